@@ -1,0 +1,268 @@
+// extern "C" surface, part 1: error string, host format helpers and the op-level entry points.
+// The op-level calls own one lazily grown device scratch area per process (activation
+// codes, split-attention partials, rope tables); they are for one caller thread at a time.
+#include <math.h>
+
+#include <vector>
+
+#include "common.h"
+
+namespace fh {
+
+int32_t qweight_upload(uint32_t wdtype, const uint8_t* raw_host, uint32_t K, uint32_t N, QWeight* out) {
+    QWeight w;
+    w.wdtype = wdtype; w.K = K; w.N = N; w.owns = true;
+    std::vector<uint8_t> qs(w.qs_bytes());
+    std::vector<uint16_t> sc((size_t)N * (K / 32));
+    repack_host(wdtype, raw_host, K, N, qs.data(), sc.data());
+    FH_HIP(hipMalloc((void**)&w.qs, std::max<size_t>(qs.size(), 16)));
+    hipError_t e = hipMalloc((void**)&w.scales, std::max<size_t>(w.scales_bytes(), 16));
+    if (e != hipSuccess) { (void)hipFree(w.qs); return fail(FORGE_HIP_ERR_HIP, "hipMalloc(scales) failed"); }
+    e = hipMemcpy(w.qs, qs.data(), qs.size(), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(w.scales, sc.data(), w.scales_bytes(), hipMemcpyHostToDevice);
+    if (e != hipSuccess) { qweight_free(&w); return fail(FORGE_HIP_ERR_HIP, std::string("weight upload: ") + hipGetErrorString(e)); }
+    *out = w;
+    return FORGE_HIP_OK;
+}
+
+void qweight_free(QWeight* w) {
+    if (w->owns) {
+        if (w->qs) (void)hipFree(w->qs);
+        if (w->scales) (void)hipFree(w->scales);
+    }
+    w->qs = nullptr; w->scales = nullptr; w->owns = false;
+}
+
+namespace {
+
+struct Scratch {
+    void* p = nullptr;
+    size_t cap = 0;
+    int32_t reserve(size_t n) {
+        if (n <= cap) return FORGE_HIP_OK;
+        if (p) { FH_HIP(hipFree(p)); p = nullptr; cap = 0; }
+        FH_HIP(hipMalloc(&p, n));
+        cap = n;
+        return FORGE_HIP_OK;
+    }
+};
+Scratch g_act;    // quantised activations: codes then scales
+Scratch g_attn;   // decode-attention partials / argmax partials
+Scratch g_rope;   // cos | sin tables
+
+inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
+
+bool valid_wdtype(uint32_t t) { return t == FORGE_HIP_Q8_0 || t == FORGE_HIP_Q4_0; }
+
+// Quantise x[M][K] into the shared scratch; returns pointers.
+int32_t quantise_into_scratch(const float* x, uint32_t M, uint32_t K, int8_t** q, uint16_t** sc, hipStream_t s) {
+    const size_t qbytes = align256((size_t)M * K);
+    const size_t sbytes = (size_t)M * (K / 32) * 2;
+    int32_t rc = g_act.reserve(qbytes + sbytes);
+    if (rc) return rc;
+    *q = reinterpret_cast<int8_t*>(g_act.p);
+    *sc = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(g_act.p) + qbytes);
+    launch_quantize_act(x, M, K, *q, *sc, s);
+    return FORGE_HIP_OK;
+}
+
+}  // namespace
+}  // namespace fh
+
+using namespace fh;
+
+struct forge_hip_qweight { QWeight w; };
+
+extern "C" {
+
+const char* forge_hip_last_error(void) { return last_error_cstr(); }
+
+int32_t forge_hip_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+float forge_hip_f16_to_f32(uint16_t bits) { return f16_to_f32_host(bits); }
+uint16_t forge_hip_f32_to_f16(float x) { return f32_to_f16_host(x); }
+
+int32_t forge_hip_quantize_f32(uint32_t wdtype, const float* data_host, uint64_t n, uint8_t* out_host) {
+    FH_CHECK(valid_wdtype(wdtype), "quantize_f32: wdtype must be Q8_0 (8) or Q4_0 (2)");
+    FH_CHECK(data_host && out_host, "quantize_f32: null pointer");
+    quantize_host(wdtype, data_host, n, out_host);
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_dequant(uint32_t wdtype, const uint8_t* data_host, uint64_t n, float* out_host) {
+    FH_CHECK(valid_wdtype(wdtype), "dequant: wdtype must be Q8_0 (8) or Q4_0 (2)");
+    FH_CHECK(data_host && out_host, "dequant: null pointer");
+    dequant_host(wdtype, data_host, n, out_host);
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_qweight_create(uint32_t wdtype, const uint8_t* raw_host, uint32_t K, uint32_t N,
+                                 forge_hip_qweight** out) {
+    FH_CHECK(out, "qweight_create: null out");
+    *out = nullptr;
+    FH_CHECK(valid_wdtype(wdtype), "qweight_create: wdtype must be Q8_0 (8) or Q4_0 (2)");
+    FH_CHECK(raw_host, "qweight_create: null weights");
+    FH_CHECK(K >= 32 && K % 32 == 0 && N >= 1, "qweight_create: K must be a positive multiple of 32 and N >= 1");
+    if (forge_hip_device_count() < 1) return fail(FORGE_HIP_ERR_NO_DEVICE, "no HIP device");
+    forge_hip_qweight* h = new forge_hip_qweight();
+    int32_t rc = qweight_upload(wdtype, raw_host, K, N, &h->w);
+    if (rc) { delete h; return rc; }
+    *out = h;
+    return FORGE_HIP_OK;
+}
+
+void forge_hip_qweight_destroy(forge_hip_qweight* w) {
+    if (!w) return;
+    qweight_free(&w->w);
+    delete w;
+}
+
+int32_t forge_hip_quantize_act(const float* x_dev, uint32_t M, uint32_t K, int8_t* q_dev, uint16_t* scales_dev,
+                               void* stream) {
+    FH_CHECK(x_dev && q_dev && scales_dev, "quantize_act: null pointer");
+    FH_CHECK(K % 32 == 0, "quantize_act: K must be a multiple of 32");
+    launch_quantize_act(x_dev, M, K, q_dev, scales_dev, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_gemv_q(const forge_hip_qweight* w, const float* x_dev, float* y_dev, void* stream) {
+    FH_CHECK(w && x_dev && y_dev, "gemv_q: null pointer");
+    FH_CHECK(gemv_k_supported(w->w.K), "gemv_q: K must be a multiple of 32, at most 16384");
+    int8_t* q; uint16_t* sc;
+    int32_t rc = quantise_into_scratch(x_dev, 1, w->w.K, &q, &sc, (hipStream_t)stream);
+    if (rc) return rc;
+    launch_gemv(w->w, q, sc, y_dev, false, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, void* stream) {
+    FH_CHECK(w && x_dev && y_dev, "gemm_q: null pointer");
+    if (M == 0) return FORGE_HIP_OK;
+    int8_t* q; uint16_t* sc;
+    int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream);
+    if (rc) return rc;
+    launch_gemm(w->w, q, sc, M, y_dev, w->w.N, false, nullptr, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, uint32_t M, int32_t* out_dev,
+                              uint32_t path, void* stream) {
+    FH_CHECK(w && x_dev && out_dev, "block_isums: null pointer");
+    FH_CHECK(path <= 1, "block_isums: path must be 0 (GEMV kernel) or 1 (MFMA GEMM kernel)");
+    if (M == 0) return FORGE_HIP_OK;
+    int8_t* q; uint16_t* sc;
+    int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream);
+    if (rc) return rc;
+    const size_t nblk = w->w.K / 32;
+    if (path == 0) {
+        FH_CHECK(gemv_k_supported(w->w.K), "block_isums: K too large for the GEMV path");
+        for (uint32_t r = 0; r < M; r++)
+            launch_gemv_isums(w->w, q + (size_t)r * w->w.K, out_dev + (size_t)r * w->w.N * nblk, (hipStream_t)stream);
+    } else {
+        // The GEMM kernel also writes y; give it the tail of the scratch as a sink.
+        Scratch& sink = g_attn;
+        rc = sink.reserve((size_t)M * w->w.N * sizeof(float));
+        if (rc) return rc;
+        launch_gemm(w->w, q, sc, M, reinterpret_cast<float*>(sink.p), w->w.N, false, out_dev, (hipStream_t)stream);
+    }
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_rms_norm(const float* x_dev, const float* w_dev, float eps, uint32_t M, uint32_t H, float* out_dev,
+                           void* stream) {
+    FH_CHECK(x_dev && w_dev && out_dev, "rms_norm: null pointer");
+    FH_CHECK(H % 4 == 0 && H >= 4, "rms_norm: H must be a multiple of 4");
+    launch_rmsnorm(x_dev, w_dev, eps, M, H, out_dev, nullptr, nullptr, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_silu_mul(const float* gate_dev, const float* up_dev, uint64_t n, float* out_dev, void* stream) {
+    FH_CHECK(gate_dev && up_dev && out_dev, "silu_mul: null pointer");
+    FH_CHECK(n % 4 == 0 && n <= 0xFFFFFFFFull, "silu_mul: n must be a multiple of 4");
+    launch_silu_mul(gate_dev, up_dev, 1, (uint32_t)n, (uint32_t)n, out_dev, nullptr, nullptr, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_rope_kv_store(float* q_dev, float* k_dev, const float* v_dev, uint16_t* k_cache_dev,
+                                uint16_t* v_cache_dev, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
+                                uint32_t head_dim, float theta, void* stream) {
+    FH_CHECK(q_dev && k_dev && v_dev && k_cache_dev && v_cache_dev, "rope_kv_store: null pointer");
+    FH_CHECK(head_dim % 2 == 0 && head_dim >= 2 && heads >= 1 && kv_heads >= 1, "rope_kv_store: bad head shape");
+    if (M == 0) return FORGE_HIP_OK;
+    const uint32_t half = head_dim / 2, n_pos = base_pos + M;
+    // rope_freqs + per-position sin_cos, emit.rs:501-517, evaluated with the host C library.
+    std::vector<float> tab((size_t)2 * n_pos * half);
+    for (uint32_t i = 0; i < half; i++) {
+        const float f = 1.0f / powf(theta, 2.0f * (float)i / (float)head_dim);
+        for (uint32_t p = 0; p < n_pos; p++) {
+            const float a = (float)p * f;
+            tab[(size_t)p * half + i] = cosf(a);
+            tab[(size_t)n_pos * half + (size_t)p * half + i] = sinf(a);
+        }
+    }
+    int32_t rc = g_rope.reserve(tab.size() * sizeof(float));
+    if (rc) return rc;
+    FH_HIP(hipMemcpyAsync(g_rope.p, tab.data(), tab.size() * sizeof(float), hipMemcpyHostToDevice, (hipStream_t)stream));
+    FH_HIP(hipStreamSynchronize((hipStream_t)stream));   // `tab` is pageable and about to go out of scope
+    const float* cos_t = reinterpret_cast<const float*>(g_rope.p);
+    const float* sin_t = cos_t + (size_t)n_pos * half;
+    launch_rope_kv_store(q_dev, k_dev, v_dev, heads * head_dim, kv_heads * head_dim, k_cache_dev, v_cache_dev, M,
+                         base_pos, nullptr, heads, kv_heads, head_dim, cos_t, sin_t, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+static int32_t check_attn_shape(const char* who, uint32_t heads, uint32_t kv_heads, uint32_t head_dim) {
+    if (!attn_head_dim_supported(head_dim)) return fail(FORGE_HIP_ERR_INVALID, std::string(who) + ": head_dim must be 64, 96 or 128");
+    if (kv_heads == 0 || heads == 0 || heads % kv_heads != 0)
+        return fail(FORGE_HIP_ERR_INVALID, std::string(who) + ": heads must be a positive multiple of kv_heads");
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_attn_prefill_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
+                                     float* out_dev, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
+                                     uint32_t head_dim, void* stream) {
+    FH_CHECK(q_dev && k_cache_dev && v_cache_dev && out_dev, "attn_prefill: null pointer");
+    int32_t rc = check_attn_shape("attn_prefill", heads, kv_heads, head_dim);
+    if (rc) return rc;
+    launch_attn_prefill(q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, M, base_pos, heads,
+                        kv_heads, head_dim, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
+                                    float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
+                                    uint32_t head_dim, void* stream) {
+    FH_CHECK(q_dev && k_cache_dev && v_cache_dev && out_dev, "attn_decode: null pointer");
+    FH_CHECK(seq_len >= 1, "attn_decode: seq_len must be at least 1");
+    int32_t rc = check_attn_shape("attn_decode", heads, kv_heads, head_dim);
+    if (rc) return rc;
+    rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
+    if (rc) return rc;
+    launch_attn_decode(q_dev, k_cache_dev, v_cache_dev, out_dev, nullptr, nullptr, seq_len, nullptr, heads, kv_heads,
+                       head_dim, g_attn.p, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void* stream) {
+    FH_CHECK(x_dev && out_dev && n >= 1, "argmax: null pointer or empty input");
+    int32_t rc = g_attn.reserve(ARGMAX_BLOCKS * 8);
+    if (rc) return rc;
+    launch_argmax(x_dev, n, out_dev, g_attn.p, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+}  // extern "C"

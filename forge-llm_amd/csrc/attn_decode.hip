@@ -1,0 +1,207 @@
+// Decode attention (attention_flash, emit.rs:656-715) over an fp16 KV cache, split along the
+// sequence so that one query fills the GPU ("flash decoding"): grid = (kv head groups,
+// DECODE_SPLITS).  HBM-bound: each K/V row is read once per group of query heads that share
+// it.  A key row of head_dim fp16 values is spread over LPK lanes (16 bytes each); the
+// lanes of a wave cover 64/LPK keys per load and every key slot keeps its own online-softmax
+// state, so the loop needs no cross-slot traffic; slots, waves and splits are merged at
+// the end with the usual (max, sum, acc) rescaling.
+#include "common.h"
+#include "device_utils.h"
+
+namespace fh {
+
+struct __attribute__((aligned(16))) Half8 { uint32_t w[4]; };
+
+__device__ __forceinline__ void unpack8(const Half8& h, float* f) {
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        f[2 * i] = f16_bits_to_f32((uint16_t)(h.w[i] & 0xFFFFu));
+        f[2 * i + 1] = f16_bits_to_f32((uint16_t)(h.w[i] >> 16));
+    }
+}
+
+// merge (m2,l2,a2) into (m,l,a)
+template <int NV>
+__device__ __forceinline__ void merge_state(float& m, float& l, float* a, float m2, float l2, const float* a2) {
+    const float mn = fmaxf(m, m2);
+    const float s1 = (m == -INFINITY) ? 0.f : __expf(m - mn);
+    const float s2 = (m2 == -INFINITY) ? 0.f : __expf(m2 - mn);
+    l = l * s1 + l2 * s2;
+#pragma unroll
+    for (int i = 0; i < NV; i++) a[i] = a[i] * s1 + a2[i] * s2;
+    m = mn;
+}
+
+// workspace record per (kv group, split, head-in-group): [HD acc][m][l]
+template <int HD, int GT>
+__global__ __launch_bounds__(256) void attn_decode_split_kernel(const float* __restrict__ q,
+                                                                const uint16_t* __restrict__ kc,
+                                                                const uint16_t* __restrict__ vc,
+                                                                float* __restrict__ ws, uint32_t seq_len_arg,
+                                                                const uint32_t* __restrict__ pos_dev, uint32_t heads,
+                                                                uint32_t kv_heads, uint32_t gsize) {
+    constexpr int LPK = HD <= 64 ? 8 : 16;   // lanes per key row
+    constexpr int KPW = 64 / LPK;            // keys per wave load
+    constexpr int REC = HD + 2;
+    __shared__ float sh[4][GT][REC];
+
+    const uint32_t seq = pos_dev ? (*pos_dev + 1) : seq_len_arg;
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t c = lane % LPK, slot = lane / LPK;
+    const bool dvalid = c * 8 < HD;
+    const uint32_t gpk = gsize / GT;   // head sub-groups per kv head
+    const uint32_t kvh = blockIdx.x / gpk, sub = blockIdx.x % gpk;
+    const uint32_t h0 = kvh * gsize + sub * GT;
+    const uint32_t split = blockIdx.y, nsplit = gridDim.y;
+    const float scale = 1.0f / sqrtf((float)HD);
+    const uint32_t kv_stride = kv_heads * HD;
+
+    uint32_t chunk = (seq + nsplit - 1) / nsplit;
+    chunk = (chunk + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
+    const uint32_t t0 = split * chunk;
+    const uint32_t t1 = min(seq, t0 + chunk);
+
+    float qf[GT][8];
+#pragma unroll
+    for (int g = 0; g < GT; g++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) qf[g][i] = dvalid ? q[(size_t)(h0 + g) * HD + c * 8 + i] : 0.f;
+
+    float m[GT], l[GT], acc[GT][8];
+#pragma unroll
+    for (int g = 0; g < GT; g++) {
+        m[g] = -INFINITY; l[g] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[g][i] = 0.f;
+    }
+
+    for (uint32_t tb = t0 + wave * KPW; tb < t1; tb += 4 * KPW) {
+        const uint32_t t = tb + slot;
+        const bool valid = t < t1;
+        Half8 kr = {{0, 0, 0, 0}}, vr = {{0, 0, 0, 0}};
+        if (valid && dvalid) {
+            const size_t off = (size_t)t * kv_stride + kvh * HD + c * 8;
+            kr = *reinterpret_cast<const Half8*>(kc + off);
+            vr = *reinterpret_cast<const Half8*>(vc + off);
+        }
+        float kf[8], vf[8];
+        unpack8(kr, kf);
+        unpack8(vr, vf);
+#pragma unroll
+        for (int g = 0; g < GT; g++) {
+            float d = 0.f;
+#pragma unroll
+            for (int i = 0; i < 8; i++) d += qf[g][i] * kf[i];
+#pragma unroll
+            for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, WAVE);
+            if (valid) {
+                const float s = d * scale;
+                const float mn = fmaxf(m[g], s);
+                const float alpha = __expf(m[g] - mn);   // m = -inf on the first key: exp(-inf) = 0
+                const float p = __expf(s - mn);
+                l[g] = l[g] * alpha + p;
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[g][i] = acc[g][i] * alpha + p * vf[i];
+                m[g] = mn;
+            }
+        }
+    }
+
+    // merge the key slots of the wave
+#pragma unroll
+    for (int g = 0; g < GT; g++) {
+#pragma unroll
+        for (int o = LPK; o < 64; o <<= 1) {
+            float m2 = __shfl_xor(m[g], o, WAVE), l2 = __shfl_xor(l[g], o, WAVE);
+            float a2[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) a2[i] = __shfl_xor(acc[g][i], o, WAVE);
+            merge_state<8>(m[g], l[g], acc[g], m2, l2, a2);
+        }
+        if (slot == 0 && dvalid) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) sh[wave][g][c * 8 + i] = acc[g][i];
+            if (c == 0) { sh[wave][g][HD] = m[g]; sh[wave][g][HD + 1] = l[g]; }
+        }
+    }
+    __syncthreads();
+    // merge the four waves: thread d of the first GT*HD threads owns one output element
+    for (uint32_t e = threadIdx.x; e < GT * HD; e += 256) {
+        const uint32_t g = e / HD, d = e % HD;
+        float mm = sh[0][g][HD], ll = sh[0][g][HD + 1], a = sh[0][g][d];
+        for (int w = 1; w < 4; w++) {
+            float a2 = sh[w][g][d];
+            merge_state<1>(mm, ll, &a, sh[w][g][HD], sh[w][g][HD + 1], &a2);
+        }
+        float* rec = ws + ((size_t)(h0 + g) * nsplit + split) * REC;
+        rec[d] = a;
+        if (d == 0) { rec[HD] = mm; rec[HD + 1] = ll; }
+    }
+}
+
+// One workgroup of HD threads per head: merge the splits, normalise, optionally quantise
+// the 32-element blocks of the output for the O projection.
+template <int HD>
+__global__ void attn_decode_combine_kernel(const float* __restrict__ ws, uint32_t nsplit, float* __restrict__ out,
+                                           int8_t* __restrict__ oq, uint16_t* __restrict__ osc) {
+    constexpr int REC = HD + 2;
+    const uint32_t h = blockIdx.x, d = threadIdx.x;
+    const float* base = ws + (size_t)h * nsplit * REC;
+    float mm = -INFINITY;
+    for (uint32_t s = 0; s < nsplit; s++) mm = fmaxf(mm, base[s * REC + HD]);
+    float num = 0.f, den = 0.f;
+    for (uint32_t s = 0; s < nsplit; s++) {
+        const float ms = base[s * REC + HD];
+        const float wgt = (ms == -INFINITY) ? 0.f : __expf(ms - mm);
+        num += wgt * base[s * REC + d];
+        den += wgt * base[s * REC + HD + 1];
+    }
+    const float o = num * (1.0f / den);
+    if (out) out[(size_t)h * HD + d] = o;
+    if (oq) {
+        float amax = fabsf(o);
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+        float inv;
+        const float sc = act_scale(amax, inv);
+        oq[(size_t)h * HD + d] = (int8_t)quant_code(o * inv);
+        if ((d & 31) == 0) osc[((size_t)h * HD + d) / 32] = f32_to_f16_bits(sc);
+    }
+}
+
+size_t attn_decode_workspace_bytes(uint32_t heads, uint32_t hd) {
+    return (size_t)heads * DECODE_SPLITS * (hd + 2) * sizeof(float);
+}
+
+bool attn_head_dim_supported(uint32_t hd) { return hd == 64 || hd == 96 || hd == 128; }
+
+namespace {
+template <int HD, int GT>
+void launch_split(const float* q, const uint16_t* kc, const uint16_t* vc, float* ws, uint32_t seq,
+                  const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, hipStream_t s) {
+    const uint32_t gsize = heads / kv_heads;
+    dim3 grid(kv_heads * (gsize / GT), DECODE_SPLITS);
+    attn_decode_split_kernel<HD, GT><<<grid, 256, 0, s>>>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, gsize);
+}
+template <int HD>
+void launch_hd(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
+               uint32_t seq, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, float* ws, hipStream_t s) {
+    const uint32_t gsize = heads / kv_heads;
+    if (gsize % 4 == 0) launch_split<HD, 4>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
+    else if (gsize % 3 == 0) launch_split<HD, 3>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
+    else if (gsize % 2 == 0) launch_split<HD, 2>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
+    else launch_split<HD, 1>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
+    attn_decode_combine_kernel<HD><<<heads, HD, 0, s>>>(ws, DECODE_SPLITS, out, oq, osc);
+}
+}  // namespace
+
+void launch_attn_decode(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
+                        uint32_t seq_len, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd,
+                        void* workspace, hipStream_t s) {
+    float* ws = reinterpret_cast<float*>(workspace);
+    if (hd == 64) launch_hd<64>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, ws, s);
+    else if (hd == 96) launch_hd<96>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, ws, s);
+    else launch_hd<128>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, ws, s);
+}
+
+}  // namespace fh

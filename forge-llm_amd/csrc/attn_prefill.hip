@@ -1,0 +1,204 @@
+// Batched-prefill causal attention (attention_flash_batch, emit.rs:754-883) over an fp16 KV
+// cache, with both matrix products on fp16 MFMA (v_mfma_f32_32x32x16_f16) and the online
+// softmax in f32.
+//
+// Workgroup = 4 waves = 128 consecutive queries of one head; each wave owns 32 queries.
+// K/V are streamed in tiles of 64 keys through LDS (K row-major, V transposed so that the
+// contraction index of P.V is contiguous per lane).
+//
+// Both products are computed transposed, S^T = K Q^T and O^T = V^T P^T.  In the 32x32 MFMA
+// result layout a lane then owns ONE query (column = lane%32) and 16 keys (or 16 head dims),
+// so the softmax row statistics are per-lane scalars (plus one exchange with lane^32), and
+// the exponentiated scores are already in the register layout the second MFMA wants for
+// its B operand.
+#include "common.h"
+#include "device_utils.h"
+
+namespace fh {
+
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int QW = 32;        // queries per wave
+constexpr int QB = 128;       // queries per workgroup
+constexpr int KT = 64;        // keys per tile
+
+template <int HD>
+__global__ __launch_bounds__(256) void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc,
+                                                           const uint16_t* __restrict__ vc, float* __restrict__ out,
+                                                           uint32_t q_stride, uint32_t out_stride, uint32_t M,
+                                                           uint32_t base_pos, uint32_t heads, uint32_t kv_heads) {
+    constexpr int KS = HD + 8;    // K tile row stride (halfs): 16-byte pad
+    constexpr int VS = KT + 4;    // V^T tile row stride (halfs): 8-byte pad
+    constexpr int PIECES = KT * HD / 8 / 256;   // 16-byte pieces per thread per tile
+    constexpr int NS = HD / 16;   // MFMA k-steps over head_dim
+    constexpr int ND = HD / 32;   // 32-wide head_dim tiles of the output
+    __shared__ __attribute__((aligned(16))) _Float16 Ks[KT * KS];
+    __shared__ __attribute__((aligned(16))) _Float16 Vt[HD * VS];
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t lq = lane & 31, lh = lane >> 5;
+    const uint32_t head = blockIdx.y, kvh = head / (heads / kv_heads);
+    // heaviest (latest) query tiles first: they stream the most keys
+    const uint32_t qtile = gridDim.x - 1 - blockIdx.x;
+    const uint32_t q0 = qtile * QB;
+    const uint32_t kv_stride = kv_heads * HD;
+    const uint32_t seq_total = base_pos + M;
+    const float scale = 1.0f / sqrtf((float)HD);
+
+    // ---- Q fragment (B operand of S^T = K Q^T): lane (lq, lh) holds q[row][16 s + 8 lh + 0..7]
+    const uint32_t qrow = q0 + wave * QW + lq;
+    const uint32_t qpos = base_pos + qrow;
+    v8h qf[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        if (qrow < M) {
+            const float4* p = reinterpret_cast<const float4*>(q + (size_t)qrow * q_stride + head * HD + 16 * s + 8 * lh);
+            float4 a = p[0], b = p[1];
+            qf[s] = (v8h){(_Float16)a.x, (_Float16)a.y, (_Float16)a.z, (_Float16)a.w,
+                          (_Float16)b.x, (_Float16)b.y, (_Float16)b.z, (_Float16)b.w};
+        } else {
+            qf[s] = (v8h){0, 0, 0, 0, 0, 0, 0, 0};
+        }
+    }
+
+    v16f oacc[ND];
+#pragma unroll
+    for (int d = 0; d < ND; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) oacc[d][r] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    const uint32_t wg_max_pos = base_pos + min(q0 + QB, M) - 1;
+    const uint32_t ntiles = wg_max_pos / KT + 1;
+    const uint32_t wave_max_pos = base_pos + min(q0 + wave * QW + QW, M) - 1;   // may underflow if wave is empty
+    const bool wave_active = q0 + wave * QW < M;
+
+    int4 kreg[PIECES], vreg[PIECES];
+    auto load_tile = [&](uint32_t kt) {
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+            const uint32_t idx = tid + 256 * i, key = idx / (HD / 8), dc = idx % (HD / 8);
+            const uint32_t t = kt * KT + key;
+            if (t < seq_total) {
+                const size_t off = (size_t)t * kv_stride + kvh * HD + dc * 8;
+                kreg[i] = *reinterpret_cast<const int4*>(kc + off);
+                vreg[i] = *reinterpret_cast<const int4*>(vc + off);
+            } else {
+                kreg[i] = make_int4(0, 0, 0, 0);
+                vreg[i] = make_int4(0, 0, 0, 0);
+            }
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int i = 0; i < PIECES; i++) {
+            const uint32_t idx = tid + 256 * i, key = idx / (HD / 8), dc = idx % (HD / 8);
+            *reinterpret_cast<int4*>(Ks + key * KS + dc * 8) = kreg[i];
+            const uint32_t w[4] = {(uint32_t)vreg[i].x, (uint32_t)vreg[i].y, (uint32_t)vreg[i].z, (uint32_t)vreg[i].w};
+            uint16_t* vt = reinterpret_cast<uint16_t*>(Vt);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                vt[(dc * 8 + 2 * e) * VS + key] = (uint16_t)(w[e] & 0xFFFFu);
+                vt[(dc * 8 + 2 * e + 1) * VS + key] = (uint16_t)(w[e] >> 16);
+            }
+        }
+    };
+
+    load_tile(0);
+    for (uint32_t kt = 0; kt < ntiles; kt++) {
+        __syncthreads();   // everyone is done reading the previous tile
+        store_tile();
+        __syncthreads();
+        if (kt + 1 < ntiles) load_tile(kt + 1);
+        if (!wave_active || kt * KT > wave_max_pos) continue;   // tile entirely in this wave's future
+
+        // ---- S^T tiles: sacc[kk][r] = score(key kt*64 + kk*32 + 8(r/4) + 4 lh + r%4, query lq)
+        v16f sacc[2];
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) sacc[kk][r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                v8h kf = *reinterpret_cast<const v8h*>(Ks + (kk * 32 + lq) * KS + 16 * s + 8 * lh);
+                sacc[kk] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], sacc[kk], 0, 0, 0);
+            }
+        }
+        // ---- causal mask + online softmax (per-lane scalars)
+        float m_tile = -INFINITY;
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const uint32_t t = kt * KT + kk * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                float s = sacc[kk][r] * scale;
+                s = (t <= qpos) ? s : -INFINITY;
+                sacc[kk][r] = s;
+                m_tile = fmaxf(m_tile, s);
+            }
+        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, WAVE));
+        const float m_new = fmaxf(m_run, m_tile);
+        // m_new is finite from the first tile on (key 0 is visible to every query)
+        const float alpha = __expf(m_run - m_new);
+        float l_tile = 0.f;
+        v8h pb[2][2];
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float p = __expf(sacc[kk][8 * j + e] - m_new);   // exp(-inf) = 0 for masked keys
+                    l_tile += p;
+                    pb[kk][j][e] = (_Float16)p;
+                }
+        l_run = l_run * alpha + l_tile;
+        m_run = m_new;
+#pragma unroll
+        for (int d = 0; d < ND; d++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[d][r] *= alpha;
+        // ---- O^T += V^T P^T
+#pragma unroll
+        for (int d = 0; d < ND; d++)
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const _Float16* vrow = Vt + (d * 32 + lq) * VS + kk * 32 + 16 * j + 4 * lh;
+                    v4h v0 = *reinterpret_cast<const v4h*>(vrow);
+                    v4h v1 = *reinterpret_cast<const v4h*>(vrow + 8);
+                    v8h vf = (v8h){v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                    oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pb[kk][j], oacc[d], 0, 0, 0);
+                }
+    }
+
+    // ---- normalise and store: lane (lq, lh) holds out[qrow][32 d + 8 g + 4 lh + 0..3]
+    const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+    if (qrow < M) {
+        const float inv_l = 1.0f / l_tot;
+        float* orow = out + (size_t)qrow * out_stride + head * HD;
+#pragma unroll
+        for (int d = 0; d < ND; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                float4 o = make_float4(oacc[d][4 * g] * inv_l, oacc[d][4 * g + 1] * inv_l, oacc[d][4 * g + 2] * inv_l,
+                                       oacc[d][4 * g + 3] * inv_l);
+                *reinterpret_cast<float4*>(orow + 32 * d + 8 * g + 4 * lh) = o;
+            }
+    }
+}
+
+void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, float* out,
+                         uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
+                         uint32_t hd, hipStream_t s) {
+    if (M == 0) return;
+    dim3 grid((M + QB - 1) / QB, heads);
+    if (hd == 64) attn_prefill_kernel<64><<<grid, 256, 0, s>>>(q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
+    else if (hd == 96) attn_prefill_kernel<96><<<grid, 256, 0, s>>>(q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
+    else attn_prefill_kernel<128><<<grid, 256, 0, s>>>(q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
+}
+
+}  // namespace fh

@@ -1,0 +1,111 @@
+// Shared declarations for libforge_hip: error plumbing, the device-side weight layout and
+// the launch functions each translation unit exports to the others.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "forge_hip.h"
+
+namespace fh {
+
+// ---- error plumbing -------------------------------------------------------------------
+void set_error(const std::string& msg);
+int32_t fail(int32_t code, const std::string& msg);
+
+#define FH_HIP(expr)                                                                                   \
+    do {                                                                                               \
+        hipError_t _e = (expr);                                                                        \
+        if (_e != hipSuccess)                                                                          \
+            return ::fh::fail(FORGE_HIP_ERR_HIP, std::string(#expr) + ": " + hipGetErrorString(_e)); \
+    } while (0)
+
+#define FH_CHECK(cond, msg)                                           \
+    do {                                                              \
+        if (!(cond)) return ::fh::fail(FORGE_HIP_ERR_INVALID, (msg)); \
+    } while (0)
+
+// ---- device weight layout ----------------------------------------------------------------
+// GGUF interleaves a 2-byte scale with every 32 quants (34- or 18-byte blocks, 2-byte
+// aligned).  On upload each matrix is split into two planes so that every lane can issue
+// aligned 16-byte loads:
+//   qs     Q8_0: int8  [N][K]      (row n = its K quants in order)
+//          Q4_0: uint8 [N][K/2]    (row n = its K/32 blocks of 16 packed bytes, byte j of a
+//                                   block = element j in the low nibble, j+16 in the high)
+//   scales fp16 bits [N][K/32]
+// The planes hold exactly the bytes of the GGUF blocks, regrouped; nothing is dequantised.
+struct QWeight {
+    uint32_t wdtype = 0, K = 0, N = 0;
+    uint8_t* qs = nullptr;
+    uint16_t* scales = nullptr;
+    bool owns = false;
+    size_t qs_row_bytes() const { return wdtype == FORGE_HIP_Q8_0 ? K : K / 2; }
+    size_t qs_bytes() const { return (size_t)N * qs_row_bytes(); }
+    size_t scales_bytes() const { return (size_t)N * (K / 32) * 2; }
+};
+
+// Split raw GGUF rows into the two planes (host side).
+void repack_host(uint32_t wdtype, const uint8_t* raw, uint32_t K, uint64_t N, uint8_t* qs, uint16_t* scales);
+
+// ---- host format helpers (format.hip) ------------------------------------------------------
+float f16_to_f32_host(uint16_t bits);
+uint16_t f32_to_f16_host(float x);
+void quantize_host(uint32_t wdtype, const float* d, uint64_t n, uint8_t* out);
+void dequant_host(uint32_t wdtype, const uint8_t* data, uint64_t n, float* out);
+const char* last_error_cstr();
+// Upload raw GGUF rows as planes into freshly allocated device memory.
+int32_t qweight_upload(uint32_t wdtype, const uint8_t* raw_host, uint32_t K, uint32_t N, QWeight* out);
+void qweight_free(QWeight* w);
+
+// ---- kernel launchers ------------------------------------------------------------------------
+// All are asynchronous on `s` and validate nothing: callers check shapes first.
+
+// elementwise.hip
+void launch_quantize_act(const float* x, uint32_t M, uint32_t K, int8_t* q, uint16_t* sc, hipStream_t s);
+// rms_norm of M rows; writes f32 `normed` if non-null and the quantised row (q, sc) if q non-null.
+void launch_rmsnorm(const float* x, const float* w, float eps, uint32_t M, uint32_t H, float* normed, int8_t* q,
+                    uint16_t* sc, hipStream_t s);
+// out = silu(gate)*up over M rows where gate = gu[r][0..I), up = gu[r][I..2I) when fused, else two
+// pointers; writes f32 out if non-null and quantised (q, sc) if q non-null.
+void launch_silu_mul(const float* gate, const float* up, uint32_t M, uint32_t I, uint32_t row_stride, float* out,
+                     int8_t* q, uint16_t* sc, hipStream_t s);
+// Interleaved-pair RoPE on q,k and fp16 cache write of k,v.  Position of row r is
+// (pos_dev ? *pos_dev : base_pos) + r.  q/k/v rows have strides q_stride/kv_stride floats.
+void launch_rope_kv_store(float* q, float* k, const float* v, uint32_t q_stride, uint32_t kv_stride, uint16_t* kc,
+                          uint16_t* vc, uint32_t M, uint32_t base_pos, const uint32_t* pos_dev, uint32_t heads,
+                          uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, hipStream_t s);
+void launch_embedding(const float* table, const uint32_t* tokens_dev, uint32_t M, uint32_t H, float* out,
+                      hipStream_t s);
+// Index of the LAST maximum.  `scratch` needs 2*ARGMAX_BLOCKS uint32/float pairs.
+constexpr uint32_t ARGMAX_BLOCKS = 256;
+void launch_argmax(const float* x, uint32_t n, uint32_t* out, void* scratch, hipStream_t s);
+void launch_advance(uint32_t* pos_dev, uint32_t* token_dev, const uint32_t* next_dev, hipStream_t s);
+
+// gemv.hip — y[n] (=|+=) sum_b f32(isum_b) * (a_s[b]*w_s[n][b]); activations already quantised.
+void launch_gemv(const QWeight& w, const int8_t* aq, const uint16_t* as, float* y, bool accumulate, hipStream_t s);
+void launch_gemv_isums(const QWeight& w, const int8_t* aq, int32_t* out, hipStream_t s);
+bool gemv_k_supported(uint32_t K);
+
+// gemm.hip — y[m][n] (=|+=) ...; aq int8 [M][K], as fp16 [M][K/32].  isums (optional) int32 [M][N][K/32].
+void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
+                 bool accumulate, int32_t* isums, hipStream_t s);
+
+// attn_decode.hip
+constexpr uint32_t DECODE_SPLITS = 32;
+size_t attn_decode_workspace_bytes(uint32_t heads, uint32_t hd);
+// seq_len = pos_dev ? *pos_dev + 1 : seq_len.  Writes f32 out if non-null and quantised (q, sc) if q non-null.
+void launch_attn_decode(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
+                        uint32_t seq_len, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd,
+                        void* workspace, hipStream_t s);
+
+// attn_prefill.hip
+// q rows / out rows have strides q_stride / out_stride floats (q may live inside a fused qkv buffer).
+void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, float* out,
+                         uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
+                         uint32_t hd, hipStream_t s);
+
+bool attn_head_dim_supported(uint32_t hd);
+
+}  // namespace fh

@@ -1,0 +1,251 @@
+// Small bandwidth-trivial kernels around the matmuls: activation quantiser, RMSNorm,
+// SiLU-gate, RoPE + fp16 KV write, embedding gather, argmax.  Each fuses the int8 block
+// quantisation of its output, because the consumer is always a quantised matmul
+// (emit.rs:1410-1440 re-quantises the same vector once per matmul; the result is identical).
+#include "common.h"
+#include "device_utils.h"
+
+namespace fh {
+
+// ---- quantize_to_q8_0_blocks_into (emit.rs:1410-1440), planes instead of 34-byte blocks ----
+__global__ __launch_bounds__(256) void quantize_act_kernel(const float* __restrict__ x, uint64_t n4,
+                                                           uint32_t* __restrict__ q, uint16_t* __restrict__ sc) {
+    uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < n4) v = reinterpret_cast<const float4*>(x)[i];
+    uint16_t sb;
+    uint32_t packed = quantize_block_part(v, sb);
+    if (i < n4) {
+        q[i] = packed;
+        if ((i & 7) == 0) sc[i >> 3] = sb;
+    }
+}
+
+void launch_quantize_act(const float* x, uint32_t M, uint32_t K, int8_t* q, uint16_t* sc, hipStream_t s) {
+    uint64_t n4 = (uint64_t)M * K / 4;
+    if (n4 == 0) return;
+    uint32_t grid = (uint32_t)((n4 + 255) / 256);
+    quantize_act_kernel<<<grid, 256, 0, s>>>(x, n4, reinterpret_cast<uint32_t*>(q), sc);
+}
+
+// ---- rms_norm (emit.rs:327-334) + optional block quantisation -------------------------------
+// One workgroup per row.  ss = sum x^2 (tree order, f32), inv = 1/sqrt(ss/n + eps),
+// out = (x*inv)*w.
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                      float eps, uint32_t H, float* __restrict__ normed,
+                                                      uint32_t* __restrict__ q, uint16_t* __restrict__ sc) {
+    __shared__ float red[4];
+    const uint32_t row = blockIdx.x, tid = threadIdx.x;
+    const float4* xr = reinterpret_cast<const float4*>(x + (size_t)row * H);
+    const uint32_t n4 = H / 4;
+    float ss = 0.f;
+    for (uint32_t i = tid; i < n4; i += 256) {
+        float4 v = xr[i];
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = wave_sum(ss);
+    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    __syncthreads();
+    ss = (red[0] + red[1]) + (red[2] + red[3]);
+    const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+    const float4* wr = reinterpret_cast<const float4*>(w);
+    const uint32_t n4_pad = (n4 + 255) / 256 * 256;
+    for (uint32_t i = tid; i < n4_pad; i += 256) {
+        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (i < n4) {
+            float4 v = xr[i], g = wr[i];
+            o.x = v.x * inv * g.x; o.y = v.y * inv * g.y; o.z = v.z * inv * g.z; o.w = v.w * inv * g.w;
+            if (normed) reinterpret_cast<float4*>(normed + (size_t)row * H)[i] = o;
+        }
+        if (q) {
+            uint16_t sb;
+            uint32_t packed = quantize_block_part(o, sb);
+            if (i < n4) {
+                q[(size_t)row * n4 + i] = packed;
+                if ((i & 7) == 0) sc[(size_t)row * (H / 32) + (i >> 3)] = sb;
+            }
+        }
+    }
+}
+
+void launch_rmsnorm(const float* x, const float* w, float eps, uint32_t M, uint32_t H, float* normed, int8_t* q,
+                    uint16_t* sc, hipStream_t s) {
+    if (M == 0) return;
+    rmsnorm_kernel<<<M, 256, 0, s>>>(x, w, eps, H, normed, reinterpret_cast<uint32_t*>(q), sc);
+}
+
+// ---- silu_mul (emit.rs:380-386) + optional block quantisation --------------------------------
+__global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                       uint32_t I4, uint32_t row_stride, uint64_t total4,
+                                                       float* __restrict__ out, uint32_t* __restrict__ q,
+                                                       uint16_t* __restrict__ sc) {
+    uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (i < total4) {
+        uint64_t r = i / I4, c = i % I4;
+        float4 g = reinterpret_cast<const float4*>(gate + r * row_stride)[c];
+        float4 u = reinterpret_cast<const float4*>(up + r * row_stride)[c];
+        o.x = (g.x / (1.0f + expf(-g.x))) * u.x;
+        o.y = (g.y / (1.0f + expf(-g.y))) * u.y;
+        o.z = (g.z / (1.0f + expf(-g.z))) * u.z;
+        o.w = (g.w / (1.0f + expf(-g.w))) * u.w;
+        if (out) reinterpret_cast<float4*>(out)[i] = o;
+    }
+    if (q) {
+        uint16_t sb;
+        uint32_t packed = quantize_block_part(o, sb);
+        if (i < total4) {
+            q[i] = packed;
+            if ((i & 7) == 0) sc[i >> 3] = sb;
+        }
+    }
+}
+
+void launch_silu_mul(const float* gate, const float* up, uint32_t M, uint32_t I, uint32_t row_stride, float* out,
+                     int8_t* q, uint16_t* sc, hipStream_t s) {
+    uint64_t total4 = (uint64_t)M * I / 4;
+    if (total4 == 0) return;
+    uint32_t grid = (uint32_t)((total4 + 255) / 256);
+    silu_mul_kernel<<<grid, 256, 0, s>>>(gate, up, I / 4, row_stride, total4, out, reinterpret_cast<uint32_t*>(q), sc);
+}
+
+// ---- rope (emit.rs:508-528) + fp16 KV write ------------------------------------------------------
+// One thread per (row, element pair).  Pair p of a head rotates (x[2p], x[2p+1]) by the
+// angle pos*freq[p]; cos/sin come from a table built on the host with the C library, so
+// they are the values the CPU path computes.
+__global__ __launch_bounds__(256) void rope_kv_store_kernel(float* __restrict__ q, float* __restrict__ k,
+                                                            const float* __restrict__ v, uint32_t q_stride,
+                                                            uint32_t kv_stride, uint16_t* __restrict__ kc,
+                                                            uint16_t* __restrict__ vc, uint32_t base_pos,
+                                                            const uint32_t* __restrict__ pos_dev, uint32_t heads,
+                                                            uint32_t kv_heads, uint32_t hd,
+                                                            const float* __restrict__ cos_t,
+                                                            const float* __restrict__ sin_t) {
+    const uint32_t r = blockIdx.y;
+    const uint32_t pos = (pos_dev ? *pos_dev : base_pos) + r;
+    const uint32_t half = hd / 2;
+    const uint32_t qp = heads * half, kp = kv_heads * half;
+    const uint32_t p = blockIdx.x * 256 + threadIdx.x;
+    if (p < qp) {
+        const uint32_t i = p % half;
+        const float c = cos_t[(size_t)pos * half + i], s = sin_t[(size_t)pos * half + i];
+        float2* ptr = reinterpret_cast<float2*>(q + (size_t)r * q_stride) + p;
+        float2 x = *ptr;
+        float2 o;
+        o.x = __fsub_rn(__fmul_rn(x.x, c), __fmul_rn(x.y, s));
+        o.y = __fadd_rn(__fmul_rn(x.x, s), __fmul_rn(x.y, c));
+        *ptr = o;
+    } else if (p < qp + kp) {
+        const uint32_t pk = p - qp, i = pk % half;
+        const float c = cos_t[(size_t)pos * half + i], s = sin_t[(size_t)pos * half + i];
+        float2* ptr = reinterpret_cast<float2*>(k + (size_t)r * kv_stride) + pk;
+        float2 x = *ptr;
+        float2 o;
+        o.x = __fsub_rn(__fmul_rn(x.x, c), __fmul_rn(x.y, s));
+        o.y = __fadd_rn(__fmul_rn(x.x, s), __fmul_rn(x.y, c));
+        *ptr = o;
+        uint32_t packed = (uint32_t)f32_to_f16_bits(o.x) | ((uint32_t)f32_to_f16_bits(o.y) << 16);
+        reinterpret_cast<uint32_t*>(kc + (size_t)pos * kv_heads * hd)[pk] = packed;
+    } else if (p < qp + 2 * kp) {
+        const uint32_t pv = p - qp - kp;
+        float2 x = reinterpret_cast<const float2*>(v + (size_t)r * kv_stride)[pv];
+        uint32_t packed = (uint32_t)f32_to_f16_bits(x.x) | ((uint32_t)f32_to_f16_bits(x.y) << 16);
+        reinterpret_cast<uint32_t*>(vc + (size_t)pos * kv_heads * hd)[pv] = packed;
+    }
+}
+
+void launch_rope_kv_store(float* q, float* k, const float* v, uint32_t q_stride, uint32_t kv_stride, uint16_t* kc,
+                          uint16_t* vc, uint32_t M, uint32_t base_pos, const uint32_t* pos_dev, uint32_t heads,
+                          uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, hipStream_t s) {
+    if (M == 0) return;
+    uint32_t per_row = (heads + 2 * kv_heads) * hd / 2;
+    dim3 grid((per_row + 255) / 256, M);
+    rope_kv_store_kernel<<<grid, 256, 0, s>>>(q, k, v, q_stride, kv_stride, kc, vc, base_pos, pos_dev, heads, kv_heads,
+                                              hd, cos_t, sin_t);
+}
+
+// ---- embedding (emit.rs:585-589) -----------------------------------------------------------------
+__global__ __launch_bounds__(256) void embedding_kernel(const float* __restrict__ table,
+                                                        const uint32_t* __restrict__ tokens, uint32_t H4,
+                                                        float* __restrict__ out) {
+    const uint32_t r = blockIdx.y;
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= H4) return;
+    const uint32_t tok = tokens[r];
+    reinterpret_cast<float4*>(out)[(size_t)r * H4 + i] = reinterpret_cast<const float4*>(table)[(size_t)tok * H4 + i];
+}
+
+void launch_embedding(const float* table, const uint32_t* tokens_dev, uint32_t M, uint32_t H, float* out,
+                      hipStream_t s) {
+    if (M == 0) return;
+    dim3 grid((H / 4 + 255) / 256, M);
+    embedding_kernel<<<grid, 256, 0, s>>>(table, tokens_dev, H / 4, out);
+}
+
+// ---- argmax (project.rs:501-503): the LAST index among equal maxima ------------------------------------
+struct ArgPair { float v; uint32_t i; };
+__device__ __forceinline__ ArgPair arg_better(ArgPair a, ArgPair b) {
+    // keep the larger value; on equality the larger index
+    bool take_b = (b.v > a.v) || (b.v == a.v && b.i > a.i);
+    return take_b ? b : a;
+}
+__device__ __forceinline__ ArgPair arg_wave(ArgPair a) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        ArgPair b;
+        b.v = __shfl_xor(a.v, o, WAVE);
+        b.i = __shfl_xor(a.i, o, WAVE);
+        a = arg_better(a, b);
+    }
+    return a;
+}
+__device__ __forceinline__ ArgPair arg_block(ArgPair a, ArgPair* sh) {
+    a = arg_wave(a);
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = a;
+    __syncthreads();
+    ArgPair r = sh[0];
+    for (int w = 1; w < 4; w++) r = arg_better(r, sh[w]);
+    return r;
+}
+
+__global__ __launch_bounds__(256) void argmax_stage1(const float* __restrict__ x, uint32_t n, ArgPair* __restrict__ part) {
+    __shared__ ArgPair sh[4];
+    ArgPair a{-INFINITY, 0};
+    bool any = false;
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
+        ArgPair b{x[i], i};
+        a = any ? arg_better(a, b) : b;
+        any = true;
+    }
+    a = arg_block(a, sh);
+    if (threadIdx.x == 0) part[blockIdx.x] = a;
+}
+__global__ __launch_bounds__(256) void argmax_stage2(const ArgPair* __restrict__ part, uint32_t nparts,
+                                                     uint32_t* __restrict__ out) {
+    __shared__ ArgPair sh[4];
+    ArgPair a{-INFINITY, 0};
+    if (threadIdx.x < nparts) a = part[threadIdx.x];
+    a = arg_block(a, sh);
+    if (threadIdx.x == 0) *out = a.i;
+}
+
+void launch_argmax(const float* x, uint32_t n, uint32_t* out, void* scratch, hipStream_t s) {
+    uint32_t blocks = (n + 255) / 256;
+    if (blocks > ARGMAX_BLOCKS) blocks = ARGMAX_BLOCKS;
+    if (blocks == 0) blocks = 1;
+    argmax_stage1<<<blocks, 256, 0, s>>>(x, n, reinterpret_cast<ArgPair*>(scratch));
+    argmax_stage2<<<1, 256, 0, s>>>(reinterpret_cast<const ArgPair*>(scratch), blocks, out);
+}
+
+// pos += 1 and, if `next` is given, token = *next (greedy feedback without a host round trip).
+__global__ void advance_kernel(uint32_t* pos, uint32_t* token, const uint32_t* next) {
+    if (threadIdx.x == 0) {
+        *pos = *pos + 1;
+        if (token && next) *token = *next;
+    }
+}
+void launch_advance(uint32_t* pos_dev, uint32_t* token_dev, const uint32_t* next_dev, hipStream_t s) {
+    advance_kernel<<<1, 64, 0, s>>>(pos_dev, token_dev, next_dev);
+}
+
+}  // namespace fh

@@ -1,0 +1,372 @@
+// extern "C" surface, part 2: the model object (MetalModel::{new, forward,
+// forward_prefill_batch, reset}, metal:4209-5981; model::{forward, forward_prefill_batched},
+// emit.rs:4029-5486) on one GPU.
+//
+// HBM layout: f32 embedding table; per layer two norm vectors and four quantised matrices
+// as planes (q|k|v rows fused into one matrix, gate|up rows fused into one — the blob stores
+// them back to back for exactly this, crates/forgellm-cli/src/main.rs:2722-2736); fp16 KV cache
+// [layer][max_seq][kv_heads*head_dim] for K and V; cos/sin tables [max_seq][head_dim/2];
+// f32 scratch for one decode step and for one prefill chunk.
+//
+// The decode step is captured once into a HIP graph (position and token live in device
+// memory so the graph never changes) and replayed per token.
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <memory>
+#include <vector>
+
+#include "common.h"
+
+namespace fh {
+
+constexpr uint32_t PREFILL_CHUNK = 4096;   // rows of scratch for batched prefill
+
+struct Layer {
+    float* attn_norm = nullptr;
+    float* ffn_norm = nullptr;
+    QWeight qkv, o, gate_up, down;
+};
+
+struct DevBuf {
+    void* p = nullptr;
+    DevBuf() = default;
+    DevBuf(const DevBuf&) = delete;
+    DevBuf& operator=(const DevBuf&) = delete;
+    ~DevBuf() { if (p) (void)hipFree(p); }
+    int32_t alloc(size_t n) {
+        FH_HIP(hipMalloc(&p, n < 16 ? 16 : n));
+        return FORGE_HIP_OK;
+    }
+    template <typename T> T* as() const { return reinterpret_cast<T*>(p); }
+};
+
+}  // namespace fh
+
+using namespace fh;
+
+struct forge_hip_model {
+    forge_hip_config cfg{};
+    uint32_t H = 0, I = 0, QKS = 0, KV = 0, QKV = 0, KMAX = 0;
+    hipStream_t stream = nullptr;
+    DevBuf embed, final_norm, norms;     // norms: [layers][2][H]
+    std::vector<Layer> layers;
+    QWeight lm_head;
+    DevBuf kcache, vcache;               // fp16 [layers][max_seq][KV]
+    DevBuf cos_t, sin_t;
+    // decode scratch
+    DevBuf x, qkv, gu, logits, aq, asc, attn_ws, state, argmax_ws;
+    // prefill scratch (chunk_rows rows)
+    DevBuf px, pqkv, pattn, pgu, paq, pasc, ptok;
+    uint32_t chunk_rows = 0;
+    // pinned host staging: [0] token, [1] next token, [2] position
+    uint32_t* h_stage = nullptr;
+    int64_t pos = 0;
+    bool use_graph = true;
+    hipGraphExec_t decode_graph = nullptr;
+
+    uint32_t* d_pos() const { return state.as<uint32_t>(); }
+    uint32_t* d_token() const { return state.as<uint32_t>() + 1; }
+    uint32_t* d_next() const { return state.as<uint32_t>() + 2; }
+    uint16_t* kc(uint32_t l) const { return kcache.as<uint16_t>() + (size_t)l * cfg.max_seq * KV; }
+    uint16_t* vc(uint32_t l) const { return vcache.as<uint16_t>() + (size_t)l * cfg.max_seq * KV; }
+
+    ~forge_hip_model() {
+        if (decode_graph) (void)hipGraphExecDestroy(decode_graph);
+        for (auto& L : layers) { qweight_free(&L.qkv); qweight_free(&L.o); qweight_free(&L.gate_up); qweight_free(&L.down); }
+        qweight_free(&lm_head);
+        if (h_stage) (void)hipHostFree(h_stage);
+        if (stream) (void)hipStreamDestroy(stream);
+    }
+};
+
+namespace {
+
+size_t wsize(uint32_t dtype, uint64_t n, uint64_t k) { return (size_t)(n * (k / 32) * (dtype == FORGE_HIP_Q8_0 ? 34 : 18)); }
+
+int32_t validate(const forge_hip_config* c) {
+    FH_CHECK(c, "config is null");
+    FH_CHECK(c->wdtype == FORGE_HIP_Q8_0 || c->wdtype == FORGE_HIP_Q4_0, "wdtype must be Q8_0 (8) or Q4_0 (2)");
+    FH_CHECK(c->lm_head_dtype == FORGE_HIP_Q8_0 || c->lm_head_dtype == FORGE_HIP_Q4_0, "lm_head_dtype must be Q8_0 (8) or Q4_0 (2)");
+    FH_CHECK(c->hidden >= 32 && c->hidden % 32 == 0, "hidden must be a positive multiple of 32");
+    FH_CHECK(c->inter >= 32 && c->inter % 32 == 0, "inter must be a positive multiple of 32");
+    FH_CHECK(c->layers >= 1 && c->vocab >= 1 && c->max_seq >= 1, "layers, vocab and max_seq must be positive");
+    FH_CHECK(c->heads >= 1 && c->kv_heads >= 1 && c->heads % c->kv_heads == 0, "heads must be a positive multiple of kv_heads");
+    FH_CHECK(attn_head_dim_supported(c->head_dim), "head_dim must be 64, 96 or 128");
+    FH_CHECK(gemv_k_supported(c->hidden) && gemv_k_supported(c->inter) && gemv_k_supported(c->heads * c->head_dim),
+             "hidden, inter and heads*head_dim must be at most 16384");
+    return FORGE_HIP_OK;
+}
+
+// Enqueue one decoder layer on the model's stream.  decode: one row, position read from
+// device memory.  prefill: M rows at positions base_pos.. .
+void enqueue_layer(forge_hip_model* m, uint32_t l, bool decode, uint32_t M, uint32_t base_pos) {
+    const forge_hip_config& c = m->cfg;
+    Layer& L = m->layers[l];
+    hipStream_t s = m->stream;
+    const uint32_t H = m->H, I = m->I, QKS = m->QKS, KV = m->KV, QKV = m->QKV;
+    float* x = decode ? m->x.as<float>() : m->px.as<float>();
+    float* qkv = decode ? m->qkv.as<float>() : m->pqkv.as<float>();
+    float* gu = decode ? m->gu.as<float>() : m->pgu.as<float>();
+    int8_t* aq = decode ? m->aq.as<int8_t>() : m->paq.as<int8_t>();
+    uint16_t* asc = decode ? m->asc.as<uint16_t>() : m->pasc.as<uint16_t>();
+
+    launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s);
+    if (decode) launch_gemv(L.qkv, aq, asc, qkv, false, s);
+    else launch_gemm(L.qkv, aq, asc, M, qkv, QKV, false, nullptr, s);
+    launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos,
+                         decode ? m->d_pos() : nullptr, c.heads, c.kv_heads, c.head_dim, m->cos_t.as<float>(),
+                         m->sin_t.as<float>(), s);
+    if (decode) {
+        launch_attn_decode(qkv, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads, c.head_dim,
+                           m->attn_ws.p, s);
+        launch_gemv(L.o, aq, asc, x, true, s);
+    } else {
+        float* attn = m->pattn.as<float>();
+        launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, s);
+        launch_quantize_act(attn, M, QKS, aq, asc, s);
+        launch_gemm(L.o, aq, asc, M, x, H, true, nullptr, s);
+    }
+    launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s);
+    if (decode) launch_gemv(L.gate_up, aq, asc, gu, false, s);
+    else launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, nullptr, s);
+    launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s);
+    if (decode) launch_gemv(L.down, aq, asc, x, true, s);
+    else launch_gemm(L.down, aq, asc, M, x, H, true, nullptr, s);
+}
+
+// Final norm of one row + lm_head GEMV + argmax.
+void enqueue_head(forge_hip_model* m, const float* xrow) {
+    hipStream_t s = m->stream;
+    launch_rmsnorm(xrow, m->final_norm.as<float>(), m->cfg.rms_eps, 1, m->H, nullptr, m->aq.as<int8_t>(),
+                   m->asc.as<uint16_t>(), s);
+    launch_gemv(m->lm_head, m->aq.as<int8_t>(), m->asc.as<uint16_t>(), m->logits.as<float>(), false, s);
+    launch_argmax(m->logits.as<float>(), m->cfg.vocab, m->d_next(), m->argmax_ws.p, s);
+}
+
+void enqueue_decode_step(forge_hip_model* m) {
+    launch_embedding(m->embed.as<float>(), m->d_token(), 1, m->H, m->x.as<float>(), m->stream);
+    for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_layer(m, l, true, 1, 0);
+    enqueue_head(m, m->x.as<float>());
+    launch_advance(m->d_pos(), m->d_token(), m->d_next(), m->stream);
+}
+
+int32_t run_decode_step(forge_hip_model* m) {
+    if (m->use_graph && !m->decode_graph) {
+        hipGraph_t g = nullptr;
+        FH_HIP(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
+        enqueue_decode_step(m);
+        hipError_t e = hipStreamEndCapture(m->stream, &g);
+        if (e != hipSuccess || !g) return fail(FORGE_HIP_ERR_HIP, std::string("graph capture failed: ") + hipGetErrorString(e));
+        e = hipGraphInstantiate(&m->decode_graph, g, nullptr, nullptr, 0);
+        (void)hipGraphDestroy(g);
+        if (e != hipSuccess) { m->decode_graph = nullptr; return fail(FORGE_HIP_ERR_HIP, std::string("graph instantiate failed: ") + hipGetErrorString(e)); }
+    }
+    if (m->decode_graph) FH_HIP(hipGraphLaunch(m->decode_graph, m->stream));
+    else { enqueue_decode_step(m); FH_HIP(hipGetLastError()); }
+    return FORGE_HIP_OK;
+}
+
+int32_t forward_common(forge_hip_model* m, uint32_t token) {
+    FH_CHECK(m, "model is null");
+    if (m->pos >= (int64_t)m->cfg.max_seq) return fail(FORGE_HIP_ERR_POSITION, "KV cache is full (pos == max_seq)");
+    if (token >= m->cfg.vocab) return fail(FORGE_HIP_ERR_POSITION, "token id out of range");
+    m->h_stage[0] = token;
+    FH_HIP(hipMemcpyAsync(m->d_token(), &m->h_stage[0], 4, hipMemcpyHostToDevice, m->stream));
+    int32_t rc = run_decode_step(m);
+    if (rc) return rc;
+    m->pos += 1;
+    return FORGE_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+uint64_t forge_hip_weights_nbytes(const forge_hip_config* c) {
+    if (!c) return 0;
+    const uint64_t H = c->hidden, I = c->inter, QKS = (uint64_t)c->heads * c->head_dim, KV = (uint64_t)c->kv_heads * c->head_dim;
+    const uint64_t per_layer = H * 4 + wsize(c->wdtype, QKS, H) + 2 * wsize(c->wdtype, KV, H) + wsize(c->wdtype, H, QKS) +
+                               H * 4 + 2 * wsize(c->wdtype, I, H) + wsize(c->wdtype, H, I);
+    return (uint64_t)c->vocab * H * 4 + c->layers * per_layer + H * 4 + wsize(c->lm_head_dtype, c->vocab, H);
+}
+
+int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob, uint64_t nbytes, forge_hip_model** out) {
+    FH_CHECK(out, "model_create: null out");
+    *out = nullptr;
+    int32_t rc = validate(cfg);
+    if (rc) return rc;
+    FH_CHECK(blob, "model_create: null weights");
+    if (nbytes != forge_hip_weights_nbytes(cfg))
+        return fail(FORGE_HIP_ERR_BLOB_SIZE, "weights blob is " + std::to_string(nbytes) + " bytes, config needs " +
+                                                 std::to_string(forge_hip_weights_nbytes(cfg)));
+    if (forge_hip_device_count() < 1) return fail(FORGE_HIP_ERR_NO_DEVICE, "no HIP device");
+
+    std::unique_ptr<forge_hip_model> m(new forge_hip_model());
+    m->cfg = *cfg;
+    const uint32_t H = m->H = cfg->hidden, I = m->I = cfg->inter;
+    const uint32_t QKS = m->QKS = cfg->heads * cfg->head_dim, KV = m->KV = cfg->kv_heads * cfg->head_dim;
+    m->QKV = QKS + 2 * KV;
+    m->KMAX = std::max(std::max(H, I), QKS);
+    const char* genv = getenv("FORGE_HIP_GRAPH");
+    m->use_graph = !(genv && genv[0] == '0');
+    FH_HIP(hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking));
+    FH_HIP(hipHostMalloc((void**)&m->h_stage, 64, hipHostMallocDefault));
+
+    // ---- weights (blob order: project.rs:342-407) ----
+    const uint8_t* p = blob;
+    rc = m->embed.alloc((size_t)cfg->vocab * H * 4);
+    if (rc) return rc;
+    FH_HIP(hipMemcpy(m->embed.p, p, (size_t)cfg->vocab * H * 4, hipMemcpyHostToDevice));
+    p += (size_t)cfg->vocab * H * 4;
+    rc = m->norms.alloc((size_t)cfg->layers * 2 * H * 4);
+    if (rc) return rc;
+    m->layers.resize(cfg->layers);
+    const uint32_t wt = cfg->wdtype;
+    for (uint32_t l = 0; l < cfg->layers; l++) {
+        Layer& L = m->layers[l];
+        L.attn_norm = m->norms.as<float>() + (size_t)(2 * l) * H;
+        L.ffn_norm = L.attn_norm + H;
+        FH_HIP(hipMemcpy(L.attn_norm, p, H * 4, hipMemcpyHostToDevice));
+        p += H * 4;
+        // q, k, v are adjacent in the blob and all have K = hidden: upload as one matrix.
+        rc = qweight_upload(wt, p, H, m->QKV, &L.qkv);
+        if (rc) return rc;
+        p += wsize(wt, m->QKV, H);
+        rc = qweight_upload(wt, p, QKS, H, &L.o);
+        if (rc) return rc;
+        p += wsize(wt, H, QKS);
+        FH_HIP(hipMemcpy(L.ffn_norm, p, H * 4, hipMemcpyHostToDevice));
+        p += H * 4;
+        rc = qweight_upload(wt, p, H, 2 * I, &L.gate_up);   // gate rows then up rows, adjacent in the blob
+        if (rc) return rc;
+        p += wsize(wt, 2 * (uint64_t)I, H);
+        rc = qweight_upload(wt, p, I, H, &L.down);
+        if (rc) return rc;
+        p += wsize(wt, H, I);
+    }
+    rc = m->final_norm.alloc(H * 4);
+    if (rc) return rc;
+    FH_HIP(hipMemcpy(m->final_norm.p, p, H * 4, hipMemcpyHostToDevice));
+    p += H * 4;
+    rc = qweight_upload(cfg->lm_head_dtype, p, H, cfg->vocab, &m->lm_head);
+    if (rc) return rc;
+
+    // ---- KV cache, rope tables ----
+    const size_t cache_bytes = (size_t)cfg->layers * cfg->max_seq * KV * 2;
+    if ((rc = m->kcache.alloc(cache_bytes)) || (rc = m->vcache.alloc(cache_bytes))) return rc;
+    {
+        const uint32_t half = cfg->head_dim / 2;
+        std::vector<float> ct((size_t)cfg->max_seq * half), st((size_t)cfg->max_seq * half);
+        for (uint32_t i = 0; i < half; i++) {
+            // rope_freqs, emit.rs:501-504; angle and sin_cos, emit.rs:514-516 — host C library
+            const float f = 1.0f / powf(cfg->rope_theta, 2.0f * (float)i / (float)cfg->head_dim);
+            for (uint32_t t = 0; t < cfg->max_seq; t++) {
+                const float a = (float)t * f;
+                ct[(size_t)t * half + i] = cosf(a);
+                st[(size_t)t * half + i] = sinf(a);
+            }
+        }
+        if ((rc = m->cos_t.alloc(ct.size() * 4)) || (rc = m->sin_t.alloc(st.size() * 4))) return rc;
+        FH_HIP(hipMemcpy(m->cos_t.p, ct.data(), ct.size() * 4, hipMemcpyHostToDevice));
+        FH_HIP(hipMemcpy(m->sin_t.p, st.data(), st.size() * 4, hipMemcpyHostToDevice));
+    }
+
+    // ---- scratch ----
+    if ((rc = m->x.alloc(H * 4)) || (rc = m->qkv.alloc(m->QKV * 4)) || (rc = m->gu.alloc(2 * (size_t)I * 4)) ||
+        (rc = m->logits.alloc((size_t)cfg->vocab * 4)) || (rc = m->aq.alloc(m->KMAX)) ||
+        (rc = m->asc.alloc(m->KMAX / 32 * 2)) || (rc = m->attn_ws.alloc(attn_decode_workspace_bytes(cfg->heads, cfg->head_dim))) ||
+        (rc = m->state.alloc(64)) || (rc = m->argmax_ws.alloc(ARGMAX_BLOCKS * 8)))
+        return rc;
+    FH_HIP(hipMemset(m->state.p, 0, 64));
+    const uint32_t R = m->chunk_rows = std::min(PREFILL_CHUNK, cfg->max_seq);
+    if ((rc = m->px.alloc((size_t)R * H * 4)) || (rc = m->pqkv.alloc((size_t)R * m->QKV * 4)) ||
+        (rc = m->pattn.alloc((size_t)R * QKS * 4)) || (rc = m->pgu.alloc((size_t)R * 2 * I * 4)) ||
+        (rc = m->paq.alloc((size_t)R * m->KMAX)) || (rc = m->pasc.alloc((size_t)R * (m->KMAX / 32) * 2)) ||
+        (rc = m->ptok.alloc((size_t)R * 4)))
+        return rc;
+    FH_HIP(hipDeviceSynchronize());
+    *out = m.release();
+    return FORGE_HIP_OK;
+}
+
+void forge_hip_model_destroy(forge_hip_model* m) {
+    if (!m) return;
+    if (m->stream) (void)hipStreamSynchronize(m->stream);
+    delete m;
+}
+
+int32_t forge_hip_forward(forge_hip_model* m, uint32_t token, float* logits_host) {
+    FH_CHECK(logits_host, "forward: null logits");
+    int32_t rc = forward_common(m, token);
+    if (rc) return rc;
+    FH_HIP(hipMemcpyAsync(logits_host, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, m->stream));
+    FH_HIP(hipStreamSynchronize(m->stream));
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_forward_greedy(forge_hip_model* m, uint32_t token, uint32_t* next_token_host) {
+    FH_CHECK(next_token_host, "forward_greedy: null out");
+    int32_t rc = forward_common(m, token);
+    if (rc) return rc;
+    FH_HIP(hipMemcpyAsync(&m->h_stage[1], m->d_next(), 4, hipMemcpyDeviceToHost, m->stream));
+    FH_HIP(hipStreamSynchronize(m->stream));
+    *next_token_host = m->h_stage[1];
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint64_t n, float* logits_host) {
+    FH_CHECK(m && tokens, "prefill_batch: null pointer");
+    FH_CHECK(n >= 1, "prefill_batch: empty token list");
+    if ((uint64_t)m->pos + n > m->cfg.max_seq)
+        return fail(FORGE_HIP_ERR_POSITION, "prompt does not fit the KV cache (pos + n > max_seq)");
+    for (uint64_t i = 0; i < n; i++)
+        if (tokens[i] >= m->cfg.vocab) return fail(FORGE_HIP_ERR_POSITION, "token id out of range");
+    hipStream_t s = m->stream;
+    uint64_t done = 0;
+    uint32_t last_rows = 0;
+    while (done < n) {
+        const uint32_t rows = (uint32_t)std::min<uint64_t>(m->chunk_rows, n - done);
+        // pageable source: the copy is complete (staged) when the call returns
+        FH_HIP(hipMemcpyAsync(m->ptok.p, tokens + done, (size_t)rows * 4, hipMemcpyHostToDevice, s));
+        launch_embedding(m->embed.as<float>(), m->ptok.as<uint32_t>(), rows, m->H, m->px.as<float>(), s);
+        for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_layer(m, l, false, rows, (uint32_t)(m->pos + done));
+        FH_HIP(hipGetLastError());
+        done += rows;
+        last_rows = rows;
+    }
+    m->pos += (int64_t)n;
+    m->h_stage[2] = (uint32_t)m->pos;
+    FH_HIP(hipMemcpyAsync(m->d_pos(), &m->h_stage[2], 4, hipMemcpyHostToDevice, s));
+    if (logits_host) {
+        enqueue_head(m, m->px.as<float>() + (size_t)(last_rows - 1) * m->H);
+        FH_HIP(hipGetLastError());
+        FH_HIP(hipMemcpyAsync(logits_host, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, s));
+    }
+    FH_HIP(hipStreamSynchronize(s));
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_reset(forge_hip_model* m) {
+    FH_CHECK(m, "reset: model is null");
+    m->pos = 0;
+    m->h_stage[2] = 0;
+    FH_HIP(hipMemcpyAsync(m->d_pos(), &m->h_stage[2], 4, hipMemcpyHostToDevice, m->stream));
+    FH_HIP(hipStreamSynchronize(m->stream));
+    return FORGE_HIP_OK;
+}
+
+int64_t forge_hip_model_pos(const forge_hip_model* m) { return m ? m->pos : -1; }
+
+int32_t forge_hip_model_read_kv(forge_hip_model* m, uint32_t layer, uint32_t which, uint16_t* out_host) {
+    FH_CHECK(m && out_host, "read_kv: null pointer");
+    FH_CHECK(layer < m->cfg.layers && which <= 1, "read_kv: layer or selector out of range");
+    FH_HIP(hipStreamSynchronize(m->stream));
+    const uint16_t* src = which == 0 ? m->kc(layer) : m->vc(layer);
+    if (m->pos > 0) FH_HIP(hipMemcpy(out_host, src, (size_t)m->pos * m->KV * 2, hipMemcpyDeviceToHost));
+    return FORGE_HIP_OK;
+}
+
+}  // extern "C"

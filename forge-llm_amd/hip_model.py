@@ -1,0 +1,97 @@
+"""HipModel — host-side mirror of the reference's GPU model object.
+
+Same surface as `MetalModel` in the reference (crates/forgellm-codegen-metal/src/lib.rs:
+`new(weights: &[u8])` :4209, `forward(token_id) -> Vec<f32>` :5070,
+`forward_prefill_batch(tokens)` :5568, `reset()` :5981), plus the CPU backend's
+`forward_prefill` signature that returns the last token's logits
+(crates/forgellm-codegen-cpu/src/emit.rs:4553).  Errors that panic in the reference raise
+ForgeHipError here.
+"""
+import ctypes as C
+
+import numpy as np
+
+
+class HipModel:
+    def __init__(self, config: dict, weights):
+        """config: dict with the forge_hip_config fields; weights: the weights.bin bytes
+        (numpy uint8 array, bytes or memoryview).  The blob is copied to the GPU."""
+        from . import Config, check, lib
+        self._lib = lib()
+        self._check = check
+        self.config = dict(config)
+        self._cfg = Config(**config)
+        w = np.frombuffer(weights, dtype=np.uint8) if not isinstance(weights, np.ndarray) else weights
+        w = np.ascontiguousarray(w, dtype=np.uint8)
+        h = C.c_void_p()
+        check(self._lib.forge_hip_model_create(C.byref(self._cfg), w.ctypes.data_as(C.c_void_p), w.size, C.byref(h)))
+        self._h = h
+        self.vocab = int(config["vocab"])
+
+    # -- MetalModel::forward / model::forward
+    def forward(self, token_id: int) -> np.ndarray:
+        out = np.empty(self.vocab, np.float32)
+        self._check(self._lib.forge_hip_forward(self._h, int(token_id), out.ctypes.data_as(C.c_void_p)))
+        return out
+
+    def forward_greedy(self, token_id: int) -> int:
+        """forward + argmax (last index among ties) on the device."""
+        nxt = C.c_uint32()
+        self._check(self._lib.forge_hip_forward_greedy(self._h, int(token_id), C.byref(nxt)))
+        return int(nxt.value)
+
+    # -- MetalModel::forward_prefill_batch: fills the cache, no logits
+    def forward_prefill_batch(self, tokens) -> None:
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        self._check(self._lib.forge_hip_prefill_batch(self._h, t.ctypes.data_as(C.c_void_p), t.size, None))
+
+    # -- model::forward_prefill: returns the last token's logits
+    def forward_prefill(self, tokens) -> np.ndarray:
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        out = np.empty(self.vocab, np.float32)
+        self._check(self._lib.forge_hip_prefill_batch(self._h, t.ctypes.data_as(C.c_void_p), t.size,
+                                                      out.ctypes.data_as(C.c_void_p)))
+        return out
+
+    def reset(self) -> None:
+        self._check(self._lib.forge_hip_reset(self._h))
+
+    @property
+    def pos(self) -> int:
+        return int(self._lib.forge_hip_model_pos(self._h))
+
+    def read_kv(self, layer: int, which: int) -> np.ndarray:
+        """Cached K (which=0) or V (1) rows [0, pos) of a layer as fp16 bit patterns."""
+        kv = self.config["kv_heads"] * self.config["head_dim"]
+        out = np.empty((self.pos, kv), np.uint16)
+        self._check(self._lib.forge_hip_model_read_kv(self._h, layer, which, out.ctypes.data_as(C.c_void_p)))
+        return out
+
+    def generate_greedy(self, prompt, n_tokens: int):
+        """The reference's greedy loop (crates/forgellm-codegen-cpu/src/project.rs:714-751 with
+        temperature 0 and repeat penalty 1.0): prefill, argmax, then feed tokens back."""
+        from .ops import argmax_host
+        logits = self.forward_prefill(prompt)
+        nxt = argmax_host(logits)
+        out = [nxt]
+        for _ in range(n_tokens - 1):
+            nxt = self.forward_greedy(nxt)
+            out.append(nxt)
+        return out
+
+    def close(self):
+        if getattr(self, "_h", None):
+            self._lib.forge_hip_model_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def weights_nbytes(config: dict) -> int:
+    from . import Config, lib
+    c = Config(**config)
+    return int(lib().forge_hip_weights_nbytes(C.byref(c)))

@@ -1,0 +1,147 @@
+"""Seeded synthetic tensors and models in the reference's on-disk formats.
+
+There are no checkpoints offline, so every workload is random-init from a seed:
+splitmix64 (counter based, so any slice can be generated independently) -> uniform ->
+Box-Muller normals in f32.  Models are written as the headerless `weights.bin` that
+`forge export-weights` produces (crates/forgellm-cli/src/main.rs:2714-2757; read back by
+crates/forgellm-codegen-cpu/src/project.rs:342-407):
+
+    embed_tokens f32 [vocab][hidden]
+    per layer: attn_norm f32 | q | k | v | o raw blocks | ffn_norm f32 | gate | up | down raw blocks
+    final_norm f32 | lm_head raw blocks
+
+With tied embeddings the lm_head bytes are the quantised embedding and the f32 table is its
+dequantisation (main.rs:2631-2693).
+"""
+from concurrent.futures import ThreadPoolExecutor
+
+import numpy as np
+
+_M64 = np.uint64(0xFFFFFFFFFFFFFFFF)
+_CHUNK = 1 << 22
+
+
+def splitmix64(seed: int, start: int, n: int) -> np.ndarray:
+    """n outputs of splitmix64 seeded with `seed`, beginning at draw index `start`."""
+    with np.errstate(over="ignore"):
+        idx = np.arange(start + 1, start + n + 1, dtype=np.uint64)
+        z = np.uint64(seed & 0xFFFFFFFFFFFFFFFF) + idx * np.uint64(0x9E3779B97F4A7C15)
+        z = (z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)
+        z = (z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)
+        return z ^ (z >> np.uint64(31))
+
+
+def _normal_chunk(seed, start_pair, npairs, std):
+    z = splitmix64(seed, 2 * start_pair, 2 * npairs)
+    u1 = ((z[0::2] >> np.uint64(11)).astype(np.float64) + 1.0) * (1.0 / 9007199254740992.0)   # (0, 1]
+    u2 = (z[1::2] >> np.uint64(11)).astype(np.float64) * (1.0 / 9007199254740992.0)           # [0, 1)
+    r = np.sqrt(-2.0 * np.log(u1)) * std
+    ang = (2.0 * np.pi) * u2
+    out = np.empty(2 * npairs, np.float32)
+    out[0::2] = r * np.cos(ang)
+    out[1::2] = r * np.sin(ang)
+    return out
+
+
+def normal(seed: int, n: int, std: float = 1.0, threads: int = 8) -> np.ndarray:
+    """n f32 normals N(0, std^2), reproducible from (seed, n) alone."""
+    npairs = (n + 1) // 2
+    starts = list(range(0, npairs, _CHUNK))
+    if len(starts) <= 1 or threads <= 1:
+        parts = [_normal_chunk(seed, s, min(_CHUNK, npairs - s), std) for s in starts]
+    else:
+        with ThreadPoolExecutor(max_workers=threads) as ex:
+            parts = list(ex.map(lambda s: _normal_chunk(seed, s, min(_CHUNK, npairs - s), std), starts))
+    out = parts[0] if len(parts) == 1 else np.concatenate(parts)
+    return out[:n]
+
+
+def uniform_ids(seed: int, n: int, vocab: int) -> np.ndarray:
+    """n token ids uniform in [0, vocab)."""
+    return (splitmix64(seed, 0, n) % np.uint64(vocab)).astype(np.uint32)
+
+
+# ---- model shapes named in the benchmark configurations ----
+def _cfg(hidden, inter, layers, heads, kv_heads, head_dim, vocab, max_seq, theta, wdtype):
+    return dict(hidden=hidden, inter=inter, layers=layers, heads=heads, kv_heads=kv_heads, head_dim=head_dim,
+                vocab=vocab, max_seq=max_seq, rms_eps=1e-5, rope_theta=theta, wdtype=wdtype, lm_head_dtype=wdtype,
+                flags=0)
+
+
+def smollm2_135m(wdtype=8, max_seq=4096):
+    return _cfg(576, 1536, 30, 9, 3, 64, 49152, max_seq, 100000.0, wdtype)
+
+
+def llama32_1b(wdtype=8, max_seq=4096):
+    return _cfg(2048, 8192, 16, 32, 8, 64, 128256, max_seq, 500000.0, wdtype)
+
+
+def llama32_3b(wdtype=8, max_seq=4096):
+    return _cfg(3072, 8192, 28, 24, 8, 128, 128256, max_seq, 500000.0, wdtype)
+
+
+def tiny(wdtype=8, max_seq=640, hidden=256, inter=512, layers=2, heads=4, kv_heads=2, head_dim=64, vocab=1000):
+    return _cfg(hidden, inter, layers, heads, kv_heads, head_dim, vocab, max_seq, 10000.0, wdtype)
+
+
+def make_weights_blob(cfg: dict, seed: int, std: float = 0.02, norm_jitter: float = 0.1, threads: int = 8) -> np.ndarray:
+    """Random-init model as weights.bin bytes (tied embeddings).  Projection weights are f32
+    N(0, std^2) quantised with the reference's quantisers; norm weights are 1 + norm_jitter*N(0,1)."""
+    from .ops import block_bytes, dequant, quantize_weights
+    H, I = cfg["hidden"], cfg["inter"]
+    QKS, KV = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"]
+    wt, lt = cfg["wdtype"], cfg["lm_head_dtype"]
+    counter = [0]
+
+    def sub_seed():
+        counter[0] += 1
+        return (seed * 1000003 + counter[0] * 7919) & 0xFFFFFFFFFFFFFFFF
+
+    def qmat(n, k, dtype):
+        return quantize_weights(dtype, normal(sub_seed(), n * k, std, threads))
+
+    def norm_vec():
+        return (1.0 + norm_jitter * normal(sub_seed(), H, 1.0, 1)).astype(np.float32)
+
+    parts = []
+    lm_raw = qmat(cfg["vocab"], H, lt)
+    embed = dequant(lt, lm_raw, cfg["vocab"] * H)
+    parts.append(embed.view(np.uint8))
+    for _ in range(cfg["layers"]):
+        parts.append(norm_vec().view(np.uint8))
+        parts.append(qmat(QKS, H, wt))
+        parts.append(qmat(KV, H, wt))
+        parts.append(qmat(KV, H, wt))
+        parts.append(qmat(H, QKS, wt))
+        parts.append(norm_vec().view(np.uint8))
+        parts.append(qmat(I, H, wt))
+        parts.append(qmat(I, H, wt))
+        parts.append(qmat(H, I, wt))
+    parts.append(norm_vec().view(np.uint8))
+    parts.append(lm_raw)
+    blob = np.concatenate(parts)
+    expect = (cfg["vocab"] * H * 4 + cfg["layers"] * (2 * H * 4 + (QKS * H + 2 * KV * H + H * QKS + 3 * I * H) // 32 * block_bytes(wt))
+              + H * 4 + cfg["vocab"] * H // 32 * block_bytes(lt))
+    assert blob.size == expect, (blob.size, expect)
+    return blob
+
+
+def gemv_bytes(n: int, k: int, wdtype: int) -> int:
+    """Algorithmic bytes of one quantised GEMV: the GGUF blocks of the matrix (34 or 18 bytes
+    per 32 weights) plus the f32 input and output vectors."""
+    from .ops import block_bytes
+    return n * (k // 32) * block_bytes(wdtype) + 4 * k + 4 * n
+
+
+def decode_weight_bytes(cfg: dict) -> int:
+    """Bytes of quantised weights (34- or 18-byte GGUF blocks) one decode step streams."""
+    from .ops import block_bytes
+    H, I = cfg["hidden"], cfg["inter"]
+    QKS, KV = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"]
+
+    def mat(n, k, dtype):
+        return n * (k // 32) * block_bytes(dtype)
+
+    wt = cfg["wdtype"]
+    per_layer = mat(QKS, H, wt) + 2 * mat(KV, H, wt) + mat(H, QKS, wt) + 2 * mat(I, H, wt) + mat(H, I, wt)
+    return cfg["layers"] * per_layer + mat(cfg["vocab"], H, cfg["lm_head_dtype"])

@@ -1,0 +1,161 @@
+/* libforge_hip — C ABI of the MI355X (gfx950) backend for ForgeLLM's quantized-Llama hot path.
+ *
+ * This is what a `forgellm-codegen-hip` crate's generated `model.rs` binds (extern "C"),
+ * in place of the Rust kernels that crates/forgellm-codegen-cpu/src/emit.rs ("emit.rs")
+ * generates and of the MSL kernels of crates/forgellm-codegen-metal/src/lib.rs ("metal").
+ * Every entry point names the reference interface it replaces.
+ *
+ * Conventions
+ *  - Every function returns a status: 0 = OK, negative = error class below.  The reference
+ *    panics on these conditions (metal:4212, project.rs:342-406); here they are codes plus a
+ *    thread-local message from forge_hip_last_error().
+ *  - "dev" pointers are device (HBM) addresses; "host" pointers are ordinary memory.
+ *  - `stream` is a hipStream_t passed as void*; NULL = the null stream.  Op-level calls are
+ *    asynchronous on that stream.  Model calls run on the model's own stream and return
+ *    after the results they hand back are complete.
+ *  - A model handle is NOT thread-safe (the reference API is `&mut self`, metal:5070).
+ *  - Arithmetic: activations are quantised per 32-element block to int8 exactly as
+ *    emit.rs:1410-1440, block dot products are exact int32 (emit.rs:1543-1553,
+ *    2522-2552), the per-block combine and everything else is f32.  KV cache is fp16.
+ */
+#ifndef FORGE_HIP_H
+#define FORGE_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FORGE_HIP_OK 0
+#define FORGE_HIP_ERR_INVALID (-1)   /* bad argument / unsupported shape */
+#define FORGE_HIP_ERR_BLOB_SIZE (-2) /* weights blob length does not match the config */
+#define FORGE_HIP_ERR_POSITION (-3)  /* cache full, or token id out of range */
+#define FORGE_HIP_ERR_NO_DEVICE (-4)
+#define FORGE_HIP_ERR_HIP (-5)       /* a HIP runtime call failed */
+
+#define FORGE_HIP_Q4_0 2u /* GGML type ids, crates/forgellm-frontend/src/gguf.rs:207-258 */
+#define FORGE_HIP_Q8_0 8u
+
+/* Mirrors the fields of ModelConfig (crates/forgellm-frontend/src/ir.rs:484-519) that the
+ * code generators read. */
+typedef struct forge_hip_config {
+    uint32_t hidden, inter, layers, heads, kv_heads, head_dim, vocab, max_seq;
+    float rms_eps, rope_theta;
+    uint32_t wdtype;        /* projection weights: FORGE_HIP_Q8_0 or FORGE_HIP_Q4_0 */
+    uint32_t lm_head_dtype; /* same coding */
+    uint32_t flags;         /* reserved, 0 */
+} forge_hip_config;
+
+typedef struct forge_hip_model forge_hip_model;
+typedef struct forge_hip_qweight forge_hip_qweight;
+
+const char* forge_hip_last_error(void);
+/* Number of visible GPUs; 0 when there is none. */
+int32_t forge_hip_device_count(void);
+
+/* ---------------- model API (replaces MetalModel, metal:4209-5981, and
+ * model::{forward, forward_prefill_batched, KVCache}, emit.rs:3954-5486) ---------------- */
+
+/* Exact byte length of the headerless weights.bin for this config (writer:
+ * crates/forgellm-cli/src/main.rs:2714-2757; reader: project.rs:342-407). */
+uint64_t forge_hip_weights_nbytes(const forge_hip_config* cfg);
+
+/* MetalModel::new(weights: &[u8]) (metal:4209).  Copies/repacks the blob into HBM; the caller
+ * keeps ownership of `weights_bin` and may free it on return. */
+int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* weights_bin_host, uint64_t nbytes,
+                               forge_hip_model** out);
+void forge_hip_model_destroy(forge_hip_model* m);
+
+/* MetalModel::forward(token_id) -> Vec<f32> (metal:5070) / model::forward (emit.rs:4029):
+ * one decode step at the current position; writes vocab logits to host memory; advances pos. */
+int32_t forge_hip_forward(forge_hip_model* m, uint32_t token, float* logits_host);
+
+/* forward() followed by argmax (project.rs:501-503: LAST index among equal maxima), with the
+ * argmax done on the device so that only 4 bytes cross PCIe. */
+int32_t forge_hip_forward_greedy(forge_hip_model* m, uint32_t token, uint32_t* next_token_host);
+
+/* MetalModel::forward_prefill_batch(tokens) (metal:5568) / model::forward_prefill_batched
+ * (emit.rs:5118): fills the KV cache for n tokens from the current position.  If
+ * `logits_host` is non-NULL it receives the logits of the LAST token (the CPU signature);
+ * NULL skips the lm_head (the Metal signature). */
+int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens_host, uint64_t n, float* logits_host);
+
+/* MetalModel::reset() (metal:5981): position back to 0. */
+int32_t forge_hip_reset(forge_hip_model* m);
+/* Current position (KVCache.len, emit.rs:3960). */
+int64_t forge_hip_model_pos(const forge_hip_model* m);
+/* Debug/parity: copy layer `layer`'s cached K (which=0) or V (which=1) rows [0,pos) to host as
+ * fp16 bit patterns, row-major [pos][kv_heads*head_dim]. */
+int32_t forge_hip_model_read_kv(forge_hip_model* m, uint32_t layer, uint32_t which, uint16_t* out_host);
+
+/* ---------------- host-side format helpers (no GPU needed) ---------------- */
+/* f16_bits_to_f32 / f32_to_f16_bits (emit.rs:1245-1264, 1460-1495). */
+float forge_hip_f16_to_f32(uint16_t bits);
+uint16_t forge_hip_f32_to_f16(float x);
+/* quantize_f32_to_q8_0 / _q4_0 (weight_loader.rs:1454-1544): n floats -> ceil(n/32) blocks. */
+int32_t forge_hip_quantize_f32(uint32_t wdtype, const float* data_host, uint64_t n, uint8_t* out_host);
+/* dequant_q8_0 / dequant_q4_0 (weight_loader.rs:860-926). */
+int32_t forge_hip_dequant(uint32_t wdtype, const uint8_t* data_host, uint64_t n, float* out_host);
+
+/* ---------------- op-level API ---------------- */
+
+/* Upload one weight matrix given as raw GGUF blocks, row-major [N][K/32] (the `weight: &[u8]`
+ * argument of matmul_vec_q8_0_KxN, emit.rs:1958).  K must be a multiple of 32. */
+int32_t forge_hip_qweight_create(uint32_t wdtype, const uint8_t* raw_host, uint32_t K, uint32_t N,
+                                 forge_hip_qweight** out);
+void forge_hip_qweight_destroy(forge_hip_qweight* w);
+
+/* quantize_to_q8_0_blocks_into (emit.rs:1410-1440) for M rows of K floats.
+ * q_dev: int8 [M][K]; scales_dev: fp16 bit patterns [M][K/32]. */
+int32_t forge_hip_quantize_act(const float* x_dev, uint32_t M, uint32_t K, int8_t* q_dev, uint16_t* scales_dev,
+                               void* stream);
+
+/* matmul_vec_q8_0_KxN / matmul_vec_q4_0_KxN (emit.rs:1926-2092, 2797-2958): y[N] = W x.
+ * x_dev f32 [K], y_dev f32 [N]. */
+int32_t forge_hip_gemv_q(const forge_hip_qweight* w, const float* x_dev, float* y_dev, void* stream);
+
+/* matmul_mat_q8_0_KxN / matmul_mat_q4_0_KxN (emit.rs:2108-2302, 3667-3817):
+ * y[M][N] = x[M][K] W^T, row-major. */
+int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, void* stream);
+
+/* The int32 block sums the two calls above combine: out_dev int32 [M][N][K/32]
+ * (dot_q8_0_q8_0 / dot_q4_0_q8_0 `vaddvq_s32(acc)`, emit.rs:1543-1553, 2522-2552).
+ * path 0 = the GEMV kernel's dot, path 1 = the MFMA GEMM kernel's tiles. */
+int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, uint32_t M, int32_t* out_dev,
+                              uint32_t path, void* stream);
+
+/* rms_norm (emit.rs:327-334) on M rows of H floats. */
+int32_t forge_hip_rms_norm(const float* x_dev, const float* w_dev, float eps, uint32_t M, uint32_t H, float* out_dev,
+                           void* stream);
+/* silu_mul (emit.rs:380-386). */
+int32_t forge_hip_silu_mul(const float* gate_dev, const float* up_dev, uint64_t n, float* out_dev, void* stream);
+
+/* rope (emit.rs:508-528) on q and k for M tokens at positions base_pos.., then the KV-cache
+ * write of k and v as fp16 (the reference's GPU backend: metal:3475-3553).
+ * q_dev f32 [M][heads*hd] (rotated in place); k_dev, v_dev f32 [M][kv_heads*hd] (k rotated in
+ * place); k_cache_dev, v_cache_dev: fp16 [max_seq][kv_heads*hd]. */
+int32_t forge_hip_rope_kv_store(float* q_dev, float* k_dev, const float* v_dev, uint16_t* k_cache_dev,
+                                uint16_t* v_cache_dev, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
+                                uint32_t head_dim, float theta, void* stream);
+
+/* attention_flash_batch (emit.rs:754-883) over an fp16 cache: causal, GQA.
+ * q_dev f32 [M][heads*hd] (already rotated); caches hold rows [0, base_pos+M);
+ * out_dev f32 [M][heads*hd]. */
+int32_t forge_hip_attn_prefill_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
+                                     float* out_dev, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
+                                     uint32_t head_dim, void* stream);
+
+/* attention_flash (emit.rs:656-715) over an fp16 cache: one query against seq_len rows.
+ * q_dev f32 [heads*hd], out_dev f32 [heads*hd]. */
+int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
+                                    float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
+                                    uint32_t head_dim, void* stream);
+
+/* argmax (project.rs:501-503): index of the LAST maximum of n floats -> *out_dev (uint32). */
+int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FORGE_HIP_H */

@@ -1,0 +1,220 @@
+"""GPU parity of the op-level entry points, through the C ABI, against the CPU oracle.
+Bit-exact for integer work (activation codes, block sums, argmax); rel 1e-3 / abs 1e-3 for f32."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+Q8, Q4 = 8, 2
+RTOL, ATOL = 1e-3, 1e-3
+
+
+def close(got, want, rtol=RTOL, atol=ATOL):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    bad = np.abs(got - want) > atol + rtol * np.abs(want)
+    assert not bad.any(), f"{bad.sum()} of {bad.size} outside tolerance; max abs err {np.max(np.abs(got - want)):.3e}"
+
+
+def act_planes(oracle, x2d):
+    """Oracle activation quantisation of each row, split into (codes int8 [M][K], scale bits [M][K/32])."""
+    M, K = x2d.shape
+    raw = np.stack([oracle.quantize_act(x2d[r]) for r in range(M)]).reshape(M, K // 32, 34)
+    codes = raw[:, :, 2:].reshape(M, K).view(np.int8)
+    bits = raw[:, :, 0].astype(np.uint16) | (raw[:, :, 1].astype(np.uint16) << 8)
+    return codes, bits
+
+
+def make_weight(fh, wd, N, K, seed):
+    w = fh.synth.normal(seed, N * K, 0.02).reshape(N, K)
+    return fh.ops.quantize_weights(wd, w)
+
+
+@pytest.mark.parametrize("M,K", [(1, 32), (1, 576), (3, 2048), (130, 8192)])
+def test_quantize_act_bit_exact(fh, oracle, torch_gpu, M, K):
+    torch = torch_gpu
+    x = fh.synth.normal(100 + K, M * K, 1.0).reshape(M, K)
+    x[0, :32] = 0.0                                        # an all-zero block: scale 1.0, codes 0
+    if K >= 64:
+        x[0, 32:64] = np.float32(1e-30)                    # scale below the fp16 range -> flushed to zero bits
+    q, sc = fh.ops.quantize_act(torch.from_numpy(x).cuda())
+    codes, bits = act_planes(oracle, x)
+    assert np.array_equal(q.cpu().numpy(), codes)
+    assert np.array_equal(sc.cpu().numpy().view(np.uint16), bits)
+
+
+@pytest.mark.parametrize("wd", [Q8, Q4])
+@pytest.mark.parametrize("N,K", [(8, 32), (13, 576), (260, 2048), (64, 8192), (70, 3072)])
+@pytest.mark.parametrize("path", [0, 1])
+def test_block_isums_bit_exact(fh, oracle, torch_gpu, wd, N, K, path):
+    torch = torch_gpu
+    M = 1 if path == 0 else 37
+    wraw = make_weight(fh, wd, N, K, seed=N + K)
+    x = fh.synth.normal(7 + K, M * K, 1.0).reshape(M, K)
+    w = fh.ops.QWeight(wd, wraw, K, N)
+    got = fh.ops.block_isums(w, torch.from_numpy(x).cuda(), path).cpu().numpy()
+    for r in range(M):
+        want = oracle.block_isums(wd, oracle.quantize_act(x[r]), wraw, K, N)
+        assert np.array_equal(got[r], want), f"row {r}"
+
+
+@pytest.mark.parametrize("path", [0, 1])
+def test_block_isums_extreme_codes(fh, oracle, torch_gpu, path):
+    """All +-127 activations against all +-127 weights: |isum| = 516128, the int32 extreme of a block."""
+    torch = torch_gpu
+    K, N = 64, 4
+    x = np.full((2, K), 3.0, np.float32); x[1] = -3.0                       # every code +-127
+    wf = np.full((N, K), 0.5, np.float32); wf[1::2] = -0.5
+    for wd, want_abs in ((Q8, 516128), (Q4, None)):
+        wraw = fh.ops.quantize_weights(wd, wf)
+        w = fh.ops.QWeight(wd, wraw, K, N)
+        for r in range(2 if path == 1 else 1):
+            xin = torch.from_numpy(x if path == 1 else x[:1]).cuda()
+            got = fh.ops.block_isums(w, xin, path).cpu().numpy()
+            want = oracle.block_isums(wd, oracle.quantize_act(x[r]), wraw, K, N)
+            assert np.array_equal(got[r], want)
+            if want_abs:
+                assert np.all(np.abs(got[r]) == want_abs)
+
+
+@pytest.mark.parametrize("wd", [Q8, Q4])
+@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 512), (8192, 2048), (576, 1536), (3072, 1029), (32, 5)])
+def test_matmul_vec_parity(fh, oracle, torch_gpu, wd, K, N):
+    torch = torch_gpu
+    wraw = make_weight(fh, wd, N, K, seed=3 * N + K)
+    x = fh.synth.normal(11 + K, K, 1.0)
+    w = fh.ops.QWeight(wd, wraw, K, N)
+    y = fh.ops.matmul_vec_q(w, torch.from_numpy(x).cuda()).cpu().numpy()
+    close(y, oracle.matmul_vec(wd, 0, x, wraw, K, N))
+
+
+@pytest.mark.parametrize("wd", [Q8, Q4])
+@pytest.mark.parametrize("M,K,N", [(1, 2048, 512), (37, 576, 960), (352, 2048, 2048), (130, 8192, 320), (129, 3072, 257)])
+def test_matmul_mat_parity(fh, oracle, torch_gpu, wd, M, K, N):
+    torch = torch_gpu
+    wraw = make_weight(fh, wd, N, K, seed=5 * N + K + M)
+    x = fh.synth.normal(13 + K, M * K, 1.0).reshape(M, K)
+    w = fh.ops.QWeight(wd, wraw, K, N)
+    y = fh.ops.matmul_mat_q(w, torch.from_numpy(x).cuda()).cpu().numpy()
+    close(y, oracle.matmul_mat(wd, 0, x, wraw, M, K, N))
+
+
+def test_matmul_vec_equals_matmul_mat_row(fh, torch_gpu):
+    """The two kernels combine the same exact block sums: rows agree to f32 summation-order noise."""
+    torch = torch_gpu
+    K, N, M = 2048, 512, 5
+    wraw = make_weight(fh, Q8, N, K, seed=77)
+    x = fh.synth.normal(78, M * K, 1.0).reshape(M, K)
+    w = fh.ops.QWeight(Q8, wraw, K, N)
+    xd = torch.from_numpy(x).cuda()
+    ym = fh.ops.matmul_mat_q(w, xd).cpu().numpy()
+    for r in range(M):
+        yv = fh.ops.matmul_vec_q(w, xd[r].contiguous()).cpu().numpy()
+        assert np.max(np.abs(yv - ym[r])) < 2e-5
+
+
+@pytest.mark.parametrize("M,H", [(1, 576), (5, 2048), (300, 3072)])
+def test_rms_norm_parity(fh, oracle, torch_gpu, M, H):
+    torch = torch_gpu
+    x = fh.synth.normal(1, M * H, 1.5).reshape(M, H)
+    g = 1.0 + 0.1 * fh.synth.normal(2, H, 1.0)
+    out = fh.ops.rms_norm(torch.from_numpy(x).cuda(), torch.from_numpy(g).cuda(), 1e-5).cpu().numpy()
+    want = np.stack([oracle.rms_norm(x[r], g, 1e-5) for r in range(M)])
+    close(out, want, rtol=1e-5, atol=1e-6)
+    k = fh.ops.rms_norm(torch.tensor([1., 2., 3., 4.], device="cuda"), torch.ones(4, device="cuda"), 1e-5).cpu().numpy()
+    close(k, np.array([1, 2, 3, 4]) / np.sqrt(7.5 + 1e-5), rtol=1e-6, atol=1e-6)      # kernels.rs:396-413
+
+
+def test_silu_mul_parity(fh, oracle, torch_gpu):
+    torch = torch_gpu
+    g = fh.synth.normal(3, 8192, 2.0)
+    u = fh.synth.normal(4, 8192, 1.0)
+    out = fh.ops.silu_mul(torch.from_numpy(g).cuda(), torch.from_numpy(u).cuda()).cpu().numpy()
+    close(out, oracle.silu_mul(g, u), rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("heads,kv_heads,hd,theta", [(32, 8, 64, 500000.0), (9, 3, 64, 100000.0), (24, 8, 128, 500000.0)])
+def test_rope_kv_store_parity(fh, oracle, torch_gpu, heads, kv_heads, hd, theta):
+    torch = torch_gpu
+    M, base = 7, 2241
+    q = fh.synth.normal(5, M * heads * hd, 1.0).reshape(M, heads * hd)
+    k = fh.synth.normal(6, M * kv_heads * hd, 1.0).reshape(M, kv_heads * hd)
+    v = fh.synth.normal(7, M * kv_heads * hd, 1.0).reshape(M, kv_heads * hd)
+    qd, kd, vd = (torch.from_numpy(a.copy()).cuda() for a in (q, k, v))
+    kc = torch.zeros((base + M, kv_heads * hd), dtype=torch.int16, device="cuda")
+    vc = torch.zeros_like(kc)
+    fh.ops.rope_kv_store(qd, kd, vd, kc, vc, base, heads, kv_heads, hd, theta)
+    for r in range(M):
+        wq = oracle.rope(q[r], base + r, hd, heads, theta)
+        wk = oracle.rope(k[r], base + r, hd, kv_heads, theta)
+        # same libm table and unfused mul/add: bit-identical on the host this runs on
+        assert np.array_equal(qd[r].cpu().numpy(), wq)
+        assert np.array_equal(kd[r].cpu().numpy(), wk)
+        assert np.array_equal(kc[base + r].cpu().numpy().view(np.uint16), oracle.f32_to_f16(wk))
+        assert np.array_equal(vc[base + r].cpu().numpy().view(np.uint16), oracle.f32_to_f16(v[r]))
+    assert int(kc[:base].abs().max()) == 0        # rows before base_pos untouched
+
+
+def _kv_cache(fh, oracle, seq, kv_heads, hd, seed):
+    k16 = oracle.f32_to_f16(fh.synth.normal(seed, seq * kv_heads * hd, 1.0)).reshape(seq, kv_heads * hd)
+    v16 = oracle.f32_to_f16(fh.synth.normal(seed + 1, seq * kv_heads * hd, 1.0)).reshape(seq, kv_heads * hd)
+    return k16, v16
+
+
+@pytest.mark.parametrize("heads,kv_heads,hd", [(32, 8, 64), (9, 3, 64), (32, 32, 96), (24, 8, 128), (8, 1, 64)])
+@pytest.mark.parametrize("seq", [1, 5, 64, 70, 900])
+def test_attention_decode_parity(fh, oracle, torch_gpu, heads, kv_heads, hd, seq):
+    torch = torch_gpu
+    k16, v16 = _kv_cache(fh, oracle, seq, kv_heads, hd, seed=seq + hd)
+    q = oracle.f16_to_f32(oracle.f32_to_f16(fh.synth.normal(9, heads * hd, 1.0)))
+    out = fh.ops.attention_flash(torch.from_numpy(q).cuda(), torch.from_numpy(k16.view(np.int16)).cuda(),
+                                 torch.from_numpy(v16.view(np.int16)).cuda(), seq, heads, kv_heads, hd).cpu().numpy()
+    close(out, oracle.attention("flash", q, k16, v16, seq, heads, kv_heads, hd))
+
+
+@pytest.mark.parametrize("heads,kv_heads,hd", [(8, 2, 64), (6, 6, 96), (6, 2, 128)])
+@pytest.mark.parametrize("M,base", [(1, 0), (33, 0), (200, 0), (131, 77), (64, 64)])
+def test_attention_prefill_parity(fh, oracle, torch_gpu, heads, kv_heads, hd, M, base):
+    torch = torch_gpu
+    seq = base + M
+    k16, v16 = _kv_cache(fh, oracle, seq, kv_heads, hd, seed=M + hd + base)
+    q = oracle.f16_to_f32(oracle.f32_to_f16(fh.synth.normal(10, M * heads * hd, 1.0))).reshape(M, heads * hd)
+    out = fh.ops.attention_flash_batch(torch.from_numpy(q).cuda(), torch.from_numpy(k16.view(np.int16)).cuda(),
+                                       torch.from_numpy(v16.view(np.int16)).cuda(), base, heads, kv_heads, hd).cpu().numpy()
+    close(out, oracle.attention("flash_batch", q, k16, v16, M, heads, kv_heads, hd, base_pos=base))
+
+
+def test_attention_reference_vectors_shape_scaled(fh, oracle, torch_gpu):
+    """The reference's deterministic attention inputs (emit.rs:6687-6741), widened to head_dim 64."""
+    torch = torch_gpu
+    hd, nh, nkv = 64, 3, 1
+    for seq in (5, 64, 70, 128, 200):
+        q = (((np.arange(nh * hd) * 7 + 3) % 41).astype(np.float32) * np.float32(0.1) - np.float32(1.0)) * np.float32(0.5)
+        k = (((np.arange(seq * hd) * 11 + 5) % 43).astype(np.float32) * np.float32(0.07) - np.float32(1.0)) * np.float32(0.3)
+        v = (((np.arange(seq * hd) * 13 + 7) % 47).astype(np.float32) * np.float32(0.05) - np.float32(0.5)) * np.float32(0.4)
+        k16, v16 = oracle.f32_to_f16(k).reshape(seq, hd), oracle.f32_to_f16(v).reshape(seq, hd)
+        want = oracle.attention("std", q, k16, v16, seq, nh, nkv, hd)
+        got = fh.ops.attention_flash(torch.from_numpy(q).cuda(), torch.from_numpy(k16.view(np.int16)).cuda(),
+                                     torch.from_numpy(v16.view(np.int16)).cuda(), seq, nh, nkv, hd).cpu().numpy()
+        assert np.max(np.abs(got - want)) < 1e-4          # the reference's own tolerance for this test
+
+
+def test_argmax_last_maximum_on_device(fh, oracle, torch_gpu):
+    torch = torch_gpu
+    x = fh.synth.normal(12, 128256, 1.0)
+    assert fh.ops.argmax(torch.from_numpy(x).cuda()) == oracle.argmax(x)
+    x[[5, 70000, 128255]] = 99.0
+    assert fh.ops.argmax(torch.from_numpy(x).cuda()) == 128255 == oracle.argmax(x)
+    x[128255] = 0.0
+    assert fh.ops.argmax(torch.from_numpy(x).cuda()) == 70000
+    assert fh.ops.argmax(torch.tensor([3.0], device="cuda")) == 0
+    assert fh.ops.argmax(torch.full((1000,), -7.0, device="cuda")) == 999
+
+
+def test_bad_shapes_are_rejected(fh, torch_gpu):
+    torch = torch_gpu
+    q = torch.zeros((4, 4 * 48), device="cuda")
+    kc = torch.zeros((4, 48), dtype=torch.int16, device="cuda")
+    with pytest.raises(fh.ForgeHipError):
+        fh.ops.attention_flash_batch(q, kc, kc, 0, 4, 1, 48)
+    with pytest.raises(fh.ForgeHipError):
+        fh.ops.attention_flash(q[0].contiguous(), kc, kc, 0, 4, 1, 64)

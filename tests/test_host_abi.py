@@ -1,0 +1,114 @@
+"""CPU-side checks of the product: the C-ABI library loads and exports every symbol the header
+declares, its host format code is bit-identical to the oracle, the synthetic generators are
+deterministic, and argument errors come back as codes (no compute calls: there is no GPU here)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+Q8, Q4 = 8, 2
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(fh):
+    header = open(os.path.join(ROOT, "include", "forge_hip.h")).read()
+    declared = sorted(set(re.findall(r"\b(forge_hip_[a-z0-9_]+)\s*\(", header)))
+    assert declared, "no declarations found in include/forge_hip.h"
+    L = fh.lib()
+    missing = [s for s in declared if not hasattr(L, s)]
+    assert not missing, f"declared but not exported: {missing}"
+    assert sorted(fh.EXPORTS) == declared
+
+
+def test_host_f16_matches_oracle_exhaustively(fh, oracle):
+    bits = np.arange(65536, dtype=np.uint16)
+    want = oracle.f16_to_f32(bits)
+    got = np.array([fh.ops.f16_to_f32(int(b)) for b in bits], np.float32)
+    nan = np.isnan(want)
+    assert np.array_equal(np.isnan(got), nan)
+    assert np.array_equal(got[~nan].view(np.uint32), want[~nan].view(np.uint32))
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(20000).astype(np.float32) * np.float32(10.0) ** rng.integers(-9, 6, 20000).astype(np.float32),
+                        np.array([2.0 ** -24, 2.0 ** -25, 1.5 * 2.0 ** -25, 1e-45, 65520.0, np.inf, -np.inf, 0.0, -0.0], np.float32)])
+    want = oracle.f32_to_f16(x)
+    got = np.array([fh.ops.f32_to_f16(float(v)) for v in x], np.uint16)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("wd", [Q8, Q4])
+def test_host_quantisers_bit_identical_to_oracle(fh, oracle, wd):
+    rng = np.random.default_rng(7)
+    v = (rng.standard_normal(32 * 5000 + 17) * 0.02).astype(np.float32)     # ragged tail block
+    v[320:352] = 0.0
+    assert np.array_equal(fh.ops.quantize_weights(wd, v), oracle.quantize_weights(wd, v))
+    raw = oracle.quantize_weights(wd, v)
+    assert np.array_equal(fh.ops.dequant(wd, raw, v.size), oracle.dequant(wd, raw, v.size))
+    assert fh.ops.quantize_weights(wd, np.zeros(0, np.float32)).size == 0
+
+
+def test_argmax_host_last_maximum(fh):
+    assert fh.ops.argmax_host(np.array([1, 5, 3, 5, 2], np.float32)) == 3
+    assert fh.ops.argmax_host(np.array([7, 7, 7], np.float32)) == 2
+
+
+def test_synth_is_deterministic_and_normal(fh):
+    a = fh.synth.normal(42, 100001, 0.02)
+    b = fh.synth.normal(42, 100001, 0.02)
+    assert np.array_equal(a, b) and a.dtype == np.float32
+    assert abs(float(a.mean())) < 3e-4 and float(a.std()) == pytest.approx(0.02, rel=0.02)
+    # counter based: a later window equals the same window of a longer draw
+    big = fh.synth.normal(42, (1 << 23) + 10, 1.0)
+    assert np.array_equal(big[:1000], fh.synth.normal(42, 1000, 1.0))
+    assert not np.array_equal(fh.synth.normal(43, 1000), fh.synth.normal(42, 1000))
+    ids = fh.synth.uniform_ids(1, 5000, 49152)
+    assert ids.max() < 49152 and len(set(ids.tolist())) > 4000
+    # splitmix64 known answer for seed 0: first output
+    assert int(fh.synth.splitmix64(0, 0, 1)[0]) == 0xE220A8397B1DCDAF
+
+
+def test_weight_stream_bytes_match_published_figures(fh):
+    """Algorithmic bytes per decode token (N*(K/32)*B + 4K + 4N per matmul)."""
+    assert fh.synth.decode_weight_bytes(fh.synth.llama32_1b(Q8)) == 1312980992
+    assert fh.synth.decode_weight_bytes(fh.synth.llama32_1b(Q4)) == 695107584
+    assert fh.synth.decode_weight_bytes(fh.synth.smollm2_135m(Q8)) == 142884864
+    assert fh.synth.decode_weight_bytes(fh.synth.llama32_3b(Q8)) == 3413360640
+
+
+def test_blob_size_contract(fh, oracle):
+    from forge_llm_amd.hip_model import weights_nbytes
+    for cfg in (fh.synth.tiny(Q8), fh.synth.tiny(Q4), fh.synth.smollm2_135m(Q8), fh.synth.llama32_1b(Q8), fh.synth.llama32_3b(Q4)):
+        assert weights_nbytes(cfg) == oracle.weights_nbytes(cfg)
+    cfg = fh.synth.tiny(Q8)
+    blob = fh.synth.make_weights_blob(cfg, seed=1)
+    assert blob.size == weights_nbytes(cfg)
+    # tied embeddings: the f32 table is the dequantised lm_head
+    H, V = cfg["hidden"], cfg["vocab"]
+    table = blob[:V * H * 4].view(np.float32)
+    lm_raw = blob[-(V * H // 32 * 34):]
+    assert np.array_equal(table, oracle.dequant(Q8, lm_raw, V * H))
+
+
+def test_errors_are_codes_not_crashes(fh):
+    L = fh.lib()
+    cfg = fh.synth.tiny(Q8)
+    blob = fh.synth.make_weights_blob(cfg, seed=1)
+    h = C.c_void_p()
+    bad = dict(cfg, head_dim=48)
+    c = fh.Config(**bad)
+    assert L.forge_hip_model_create(C.byref(c), blob.ctypes.data_as(C.c_void_p), blob.size, C.byref(h)) == fh.ERR_INVALID
+    assert b"head_dim" in L.forge_hip_last_error()
+    c = fh.Config(**dict(cfg, wdtype=12))
+    assert L.forge_hip_model_create(C.byref(c), blob.ctypes.data_as(C.c_void_p), blob.size, C.byref(h)) == fh.ERR_INVALID
+    c = fh.Config(**cfg)
+    rc = L.forge_hip_model_create(C.byref(c), blob.ctypes.data_as(C.c_void_p), blob.size - 1, C.byref(h))
+    assert rc == fh.ERR_BLOB_SIZE and not h.value        # the reference panics on a short blob (project.rs:342-406)
+    with pytest.raises(fh.ForgeHipError):
+        fh.HipModel(cfg, blob[:-5])
+    assert L.forge_hip_quantize_f32(99, None, 0, None) == fh.ERR_INVALID
+    w = C.c_void_p()
+    assert L.forge_hip_qweight_create(Q8, blob.ctypes.data_as(C.c_void_p), 48, 4, C.byref(w)) == fh.ERR_INVALID
+    if fh.device_count() == 0:
+        rc = L.forge_hip_model_create(C.byref(c), blob.ctypes.data_as(C.c_void_p), blob.size, C.byref(h))
+        assert rc == fh.ERR_NO_DEVICE                     # metal:4212 `expect("no Metal device found")`
