@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libforge_hip.so")
 
 Q4_0 = 2
 Q8_0 = 8
+FLAG_EXACT = 1   # config.flags / op flags: order-faithful f32 arithmetic (bit-identical to the CPU path)
 
 OK = 0
 ERR_INVALID = -1
@@ -28,7 +29,7 @@ EXPORTS = [
     "forge_hip_last_error", "forge_hip_device_count", "forge_hip_weights_nbytes", "forge_hip_model_create",
     "forge_hip_model_destroy", "forge_hip_forward", "forge_hip_forward_greedy", "forge_hip_prefill_batch",
     "forge_hip_reset", "forge_hip_model_pos", "forge_hip_model_read_kv", "forge_hip_f16_to_f32",
-    "forge_hip_f32_to_f16", "forge_hip_quantize_f32", "forge_hip_dequant", "forge_hip_qweight_create",
+    "forge_hip_f32_to_f16", "forge_hip_quantize_f32", "forge_hip_expf_host", "forge_hip_dequant", "forge_hip_qweight_create",
     "forge_hip_qweight_destroy", "forge_hip_quantize_act", "forge_hip_gemv_q", "forge_hip_gemm_q",
     "forge_hip_block_isums", "forge_hip_rms_norm", "forge_hip_silu_mul", "forge_hip_rope_kv_store",
     "forge_hip_attn_prefill_f16kv", "forge_hip_attn_decode_f16kv", "forge_hip_argmax",
@@ -100,7 +101,9 @@ def lib():
     L.forge_hip_gemv_q.restype = i32
     L.forge_hip_gemv_q.argtypes = [vp, vp, vp, vp]
     L.forge_hip_gemm_q.restype = i32
-    L.forge_hip_gemm_q.argtypes = [vp, vp, u32, vp, vp]
+    L.forge_hip_gemm_q.argtypes = [vp, vp, u32, vp, u32, vp]
+    L.forge_hip_expf_host.restype = i32
+    L.forge_hip_expf_host.argtypes = [vp, u64, vp]
     L.forge_hip_block_isums.restype = i32
     L.forge_hip_block_isums.argtypes = [vp, vp, u32, vp, u32, vp]
     L.forge_hip_rms_norm.restype = i32
@@ -110,9 +113,9 @@ def lib():
     L.forge_hip_rope_kv_store.restype = i32
     L.forge_hip_rope_kv_store.argtypes = [vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, C.c_float, vp]
     L.forge_hip_attn_prefill_f16kv.restype = i32
-    L.forge_hip_attn_prefill_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, vp]
+    L.forge_hip_attn_prefill_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]
     L.forge_hip_attn_decode_f16kv.restype = i32
-    L.forge_hip_attn_decode_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, vp]
+    L.forge_hip_attn_decode_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, vp]
     L.forge_hip_argmax.restype = i32
     L.forge_hip_argmax.argtypes = [vp, u32, vp, vp]
     _lib = L
@@ -136,4 +139,4 @@ def require_gpu():
 from .hip_model import HipModel  # noqa: E402
 from . import ops, synth  # noqa: E402
 
-__all__ = ["HipModel", "ops", "synth", "Config", "ForgeHipError", "lib", "check", "device_count", "Q4_0", "Q8_0"]
+__all__ = ["HipModel", "ops", "synth", "Config", "ForgeHipError", "lib", "check", "device_count", "Q4_0", "Q8_0", "FLAG_EXACT"]

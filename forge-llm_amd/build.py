@@ -11,10 +11,11 @@ BUILD = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libforge_hip.so")
 
 SOURCES = ["format.hip", "elementwise.hip", "gemv.hip", "gemm.hip", "attn_decode.hip", "attn_prefill.hip",
-           "api.hip", "model.hip"]
+           "attn_exact.hip", "api.hip", "model.hip"]
 
 # -packed-fp32-ops off: keep hipcc from forming packed FP32 instructions.
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
+# -ffp-contract=off: the CPU path never fuses a*b+c; kernels say fmaf() where a fused op is meant.
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-ffp-contract=off",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-I", INCLUDE, "-I", CSRC]
 

@@ -6,6 +6,7 @@
 #include <vector>
 
 #include "common.h"
+#include "expf_ref.h"
 
 namespace fh {
 
@@ -136,18 +137,20 @@ int32_t forge_hip_gemv_q(const forge_hip_qweight* w, const float* x_dev, float* 
     int8_t* q; uint16_t* sc;
     int32_t rc = quantise_into_scratch(x_dev, 1, w->w.K, &q, &sc, (hipStream_t)stream);
     if (rc) return rc;
-    launch_gemv(w->w, q, sc, y_dev, false, (hipStream_t)stream);
+    launch_gemv(w->w, q, sc, y_dev, false, GemvOrder::MatmulVec, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }
 
-int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, void* stream) {
+int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, uint32_t flags,
+                         void* stream) {
     FH_CHECK(w && x_dev && y_dev, "gemm_q: null pointer");
+    FH_CHECK((flags & ~FORGE_HIP_FLAG_EXACT) == 0, "gemm_q: unknown flag bits");
     if (M == 0) return FORGE_HIP_OK;
     int8_t* q; uint16_t* sc;
     int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream);
     if (rc) return rc;
-    launch_gemm(w->w, q, sc, M, y_dev, w->w.N, false, nullptr, (hipStream_t)stream);
+    launch_gemm(w->w, q, sc, M, y_dev, w->w.N, false, (flags & FORGE_HIP_FLAG_EXACT) != 0, nullptr, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }
@@ -170,7 +173,7 @@ int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, ui
         Scratch& sink = g_attn;
         rc = sink.reserve((size_t)M * w->w.N * sizeof(float));
         if (rc) return rc;
-        launch_gemm(w->w, q, sc, M, reinterpret_cast<float*>(sink.p), w->w.N, false, out_dev, (hipStream_t)stream);
+        launch_gemm(w->w, q, sc, M, reinterpret_cast<float*>(sink.p), w->w.N, false, true, out_dev, (hipStream_t)stream);
     }
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
@@ -179,7 +182,7 @@ int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, ui
 int32_t forge_hip_rms_norm(const float* x_dev, const float* w_dev, float eps, uint32_t M, uint32_t H, float* out_dev,
                            void* stream) {
     FH_CHECK(x_dev && w_dev && out_dev, "rms_norm: null pointer");
-    FH_CHECK(H % 4 == 0 && H >= 4, "rms_norm: H must be a multiple of 4");
+    FH_CHECK(H % 4 == 0 && H >= 4 && H <= 16352, "rms_norm: H must be a multiple of 4, at most 16352");
     launch_rmsnorm(x_dev, w_dev, eps, M, H, out_dev, nullptr, nullptr, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
@@ -231,28 +234,45 @@ static int32_t check_attn_shape(const char* who, uint32_t heads, uint32_t kv_hea
 
 int32_t forge_hip_attn_prefill_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                      float* out_dev, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
-                                     uint32_t head_dim, void* stream) {
+                                     uint32_t head_dim, uint32_t flags, void* stream) {
     FH_CHECK(q_dev && k_cache_dev && v_cache_dev && out_dev, "attn_prefill: null pointer");
+    FH_CHECK((flags & ~FORGE_HIP_FLAG_EXACT) == 0, "attn_prefill: unknown flag bits");
     int32_t rc = check_attn_shape("attn_prefill", heads, kv_heads, head_dim);
     if (rc) return rc;
-    launch_attn_prefill(q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, M, base_pos, heads,
-                        kv_heads, head_dim, (hipStream_t)stream);
+    if (flags & FORGE_HIP_FLAG_EXACT)
+        launch_attn_exact(true, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr,
+                          nullptr, M, base_pos, nullptr, heads, kv_heads, head_dim, (hipStream_t)stream);
+    else
+        launch_attn_prefill(q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, M, base_pos,
+                            heads, kv_heads, head_dim, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }
 
 int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                     float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
-                                    uint32_t head_dim, void* stream) {
+                                    uint32_t head_dim, uint32_t flags, void* stream) {
     FH_CHECK(q_dev && k_cache_dev && v_cache_dev && out_dev, "attn_decode: null pointer");
     FH_CHECK(seq_len >= 1, "attn_decode: seq_len must be at least 1");
+    FH_CHECK((flags & ~FORGE_HIP_FLAG_EXACT) == 0, "attn_decode: unknown flag bits");
     int32_t rc = check_attn_shape("attn_decode", heads, kv_heads, head_dim);
     if (rc) return rc;
-    rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
-    if (rc) return rc;
-    launch_attn_decode(q_dev, k_cache_dev, v_cache_dev, out_dev, nullptr, nullptr, seq_len, nullptr, heads, kv_heads,
-                       head_dim, g_attn.p, (hipStream_t)stream);
+    if (flags & FORGE_HIP_FLAG_EXACT) {
+        launch_attn_exact(false, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr,
+                          nullptr, 1, seq_len - 1, nullptr, heads, kv_heads, head_dim, (hipStream_t)stream);
+    } else {
+        rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
+        if (rc) return rc;
+        launch_attn_decode(q_dev, k_cache_dev, v_cache_dev, out_dev, nullptr, nullptr, seq_len, nullptr, heads, kv_heads,
+                           head_dim, g_attn.p, (hipStream_t)stream);
+    }
     FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_expf_host(const float* x_host, uint64_t n, float* out_host) {
+    FH_CHECK(x_host && out_host, "expf_host: null pointer");
+    for (uint64_t i = 0; i < n; i++) out_host[i] = expf_ref<true>(x_host[i]);
     return FORGE_HIP_OK;
 }
 

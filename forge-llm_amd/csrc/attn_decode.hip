@@ -91,7 +91,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const float* __r
         for (int g = 0; g < GT; g++) {
             float d = 0.f;
 #pragma unroll
-            for (int i = 0; i < 8; i++) d += qf[g][i] * kf[i];
+            for (int i = 0; i < 8; i++) d = fmaf(qf[g][i], kf[i], d);
 #pragma unroll
             for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, WAVE);
             if (valid) {
@@ -99,9 +99,9 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const float* __r
                 const float mn = fmaxf(m[g], s);
                 const float alpha = __expf(m[g] - mn);   // m = -inf on the first key: exp(-inf) = 0
                 const float p = __expf(s - mn);
-                l[g] = l[g] * alpha + p;
+                l[g] = fmaf(l[g], alpha, p);
 #pragma unroll
-                for (int i = 0; i < 8; i++) acc[g][i] = acc[g][i] * alpha + p * vf[i];
+                for (int i = 0; i < 8; i++) acc[g][i] = fmaf(acc[g][i], alpha, p * vf[i]);
                 m[g] = mn;
             }
         }

@@ -1,0 +1,123 @@
+// Order-faithful attention over the fp16 KV cache: attention_flash (emit.rs:656-715) and
+// attention_flash_batch (emit.rs:754-883) with every f32 operation in the reference's own
+// order — sequential q.k dots, 64-key blocks, block maximum, exp via the C library's
+// algorithm, sequential block sums, and the two kernels' different P.V accumulation orders
+// (flash: block-local sum then add; flash_batch: straight into the accumulator).
+//
+// This is the attention the model uses when it is created with FORGE_HIP_FLAG_EXACT: its
+// output is bit-identical to the CPU path, which is what it takes for greedy tokens to be
+// identical, because the output is quantised to int8 next and one flipped code cascades.
+// It is a VALU kernel: one workgroup per (query row, head), keys across lanes for the
+// scores, head dims across lanes for P.V.  The MFMA / split-sequence kernels are the fast
+// path and agree with it to the float tolerance.
+#include "common.h"
+#include "device_utils.h"
+#include "expf_ref.h"
+
+namespace fh {
+
+constexpr int XB = 64;   // FLASH_ATTN_BLOCK_SIZE, emit.rs:201
+
+template <int HD, bool BATCH>
+__global__ void attn_exact_kernel(const float* __restrict__ q, uint32_t q_stride, const uint16_t* __restrict__ kc,
+                                  const uint16_t* __restrict__ vc, float* __restrict__ out, uint32_t out_stride,
+                                  int8_t* __restrict__ oq, uint16_t* __restrict__ osc, uint32_t base_pos,
+                                  const uint32_t* __restrict__ pos_dev, uint32_t heads, uint32_t kv_heads) {
+    __shared__ float qs[HD];
+    __shared__ float e[XB];
+    __shared__ float red[2];
+    const uint32_t tid = threadIdx.x;
+    const uint32_t h = blockIdx.x, r = blockIdx.y;
+    const uint32_t kvh = h / (heads / kv_heads);
+    const uint32_t qpos = (pos_dev ? *pos_dev : base_pos) + r;
+    const uint32_t seq = qpos + 1;
+    const uint32_t kv_stride = kv_heads * HD;
+    const float scale = 1.0f / sqrtf((float)HD);
+
+    if (tid < HD) qs[tid] = q[(size_t)r * q_stride + h * HD + tid];
+    __syncthreads();
+
+    float m_i = -INFINITY, l_i = 0.f, acc = 0.f;   // acc: head dim `tid`
+    for (uint32_t bs = 0; bs < seq; bs += XB) {
+        const uint32_t bl = min((uint32_t)XB, seq - bs);
+        // ---- scores: thread bi owns key bs+bi; sum += q[i]*k[i] in order, then * scale
+        float s = -INFINITY;
+        if (tid < bl) {
+            const uint16_t* krow = kc + (size_t)(bs + tid) * kv_stride + kvh * HD;
+            float sum = 0.f;
+#pragma unroll
+            for (int c = 0; c < HD / 8; c++) {
+                const uint4 w = *reinterpret_cast<const uint4*>(krow + c * 8);
+                const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    sum = sum + qs[c * 8 + 2 * j] * f16_bits_to_f32((uint16_t)(ww[j] & 0xFFFFu));
+                    sum = sum + qs[c * 8 + 2 * j + 1] * f16_bits_to_f32((uint16_t)(ww[j] >> 16));
+                }
+            }
+            s = sum * scale;
+        }
+        // ---- block maximum (order-free), running maximum, rescale
+        if (tid < 64) {
+            const float mb = wave_max(s);
+            if (tid == 0) red[0] = mb;
+        }
+        __syncthreads();
+        const float m_block = red[0];
+        const float m_prev = m_i;
+        if (m_block > m_i) m_i = m_block;
+        const float exp_scale = expf_ref<true>(m_prev - m_i);
+        l_i = l_i * exp_scale;
+        acc = acc * exp_scale;
+        if (tid < bl) e[tid] = expf_ref<true>(s - m_i);
+        __syncthreads();
+        // ---- l_block: sequential over the block (every thread redundantly: same bits)
+        float l_block = 0.f;
+        for (uint32_t bi = 0; bi < bl; bi++) l_block = l_block + e[bi];
+        l_i = l_i + l_block;
+        // ---- P.V for head dim tid
+        if (tid < HD) {
+            const uint16_t* vcol = vc + (size_t)bs * kv_stride + kvh * HD + tid;
+            if (BATCH) {
+                for (uint32_t bi = 0; bi < bl; bi++) acc = acc + e[bi] * f16_bits_to_f32(vcol[(size_t)bi * kv_stride]);
+            } else {
+                float sum = 0.f;
+                for (uint32_t bi = 0; bi < bl; bi++) sum = sum + e[bi] * f16_bits_to_f32(vcol[(size_t)bi * kv_stride]);
+                acc = acc + sum;
+            }
+        }
+        __syncthreads();   // e[] and red[] are rewritten by the next block
+    }
+    const float inv_l = 1.0f / l_i;
+    const float o = acc * inv_l;
+    if (tid < HD && out) out[(size_t)r * out_stride + h * HD + tid] = o;
+    if (oq) {
+        // int8 block quantisation of the output row (blocks of 32 head dims), for the O projection
+        float amax = tid < HD ? fabsf(o) : 0.f;
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+        float inv;
+        const float sc = act_scale(amax, inv);
+        if (tid < HD) {
+            const size_t idx = (size_t)r * heads * HD + h * HD + tid;
+            oq[idx] = (int8_t)quant_code(o * inv);
+            if ((tid & 31) == 0) osc[idx / 32] = f32_to_f16_bits(sc);
+        }
+    }
+}
+
+void launch_attn_exact(bool batch_order, const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc,
+                       float* out, uint32_t out_stride, int8_t* oq, uint16_t* osc, uint32_t M, uint32_t base_pos,
+                       const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s) {
+    if (M == 0) return;
+    dim3 grid(heads, M);
+    const uint32_t threads = hd <= 64 ? 64 : 128;
+#define FH_AX(HD_, B_) \
+    attn_exact_kernel<HD_, B_><<<grid, threads, 0, s>>>(q, q_stride, kc, vc, out, out_stride, oq, osc, base_pos, pos_dev, heads, kv_heads)
+    if (hd == 64) { if (batch_order) FH_AX(64, true); else FH_AX(64, false); }
+    else if (hd == 96) { if (batch_order) FH_AX(96, true); else FH_AX(96, false); }
+    else { if (batch_order) FH_AX(128, true); else FH_AX(128, false); }
+#undef FH_AX
+}
+
+}  // namespace fh

@@ -84,13 +84,17 @@ void launch_argmax(const float* x, uint32_t n, uint32_t* out, void* scratch, hip
 void launch_advance(uint32_t* pos_dev, uint32_t* token_dev, const uint32_t* next_dev, hipStream_t s);
 
 // gemv.hip — y[n] (=|+=) sum_b f32(isum_b) * (a_s[b]*w_s[n][b]); activations already quantised.
-void launch_gemv(const QWeight& w, const int8_t* aq, const uint16_t* as, float* y, bool accumulate, hipStream_t s);
+// `order` selects which rows take the reference's 4-accumulator (dot1) order instead of the sequential one.
+enum class GemvOrder { MatmulVec, LmHead, LmHeadAfterPrefill };
+void launch_gemv(const QWeight& w, const int8_t* aq, const uint16_t* as, float* y, bool accumulate, GemvOrder order,
+                 hipStream_t s);
 void launch_gemv_isums(const QWeight& w, const int8_t* aq, int32_t* out, hipStream_t s);
 bool gemv_k_supported(uint32_t K);
 
 // gemm.hip — y[m][n] (=|+=) ...; aq int8 [M][K], as fp16 [M][K/32].  isums (optional) int32 [M][N][K/32].
+// exact: unfused multiply/add per block (bit-identical to the CPU path); otherwise one FMA per block.
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
-                 bool accumulate, int32_t* isums, hipStream_t s);
+                 bool accumulate, bool exact, int32_t* isums, hipStream_t s);
 
 // attn_decode.hip
 constexpr uint32_t DECODE_SPLITS = 32;
@@ -107,5 +111,12 @@ void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, 
                          uint32_t hd, hipStream_t s);
 
 bool attn_head_dim_supported(uint32_t hd);
+
+// attn_exact.hip — order-faithful attention (one workgroup per row and head).  batch_order selects
+// attention_flash_batch's accumulation order, otherwise attention_flash's.  Row r sits at position
+// (pos_dev ? *pos_dev : base_pos) + r and sees keys [0, that position].
+void launch_attn_exact(bool batch_order, const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc,
+                       float* out, uint32_t out_stride, int8_t* oq, uint16_t* osc, uint32_t M, uint32_t base_pos,
+                       const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s);
 
 }  // namespace fh

@@ -4,6 +4,7 @@
 // (emit.rs:1410-1440 re-quantises the same vector once per matmul; the result is identical).
 #include "common.h"
 #include "device_utils.h"
+#include "expf_ref.h"
 
 namespace fh {
 
@@ -29,24 +30,36 @@ void launch_quantize_act(const float* x, uint32_t M, uint32_t K, int8_t* q, uint
 }
 
 // ---- rms_norm (emit.rs:327-334) + optional block quantisation -------------------------------
-// One workgroup per row.  ss = sum x^2 (tree order, f32), inv = 1/sqrt(ss/n + eps),
-// out = (x*inv)*w.
+// One workgroup per row.  The sum of squares follows the reference's dot_f32 on its primary
+// (aarch64) path bit for bit (emit.rs:272-295): sixteen fused-multiply-add accumulators over
+// elements i mod 16, combined as (s[i]+s[i+4]) + (s[i+8]+s[i+12]) for i < 4, then pairwise,
+// then the H mod 16 tail added in order.  inv = 1/sqrt(ss/n + eps), out = (x*inv)*w.
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                       float eps, uint32_t H, float* __restrict__ normed,
                                                       uint32_t* __restrict__ q, uint16_t* __restrict__ sc) {
-    __shared__ float red[4];
+    extern __shared__ float xs[];          // the row, then 16 partial sums, then the result
     const uint32_t row = blockIdx.x, tid = threadIdx.x;
     const float4* xr = reinterpret_cast<const float4*>(x + (size_t)row * H);
     const uint32_t n4 = H / 4;
-    float ss = 0.f;
-    for (uint32_t i = tid; i < n4; i += 256) {
-        float4 v = xr[i];
-        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-    }
-    ss = wave_sum(ss);
-    if ((tid & 63) == 0) red[tid >> 6] = ss;
+    for (uint32_t i = tid; i < n4; i += 256) reinterpret_cast<float4*>(xs)[i] = xr[i];
     __syncthreads();
-    ss = (red[0] + red[1]) + (red[2] + red[3]);
+    float* part = xs + H;
+    if (tid < 16) {
+        float s = 0.f;
+        const uint32_t chunks = H / 16;
+        for (uint32_t c = 0; c < chunks; c++) { const float v = xs[c * 16 + tid]; s = fmaf(v, v, s); }
+        part[tid] = s;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float t[4];
+        for (int i = 0; i < 4; i++) t[i] = (part[i] + part[4 + i]) + (part[8 + i] + part[12 + i]);
+        float r = (t[0] + t[1]) + (t[2] + t[3]);
+        for (uint32_t i = H / 16 * 16; i < H; i++) r = r + xs[i] * xs[i];
+        part[16] = r;
+    }
+    __syncthreads();
+    const float ss = part[16];
     const float inv = 1.0f / sqrtf(ss / (float)H + eps);
     const float4* wr = reinterpret_cast<const float4*>(w);
     const uint32_t n4_pad = (n4 + 255) / 256 * 256;
@@ -71,7 +84,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
 void launch_rmsnorm(const float* x, const float* w, float eps, uint32_t M, uint32_t H, float* normed, int8_t* q,
                     uint16_t* sc, hipStream_t s) {
     if (M == 0) return;
-    rmsnorm_kernel<<<M, 256, 0, s>>>(x, w, eps, H, normed, reinterpret_cast<uint32_t*>(q), sc);
+    rmsnorm_kernel<<<M, 256, (H + 32) * sizeof(float), s>>>(x, w, eps, H, normed, reinterpret_cast<uint32_t*>(q), sc);
 }
 
 // ---- silu_mul (emit.rs:380-386) + optional block quantisation --------------------------------
@@ -85,10 +98,11 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
         uint64_t r = i / I4, c = i % I4;
         float4 g = reinterpret_cast<const float4*>(gate + r * row_stride)[c];
         float4 u = reinterpret_cast<const float4*>(up + r * row_stride)[c];
-        o.x = (g.x / (1.0f + expf(-g.x))) * u.x;
-        o.y = (g.y / (1.0f + expf(-g.y))) * u.y;
-        o.z = (g.z / (1.0f + expf(-g.z))) * u.z;
-        o.w = (g.w / (1.0f + expf(-g.w))) * u.w;
+        // exp as the CPU's C library computes it: the result is quantised to int8 next
+        o.x = (g.x / (1.0f + expf_ref<true>(-g.x))) * u.x;
+        o.y = (g.y / (1.0f + expf_ref<true>(-g.y))) * u.y;
+        o.z = (g.z / (1.0f + expf_ref<true>(-g.z))) * u.z;
+        o.w = (g.w / (1.0f + expf_ref<true>(-g.w))) * u.w;
         if (out) reinterpret_cast<float4*>(out)[i] = o;
     }
     if (q) {

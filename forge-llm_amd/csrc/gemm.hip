@@ -26,7 +26,9 @@ __device__ __forceinline__ uint32_t nib_minus8(uint32_t x) {
     return ((x | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
 }
 
-template <bool Q4, bool DUMP>
+// EXACT: block products are multiplied and added unfused, in block order, which is bit for bit the
+// reference's `r += s * f32(isum)`; otherwise one fused multiply-add per block (faster, last-bit different).
+template <bool Q4, bool DUMP, bool EXACT>
 __global__ __launch_bounds__(256) void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ wsc,
                                                      const int8_t* __restrict__ aq, const uint16_t* __restrict__ asc,
                                                      float* __restrict__ y, int32_t* __restrict__ isums, uint32_t M,
@@ -159,10 +161,14 @@ __global__ __launch_bounds__(256) void gemm_q_kernel(const uint8_t* __restrict__
                     v16i isum = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tm], bf[tn], z, 0, 0, 0);
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        acc[tm][tn][4 * g + 0] += (sa[g].x * sw) * (float)isum[4 * g + 0];
-                        acc[tm][tn][4 * g + 1] += (sa[g].y * sw) * (float)isum[4 * g + 1];
-                        acc[tm][tn][4 * g + 2] += (sa[g].z * sw) * (float)isum[4 * g + 2];
-                        acc[tm][tn][4 * g + 3] += (sa[g].w * sw) * (float)isum[4 * g + 3];
+                        const float sv[4] = {sa[g].x, sa[g].y, sa[g].z, sa[g].w};
+#pragma unroll
+                        for (int e = 0; e < 4; e++) {
+                            float& c = acc[tm][tn][4 * g + e];
+                            const float f = (float)isum[4 * g + e];
+                            if (EXACT) c = c + (sv[e] * sw) * f;
+                            else c = fmaf(sv[e] * sw, f, c);
+                        }
                     }
                     if (DUMP) {
                         const uint32_t b = k0 / 32 + kb;
@@ -197,18 +203,23 @@ __global__ __launch_bounds__(256) void gemm_q_kernel(const uint8_t* __restrict__
 }
 
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
-                 bool accumulate, int32_t* isums, hipStream_t s) {
+                 bool accumulate, bool exact, int32_t* isums, hipStream_t s) {
     if (M == 0) return;
     dim3 grid((w.N + BN - 1) / BN, (M + BM - 1) / BM);
     const int accf = accumulate ? 1 : 0;
     const bool q4 = w.wdtype == FORGE_HIP_Q4_0;
+#define FH_GEMM_LAUNCH(Q4_, DUMP_, EXACT_) \
+    gemm_q_kernel<Q4_, DUMP_, EXACT_><<<grid, 256, 0, s>>>(w.qs, w.scales, aq, as, y, isums, M, w.N, w.K, ldy, accf)
     if (q4) {
-        if (isums) gemm_q_kernel<true, true><<<grid, 256, 0, s>>>(w.qs, w.scales, aq, as, y, isums, M, w.N, w.K, ldy, accf);
-        else gemm_q_kernel<true, false><<<grid, 256, 0, s>>>(w.qs, w.scales, aq, as, y, isums, M, w.N, w.K, ldy, accf);
+        if (isums) FH_GEMM_LAUNCH(true, true, true);
+        else if (exact) FH_GEMM_LAUNCH(true, false, true);
+        else FH_GEMM_LAUNCH(true, false, false);
     } else {
-        if (isums) gemm_q_kernel<false, true><<<grid, 256, 0, s>>>(w.qs, w.scales, aq, as, y, isums, M, w.N, w.K, ldy, accf);
-        else gemm_q_kernel<false, false><<<grid, 256, 0, s>>>(w.qs, w.scales, aq, as, y, isums, M, w.N, w.K, ldy, accf);
+        if (isums) FH_GEMM_LAUNCH(false, true, true);
+        else if (exact) FH_GEMM_LAUNCH(false, false, true);
+        else FH_GEMM_LAUNCH(false, false, false);
     }
+#undef FH_GEMM_LAUNCH
 }
 
 }  // namespace fh

@@ -90,11 +90,15 @@ int32_t validate(const forge_hip_config* c) {
     FH_CHECK(c, "config is null");
     FH_CHECK(c->wdtype == FORGE_HIP_Q8_0 || c->wdtype == FORGE_HIP_Q4_0, "wdtype must be Q8_0 (8) or Q4_0 (2)");
     FH_CHECK(c->lm_head_dtype == FORGE_HIP_Q8_0 || c->lm_head_dtype == FORGE_HIP_Q4_0, "lm_head_dtype must be Q8_0 (8) or Q4_0 (2)");
-    FH_CHECK(c->hidden >= 32 && c->hidden % 32 == 0, "hidden must be a positive multiple of 32");
+    FH_CHECK(c->hidden >= 32 && c->hidden % 32 == 0 && c->hidden <= 16352, "hidden must be a multiple of 32 in [32, 16352]");
     FH_CHECK(c->inter >= 32 && c->inter % 32 == 0, "inter must be a positive multiple of 32");
     FH_CHECK(c->layers >= 1 && c->vocab >= 1 && c->max_seq >= 1, "layers, vocab and max_seq must be positive");
     FH_CHECK(c->heads >= 1 && c->kv_heads >= 1 && c->heads % c->kv_heads == 0, "heads must be a positive multiple of kv_heads");
     FH_CHECK(attn_head_dim_supported(c->head_dim), "head_dim must be 64, 96 or 128");
+    FH_CHECK((c->flags & ~FORGE_HIP_FLAG_EXACT) == 0, "unknown bits in flags");
+    // The reference switches to its non-flash attention (a different summation order) when
+    // max_seq_len <= 512 (emit.rs:126-128); the order-faithful kernels follow the flash variants only.
+    FH_CHECK(!(c->flags & FORGE_HIP_FLAG_EXACT) || c->max_seq > 512, "FORGE_HIP_FLAG_EXACT needs max_seq > 512");
     FH_CHECK(gemv_k_supported(c->hidden) && gemv_k_supported(c->inter) && gemv_k_supported(c->heads * c->head_dim),
              "hidden, inter and heads*head_dim must be at most 16384");
     return FORGE_HIP_OK;
@@ -113,43 +117,54 @@ void enqueue_layer(forge_hip_model* m, uint32_t l, bool decode, uint32_t M, uint
     int8_t* aq = decode ? m->aq.as<int8_t>() : m->paq.as<int8_t>();
     uint16_t* asc = decode ? m->asc.as<uint16_t>() : m->pasc.as<uint16_t>();
 
+    const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
+    const GemvOrder mv = GemvOrder::MatmulVec;
     launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s);
-    if (decode) launch_gemv(L.qkv, aq, asc, qkv, false, s);
-    else launch_gemm(L.qkv, aq, asc, M, qkv, QKV, false, nullptr, s);
+    if (decode) launch_gemv(L.qkv, aq, asc, qkv, false, mv, s);
+    else launch_gemm(L.qkv, aq, asc, M, qkv, QKV, false, exact, nullptr, s);
     launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos,
                          decode ? m->d_pos() : nullptr, c.heads, c.kv_heads, c.head_dim, m->cos_t.as<float>(),
                          m->sin_t.as<float>(), s);
     if (decode) {
-        launch_attn_decode(qkv, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads, c.head_dim,
-                           m->attn_ws.p, s);
-        launch_gemv(L.o, aq, asc, x, true, s);
+        if (exact)
+            launch_attn_exact(false, qkv, QKV, m->kc(l), m->vc(l), nullptr, QKS, aq, asc, 1, 0, m->d_pos(), c.heads,
+                              c.kv_heads, c.head_dim, s);
+        else
+            launch_attn_decode(qkv, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads,
+                               c.head_dim, m->attn_ws.p, s);
+        launch_gemv(L.o, aq, asc, x, true, mv, s);
     } else {
         float* attn = m->pattn.as<float>();
-        launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, s);
+        if (exact)
+            launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr,
+                              c.heads, c.kv_heads, c.head_dim, s);
+        else
+            launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, s);
         launch_quantize_act(attn, M, QKS, aq, asc, s);
-        launch_gemm(L.o, aq, asc, M, x, H, true, nullptr, s);
+        launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s);
     }
     launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s);
-    if (decode) launch_gemv(L.gate_up, aq, asc, gu, false, s);
-    else launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, nullptr, s);
+    if (decode) launch_gemv(L.gate_up, aq, asc, gu, false, mv, s);
+    else launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s);
     launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s);
-    if (decode) launch_gemv(L.down, aq, asc, x, true, s);
-    else launch_gemm(L.down, aq, asc, M, x, H, true, nullptr, s);
+    if (decode) launch_gemv(L.down, aq, asc, x, true, mv, s);
+    else launch_gemm(L.down, aq, asc, M, x, H, true, exact, nullptr, s);
 }
 
 // Final norm of one row + lm_head GEMV + argmax.
-void enqueue_head(forge_hip_model* m, const float* xrow) {
+void enqueue_head(forge_hip_model* m, const float* xrow, bool after_prefill) {
     hipStream_t s = m->stream;
     launch_rmsnorm(xrow, m->final_norm.as<float>(), m->cfg.rms_eps, 1, m->H, nullptr, m->aq.as<int8_t>(),
                    m->asc.as<uint16_t>(), s);
-    launch_gemv(m->lm_head, m->aq.as<int8_t>(), m->asc.as<uint16_t>(), m->logits.as<float>(), false, s);
+    launch_gemv(m->lm_head, m->aq.as<int8_t>(), m->asc.as<uint16_t>(), m->logits.as<float>(), false,
+                after_prefill ? GemvOrder::LmHeadAfterPrefill : GemvOrder::LmHead, s);
     launch_argmax(m->logits.as<float>(), m->cfg.vocab, m->d_next(), m->argmax_ws.p, s);
 }
 
 void enqueue_decode_step(forge_hip_model* m) {
     launch_embedding(m->embed.as<float>(), m->d_token(), 1, m->H, m->x.as<float>(), m->stream);
     for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_layer(m, l, true, 1, 0);
-    enqueue_head(m, m->x.as<float>());
+    enqueue_head(m, m->x.as<float>(), false);
     launch_advance(m->d_pos(), m->d_token(), m->d_next(), m->stream);
 }
 
@@ -341,7 +356,7 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint
     m->h_stage[2] = (uint32_t)m->pos;
     FH_HIP(hipMemcpyAsync(m->d_pos(), &m->h_stage[2], 4, hipMemcpyHostToDevice, s));
     if (logits_host) {
-        enqueue_head(m, m->px.as<float>() + (size_t)(last_rows - 1) * m->H);
+        enqueue_head(m, m->px.as<float>() + (size_t)(last_rows - 1) * m->H, true);
         FH_HIP(hipGetLastError());
         FH_HIP(hipMemcpyAsync(logits_host, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, s));
     }

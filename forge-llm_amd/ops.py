@@ -121,7 +121,16 @@ def matmul_vec_q(w: QWeight, x):
     return y
 
 
-def matmul_mat_q(w: QWeight, x):
+def expf_host(x) -> np.ndarray:
+    """exp as the GPU kernels evaluate it (host twin; bit-identical to the C library's expf)."""
+    from . import check, lib
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty_like(x)
+    check(lib().forge_hip_expf_host(x.ctypes.data_as(C.c_void_p), x.size, out.ctypes.data_as(C.c_void_p)))
+    return out
+
+
+def matmul_mat_q(w: QWeight, x, flags=0):
     """matmul_mat_q8_0_KxN / matmul_mat_q4_0_KxN: x f32 [M][K] -> f32 [M][N]."""
     from . import check, lib
     torch = _torch()
@@ -130,7 +139,7 @@ def matmul_mat_q(w: QWeight, x):
         raise ValueError("input must be [M][K]")
     M = x.shape[0]
     y = torch.empty((M, w.N), dtype=torch.float32, device=x.device)
-    check(lib().forge_hip_gemm_q(w._h, _ptr(x), M, _ptr(y), _stream()))
+    check(lib().forge_hip_gemm_q(w._h, _ptr(x), M, _ptr(y), flags, _stream()))
     return y
 
 
@@ -178,7 +187,7 @@ def rope_kv_store(q, k, v, k_cache, v_cache, base_pos, heads, kv_heads, head_dim
                                         kv_heads, head_dim, theta, _stream()))
 
 
-def attention_flash_batch(q, k_cache, v_cache, base_pos, heads, kv_heads, head_dim):
+def attention_flash_batch(q, k_cache, v_cache, base_pos, heads, kv_heads, head_dim, flags=0):
     """attention_flash_batch over an fp16 cache: q f32 [M][heads*hd] -> f32 [M][heads*hd]."""
     from . import check, lib
     torch = _torch()
@@ -189,11 +198,11 @@ def attention_flash_batch(q, k_cache, v_cache, base_pos, heads, kv_heads, head_d
         raise ValueError("cache holds fewer than base_pos + M rows")
     out = torch.empty_like(q)
     check(lib().forge_hip_attn_prefill_f16kv(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), M, base_pos, heads,
-                                             kv_heads, head_dim, _stream()))
+                                             kv_heads, head_dim, flags, _stream()))
     return out
 
 
-def attention_flash(q, k_cache, v_cache, seq_len, heads, kv_heads, head_dim):
+def attention_flash(q, k_cache, v_cache, seq_len, heads, kv_heads, head_dim, flags=0):
     """attention_flash over an fp16 cache: one query f32 [heads*hd] against seq_len rows."""
     from . import check, lib
     torch = _torch()
@@ -203,7 +212,7 @@ def attention_flash(q, k_cache, v_cache, seq_len, heads, kv_heads, head_dim):
         raise ValueError("cache holds fewer than seq_len rows")
     out = torch.empty_like(q)
     check(lib().forge_hip_attn_decode_f16kv(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), seq_len, heads, kv_heads,
-                                            head_dim, _stream()))
+                                            head_dim, flags, _stream()))
     return out
 
 

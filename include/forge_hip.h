@@ -34,6 +34,14 @@ extern "C" {
 #define FORGE_HIP_ERR_NO_DEVICE (-4)
 #define FORGE_HIP_ERR_HIP (-5)       /* a HIP runtime call failed */
 
+/* Bit for config.flags and for the `flags` argument of the op-level calls.
+ * EXACT: every f32 operation follows the CPU path's own order (sequential block combine without
+ * fused multiply-add, 64-key attention blocks with sequential sums, the C library's expf), so
+ * results are bit-identical to the CPU path and greedy tokens are identical.  Without it the
+ * prefill GEMM fuses its per-block multiply-add and attention runs on the MFMA / split-sequence
+ * kernels: same integer block sums, f32 results within rel 1e-3 / abs 1e-3, much faster. */
+#define FORGE_HIP_FLAG_EXACT 1u
+
 #define FORGE_HIP_Q4_0 2u /* GGML type ids, crates/forgellm-frontend/src/gguf.rs:207-258 */
 #define FORGE_HIP_Q8_0 8u
 
@@ -44,7 +52,7 @@ typedef struct forge_hip_config {
     float rms_eps, rope_theta;
     uint32_t wdtype;        /* projection weights: FORGE_HIP_Q8_0 or FORGE_HIP_Q4_0 */
     uint32_t lm_head_dtype; /* same coding */
-    uint32_t flags;         /* reserved, 0 */
+    uint32_t flags;         /* 0 or FORGE_HIP_FLAG_EXACT */
 } forge_hip_config;
 
 typedef struct forge_hip_model forge_hip_model;
@@ -95,6 +103,10 @@ float forge_hip_f16_to_f32(uint16_t bits);
 uint16_t forge_hip_f32_to_f16(float x);
 /* quantize_f32_to_q8_0 / _q4_0 (weight_loader.rs:1454-1544): n floats -> ceil(n/32) blocks. */
 int32_t forge_hip_quantize_f32(uint32_t wdtype, const float* data_host, uint64_t n, uint8_t* out_host);
+/* f32::exp as the GPU kernels evaluate it (silu_mul emit.rs:384, softmax emit.rs:688-699): the
+ * table-driven binary64 algorithm of the C library's expf, so that CPU and GPU agree bit for bit.
+ * This is its host twin, exported so that it can be checked against the C library. */
+int32_t forge_hip_expf_host(const float* x_host, uint64_t n, float* out_host);
 /* dequant_q8_0 / dequant_q4_0 (weight_loader.rs:860-926). */
 int32_t forge_hip_dequant(uint32_t wdtype, const uint8_t* data_host, uint64_t n, float* out_host);
 
@@ -117,7 +129,8 @@ int32_t forge_hip_gemv_q(const forge_hip_qweight* w, const float* x_dev, float* 
 
 /* matmul_mat_q8_0_KxN / matmul_mat_q4_0_KxN (emit.rs:2108-2302, 3667-3817):
  * y[M][N] = x[M][K] W^T, row-major. */
-int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, void* stream);
+int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, uint32_t flags,
+                         void* stream);
 
 /* The int32 block sums the two calls above combine: out_dev int32 [M][N][K/32]
  * (dot_q8_0_q8_0 / dot_q4_0_q8_0 `vaddvq_s32(acc)`, emit.rs:1543-1553, 2522-2552).
@@ -144,13 +157,13 @@ int32_t forge_hip_rope_kv_store(float* q_dev, float* k_dev, const float* v_dev, 
  * out_dev f32 [M][heads*hd]. */
 int32_t forge_hip_attn_prefill_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                      float* out_dev, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
-                                     uint32_t head_dim, void* stream);
+                                     uint32_t head_dim, uint32_t flags, void* stream);
 
 /* attention_flash (emit.rs:656-715) over an fp16 cache: one query against seq_len rows.
  * q_dev f32 [heads*hd], out_dev f32 [heads*hd]. */
 int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                     float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
-                                    uint32_t head_dim, void* stream);
+                                    uint32_t head_dim, uint32_t flags, void* stream);
 
 /* argmax (project.rs:501-503): index of the LAST maximum of n floats -> *out_dev (uint32). */
 int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void* stream);

@@ -807,6 +807,8 @@ void fo_rope_table(int64_t n_pos, int head_dim, float theta, float* cos_out, flo
 }
 float fo_quantize_kv(const float* v, int64_t n, int8_t* out) { return quantize_kv(v, n, out); }
 uint32_t fo_argmax(const float* v, int64_t n) { return argmax_last(v, n); }
+// The C library's expf (what Rust's f32::exp calls on Linux), element-wise.
+void fo_expf_array(const float* x, int64_t n, float* out) { for (int64_t i = 0; i < n; i++) out[i] = expf(x[i]); }
 
 // Attention over an externally supplied cache.  kvmode 0: k,v are int8 with ks/vs scales;
 // kvmode 1: k,v are fp16 bit patterns.  kind 0 standard, 1 flash, 2 flash_batch (then q is

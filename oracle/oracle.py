@@ -76,6 +76,7 @@ def lib():
     L.fo_rope_table.argtypes = [i64, i32, f32, vp, vp]
     L.fo_quantize_kv.restype = f32
     L.fo_quantize_kv.argtypes = [vp, i64, vp]
+    L.fo_expf_array.argtypes = [vp, i64, vp]
     L.fo_argmax.restype = C.c_uint32
     L.fo_argmax.argtypes = [vp, i64]
     L.fo_attention.argtypes = [i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32]
@@ -210,6 +211,14 @@ def quantize_kv(v):
     out = np.empty(v.size, np.int8)
     scale = lib().fo_quantize_kv(_p(v), v.size, _p(out))
     return out, float(scale)
+
+
+def expf(x):
+    """The C library's expf, element-wise."""
+    x = _f32(x)
+    out = np.empty_like(x)
+    lib().fo_expf_array(_p(x), x.size, _p(out))
+    return out
 
 
 def argmax(v):

@@ -1,5 +1,11 @@
 """GPU parity of the model API (create / forward / forward_prefill_batch / reset) against the
-oracle model with variant-A arithmetic and an fp16 KV cache, on seeded synthetic models."""
+oracle model (aarch64 arithmetic, fp16 KV cache) on seeded synthetic models.
+
+With FLAG_EXACT every f32 operation is in the CPU path's order, so logits are compared bit for
+bit and greedy tokens must be identical.  Without it (MFMA attention, split-sequence decode
+attention, fused GEMM combine) each kernel is within 1e-3 of the oracle on identical inputs
+(tests/test_gpu_ops.py), but int8 activation quantisation amplifies such differences from layer
+to layer on random-init weights, so end-to-end the fast mode is only held to a loose bound."""
 import numpy as np
 import pytest
 
@@ -7,12 +13,19 @@ pytestmark = pytest.mark.gpu
 
 Q8, Q4 = 8, 2
 A, KV_F16 = 0, 1
+EXACT = 1
 
 
 def close(got, want, rtol=1e-3, atol=1e-3):
     got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
     bad = np.abs(got - want) > atol + rtol * np.abs(want)
     assert not bad.any(), f"{bad.sum()} of {bad.size} outside tolerance; max abs err {np.max(np.abs(got - want)):.3e}"
+
+
+def same_bits(got, want):
+    got, want = np.ascontiguousarray(got, np.float32), np.ascontiguousarray(want, np.float32)
+    diff = got.view(np.uint32) != want.view(np.uint32)
+    assert not diff.any(), f"{diff.sum()} of {diff.size} differ in bits; max abs err {np.max(np.abs(got - want)):.3e}"
 
 
 def greedy_oracle(oracle, om, prompt, n):
@@ -23,40 +36,61 @@ def greedy_oracle(oracle, om, prompt, n):
     return out
 
 
-@pytest.mark.parametrize("wd", [Q8, Q4])
-def test_tiny_model_logits_and_cache(fh, oracle, torch_gpu, wd):
+def tiny_cfg(fh, wd, flags):
     cfg = fh.synth.tiny(wdtype=wd, max_seq=640, hidden=256, inter=512, layers=2, heads=4, kv_heads=2, head_dim=64, vocab=1000)
+    cfg["flags"] = flags
+    return cfg
+
+
+@pytest.mark.parametrize("wd", [Q8, Q4])
+def test_tiny_model_exact_mode_is_bit_identical(fh, oracle, torch_gpu, wd):
+    cfg = tiny_cfg(fh, wd, EXACT)
     blob = fh.synth.make_weights_blob(cfg, seed=11)
     toks = fh.synth.uniform_ids(12, 40, cfg["vocab"])
     gm = fh.HipModel(cfg, blob)
     om = oracle.Model(cfg, blob, A, KV_F16)
-    # batched prefill: last-token logits and the fp16 cache contents
     gl = gm.forward_prefill(toks)
     ol = om.prefill_batched(toks)
     assert gm.pos == om.pos == 40
-    close(gl, ol)
+    same_bits(gl, ol)
     for layer in range(cfg["layers"]):
         for which in (0, 1):
-            got = oracle.f16_to_f32(gm.read_kv(layer, which))
-            close(got, om.read_kv(layer, which), rtol=2e-3, atol=2e-3)
-    # decode steps continue from the cache
-    for t in (3, 999, 0):
-        close(gm.forward(t), om.forward(t))
+            same_bits(oracle.f16_to_f32(gm.read_kv(layer, which)), om.read_kv(layer, which))
+    for t in (3, 999, 0):                                   # decode steps continue from the cache
+        same_bits(gm.forward(t), om.forward(t))
     assert gm.pos == om.pos == 43
-    # per-token path from scratch equals the batched path (the reference's consistency claim)
-    gm.reset()
+    # per-token path from scratch (the reference takes it for prompts under 8 tokens)
+    gm.reset(); om.reset()
     assert gm.pos == 0
-    for t in toks:
-        last = gm.forward(int(t))
-    close(last, gl, rtol=1e-3, atol=1e-3)
-    # reset reproduces
+    for t in toks[:7]:
+        same_bits(gm.forward(int(t)), om.forward(int(t)))
     gm.reset()
-    again = gm.forward_prefill(toks)
-    assert np.array_equal(again, gl)
+    same_bits(gm.forward_prefill(toks), gl)                 # reset reproduces
+    gm.close()
+
+
+@pytest.mark.parametrize("wd", [Q8, Q4])
+def test_tiny_model_fast_mode(fh, oracle, torch_gpu, wd):
+    cfg = tiny_cfg(fh, wd, 0)
+    blob = fh.synth.make_weights_blob(cfg, seed=11)
+    toks = fh.synth.uniform_ids(12, 40, cfg["vocab"])
+    gm = fh.HipModel(cfg, blob)
+    om = oracle.Model(cfg, blob, A, KV_F16)
+    gl = gm.forward_prefill(toks)
+    ol = om.prefill_batched(toks)
+    # layer 0's K/V depend only on embedding -> rms_norm -> GEMM -> rope: within tolerance
+    for which in (0, 1):
+        close(oracle.f16_to_f32(gm.read_kv(0, which)), om.read_kv(0, which), rtol=2e-3, atol=2e-3)
+    # end to end: loose (quantisation amplifies the 1e-3 differences of the MFMA attention)
+    assert np.max(np.abs(gl - ol)) < 0.1 * max(1.0, float(np.std(ol)) * 4)
+    assert np.corrcoef(gl, ol)[0, 1] > 0.995
     # Metal-style signature: fill the cache without logits, then forward(last)
     gm.reset()
     gm.forward_prefill_batch(toks[:-1])
-    close(gm.forward(int(toks[-1])), gl)
+    last = gm.forward(int(toks[-1]))
+    assert np.corrcoef(last, gl)[0, 1] > 0.995
+    gm.reset()
+    assert np.array_equal(gm.forward_prefill(toks), gl)     # deterministic
     gm.close()
 
 
@@ -88,11 +122,14 @@ def test_error_codes_on_device(fh, torch_gpu):
         gm.forward(cfg["vocab"])
     assert e.value.code == fh.ERR_POSITION
     gm.close()
+    with pytest.raises(fh.ForgeHipError) as e:          # exact mode follows the flash kernels only
+        fh.HipModel(dict(cfg, flags=EXACT), blob)
+    assert e.value.code == fh.ERR_INVALID
 
 
 def test_prefill_in_chunks_equals_one_shot(fh, torch_gpu):
     """Prefilling 90 tokens as 50 + 40 (second call starts at base_pos 50) equals one call of 90."""
-    cfg = fh.synth.tiny(wdtype=Q8, max_seq=640)
+    cfg = tiny_cfg(fh, Q8, EXACT)
     blob = fh.synth.make_weights_blob(cfg, seed=5)
     toks = fh.synth.uniform_ids(6, 90, cfg["vocab"])
     gm = fh.HipModel(cfg, blob)
@@ -100,13 +137,30 @@ def test_prefill_in_chunks_equals_one_shot(fh, torch_gpu):
     gm.reset()
     gm.forward_prefill_batch(toks[:50])
     two = gm.forward_prefill(toks[50:])
-    close(two, one, rtol=1e-4, atol=1e-4)
+    same_bits(two, one)
     gm.close()
+
+
+def test_graph_replay_matches_eager(fh, torch_gpu, monkeypatch):
+    """The captured decode step, replayed many times with host work in between, equals eager launches."""
+    cfg = tiny_cfg(fh, Q8, 0)
+    blob = fh.synth.make_weights_blob(cfg, seed=8)
+    toks = fh.synth.uniform_ids(9, 12, cfg["vocab"])
+    monkeypatch.setenv("FORGE_HIP_GRAPH", "0")
+    eager = fh.HipModel(cfg, blob)
+    monkeypatch.setenv("FORGE_HIP_GRAPH", "1")
+    graph = fh.HipModel(cfg, blob)
+    for t in toks:
+        a = eager.forward(int(t))
+        b = graph.forward(int(t))
+        assert np.array_equal(a, b)
+    eager.close(); graph.close()
 
 
 def test_smollm2_135m_greedy_64_tokens_identical(fh, oracle, torch_gpu):
     """SmolLM2-135M-shape Q8_0 model, random-init: 32-token prompt, 64 greedy tokens, identical ids."""
     cfg = fh.synth.smollm2_135m(Q8, max_seq=1024)
+    cfg["flags"] = EXACT
     blob = fh.synth.make_weights_blob(cfg, seed=135)
     prompt = fh.synth.uniform_ids(136, 32, cfg["vocab"])
     gm = fh.HipModel(cfg, blob)
@@ -114,4 +168,5 @@ def test_smollm2_135m_greedy_64_tokens_identical(fh, oracle, torch_gpu):
     got = gm.generate_greedy(prompt, 64)
     want = greedy_oracle(oracle, om, prompt, 64)
     assert got == want
+    same_bits(gm.forward(got[-1]), om.forward(want[-1]))    # and the 65th step's logits, bit for bit
     gm.close()
