@@ -1,0 +1,204 @@
+"""Benchmark: Llama-3.2-1B-shape Q8_0 model (random-init from a seed) on ONE MI355X.
+
+A "step" is one greedy decode token (forward + on-device argmax + 4-byte read-back).  The
+script prefills a 2502-token prompt (timed: prefill tok/s), then runs W warm-up and K timed
+decode steps at that context, and prints ONE JSON line.  Weights, KV cache and activations are
+resident in HBM when the timed regions start.
+
+roofline: the decode step's dominant kernel, the quantised GEMV.  `achieved` = algorithmic bytes
+(GGUF block bytes of every matrix + its f32 input and output vectors) of the GEMV launches of one
+token / their summed device time, measured with HIP events around every launch by the library's
+forward_profile on the model's own stream.  `peak` = 8 TB/s (MI355X HBM3E).
+
+cpu_baseline: the CPU restatement of the reference's generated kernels (oracle/), in the arithmetic
+the reference runs on an x86 host (f32 activations x dequantised weights, int8 KV), per-token decode,
+timed on this host's cores on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+from __graft_entry__ import load_package  # noqa: E402
+
+HBM_PEAK_GBS = 8000.0
+MFMA_I8_PEAK_TOPS = 5000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+PROMPT_TOKENS = 2502
+
+
+def gemv_launch_bytes(fh, cfg):
+    """Algorithmic bytes of the GEMV launches of one decode step, per stage."""
+    H, I = cfg["hidden"], cfg["inter"]
+    QKS, KV = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"]
+    wt, g = cfg["wdtype"], fh.synth.gemv_bytes
+    L = cfg["layers"]
+    return {
+        "qkv_matmul": L * (g(QKS, H, wt) + 2 * g(KV, H, wt)),
+        "o_matmul": L * g(H, QKS, wt),
+        "gate_up_matmul": L * 2 * g(I, H, wt),
+        "down_matmul": L * g(H, I, wt),
+        "lm_head_matmul": g(cfg["vocab"], H, cfg["lm_head_dtype"]),
+    }
+
+
+def prefill_flops(cfg, m):
+    H, I = cfg["hidden"], cfg["inter"]
+    QKS, KV = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"]
+    gemm = 2 * m * cfg["layers"] * (H * QKS + 2 * H * KV + QKS * H + 2 * H * I + I * H)
+    attn = cfg["layers"] * 4 * cfg["head_dim"] * cfg["heads"] * m * (m + 1) // 2
+    return gemm, attn
+
+
+def cpu_baseline(fh, cfg, blob, prompt, budget_s=20.0):
+    from oracle import oracle
+    om = oracle.Model(cfg, blob, oracle.VARIANT_B, oracle.KV_INT8)
+    threads = oracle.num_threads()
+    ctx = 8
+    for t in prompt[:ctx]:
+        logits = om.forward(int(t))          # per-token path fills a short cache
+    tok = oracle.argmax(logits)
+    t0 = time.perf_counter()
+    n = 0
+    while n < 32 and (time.perf_counter() - t0 < budget_s or n < 2):
+        tok = oracle.argmax(om.forward(tok))
+        n += 1
+    dt = time.perf_counter() - t0
+    om.close()
+    return {"value": n / dt, "unit": "tok/s", "cores": threads, "kind": "port",
+            "sample": f"{n} greedy decode tokens after an {ctx}-token prompt, same model and weights; f32 x dequantised-weight "
+                      f"arithmetic of the reference's x86 build, int8 KV, OpenMP over rows with {threads} threads"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--seed", type=int, default=1)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU; --gpus must be 1 (no multi-GPU path exists to run)", file=sys.stderr)
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    fh = load_package()
+    fh.require_gpu()
+    cfg = fh.synth.llama32_1b(fh.Q8_0, max_seq=4096)
+    t0 = time.perf_counter()
+    blob = fh.synth.make_weights_blob(cfg, seed=args.seed, threads=16)
+    t_gen = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    model = fh.HipModel(cfg, blob)
+    t_load = time.perf_counter() - t0
+    prompt = fh.synth.uniform_ids(args.seed + 1, PROMPT_TOKENS, cfg["vocab"])
+
+    # ---- prefill: one warm-up pass, then timed
+    model.forward_prefill_batch(prompt)
+    model.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    logits = model.forward_prefill(prompt)
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    tok = fh.ops.argmax_host(logits)
+
+    # ---- decode at context ~2502: W warm-up steps, K timed steps
+    for _ in range(args.warmup):
+        tok = model.forward_greedy(tok)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        tok = model.forward_greedy(tok)
+    torch.cuda.synchronize()
+    t_decode = time.perf_counter() - t0
+
+    # ---- per-kernel device time of the decode step (events around every launch)
+    prof_steps = 8
+    stage_ms, stage_n = {}, {}
+    for _ in range(prof_steps):
+        p = model.forward_profile(tok)
+        for s, (ms, n) in p.items():
+            stage_ms[s] = stage_ms.get(s, 0.0) + ms
+            stage_n[s] = stage_n.get(s, 0) + n
+    gbytes = gemv_launch_bytes(fh, cfg)
+    gemv_ms = sum(stage_ms[s] for s in gbytes) / prof_steps
+    gemv_launches = sum(stage_n[s] for s in gbytes) // prof_steps
+    gemv_bytes_total = sum(gbytes.values())
+    achieved = gemv_bytes_total / (gemv_ms * 1e-3) / 1e9
+    per_stage = {s: {"GB/s": round(gbytes[s] / (stage_ms[s] / prof_steps * 1e-3) / 1e9, 1),
+                     "us_per_launch": round(stage_ms[s] / stage_n[s] * 1e3, 2)} for s in gbytes}
+
+    # ---- prefill kernels (GEMM / attention) from prefill_profile
+    model.reset()
+    pp = model.prefill_profile(prompt)
+    gemm_flops, attn_flops = prefill_flops(cfg, PROMPT_TOKENS)
+    gemm_ms = sum(pp[s][0] for s in ("qkv_matmul", "o_matmul", "gate_up_matmul", "down_matmul"))
+    attn_ms = pp["attention"][0]
+
+    # ---- short-context decode for reference (64-token style run of the reference's decode benchmark)
+    model.reset()
+    tok2 = fh.ops.argmax_host(model.forward_prefill(prompt[:32]))
+    for _ in range(4):
+        tok2 = model.forward_greedy(tok2)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        tok2 = model.forward_greedy(tok2)
+    torch.cuda.synchronize()
+    t_decode_short = time.perf_counter() - t0
+    model.close()
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "gemv_hbm_traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get("bytes_per_launch")
+
+    out = {
+        "metric": "decode tok/s (Llama-3.2-1B Q8_0, 1 GPU)",
+        "value": args.steps / t_decode,
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": t_decode / args.steps * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 block dots (exact int32) + f32 combine; fp16 KV",
+        "data": "synthetic",
+        "config": {"workload": f"Llama-3.2-1B shape, Q8_0, random-init seed {args.seed}: {PROMPT_TOKENS}-token prompt, "
+                               f"then greedy decode at that context", "prompt_tokens": PROMPT_TOKENS,
+                   "decode_context": PROMPT_TOKENS + args.warmup, "mode": "fast (MFMA prefill, split-seq decode attention)"},
+        "prefill_tok_per_s": PROMPT_TOKENS / t_prefill,
+        "prefill_ms": t_prefill * 1e3,
+        "decode_tok_per_s_short_context": args.steps / t_decode_short,
+        "decode_weight_stream_GBps_end_to_end": fh.synth.decode_weight_bytes(cfg) * args.steps / t_decode / 1e9,
+        "roofline": {"kernel": "gemv_kernel (quantised GEMV, all launches of one decode step)", "bound": "hbm",
+                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                     "traffic": traffic, "bytes_per_launch": gemv_bytes_total / gemv_launches,
+                     "us_per_launch": gemv_ms * 1e3 / gemv_launches, "launches_per_step": gemv_launches,
+                     "per_stage": per_stage},
+        "prefill_rooflines": {
+            "gemm": {"bound": "mfma", "achieved": gemm_flops / (gemm_ms * 1e-3) / 1e12, "peak": MFMA_I8_PEAK_TOPS,
+                     "unit": "TOP/s (int8)", "frac": gemm_flops / (gemm_ms * 1e-3) / 1e12 / MFMA_I8_PEAK_TOPS, "ms": gemm_ms},
+            "attention": {"bound": "mfma", "achieved": attn_flops / (attn_ms * 1e-3) / 1e12, "peak": MFMA_F16_PEAK_TFLOPS,
+                          "unit": "TFLOP/s (fp16)", "frac": attn_flops / (attn_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
+                          "ms": attn_ms},
+        },
+        "decode_stage_us": {s: round(stage_ms[s] / prof_steps * 1e3, 1) for s in stage_ms},
+        "setup_s": {"generate_weights": round(t_gen, 1), "upload_and_repack": round(t_load, 1)},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(fh, cfg, blob, prompt)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -145,18 +145,28 @@ template <int HD>
 __global__ void attn_decode_combine_kernel(const float* __restrict__ ws, uint32_t nsplit, float* __restrict__ out,
                                            int8_t* __restrict__ oq, uint16_t* __restrict__ osc) {
     constexpr int REC = HD + 2;
+    __shared__ float wgt_s[DECODE_SPLITS];
+    __shared__ float den_s;
     const uint32_t h = blockIdx.x, d = threadIdx.x;
     const float* base = ws + (size_t)h * nsplit * REC;
-    float mm = -INFINITY;
-    for (uint32_t s = 0; s < nsplit; s++) mm = fmaxf(mm, base[s * REC + HD]);
-    float num = 0.f, den = 0.f;
-    for (uint32_t s = 0; s < nsplit; s++) {
-        const float ms = base[s * REC + HD];
+    // lanes 0..nsplit-1 of the first wave fetch the split maxima and sums in parallel
+    if (d < 64) {
+        const float ms = d < nsplit ? base[d * REC + HD] : -INFINITY;
+        const float ls = d < nsplit ? base[d * REC + HD + 1] : 0.f;
+        const float mm = wave_max(ms);
         const float wgt = (ms == -INFINITY) ? 0.f : __expf(ms - mm);
-        num += wgt * base[s * REC + d];
-        den += wgt * base[s * REC + HD + 1];
+        const float den = wave_sum(wgt * ls);
+        if (d < nsplit) wgt_s[d] = wgt;
+        if (d == 0) den_s = den;
     }
-    const float o = num * (1.0f / den);
+    __syncthreads();
+    float part[DECODE_SPLITS];
+#pragma unroll
+    for (uint32_t s = 0; s < DECODE_SPLITS; s++) part[s] = s < nsplit ? base[s * REC + d] : 0.f;   // all loads in flight
+    float num = 0.f;
+#pragma unroll
+    for (uint32_t s = 0; s < DECODE_SPLITS; s++) num = fmaf(wgt_s[s < nsplit ? s : 0], part[s], num);
+    const float o = num * (1.0f / den_s);
     if (out) out[(size_t)h * HD + d] = o;
     if (oq) {
         float amax = fabsf(o);

@@ -47,7 +47,15 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
     if (tid < 16) {
         float s = 0.f;
         const uint32_t chunks = H / 16;
-        for (uint32_t c = 0; c < chunks; c++) { const float v = xs[c * 16 + tid]; s = fmaf(v, v, s); }
+        uint32_t c = 0;
+        for (; c + 8 <= chunks; c += 8) {      // eight LDS reads in flight, then the dependent FMAs
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = xs[(c + i) * 16 + tid];
+#pragma unroll
+            for (int i = 0; i < 8; i++) s = fmaf(v[i], v[i], s);
+        }
+        for (; c < chunks; c++) { const float v = xs[c * 16 + tid]; s = fmaf(v, v, s); }
         part[tid] = s;
     }
     __syncthreads();

@@ -48,7 +48,15 @@ struct GemvArgs {
 __device__ __forceinline__ float ordered_sum(const float* p, uint32_t nblk, bool dot1) {
     if (!dot1) {
         float r = 0.f;
-        for (uint32_t b = 0; b < nblk; b++) r = r + p[b];
+        uint32_t b = 0;
+        for (; b + 8 <= nblk; b += 8) {          // eight LDS reads in flight, then the dependent adds
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = p[b + i];
+#pragma unroll
+            for (int i = 0; i < 8; i++) r = r + v[i];
+        }
+        for (; b < nblk; b++) r = r + p[b];
         return r;
     }
     float fa0 = 0.f, fa1 = 0.f, fa2 = 0.f, fa3 = 0.f;
@@ -172,18 +180,20 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
 
 namespace {
 
-uint32_t rows_per_group(uint32_t nblk) {
-    if (nblk <= 32) return 64;
-    if (nblk <= 64) return 32;
-    if (nblk <= 128) return 16;
-    if (nblk <= 256) return 8;
-    return 4;
+// Rows per ordered-sum group.  One lane per row walks the block products in order, so a group costs
+// about the same time whatever its size: large groups amortise it (lm_head), small groups keep every
+// CU busy on the small matrices.  Bounded above by the LDS the products need.
+uint32_t rows_per_group(uint32_t nblk, uint32_t N, uint32_t rw) {
+    uint32_t cap = nblk <= 32 ? 64 : nblk <= 64 ? 32 : nblk <= 128 ? 16 : nblk <= 256 ? 8 : 4;
+    uint32_t want = N / 4096 / rw * rw;          // aim for >= 4096 groups, i.e. >= 4 waves per SIMD
+    if (want < rw) want = rw;
+    return want < cap ? want : cap;
 }
 
 template <bool Q4, int NCH, int RW, bool ISUMS>
 void launch_one(GemvArgs a, hipStream_t s) {
     const uint32_t nblk = a.K / 32;
-    a.rc = rows_per_group(nblk);
+    a.rc = rows_per_group(nblk, a.N, RW);
     const uint32_t ngroups = (a.N + a.rc - 1) / a.rc;
     uint32_t grid = (ngroups + 3) / 4;
     if (grid > 256 * 8) grid = 256 * 8;

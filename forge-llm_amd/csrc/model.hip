@@ -66,6 +66,11 @@ struct forge_hip_model {
     int64_t pos = 0;
     bool use_graph = true;
     hipGraphExec_t decode_graph = nullptr;
+    // forward_profile: while `prof_on`, every launch is bracketed by a pair of events tagged with its stage
+    bool prof_on = false;
+    std::vector<hipEvent_t> prof_ev;
+    std::vector<int> prof_stage;
+    size_t prof_used = 0;
 
     uint32_t* d_pos() const { return state.as<uint32_t>(); }
     uint32_t* d_token() const { return state.as<uint32_t>() + 1; }
@@ -75,6 +80,7 @@ struct forge_hip_model {
 
     ~forge_hip_model() {
         if (decode_graph) (void)hipGraphExecDestroy(decode_graph);
+        for (hipEvent_t e : prof_ev) (void)hipEventDestroy(e);
         for (auto& L : layers) { qweight_free(&L.qkv); qweight_free(&L.o); qweight_free(&L.gate_up); qweight_free(&L.down); }
         qweight_free(&lm_head);
         if (h_stage) (void)hipHostFree(h_stage);
@@ -83,6 +89,45 @@ struct forge_hip_model {
 };
 
 namespace {
+
+// Stage ids of forward_profile / prefill_profile (the order of FORGE_HIP_STAGE_* in forge_hip.h).
+enum Stage { ST_EMBED = 0, ST_RMSNORM, ST_QKV, ST_ROPE, ST_ATTN, ST_QUANT, ST_O, ST_GATE_UP, ST_SILU, ST_DOWN, ST_LM_HEAD,
+             ST_ARGMAX, ST_COUNT };
+static_assert(ST_COUNT == FORGE_HIP_NUM_STAGES, "stage table out of step with forge_hip.h");
+
+// Brackets the launches of one scope with two events while the model is profiling.
+struct StageMark {
+    forge_hip_model* m;
+    StageMark(forge_hip_model* model, int stage) : m(model) {
+        if (!m->prof_on) return;
+        if (m->prof_used + 2 > m->prof_ev.size()) {
+            for (int i = 0; i < 2; i++) {
+                hipEvent_t e = nullptr;
+                if (hipEventCreate(&e) != hipSuccess) { m->prof_on = false; return; }
+                m->prof_ev.push_back(e);
+            }
+        }
+        m->prof_stage.push_back(stage);
+        (void)hipEventRecord(m->prof_ev[m->prof_used], m->stream);
+    }
+    ~StageMark() {
+        if (!m->prof_on) return;
+        (void)hipEventRecord(m->prof_ev[m->prof_used + 1], m->stream);
+        m->prof_used += 2;
+    }
+};
+
+// Sum the bracketed times per stage (milliseconds) after the stream has drained.
+int32_t collect_profile(forge_hip_model* m, float* stage_ms, uint32_t* stage_launches) {
+    for (int i = 0; i < ST_COUNT; i++) { stage_ms[i] = 0.f; if (stage_launches) stage_launches[i] = 0; }
+    for (size_t i = 0; i * 2 < m->prof_used; i++) {
+        float ms = 0.f;
+        FH_HIP(hipEventElapsedTime(&ms, m->prof_ev[2 * i], m->prof_ev[2 * i + 1]));
+        stage_ms[m->prof_stage[i]] += ms;
+        if (stage_launches) stage_launches[m->prof_stage[i]] += 1;
+    }
+    return FORGE_HIP_OK;
+}
 
 size_t wsize(uint32_t dtype, uint64_t n, uint64_t k) { return (size_t)(n * (k / 32) * (dtype == FORGE_HIP_Q8_0 ? 34 : 18)); }
 
@@ -119,50 +164,75 @@ void enqueue_layer(forge_hip_model* m, uint32_t l, bool decode, uint32_t M, uint
 
     const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
     const GemvOrder mv = GemvOrder::MatmulVec;
-    launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s);
-    if (decode) launch_gemv(L.qkv, aq, asc, qkv, false, mv, s);
-    else launch_gemm(L.qkv, aq, asc, M, qkv, QKV, false, exact, nullptr, s);
-    launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos,
-                         decode ? m->d_pos() : nullptr, c.heads, c.kv_heads, c.head_dim, m->cos_t.as<float>(),
-                         m->sin_t.as<float>(), s);
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
+    {
+        StageMark t(m, ST_QKV);
+        if (decode) launch_gemv(L.qkv, aq, asc, qkv, false, mv, s);
+        else launch_gemm(L.qkv, aq, asc, M, qkv, QKV, false, exact, nullptr, s);
+    }
+    {
+        StageMark t(m, ST_ROPE);
+        launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos,
+                             decode ? m->d_pos() : nullptr, c.heads, c.kv_heads, c.head_dim, m->cos_t.as<float>(),
+                             m->sin_t.as<float>(), s);
+    }
     if (decode) {
-        if (exact)
-            launch_attn_exact(false, qkv, QKV, m->kc(l), m->vc(l), nullptr, QKS, aq, asc, 1, 0, m->d_pos(), c.heads,
-                              c.kv_heads, c.head_dim, s);
-        else
-            launch_attn_decode(qkv, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads,
-                               c.head_dim, m->attn_ws.p, s);
-        launch_gemv(L.o, aq, asc, x, true, mv, s);
+        {
+            StageMark t(m, ST_ATTN);
+            if (exact)
+                launch_attn_exact(false, qkv, QKV, m->kc(l), m->vc(l), nullptr, QKS, aq, asc, 1, 0, m->d_pos(), c.heads,
+                                  c.kv_heads, c.head_dim, s);
+            else
+                launch_attn_decode(qkv, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads,
+                                   c.head_dim, m->attn_ws.p, s);
+        }
+        { StageMark t(m, ST_O); launch_gemv(L.o, aq, asc, x, true, mv, s); }
     } else {
         float* attn = m->pattn.as<float>();
-        if (exact)
-            launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr,
-                              c.heads, c.kv_heads, c.head_dim, s);
-        else
-            launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, s);
-        launch_quantize_act(attn, M, QKS, aq, asc, s);
-        launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s);
+        {
+            StageMark t(m, ST_ATTN);
+            if (exact)
+                launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr,
+                                  c.heads, c.kv_heads, c.head_dim, s);
+            else
+                launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads,
+                                    c.head_dim, s);
+        }
+        { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
+        { StageMark t(m, ST_O); launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s); }
     }
-    launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s);
-    if (decode) launch_gemv(L.gate_up, aq, asc, gu, false, mv, s);
-    else launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s);
-    launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s);
-    if (decode) launch_gemv(L.down, aq, asc, x, true, mv, s);
-    else launch_gemm(L.down, aq, asc, M, x, H, true, exact, nullptr, s);
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
+    {
+        StageMark t(m, ST_GATE_UP);
+        if (decode) launch_gemv(L.gate_up, aq, asc, gu, false, mv, s);
+        else launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s);
+    }
+    { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s); }
+    {
+        StageMark t(m, ST_DOWN);
+        if (decode) launch_gemv(L.down, aq, asc, x, true, mv, s);
+        else launch_gemm(L.down, aq, asc, M, x, H, true, exact, nullptr, s);
+    }
 }
 
 // Final norm of one row + lm_head GEMV + argmax.
 void enqueue_head(forge_hip_model* m, const float* xrow, bool after_prefill) {
     hipStream_t s = m->stream;
-    launch_rmsnorm(xrow, m->final_norm.as<float>(), m->cfg.rms_eps, 1, m->H, nullptr, m->aq.as<int8_t>(),
-                   m->asc.as<uint16_t>(), s);
-    launch_gemv(m->lm_head, m->aq.as<int8_t>(), m->asc.as<uint16_t>(), m->logits.as<float>(), false,
-                after_prefill ? GemvOrder::LmHeadAfterPrefill : GemvOrder::LmHead, s);
-    launch_argmax(m->logits.as<float>(), m->cfg.vocab, m->d_next(), m->argmax_ws.p, s);
+    {
+        StageMark t(m, ST_RMSNORM);
+        launch_rmsnorm(xrow, m->final_norm.as<float>(), m->cfg.rms_eps, 1, m->H, nullptr, m->aq.as<int8_t>(),
+                       m->asc.as<uint16_t>(), s);
+    }
+    {
+        StageMark t(m, ST_LM_HEAD);
+        launch_gemv(m->lm_head, m->aq.as<int8_t>(), m->asc.as<uint16_t>(), m->logits.as<float>(), false,
+                    after_prefill ? GemvOrder::LmHeadAfterPrefill : GemvOrder::LmHead, s);
+    }
+    { StageMark t(m, ST_ARGMAX); launch_argmax(m->logits.as<float>(), m->cfg.vocab, m->d_next(), m->argmax_ws.p, s); }
 }
 
 void enqueue_decode_step(forge_hip_model* m) {
-    launch_embedding(m->embed.as<float>(), m->d_token(), 1, m->H, m->x.as<float>(), m->stream);
+    { StageMark t(m, ST_EMBED); launch_embedding(m->embed.as<float>(), m->d_token(), 1, m->H, m->x.as<float>(), m->stream); }
     for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_layer(m, l, true, 1, 0);
     enqueue_head(m, m->x.as<float>(), false);
     launch_advance(m->d_pos(), m->d_token(), m->d_next(), m->stream);
@@ -362,6 +432,31 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint
     }
     FH_HIP(hipStreamSynchronize(s));
     return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_forward_profile(forge_hip_model* m, uint32_t token, float* stage_ms, uint32_t* stage_launches) {
+    FH_CHECK(m && stage_ms, "forward_profile: null pointer");
+    if (m->pos >= (int64_t)m->cfg.max_seq) return fail(FORGE_HIP_ERR_POSITION, "KV cache is full (pos == max_seq)");
+    if (token >= m->cfg.vocab) return fail(FORGE_HIP_ERR_POSITION, "token id out of range");
+    m->h_stage[0] = token;
+    FH_HIP(hipMemcpyAsync(m->d_token(), &m->h_stage[0], 4, hipMemcpyHostToDevice, m->stream));
+    m->prof_on = true; m->prof_used = 0; m->prof_stage.clear();
+    enqueue_decode_step(m);            // eager launches, each bracketed by events
+    m->prof_on = false;
+    FH_HIP(hipGetLastError());
+    FH_HIP(hipStreamSynchronize(m->stream));
+    m->pos += 1;
+    return collect_profile(m, stage_ms, stage_launches);
+}
+
+int32_t forge_hip_prefill_profile(forge_hip_model* m, const uint32_t* tokens, uint64_t n, float* stage_ms,
+                                  uint32_t* stage_launches) {
+    FH_CHECK(m && stage_ms, "prefill_profile: null pointer");
+    m->prof_on = true; m->prof_used = 0; m->prof_stage.clear();
+    int32_t rc = forge_hip_prefill_batch(m, tokens, n, nullptr);
+    m->prof_on = false;
+    if (rc) return rc;
+    return collect_profile(m, stage_ms, stage_launches);
 }
 
 int32_t forge_hip_reset(forge_hip_model* m) {

@@ -53,6 +53,24 @@ class HipModel:
                                                       out.ctypes.data_as(C.c_void_p)))
         return out
 
+    # -- MetalModel::forward_profile: per-stage device time of one eager decode step
+    STAGES = ("embedding", "rms_norm", "qkv_matmul", "rope_kv_store", "attention", "quantize_act", "o_matmul",
+              "gate_up_matmul", "silu_mul", "down_matmul", "lm_head_matmul", "argmax")
+
+    def forward_profile(self, token_id: int) -> dict:
+        """{stage: (milliseconds, launches)} for one decode step launched eagerly with events around each kernel."""
+        ms = (C.c_float * len(self.STAGES))()
+        n = (C.c_uint32 * len(self.STAGES))()
+        self._check(self._lib.forge_hip_forward_profile(self._h, int(token_id), ms, n))
+        return {s: (float(ms[i]), int(n[i])) for i, s in enumerate(self.STAGES)}
+
+    def prefill_profile(self, tokens) -> dict:
+        t = np.ascontiguousarray(tokens, dtype=np.uint32)
+        ms = (C.c_float * len(self.STAGES))()
+        n = (C.c_uint32 * len(self.STAGES))()
+        self._check(self._lib.forge_hip_prefill_profile(self._h, t.ctypes.data_as(C.c_void_p), t.size, ms, n))
+        return {s: (float(ms[i]), int(n[i])) for i, s in enumerate(self.STAGES)}
+
     def reset(self) -> None:
         self._check(self._lib.forge_hip_reset(self._h))
 

@@ -89,6 +89,20 @@ int32_t forge_hip_forward_greedy(forge_hip_model* m, uint32_t token, uint32_t* n
  * NULL skips the lm_head (the Metal signature). */
 int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens_host, uint64_t n, float* logits_host);
 
+/* MetalModel::forward_profile (metal:5307-5330: one decode step with a wait per stage, timings
+ * printed).  Here: one decode step launched eagerly with a pair of events around every kernel
+ * launch; stage_ms_host[FORGE_HIP_NUM_STAGES] receives the summed device time per stage in
+ * milliseconds, stage_launches_host (may be NULL) the number of launches.  The position advances
+ * like forward(); no logits are returned.  prefill_profile does the same for a batched prefill. */
+#define FORGE_HIP_NUM_STAGES 12
+#define FORGE_HIP_STAGE_NAMES                                                                                  \
+    "embedding", "rms_norm", "qkv_matmul", "rope_kv_store", "attention", "quantize_act", "o_matmul", "gate_up_matmul", \
+        "silu_mul", "down_matmul", "lm_head_matmul", "argmax"
+int32_t forge_hip_forward_profile(forge_hip_model* m, uint32_t token, float* stage_ms_host,
+                                  uint32_t* stage_launches_host);
+int32_t forge_hip_prefill_profile(forge_hip_model* m, const uint32_t* tokens_host, uint64_t n, float* stage_ms_host,
+                                  uint32_t* stage_launches_host);
+
 /* MetalModel::reset() (metal:5981): position back to 0. */
 int32_t forge_hip_reset(forge_hip_model* m);
 /* Current position (KVCache.len, emit.rs:3960). */
