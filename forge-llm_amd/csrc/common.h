@@ -80,8 +80,9 @@ void launch_embedding(const float* table, const uint32_t* tokens_dev, uint32_t M
                       hipStream_t s);
 // Index of the LAST maximum.  `scratch` needs 2*ARGMAX_BLOCKS uint32/float pairs.
 constexpr uint32_t ARGMAX_BLOCKS = 256;
-void launch_argmax(const float* x, uint32_t n, uint32_t* out, void* scratch, hipStream_t s);
-void launch_advance(uint32_t* pos_dev, uint32_t* token_dev, const uint32_t* next_dev, hipStream_t s);
+// If pos_dev is given, the final stage also advances the decode state: *pos_dev += 1, *token_dev = *out.
+void launch_argmax(const float* x, uint32_t n, uint32_t* out, void* scratch, uint32_t* pos_dev, uint32_t* token_dev,
+                   hipStream_t s);
 
 // gemv.hip — y[n] (=|+=) sum_b f32(isum_b) * (a_s[b]*w_s[n][b]); activations already quantised.
 // `order` selects which rows take the reference's 4-accumulator (dot1) order instead of the sequential one.
@@ -90,6 +91,19 @@ void launch_gemv(const QWeight& w, const int8_t* aq, const uint16_t* as, float* 
                  hipStream_t s);
 void launch_gemv_isums(const QWeight& w, const int8_t* aq, int32_t* out, hipStream_t s);
 bool gemv_k_supported(uint32_t K);
+// Fused decode variants (one launch instead of three): rms_norm + activation quantiser in the prologue.
+bool gemv_norm_fusable(uint32_t K);
+bool gemv_silu_fusable(uint32_t K);
+// y = W * quant(rms_norm(x))
+void launch_gemv_norm(const QWeight& w, const float* x, const float* norm_w, float eps, float* y, GemvOrder order,
+                      hipStream_t s);
+// fused [q;k;v] matrix: q rows -> q_out (rotated), k rows -> K cache (rotated, fp16), v rows -> V cache, at *pos_dev
+void launch_gemv_norm_rope_kv(const QWeight& wqkv, const float* x, const float* norm_w, float eps, float* q_out,
+                              uint16_t* kc, uint16_t* vc, const float* cos_t, const float* sin_t,
+                              const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s);
+// fused [gate;up] matrix: quant(silu(gate)*up) -> (oq, osc)
+void launch_gemv_norm_silu_quant(const QWeight& wgu, const float* x, const float* norm_w, float eps, int8_t* oq,
+                                 uint16_t* osc, hipStream_t s);
 
 // gemm.hip — y[m][n] (=|+=) ...; aq int8 [M][K], as fp16 [M][K/32].  isums (optional) int32 [M][N][K/32].
 // exact: unfused multiply/add per block (bit-identical to the CPU path); otherwise one FMA per block.

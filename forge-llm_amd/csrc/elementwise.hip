@@ -242,32 +242,28 @@ __global__ __launch_bounds__(256) void argmax_stage1(const float* __restrict__ x
     a = arg_block(a, sh);
     if (threadIdx.x == 0) part[blockIdx.x] = a;
 }
+// Final stage; optionally also advances the decode state (pos += 1, token = winner) so that the
+// step needs no separate launch for it.
 __global__ __launch_bounds__(256) void argmax_stage2(const ArgPair* __restrict__ part, uint32_t nparts,
-                                                     uint32_t* __restrict__ out) {
+                                                     uint32_t* __restrict__ out, uint32_t* pos, uint32_t* token) {
     __shared__ ArgPair sh[4];
     ArgPair a{-INFINITY, 0};
     if (threadIdx.x < nparts) a = part[threadIdx.x];
     a = arg_block(a, sh);
-    if (threadIdx.x == 0) *out = a.i;
+    if (threadIdx.x == 0) {
+        *out = a.i;
+        if (pos) *pos = *pos + 1;
+        if (token) *token = a.i;
+    }
 }
 
-void launch_argmax(const float* x, uint32_t n, uint32_t* out, void* scratch, hipStream_t s) {
+void launch_argmax(const float* x, uint32_t n, uint32_t* out, void* scratch, uint32_t* pos_dev, uint32_t* token_dev,
+                   hipStream_t s) {
     uint32_t blocks = (n + 255) / 256;
     if (blocks > ARGMAX_BLOCKS) blocks = ARGMAX_BLOCKS;
     if (blocks == 0) blocks = 1;
     argmax_stage1<<<blocks, 256, 0, s>>>(x, n, reinterpret_cast<ArgPair*>(scratch));
-    argmax_stage2<<<1, 256, 0, s>>>(reinterpret_cast<const ArgPair*>(scratch), blocks, out);
-}
-
-// pos += 1 and, if `next` is given, token = *next (greedy feedback without a host round trip).
-__global__ void advance_kernel(uint32_t* pos, uint32_t* token, const uint32_t* next) {
-    if (threadIdx.x == 0) {
-        *pos = *pos + 1;
-        if (token && next) *token = *next;
-    }
-}
-void launch_advance(uint32_t* pos_dev, uint32_t* token_dev, const uint32_t* next_dev, hipStream_t s) {
-    advance_kernel<<<1, 64, 0, s>>>(pos_dev, token_dev, next_dev);
+    argmax_stage2<<<1, 256, 0, s>>>(reinterpret_cast<const ArgPair*>(scratch), blocks, out, pos_dev, token_dev);
 }
 
 }  // namespace fh

@@ -17,8 +17,17 @@
 // order (dot8/dot4: one accumulator, emit.rs:1770-1877; the N%4 tail rows of dot1: four
 // interleaved accumulators, emit.rs:1558-1571).  Multiplies and adds are not fused (Rust
 // never contracts).
+//
+// A kernel boundary costs several microseconds on this GPU, more than streaming a small
+// matrix, so the decode step's neighbours are fused in:
+//   prologue  RmsNorm: rms_norm (emit.rs:327-334, the 16-lane FMA order of emit.rs:272-295) and the
+//             activation quantiser (emit.rs:1410-1440), recomputed by every workgroup from x
+//   epilogue  Add: residual_add (emit.rs:455-459);  RopeKv: rope (emit.rs:508-528) on the q and k
+//             rows and the fp16 KV-cache write;  SiluQuant: silu_mul (emit.rs:380-386) of the gate
+//             and up rows of a fused [gate;up] matrix and the quantisation of the result.
 #include "common.h"
 #include "device_utils.h"
+#include "expf_ref.h"
 
 namespace fh {
 
@@ -30,18 +39,40 @@ __device__ __forceinline__ int dot16(int4 w, int4 a, int acc) {
     return acc;
 }
 
+enum class Pro { Quant, RmsNorm };
+enum class Epi { Store, Add, RopeKv, SiluQuant, Isums };
+
+struct Segment { uint32_t start, len, chunk; };   // one reference matmul inside a fused matrix
+
 struct GemvArgs {
     const uint8_t* qs;
     const uint16_t* ws;
+    uint32_t K, N;
+    uint32_t rc;             // rows per ordered-sum group (per wave)
+    Segment seg[3];          // row ranges of the reference matmuls (tail rule applies per matmul)
+    uint32_t nseg, tail_mod;
+    // Pro::Quant
     const int8_t* aq;
     const uint16_t* as;
+    // Pro::RmsNorm
+    const float* x;
+    const float* norm_w;
+    float eps;
+    // Epi::Store / Add / Isums
     float* y;
     int32_t* isums;
-    uint32_t K, N;
-    uint32_t rc;          // rows per ordered-sum group (per wave)
-    uint32_t chunk;       // 0, or 256: rows are grouped in chunks of this many for the tail rule
-    uint32_t tail_mod;    // the last (len % tail_mod) rows of a chunk use the 4-accumulator order
-    int accumulate;
+    // Epi::RopeKv: rows [0,QKS) -> q_out f32 (rotated); [QKS,QKS+KV) -> kc (rotated, fp16); rest -> vc (fp16)
+    float* q_out;
+    uint16_t* kc;
+    uint16_t* vc;
+    const float* cos_t;
+    const float* sin_t;
+    const uint32_t* pos_dev;
+    uint32_t qks, kv, hd;
+    // Epi::SiluQuant: rows [0,I) gate, [I,2I) up -> oq int8 [I], osc fp16 [I/32]
+    int8_t* oq;
+    uint16_t* osc;
+    uint32_t inter;
 };
 
 // Ordered sum of one row's block products p[0..nblk): sequential, or the dot1 order.
@@ -72,75 +103,180 @@ __device__ __forceinline__ float ordered_sum(const float* p, uint32_t nblk, bool
 }
 
 __device__ __forceinline__ bool row_is_dot1(uint32_t row, const GemvArgs& a) {
-    const uint32_t base = a.chunk ? (row / a.chunk) * a.chunk : 0;
-    const uint32_t len = a.chunk ? min(a.chunk, a.N - base) : a.N;
-    return (row - base) >= len - (len % a.tail_mod);
+    for (uint32_t s = 0; s < a.nseg; s++) {
+        const Segment sg = a.seg[s];
+        if (row >= sg.start && row < sg.start + sg.len) {
+            const uint32_t i = row - sg.start;
+            const uint32_t base = sg.chunk ? (i / sg.chunk) * sg.chunk : 0;
+            const uint32_t len = sg.chunk ? min(sg.chunk, sg.len - base) : sg.len;
+            return (i - base) >= len - (len % a.tail_mod);
+        }
+    }
+    return false;
 }
 
-// Q4 = false: Q8_0 planes; Q4 = true: Q4_0 planes.  ISUMS: write the int32 block sums instead of y.
-template <bool Q4, int NCH, int RW, bool ISUMS>
-__global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
+template <bool Q4, int NCH, int RW, int WAVES, Pro PRO, Epi EPI>
+__global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
     extern __shared__ float lds[];
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    constexpr uint32_t THREADS = WAVES * 64;
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t K = a.K, N = a.N, nblk = K / 32;
     const uint32_t pstride = nblk + 1;                       // +1: conflict-free column reads
     float* prod = lds + (size_t)wave * a.rc * pstride;
+    float* shared_tail = lds + (size_t)WAVES * a.rc * pstride;   // prologue / epilogue scratch
+
+    uint32_t blk[NCH];
+    bool own[NCH];                                           // this lane reports block blk[j]
+#pragma unroll
+    for (int j = 0; j < NCH; j++) {
+        if (Q4) { blk[j] = j * 64 + lane; own[j] = blk[j] < nblk; }
+        else { const uint32_t off = j * 1024 + lane * 16; blk[j] = off / 32; own[j] = off < K && !(lane & 1); }
+    }
+
+    // ---- row groups.  Standard: wave w of workgroup-group g0 owns rows [(g0+w) rc, +rc).
+    //      SiluQuant (WAVES = 16, rc = 4): workgroup G owns inter indices [32 G, +32): waves 0..7 take the
+    //      gate rows, waves 8..15 the up rows, four rows each.
+    const uint32_t ngroups = EPI == Epi::SiluQuant ? (a.inter + 31) / 32 : (N + a.rc - 1) / a.rc;
+    const uint32_t gstep = EPI == Epi::SiluQuant ? 1 : WAVES;
+    auto rows_of = [&](uint32_t g0, uint32_t& row_base, uint32_t& row_end) -> bool {
+        if (EPI == Epi::SiluQuant) {
+            const uint32_t i0 = g0 * 32 + (wave & 7) * 4;
+            row_base = (wave >> 3) * a.inter + i0;
+            row_end = (wave >> 3) * a.inter + min(a.inter, i0 + 4);
+            return i0 < a.inter;
+        }
+        const uint32_t g = g0 + wave;                        // may be >= ngroups: idle but keeps the barriers uniform
+        row_base = g * a.rc;
+        row_end = min(N, row_base + a.rc);
+        return g < ngroups;
+    };
+
+    int4 wv[RW][NCH];
+    uint16_t wsb[RW][NCH];
+    auto load_rows = [&](uint32_t row0, uint32_t row_end) {
+#pragma unroll
+        for (int r = 0; r < RW; r++) {
+            const uint32_t row = min(row0 + r, row_end - 1);
+#pragma unroll
+            for (int j = 0; j < NCH; j++) {
+                if (Q4) {
+                    if (blk[j] < nblk) {
+                        wv[r][j] = *reinterpret_cast<const int4*>(a.qs + ((size_t)row * nblk + blk[j]) * 16);
+                        wsb[r][j] = a.ws[(size_t)row * nblk + blk[j]];
+                    } else { wv[r][j] = make_int4(0, 0, 0, 0); wsb[r][j] = 0; }
+                } else {
+                    const uint32_t off = j * 1024 + lane * 16;
+                    if (off < K) {
+                        wv[r][j] = *reinterpret_cast<const int4*>(a.qs + (size_t)row * K + off);
+                        wsb[r][j] = a.ws[(size_t)row * nblk + blk[j]];
+                    } else { wv[r][j] = make_int4(0, 0, 0, 0); wsb[r][j] = 0; }
+                }
+            }
+        }
+    };
+
+    // Weights do not depend on the activations: start streaming the first rows before the prologue.
+    bool prefetched = false;
+    {
+        uint32_t rb, re;
+        const uint32_t g0 = blockIdx.x * gstep;
+        if (g0 < ngroups && rows_of(g0, rb, re) && rb < re) { load_rows(rb, re); prefetched = true; }
+    }
 
     // ---- activation fragment, resident for the whole kernel
     int4 av[NCH], av2[Q4 ? NCH : 1];
     int asum8[Q4 ? NCH : 1];
     float asf[NCH];
-    uint32_t blk[NCH];
-    bool own[NCH];                                           // this lane reports block blk[j]
+    if (PRO == Pro::RmsNorm) {
+        // rms_norm of x[K] in the reference's summation order, then block quantisation, all in-kernel
+        float* xs = shared_tail;                              // K floats + 17
+        float* part = xs + K;
+        for (uint32_t i = tid; i < K / 4; i += THREADS) reinterpret_cast<float4*>(xs)[i] = reinterpret_cast<const float4*>(a.x)[i];
+        __syncthreads();
+        if (tid < 16) {
+            float s = 0.f;
+            const uint32_t chunks = K / 16;
+            uint32_t c = 0;
+            for (; c + 8 <= chunks; c += 8) {
+                float v[8];
 #pragma unroll
-    for (int j = 0; j < NCH; j++) {
-        if (Q4) {
-            const uint32_t b = j * 64 + lane;
-            blk[j] = b; own[j] = b < nblk;
-            if (own[j]) {
-                av[j] = *reinterpret_cast<const int4*>(a.aq + (size_t)b * 32);
-                av2[j] = *reinterpret_cast<const int4*>(a.aq + (size_t)b * 32 + 16);
-                const int4 ones = make_int4(0x01010101, 0x01010101, 0x01010101, 0x01010101);
-                asum8[j] = 8 * dot16(ones, av2[j], dot16(ones, av[j], 0));
-            } else {
-                av[j] = av2[j] = make_int4(0, 0, 0, 0); asum8[j] = 0;
+                for (int i = 0; i < 8; i++) v[i] = xs[(c + i) * 16 + tid];
+#pragma unroll
+                for (int i = 0; i < 8; i++) s = fmaf(v[i], v[i], s);
             }
-        } else {
-            const uint32_t off = j * 1024 + lane * 16;
-            blk[j] = off / 32; own[j] = off < K && !(lane & 1);
-            av[j] = off < K ? *reinterpret_cast<const int4*>(a.aq + off) : make_int4(0, 0, 0, 0);
+            for (; c < chunks; c++) { const float v = xs[c * 16 + tid]; s = fmaf(v, v, s); }
+            part[tid] = s;
         }
-        asf[j] = (!ISUMS && blk[j] < nblk) ? f16_bits_to_f32(a.as[blk[j]]) : 0.f;
+        __syncthreads();
+        if (tid == 0) {
+            float t[4];
+            for (int i = 0; i < 4; i++) t[i] = (part[i] + part[4 + i]) + (part[8 + i] + part[12 + i]);
+            float r = (t[0] + t[1]) + (t[2] + t[3]);
+            for (uint32_t i = K / 16 * 16; i < K; i++) r = r + xs[i] * xs[i];
+            part[16] = r;
+        }
+        __syncthreads();
+        const float inv_rms = 1.0f / sqrtf(part[16] / (float)K + a.eps);
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            // the 16 (Q8 layout) or 32 (Q4 layout) consecutive elements this lane holds of chunk j
+            const uint32_t e0 = Q4 ? (j * 64 + lane) * 32 : j * 1024 + lane * 16;
+            constexpr int CNT = Q4 ? 32 : 16;
+            float v[CNT];
+            float amax = 0.f;
+            const bool in = e0 < K;
+#pragma unroll
+            for (int i = 0; i < CNT / 4; i++) {
+                float4 xv = make_float4(0.f, 0.f, 0.f, 0.f), wv4 = xv;
+                if (in) { xv = reinterpret_cast<const float4*>(xs + e0)[i]; wv4 = reinterpret_cast<const float4*>(a.norm_w + e0)[i]; }
+                v[4 * i] = xv.x * inv_rms * wv4.x; v[4 * i + 1] = xv.y * inv_rms * wv4.y;
+                v[4 * i + 2] = xv.z * inv_rms * wv4.z; v[4 * i + 3] = xv.w * inv_rms * wv4.w;
+            }
+#pragma unroll
+            for (int i = 0; i < CNT; i++) amax = fmaxf(amax, fabsf(v[i]));
+            if (!Q4) amax = fmaxf(amax, __shfl_xor(amax, 1, WAVE));   // the other half of the block
+            float inv;
+            const float sc = act_scale(amax, inv);
+            asf[j] = in ? f16_bits_to_f32(f32_to_f16_bits(sc)) : 0.f;
+            uint32_t pk[CNT / 4];
+#pragma unroll
+            for (int i = 0; i < CNT / 4; i++) {
+                pk[i] = ((uint32_t)quant_code(v[4 * i] * inv) & 0xFFu) | (((uint32_t)quant_code(v[4 * i + 1] * inv) & 0xFFu) << 8) |
+                        (((uint32_t)quant_code(v[4 * i + 2] * inv) & 0xFFu) << 16) | (((uint32_t)quant_code(v[4 * i + 3] * inv) & 0xFFu) << 24);
+            }
+            av[j] = make_int4((int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]);
+            if (Q4) av2[j] = make_int4((int)pk[CNT / 4 - 4], (int)pk[CNT / 4 - 3], (int)pk[CNT / 4 - 2], (int)pk[CNT / 4 - 1]);
+        }
+        __syncthreads();   // xs is free again (SiluQuant reuses the tail)
+    } else {
+#pragma unroll
+        for (int j = 0; j < NCH; j++) {
+            if (Q4) {
+                if (own[j]) {
+                    av[j] = *reinterpret_cast<const int4*>(a.aq + (size_t)blk[j] * 32);
+                    av2[j] = *reinterpret_cast<const int4*>(a.aq + (size_t)blk[j] * 32 + 16);
+                } else { av[j] = av2[j] = make_int4(0, 0, 0, 0); }
+            } else {
+                const uint32_t off = j * 1024 + lane * 16;
+                av[j] = off < K ? *reinterpret_cast<const int4*>(a.aq + off) : make_int4(0, 0, 0, 0);
+            }
+            asf[j] = (EPI != Epi::Isums && blk[j] < nblk) ? f16_bits_to_f32(a.as[blk[j]]) : 0.f;
+        }
+    }
+    if (Q4) {
+        const int4 ones = make_int4(0x01010101, 0x01010101, 0x01010101, 0x01010101);
+#pragma unroll
+        for (int j = 0; j < NCH; j++) asum8[j] = 8 * dot16(ones, av2[j], dot16(ones, av[j], 0));
     }
 
-    const uint32_t ngroups = (N + a.rc - 1) / a.rc;
-    for (uint32_t g0 = blockIdx.x * 4; g0 < ngroups; g0 += gridDim.x * 4) {
-        const uint32_t g = g0 + wave;                         // may be >= ngroups: idle but keeps the barriers uniform
-        const uint32_t row_base = g * a.rc;
-        if (g < ngroups) {
+    for (uint32_t g0 = blockIdx.x * gstep; g0 < ngroups; g0 += gridDim.x * gstep) {
+        uint32_t row_base, row_end;   // this wave's rows [row_base, row_end)
+        const bool wave_on = rows_of(g0, row_base, row_end);
+        if (wave_on) {
             for (uint32_t sub = 0; sub < a.rc; sub += RW) {
-                if (row_base + sub >= N) break;
-                int4 wv[RW][NCH];
-                uint16_t wsb[RW][NCH];
-#pragma unroll
-                for (int r = 0; r < RW; r++) {
-                    const uint32_t row = min(row_base + sub + r, N - 1);
-#pragma unroll
-                    for (int j = 0; j < NCH; j++) {
-                        if (Q4) {
-                            if (blk[j] < nblk) {
-                                wv[r][j] = *reinterpret_cast<const int4*>(a.qs + ((size_t)row * nblk + blk[j]) * 16);
-                                wsb[r][j] = a.ws[(size_t)row * nblk + blk[j]];
-                            } else { wv[r][j] = make_int4(0, 0, 0, 0); wsb[r][j] = 0; }
-                        } else {
-                            const uint32_t off = j * 1024 + lane * 16;
-                            if (off < K) {
-                                wv[r][j] = *reinterpret_cast<const int4*>(a.qs + (size_t)row * K + off);
-                                wsb[r][j] = a.ws[(size_t)row * nblk + blk[j]];
-                            } else { wv[r][j] = make_int4(0, 0, 0, 0); wsb[r][j] = 0; }
-                        }
-                    }
-                }
+                if (row_base + sub >= row_end) break;
+                if (!prefetched) load_rows(row_base + sub, row_end);
+                prefetched = false;
 #pragma unroll
                 for (int r = 0; r < RW; r++) {
                     const uint32_t row = row_base + sub + r;
@@ -157,24 +293,64 @@ __global__ __launch_bounds__(256) void gemv_kernel(GemvArgs a) {
                             const int half = dot16(wv[r][j], av[j], 0);
                             isum = half + __shfl_xor(half, 1, WAVE);
                         }
-                        if (own[j] && row < N) {
-                            if (ISUMS) a.isums[(size_t)row * nblk + blk[j]] = isum;
+                        if (own[j] && row < row_end) {
+                            if (EPI == Epi::Isums) a.isums[(size_t)row * nblk + blk[j]] = isum;
                             else prod[(sub + r) * pstride + blk[j]] = (asf[j] * f16_bits_to_f32(wsb[r][j])) * (float)isum;
                         }
                     }
                 }
             }
         }
-        if (!ISUMS) {
-            __syncthreads();
-            const uint32_t row = row_base + lane;
-            if (g < ngroups && lane < a.rc && row < N) {
-                const float r = ordered_sum(prod + lane * pstride, nblk, row_is_dot1(row, a));
-                a.y[row] = a.accumulate ? a.y[row] + r : r;
+        prefetched = false;
+        if (EPI == Epi::Isums) continue;
+        __syncthreads();
+        // ---- ordered sums: lane i of the wave owns row row_base + i
+        const uint32_t row = row_base + lane;
+        const bool active = wave_on && lane < a.rc && row < row_end;
+        float r = 0.f;
+        if (active) r = ordered_sum(prod + lane * pstride, nblk, row_is_dot1(row, a));
+        if (EPI == Epi::Store) {
+            if (active) a.y[row] = r;
+        } else if (EPI == Epi::Add) {
+            if (active) a.y[row] = a.y[row] + r;
+        } else if (EPI == Epi::RopeKv) {
+            // rows 2i, 2i+1 of a head sit in lanes 2i, 2i+1 (row_base and rc are even)
+            const float other = __shfl_xor(r, 1, WAVE);
+            if (active) {
+                const uint32_t pos = *a.pos_dev;
+                if (row < a.qks + a.kv) {
+                    const uint32_t d = row < a.qks ? row % a.hd : (row - a.qks) % a.hd;
+                    const float c = a.cos_t[(size_t)pos * (a.hd / 2) + d / 2], s = a.sin_t[(size_t)pos * (a.hd / 2) + d / 2];
+                    const float o = (row & 1) ? other * s + r * c : r * c - other * s;
+                    if (row < a.qks) a.q_out[row] = o;
+                    else a.kc[(size_t)pos * a.kv + (row - a.qks)] = f32_to_f16_bits(o);
+                } else {
+                    a.vc[(size_t)pos * a.kv + (row - a.qks - a.kv)] = f32_to_f16_bits(r);
+                }
             }
-            // no second barrier: the product area is private to the wave and LDS operations of
-            // one wave execute in order
+        } else if (EPI == Epi::SiluQuant) {
+            float* res = shared_tail;                         // [64]: gate 0..31, up 32..63
+            if (active) res[(wave >> 3) * 32 + (wave & 7) * 4 + lane] = r;
+            __syncthreads();
+            if (tid < 32) {
+                const uint32_t i = g0 * 32 + tid;
+                const bool in = i < a.inter;
+                const float gx = in ? res[tid] : 0.f, ux = in ? res[32 + tid] : 0.f;
+                const float o = in ? (gx / (1.0f + expf_ref<true>(-gx))) * ux : 0.f;
+                float amax = fabsf(o);
+#pragma unroll
+                for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+                float inv;
+                const float sc = act_scale(amax, inv);
+                if (in) {
+                    a.oq[i] = (int8_t)quant_code(o * inv);
+                    if (tid == 0) a.osc[i / 32] = f32_to_f16_bits(sc);
+                }
+            }
+            // the next iteration's first barrier orders these reads before res[] is rewritten
         }
+        // the product area is private to the wave and LDS operations of one wave execute in order,
+        // so no barrier is needed before the next group overwrites it
     }
 }
 
@@ -187,42 +363,75 @@ uint32_t rows_per_group(uint32_t nblk, uint32_t N, uint32_t rw) {
     uint32_t cap = nblk <= 32 ? 64 : nblk <= 64 ? 32 : nblk <= 128 ? 16 : nblk <= 256 ? 8 : 4;
     uint32_t want = N / 4096 / rw * rw;          // aim for >= 4096 groups, i.e. >= 4 waves per SIMD
     if (want < rw) want = rw;
+    want &= ~1u;                                 // rope pairs need both rows of a pair in one group
+    if (want < 2) want = 2;
     return want < cap ? want : cap;
 }
 
-template <bool Q4, int NCH, int RW, bool ISUMS>
-void launch_one(GemvArgs a, hipStream_t s) {
-    const uint32_t nblk = a.K / 32;
-    a.rc = rows_per_group(nblk, a.N, RW);
-    const uint32_t ngroups = (a.N + a.rc - 1) / a.rc;
-    uint32_t grid = (ngroups + 3) / 4;
-    if (grid > 256 * 8) grid = 256 * 8;
-    const size_t lds = ISUMS ? 0 : (size_t)4 * a.rc * (nblk + 1) * sizeof(float);
-    gemv_kernel<Q4, NCH, RW, ISUMS><<<grid, 256, lds, s>>>(a);
+constexpr size_t LDS_LIMIT = 64 * 1024;
+size_t lds_tail_bytes(bool norm, bool silu, uint32_t K) {
+    size_t tail = norm ? (size_t)(K + 32) * sizeof(float) : 0;
+    if (silu && tail < 64 * sizeof(float)) tail = 64 * sizeof(float);
+    return tail;
 }
 
-template <bool ISUMS>
-void dispatch(const QWeight& w, GemvArgs a, hipStream_t s) {
-    if (w.wdtype == FORGE_HIP_Q8_0) {
-        const uint32_t nch = (w.K + 1023) / 1024;
+template <bool Q4, int NCH, int RW, Pro PRO, Epi EPI>
+void launch_one(GemvArgs a, hipStream_t s) {
+    constexpr int WAVES = EPI == Epi::SiluQuant ? 16 : 4;
+    const uint32_t nblk = a.K / 32;
+    const size_t tail = lds_tail_bytes(PRO == Pro::RmsNorm, EPI == Epi::SiluQuant, a.K);
+    a.rc = EPI == Epi::SiluQuant ? 4 : rows_per_group(nblk, a.N, RW);
+    // shrink the group if the products and the prologue's copy of x do not fit LDS together
+    constexpr uint32_t step = RW < 2 ? 2 : RW;
+    while (EPI != Epi::SiluQuant && a.rc > step && (size_t)WAVES * a.rc * (nblk + 1) * sizeof(float) + tail > LDS_LIMIT) a.rc -= step;
+    const uint32_t ngroups = EPI == Epi::SiluQuant ? (a.inter + 31) / 32 : ((a.N + a.rc - 1) / a.rc + WAVES - 1) / WAVES;
+    uint32_t grid = ngroups;
+    if (grid > 256 * 8) grid = 256 * 8;
+    const size_t lds = EPI == Epi::Isums ? 0 : (size_t)WAVES * a.rc * (nblk + 1) * sizeof(float);
+    gemv_kernel<Q4, NCH, (EPI == Epi::SiluQuant ? (RW > 4 ? 4 : RW) : RW), WAVES, PRO, EPI><<<grid, WAVES * 64, lds + tail, s>>>(a);
+}
+
+template <Pro PRO, Epi EPI>
+void dispatch(uint32_t wdtype, const GemvArgs& a, hipStream_t s) {
+    // SiluQuant walks 16 rows per wave; RW must divide 16 (it always does)
+    if (wdtype == FORGE_HIP_Q8_0) {
+        const uint32_t nch = (a.K + 1023) / 1024;
         switch (nch) {
-            case 1: launch_one<false, 1, 4, ISUMS>(a, s); break;
-            case 2: launch_one<false, 2, 4, ISUMS>(a, s); break;
-            case 3: launch_one<false, 3, 2, ISUMS>(a, s); break;
-            case 4: launch_one<false, 4, 2, ISUMS>(a, s); break;
-            case 5: case 6: launch_one<false, 6, 2, ISUMS>(a, s); break;
-            case 7: case 8: launch_one<false, 8, 1, ISUMS>(a, s); break;
-            default: launch_one<false, 16, 1, ISUMS>(a, s); break;
+            case 1: launch_one<false, 1, 4, PRO, EPI>(a, s); break;
+            case 2: launch_one<false, 2, 4, PRO, EPI>(a, s); break;
+            case 3: launch_one<false, 3, 2, PRO, EPI>(a, s); break;
+            case 4: launch_one<false, 4, 2, PRO, EPI>(a, s); break;
+            case 5: case 6: launch_one<false, 6, 2, PRO, EPI>(a, s); break;
+            case 7: case 8: launch_one<false, 8, 1, PRO, EPI>(a, s); break;
+            default: launch_one<false, 16, 1, PRO, EPI>(a, s); break;
         }
     } else {
-        const uint32_t nch = (w.K + 2047) / 2048;
+        const uint32_t nch = (a.K + 2047) / 2048;
         switch (nch) {
-            case 1: launch_one<true, 1, 4, ISUMS>(a, s); break;
-            case 2: launch_one<true, 2, 4, ISUMS>(a, s); break;
-            case 3: case 4: launch_one<true, 4, 2, ISUMS>(a, s); break;
-            default: launch_one<true, 8, 1, ISUMS>(a, s); break;
+            case 1: launch_one<true, 1, 4, PRO, EPI>(a, s); break;
+            case 2: launch_one<true, 2, 4, PRO, EPI>(a, s); break;
+            case 3: case 4: launch_one<true, 4, 2, PRO, EPI>(a, s); break;
+            default: launch_one<true, 8, 1, PRO, EPI>(a, s); break;
         }
     }
+}
+
+// matmul_vec chunks rows by 256 once the matrix reaches 1 MB of GGUF bytes (emit.rs:1937,1971); the
+// lm_head GEMV always chunks, with an 8-row tail rule after batched prefill (emit.rs:5455-5470).
+Segment make_segment(uint32_t wdtype, uint32_t K, uint32_t start, uint32_t len, GemvOrder order) {
+    const size_t raw_bytes = (size_t)len * (K / 32) * (wdtype == FORGE_HIP_Q8_0 ? 34 : 18);
+    Segment sg;
+    sg.start = start; sg.len = len;
+    sg.chunk = (order != GemvOrder::MatmulVec || raw_bytes >= 1000000) ? 256 : 0;
+    return sg;
+}
+
+GemvArgs base_args(const QWeight& w, GemvOrder order) {
+    GemvArgs a{};
+    a.qs = w.qs; a.ws = w.scales; a.K = w.K; a.N = w.N;
+    a.nseg = 1; a.seg[0] = make_segment(w.wdtype, w.K, 0, w.N, order);
+    a.tail_mod = order == GemvOrder::LmHeadAfterPrefill ? 8 : 4;
+    return a;
 }
 
 }  // namespace
@@ -230,24 +439,58 @@ void dispatch(const QWeight& w, GemvArgs a, hipStream_t s) {
 // Largest K the register-resident activation fragment covers.
 bool gemv_k_supported(uint32_t K) { return K % 32 == 0 && K >= 32 && K <= 16384; }
 
+// Whether the fused prologue / epilogue variants fit LDS for this K (else the caller launches the
+// separate kernels).
+bool gemv_norm_fusable(uint32_t K) {
+    return gemv_k_supported(K) && (size_t)4 * 4 * (K / 32 + 1) * sizeof(float) + lds_tail_bytes(true, false, K) <= LDS_LIMIT;
+}
+bool gemv_silu_fusable(uint32_t K) {
+    return gemv_k_supported(K) && (size_t)16 * 4 * (K / 32 + 1) * sizeof(float) + lds_tail_bytes(true, true, K) <= LDS_LIMIT;
+}
+
 void launch_gemv(const QWeight& w, const int8_t* aq, const uint16_t* as, float* y, bool accumulate, GemvOrder order,
                  hipStream_t s) {
-    GemvArgs a{};
-    a.qs = w.qs; a.ws = w.scales; a.aq = aq; a.as = as; a.y = y; a.isums = nullptr; a.K = w.K; a.N = w.N;
-    a.accumulate = accumulate ? 1 : 0;
-    // matmul_vec: chunks of 256 rows once the matrix reaches 1 MB of GGUF bytes (emit.rs:1937,1971);
-    // the lm_head GEMV always chunks, with an 8-row tail rule after batched prefill (emit.rs:5455-5470).
-    const size_t raw_bytes = (size_t)w.N * (w.K / 32) * (w.wdtype == FORGE_HIP_Q8_0 ? 34 : 18);
-    a.chunk = (order != GemvOrder::MatmulVec || raw_bytes >= 1000000) ? 256 : 0;
-    a.tail_mod = order == GemvOrder::LmHeadAfterPrefill ? 8 : 4;
-    dispatch<false>(w, a, s);
+    GemvArgs a = base_args(w, order);
+    a.aq = aq; a.as = as; a.y = y;
+    if (accumulate) dispatch<Pro::Quant, Epi::Add>(w.wdtype, a, s);
+    else dispatch<Pro::Quant, Epi::Store>(w.wdtype, a, s);
 }
 
 void launch_gemv_isums(const QWeight& w, const int8_t* aq, int32_t* out, hipStream_t s) {
-    GemvArgs a{};
-    a.qs = w.qs; a.ws = w.scales; a.aq = aq; a.as = nullptr; a.y = nullptr; a.isums = out; a.K = w.K; a.N = w.N;
-    a.tail_mod = 4;
-    dispatch<true>(w, a, s);
+    GemvArgs a = base_args(w, GemvOrder::MatmulVec);
+    a.aq = aq; a.isums = out;
+    dispatch<Pro::Quant, Epi::Isums>(w.wdtype, a, s);
+}
+
+void launch_gemv_norm(const QWeight& w, const float* x, const float* norm_w, float eps, float* y, GemvOrder order,
+                      hipStream_t s) {
+    GemvArgs a = base_args(w, order);
+    a.x = x; a.norm_w = norm_w; a.eps = eps; a.y = y;
+    dispatch<Pro::RmsNorm, Epi::Store>(w.wdtype, a, s);
+}
+
+void launch_gemv_norm_rope_kv(const QWeight& wqkv, const float* x, const float* norm_w, float eps, float* q_out,
+                              uint16_t* kc, uint16_t* vc, const float* cos_t, const float* sin_t,
+                              const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s) {
+    GemvArgs a = base_args(wqkv, GemvOrder::MatmulVec);
+    a.x = x; a.norm_w = norm_w; a.eps = eps;
+    a.q_out = q_out; a.kc = kc; a.vc = vc; a.cos_t = cos_t; a.sin_t = sin_t; a.pos_dev = pos_dev;
+    a.qks = heads * hd; a.kv = kv_heads * hd; a.hd = hd;
+    a.nseg = 3;
+    a.seg[0] = make_segment(wqkv.wdtype, wqkv.K, 0, a.qks, GemvOrder::MatmulVec);
+    a.seg[1] = make_segment(wqkv.wdtype, wqkv.K, a.qks, a.kv, GemvOrder::MatmulVec);
+    a.seg[2] = make_segment(wqkv.wdtype, wqkv.K, a.qks + a.kv, a.kv, GemvOrder::MatmulVec);
+    dispatch<Pro::RmsNorm, Epi::RopeKv>(wqkv.wdtype, a, s);
+}
+
+void launch_gemv_norm_silu_quant(const QWeight& wgu, const float* x, const float* norm_w, float eps, int8_t* oq,
+                                 uint16_t* osc, hipStream_t s) {
+    GemvArgs a = base_args(wgu, GemvOrder::MatmulVec);
+    a.x = x; a.norm_w = norm_w; a.eps = eps; a.oq = oq; a.osc = osc; a.inter = wgu.N / 2;
+    a.nseg = 2;
+    a.seg[0] = make_segment(wgu.wdtype, wgu.K, 0, a.inter, GemvOrder::MatmulVec);
+    a.seg[1] = make_segment(wgu.wdtype, wgu.K, a.inter, a.inter, GemvOrder::MatmulVec);
+    dispatch<Pro::RmsNorm, Epi::SiluQuant>(wgu.wdtype, a, s);
 }
 
 }  // namespace fh

@@ -65,6 +65,7 @@ struct forge_hip_model {
     uint32_t* h_stage = nullptr;
     int64_t pos = 0;
     bool use_graph = true;
+    bool fuse_norm = false, fuse_silu = false;   // fused GEMV prologue/epilogue variants fit LDS for this model
     hipGraphExec_t decode_graph = nullptr;
     // forward_profile: while `prof_on`, every launch is bracketed by a pair of events tagged with its stage
     bool prof_on = false;
@@ -149,93 +150,133 @@ int32_t validate(const forge_hip_config* c) {
     return FORGE_HIP_OK;
 }
 
-// Enqueue one decoder layer on the model's stream.  decode: one row, position read from
-// device memory.  prefill: M rows at positions base_pos.. .
-void enqueue_layer(forge_hip_model* m, uint32_t l, bool decode, uint32_t M, uint32_t base_pos) {
+// Attention + O projection of one decode row; q is in qkv[0, QKS), attention output goes out quantised.
+void enqueue_decode_attention(forge_hip_model* m, uint32_t l, const float* q, uint32_t q_stride) {
+    const forge_hip_config& c = m->cfg;
+    hipStream_t s = m->stream;
+    const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
+    int8_t* aq = m->aq.as<int8_t>();
+    uint16_t* asc = m->asc.as<uint16_t>();
+    {
+        StageMark t(m, ST_ATTN);
+        if (exact)
+            launch_attn_exact(false, q, q_stride, m->kc(l), m->vc(l), nullptr, m->QKS, aq, asc, 1, 0, m->d_pos(), c.heads,
+                              c.kv_heads, c.head_dim, s);
+        else
+            launch_attn_decode(q, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads, c.head_dim,
+                               m->attn_ws.p, s);
+    }
+    { StageMark t(m, ST_O); launch_gemv(m->layers[l].o, aq, asc, m->x.as<float>(), true, GemvOrder::MatmulVec, s); }
+}
+
+// One decoder layer of the decode step (one row, position read from device memory).  Six launches
+// when the fused GEMV variants fit LDS: [norm+quant | qkv GEMV | rope + KV write], attention split,
+// attention merge + quant, [o GEMV | residual], [norm+quant | gate/up GEMV | silu*up + quant],
+// [down GEMV | residual].
+void enqueue_decode_layer(forge_hip_model* m, uint32_t l) {
     const forge_hip_config& c = m->cfg;
     Layer& L = m->layers[l];
     hipStream_t s = m->stream;
     const uint32_t H = m->H, I = m->I, QKS = m->QKS, KV = m->KV, QKV = m->QKV;
-    float* x = decode ? m->x.as<float>() : m->px.as<float>();
-    float* qkv = decode ? m->qkv.as<float>() : m->pqkv.as<float>();
-    float* gu = decode ? m->gu.as<float>() : m->pgu.as<float>();
-    int8_t* aq = decode ? m->aq.as<int8_t>() : m->paq.as<int8_t>();
-    uint16_t* asc = decode ? m->asc.as<uint16_t>() : m->pasc.as<uint16_t>();
-
-    const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
+    float* x = m->x.as<float>();
+    float* qkv = m->qkv.as<float>();
+    float* gu = m->gu.as<float>();
+    int8_t* aq = m->aq.as<int8_t>();
+    uint16_t* asc = m->asc.as<uint16_t>();
     const GemvOrder mv = GemvOrder::MatmulVec;
-    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
-    {
+    if (m->fuse_norm) {
         StageMark t(m, ST_QKV);
-        if (decode) launch_gemv(L.qkv, aq, asc, qkv, false, mv, s);
-        else launch_gemm(L.qkv, aq, asc, M, qkv, QKV, false, exact, nullptr, s);
-    }
-    {
-        StageMark t(m, ST_ROPE);
-        launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos,
-                             decode ? m->d_pos() : nullptr, c.heads, c.kv_heads, c.head_dim, m->cos_t.as<float>(),
-                             m->sin_t.as<float>(), s);
-    }
-    if (decode) {
-        {
-            StageMark t(m, ST_ATTN);
-            if (exact)
-                launch_attn_exact(false, qkv, QKV, m->kc(l), m->vc(l), nullptr, QKS, aq, asc, 1, 0, m->d_pos(), c.heads,
-                                  c.kv_heads, c.head_dim, s);
-            else
-                launch_attn_decode(qkv, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads,
-                                   c.head_dim, m->attn_ws.p, s);
-        }
-        { StageMark t(m, ST_O); launch_gemv(L.o, aq, asc, x, true, mv, s); }
+        launch_gemv_norm_rope_kv(L.qkv, x, L.attn_norm, c.rms_eps, qkv, m->kc(l), m->vc(l), m->cos_t.as<float>(),
+                                 m->sin_t.as<float>(), m->d_pos(), c.heads, c.kv_heads, c.head_dim, s);
+        // q now sits compact in qkv[0, QKS)
     } else {
-        float* attn = m->pattn.as<float>();
+        { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, 1, H, nullptr, aq, asc, s); }
+        { StageMark t(m, ST_QKV); launch_gemv(L.qkv, aq, asc, qkv, false, mv, s); }
         {
-            StageMark t(m, ST_ATTN);
-            if (exact)
-                launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr,
-                                  c.heads, c.kv_heads, c.head_dim, s);
-            else
-                launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads,
-                                    c.head_dim, s);
+            StageMark t(m, ST_ROPE);
+            launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), 1, 0, m->d_pos(), c.heads,
+                                 c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), s);
         }
-        { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
-        { StageMark t(m, ST_O); launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s); }
     }
-    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
-    {
+    enqueue_decode_attention(m, l, qkv, QKS);
+    if (m->fuse_silu) {
         StageMark t(m, ST_GATE_UP);
-        if (decode) launch_gemv(L.gate_up, aq, asc, gu, false, mv, s);
-        else launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s);
+        launch_gemv_norm_silu_quant(L.gate_up, x, L.ffn_norm, c.rms_eps, aq, asc, s);
+    } else {
+        { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, 1, H, nullptr, aq, asc, s); }
+        { StageMark t(m, ST_GATE_UP); launch_gemv(L.gate_up, aq, asc, gu, false, mv, s); }
+        { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, 1, I, 2 * I, nullptr, aq, asc, s); }
     }
-    { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s); }
-    {
-        StageMark t(m, ST_DOWN);
-        if (decode) launch_gemv(L.down, aq, asc, x, true, mv, s);
-        else launch_gemm(L.down, aq, asc, M, x, H, true, exact, nullptr, s);
-    }
+    { StageMark t(m, ST_DOWN); launch_gemv(L.down, aq, asc, x, true, mv, s); }
 }
 
-// Final norm of one row + lm_head GEMV + argmax.
-void enqueue_head(forge_hip_model* m, const float* xrow, bool after_prefill) {
+// One decoder layer of a batched prefill: M rows at positions base_pos.. .
+void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t base_pos) {
+    const forge_hip_config& c = m->cfg;
+    Layer& L = m->layers[l];
     hipStream_t s = m->stream;
+    const uint32_t H = m->H, I = m->I, QKS = m->QKS, KV = m->KV, QKV = m->QKV;
+    float* x = m->px.as<float>();
+    float* qkv = m->pqkv.as<float>();
+    float* gu = m->pgu.as<float>();
+    float* attn = m->pattn.as<float>();
+    int8_t* aq = m->paq.as<int8_t>();
+    uint16_t* asc = m->pasc.as<uint16_t>();
+    const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
+    { StageMark t(m, ST_QKV); launch_gemm(L.qkv, aq, asc, M, qkv, QKV, false, exact, nullptr, s); }
     {
-        StageMark t(m, ST_RMSNORM);
-        launch_rmsnorm(xrow, m->final_norm.as<float>(), m->cfg.rms_eps, 1, m->H, nullptr, m->aq.as<int8_t>(),
-                       m->asc.as<uint16_t>(), s);
+        StageMark t(m, ST_ROPE);
+        launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos, nullptr, c.heads,
+                             c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), s);
     }
     {
+        StageMark t(m, ST_ATTN);
+        if (exact)
+            launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads,
+                              c.kv_heads, c.head_dim, s);
+        else
+            launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, s);
+    }
+    { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
+    { StageMark t(m, ST_O); launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s); }
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
+    { StageMark t(m, ST_GATE_UP); launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s); }
+    { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s); }
+    { StageMark t(m, ST_DOWN); launch_gemm(L.down, aq, asc, M, x, H, true, exact, nullptr, s); }
+}
+
+// Final norm of one row + lm_head GEMV + argmax (+ pos/token advance when `advance`).
+void enqueue_head(forge_hip_model* m, const float* xrow, bool after_prefill, bool advance) {
+    hipStream_t s = m->stream;
+    const GemvOrder order = after_prefill ? GemvOrder::LmHeadAfterPrefill : GemvOrder::LmHead;
+    // The lm_head runs thousands of workgroups; repeating the norm prologue in each costs more than the
+    // one extra launch, so the fused form is used only for small vocabularies.
+    if (m->fuse_norm && m->cfg.vocab <= 16384) {
         StageMark t(m, ST_LM_HEAD);
-        launch_gemv(m->lm_head, m->aq.as<int8_t>(), m->asc.as<uint16_t>(), m->logits.as<float>(), false,
-                    after_prefill ? GemvOrder::LmHeadAfterPrefill : GemvOrder::LmHead, s);
+        launch_gemv_norm(m->lm_head, xrow, m->final_norm.as<float>(), m->cfg.rms_eps, m->logits.as<float>(), order, s);
+    } else {
+        {
+            StageMark t(m, ST_RMSNORM);
+            launch_rmsnorm(xrow, m->final_norm.as<float>(), m->cfg.rms_eps, 1, m->H, nullptr, m->aq.as<int8_t>(),
+                           m->asc.as<uint16_t>(), s);
+        }
+        {
+            StageMark t(m, ST_LM_HEAD);
+            launch_gemv(m->lm_head, m->aq.as<int8_t>(), m->asc.as<uint16_t>(), m->logits.as<float>(), false, order, s);
+        }
     }
-    { StageMark t(m, ST_ARGMAX); launch_argmax(m->logits.as<float>(), m->cfg.vocab, m->d_next(), m->argmax_ws.p, s); }
+    {
+        StageMark t(m, ST_ARGMAX);
+        launch_argmax(m->logits.as<float>(), m->cfg.vocab, m->d_next(), m->argmax_ws.p, advance ? m->d_pos() : nullptr,
+                      advance ? m->d_token() : nullptr, s);
+    }
 }
 
 void enqueue_decode_step(forge_hip_model* m) {
     { StageMark t(m, ST_EMBED); launch_embedding(m->embed.as<float>(), m->d_token(), 1, m->H, m->x.as<float>(), m->stream); }
-    for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_layer(m, l, true, 1, 0);
-    enqueue_head(m, m->x.as<float>(), false);
-    launch_advance(m->d_pos(), m->d_token(), m->d_next(), m->stream);
+    for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_decode_layer(m, l);
+    enqueue_head(m, m->x.as<float>(), false, true);
 }
 
 int32_t run_decode_step(forge_hip_model* m) {
@@ -297,6 +338,10 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
     m->KMAX = std::max(std::max(H, I), QKS);
     const char* genv = getenv("FORGE_HIP_GRAPH");
     m->use_graph = !(genv && genv[0] == '0');
+    const char* fenv = getenv("FORGE_HIP_FUSE");
+    const bool fuse_ok = !(fenv && fenv[0] == '0');
+    m->fuse_norm = fuse_ok && gemv_norm_fusable(H);
+    m->fuse_silu = fuse_ok && gemv_silu_fusable(H);
     FH_HIP(hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking));
     FH_HIP(hipHostMalloc((void**)&m->h_stage, 64, hipHostMallocDefault));
 
@@ -417,7 +462,7 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint
         // pageable source: the copy is complete (staged) when the call returns
         FH_HIP(hipMemcpyAsync(m->ptok.p, tokens + done, (size_t)rows * 4, hipMemcpyHostToDevice, s));
         launch_embedding(m->embed.as<float>(), m->ptok.as<uint32_t>(), rows, m->H, m->px.as<float>(), s);
-        for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_layer(m, l, false, rows, (uint32_t)(m->pos + done));
+        for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_prefill_layer(m, l, rows, (uint32_t)(m->pos + done));
         FH_HIP(hipGetLastError());
         done += rows;
         last_rows = rows;
@@ -426,7 +471,7 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint
     m->h_stage[2] = (uint32_t)m->pos;
     FH_HIP(hipMemcpyAsync(m->d_pos(), &m->h_stage[2], 4, hipMemcpyHostToDevice, s));
     if (logits_host) {
-        enqueue_head(m, m->px.as<float>() + (size_t)(last_rows - 1) * m->H, true);
+        enqueue_head(m, m->px.as<float>() + (size_t)(last_rows - 1) * m->H, true, false);
         FH_HIP(hipGetLastError());
         FH_HIP(hipMemcpyAsync(logits_host, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, s));
     }
