@@ -402,7 +402,7 @@ void dispatch(uint32_t wdtype, const GemvArgs& a, hipStream_t s) {
             case 3: launch_one<false, 3, 2, PRO, EPI>(a, s); break;
             case 4: launch_one<false, 4, 2, PRO, EPI>(a, s); break;
             case 5: case 6: launch_one<false, 6, 2, PRO, EPI>(a, s); break;
-            case 7: case 8: launch_one<false, 8, 1, PRO, EPI>(a, s); break;
+            case 7: case 8: launch_one<false, 8, 2, PRO, EPI>(a, s); break;
             default: launch_one<false, 16, 1, PRO, EPI>(a, s); break;
         }
     } else {
