@@ -7,8 +7,9 @@ resident in HBM when the timed regions start.
 
 roofline: the decode step's dominant kernel, the quantised GEMV.  `achieved` = algorithmic bytes
 (GGUF block bytes of every matrix + its f32 input and output vectors) of the GEMV launches of one
-token / their summed device time, measured with HIP events around every launch by the library's
-forward_profile on the model's own stream.  `peak` = 8 TB/s (MI355X HBM3E).
+token / their summed device time, measured live by the library's forward_profile with a pair of HIP
+events attached to every kernel dispatch on the model's own stream (the kernel's begin-to-end time, the
+figure a kernel trace reports).  `peak` = 8 TB/s (MI355X HBM3E).
 
 cpu_baseline: the CPU restatement of the reference's generated kernels (oracle/), in the arithmetic
 the reference runs on an x86 host (f32 activations x dequantised weights, int8 KV), per-token decode,
@@ -28,6 +29,10 @@ HBM_PEAK_GBS = 8000.0
 MFMA_I8_PEAK_TOPS = 5000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 PROMPT_TOKENS = 2502
+# HBM bytes per GEMV launch of this workload, averaged over the 65 GEMV launches of one decode step: FETCH_SIZE and
+# WRITE_SIZE counters of two profiler runs of this script, each scaled by what the same counter reads for the 1 GiB
+# copy of --calibrate-copy (FETCH_SIZE x2.000, WRITE_SIZE x1.000).  Summary: profiles/gemv_hbm_traffic_pmc.md.
+GEMV_HBM_BYTES_PER_LAUNCH = 20.46e6 + 0.02e6      # fetched + written
 
 
 def gemv_launch_bytes(fh, cfg):
@@ -80,6 +85,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one 1 GiB device-to-device copy kernel (known HBM traffic, for scaling counter readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU; --gpus must be 1 (no multi-GPU path exists to run)", file=sys.stderr)
@@ -153,12 +160,15 @@ def main():
     torch.cuda.synchronize()
     t_decode_short = time.perf_counter() - t0
     model.close()
+    if args.calibrate_copy:
+        src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)     # 1 GiB
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        dst.copy_(src)                                                                 # reads 1 GiB, writes 1 GiB
+        torch.cuda.synchronize()
+        del src, dst
 
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "gemv_hbm_traffic.json")
-    if os.path.exists(tpath):
-        with open(tpath) as f:
-            traffic = json.load(f).get("bytes_per_launch")
+    traffic = GEMV_HBM_BYTES_PER_LAUNCH if cfg["wdtype"] == fh.Q8_0 else None
 
     out = {
         "metric": "decode tok/s (Llama-3.2-1B Q8_0, 1 GPU)",

@@ -191,7 +191,7 @@ void launch_split(const float* q, const uint16_t* kc, const uint16_t* vc, float*
                   const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, hipStream_t s) {
     const uint32_t gsize = heads / kv_heads;
     dim3 grid(kv_heads * (gsize / GT), DECODE_SPLITS);
-    attn_decode_split_kernel<HD, GT><<<grid, 256, 0, s>>>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, gsize);
+    fh::launch(attn_decode_split_kernel<HD, GT>, grid, 256, 0, s, q, kc, vc, ws, seq, pos_dev, heads, kv_heads, gsize);
 }
 template <int HD>
 void launch_hd(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
@@ -201,7 +201,7 @@ void launch_hd(const float* q, const uint16_t* kc, const uint16_t* vc, float* ou
     else if (gsize % 3 == 0) launch_split<HD, 3>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
     else if (gsize % 2 == 0) launch_split<HD, 2>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
     else launch_split<HD, 1>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
-    attn_decode_combine_kernel<HD><<<heads, HD, 0, s>>>(ws, DECODE_SPLITS, out, oq, osc);
+    fh::launch(attn_decode_combine_kernel<HD>, heads, HD, 0, s, ws, DECODE_SPLITS, out, oq, osc);
 }
 }  // namespace
 

@@ -113,7 +113,7 @@ void launch_attn_exact(bool batch_order, const float* q, uint32_t q_stride, cons
     dim3 grid(heads, M);
     const uint32_t threads = hd <= 64 ? 64 : 128;
 #define FH_AX(HD_, B_) \
-    attn_exact_kernel<HD_, B_><<<grid, threads, 0, s>>>(q, q_stride, kc, vc, out, out_stride, oq, osc, base_pos, pos_dev, heads, kv_heads)
+    fh::launch(attn_exact_kernel<HD_, B_>, grid, threads, 0, s, q, q_stride, kc, vc, out, out_stride, oq, osc, base_pos, pos_dev, heads, kv_heads)
     if (hd == 64) { if (batch_order) FH_AX(64, true); else FH_AX(64, false); }
     else if (hd == 96) { if (batch_order) FH_AX(96, true); else FH_AX(96, false); }
     else { if (batch_order) FH_AX(128, true); else FH_AX(128, false); }

@@ -196,9 +196,9 @@ void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, 
                          uint32_t hd, hipStream_t s) {
     if (M == 0) return;
     dim3 grid((M + QB - 1) / QB, heads);
-    if (hd == 64) attn_prefill_kernel<64><<<grid, 256, 0, s>>>(q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
-    else if (hd == 96) attn_prefill_kernel<96><<<grid, 256, 0, s>>>(q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
-    else attn_prefill_kernel<128><<<grid, 256, 0, s>>>(q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
+    if (hd == 64) fh::launch(attn_prefill_kernel<64>, grid, 256, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
+    else if (hd == 96) fh::launch(attn_prefill_kernel<96>, grid, 256, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
+    else fh::launch(attn_prefill_kernel<128>, grid, 256, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
 }
 
 }  // namespace fh

@@ -3,6 +3,7 @@
 #pragma once
 
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 
 #include <string>
@@ -26,6 +27,28 @@ int32_t fail(int32_t code, const std::string& msg);
     do {                                                              \
         if (!(cond)) return ::fh::fail(FORGE_HIP_ERR_INVALID, (msg)); \
     } while (0)
+
+// ---- kernel launch -------------------------------------------------------------------------
+// Every kernel of the library is launched through fh::launch.  While a LaunchProbe is installed on
+// the calling thread (forward_profile / prefill_profile), each launch asks it for a pair of events
+// and attaches them to the dispatch itself, so that their elapsed time is the kernel's own begin-to-end
+// device time (the dispatch timestamps a kernel trace reports), free of the cost of recording events
+// around it on the stream.
+struct LaunchProbe {
+    virtual bool next(hipEvent_t* start, hipEvent_t* stop) = 0;
+    virtual ~LaunchProbe() = default;
+};
+LaunchProbe*& launch_probe();      // thread-local slot, null when not profiling
+
+template <typename... KArgs, typename... Args>
+inline void launch(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds_bytes, hipStream_t s, Args... args) {
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    LaunchProbe* p = launch_probe();
+    if (p && p->next(&e0, &e1))
+        hipExtLaunchKernelGGL(kernel, grid, block, (uint32_t)lds_bytes, s, e0, e1, 0, static_cast<KArgs>(args)...);
+    else
+        hipLaunchKernelGGL(kernel, grid, block, (uint32_t)lds_bytes, s, static_cast<KArgs>(args)...);
+}
 
 // ---- device weight layout ----------------------------------------------------------------
 // GGUF interleaves a 2-byte scale with every 32 quants (34- or 18-byte blocks, 2-byte

@@ -26,7 +26,7 @@ void launch_quantize_act(const float* x, uint32_t M, uint32_t K, int8_t* q, uint
     uint64_t n4 = (uint64_t)M * K / 4;
     if (n4 == 0) return;
     uint32_t grid = (uint32_t)((n4 + 255) / 256);
-    quantize_act_kernel<<<grid, 256, 0, s>>>(x, n4, reinterpret_cast<uint32_t*>(q), sc);
+    fh::launch(quantize_act_kernel, grid, 256, 0, s, x, n4, reinterpret_cast<uint32_t*>(q), sc);
 }
 
 // ---- rms_norm (emit.rs:327-334) + optional block quantisation -------------------------------
@@ -92,7 +92,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
 void launch_rmsnorm(const float* x, const float* w, float eps, uint32_t M, uint32_t H, float* normed, int8_t* q,
                     uint16_t* sc, hipStream_t s) {
     if (M == 0) return;
-    rmsnorm_kernel<<<M, 256, (H + 32) * sizeof(float), s>>>(x, w, eps, H, normed, reinterpret_cast<uint32_t*>(q), sc);
+    fh::launch(rmsnorm_kernel, M, 256, (H + 32) * sizeof(float), s, x, w, eps, H, normed, reinterpret_cast<uint32_t*>(q), sc);
 }
 
 // ---- silu_mul (emit.rs:380-386) + optional block quantisation --------------------------------
@@ -128,7 +128,7 @@ void launch_silu_mul(const float* gate, const float* up, uint32_t M, uint32_t I,
     uint64_t total4 = (uint64_t)M * I / 4;
     if (total4 == 0) return;
     uint32_t grid = (uint32_t)((total4 + 255) / 256);
-    silu_mul_kernel<<<grid, 256, 0, s>>>(gate, up, I / 4, row_stride, total4, out, reinterpret_cast<uint32_t*>(q), sc);
+    fh::launch(silu_mul_kernel, grid, 256, 0, s, gate, up, I / 4, row_stride, total4, out, reinterpret_cast<uint32_t*>(q), sc);
 }
 
 // ---- rope (emit.rs:508-528) + fp16 KV write ------------------------------------------------------
@@ -182,7 +182,7 @@ void launch_rope_kv_store(float* q, float* k, const float* v, uint32_t q_stride,
     if (M == 0) return;
     uint32_t per_row = (heads + 2 * kv_heads) * hd / 2;
     dim3 grid((per_row + 255) / 256, M);
-    rope_kv_store_kernel<<<grid, 256, 0, s>>>(q, k, v, q_stride, kv_stride, kc, vc, base_pos, pos_dev, heads, kv_heads,
+    fh::launch(rope_kv_store_kernel, grid, 256, 0, s, q, k, v, q_stride, kv_stride, kc, vc, base_pos, pos_dev, heads, kv_heads,
                                               hd, cos_t, sin_t);
 }
 
@@ -201,7 +201,7 @@ void launch_embedding(const float* table, const uint32_t* tokens_dev, uint32_t M
                       hipStream_t s) {
     if (M == 0) return;
     dim3 grid((H / 4 + 255) / 256, M);
-    embedding_kernel<<<grid, 256, 0, s>>>(table, tokens_dev, H / 4, out);
+    fh::launch(embedding_kernel, grid, 256, 0, s, table, tokens_dev, H / 4, out);
 }
 
 // ---- argmax (project.rs:501-503): the LAST index among equal maxima ------------------------------------
@@ -262,8 +262,8 @@ void launch_argmax(const float* x, uint32_t n, uint32_t* out, void* scratch, uin
     uint32_t blocks = (n + 255) / 256;
     if (blocks > ARGMAX_BLOCKS) blocks = ARGMAX_BLOCKS;
     if (blocks == 0) blocks = 1;
-    argmax_stage1<<<blocks, 256, 0, s>>>(x, n, reinterpret_cast<ArgPair*>(scratch));
-    argmax_stage2<<<1, 256, 0, s>>>(reinterpret_cast<const ArgPair*>(scratch), blocks, out, pos_dev, token_dev);
+    fh::launch(argmax_stage1, blocks, 256, 0, s, x, n, reinterpret_cast<ArgPair*>(scratch));
+    fh::launch(argmax_stage2, 1, 256, 0, s, reinterpret_cast<const ArgPair*>(scratch), blocks, out, pos_dev, token_dev);
 }
 
 }  // namespace fh

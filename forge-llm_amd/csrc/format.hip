@@ -21,6 +21,11 @@ void set_error(const std::string& msg) { g_error = msg; }
 int32_t fail(int32_t code, const std::string& msg) { g_error = msg; return code; }
 const char* last_error_cstr() { return g_error.c_str(); }
 
+LaunchProbe*& launch_probe() {
+    static thread_local LaunchProbe* probe = nullptr;
+    return probe;
+}
+
 // f16_bits_to_f32, emit.rs:1245-1264
 float f16_to_f32_host(uint16_t h) {
     const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;

@@ -223,7 +223,7 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
     const int accf = accumulate ? 1 : 0;
     const bool q4 = w.wdtype == FORGE_HIP_Q4_0;
 #define FH_GEMM_LAUNCH(Q4_, DUMP_, EXACT_) \
-    gemm_q_kernel<Q4_, DUMP_, EXACT_><<<grid, 256, 0, s>>>(w.qs, w.scales, aq, as, y, isums, M, w.N, w.K, ldy, accf)
+    fh::launch(gemm_q_kernel<Q4_, DUMP_, EXACT_>, grid, 256, 0, s, w.qs, w.scales, aq, as, y, isums, M, w.N, w.K, ldy, accf)
     if (q4) {
         if (isums) FH_GEMM_LAUNCH(true, true, true);
         else if (exact) FH_GEMM_LAUNCH(true, false, true);

@@ -388,7 +388,7 @@ void launch_one(GemvArgs a, hipStream_t s) {
     uint32_t grid = ngroups;
     if (grid > 256 * 8) grid = 256 * 8;
     const size_t lds = EPI == Epi::Isums ? 0 : (size_t)WAVES * a.rc * (nblk + 1) * sizeof(float);
-    gemv_kernel<Q4, NCH, (EPI == Epi::SiluQuant ? (RW > 4 ? 4 : RW) : RW), WAVES, PRO, EPI><<<grid, WAVES * 64, lds + tail, s>>>(a);
+    fh::launch(gemv_kernel<Q4, NCH, (EPI == Epi::SiluQuant ? (RW > 4 ? 4 : RW) : RW), WAVES, PRO, EPI>, grid, WAVES * 64, lds + tail, s, a);
 }
 
 template <Pro PRO, Epi EPI>

@@ -67,8 +67,9 @@ struct forge_hip_model {
     bool use_graph = true;
     bool fuse_norm = false, fuse_silu = false;   // fused GEMV prologue/epilogue variants fit LDS for this model
     hipGraphExec_t decode_graph = nullptr;
-    // forward_profile: while `prof_on`, every launch is bracketed by a pair of events tagged with its stage
-    bool prof_on = false;
+    // forward_profile / prefill_profile: one event pair per kernel launch, tagged with the stage of the
+    // enclosing StageMark (ST_COUNT = outside any stage, not measured)
+    int prof_cur = 0;
     std::vector<hipEvent_t> prof_ev;
     std::vector<int> prof_stage;
     size_t prof_used = 0;
@@ -96,29 +97,41 @@ enum Stage { ST_EMBED = 0, ST_RMSNORM, ST_QKV, ST_ROPE, ST_ATTN, ST_QUANT, ST_O,
              ST_ARGMAX, ST_COUNT };
 static_assert(ST_COUNT == FORGE_HIP_NUM_STAGES, "stage table out of step with forge_hip.h");
 
-// Brackets the launches of one scope with two events while the model is profiling.
+// While the model is profiling, names the stage that the launches of one scope are counted under.
 struct StageMark {
     forge_hip_model* m;
-    StageMark(forge_hip_model* model, int stage) : m(model) {
-        if (!m->prof_on) return;
+    int saved;
+    StageMark(forge_hip_model* model, int stage) : m(model), saved(model->prof_cur) { m->prof_cur = stage; }
+    ~StageMark() { m->prof_cur = saved; }
+};
+
+// Hands every kernel launch of a profiled pass its own pair of events (fh::launch attaches them to the
+// dispatch) and remembers the stage it belongs to.
+struct ModelProbe : LaunchProbe {
+    forge_hip_model* m;
+    explicit ModelProbe(forge_hip_model* model) : m(model) {
+        m->prof_used = 0; m->prof_stage.clear(); m->prof_cur = ST_COUNT;
+        launch_probe() = this;
+    }
+    ~ModelProbe() override { launch_probe() = nullptr; }
+    bool next(hipEvent_t* start, hipEvent_t* stop) override {
+        if (m->prof_cur == ST_COUNT) return false;
         if (m->prof_used + 2 > m->prof_ev.size()) {
             for (int i = 0; i < 2; i++) {
                 hipEvent_t e = nullptr;
-                if (hipEventCreate(&e) != hipSuccess) { m->prof_on = false; return; }
+                if (hipEventCreate(&e) != hipSuccess) return false;
                 m->prof_ev.push_back(e);
             }
         }
-        m->prof_stage.push_back(stage);
-        (void)hipEventRecord(m->prof_ev[m->prof_used], m->stream);
-    }
-    ~StageMark() {
-        if (!m->prof_on) return;
-        (void)hipEventRecord(m->prof_ev[m->prof_used + 1], m->stream);
+        *start = m->prof_ev[m->prof_used];
+        *stop = m->prof_ev[m->prof_used + 1];
+        m->prof_stage.push_back(m->prof_cur);
         m->prof_used += 2;
+        return true;
     }
 };
 
-// Sum the bracketed times per stage (milliseconds) after the stream has drained.
+// Sum the kernels' device times per stage (milliseconds) after the stream has drained.
 int32_t collect_profile(forge_hip_model* m, float* stage_ms, uint32_t* stage_launches) {
     for (int i = 0; i < ST_COUNT; i++) { stage_ms[i] = 0.f; if (stage_launches) stage_launches[i] = 0; }
     for (size_t i = 0; i * 2 < m->prof_used; i++) {
@@ -485,9 +498,10 @@ int32_t forge_hip_forward_profile(forge_hip_model* m, uint32_t token, float* sta
     if (token >= m->cfg.vocab) return fail(FORGE_HIP_ERR_POSITION, "token id out of range");
     m->h_stage[0] = token;
     FH_HIP(hipMemcpyAsync(m->d_token(), &m->h_stage[0], 4, hipMemcpyHostToDevice, m->stream));
-    m->prof_on = true; m->prof_used = 0; m->prof_stage.clear();
-    enqueue_decode_step(m);            // eager launches, each bracketed by events
-    m->prof_on = false;
+    {
+        ModelProbe probe(m);
+        enqueue_decode_step(m);        // eager launches, each carrying its own pair of events
+    }
     FH_HIP(hipGetLastError());
     FH_HIP(hipStreamSynchronize(m->stream));
     m->pos += 1;
@@ -497,10 +511,13 @@ int32_t forge_hip_forward_profile(forge_hip_model* m, uint32_t token, float* sta
 int32_t forge_hip_prefill_profile(forge_hip_model* m, const uint32_t* tokens, uint64_t n, float* stage_ms,
                                   uint32_t* stage_launches) {
     FH_CHECK(m && stage_ms, "prefill_profile: null pointer");
-    m->prof_on = true; m->prof_used = 0; m->prof_stage.clear();
-    int32_t rc = forge_hip_prefill_batch(m, tokens, n, nullptr);
-    m->prof_on = false;
+    int32_t rc;
+    {
+        ModelProbe probe(m);
+        rc = forge_hip_prefill_batch(m, tokens, n, nullptr);
+    }
     if (rc) return rc;
+    FH_HIP(hipStreamSynchronize(m->stream));
     return collect_profile(m, stage_ms, stage_launches);
 }
 

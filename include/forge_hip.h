@@ -90,9 +90,10 @@ int32_t forge_hip_forward_greedy(forge_hip_model* m, uint32_t token, uint32_t* n
 int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens_host, uint64_t n, float* logits_host);
 
 /* MetalModel::forward_profile (metal:5307-5330: one decode step with a wait per stage, timings
- * printed).  Here: one decode step launched eagerly with a pair of events around every kernel
- * launch; stage_ms_host[FORGE_HIP_NUM_STAGES] receives the summed device time per stage in
- * milliseconds, stage_launches_host (may be NULL) the number of launches.  The position advances
+ * printed).  Here: one decode step launched eagerly with a pair of events attached to every kernel
+ * dispatch (begin and end of the kernel itself, the times a kernel trace reports);
+ * stage_ms_host[FORGE_HIP_NUM_STAGES] receives the summed kernel time per stage in milliseconds,
+ * stage_launches_host (may be NULL) the number of kernel launches.  The position advances
  * like forward(); no logits are returned.  prefill_profile does the same for a batched prefill. */
 #define FORGE_HIP_NUM_STAGES 12
 #define FORGE_HIP_STAGE_NAMES                                                                                  \
