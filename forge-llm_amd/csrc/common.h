@@ -7,6 +7,7 @@
 #include <stdint.h>
 
 #include <string>
+#include <vector>
 
 #include "forge_hip.h"
 
@@ -155,5 +156,27 @@ bool attn_head_dim_supported(uint32_t hd);
 void launch_attn_exact(bool batch_order, const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc,
                        float* out, uint32_t out_stride, int8_t* oq, uint16_t* osc, uint32_t M, uint32_t base_pos,
                        const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s);
+
+// decode_persistent.hip — the whole decode step as one resident kernel (fast mode only)
+struct PdLayerIn {
+    const QWeight* qkv;
+    const QWeight* o;
+    const QWeight* gate_up;
+    const QWeight* down;
+    const float* attn_norm;
+    const float* ffn_norm;
+    uint16_t* kc;
+    uint16_t* vc;
+};
+struct PdState;
+// Leaves *out null (returning OK) when the shape or device is not covered; `state` = {position, token, next token, abort flag}.
+int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layers, const QWeight& lm_head, const float* embed,
+                  const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, PdState** out);
+void pd_destroy(PdState* st);
+int32_t pd_enqueue(PdState* st, bool profile, hipStream_t s);
+// Call with the abort flag read back after the stream drained; resets the exchange buffers and fails if it is set.
+int32_t pd_after_sync(PdState* st, uint32_t abort_flag, hipStream_t s);
+// Milliseconds between the phase starts of the last profiled step: six per layer, then head and argmax.
+int32_t pd_phase_ms(PdState* st, std::vector<float>* out, hipStream_t s);
 
 }  // namespace fh

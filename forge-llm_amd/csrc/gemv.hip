@@ -28,6 +28,7 @@
 #include "common.h"
 #include "device_utils.h"
 #include "expf_ref.h"
+#include "gemv_order.h"
 
 namespace fh {
 
@@ -42,7 +43,6 @@ __device__ __forceinline__ int dot16(int4 w, int4 a, int acc) {
 enum class Pro { Quant, RmsNorm };
 enum class Epi { Store, Add, RopeKv, SiluQuant, Isums };
 
-struct Segment { uint32_t start, len, chunk; };   // one reference matmul inside a fused matrix
 
 struct GemvArgs {
     const uint8_t* qs;
@@ -75,44 +75,8 @@ struct GemvArgs {
     uint32_t inter;
 };
 
-// Ordered sum of one row's block products p[0..nblk): sequential, or the dot1 order.
-__device__ __forceinline__ float ordered_sum(const float* p, uint32_t nblk, bool dot1) {
-    if (!dot1) {
-        float r = 0.f;
-        uint32_t b = 0;
-        for (; b + 8 <= nblk; b += 8) {          // eight LDS reads in flight, then the dependent adds
-            float v[8];
-#pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = p[b + i];
-#pragma unroll
-            for (int i = 0; i < 8; i++) r = r + v[i];
-        }
-        for (; b < nblk; b++) r = r + p[b];
-        return r;
-    }
-    float fa0 = 0.f, fa1 = 0.f, fa2 = 0.f, fa3 = 0.f;
-    const uint32_t groups = nblk / 4;
-    for (uint32_t g = 0; g < groups; g++) {
-        fa0 = fa0 + p[4 * g]; fa1 = fa1 + p[4 * g + 1]; fa2 = fa2 + p[4 * g + 2]; fa3 = fa3 + p[4 * g + 3];
-    }
-    const uint32_t tail = groups * 4;
-    if (tail < nblk) fa0 = fa0 + p[tail];
-    if (tail + 1 < nblk) fa1 = fa1 + p[tail + 1];
-    if (tail + 2 < nblk) fa2 = fa2 + p[tail + 2];
-    return ((fa0 + fa1) + fa2) + fa3;
-}
-
 __device__ __forceinline__ bool row_is_dot1(uint32_t row, const GemvArgs& a) {
-    for (uint32_t s = 0; s < a.nseg; s++) {
-        const Segment sg = a.seg[s];
-        if (row >= sg.start && row < sg.start + sg.len) {
-            const uint32_t i = row - sg.start;
-            const uint32_t base = sg.chunk ? (i / sg.chunk) * sg.chunk : 0;
-            const uint32_t len = sg.chunk ? min(sg.chunk, sg.len - base) : sg.len;
-            return (i - base) >= len - (len % a.tail_mod);
-        }
-    }
-    return false;
+    return segment_row_is_dot1(row, a.seg, a.nseg, a.tail_mod);
 }
 
 template <bool Q4, int NCH, int RW, int WAVES, Pro PRO, Epi EPI>
@@ -416,20 +380,10 @@ void dispatch(uint32_t wdtype, const GemvArgs& a, hipStream_t s) {
     }
 }
 
-// matmul_vec chunks rows by 256 once the matrix reaches 1 MB of GGUF bytes (emit.rs:1937,1971); the
-// lm_head GEMV always chunks, with an 8-row tail rule after batched prefill (emit.rs:5455-5470).
-Segment make_segment(uint32_t wdtype, uint32_t K, uint32_t start, uint32_t len, GemvOrder order) {
-    const size_t raw_bytes = (size_t)len * (K / 32) * (wdtype == FORGE_HIP_Q8_0 ? 34 : 18);
-    Segment sg;
-    sg.start = start; sg.len = len;
-    sg.chunk = (order != GemvOrder::MatmulVec || raw_bytes >= 1000000) ? 256 : 0;
-    return sg;
-}
-
 GemvArgs base_args(const QWeight& w, GemvOrder order) {
     GemvArgs a{};
     a.qs = w.qs; a.ws = w.scales; a.K = w.K; a.N = w.N;
-    a.nseg = 1; a.seg[0] = make_segment(w.wdtype, w.K, 0, w.N, order);
+    a.nseg = 1; a.seg[0] = make_segment(w.wdtype, w.K, 0, w.N, order != GemvOrder::MatmulVec);
     a.tail_mod = order == GemvOrder::LmHeadAfterPrefill ? 8 : 4;
     return a;
 }
@@ -477,9 +431,9 @@ void launch_gemv_norm_rope_kv(const QWeight& wqkv, const float* x, const float* 
     a.q_out = q_out; a.kc = kc; a.vc = vc; a.cos_t = cos_t; a.sin_t = sin_t; a.pos_dev = pos_dev;
     a.qks = heads * hd; a.kv = kv_heads * hd; a.hd = hd;
     a.nseg = 3;
-    a.seg[0] = make_segment(wqkv.wdtype, wqkv.K, 0, a.qks, GemvOrder::MatmulVec);
-    a.seg[1] = make_segment(wqkv.wdtype, wqkv.K, a.qks, a.kv, GemvOrder::MatmulVec);
-    a.seg[2] = make_segment(wqkv.wdtype, wqkv.K, a.qks + a.kv, a.kv, GemvOrder::MatmulVec);
+    a.seg[0] = make_segment(wqkv.wdtype, wqkv.K, 0, a.qks, false);
+    a.seg[1] = make_segment(wqkv.wdtype, wqkv.K, a.qks, a.kv, false);
+    a.seg[2] = make_segment(wqkv.wdtype, wqkv.K, a.qks + a.kv, a.kv, false);
     dispatch<Pro::RmsNorm, Epi::RopeKv>(wqkv.wdtype, a, s);
 }
 
@@ -488,8 +442,8 @@ void launch_gemv_norm_silu_quant(const QWeight& wgu, const float* x, const float
     GemvArgs a = base_args(wgu, GemvOrder::MatmulVec);
     a.x = x; a.norm_w = norm_w; a.eps = eps; a.oq = oq; a.osc = osc; a.inter = wgu.N / 2;
     a.nseg = 2;
-    a.seg[0] = make_segment(wgu.wdtype, wgu.K, 0, a.inter, GemvOrder::MatmulVec);
-    a.seg[1] = make_segment(wgu.wdtype, wgu.K, a.inter, a.inter, GemvOrder::MatmulVec);
+    a.seg[0] = make_segment(wgu.wdtype, wgu.K, 0, a.inter, false);
+    a.seg[1] = make_segment(wgu.wdtype, wgu.K, a.inter, a.inter, false);
     dispatch<Pro::RmsNorm, Epi::SiluQuant>(wgu.wdtype, a, s);
 }
 

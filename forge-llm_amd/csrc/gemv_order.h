@@ -1,0 +1,69 @@
+// The order in which the reference's decode GEMV adds a row's per-block products, shared by the
+// GEMV kernels: which rows take the four-accumulator (dot1) order and the ordered sum itself.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "forge_hip.h"
+
+namespace fh {
+
+// One reference matmul inside a (possibly fused) matrix: rows [start, start+len), processed by the
+// reference in chunks of `chunk` rows (0 = unchunked).
+struct Segment { uint32_t start, len, chunk; };
+
+// matmul_vec chunks rows by 256 once the matrix reaches 1 MB of GGUF bytes (emit.rs:1937,1971); the
+// lm_head GEMV always chunks (emit.rs:5455-5470).
+inline Segment make_segment(uint32_t wdtype, uint32_t K, uint32_t start, uint32_t len, bool always_chunk) {
+    const size_t raw_bytes = (size_t)len * (K / 32) * (wdtype == FORGE_HIP_Q8_0 ? 34 : 18);
+    Segment sg;
+    sg.start = start; sg.len = len;
+    sg.chunk = (always_chunk || raw_bytes >= 1000000) ? 256 : 0;
+    return sg;
+}
+
+// Rows of a chunk are taken 8 (then 4) at a time by dot8/dot4; the last len % tail_mod rows of each chunk go
+// through dot1, whose block products are added by four interleaved accumulators (emit.rs:1558-1571).
+__device__ __forceinline__ bool segment_row_is_dot1(uint32_t row, const Segment* seg, uint32_t nseg, uint32_t tail_mod) {
+    for (uint32_t s = 0; s < nseg; s++) {
+        const Segment sg = seg[s];
+        if (row >= sg.start && row < sg.start + sg.len) {
+            const uint32_t i = row - sg.start;
+            const uint32_t base = sg.chunk ? (i / sg.chunk) * sg.chunk : 0;
+            const uint32_t len = sg.chunk ? min(sg.chunk, sg.len - base) : sg.len;
+            return (i - base) >= len - (len % tail_mod);
+        }
+    }
+    return false;
+}
+
+// Ordered sum of one row's block products p[0..nblk): sequential (dot8/dot4, emit.rs:1770-1877), or the
+// dot1 order.  Adds are never fused with the multiplies that made the products.
+__device__ __forceinline__ float ordered_sum(const float* p, uint32_t nblk, bool dot1) {
+    if (!dot1) {
+        float r = 0.f;
+        uint32_t b = 0;
+        for (; b + 8 <= nblk; b += 8) {          // eight LDS reads in flight, then the dependent adds
+            float v[8];
+#pragma unroll
+            for (int i = 0; i < 8; i++) v[i] = p[b + i];
+#pragma unroll
+            for (int i = 0; i < 8; i++) r = r + v[i];
+        }
+        for (; b < nblk; b++) r = r + p[b];
+        return r;
+    }
+    float fa0 = 0.f, fa1 = 0.f, fa2 = 0.f, fa3 = 0.f;
+    const uint32_t groups = nblk / 4;
+    for (uint32_t g = 0; g < groups; g++) {
+        fa0 = fa0 + p[4 * g]; fa1 = fa1 + p[4 * g + 1]; fa2 = fa2 + p[4 * g + 2]; fa3 = fa3 + p[4 * g + 3];
+    }
+    const uint32_t tail = groups * 4;
+    if (tail < nblk) fa0 = fa0 + p[tail];
+    if (tail + 1 < nblk) fa1 = fa1 + p[tail + 1];
+    if (tail + 2 < nblk) fa2 = fa2 + p[tail + 2];
+    return ((fa0 + fa1) + fa2) + fa3;
+}
+
+}  // namespace fh

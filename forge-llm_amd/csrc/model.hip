@@ -67,6 +67,7 @@ struct forge_hip_model {
     bool use_graph = true;
     bool fuse_norm = false, fuse_silu = false;   // fused GEMV prologue/epilogue variants fit LDS for this model
     hipGraphExec_t decode_graph = nullptr;
+    PdState* pd = nullptr;               // the decode step as one resident kernel, when the shape is covered
     // forward_profile / prefill_profile: one event pair per kernel launch, tagged with the stage of the
     // enclosing StageMark (ST_COUNT = outside any stage, not measured)
     int prof_cur = 0;
@@ -82,6 +83,7 @@ struct forge_hip_model {
 
     ~forge_hip_model() {
         if (decode_graph) (void)hipGraphExecDestroy(decode_graph);
+        pd_destroy(pd);
         for (hipEvent_t e : prof_ev) (void)hipEventDestroy(e);
         for (auto& L : layers) { qweight_free(&L.qkv); qweight_free(&L.o); qweight_free(&L.gate_up); qweight_free(&L.down); }
         qweight_free(&lm_head);
@@ -293,6 +295,7 @@ void enqueue_decode_step(forge_hip_model* m) {
 }
 
 int32_t run_decode_step(forge_hip_model* m) {
+    if (m->pd) return pd_enqueue(m->pd, false, m->stream);
     if (m->use_graph && !m->decode_graph) {
         hipGraph_t g = nullptr;
         FH_HIP(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
@@ -305,6 +308,14 @@ int32_t run_decode_step(forge_hip_model* m) {
     }
     if (m->decode_graph) FH_HIP(hipGraphLaunch(m->decode_graph, m->stream));
     else { enqueue_decode_step(m); FH_HIP(hipGetLastError()); }
+    return FORGE_HIP_OK;
+}
+
+// Reads back {next token, abort flag} after a decode step and waits for the stream.
+int32_t finish_decode_step(forge_hip_model* m) {
+    FH_HIP(hipMemcpyAsync(&m->h_stage[4], m->d_next(), 8, hipMemcpyDeviceToHost, m->stream));
+    FH_HIP(hipStreamSynchronize(m->stream));
+    if (m->pd) return pd_after_sync(m->pd, m->h_stage[5], m->stream);
     return FORGE_HIP_OK;
 }
 
@@ -430,6 +441,17 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
         (rc = m->paq.alloc((size_t)R * m->KMAX)) || (rc = m->pasc.alloc((size_t)R * (m->KMAX / 32) * 2)) ||
         (rc = m->ptok.alloc((size_t)R * 4)))
         return rc;
+    const char* penv = getenv("FORGE_HIP_PERSIST");
+    if (penv && penv[0] == '1') {   // opt-in while the kernel sequence is still the faster step
+        std::vector<PdLayerIn> pl(cfg->layers);
+        for (uint32_t l = 0; l < cfg->layers; l++) {
+            Layer& L = m->layers[l];
+            pl[l] = PdLayerIn{&L.qkv, &L.o, &L.gate_up, &L.down, L.attn_norm, L.ffn_norm, m->kc(l), m->vc(l)};
+        }
+        rc = pd_create(*cfg, pl, m->lm_head, m->embed.as<float>(), m->final_norm.as<float>(), m->cos_t.as<float>(),
+                       m->sin_t.as<float>(), m->logits.as<float>(), m->state.as<uint32_t>(), &m->pd);
+        if (rc) return rc;
+    }
     FH_HIP(hipDeviceSynchronize());
     *out = m.release();
     return FORGE_HIP_OK;
@@ -446,17 +468,16 @@ int32_t forge_hip_forward(forge_hip_model* m, uint32_t token, float* logits_host
     int32_t rc = forward_common(m, token);
     if (rc) return rc;
     FH_HIP(hipMemcpyAsync(logits_host, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, m->stream));
-    FH_HIP(hipStreamSynchronize(m->stream));
-    return FORGE_HIP_OK;
+    return finish_decode_step(m);
 }
 
 int32_t forge_hip_forward_greedy(forge_hip_model* m, uint32_t token, uint32_t* next_token_host) {
     FH_CHECK(next_token_host, "forward_greedy: null out");
     int32_t rc = forward_common(m, token);
     if (rc) return rc;
-    FH_HIP(hipMemcpyAsync(&m->h_stage[1], m->d_next(), 4, hipMemcpyDeviceToHost, m->stream));
-    FH_HIP(hipStreamSynchronize(m->stream));
-    *next_token_host = m->h_stage[1];
+    rc = finish_decode_step(m);
+    if (rc) return rc;
+    *next_token_host = m->h_stage[4];
     return FORGE_HIP_OK;
 }
 
@@ -498,6 +519,26 @@ int32_t forge_hip_forward_profile(forge_hip_model* m, uint32_t token, float* sta
     if (token >= m->cfg.vocab) return fail(FORGE_HIP_ERR_POSITION, "token id out of range");
     m->h_stage[0] = token;
     FH_HIP(hipMemcpyAsync(m->d_token(), &m->h_stage[0], 4, hipMemcpyHostToDevice, m->stream));
+    if (m->pd) {
+        // one kernel: the stages are its phases, timed by the kernel's own clock stamps
+        int32_t rc = pd_enqueue(m->pd, true, m->stream);
+        if (rc) return rc;
+        rc = finish_decode_step(m);
+        if (rc) return rc;
+        m->pos += 1;
+        std::vector<float> ph;
+        rc = pd_phase_ms(m->pd, &ph, m->stream);
+        if (rc) return rc;
+        for (int i = 0; i < ST_COUNT; i++) { stage_ms[i] = 0.f; if (stage_launches) stage_launches[i] = 0; }
+        static const int phase_stage[6] = {ST_QKV, ST_ATTN, ST_ATTN, ST_O, ST_GATE_UP, ST_DOWN};
+        for (size_t i = 0; i < ph.size(); i++) {
+            const size_t nl = 6 * (size_t)m->cfg.layers;
+            const int st = i < nl ? phase_stage[i % 6] : (i == nl ? ST_LM_HEAD : ST_ARGMAX);
+            stage_ms[st] += ph[i];
+            if (stage_launches) stage_launches[st] += 1;
+        }
+        return FORGE_HIP_OK;
+    }
     {
         ModelProbe probe(m);
         enqueue_decode_step(m);        // eager launches, each carrying its own pair of events
@@ -519,6 +560,16 @@ int32_t forge_hip_prefill_profile(forge_hip_model* m, const uint32_t* tokens, ui
     if (rc) return rc;
     FH_HIP(hipStreamSynchronize(m->stream));
     return collect_profile(m, stage_ms, stage_launches);
+}
+
+int32_t forge_hip_model_decode_launches(const forge_hip_model* m) {
+    if (!m) return -1;
+    if (m->pd) return 1;
+    const bool exact = (m->cfg.flags & FORGE_HIP_FLAG_EXACT) != 0;
+    const int attn = exact ? 1 : 2;
+    const int layer = (m->fuse_norm ? 1 : 3) + attn + 1 + (m->fuse_silu ? 1 : 3) + 1;
+    const int head = ((m->fuse_norm && m->cfg.vocab <= 16384) ? 1 : 2) + 2;
+    return 1 + (int)m->cfg.layers * layer + head;
 }
 
 int32_t forge_hip_reset(forge_hip_model* m) {

@@ -75,6 +75,11 @@ class HipModel:
         self._check(self._lib.forge_hip_reset(self._h))
 
     @property
+    def decode_launches(self) -> int:
+        """Kernel launches per decode step: 1 when the step runs as one resident kernel."""
+        return int(self._lib.forge_hip_model_decode_launches(self._h))
+
+    @property
     def pos(self) -> int:
         return int(self._lib.forge_hip_model_pos(self._h))
 

@@ -94,7 +94,10 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens_host,
  * dispatch (begin and end of the kernel itself, the times a kernel trace reports);
  * stage_ms_host[FORGE_HIP_NUM_STAGES] receives the summed kernel time per stage in milliseconds,
  * stage_launches_host (may be NULL) the number of kernel launches.  The position advances
- * like forward(); no logits are returned.  prefill_profile does the same for a batched prefill. */
+ * like forward(); no logits are returned.  prefill_profile does the same for a batched prefill.
+ * When the decode step is one resident kernel (forge_hip_model_decode_launches() == 1) its phases are the
+ * stages: the kernel stamps the device wall clock at the start of each phase and the differences are
+ * reported ("attention" = split + merge phases; "launches" then counts phases). */
 #define FORGE_HIP_NUM_STAGES 12
 #define FORGE_HIP_STAGE_NAMES                                                                                  \
     "embedding", "rms_norm", "qkv_matmul", "rope_kv_store", "attention", "quantize_act", "o_matmul", "gate_up_matmul", \
@@ -103,6 +106,11 @@ int32_t forge_hip_forward_profile(forge_hip_model* m, uint32_t token, float* sta
                                   uint32_t* stage_launches_host);
 int32_t forge_hip_prefill_profile(forge_hip_model* m, const uint32_t* tokens_host, uint64_t n, float* stage_ms_host,
                                   uint32_t* stage_launches_host);
+
+/* Kernel launches one decode step costs on this model: 1 when the whole step runs as one resident kernel
+ * (fast mode, covered shapes), otherwise the length of the kernel sequence.  The Metal backend's counterpart
+ * is the fixed encoder sequence of MetalModel::forward (metal:5070-5300). */
+int32_t forge_hip_model_decode_launches(const forge_hip_model* m);
 
 /* MetalModel::reset() (metal:5981): position back to 0. */
 int32_t forge_hip_reset(forge_hip_model* m);

@@ -146,6 +146,7 @@ def test_graph_replay_matches_eager(fh, torch_gpu, monkeypatch):
     cfg = tiny_cfg(fh, Q8, 0)
     blob = fh.synth.make_weights_blob(cfg, seed=8)
     toks = fh.synth.uniform_ids(9, 12, cfg["vocab"])
+    monkeypatch.setenv("FORGE_HIP_PERSIST", "0")          # the kernel-sequence step is what a graph captures
     monkeypatch.setenv("FORGE_HIP_GRAPH", "0")
     eager = fh.HipModel(cfg, blob)
     monkeypatch.setenv("FORGE_HIP_GRAPH", "1")
@@ -173,6 +174,65 @@ def test_fused_decode_kernels_equal_separate_kernels(fh, torch_gpu, monkeypatch,
     for which in (0, 1):
         assert np.array_equal(fused.read_kv(1, which), plain.read_kv(1, which))
     plain.close(); fused.close()
+
+
+def persistent_pair(fh, cfg, blob, monkeypatch):
+    monkeypatch.setenv("FORGE_HIP_PERSIST", "0")
+    seq = fh.HipModel(cfg, blob)
+    monkeypatch.setenv("FORGE_HIP_PERSIST", "1")
+    one = fh.HipModel(cfg, blob)
+    assert one.decode_launches == 1 and seq.decode_launches > 1
+    return seq, one
+
+
+@pytest.mark.parametrize("wd", [Q8, Q4])
+def test_persistent_decode_kernel_equals_kernel_sequence(fh, torch_gpu, monkeypatch, wd):
+    """Fast mode: the decode step as one resident kernel (tagged hand-over between workgroups instead of kernel
+    boundaries) gives the same bits as the sequence of kernels: logits, greedy tokens and the KV cache."""
+    cfg = tiny_cfg(fh, wd, 0)
+    blob = fh.synth.make_weights_blob(cfg, seed=41)
+    toks = fh.synth.uniform_ids(42, 120, cfg["vocab"])
+    seq, one = persistent_pair(fh, cfg, blob, monkeypatch)
+    for t in toks[:20]:                                     # from an empty cache, token by token
+        same_bits(one.forward(int(t)), seq.forward(int(t)))
+    seq.reset(); one.reset()
+    same_bits(one.forward_prefill(toks[:75]), seq.forward_prefill(toks[:75]))    # same prefill kernels in both
+    for t in toks[75:]:
+        assert one.forward_greedy(int(t)) == seq.forward_greedy(int(t))
+    same_bits(one.forward(7), seq.forward(7))
+    assert one.pos == seq.pos == 121
+    for layer in range(cfg["layers"]):
+        for which in (0, 1):
+            assert np.array_equal(one.read_kv(layer, which), seq.read_kv(layer, which))
+    seq.close(); one.close()
+
+
+@pytest.mark.parametrize("shape", ["smollm2_135m", "llama_1b_2layers"])
+def test_persistent_decode_kernel_real_shapes(fh, torch_gpu, monkeypatch, shape):
+    """Same check on the shapes that matter: SmolLM2-135M (hidden 576, 9 heads over 3 KV heads: partial weight
+    units, three heads per group) and the Llama-3.2-1B layer shape at a context that spans every split."""
+    if shape == "smollm2_135m":
+        cfg = fh.synth.smollm2_135m(Q8, max_seq=1024)
+        n_prompt = 300
+    else:
+        cfg = fh.synth.llama32_1b(Q8, max_seq=2048)
+        cfg["layers"], cfg["vocab"] = 2, 32000
+        n_prompt = 1500
+    blob = fh.synth.make_weights_blob(cfg, seed=77, threads=16)
+    toks = fh.synth.uniform_ids(78, n_prompt + 12, cfg["vocab"])
+    seq, one = persistent_pair(fh, cfg, blob, monkeypatch)
+    seq.forward_prefill_batch(toks[:n_prompt]); one.forward_prefill_batch(toks[:n_prompt])
+    for t in toks[n_prompt:n_prompt + 6]:
+        same_bits(one.forward(int(t)), seq.forward(int(t)))
+    a = b = int(toks[n_prompt + 6])
+    for _ in range(6):
+        a, b = one.forward_greedy(a), seq.forward_greedy(b)
+        assert a == b
+    assert np.array_equal(one.read_kv(cfg["layers"] - 1, 0), seq.read_kv(cfg["layers"] - 1, 0))
+    prof = one.forward_profile(a)                           # the stamped run is an ordinary step
+    assert prof["lm_head_matmul"][0] > 0 and prof["qkv_matmul"][1] == cfg["layers"]
+    assert one.forward_greedy(3) is not None
+    seq.close(); one.close()
 
 
 def test_smollm2_135m_greedy_64_tokens_identical(fh, oracle, torch_gpu):
