@@ -26,10 +26,19 @@
 // leaves, and the host reports an error instead of hanging.
 //
 // Weights do not depend on activations: each phase issues the loads of its first weight units before it
-// starts waiting for its inputs, so HBM latency overlaps the hand-over.
+// starts waiting for its inputs, so HBM latency overlaps the hand-over.  Vector loads of a wave return in
+// issue order on this architecture, so a wave that has weights in flight cannot see a polled element
+// before those weights have landed.  The waves of a workgroup are therefore split: the first
+// PD_POLL_WAVES ("pollers") fetch the phase's input first and issue their weight loads afterwards, the
+// others ("streamers") issue weight loads at once and touch no other global memory until they consume
+// them.  For the same reason the per-layer descriptors travel as kernel arguments (scalar loads, a
+// counter of their own) and everything a wave needs besides weights (norm weights, rope factors, the
+// residual) is requested before its weights are.
 //
 // The arithmetic is that of the separate kernels (gemv.hip, attn_decode.hip, elementwise.hip), value for
 // value: the same block products, the same ordered sums, the same split boundaries and merge order.
+#include <stddef.h>
+
 #include <algorithm>
 #include <memory>
 #include <vector>
@@ -43,12 +52,18 @@ namespace fh {
 
 namespace {
 
-constexpr int PD_THREADS = 1024;
+constexpr int PD_THREADS = 512;
 constexpr int PD_WAVES = PD_THREADS / 64;
-constexpr int PD_D = 8;                       // weight units (1 KB) a wave holds in registers per round
+constexpr int PD_D = 16;                      // weight units (1 KB) a wave holds in registers per round
 constexpr uint32_t PD_MAX_TILE_ROWS = 128;
 constexpr uint32_t PD_LDS_BYTES = 64 * 1024;
 constexpr uint32_t PD_MISC_BYTES = 2048;
+constexpr int PD_POLL_WAVES = 2;              // waves that fetch a phase's input; the others stream weights
+constexpr int PD_POLL_THREADS = PD_POLL_WAVES * 64;
+constexpr int PD_STREAM_WAVES = PD_WAVES - PD_POLL_WAVES;
+constexpr int PD_POLL_N = 20;                 // tagged elements a poller thread takes per round trip
+// misc LDS (floats): [0,32) norm partial sums, [40] hint flag, [64,128) phase scratch
+constexpr int PD_MISC_HINT = 40, PD_MISC_SCRATCH = 64;
 
 struct PdGemv {
     const uint8_t* qs;
@@ -60,16 +75,20 @@ struct PdGemv {
     Segment seg[3];
 };
 
+// What differs from layer to layer: addresses only.  The shapes of the four matrices are shared.
 struct PdLayer {
-    PdGemv qkv, o, gu, down;
+    const uint8_t* qs[4];      // qkv, o, gate_up, down
+    const uint16_t* ws[4];
     const float* attn_norm;
     const float* ffn_norm;
     uint16_t* kc;
     uint16_t* vc;
 };
+constexpr uint32_t PD_MAX_LAYERS = 34;       // the descriptors travel as kernel arguments (4 KB in all)
+enum { PD_QKV = 0, PD_O = 1, PD_GU = 2, PD_DOWN = 3 };
 
 struct PdArgs {
-    const PdLayer* layers;
+    PdGemv shape[4];           // qkv, o, gate_up, down with null addresses
     PdGemv lm;
     uint32_t n_layers, H, I, QKS, KV, heads, kv_heads, gt;
     float eps;
@@ -88,9 +107,44 @@ struct PdArgs {
     float* logits;
     uint32_t* state;   // [0] position  [1] token  [2] next token  [3] abort flag
     uint32_t tag_base, spin_limit;
+    uint32_t q4, lm_q4;                        // weight formats: projections, lm_head
     uint32_t off_act_s, off_misc, off_big;     // LDS byte offsets (activation codes sit at 0)
     unsigned long long* stamps;                // optional: wall clock at the start of every phase (workgroup 0)
+    // Kernel arguments are read with scalar loads, which have their own completion counter: a wave can
+    // fetch a descriptor while its weight loads are in flight without waiting for them.
+    PdLayer layers[PD_MAX_LAYERS];
 };
+static_assert(sizeof(PdArgs) <= 4096, "kernel arguments exceed 4 KB");
+
+// ---- plain global accesses -------------------------------------------------------------------------------
+// Pointers that reach the kernel through descriptors in memory have lost their address space; a load through
+// them would be a FLAT instruction, whose completion the compiler can only order with a full wait.  These
+// say "global" explicitly.
+typedef uint32_t pd_u32x4 __attribute__((ext_vector_type(4)));
+template <typename T>
+__device__ __forceinline__ T ldg(const T* p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    if constexpr (sizeof(T) == 16) {
+        const pd_u32x4 v = *(const __attribute__((address_space(1))) pd_u32x4*)(uintptr_t)p;
+        T r;
+        __builtin_memcpy(&r, &v, 16);
+        return r;
+    } else {
+        static_assert(sizeof(T) <= 8, "ldg: scalar or 16-byte types only");
+        return *(const __attribute__((address_space(1))) T*)(uintptr_t)p;
+    }
+#else
+    return *p;
+#endif
+}
+template <typename T>
+__device__ __forceinline__ void stg(T* p, T v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    *(__attribute__((address_space(1))) T*)(uintptr_t)p = v;
+#else
+    *p = v;
+#endif
+}
 
 // ---- coherent (agent-scope, L2-bypassing) accesses ----------------------------------------------------
 __device__ __forceinline__ uint64_t ldc64(const uint64_t* p) {
@@ -125,19 +179,37 @@ __device__ __forceinline__ uint32_t poll(const uint64_t* p, uint32_t tag, const 
     return (uint32_t)w;
 }
 
+// Thousands of threads re-reading a buffer that is not ready yet would flood the memory fabric the weight
+// stream needs.  After a first attempt that found something missing, the pollers of a workgroup therefore
+// wait (on an LDS flag) until thread 0 has seen one watched element of the buffer arrive, which in a
+// balanced phase is when the rest is about to.
+struct Hint { const uint64_t* sentinel; volatile uint32_t* flag; };
+
 // Up to N elements per thread: all loads are issued before any tag is looked at, so a hand-over costs one
 // memory round trip however many elements a thread takes; only elements still carrying another tag are re-read.
 template <int N, typename Addr>
-__device__ __forceinline__ void poll_many(Addr addr, uint32_t n, uint32_t tag, uint32_t* out, const PdCtx& cx) {
+__device__ __forceinline__ void poll_many(Addr addr, uint32_t n, uint32_t tag, uint32_t* out, const PdCtx& cx, Hint hint) {
     uint64_t w[N];
 #pragma unroll
     for (int i = 0; i < N; i++) w[i] = (uint32_t)i < n ? ldc64(addr(i)) : ((uint64_t)tag << 32);
+    if (hint.flag && cx.tid == 0) {
+        (void)poll(hint.sentinel, tag, cx);
+        *hint.flag = tag;
+    }
     uint32_t spins = 0;
+    bool waited = hint.flag == nullptr;
     for (;;) {
         bool ok = true;
 #pragma unroll
         for (int i = 0; i < N; i++) ok = ok && (uint32_t)(w[i] >> 32) == tag;
         if (ok) break;
+        if (!waited) {
+            uint32_t s2 = 0;
+            while (*hint.flag != tag && *cx.sh_abort == 0 && ++s2 < cx.spin_limit) __builtin_amdgcn_s_sleep(4);
+            waited = true;
+        } else {
+            __builtin_amdgcn_s_sleep(2);
+        }
         ++spins;
         if (spins > cx.spin_limit ||
             ((spins & 1023u) == 0 && __hip_atomic_load(cx.abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
@@ -145,7 +217,6 @@ __device__ __forceinline__ void poll_many(Addr addr, uint32_t n, uint32_t tag, u
             __hip_atomic_store(cx.abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             break;
         }
-        __builtin_amdgcn_s_sleep(2);
 #pragma unroll
         for (int i = 0; i < N; i++)
             if ((uint32_t)(w[i] >> 32) != tag) w[i] = ldc64(addr(i));
@@ -154,25 +225,21 @@ __device__ __forceinline__ void poll_many(Addr addr, uint32_t n, uint32_t tag, u
     for (int i = 0; i < N; i++) out[i] = (uint32_t)w[i];
 }
 
-// A whole vector of `count` elements, four per thread and pass; `put(index, payload)` stores each.
-template <typename Put>
-__device__ __forceinline__ void poll_vec(const uint64_t* base, uint32_t count, uint32_t tag, const PdCtx& cx, Put put) {
-    for (uint32_t i0 = cx.tid; i0 < count; i0 += 4 * PD_THREADS) {
-        uint32_t v[4];
-        const uint32_t n = (count - i0 + PD_THREADS - 1) / PD_THREADS;
-        poll_many<4>([&](int i) { return base + i0 + (uint32_t)i * PD_THREADS; }, n < 4 ? n : 4, tag, v, cx);
+// A whole vector of `count` elements fetched by the first `nthreads` threads of the workgroup, N per thread and
+// round trip; `put(index, payload)` stores each.  Threads past nthreads return at once.
+template <int N, typename Put>
+__device__ __forceinline__ void poll_vec(const uint64_t* base, uint32_t count, uint32_t tag, uint32_t nthreads, const PdCtx& cx,
+                                         Hint hint, Put put) {
+    if (cx.tid >= nthreads) return;
+    for (uint32_t i0 = cx.tid; i0 < count; i0 += N * nthreads) {
+        uint32_t v[N];
+        const uint32_t n = (count - i0 + nthreads - 1) / nthreads;
+        poll_many<N>([&](int i) { return base + i0 + (uint32_t)i * nthreads; }, n < (uint32_t)N ? n : (uint32_t)N, tag, v, cx, hint);
+        hint.flag = nullptr;      // later passes: the buffer is known to be arriving
 #pragma unroll
-        for (int i = 0; i < 4; i++)
-            if (i0 + (uint32_t)i * PD_THREADS < count) put(i0 + (uint32_t)i * PD_THREADS, v[i]);
+        for (int i = 0; i < N; i++)
+            if (i0 + (uint32_t)i * nthreads < count) put(i0 + (uint32_t)i * nthreads, v[i]);
     }
-}
-
-// Thousands of threads re-reading a buffer that is not ready yet would flood the memory fabric the weight
-// stream needs.  One lane per workgroup watches a single element first; the full read starts when that
-// element has arrived, which in a balanced phase is when the rest is about to.
-__device__ __forceinline__ void wait_hint(const uint64_t* sentinel, uint32_t tag, const PdCtx& cx) {
-    if (cx.tid == 0) (void)poll(sentinel, tag, cx);
-    __syncthreads();
 }
 
 __device__ __forceinline__ int dot16(int4 w, int4 a, int acc) {
@@ -185,8 +252,9 @@ __device__ __forceinline__ int dot16(int4 w, int4 a, int acc) {
 
 // ---- prologues: the activation vector of a GEMV phase, quantised, in LDS ------------------------------
 // rms_norm (emit.rs:327-334, 16-lane FMA order of emit.rs:272-295) + activation quantiser (emit.rs:1410-1440).
-// xs must already hold x[0..H); `part` is 32 floats of LDS.
-__device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict__ norm_w, float eps, uint32_t H,
+// xs must already hold x[0..H); `part` is 32 floats of LDS; nw0 = norm_w[4 tid .. 4 tid + 4), requested by the
+// caller before any weight load of this wave.
+__device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict__ norm_w, float4 nw0, float eps, uint32_t H,
                                               uint32_t* aq_lds, float* as_lds, float* part, const PdCtx& cx) {
     const uint32_t tid = cx.tid;
     __syncthreads();
@@ -216,7 +284,7 @@ __device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict
     const float inv_rms = 1.0f / sqrtf(part[16] / (float)H + eps);
     for (uint32_t e0 = tid * 4; e0 < H; e0 += PD_THREADS * 4) {
         const float4 xv = *reinterpret_cast<const float4*>(xs + e0);
-        const float4 wv = *reinterpret_cast<const float4*>(norm_w + e0);
+        const float4 wv = e0 == tid * 4 ? nw0 : ldg(reinterpret_cast<const float4*>(norm_w + e0));
         const float4 v = make_float4(xv.x * inv_rms * wv.x, xv.y * inv_rms * wv.y, xv.z * inv_rms * wv.z, xv.w * inv_rms * wv.w);
         uint16_t sb;
         const uint32_t pk = quantize_block_part(v, sb);
@@ -226,123 +294,125 @@ __device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict
     __syncthreads();
 }
 
-// An already quantised vector (codes then scales, tagged) from another phase.
+// An already quantised vector (codes then scales, tagged) from another phase; fetched by the poller waves.
 __device__ __forceinline__ void pd_load_aq(const uint64_t* t, uint32_t tag, uint32_t K, uint32_t* aq_lds, float* as_lds,
-                                           const PdCtx& cx) {
+                                           float* misc, const PdCtx& cx) {
     const uint32_t nq = K / 4, ns = K / 32;
-    wait_hint(t + nq + ns - 1, tag, cx);
-    poll_vec(t, nq + ns, tag, cx, [&](uint32_t i, uint32_t p) {
+    const Hint hint{t + nq + ns - 1, reinterpret_cast<volatile uint32_t*>(misc + PD_MISC_HINT)};
+    poll_vec<PD_POLL_N>(t, nq + ns, tag, PD_POLL_THREADS, cx, hint, [&](uint32_t i, uint32_t p) {
         if (i < nq) aq_lds[i] = p;
         else as_lds[i - nq] = f16_bits_to_f32((uint16_t)p);
     });
-    __syncthreads();
+}
+
+// The residual stream (tagged) into LDS as floats; fetched by the poller waves.
+__device__ __forceinline__ void pd_load_x(const uint64_t* tx, uint32_t tag, uint32_t H, float* xs, float* misc, const PdCtx& cx) {
+    const Hint hint{tx + H - 1, reinterpret_cast<volatile uint32_t*>(misc + PD_MISC_HINT)};
+    poll_vec<PD_POLL_N>(tx, H, tag, PD_POLL_THREADS, cx, hint, [&](uint32_t i, uint32_t p) { xs[i] = __uint_as_float(p); });
 }
 
 // ---- the GEMV of a phase ------------------------------------------------------------------------------
+// One generic routine serves all five matrices (its code exists once: the kernel is a loop over steps, and an
+// instruction cache that has to refill at every phase costs more than the branches).  What differs between
+// the matrices is data: the shape, where the activation vector comes from and what happens to a finished row.
+enum { PRO_NORM = 0, PRO_AQ = 1 };
+enum { EPI_ROPE = 0, EPI_ADD = 1, EPI_SILU = 2, EPI_LOGITS = 3 };
+
+struct GemvJob {
+    const PdGemv* g;           // shape, in the kernel arguments
+    const uint8_t* qs;
+    const uint16_t* ws;
+    bool q4;
+    int pro, epi;
+    const float* norm_w;       // PRO_NORM
+    const uint64_t* tin;       // tagged input: residual stream (PRO_NORM) or quantised vector (PRO_AQ)
+    uint32_t tin_tag;          // 0 with PRO_NORM: the input is the embedding row
+    uint32_t in_len;           // elements of the input vector (= K)
+    uint32_t tag_out;
+    uint32_t res_tag;          // EPI_ADD: tag of the residual's current version (0: embedding row)
+    uint16_t* kc;              // EPI_ROPE
+    uint16_t* vc;
+};
+
 struct WReg { int4 v[PD_D]; uint32_t s[PD_D]; };
 
-__device__ __forceinline__ uint32_t pd_tile_rows(const PdGemv& g, uint32_t tile) {
-    return g.inter ? 64u : min(g.T, g.N - tile * g.T);
+// Rows of a tile: [row0, row0 + split) and, for the fused [gate;up] matrix, the matching rows `jump` further on.
+// Everything here is wave-uniform and meant to live in scalar registers.
+struct TilePos {
+    uint32_t rows, row0, split, jump;
+};
+__device__ __forceinline__ TilePos pd_tile(const PdGemv& g, uint32_t tile) {
+    TilePos t;
+    if (g.inter) { t.rows = 64; t.row0 = tile * 32; t.split = 32; t.jump = g.inter - 32; }
+    else { t.rows = min(g.T, g.N - tile * g.T); t.row0 = tile * g.T; t.split = 0xFFFFFFFFu; t.jump = 0; }
+    return t;
 }
-__device__ __forceinline__ uint32_t pd_tile_row(const PdGemv& g, uint32_t tile, uint32_t lr) {
-    if (g.inter) return lr < 32 ? tile * 32 + lr : g.inter + tile * 32 + (lr - 32);
-    return tile * g.T + lr;
-}
+__device__ __forceinline__ uint32_t pd_row(const TilePos& t, uint32_t lr) { return t.row0 + lr + (lr >= t.split ? t.jump : 0u); }
+__device__ __forceinline__ uint32_t sdiv(uint32_t a, uint32_t b) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)(a / b)); }
 
-// Unit u of a tile = weight unit (u % U) of tile row (u / U); wave w takes units w, w + 16, ...; a round is
-// PD_D units per wave, all loads issued before any is used.
+// The weight streamers of a workgroup (waves PD_POLL_WAVES .. PD_WAVES-1, numbered sw = 0 .. PD_STREAM_WAVES-1) split a
+// tile by rows: streamer sw takes tile rows sw, sw + PD_STREAM_WAVES, ... and walks each row's U weight units (1 KB:
+// 32 Q8_0 blocks, two lanes per block, or 64 Q4_0 blocks) in order.  Position p of that walk is unit p % U of the
+// wave's (p / U)-th row; a round is PD_D consecutive positions, all loaded before any is used.
 template <bool Q4>
-__device__ __forceinline__ void pd_load_round(const PdGemv& g, uint32_t tile, uint32_t round, const PdCtx& cx, WReg& W) {
-    const uint32_t units = tile < g.ntiles ? pd_tile_rows(g, tile) * g.U : 0;
+__device__ __forceinline__ void pd_load_round(const GemvJob& job, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane, WReg& W) {
+    constexpr uint32_t BPU = Q4 ? 64 : 32, BPB = Q4 ? 16 : 32;
+    const uint32_t U = job.g->U, nblk = job.g->nblk;
+    const uint32_t lb = Q4 ? lane : lane >> 1;
+    const uint32_t q = sdiv(round * PD_D, U);
+    uint32_t j = round * PD_D - q * U, lr = sw + q * PD_STREAM_WAVES;
 #pragma unroll
     for (int d = 0; d < PD_D; d++) {
-        const uint32_t u = (round * PD_D + d) * PD_WAVES + cx.wave;
         W.v[d] = make_int4(0, 0, 0, 0);
         W.s[d] = 0;
-        if (u < units) {
-            const uint32_t lr = u / g.U, j = u - lr * g.U;
-            const size_t row = pd_tile_row(g, tile, lr);
-            if (Q4) {
-                const uint32_t blk = j * 64 + cx.lane;
-                if (blk < g.nblk) {
-                    W.v[d] = *reinterpret_cast<const int4*>(g.qs + (row * g.nblk + blk) * 16);
-                    W.s[d] = g.ws[row * g.nblk + blk];
-                }
-            } else {
-                const uint32_t off = j * 1024 + cx.lane * 16;
-                if (off < g.K) {
-                    W.v[d] = *reinterpret_cast<const int4*>(g.qs + row * g.K + off);
-                    W.s[d] = g.ws[row * g.nblk + off / 32];
-                }
+        if (lr < t.rows) {                                        // wave-uniform
+            const uint32_t blk0 = pd_row(t, lr) * nblk + j * BPU;    // first block of the unit (fits 32 bits: N K / 32)
+            if (j * BPU + lb < nblk) {
+                W.v[d] = ldg(reinterpret_cast<const int4*>(job.qs + (size_t)blk0 * BPB) + lane);
+                W.s[d] = ldg(job.ws + blk0 + lb);
             }
         }
+        j += 1;
+        if (j == U) { j = 0; lr += PD_STREAM_WAVES; }
     }
 }
 
 // Exact int32 block dots on v_dot4, one f32 product (a_s*w_s)*f32(isum) per block parked in LDS.
 template <bool Q4>
-__device__ __forceinline__ void pd_compute_round(const PdGemv& g, uint32_t tile, uint32_t round, const PdCtx& cx, const WReg& W,
+__device__ __forceinline__ void pd_compute_round(const GemvJob& job, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane, const WReg& W,
                                                  const uint32_t* aq_lds, const float* as_lds, float* prod, uint32_t pstride) {
-    const uint32_t units = pd_tile_rows(g, tile) * g.U;
+    constexpr uint32_t BPU = Q4 ? 64 : 32;
+    const uint32_t U = job.g->U, nblk = job.g->nblk;
+    const uint32_t lb = Q4 ? lane : lane >> 1;
+    const uint32_t q = sdiv(round * PD_D, U);
+    uint32_t j = round * PD_D - q * U, lr = sw + q * PD_STREAM_WAVES;
 #pragma unroll
     for (int d = 0; d < PD_D; d++) {
-        const uint32_t u = (round * PD_D + d) * PD_WAVES + cx.wave;
-        if (u < units) {
-            const uint32_t lr = u / g.U, j = u - lr * g.U;
+        if (lr < t.rows) {                                        // wave-uniform
+            const uint32_t b = j * BPU + lb;
+            const bool in = b < nblk;
+            const uint32_t bs = in ? b : 0;
+            int isum;
             if (Q4) {
-                const uint32_t blk = j * 64 + cx.lane;
-                if (blk < g.nblk) {
-                    const int4 a0 = *reinterpret_cast<const int4*>(aq_lds + blk * 8);
-                    const int4 a1 = *reinterpret_cast<const int4*>(aq_lds + blk * 8 + 4);
-                    const int4 w = W.v[d];
-                    const int m = 0x0F0F0F0F;
-                    const int4 lo = make_int4(w.x & m, w.y & m, w.z & m, w.w & m);
-                    const int4 hi = make_int4((w.x >> 4) & m, (w.y >> 4) & m, (w.z >> 4) & m, (w.w >> 4) & m);
-                    const int4 ones = make_int4(0x01010101, 0x01010101, 0x01010101, 0x01010101);
-                    const int asum8 = 8 * dot16(ones, a1, dot16(ones, a0, 0));
-                    const int isum = dot16(hi, a1, dot16(lo, a0, 0)) - asum8;
-                    prod[lr * pstride + blk] = (as_lds[blk] * f16_bits_to_f32((uint16_t)W.s[d])) * (float)isum;
-                }
+                const int4 a0 = *reinterpret_cast<const int4*>(aq_lds + bs * 8);
+                const int4 a1 = *reinterpret_cast<const int4*>(aq_lds + bs * 8 + 4);
+                const int4 w = W.v[d];
+                const int m = 0x0F0F0F0F;
+                const int4 lo = make_int4(w.x & m, w.y & m, w.z & m, w.w & m);
+                const int4 hi = make_int4((w.x >> 4) & m, (w.y >> 4) & m, (w.z >> 4) & m, (w.w >> 4) & m);
+                const int4 ones = make_int4(0x01010101, 0x01010101, 0x01010101, 0x01010101);
+                const int asum8 = 8 * dot16(ones, a1, dot16(ones, a0, 0));
+                isum = dot16(hi, a1, dot16(lo, a0, 0)) - asum8;
             } else {
-                const uint32_t off = j * 1024 + cx.lane * 16;
-                const bool in = off < g.K;
-                const int4 a = in ? *reinterpret_cast<const int4*>(aq_lds + off / 4) : make_int4(0, 0, 0, 0);
-                const int half = dot16(W.v[d], a, 0);
-                const int isum = half + __shfl_xor(half, 1, WAVE);
-                if (in && !(cx.lane & 1u))
-                    prod[lr * pstride + off / 32] = (as_lds[off / 32] * f16_bits_to_f32((uint16_t)W.s[d])) * (float)isum;
+                const int4 a = *reinterpret_cast<const int4*>(aq_lds + bs * 8 + (lane & 1u) * 4);
+                const int half = dot16(W.v[d], a, 0);             // W is zero where the lane is past the row
+                // the other half of the block sits in the neighbouring lane: quad_perm [1,0,3,2]
+                isum = half + __builtin_amdgcn_update_dpp(0, half, 0xB1, 0xF, 0xF, false);
             }
+            if (in && (Q4 || !(lane & 1u))) prod[lr * pstride + b] = (as_lds[b] * f16_bits_to_f32((uint16_t)W.s[d])) * (float)isum;
         }
-    }
-}
-
-// Runs the tiles of this workgroup.  `epi(tile, lr, row, value, active)` is called by whole waves (lanes past
-// the tile's rows come with active = false) once the ordered sum of a row is known.
-// `pre(tile, lr, row, active)` runs before the sums: the place to start loads the epilogue will need.
-template <bool Q4, typename Pre, typename Epi>
-__device__ __forceinline__ void pd_gemv(const PdGemv& g, bool prefetched, WReg& W, const uint32_t* aq_lds, const float* as_lds,
-                                        float* prod, const PdCtx& cx, Pre pre, Epi epi) {
-    const uint32_t pstride = g.nblk + 1;                    // +1: conflict-free column reads
-    for (uint32_t tile = cx.wg; tile < g.ntiles; tile += cx.G) {
-        const uint32_t rows = pd_tile_rows(g, tile);
-        const uint32_t rounds = (rows * g.U + PD_D * PD_WAVES - 1) / (PD_D * PD_WAVES);
-        for (uint32_t r = 0; r < rounds; r++) {
-            if (!(prefetched && r == 0)) pd_load_round<Q4>(g, tile, r, cx, W);
-            pd_compute_round<Q4>(g, tile, r, cx, W, aq_lds, as_lds, prod, pstride);
-        }
-        // the next tile's first loads fly while this tile's rows are summed
-        prefetched = tile + cx.G < g.ntiles;
-        if (prefetched) pd_load_round<Q4>(g, tile + cx.G, 0, cx, W);
-        if (cx.tid < ((rows + 63u) & ~63u)) pre(tile, cx.tid, pd_tile_row(g, tile, cx.tid < rows ? cx.tid : 0), cx.tid < rows);
-        __syncthreads();
-        if (cx.tid < ((rows + 63u) & ~63u)) {
-            const bool active = cx.tid < rows;
-            const uint32_t row = pd_tile_row(g, tile, active ? cx.tid : 0);
-            float v = 0.f;
-            if (active) v = ordered_sum(prod + cx.tid * pstride, g.nblk, segment_row_is_dot1(row, g.seg, g.nseg, g.tail_mod));
-            epi(tile, cx.tid, row, v, active);
-        }
-        __syncthreads();
+        j += 1;
+        if (j == U) { j = 0; lr += PD_STREAM_WAVES; }
     }
 }
 
@@ -374,12 +444,12 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float* a, float 
 // keeps the per-thread state small.  Keys before this position come from the cache, this position's K/V
 // row and q from the tagged buffers P1 filled.
 template <int HD>
-__device__ __forceinline__ void pd_attn_split(const PdArgs& a, const PdLayer& L, uint32_t pos, uint32_t tag_in, uint32_t tag_out,
-                                              float* big, const PdCtx& cx) {
+__device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* kc, const uint16_t* vc, uint32_t pos, uint32_t tag_in,
+                                              uint32_t tag_out, float* big, const PdCtx& cx) {
     constexpr int LPK = HD <= 64 ? 8 : 16;
     constexpr int KPW = 64 / LPK;
     constexpr int REC = HD + 2;
-    const uint32_t g = cx.wave >> 2, wave = cx.wave & 3u, lane = cx.lane;
+    const uint32_t wave = cx.wave & 3u, lane = cx.lane;
     float* sh = big;                                                  // [4 waves][4][REC]
     float* q_lds = sh + 16 * REC;                                     // [gt][HD]
     uint32_t* kvn = reinterpret_cast<uint32_t*>(q_lds + 4 * HD);      // [2][HD] fp16 bits of this position's K and V
@@ -407,14 +477,14 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const PdLayer& L,
             const uint64_t* pkv = a.tkv + (e < HD ? kvh * HD + e : a.KV + kvh * HD + (e - HD));
             uint32_t v[2];
             // one batch: an element that is not needed re-reads the needed one
-            poll_many<2>([&](int i) { return (i == 0 ? need_q : !need_kv) ? pq : pkv; }, 2, tag_in, v, cx);
+            poll_many<2>([&](int i) { return (i == 0 ? need_q : !need_kv) ? pq : pkv; }, 2, tag_in, v, cx, Hint{nullptr, nullptr});
             if (need_q) q_lds[e] = __uint_as_float(v[0]);
             if (need_kv) kvn[e] = v[1];
         }
         __syncthreads();
         if (*cx.sh_abort) return;
 
-        if (g < gt) {
+        for (uint32_t g = cx.wave >> 2; g < gt; g += PD_WAVES / 4) {
             float qf[8], acc[8], m = -INFINITY, l = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; i++) { acc[i] = 0.f; qf[i] = dvalid ? q_lds[g * HD + c * 8 + i] : 0.f; }
@@ -435,8 +505,8 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const PdLayer& L,
                             }
                         } else {
                             const size_t off = (size_t)t * kv_stride + kvh * HD + c * 8;
-                            kr[u] = *reinterpret_cast<const Half8*>(L.kc + off);
-                            vr[u] = *reinterpret_cast<const Half8*>(L.vc + off);
+                            kr[u] = ldg(reinterpret_cast<const Half8*>(kc + off));
+                            vr[u] = ldg(reinterpret_cast<const Half8*>(vc + off));
                         }
                     }
                 }
@@ -506,11 +576,12 @@ __device__ __forceinline__ void pd_attn_combine(const PdArgs& a, uint32_t tag_in
                                                 const PdCtx& cx) {
     constexpr int REC = HD + 2;
     const uint32_t d = cx.tid;
-    float* wgt_s = misc + 64;                    // [DECODE_SPLITS] + den
+    float* wgt_s = misc + PD_MISC_SCRATCH;                    // [DECODE_SPLITS] + den
     float* recs = big;                           // [DECODE_SPLITS][REC]
     for (uint32_t h = cx.wg; h < a.heads; h += cx.G) {
         const uint64_t* base = a.tws + (size_t)h * DECODE_SPLITS * REC;
-        poll_vec(base, DECODE_SPLITS * REC, tag_in, cx, [&](uint32_t i, uint32_t p) { recs[i] = __uint_as_float(p); });
+        poll_vec<4>(base, DECODE_SPLITS * REC, tag_in, PD_THREADS, cx, Hint{nullptr, nullptr},
+                    [&](uint32_t i, uint32_t p) { recs[i] = __uint_as_float(p); });
         __syncthreads();
         if (*cx.sh_abort) return;
         if (d < 64) {
@@ -559,7 +630,7 @@ __device__ __forceinline__ ArgPair arg_wg(ArgPair a, float* misc, const PdCtx& c
         b.i = __shfl_xor(a.i, o, WAVE);
         a = arg_better(a, b);
     }
-    ArgPair* sh = reinterpret_cast<ArgPair*>(misc + 64);
+    ArgPair* sh = reinterpret_cast<ArgPair*>(misc + PD_MISC_SCRATCH);
     __syncthreads();
     if (cx.lane == 0) sh[cx.wave] = a;
     __syncthreads();
@@ -568,16 +639,136 @@ __device__ __forceinline__ ArgPair arg_wg(ArgPair a, float* misc, const PdCtx& c
     return r;
 }
 
-#define PD_EXIT_IF_ABORTED() do { if (*cx.sh_abort) return; } while (0)
-#define PD_STAMP(idx) do { if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[idx] = wall_clock64(); } while (0)
 
-template <bool Q4, bool LMQ4, int HD>
+// One GEMV phase of this workgroup: inputs, tiles, epilogues.
+//   inputs    the streamers issue the first weight loads of their rows at once; the poller wave fetches the activation
+//             vector (it never has weights in flight, so nothing delays what it polls)
+//   tiles     compute a round from registers, issue the next round (or the next tile's first), sum, finish the rows
+template <bool Q4, int HD>
+__device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& job, const float* emb, uint32_t pos, uint32_t* aq_lds,
+                                              float* as_lds, float* misc, float* big, ArgPair& best, const PdCtx& cx) {
+    const PdGemv& g = *job.g;
+    if (cx.wg >= g.ntiles) return;
+    const bool streamer = cx.wave >= (uint32_t)PD_POLL_WAVES;
+    const uint32_t sw = cx.wave - PD_POLL_WAVES;
+    const uint32_t pstride = g.nblk + 1;                    // +1: conflict-free column reads
+    const uint32_t K = job.in_len, U = g.U;
+    WReg W;
+    TilePos t = pd_tile(g, cx.wg);
+
+    // ---- inputs (norm weights are requested before this wave's weights: loads return in order)
+    float4 nw = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (job.pro == PRO_NORM && cx.tid * 4 < K) nw = ldg(reinterpret_cast<const float4*>(job.norm_w + cx.tid * 4));
+    if (streamer) {
+        pd_load_round<Q4>(job, t, 0, sw, cx.lane, W);
+    } else {
+        if (job.pro == PRO_AQ) pd_load_aq(job.tin, job.tin_tag, K, aq_lds, as_lds, misc, cx);
+        else if (job.tin_tag) pd_load_x(job.tin, job.tin_tag, K, big, misc, cx);
+        else for (uint32_t i = cx.tid; i < K; i += PD_POLL_THREADS) big[i] = emb[i];
+    }
+    __syncthreads();
+    if (*cx.sh_abort) return;
+    // the norm reads big[0..K); the products reuse the area afterwards
+    if (job.pro == PRO_NORM) pd_norm_quant(big, job.norm_w, nw, a.eps, K, aq_lds, as_lds, misc, cx);
+
+    // ---- tiles
+#pragma nounroll
+    for (uint32_t tile = cx.wg; tile < g.ntiles; tile += cx.G) {
+        const uint32_t rounds = ((t.rows + PD_STREAM_WAVES - 1) / PD_STREAM_WAVES * U + PD_D - 1) / PD_D;
+        const bool more = tile + cx.G < g.ntiles;
+        const TilePos tn = more ? pd_tile(g, tile + cx.G) : t;
+        // what the epilogue needs from global memory is requested early (by wave 0, which streams nothing, for tiles of
+        // up to 64 rows)
+        const bool mine = cx.tid < t.rows;
+        const uint32_t row = pd_row(t, mine ? cx.tid : 0);
+        float rc = 0.f, rs = 0.f;
+        uint64_t res_w = 0;
+        float res_e = 0.f;
+        if (mine) {
+            if (job.epi == EPI_ROPE && row < a.QKS + a.KV) {
+                const uint32_t d = row < a.QKS ? row % HD : (row - a.QKS) % HD;
+                rc = a.cos_t[(size_t)pos * (HD / 2) + d / 2];
+                rs = a.sin_t[(size_t)pos * (HD / 2) + d / 2];
+            } else if (job.epi == EPI_ADD) {
+                if (job.res_tag) res_w = ldc64(a.tx + row);   // in flight while the tile is computed; the tag is checked below
+                else res_e = emb[row];
+            }
+        }
+        if (streamer) {
+#pragma nounroll
+            for (uint32_t r = 0; r < rounds; r++) {
+                pd_compute_round<Q4>(job, t, r, sw, cx.lane, W, aq_lds, as_lds, big, pstride);
+                if (r + 1 < rounds) pd_load_round<Q4>(job, t, r + 1, sw, cx.lane, W);
+                else if (more) pd_load_round<Q4>(job, tn, 0, sw, cx.lane, W);
+            }
+        }
+        __syncthreads();
+        if (cx.tid < ((t.rows + 63u) & ~63u)) {
+            float v = 0.f;
+            if (mine) v = ordered_sum(big + cx.tid * pstride, g.nblk, segment_row_is_dot1(row, g.seg, g.nseg, g.tail_mod));
+            if (job.epi == EPI_ROPE) {
+                // rope (emit.rs:508-528): rows 2i, 2i+1 of a head sit in neighbouring lanes
+                const float other = __shfl_xor(v, 1, WAVE);
+                if (mine) {
+                    if (row < a.QKS + a.KV) {
+                        const float o = (row & 1u) ? other * rs + v * rc : v * rc - other * rs;
+                        if (row < a.QKS) {
+                            stc64(a.tq + row, job.tag_out, __float_as_uint(o));
+                        } else {
+                            const uint16_t hb = f32_to_f16_bits(o);
+                            stg(job.kc + (size_t)pos * a.KV + (row - a.QKS), hb);
+                            stc64(a.tkv + (row - a.QKS), job.tag_out, hb);
+                        }
+                    } else {
+                        const uint16_t hb = f32_to_f16_bits(v);
+                        stg(job.vc + (size_t)pos * a.KV + (row - a.QKS - a.KV), hb);
+                        stc64(a.tkv + a.KV + (row - a.QKS - a.KV), job.tag_out, hb);
+                    }
+                }
+            } else if (job.epi == EPI_ADD) {
+                if (mine) {
+                    float res = res_e;
+                    if (job.res_tag)
+                        res = __uint_as_float((uint32_t)(res_w >> 32) == job.res_tag ? (uint32_t)res_w : poll(a.tx + row, job.res_tag, cx));
+                    stc64(a.tx + row, job.tag_out, __float_as_uint(res + v));       // residual_add, emit.rs:455-459
+                }
+            } else if (job.epi == EPI_SILU) {
+                // lanes 0..31 hold the gate rows of inter indices [32 tile, +32), lanes 32..63 the up rows
+                const uint32_t lr = cx.tid;
+                const float ux = __shfl(v, (cx.lane & 31u) + 32, WAVE);
+                if (lr < 32) {
+                    const float o = (v / (1.0f + expf_ref<true>(-v))) * ux;          // silu_mul, emit.rs:380-386
+                    float amax = fabsf(o);
+#pragma unroll
+                    for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+                    float inv;
+                    const float sc = act_scale(amax, inv);
+                    const uint32_t code = (uint32_t)quant_code(o * inv) & 0xFFu;
+                    const uint32_t bl = lr & ~3u;
+                    const uint32_t pk = __shfl(code, bl, WAVE) | (__shfl(code, bl + 1, WAVE) << 8) | (__shfl(code, bl + 2, WAVE) << 16) |
+                                        (__shfl(code, bl + 3, WAVE) << 24);
+                    if ((lr & 3u) == 0) stc64(a.taq2 + tile * 8 + lr / 4, job.tag_out, pk);
+                    if (lr == 0) stc64(a.taq2 + a.I / 4 + tile, job.tag_out, f32_to_f16_bits(sc));
+                }
+            } else {
+                if (mine) {
+                    a.logits[row] = v;
+                    best = arg_better(best, ArgPair{v, row});
+                }
+            }
+        }
+        __syncthreads();
+        t = tn;
+    }
+}
+
+template <int HD>
 __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     __shared__ uint32_t sh_abort;
     uint32_t* aq_lds = reinterpret_cast<uint32_t*>(smem);
     float* as_lds = reinterpret_cast<float*>(smem + a.off_act_s);
-    float* misc = reinterpret_cast<float*>(smem + a.off_misc);       // [0,32) norm partials, [64, ...) phase scratch
+    float* misc = reinterpret_cast<float*>(smem + a.off_misc);
     float* big = reinterpret_cast<float*>(smem + a.off_big);         // x copy / block products / attention scratch
 
     PdCtx cx;
@@ -589,189 +780,77 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     cx.spin_limit = a.spin_limit;
     cx.sh_abort = &sh_abort;
     cx.abort_flag = a.state + 3;
-    if (cx.tid == 0) sh_abort = 0;
+    if (cx.tid == 0) { sh_abort = 0; reinterpret_cast<uint32_t*>(misc)[PD_MISC_HINT] = 0; }
     __syncthreads();
 
     const uint32_t pos = a.state[0], token = a.state[1];
-    const uint32_t H = a.H;
-    const float* emb = a.embed + (size_t)token * H;
-    uint32_t tag = a.tag_base;            // tag of phase instance k of this launch = tag_base + k
-    uint32_t x_tag = 0;                   // tag of the current version of tx (0: x is still the embedding row)
-    uint32_t stamp = 0;
-    WReg W;
-
-    {
-        const PdGemv& g0 = a.layers[0].qkv;
-        pd_load_round<Q4>(g0, cx.wg, 0, cx, W);
-    }
-    for (uint32_t l = 0; l < a.n_layers; l++) {
-        const PdLayer& L = a.layers[l];
-        // ---------------- P1: norm | qkv GEMV | rope + KV ----------------
-        PD_STAMP(stamp++);
-        const uint32_t t1 = ++tag;
-        if (cx.wg < L.qkv.ntiles) {
-            if (x_tag) {
-                wait_hint(a.tx + H - 1, x_tag, cx);
-                poll_vec(a.tx, H, x_tag, cx, [&](uint32_t i, uint32_t p) { big[i] = __uint_as_float(p); });
-            } else {
-                for (uint32_t i = cx.tid; i < H; i += PD_THREADS) big[i] = emb[i];
-            }
-            __syncthreads();
-            PD_EXIT_IF_ABORTED();
-            // the norm reads big[0..H); the products reuse the area afterwards
-            pd_norm_quant(big, L.attn_norm, a.eps, H, aq_lds, as_lds, misc, cx);
-            float rc = 0.f, rs = 0.f;
-            pd_gemv<Q4>(L.qkv, true, W, aq_lds, as_lds, big, cx, [&](uint32_t, uint32_t, uint32_t row, bool active) {
-                if (active && row < a.QKS + a.KV) {
-                    const uint32_t d = row < a.QKS ? row % HD : (row - a.QKS) % HD;
-                    rc = a.cos_t[(size_t)pos * (HD / 2) + d / 2];
-                    rs = a.sin_t[(size_t)pos * (HD / 2) + d / 2];
-                }
-            }, [&](uint32_t, uint32_t, uint32_t row, float r, bool active) {
-                // rope (emit.rs:508-528): rows 2i, 2i+1 of a head sit in neighbouring lanes
-                const float other = __shfl_xor(r, 1, WAVE);
-                if (!active) return;
-                if (row < a.QKS + a.KV) {
-                    const float c = rc, s = rs;
-                    const float o = (row & 1u) ? other * s + r * c : r * c - other * s;
-                    if (row < a.QKS) {
-                        stc64(a.tq + row, t1, __float_as_uint(o));
-                    } else {
-                        const uint16_t hb = f32_to_f16_bits(o);
-                        L.kc[(size_t)pos * a.KV + (row - a.QKS)] = hb;
-                        stc64(a.tkv + (row - a.QKS), t1, hb);
-                    }
-                } else {
-                    const uint16_t hb = f32_to_f16_bits(r);
-                    L.vc[(size_t)pos * a.KV + (row - a.QKS - a.KV)] = hb;
-                    stc64(a.tkv + a.KV + (row - a.QKS - a.KV), t1, hb);
-                }
-            });
-        }
-        // ---------------- P2: attention, split along the sequence ----------------
-        PD_STAMP(stamp++);
-        const uint32_t t2 = ++tag;
-        pd_attn_split<HD>(a, L, pos, t1, t2, big, cx);
-        PD_EXIT_IF_ABORTED();
-        // ---------------- P3: merge the splits, quantise ----------------
-        PD_STAMP(stamp++);
-        const uint32_t t3 = ++tag;
-        pd_attn_combine<HD>(a, t2, t3, misc, big, cx);
-        PD_EXIT_IF_ABORTED();
-        // ---------------- P4: O GEMV + residual ----------------
-        PD_STAMP(stamp++);
-        const uint32_t t4 = ++tag;
-        if (cx.wg < L.o.ntiles) {
-            pd_load_round<Q4>(L.o, cx.wg, 0, cx, W);
-            pd_load_aq(a.taq, t3, a.QKS, aq_lds, as_lds, cx);
-            PD_EXIT_IF_ABORTED();
-            const uint32_t xin = x_tag;
-            uint64_t res_w = 0;
-            float res_e = 0.f;
-            pd_gemv<Q4>(L.o, true, W, aq_lds, as_lds, big, cx, [&](uint32_t, uint32_t, uint32_t row, bool active) {
-                if (!active) return;
-                if (xin) res_w = ldc64(a.tx + row);       // in flight while the rows are summed; the tag is checked below
-                else res_e = emb[row];
-            }, [&](uint32_t, uint32_t, uint32_t row, float r, bool active) {
-                if (!active) return;
-                float res = res_e;
-                if (xin) res = __uint_as_float((uint32_t)(res_w >> 32) == xin ? (uint32_t)res_w : poll(a.tx + row, xin, cx));
-                stc64(a.tx + row, t4, __float_as_uint(res + r));       // residual_add, emit.rs:455-459
-            });
-            PD_EXIT_IF_ABORTED();
-        }
-        x_tag = t4;
-        // ---------------- P5: norm | gate/up GEMV | silu*up, quantise ----------------
-        PD_STAMP(stamp++);
-        const uint32_t t5 = ++tag;
-        if (cx.wg < L.gu.ntiles) {
-            pd_load_round<Q4>(L.gu, cx.wg, 0, cx, W);
-            wait_hint(a.tx + H - 1, x_tag, cx);
-            poll_vec(a.tx, H, x_tag, cx, [&](uint32_t i, uint32_t p) { big[i] = __uint_as_float(p); });
-            __syncthreads();
-            PD_EXIT_IF_ABORTED();
-            pd_norm_quant(big, L.ffn_norm, a.eps, H, aq_lds, as_lds, misc, cx);
-            pd_gemv<Q4>(L.gu, true, W, aq_lds, as_lds, big, cx, [](uint32_t, uint32_t, uint32_t, bool) {},
-                        [&](uint32_t tile, uint32_t lr, uint32_t, float r, bool) {
-                // lanes 0..31 hold the gate rows of inter indices [32 tile, +32), lanes 32..63 the up rows
-                const float ux = __shfl(r, (cx.lane & 31u) + 32, WAVE);
-                if (lr >= 32) return;
-                const float o = (r / (1.0f + expf_ref<true>(-r))) * ux;          // silu_mul, emit.rs:380-386
-                float amax = fabsf(o);
-#pragma unroll
-                for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
-                float inv;
-                const float sc = act_scale(amax, inv);
-                const uint32_t code = (uint32_t)quant_code(o * inv) & 0xFFu;
-                const uint32_t bl = lr & ~3u;
-                const uint32_t pk = __shfl(code, bl, WAVE) | (__shfl(code, bl + 1, WAVE) << 8) | (__shfl(code, bl + 2, WAVE) << 16) |
-                                    (__shfl(code, bl + 3, WAVE) << 24);
-                if ((lr & 3u) == 0) stc64(a.taq2 + tile * 8 + lr / 4, t5, pk);
-                if (lr == 0) stc64(a.taq2 + a.I / 4 + tile, t5, f32_to_f16_bits(sc));
-            });
-        }
-        // ---------------- P6: down GEMV + residual ----------------
-        PD_STAMP(stamp++);
-        const uint32_t t6 = ++tag;
-        if (cx.wg < L.down.ntiles) {
-            pd_load_round<Q4>(L.down, cx.wg, 0, cx, W);
-            pd_load_aq(a.taq2, t5, a.I, aq_lds, as_lds, cx);
-            PD_EXIT_IF_ABORTED();
-            uint64_t res_w = 0;
-            pd_gemv<Q4>(L.down, true, W, aq_lds, as_lds, big, cx, [&](uint32_t, uint32_t, uint32_t row, bool active) {
-                if (active) res_w = ldc64(a.tx + row);
-            }, [&](uint32_t, uint32_t, uint32_t row, float r, bool active) {
-                if (!active) return;
-                const float res = __uint_as_float((uint32_t)(res_w >> 32) == t4 ? (uint32_t)res_w : poll(a.tx + row, t4, cx));
-                stc64(a.tx + row, t6, __float_as_uint(res + r));
-            });
-            PD_EXIT_IF_ABORTED();
-        }
-        x_tag = t6;
-        if (l + 1 < a.n_layers) pd_load_round<Q4>(a.layers[l + 1].qkv, cx.wg, 0, cx, W);
-    }
-
-    // ---------------- head: final norm | lm_head GEMV | argmax ----------------
-    PD_STAMP(stamp++);
-    const uint32_t th = ++tag;
+    const float* emb = a.embed + (size_t)token * a.H;
+    const uint32_t L = a.n_layers;
     ArgPair best{-INFINITY, 0};
-    if (cx.wg < a.lm.ntiles) {
-        WReg WL;
-        pd_load_round<LMQ4>(a.lm, cx.wg, 0, cx, WL);
-        wait_hint(a.tx + H - 1, x_tag, cx);
-        poll_vec(a.tx, H, x_tag, cx, [&](uint32_t i, uint32_t p) { big[i] = __uint_as_float(p); });
-        __syncthreads();
-        PD_EXIT_IF_ABORTED();
-        pd_norm_quant(big, a.final_norm, a.eps, H, aq_lds, as_lds, misc, cx);
-        pd_gemv<LMQ4>(a.lm, true, WL, aq_lds, as_lds, big, cx, [](uint32_t, uint32_t, uint32_t, bool) {},
-                      [&](uint32_t, uint32_t, uint32_t row, float r, bool active) {
-            if (!active) return;
-            a.logits[row] = r;
-            best = arg_better(best, ArgPair{r, row});
-        });
+
+    // steps 4 l + {0: qkv, 1: attention then o, 2: gate/up, 3: down}; step 4 L: lm_head.  Phase instance k of this
+    // launch carries tag tag_base + k: per layer 1 qkv, 2 attention split, 3 attention merge, 4 o, 5 gate/up, 6 down.
+#pragma nounroll
+    for (uint32_t step = 0; step <= 4 * L; step++) {
+        const bool is_lm = step == 4 * L;
+        const uint32_t l = is_lm ? L - 1 : step >> 2, ph = is_lm ? 4u : (step & 3u);
+        const uint32_t base = a.tag_base + 6 * l;
+        const uint32_t x_in = l ? base : 0;                  // tag of x entering layer l (0: still the embedding row)
+        if (ph == 1) {
+            if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * l + 1] = wall_clock64();
+            pd_attn_split<HD>(a, a.layers[l].kc, a.layers[l].vc, pos, base + 1, base + 2, big, cx);
+            if (sh_abort) return;
+            if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * l + 2] = wall_clock64();
+            pd_attn_combine<HD>(a, base + 2, base + 3, misc, big, cx);
+            if (sh_abort) return;
+        }
+        if (a.stamps && cx.wg == 0 && cx.tid == 0) {
+            static const int slot[5] = {0, 3, 4, 5, 6};
+            a.stamps[6 * l + slot[ph]] = wall_clock64();
+        }
+        GemvJob job;
+        job.g = is_lm ? &a.lm : &a.shape[ph];
+        job.qs = is_lm ? a.lm.qs : a.layers[l].qs[ph];
+        job.ws = is_lm ? a.lm.ws : a.layers[l].ws[ph];
+        job.q4 = is_lm ? a.lm_q4 != 0 : a.q4 != 0;
+        job.pro = (ph == 1 || ph == 3) ? PRO_AQ : PRO_NORM;
+        job.epi = ph == 0 ? EPI_ROPE : ph == 2 ? EPI_SILU : ph == 4 ? EPI_LOGITS : EPI_ADD;
+        job.norm_w = ph == 0 ? a.layers[l].attn_norm : ph == 2 ? a.layers[l].ffn_norm : a.final_norm;
+        job.tin = ph == 1 ? a.taq : ph == 3 ? a.taq2 : a.tx;
+        job.tin_tag = ph == 0 ? x_in : ph == 1 ? base + 3 : ph == 2 ? base + 4 : ph == 3 ? base + 5 : base + 6;
+        job.in_len = ph == 1 ? a.QKS : ph == 3 ? a.I : a.H;
+        job.tag_out = is_lm ? 0 : base + (ph == 0 ? 1u : ph == 1 ? 4u : ph == 2 ? 5u : 6u);
+        job.res_tag = ph == 1 ? x_in : base + 4;
+        job.kc = a.layers[l].kc;
+        job.vc = a.layers[l].vc;
+        if (job.q4) pd_gemv_phase<true, HD>(a, job, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        else pd_gemv_phase<false, HD>(a, job, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        if (sh_abort) return;
     }
+
+    // ---------------- argmax (and the position / token advance) ----------------
+    const uint32_t th = a.tag_base + 6 * L + 1;
     best = arg_wg(best, misc, cx);
     if (cx.tid == 0) {
         stc64(a.tpart + 2 * cx.wg, th, __float_as_uint(best.v));
         stc64(a.tpart + 2 * cx.wg + 1, th, best.i);
     }
-    PD_STAMP(stamp++);
+    if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * L + 1] = wall_clock64();
     if (cx.wg == 0) {
         ArgPair p{-INFINITY, 0};
-        if (cx.tid < cx.G) {
+        for (uint32_t w = cx.tid; w < cx.G; w += PD_THREADS) {
             uint32_t v[2];
-            poll_many<2>([&](int i) { return a.tpart + 2 * cx.tid + (uint32_t)i; }, 2, th, v, cx);
-            p.v = __uint_as_float(v[0]);
-            p.i = v[1];
+            poll_many<2>([&](int i) { return a.tpart + 2 * w + (uint32_t)i; }, 2, th, v, cx, Hint{nullptr, nullptr});
+            p = arg_better(p, ArgPair{__uint_as_float(v[0]), v[1]});
         }
         p = arg_wg(p, misc, cx);
-        PD_EXIT_IF_ABORTED();
+        if (sh_abort) return;
         if (cx.tid == 0) {
             a.state[2] = p.i;
             a.state[1] = p.i;
             a.state[0] = pos + 1;
+            if (a.stamps) a.stamps[6 * L + 2] = wall_clock64();
         }
-        PD_STAMP(stamp++);
     }
 }
 
@@ -830,19 +909,10 @@ bool plan_gemv(const QWeight& w, uint32_t inter, uint32_t nseg, const Segment* s
     return true;
 }
 
-template <bool Q4, bool LMQ4, int HD>
-hipError_t launch_pd(const PdState* st, hipStream_t s) {
-    void* kargs[] = {const_cast<PdArgs*>(&st->args)};
-    return hipLaunchCooperativeKernel(reinterpret_cast<void*>(decode_step_kernel<Q4, LMQ4, HD>), dim3(st->grid), dim3(PD_THREADS), kargs,
-                                      st->lds, s);
-}
-
 template <int HD>
 hipError_t launch_pd_hd(const PdState* st, hipStream_t s) {
-    if (!st->q4 && !st->lmq4) return launch_pd<false, false, HD>(st, s);
-    if (st->q4 && st->lmq4) return launch_pd<true, true, HD>(st, s);
-    if (st->q4) return launch_pd<true, false, HD>(st, s);
-    return hipErrorInvalidValue;
+    void* kargs[] = {const_cast<PdArgs*>(&st->args)};
+    return hipLaunchCooperativeKernel(reinterpret_cast<void*>(decode_step_kernel<HD>), dim3(st->grid), dim3(PD_THREADS), kargs, st->lds, s);
 }
 
 }  // namespace
@@ -856,7 +926,6 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     *out = nullptr;
     if (c.flags & FORGE_HIP_FLAG_EXACT) return FORGE_HIP_OK;
     if (c.head_dim != 64 && c.head_dim != 128) return FORGE_HIP_OK;
-    if (c.wdtype == FORGE_HIP_Q8_0 && c.lm_head_dtype == FORGE_HIP_Q4_0) return FORGE_HIP_OK;
     int dev = 0, coop = 0, cus = 0, khz = 0;
     FH_HIP(hipGetDevice(&dev));
     FH_HIP(hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev));
@@ -886,18 +955,25 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     if ((H + 32) * 4 > big || attn_bytes > big || DECODE_SPLITS * (hd + 2) * 4 > big) return FORGE_HIP_OK;
     st->lds = a.off_big + big;
 
-    std::vector<PdLayer> hl(layers.size());
-    for (size_t l = 0; l < layers.size(); l++) {
-        const PdLayerIn& in = layers[l];
-        PdLayer& L = hl[l];
+    if (layers.empty() || layers.size() > PD_MAX_LAYERS) return FORGE_HIP_OK;
+    {
+        const PdLayerIn& in = layers[0];
         const uint32_t wt = c.wdtype;
         Segment sq[3] = {make_segment(wt, H, 0, QKS, false), make_segment(wt, H, QKS, KV, false), make_segment(wt, H, QKS + KV, KV, false)};
         Segment so[1] = {make_segment(wt, QKS, 0, H, false)};
         Segment sg[2] = {make_segment(wt, H, 0, I, false), make_segment(wt, H, I, I, false)};
         Segment sd[1] = {make_segment(wt, I, 0, H, false)};
-        if (!plan_gemv(*in.qkv, 0, 3, sq, 4, st->grid, big, &L.qkv) || !plan_gemv(*in.o, 0, 1, so, 4, st->grid, big, &L.o) ||
-            !plan_gemv(*in.gate_up, I, 2, sg, 4, st->grid, big, &L.gu) || !plan_gemv(*in.down, 0, 1, sd, 4, st->grid, big, &L.down))
+        if (!plan_gemv(*in.qkv, 0, 3, sq, 4, st->grid, big, &a.shape[PD_QKV]) || !plan_gemv(*in.o, 0, 1, so, 4, st->grid, big, &a.shape[PD_O]) ||
+            !plan_gemv(*in.gate_up, I, 2, sg, 4, st->grid, big, &a.shape[PD_GU]) ||
+            !plan_gemv(*in.down, 0, 1, sd, 4, st->grid, big, &a.shape[PD_DOWN]))
             return FORGE_HIP_OK;
+        for (int k = 0; k < 4; k++) { a.shape[k].qs = nullptr; a.shape[k].ws = nullptr; }
+    }
+    for (size_t l = 0; l < layers.size(); l++) {
+        const PdLayerIn& in = layers[l];
+        PdLayer& L = a.layers[l];
+        const QWeight* w[4] = {in.qkv, in.o, in.gate_up, in.down};
+        for (int k = 0; k < 4; k++) { L.qs[k] = w[k]->qs; L.ws[k] = w[k]->scales; }
         L.attn_norm = in.attn_norm; L.ffn_norm = in.ffn_norm; L.kc = in.kc; L.vc = in.vc;
     }
     {
@@ -908,19 +984,12 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     {
         int per_cu = 0;
         hipError_t e = hipErrorInvalidValue;
-        const bool q4 = st->q4, lq4 = st->lmq4;
-#define PD_OCC(Q, LQ, HDV) e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_step_kernel<Q, LQ, HDV>, PD_THREADS, st->lds)
-        if (hd == 64) { if (!q4) PD_OCC(false, false, 64); else if (lq4) PD_OCC(true, true, 64); else PD_OCC(true, false, 64); }
-        else { if (!q4) PD_OCC(false, false, 128); else if (lq4) PD_OCC(true, true, 128); else PD_OCC(true, false, 128); }
-#undef PD_OCC
+e = hd == 64 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_step_kernel<64>, PD_THREADS, st->lds)
+                     : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_step_kernel<128>, PD_THREADS, st->lds);
         if (e != hipSuccess || per_cu < 1) { (void)hipGetLastError(); return FORGE_HIP_OK; }
     }
 
-    PdLayer* dl = dev_alloc<PdLayer>(hl.size() * sizeof(PdLayer), st->owned);
-    if (!dl) return fail(FORGE_HIP_ERR_HIP, "persistent decode: out of device memory");
-    FH_HIP(hipMemcpy(dl, hl.data(), hl.size() * sizeof(PdLayer), hipMemcpyHostToDevice));
-    a.layers = dl;
-    a.n_layers = (uint32_t)hl.size();
+    a.n_layers = (uint32_t)layers.size();
     a.H = H; a.I = I; a.QKS = QKS; a.KV = KV; a.heads = c.heads; a.kv_heads = c.kv_heads;
     a.eps = c.rms_eps;
     a.embed = embed; a.final_norm = final_norm; a.cos_t = cos_t; a.sin_t = sin_t;
@@ -942,6 +1011,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     a.tpart = t;
     a.tag_base = 0;
     a.spin_limit = 400000;
+    a.q4 = st->q4; a.lm_q4 = st->lmq4;
     st->tags_per_launch = 6 * a.n_layers + 1;
     st->n_stamps = 6 * a.n_layers + 3;
     a.stamps = nullptr;
