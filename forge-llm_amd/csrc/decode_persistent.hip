@@ -55,7 +55,7 @@ namespace {
 constexpr int PD_THREADS = 512;
 constexpr int PD_WAVES = PD_THREADS / 64;
 constexpr int PD_D = 16;                      // weight units (1 KB) a wave holds in registers per round
-constexpr uint32_t PD_MAX_TILE_ROWS = 128;
+constexpr uint32_t PD_MAX_TILE_ROWS = 128;      // = 64 PD_POLL_WAVES: the pollers own a tile's rows
 constexpr uint32_t PD_LDS_BYTES = 64 * 1024;
 constexpr uint32_t PD_MISC_BYTES = 2048;
 constexpr int PD_POLL_WAVES = 2;              // waves that fetch a phase's input; the others stream weights
@@ -85,11 +85,10 @@ struct PdLayer {
     uint16_t* vc;
 };
 constexpr uint32_t PD_MAX_LAYERS = 34;       // the descriptors travel as kernel arguments (4 KB in all)
-enum { PD_QKV = 0, PD_O = 1, PD_GU = 2, PD_DOWN = 3 };
+enum { PD_QKV = 0, PD_O = 1, PD_GU = 2, PD_DOWN = 3, PD_LM = 4 };
 
 struct PdArgs {
-    PdGemv shape[4];           // qkv, o, gate_up, down with null addresses
-    PdGemv lm;
+    PdGemv shape[5];           // qkv, o, gate_up, down (addresses per layer, below) and lm_head (addresses here)
     uint32_t n_layers, H, I, QKS, KV, heads, kv_heads, gt;
     float eps;
     const float* embed;
@@ -108,6 +107,7 @@ struct PdArgs {
     uint32_t* state;   // [0] position  [1] token  [2] next token  [3] abort flag
     uint32_t tag_base, spin_limit;
     uint32_t q4, lm_q4;                        // weight formats: projections, lm_head
+    uint32_t use_hint;                         // pollers wait for one watched element before re-reading a whole buffer
     uint32_t off_act_s, off_misc, off_big;     // LDS byte offsets (activation codes sit at 0)
     unsigned long long* stamps;                // optional: wall clock at the start of every phase (workgroup 0)
     // Kernel arguments are read with scalar loads, which have their own completion counter: a wave can
@@ -258,27 +258,35 @@ __device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict
                                               uint32_t* aq_lds, float* as_lds, float* part, const PdCtx& cx) {
     const uint32_t tid = cx.tid;
     __syncthreads();
-    if (tid < 16) {
+    if (tid < 64) {
+        // lane i < 16 owns accumulator i: x[i], x[16 + i], ... added in order with FMAs.  The reads of the next eight
+        // values are issued before the current eight are consumed, so LDS latency stays off the dependent chain.
         float s = 0.f;
-        const uint32_t chunks = H / 16;
+        const uint32_t chunks = H / 16, i16 = tid & 15u;
         uint32_t c = 0;
-        for (; c + 8 <= chunks; c += 8) {
-            float v[8];
+        if (chunks >= 8) {
+            float v[8], w[8];
 #pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = xs[(c + i) * 16 + tid];
+            for (int i = 0; i < 8; i++) v[i] = xs[i * 16 + i16];
+            for (c = 8; c + 8 <= chunks; c += 8) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) w[i] = xs[(c + i) * 16 + i16];
+#pragma unroll
+                for (int i = 0; i < 8; i++) s = fmaf(v[i], v[i], s);
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[i] = w[i];
+            }
 #pragma unroll
             for (int i = 0; i < 8; i++) s = fmaf(v[i], v[i], s);
         }
-        for (; c < chunks; c++) { const float v = xs[c * 16 + tid]; s = fmaf(v, v, s); }
-        part[tid] = s;
-    }
-    __syncthreads();
-    if (tid == 0) {
-        float t[4];
-        for (int i = 0; i < 4; i++) t[i] = (part[i] + part[4 + i]) + (part[8 + i] + part[12 + i]);
-        float r = (t[0] + t[1]) + (t[2] + t[3]);
-        for (uint32_t i = H / 16 * 16; i < H; i++) r = r + xs[i] * xs[i];
-        part[16] = r;
+        for (; c < chunks; c++) { const float v = xs[c * 16 + i16]; s = fmaf(v, v, s); }
+        // (p[i] + p[4+i]) + (p[8+i] + p[12+i]) for i = 0..3, then (t0 + t1) + (t2 + t3)
+        const float t = (s + __shfl(s, (tid + 4) & 63, WAVE)) + (__shfl(s, (tid + 8) & 63, WAVE) + __shfl(s, (tid + 12) & 63, WAVE));
+        float r = (t + __shfl(t, (tid + 1) & 63, WAVE)) + (__shfl(t, (tid + 2) & 63, WAVE) + __shfl(t, (tid + 3) & 63, WAVE));
+        if (tid == 0) {
+            for (uint32_t i = H / 16 * 16; i < H; i++) r = r + xs[i] * xs[i];
+            part[16] = r;
+        }
     }
     __syncthreads();
     const float inv_rms = 1.0f / sqrtf(part[16] / (float)H + eps);
@@ -296,9 +304,9 @@ __device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict
 
 // An already quantised vector (codes then scales, tagged) from another phase; fetched by the poller waves.
 __device__ __forceinline__ void pd_load_aq(const uint64_t* t, uint32_t tag, uint32_t K, uint32_t* aq_lds, float* as_lds,
-                                           float* misc, const PdCtx& cx) {
+                                           float* misc, bool use_hint, const PdCtx& cx) {
     const uint32_t nq = K / 4, ns = K / 32;
-    const Hint hint{t + nq + ns - 1, reinterpret_cast<volatile uint32_t*>(misc + PD_MISC_HINT)};
+    const Hint hint{t + nq + ns - 1, use_hint ? reinterpret_cast<volatile uint32_t*>(misc + PD_MISC_HINT) : nullptr};
     poll_vec<PD_POLL_N>(t, nq + ns, tag, PD_POLL_THREADS, cx, hint, [&](uint32_t i, uint32_t p) {
         if (i < nq) aq_lds[i] = p;
         else as_lds[i - nq] = f16_bits_to_f32((uint16_t)p);
@@ -306,8 +314,9 @@ __device__ __forceinline__ void pd_load_aq(const uint64_t* t, uint32_t tag, uint
 }
 
 // The residual stream (tagged) into LDS as floats; fetched by the poller waves.
-__device__ __forceinline__ void pd_load_x(const uint64_t* tx, uint32_t tag, uint32_t H, float* xs, float* misc, const PdCtx& cx) {
-    const Hint hint{tx + H - 1, reinterpret_cast<volatile uint32_t*>(misc + PD_MISC_HINT)};
+__device__ __forceinline__ void pd_load_x(const uint64_t* tx, uint32_t tag, uint32_t H, float* xs, float* misc, bool use_hint,
+                                          const PdCtx& cx) {
+    const Hint hint{tx + H - 1, use_hint ? reinterpret_cast<volatile uint32_t*>(misc + PD_MISC_HINT) : nullptr};
     poll_vec<PD_POLL_N>(tx, H, tag, PD_POLL_THREADS, cx, hint, [&](uint32_t i, uint32_t p) { xs[i] = __uint_as_float(p); });
 }
 
@@ -319,7 +328,7 @@ enum { PRO_NORM = 0, PRO_AQ = 1 };
 enum { EPI_ROPE = 0, EPI_ADD = 1, EPI_SILU = 2, EPI_LOGITS = 3 };
 
 struct GemvJob {
-    const PdGemv* g;           // shape, in the kernel arguments
+    uint32_t which;            // index of the shape in the kernel arguments (PD_QKV .. PD_LM)
     const uint8_t* qs;
     const uint16_t* ws;
     bool q4;
@@ -336,28 +345,40 @@ struct GemvJob {
 
 struct WReg { int4 v[PD_D]; uint32_t s[PD_D]; };
 
+__device__ __forceinline__ uint32_t sgpr(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+
+// The scalar fields of a shape, read once per phase into scalar registers.
+struct Shape { uint32_t K, N, nblk, U, T, ntiles, inter; };
+__device__ __forceinline__ Shape pd_shape(const PdGemv& g) {
+    Shape h;
+    h.K = sgpr(g.K); h.N = sgpr(g.N); h.nblk = sgpr(g.nblk); h.U = sgpr(g.U); h.T = sgpr(g.T); h.ntiles = sgpr(g.ntiles);
+    h.inter = sgpr(g.inter);
+    return h;
+}
+
 // Rows of a tile: [row0, row0 + split) and, for the fused [gate;up] matrix, the matching rows `jump` further on.
 // Everything here is wave-uniform and meant to live in scalar registers.
 struct TilePos {
     uint32_t rows, row0, split, jump;
 };
-__device__ __forceinline__ TilePos pd_tile(const PdGemv& g, uint32_t tile) {
+__device__ __forceinline__ TilePos pd_tile(const Shape& g, uint32_t tile) {
     TilePos t;
     if (g.inter) { t.rows = 64; t.row0 = tile * 32; t.split = 32; t.jump = g.inter - 32; }
     else { t.rows = min(g.T, g.N - tile * g.T); t.row0 = tile * g.T; t.split = 0xFFFFFFFFu; t.jump = 0; }
     return t;
 }
 __device__ __forceinline__ uint32_t pd_row(const TilePos& t, uint32_t lr) { return t.row0 + lr + (lr >= t.split ? t.jump : 0u); }
-__device__ __forceinline__ uint32_t sdiv(uint32_t a, uint32_t b) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)(a / b)); }
+__device__ __forceinline__ uint32_t sdiv(uint32_t a, uint32_t b) { return sgpr(a / b); }
 
 // The weight streamers of a workgroup (waves PD_POLL_WAVES .. PD_WAVES-1, numbered sw = 0 .. PD_STREAM_WAVES-1) split a
 // tile by rows: streamer sw takes tile rows sw, sw + PD_STREAM_WAVES, ... and walks each row's U weight units (1 KB:
 // 32 Q8_0 blocks, two lanes per block, or 64 Q4_0 blocks) in order.  Position p of that walk is unit p % U of the
 // wave's (p / U)-th row; a round is PD_D consecutive positions, all loaded before any is used.
 template <bool Q4>
-__device__ __forceinline__ void pd_load_round(const GemvJob& job, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane, WReg& W) {
+__device__ __forceinline__ void pd_load_round(const GemvJob& job, const Shape& h, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane,
+                                              WReg& W) {
     constexpr uint32_t BPU = Q4 ? 64 : 32, BPB = Q4 ? 16 : 32;
-    const uint32_t U = job.g->U, nblk = job.g->nblk;
+    const uint32_t U = h.U, nblk = h.nblk;
     const uint32_t lb = Q4 ? lane : lane >> 1;
     const uint32_t q = sdiv(round * PD_D, U);
     uint32_t j = round * PD_D - q * U, lr = sw + q * PD_STREAM_WAVES;
@@ -365,7 +386,7 @@ __device__ __forceinline__ void pd_load_round(const GemvJob& job, const TilePos&
     for (int d = 0; d < PD_D; d++) {
         W.v[d] = make_int4(0, 0, 0, 0);
         W.s[d] = 0;
-        if (lr < t.rows) {                                        // wave-uniform
+        if (lr < t.rows) {                                        // wave-uniform (scalar compare and branch)
             const uint32_t blk0 = pd_row(t, lr) * nblk + j * BPU;    // first block of the unit (fits 32 bits: N K / 32)
             if (j * BPU + lb < nblk) {
                 W.v[d] = ldg(reinterpret_cast<const int4*>(job.qs + (size_t)blk0 * BPB) + lane);
@@ -377,18 +398,36 @@ __device__ __forceinline__ void pd_load_round(const GemvJob& job, const TilePos&
     }
 }
 
+// What a weight prefetch needs to know about a matrix.
+struct Mat {
+    uint32_t which;            // shape index; valid == false: nothing follows
+    const uint8_t* qs;
+    const uint16_t* ws;
+    bool q4, valid;
+};
+template <int FMT>
+__device__ __forceinline__ void pd_load_first(const PdArgs& a, const Mat& m, uint32_t wg, uint32_t sw, uint32_t lane, WReg& W) {
+    const Shape h = pd_shape(a.shape[m.which]);
+    if (wg >= h.ntiles) return;
+    const TilePos t = pd_tile(h, wg);
+    GemvJob j{};
+    j.qs = m.qs; j.ws = m.ws;
+    if (FMT == 1 || (FMT == 2 && m.q4)) pd_load_round<true>(j, h, t, 0, sw, lane, W);
+    else pd_load_round<false>(j, h, t, 0, sw, lane, W);
+}
+
 // Exact int32 block dots on v_dot4, one f32 product (a_s*w_s)*f32(isum) per block parked in LDS.
 template <bool Q4>
-__device__ __forceinline__ void pd_compute_round(const GemvJob& job, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane, const WReg& W,
+__device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane, const WReg& W,
                                                  const uint32_t* aq_lds, const float* as_lds, float* prod, uint32_t pstride) {
     constexpr uint32_t BPU = Q4 ? 64 : 32;
-    const uint32_t U = job.g->U, nblk = job.g->nblk;
+    const uint32_t U = h.U, nblk = h.nblk;
     const uint32_t lb = Q4 ? lane : lane >> 1;
     const uint32_t q = sdiv(round * PD_D, U);
     uint32_t j = round * PD_D - q * U, lr = sw + q * PD_STREAM_WAVES;
 #pragma unroll
     for (int d = 0; d < PD_D; d++) {
-        if (lr < t.rows) {                                        // wave-uniform
+        if (lr < t.rows) {                                        // wave-uniform (scalar compare and branch)
             const uint32_t b = j * BPU + lb;
             const bool in = b < nblk;
             const uint32_t bs = in ? b : 0;
@@ -644,26 +683,31 @@ __device__ __forceinline__ ArgPair arg_wg(ArgPair a, float* misc, const PdCtx& c
 //   inputs    the streamers issue the first weight loads of their rows at once; the poller wave fetches the activation
 //             vector (it never has weights in flight, so nothing delays what it polls)
 //   tiles     compute a round from registers, issue the next round (or the next tile's first), sum, finish the rows
-template <bool Q4, int HD>
-__device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& job, const float* emb, uint32_t pos, uint32_t* aq_lds,
-                                              float* as_lds, float* misc, float* big, ArgPair& best, const PdCtx& cx) {
-    const PdGemv& g = *job.g;
-    if (cx.wg >= g.ntiles) return;
+template <bool Q4, int HD, int FMT>
+__device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& job, const Mat& next, bool early, WReg& W, const float* emb,
+                                              uint32_t pos, uint32_t* aq_lds, float* as_lds, float* misc, float* big, ArgPair& best,
+                                              const PdCtx& cx) {
+    const PdGemv& g = a.shape[job.which];
+    const Shape h = pd_shape(g);
     const bool streamer = cx.wave >= (uint32_t)PD_POLL_WAVES;
     const uint32_t sw = cx.wave - PD_POLL_WAVES;
-    const uint32_t pstride = g.nblk + 1;                    // +1: conflict-free column reads
-    const uint32_t K = job.in_len, U = g.U;
-    WReg W;
-    TilePos t = pd_tile(g, cx.wg);
+    if (cx.wg >= h.ntiles) {
+        // nothing to do here; the streamers still start on the matrix that follows
+        if (streamer && next.valid) pd_load_first<FMT>(a, next, cx.wg, sw, cx.lane, W);
+        return;
+    }
+    const uint32_t pstride = h.nblk + 1;                    // +1: conflict-free column reads
+    const uint32_t K = job.in_len, U = h.U;
+    TilePos t = pd_tile(h, cx.wg);
 
     // ---- inputs (norm weights are requested before this wave's weights: loads return in order)
     float4 nw = make_float4(0.f, 0.f, 0.f, 0.f);
     if (job.pro == PRO_NORM && cx.tid * 4 < K) nw = ldg(reinterpret_cast<const float4*>(job.norm_w + cx.tid * 4));
     if (streamer) {
-        pd_load_round<Q4>(job, t, 0, sw, cx.lane, W);
+        if (!early) pd_load_round<Q4>(job, h, t, 0, sw, cx.lane, W);      // otherwise the previous phase's tail issued them
     } else {
-        if (job.pro == PRO_AQ) pd_load_aq(job.tin, job.tin_tag, K, aq_lds, as_lds, misc, cx);
-        else if (job.tin_tag) pd_load_x(job.tin, job.tin_tag, K, big, misc, cx);
+        if (job.pro == PRO_AQ) pd_load_aq(job.tin, job.tin_tag, K, aq_lds, as_lds, misc, a.use_hint != 0, cx);
+        else if (job.tin_tag) pd_load_x(job.tin, job.tin_tag, K, big, misc, a.use_hint != 0, cx);
         else for (uint32_t i = cx.tid; i < K; i += PD_POLL_THREADS) big[i] = emb[i];
     }
     __syncthreads();
@@ -673,10 +717,10 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
 
     // ---- tiles
 #pragma nounroll
-    for (uint32_t tile = cx.wg; tile < g.ntiles; tile += cx.G) {
+    for (uint32_t tile = cx.wg; tile < h.ntiles; tile += cx.G) {
         const uint32_t rounds = ((t.rows + PD_STREAM_WAVES - 1) / PD_STREAM_WAVES * U + PD_D - 1) / PD_D;
-        const bool more = tile + cx.G < g.ntiles;
-        const TilePos tn = more ? pd_tile(g, tile + cx.G) : t;
+        const bool more = tile + cx.G < h.ntiles;
+        const TilePos tn = more ? pd_tile(h, tile + cx.G) : t;
         // what the epilogue needs from global memory is requested early (by wave 0, which streams nothing, for tiles of
         // up to 64 rows)
         const bool mine = cx.tid < t.rows;
@@ -697,15 +741,22 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
         if (streamer) {
 #pragma nounroll
             for (uint32_t r = 0; r < rounds; r++) {
-                pd_compute_round<Q4>(job, t, r, sw, cx.lane, W, aq_lds, as_lds, big, pstride);
-                if (r + 1 < rounds) pd_load_round<Q4>(job, t, r + 1, sw, cx.lane, W);
-                else if (more) pd_load_round<Q4>(job, tn, 0, sw, cx.lane, W);
+                pd_compute_round<Q4>(h, t, r, sw, cx.lane, W, aq_lds, as_lds, big, pstride);
+                if (r + 1 < rounds) pd_load_round<Q4>(job, h, t, r + 1, sw, cx.lane, W);
             }
         }
         __syncthreads();
+        // While the pollers (which own every row of a tile: at most 64 PD_POLL_WAVES rows) sum and finish the rows, the
+        // streamers start on what comes next: the next tile, or the next matrix.  Issuing a wave's loads takes about as
+        // long as the data takes to arrive (the memory pipeline holds only so many misses), so it must not sit between
+        // the products and the sums.
+        if (streamer) {
+            if (more) pd_load_round<Q4>(job, h, tn, 0, sw, cx.lane, W);
+            else if (next.valid) pd_load_first<FMT>(a, next, cx.wg, sw, cx.lane, W);
+        }
         if (cx.tid < ((t.rows + 63u) & ~63u)) {
             float v = 0.f;
-            if (mine) v = ordered_sum(big + cx.tid * pstride, g.nblk, segment_row_is_dot1(row, g.seg, g.nseg, g.tail_mod));
+            if (mine) v = ordered_sum(big + cx.tid * pstride, h.nblk, segment_row_is_dot1(row, g.seg, g.nseg, g.tail_mod));
             if (job.epi == EPI_ROPE) {
                 // rope (emit.rs:508-528): rows 2i, 2i+1 of a head sit in neighbouring lanes
                 const float other = __shfl_xor(v, 1, WAVE);
@@ -757,12 +808,17 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
                 }
             }
         }
-        __syncthreads();
+        // before the next tile's products overwrite this tile's; after the last tile nothing touches LDS until the
+        // next phase's inputs are in (the streamers only issue loads, the pollers write what they poll), so the pollers
+        // need not wait for the streamers' loads to be issued
+        if (more) __syncthreads();
         t = tn;
     }
 }
 
-template <int HD>
+// FMT: which weight formats the kernel carries code for (0: Q8_0 only, 1: Q4_0 only, 2: both) -- a kernel that
+// fits the instruction cache matters more than one binary for all models.
+template <int HD, int FMT>
 __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     __shared__ uint32_t sh_abort;
@@ -787,6 +843,8 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     const float* emb = a.embed + (size_t)token * a.H;
     const uint32_t L = a.n_layers;
     ArgPair best{-INFINITY, 0};
+    WReg W;
+    bool early = false;
 
     // steps 4 l + {0: qkv, 1: attention then o, 2: gate/up, 3: down}; step 4 L: lm_head.  Phase instance k of this
     // launch carries tag tag_base + k: per layer 1 qkv, 2 attention split, 3 attention merge, 4 o, 5 gate/up, 6 down.
@@ -809,10 +867,22 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
             a.stamps[6 * l + slot[ph]] = wall_clock64();
         }
         GemvJob job;
-        job.g = is_lm ? &a.lm : &a.shape[ph];
-        job.qs = is_lm ? a.lm.qs : a.layers[l].qs[ph];
-        job.ws = is_lm ? a.lm.ws : a.layers[l].ws[ph];
+        job.which = ph;
+        job.qs = is_lm ? a.shape[PD_LM].qs : a.layers[l].qs[ph];
+        job.ws = is_lm ? a.shape[PD_LM].ws : a.layers[l].ws[ph];
         job.q4 = is_lm ? a.lm_q4 != 0 : a.q4 != 0;
+        Mat next;
+        {
+            const uint32_t ns = step + 1;
+            const bool n_lm = ns == 4 * L;
+            const uint32_t nl = n_lm ? L - 1 : ns >> 2, nph = n_lm ? 4u : (ns & 3u);
+            // the O projection follows attention, which needs every wave at once: its (few) weights are loaded when it starts
+            next.valid = ns <= 4 * L && nph != 1;
+            next.which = nph;
+            next.qs = n_lm ? a.shape[PD_LM].qs : a.layers[next.valid ? nl : 0].qs[nph & 3u];
+            next.ws = n_lm ? a.shape[PD_LM].ws : a.layers[next.valid ? nl : 0].ws[nph & 3u];
+            next.q4 = n_lm ? a.lm_q4 != 0 : a.q4 != 0;
+        }
         job.pro = (ph == 1 || ph == 3) ? PRO_AQ : PRO_NORM;
         job.epi = ph == 0 ? EPI_ROPE : ph == 2 ? EPI_SILU : ph == 4 ? EPI_LOGITS : EPI_ADD;
         job.norm_w = ph == 0 ? a.layers[l].attn_norm : ph == 2 ? a.layers[l].ffn_norm : a.final_norm;
@@ -823,8 +893,9 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         job.res_tag = ph == 1 ? x_in : base + 4;
         job.kc = a.layers[l].kc;
         job.vc = a.layers[l].vc;
-        if (job.q4) pd_gemv_phase<true, HD>(a, job, emb, pos, aq_lds, as_lds, misc, big, best, cx);
-        else pd_gemv_phase<false, HD>(a, job, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT>(a, job, next, early, W, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        else pd_gemv_phase<false, HD, FMT>(a, job, next, early, W, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        early = next.valid;
         if (sh_abort) return;
     }
 
@@ -910,9 +981,14 @@ bool plan_gemv(const QWeight& w, uint32_t inter, uint32_t nseg, const Segment* s
 }
 
 template <int HD>
+const void* pd_kernel(const PdState* st) {
+    if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2>);
+    return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 1>) : reinterpret_cast<const void*>(decode_step_kernel<HD, 0>);
+}
+template <int HD>
 hipError_t launch_pd_hd(const PdState* st, hipStream_t s) {
     void* kargs[] = {const_cast<PdArgs*>(&st->args)};
-    return hipLaunchCooperativeKernel(reinterpret_cast<void*>(decode_step_kernel<HD>), dim3(st->grid), dim3(PD_THREADS), kargs, st->lds, s);
+    return hipLaunchCooperativeKernel(pd_kernel<HD>(st), dim3(st->grid), dim3(PD_THREADS), kargs, st->lds, s);
 }
 
 }  // namespace
@@ -978,14 +1054,13 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     }
     {
         Segment sl[1] = {make_segment(c.lm_head_dtype, H, 0, c.vocab, true)};
-        if (!plan_gemv(lm_head, 0, 1, sl, 4, st->grid, big, &a.lm)) return FORGE_HIP_OK;
+        if (!plan_gemv(lm_head, 0, 1, sl, 4, st->grid, big, &a.shape[PD_LM])) return FORGE_HIP_OK;
     }
     // cooperative residency: one workgroup per CU must fit
     {
         int per_cu = 0;
         hipError_t e = hipErrorInvalidValue;
-e = hd == 64 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_step_kernel<64>, PD_THREADS, st->lds)
-                     : hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_step_kernel<128>, PD_THREADS, st->lds);
+e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, hd == 64 ? pd_kernel<64>(st.get()) : pd_kernel<128>(st.get()), PD_THREADS, st->lds);
         if (e != hipSuccess || per_cu < 1) { (void)hipGetLastError(); return FORGE_HIP_OK; }
     }
 
@@ -1012,6 +1087,7 @@ e = hd == 64 ? hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, decode_step
     a.tag_base = 0;
     a.spin_limit = 400000;
     a.q4 = st->q4; a.lm_q4 = st->lmq4;
+    { const char* e = getenv("FORGE_HIP_PD_HINT"); a.use_hint = (e && e[0] == '0') ? 0 : 1; }
     st->tags_per_launch = 6 * a.n_layers + 1;
     st->n_stamps = 6 * a.n_layers + 3;
     a.stamps = nullptr;

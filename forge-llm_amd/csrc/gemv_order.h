@@ -42,12 +42,22 @@ __device__ __forceinline__ bool segment_row_is_dot1(uint32_t row, const Segment*
 // dot1 order.  Adds are never fused with the multiplies that made the products.
 __device__ __forceinline__ float ordered_sum(const float* p, uint32_t nblk, bool dot1) {
     if (!dot1) {
+        // the adds form one dependent chain; the reads of the next eight products are issued before the current
+        // eight are added, so that LDS latency stays off that chain
         float r = 0.f;
         uint32_t b = 0;
-        for (; b + 8 <= nblk; b += 8) {          // eight LDS reads in flight, then the dependent adds
-            float v[8];
+        if (nblk >= 8) {
+            float v[8], w[8];
 #pragma unroll
-            for (int i = 0; i < 8; i++) v[i] = p[b + i];
+            for (int i = 0; i < 8; i++) v[i] = p[i];
+            for (b = 8; b + 8 <= nblk; b += 8) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) w[i] = p[b + i];
+#pragma unroll
+                for (int i = 0; i < 8; i++) r = r + v[i];
+#pragma unroll
+                for (int i = 0; i < 8; i++) v[i] = w[i];
+            }
 #pragma unroll
             for (int i = 0; i < 8; i++) r = r + v[i];
         }
