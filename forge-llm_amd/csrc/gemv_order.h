@@ -42,24 +42,38 @@ __device__ __forceinline__ bool segment_row_is_dot1(uint32_t row, const Segment*
 // dot1 order.  Adds are never fused with the multiplies that made the products.
 __device__ __forceinline__ float ordered_sum(const float* p, uint32_t nblk, bool dot1) {
     if (!dot1) {
-        // the adds form one dependent chain; the reads of the next eight products are issued before the current
-        // eight are added, so that LDS latency stays off that chain
+        // the adds form one dependent chain; two register sets alternate so that the reads of the next eight products
+        // are in flight while the current eight are added
         float r = 0.f;
         uint32_t b = 0;
         if (nblk >= 8) {
             float v[8], w[8];
 #pragma unroll
             for (int i = 0; i < 8; i++) v[i] = p[i];
-            for (b = 8; b + 8 <= nblk; b += 8) {
+            b = 8;                                   // v holds products [b - 8, b)
+            while (b + 16 <= nblk) {
 #pragma unroll
                 for (int i = 0; i < 8; i++) w[i] = p[b + i];
 #pragma unroll
                 for (int i = 0; i < 8; i++) r = r + v[i];
 #pragma unroll
-                for (int i = 0; i < 8; i++) v[i] = w[i];
-            }
+                for (int i = 0; i < 8; i++) v[i] = p[b + 8 + i];
 #pragma unroll
-            for (int i = 0; i < 8; i++) r = r + v[i];
+                for (int i = 0; i < 8; i++) r = r + w[i];
+                b += 16;
+            }
+            if (b + 8 <= nblk) {
+#pragma unroll
+                for (int i = 0; i < 8; i++) w[i] = p[b + i];
+#pragma unroll
+                for (int i = 0; i < 8; i++) r = r + v[i];
+#pragma unroll
+                for (int i = 0; i < 8; i++) r = r + w[i];
+                b += 8;
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; i++) r = r + v[i];
+            }
         }
         for (; b < nblk; b++) r = r + p[b];
         return r;
