@@ -5,11 +5,13 @@ script prefills a 2502-token prompt (timed: prefill tok/s), then runs W warm-up 
 decode steps at that context, and prints ONE JSON line.  Weights, KV cache and activations are
 resident in HBM when the timed regions start.
 
-roofline: the decode step's dominant kernel, the quantised GEMV.  `achieved` = algorithmic bytes
-(GGUF block bytes of every matrix + its f32 input and output vectors) of the GEMV launches of one
-token / their summed device time, measured live by the library's forward_profile with a pair of HIP
-events attached to every kernel dispatch on the model's own stream (the kernel's begin-to-end time, the
-figure a kernel trace reports).  `peak` = 8 TB/s (MI355X HBM3E).
+roofline: the decode step's dominant kernel.  By default the whole step is ONE resident kernel
+(decode_step_kernel): `achieved` = algorithmic bytes of one token (GGUF block bytes of every matrix + the
+f32 input and output vectors of each GEMV + the fp16 K/V rows attention reads) / the kernel's duration,
+measured live by the library's forward_profile from the kernel's own clock stamps (one per phase, summed).
+With FORGE_HIP_PERSIST=0 the step is a sequence of kernels and the figure is that of the quantised GEMV
+launches, each timed by a pair of HIP events attached to its dispatch.  The line also carries the other
+path's figures under "kernel_sequence_path".  `peak` = 8 TB/s (MI355X HBM3E).
 
 cpu_baseline: the CPU restatement of the reference's generated kernels (oracle/), in the arithmetic
 the reference runs on an x86 host (f32 activations x dequantised weights, int8 KV), per-token decode,
@@ -33,6 +35,9 @@ PROMPT_TOKENS = 2502
 # WRITE_SIZE counters of two profiler runs of this script, each scaled by what the same counter reads for the 1 GiB
 # copy of --calibrate-copy (FETCH_SIZE x2.000, WRITE_SIZE x1.000).  Summary: profiles/gemv_hbm_traffic_pmc.md.
 GEMV_HBM_BYTES_PER_LAUNCH = 20.46e6 + 0.02e6      # fetched + written
+# The same for one launch of the resident decode kernel (the whole step) at this context: 1 400.9 MB fetched + 13.3 MB
+# written.  Summary: profiles/decode_step_kernel_hbm_traffic_pmc.md.
+STEP_KERNEL_HBM_BYTES_PER_LAUNCH = 1414.2e6
 
 
 def gemv_launch_bytes(fh, cfg):
@@ -78,6 +83,53 @@ def cpu_baseline(fh, cfg, blob, prompt, budget_s=20.0):
                       f"arithmetic of the reference's x86 build, int8 KV, OpenMP over rows with {threads} threads"}
 
 
+def decode_profile(fh, model, cfg, tok, context, prof_steps=8):
+    """Per-stage device time of the decode step and the roofline of its dominant kernel."""
+    stage_ms, stage_n = {}, {}
+    for _ in range(prof_steps):
+        p = model.forward_profile(tok)
+        for s, (ms, n) in p.items():
+            stage_ms[s] = stage_ms.get(s, 0.0) + ms / prof_steps
+            stage_n[s] = stage_n.get(s, 0) + n
+    gbytes = gemv_launch_bytes(fh, cfg)
+    gemv_bytes_total = sum(gbytes.values())
+    per_stage = {s: {"GB/s": round(gbytes[s] / (stage_ms[s] * 1e-3) / 1e9, 1), "us_per_token": round(stage_ms[s] * 1e3, 1)} for s in gbytes}
+    stage_us = {s: round(v * 1e3, 1) for s, v in stage_ms.items() if v > 0}
+    if model.decode_launches == 1:
+        # one resident kernel per token: its phases are the stages, timed by the kernel's own clock stamps
+        kv_bytes = cfg["layers"] * 2 * context * cfg["kv_heads"] * cfg["head_dim"] * 2
+        total = gemv_bytes_total + kv_bytes
+        kernel_ms = sum(stage_ms.values())
+        achieved = total / (kernel_ms * 1e-3) / 1e9
+        roof = {"kernel": "decode_step_kernel (the whole decode step: every quantised GEMV, decode attention, norms, argmax)",
+                "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                "traffic": STEP_KERNEL_HBM_BYTES_PER_LAUNCH, "bytes_per_launch": total, "us_per_launch": kernel_ms * 1e3,
+                "launches_per_step": 1, "weights_and_vectors_bytes": gemv_bytes_total, "kv_cache_bytes": kv_bytes,
+                "per_phase": per_stage}
+    else:
+        gemv_ms = sum(stage_ms[s] for s in gbytes)
+        launches = sum(stage_n[s] for s in gbytes) // prof_steps
+        achieved = gemv_bytes_total / (gemv_ms * 1e-3) / 1e9
+        roof = {"kernel": "gemv_kernel (quantised GEMV, all launches of one decode step)", "bound": "hbm", "achieved": achieved,
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+                "traffic": GEMV_HBM_BYTES_PER_LAUNCH if cfg["wdtype"] == fh.Q8_0 else None,
+                "bytes_per_launch": gemv_bytes_total / launches, "us_per_launch": gemv_ms * 1e3 / launches,
+                "launches_per_step": launches, "per_stage": per_stage}
+    return roof, stage_us
+
+
+def timed_decode(model, tok, warmup, steps):
+    import torch
+    for _ in range(warmup):
+        tok = model.forward_greedy(tok)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        tok = model.forward_greedy(tok)
+    torch.cuda.synchronize()
+    return time.perf_counter() - t0, tok
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -85,6 +137,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-alt", action="store_true", help="skip the second model that measures the kernel-sequence decode step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (known HBM traffic, for scaling counter readings)")
     args = ap.parse_args()
@@ -116,30 +169,8 @@ def main():
     tok = fh.ops.argmax_host(logits)
 
     # ---- decode at context ~2502: W warm-up steps, K timed steps
-    for _ in range(args.warmup):
-        tok = model.forward_greedy(tok)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        tok = model.forward_greedy(tok)
-    torch.cuda.synchronize()
-    t_decode = time.perf_counter() - t0
-
-    # ---- per-kernel device time of the decode step (events around every launch)
-    prof_steps = 8
-    stage_ms, stage_n = {}, {}
-    for _ in range(prof_steps):
-        p = model.forward_profile(tok)
-        for s, (ms, n) in p.items():
-            stage_ms[s] = stage_ms.get(s, 0.0) + ms
-            stage_n[s] = stage_n.get(s, 0) + n
-    gbytes = gemv_launch_bytes(fh, cfg)
-    gemv_ms = sum(stage_ms[s] for s in gbytes) / prof_steps
-    gemv_launches = sum(stage_n[s] for s in gbytes) // prof_steps
-    gemv_bytes_total = sum(gbytes.values())
-    achieved = gemv_bytes_total / (gemv_ms * 1e-3) / 1e9
-    per_stage = {s: {"GB/s": round(gbytes[s] / (stage_ms[s] / prof_steps * 1e-3) / 1e9, 1),
-                     "us_per_launch": round(stage_ms[s] / stage_n[s] * 1e3, 2)} for s in gbytes}
+    t_decode, tok = timed_decode(model, tok, args.warmup, args.steps)
+    roofline, stage_us = decode_profile(fh, model, cfg, tok, PROMPT_TOKENS + args.warmup + args.steps)
 
     # ---- prefill kernels (GEMM / attention) from prefill_profile
     model.reset()
@@ -151,15 +182,24 @@ def main():
     # ---- short-context decode for reference (64-token style run of the reference's decode benchmark)
     model.reset()
     tok2 = fh.ops.argmax_host(model.forward_prefill(prompt[:32]))
-    for _ in range(4):
-        tok2 = model.forward_greedy(tok2)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        tok2 = model.forward_greedy(tok2)
-    torch.cuda.synchronize()
-    t_decode_short = time.perf_counter() - t0
+    t_decode_short, _ = timed_decode(model, tok2, 4, args.steps)
+    path = "one resident kernel per token" if model.decode_launches == 1 else f"{model.decode_launches} kernels per token (graph replay)"
     model.close()
+
+    # ---- the other decode path, for comparison: the step as a sequence of kernels
+    alt = None
+    if not args.no_alt and os.environ.get("FORGE_HIP_PERSIST", "1") != "0":
+        os.environ["FORGE_HIP_PERSIST"] = "0"
+        try:
+            m2 = fh.HipModel(cfg, blob)
+            tk = fh.ops.argmax_host(m2.forward_prefill(prompt))
+            t2, tk = timed_decode(m2, tk, args.warmup, args.steps)
+            roof2, stage2 = decode_profile(fh, m2, cfg, tk, PROMPT_TOKENS + args.warmup + args.steps)
+            alt = {"path": f"{m2.decode_launches} kernels per token (graph replay)", "decode_tok_per_s": args.steps / t2,
+                   "roofline": roof2, "decode_stage_us": stage2}
+            m2.close()
+        finally:
+            os.environ["FORGE_HIP_PERSIST"] = "1"
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)     # 1 GiB
         dst = torch.empty_like(src)
@@ -167,8 +207,6 @@ def main():
         dst.copy_(src)                                                                 # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
-
-    traffic = GEMV_HBM_BYTES_PER_LAUNCH if cfg["wdtype"] == fh.Q8_0 else None
 
     out = {
         "metric": "decode tok/s (Llama-3.2-1B Q8_0, 1 GPU)",
@@ -185,16 +223,13 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"Llama-3.2-1B shape, Q8_0, random-init seed {args.seed}: {PROMPT_TOKENS}-token prompt, "
                                f"then greedy decode at that context", "prompt_tokens": PROMPT_TOKENS,
-                   "decode_context": PROMPT_TOKENS + args.warmup, "mode": "fast (MFMA prefill, split-seq decode attention)"},
+                   "decode_context": PROMPT_TOKENS + args.warmup, "mode": "fast (MFMA prefill, split-seq decode attention)",
+                   "decode_path": path},
         "prefill_tok_per_s": PROMPT_TOKENS / t_prefill,
         "prefill_ms": t_prefill * 1e3,
         "decode_tok_per_s_short_context": args.steps / t_decode_short,
         "decode_weight_stream_GBps_end_to_end": fh.synth.decode_weight_bytes(cfg) * args.steps / t_decode / 1e9,
-        "roofline": {"kernel": "gemv_kernel (quantised GEMV, all launches of one decode step)", "bound": "hbm",
-                     "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                     "traffic": traffic, "bytes_per_launch": gemv_bytes_total / gemv_launches,
-                     "us_per_launch": gemv_ms * 1e3 / gemv_launches, "launches_per_step": gemv_launches,
-                     "per_stage": per_stage},
+        "roofline": roofline,
         "prefill_rooflines": {
             "gemm": {"bound": "mfma", "achieved": gemm_flops / (gemm_ms * 1e-3) / 1e12, "peak": MFMA_I8_PEAK_TOPS,
                      "unit": "TOP/s (int8)", "frac": gemm_flops / (gemm_ms * 1e-3) / 1e12 / MFMA_I8_PEAK_TOPS, "ms": gemm_ms},
@@ -202,7 +237,8 @@ def main():
                           "unit": "TFLOP/s (fp16)", "frac": attn_flops / (attn_ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS,
                           "ms": attn_ms},
         },
-        "decode_stage_us": {s: round(stage_ms[s] / prof_steps * 1e3, 1) for s in stage_ms},
+        "decode_stage_us": stage_us,
+        "kernel_sequence_path": alt,
         "setup_s": {"generate_weights": round(t_gen, 1), "upload_and_repack": round(t_load, 1)},
     }
     if not args.no_cpu_baseline:

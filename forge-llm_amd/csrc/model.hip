@@ -442,7 +442,7 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
         (rc = m->ptok.alloc((size_t)R * 4)))
         return rc;
     const char* penv = getenv("FORGE_HIP_PERSIST");
-    if (penv && penv[0] == '1') {   // opt-in while the kernel sequence is still the faster step
+    if (!(penv && penv[0] == '0')) {
         std::vector<PdLayerIn> pl(cfg->layers);
         for (uint32_t l = 0; l < cfg->layers; l++) {
             Layer& L = m->layers[l];
