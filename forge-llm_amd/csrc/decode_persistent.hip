@@ -416,10 +416,13 @@ __device__ __forceinline__ void pd_load_first(const PdArgs& a, const Mat& m, uin
     else pd_load_round<false>(j, h, t, 0, sw, lane, W);
 }
 
-// Exact int32 block dots on v_dot4, one f32 product (a_s*w_s)*f32(isum) per block parked in LDS.
-template <bool Q4>
+// Exact int32 block dots on v_dot4 and one f32 product (a_s*w_s)*f32(isum) per block.
+//   ORDERED   the products are parked in LDS (prod[row][block]) and summed later in the reference's order
+//   otherwise each lane adds its products of a row as they come (`acc`, carried across rounds) and the wave folds
+//             them when the row's last unit is done: rowsum[row].  Same terms, another order of addition.
+template <bool Q4, bool ORDERED>
 __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane, const WReg& W,
-                                                 const uint32_t* aq_lds, const float* as_lds, float* prod, uint32_t pstride) {
+                                                 const uint32_t* aq_lds, const float* as_lds, float* prod, uint32_t pstride, float& acc) {
     constexpr uint32_t BPU = Q4 ? 64 : 32;
     const uint32_t U = h.U, nblk = h.nblk;
     const uint32_t lb = Q4 ? lane : lane >> 1;
@@ -446,9 +449,23 @@ __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& 
                 const int4 a = *reinterpret_cast<const int4*>(aq_lds + bs * 8 + (lane & 1u) * 4);
                 const int half = dot16(W.v[d], a, 0);             // W is zero where the lane is past the row
                 // the other half of the block sits in the neighbouring lane: quad_perm [1,0,3,2]
-                isum = half + __builtin_amdgcn_update_dpp(0, half, 0xB1, 0xF, 0xF, false);
+                isum = ORDERED ? half + __builtin_amdgcn_update_dpp(0, half, 0xB1, 0xF, 0xF, false) : half;
             }
-            if (in && (Q4 || !(lane & 1u))) prod[lr * pstride + b] = (as_lds[b] * f16_bits_to_f32((uint16_t)W.s[d])) * (float)isum;
+            if (ORDERED) {
+                if (in && (Q4 || !(lane & 1u))) prod[lr * pstride + b] = (as_lds[b] * f16_bits_to_f32((uint16_t)W.s[d])) * (float)isum;
+            } else {
+                if (in) acc += (as_lds[b] * f16_bits_to_f32((uint16_t)W.s[d])) * (float)isum;   // Q8_0: each lane its half block
+                if (j == U - 1) {                                     // wave-uniform: the row is complete
+                    // fold the 16 lanes of each DPP row (pairs, quads, halves, row); the epilogue adds the four row sums
+                    float r = acc;
+                    r += __builtin_amdgcn_update_dpp(0.f, r, 0xB1, 0xF, 0xF, false);     // quad_perm [1,0,3,2]
+                    r += __builtin_amdgcn_update_dpp(0.f, r, 0x4E, 0xF, 0xF, false);     // quad_perm [2,3,0,1]
+                    r += __builtin_amdgcn_update_dpp(0.f, r, 0x141, 0xF, 0xF, false);    // row_half_mirror
+                    r += __builtin_amdgcn_update_dpp(0.f, r, 0x140, 0xF, 0xF, false);    // row_mirror
+                    if ((lane & 15u) == 0) prod[lr * 4 + (lane >> 4)] = r;
+                    acc = 0.f;
+                }
+            }
         }
         j += 1;
         if (j == U) { j = 0; lr += PD_STREAM_WAVES; }
@@ -683,7 +700,7 @@ __device__ __forceinline__ ArgPair arg_wg(ArgPair a, float* misc, const PdCtx& c
 //   inputs    the streamers issue the first weight loads of their rows at once; the poller wave fetches the activation
 //             vector (it never has weights in flight, so nothing delays what it polls)
 //   tiles     compute a round from registers, issue the next round (or the next tile's first), sum, finish the rows
-template <bool Q4, int HD, int FMT>
+template <bool Q4, int HD, int FMT, bool ORDERED>
 __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& job, const Mat& next, bool early, WReg& W, const float* emb,
                                               uint32_t pos, uint32_t* aq_lds, float* as_lds, float* misc, float* big, ArgPair& best,
                                               const PdCtx& cx) {
@@ -716,6 +733,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     if (job.pro == PRO_NORM) pd_norm_quant(big, job.norm_w, nw, a.eps, K, aq_lds, as_lds, misc, cx);
 
     // ---- tiles
+    float acc = 0.f;
 #pragma nounroll
     for (uint32_t tile = cx.wg; tile < h.ntiles; tile += cx.G) {
         const uint32_t rounds = ((t.rows + PD_STREAM_WAVES - 1) / PD_STREAM_WAVES * U + PD_D - 1) / PD_D;
@@ -741,7 +759,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
         if (streamer) {
 #pragma nounroll
             for (uint32_t r = 0; r < rounds; r++) {
-                pd_compute_round<Q4>(h, t, r, sw, cx.lane, W, aq_lds, as_lds, big, pstride);
+                pd_compute_round<Q4, ORDERED>(h, t, r, sw, cx.lane, W, aq_lds, as_lds, big, pstride, acc);
                 if (r + 1 < rounds) pd_load_round<Q4>(job, h, t, r + 1, sw, cx.lane, W);
             }
         }
@@ -756,7 +774,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
         }
         if (cx.tid < ((t.rows + 63u) & ~63u)) {
             float v = 0.f;
-            if (mine) v = ordered_sum(big + cx.tid * pstride, h.nblk, segment_row_is_dot1(row, g.seg, g.nseg, g.tail_mod));
+            if (mine) v = ORDERED ? ordered_sum(big + cx.tid * pstride, h.nblk, segment_row_is_dot1(row, g.seg, g.nseg, g.tail_mod)) : (big[cx.tid * 4] + big[cx.tid * 4 + 1]) + (big[cx.tid * 4 + 2] + big[cx.tid * 4 + 3]);
             if (job.epi == EPI_ROPE) {
                 // rope (emit.rs:508-528): rows 2i, 2i+1 of a head sit in neighbouring lanes
                 const float other = __shfl_xor(v, 1, WAVE);
@@ -818,7 +836,9 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
 
 // FMT: which weight formats the kernel carries code for (0: Q8_0 only, 1: Q4_0 only, 2: both) -- a kernel that
 // fits the instruction cache matters more than one binary for all models.
-template <int HD, int FMT>
+// ORD: the GEMV rows are summed in the reference's block order (bit-identical to the kernel sequence) instead of as the
+// products come.
+template <int HD, int FMT, bool ORD>
 __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     __shared__ uint32_t sh_abort;
@@ -893,8 +913,8 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         job.res_tag = ph == 1 ? x_in : base + 4;
         job.kc = a.layers[l].kc;
         job.vc = a.layers[l].vc;
-        if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT>(a, job, next, early, W, emb, pos, aq_lds, as_lds, misc, big, best, cx);
-        else pd_gemv_phase<false, HD, FMT>(a, job, next, early, W, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT, ORD>(a, job, next, early, W, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        else pd_gemv_phase<false, HD, FMT, ORD>(a, job, next, early, W, emb, pos, aq_lds, as_lds, misc, big, best, cx);
         early = next.valid;
         if (sh_abort) return;
     }
@@ -941,7 +961,7 @@ struct PdState {
     PdArgs args{};
     std::vector<void*> owned;
     uint32_t grid = 0, lds = 0, hd = 0, tags_per_launch = 0, n_stamps = 0;
-    bool q4 = false, lmq4 = false;
+    bool q4 = false, lmq4 = false, ordered = false;
     size_t tagged_bytes = 0;
     void* tagged_base = nullptr;
     std::vector<unsigned long long> stamps_host;
@@ -980,11 +1000,13 @@ bool plan_gemv(const QWeight& w, uint32_t inter, uint32_t nseg, const Segment* s
     return true;
 }
 
-template <int HD>
-const void* pd_kernel(const PdState* st) {
-    if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2>);
-    return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 1>) : reinterpret_cast<const void*>(decode_step_kernel<HD, 0>);
+template <int HD, bool ORD>
+const void* pd_kernel_ord(const PdState* st) {
+    if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2, ORD>);
+    return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 1, ORD>) : reinterpret_cast<const void*>(decode_step_kernel<HD, 0, ORD>);
 }
+template <int HD>
+const void* pd_kernel(const PdState* st) { return st->ordered ? pd_kernel_ord<HD, true>(st) : pd_kernel_ord<HD, false>(st); }
 template <int HD>
 hipError_t launch_pd_hd(const PdState* st, hipStream_t s) {
     void* kargs[] = {const_cast<PdArgs*>(&st->args)};
@@ -1020,6 +1042,8 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     st->q4 = c.wdtype == FORGE_HIP_Q4_0;
     st->lmq4 = c.lm_head_dtype == FORGE_HIP_Q4_0;
     st->wall_khz = khz;
+    // FORGE_HIP_PD_ORDERED=1: GEMV rows summed in the reference's block order, bit-identical to the kernel sequence
+    { const char* e = getenv("FORGE_HIP_PD_ORDERED"); st->ordered = e && e[0] == '1'; }
 
     // LDS: activation codes | activation scales | misc | big
     a.off_act_s = round_up(kmax, 16);
