@@ -54,7 +54,7 @@ namespace {
 
 constexpr int PD_THREADS = 512;
 constexpr int PD_WAVES = PD_THREADS / 64;
-constexpr int PD_D = 16;                      // weight units (1 KB) a wave holds in registers per round
+constexpr int PD_D = 8;                       // weight units (1 KB) a wave holds in registers per round
 constexpr uint32_t PD_MAX_TILE_ROWS = 128;      // = 64 PD_POLL_WAVES: the pollers own a tile's rows
 constexpr uint32_t PD_LDS_BYTES = 64 * 1024;
 constexpr uint32_t PD_MISC_BYTES = 2048;
@@ -62,7 +62,7 @@ constexpr int PD_POLL_WAVES = 2;              // waves that fetch a phase's inpu
 constexpr int PD_POLL_THREADS = PD_POLL_WAVES * 64;
 constexpr int PD_STREAM_WAVES = PD_WAVES - PD_POLL_WAVES;
 constexpr int PD_POLL_N = 20;                 // tagged elements a poller thread takes per round trip
-// misc LDS (floats): [0,32) norm partial sums, [40] hint flag, [64,128) phase scratch
+// misc LDS (floats): [0,33) norm partial sums, [40] hint flag, [64,128) phase scratch
 constexpr int PD_MISC_HINT = 40, PD_MISC_SCRATCH = 64;
 
 struct PdGemv {
@@ -254,11 +254,32 @@ __device__ __forceinline__ int dot16(int4 w, int4 a, int acc) {
 // rms_norm (emit.rs:327-334, 16-lane FMA order of emit.rs:272-295) + activation quantiser (emit.rs:1410-1440).
 // xs must already hold x[0..H); `part` is 32 floats of LDS; nw0 = norm_w[4 tid .. 4 tid + 4), requested by the
 // caller before any weight load of this wave.
+// ORDERED: the sum of squares in the reference's order (16 accumulators walked in sequence); otherwise every thread
+// squares its own elements and the workgroup folds them (same terms, another order of addition).
+template <bool ORDERED>
 __device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict__ norm_w, float4 nw0, float eps, uint32_t H,
                                               uint32_t* aq_lds, float* as_lds, float* part, const PdCtx& cx) {
     const uint32_t tid = cx.tid;
     __syncthreads();
-    if (tid < 64) {
+    if (!ORDERED) {
+        float s = 0.f;
+        for (uint32_t e0 = tid * 4; e0 < H; e0 += PD_THREADS * 4) {
+            const float4 xv = *reinterpret_cast<const float4*>(xs + e0);
+            s += (xv.x * xv.x + xv.y * xv.y) + (xv.z * xv.z + xv.w * xv.w);
+        }
+        s += __builtin_amdgcn_update_dpp(0.f, s, 0xB1, 0xF, 0xF, false);      // quad_perm [1,0,3,2]
+        s += __builtin_amdgcn_update_dpp(0.f, s, 0x4E, 0xF, 0xF, false);      // quad_perm [2,3,0,1]
+        s += __builtin_amdgcn_update_dpp(0.f, s, 0x141, 0xF, 0xF, false);     // row_half_mirror
+        s += __builtin_amdgcn_update_dpp(0.f, s, 0x140, 0xF, 0xF, false);     // row_mirror
+        if ((tid & 15u) == 0) part[tid >> 4] = s;                             // PD_THREADS / 16 = 32 partial sums
+        __syncthreads();
+        if (tid == 0) {
+            float r = 0.f;
+#pragma unroll
+            for (int i = 0; i < PD_THREADS / 16; i++) r += part[i];
+            part[PD_THREADS / 16] = r;
+        }
+    } else if (tid < 64) {
         // lane i < 16 owns accumulator i: x[i], x[16 + i], ... added in order with FMAs.  The reads of the next eight
         // values are issued before the current eight are consumed, so LDS latency stays off the dependent chain.
         float s = 0.f;
@@ -285,11 +306,11 @@ __device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict
         float r = (t + __shfl(t, (tid + 1) & 63, WAVE)) + (__shfl(t, (tid + 2) & 63, WAVE) + __shfl(t, (tid + 3) & 63, WAVE));
         if (tid == 0) {
             for (uint32_t i = H / 16 * 16; i < H; i++) r = r + xs[i] * xs[i];
-            part[16] = r;
+            part[PD_THREADS / 16] = r;
         }
     }
     __syncthreads();
-    const float inv_rms = 1.0f / sqrtf(part[16] / (float)H + eps);
+    const float inv_rms = 1.0f / sqrtf(part[PD_THREADS / 16] / (float)H + eps);
     for (uint32_t e0 = tid * 4; e0 < H; e0 += PD_THREADS * 4) {
         const float4 xv = *reinterpret_cast<const float4*>(xs + e0);
         const float4 wv = e0 == tid * 4 ? nw0 : ldg(reinterpret_cast<const float4*>(norm_w + e0));
@@ -374,6 +395,9 @@ __device__ __forceinline__ uint32_t sdiv(uint32_t a, uint32_t b) { return sgpr(a
 // tile by rows: streamer sw takes tile rows sw, sw + PD_STREAM_WAVES, ... and walks each row's U weight units (1 KB:
 // 32 Q8_0 blocks, two lanes per block, or 64 Q4_0 blocks) in order.  Position p of that walk is unit p % U of the
 // wave's (p / U)-th row; a round is PD_D consecutive positions, all loaded before any is used.
+// Every slot issues its two loads whatever the shape (slots past the wave's rows and lanes past a row's end re-read a
+// valid address and their data is ignored): the number of loads in flight is then known at compile time and a round can
+// be consumed while the next one is still arriving.
 template <bool Q4>
 __device__ __forceinline__ void pd_load_round(const GemvJob& job, const Shape& h, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane,
                                               WReg& W) {
@@ -384,15 +408,12 @@ __device__ __forceinline__ void pd_load_round(const GemvJob& job, const Shape& h
     uint32_t j = round * PD_D - q * U, lr = sw + q * PD_STREAM_WAVES;
 #pragma unroll
     for (int d = 0; d < PD_D; d++) {
-        W.v[d] = make_int4(0, 0, 0, 0);
-        W.s[d] = 0;
-        if (lr < t.rows) {                                        // wave-uniform (scalar compare and branch)
-            const uint32_t blk0 = pd_row(t, lr) * nblk + j * BPU;    // first block of the unit (fits 32 bits: N K / 32)
-            if (j * BPU + lb < nblk) {
-                W.v[d] = ldg(reinterpret_cast<const int4*>(job.qs + (size_t)blk0 * BPB) + lane);
-                W.s[d] = ldg(job.ws + blk0 + lb);
-            }
-        }
+        const uint32_t lrc = lr < t.rows ? lr : 0;                // a tile has at least one row
+        const uint32_t b = j * BPU + lb;
+        const uint32_t bc = b < nblk ? b : nblk - 1;
+        const uint32_t bi = pd_row(t, lrc) * nblk + bc;             // block index in the matrix (fits 32 bits: N K / 32)
+        W.v[d] = ldg(reinterpret_cast<const int4*>(job.qs + (size_t)bi * BPB + (Q4 ? 0u : (lane & 1u) * 16u)));
+        W.s[d] = ldg(job.ws + bi);
         j += 1;
         if (j == U) { j = 0; lr += PD_STREAM_WAVES; }
     }
@@ -447,7 +468,7 @@ __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& 
                 isum = dot16(hi, a1, dot16(lo, a0, 0)) - asum8;
             } else {
                 const int4 a = *reinterpret_cast<const int4*>(aq_lds + bs * 8 + (lane & 1u) * 4);
-                const int half = dot16(W.v[d], a, 0);             // W is zero where the lane is past the row
+                const int half = in ? dot16(W.v[d], a, 0) : 0;    // lanes past the row's end hold another block's data
                 // the other half of the block sits in the neighbouring lane: quad_perm [1,0,3,2]
                 isum = ORDERED ? half + __builtin_amdgcn_update_dpp(0, half, 0xB1, 0xF, 0xF, false) : half;
             }
@@ -701,7 +722,7 @@ __device__ __forceinline__ ArgPair arg_wg(ArgPair a, float* misc, const PdCtx& c
 //             vector (it never has weights in flight, so nothing delays what it polls)
 //   tiles     compute a round from registers, issue the next round (or the next tile's first), sum, finish the rows
 template <bool Q4, int HD, int FMT, bool ORDERED>
-__device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& job, const Mat& next, bool early, WReg& W, const float* emb,
+__device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& job, const Mat& next, bool early, WReg& W, WReg& W1, const float* emb,
                                               uint32_t pos, uint32_t* aq_lds, float* as_lds, float* misc, float* big, ArgPair& best,
                                               const PdCtx& cx) {
     const PdGemv& g = a.shape[job.which];
@@ -730,7 +751,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     __syncthreads();
     if (*cx.sh_abort) return;
     // the norm reads big[0..K); the products reuse the area afterwards
-    if (job.pro == PRO_NORM) pd_norm_quant(big, job.norm_w, nw, a.eps, K, aq_lds, as_lds, misc, cx);
+    if (job.pro == PRO_NORM) pd_norm_quant<ORDERED>(big, job.norm_w, nw, a.eps, K, aq_lds, as_lds, misc, cx);
 
     // ---- tiles
     float acc = 0.f;
@@ -757,10 +778,16 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
             }
         }
         if (streamer) {
+            // two register sets alternate: a round is computed while the next one is arriving; round 0 of a tile is
+            // always in W
 #pragma nounroll
-            for (uint32_t r = 0; r < rounds; r++) {
+            for (uint32_t r = 0; r < rounds; r += 2) {
+                if (r + 1 < rounds) pd_load_round<Q4>(job, h, t, r + 1, sw, cx.lane, W1);
                 pd_compute_round<Q4, ORDERED>(h, t, r, sw, cx.lane, W, aq_lds, as_lds, big, pstride, acc);
-                if (r + 1 < rounds) pd_load_round<Q4>(job, h, t, r + 1, sw, cx.lane, W);
+                if (r + 1 < rounds) {
+                    if (r + 2 < rounds) pd_load_round<Q4>(job, h, t, r + 2, sw, cx.lane, W);
+                    pd_compute_round<Q4, ORDERED>(h, t, r + 1, sw, cx.lane, W1, aq_lds, as_lds, big, pstride, acc);
+                }
             }
         }
         __syncthreads();
@@ -863,7 +890,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     const float* emb = a.embed + (size_t)token * a.H;
     const uint32_t L = a.n_layers;
     ArgPair best{-INFINITY, 0};
-    WReg W;
+    WReg W, W1;
     bool early = false;
 
     // steps 4 l + {0: qkv, 1: attention then o, 2: gate/up, 3: down}; step 4 L: lm_head.  Phase instance k of this
@@ -913,8 +940,8 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         job.res_tag = ph == 1 ? x_in : base + 4;
         job.kc = a.layers[l].kc;
         job.vc = a.layers[l].vc;
-        if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT, ORD>(a, job, next, early, W, emb, pos, aq_lds, as_lds, misc, big, best, cx);
-        else pd_gemv_phase<false, HD, FMT, ORD>(a, job, next, early, W, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT, ORD>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        else pd_gemv_phase<false, HD, FMT, ORD>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
         early = next.valid;
         if (sh_abort) return;
     }
