@@ -547,6 +547,22 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
         const uint32_t t0 = split * chunk;
         const uint32_t t1 = min(seq, t0 + chunk);
         const bool has_new = t0 <= pos && pos < t1;
+        // The cached K/V rows do not depend on q: the first key blocks of this wave are requested before q is awaited (loads
+        // return in order, so the wait for q then costs the longer of the two latencies, not their sum).
+        constexpr int UNR = 4;        // key blocks whose K/V loads are issued together
+        const uint32_t tbw = t0 + wave * KPW;
+        Half8 kr0[UNR], vr0[UNR];
+#pragma unroll
+        for (int u = 0; u < UNR; u++) {
+            const uint32_t t = tbw + u * 4 * KPW + slot;
+            kr0[u] = Half8{{0, 0, 0, 0}};
+            vr0[u] = Half8{{0, 0, 0, 0}};
+            if (t < t1 && dvalid && t != pos) {
+                const size_t off = (size_t)t * kv_stride + kvh * HD + c * 8;
+                kr0[u] = ldg(reinterpret_cast<const Half8*>(kc + off));
+                vr0[u] = ldg(reinterpret_cast<const Half8*>(vc + off));
+            }
+        }
         // q is awaited even when the split is empty: the wait orders this item's records after the previous layer's readers
         for (uint32_t e = cx.tid; e < gt * HD || (has_new && e < 2 * HD); e += PD_THREADS) {
             const bool need_q = e < gt * HD, need_kv = has_new && e < 2 * HD;
@@ -560,20 +576,30 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
         }
         __syncthreads();
         if (*cx.sh_abort) return;
+#pragma unroll
+        for (int u = 0; u < UNR; u++) {                      // this position's row arrived with q
+            const uint32_t t = tbw + u * 4 * KPW + slot;
+            if (t == pos && t < t1 && dvalid) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    kr0[u].w[i] = (kvn[c * 8 + 2 * i] & 0xFFFFu) | (kvn[c * 8 + 2 * i + 1] << 16);
+                    vr0[u].w[i] = (kvn[HD + c * 8 + 2 * i] & 0xFFFFu) | (kvn[HD + c * 8 + 2 * i + 1] << 16);
+                }
+            }
+        }
 
         for (uint32_t g = cx.wave >> 2; g < gt; g += PD_WAVES / 4) {
             float qf[8], acc[8], m = -INFINITY, l = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; i++) { acc[i] = 0.f; qf[i] = dvalid ? q_lds[g * HD + c * 8 + i] : 0.f; }
-            constexpr int UNR = 4;        // key blocks whose K/V loads are issued together
-            for (uint32_t tb0 = t0 + wave * KPW; tb0 < t1; tb0 += UNR * 4 * KPW) {
+            for (uint32_t tb0 = tbw; tb0 < t1; tb0 += UNR * 4 * KPW) {
                 Half8 kr[UNR], vr[UNR];
 #pragma unroll
                 for (int u = 0; u < UNR; u++) {
                     const uint32_t t = tb0 + u * 4 * KPW + slot;
-                    kr[u] = Half8{{0, 0, 0, 0}};
-                    vr[u] = Half8{{0, 0, 0, 0}};
-                    if (t < t1 && dvalid) {
+                    kr[u] = kr0[u];
+                    vr[u] = vr0[u];
+                    if (tb0 != tbw && t < t1 && dvalid) {
                         if (t == pos) {
 #pragma unroll
                             for (int i = 0; i < 4; i++) {
@@ -585,6 +611,9 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
                             kr[u] = ldg(reinterpret_cast<const Half8*>(kc + off));
                             vr[u] = ldg(reinterpret_cast<const Half8*>(vc + off));
                         }
+                    } else if (tb0 != tbw) {
+                        kr[u] = Half8{{0, 0, 0, 0}};
+                        vr[u] = Half8{{0, 0, 0, 0}};
                     }
                 }
 #pragma unroll
@@ -657,7 +686,7 @@ __device__ __forceinline__ void pd_attn_combine(const PdArgs& a, uint32_t tag_in
     float* recs = big;                           // [DECODE_SPLITS][REC]
     for (uint32_t h = cx.wg; h < a.heads; h += cx.G) {
         const uint64_t* base = a.tws + (size_t)h * DECODE_SPLITS * REC;
-        poll_vec<4>(base, DECODE_SPLITS * REC, tag_in, PD_THREADS, cx, Hint{nullptr, nullptr},
+        poll_vec<(DECODE_SPLITS * REC + PD_THREADS - 1) / PD_THREADS>(base, DECODE_SPLITS * REC, tag_in, PD_THREADS, cx, Hint{nullptr, nullptr},
                     [&](uint32_t i, uint32_t p) { recs[i] = __uint_as_float(p); });
         __syncthreads();
         if (*cx.sh_abort) return;
@@ -833,7 +862,8 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
                 const uint32_t lr = cx.tid;
                 const float ux = __shfl(v, (cx.lane & 31u) + 32, WAVE);
                 if (lr < 32) {
-                    const float o = (v / (1.0f + expf_ref<true>(-v))) * ux;          // silu_mul, emit.rs:380-386
+                    // silu_mul, emit.rs:380-386; the C library's expf bit for bit where the reference order is asked for
+                    const float o = (v / (1.0f + (ORDERED ? expf_ref<true>(-v) : __expf(-v)))) * ux;
                     float amax = fabsf(o);
 #pragma unroll
                     for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
