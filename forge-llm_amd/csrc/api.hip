@@ -169,6 +169,7 @@ int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, ui
         for (uint32_t r = 0; r < M; r++)
             launch_gemv_isums(w->w, q + (size_t)r * w->w.K, out_dev + (size_t)r * w->w.N * nblk, (hipStream_t)stream);
     } else {
+        FH_CHECK((uint64_t)M * w->w.N * nblk * 4 < 0x7FFFFFFFull, "block_isums: more than 2 GiB of block sums in one call");
         // The GEMM kernel also writes y; give it the tail of the scratch as a sink.
         Scratch& sink = g_attn;
         rc = sink.reserve((size_t)M * w->w.N * sizeof(float));

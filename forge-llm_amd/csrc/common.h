@@ -173,7 +173,9 @@ struct PdState;
 int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layers, const QWeight& lm_head, const float* embed,
                   const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, PdState** out);
 void pd_destroy(PdState* st);
-int32_t pd_enqueue(PdState* st, bool profile, hipStream_t s);
+int32_t pd_enqueue(PdState* st, bool profile, uint32_t token, hipStream_t s);
+// Spins on the host word the kernel writes last; false = not available, wait for the stream instead.
+bool pd_wait_token(PdState* st, uint32_t* next);
 // Call with the abort flag read back after the stream drained; resets the exchange buffers and fails if it is set.
 int32_t pd_after_sync(PdState* st, uint32_t abort_flag, hipStream_t s);
 // Milliseconds between the phase starts of the last profiled step: six per layer, then head and argmax.

@@ -43,6 +43,8 @@
 #include <memory>
 #include <vector>
 
+#include <chrono>
+
 #include "common.h"
 #include "device_utils.h"
 #include "expf_ref.h"
@@ -106,6 +108,9 @@ struct PdArgs {
     float* logits;
     uint32_t* state;   // [0] position  [1] token  [2] next token  [3] abort flag
     uint32_t tag_base, spin_limit;
+    uint32_t token, token_from_arg;            // the step's input token when the host passes it with the launch
+    unsigned long long* host_out;              // host-mapped {next token, launch number}: written last, or null
+    uint32_t host_seq;
     uint32_t q4, lm_q4;                        // weight formats: projections, lm_head
     uint32_t use_hint;                         // pollers wait for one watched element before re-reading a whole buffer
     uint32_t off_act_s, off_misc, off_big;     // LDS byte offsets (activation codes sit at 0)
@@ -916,7 +921,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     if (cx.tid == 0) { sh_abort = 0; reinterpret_cast<uint32_t*>(misc)[PD_MISC_HINT] = 0; }
     __syncthreads();
 
-    const uint32_t pos = a.state[0], token = a.state[1];
+    const uint32_t pos = a.state[0], token = a.token_from_arg ? a.token : a.state[1];
     const float* emb = a.embed + (size_t)token * a.H;
     const uint32_t L = a.n_layers;
     ArgPair best{-INFINITY, 0};
@@ -998,6 +1003,9 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
             a.state[1] = p.i;
             a.state[0] = pos + 1;
             if (a.stamps) a.stamps[6 * L + 2] = wall_clock64();
+            // the host may be spinning on this word instead of waiting for the stream
+            if (a.host_out)
+                __hip_atomic_store(a.host_out, ((unsigned long long)a.host_seq << 32) | p.i, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
         }
     }
 }
@@ -1023,7 +1031,13 @@ struct PdState {
     void* tagged_base = nullptr;
     std::vector<unsigned long long> stamps_host;
     int wall_khz = 0;
-    ~PdState() { for (void* p : owned) (void)hipFree(p); }
+    unsigned long long* host_out = nullptr;    // pinned, mapped into the device's address space
+    unsigned long long* host_out_dev = nullptr;
+    uint32_t seq = 0;
+    ~PdState() {
+        for (void* p : owned) (void)hipFree(p);
+        if (host_out) (void)hipHostFree(host_out);
+    }
 };
 
 namespace {
@@ -1169,6 +1183,23 @@ e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, hd == 64 ? pd_kernel<6
     a.spin_limit = 400000;
     a.q4 = st->q4; a.lm_q4 = st->lmq4;
     { const char* e = getenv("FORGE_HIP_PD_HINT"); a.use_hint = (e && e[0] == '0') ? 0 : 1; }
+    a.token = 0; a.token_from_arg = 0; a.host_out = nullptr; a.host_seq = 0;
+    if (!(getenv("FORGE_HIP_PD_HOSTWORD") && getenv("FORGE_HIP_PD_HOSTWORD")[0] == '0')) {
+        void* hp = nullptr;
+        if (hipHostMalloc(&hp, 64, hipHostMallocMapped) == hipSuccess) {
+            void* dp = nullptr;
+            if (hipHostGetDevicePointer(&dp, hp, 0) == hipSuccess) {
+                st->host_out = reinterpret_cast<unsigned long long*>(hp);
+                st->host_out_dev = reinterpret_cast<unsigned long long*>(dp);
+                st->host_out[0] = 0;
+            } else {
+                (void)hipGetLastError();
+                (void)hipHostFree(hp);
+            }
+        } else {
+            (void)hipGetLastError();
+        }
+    }
     st->tags_per_launch = 6 * a.n_layers + 1;
     st->n_stamps = 6 * a.n_layers + 3;
     a.stamps = nullptr;
@@ -1176,10 +1207,14 @@ e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, hd == 64 ? pd_kernel<6
     return FORGE_HIP_OK;
 }
 
-// Enqueue one decode step (token and position are in `state`).  With `profile` the kernel also records
-// the wall clock at the start of every phase.
-int32_t pd_enqueue(PdState* st, bool profile, hipStream_t s) {
+// Enqueue one decode step at the position in `state` for `token` (travels as a kernel argument).  With `profile`
+// the kernel also records the wall clock at the start of every phase.
+int32_t pd_enqueue(PdState* st, bool profile, uint32_t token, hipStream_t s) {
     PdArgs& a = st->args;
+    a.token = token;
+    a.token_from_arg = 1;
+    a.host_out = st->host_out_dev;
+    if (a.host_out) a.host_seq = ++st->seq;
     if (a.tag_base > 0xF0000000u) {      // tags are about to wrap: start again from zeroed buffers
         FH_HIP(hipMemsetAsync(st->tagged_base, 0, st->tagged_bytes, s));
         a.tag_base = 0;
@@ -1195,6 +1230,22 @@ int32_t pd_enqueue(PdState* st, bool profile, hipStream_t s) {
     if (e != hipSuccess) return fail(FORGE_HIP_ERR_HIP, std::string("persistent decode launch: ") + hipGetErrorString(e));
     a.tag_base += st->tags_per_launch;
     return FORGE_HIP_OK;
+}
+
+// Waits for the next token of the step enqueued last by watching the word the kernel writes into host memory
+// when its result is final (a few microseconds earlier than the stream reports completion, and without a
+// device-to-host copy).  Returns false if the word is not in use or did not arrive in time: the caller then
+// waits for the stream and reads the state from the device.
+bool pd_wait_token(PdState* st, uint32_t* next) {
+    if (!st->host_out || !st->args.host_out) return false;
+    const volatile unsigned long long* w = st->host_out;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (uint32_t spin = 0;; spin++) {
+        const unsigned long long v = *w;
+        if ((uint32_t)(v >> 32) == st->seq) { *next = (uint32_t)v; return true; }
+        if ((spin & 1023u) == 1023u &&
+            std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(200)) return false;
+    }
 }
 
 // After the stream has drained: did every workgroup get through?  (state[3] is the abort flag.)

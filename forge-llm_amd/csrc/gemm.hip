@@ -13,9 +13,18 @@
 // kernel: 32 VALU instructions (128 cycles) per 64 cycles of MFMA.
 //
 // Tiling: 256 threads = 4 waves (2x2), workgroup tile 128 (m) x 128 (n), wave tile 64x64 = 2x2 MFMA
-// tiles, K step 128 (4 blocks) staged through padded LDS.  Activations are the MFMA A operand (rows),
-// weights the B operand (columns): a lane's 16 results share one weight row n, stores are contiguous in n.
+// tiles, K step 128 (4 blocks).  Activations are the MFMA A operand (rows), weights the B operand
+// (columns): a lane's 16 results share one weight row n, stores are contiguous in n.
 // Two waves per SIMD (<= 256 VGPRs) so that MFMA results land in ordinary VGPRs, not AccVGPRs.
+//
+// Data movement: int8 operand tiles go from global memory straight into LDS (buffer loads with the LDS
+// destination; Q4_0 weights pass through registers to have their nibbles expanded), into one of two
+// buffers, so that a stage needs one barrier and the loads of stage s+1 fly under the arithmetic of
+// stage s.  LDS rows are 128 B, unpadded; the 16-byte chunk c of row r sits at position
+// c ^ ((r >> 1) & 7), which makes the fragment reads (32 rows x one chunk) free of bank conflicts.
+// All global accesses go through buffer descriptors: rows past the end of a matrix read as zero and
+// stores past the end are dropped by the hardware's range check, so the loops carry no predication.
+// A K tail (K % 128) reads whatever follows in the row-major matrix; those blocks get scale 0.
 #include "common.h"
 #include "device_utils.h"
 
@@ -27,8 +36,15 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 
 constexpr int BM = 128, BN = 128, BK = 128;   // BK in elements (= bytes of int8)
-constexpr int LDS_STRIDE = BK + 16;           // padded row stride: conflict-free 16-byte reads
 constexpr int KB = BK / 32;                   // quant blocks per stage
+constexpr int TILE_BYTES = BM * BK;           // one operand tile of one stage in LDS
+// LDS map: A tiles [2], B tiles [2], A scales [2][128 rows][4] fp16, B scales likewise, 512 zero bytes
+constexpr int LDS_A = 0, LDS_B = 2 * TILE_BYTES, LDS_ASC = 4 * TILE_BYTES, LDS_BSC = LDS_ASC + 2 * BM * KB * 2,
+              LDS_ZERO = LDS_BSC + 2 * BN * KB * 2, GEMM_LDS_BYTES = LDS_ZERO + 512;
+constexpr uint32_t RSRC_FLAGS = 0x00020000;   // raw buffer, 32-bit data format
+constexpr uint32_t OOB = 0x80000000u;         // an offset no descriptor here covers
+
+#define FH_LDS3(p) ((__attribute__((address_space(3))) void*)(p))
 
 // (c - 8) for each of four nibble codes c held in the low nibbles of the four bytes.
 __device__ __forceinline__ uint32_t nib_minus8(uint32_t x) {
@@ -41,16 +57,92 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ wsc, const int8_t* __restrict__ aq,
                    const uint16_t* __restrict__ asc, float* __restrict__ y, int32_t* __restrict__ isums, uint32_t M,
                    uint32_t N, uint32_t K, uint32_t ldy, int accumulate) {
-    __shared__ __attribute__((aligned(16))) int8_t As[BM * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) int8_t Bs[BN * LDS_STRIDE];
-    __shared__ uint16_t Asc[KB][BM];     // fp16 scale bits
-    __shared__ uint16_t Bsc[KB][BN];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t tid = threadIdx.x, lane = tid & 63;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // uniform: the compiler keeps it scalar
     const uint32_t wm = wave >> 1, wn = wave & 1;
     const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
     const uint32_t nblk = K / 32;
     const uint32_t lrow = lane & 31, lhalf = lane >> 5;
+    const uint32_t wrow = Q4 ? K / 2 : K;   // bytes of one weight row
+
+    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)aq, 0, M * K, RSRC_FLAGS);
+    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void*)wq, 0, N * wrow, RSRC_FLAGS);
+    const __amdgpu_buffer_rsrc_t ras = __builtin_amdgcn_make_buffer_rsrc((void*)asc, 0, M * nblk * 2, RSRC_FLAGS);
+    const __amdgpu_buffer_rsrc_t rdump = __builtin_amdgcn_make_buffer_rsrc((void*)isums, 0, DUMP ? M * N * nblk * 4 : 0, RSRC_FLAGS);
+    const __amdgpu_buffer_rsrc_t rws = __builtin_amdgcn_make_buffer_rsrc((void*)wsc, 0, N * nblk * 2, RSRC_FLAGS);
+
+    // ---- loader mapping: load i of wave w fills LDS rows (4i + w) * 8 .. + 8 of a tile, lane -> (row, position)
+    const uint32_t ld_row = wave * 8 + (lane >> 3);                        // + 32 i
+    const uint32_t ld_chunk = (lane & 7) ^ ((ld_row >> 1) & 7);            // global chunk for LDS position lane & 7
+    const uint32_t a_voff = (m0 + ld_row) * K + ld_chunk * 16;             // + 32 i K + k0
+    const uint32_t w_voff = (n0 + ld_row) * K + ld_chunk * 16;             // Q8_0 only
+    // Q4_0: piece idx = tid + 256 i: row = idx / 4, block = idx % 4 (16 packed bytes -> 32 codes)
+    const uint32_t q4_row = tid >> 2, q4_blk = tid & 3;                    // + 64 i
+    const uint32_t q4_voff = ((n0 + q4_row) * nblk + q4_blk) * 16;         // + 64 i nblk 16 + (k0/32) 16
+    // scales: threads 0..127 take activation row tid, threads 128..255 weight row tid - 128
+    const bool sc_is_a = wave < 2;
+    const uint32_t sc_row = tid & 127;
+    const uint32_t sc_voff = ((sc_is_a ? m0 : n0) + sc_row) * nblk * 2;
+
+    v4i rb[2];
+    uint32_t rs[KB];
+
+    auto issue_stage = [&](uint32_t k0, uint32_t buf) {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, FH_LDS3(lds + LDS_A + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
+                                                     a_voff + i * 32 * K + k0, 0, 0, 0);
+        if (Q4) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, q4_voff + i * 64 * nblk * 16 + (k0 / 32) * 16, 0, 0);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, FH_LDS3(lds + LDS_B + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
+                                                         w_voff + i * 32 * K + k0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int b = 0; b < KB; b++) {
+            const uint32_t v = sc_is_a ? __builtin_amdgcn_raw_buffer_load_b16(ras, sc_voff + b * 2 + (k0 / 32) * 2, 0, 0)
+                                       : __builtin_amdgcn_raw_buffer_load_b16(rws, sc_voff + b * 2 + (k0 / 32) * 2, 0, 0);
+            rs[b] = (k0 / 32 + b < nblk) ? (v & 0xFFFFu) : 0u;
+        }
+    };
+
+    // what passes through registers: expanded Q4_0 codes and the scales
+    auto commit_stage = [&](uint32_t buf) {
+        if (Q4) {
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const uint32_t row = q4_row + 64 * i, sw = (row >> 1) & 7;
+                const v4i p = rb[i];
+                const uint32_t m = 0x0F0F0F0Fu;
+                v4i lo, hi;
+                lo.x = nib_minus8((uint32_t)p.x & m); lo.y = nib_minus8((uint32_t)p.y & m);
+                lo.z = nib_minus8((uint32_t)p.z & m); lo.w = nib_minus8((uint32_t)p.w & m);
+                hi.x = nib_minus8(((uint32_t)p.x >> 4) & m); hi.y = nib_minus8(((uint32_t)p.y >> 4) & m);
+                hi.z = nib_minus8(((uint32_t)p.z >> 4) & m); hi.w = nib_minus8(((uint32_t)p.w >> 4) & m);
+                uint8_t* base = lds + LDS_B + buf * TILE_BYTES + row * BK;
+                *reinterpret_cast<v4i*>(base + ((q4_blk * 2) ^ sw) * 16) = lo;       // elements 0..15 of the block
+                *reinterpret_cast<v4i*>(base + ((q4_blk * 2 + 1) ^ sw) * 16) = hi;   // elements 16..31
+            }
+        }
+        uint2 pk;
+        pk.x = rs[0] | (rs[1] << 16);
+        pk.y = rs[2] | (rs[3] << 16);
+        *reinterpret_cast<uint2*>(lds + (sc_is_a ? LDS_ASC : LDS_BSC) + buf * (BM * KB * 2) + sc_row * (KB * 2)) = pk;
+    };
+
+    // ---- fragment addresses (bytes from the start of a tile / of a scale table)
+    const uint32_t f_sw = (lrow >> 1) & 7;
+    const uint32_t fa_off = (wm * 64 + lrow) * BK + ((lhalf ^ f_sw) * 16);          // chunk of block kb: ^ (kb * 32)
+    const uint32_t fb_off = (wn * 64 + lrow) * BK + ((lhalf ^ f_sw) * 16);
+    // scale operand of the rank-1 product: lanes 0..31 hold k = 0 (the scale), lanes 32..63 read zeros
+    const uint32_t sa_off = lhalf ? (uint32_t)LDS_ZERO : LDS_ASC + (wm * 64 + lrow) * (KB * 2);
+    const uint32_t sb_off = lhalf ? (uint32_t)LDS_ZERO : LDS_BSC + (wn * 64 + lrow) * (KB * 2);
+    const uint32_t s_buf_stride = lhalf ? 0u : (uint32_t)(BM * KB * 2);
 
     float acc[2][2][16];
 #pragma unroll
@@ -60,113 +152,54 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[a][b][r] = 0.f;
 
-    // staging registers (global -> regs -> LDS)
-    int4 ra[4];
-    int4 rb[Q4 ? 2 : 4];
-    uint16_t rs[KB];
+    if (tid < 128) reinterpret_cast<uint32_t*>(lds + LDS_ZERO)[tid] = 0u;
 
-    auto load_stage = [&](uint32_t k0) {
-        // activations: 128 rows x 128 B; thread t takes 16-byte piece (t + 256 i): row = idx/8, c = idx%8
+    struct Frag {
+        v4i af[2], bf[2];
+        uint32_t sa[2], sb[2];
+    };
+    auto read_frag = [&](Frag& f, uint32_t buf, int kb) {
+        const uint8_t* A = lds + LDS_A + buf * TILE_BYTES;
+        const uint8_t* B = lds + LDS_B + buf * TILE_BYTES;
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t idx = tid + 256 * i, row = idx >> 3, c = idx & 7;
-            const uint32_t m = m0 + row, k = k0 + c * 16;
-            ra[i] = (m < M && k < K) ? *reinterpret_cast<const int4*>(aq + (size_t)m * K + k) : make_int4(0, 0, 0, 0);
-        }
-        if (Q4) {
-            // weights: 128 rows x 4 blocks x 16 packed bytes; piece idx: row = idx/4, blk = idx%4
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const uint32_t idx = tid + 256 * i, row = idx >> 2, bl = idx & 3;
-                const uint32_t n = n0 + row, b = k0 / 32 + bl;
-                rb[i] = (n < N && b < nblk) ? *reinterpret_cast<const int4*>(wq + ((size_t)n * nblk + b) * 16)
-                                            : make_int4(0x88888888, 0x88888888, 0x88888888, 0x88888888);
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t idx = tid + 256 * i, row = idx >> 3, c = idx & 7;
-                const uint32_t n = n0 + row, k = k0 + c * 16;
-                rb[i] = (n < N && k < K) ? *reinterpret_cast<const int4*>(wq + (size_t)n * K + k) : make_int4(0, 0, 0, 0);
-            }
-        }
-        // scales: threads 0..127 take activation row t, threads 128..255 weight row t-128
-        {
-            const bool is_a = tid < 128;
-            const uint32_t row = is_a ? tid : tid - 128;
-            const uint32_t g = (is_a ? m0 : n0) + row;
-            const bool ok = is_a ? (g < M) : (g < N);
-            const uint16_t* src = (is_a ? asc : wsc) + (size_t)g * nblk + k0 / 32;
-#pragma unroll
-            for (int b = 0; b < KB; b++) rs[b] = (ok && k0 / 32 + b < nblk) ? src[b] : (uint16_t)0;
+        for (int t = 0; t < 2; t++) {
+            f.af[t] = *reinterpret_cast<const v4i*>(A + ((fa_off ^ (kb * 32)) + t * 32 * BK));
+            f.bf[t] = *reinterpret_cast<const v4i*>(B + ((fb_off ^ (kb * 32)) + t * 32 * BK));
+            f.sa[t] = *reinterpret_cast<const uint16_t*>(lds + sa_off + buf * s_buf_stride + (lhalf ? 0 : t * 32 * KB * 2) + kb * 2);
+            f.sb[t] = *reinterpret_cast<const uint16_t*>(lds + sb_off + buf * s_buf_stride + (lhalf ? 0 : t * 32 * KB * 2) + kb * 2);
         }
     };
-
-    auto store_stage = [&]() {
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const uint32_t idx = tid + 256 * i, row = idx >> 3, c = idx & 7;
-            *reinterpret_cast<int4*>(As + row * LDS_STRIDE + c * 16) = ra[i];
-        }
-        if (Q4) {
-#pragma unroll
-            for (int i = 0; i < 2; i++) {
-                const uint32_t idx = tid + 256 * i, row = idx >> 2, bl = idx & 3;
-                const int4 p = rb[i];
-                const uint32_t m = 0x0F0F0F0Fu;
-                int4 lo, hi;
-                lo.x = nib_minus8((uint32_t)p.x & m); lo.y = nib_minus8((uint32_t)p.y & m);
-                lo.z = nib_minus8((uint32_t)p.z & m); lo.w = nib_minus8((uint32_t)p.w & m);
-                hi.x = nib_minus8(((uint32_t)p.x >> 4) & m); hi.y = nib_minus8(((uint32_t)p.y >> 4) & m);
-                hi.z = nib_minus8(((uint32_t)p.z >> 4) & m); hi.w = nib_minus8(((uint32_t)p.w >> 4) & m);
-                *reinterpret_cast<int4*>(Bs + row * LDS_STRIDE + bl * 32) = lo;       // elements 0..15
-                *reinterpret_cast<int4*>(Bs + row * LDS_STRIDE + bl * 32 + 16) = hi;  // elements 16..31
-            }
-        } else {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t idx = tid + 256 * i, row = idx >> 3, c = idx & 7;
-                *reinterpret_cast<int4*>(Bs + row * LDS_STRIDE + c * 16) = rb[i];
-            }
-        }
-        {
-            const bool is_a = tid < 128;
-            const uint32_t row = is_a ? tid : tid - 128;
-#pragma unroll
-            for (int b = 0; b < KB; b++) {
-                if (is_a) Asc[b][row] = rs[b];
-                else Bsc[b][row] = rs[b];
-            }
-        }
+    auto scale_operand = [](uint32_t bits) {
+        const _Float16 z = (_Float16)0.0f;
+        return (v8h){__builtin_bit_cast(_Float16, (uint16_t)bits), z, z, z, z, z, z, z};
     };
 
     const v16i zero_i = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     const v16f zero_f = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    load_stage(0);
-    for (uint32_t k0 = 0; k0 < K; k0 += BK) {
-        __syncthreads();   // previous stage fully consumed
-        store_stage();
-        __syncthreads();
-        if (k0 + BK < K) load_stage(k0 + BK);   // prefetch next stage into registers
-#pragma unroll 1
-        for (int kb = 0; kb < KB; kb++) {
-            v4i af[2], bf[2];
-            v8h sa[2], sb[2];
+
+    const uint32_t stages = (K + BK - 1) / BK;
+    issue_stage(0, 0);
+    commit_stage(0);
+    __builtin_amdgcn_s_waitcnt(0);      // vmcnt(0): the tiles of stage 0 are in LDS
+    __syncthreads();
+
+    for (uint32_t s = 0; s < stages; s++) {
+        const uint32_t buf = s & 1;
+        // unconditionally: past the last stage this fetches blocks that do not exist (zeros or the next row's
+        // bytes, never used), which keeps the loop body one straight block of code
+        issue_stage((s + 1) * BK, buf ^ 1);
+
+        Frag fr[2];
+        read_frag(fr[0], buf, 0);
+        v16i isum = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[0].af[0], fr[0].bf[0], zero_i, 0, 0, 0);
+        v16f S = __builtin_amdgcn_mfma_f32_32x32x16_f16(scale_operand(fr[0].sa[0]), scale_operand(fr[0].sb[0]), zero_f, 0, 0, 0);
 #pragma unroll
-            for (int t = 0; t < 2; t++) {
-                af[t] = *reinterpret_cast<const v4i*>(As + (wm * 64 + t * 32 + lrow) * LDS_STRIDE + kb * 32 + lhalf * 16);
-                bf[t] = *reinterpret_cast<const v4i*>(Bs + (wn * 64 + t * 32 + lrow) * LDS_STRIDE + kb * 32 + lhalf * 16);
-                // operands of the rank-1 scale product: the scale in k = 0 (lanes 0..31), zeros elsewhere
-                const uint16_t sab = lhalf ? (uint16_t)0 : Asc[kb][wm * 64 + t * 32 + lrow];
-                const uint16_t sbb = lhalf ? (uint16_t)0 : Bsc[kb][wn * 64 + t * 32 + lrow];
-                const _Float16 z = (_Float16)0.0f;
-                sa[t] = (v8h){__builtin_bit_cast(_Float16, sab), z, z, z, z, z, z, z};
-                sb[t] = (v8h){__builtin_bit_cast(_Float16, sbb), z, z, z, z, z, z, z};
-            }
-            // four tiles, software-pipelined by one: the MFMAs of tile t+1 are issued before tile t is combined,
-            // so the matrix unit works while the VALU scales, and only two tiles of temporaries are live
-            v16i isum = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[0], bf[0], zero_i, 0, 0, 0);
-            v16f S = __builtin_amdgcn_mfma_f32_32x32x16_f16(sa[0], sb[0], zero_f, 0, 0, 0);
+        for (int kb = 0; kb < KB; kb++) {
+            Frag& f = fr[kb & 1];
+            Frag& fnext = fr[(kb + 1) & 1];
+            if (kb + 1 < KB) read_frag(fnext, buf, kb + 1);
+            // four tiles, software-pipelined by one (across blocks too): the MFMAs of the next tile are issued
+            // before this one is combined, so the matrix unit works while the VALU scales
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 const int tm = t >> 1, tn = t & 1;
@@ -174,65 +207,100 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                 v16f S_n = zero_f;
                 if (t < 3) {
                     const int tm2 = (t + 1) >> 1, tn2 = (t + 1) & 1;
-                    isum_n = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tm2], bf[tn2], zero_i, 0, 0, 0);
-                    S_n = __builtin_amdgcn_mfma_f32_32x32x16_f16(sa[tm2], sb[tn2], zero_f, 0, 0, 0);
+                    isum_n = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.af[tm2], f.bf[tn2], zero_i, 0, 0, 0);
+                    S_n = __builtin_amdgcn_mfma_f32_32x32x16_f16(scale_operand(f.sa[tm2]), scale_operand(f.sb[tn2]), zero_f, 0, 0, 0);
+                } else if (kb + 1 < KB) {
+                    isum_n = __builtin_amdgcn_mfma_i32_32x32x32_i8(fnext.af[0], fnext.bf[0], zero_i, 0, 0, 0);
+                    S_n = __builtin_amdgcn_mfma_f32_32x32x16_f16(scale_operand(fnext.sa[0]), scale_operand(fnext.sb[0]), zero_f, 0, 0, 0);
                 }
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    const float f = (float)isum[r];
-                    if (EXACT) acc[tm][tn][r] = acc[tm][tn][r] + S[r] * f;
-                    else acc[tm][tn][r] = fmaf(S[r], f, acc[tm][tn][r]);
+                    const float fl = (float)isum[r];
+                    if (EXACT) acc[tm][tn][r] = acc[tm][tn][r] + S[r] * fl;
+                    else acc[tm][tn][r] = fmaf(S[r], fl, acc[tm][tn][r]);
                 }
                 if (DUMP) {
-                    const uint32_t b = k0 / 32 + kb;
+                    const uint32_t b = s * KB + kb;
                     const uint32_t n = n0 + wn * 64 + tn * 32 + lrow;
+                    const uint32_t mb = m0 + wm * 64 + tm * 32 + 4 * lhalf;
+                    const uint32_t base = (n < N && b < nblk) ? ((mb * N + n) * nblk + b) * 4 : OOB;
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const uint32_t m = m0 + wm * 64 + tm * 32 + 8 * (r >> 2) + 4 * lhalf + (r & 3);
-                        if (m < M && n < N && b < nblk) isums[((size_t)m * N + n) * nblk + b] = isum[r];
-                    }
+                    for (int r = 0; r < 16; r++)
+                        __builtin_amdgcn_raw_buffer_store_b32((uint32_t)isum[r], rdump, base + (8 * (r >> 2) + (r & 3)) * N * nblk * 4, 0, 0);
                 }
                 isum = isum_n;
                 S = S_n;
+                __builtin_amdgcn_sched_barrier(0);   // keep the tiles in this order: one tile of temporaries ahead, no more
             }
         }
+        commit_stage(buf ^ 1);
+        __builtin_amdgcn_s_waitcnt(0);   // this wave's share of stage s+1 has landed
+        __syncthreads();
     }
 
-    // epilogue: lane holds column n = lrow, rows 8g + 4*lhalf + (r&3)
+    // epilogue: lane holds column n = lrow, rows 8g + 4*lhalf + (r&3); the descriptor drops rows >= M
+    const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc((void*)y, 0, M * ldy * 4, RSRC_FLAGS);
 #pragma unroll
     for (int tm = 0; tm < 2; tm++)
 #pragma unroll
         for (int tn = 0; tn < 2; tn++) {
             const uint32_t n = n0 + wn * 64 + tn * 32 + lrow;
+            const uint32_t mb = m0 + wm * 64 + tm * 32 + 4 * lhalf;
+            const uint32_t base = n < N ? (mb * ldy + n) * 4 : OOB;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
-                const uint32_t m = m0 + wm * 64 + tm * 32 + 8 * (r >> 2) + 4 * lhalf + (r & 3);
-                if (m < M && n < N) {
-                    float* p = y + (size_t)m * ldy + n;
-                    if (accumulate) *p = *p + acc[tm][tn][r];
-                    else *p = acc[tm][tn][r];
-                }
+                const uint32_t off = base + (8 * (r >> 2) + (r & 3)) * ldy * 4;
+                float v = acc[tm][tn][r];
+                if (accumulate) v = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ry, off, 0, 0)) + v;
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), ry, off, 0, 0);
             }
         }
 }
 
+// The kernel addresses each matrix with 32-bit byte offsets below 2^31: larger problems are cut into
+// row ranges of the activations and of the weights, one launch each.
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
                  bool accumulate, bool exact, int32_t* isums, hipStream_t s) {
-    if (M == 0) return;
-    dim3 grid((w.N + BN - 1) / BN, (M + BM - 1) / BM);
+    if (M == 0 || w.N == 0) return;
     const int accf = accumulate ? 1 : 0;
     const bool q4 = w.wdtype == FORGE_HIP_Q4_0;
-#define FH_GEMM_LAUNCH(Q4_, DUMP_, EXACT_) \
-    fh::launch(gemm_q_kernel<Q4_, DUMP_, EXACT_>, grid, 256, 0, s, w.qs, w.scales, aq, as, y, isums, M, w.N, w.K, ldy, accf)
-    if (q4) {
-        if (isums) FH_GEMM_LAUNCH(true, true, true);
-        else if (exact) FH_GEMM_LAUNCH(true, false, true);
-        else FH_GEMM_LAUNCH(true, false, false);
-    } else {
-        if (isums) FH_GEMM_LAUNCH(false, true, true);
-        else if (exact) FH_GEMM_LAUNCH(false, false, true);
-        else FH_GEMM_LAUNCH(false, false, false);
-    }
+    const uint64_t LIMIT = 0x7FFFFFFFull - 2 * BK;
+    const uint64_t nblk = w.K / 32;
+    const uint64_t per_m = std::max<uint64_t>(w.K, (uint64_t)ldy * 4);
+    const uint64_t per_n = std::max<uint64_t>(w.qs_row_bytes(), nblk * 2);
+    // a whole dimension in one launch when it fits, else steps of whole tiles
+    const uint64_t m_fit = LIMIT / per_m, n_fit = LIMIT / per_n;
+    const uint32_t m_step = M <= m_fit ? M : (uint32_t)std::max<uint64_t>(BM, m_fit / BM * BM);
+    const uint32_t n_step = w.N <= n_fit ? w.N : (uint32_t)std::max<uint64_t>(BN, n_fit / BN * BN);
+#define FH_GEMM_LAUNCH(Q4_, DUMP_, EXACT_)                                                                              \
+    do {                                                                                                                \
+        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, DUMP_, EXACT_>,           \
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES); \
+        (void)lds_ok;                                                                                                   \
+        fh::launch(gemm_q_kernel<Q4_, DUMP_, EXACT_>, grid, 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c, y_c, is_c, mc, \
+                   nc, w.K, ldy, accf);                                                                                 \
+    } while (0)
+    for (uint32_t mlo = 0; mlo < M; mlo += m_step)
+        for (uint32_t nlo = 0; nlo < w.N; nlo += n_step) {
+            const uint32_t mc = std::min(m_step, M - mlo), nc = std::min(n_step, w.N - nlo);
+            const uint8_t* wq = w.qs + (size_t)nlo * w.qs_row_bytes();
+            const uint16_t* wsc = w.scales + (size_t)nlo * nblk;
+            const int8_t* aq_c = aq + (size_t)mlo * w.K;
+            const uint16_t* as_c = as + (size_t)mlo * nblk;
+            float* y_c = y + (size_t)mlo * ldy + nlo;
+            // block sums of a sub-problem are laid out [mc][nc][nblk]: only whole problems are dumped
+            int32_t* is_c = isums;
+            dim3 grid((nc + BN - 1) / BN, (mc + BM - 1) / BM);
+            if (q4) {
+                if (isums) FH_GEMM_LAUNCH(true, true, true);
+                else if (exact) FH_GEMM_LAUNCH(true, false, true);
+                else FH_GEMM_LAUNCH(true, false, false);
+            } else {
+                if (isums) FH_GEMM_LAUNCH(false, true, true);
+                else if (exact) FH_GEMM_LAUNCH(false, false, true);
+                else FH_GEMM_LAUNCH(false, false, false);
+            }
+        }
 #undef FH_GEMM_LAUNCH
 }
 

@@ -294,8 +294,10 @@ void enqueue_decode_step(forge_hip_model* m) {
     enqueue_head(m, m->x.as<float>(), false, true);
 }
 
-int32_t run_decode_step(forge_hip_model* m) {
-    if (m->pd) return pd_enqueue(m->pd, false, m->stream);
+int32_t run_decode_step(forge_hip_model* m, uint32_t token) {
+    if (m->pd) return pd_enqueue(m->pd, false, token, m->stream);   // the token rides with the launch
+    m->h_stage[0] = token;
+    FH_HIP(hipMemcpyAsync(m->d_token(), &m->h_stage[0], 4, hipMemcpyHostToDevice, m->stream));
     if (m->use_graph && !m->decode_graph) {
         hipGraph_t g = nullptr;
         FH_HIP(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
@@ -323,9 +325,7 @@ int32_t forward_common(forge_hip_model* m, uint32_t token) {
     FH_CHECK(m, "model is null");
     if (m->pos >= (int64_t)m->cfg.max_seq) return fail(FORGE_HIP_ERR_POSITION, "KV cache is full (pos == max_seq)");
     if (token >= m->cfg.vocab) return fail(FORGE_HIP_ERR_POSITION, "token id out of range");
-    m->h_stage[0] = token;
-    FH_HIP(hipMemcpyAsync(m->d_token(), &m->h_stage[0], 4, hipMemcpyHostToDevice, m->stream));
-    int32_t rc = run_decode_step(m);
+    int32_t rc = run_decode_step(m, token);
     if (rc) return rc;
     m->pos += 1;
     return FORGE_HIP_OK;
@@ -475,6 +475,8 @@ int32_t forge_hip_forward_greedy(forge_hip_model* m, uint32_t token, uint32_t* n
     FH_CHECK(next_token_host, "forward_greedy: null out");
     int32_t rc = forward_common(m, token);
     if (rc) return rc;
+    // the resident kernel hands the token over through host memory as soon as it is final
+    if (m->pd && pd_wait_token(m->pd, next_token_host)) return FORGE_HIP_OK;
     rc = finish_decode_step(m);
     if (rc) return rc;
     *next_token_host = m->h_stage[4];
@@ -517,11 +519,9 @@ int32_t forge_hip_forward_profile(forge_hip_model* m, uint32_t token, float* sta
     FH_CHECK(m && stage_ms, "forward_profile: null pointer");
     if (m->pos >= (int64_t)m->cfg.max_seq) return fail(FORGE_HIP_ERR_POSITION, "KV cache is full (pos == max_seq)");
     if (token >= m->cfg.vocab) return fail(FORGE_HIP_ERR_POSITION, "token id out of range");
-    m->h_stage[0] = token;
-    FH_HIP(hipMemcpyAsync(m->d_token(), &m->h_stage[0], 4, hipMemcpyHostToDevice, m->stream));
     if (m->pd) {
         // one kernel: the stages are its phases, timed by the kernel's own clock stamps
-        int32_t rc = pd_enqueue(m->pd, true, m->stream);
+        int32_t rc = pd_enqueue(m->pd, true, token, m->stream);
         if (rc) return rc;
         rc = finish_decode_step(m);
         if (rc) return rc;
@@ -539,6 +539,8 @@ int32_t forge_hip_forward_profile(forge_hip_model* m, uint32_t token, float* sta
         }
         return FORGE_HIP_OK;
     }
+    m->h_stage[0] = token;
+    FH_HIP(hipMemcpyAsync(m->d_token(), &m->h_stage[0], 4, hipMemcpyHostToDevice, m->stream));
     {
         ModelProbe probe(m);
         enqueue_decode_step(m);        // eager launches, each carrying its own pair of events
