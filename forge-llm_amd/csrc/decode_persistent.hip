@@ -1026,7 +1026,7 @@ struct PdState {
     PdArgs args{};
     std::vector<void*> owned;
     uint32_t grid = 0, lds = 0, hd = 0, tags_per_launch = 0, n_stamps = 0;
-    bool q4 = false, lmq4 = false, ordered = false;
+    bool q4 = false, lmq4 = false, ordered = false, cooperative = true;
     size_t tagged_bytes = 0;
     void* tagged_base = nullptr;
     std::vector<unsigned long long> stamps_host;
@@ -1081,6 +1081,7 @@ const void* pd_kernel(const PdState* st) { return st->ordered ? pd_kernel_ord<HD
 template <int HD>
 hipError_t launch_pd_hd(const PdState* st, hipStream_t s) {
     void* kargs[] = {const_cast<PdArgs*>(&st->args)};
+    if (!st->cooperative) return hipLaunchKernel(pd_kernel<HD>(st), dim3(st->grid), dim3(PD_THREADS), kargs, st->lds, s);
     return hipLaunchCooperativeKernel(pd_kernel<HD>(st), dim3(st->grid), dim3(PD_THREADS), kargs, st->lds, s);
 }
 
@@ -1184,6 +1185,10 @@ e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, hd == 64 ? pd_kernel<6
     a.q4 = st->q4; a.lm_q4 = st->lmq4;
     { const char* e = getenv("FORGE_HIP_PD_HINT"); a.use_hint = (e && e[0] == '0') ? 0 : 1; }
     a.token = 0; a.token_from_arg = 0; a.host_out = nullptr; a.host_seq = 0;
+    // All workgroups are co-resident by construction (one per CU, checked above), and every wait in the kernel is
+    // bounded, so an ordinary launch is enough; it costs ~7 us less per step than a cooperative one.
+    // FORGE_HIP_PD_COOP=1 asks for the cooperative launch (which re-checks residency on every launch).
+    { const char* e = getenv("FORGE_HIP_PD_COOP"); st->cooperative = e && e[0] == '1'; }
     if (!(getenv("FORGE_HIP_PD_HOSTWORD") && getenv("FORGE_HIP_PD_HOSTWORD")[0] == '0')) {
         void* hp = nullptr;
         if (hipHostMalloc(&hp, 64, hipHostMallocMapped) == hipSuccess) {

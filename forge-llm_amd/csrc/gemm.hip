@@ -7,10 +7,18 @@
 //   * the scale products a_s[m]*w_s[n] of that tile are a rank-1 outer product of fp16 values, exact in
 //     f32 (11-bit x 11-bit significands): one v_mfma_f32_32x32x16_f16 with the scales in k = 0 and zeros
 //     elsewhere (fp16 subnormal scales included; the unit does not flush them).
-// The scaling itself is elementwise in (m, n, b) and has to be done on the VALU: int->float and one
-// multiply-add per element (in exact mode multiply then add, which is bit for bit the reference's
-// `r += (a_scale*w_scale) * f32(isum)` in block order).  That VALU work, not the matrix unit, bounds the
-// kernel: 32 VALU instructions (128 cycles) per 64 cycles of MFMA.
+// The scaling itself is elementwise in (m, n, b) and has to be done on the VALU.  In exact mode that is
+// int->float, multiply, add per element: bit for bit the reference's `r += (a_scale*w_scale) * f32(isum)` in
+// block order.  That VALU work, not the matrix unit, bounds the kernel (32 VALU instructions = 128 cycles per
+// 64 cycles of MFMA), so the fast mode halves it by never converting: the integer MFMA starts from
+// C = 0x4B400000 in every element, which makes its int32 result, read as f32, the number 12582912 + isum
+// exactly (|isum| <= 516128 < 2^22), and one FMA per element adds S * (12582912 + isum).  To keep the
+// accumulators near their true size the bias alternates in sign: in odd blocks the activation codes are
+// negated before the MFMA and the weight scale carries a minus sign, which adds S * (isum - 12582912).  What
+// is left of the bias after 8 blocks, 12582912 * sum_b (+-)S_b, is itself a product of the scales: one more
+// f16 MFMA (k = the 8 blocks) gives it, and one FMA per element takes it out.  Block sums stay exact; the
+// f32 accumulation carries a rounding error of about 2e-5 of the typical output (measured; 1e-7 in the
+// cvt + FMA form), inside the 1e-3 the fast mode is held to.
 //
 // Tiling: 256 threads = 4 waves (2x2), workgroup tile 128 (m) x 128 (n), wave tile 64x64 = 2x2 MFMA
 // tiles, K step 128 (4 blocks).  Activations are the MFMA A operand (rows), weights the B operand
@@ -39,12 +47,21 @@ constexpr int BM = 128, BN = 128, BK = 128;   // BK in elements (= bytes of int8
 constexpr int KB = BK / 32;                   // quant blocks per stage
 constexpr int TILE_BYTES = BM * BK;           // one operand tile of one stage in LDS
 // LDS map: A tiles [2], B tiles [2], A scales [2][128 rows][4] fp16, B scales likewise, 512 zero bytes
-constexpr int LDS_A = 0, LDS_B = 2 * TILE_BYTES, LDS_ASC = 4 * TILE_BYTES, LDS_BSC = LDS_ASC + 2 * BM * KB * 2,
-              LDS_ZERO = LDS_BSC + 2 * BN * KB * 2, GEMM_LDS_BYTES = LDS_ZERO + 512;
+// scale tables: [4 stage slots][128 rows][4 blocks] fp16, slot = stage & 3 (rows 8 bytes apart: 32 rows, 32 banks)
+constexpr int SC_ROW = KB * 2, SC_SLOT = BM * SC_ROW;
+constexpr int LDS_A = 0, LDS_B = 2 * TILE_BYTES, LDS_ASC = 4 * TILE_BYTES, LDS_BSC = LDS_ASC + 4 * SC_SLOT,
+              LDS_ZERO = LDS_BSC + 4 * SC_SLOT, GEMM_LDS_BYTES = LDS_ZERO + 512;
+constexpr uint32_t MAGIC_BITS = 0x4B400000u;  // 12582912.0f = 1.5 * 2^23: ulp 1, room for +-2^22
 constexpr uint32_t RSRC_FLAGS = 0x00020000;   // raw buffer, 32-bit data format
 constexpr uint32_t OOB = 0x80000000u;         // an offset no descriptor here covers
 
 #define FH_LDS3(p) ((__attribute__((address_space(3))) void*)(p))
+
+// -x for each of four int8 codes (none is -128).
+__device__ __forceinline__ uint32_t neg4(uint32_t x) {
+    const uint32_t y = ~x;
+    return ((y & 0x7F7F7F7Fu) + 0x01010101u) ^ (y & 0x80808080u);
+}
 
 // (c - 8) for each of four nibble codes c held in the low nibbles of the four bytes.
 __device__ __forceinline__ uint32_t nib_minus8(uint32_t x) {
@@ -58,6 +75,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                    const uint16_t* __restrict__ asc, float* __restrict__ y, int32_t* __restrict__ isums, uint32_t M,
                    uint32_t N, uint32_t K, uint32_t ldy, int accumulate) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr bool MAGIC = !EXACT && !DUMP;
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // uniform: the compiler keeps it scalar
@@ -112,7 +130,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     };
 
     // what passes through registers: expanded Q4_0 codes and the scales
-    auto commit_stage = [&](uint32_t buf) {
+    auto commit_stage = [&](uint32_t buf, uint32_t slot) {
         if (Q4) {
 #pragma unroll
             for (int i = 0; i < 2; i++) {
@@ -120,10 +138,20 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                 const v4i p = rb[i];
                 const uint32_t m = 0x0F0F0F0Fu;
                 v4i lo, hi;
+                if (MAGIC) {
+                    // 16 (c - 8) per byte: the biased accumulation resolves sums in units of 1 against a bias of 2^23,
+                    // and 4-bit codes leave 4 bits of headroom (|16 isum| <= 520192); the epilogue divides by 16
+                    const uint32_t h = 0xF0F0F0F0u, b = 0x80808080u;
+                    lo.x = (int)((((uint32_t)p.x & m) << 4) ^ b); lo.y = (int)((((uint32_t)p.y & m) << 4) ^ b);
+                    lo.z = (int)((((uint32_t)p.z & m) << 4) ^ b); lo.w = (int)((((uint32_t)p.w & m) << 4) ^ b);
+                    hi.x = (int)(((uint32_t)p.x & h) ^ b); hi.y = (int)(((uint32_t)p.y & h) ^ b);
+                    hi.z = (int)(((uint32_t)p.z & h) ^ b); hi.w = (int)(((uint32_t)p.w & h) ^ b);
+                } else {
                 lo.x = nib_minus8((uint32_t)p.x & m); lo.y = nib_minus8((uint32_t)p.y & m);
                 lo.z = nib_minus8((uint32_t)p.z & m); lo.w = nib_minus8((uint32_t)p.w & m);
                 hi.x = nib_minus8(((uint32_t)p.x >> 4) & m); hi.y = nib_minus8(((uint32_t)p.y >> 4) & m);
                 hi.z = nib_minus8(((uint32_t)p.z >> 4) & m); hi.w = nib_minus8(((uint32_t)p.w >> 4) & m);
+                }
                 uint8_t* base = lds + LDS_B + buf * TILE_BYTES + row * BK;
                 *reinterpret_cast<v4i*>(base + ((q4_blk * 2) ^ sw) * 16) = lo;       // elements 0..15 of the block
                 *reinterpret_cast<v4i*>(base + ((q4_blk * 2 + 1) ^ sw) * 16) = hi;   // elements 16..31
@@ -132,7 +160,8 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         uint2 pk;
         pk.x = rs[0] | (rs[1] << 16);
         pk.y = rs[2] | (rs[3] << 16);
-        *reinterpret_cast<uint2*>(lds + (sc_is_a ? LDS_ASC : LDS_BSC) + buf * (BM * KB * 2) + sc_row * (KB * 2)) = pk;
+        if (MAGIC && !sc_is_a) { pk.x ^= 0x80000000u; pk.y ^= 0x80000000u; }   // odd blocks: minus sign on the weight scale
+        *reinterpret_cast<uint2*>(lds + (sc_is_a ? LDS_ASC : LDS_BSC) + slot * SC_SLOT + sc_row * SC_ROW) = pk;
     };
 
     // ---- fragment addresses (bytes from the start of a tile / of a scale table)
@@ -140,9 +169,10 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     const uint32_t fa_off = (wm * 64 + lrow) * BK + ((lhalf ^ f_sw) * 16);          // chunk of block kb: ^ (kb * 32)
     const uint32_t fb_off = (wn * 64 + lrow) * BK + ((lhalf ^ f_sw) * 16);
     // scale operand of the rank-1 product: lanes 0..31 hold k = 0 (the scale), lanes 32..63 read zeros
-    const uint32_t sa_off = lhalf ? (uint32_t)LDS_ZERO : LDS_ASC + (wm * 64 + lrow) * (KB * 2);
-    const uint32_t sb_off = lhalf ? (uint32_t)LDS_ZERO : LDS_BSC + (wn * 64 + lrow) * (KB * 2);
-    const uint32_t s_buf_stride = lhalf ? 0u : (uint32_t)(BM * KB * 2);
+    const uint32_t sa_off = lhalf ? (uint32_t)LDS_ZERO : LDS_ASC + (wm * 64 + lrow) * SC_ROW;
+    const uint32_t sb_off = lhalf ? (uint32_t)LDS_ZERO : LDS_BSC + (wn * 64 + lrow) * SC_ROW;
+    const uint32_t s_slot_stride = lhalf ? 0u : (uint32_t)SC_SLOT;
+    const uint32_t s_t_stride = lhalf ? 0u : (uint32_t)(32 * SC_ROW);
 
     float acc[2][2][16];
 #pragma unroll
@@ -158,15 +188,19 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         v4i af[2], bf[2];
         uint32_t sa[2], sb[2];
     };
-    auto read_frag = [&](Frag& f, uint32_t buf, int kb) {
+    auto read_frag = [&](Frag& f, uint32_t buf, uint32_t slot, int kb) {
         const uint8_t* A = lds + LDS_A + buf * TILE_BYTES;
         const uint8_t* B = lds + LDS_B + buf * TILE_BYTES;
 #pragma unroll
         for (int t = 0; t < 2; t++) {
             f.af[t] = *reinterpret_cast<const v4i*>(A + ((fa_off ^ (kb * 32)) + t * 32 * BK));
             f.bf[t] = *reinterpret_cast<const v4i*>(B + ((fb_off ^ (kb * 32)) + t * 32 * BK));
-            f.sa[t] = *reinterpret_cast<const uint16_t*>(lds + sa_off + buf * s_buf_stride + (lhalf ? 0 : t * 32 * KB * 2) + kb * 2);
-            f.sb[t] = *reinterpret_cast<const uint16_t*>(lds + sb_off + buf * s_buf_stride + (lhalf ? 0 : t * 32 * KB * 2) + kb * 2);
+            f.sa[t] = *reinterpret_cast<const uint16_t*>(lds + sa_off + slot * s_slot_stride + t * s_t_stride + kb * 2);
+            f.sb[t] = *reinterpret_cast<const uint16_t*>(lds + sb_off + slot * s_slot_stride + t * s_t_stride + kb * 2);
+            if (MAGIC && (kb & 1)) {
+                f.af[t].x = (int)neg4((uint32_t)f.af[t].x); f.af[t].y = (int)neg4((uint32_t)f.af[t].y);
+                f.af[t].z = (int)neg4((uint32_t)f.af[t].z); f.af[t].w = (int)neg4((uint32_t)f.af[t].w);
+            }
         }
     };
     auto scale_operand = [](uint32_t bits) {
@@ -177,48 +211,64 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     const v16i zero_i = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     const v16f zero_f = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
+    v16i c_in = zero_i;                 // C operand of the integer MFMA: zeros, or the bias that makes the result a float
+    if (MAGIC) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) c_in[r] = (int)MAGIC_BITS;
+    }
+
     const uint32_t stages = (K + BK - 1) / BK;
     issue_stage(0, 0);
-    commit_stage(0);
+    commit_stage(0, 0);
     __builtin_amdgcn_s_waitcnt(0);      // vmcnt(0): the tiles of stage 0 are in LDS
     __syncthreads();
 
-    for (uint32_t s = 0; s < stages; s++) {
-        const uint32_t buf = s & 1;
+    // One stage: 4 blocks out of LDS buffer `buf` while the next stage's tiles fly into the other one.
+    auto run_stage = [&](uint32_t s, uint32_t buf) {
+        const uint32_t slot = s & 3;
         // unconditionally: past the last stage this fetches blocks that do not exist (zeros or the next row's
-        // bytes, never used), which keeps the loop body one straight block of code
+        // bytes, with scale 0), which keeps the loop body one straight block of code
         issue_stage((s + 1) * BK, buf ^ 1);
 
         Frag fr[2];
-        read_frag(fr[0], buf, 0);
-        v16i isum = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[0].af[0], fr[0].bf[0], zero_i, 0, 0, 0);
+        read_frag(fr[0], buf, slot, 0);
+        v16i isum = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[0].af[0], fr[0].bf[0], c_in, 0, 0, 0);
         v16f S = __builtin_amdgcn_mfma_f32_32x32x16_f16(scale_operand(fr[0].sa[0]), scale_operand(fr[0].sb[0]), zero_f, 0, 0, 0);
 #pragma unroll
         for (int kb = 0; kb < KB; kb++) {
             Frag& f = fr[kb & 1];
             Frag& fnext = fr[(kb + 1) & 1];
-            if (kb + 1 < KB) read_frag(fnext, buf, kb + 1);
+            if (kb + 1 < KB) read_frag(fnext, buf, slot, kb + 1);
             // four tiles, software-pipelined by one (across blocks too): the MFMAs of the next tile are issued
             // before this one is combined, so the matrix unit works while the VALU scales
 #pragma unroll
             for (int t = 0; t < 4; t++) {
                 const int tm = t >> 1, tn = t & 1;
+                // next tile's two MFMAs, with this tile's combine split between them: the second MFMA would
+                // otherwise wait (in order, blocking the FMAs behind it) for the first to clear the matrix pipe
+                const bool has_next = t < 3 || kb + 1 < KB;
+                const Frag& fn = t < 3 ? f : fnext;
+                const int tm2 = t < 3 ? (t + 1) >> 1 : 0, tn2 = t < 3 ? (t + 1) & 1 : 0;
                 v16i isum_n = zero_i;
                 v16f S_n = zero_f;
-                if (t < 3) {
-                    const int tm2 = (t + 1) >> 1, tn2 = (t + 1) & 1;
-                    isum_n = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.af[tm2], f.bf[tn2], zero_i, 0, 0, 0);
-                    S_n = __builtin_amdgcn_mfma_f32_32x32x16_f16(scale_operand(f.sa[tm2]), scale_operand(f.sb[tn2]), zero_f, 0, 0, 0);
-                } else if (kb + 1 < KB) {
-                    isum_n = __builtin_amdgcn_mfma_i32_32x32x32_i8(fnext.af[0], fnext.bf[0], zero_i, 0, 0, 0);
-                    S_n = __builtin_amdgcn_mfma_f32_32x32x16_f16(scale_operand(fnext.sa[0]), scale_operand(fnext.sb[0]), zero_f, 0, 0, 0);
-                }
+                if (has_next) isum_n = __builtin_amdgcn_mfma_i32_32x32x32_i8(fn.af[tm2], fn.bf[tn2], c_in, 0, 0, 0);
+                const v16f biased = __builtin_bit_cast(v16f, isum);   // fast mode: 12582912 +- isum, exactly
+                auto combine = [&](int r) {
+                    if (MAGIC) {
+                        acc[tm][tn][r] = fmaf(S[r], biased[r], acc[tm][tn][r]);
+                    } else {
+                        const float fl = (float)isum[r];
+                        if (EXACT) acc[tm][tn][r] = acc[tm][tn][r] + S[r] * fl;
+                        else acc[tm][tn][r] = fmaf(S[r], fl, acc[tm][tn][r]);
+                    }
+                };
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const float fl = (float)isum[r];
-                    if (EXACT) acc[tm][tn][r] = acc[tm][tn][r] + S[r] * fl;
-                    else acc[tm][tn][r] = fmaf(S[r], fl, acc[tm][tn][r]);
-                }
+                for (int r = 0; r < 8; r++) combine(r);
+                __builtin_amdgcn_sched_barrier(0);
+                if (has_next)
+                    S_n = __builtin_amdgcn_mfma_f32_32x32x16_f16(scale_operand(fn.sa[tm2]), scale_operand(fn.sb[tn2]), zero_f, 0, 0, 0);
+#pragma unroll
+                for (int r = 8; r < 16; r++) combine(r);
                 if (DUMP) {
                     const uint32_t b = s * KB + kb;
                     const uint32_t n = n0 + wn * 64 + tn * 32 + lrow;
@@ -233,9 +283,40 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                 __builtin_amdgcn_sched_barrier(0);   // keep the tiles in this order: one tile of temporaries ahead, no more
             }
         }
-        commit_stage(buf ^ 1);
+        commit_stage(buf ^ 1, (s + 1) & 3);
         __builtin_amdgcn_s_waitcnt(0);   // this wave's share of stage s+1 has landed
         __syncthreads();
+    };
+
+    // Stages go in pairs (an odd count runs one stage of zero scales).  After a pair the fast mode removes what
+    // the 8 blocks left of the bias: 12582912 * sum_b a_s[m][b] * (+-w_s[n][b]), the sum being one f16 MFMA.
+    const uint32_t ta_off = lhalf ? (uint32_t)LDS_ZERO : LDS_ASC + (wm * 64 + lrow) * SC_ROW;
+    const uint32_t tb_off = lhalf ? (uint32_t)LDS_ZERO : LDS_BSC + (wn * 64 + lrow) * SC_ROW;
+    for (uint32_t s = 0; s < stages; s += 2) {
+        run_stage(s, 0);
+        run_stage(s + 1, 1);
+        if (MAGIC) {
+            const uint32_t pair = lhalf ? 0u : (s & 2u) * (uint32_t)SC_SLOT;      // slots {0,1} or {2,3}
+            typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+            v8h ta[2], tb[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const v4h a0 = *reinterpret_cast<const v4h*>(lds + ta_off + pair + t * s_t_stride);
+                const v4h a1 = *reinterpret_cast<const v4h*>(lds + ta_off + pair + s_slot_stride + t * s_t_stride);
+                const v4h b0 = *reinterpret_cast<const v4h*>(lds + tb_off + pair + t * s_t_stride);
+                const v4h b1 = *reinterpret_cast<const v4h*>(lds + tb_off + pair + s_slot_stride + t * s_t_stride);
+                ta[t] = (v8h){a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                tb[t] = (v8h){b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+            }
+#pragma unroll
+            for (int t = 0; t < 4; t++) {
+                const int tm = t >> 1, tn = t & 1;
+                const v16f T = __builtin_amdgcn_mfma_f32_32x32x16_f16(ta[tm], tb[tn], zero_f, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    acc[tm][tn][r] = fmaf(-__builtin_bit_cast(float, MAGIC_BITS), T[r], acc[tm][tn][r]);
+            }
+        }
     }
 
     // epilogue: lane holds column n = lrow, rows 8g + 4*lhalf + (r&3); the descriptor drops rows >= M
@@ -251,6 +332,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
             for (int r = 0; r < 16; r++) {
                 const uint32_t off = base + (8 * (r >> 2) + (r & 3)) * ldy * 4;
                 float v = acc[tm][tn][r];
+                if (MAGIC && Q4) v *= 0.0625f;
                 if (accumulate) v = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ry, off, 0, 0)) + v;
                 __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), ry, off, 0, 0);
             }
