@@ -1,0 +1,162 @@
+"""GPU parity at the sizes the benchmark configurations name (Llama-3.2-1B projection shapes, 2.5k-token
+batches, 3k-token attention, 8k-token caches, the Llama-3.2-3B layer shape), through the C ABI.
+
+The oracle would need minutes for whole outputs at these sizes, so each test runs the GPU on the full
+problem and compares the parts the oracle can do in seconds, using what the operations guarantee:
+  * a GEMM row depends only on its own activation row, an attention row only on its own query and the keys
+    up to its position: sampled rows are checked against the oracle run on exactly those rows;
+  * the same rows computed alone on the GPU must equal the rows of the full launch bit for bit
+    (tiling, batching and chunking may not change a result)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+Q8, Q4 = 8, 2
+A, KV_F16 = 0, 1
+EXACT = 1
+RTOL, ATOL = 1e-3, 1e-3
+
+
+def close(got, want, rtol=RTOL, atol=ATOL):
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    bad = np.abs(got - want) > atol + rtol * np.abs(want)
+    assert not bad.any(), f"{bad.sum()} of {bad.size} outside tolerance; max abs err {np.max(np.abs(got - want)):.3e}"
+
+
+def same_bits(got, want):
+    got, want = np.ascontiguousarray(got, np.float32), np.ascontiguousarray(want, np.float32)
+    diff = got.view(np.uint32) != want.view(np.uint32)
+    assert not diff.any(), f"{diff.sum()} of {diff.size} differ in bits; max abs err {np.max(np.abs(got - want)):.3e}"
+
+
+_weights = {}
+
+
+def weight(fh, wd, K, N):
+    """Seeded N(0, 0.02) weights quantised with the reference's quantiser; cached per shape."""
+    key = (wd, K, N)
+    if key not in _weights:
+        w = fh.synth.normal(1000 + K + 3 * N, N * K, 0.02).reshape(N, K)
+        raw = fh.ops.quantize_weights(wd, w)
+        _weights[key] = (raw, fh.ops.QWeight(wd, raw, K, N))
+    return _weights[key]
+
+
+def sample_rows(M, seed):
+    """First and last rows, the rows either side of every 128-row tile edge that exists, and a few random ones."""
+    rows = {0, M - 1}
+    for edge in (127, 128, 255, 256, 1023, 1024, 2047, 2048):
+        if edge < M:
+            rows.add(edge)
+    rng = np.random.default_rng(seed)
+    rows.update(int(r) for r in rng.integers(0, M, 6))
+    return sorted(rows)
+
+
+# ---------------- isolated GEMV, M = 1 ----------------
+@pytest.mark.parametrize("wd", [Q8, Q4])
+@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 512), (2048, 8192), (8192, 2048), (2048, 128256)])
+def test_gemv_llama_1b_shapes_bit_exact(fh, oracle, torch_gpu, wd, K, N):
+    """matmul_vec at every projection shape of Llama-3.2-1B, the LM head included: identical bits."""
+    torch = torch_gpu
+    raw, w = weight(fh, wd, K, N)
+    x = fh.synth.normal(21 + K + N, K, 1.0)
+    y = fh.ops.matmul_vec_q(w, torch.from_numpy(x).cuda()).cpu().numpy()
+    same_bits(y, oracle.matmul_vec(wd, 0, x, raw, K, N))
+
+
+# ---------------- batched-prefill GEMM ----------------
+@pytest.mark.parametrize("wd", [Q8, Q4])
+@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 512), (2048, 8192), (8192, 2048)])
+@pytest.mark.parametrize("M", [352, 902, 1603, 2502])
+def test_gemm_llama_1b_shapes(fh, oracle, torch_gpu, wd, K, N, M):
+    torch = torch_gpu
+    raw, w = weight(fh, wd, K, N)
+    x = fh.synth.normal(31 + M + K, M * K, 1.0).reshape(M, K)
+    rows = sample_rows(M, M + K + N)
+    xd = torch.from_numpy(x).cuda()
+    want = oracle.matmul_mat(wd, 0, x[rows], raw, len(rows), K, N)
+    exact = fh.ops.matmul_mat_q(w, xd, EXACT).cpu().numpy()
+    fast = fh.ops.matmul_mat_q(w, xd, 0).cpu().numpy()
+    same_bits(exact[rows], want)
+    close(fast[rows], want)
+    # every row of the fast result against the exact one (same block sums, different f32 evaluation)
+    close(fast, exact)
+    # the sampled rows as a batch of their own: same bits as inside the full batch
+    xs = torch.from_numpy(np.ascontiguousarray(x[rows])).cuda()
+    same_bits(fh.ops.matmul_mat_q(w, xs, EXACT).cpu().numpy(), exact[rows])
+    same_bits(fh.ops.matmul_mat_q(w, xs, 0).cpu().numpy(), fast[rows])
+
+
+# ---------------- attention over an fp16 cache ----------------
+def kv_cache(fh, oracle, seq, kv_heads, hd, seed):
+    k = fh.synth.normal(seed, seq * kv_heads * hd, 1.0)
+    v = fh.synth.normal(seed + 1, seq * kv_heads * hd, 1.0)
+    return (oracle.f32_to_f16(k).reshape(seq, kv_heads * hd), oracle.f32_to_f16(v).reshape(seq, kv_heads * hd))
+
+
+def dev16(torch, a):
+    return torch.from_numpy(a.view(np.int16)).cuda()
+
+
+@pytest.mark.parametrize("heads,kv_heads,hd", [(32, 8, 64), (32, 32, 96)])
+@pytest.mark.parametrize("seq", [801, 1501, 3001])
+def test_attention_prefill_long_sequences(fh, oracle, torch_gpu, heads, kv_heads, hd, seq):
+    """attention_flash_batch over the whole sequence; sampled rows against the oracle's batch kernel run for
+    that single row at its position (row r of a batch sees keys 0..r)."""
+    torch = torch_gpu
+    k16, v16 = kv_cache(fh, oracle, seq, kv_heads, hd, seed=seq + hd)
+    q = fh.synth.normal(40 + seq, seq * heads * hd, 1.0).reshape(seq, heads * hd)
+    q16 = oracle.f16_to_f32(oracle.f32_to_f16(q))            # the MFMA kernel rounds q to fp16: give it such queries
+    kd, vd = dev16(torch, k16), dev16(torch, v16)
+    exact = fh.ops.attention_flash_batch(torch.from_numpy(q).cuda(), kd, vd, 0, heads, kv_heads, hd, EXACT).cpu().numpy()
+    fast = fh.ops.attention_flash_batch(torch.from_numpy(q16).cuda(), kd, vd, 0, heads, kv_heads, hd, 0).cpu().numpy()
+    for r in sample_rows(seq, seq + hd):
+        same_bits(exact[r], oracle.attention("flash_batch", q[r], k16, v16, 1, heads, kv_heads, hd, base_pos=r))
+        close(fast[r], oracle.attention("flash_batch", q16[r], k16, v16, 1, heads, kv_heads, hd, base_pos=r))
+    # a second chunk appended to an existing cache (base_pos > 0) reproduces the rows of the one-shot call
+    cut = seq // 2 + 3
+    tail_e = fh.ops.attention_flash_batch(torch.from_numpy(np.ascontiguousarray(q[cut:])).cuda(), kd, vd, cut, heads, kv_heads,
+                                          hd, EXACT).cpu().numpy()
+    same_bits(tail_e, exact[cut:])
+    tail_f = fh.ops.attention_flash_batch(torch.from_numpy(np.ascontiguousarray(q16[cut:])).cuda(), kd, vd, cut, heads,
+                                          kv_heads, hd, 0).cpu().numpy()
+    close(tail_f, fast[cut:])
+
+
+@pytest.mark.parametrize("heads,kv_heads,hd", [(32, 8, 64), (32, 32, 96)])
+@pytest.mark.parametrize("seq", [900, 2250, 8192])
+def test_attention_decode_long_caches(fh, oracle, torch_gpu, heads, kv_heads, hd, seq):
+    torch = torch_gpu
+    k16, v16 = kv_cache(fh, oracle, seq, kv_heads, hd, seed=seq + 7 * hd)
+    q = fh.synth.normal(50 + seq, heads * hd, 1.0)
+    want = oracle.attention("flash", q, k16, v16, seq, heads, kv_heads, hd)
+    qd, kd, vd = torch.from_numpy(q).cuda(), dev16(torch, k16), dev16(torch, v16)
+    same_bits(fh.ops.attention_flash(qd, kd, vd, seq, heads, kv_heads, hd, EXACT).cpu().numpy(), want)
+    close(fh.ops.attention_flash(qd, kd, vd, seq, heads, kv_heads, hd, 0).cpu().numpy(), want)
+
+
+# ---------------- Llama-3.2-3B layer shape end to end ----------------
+def test_llama_3b_shape_two_layers_identical_tokens(fh, oracle, torch_gpu):
+    """Llama-3.2-3B shape (hidden 3072, 24 heads over 8 KV heads, head_dim 128, intermediate 8192, vocabulary
+    128256), Q8_0, cut to 2 of its 28 layers and a 300-token prompt so that the CPU oracle finishes in seconds:
+    batched prefill, then greedy decode -- identical token ids and bit-identical logits in exact mode."""
+    cfg = fh.synth.llama32_3b(Q8, max_seq=1024)
+    cfg["layers"] = 2
+    cfg["flags"] = EXACT
+    blob = fh.synth.make_weights_blob(cfg, seed=3, threads=16)
+    prompt = fh.synth.uniform_ids(4, 300, cfg["vocab"])
+    gm = fh.HipModel(cfg, blob)
+    om = oracle.Model(cfg, blob, A, KV_F16)
+    glog = gm.forward_prefill(prompt)
+    olog = om.prefill_batched(prompt)
+    same_bits(glog, olog)
+    tok = oracle.argmax(olog)
+    for _ in range(8):
+        gl, ol = gm.forward(tok), om.forward(tok)
+        same_bits(gl, ol)
+        tok = oracle.argmax(ol)
+    for which in (0, 1):
+        same_bits(oracle.f16_to_f32(gm.read_kv(1, which)), om.read_kv(1, which))
+    gm.close(); om.close()

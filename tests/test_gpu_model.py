@@ -233,13 +233,18 @@ def test_persistent_decode_kernel_default_summation(fh, oracle, torch_gpu, monke
     seq.close(); one.close()
 
 
-@pytest.mark.parametrize("shape", ["smollm2_135m", "llama_1b_2layers"])
+@pytest.mark.parametrize("shape", ["smollm2_135m", "llama_1b_2layers", "llama_3b_2layers"])
 def test_persistent_decode_kernel_real_shapes(fh, torch_gpu, monkeypatch, shape):
     """Same check on the shapes that matter: SmolLM2-135M (hidden 576, 9 heads over 3 KV heads: partial weight
-    units, three heads per group) and the Llama-3.2-1B layer shape at a context that spans every split."""
+    units, three heads per group), the Llama-3.2-1B layer shape at a context that spans every split, and the
+    Llama-3.2-3B layer shape (hidden 3072: three weight units per row, head_dim 128, three heads per group)."""
     if shape == "smollm2_135m":
         cfg = fh.synth.smollm2_135m(Q8, max_seq=1024)
         n_prompt = 300
+    elif shape == "llama_3b_2layers":
+        cfg = fh.synth.llama32_3b(Q8, max_seq=1024)
+        cfg["layers"], cfg["vocab"] = 2, 32000
+        n_prompt = 700
     else:
         cfg = fh.synth.llama32_1b(Q8, max_seq=2048)
         cfg["layers"], cfg["vocab"] = 2, 32000
