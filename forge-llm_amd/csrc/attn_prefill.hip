@@ -3,8 +3,12 @@
 // softmax in f32.
 //
 // Workgroup = 4 waves = 128 consecutive queries of one head; each wave owns 32 queries.
-// K/V are streamed in tiles of 64 keys through LDS (K row-major, V transposed so that the
-// contraction index of P.V is contiguous per lane).
+// K/V are streamed in tiles of 64 keys through two LDS buffers (K row-major, V transposed so that
+// the contraction index of P.V is contiguous per lane; a thread fetches 4 head dims of two
+// consecutive keys and writes the pairs as dwords).  Scores stay in the base-2 domain
+// (s * scale * log2 e) so that the exponential is one v_exp_f32 after one FMA; keys are masked only in
+// tiles that reach past the wave's first query, and the accumulators are rescaled only when some
+// query of the wave saw a new maximum.
 //
 // Both products are computed transposed, S^T = K Q^T and O^T = V^T P^T.  In the 32x32 MFMA
 // result layout a lane then owns ONE query (column = lane%32) and 16 keys (or 16 head dims),
@@ -25,17 +29,20 @@ constexpr int QB = 128;       // queries per workgroup
 constexpr int KT = 64;        // keys per tile
 
 template <int HD>
-__global__ __launch_bounds__(256) void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc,
                                                            const uint16_t* __restrict__ vc, float* __restrict__ out,
                                                            uint32_t q_stride, uint32_t out_stride, uint32_t M,
                                                            uint32_t base_pos, uint32_t heads, uint32_t kv_heads) {
     constexpr int KS = HD + 8;    // K tile row stride (halfs): 16-byte pad
     constexpr int VS = KT + 4;    // V^T tile row stride (halfs): 8-byte pad
-    constexpr int PIECES = KT * HD / 8 / 256;   // 16-byte pieces per thread per tile
+    constexpr int KPIECES = KT * HD / 8 / 256;   // 16-byte pieces of K per thread per tile
+    constexpr int VITEMS = KT * HD / 8 / 256;    // (key pair, 4 dims) items of V per thread per tile
+    constexpr int DG = HD / 4;    // groups of 4 head dims
     constexpr int NS = HD / 16;   // MFMA k-steps over head_dim
     constexpr int ND = HD / 32;   // 32-wide head_dim tiles of the output
-    __shared__ __attribute__((aligned(16))) _Float16 Ks[KT * KS];
-    __shared__ __attribute__((aligned(16))) _Float16 Vt[HD * VS];
+    // two tiles each: the loads of tile t+1 are written while tile t is read, one barrier per tile
+    __shared__ __attribute__((aligned(16))) _Float16 Ks[2][KT * KS];
+    __shared__ __attribute__((aligned(16))) _Float16 Vt[2][HD * VS];
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t lq = lane & 31, lh = lane >> 5;
@@ -45,7 +52,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const float* __restri
     const uint32_t q0 = qtile * QB;
     const uint32_t kv_stride = kv_heads * HD;
     const uint32_t seq_total = base_pos + M;
-    const float scale = 1.0f / sqrtf((float)HD);
+    // scores are kept in the base-2 domain: s * (scale * log2 e), so that exp is the bare v_exp_f32
+    const float c2 = (1.0f / sqrtf((float)HD)) * 1.4426950408889634f;
 
     // ---- Q fragment (B operand of S^T = K Q^T): lane (lq, lh) holds q[row][16 s + 8 lh + 0..7]
     const uint32_t qrow = q0 + wave * QW + lq;
@@ -73,106 +81,126 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(const float* __restri
     const uint32_t wg_max_pos = base_pos + min(q0 + QB, M) - 1;
     const uint32_t ntiles = wg_max_pos / KT + 1;
     const uint32_t wave_max_pos = base_pos + min(q0 + wave * QW + QW, M) - 1;   // may underflow if wave is empty
+    const uint32_t wave_min_pos = base_pos + q0 + wave * QW;                    // position of the wave's first query
     const bool wave_active = q0 + wave * QW < M;
 
-    int4 kreg[PIECES], vreg[PIECES];
+    int4 kreg[KPIECES];
+    uint2 va[VITEMS], vb[VITEMS];
     auto load_tile = [&](uint32_t kt) {
 #pragma unroll
-        for (int i = 0; i < PIECES; i++) {
+        for (int i = 0; i < KPIECES; i++) {
             const uint32_t idx = tid + 256 * i, key = idx / (HD / 8), dc = idx % (HD / 8);
             const uint32_t t = kt * KT + key;
-            if (t < seq_total) {
-                const size_t off = (size_t)t * kv_stride + kvh * HD + dc * 8;
-                kreg[i] = *reinterpret_cast<const int4*>(kc + off);
-                vreg[i] = *reinterpret_cast<const int4*>(vc + off);
-            } else {
-                kreg[i] = make_int4(0, 0, 0, 0);
-                vreg[i] = make_int4(0, 0, 0, 0);
-            }
+            kreg[i] = t < seq_total ? *reinterpret_cast<const int4*>(kc + (size_t)t * kv_stride + kvh * HD + dc * 8)
+                                    : make_int4(0, 0, 0, 0);
+        }
+        // V: an item is 4 head dims of two consecutive keys (seq rows t, t+1)
+#pragma unroll
+        for (int i = 0; i < VITEMS; i++) {
+            const uint32_t idx = tid + 256 * i, kp = idx / DG, dg = idx % DG;
+            const uint32_t t = kt * KT + 2 * kp;
+            const uint16_t* src = vc + (size_t)t * kv_stride + kvh * HD + dg * 4;
+            va[i] = t < seq_total ? *reinterpret_cast<const uint2*>(src) : make_uint2(0, 0);
+            vb[i] = t + 1 < seq_total ? *reinterpret_cast<const uint2*>(src + kv_stride) : make_uint2(0, 0);
         }
     };
-    auto store_tile = [&]() {
+    auto store_tile = [&](uint32_t buf) {
 #pragma unroll
-        for (int i = 0; i < PIECES; i++) {
+        for (int i = 0; i < KPIECES; i++) {
             const uint32_t idx = tid + 256 * i, key = idx / (HD / 8), dc = idx % (HD / 8);
-            *reinterpret_cast<int4*>(Ks + key * KS + dc * 8) = kreg[i];
-            const uint32_t w[4] = {(uint32_t)vreg[i].x, (uint32_t)vreg[i].y, (uint32_t)vreg[i].z, (uint32_t)vreg[i].w};
-            uint16_t* vt = reinterpret_cast<uint16_t*>(Vt);
+            *reinterpret_cast<int4*>(&Ks[buf][key * KS + dc * 8]) = kreg[i];
+        }
+        // V^T[d][key]: the two keys' values of one head dim side by side in a dword
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                vt[(dc * 8 + 2 * e) * VS + key] = (uint16_t)(w[e] & 0xFFFFu);
-                vt[(dc * 8 + 2 * e + 1) * VS + key] = (uint16_t)(w[e] >> 16);
-            }
+        for (int i = 0; i < VITEMS; i++) {
+            const uint32_t idx = tid + 256 * i, kp = idx / DG, dg = idx % DG;
+            uint32_t* vt = reinterpret_cast<uint32_t*>(&Vt[buf][(dg * 4) * VS + 2 * kp]);
+            vt[0 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].x, va[i].x, 0x05040100u);
+            vt[1 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].x, va[i].x, 0x07060302u);
+            vt[2 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].y, va[i].y, 0x05040100u);
+            vt[3 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].y, va[i].y, 0x07060302u);
         }
     };
 
     load_tile(0);
+    store_tile(0);
+    __syncthreads();
     for (uint32_t kt = 0; kt < ntiles; kt++) {
-        __syncthreads();   // everyone is done reading the previous tile
-        store_tile();
-        __syncthreads();
-        if (kt + 1 < ntiles) load_tile(kt + 1);
-        if (!wave_active || kt * KT > wave_max_pos) continue;   // tile entirely in this wave's future
-
-        // ---- S^T tiles: sacc[kk][r] = score(key kt*64 + kk*32 + 8(r/4) + 4 lh + r%4, query lq)
-        v16f sacc[2];
+        const uint32_t buf = kt & 1;
+        if (kt + 1 < ntiles) load_tile(kt + 1);          // in flight while this tile is computed
+        if (wave_active && kt * KT <= wave_max_pos) {    // else the tile lies entirely in this wave's future
+            const _Float16* Kb = Ks[buf];
+            const _Float16* Vb = Vt[buf];
+            // ---- S^T tiles: sacc[kk][r] = q . k for key kt*64 + kk*32 + 8(r/4) + 4 lh + r%4, query lq
+            v16f sacc[2];
 #pragma unroll
-        for (int kk = 0; kk < 2; kk++) {
+            for (int kk = 0; kk < 2; kk++) {
 #pragma unroll
-            for (int r = 0; r < 16; r++) sacc[kk][r] = 0.f;
+                for (int r = 0; r < 16; r++) sacc[kk][r] = 0.f;
 #pragma unroll
-            for (int s = 0; s < NS; s++) {
-                v8h kf = *reinterpret_cast<const v8h*>(Ks + (kk * 32 + lq) * KS + 16 * s + 8 * lh);
-                sacc[kk] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], sacc[kk], 0, 0, 0);
-            }
-        }
-        // ---- causal mask + online softmax (per-lane scalars)
-        float m_tile = -INFINITY;
-#pragma unroll
-        for (int kk = 0; kk < 2; kk++)
-#pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const uint32_t t = kt * KT + kk * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                float s = sacc[kk][r] * scale;
-                s = (t <= qpos) ? s : -INFINITY;
-                sacc[kk][r] = s;
-                m_tile = fmaxf(m_tile, s);
-            }
-        m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, WAVE));
-        const float m_new = fmaxf(m_run, m_tile);
-        // m_new is finite from the first tile on (key 0 is visible to every query)
-        const float alpha = __expf(m_run - m_new);
-        float l_tile = 0.f;
-        v8h pb[2][2];
-#pragma unroll
-        for (int kk = 0; kk < 2; kk++)
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const float p = __expf(sacc[kk][8 * j + e] - m_new);   // exp(-inf) = 0 for masked keys
-                    l_tile += p;
-                    pb[kk][j][e] = (_Float16)p;
+                for (int s = 0; s < NS; s++) {
+                    v8h kf = *reinterpret_cast<const v8h*>(Kb + (kk * 32 + lq) * KS + 16 * s + 8 * lh);
+                    sacc[kk] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], sacc[kk], 0, 0, 0);
                 }
-        l_run = l_run * alpha + l_tile;
-        m_run = m_new;
+            }
+            // ---- causal mask: only tiles that reach past the wave's first query have masked keys
+            if (kt * KT + KT - 1 > wave_min_pos) {
 #pragma unroll
-        for (int d = 0; d < ND; d++)
+                for (int kk = 0; kk < 2; kk++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) oacc[d][r] *= alpha;
-        // ---- O^T += V^T P^T
-#pragma unroll
-        for (int d = 0; d < ND; d++)
+                    for (int r = 0; r < 16; r++) {
+                        const uint32_t t = kt * KT + kk * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                        sacc[kk][r] = (t <= qpos) ? sacc[kk][r] : -INFINITY;
+                    }
+            }
+            // ---- online softmax in base 2 (per-lane scalars: a lane owns one query)
+            float m_tile = -INFINITY;
 #pragma unroll
             for (int kk = 0; kk < 2; kk++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const _Float16* vrow = Vt + (d * 32 + lq) * VS + kk * 32 + 16 * j + 4 * lh;
-                    v4h v0 = *reinterpret_cast<const v4h*>(vrow);
-                    v4h v1 = *reinterpret_cast<const v4h*>(vrow + 8);
-                    v8h vf = (v8h){v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-                    oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pb[kk][j], oacc[d], 0, 0, 0);
-                }
+                for (int r = 0; r < 16; r++) m_tile = fmaxf(m_tile, sacc[kk][r]);
+            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, WAVE)) * c2;      // c2 > 0: max commutes with the scaling
+            const float m_new = fmaxf(m_run, m_tile);
+            // m_new is finite from the first tile on (key 0 is visible to every query)
+            float l_tile = 0.f;
+            v8h pb[2][2];
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const float p = __builtin_amdgcn_exp2f(fmaf(sacc[kk][8 * j + e], c2, -m_new));   // 2^-inf = 0 for masked keys
+                        l_tile += p;
+                        pb[kk][j][e] = (_Float16)p;
+                    }
+            // rescale what has been accumulated, unless no query of the wave saw a new maximum
+            if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
+                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                l_run *= alpha;
+#pragma unroll
+                for (int d = 0; d < ND; d++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) oacc[d][r] *= alpha;
+            }
+            l_run += l_tile;
+            m_run = m_new;
+            // ---- O^T += V^T P^T
+#pragma unroll
+            for (int d = 0; d < ND; d++)
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++) {
+                        const _Float16* vrow = Vb + (d * 32 + lq) * VS + kk * 32 + 16 * j + 4 * lh;
+                        v4h v0 = *reinterpret_cast<const v4h*>(vrow);
+                        v4h v1 = *reinterpret_cast<const v4h*>(vrow + 8);
+                        v8h vf = (v8h){v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                        oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pb[kk][j], oacc[d], 0, 0, 0);
+                    }
+        }
+        if (kt + 1 < ntiles) store_tile(buf ^ 1);   // nobody reads that buffer: its tile was finished before the last barrier
+        __syncthreads();
     }
 
     // ---- normalise and store: lane (lq, lh) holds out[qrow][32 d + 8 g + 4 lh + 0..3]
