@@ -2,7 +2,9 @@
 // cache, with both matrix products on fp16 MFMA (v_mfma_f32_32x32x16_f16) and the online
 // softmax in f32.
 //
-// Workgroup = 4 waves = 128 consecutive queries of one head; each wave owns 32 queries.
+// Workgroup = 8 waves = 128 consecutive queries of one head: four groups of 32 queries, each shared by two
+// waves that take one half (32 keys) of every key tile and merge their (max, sum, output) once at the end, so
+// that the longest chain of dependent tile steps (the last query tile's) is worked on by twice the waves.
 // K/V are streamed in tiles of 64 keys through two LDS buffers (K row-major, V transposed so that
 // the contraction index of P.V is contiguous per lane; a thread fetches 4 head dims of two
 // consecutive keys and writes the pairs as dwords).  Scores stay in the base-2 domain
@@ -24,31 +26,40 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int QW = 32;        // queries per wave
+constexpr int QW = 32;        // queries per wave pair
 constexpr int QB = 128;       // queries per workgroup
 constexpr int KT = 64;        // keys per tile
+constexpr int AP_THREADS = 512;
 
 template <int HD>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc,
-                                                           const uint16_t* __restrict__ vc, float* __restrict__ out,
-                                                           uint32_t q_stride, uint32_t out_stride, uint32_t M,
-                                                           uint32_t base_pos, uint32_t heads, uint32_t kv_heads) {
+__global__ __launch_bounds__(AP_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
+void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+                         float* __restrict__ out, uint32_t q_stride, uint32_t out_stride, uint32_t M, uint32_t base_pos,
+                         uint32_t heads, uint32_t kv_heads) {
     constexpr int KS = HD + 8;    // K tile row stride (halfs): 16-byte pad
     constexpr int VS = KT + 4;    // V^T tile row stride (halfs): 8-byte pad
-    constexpr int KPIECES = KT * HD / 8 / 256;   // 16-byte pieces of K per thread per tile
-    constexpr int VITEMS = KT * HD / 8 / 256;    // (key pair, 4 dims) items of V per thread per tile
+    constexpr int KTOTAL = KT * HD / 8;          // 16-byte pieces of K per tile
+    constexpr int VTOTAL = KT * HD / 8;          // (key pair, 4 dims) items of V per tile
+    constexpr int KPIECES = (KTOTAL + AP_THREADS - 1) / AP_THREADS, VITEMS = (VTOTAL + AP_THREADS - 1) / AP_THREADS;
     constexpr int DG = HD / 4;    // groups of 4 head dims
     constexpr int NS = HD / 16;   // MFMA k-steps over head_dim
     constexpr int ND = HD / 32;   // 32-wide head_dim tiles of the output
+    constexpr int KBYTES = KT * KS * 2, VBYTES = HD * VS * 2;
+    constexpr int MERGE_FLOATS = 2 + ND * 16;    // per lane: m, l and the output accumulators
+    static_assert(2 * (KBYTES + VBYTES) >= 4 * 64 * MERGE_FLOATS * 4, "the merge reuses the tile buffers");
     // two tiles each: the loads of tile t+1 are written while tile t is read, one barrier per tile
-    __shared__ __attribute__((aligned(16))) _Float16 Ks[2][KT * KS];
-    __shared__ __attribute__((aligned(16))) _Float16 Vt[2][HD * VS];
+    __shared__ __attribute__((aligned(16))) uint8_t smem[2 * (KBYTES + VBYTES)];
+    auto Ks = [&](uint32_t buf) { return reinterpret_cast<_Float16*>(smem + buf * KBYTES); };
+    auto Vt = [&](uint32_t buf) { return reinterpret_cast<_Float16*>(smem + 2 * KBYTES + buf * VBYTES); };
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t qg = wave >> 1, kh = wave & 1;      // query group of 32, half of every key tile
     const uint32_t lq = lane & 31, lh = lane >> 5;
-    const uint32_t head = blockIdx.y, kvh = head / (heads / kv_heads);
-    // heaviest (latest) query tiles first: they stream the most keys
-    const uint32_t qtile = gridDim.x - 1 - blockIdx.x;
+    // tile-major order, heaviest (latest) query tiles first: they stream the most keys, and whatever does not fit the
+    // machine at once is the light end, handed out as the first workgroups finish
+    const uint32_t head = blockIdx.x % heads, kvh = head / (heads / kv_heads);
+    const uint32_t ntq = gridDim.x / heads;
+    const uint32_t qtile = ntq - 1 - blockIdx.x / heads;
     const uint32_t q0 = qtile * QB;
     const uint32_t kv_stride = kv_heads * HD;
     const uint32_t seq_total = base_pos + M;
@@ -56,7 +67,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     const float c2 = (1.0f / sqrtf((float)HD)) * 1.4426950408889634f;
 
     // ---- Q fragment (B operand of S^T = K Q^T): lane (lq, lh) holds q[row][16 s + 8 lh + 0..7]
-    const uint32_t qrow = q0 + wave * QW + lq;
+    const uint32_t qrow = q0 + qg * QW + lq;
     const uint32_t qpos = base_pos + qrow;
     v8h qf[NS];
 #pragma unroll
@@ -80,45 +91,47 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
 
     const uint32_t wg_max_pos = base_pos + min(q0 + QB, M) - 1;
     const uint32_t ntiles = wg_max_pos / KT + 1;
-    const uint32_t wave_max_pos = base_pos + min(q0 + wave * QW + QW, M) - 1;   // may underflow if wave is empty
-    const uint32_t wave_min_pos = base_pos + q0 + wave * QW;                    // position of the wave's first query
-    const bool wave_active = q0 + wave * QW < M;
+    const uint32_t wave_max_pos = base_pos + min(q0 + qg * QW + QW, M) - 1;   // may underflow if the group is empty
+    const uint32_t wave_min_pos = base_pos + q0 + qg * QW;                    // position of the group's first query
+    const bool wave_active = q0 + qg * QW < M;
 
     int4 kreg[KPIECES];
     uint2 va[VITEMS], vb[VITEMS];
     auto load_tile = [&](uint32_t kt) {
 #pragma unroll
         for (int i = 0; i < KPIECES; i++) {
-            const uint32_t idx = tid + 256 * i, key = idx / (HD / 8), dc = idx % (HD / 8);
+            const uint32_t idx = tid + AP_THREADS * i, key = idx / (HD / 8), dc = idx % (HD / 8);
             const uint32_t t = kt * KT + key;
-            kreg[i] = t < seq_total ? *reinterpret_cast<const int4*>(kc + (size_t)t * kv_stride + kvh * HD + dc * 8)
-                                    : make_int4(0, 0, 0, 0);
+            kreg[i] = (idx < KTOTAL && t < seq_total) ? *reinterpret_cast<const int4*>(kc + (size_t)t * kv_stride + kvh * HD + dc * 8)
+                                                     : make_int4(0, 0, 0, 0);
         }
         // V: an item is 4 head dims of two consecutive keys (seq rows t, t+1)
 #pragma unroll
         for (int i = 0; i < VITEMS; i++) {
-            const uint32_t idx = tid + 256 * i, kp = idx / DG, dg = idx % DG;
+            const uint32_t idx = tid + AP_THREADS * i, kp = idx / DG, dg = idx % DG;
             const uint32_t t = kt * KT + 2 * kp;
             const uint16_t* src = vc + (size_t)t * kv_stride + kvh * HD + dg * 4;
-            va[i] = t < seq_total ? *reinterpret_cast<const uint2*>(src) : make_uint2(0, 0);
-            vb[i] = t + 1 < seq_total ? *reinterpret_cast<const uint2*>(src + kv_stride) : make_uint2(0, 0);
+            va[i] = (idx < VTOTAL && t < seq_total) ? *reinterpret_cast<const uint2*>(src) : make_uint2(0, 0);
+            vb[i] = (idx < VTOTAL && t + 1 < seq_total) ? *reinterpret_cast<const uint2*>(src + kv_stride) : make_uint2(0, 0);
         }
     };
     auto store_tile = [&](uint32_t buf) {
 #pragma unroll
         for (int i = 0; i < KPIECES; i++) {
-            const uint32_t idx = tid + 256 * i, key = idx / (HD / 8), dc = idx % (HD / 8);
-            *reinterpret_cast<int4*>(&Ks[buf][key * KS + dc * 8]) = kreg[i];
+            const uint32_t idx = tid + AP_THREADS * i, key = idx / (HD / 8), dc = idx % (HD / 8);
+            if (idx < KTOTAL) *reinterpret_cast<int4*>(Ks(buf) + key * KS + dc * 8) = kreg[i];
         }
         // V^T[d][key]: the two keys' values of one head dim side by side in a dword
 #pragma unroll
         for (int i = 0; i < VITEMS; i++) {
-            const uint32_t idx = tid + 256 * i, kp = idx / DG, dg = idx % DG;
-            uint32_t* vt = reinterpret_cast<uint32_t*>(&Vt[buf][(dg * 4) * VS + 2 * kp]);
-            vt[0 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].x, va[i].x, 0x05040100u);
-            vt[1 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].x, va[i].x, 0x07060302u);
-            vt[2 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].y, va[i].y, 0x05040100u);
-            vt[3 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].y, va[i].y, 0x07060302u);
+            const uint32_t idx = tid + AP_THREADS * i, kp = idx / DG, dg = idx % DG;
+            if (idx < VTOTAL) {
+                uint32_t* vt = reinterpret_cast<uint32_t*>(Vt(buf) + (dg * 4) * VS + 2 * kp);
+                vt[0 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].x, va[i].x, 0x05040100u);
+                vt[1 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].x, va[i].x, 0x07060302u);
+                vt[2 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].y, va[i].y, 0x05040100u);
+                vt[3 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].y, va[i].y, 0x07060302u);
+            }
         }
     };
 
@@ -128,55 +141,49 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
     for (uint32_t kt = 0; kt < ntiles; kt++) {
         const uint32_t buf = kt & 1;
         if (kt + 1 < ntiles) load_tile(kt + 1);          // in flight while this tile is computed
-        if (wave_active && kt * KT <= wave_max_pos) {    // else the tile lies entirely in this wave's future
-            const _Float16* Kb = Ks[buf];
-            const _Float16* Vb = Vt[buf];
-            // ---- S^T tiles: sacc[kk][r] = q . k for key kt*64 + kk*32 + 8(r/4) + 4 lh + r%4, query lq
-            v16f sacc[2];
+        const uint32_t k0 = kt * KT + kh * 32;            // this wave's 32 keys of the tile
+        if (wave_active && k0 <= wave_max_pos) {         // else they lie entirely in the group's future
+            const _Float16* Kb = Ks(buf);
+            const _Float16* Vb = Vt(buf);
+            // ---- S^T tile: sacc[r] = q . k for key k0 + 8(r/4) + 4 lh + r%4, query lq
+            v16f sacc;
 #pragma unroll
-            for (int kk = 0; kk < 2; kk++) {
+            for (int r = 0; r < 16; r++) sacc[r] = 0.f;
 #pragma unroll
-                for (int r = 0; r < 16; r++) sacc[kk][r] = 0.f;
-#pragma unroll
-                for (int s = 0; s < NS; s++) {
-                    v8h kf = *reinterpret_cast<const v8h*>(Kb + (kk * 32 + lq) * KS + 16 * s + 8 * lh);
-                    sacc[kk] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], sacc[kk], 0, 0, 0);
-                }
+            for (int s = 0; s < NS; s++) {
+                v8h kf = *reinterpret_cast<const v8h*>(Kb + (kh * 32 + lq) * KS + 16 * s + 8 * lh);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], sacc, 0, 0, 0);
             }
-            // ---- causal mask: only tiles that reach past the wave's first query have masked keys
-            if (kt * KT + KT - 1 > wave_min_pos) {
+            // ---- causal mask: only keys past the group's first query can be masked for some query
+            if (k0 + 31 > wave_min_pos) {
 #pragma unroll
-                for (int kk = 0; kk < 2; kk++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const uint32_t t = kt * KT + kk * 32 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                        sacc[kk][r] = (t <= qpos) ? sacc[kk][r] : -INFINITY;
-                    }
+                for (int r = 0; r < 16; r++) {
+                    const uint32_t t = k0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                    sacc[r] = (t <= qpos) ? sacc[r] : -INFINITY;
+                }
             }
             // ---- online softmax in base 2 (per-lane scalars: a lane owns one query)
             float m_tile = -INFINITY;
 #pragma unroll
-            for (int kk = 0; kk < 2; kk++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) m_tile = fmaxf(m_tile, sacc[kk][r]);
+            for (int r = 0; r < 16; r++) m_tile = fmaxf(m_tile, sacc[r]);
             m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, WAVE)) * c2;      // c2 > 0: max commutes with the scaling
             const float m_new = fmaxf(m_run, m_tile);
-            // m_new is finite from the first tile on (key 0 is visible to every query)
+            // a query that has seen no key yet (all of this half tile masked for it) keeps m = -inf: exponentiate
+            // against 0 instead, every p is then 2^-inf = 0
+            const float m_exp = m_new == -INFINITY ? 0.f : m_new;
             float l_tile = 0.f;
-            v8h pb[2][2];
+            v8h pb[2];
 #pragma unroll
-            for (int kk = 0; kk < 2; kk++)
+            for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int j = 0; j < 2; j++)
-#pragma unroll
-                    for (int e = 0; e < 8; e++) {
-                        const float p = __builtin_amdgcn_exp2f(fmaf(sacc[kk][8 * j + e], c2, -m_new));   // 2^-inf = 0 for masked keys
-                        l_tile += p;
-                        pb[kk][j][e] = (_Float16)p;
-                    }
+                for (int e = 0; e < 8; e++) {
+                    const float p = __builtin_amdgcn_exp2f(fmaf(sacc[8 * j + e], c2, -m_exp));   // 2^-inf = 0 for masked keys
+                    l_tile += p;
+                    pb[j][e] = (_Float16)p;
+                }
             // rescale what has been accumulated, unless no query of the wave saw a new maximum
             if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
-                const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+                const float alpha = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
                 l_run *= alpha;
 #pragma unroll
                 for (int d = 0; d < ND; d++)
@@ -185,22 +192,43 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2))) void a
             }
             l_run += l_tile;
             m_run = m_new;
-            // ---- O^T += V^T P^T
+            // ---- O^T += V^T P^T over this wave's 32 keys
 #pragma unroll
             for (int d = 0; d < ND; d++)
 #pragma unroll
-                for (int kk = 0; kk < 2; kk++)
-#pragma unroll
-                    for (int j = 0; j < 2; j++) {
-                        const _Float16* vrow = Vb + (d * 32 + lq) * VS + kk * 32 + 16 * j + 4 * lh;
-                        v4h v0 = *reinterpret_cast<const v4h*>(vrow);
-                        v4h v1 = *reinterpret_cast<const v4h*>(vrow + 8);
-                        v8h vf = (v8h){v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-                        oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pb[kk][j], oacc[d], 0, 0, 0);
-                    }
+                for (int j = 0; j < 2; j++) {
+                    const _Float16* vrow = Vb + (d * 32 + lq) * VS + kh * 32 + 16 * j + 4 * lh;
+                    v4h v0 = *reinterpret_cast<const v4h*>(vrow);
+                    v4h v1 = *reinterpret_cast<const v4h*>(vrow + 8);
+                    v8h vf = (v8h){v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                    oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pb[j], oacc[d], 0, 0, 0);
+                }
         }
         if (kt + 1 < ntiles) store_tile(buf ^ 1);   // nobody reads that buffer: its tile was finished before the last barrier
         __syncthreads();
+    }
+
+    // ---- the two waves of a query group merge their halves: the odd one hands (m, l, O) over through LDS
+    float* mg = reinterpret_cast<float*>(smem) + (qg * 64 + lane) * MERGE_FLOATS;
+    if (kh == 1) {
+        mg[0] = m_run;
+        mg[1] = l_run;
+#pragma unroll
+        for (int d = 0; d < ND; d++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) mg[2 + d * 16 + r] = oacc[d][r];
+    }
+    __syncthreads();
+    if (kh == 1) return;
+    {
+        const float m1 = mg[0], l1 = mg[1];
+        const float m = fmaxf(m_run, m1);            // finite: key 0 is in the even wave's half and visible to every query
+        const float a0 = __builtin_amdgcn_exp2f(m_run - m), a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - m);
+        l_run = l_run * a0 + l1 * a1;
+#pragma unroll
+        for (int d = 0; d < ND; d++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) oacc[d][r] = oacc[d][r] * a0 + mg[2 + d * 16 + r] * a1;
     }
 
     // ---- normalise and store: lane (lq, lh) holds out[qrow][32 d + 8 g + 4 lh + 0..3]
@@ -223,10 +251,10 @@ void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, 
                          uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
                          uint32_t hd, hipStream_t s) {
     if (M == 0) return;
-    dim3 grid((M + QB - 1) / QB, heads);
-    if (hd == 64) fh::launch(attn_prefill_kernel<64>, grid, 256, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
-    else if (hd == 96) fh::launch(attn_prefill_kernel<96>, grid, 256, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
-    else fh::launch(attn_prefill_kernel<128>, grid, 256, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
+    dim3 grid(((M + QB - 1) / QB) * heads);
+    if (hd == 64) fh::launch(attn_prefill_kernel<64>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
+    else if (hd == 96) fh::launch(attn_prefill_kernel<96>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
+    else fh::launch(attn_prefill_kernel<128>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
 }
 
 }  // namespace fh
