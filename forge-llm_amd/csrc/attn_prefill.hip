@@ -31,11 +31,14 @@ constexpr int QB = 128;       // queries per workgroup
 constexpr int KT = 64;        // keys per tile
 constexpr int AP_THREADS = 512;
 
-template <int HD>
+// QUANT: instead of f32 rows the kernel writes what the o projection's GEMM reads, the activation quantiser's int8
+// codes oq[M][heads*HD] and fp16 scales osc[M][heads*HD/32] of the same values (a 32-element block is one 32-wide
+// head_dim tile of one query: 16 values in this lane, 16 in lane ^ 32).
+template <int HD, bool QUANT>
 __global__ __launch_bounds__(AP_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
 void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
                          float* __restrict__ out, uint32_t q_stride, uint32_t out_stride, uint32_t M, uint32_t base_pos,
-                         uint32_t heads, uint32_t kv_heads) {
+                         uint32_t heads, uint32_t kv_heads, int8_t* __restrict__ oq, uint16_t* __restrict__ osc) {
     constexpr int KS = HD + 8;    // K tile row stride (halfs): 16-byte pad
     constexpr int VS = KT + 4;    // V^T tile row stride (halfs): 8-byte pad
     constexpr int KTOTAL = KT * HD / 8;          // 16-byte pieces of K per tile
@@ -233,6 +236,29 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
 
     // ---- normalise and store: lane (lq, lh) holds out[qrow][32 d + 8 g + 4 lh + 0..3]
     const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+    if (QUANT) {
+        const float inv_l = 1.0f / l_tot;
+        const uint32_t width = heads * HD;
+#pragma unroll
+        for (int d = 0; d < ND; d++) {
+            float o[16], amax = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; r++) { o[r] = oacc[d][r] * inv_l; amax = fmaxf(amax, fabsf(o[r])); }
+            amax = fmaxf(amax, __shfl_xor(amax, 32, WAVE));
+            float inv;
+            const float sc = act_scale(amax, inv);
+            if (qrow < M) {
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const uint32_t pk = ((uint32_t)quant_code(o[4 * g] * inv) & 0xFFu) | (((uint32_t)quant_code(o[4 * g + 1] * inv) & 0xFFu) << 8) |
+                                        (((uint32_t)quant_code(o[4 * g + 2] * inv) & 0xFFu) << 16) | (((uint32_t)quant_code(o[4 * g + 3] * inv) & 0xFFu) << 24);
+                    *reinterpret_cast<uint32_t*>(oq + (size_t)qrow * width + head * HD + 32 * d + 8 * g + 4 * lh) = pk;
+                }
+                if (lh == 0) osc[(size_t)qrow * (width / 32) + head * (HD / 32) + d] = f32_to_f16_bits(sc);
+            }
+        }
+        return;
+    }
     if (qrow < M) {
         const float inv_l = 1.0f / l_tot;
         float* orow = out + (size_t)qrow * out_stride + head * HD;
@@ -252,9 +278,21 @@ void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, 
                          uint32_t hd, hipStream_t s) {
     if (M == 0) return;
     dim3 grid(((M + QB - 1) / QB) * heads);
-    if (hd == 64) fh::launch(attn_prefill_kernel<64>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
-    else if (hd == 96) fh::launch(attn_prefill_kernel<96>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
-    else fh::launch(attn_prefill_kernel<128>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads);
+    int8_t* nq = nullptr;
+    uint16_t* ns = nullptr;
+    if (hd == 64) fh::launch(attn_prefill_kernel<64, false>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, nq, ns);
+    else if (hd == 96) fh::launch(attn_prefill_kernel<96, false>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, nq, ns);
+    else fh::launch(attn_prefill_kernel<128, false>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, nq, ns);
+}
+
+void launch_attn_prefill_quant(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, int8_t* oq, uint16_t* osc,
+                               uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s) {
+    if (M == 0) return;
+    dim3 grid(((M + QB - 1) / QB) * heads);
+    float* no = nullptr;
+    if (hd == 64) fh::launch(attn_prefill_kernel<64, true>, grid, AP_THREADS, 0, s, q, kc, vc, no, q_stride, 0u, M, base_pos, heads, kv_heads, oq, osc);
+    else if (hd == 96) fh::launch(attn_prefill_kernel<96, true>, grid, AP_THREADS, 0, s, q, kc, vc, no, q_stride, 0u, M, base_pos, heads, kv_heads, oq, osc);
+    else fh::launch(attn_prefill_kernel<128, true>, grid, AP_THREADS, 0, s, q, kc, vc, no, q_stride, 0u, M, base_pos, heads, kv_heads, oq, osc);
 }
 
 }  // namespace fh

@@ -148,6 +148,11 @@ void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, 
                          uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
                          uint32_t hd, hipStream_t s);
 
+// The same attention, written as the activation quantiser's output of its rows: int8 codes oq[M][heads*hd] and fp16 scales
+// osc[M][heads*hd/32] (bit-identical to launch_attn_prefill followed by launch_quantize_act).
+void launch_attn_prefill_quant(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, int8_t* oq, uint16_t* osc,
+                               uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s);
+
 bool attn_head_dim_supported(uint32_t hd);
 
 // attn_exact.hip — order-faithful attention (one workgroup per row and head).  batch_order selects

@@ -60,6 +60,7 @@ struct forge_hip_model {
     DevBuf x, qkv, gu, logits, aq, asc, attn_ws, state, argmax_ws;
     // prefill scratch (chunk_rows rows)
     DevBuf px, pqkv, pattn, pgu, paq, pasc, ptok;
+    bool prefill_fuse_quant = true;              // fast mode: attention writes int8 codes + scales (FORGE_HIP_FUSE=0: separate quantiser)
     uint32_t chunk_rows = 0;
     // pinned host staging: [0] token, [1] next token, [2] position
     uint32_t* h_stage = nullptr;
@@ -245,15 +246,17 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
         launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos, nullptr, c.heads,
                              c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), s);
     }
-    {
+    if (exact) {
+        { StageMark t(m, ST_ATTN); launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, s); }
+        { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
+    } else if (m->prefill_fuse_quant) {
+        // the attention kernel writes the o projection's quantised input itself
         StageMark t(m, ST_ATTN);
-        if (exact)
-            launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads,
-                              c.kv_heads, c.head_dim, s);
-        else
-            launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, s);
+        launch_attn_prefill_quant(qkv, QKV, m->kc(l), m->vc(l), aq, asc, M, base_pos, c.heads, c.kv_heads, c.head_dim, s);
+    } else {
+        { StageMark t(m, ST_ATTN); launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, s); }
+        { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
     }
-    { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
     { StageMark t(m, ST_O); launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s); }
     { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
     { StageMark t(m, ST_GATE_UP); launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s); }
@@ -366,6 +369,7 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
     const bool fuse_ok = !(fenv && fenv[0] == '0');
     m->fuse_norm = fuse_ok && gemv_norm_fusable(H);
     m->fuse_silu = fuse_ok && gemv_silu_fusable(H);
+    m->prefill_fuse_quant = fuse_ok;
     FH_HIP(hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking));
     FH_HIP(hipHostMalloc((void**)&m->h_stage, 64, hipHostMallocDefault));
 

@@ -176,6 +176,30 @@ def test_fused_decode_kernels_equal_separate_kernels(fh, torch_gpu, monkeypatch,
     plain.close(); fused.close()
 
 
+@pytest.mark.parametrize("shape", ["tiny", "smollm2_135m_4layers", "llama_3b_1layer"])
+def test_prefill_attention_with_quantising_epilogue_equals_separate_kernels(fh, torch_gpu, monkeypatch, shape):
+    """Fast-mode prefill: the attention kernel that writes the o projection's int8 input itself gives the same bits
+    (logits and KV cache) as attention -> f32 rows -> activation quantiser."""
+    if shape == "tiny":
+        cfg, n = tiny_cfg(fh, Q8, 0), 90
+    elif shape == "llama_3b_1layer":
+        cfg, n = fh.synth.llama32_3b(Q8, max_seq=512), 260
+        cfg["layers"], cfg["vocab"] = 1, 8000
+    else:
+        cfg, n = fh.synth.smollm2_135m(Q8, max_seq=512), 300
+        cfg["layers"] = 4
+    blob = fh.synth.make_weights_blob(cfg, seed=87, threads=16)
+    toks = fh.synth.uniform_ids(88, n, cfg["vocab"])
+    monkeypatch.setenv("FORGE_HIP_FUSE", "0")
+    plain = fh.HipModel(cfg, blob)
+    monkeypatch.setenv("FORGE_HIP_FUSE", "1")
+    fused = fh.HipModel(cfg, blob)
+    same_bits(fused.forward_prefill(toks), plain.forward_prefill(toks))
+    for which in (0, 1):
+        assert np.array_equal(fused.read_kv(cfg["layers"] - 1, which), plain.read_kv(cfg["layers"] - 1, which))
+    plain.close(); fused.close()
+
+
 def persistent_pair(fh, cfg, blob, monkeypatch, ordered=True):
     """The kernel-sequence model and the one-kernel model.  ordered: the one-kernel step sums GEMV rows in the
     reference's block order (then it is bit-identical to the sequence) instead of as the products come."""
