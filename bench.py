@@ -130,6 +130,61 @@ def timed_decode(model, tok, warmup, steps):
     return time.perf_counter() - t0, tok
 
 
+def ops_table(fh, reps=10):
+    """The isolated kernels at the sizes of the benchmark configurations (GEMV and GEMM at Llama-3.2-1B projection
+    shapes, prefill attention at 801/1501/3001 tokens, decode attention over 900/2250/8192-token caches), `reps` calls
+    each in a fixed order, timed with events on the stream the ops launch on.  An op-level call quantises its f32
+    activations first, so its wall time is that of two kernels; a kernel trace of this mode gives each kernel alone."""
+    import numpy as np
+    import torch
+    ops = fh.ops
+    rows = []
+
+    def timed(fn):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
+
+    shapes = [(2048, 2048), (2048, 512), (2048, 8192), (8192, 2048), (2048, 128256)]
+    for wd, name in ((fh.Q8_0, "Q8_0"), (fh.Q4_0, "Q4_0")):
+        bpb = 34 if wd == fh.Q8_0 else 18
+        for K, N in shapes:
+            w = ops.QWeight(wd, ops.quantize_weights(wd, fh.synth.normal(K + N, N * K, 0.02)), K, N)
+            x = torch.from_numpy(fh.synth.normal(7, K, 1.0)).cuda()
+            us = timed(lambda: ops.matmul_vec_q(w, x))
+            rows.append({"op": "gemv", "fmt": name, "K": K, "N": N, "us_per_call": round(us, 2),
+                         "weight_bytes": N * (K // 32) * bpb})
+            if N <= 8192:
+                for M in (352, 902, 1603, 2502):
+                    xm = torch.from_numpy(fh.synth.normal(8, M * K, 1.0).reshape(M, K)).cuda()
+                    us = timed(lambda: ops.matmul_mat_q(w, xm))
+                    rows.append({"op": "gemm", "fmt": name, "M": M, "K": K, "N": N, "us_per_call": round(us, 2),
+                                 "int8_ops": 2 * M * K * N})
+            w.close()
+    for heads, kvh, hd in ((32, 8, 64), (32, 32, 96)):
+        for seq in (801, 1501, 3001):
+            q = torch.from_numpy(fh.synth.normal(9, seq * heads * hd, 1.0).reshape(seq, heads * hd)).cuda()
+            k = torch.from_numpy(fh.synth.normal(10, seq * kvh * hd, 1.0).reshape(seq, kvh * hd)).cuda().half().view(torch.int16)
+            v = torch.from_numpy(fh.synth.normal(11, seq * kvh * hd, 1.0).reshape(seq, kvh * hd)).cuda().half().view(torch.int16)
+            us = timed(lambda: ops.attention_flash_batch(q, k, v, 0, heads, kvh, hd))
+            rows.append({"op": "attention_prefill", "heads": heads, "kv_heads": kvh, "head_dim": hd, "seq": seq,
+                         "us_per_call": round(us, 2), "flops": 4 * heads * hd * seq * (seq + 1) // 2})
+        for seq in (900, 2250, 8192):
+            q1 = torch.from_numpy(fh.synth.normal(12, heads * hd, 1.0)).cuda()
+            k = torch.from_numpy(fh.synth.normal(13, seq * kvh * hd, 1.0).reshape(seq, kvh * hd)).cuda().half().view(torch.int16)
+            v = torch.from_numpy(fh.synth.normal(14, seq * kvh * hd, 1.0).reshape(seq, kvh * hd)).cuda().half().view(torch.int16)
+            us = timed(lambda: ops.attention_flash(q1, k, v, seq, heads, kvh, hd))
+            rows.append({"op": "attention_decode", "heads": heads, "kv_heads": kvh, "head_dim": hd, "cache": seq,
+                         "us_per_call": round(us, 2), "kv_bytes": 2 * seq * kvh * hd * 2})
+    print(json.dumps({"ops_table": rows, "reps": reps}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -140,6 +195,8 @@ def main():
     ap.add_argument("--no-alt", action="store_true", help="skip the second model that measures the kernel-sequence decode step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (known HBM traffic, for scaling counter readings)")
+    ap.add_argument("--ops-table", action="store_true",
+                    help="instead of the model benchmark, run the isolated kernels at the benchmark configurations' sizes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures ONE GPU; --gpus must be 1 (no multi-GPU path exists to run)", file=sys.stderr)
@@ -149,6 +206,9 @@ def main():
     import torch
     fh = load_package()
     fh.require_gpu()
+    if args.ops_table:
+        ops_table(fh)
+        return
     cfg = fh.synth.llama32_1b(fh.Q8_0, max_seq=4096)
     t0 = time.perf_counter()
     blob = fh.synth.make_weights_blob(cfg, seed=args.seed, threads=16)
