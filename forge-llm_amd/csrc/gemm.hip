@@ -69,7 +69,9 @@ __device__ __forceinline__ uint32_t nib_minus8(uint32_t x) {
 }
 
 // EXACT: multiply then add per block (bit-identical to the CPU path); otherwise one FMA per block.
-template <bool Q4, bool DUMP, bool EXACT>
+// TM: 32-row tiles per wave along m.  2 = the 128-row workgroup tile; 1 = a 64-row tile for problems so small that even
+// twice the workgroups leave CUs idle (a workgroup's time per K stage halves with its tile).
+template <bool Q4, bool DUMP, bool EXACT, int TM>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ wsc, const int8_t* __restrict__ aq,
                    const uint16_t* __restrict__ asc, float* __restrict__ y, int32_t* __restrict__ isums, uint32_t M,
@@ -80,7 +82,8 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // uniform: the compiler keeps it scalar
     const uint32_t wm = wave >> 1, wn = wave & 1;
-    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    constexpr int WM = 32 * TM;                  // rows of a wave's tile
+    const uint32_t m0 = blockIdx.y * (2 * WM), n0 = blockIdx.x * BN;
     const uint32_t nblk = K / 32;
     const uint32_t lrow = lane & 31, lhalf = lane >> 5;
     const uint32_t wrow = Q4 ? K / 2 : K;   // bytes of one weight row
@@ -109,7 +112,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
 
     auto issue_stage = [&](uint32_t k0, uint32_t buf) {
 #pragma unroll
-        for (int i = 0; i < 4; i++)
+        for (int i = 0; i < 2 * TM; i++)
             __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, FH_LDS3(lds + LDS_A + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
                                                      a_voff + i * 32 * K + k0, 0, 0, 0);
         if (Q4) {
@@ -166,17 +169,17 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
 
     // ---- fragment addresses (bytes from the start of a tile / of a scale table)
     const uint32_t f_sw = (lrow >> 1) & 7;
-    const uint32_t fa_off = (wm * 64 + lrow) * BK + ((lhalf ^ f_sw) * 16);          // chunk of block kb: ^ (kb * 32)
+    const uint32_t fa_off = (wm * WM + lrow) * BK + ((lhalf ^ f_sw) * 16);          // chunk of block kb: ^ (kb * 32)
     const uint32_t fb_off = (wn * 64 + lrow) * BK + ((lhalf ^ f_sw) * 16);
     // scale operand of the rank-1 product: lanes 0..31 hold k = 0 (the scale), lanes 32..63 read zeros
-    const uint32_t sa_off = lhalf ? (uint32_t)LDS_ZERO : LDS_ASC + (wm * 64 + lrow) * SC_ROW;
+    const uint32_t sa_off = lhalf ? (uint32_t)LDS_ZERO : LDS_ASC + (wm * WM + lrow) * SC_ROW;
     const uint32_t sb_off = lhalf ? (uint32_t)LDS_ZERO : LDS_BSC + (wn * 64 + lrow) * SC_ROW;
     const uint32_t s_slot_stride = lhalf ? 0u : (uint32_t)SC_SLOT;
     const uint32_t s_t_stride = lhalf ? 0u : (uint32_t)(32 * SC_ROW);
 
-    float acc[2][2][16];
+    float acc[TM][2][16];
 #pragma unroll
-    for (int a = 0; a < 2; a++)
+    for (int a = 0; a < TM; a++)
 #pragma unroll
         for (int b = 0; b < 2; b++)
 #pragma unroll
@@ -185,18 +188,21 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     if (tid < 128) reinterpret_cast<uint32_t*>(lds + LDS_ZERO)[tid] = 0u;
 
     struct Frag {
-        v4i af[2], bf[2];
-        uint32_t sa[2], sb[2];
+        v4i af[TM], bf[2];
+        uint32_t sa[TM], sb[2];
     };
     auto read_frag = [&](Frag& f, uint32_t buf, uint32_t slot, int kb) {
         const uint8_t* A = lds + LDS_A + buf * TILE_BYTES;
         const uint8_t* B = lds + LDS_B + buf * TILE_BYTES;
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-            f.af[t] = *reinterpret_cast<const v4i*>(A + ((fa_off ^ (kb * 32)) + t * 32 * BK));
             f.bf[t] = *reinterpret_cast<const v4i*>(B + ((fb_off ^ (kb * 32)) + t * 32 * BK));
-            f.sa[t] = *reinterpret_cast<const uint16_t*>(lds + sa_off + slot * s_slot_stride + t * s_t_stride + kb * 2);
             f.sb[t] = *reinterpret_cast<const uint16_t*>(lds + sb_off + slot * s_slot_stride + t * s_t_stride + kb * 2);
+        }
+#pragma unroll
+        for (int t = 0; t < TM; t++) {
+            f.af[t] = *reinterpret_cast<const v4i*>(A + ((fa_off ^ (kb * 32)) + t * 32 * BK));
+            f.sa[t] = *reinterpret_cast<const uint16_t*>(lds + sa_off + slot * s_slot_stride + t * s_t_stride + kb * 2);
             if (MAGIC && (kb & 1)) {
                 f.af[t].x = (int)neg4((uint32_t)f.af[t].x); f.af[t].y = (int)neg4((uint32_t)f.af[t].y);
                 f.af[t].z = (int)neg4((uint32_t)f.af[t].z); f.af[t].w = (int)neg4((uint32_t)f.af[t].w);
@@ -241,14 +247,15 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
             if (kb + 1 < KB) read_frag(fnext, buf, slot, kb + 1);
             // four tiles, software-pipelined by one (across blocks too): the MFMAs of the next tile are issued
             // before this one is combined, so the matrix unit works while the VALU scales
+            constexpr int NT = 2 * TM;           // MFMA tiles of a wave
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
+            for (int t = 0; t < NT; t++) {
                 const int tm = t >> 1, tn = t & 1;
                 // next tile's two MFMAs, with this tile's combine split between them: the second MFMA would
                 // otherwise wait (in order, blocking the FMAs behind it) for the first to clear the matrix pipe
-                const bool has_next = t < 3 || kb + 1 < KB;
-                const Frag& fn = t < 3 ? f : fnext;
-                const int tm2 = t < 3 ? (t + 1) >> 1 : 0, tn2 = t < 3 ? (t + 1) & 1 : 0;
+                const bool has_next = t < NT - 1 || kb + 1 < KB;
+                const Frag& fn = t < NT - 1 ? f : fnext;
+                const int tm2 = t < NT - 1 ? (t + 1) >> 1 : 0, tn2 = t < NT - 1 ? (t + 1) & 1 : 0;
                 v16i isum_n = zero_i;
                 v16f S_n = zero_f;
                 if (has_next) isum_n = __builtin_amdgcn_mfma_i32_32x32x32_i8(fn.af[tm2], fn.bf[tn2], c_in, 0, 0, 0);
@@ -272,7 +279,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                 if (DUMP) {
                     const uint32_t b = s * KB + kb;
                     const uint32_t n = n0 + wn * 64 + tn * 32 + lrow;
-                    const uint32_t mb = m0 + wm * 64 + tm * 32 + 4 * lhalf;
+                    const uint32_t mb = m0 + wm * WM + tm * 32 + 4 * lhalf;
                     const uint32_t base = (n < N && b < nblk) ? ((mb * N + n) * nblk + b) * 4 : OOB;
 #pragma unroll
                     for (int r = 0; r < 16; r++)
@@ -290,7 +297,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
 
     // Stages go in pairs (an odd count runs one stage of zero scales).  After a pair the fast mode removes what
     // the 8 blocks left of the bias: 12582912 * sum_b a_s[m][b] * (+-w_s[n][b]), the sum being one f16 MFMA.
-    const uint32_t ta_off = lhalf ? (uint32_t)LDS_ZERO : LDS_ASC + (wm * 64 + lrow) * SC_ROW;
+    const uint32_t ta_off = lhalf ? (uint32_t)LDS_ZERO : LDS_ASC + (wm * WM + lrow) * SC_ROW;
     const uint32_t tb_off = lhalf ? (uint32_t)LDS_ZERO : LDS_BSC + (wn * 64 + lrow) * SC_ROW;
     for (uint32_t s = 0; s < stages; s += 2) {
         run_stage(s, 0);
@@ -298,18 +305,21 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         if (MAGIC) {
             const uint32_t pair = lhalf ? 0u : (s & 2u) * (uint32_t)SC_SLOT;      // slots {0,1} or {2,3}
             typedef _Float16 v4h __attribute__((ext_vector_type(4)));
-            v8h ta[2], tb[2];
+            v8h ta[TM], tb[2];
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-                const v4h a0 = *reinterpret_cast<const v4h*>(lds + ta_off + pair + t * s_t_stride);
-                const v4h a1 = *reinterpret_cast<const v4h*>(lds + ta_off + pair + s_slot_stride + t * s_t_stride);
                 const v4h b0 = *reinterpret_cast<const v4h*>(lds + tb_off + pair + t * s_t_stride);
                 const v4h b1 = *reinterpret_cast<const v4h*>(lds + tb_off + pair + s_slot_stride + t * s_t_stride);
-                ta[t] = (v8h){a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
                 tb[t] = (v8h){b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
             }
 #pragma unroll
-            for (int t = 0; t < 4; t++) {
+            for (int t = 0; t < TM; t++) {
+                const v4h a0 = *reinterpret_cast<const v4h*>(lds + ta_off + pair + t * s_t_stride);
+                const v4h a1 = *reinterpret_cast<const v4h*>(lds + ta_off + pair + s_slot_stride + t * s_t_stride);
+                ta[t] = (v8h){a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+            }
+#pragma unroll
+            for (int t = 0; t < 2 * TM; t++) {
                 const int tm = t >> 1, tn = t & 1;
                 const v16f T = __builtin_amdgcn_mfma_f32_32x32x16_f16(ta[tm], tb[tn], zero_f, 0, 0, 0);
 #pragma unroll
@@ -322,11 +332,11 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     // epilogue: lane holds column n = lrow, rows 8g + 4*lhalf + (r&3); the descriptor drops rows >= M
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc((void*)y, 0, M * ldy * 4, RSRC_FLAGS);
 #pragma unroll
-    for (int tm = 0; tm < 2; tm++)
+    for (int tm = 0; tm < TM; tm++)
 #pragma unroll
         for (int tn = 0; tn < 2; tn++) {
             const uint32_t n = n0 + wn * 64 + tn * 32 + lrow;
-            const uint32_t mb = m0 + wm * 64 + tm * 32 + 4 * lhalf;
+            const uint32_t mb = m0 + wm * WM + tm * 32 + 4 * lhalf;
             const uint32_t base = n < N ? (mb * ldy + n) * 4 : OOB;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
@@ -354,13 +364,24 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
     const uint64_t m_fit = LIMIT / per_m, n_fit = LIMIT / per_n;
     const uint32_t m_step = M <= m_fit ? M : (uint32_t)std::max<uint64_t>(BM, m_fit / BM * BM);
     const uint32_t n_step = w.N <= n_fit ? w.N : (uint32_t)std::max<uint64_t>(BN, n_fit / BN * BN);
-#define FH_GEMM_LAUNCH(Q4_, DUMP_, EXACT_)                                                                              \
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 256;
+        return n > 0 ? n : 256;
+    }();
+#define FH_GEMM_LAUNCH_TM(Q4_, DUMP_, EXACT_, TM_)                                                                        \
     do {                                                                                                                \
-        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, DUMP_, EXACT_>,           \
+        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, DUMP_, EXACT_, TM_>,      \
                                                              hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES); \
         (void)lds_ok;                                                                                                   \
-        fh::launch(gemm_q_kernel<Q4_, DUMP_, EXACT_>, grid, 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c, y_c, is_c, mc, \
-                   nc, w.K, ldy, accf);                                                                                 \
+        dim3 grid((nc + BN - 1) / BN, (mc + 64 * TM_ - 1) / (64 * TM_));                                                \
+        fh::launch(gemm_q_kernel<Q4_, DUMP_, EXACT_, TM_>, grid, 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c, y_c, is_c, \
+                   mc, nc, w.K, ldy, accf);                                                                             \
+    } while (0)
+#define FH_GEMM_LAUNCH(Q4_, DUMP_, EXACT_)                         \
+    do {                                                           \
+        if (small_tiles) FH_GEMM_LAUNCH_TM(Q4_, DUMP_, EXACT_, 1); \
+        else FH_GEMM_LAUNCH_TM(Q4_, DUMP_, EXACT_, 2);             \
     } while (0)
     for (uint32_t mlo = 0; mlo < M; mlo += m_step)
         for (uint32_t nlo = 0; nlo < w.N; nlo += n_step) {
@@ -372,7 +393,10 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
             float* y_c = y + (size_t)mlo * ldy + nlo;
             // block sums of a sub-problem are laid out [mc][nc][nblk]: only whole problems are dumped
             int32_t* is_c = isums;
-            dim3 grid((nc + BN - 1) / BN, (mc + BM - 1) / BM);
+            // 64-row tiles when even those leave no CU with more than one workgroup: a workgroup's time per K stage
+            // halves with its tile, and a larger tile would only leave more CUs idle
+            const uint64_t tiles64 = (uint64_t)((nc + BN - 1) / BN) * ((mc + 63) / 64);
+            const bool small_tiles = tiles64 <= (uint64_t)cus && mc > 64;
             if (q4) {
                 if (isums) FH_GEMM_LAUNCH(true, true, true);
                 else if (exact) FH_GEMM_LAUNCH(true, false, true);
@@ -384,6 +408,7 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
             }
         }
 #undef FH_GEMM_LAUNCH
+#undef FH_GEMM_LAUNCH_TM
 }
 
 }  // namespace fh
