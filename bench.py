@@ -35,9 +35,9 @@ PROMPT_TOKENS = 2502
 # WRITE_SIZE counters of two profiler runs of this script, each scaled by what the same counter reads for the 1 GiB
 # copy of --calibrate-copy (FETCH_SIZE x2.000, WRITE_SIZE x1.000).  Summary: profiles/gemv_hbm_traffic_pmc.md.
 GEMV_HBM_BYTES_PER_LAUNCH = 20.46e6 + 0.02e6      # fetched + written
-# The same for one launch of the resident decode kernel (the whole step) at this context: 1 421.6 MB fetched + 12.2 MB
+# The same for one launch of the resident decode kernel (the whole step) at this context: 1 433.6 MB fetched + 13.3 MB
 # written.  Summary: profiles/decode_step_kernel_hbm_traffic_pmc.md.
-STEP_KERNEL_HBM_BYTES_PER_LAUNCH = 1433.8e6
+STEP_KERNEL_HBM_BYTES_PER_LAUNCH = 1446.9e6
 
 
 def gemv_launch_bytes(fh, cfg):
