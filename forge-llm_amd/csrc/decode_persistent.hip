@@ -265,7 +265,7 @@ template <bool ORDERED>
 __device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict__ norm_w, float4 nw0, float eps, uint32_t H,
                                               uint32_t* aq_lds, float* as_lds, float* part, const PdCtx& cx) {
     const uint32_t tid = cx.tid;
-    __syncthreads();
+    float ss;                      // sum of squares of the row (the caller's barrier made xs visible)
     if (!ORDERED) {
         float s = 0.f;
         for (uint32_t e0 = tid * 4; e0 < H; e0 += PD_THREADS * 4) {
@@ -278,13 +278,16 @@ __device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict
         s += __builtin_amdgcn_update_dpp(0.f, s, 0x140, 0xF, 0xF, false);     // row_mirror
         if ((tid & 15u) == 0) part[tid >> 4] = s;                             // PD_THREADS / 16 = 32 partial sums
         __syncthreads();
-        if (tid == 0) {
-            float r = 0.f;
-#pragma unroll
-            for (int i = 0; i < PD_THREADS / 16; i++) r += part[i];
-            part[PD_THREADS / 16] = r;
-        }
-    } else if (tid < 64) {
+        // every thread adds the 32 partial sums itself (two per lane, then the same folds): no second barrier
+        static_assert(PD_THREADS / 16 == 32, "two partial sums per lane of a 16-lane row");
+        float r = part[tid & 15u] + part[16 + (tid & 15u)];
+        r += __builtin_amdgcn_update_dpp(0.f, r, 0xB1, 0xF, 0xF, false);
+        r += __builtin_amdgcn_update_dpp(0.f, r, 0x4E, 0xF, 0xF, false);
+        r += __builtin_amdgcn_update_dpp(0.f, r, 0x141, 0xF, 0xF, false);
+        r += __builtin_amdgcn_update_dpp(0.f, r, 0x140, 0xF, 0xF, false);
+        ss = r;
+    } else {
+      if (tid < 64) {
         // lane i < 16 owns accumulator i: x[i], x[16 + i], ... added in order with FMAs.  The reads of the next eight
         // values are issued before the current eight are consumed, so LDS latency stays off the dependent chain.
         float s = 0.f;
@@ -313,9 +316,11 @@ __device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict
             for (uint32_t i = H / 16 * 16; i < H; i++) r = r + xs[i] * xs[i];
             part[PD_THREADS / 16] = r;
         }
+      }
+      __syncthreads();
+      ss = part[PD_THREADS / 16];
     }
-    __syncthreads();
-    const float inv_rms = 1.0f / sqrtf(part[PD_THREADS / 16] / (float)H + eps);
+    const float inv_rms = 1.0f / sqrtf(ss / (float)H + eps);
     for (uint32_t e0 = tid * 4; e0 < H; e0 += PD_THREADS * 4) {
         const float4 xv = *reinterpret_cast<const float4*>(xs + e0);
         const float4 wv = e0 == tid * 4 ? nw0 : ldg(reinterpret_cast<const float4*>(norm_w + e0));
