@@ -267,24 +267,12 @@ __device__ __forceinline__ void pd_norm_quant(float* xs, const float* __restrict
     const uint32_t tid = cx.tid;
     float ss;                      // sum of squares of the row (the caller's barrier made xs visible)
     if (!ORDERED) {
-        float s = 0.f;
-        for (uint32_t e0 = tid * 4; e0 < H; e0 += PD_THREADS * 4) {
-            const float4 xv = *reinterpret_cast<const float4*>(xs + e0);
-            s += (xv.x * xv.x + xv.y * xv.y) + (xv.z * xv.z + xv.w * xv.w);
-        }
-        s += __builtin_amdgcn_update_dpp(0.f, s, 0xB1, 0xF, 0xF, false);      // quad_perm [1,0,3,2]
-        s += __builtin_amdgcn_update_dpp(0.f, s, 0x4E, 0xF, 0xF, false);      // quad_perm [2,3,0,1]
-        s += __builtin_amdgcn_update_dpp(0.f, s, 0x141, 0xF, 0xF, false);     // row_half_mirror
-        s += __builtin_amdgcn_update_dpp(0.f, s, 0x140, 0xF, 0xF, false);     // row_mirror
-        if ((tid & 15u) == 0) part[tid >> 4] = s;                             // PD_THREADS / 16 = 32 partial sums
-        __syncthreads();
-        // every thread adds the 32 partial sums itself (two per lane, then the same folds): no second barrier
-        static_assert(PD_THREADS / 16 == 32, "two partial sums per lane of a 16-lane row");
-        float r = part[tid & 15u] + part[16 + (tid & 15u)];
-        r += __builtin_amdgcn_update_dpp(0.f, r, 0xB1, 0xF, 0xF, false);
-        r += __builtin_amdgcn_update_dpp(0.f, r, 0x4E, 0xF, 0xF, false);
-        r += __builtin_amdgcn_update_dpp(0.f, r, 0x141, 0xF, 0xF, false);
-        r += __builtin_amdgcn_update_dpp(0.f, r, 0x140, 0xF, 0xF, false);
+        // the pollers left the squares of what they fetched as 8 partial sums (one per 16 lanes): every thread folds them
+        static_assert(PD_POLL_THREADS / 16 == 8, "eight partial sums");
+        float r = part[tid & 7u];
+        r += __builtin_amdgcn_update_dpp(0.f, r, 0xB1, 0xF, 0xF, false);      // quad_perm [1,0,3,2]
+        r += __builtin_amdgcn_update_dpp(0.f, r, 0x4E, 0xF, 0xF, false);      // quad_perm [2,3,0,1]
+        r += __builtin_amdgcn_update_dpp(0.f, r, 0x141, 0xF, 0xF, false);     // row_half_mirror: lanes 0..7 <-> 7..0
         ss = r;
     } else {
       if (tid < 64) {
@@ -345,10 +333,15 @@ __device__ __forceinline__ void pd_load_aq(const uint64_t* t, uint32_t tag, uint
 }
 
 // The residual stream (tagged) into LDS as floats; fetched by the poller waves.
+// `ssq` collects the squares of what this thread fetched.
 __device__ __forceinline__ void pd_load_x(const uint64_t* tx, uint32_t tag, uint32_t H, float* xs, float* misc, bool use_hint,
-                                          const PdCtx& cx) {
+                                          const PdCtx& cx, float& ssq) {
     const Hint hint{tx + H - 1, use_hint ? reinterpret_cast<volatile uint32_t*>(misc + PD_MISC_HINT) : nullptr};
-    poll_vec<PD_POLL_N>(tx, H, tag, PD_POLL_THREADS, cx, hint, [&](uint32_t i, uint32_t p) { xs[i] = __uint_as_float(p); });
+    poll_vec<PD_POLL_N>(tx, H, tag, PD_POLL_THREADS, cx, hint, [&](uint32_t i, uint32_t p) {
+        const float v = __uint_as_float(p);
+        xs[i] = v;
+        ssq += v * v;
+    });
 }
 
 // ---- the GEMV of a phase ------------------------------------------------------------------------------
@@ -783,9 +776,18 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     if (streamer) {
         if (!early) pd_load_round<Q4>(job, h, t, 0, sw, cx.lane, W);      // otherwise the previous phase's tail issued them
     } else {
+        float ssq = 0.f;
         if (job.pro == PRO_AQ) pd_load_aq(job.tin, job.tin_tag, K, aq_lds, as_lds, misc, a.use_hint != 0, cx);
-        else if (job.tin_tag) pd_load_x(job.tin, job.tin_tag, K, big, misc, a.use_hint != 0, cx);
-        else for (uint32_t i = cx.tid; i < K; i += PD_POLL_THREADS) big[i] = emb[i];
+        else if (job.tin_tag) pd_load_x(job.tin, job.tin_tag, K, big, misc, a.use_hint != 0, cx, ssq);
+        else for (uint32_t i = cx.tid; i < K; i += PD_POLL_THREADS) { const float v = emb[i]; big[i] = v; ssq += v * v; }
+        if (!ORDERED && job.pro == PRO_NORM) {
+            // the pollers square what they fetched: the sum of squares needs no pass (and no barrier) of its own
+            ssq += __builtin_amdgcn_update_dpp(0.f, ssq, 0xB1, 0xF, 0xF, false);      // quad_perm [1,0,3,2]
+            ssq += __builtin_amdgcn_update_dpp(0.f, ssq, 0x4E, 0xF, 0xF, false);      // quad_perm [2,3,0,1]
+            ssq += __builtin_amdgcn_update_dpp(0.f, ssq, 0x141, 0xF, 0xF, false);     // row_half_mirror
+            ssq += __builtin_amdgcn_update_dpp(0.f, ssq, 0x140, 0xF, 0xF, false);     // row_mirror
+            if ((cx.tid & 15u) == 0) misc[cx.tid >> 4] = ssq;                         // PD_POLL_THREADS / 16 = 8 partial sums
+        }
     }
     __syncthreads();
     if (*cx.sh_abort) return;
