@@ -62,6 +62,13 @@ def lib():
         return _lib
     if not os.path.exists(LIB_PATH):
         raise ForgeHipError(ERR_NO_DEVICE, f"{LIB_PATH} not built; run `python forge-llm_amd/build.py`")
+    # The Python host side uses PyTorch for device memory and streams, and PyTorch brings its own copy of the HIP
+    # runtime: it has to be in the process first, so that the library binds to that same copy (loaded the other way
+    # round, the two runtimes do not see each other's device).
+    try:
+        import torch  # noqa: F401
+    except ImportError:
+        pass
     L = C.CDLL(LIB_PATH)
     vp, u32, u64, i32 = C.c_void_p, C.c_uint32, C.c_uint64, C.c_int32
     L.forge_hip_last_error.restype = C.c_char_p
