@@ -192,6 +192,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--seed", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-gguf", action="store_true", help="create the model from the weights blob instead of from a GGUF file")
     ap.add_argument("--no-alt", action="store_true", help="skip the second model that measures the kernel-sequence decode step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (known HBM traffic, for scaling counter readings)")
@@ -219,9 +220,27 @@ def main():
     t0 = time.perf_counter()
     blob = fh.synth.make_weights_blob(cfg, seed=args.seed, threads=16)
     t_gen = time.perf_counter() - t0
-    t0 = time.perf_counter()
-    model = fh.HipModel(cfg, blob)
-    t_load = time.perf_counter() - t0
+    # The model arrives the way a user's does: as a GGUF file that the library parses, converts and uploads
+    # (--no-gguf: hand the weights blob over directly).
+    gguf_info = None
+    if args.no_gguf:
+        t0 = time.perf_counter()
+        model = fh.HipModel(cfg, blob)
+        t_load = time.perf_counter() - t0
+    else:
+        import tempfile
+        with tempfile.TemporaryDirectory() as tmp:
+            path = os.path.join(tmp, "model.gguf")
+            t0 = time.perf_counter()
+            fh.gguf.model_to_gguf(cfg, blob, tied=True, path=path)
+            t_write = time.perf_counter() - t0
+            nbytes = os.path.getsize(path)
+            t0 = time.perf_counter()
+            model = fh.HipModel.from_gguf(path, max_seq=cfg["max_seq"])
+            t_load = time.perf_counter() - t0
+        assert {k: model.config[k] for k in cfg if k not in ("rms_eps", "rope_theta")} == {k: cfg[k] for k in cfg if k not in ("rms_eps", "rope_theta")}
+        gguf_info = {"file_bytes": nbytes, "write_s": round(t_write, 2), "parse_convert_upload_s": round(t_load, 2),
+                     "GB_per_s": round(nbytes / t_load / 1e9, 2)}
     prompt = fh.synth.uniform_ids(args.seed + 1, PROMPT_TOKENS, cfg["vocab"])
 
     # ---- prefill: one warm-up pass, then timed
@@ -310,6 +329,7 @@ def main():
         "decode_stage_us": stage_us,
         "kernel_sequence_path": alt,
         "setup_s": {"generate_weights": round(t_gen, 1), "upload_and_repack": round(t_load, 1)},
+        "gguf_load": gguf_info,
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(fh, cfg, blob, prompt)

@@ -33,6 +33,10 @@ EXPORTS = [
     "forge_hip_qweight_destroy", "forge_hip_quantize_act", "forge_hip_gemv_q", "forge_hip_gemm_q",
     "forge_hip_block_isums", "forge_hip_rms_norm", "forge_hip_silu_mul", "forge_hip_rope_kv_store",
     "forge_hip_attn_prefill_f16kv", "forge_hip_attn_decode_f16kv", "forge_hip_argmax",
+    "forge_hip_gguf_open", "forge_hip_gguf_parse", "forge_hip_gguf_close", "forge_hip_gguf_version", "forge_hip_gguf_alignment",
+    "forge_hip_gguf_tensor_data_offset", "forge_hip_gguf_tensor_count", "forge_hip_gguf_metadata_count", "forge_hip_gguf_tensor",
+    "forge_hip_gguf_find_tensor", "forge_hip_gguf_meta", "forge_hip_gguf_config", "forge_hip_gguf_export_weights",
+    "forge_hip_model_create_from_gguf",
 ]
 
 
@@ -150,6 +154,6 @@ def require_gpu():
 
 
 from .hip_model import HipModel  # noqa: E402
-from . import ops, synth  # noqa: E402
+from . import gguf, ops, synth  # noqa: E402
 
 __all__ = ["HipModel", "ops", "synth", "Config", "ForgeHipError", "lib", "check", "device_count", "Q4_0", "Q8_0", "FLAG_EXACT"]

@@ -11,7 +11,7 @@ BUILD = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libforge_hip.so")
 
 SOURCES = ["format.hip", "elementwise.hip", "gemv.hip", "gemm.hip", "attn_decode.hip", "attn_prefill.hip",
-           "attn_exact.hip", "decode_persistent.hip", "api.hip", "model.hip"]
+           "attn_exact.hip", "decode_persistent.hip", "api.hip", "model.hip", "gguf.cpp"]
 
 # -packed-fp32-ops off: keep hipcc from forming packed FP32 instructions.
 # -ffp-contract=off: the CPU path never fuses a*b+c; kernels say fmaf() where a fused op is meant.
@@ -28,7 +28,7 @@ def _hipcc():
 
 
 def _compile(src):
-    obj = os.path.join(BUILD, src.replace(".hip", ".o"))
+    obj = os.path.join(BUILD, os.path.splitext(src)[0] + ".o")
     cmd = [_hipcc(), *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass warns that it does not know the packed-fp32 feature: harmless, filter it

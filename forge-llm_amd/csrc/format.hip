@@ -145,7 +145,8 @@ void quantize_host(uint32_t wdtype, const float* d, uint64_t n, uint8_t* out) {
 // dequant_q8_0 / dequant_q4_0, weight_loader.rs:860-926
 void dequant_host(uint32_t wdtype, const uint8_t* data, uint64_t n, float* out) {
     const uint64_t nb = (n + 31) / 32;
-    for (uint64_t b = 0; b < nb; b++) {
+    parallel_blocks(nb, [&](uint64_t b0, uint64_t b1) {
+    for (uint64_t b = b0; b < b1; b++) {
         if (wdtype == FORGE_HIP_Q8_0) {
             const uint8_t* blk = data + b * 34;
             const float sc = f16_to_f32_host((uint16_t)(blk[0] | (blk[1] << 8)));
@@ -160,6 +161,7 @@ void dequant_host(uint32_t wdtype, const uint8_t* data, uint64_t n, float* out) 
             }
         }
     }
+    });
 }
 
 void repack_host(uint32_t wdtype, const uint8_t* raw, uint32_t K, uint64_t N, uint8_t* qs, uint16_t* scales) {

@@ -1,0 +1,508 @@
+// GGUF on the input side of the hot path (host code only): the file parser, the model configuration read from
+// its metadata, and the conversion of its tensors into the headerless weights blob that forge_hip_model_create takes.
+//
+//   parse            crates/forgellm-frontend/src/gguf.rs:484-551 (header, metadata, tensor descriptors, alignment)
+//   config           crates/forgellm-cli/src/main.rs:700-830 (metadata keys, defaults, majority vote on the dtype)
+//   tensor names     crates/forgellm-frontend/src/weight_loader.rs:400-447 (gguf_name_to_hf)
+//   blob order       crates/forgellm-cli/src/main.rs:2714-2757 (export-weights)
+//
+// A file is memory-mapped and tensors are converted straight from the mapping into the caller's buffer.
+#include <errno.h>
+#include <fcntl.h>
+#include <stdio.h>
+#include <string.h>
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <unistd.h>
+
+#include <map>
+#include <memory>
+#include <new>
+
+#include "common.h"
+
+namespace {
+
+constexpr uint32_t GGUF_MAGIC = 0x46554747u;      // "GGUF", gguf.rs:18
+constexpr uint64_t DEFAULT_ALIGNMENT = 32;         // gguf.rs:21
+
+enum : uint32_t { T_F32 = 0, T_F16 = 1, T_Q4_0 = 2, T_Q8_0 = 8, T_BF16 = 30 };
+
+// Elements per block and bytes per block of every GGML type id the reference knows (gguf.rs:207-258);
+// other ids are refused (GGUFError::UnsupportedGGMLType).
+bool ggml_type_layout(uint32_t id, uint32_t* block, uint32_t* bytes) {
+    static const struct { uint32_t id, block, bytes; } t[] = {
+        {0, 1, 4},     {1, 1, 2},     {2, 32, 18},   {3, 32, 20},   {6, 32, 22},   {7, 32, 24},   {8, 32, 34},  {9, 32, 40},
+        {10, 256, 84}, {11, 256, 110}, {12, 256, 144}, {13, 256, 176}, {14, 256, 210}, {15, 256, 292}, {16, 256, 66}, {17, 256, 74},
+        {18, 256, 98}, {19, 256, 50},  {20, 32, 18},  {21, 256, 110}, {22, 256, 82},  {23, 32, 36},   {24, 1, 1},   {25, 1, 2},
+        {26, 1, 4},    {27, 1, 8},    {28, 1, 8},    {29, 256, 56},  {30, 1, 2}};
+    for (const auto& e : t)
+        if (e.id == id) { *block = e.block; *bytes = e.bytes; return true; }
+    return false;
+}
+
+struct MetaValue {
+    uint32_t type = 0;           // GGUF value type id 0..12
+    uint64_t bits = 0;           // scalars: the value's bytes, little endian, zero-extended
+    std::string str;             // type 8
+    uint32_t elem_type = 0;      // type 9
+    uint64_t count = 0;          // type 9: number of elements (elements themselves are skipped, only counted)
+};
+
+struct TensorInfo {
+    std::string name;
+    uint32_t n_dims = 0;
+    uint64_t dims[4] = {0, 0, 0, 0};
+    uint32_t type = 0;
+    uint64_t offset = 0;         // from the start of the tensor data section
+    uint64_t numel() const { uint64_t n = 1; for (uint32_t i = 0; i < n_dims; i++) n *= dims[i]; return n; }
+    uint64_t data_size() const {                              // gguf.rs:278-284
+        uint32_t block = 1, bytes = 0;
+        ggml_type_layout(type, &block, &bytes);
+        return (numel() + block - 1) / block * bytes;
+    }
+};
+
+struct Reader {
+    const uint8_t* p;
+    uint64_t n, pos = 0;
+    bool ok = true;
+    bool take(void* dst, uint64_t k) {
+        if (!ok || k > n - pos) { ok = false; memset(dst, 0, k); return false; }
+        memcpy(dst, p + pos, k);
+        pos += k;
+        return true;
+    }
+    template <typename T> T get() { T v{}; take(&v, sizeof(T)); return v; }
+    bool str(std::string* s) {
+        const uint64_t len = get<uint64_t>();
+        if (!ok || len > n - pos) { ok = false; return false; }
+        s->assign(reinterpret_cast<const char*>(p + pos), len);
+        pos += len;
+        return true;
+    }
+};
+
+bool valid_utf8(const std::string& s) {
+    size_t i = 0;
+    while (i < s.size()) {
+        const uint8_t c = (uint8_t)s[i];
+        int extra = c < 0x80 ? 0 : (c >> 5) == 6 ? 1 : (c >> 4) == 14 ? 2 : (c >> 3) == 30 ? 3 : -1;
+        if (extra < 0 || i + extra >= s.size() + (extra == 0)) return false;
+        for (int k = 1; k <= extra; k++)
+            if (((uint8_t)s[i + k] >> 6) != 2) return false;
+        i += extra + 1;
+    }
+    return true;
+}
+
+}  // namespace
+
+struct forge_hip_gguf {
+    const uint8_t* data = nullptr;
+    uint64_t nbytes = 0;
+    void* map = nullptr;          // set when the library mapped the file itself
+    uint64_t map_len = 0;
+    uint32_t version = 0;
+    uint64_t alignment = DEFAULT_ALIGNMENT, tensor_data_offset = 0;
+    std::map<std::string, MetaValue> meta;
+    std::vector<TensorInfo> tensors;
+    ~forge_hip_gguf() { if (map) munmap(map, map_len); }
+    const MetaValue* find(const std::string& k) const { auto it = meta.find(k); return it == meta.end() ? nullptr : &it->second; }
+    const TensorInfo* tensor(const std::string& name) const {
+        for (const auto& t : tensors) if (t.name == name) return &t;
+        return nullptr;
+    }
+    bool get_u32(const std::string& k, uint32_t* out) const {         // gguf.rs:306-308: a Uint32 value only
+        const MetaValue* v = find(k);
+        if (!v || v->type != 4) return false;
+        *out = (uint32_t)v->bits;
+        return true;
+    }
+    bool get_u64(const std::string& k, uint64_t* out) const {         // gguf.rs:311-317: Uint64, or Uint32 widened
+        const MetaValue* v = find(k);
+        if (!v || (v->type != 10 && v->type != 4)) return false;
+        *out = v->bits;
+        return true;
+    }
+    bool get_f32(const std::string& k, float* out) const {
+        const MetaValue* v = find(k);
+        if (!v || v->type != 6) return false;
+        const uint32_t b = (uint32_t)v->bits;
+        memcpy(out, &b, 4);
+        return true;
+    }
+};
+
+namespace {
+
+using fh::fail;
+
+// One metadata value (gguf.rs:447-476).  Array elements are parsed (they may be strings or nested arrays) but not kept.
+int32_t read_value(Reader& r, uint32_t type, MetaValue* v, int depth) {
+    static const int width[13] = {1, 1, 2, 2, 4, 4, 4, 1, 0, 0, 8, 8, 8};
+    if (type > 12) return fail(FORGE_HIP_ERR_INVALID, "gguf: unsupported metadata value type: " + std::to_string(type));
+    if (v) v->type = type;
+    if (type == 8) {
+        std::string s;
+        if (!r.str(&s)) return fail(FORGE_HIP_ERR_INVALID, "gguf: file ends inside a metadata string");
+        if (!valid_utf8(s)) return fail(FORGE_HIP_ERR_INVALID, "gguf: invalid UTF-8 in string");
+        if (v) v->str = std::move(s);
+        return FORGE_HIP_OK;
+    }
+    if (type == 9) {
+        const uint32_t et = r.get<uint32_t>();
+        const uint64_t count = r.get<uint64_t>();
+        if (!r.ok) return fail(FORGE_HIP_ERR_INVALID, "gguf: file ends inside a metadata array");
+        if (depth > 8) return fail(FORGE_HIP_ERR_INVALID, "gguf: metadata arrays nested too deeply");
+        if (v) { v->elem_type = et; v->count = count; }
+        if (et <= 12 && width[et]) {                        // fixed-width elements: skip them in one step
+            if (count > (r.n - r.pos) / width[et]) return fail(FORGE_HIP_ERR_INVALID, "gguf: file ends inside a metadata array");
+            r.pos += count * width[et];
+            return FORGE_HIP_OK;
+        }
+        for (uint64_t i = 0; i < count; i++) {
+            const int32_t rc = read_value(r, et, nullptr, depth + 1);
+            if (rc) return rc;
+        }
+        return FORGE_HIP_OK;
+    }
+    uint64_t bits = 0;
+    if (!r.take(&bits, width[type])) return fail(FORGE_HIP_ERR_INVALID, "gguf: file ends inside a metadata value");
+    if (type == 7) bits = bits != 0;                        // read_bool, gguf.rs:436-438
+    if (v) v->bits = bits;
+    return FORGE_HIP_OK;
+}
+
+int32_t parse_into(forge_hip_gguf* g) {
+    Reader r{g->data, g->nbytes};
+    const uint32_t magic = r.get<uint32_t>();
+    if (!r.ok) return fail(FORGE_HIP_ERR_INVALID, "gguf: file shorter than its header");
+    if (magic != GGUF_MAGIC) {
+        char buf[64];
+        snprintf(buf, sizeof buf, "gguf: invalid GGUF magic number: got 0x%08X", magic);
+        return fail(FORGE_HIP_ERR_INVALID, buf);
+    }
+    g->version = r.get<uint32_t>();
+    if (r.ok && g->version != 2 && g->version != 3)
+        return fail(FORGE_HIP_ERR_INVALID, "gguf: unsupported GGUF version: " + std::to_string(g->version) + " (supported: 2, 3)");
+    const uint64_t n_tensors = r.get<uint64_t>(), n_meta = r.get<uint64_t>();
+    if (!r.ok) return fail(FORGE_HIP_ERR_INVALID, "gguf: file shorter than its header");
+    for (uint64_t i = 0; i < n_meta; i++) {
+        std::string key;
+        if (!r.str(&key)) return fail(FORGE_HIP_ERR_INVALID, "gguf: file ends inside the metadata");
+        if (!valid_utf8(key)) return fail(FORGE_HIP_ERR_INVALID, "gguf: invalid UTF-8 in string");
+        const uint32_t type = r.get<uint32_t>();
+        if (!r.ok) return fail(FORGE_HIP_ERR_INVALID, "gguf: file ends inside the metadata");
+        MetaValue v;
+        const int32_t rc = read_value(r, type, &v, 0);
+        if (rc) return rc;
+        g->meta[key] = std::move(v);                        // a repeated key keeps the last value (HashMap::insert)
+    }
+    for (uint64_t i = 0; i < n_tensors; i++) {
+        TensorInfo t;
+        if (!r.str(&t.name)) return fail(FORGE_HIP_ERR_INVALID, "gguf: file ends inside the tensor descriptors");
+        if (!valid_utf8(t.name)) return fail(FORGE_HIP_ERR_INVALID, "gguf: invalid UTF-8 in string");
+        t.n_dims = r.get<uint32_t>();
+        if (r.ok && t.n_dims > 4)
+            return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor dimension count " + std::to_string(t.n_dims) + " exceeds maximum (4)");
+        for (uint32_t d = 0; d < t.n_dims; d++) t.dims[d] = r.get<uint64_t>();
+        t.type = r.get<uint32_t>();
+        t.offset = r.get<uint64_t>();
+        if (!r.ok) return fail(FORGE_HIP_ERR_INVALID, "gguf: file ends inside the tensor descriptors");
+        uint32_t block, bytes;
+        if (!ggml_type_layout(t.type, &block, &bytes))
+            return fail(FORGE_HIP_ERR_INVALID, "gguf: unsupported GGML type ID: " + std::to_string(t.type));
+        g->tensors.push_back(std::move(t));
+    }
+    uint32_t al = 0;
+    g->alignment = g->get_u32("general.alignment", &al) ? al : DEFAULT_ALIGNMENT;
+    if (g->alignment == 0) return fail(FORGE_HIP_ERR_INVALID, "gguf: general.alignment is 0");
+    g->tensor_data_offset = (r.pos + g->alignment - 1) / g->alignment * g->alignment;
+    return FORGE_HIP_OK;
+}
+
+// ---- tensors -> blob --------------------------------------------------------------------------------------
+
+// GGUF name of a tensor the blob needs (inverse of gguf_name_to_hf, weight_loader.rs:400-447).
+std::string blk(uint32_t l, const char* suffix) { return "blk." + std::to_string(l) + "." + suffix; }
+
+struct Source {
+    const TensorInfo* t;
+    const uint8_t* bytes;
+};
+
+int32_t locate(const forge_hip_gguf* g, const std::string& name, uint64_t numel, Source* out) {
+    const TensorInfo* t = g->tensor(name);
+    if (!t) return fail(FORGE_HIP_ERR_INVALID, "gguf: weight not found: " + name);
+    if (t->numel() != numel)
+        return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor " + name + " has " + std::to_string(t->numel()) + " elements, the configuration needs " +
+                                               std::to_string(numel));
+    const uint64_t start = g->tensor_data_offset + t->offset, size = t->data_size();
+    if (start > g->nbytes || size > g->nbytes - start)
+        return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor " + name + " extends past end of file");      // weight_loader.rs:172-177
+    out->t = t;
+    out->bytes = g->data + start;
+    return FORGE_HIP_OK;
+}
+
+// f32 values of a tensor (weight_loader.rs:809-855 for the dense types, :860-926 for the two block formats).
+int32_t to_f32(const Source& s, uint64_t numel, float* out) {
+    switch (s.t->type) {
+        case T_F32: memcpy(out, s.bytes, numel * 4); return FORGE_HIP_OK;
+        case T_F16:
+            for (uint64_t i = 0; i < numel; i++) out[i] = fh::f16_to_f32_host((uint16_t)(s.bytes[2 * i] | (s.bytes[2 * i + 1] << 8)));
+            return FORGE_HIP_OK;
+        case T_BF16:
+            for (uint64_t i = 0; i < numel; i++) {
+                const uint32_t b = ((uint32_t)(s.bytes[2 * i] | (s.bytes[2 * i + 1] << 8))) << 16;
+                memcpy(out + i, &b, 4);
+            }
+            return FORGE_HIP_OK;
+        case T_Q8_0: fh::dequant_host(FORGE_HIP_Q8_0, s.bytes, numel, out); return FORGE_HIP_OK;
+        case T_Q4_0: fh::dequant_host(FORGE_HIP_Q4_0, s.bytes, numel, out); return FORGE_HIP_OK;
+        default:
+            return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor " + s.t->name + " has GGML type " + std::to_string(s.t->type) +
+                                                   "; this library reads F32, F16, BF16, Q8_0 and Q4_0 tensors");
+    }
+}
+
+uint64_t qbytes(uint32_t wdtype, uint64_t numel) { return numel / 32 * (wdtype == FORGE_HIP_Q8_0 ? 34 : 18); }
+
+// A projection matrix in the blob's format: the file's bytes when it already has that format, otherwise its values
+// quantised again with the reference's weight quantiser (weight_loader.rs:1454-1544).
+int32_t write_quantised(const forge_hip_gguf* g, const std::string& name, uint32_t wdtype, uint64_t numel, uint8_t* out) {
+    Source s;
+    int32_t rc = locate(g, name, numel, &s);
+    if (rc) return rc;
+    if (s.t->type == wdtype) { memcpy(out, s.bytes, qbytes(wdtype, numel)); return FORGE_HIP_OK; }
+    std::vector<float> v(numel);
+    rc = to_f32(s, numel, v.data());
+    if (rc) return rc;
+    fh::quantize_host(wdtype, v.data(), numel, out);
+    return FORGE_HIP_OK;
+}
+
+int32_t write_f32(const forge_hip_gguf* g, const std::string& name, uint64_t numel, uint8_t* out) {
+    Source s;
+    const int32_t rc = locate(g, name, numel, &s);
+    if (rc) return rc;
+    return to_f32(s, numel, reinterpret_cast<float*>(out));
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t forge_hip_gguf_parse(const uint8_t* data_host, uint64_t nbytes, forge_hip_gguf** out) {
+    FH_CHECK(out, "gguf_parse: null out");
+    *out = nullptr;
+    FH_CHECK(data_host || nbytes == 0, "gguf_parse: null data");
+    std::unique_ptr<forge_hip_gguf> g(new forge_hip_gguf());
+    g->data = data_host;
+    g->nbytes = nbytes;
+    const int32_t rc = parse_into(g.get());
+    if (rc) return rc;
+    *out = g.release();
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_gguf_open(const char* path, forge_hip_gguf** out) {
+    FH_CHECK(out, "gguf_open: null out");
+    *out = nullptr;
+    FH_CHECK(path, "gguf_open: null path");
+    const int fd = open(path, O_RDONLY);
+    if (fd < 0) return fh::fail(FORGE_HIP_ERR_INVALID, std::string("gguf_open: cannot open ") + path + ": " + strerror(errno));
+    struct stat st;
+    if (fstat(fd, &st) != 0 || st.st_size <= 0) {
+        close(fd);
+        return fh::fail(FORGE_HIP_ERR_INVALID, std::string("gguf_open: cannot read ") + path);
+    }
+    void* map = mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
+    close(fd);
+    if (map == MAP_FAILED) return fh::fail(FORGE_HIP_ERR_INVALID, std::string("gguf_open: cannot map ") + path + ": " + strerror(errno));
+    std::unique_ptr<forge_hip_gguf> g(new forge_hip_gguf());
+    g->map = map;
+    g->map_len = (uint64_t)st.st_size;
+    g->data = reinterpret_cast<const uint8_t*>(map);
+    g->nbytes = g->map_len;
+    const int32_t rc = parse_into(g.get());
+    if (rc) return rc;
+    *out = g.release();
+    return FORGE_HIP_OK;
+}
+
+void forge_hip_gguf_close(forge_hip_gguf* g) { delete g; }
+
+uint32_t forge_hip_gguf_version(const forge_hip_gguf* g) { return g ? g->version : 0; }
+uint64_t forge_hip_gguf_alignment(const forge_hip_gguf* g) { return g ? g->alignment : 0; }
+uint64_t forge_hip_gguf_tensor_data_offset(const forge_hip_gguf* g) { return g ? g->tensor_data_offset : 0; }
+uint64_t forge_hip_gguf_tensor_count(const forge_hip_gguf* g) { return g ? g->tensors.size() : 0; }
+uint64_t forge_hip_gguf_metadata_count(const forge_hip_gguf* g) { return g ? g->meta.size() : 0; }
+
+int32_t forge_hip_gguf_tensor(const forge_hip_gguf* g, uint64_t index, const char** name, uint32_t* n_dims, uint64_t* dims4,
+                              uint32_t* ggml_type, uint64_t* offset, uint64_t* data_size) {
+    FH_CHECK(g, "gguf_tensor: null handle");
+    FH_CHECK(index < g->tensors.size(), "gguf_tensor: index out of range");
+    const TensorInfo& t = g->tensors[index];
+    if (name) *name = t.name.c_str();
+    if (n_dims) *n_dims = t.n_dims;
+    if (dims4) for (int i = 0; i < 4; i++) dims4[i] = t.dims[i];
+    if (ggml_type) *ggml_type = t.type;
+    if (offset) *offset = t.offset;
+    if (data_size) *data_size = t.data_size();
+    return FORGE_HIP_OK;
+}
+
+int64_t forge_hip_gguf_find_tensor(const forge_hip_gguf* g, const char* name) {
+    if (!g || !name) return -1;
+    for (size_t i = 0; i < g->tensors.size(); i++)
+        if (g->tensors[i].name == name) return (int64_t)i;
+    return -1;
+}
+
+int32_t forge_hip_gguf_meta(const forge_hip_gguf* g, const char* key, uint32_t* type, uint64_t* bits, const char** str,
+                            uint32_t* elem_type, uint64_t* count) {
+    FH_CHECK(g && key, "gguf_meta: null argument");
+    const MetaValue* v = g->find(key);
+    if (!v) return fh::fail(FORGE_HIP_ERR_INVALID, std::string("gguf_meta: no such key: ") + key);
+    if (type) *type = v->type;
+    if (bits) *bits = v->bits;
+    if (str) *str = v->type == 8 ? v->str.c_str() : nullptr;
+    if (elem_type) *elem_type = v->elem_type;
+    if (count) *count = v->count;
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_t flags, forge_hip_config* out) {
+    FH_CHECK(g && out, "gguf_config: null argument");
+    const MetaValue* arch_v = g->find("general.architecture");
+    const std::string arch = arch_v && arch_v->type == 8 ? arch_v->str : "unknown";
+    // The kernels here cover the plain Llama layer: no QKV bias (qwen2), no GeLU or embedding scale (gemma), no fused
+    // QKV (phi3).  Mistral is that layer plus an optional sliding window.
+    if (arch != "llama" && arch != "mistral") return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: unsupported GGUF architecture: " + arch);
+    const std::string p = arch + ".";
+    uint32_t hidden = 0, layers = 0, heads = 0, kv_heads = 0, inter = 0;
+    g->get_u32(p + "embedding_length", &hidden);
+    g->get_u32(p + "block_count", &layers);
+    g->get_u32(p + "attention.head_count", &heads);
+    if (!g->get_u32(p + "attention.head_count_kv", &kv_heads)) kv_heads = heads;
+    if (hidden == 0 || layers == 0 || heads == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: could not extract model config from GGUF metadata");
+    if (!g->get_u32(p + "feed_forward_length", &inter)) inter = hidden * 4;
+    uint64_t vocab = 32000, ctx = 2048;
+    const MetaValue* tokens = g->find("tokenizer.ggml.tokens");
+    if (tokens && tokens->type == 9) vocab = tokens->count;
+    else g->get_u64(p + "vocab_size", &vocab);
+    g->get_u64(p + "context_length", &ctx);
+    float eps = 1e-5f, theta = 10000.0f;
+    g->get_f32(p + "attention.layer_norm_rms_epsilon", &eps);
+    g->get_f32(p + "rope.freq_base", &theta);
+    uint32_t window = 0;
+    const bool has_window = g->get_u32(p + "attention.sliding_window", &window);
+
+    // majority vote over the projection tensors (main.rs:479-555)
+    uint64_t q8 = 0, q4 = 0, q4k = 0, f16 = 0, f32 = 0;
+    for (const auto& t : g->tensors) {
+        const std::string& n = t.name;
+        const bool proj = n.find(".weight") != std::string::npos && n.find("token_embd") == std::string::npos &&
+                          n.find("output.weight") == std::string::npos && n.find("_norm") == std::string::npos;
+        if (!proj) continue;
+        switch (t.type) {
+            case T_Q8_0: q8++; break;
+            case T_Q4_0: q4++; break;
+            case 12: q4k++; break;
+            case T_F16: case T_BF16: f16++; break;
+            case T_F32: f32++; break;
+            case 3: case 20: case 23: case 6: case 7: case 9: case 10: case 11: case 13: case 14: case 15: case 16: case 17: case 22:
+            case 18: case 21: case 19: case 29: q8++; break;
+            default: break;
+        }
+    }
+    const uint64_t total = q8 + q4 + q4k + f16 + f32;
+    uint32_t wdtype = 0;
+    if (total && q4k <= total / 2) {
+        if (q8 > total / 2) wdtype = FORGE_HIP_Q8_0;
+        else if (q4 > total / 2) wdtype = FORGE_HIP_Q4_0;
+    }
+    if (!wdtype) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: the projection weights are neither mostly Q8_0 nor mostly Q4_0");
+    // lm_head: the type of output.weight after loading (main.rs:567-581, gguf.rs:168-205); without that tensor the
+    // embedding table serves, converted to the projections' format
+    uint32_t lm = wdtype;
+    const TensorInfo* ot = g->tensor("output.weight");
+    if (!ot) ot = g->tensor("lm_head.weight");
+    if (ot) {
+        if (ot->type == T_Q4_0) lm = FORGE_HIP_Q4_0;
+        else if (ot->type == T_Q8_0) lm = FORGE_HIP_Q8_0;
+        else if (ot->type == T_F32 || ot->type == T_F16 || ot->type == T_BF16) lm = wdtype;   // dense: quantised like the projections
+        else return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: output.weight has GGML type " + std::to_string(ot->type) +
+                                                       "; this library reads F32, F16, BF16, Q8_0 and Q4_0 tensors");
+    }
+    const uint64_t seq = max_seq ? max_seq : ctx;
+    if (has_window && window < seq)
+        return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: sliding-window attention (window " + std::to_string(window) + ") is not supported for max_seq " +
+                                                   std::to_string(seq));
+    FH_CHECK(vocab <= 0xFFFFFFFFull && seq <= 0xFFFFFFFFull, "gguf: vocabulary or context length out of range");
+    forge_hip_config c{};
+    c.hidden = hidden; c.inter = inter; c.layers = layers; c.heads = heads; c.kv_heads = kv_heads;
+    c.head_dim = hidden / heads;                     // main.rs:731
+    c.vocab = (uint32_t)vocab; c.max_seq = (uint32_t)seq;
+    c.rms_eps = eps; c.rope_theta = theta;
+    c.wdtype = wdtype; c.lm_head_dtype = lm; c.flags = flags;
+    *out = c;
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_gguf_export_weights(const forge_hip_gguf* g, const forge_hip_config* c, uint8_t* out_host, uint64_t nbytes) {
+    FH_CHECK(g && c && out_host, "gguf_export_weights: null argument");
+    FH_CHECK(c->wdtype == FORGE_HIP_Q8_0 || c->wdtype == FORGE_HIP_Q4_0, "gguf_export_weights: wdtype must be Q8_0 or Q4_0");
+    FH_CHECK(c->lm_head_dtype == FORGE_HIP_Q8_0 || c->lm_head_dtype == FORGE_HIP_Q4_0, "gguf_export_weights: lm_head_dtype must be Q8_0 or Q4_0");
+    FH_CHECK(c->hidden % 32 == 0 && c->inter % 32 == 0 && (c->heads * c->head_dim) % 32 == 0, "gguf_export_weights: row lengths must be multiples of 32");
+    const uint64_t need = forge_hip_weights_nbytes(c);
+    if (nbytes != need)
+        return fh::fail(FORGE_HIP_ERR_BLOB_SIZE, "gguf_export_weights: buffer is " + std::to_string(nbytes) + " bytes, config needs " + std::to_string(need));
+    const uint64_t H = c->hidden, I = c->inter, QKS = (uint64_t)c->heads * c->head_dim, KV = (uint64_t)c->kv_heads * c->head_dim, V = c->vocab;
+    const uint32_t wt = c->wdtype;
+    uint8_t* p = out_host;
+    int32_t rc;
+#define FH_STEP(call, bytes) do { rc = (call); if (rc) return rc; p += (bytes); } while (0)
+    // the embedding table is always f32 in the blob (main.rs:2690-2722)
+    FH_STEP(write_f32(g, "token_embd.weight", V * H, p), V * H * 4);
+    for (uint32_t l = 0; l < c->layers; l++) {
+        FH_STEP(write_f32(g, blk(l, "attn_norm.weight"), H, p), H * 4);
+        FH_STEP(write_quantised(g, blk(l, "attn_q.weight"), wt, QKS * H, p), qbytes(wt, QKS * H));
+        FH_STEP(write_quantised(g, blk(l, "attn_k.weight"), wt, KV * H, p), qbytes(wt, KV * H));
+        FH_STEP(write_quantised(g, blk(l, "attn_v.weight"), wt, KV * H, p), qbytes(wt, KV * H));
+        FH_STEP(write_quantised(g, blk(l, "attn_output.weight"), wt, H * QKS, p), qbytes(wt, H * QKS));
+        FH_STEP(write_f32(g, blk(l, "ffn_norm.weight"), H, p), H * 4);
+        FH_STEP(write_quantised(g, blk(l, "ffn_gate.weight"), wt, I * H, p), qbytes(wt, I * H));
+        FH_STEP(write_quantised(g, blk(l, "ffn_up.weight"), wt, I * H, p), qbytes(wt, I * H));
+        FH_STEP(write_quantised(g, blk(l, "ffn_down.weight"), wt, H * I, p), qbytes(wt, H * I));
+    }
+    FH_STEP(write_f32(g, "output_norm.weight", H, p), H * 4);
+    // lm_head: output.weight, or the embedding table of a model with tied weights (main.rs:2632-2676)
+    const char* lm_name = g->tensor("output.weight") ? "output.weight" : g->tensor("lm_head.weight") ? "lm_head.weight" : "token_embd.weight";
+    FH_STEP(write_quantised(g, lm_name, c->lm_head_dtype, V * H, p), qbytes(c->lm_head_dtype, V * H));
+#undef FH_STEP
+    if ((uint64_t)(p - out_host) != need) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf_export_weights: internal size mismatch");
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_model_create_from_gguf(const char* path, uint32_t max_seq, uint32_t flags, forge_hip_model** out) {
+    FH_CHECK(out, "model_create_from_gguf: null out");
+    *out = nullptr;
+    forge_hip_gguf* g = nullptr;
+    int32_t rc = forge_hip_gguf_open(path, &g);
+    if (rc) return rc;
+    std::unique_ptr<forge_hip_gguf> hold(g);
+    forge_hip_config c;
+    rc = forge_hip_gguf_config(g, max_seq, flags, &c);
+    if (rc) return rc;
+    const uint64_t n = forge_hip_weights_nbytes(&c);
+    std::unique_ptr<uint8_t[]> blob(new (std::nothrow) uint8_t[n]);
+    if (!blob) return fh::fail(FORGE_HIP_ERR_INVALID, "model_create_from_gguf: out of host memory for " + std::to_string(n) + " bytes");
+    rc = forge_hip_gguf_export_weights(g, &c, blob.get(), n);
+    if (rc) return rc;
+    return forge_hip_model_create(&c, blob.get(), n, out);
+}
+
+}  // extern "C"

@@ -28,6 +28,26 @@ class HipModel:
         self._h = h
         self.vocab = int(config["vocab"])
 
+    @classmethod
+    def from_gguf(cls, path: str, max_seq: int = 0, flags: int = 0):
+        """Model straight from a GGUF file: what the reference does with `forge export-weights` + `Model::new`
+        (crates/forgellm-cli/src/main.rs:2585-2757).  max_seq = 0 takes the file's context length."""
+        from . import check, lib
+        from .gguf import GgufFile, _declare
+        L = lib()
+        _declare(L)
+        g = GgufFile(path)
+        cfg = g.config(max_seq, flags)
+        g.close()
+        self = cls.__new__(cls)
+        self._lib, self._check = L, check
+        self.config = cfg
+        h = C.c_void_p()
+        check(L.forge_hip_model_create_from_gguf(path.encode(), max_seq, flags, C.byref(h)))
+        self._h = h
+        self.vocab = int(cfg["vocab"])
+        return self
+
     # -- MetalModel::forward / model::forward
     def forward(self, token_id: int) -> np.ndarray:
         out = np.empty(self.vocab, np.float32)

@@ -191,6 +191,54 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
 /* argmax (project.rs:501-503): index of the LAST maximum of n floats -> *out_dev (uint32). */
 int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void* stream);
 
+/* ---------------- GGUF input (host code; no GPU needed except for the last call) ----------------
+ * The reference reads a model from a GGUF file in three steps: gguf::parse (crates/forgellm-frontend/src/gguf.rs:484-551),
+ * load_config (crates/forgellm-cli/src/main.rs:700-830) and `forge export-weights` (main.rs:2585-2757, tensor names
+ * mapped by weight_loader.rs:400-447), whose output file is the blob forge_hip_model_create takes.  These entry points are
+ * those three steps.  Supported: architectures "llama" and "mistral" (without a sliding window shorter than max_seq);
+ * tensors of GGML type F32, F16, BF16, Q8_0 or Q4_0; projections mostly Q8_0 or mostly Q4_0 (the reference's majority vote). */
+typedef struct forge_hip_gguf forge_hip_gguf;
+
+/* gguf::parse over a file (memory-mapped until close) or over bytes the caller keeps alive until close.  Failures are
+ * FORGE_HIP_ERR_INVALID with the reference's GGUFError text (invalid magic, unsupported version, unsupported GGML
+ * type / metadata value type, invalid UTF-8, more than 4 dimensions) or a message saying where the file ends early. */
+int32_t forge_hip_gguf_open(const char* path, forge_hip_gguf** out);
+int32_t forge_hip_gguf_parse(const uint8_t* data_host, uint64_t nbytes, forge_hip_gguf** out);
+void forge_hip_gguf_close(forge_hip_gguf* g);
+
+/* Fields of GGUFFile (gguf.rs:287-297). */
+uint32_t forge_hip_gguf_version(const forge_hip_gguf* g);
+uint64_t forge_hip_gguf_alignment(const forge_hip_gguf* g);
+uint64_t forge_hip_gguf_tensor_data_offset(const forge_hip_gguf* g);
+uint64_t forge_hip_gguf_tensor_count(const forge_hip_gguf* g);
+uint64_t forge_hip_gguf_metadata_count(const forge_hip_gguf* g);
+/* GGUFTensorInfo (gguf.rs:262-285) of tensor `index`; any output pointer may be NULL.  `name` stays valid until close;
+ * dims4 receives 4 values (unused ones 0); data_size = ceil(numel / block) * bytes per block. */
+int32_t forge_hip_gguf_tensor(const forge_hip_gguf* g, uint64_t index, const char** name, uint32_t* n_dims, uint64_t* dims4,
+                              uint32_t* ggml_type, uint64_t* offset, uint64_t* data_size);
+/* GGUFFile::tensor (gguf.rs:338-340): index of the tensor of that name, or -1. */
+int64_t forge_hip_gguf_find_tensor(const forge_hip_gguf* g, const char* name);
+/* One metadata value: its GGUF type id (0..12); `bits` = the bytes of a scalar, little endian, zero-extended (a bool is 0 or
+ * 1); `str` for type 8 (else NULL); element type and element count for type 9 (array elements are not kept).
+ * Unknown key: FORGE_HIP_ERR_INVALID. */
+int32_t forge_hip_gguf_meta(const forge_hip_gguf* g, const char* key, uint32_t* type, uint64_t* bits, const char** str,
+                            uint32_t* elem_type, uint64_t* count);
+
+/* load_config (main.rs:700-830): `<arch>.embedding_length`, `.block_count`, `.attention.head_count`, `.attention.head_count_kv`
+ * (default: head_count), `.feed_forward_length` (4 x hidden), vocabulary = length of `tokenizer.ggml.tokens`, else
+ * `<arch>.vocab_size`, else 32000; `.context_length` (2048), `.attention.layer_norm_rms_epsilon` (1e-5), `.rope.freq_base`
+ * (10000); head_dim = hidden / heads; weight format by majority vote over the projection tensors; lm_head format from
+ * `output.weight` (absent: tied to the embedding, stored in the projections' format).  max_seq = 0 takes the file's context
+ * length. */
+int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_t flags, forge_hip_config* out);
+/* `forge export-weights` (main.rs:2585-2757) into the caller's buffer of exactly forge_hip_weights_nbytes(cfg) bytes:
+ * f32 embedding table, per layer attn_norm | q | k | v | o | ffn_norm | gate | up | down, final norm, lm_head.  A tensor
+ * stored in another format than the blob needs is converted with the reference's own routines (dequant
+ * weight_loader.rs:809-926, quantisers :1454-1544). */
+int32_t forge_hip_gguf_export_weights(const forge_hip_gguf* g, const forge_hip_config* cfg, uint8_t* out_host, uint64_t nbytes);
+/* open + config + export_weights + forge_hip_model_create. */
+int32_t forge_hip_model_create_from_gguf(const char* path, uint32_t max_seq, uint32_t flags, forge_hip_model** out);
+
 #ifdef __cplusplus
 }
 #endif

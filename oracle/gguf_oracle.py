@@ -1,0 +1,241 @@
+"""TEST INFRASTRUCTURE ONLY — CPU restatement of the reference's GGUF input path, used by tests/ as the checker of
+the library's reader.  Nothing the product ships imports this file.
+
+Follows, step by step:
+  parse            crates/forgellm-frontend/src/gguf.rs:484-551 (reader helpers :367-481)
+  GGMLType sizes   gguf.rs:207-258;  GGUFTensorInfo::data_size gguf.rs:278-284
+  load_config      crates/forgellm-cli/src/main.rs:700-830, dtype vote :479-555, lm_head dtype :567-581
+  tensor names     crates/forgellm-frontend/src/weight_loader.rs:400-447
+  export-weights   crates/forgellm-cli/src/main.rs:2585-2757 (blob order :2714-2757)
+  dense dequant    weight_loader.rs:827-855; Q8_0 / Q4_0 dequant and the weight quantisers come from forge_oracle.cpp
+
+Pinned by the reference's own unit tests for this path (gguf.rs:606-769: minimal v3 file, several tensors with
+metadata, version 2, bad magic, unsupported version, data sizes, alignment), restated as byte strings in
+tests/test_gguf.py.  Where a GGUF tensor is stored in another format than the blob needs, the reference's exporter
+writes bytes its own generated reader cannot consume (main.rs:2603-2626 handles only f32 -> Q4_0); this restatement
+converts with the reference's dequantisers and quantisers instead, and says so here: that conversion is parity
+unpinned (no reference test or fixture covers it).
+"""
+import struct
+
+import numpy as np
+
+MAGIC = 0x46554747
+DEFAULT_ALIGNMENT = 32
+
+# id: (elements per block, bytes per block), gguf.rs:207-258
+TYPE_LAYOUT = {0: (1, 4), 1: (1, 2), 2: (32, 18), 3: (32, 20), 6: (32, 22), 7: (32, 24), 8: (32, 34), 9: (32, 40), 10: (256, 84),
+               11: (256, 110), 12: (256, 144), 13: (256, 176), 14: (256, 210), 15: (256, 292), 16: (256, 66), 17: (256, 74),
+               18: (256, 98), 19: (256, 50), 20: (32, 18), 21: (256, 110), 22: (256, 82), 23: (32, 36), 24: (1, 1), 25: (1, 2),
+               26: (1, 4), 27: (1, 8), 28: (1, 8), 29: (256, 56), 30: (1, 2)}
+
+
+class GgufError(ValueError):
+    pass
+
+
+class _Reader:
+    def __init__(self, data):
+        self.d, self.pos = bytes(data), 0
+
+    def take(self, fmt):
+        n = struct.calcsize(fmt)
+        if self.pos + n > len(self.d):
+            raise GgufError("unexpected end of file")
+        v = struct.unpack_from(fmt, self.d, self.pos)[0]
+        self.pos += n
+        return v
+
+    def string(self):
+        n = self.take("<Q")
+        if self.pos + n > len(self.d):
+            raise GgufError("unexpected end of file")
+        raw = self.d[self.pos:self.pos + n]
+        self.pos += n
+        try:
+            return raw.decode("utf-8")
+        except UnicodeDecodeError:
+            raise GgufError("invalid UTF-8 in string")
+
+    def value(self, t):
+        fmts = {0: "<B", 1: "<b", 2: "<H", 3: "<h", 4: "<I", 5: "<i", 6: "<f", 10: "<Q", 11: "<q", 12: "<d"}
+        if t in fmts:
+            return (t, self.take(fmts[t]))
+        if t == 7:
+            return (t, self.take("<B") != 0)
+        if t == 8:
+            return (t, self.string())
+        if t == 9:
+            et = self.take("<I")
+            n = self.take("<Q")
+            return (t, (et, [self.value(et) for _ in range(n)]))
+        raise GgufError(f"unsupported metadata value type: {t}")
+
+
+def parse(data) -> dict:
+    r = _Reader(data)
+    magic = r.take("<I")
+    if magic != MAGIC:
+        raise GgufError(f"invalid GGUF magic number: got 0x{magic:08X}")
+    version = r.take("<I")
+    if version not in (2, 3):
+        raise GgufError(f"unsupported GGUF version: {version} (supported: 2, 3)")
+    n_tensors, n_meta = r.take("<Q"), r.take("<Q")
+    meta = {}
+    for _ in range(n_meta):
+        key = r.string()
+        meta[key] = r.value(r.take("<I"))
+    tensors = []
+    for _ in range(n_tensors):
+        name = r.string()
+        nd = r.take("<I")
+        if nd > 4:
+            raise GgufError(f"tensor dimension count {nd} exceeds maximum (4)")
+        dims = [r.take("<Q") for _ in range(nd)]
+        gtype = r.take("<I")
+        if gtype not in TYPE_LAYOUT:
+            raise GgufError(f"unsupported GGML type ID: {gtype}")
+        tensors.append({"name": name, "dimensions": dims, "ggml_type": gtype, "offset": r.take("<Q")})
+    al = meta.get("general.alignment")
+    alignment = al[1] if al is not None and al[0] == 4 else DEFAULT_ALIGNMENT
+    return {"version": version, "metadata": meta, "tensors": tensors, "alignment": alignment,
+            "tensor_data_offset": (r.pos + alignment - 1) // alignment * alignment}
+
+
+def numel(t) -> int:
+    n = 1
+    for d in t["dimensions"]:
+        n *= d
+    return n
+
+
+def data_size(t) -> int:
+    block, nbytes = TYPE_LAYOUT[t["ggml_type"]]
+    return (numel(t) + block - 1) // block * nbytes
+
+
+def _get(g, key, types):
+    v = g["metadata"].get(key)
+    return v[1] if v is not None and v[0] in types else None
+
+
+def config(g, max_seq=0, flags=0) -> dict:
+    arch = _get(g, "general.architecture", (8,)) or "unknown"
+    if arch not in ("llama", "mistral"):
+        raise GgufError(f"unsupported GGUF architecture: {arch}")
+    p = arch + "."
+    hidden = _get(g, p + "embedding_length", (4,)) or 0
+    layers = _get(g, p + "block_count", (4,)) or 0
+    heads = _get(g, p + "attention.head_count", (4,)) or 0
+    kv = _get(g, p + "attention.head_count_kv", (4,))
+    kv = heads if kv is None else kv
+    if hidden == 0 or layers == 0 or heads == 0:
+        raise GgufError("could not extract model config from GGUF metadata")
+    inter = _get(g, p + "feed_forward_length", (4,))
+    inter = hidden * 4 if inter is None else inter
+    tokens = g["metadata"].get("tokenizer.ggml.tokens")
+    if tokens is not None and tokens[0] == 9:
+        vocab = len(tokens[1][1])
+    else:
+        vocab = _get(g, p + "vocab_size", (10, 4))
+        vocab = 32000 if vocab is None else vocab
+    ctx = _get(g, p + "context_length", (10, 4))
+    ctx = 2048 if ctx is None else ctx
+    eps = _get(g, p + "attention.layer_norm_rms_epsilon", (6,))
+    theta = _get(g, p + "rope.freq_base", (6,))
+    q8 = q4 = q4k = f16 = f32 = 0
+    as_q8 = {3, 20, 23, 6, 7, 9, 10, 11, 13, 14, 15, 16, 17, 22, 18, 21, 19, 29}
+    for t in g["tensors"]:
+        n = t["name"]
+        if not (".weight" in n and "token_embd" not in n and "output.weight" not in n and "_norm" not in n):
+            continue
+        ty = t["ggml_type"]
+        if ty == 8 or ty in as_q8:
+            q8 += 1
+        elif ty == 2:
+            q4 += 1
+        elif ty == 12:
+            q4k += 1
+        elif ty in (1, 30):
+            f16 += 1
+        elif ty == 0:
+            f32 += 1
+    total = q8 + q4 + q4k + f16 + f32
+    if total == 0 or q4k > total // 2:
+        raise GgufError("projection weights are neither mostly Q8_0 nor mostly Q4_0")
+    if q8 > total // 2:
+        wd = 8
+    elif q4 > total // 2:
+        wd = 2
+    else:
+        raise GgufError("projection weights are neither mostly Q8_0 nor mostly Q4_0")
+    lm = wd
+    ot = next((t for t in g["tensors"] if t["name"] in ("output.weight", "lm_head.weight")), None)
+    if ot is not None:
+        if ot["ggml_type"] in (2, 8):
+            lm = ot["ggml_type"]
+        elif ot["ggml_type"] not in (0, 1, 30):
+            raise GgufError("output.weight has an unsupported GGML type")
+    seq = max_seq or ctx
+    window = _get(g, p + "attention.sliding_window", (4,))
+    if window is not None and window < seq:
+        raise GgufError("sliding-window attention is not supported")
+    f = np.float32
+    return {"hidden": hidden, "inter": inter, "layers": layers, "heads": heads, "kv_heads": kv, "head_dim": hidden // heads,
+            "vocab": vocab, "max_seq": seq, "rms_eps": float(f(1e-5) if eps is None else f(eps)),
+            "rope_theta": float(f(10000.0) if theta is None else f(theta)), "wdtype": wd, "lm_head_dtype": lm, "flags": flags}
+
+
+def _tensor_f32(oracle, g, data, t):
+    n = numel(t)
+    start = g["tensor_data_offset"] + t["offset"]
+    raw = np.frombuffer(data, np.uint8, data_size(t), start)
+    ty = t["ggml_type"]
+    if ty == 0:
+        return raw.view("<f4").copy()
+    if ty == 1:
+        return oracle.f16_to_f32(raw.view("<u2"))
+    if ty == 30:
+        return (raw.view("<u2").astype(np.uint32) << 16).view(np.float32)
+    if ty in (8, 2):
+        return oracle.dequant(ty, raw, n)
+    raise GgufError(f"tensor {t['name']}: unsupported GGML type {ty}")
+
+
+def export_weights(oracle, g, data, cfg) -> np.ndarray:
+    """The weights.bin bytes for `cfg` (main.rs:2714-2757).  `oracle` is the oracle.oracle module."""
+    data = bytes(data)
+    by_name = {t["name"]: t for t in g["tensors"]}
+
+    def find(name, n):
+        t = by_name.get(name)
+        if t is None:
+            raise GgufError(f"weight not found: {name}")
+        if numel(t) != n:
+            raise GgufError(f"tensor {name} has the wrong number of elements")
+        if g["tensor_data_offset"] + t["offset"] + data_size(t) > len(data):
+            raise GgufError(f"tensor {name} extends past end of file")
+        return t
+
+    def f32(name, n):
+        return _tensor_f32(oracle, g, data, find(name, n)).astype("<f4").view(np.uint8)
+
+    def quant(name, n, wd):
+        t = find(name, n)
+        if t["ggml_type"] == wd:
+            return np.frombuffer(data, np.uint8, data_size(t), g["tensor_data_offset"] + t["offset"])
+        return oracle.quantize_weights(wd, _tensor_f32(oracle, g, data, t))
+
+    H, I = cfg["hidden"], cfg["inter"]
+    QKS, KV, V = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"], cfg["vocab"]
+    wd = cfg["wdtype"]
+    parts = [f32("token_embd.weight", V * H)]
+    for l in range(cfg["layers"]):
+        b = f"blk.{l}."
+        parts += [f32(b + "attn_norm.weight", H), quant(b + "attn_q.weight", QKS * H, wd), quant(b + "attn_k.weight", KV * H, wd),
+                  quant(b + "attn_v.weight", KV * H, wd), quant(b + "attn_output.weight", H * QKS, wd), f32(b + "ffn_norm.weight", H),
+                  quant(b + "ffn_gate.weight", I * H, wd), quant(b + "ffn_up.weight", I * H, wd), quant(b + "ffn_down.weight", H * I, wd)]
+    parts.append(f32("output_norm.weight", H))
+    lm_name = "output.weight" if "output.weight" in by_name else "lm_head.weight" if "lm_head.weight" in by_name else "token_embd.weight"
+    parts.append(quant(lm_name, V * H, cfg["lm_head_dtype"]))
+    return np.concatenate([np.ascontiguousarray(p, np.uint8) for p in parts])

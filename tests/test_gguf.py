@@ -1,0 +1,343 @@
+"""GGUF input: the library's parser / config reader / weights exporter against the reference's own unit-test vectors
+(crates/forgellm-frontend/src/gguf.rs:606-769, restated as the byte strings those tests build), against the Python
+restatement in oracle/gguf_oracle.py, and through round trips of seeded synthetic models.  Host code only, except
+the last test, which loads a model from a GGUF file onto the GPU."""
+import struct
+
+import numpy as np
+import pytest
+
+Q8, Q4 = 8, 2
+
+
+@pytest.fixture(scope="module")
+def gg(fh):
+    return fh.gguf
+
+
+@pytest.fixture(scope="module")
+def go():
+    from oracle import gguf_oracle
+    return gguf_oracle
+
+
+def both(fh, go, data):
+    """Parse with the library and with the oracle; check that they agree on everything a GGUFFile holds."""
+    lib_file = fh.gguf.GgufFile(data)
+    ora = go.parse(data)
+    assert lib_file.version == ora["version"]
+    assert lib_file.alignment == ora["alignment"]
+    assert lib_file.tensor_data_offset == ora["tensor_data_offset"]
+    assert lib_file.metadata_count == len(ora["metadata"])
+    assert len(lib_file.tensors) == len(ora["tensors"])
+    for a, b in zip(lib_file.tensors, ora["tensors"]):
+        assert a["name"] == b["name"] and a["dimensions"] == b["dimensions"]
+        assert a["ggml_type"] == b["ggml_type"] and a["offset"] == b["offset"]
+        assert a["data_size"] == go.data_size(b)
+    for key, (vtype, value) in ora["metadata"].items():
+        got = lib_file.meta(key)
+        if vtype == 9:
+            assert got == (value[0], len(value[1])), key
+        elif vtype in (6, 12):
+            assert np.float64(got) == np.float64(value) or (np.isnan(got) and np.isnan(value)), key
+        else:
+            assert got == value, key
+    return lib_file, ora
+
+
+def err(fh, data):
+    with pytest.raises(fh.ForgeHipError) as e:
+        fh.gguf.GgufFile(data)
+    assert e.value.code == fh.ERR_INVALID
+    return str(e.value)
+
+
+# ---------------- the reference's unit tests (gguf.rs:606-769) ----------------
+def test_reference_parse_minimal_gguf_v3(fh, gg, go):
+    data = gg.write_gguf([("general.architecture", gg.STRING, "llama")], [("token_embd.weight", [32000, 2048], gg.F16, None)])
+    f, _ = both(fh, go, data)
+    assert f.version == 3
+    assert f.meta("general.architecture") == "llama"
+    assert len(f.tensors) == 1
+    assert f.tensors[0]["name"] == "token_embd.weight"
+    assert f.tensors[0]["dimensions"] == [32000, 2048]
+    assert f.tensors[0]["ggml_type"] == gg.F16
+
+
+def test_reference_parse_with_multiple_tensors(fh, gg, go):
+    # offsets as in the reference's test: 0, 4096, 8192 (descriptors only, no data section)
+    meta = [("general.architecture", gg.STRING, "llama"), ("llama.embedding_length", gg.U32, 2048),
+            ("llama.attention.layer_norm_rms_epsilon", gg.FLOAT32, 1e-5)]
+    head = struct.pack("<IIQQ", gg.MAGIC, 3, 3, 3)
+    for k, t, v in meta:
+        head += struct.pack("<Q", len(k)) + k.encode() + struct.pack("<I", t) + gg.encode_value(t, v)
+    for name, dims, ty, off in [("token_embd.weight", [32000, 2048], 1, 0), ("blk.0.attn_q.weight", [2048, 2048], 8, 4096),
+                                ("blk.0.ffn_gate.weight", [5632, 2048], 2, 8192)]:
+        head += struct.pack("<Q", len(name)) + name.encode() + struct.pack("<I", len(dims))
+        head += b"".join(struct.pack("<Q", d) for d in dims) + struct.pack("<IQ", ty, off)
+    f, _ = both(fh, go, head)
+    assert len(f.tensors) == 3
+    assert f.meta("llama.embedding_length") == 2048
+    assert f.meta("llama.attention.layer_norm_rms_epsilon") == float(np.float32(1e-5))
+    q = f.tensor("blk.0.attn_q.weight")
+    assert q["ggml_type"] == Q8 and int(np.prod(q["dimensions"])) == 2048 * 2048 and q["offset"] == 4096
+    assert f.tensor("blk.0.ffn_gate.weight")["offset"] == 8192
+    assert f.tensor("nope") is None
+
+
+def test_reference_parse_v2(fh, gg, go):
+    f, _ = both(fh, go, gg.write_gguf([], [], version=2))
+    assert f.version == 2 and f.tensors == []
+
+
+def test_reference_reject_invalid_magic(fh, go):
+    data = bytearray(32)
+    data[0:4] = struct.pack("<I", 0xDEADBEEF)
+    assert "invalid GGUF magic number: got 0xDEADBEEF" in err(fh, bytes(data))
+    with pytest.raises(go.GgufError, match="0xDEADBEEF"):
+        go.parse(bytes(data))
+
+
+def test_reference_reject_unsupported_version(fh, gg, go):
+    data = struct.pack("<IIQQ", gg.MAGIC, 99, 0, 0)
+    assert "unsupported GGUF version: 99 (supported: 2, 3)" in err(fh, data)
+    with pytest.raises(go.GgufError, match="99"):
+        go.parse(data)
+
+
+def test_reference_tensor_data_size(fh, gg, go):
+    data = gg.write_gguf([], [("test", [32000, 2048], gg.F16, None), ("test2", [2048, 2048], gg.Q4_0, None)])
+    f, _ = both(fh, go, data)
+    assert f.tensors[0]["data_size"] == 32000 * 2048 * 2
+    assert f.tensors[1]["data_size"] == (2048 * 2048 // 32) * 18
+
+
+def test_reference_alignment_calculation(fh, gg, go):
+    f, _ = both(fh, go, gg.write_gguf([], []))
+    assert f.alignment == 32 and f.tensor_data_offset % 32 == 0
+    # 24 header bytes round up to one alignment unit
+    assert f.tensor_data_offset == 32
+
+
+# ---------------- beyond the reference's tests ----------------
+def test_every_metadata_type_and_nested_arrays(fh, gg, go):
+    meta = [("a.u8", gg.U8, 200), ("a.i8", gg.I8, -100), ("a.u16", gg.U16, 60000), ("a.i16", gg.I16, -30000),
+            ("a.u32", gg.U32, 4000000000), ("a.i32", gg.I32, -2000000000), ("a.f32", gg.FLOAT32, 0.1), ("a.true", gg.BOOL, 1),
+            ("a.false", gg.BOOL, 0), ("a.str", gg.STRING, "héllo wörld ✓"), ("a.empty", gg.STRING, ""),
+            ("a.u64", gg.U64, 2 ** 63 + 5), ("a.i64", gg.I64, -2 ** 62), ("a.f64", gg.FLOAT64, 1e300),
+            ("arr.u32", gg.ARRAY, (gg.U32, [1, 2, 3])), ("arr.str", gg.ARRAY, (gg.STRING, ["a", "bc", ""])),
+            ("arr.empty", gg.ARRAY, (gg.FLOAT64, [])),
+            ("arr.nested", gg.ARRAY, (gg.ARRAY, [(gg.U8, [1, 2]), (gg.STRING, ["x"]), (gg.ARRAY, [(gg.I16, [-1])])])),
+            ("general.alignment", gg.U32, 64)]
+    data = gg.write_gguf(meta, [("t", [3], gg.F32, np.arange(3, dtype=np.float32))], alignment=64)
+    f, o = both(fh, go, data)
+    assert f.alignment == 64 and f.tensor_data_offset % 64 == 0
+    assert f.meta("a.i8") == -100 and f.meta("a.i64") == -2 ** 62 and f.meta("a.u64") == 2 ** 63 + 5
+    assert f.meta("a.true") is True and f.meta("a.false") is False
+    assert f.meta("a.str") == "héllo wörld ✓"
+    assert f.meta("arr.nested") == (gg.ARRAY, 3)
+    assert f.meta("missing") is None
+    # the data really sits at tensor_data_offset
+    assert np.frombuffer(data, np.float32, 3, f.tensor_data_offset).tolist() == [0.0, 1.0, 2.0]
+
+
+def test_a_repeated_key_keeps_the_last_value(fh, gg, go):
+    f, _ = both(fh, go, gg.write_gguf([("k", gg.U32, 1), ("k", gg.U32, 2)], []))
+    assert f.meta("k") == 2 and f.metadata_count == 1
+
+
+def test_parse_errors(fh, gg, go):
+    good = gg.write_gguf([("general.architecture", gg.STRING, "llama")], [("t", [4, 4], gg.F32, None)])
+    assert "unsupported GGML type ID: 5" in err(fh, gg.write_gguf([], [("t", [4], 5, None)]))
+    assert "unsupported GGML type ID: 31" in err(fh, gg.write_gguf([], [("t", [4], 31, None)]))
+    assert "tensor dimension count 5 exceeds maximum (4)" in err(fh, gg.write_gguf([], [("t", [1, 1, 1, 1, 1], gg.F32, None)]))
+    bad_type = struct.pack("<IIQQ", gg.MAGIC, 3, 0, 1) + struct.pack("<Q", 1) + b"k" + struct.pack("<I", 13)
+    assert "unsupported metadata value type: 13" in err(fh, bad_type)
+    bad_utf8 = struct.pack("<IIQQ", gg.MAGIC, 3, 0, 1) + struct.pack("<Q", 1) + b"k" + struct.pack("<I", 8) + struct.pack("<Q", 2) + b"\xff\xfe"
+    assert "invalid UTF-8" in err(fh, bad_utf8)
+    with pytest.raises(go.GgufError, match="UTF-8"):
+        go.parse(bad_utf8)
+    # every proper prefix of a good file is refused (never read past the end), the whole file is accepted
+    for cut in range(len(good)):
+        err(fh, good[:cut])
+        with pytest.raises(go.GgufError):
+            go.parse(good[:cut])
+    both(fh, go, good)
+    # a string length that points far past the end
+    huge = struct.pack("<IIQQ", gg.MAGIC, 3, 0, 1) + struct.pack("<Q", 2 ** 62)
+    err(fh, huge)
+    # an array count that points far past the end
+    huge_arr = struct.pack("<IIQQ", gg.MAGIC, 3, 0, 1) + struct.pack("<Q", 1) + b"k" + struct.pack("<IIQ", 9, 4, 2 ** 61)
+    err(fh, huge_arr)
+
+
+@pytest.mark.parametrize("wd", [Q8, Q4])
+@pytest.mark.parametrize("tied", [True, False])
+def test_synthetic_model_round_trip(fh, gg, go, oracle, wd, tied, tmp_path):
+    """blob -> GGUF file -> (library) config + blob: identical bytes, identical configuration; same through the oracle."""
+    cfg = fh.synth.tiny(wd, max_seq=640)
+    blob = fh.synth.make_weights_blob(cfg, seed=11)
+    path = str(tmp_path / "m.gguf")
+    data = gg.model_to_gguf(cfg, blob, tied=tied, path=path, tokens=tied)
+    for source in (path, data):
+        f = gg.GgufFile(source)
+        got = f.config()
+        assert {k: got[k] for k in cfg if k not in ("rms_eps", "rope_theta")} == {k: cfg[k] for k in cfg if k not in ("rms_eps", "rope_theta")}
+        assert np.float32(got["rms_eps"]) == np.float32(cfg["rms_eps"]) and np.float32(got["rope_theta"]) == np.float32(cfg["rope_theta"])
+        out = f.export_weights(got)
+        assert out.size == blob.size and np.array_equal(out, blob)
+        assert f.config(max_seq=128, flags=1)["max_seq"] == 128 and f.config(max_seq=128, flags=1)["flags"] == 1
+        f.close()
+    o = go.parse(data)
+    ocfg = go.config(o)
+    assert ocfg == got
+    assert np.array_equal(go.export_weights(oracle, o, data, ocfg), blob)
+
+
+def test_tensors_in_other_formats_are_converted_like_the_oracle_does(fh, gg, go, oracle):
+    """A Q8_0 model whose norms are F16, one projection F32, one BF16, one Q4_0, with an F16 embedding and a Q4_0 output
+    matrix: the exporter dequantises / requantises with the reference's routines; library == oracle, byte for byte."""
+    cfg = fh.synth.tiny(Q8, max_seq=640)
+    blob = fh.synth.make_weights_blob(cfg, seed=12)
+    t = gg.split_blob(cfg, blob)
+    H, V = cfg["hidden"], cfg["vocab"]
+
+    def f32_of(name):
+        dims, ty, raw = t[name]
+        n = int(np.prod(dims))
+        return raw.view(np.float32).copy() if ty == gg.F32 else oracle.dequant(ty, raw, n)
+
+    def as_f16(x):
+        return oracle.f32_to_f16(x).astype("<u2").view(np.uint8)
+
+    t["blk.0.attn_norm.weight"] = ([H], gg.F16, as_f16(f32_of("blk.0.attn_norm.weight")))
+    t["blk.0.attn_q.weight"] = (t["blk.0.attn_q.weight"][0], gg.F32, f32_of("blk.0.attn_q.weight").view(np.uint8))
+    bf = (f32_of("blk.1.ffn_up.weight").view(np.uint32) >> 16).astype("<u2").view(np.uint8)
+    t["blk.1.ffn_up.weight"] = (t["blk.1.ffn_up.weight"][0], gg.BF16, bf)
+    t["blk.1.attn_v.weight"] = (t["blk.1.attn_v.weight"][0], gg.Q4_0, oracle.quantize_weights(Q4, f32_of("blk.1.attn_v.weight")))
+    t["token_embd.weight"] = ([H, V], gg.F16, as_f16(f32_of("token_embd.weight")))
+    t["output.weight"] = ([H, V], gg.Q4_0, oracle.quantize_weights(Q4, f32_of("output.weight")))
+    meta = [("general.architecture", gg.STRING, "llama"), ("llama.embedding_length", gg.U32, H), ("llama.block_count", gg.U32, cfg["layers"]),
+            ("llama.attention.head_count", gg.U32, cfg["heads"]), ("llama.attention.head_count_kv", gg.U32, cfg["kv_heads"]),
+            ("llama.feed_forward_length", gg.U32, cfg["inter"]), ("llama.vocab_size", gg.U64, V), ("llama.context_length", gg.U64, 640),
+            ("llama.attention.layer_norm_rms_epsilon", gg.FLOAT32, cfg["rms_eps"]), ("llama.rope.freq_base", gg.FLOAT32, cfg["rope_theta"])]
+    data = gg.write_gguf(meta, [(n, d, g, b) for n, (d, g, b) in t.items()])
+    f = gg.GgufFile(data)
+    got = f.config()
+    assert got["wdtype"] == Q8 and got["lm_head_dtype"] == Q4 and got["vocab"] == V and got["max_seq"] == 640
+    o = go.parse(data)
+    assert go.config(o) == got
+    out = f.export_weights(got)
+    want = go.export_weights(oracle, o, data, got)
+    assert out.size == want.size and np.array_equal(out, want)
+    # untouched tensors came through verbatim
+    same = gg.split_blob(got, out)
+    for name in ("blk.0.attn_k.weight", "blk.1.ffn_down.weight", "output_norm.weight"):
+        assert np.array_equal(same[name][2], t[name][2])
+    # F32 -> Q8_0 of values that were Q8_0 to begin with reproduces the blocks' values
+    assert np.array_equal(oracle.dequant(Q8, same["blk.0.attn_q.weight"][2], H * cfg["heads"] * cfg["head_dim"]), f32_of("blk.0.attn_q.weight"))
+
+
+def test_config_defaults_and_refusals(fh, gg, go):
+    def make(meta, tensors=(("blk.0.attn_q.weight", [64, 64], gg.Q8_0, None),)):
+        return gg.write_gguf(meta, list(tensors))
+
+    base = [("general.architecture", gg.STRING, "llama"), ("llama.embedding_length", gg.U32, 64), ("llama.block_count", gg.U32, 1),
+            ("llama.attention.head_count", gg.U32, 1)]
+    f = gg.GgufFile(make(base))
+    c = f.config()
+    o = go.config(go.parse(make(base)))
+    assert c == o
+    # defaults of main.rs:716-757
+    assert (c["kv_heads"], c["inter"], c["vocab"], c["max_seq"], c["head_dim"]) == (1, 256, 32000, 2048, 64)
+    assert np.float32(c["rms_eps"]) == np.float32(1e-5) and c["rope_theta"] == 10000.0
+    assert c["wdtype"] == Q8 and c["lm_head_dtype"] == Q8
+
+    def refused(meta, tensors=None, text=""):
+        data = make(meta) if tensors is None else make(meta, tensors)
+        g = gg.GgufFile(data)
+        with pytest.raises(fh.ForgeHipError) as e:
+            g.config()
+        assert text in str(e.value)
+        with pytest.raises(go.GgufError):
+            go.config(go.parse(data))
+
+    refused([("general.architecture", gg.STRING, "qwen2")] + base[1:], text="unsupported GGUF architecture: qwen2")
+    refused(base[1:], text="unsupported GGUF architecture: unknown")
+    refused(base[:2], text="could not extract model config")
+    # get_u32 takes a Uint32 value only (gguf.rs:306-308): the same key as u64 does not count
+    refused([base[0], ("llama.embedding_length", gg.U64, 64)] + base[2:], text="could not extract model config")
+    refused(base, tensors=(("blk.0.attn_q.weight", [64, 64], gg.F16, None),), text="neither mostly Q8_0 nor mostly Q4_0")
+    refused(base, tensors=(("blk.0.attn_q.weight", [256, 64], 12, None),), text="neither mostly Q8_0 nor mostly Q4_0")
+    refused(base, tensors=(("blk.0.attn_q.weight", [64, 64], gg.Q8_0, None), ("output.weight", [256, 64], 14, None)), text="output.weight")
+    refused(base + [("llama.attention.sliding_window", gg.U32, 1024)], text="sliding-window")
+    # the vote: 2 x Q4_0 against 1 x Q8_0
+    vote = (("blk.0.attn_q.weight", [64, 64], gg.Q4_0, None), ("blk.0.attn_k.weight", [64, 64], gg.Q4_0, None),
+            ("blk.0.ffn_up.weight", [64, 64], gg.Q8_0, None), ("blk.0.attn_norm.weight", [64], gg.F32, None),
+            ("token_embd.weight", [64, 10], gg.F16, None))
+    assert gg.GgufFile(make(base, vote)).config()["wdtype"] == Q4
+
+
+def test_export_errors(fh, gg):
+    cfg = fh.synth.tiny(Q8, max_seq=640)
+    blob = fh.synth.make_weights_blob(cfg, seed=13)
+    t = gg.split_blob(cfg, blob)
+    meta = [("general.architecture", gg.STRING, "llama")]
+
+    def export(tensors, c=cfg):
+        f = gg.GgufFile(gg.write_gguf(meta, [(n, d, g, b) for n, (d, g, b) in tensors.items()]))
+        with pytest.raises(fh.ForgeHipError) as e:
+            f.export_weights(c)
+        return str(e.value)
+
+    missing = dict(t)
+    del missing["blk.1.ffn_gate.weight"]
+    assert "weight not found: blk.1.ffn_gate.weight" in export(missing)
+    wrong = dict(t)
+    wrong["blk.0.attn_k.weight"] = ([cfg["hidden"], 8], Q8, t["blk.0.attn_k.weight"][2][:8 * cfg["hidden"] // 32 * 34])
+    assert "blk.0.attn_k.weight has" in export(wrong)
+    kq = dict(t)
+    d = kq["blk.0.ffn_down.weight"][0]
+    kq["blk.0.ffn_down.weight"] = (d, 14, np.zeros(int(np.prod(d)) // 256 * 210, np.uint8))
+    assert "reads F32, F16, BF16, Q8_0 and Q4_0" in export(kq)
+    # a data section cut short: the last tensor extends past the end of the file
+    data = gg.write_gguf(meta, [(n, d, g, b) for n, (d, g, b) in t.items()])
+    f = gg.GgufFile(data[:-4096])
+    with pytest.raises(fh.ForgeHipError) as e:
+        f.export_weights(cfg)
+    assert "extends past end of file" in str(e.value)
+    # wrong buffer size
+    from ctypes import byref, c_void_p
+    f = gg.GgufFile(data)
+    c = fh.Config(**cfg)
+    out = np.empty(16, np.uint8)
+    assert fh.lib().forge_hip_gguf_export_weights(f._h, byref(c), out.ctypes.data_as(c_void_p), 16) == fh.ERR_BLOB_SIZE
+    with pytest.raises(fh.ForgeHipError):
+        gg.GgufFile("/nonexistent/dir/model.gguf")
+
+
+@pytest.mark.gpu
+def test_model_from_gguf_equals_model_from_blob(fh, gg, torch_gpu, tmp_path):
+    """forge_hip_model_create_from_gguf: same logits, same greedy tokens, same cache as the model built from the blob."""
+    for wd in (Q8, Q4):
+        cfg = fh.synth.tiny(wd, max_seq=640)
+        blob = fh.synth.make_weights_blob(cfg, seed=14)
+        path = str(tmp_path / f"m{wd}.gguf")
+        gg.model_to_gguf(cfg, blob, tied=True, path=path)
+        a, b = fh.HipModel(cfg, blob), fh.HipModel.from_gguf(path)
+        assert b.config == {**cfg, "rms_eps": b.config["rms_eps"], "rope_theta": b.config["rope_theta"]}
+        prompt = fh.synth.uniform_ids(5, 40, cfg["vocab"])
+        la, lb = a.forward_prefill(prompt), b.forward_prefill(prompt)
+        assert np.array_equal(la.view(np.uint32), lb.view(np.uint32))
+        tok = fh.ops.argmax_host(la)
+        for _ in range(6):
+            ta, tb = a.forward_greedy(tok), b.forward_greedy(tok)
+            assert ta == tb
+            tok = ta
+        assert np.array_equal(a.read_kv(1, 0), b.read_kv(1, 0))
+        a.close(); b.close()
+        # a smaller cache than the file's context length, and the exact mode
+        c = fh.HipModel.from_gguf(path, max_seq=600, flags=fh.FLAG_EXACT)
+        assert c.config["max_seq"] == 600 and c.config["flags"] == fh.FLAG_EXACT
+        c.forward_prefill(prompt)
+        c.close()
