@@ -36,7 +36,7 @@ EXPORTS = [
     "forge_hip_gguf_open", "forge_hip_gguf_parse", "forge_hip_gguf_close", "forge_hip_gguf_version", "forge_hip_gguf_alignment",
     "forge_hip_gguf_tensor_data_offset", "forge_hip_gguf_tensor_count", "forge_hip_gguf_metadata_count", "forge_hip_gguf_tensor",
     "forge_hip_gguf_find_tensor", "forge_hip_gguf_meta", "forge_hip_gguf_config", "forge_hip_gguf_export_weights",
-    "forge_hip_model_create_from_gguf",
+    "forge_hip_model_create_from_gguf", "forge_hip_model_set_repeat_penalty", "forge_hip_apply_repeat_penalty", "forge_hip_sample",
 ]
 
 
@@ -135,6 +135,12 @@ def lib():
     L.forge_hip_attn_decode_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, vp]
     L.forge_hip_argmax.restype = i32
     L.forge_hip_argmax.argtypes = [vp, u32, vp, vp]
+    L.forge_hip_model_set_repeat_penalty.restype = i32
+    L.forge_hip_model_set_repeat_penalty.argtypes = [vp, C.c_float]
+    L.forge_hip_apply_repeat_penalty.restype = i32
+    L.forge_hip_apply_repeat_penalty.argtypes = [vp, u64, vp, u64, C.c_float]
+    L.forge_hip_sample.restype = i32
+    L.forge_hip_sample.argtypes = [vp, u64, C.c_float, u64, C.c_float, C.POINTER(u64), C.POINTER(u32)]
     _lib = L
     return L
 

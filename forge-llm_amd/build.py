@@ -11,7 +11,7 @@ BUILD = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libforge_hip.so")
 
 SOURCES = ["format.hip", "elementwise.hip", "gemv.hip", "gemm.hip", "attn_decode.hip", "attn_prefill.hip",
-           "attn_exact.hip", "decode_persistent.hip", "api.hip", "model.hip", "gguf.cpp"]
+           "attn_exact.hip", "decode_persistent.hip", "api.hip", "model.hip", "gguf.cpp", "sampling.cpp"]
 
 # -packed-fp32-ops off: keep hipcc from forming packed FP32 instructions.
 # -ffp-contract=off: the CPU path never fuses a*b+c; kernels say fmaf() where a fused op is meant.

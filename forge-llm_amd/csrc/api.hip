@@ -281,7 +281,7 @@ int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void
     FH_CHECK(x_dev && out_dev && n >= 1, "argmax: null pointer or empty input");
     int32_t rc = g_attn.reserve(ARGMAX_BLOCKS * 8);
     if (rc) return rc;
-    launch_argmax(x_dev, n, out_dev, g_attn.p, nullptr, nullptr, (hipStream_t)stream);
+    launch_argmax(x_dev, n, out_dev, g_attn.p, nullptr, nullptr, nullptr, 1.0f, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }

@@ -100,13 +100,13 @@ void launch_silu_mul(const float* gate, const float* up, uint32_t M, uint32_t I,
 void launch_rope_kv_store(float* q, float* k, const float* v, uint32_t q_stride, uint32_t kv_stride, uint16_t* kc,
                           uint16_t* vc, uint32_t M, uint32_t base_pos, const uint32_t* pos_dev, uint32_t heads,
                           uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, hipStream_t s);
-void launch_embedding(const float* table, const uint32_t* tokens_dev, uint32_t M, uint32_t H, float* out,
+void launch_embedding(const float* table, const uint32_t* tokens_dev, uint32_t M, uint32_t H, float* out, uint32_t* counts,
                       hipStream_t s);
 // Index of the LAST maximum.  `scratch` needs 2*ARGMAX_BLOCKS uint32/float pairs.
 constexpr uint32_t ARGMAX_BLOCKS = 256;
 // If pos_dev is given, the final stage also advances the decode state: *pos_dev += 1, *token_dev = *out.
 void launch_argmax(const float* x, uint32_t n, uint32_t* out, void* scratch, uint32_t* pos_dev, uint32_t* token_dev,
-                   hipStream_t s);
+                   const uint32_t* counts, float penalty, hipStream_t s);
 
 // gemv.hip — y[n] (=|+=) sum_b f32(isum_b) * (a_s[b]*w_s[n][b]); activations already quantised.
 // `order` selects which rows take the reference's 4-accumulator (dot1) order instead of the sequential one.
@@ -176,7 +176,9 @@ struct PdLayerIn {
 struct PdState;
 // Leaves *out null (returning OK) when the shape or device is not covered; `state` = {position, token, next token, abort flag}.
 int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layers, const QWeight& lm_head, const float* embed,
-                  const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, PdState** out);
+                  const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, uint32_t* counts,
+                  PdState** out);
+int32_t pd_set_repeat_penalty(PdState* st, float penalty);
 void pd_destroy(PdState* st);
 int32_t pd_enqueue(PdState* st, bool profile, uint32_t token, hipStream_t s);
 // Spins on the host word the kernel writes last; false = not available, wait for the stream instead.

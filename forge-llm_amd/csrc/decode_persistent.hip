@@ -112,6 +112,8 @@ struct PdArgs {
     unsigned long long* host_out;              // host-mapped {next token, launch number}: written last, or null
     uint32_t host_seq;
     uint32_t q4, lm_q4;                        // weight formats: projections, lm_head
+    uint32_t* counts;                          // u32 [vocab]: times each token id has been fed (this step's token is added here)
+    float penalty;                             // > 1: the argmax is taken over the penalised logits
     uint32_t use_hint;                         // pollers wait for one watched element before re-reading a whole buffer
     uint32_t off_act_s, off_misc, off_big;     // LDS byte offsets (activation codes sit at 0)
     unsigned long long* stamps;                // optional: wall clock at the start of every phase (workgroup 0)
@@ -161,6 +163,7 @@ __device__ __forceinline__ void stc64(uint64_t* p, uint32_t tag, uint32_t payloa
 
 struct PdCtx {
     uint32_t tid, lane, wave, wg, G;
+    uint32_t token;          // the token this step feeds
     uint32_t spin_limit;
     uint32_t* sh_abort;      // LDS
     uint32_t* abort_flag;    // global
@@ -753,7 +756,7 @@ __device__ __forceinline__ ArgPair arg_wg(ArgPair a, float* misc, const PdCtx& c
 //   inputs    the streamers issue the first weight loads of their rows at once; the poller wave fetches the activation
 //             vector (it never has weights in flight, so nothing delays what it polls)
 //   tiles     compute a round from registers, issue the next round (or the next tile's first), sum, finish the rows
-template <bool Q4, int HD, int FMT, bool ORDERED>
+template <bool Q4, int HD, int FMT, bool ORDERED, bool PEN>
 __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& job, const Mat& next, bool early, WReg& W, WReg& W1, const float* emb,
                                               uint32_t pos, uint32_t* aq_lds, float* as_lds, float* misc, float* big, ArgPair& best,
                                               const PdCtx& cx) {
@@ -891,6 +894,15 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
             } else {
                 if (mine) {
                     a.logits[row] = v;
+                    // apply_repeat_penalty (project.rs:505-513) before the argmax.  The thread that owns the row of the
+                    // token being fed is the only one in the grid to touch that counter: it adds this step's occurrence.
+                    // (A kernel built without PEN counts the token in its last stage and never reads the counters.)
+                    if (PEN) {
+                        const bool fed = row == cx.token;
+                        const uint32_t c = a.counts[row] + (fed ? 1u : 0u);
+                        if (fed) a.counts[row] = c;
+                        if (a.penalty > 1.0f) v = repeat_penalised(v, c, a.penalty);
+                    }
                     best = arg_better(best, ArgPair{v, row});
                 }
             }
@@ -907,7 +919,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
 // fits the instruction cache matters more than one binary for all models.
 // ORD: the GEMV rows are summed in the reference's block order (bit-identical to the kernel sequence) instead of as the
 // products come.
-template <int HD, int FMT, bool ORD>
+template <int HD, int FMT, bool ORD, bool PEN>
 __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     __shared__ uint32_t sh_abort;
@@ -930,6 +942,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
 
     const uint32_t pos = a.state[0], token = a.token_from_arg ? a.token : a.state[1];
     const float* emb = a.embed + (size_t)token * a.H;
+    cx.token = token;
     const uint32_t L = a.n_layers;
     ArgPair best{-INFINITY, 0};
     WReg W, W1;
@@ -982,8 +995,8 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         job.res_tag = ph == 1 ? x_in : base + 4;
         job.kc = a.layers[l].kc;
         job.vc = a.layers[l].vc;
-        if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT, ORD>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
-        else pd_gemv_phase<false, HD, FMT, ORD>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        else pd_gemv_phase<false, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
         early = next.valid;
         if (sh_abort) return;
     }
@@ -1009,6 +1022,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
             a.state[2] = p.i;
             a.state[1] = p.i;
             a.state[0] = pos + 1;
+            if (!PEN) a.counts[token] += 1;          // nobody read the counters in this launch
             if (a.stamps) a.stamps[6 * L + 2] = wall_clock64();
             // the host may be spinning on this word instead of waiting for the stream
             if (a.host_out)
@@ -1078,13 +1092,18 @@ bool plan_gemv(const QWeight& w, uint32_t inter, uint32_t nseg, const Segment* s
     return true;
 }
 
-template <int HD, bool ORD>
+template <int HD, bool ORD, bool PEN>
 const void* pd_kernel_ord(const PdState* st) {
-    if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2, ORD>);
-    return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 1, ORD>) : reinterpret_cast<const void*>(decode_step_kernel<HD, 0, ORD>);
+    if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2, ORD, PEN>);
+    return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 1, ORD, PEN>) : reinterpret_cast<const void*>(decode_step_kernel<HD, 0, ORD, PEN>);
 }
+// The repeat penalty is code of its own in the lm_head epilogue: the default kernel is built without it (the ordered
+// variants always carry it).
 template <int HD>
-const void* pd_kernel(const PdState* st) { return st->ordered ? pd_kernel_ord<HD, true>(st) : pd_kernel_ord<HD, false>(st); }
+const void* pd_kernel(const PdState* st) {
+    if (st->ordered) return pd_kernel_ord<HD, true, true>(st);
+    return st->args.penalty > 1.0f ? pd_kernel_ord<HD, false, true>(st) : pd_kernel_ord<HD, false, false>(st);
+}
 template <int HD>
 hipError_t launch_pd_hd(const PdState* st, hipStream_t s) {
     void* kargs[] = {const_cast<PdArgs*>(&st->args)};
@@ -1099,7 +1118,8 @@ void pd_destroy(PdState* st) { delete st; }
 // Plans the persistent decode step for a model.  Leaves *out null (and returns OK) when the shape or the
 // device is outside what the kernel covers; the caller then keeps the multi-kernel step.
 int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layers, const QWeight& lm_head, const float* embed,
-                  const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, PdState** out) {
+                  const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, uint32_t* counts,
+                  PdState** out) {
     *out = nullptr;
     if (c.flags & FORGE_HIP_FLAG_EXACT) return FORGE_HIP_OK;
     if (c.head_dim != 64 && c.head_dim != 128) return FORGE_HIP_OK;
@@ -1172,6 +1192,7 @@ e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, hd == 64 ? pd_kernel<6
     a.eps = c.rms_eps;
     a.embed = embed; a.final_norm = final_norm; a.cos_t = cos_t; a.sin_t = sin_t;
     a.logits = logits; a.state = state;
+    a.counts = counts; a.penalty = 1.0f;
     // one allocation for all tagged buffers (zeroed: tag 0 is never expected)
     const size_t n_tx = H, n_tq = QKS, n_tkv = 2 * (size_t)KV, n_tws = (size_t)c.heads * DECODE_SPLITS * (hd + 2),
                  n_taq = QKS / 4 + QKS / 32, n_taq2 = I / 4 + I / 32, n_tpart = 2 * (size_t)st->grid;
@@ -1216,6 +1237,20 @@ e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, hd == 64 ? pd_kernel<6
     st->n_stamps = 6 * a.n_layers + 3;
     a.stamps = nullptr;
     *out = st.release();
+    return FORGE_HIP_OK;
+}
+
+// A penalty > 1 selects the kernel variant that carries the penalty code: check that it, too, fits one workgroup per CU.
+int32_t pd_set_repeat_penalty(PdState* st, float penalty) {
+    const float old = st->args.penalty;
+    st->args.penalty = penalty;
+    int per_cu = 0;
+    const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, st->hd == 64 ? pd_kernel<64>(st) : pd_kernel<128>(st), PD_THREADS, st->lds);
+    if (e != hipSuccess || per_cu < 1) {
+        (void)hipGetLastError();
+        st->args.penalty = old;
+        return fail(FORGE_HIP_ERR_HIP, "persistent decode: the kernel variant with the repeat penalty does not fit the device");
+    }
     return FORGE_HIP_OK;
 }
 

@@ -37,6 +37,13 @@ __device__ __forceinline__ float act_scale(float absmax, float& inv) {
     return s;
 }
 
+// apply_repeat_penalty (project.rs:505-513) for one logit whose token occurs `count` times in the list: the reference
+// applies the penalty once per occurrence, so this is `count` successive divisions (or multiplications), not a power.
+__device__ __forceinline__ float repeat_penalised(float v, uint32_t count, float penalty) {
+    for (uint32_t k = 0; k < count; k++) v = v > 0.0f ? v / penalty : v * penalty;
+    return v;
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);

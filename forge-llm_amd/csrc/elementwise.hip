@@ -187,21 +187,23 @@ void launch_rope_kv_store(float* q, float* k, const float* v, uint32_t q_stride,
 }
 
 // ---- embedding (emit.rs:585-589) -----------------------------------------------------------------
+// `counts` (optional): how often each token id has been fed to the model; the row's first thread counts its token.
 __global__ __launch_bounds__(256) void embedding_kernel(const float* __restrict__ table,
                                                         const uint32_t* __restrict__ tokens, uint32_t H4,
-                                                        float* __restrict__ out) {
+                                                        float* __restrict__ out, uint32_t* __restrict__ counts) {
     const uint32_t r = blockIdx.y;
     const uint32_t i = blockIdx.x * 256 + threadIdx.x;
     if (i >= H4) return;
     const uint32_t tok = tokens[r];
+    if (counts && i == 0) atomicAdd(counts + tok, 1u);
     reinterpret_cast<float4*>(out)[(size_t)r * H4 + i] = reinterpret_cast<const float4*>(table)[(size_t)tok * H4 + i];
 }
 
-void launch_embedding(const float* table, const uint32_t* tokens_dev, uint32_t M, uint32_t H, float* out,
+void launch_embedding(const float* table, const uint32_t* tokens_dev, uint32_t M, uint32_t H, float* out, uint32_t* counts,
                       hipStream_t s) {
     if (M == 0) return;
     dim3 grid((H / 4 + 255) / 256, M);
-    fh::launch(embedding_kernel, grid, 256, 0, s, table, tokens_dev, H / 4, out);
+    fh::launch(embedding_kernel, grid, 256, 0, s, table, tokens_dev, H / 4, out, counts);
 }
 
 // ---- argmax (project.rs:501-503): the LAST index among equal maxima ------------------------------------
@@ -230,12 +232,15 @@ __device__ __forceinline__ ArgPair arg_block(ArgPair a, ArgPair* sh) {
     return r;
 }
 
-__global__ __launch_bounds__(256) void argmax_stage1(const float* __restrict__ x, uint32_t n, ArgPair* __restrict__ part) {
+// `counts` (optional): apply_repeat_penalty (project.rs:505-513) on the fly, once per time the token was fed.
+__global__ __launch_bounds__(256) void argmax_stage1(const float* __restrict__ x, uint32_t n, ArgPair* __restrict__ part,
+                                                     const uint32_t* __restrict__ counts, float penalty) {
     __shared__ ArgPair sh[4];
     ArgPair a{-INFINITY, 0};
     bool any = false;
     for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) {
         ArgPair b{x[i], i};
+        if (counts) b.v = repeat_penalised(b.v, counts[i], penalty);
         a = any ? arg_better(a, b) : b;
         any = true;
     }
@@ -258,11 +263,11 @@ __global__ __launch_bounds__(256) void argmax_stage2(const ArgPair* __restrict__
 }
 
 void launch_argmax(const float* x, uint32_t n, uint32_t* out, void* scratch, uint32_t* pos_dev, uint32_t* token_dev,
-                   hipStream_t s) {
+                   const uint32_t* counts, float penalty, hipStream_t s) {
     uint32_t blocks = (n + 255) / 256;
     if (blocks > ARGMAX_BLOCKS) blocks = ARGMAX_BLOCKS;
     if (blocks == 0) blocks = 1;
-    fh::launch(argmax_stage1, blocks, 256, 0, s, x, n, reinterpret_cast<ArgPair*>(scratch));
+    fh::launch(argmax_stage1, blocks, 256, 0, s, x, n, reinterpret_cast<ArgPair*>(scratch), counts, penalty);
     fh::launch(argmax_stage2, 1, 256, 0, s, reinterpret_cast<const ArgPair*>(scratch), blocks, out, pos_dev, token_dev);
 }
 

@@ -58,6 +58,8 @@ struct forge_hip_model {
     DevBuf cos_t, sin_t;
     // decode scratch
     DevBuf x, qkv, gu, logits, aq, asc, attn_ws, state, argmax_ws;
+    DevBuf counts;                       // u32 [vocab]: how often each token id has been fed since the last reset
+    float repeat_penalty = 1.0f;         // > 1: forward_greedy picks the maximum of the penalised logits
     // prefill scratch (chunk_rows rows)
     DevBuf px, pqkv, pattn, pgu, paq, pasc, ptok;
     bool prefill_fuse_quant = true;              // fast mode: attention writes int8 codes + scales (FORGE_HIP_FUSE=0: separate quantiser)
@@ -286,13 +288,15 @@ void enqueue_head(forge_hip_model* m, const float* xrow, bool after_prefill, boo
     }
     {
         StageMark t(m, ST_ARGMAX);
+        // the token sampled right after a prefill is not penalised (project.rs:719-720), those inside the loop are (:742-744)
+        const bool pen = !after_prefill && m->repeat_penalty > 1.0f;
         launch_argmax(m->logits.as<float>(), m->cfg.vocab, m->d_next(), m->argmax_ws.p, advance ? m->d_pos() : nullptr,
-                      advance ? m->d_token() : nullptr, s);
+                      advance ? m->d_token() : nullptr, pen ? m->counts.as<uint32_t>() : nullptr, m->repeat_penalty, s);
     }
 }
 
 void enqueue_decode_step(forge_hip_model* m) {
-    { StageMark t(m, ST_EMBED); launch_embedding(m->embed.as<float>(), m->d_token(), 1, m->H, m->x.as<float>(), m->stream); }
+    { StageMark t(m, ST_EMBED); launch_embedding(m->embed.as<float>(), m->d_token(), 1, m->H, m->x.as<float>(), m->counts.as<uint32_t>(), m->stream); }
     for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_decode_layer(m, l);
     enqueue_head(m, m->x.as<float>(), false, true);
 }
@@ -436,9 +440,10 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
     if ((rc = m->x.alloc(H * 4)) || (rc = m->qkv.alloc(m->QKV * 4)) || (rc = m->gu.alloc(2 * (size_t)I * 4)) ||
         (rc = m->logits.alloc((size_t)cfg->vocab * 4)) || (rc = m->aq.alloc(m->KMAX)) ||
         (rc = m->asc.alloc(m->KMAX / 32 * 2)) || (rc = m->attn_ws.alloc(attn_decode_workspace_bytes(cfg->heads, cfg->head_dim))) ||
-        (rc = m->state.alloc(64)) || (rc = m->argmax_ws.alloc(ARGMAX_BLOCKS * 8)))
+        (rc = m->state.alloc(64)) || (rc = m->argmax_ws.alloc(ARGMAX_BLOCKS * 8)) || (rc = m->counts.alloc((size_t)cfg->vocab * 4)))
         return rc;
     FH_HIP(hipMemset(m->state.p, 0, 64));
+    FH_HIP(hipMemset(m->counts.p, 0, (size_t)cfg->vocab * 4));
     const uint32_t R = m->chunk_rows = std::min(PREFILL_CHUNK, cfg->max_seq);
     if ((rc = m->px.alloc((size_t)R * H * 4)) || (rc = m->pqkv.alloc((size_t)R * m->QKV * 4)) ||
         (rc = m->pattn.alloc((size_t)R * QKS * 4)) || (rc = m->pgu.alloc((size_t)R * 2 * I * 4)) ||
@@ -453,7 +458,7 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
             pl[l] = PdLayerIn{&L.qkv, &L.o, &L.gate_up, &L.down, L.attn_norm, L.ffn_norm, m->kc(l), m->vc(l)};
         }
         rc = pd_create(*cfg, pl, m->lm_head, m->embed.as<float>(), m->final_norm.as<float>(), m->cos_t.as<float>(),
-                       m->sin_t.as<float>(), m->logits.as<float>(), m->state.as<uint32_t>(), &m->pd);
+                       m->sin_t.as<float>(), m->logits.as<float>(), m->state.as<uint32_t>(), m->counts.as<uint32_t>(), &m->pd);
         if (rc) return rc;
     }
     FH_HIP(hipDeviceSynchronize());
@@ -501,7 +506,7 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint
         const uint32_t rows = (uint32_t)std::min<uint64_t>(m->chunk_rows, n - done);
         // pageable source: the copy is complete (staged) when the call returns
         FH_HIP(hipMemcpyAsync(m->ptok.p, tokens + done, (size_t)rows * 4, hipMemcpyHostToDevice, s));
-        launch_embedding(m->embed.as<float>(), m->ptok.as<uint32_t>(), rows, m->H, m->px.as<float>(), s);
+        launch_embedding(m->embed.as<float>(), m->ptok.as<uint32_t>(), rows, m->H, m->px.as<float>(), m->counts.as<uint32_t>(), s);
         for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_prefill_layer(m, l, rows, (uint32_t)(m->pos + done));
         FH_HIP(hipGetLastError());
         done += rows;
@@ -583,7 +588,23 @@ int32_t forge_hip_reset(forge_hip_model* m) {
     m->pos = 0;
     m->h_stage[2] = 0;
     FH_HIP(hipMemcpyAsync(m->d_pos(), &m->h_stage[2], 4, hipMemcpyHostToDevice, m->stream));
+    FH_HIP(hipMemsetAsync(m->counts.p, 0, (size_t)m->cfg.vocab * 4, m->stream));      // recent_tokens starts empty again
     FH_HIP(hipStreamSynchronize(m->stream));
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_model_set_repeat_penalty(forge_hip_model* m, float penalty) {
+    FH_CHECK(m, "set_repeat_penalty: model is null");
+    FH_CHECK(penalty == penalty && penalty > 0.0f, "set_repeat_penalty: the penalty must be a positive number");
+    if (penalty == m->repeat_penalty) return FORGE_HIP_OK;
+    FH_HIP(hipStreamSynchronize(m->stream));
+    if (m->pd) {
+        const int32_t rc = pd_set_repeat_penalty(m->pd, penalty);
+        if (rc) return rc;
+    }
+    m->repeat_penalty = penalty;
+    // the captured kernel sequence carries the old value in its launch arguments: capture again at the next step
+    if (m->decode_graph) { (void)hipGraphExecDestroy(m->decode_graph); m->decode_graph = nullptr; }
     return FORGE_HIP_OK;
 }
 

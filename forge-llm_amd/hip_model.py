@@ -122,6 +122,37 @@ class HipModel:
             out.append(nxt)
         return out
 
+    def set_repeat_penalty(self, penalty: float) -> None:
+        """With a penalty > 1, forward_greedy takes the argmax of the logits after apply_repeat_penalty over every token
+        fed since the last reset (project.rs:505-513, 742-744), on the device."""
+        self._check(self._lib.forge_hip_model_set_repeat_penalty(self._h, float(penalty)))
+
+    def generate(self, prompt, max_tokens: int = 128, temperature: float = 0.0, top_k: int = 0, top_p: float = 0.9,
+                 repeat_penalty: float = 1.1, seed: int = 0xdeadbeef12345678, eos=()):
+        """The generation loop of the generated main.rs with its defaults (project.rs:607-612, 714-751): prefill, sample
+        (no penalty on the first token), then per token: stop on EOS, feed it, penalise every token fed so far, sample.
+        Greedy decoding (temperature <= 0) stays on the device; with a temperature the logits come back and the
+        host-side sampler runs."""
+        from .ops import apply_repeat_penalty, sample
+        rng = seed
+        logits = self.forward_prefill(prompt)
+        nxt, rng = sample(logits, temperature, top_k, top_p, rng)
+        recent = [int(t) for t in prompt]
+        out = []
+        self.set_repeat_penalty(repeat_penalty)
+        for _ in range(max_tokens):
+            if nxt in eos:
+                break
+            out.append(nxt)
+            recent.append(nxt)
+            if temperature <= 0.0:
+                nxt = self.forward_greedy(nxt)
+            else:
+                logits = self.forward(nxt)
+                apply_repeat_penalty(logits, recent, repeat_penalty)
+                nxt, rng = sample(logits, temperature, top_k, top_p, rng)
+        return out
+
     def close(self):
         if getattr(self, "_h", None):
             self._lib.forge_hip_model_destroy(self._h)

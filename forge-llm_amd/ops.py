@@ -68,6 +68,25 @@ def argmax_host(logits) -> int:
     return int(v.size - 1 - np.argmax(v[::-1]))
 
 
+def apply_repeat_penalty(logits, recent_tokens, penalty: float) -> None:
+    """apply_repeat_penalty (project.rs:505-513), in place on a float32 array."""
+    from . import check, lib
+    assert logits.dtype == np.float32 and logits.flags.c_contiguous
+    r = np.ascontiguousarray(recent_tokens, dtype=np.uint32)
+    check(lib().forge_hip_apply_repeat_penalty(logits.ctypes.data_as(C.c_void_p), logits.size, r.ctypes.data_as(C.c_void_p), r.size,
+                                               float(penalty)))
+
+
+def sample(logits, temperature: float, top_k: int, top_p: float, rng_state: int):
+    """sample (project.rs:515-555): returns (token, new rng state).  `logits` (float32) is overwritten, as in the reference."""
+    from . import check, lib
+    assert logits.dtype == np.float32 and logits.flags.c_contiguous
+    state, out = C.c_uint64(rng_state), C.c_uint32()
+    check(lib().forge_hip_sample(logits.ctypes.data_as(C.c_void_p), logits.size, float(temperature), int(top_k), float(top_p),
+                                 C.byref(state), C.byref(out)))
+    return int(out.value), int(state.value)
+
+
 # ---------------- device ops ----------------
 
 class QWeight:

@@ -239,6 +239,30 @@ int32_t forge_hip_gguf_export_weights(const forge_hip_gguf* g, const forge_hip_c
 /* open + config + export_weights + forge_hip_model_create. */
 int32_t forge_hip_model_create_from_gguf(const char* path, uint32_t max_seq, uint32_t flags, forge_hip_model** out);
 
+/* ---------------- sampling (the loop of the generated main.rs, project.rs:714-751) ----------------
+ * The reference's default generation is greedy WITH a repeat penalty of 1.1 (project.rs:607-611): after every
+ * `forward` it runs apply_repeat_penalty over all tokens fed so far (prompt and generated, once per occurrence) and then
+ * takes the argmax.  The model keeps that occurrence count per token id on the device (prefill and decode steps add to
+ * it, reset clears it); with a penalty > 1 set here, forge_hip_forward_greedy returns the last maximum of the penalised
+ * logits, bit for bit what apply_repeat_penalty + argmax give on the logits of forge_hip_forward.  The logits handed
+ * back by forge_hip_forward / forge_hip_prefill_batch stay unpenalised, as the reference's `forward` returns them, and
+ * the token after a prefill is the caller's argmax of those (the reference does not penalise it, project.rs:719-720).
+ * penalty <= 1 switches the penalty off (the reference's `if penalty <= 1.0 { return; }`). */
+int32_t forge_hip_model_set_repeat_penalty(forge_hip_model* m, float penalty);
+
+/* apply_repeat_penalty (project.rs:505-513) on host logits: for each entry of `recent`, in order,
+ * `l > 0 ? l /= penalty : l *= penalty`. */
+int32_t forge_hip_apply_repeat_penalty(float* logits_host, uint64_t n, const uint32_t* recent_host, uint64_t n_recent,
+                                       float penalty);
+/* sample (project.rs:515-555) on host logits, which it overwrites like the reference's `&mut [f32]`: temperature,
+ * softmax with sequential f32 sums, top-k, top-p (the entry that crosses the threshold is dropped too, as in the
+ * reference), renormalisation, one xorshift64 step of *rng_state, `r = state as f32 / u64::MAX as f32`, first index whose
+ * running sum reaches r (else the last index).  temperature <= 0: the last maximum, state untouched.  A NaN logit is
+ * FORGE_HIP_ERR_INVALID (the reference panics).  Among equal probabilities the lower index sorts first (the
+ * reference's unstable sort leaves that order open). */
+int32_t forge_hip_sample(float* logits_host, uint64_t n, float temperature, uint64_t top_k, float top_p, uint64_t* rng_state,
+                         uint32_t* out);
+
 #ifdef __cplusplus
 }
 #endif
