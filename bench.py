@@ -35,9 +35,9 @@ PROMPT_TOKENS = 2502
 # WRITE_SIZE counters of two profiler runs of this script, each scaled by what the same counter reads for the 1 GiB
 # copy of --calibrate-copy (FETCH_SIZE x2.000, WRITE_SIZE x1.000).  Summary: profiles/gemv_hbm_traffic_pmc.md.
 GEMV_HBM_BYTES_PER_LAUNCH = 20.46e6 + 0.02e6      # fetched + written
-# The same for one launch of the resident decode kernel (the whole step) at this context: 1 433.6 MB fetched + 13.3 MB
+# The same for one launch of the resident decode kernel (the whole step) at this context: 1 436.9 MB fetched + 13.8 MB
 # written.  Summary: profiles/decode_step_kernel_hbm_traffic_pmc.md.
-STEP_KERNEL_HBM_BYTES_PER_LAUNCH = 1446.9e6
+STEP_KERNEL_HBM_BYTES_PER_LAUNCH = 1450.7e6
 
 
 def gemv_launch_bytes(fh, cfg):
@@ -271,6 +271,12 @@ def main():
     tok2 = fh.ops.argmax_host(model.forward_prefill(prompt[:32]))
     t_decode_short, _ = timed_decode(model, tok2, 4, args.steps)
     path = "one resident kernel per token" if model.decode_launches == 1 else f"{model.decode_launches} kernels per token (graph replay)"
+
+    # ---- the reference's default loop: greedy with repeat penalty 1.1 over every token fed (project.rs:607-611, 742-744)
+    model.reset()
+    model.set_repeat_penalty(1.1)
+    tok3 = fh.ops.argmax_host(model.forward_prefill(prompt))
+    t_decode_pen, _ = timed_decode(model, tok3, args.warmup, args.steps)
     model.close()
 
     # ---- the other decode path, for comparison: the step as a sequence of kernels
@@ -317,6 +323,7 @@ def main():
         "prefill_tok_per_s": PROMPT_TOKENS / t_prefill,
         "prefill_ms": t_prefill * 1e3,
         "decode_tok_per_s_short_context": args.steps / t_decode_short,
+        "decode_tok_per_s_repeat_penalty_1.1": args.steps / t_decode_pen,
         "decode_weight_stream_GBps_end_to_end": fh.synth.decode_weight_bytes(cfg) * args.steps / t_decode / 1e9,
         "roofline": roofline,
         "prefill_rooflines": {
