@@ -246,25 +246,128 @@ int32_t locate(const forge_hip_gguf* g, const std::string& name, uint64_t numel,
     return FORGE_HIP_OK;
 }
 
-// f32 values of a tensor (weight_loader.rs:809-855 for the dense types, :860-926 for the two block formats).
-int32_t to_f32(const Source& s, uint64_t numel, float* out) {
-    switch (s.t->type) {
-        case T_F32: memcpy(out, s.bytes, numel * 4); return FORGE_HIP_OK;
-        case T_F16:
-            for (uint64_t i = 0; i < numel; i++) out[i] = fh::f16_to_f32_host((uint16_t)(s.bytes[2 * i] | (s.bytes[2 * i + 1] << 8)));
-            return FORGE_HIP_OK;
-        case T_BF16:
-            for (uint64_t i = 0; i < numel; i++) {
-                const uint32_t b = ((uint32_t)(s.bytes[2 * i] | (s.bytes[2 * i + 1] << 8))) << 16;
-                memcpy(out + i, &b, 4);
-            }
-            return FORGE_HIP_OK;
-        case T_Q8_0: fh::dequant_host(FORGE_HIP_Q8_0, s.bytes, numel, out); return FORGE_HIP_OK;
-        case T_Q4_0: fh::dequant_host(FORGE_HIP_Q4_0, s.bytes, numel, out); return FORGE_HIP_OK;
-        default:
-            return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor " + s.t->name + " has GGML type " + std::to_string(s.t->type) +
-                                                   "; this library reads F32, F16, BF16, Q8_0 and Q4_0 tensors");
+// ---- the other block formats the reference's loader reads (weight_loader.rs:809-825) --------------------------------
+// Values in the reference's order of f32 operations (no fused multiply-add: this file is built with -ffp-contract=off).
+
+// get_scale_min_k4, weight_loader.rs:977-987: 6-bit scale and minimum j of the 12 packed bytes of a K-quant super-block.
+void scale_min_k4(int j, const uint8_t* sc, uint8_t* scale, uint8_t* mn) {
+    if (j < 4) { *scale = sc[j] & 63; *mn = sc[j + 4] & 63; }
+    else { *scale = (uint8_t)((sc[j + 4] & 0x0F) | ((sc[j - 4] >> 6) << 4)); *mn = (uint8_t)((sc[j + 4] >> 4) | ((sc[j] >> 6) << 4)); }
+}
+float half_at(const uint8_t* p) { return fh::f16_to_f32_host((uint16_t)(p[0] | (p[1] << 8))); }
+
+// dequant_q4_1, weight_loader.rs:931-965: 20 bytes = f16 scale, f16 minimum, 16 bytes of nibbles; q * scale + min.
+void dequant_q4_1(const uint8_t* d, uint64_t n, float* out) {
+    for (uint64_t b = 0; b * 32 < n; b++) {
+        const uint8_t* blk = d + b * 20;
+        const float scale = half_at(blk), mn = half_at(blk + 2);
+        for (uint64_t j = 0; j < 16; j++) {
+            const float lo = (float)(blk[4 + j] & 0x0F), hi = (float)(blk[4 + j] >> 4);
+            if (b * 32 + j < n) out[b * 32 + j] = lo * scale + mn;
+            if (b * 32 + j + 16 < n) out[b * 32 + j + 16] = hi * scale + mn;
+        }
     }
+}
+// dequant_q4_k (weight_loader.rs:1146-1201) and dequant_q5_k (:1071-1135): 256 elements in four chunks of 64, each with
+// two (scale, minimum) pairs; value = (d * sc) * q - (dmin * m).  Q5_K adds one high bit per element from `qh`.
+void dequant_q45_k(bool five, const uint8_t* d, uint64_t n, float* out) {
+    const uint64_t bytes = five ? 176 : 144;
+    for (uint64_t b = 0; b * 256 < n; b++) {
+        const uint8_t* blk = d + b * bytes;
+        const float dd = half_at(blk), dmin = half_at(blk + 2);
+        const uint8_t* scales = blk + 4;
+        const uint8_t* qh = blk + 16;                       // Q5_K only
+        const uint8_t* qs = blk + (five ? 48 : 16);
+        for (int chunk = 0; chunk < 4; chunk++) {
+            uint8_t sc1, m1, sc2, m2;
+            scale_min_k4(2 * chunk, scales, &sc1, &m1);
+            scale_min_k4(2 * chunk + 1, scales, &sc2, &m2);
+            const float d1 = dd * (float)sc1, mm1 = dmin * (float)m1, d2 = dd * (float)sc2, mm2 = dmin * (float)m2;
+            const uint8_t u1 = (uint8_t)(1u << (2 * chunk)), u2 = (uint8_t)(2u << (2 * chunk));
+            for (uint64_t l = 0; l < 32; l++) {
+                const uint64_t o = b * 256 + chunk * 64 + l;
+                const uint8_t q = qs[chunk * 32 + l];
+                const uint32_t lo = (q & 0x0F) + ((five && (qh[l] & u1)) ? 16u : 0u);
+                const uint32_t hi = (q >> 4) + ((five && (qh[l] & u2)) ? 16u : 0u);
+                if (o < n) out[o] = d1 * (float)lo - mm1;
+                if (o + 32 < n) out[o + 32] = d2 * (float)hi - mm2;
+            }
+        }
+    }
+}
+// dequant_q6_k, weight_loader.rs:997-1057: 210 bytes = 128 low nibbles, 64 bytes of high bit pairs, 16 int8 scales, f16 d;
+// two halves of 128 elements, four interleaved values per step; value = (d * sc) * (q - 32).
+void dequant_q6_k(const uint8_t* d, uint64_t n, float* out) {
+    for (uint64_t b = 0; b * 256 < n; b++) {
+        const uint8_t* blk = d + b * 210;
+        const uint8_t *ql = blk, *qh = blk + 128;
+        const int8_t* sc = reinterpret_cast<const int8_t*>(blk + 192);
+        const float dd = half_at(blk + 208);
+        for (uint64_t half = 0; half < 2; half++) {
+            const uint8_t *l4 = ql + 64 * half, *h2 = qh + 32 * half;
+            const int8_t* s = sc + 8 * half;
+            for (uint64_t l = 0; l < 32; l++) {
+                const int is = (int)(l / 16);
+                const int q1 = (int)((l4[l] & 0x0F) | ((h2[l] & 3) << 4)) - 32;
+                const int q2 = (int)((l4[l + 32] & 0x0F) | (((h2[l] >> 2) & 3) << 4)) - 32;
+                const int q3 = (int)((l4[l] >> 4) | (((h2[l] >> 4) & 3) << 4)) - 32;
+                const int q4 = (int)((l4[l + 32] >> 4) | (((h2[l] >> 6) & 3) << 4)) - 32;
+                const uint64_t o = b * 256 + 128 * half + l;
+                if (o < n) out[o] = dd * (float)s[is] * (float)q1;
+                if (o + 32 < n) out[o + 32] = dd * (float)s[is + 2] * (float)q2;
+                if (o + 64 < n) out[o + 64] = dd * (float)s[is + 4] * (float)q3;
+                if (o + 96 < n) out[o + 96] = dd * (float)s[is + 6] * (float)q4;
+            }
+        }
+    }
+}
+// dequant_q8_k, weight_loader.rs:1206-1229: f32 scale + 256 int8 (+ 32 bytes of block sums that are not used).
+void dequant_q8_k(const uint8_t* d, uint64_t n, float* out) {
+    for (uint64_t b = 0; b * 256 < n; b++) {
+        const uint8_t* blk = d + b * 292;
+        float scale;
+        memcpy(&scale, blk, 4);
+        for (uint64_t j = 0; j < 256 && b * 256 + j < n; j++) out[b * 256 + j] = scale * (float)(int8_t)blk[4 + j];
+    }
+}
+
+// Types whose tensors the reference's loader turns into Q8_0 when it reads them (weight_loader.rs:219-229).
+bool requantised_on_load(uint32_t type) { return type == 3 || type == 12 || type == 13 || type == 14 || type == 15; }
+
+// `dequantize` of weight_loader.rs:809-825 for the types this library reads.
+bool dequant_ggml(uint32_t type, const uint8_t* d, uint64_t n, float* out) {
+    switch (type) {
+        case T_F32: memcpy(out, d, n * 4); return true;
+        case T_F16: for (uint64_t i = 0; i < n; i++) out[i] = half_at(d + 2 * i); return true;
+        case T_BF16:
+            for (uint64_t i = 0; i < n; i++) { const uint32_t b = ((uint32_t)(d[2 * i] | (d[2 * i + 1] << 8))) << 16; memcpy(out + i, &b, 4); }
+            return true;
+        case T_Q8_0: fh::dequant_host(FORGE_HIP_Q8_0, d, n, out); return true;
+        case T_Q4_0: fh::dequant_host(FORGE_HIP_Q4_0, d, n, out); return true;
+        case 3: dequant_q4_1(d, n, out); return true;
+        case 12: dequant_q45_k(false, d, n, out); return true;
+        case 13: dequant_q45_k(true, d, n, out); return true;
+        case 14: dequant_q6_k(d, n, out); return true;
+        case 15: dequant_q8_k(d, n, out); return true;
+        default: return false;
+    }
+}
+
+const char* const SUPPORTED_TYPES = "F32, F16, BF16, Q8_0, Q4_0, Q4_1, Q4_K, Q5_K, Q6_K and Q8_K";
+
+// f32 values of a tensor as the reference holds it after loading: dense types and Q8_0 / Q4_0 decode directly
+// (weight_loader.rs:809-926); any other quantised type is first turned into Q8_0 blocks by the loader
+// (dequantise, quantize_f32_to_q8_0: weight_loader.rs:219-229), so its values are those of the Q8_0 blocks.
+int32_t to_f32(const Source& s, uint64_t numel, float* out) {
+    if (!dequant_ggml(s.t->type, s.bytes, numel, out))
+        return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor " + s.t->name + " has GGML type " + std::to_string(s.t->type) +
+                                               "; this library reads " + SUPPORTED_TYPES + " tensors");
+    if (requantised_on_load(s.t->type)) {
+        std::vector<uint8_t> q8((numel + 31) / 32 * 34);
+        fh::quantize_host(FORGE_HIP_Q8_0, out, numel, q8.data());
+        fh::dequant_host(FORGE_HIP_Q8_0, q8.data(), numel, out);
+    }
+    return FORGE_HIP_OK;
 }
 
 uint64_t qbytes(uint32_t wdtype, uint64_t numel) { return numel / 32 * (wdtype == FORGE_HIP_Q8_0 ? 34 : 18); }
@@ -374,6 +477,13 @@ int32_t forge_hip_gguf_meta(const forge_hip_gguf* g, const char* key, uint32_t* 
     return FORGE_HIP_OK;
 }
 
+int32_t forge_hip_dequant_ggml(uint32_t ggml_type, const uint8_t* data_host, uint64_t n, float* out_host) {
+    FH_CHECK(data_host && out_host, "dequant_ggml: null pointer");
+    if (!dequant_ggml(ggml_type, data_host, n, out_host))
+        return fh::fail(FORGE_HIP_ERR_INVALID, "dequant_ggml: GGML type " + std::to_string(ggml_type) + " is not one of " + SUPPORTED_TYPES);
+    return FORGE_HIP_OK;
+}
+
 int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_t flags, forge_hip_config* out) {
     FH_CHECK(g && out, "gguf_config: null argument");
     const MetaValue* arch_v = g->find("general.architecture");
@@ -434,8 +544,9 @@ int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_
         if (ot->type == T_Q4_0) lm = FORGE_HIP_Q4_0;
         else if (ot->type == T_Q8_0) lm = FORGE_HIP_Q8_0;
         else if (ot->type == T_F32 || ot->type == T_F16 || ot->type == T_BF16) lm = wdtype;   // dense: quantised like the projections
+        else if (requantised_on_load(ot->type)) lm = FORGE_HIP_Q8_0;                          // GGMLType::to_dtype, gguf.rs:168-205
         else return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: output.weight has GGML type " + std::to_string(ot->type) +
-                                                       "; this library reads F32, F16, BF16, Q8_0 and Q4_0 tensors");
+                                                       "; this library reads " + SUPPORTED_TYPES + " tensors");
     }
     const uint64_t seq = max_seq ? max_seq : ctx;
     if (has_window && window < seq)

@@ -13,6 +13,7 @@ import numpy as np
 
 MAGIC = 0x46554747          # gguf.rs:18
 F32, F16, Q4_0, Q8_0, BF16 = 0, 1, 2, 8, 30
+Q4_1, Q4_K, Q5_K, Q6_K, Q8_K = 3, 12, 13, 14, 15
 
 # GGUF metadata value type ids (gguf.rs:447-476)
 U8, I8, U16, I16, U32, I32, FLOAT32, BOOL, STRING, ARRAY, U64, I64, FLOAT64 = range(13)
@@ -130,6 +131,17 @@ def model_to_gguf(cfg: dict, blob: np.ndarray, tied: bool = True, arch: str = "l
     return write_gguf(meta, [(n, d, g, b) for n, (d, g, b) in t.items()], path=path)
 
 
+def dequant_ggml(ggml_type: int, data, n: int) -> np.ndarray:
+    """`dequantize` of the reference's loader (weight_loader.rs:809-825) for one tensor's bytes."""
+    from . import check, lib
+    L = lib()
+    _declare(L)
+    raw = np.ascontiguousarray(np.frombuffer(data, np.uint8) if not isinstance(data, np.ndarray) else data, np.uint8)
+    out = np.empty(n, np.float32)
+    check(L.forge_hip_dequant_ggml(ggml_type, raw.ctypes.data_as(C.c_void_p), n, out.ctypes.data_as(C.c_void_p)))
+    return out
+
+
 class GgufFile:
     """A parsed GGUF file: `GGUFFile` of the reference (gguf.rs:287-341) on the library's parser."""
 
@@ -233,6 +245,8 @@ def _declare(L):
     L.forge_hip_gguf_config.argtypes = [vp, u32, u32, C.POINTER(Config)]
     L.forge_hip_gguf_export_weights.restype = i32
     L.forge_hip_gguf_export_weights.argtypes = [vp, C.POINTER(Config), vp, u64]
+    L.forge_hip_dequant_ggml.restype = i32
+    L.forge_hip_dequant_ggml.argtypes = [u32, vp, u64, vp]
     L.forge_hip_model_create_from_gguf.restype = i32
     L.forge_hip_model_create_from_gguf.argtypes = [C.c_char_p, u32, u32, C.POINTER(vp)]
     L._gguf_declared = True

@@ -196,7 +196,10 @@ int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void
  * load_config (crates/forgellm-cli/src/main.rs:700-830) and `forge export-weights` (main.rs:2585-2757, tensor names
  * mapped by weight_loader.rs:400-447), whose output file is the blob forge_hip_model_create takes.  These entry points are
  * those three steps.  Supported: architectures "llama" and "mistral" (without a sliding window shorter than max_seq);
- * tensors of GGML type F32, F16, BF16, Q8_0 or Q4_0; projections mostly Q8_0 or mostly Q4_0 (the reference's majority vote). */
+ * tensors of GGML type F32, F16, BF16, Q8_0, Q4_0 and -- turned into Q8_0 blocks when they are read, as the reference's loader
+ * does (weight_loader.rs:219-229) -- Q4_1, Q4_K, Q5_K, Q6_K, Q8_K; projections mostly Q8_0 or mostly Q4_0 by the reference's
+ * majority vote, which counts those other types as Q8_0 (a file whose projections are mostly Q4_K is refused: the reference
+ * runs it on Q4_K kernels of its own). */
 typedef struct forge_hip_gguf forge_hip_gguf;
 
 /* gguf::parse over a file (memory-mapped until close) or over bytes the caller keeps alive until close.  Failures are
@@ -236,6 +239,9 @@ int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_
  * stored in another format than the blob needs is converted with the reference's own routines (dequant
  * weight_loader.rs:809-926, quantisers :1454-1544). */
 int32_t forge_hip_gguf_export_weights(const forge_hip_gguf* g, const forge_hip_config* cfg, uint8_t* out_host, uint64_t nbytes);
+/* `dequantize` (weight_loader.rs:809-825) for one tensor's bytes: GGML types F32 (0), F16 (1), BF16 (30), Q8_0 (8), Q4_0 (2),
+ * Q4_1 (3), Q4_K (12), Q5_K (13), Q6_K (14), Q8_K (15); n = number of elements. */
+int32_t forge_hip_dequant_ggml(uint32_t ggml_type, const uint8_t* data_host, uint64_t n, float* out_host);
 /* open + config + export_weights + forge_hip_model_create. */
 int32_t forge_hip_model_create_from_gguf(const char* path, uint32_t max_seq, uint32_t flags, forge_hip_model** out);
 

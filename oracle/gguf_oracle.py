@@ -10,8 +10,9 @@ Follows, step by step:
   dense dequant    weight_loader.rs:827-855; Q8_0 / Q4_0 dequant and the weight quantisers come from forge_oracle.cpp
 
 Pinned by the reference's own unit tests for this path (gguf.rs:606-769: minimal v3 file, several tensors with
-metadata, version 2, bad magic, unsupported version, data sizes, alignment), restated as byte strings in
-tests/test_gguf.py.  Where a GGUF tensor is stored in another format than the blob needs, the reference's exporter
+metadata, version 2, bad magic, unsupported version, data sizes, alignment; weight_loader.rs:3245-3259 and :3422-3656:
+the Q4_1, Q4_K, Q5_K and Q6_K dequantiser fixtures), restated as byte strings in tests/test_gguf.py.  Q8_K has no
+reference fixture: pinned by its closed form (scale * int8) only.  Where a GGUF tensor is stored in another format than the blob needs, the reference's exporter
 writes bytes its own generated reader cannot consume (main.rs:2603-2626 handles only f32 -> Q4_0); this restatement
 converts with the reference's dequantisers and quantisers instead, and says so here: that conversion is parity
 unpinned (no reference test or fixture covers it).
@@ -174,6 +175,8 @@ def config(g, max_seq=0, flags=0) -> dict:
     if ot is not None:
         if ot["ggml_type"] in (2, 8):
             lm = ot["ggml_type"]
+        elif ot["ggml_type"] in REQUANTISED_ON_LOAD:
+            lm = 8
         elif ot["ggml_type"] not in (0, 1, 30):
             raise GgufError("output.weight has an unsupported GGML type")
     seq = max_seq or ctx
@@ -186,20 +189,93 @@ def config(g, max_seq=0, flags=0) -> dict:
             "rope_theta": float(f(10000.0) if theta is None else f(theta)), "wdtype": wd, "lm_head_dtype": lm, "flags": flags}
 
 
-def _tensor_f32(oracle, g, data, t):
-    n = numel(t)
-    start = g["tensor_data_offset"] + t["offset"]
-    raw = np.frombuffer(data, np.uint8, data_size(t), start)
-    ty = t["ggml_type"]
+F = np.float32
+REQUANTISED_ON_LOAD = (3, 12, 13, 14, 15)      # Q4_1, Q4_K, Q5_K, Q6_K, Q8_K become Q8_0 blocks when read, weight_loader.rs:219-229
+
+
+def _half(oracle, blocks, off):
+    return oracle.f16_to_f32(blocks[:, off:off + 2].copy().view("<u2")[:, 0]).astype(F)
+
+
+def _scale_min_k4(sc):
+    """get_scale_min_k4 (weight_loader.rs:977-987) for j = 0..7 of every block: two uint8 arrays [nblocks][8]."""
+    s = np.empty((sc.shape[0], 8), np.uint8)
+    m = np.empty((sc.shape[0], 8), np.uint8)
+    s[:, :4] = sc[:, 0:4] & 63
+    m[:, :4] = sc[:, 4:8] & 63
+    s[:, 4:] = (sc[:, 8:12] & 0x0F) | ((sc[:, 0:4] >> 6) << 4)
+    m[:, 4:] = (sc[:, 8:12] >> 4) | ((sc[:, 4:8] >> 6) << 4)
+    return s, m
+
+
+def dequant_ggml(oracle, ty, raw, n):
+    """`dequantize` (weight_loader.rs:809-825), numpy float32 in the reference's order of operations."""
+    raw = np.frombuffer(raw, np.uint8) if not isinstance(raw, np.ndarray) else raw
     if ty == 0:
-        return raw.view("<f4").copy()
+        return raw[:4 * n].view("<f4").copy()
     if ty == 1:
-        return oracle.f16_to_f32(raw.view("<u2"))
+        return oracle.f16_to_f32(raw[:2 * n].view("<u2"))
     if ty == 30:
-        return (raw.view("<u2").astype(np.uint32) << 16).view(np.float32)
+        return (raw[:2 * n].view("<u2").astype(np.uint32) << 16).view(np.float32)
     if ty in (8, 2):
         return oracle.dequant(ty, raw, n)
-    raise GgufError(f"tensor {t['name']}: unsupported GGML type {ty}")
+    block, nbytes = TYPE_LAYOUT[ty]
+    nb = (n + block - 1) // block
+    b = raw[:nb * nbytes].reshape(nb, nbytes)
+    out = np.empty((nb, block), F)
+    if ty == 3:                                   # Q4_1, weight_loader.rs:931-965
+        scale, mn = _half(oracle, b, 0)[:, None], _half(oracle, b, 2)[:, None]
+        out[:, :16] = (b[:, 4:] & 0x0F).astype(F) * scale + mn
+        out[:, 16:] = (b[:, 4:] >> 4).astype(F) * scale + mn
+    elif ty in (12, 13):                          # Q4_K :1146-1201, Q5_K :1071-1135
+        d, dmin = _half(oracle, b, 0), _half(oracle, b, 2)
+        s, m = _scale_min_k4(b[:, 4:16])
+        qs = b[:, (48 if ty == 13 else 16):].reshape(nb, 4, 32)
+        lo, hi = (qs & 0x0F).astype(np.uint32), (qs >> 4).astype(np.uint32)
+        if ty == 13:
+            qh = b[:, 16:48]
+            for c in range(4):
+                lo[:, c] += np.where(qh & (1 << (2 * c)), 16, 0).astype(np.uint32)
+                hi[:, c] += np.where(qh & (2 << (2 * c)), 16, 0).astype(np.uint32)
+        o = out.reshape(nb, 4, 64)
+        for c in range(4):
+            d1, m1 = (d * s[:, 2 * c].astype(F))[:, None], (dmin * m[:, 2 * c].astype(F))[:, None]
+            d2, m2 = (d * s[:, 2 * c + 1].astype(F))[:, None], (dmin * m[:, 2 * c + 1].astype(F))[:, None]
+            o[:, c, :32] = d1 * lo[:, c].astype(F) - m1
+            o[:, c, 32:] = d2 * hi[:, c].astype(F) - m2
+    elif ty == 14:                                # Q6_K, weight_loader.rs:997-1057
+        ql, qh = b[:, :128].reshape(nb, 2, 64), b[:, 128:192].reshape(nb, 2, 32)
+        sc = b[:, 192:208].view(np.int8).reshape(nb, 2, 8).astype(F)
+        d = _half(oracle, b, 208)[:, None, None]
+        o = out.reshape(nb, 2, 4, 32)
+        q = np.empty((nb, 2, 4, 32), np.int32)
+        q[:, :, 0] = (ql[:, :, :32] & 0x0F) | ((qh & 3) << 4)
+        q[:, :, 1] = (ql[:, :, 32:] & 0x0F) | (((qh >> 2) & 3) << 4)
+        q[:, :, 2] = (ql[:, :, :32] >> 4) | (((qh >> 4) & 3) << 4)
+        q[:, :, 3] = (ql[:, :, 32:] >> 4) | (((qh >> 6) & 3) << 4)
+        q -= 32
+        for k in range(4):
+            scale = np.repeat(sc[:, :, 2 * k:2 * k + 2], 16, axis=2)          # is = l / 16 picks scale 2k or 2k + 1
+            o[:, :, k] = d * scale * q[:, :, k].astype(F)
+    elif ty == 15:                                # Q8_K, weight_loader.rs:1206-1229
+        scale = b[:, :4].copy().view("<f4")
+        out[:] = scale * b[:, 4:260].view(np.int8).astype(F)
+    else:
+        raise GgufError(f"unsupported GGML type {ty}")
+    return out.reshape(-1)[:n].copy()
+
+
+def _tensor_f32(oracle, g, data, t):
+    """The tensor's values as the reference holds them after loading."""
+    n = numel(t)
+    raw = np.frombuffer(data, np.uint8, data_size(t), g["tensor_data_offset"] + t["offset"])
+    ty = t["ggml_type"]
+    if ty not in (0, 1, 30, 8, 2) + REQUANTISED_ON_LOAD:
+        raise GgufError(f"tensor {t['name']}: unsupported GGML type {ty}")
+    v = dequant_ggml(oracle, ty, raw, n)
+    if ty in REQUANTISED_ON_LOAD:
+        v = oracle.dequant(8, oracle.quantize_weights(8, v), n)
+    return v
 
 
 def export_weights(oracle, g, data, cfg) -> np.ndarray:

@@ -269,7 +269,11 @@ def test_config_defaults_and_refusals(fh, gg, go):
     refused([base[0], ("llama.embedding_length", gg.U64, 64)] + base[2:], text="could not extract model config")
     refused(base, tensors=(("blk.0.attn_q.weight", [64, 64], gg.F16, None),), text="neither mostly Q8_0 nor mostly Q4_0")
     refused(base, tensors=(("blk.0.attn_q.weight", [256, 64], 12, None),), text="neither mostly Q8_0 nor mostly Q4_0")
-    refused(base, tensors=(("blk.0.attn_q.weight", [64, 64], gg.Q8_0, None), ("output.weight", [256, 64], 14, None)), text="output.weight")
+    refused(base, tensors=(("blk.0.attn_q.weight", [64, 64], gg.Q8_0, None), ("output.weight", [256, 64], 10, None)), text="output.weight")
+    # a Q6_K output matrix is read as Q8_0 (GGMLType::to_dtype, gguf.rs:168-205); Q5_K projections vote as Q8_0 (main.rs:509-531)
+    kq = (("blk.0.attn_q.weight", [256, 64], gg.Q5_K, None), ("output.weight", [256, 64], gg.Q6_K, None))
+    ck = gg.GgufFile(make(base, kq)).config()
+    assert (ck["wdtype"], ck["lm_head_dtype"]) == (Q8, Q8) and ck == go.config(go.parse(make(base, kq)))
     refused(base + [("llama.attention.sliding_window", gg.U32, 1024)], text="sliding-window")
     # the vote: 2 x Q4_0 against 1 x Q8_0
     vote = (("blk.0.attn_q.weight", [64, 64], gg.Q4_0, None), ("blk.0.attn_k.weight", [64, 64], gg.Q4_0, None),
@@ -298,8 +302,8 @@ def test_export_errors(fh, gg):
     assert "blk.0.attn_k.weight has" in export(wrong)
     kq = dict(t)
     d = kq["blk.0.ffn_down.weight"][0]
-    kq["blk.0.ffn_down.weight"] = (d, 14, np.zeros(int(np.prod(d)) // 256 * 210, np.uint8))
-    assert "reads F32, F16, BF16, Q8_0 and Q4_0" in export(kq)
+    kq["blk.0.ffn_down.weight"] = (d, 11, np.zeros(int(np.prod(d)) // 256 * 110, np.uint8))      # Q3_K
+    assert "this library reads F32, F16, BF16, Q8_0, Q4_0, Q4_1, Q4_K, Q5_K, Q6_K and Q8_K tensors" in export(kq)
     # a data section cut short: the last tensor extends past the end of the file
     data = gg.write_gguf(meta, [(n, d, g, b) for n, (d, g, b) in t.items()])
     f = gg.GgufFile(data[:-4096])
@@ -314,6 +318,178 @@ def test_export_errors(fh, gg):
     assert fh.lib().forge_hip_gguf_export_weights(f._h, byref(c), out.ctypes.data_as(c_void_p), 16) == fh.ERR_BLOB_SIZE
     with pytest.raises(fh.ForgeHipError):
         gg.GgufFile("/nonexistent/dir/model.gguf")
+
+
+# ---------------- the other block formats the reference's loader reads ----------------
+def f16le(bits):
+    return struct.pack("<H", bits)
+
+
+def dq(fh, go, oracle, ty, block, n):
+    """Dequantise with the library and with the oracle; they must agree bit for bit."""
+    a = fh.gguf.dequant_ggml(ty, np.frombuffer(bytes(block), np.uint8), n)
+    b = go.dequant_ggml(oracle, ty, np.frombuffer(bytes(block), np.uint8), n)
+    assert a.shape == (n,) and np.array_equal(a.view(np.uint32), np.asarray(b, np.float32).view(np.uint32))
+    return a
+
+
+def test_reference_dequant_q4_1_basic(fh, gg, go, oracle):
+    """weight_loader.rs:3245-3259: scale 2.0, minimum 1.0, all nibbles 0 -> 1.0 everywhere."""
+    block = f16le(0x4000) + f16le(0x3C00) + bytes(16)
+    assert np.all(np.abs(dq(fh, go, oracle, gg.Q4_1, block, 32) - 1.0) < 1e-6)
+
+
+def test_reference_dequant_q4_k(fh, gg, go, oracle):
+    """weight_loader.rs:3422-3478."""
+    block = bytearray(144)
+    block[0:2] = f16le(0x3C00)
+    for i in (4, 5, 6, 7, 12, 13, 14, 15):
+        block[i] = 1
+    assert np.all(np.abs(dq(fh, go, oracle, gg.Q4_K, block, 256)) < 1e-6)
+    block = bytearray(144)
+    block[0:2], block[2:4] = f16le(0x4000), f16le(0x3C00)
+    block[4], block[8] = 3, 2
+    for i in range(32):
+        block[16 + i] = 0x05
+    out = dq(fh, go, oracle, gg.Q4_K, block, 256)
+    assert np.all(np.abs(out[:32] - 28.0) < 1e-4)
+
+
+def test_reference_dequant_q5_k(fh, gg, go, oracle):
+    """weight_loader.rs:3481-3560."""
+    block = bytearray(176)
+    block[0:2] = f16le(0x3C00)
+    for i in (4, 5, 6, 7, 12, 13, 14, 15):
+        block[i] = 1
+    assert np.all(np.abs(dq(fh, go, oracle, gg.Q5_K, block, 256)) < 1e-6)
+    block = bytearray(176)
+    block[0:2] = f16le(0x3C00)
+    block[4], block[16], block[48] = 1, 0x01, 0x03
+    assert abs(dq(fh, go, oracle, gg.Q5_K, block, 256)[0] - 19.0) < 1e-4
+    block = bytearray(176)
+    block[0:2] = f16le(0x3C00)
+    block[5], block[16], block[48] = 2, 0x02, 0x70
+    assert abs(dq(fh, go, oracle, gg.Q5_K, block, 256)[32] - 46.0) < 1e-4
+
+
+def test_reference_dequant_q6_k(fh, gg, go, oracle):
+    """weight_loader.rs:3562-3656."""
+    block = bytearray(210)
+    block[208:210] = f16le(0x3C00)
+    for i in range(192, 208):
+        block[i] = 1
+    assert np.all(np.abs(dq(fh, go, oracle, gg.Q6_K, block, 256) + 32.0) < 1e-4)
+    block = bytearray(210)
+    block[208:210] = f16le(0x3800)
+    block[192], block[0], block[128] = 2, 0x0A, 0x02
+    assert abs(dq(fh, go, oracle, gg.Q6_K, block, 256)[0] - 10.0) < 1e-4
+    block = bytearray(210)
+    block[208:210] = f16le(0x3C00)
+    for i in range(192, 208):
+        block[i] = 1
+    block[0], block[32], block[128] = 0x31, 0x52, 0xE4
+    out = dq(fh, go, oracle, gg.Q6_K, block, 256)
+    assert [abs(out[i] - w) < 1e-4 for i, w in ((0, -31.0), (32, -14.0), (64, 3.0), (96, 21.0))] == [True] * 4
+
+
+def random_blocks(ty, nblocks, seed):
+    """Random bytes with sane scale fields (finite f16 / f32 in the positions that hold them)."""
+    rng = np.random.default_rng(seed)
+    nbytes = {3: 20, 12: 144, 13: 176, 14: 210, 15: 292}[ty]
+    b = rng.integers(0, 256, (nblocks, nbytes), dtype=np.uint8)
+    halves = {3: (0, 2), 12: (0, 2), 13: (0, 2), 14: (208,), 15: ()}[ty]
+    for off in halves:
+        b[:, off:off + 2] = (rng.normal(0, 0.05, nblocks).astype(np.float16)).view(np.uint8).reshape(nblocks, 2)
+    if ty == 15:
+        b[:, 0:4] = rng.normal(0, 0.05, nblocks).astype(np.float32).view(np.uint8).reshape(nblocks, 4)
+    return b.reshape(-1)
+
+
+@pytest.mark.parametrize("ty", [3, 12, 13, 14, 15])
+def test_dequantisers_on_random_blocks_and_closed_forms(fh, gg, go, oracle, ty):
+    per = 32 if ty == 3 else 256
+    raw = random_blocks(ty, 37, 50 + ty)
+    out = dq(fh, go, oracle, ty, raw, 37 * per)
+    assert np.all(np.isfinite(out))
+    # a ragged element count stops inside the last block
+    assert np.array_equal(dq(fh, go, oracle, ty, raw, 36 * per + 5), out[:36 * per + 5])
+    # an element-by-element float64 evaluation of the format's definition, independent of both implementations
+    b = raw.reshape(37, -1)[3]
+    h = lambda o: float(np.frombuffer(bytes(b[o:o + 2]), np.float16)[0])
+    want = np.zeros(per)
+    if ty == 3:
+        for j in range(16):
+            want[j] = (int(b[4 + j]) & 15) * h(0) + h(2)
+            want[j + 16] = (int(b[4 + j]) >> 4) * h(0) + h(2)
+    elif ty in (12, 13):
+        sc = b[4:16]
+        for j in range(8):
+            sc = [int(x) for x in b[4:16]]
+            s, m = (sc[j] & 63, sc[j + 4] & 63) if j < 4 else ((sc[j + 4] & 15) | ((sc[j - 4] >> 6) << 4), (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4))
+            qs = b[(48 if ty == 13 else 16):]
+            for l in range(32):
+                q = int(qs[(j // 2) * 32 + l])
+                v = (q >> 4) if j % 2 else (q & 15)
+                if ty == 13 and (int(b[16 + l]) >> j) & 1:
+                    v += 16
+                want[j * 32 + l] = h(0) * s * v - h(2) * m
+    elif ty == 14:
+        ql, qh, sc, d = b[:128], b[128:192], b[192:208].view(np.int8), h(208)
+        for e in range(256):
+            half, r = divmod(e, 128)
+            k, l = divmod(r, 32)
+            lo = int(ql[64 * half + l + (32 if k in (1, 3) else 0)])
+            nib = (lo >> 4) if k >= 2 else (lo & 15)
+            hi2 = (int(qh[32 * half + l]) >> (2 * k)) & 3
+            want[e] = d * int(sc[8 * half + 2 * k + l // 16]) * ((nib | (hi2 << 4)) - 32)
+    else:
+        scale = float(np.frombuffer(bytes(b[:4]), np.float32)[0])
+        want = scale * b[4:260].view(np.int8).astype(np.float64)
+    assert np.allclose(out[3 * per:4 * per], want, rtol=1e-5, atol=1e-6)
+
+
+def test_unsupported_type_for_dequant(fh, gg):
+    with pytest.raises(fh.ForgeHipError):
+        gg.dequant_ggml(11, np.zeros(110, np.uint8), 256)
+
+
+def test_k_quant_tensors_are_read_as_q8_0_like_the_reference_loader_does(fh, gg, go, oracle):
+    """A Q8_0 model file in which the embedding is Q6_K (what llama.cpp writes into many files), one projection Q5_K, one
+    Q4_K, one Q4_1 and the output matrix Q6_K: each becomes Q8_0 blocks on load (weight_loader.rs:219-229), the f32
+    embedding table is the dequantised Q8_0 form (main.rs:2700-2705).  Library == oracle byte for byte; and the
+    closed form: requantised tensor == quantize_q8_0(dequant(raw))."""
+    cfg = fh.synth.tiny(Q8, max_seq=640, hidden=256, inter=512, vocab=1024)
+    blob = fh.synth.make_weights_blob(cfg, seed=15)
+    t = gg.split_blob(cfg, blob)
+    H, V = cfg["hidden"], cfg["vocab"]
+    swaps = {"token_embd.weight": gg.Q6_K, "output.weight": gg.Q6_K, "blk.0.ffn_up.weight": gg.Q5_K, "blk.1.attn_q.weight": gg.Q4_K,
+             "blk.1.ffn_down.weight": gg.Q4_1, "blk.0.attn_k.weight": gg.Q8_K}
+    raws = {}
+    for i, (name, ty) in enumerate(swaps.items()):
+        n = int(np.prod(t[name][0]))
+        per = 32 if ty == 3 else 256
+        raws[name] = random_blocks(ty, n // per, 70 + i)
+        t[name] = (t[name][0], ty, raws[name])
+    meta = [("general.architecture", gg.STRING, "llama"), ("llama.embedding_length", gg.U32, H), ("llama.block_count", gg.U32, cfg["layers"]),
+            ("llama.attention.head_count", gg.U32, cfg["heads"]), ("llama.attention.head_count_kv", gg.U32, cfg["kv_heads"]),
+            ("llama.feed_forward_length", gg.U32, cfg["inter"]), ("llama.vocab_size", gg.U32, V), ("llama.context_length", gg.U32, 640),
+            ("llama.attention.layer_norm_rms_epsilon", gg.FLOAT32, cfg["rms_eps"]), ("llama.rope.freq_base", gg.FLOAT32, cfg["rope_theta"])]
+    data = gg.write_gguf(meta, [(n, d, g, b) for n, (d, g, b) in t.items()])
+    f = gg.GgufFile(data)
+    got = f.config()
+    assert (got["wdtype"], got["lm_head_dtype"]) == (Q8, Q8)
+    o = go.parse(data)
+    assert go.config(o) == got
+    out = f.export_weights(got)
+    assert np.array_equal(out, go.export_weights(oracle, o, data, got))
+    parts = gg.split_blob(got, out)
+    for name, ty in swaps.items():
+        n = int(np.prod(t[name][0]))
+        q8 = oracle.quantize_weights(Q8, gg.dequant_ggml(ty, raws[name], n))
+        if name == "token_embd.weight":
+            assert np.array_equal(parts[name][2].view(np.float32), oracle.dequant(Q8, q8, n))
+        else:
+            assert np.array_equal(parts[name][2], q8), name
 
 
 @pytest.mark.gpu
