@@ -128,12 +128,12 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         for (int b = 0; b < KB; b++) {
             const uint32_t v = sc_is_a ? __builtin_amdgcn_raw_buffer_load_b16(ras, sc_voff + b * 2 + (k0 / 32) * 2, 0, 0)
                                        : __builtin_amdgcn_raw_buffer_load_b16(rws, sc_voff + b * 2 + (k0 / 32) * 2, 0, 0);
-            rs[b] = (k0 / 32 + b < nblk) ? (v & 0xFFFFu) : 0u;
+            rs[b] = v;              // looked at only when the stage is committed: nothing at the start of a stage waits for it
         }
     };
 
     // what passes through registers: expanded Q4_0 codes and the scales
-    auto commit_stage = [&](uint32_t buf, uint32_t slot) {
+    auto commit_stage = [&](uint32_t buf, uint32_t slot, uint32_t blk0) {
         if (Q4) {
 #pragma unroll
             for (int i = 0; i < 2; i++) {
@@ -160,9 +160,13 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                 *reinterpret_cast<v4i*>(base + ((q4_blk * 2 + 1) ^ sw) * 16) = hi;   // elements 16..31
             }
         }
+        // blocks past the end of K (they hold the next row's scales) count with scale 0
+        uint32_t sc4[KB];
+#pragma unroll
+        for (int b = 0; b < KB; b++) sc4[b] = (blk0 + b < nblk) ? (rs[b] & 0xFFFFu) : 0u;
         uint2 pk;
-        pk.x = rs[0] | (rs[1] << 16);
-        pk.y = rs[2] | (rs[3] << 16);
+        pk.x = sc4[0] | (sc4[1] << 16);
+        pk.y = sc4[2] | (sc4[3] << 16);
         if (MAGIC && !sc_is_a) { pk.x ^= 0x80000000u; pk.y ^= 0x80000000u; }   // odd blocks: minus sign on the weight scale
         *reinterpret_cast<uint2*>(lds + (sc_is_a ? LDS_ASC : LDS_BSC) + slot * SC_SLOT + sc_row * SC_ROW) = pk;
     };
@@ -225,7 +229,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
 
     const uint32_t stages = (K + BK - 1) / BK;
     issue_stage(0, 0);
-    commit_stage(0, 0);
+    commit_stage(0, 0, 0);
     __builtin_amdgcn_s_waitcnt(0);      // vmcnt(0): the tiles of stage 0 are in LDS
     __syncthreads();
 
@@ -290,7 +294,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                 __builtin_amdgcn_sched_barrier(0);   // keep the tiles in this order: one tile of temporaries ahead, no more
             }
         }
-        commit_stage(buf ^ 1, (s + 1) & 3);
+        commit_stage(buf ^ 1, (s + 1) & 3, (s + 1) * KB);
         __builtin_amdgcn_s_waitcnt(0);   // this wave's share of stage s+1 has landed
         __syncthreads();
     };
