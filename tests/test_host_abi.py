@@ -127,3 +127,53 @@ def test_errors_are_codes_not_crashes(fh):
     if fh.device_count() == 0:
         rc = L.forge_hip_model_create(C.byref(c), blob.ctypes.data_as(C.c_void_p), blob.size, C.byref(h))
         assert rc == fh.ERR_NO_DEVICE                     # metal:4212 `expect("no Metal device found")`
+
+
+def test_header_is_plain_c_and_the_library_links_from_c(fh, tmp_path):
+    """include/forge_hip.h compiles as strict C99, and a C program linked against the library calls its host-side
+    entry points (no GPU involved): f16 conversion, the GGUF parser on a buffer in memory, the sampler."""
+    import shutil
+    import subprocess
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler")
+    src = tmp_path / "abi.c"
+    src.write_text(r'''
+#include <stdio.h>
+#include <string.h>
+#include "forge_hip.h"
+int main(void) {
+    /* GGUF v3 header with no metadata and no tensors */
+    unsigned char g[24];
+    unsigned int magic = 0x46554747u, version = 3u;
+    unsigned long long zero = 0;
+    forge_hip_gguf* f = 0;
+    forge_hip_config cfg;
+    float logits[4] = {0.1f, 2.0f, 2.0f, -1.0f};
+    uint64_t state = 1;
+    uint32_t tok = 99;
+    memcpy(g, &magic, 4); memcpy(g + 4, &version, 4); memcpy(g + 8, &zero, 8); memcpy(g + 16, &zero, 8);
+    if (forge_hip_f32_to_f16(1.0f) != 0x3C00 || forge_hip_f16_to_f32(0xC000) != -2.0f) return 1;
+    if (forge_hip_gguf_parse(g, sizeof g, &f) != FORGE_HIP_OK) return 2;
+    if (forge_hip_gguf_version(f) != 3 || forge_hip_gguf_tensor_count(f) != 0 || forge_hip_gguf_tensor_data_offset(f) != 32) return 3;
+    if (forge_hip_gguf_config(f, 0, 0, &cfg) != FORGE_HIP_ERR_INVALID) return 4;      /* no architecture key */
+    if (strstr(forge_hip_last_error(), "unsupported GGUF architecture") == 0) return 5;
+    forge_hip_gguf_close(f);
+    g[0] = 0;
+    if (forge_hip_gguf_parse(g, sizeof g, &f) != FORGE_HIP_ERR_INVALID || f != 0) return 6;
+    if (forge_hip_sample(logits, 4, 0.0f, 0, 0.9f, &state, &tok) != FORGE_HIP_OK || tok != 2 || state != 1) return 7;
+    if (forge_hip_model_create(0, 0, 0, 0) == FORGE_HIP_OK) return 8;
+    printf("ok\n");
+    return 0;
+}
+''')
+    exe = tmp_path / "abi"
+    inc = os.path.join(ROOT, "include")
+    libdir = os.path.dirname(fh.LIB_PATH)
+    r = subprocess.run([gcc, "-std=c99", "-pedantic", "-Wall", "-Wextra", "-Werror", "-I", inc, str(src), "-o", str(exe),
+                        "-L", libdir, "-lforge_hip", "-Wl,-rpath," + libdir, "-Wl,-rpath,/opt/rocm/lib"],
+                       capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    env = dict(os.environ, LD_LIBRARY_PATH=libdir + ":/opt/rocm/lib:" + os.environ.get("LD_LIBRARY_PATH", ""))
+    r = subprocess.run([str(exe)], capture_output=True, text=True, env=env, timeout=120)
+    assert r.returncode == 0 and r.stdout.strip() == "ok", (r.returncode, r.stdout, r.stderr)
