@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libforge_hip.so")
 Q4_0 = 2
 Q8_0 = 8
 FLAG_EXACT = 1   # config.flags / op flags: order-faithful f32 arithmetic (bit-identical to the CPU path)
+FLAG_QKV_BIAS = 2   # config.flags: q, k, v projections add a bias vector before RoPE (Qwen2); the blob carries the vectors
 
 OK = 0
 ERR_INVALID = -1

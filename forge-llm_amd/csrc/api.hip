@@ -221,7 +221,7 @@ int32_t forge_hip_rope_kv_store(float* q_dev, float* k_dev, const float* v_dev, 
     const float* cos_t = reinterpret_cast<const float*>(g_rope.p);
     const float* sin_t = cos_t + (size_t)n_pos * half;
     launch_rope_kv_store(q_dev, k_dev, v_dev, heads * head_dim, kv_heads * head_dim, k_cache_dev, v_cache_dev, M,
-                         base_pos, nullptr, heads, kv_heads, head_dim, cos_t, sin_t, (hipStream_t)stream);
+                         base_pos, nullptr, heads, kv_heads, head_dim, cos_t, sin_t, nullptr, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }

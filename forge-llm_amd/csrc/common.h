@@ -99,7 +99,7 @@ void launch_silu_mul(const float* gate, const float* up, uint32_t M, uint32_t I,
 // (pos_dev ? *pos_dev : base_pos) + r.  q/k/v rows have strides q_stride/kv_stride floats.
 void launch_rope_kv_store(float* q, float* k, const float* v, uint32_t q_stride, uint32_t kv_stride, uint16_t* kc,
                           uint16_t* vc, uint32_t M, uint32_t base_pos, const uint32_t* pos_dev, uint32_t heads,
-                          uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, hipStream_t s);
+                          uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, const float* bias, hipStream_t s);
 void launch_embedding(const float* table, const uint32_t* tokens_dev, uint32_t M, uint32_t H, float* out, uint32_t* counts,
                       hipStream_t s);
 // Index of the LAST maximum.  `scratch` needs 2*ARGMAX_BLOCKS uint32/float pairs.
@@ -122,7 +122,7 @@ bool gemv_silu_fusable(uint32_t K);
 void launch_gemv_norm(const QWeight& w, const float* x, const float* norm_w, float eps, float* y, GemvOrder order,
                       hipStream_t s);
 // fused [q;k;v] matrix: q rows -> q_out (rotated), k rows -> K cache (rotated, fp16), v rows -> V cache, at *pos_dev
-void launch_gemv_norm_rope_kv(const QWeight& wqkv, const float* x, const float* norm_w, float eps, float* q_out,
+void launch_gemv_norm_rope_kv(const QWeight& wqkv, const float* x, const float* norm_w, float eps, const float* bias, float* q_out,
                               uint16_t* kc, uint16_t* vc, const float* cos_t, const float* sin_t,
                               const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s);
 // fused [gate;up] matrix: quant(silu(gate)*up) -> (oq, osc)

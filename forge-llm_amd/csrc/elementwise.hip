@@ -142,7 +142,9 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(float* __restrict__ 
                                                             const uint32_t* __restrict__ pos_dev, uint32_t heads,
                                                             uint32_t kv_heads, uint32_t hd,
                                                             const float* __restrict__ cos_t,
-                                                            const float* __restrict__ sin_t) {
+                                                            const float* __restrict__ sin_t,
+                                                            const float* __restrict__ bias) {
+    // bias (optional): q | k | v bias vectors, added before the rotation (Qwen2, emit.rs:4105-4120)
     const uint32_t r = blockIdx.y;
     const uint32_t pos = (pos_dev ? *pos_dev : base_pos) + r;
     const uint32_t half = hd / 2;
@@ -153,6 +155,7 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(float* __restrict__ 
         const float c = cos_t[(size_t)pos * half + i], s = sin_t[(size_t)pos * half + i];
         float2* ptr = reinterpret_cast<float2*>(q + (size_t)r * q_stride) + p;
         float2 x = *ptr;
+        if (bias) { x.x = x.x + bias[2 * p]; x.y = x.y + bias[2 * p + 1]; }
         float2 o;
         o.x = __fsub_rn(__fmul_rn(x.x, c), __fmul_rn(x.y, s));
         o.y = __fadd_rn(__fmul_rn(x.x, s), __fmul_rn(x.y, c));
@@ -162,6 +165,7 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(float* __restrict__ 
         const float c = cos_t[(size_t)pos * half + i], s = sin_t[(size_t)pos * half + i];
         float2* ptr = reinterpret_cast<float2*>(k + (size_t)r * kv_stride) + pk;
         float2 x = *ptr;
+        if (bias) { x.x = x.x + bias[2 * qp + 2 * pk]; x.y = x.y + bias[2 * qp + 2 * pk + 1]; }
         float2 o;
         o.x = __fsub_rn(__fmul_rn(x.x, c), __fmul_rn(x.y, s));
         o.y = __fadd_rn(__fmul_rn(x.x, s), __fmul_rn(x.y, c));
@@ -171,6 +175,7 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(float* __restrict__ 
     } else if (p < qp + 2 * kp) {
         const uint32_t pv = p - qp - kp;
         float2 x = reinterpret_cast<const float2*>(v + (size_t)r * kv_stride)[pv];
+        if (bias) { x.x = x.x + bias[2 * (qp + kp) + 2 * pv]; x.y = x.y + bias[2 * (qp + kp) + 2 * pv + 1]; }
         uint32_t packed = (uint32_t)f32_to_f16_bits(x.x) | ((uint32_t)f32_to_f16_bits(x.y) << 16);
         reinterpret_cast<uint32_t*>(vc + (size_t)pos * kv_heads * hd)[pv] = packed;
     }
@@ -178,12 +183,12 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(float* __restrict__ 
 
 void launch_rope_kv_store(float* q, float* k, const float* v, uint32_t q_stride, uint32_t kv_stride, uint16_t* kc,
                           uint16_t* vc, uint32_t M, uint32_t base_pos, const uint32_t* pos_dev, uint32_t heads,
-                          uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, hipStream_t s) {
+                          uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, const float* bias, hipStream_t s) {
     if (M == 0) return;
     uint32_t per_row = (heads + 2 * kv_heads) * hd / 2;
     dim3 grid((per_row + 255) / 256, M);
     fh::launch(rope_kv_store_kernel, grid, 256, 0, s, q, k, v, q_stride, kv_stride, kc, vc, base_pos, pos_dev, heads, kv_heads,
-                                              hd, cos_t, sin_t);
+                                              hd, cos_t, sin_t, bias);
 }
 
 // ---- embedding (emit.rs:585-589) -----------------------------------------------------------------

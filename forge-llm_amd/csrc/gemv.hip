@@ -68,6 +68,7 @@ struct GemvArgs {
     const float* cos_t;
     const float* sin_t;
     const uint32_t* pos_dev;
+    const float* bias;       // optional: q | k | v bias, added before the rotation (Qwen2, emit.rs:4105-4120)
     uint32_t qks, kv, hd;
     // Epi::SiluQuant: rows [0,I) gate, [I,2I) up -> oq int8 [I], osc fp16 [I/32]
     int8_t* oq;
@@ -279,6 +280,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
             if (active) a.y[row] = a.y[row] + r;
         } else if (EPI == Epi::RopeKv) {
             // rows 2i, 2i+1 of a head sit in lanes 2i, 2i+1 (row_base and rc are even)
+            if (a.bias && active) r = r + a.bias[row];
             const float other = __shfl_xor(r, 1, WAVE);
             if (active) {
                 const uint32_t pos = *a.pos_dev;
@@ -423,12 +425,13 @@ void launch_gemv_norm(const QWeight& w, const float* x, const float* norm_w, flo
     dispatch<Pro::RmsNorm, Epi::Store>(w.wdtype, a, s);
 }
 
-void launch_gemv_norm_rope_kv(const QWeight& wqkv, const float* x, const float* norm_w, float eps, float* q_out,
+void launch_gemv_norm_rope_kv(const QWeight& wqkv, const float* x, const float* norm_w, float eps, const float* bias, float* q_out,
                               uint16_t* kc, uint16_t* vc, const float* cos_t, const float* sin_t,
                               const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s) {
     GemvArgs a = base_args(wqkv, GemvOrder::MatmulVec);
     a.x = x; a.norm_w = norm_w; a.eps = eps;
     a.q_out = q_out; a.kc = kc; a.vc = vc; a.cos_t = cos_t; a.sin_t = sin_t; a.pos_dev = pos_dev;
+    a.bias = bias;
     a.qks = heads * hd; a.kv = kv_heads * hd; a.hd = hd;
     a.nseg = 3;
     a.seg[0] = make_segment(wqkv.wdtype, wqkv.K, 0, a.qks, false);

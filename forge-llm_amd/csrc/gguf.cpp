@@ -488,9 +488,11 @@ int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_
     FH_CHECK(g && out, "gguf_config: null argument");
     const MetaValue* arch_v = g->find("general.architecture");
     const std::string arch = arch_v && arch_v->type == 8 ? arch_v->str : "unknown";
-    // The kernels here cover the plain Llama layer: no QKV bias (qwen2), no GeLU or embedding scale (gemma), no fused
-    // QKV (phi3).  Mistral is that layer plus an optional sliding window.
-    if (arch != "llama" && arch != "mistral") return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: unsupported GGUF architecture: " + arch);
+    // The kernels here cover the Llama layer, with the QKV bias of Qwen2 (main.rs:770: the bias goes with the
+    // architecture): no GeLU or embedding scale (gemma), no fused QKV (phi3).  Mistral is the Llama layer plus an optional
+    // sliding window.
+    if (arch != "llama" && arch != "mistral" && arch != "qwen2")
+        return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: unsupported GGUF architecture: " + arch);
     const std::string p = arch + ".";
     uint32_t hidden = 0, layers = 0, heads = 0, kv_heads = 0, inter = 0;
     g->get_u32(p + "embedding_length", &hidden);
@@ -558,7 +560,8 @@ int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_
     c.head_dim = hidden / heads;                     // main.rs:731
     c.vocab = (uint32_t)vocab; c.max_seq = (uint32_t)seq;
     c.rms_eps = eps; c.rope_theta = theta;
-    c.wdtype = wdtype; c.lm_head_dtype = lm; c.flags = flags;
+    c.wdtype = wdtype; c.lm_head_dtype = lm;
+    c.flags = flags | (arch == "qwen2" ? FORGE_HIP_FLAG_QKV_BIAS : 0u);
     *out = c;
     return FORGE_HIP_OK;
 }
@@ -583,6 +586,11 @@ int32_t forge_hip_gguf_export_weights(const forge_hip_gguf* g, const forge_hip_c
         FH_STEP(write_quantised(g, blk(l, "attn_q.weight"), wt, QKS * H, p), qbytes(wt, QKS * H));
         FH_STEP(write_quantised(g, blk(l, "attn_k.weight"), wt, KV * H, p), qbytes(wt, KV * H));
         FH_STEP(write_quantised(g, blk(l, "attn_v.weight"), wt, KV * H, p), qbytes(wt, KV * H));
+        if (c->flags & FORGE_HIP_FLAG_QKV_BIAS) {             // main.rs:2737-2742
+            FH_STEP(write_f32(g, blk(l, "attn_q.bias"), QKS, p), QKS * 4);
+            FH_STEP(write_f32(g, blk(l, "attn_k.bias"), KV, p), KV * 4);
+            FH_STEP(write_f32(g, blk(l, "attn_v.bias"), KV, p), KV * 4);
+        }
         FH_STEP(write_quantised(g, blk(l, "attn_output.weight"), wt, H * QKS, p), qbytes(wt, H * QKS));
         FH_STEP(write_f32(g, blk(l, "ffn_norm.weight"), H, p), H * 4);
         FH_STEP(write_quantised(g, blk(l, "ffn_gate.weight"), wt, I * H, p), qbytes(wt, I * H));

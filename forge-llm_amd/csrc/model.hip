@@ -28,6 +28,7 @@ struct Layer {
     float* attn_norm = nullptr;
     float* ffn_norm = nullptr;
     QWeight qkv, o, gate_up, down;
+    float* qkv_bias = nullptr;           // [QKS + 2 KV]: q | k | v bias, in the row order of the fused qkv matrix (FLAG_QKV_BIAS)
 };
 
 struct DevBuf {
@@ -52,6 +53,7 @@ struct forge_hip_model {
     uint32_t H = 0, I = 0, QKS = 0, KV = 0, QKV = 0, KMAX = 0;
     hipStream_t stream = nullptr;
     DevBuf embed, final_norm, norms;     // norms: [layers][2][H]
+    DevBuf biases;                       // [layers][QKS + 2 KV] f32 (FLAG_QKV_BIAS)
     std::vector<Layer> layers;
     QWeight lm_head;
     DevBuf kcache, vcache;               // fp16 [layers][max_seq][KV]
@@ -159,7 +161,7 @@ int32_t validate(const forge_hip_config* c) {
     FH_CHECK(c->layers >= 1 && c->vocab >= 1 && c->max_seq >= 1, "layers, vocab and max_seq must be positive");
     FH_CHECK(c->heads >= 1 && c->kv_heads >= 1 && c->heads % c->kv_heads == 0, "heads must be a positive multiple of kv_heads");
     FH_CHECK(attn_head_dim_supported(c->head_dim), "head_dim must be 64, 96 or 128");
-    FH_CHECK((c->flags & ~FORGE_HIP_FLAG_EXACT) == 0, "unknown bits in flags");
+    FH_CHECK((c->flags & ~(FORGE_HIP_FLAG_EXACT | FORGE_HIP_FLAG_QKV_BIAS)) == 0, "unknown bits in flags");
     // The reference switches to its non-flash attention (a different summation order) when
     // max_seq_len <= 512 (emit.rs:126-128); the order-faithful kernels follow the flash variants only.
     FH_CHECK(!(c->flags & FORGE_HIP_FLAG_EXACT) || c->max_seq > 512, "FORGE_HIP_FLAG_EXACT needs max_seq > 512");
@@ -204,7 +206,7 @@ void enqueue_decode_layer(forge_hip_model* m, uint32_t l) {
     const GemvOrder mv = GemvOrder::MatmulVec;
     if (m->fuse_norm) {
         StageMark t(m, ST_QKV);
-        launch_gemv_norm_rope_kv(L.qkv, x, L.attn_norm, c.rms_eps, qkv, m->kc(l), m->vc(l), m->cos_t.as<float>(),
+        launch_gemv_norm_rope_kv(L.qkv, x, L.attn_norm, c.rms_eps, L.qkv_bias, qkv, m->kc(l), m->vc(l), m->cos_t.as<float>(),
                                  m->sin_t.as<float>(), m->d_pos(), c.heads, c.kv_heads, c.head_dim, s);
         // q now sits compact in qkv[0, QKS)
     } else {
@@ -213,7 +215,7 @@ void enqueue_decode_layer(forge_hip_model* m, uint32_t l) {
         {
             StageMark t(m, ST_ROPE);
             launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), 1, 0, m->d_pos(), c.heads,
-                                 c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), s);
+                                 c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s);
         }
     }
     enqueue_decode_attention(m, l, qkv, QKS);
@@ -246,7 +248,7 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
     {
         StageMark t(m, ST_ROPE);
         launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos, nullptr, c.heads,
-                             c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), s);
+                             c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s);
     }
     if (exact) {
         { StageMark t(m, ST_ATTN); launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, s); }
@@ -346,7 +348,8 @@ uint64_t forge_hip_weights_nbytes(const forge_hip_config* c) {
     if (!c) return 0;
     const uint64_t H = c->hidden, I = c->inter, QKS = (uint64_t)c->heads * c->head_dim, KV = (uint64_t)c->kv_heads * c->head_dim;
     const uint64_t per_layer = H * 4 + wsize(c->wdtype, QKS, H) + 2 * wsize(c->wdtype, KV, H) + wsize(c->wdtype, H, QKS) +
-                               H * 4 + 2 * wsize(c->wdtype, I, H) + wsize(c->wdtype, H, I);
+                               H * 4 + 2 * wsize(c->wdtype, I, H) + wsize(c->wdtype, H, I) +
+                               ((c->flags & FORGE_HIP_FLAG_QKV_BIAS) ? (QKS + 2 * KV) * 4 : 0);
     return (uint64_t)c->vocab * H * 4 + c->layers * per_layer + H * 4 + wsize(c->lm_head_dtype, c->vocab, H);
 }
 
@@ -386,6 +389,11 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
     rc = m->norms.alloc((size_t)cfg->layers * 2 * H * 4);
     if (rc) return rc;
     m->layers.resize(cfg->layers);
+    const bool has_bias = (cfg->flags & FORGE_HIP_FLAG_QKV_BIAS) != 0;
+    if (has_bias) {
+        rc = m->biases.alloc((size_t)cfg->layers * m->QKV * 4);
+        if (rc) return rc;
+    }
     const uint32_t wt = cfg->wdtype;
     for (uint32_t l = 0; l < cfg->layers; l++) {
         Layer& L = m->layers[l];
@@ -397,6 +405,11 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
         rc = qweight_upload(wt, p, H, m->QKV, &L.qkv);
         if (rc) return rc;
         p += wsize(wt, m->QKV, H);
+        if (has_bias) {                                       // q_bias | k_bias | v_bias, project.rs:286-292
+            L.qkv_bias = m->biases.as<float>() + (size_t)l * m->QKV;
+            FH_HIP(hipMemcpy(L.qkv_bias, p, (size_t)m->QKV * 4, hipMemcpyHostToDevice));
+            p += (size_t)m->QKV * 4;
+        }
         rc = qweight_upload(wt, p, QKS, H, &L.o);
         if (rc) return rc;
         p += wsize(wt, H, QKS);
@@ -451,7 +464,8 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
         (rc = m->ptok.alloc((size_t)R * 4)))
         return rc;
     const char* penv = getenv("FORGE_HIP_PERSIST");
-    if (!(penv && penv[0] == '0')) {
+    // a model with QKV bias decodes with the kernel sequence (the resident kernel has no bias in its qkv epilogue)
+    if (!(penv && penv[0] == '0') && !has_bias) {
         std::vector<PdLayerIn> pl(cfg->layers);
         for (uint32_t l = 0; l < cfg->layers; l++) {
             Layer& L = m->layers[l];

@@ -92,6 +92,10 @@ def split_blob(cfg: dict, blob: np.ndarray) -> dict:
         take(f"blk.{l}.attn_q.weight", QKS, H, wt)
         take(f"blk.{l}.attn_k.weight", KV, H, wt)
         take(f"blk.{l}.attn_v.weight", KV, H, wt)
+        if cfg.get("flags", 0) & 2:
+            take(f"blk.{l}.attn_q.bias", 1, QKS, F32)
+            take(f"blk.{l}.attn_k.bias", 1, KV, F32)
+            take(f"blk.{l}.attn_v.bias", 1, KV, F32)
         take(f"blk.{l}.attn_output.weight", H, QKS, wt)
         take(f"blk.{l}.ffn_norm.weight", 1, H, F32)
         take(f"blk.{l}.ffn_gate.weight", I, H, wt)
@@ -103,12 +107,14 @@ def split_blob(cfg: dict, blob: np.ndarray) -> dict:
     return out
 
 
-def model_to_gguf(cfg: dict, blob: np.ndarray, tied: bool = True, arch: str = "llama", path=None, tokens: bool = False) -> bytes:
+def model_to_gguf(cfg: dict, blob: np.ndarray, tied: bool = True, arch: str = None, path=None, tokens: bool = False) -> bytes:
     """A weights blob as a GGUF v3 file with the metadata keys load_config reads (main.rs:700-830).
     tied=True stores the embedding once, as the quantised `token_embd.weight` (what llama.cpp does for models with tied
     embeddings; the blob's f32 table must then be the dequantised lm_head, as `synth.make_weights_blob` makes it);
     tied=False stores the f32 table and `output.weight`.  tokens=True also writes a `tokenizer.ggml.tokens` array of
     `vocab` one-character strings, the key the vocabulary size is read from first."""
+    if arch is None:
+        arch = "qwen2" if cfg.get("flags", 0) & 2 else "llama"       # the reference ties QKV bias to the architecture
     t = split_blob(cfg, blob)
     if tied:
         dims, gtype, data = t.pop("output.weight")

@@ -107,11 +107,14 @@ def make_weights_blob(cfg: dict, seed: int, std: float = 0.02, norm_jitter: floa
     lm_raw = qmat(cfg["vocab"], H, lt)
     embed = dequant(lt, lm_raw, cfg["vocab"] * H)
     parts.append(embed.view(np.uint8))
+    has_bias = bool(cfg.get("flags", 0) & 2)
     for _ in range(cfg["layers"]):
         parts.append(norm_vec().view(np.uint8))
         parts.append(qmat(QKS, H, wt))
         parts.append(qmat(KV, H, wt))
         parts.append(qmat(KV, H, wt))
+        if has_bias:                                        # q_bias | k_bias | v_bias, f32 (project.rs:286-292)
+            parts.append(normal(sub_seed(), QKS + 2 * KV, 0.5, 1).astype(np.float32).view(np.uint8))
         parts.append(qmat(H, QKS, wt))
         parts.append(norm_vec().view(np.uint8))
         parts.append(qmat(I, H, wt))
@@ -120,7 +123,8 @@ def make_weights_blob(cfg: dict, seed: int, std: float = 0.02, norm_jitter: floa
     parts.append(norm_vec().view(np.uint8))
     parts.append(lm_raw)
     blob = np.concatenate(parts)
-    expect = (cfg["vocab"] * H * 4 + cfg["layers"] * (2 * H * 4 + (QKS * H + 2 * KV * H + H * QKS + 3 * I * H) // 32 * block_bytes(wt))
+    expect = (cfg["vocab"] * H * 4 + cfg["layers"] * (2 * H * 4 + (QKS * H + 2 * KV * H + H * QKS + 3 * I * H) // 32 * block_bytes(wt)
+                                                       + ((QKS + 2 * KV) * 4 if has_bias else 0))
               + H * 4 + cfg["vocab"] * H // 32 * block_bytes(lt))
     assert blob.size == expect, (blob.size, expect)
     return blob

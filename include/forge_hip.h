@@ -41,6 +41,10 @@ extern "C" {
  * prefill GEMM fuses its per-block multiply-add and attention runs on the MFMA / split-sequence
  * kernels: same integer block sums, f32 results within rel 1e-3 / abs 1e-3, much faster. */
 #define FORGE_HIP_FLAG_EXACT 1u
+/* Bit for config.flags only.  QKV_BIAS: the q, k and v projections add a bias vector before RoPE (Qwen2,
+ * emit.rs:3906-3915, 4105-4120) and the weights blob carries, per layer after the v weights, q_bias [heads*head_dim],
+ * k_bias and v_bias [kv_heads*head_dim] as f32 (project.rs:286-292).  Such a model decodes with the kernel sequence. */
+#define FORGE_HIP_FLAG_QKV_BIAS 2u
 
 #define FORGE_HIP_Q4_0 2u /* GGML type ids, crates/forgellm-frontend/src/gguf.rs:207-258 */
 #define FORGE_HIP_Q8_0 8u
@@ -52,7 +56,7 @@ typedef struct forge_hip_config {
     float rms_eps, rope_theta;
     uint32_t wdtype;        /* projection weights: FORGE_HIP_Q8_0 or FORGE_HIP_Q4_0 */
     uint32_t lm_head_dtype; /* same coding */
-    uint32_t flags;         /* 0 or FORGE_HIP_FLAG_EXACT */
+    uint32_t flags;         /* FORGE_HIP_FLAG_EXACT, FORGE_HIP_FLAG_QKV_BIAS, both or neither */
 } forge_hip_config;
 
 typedef struct forge_hip_model forge_hip_model;
@@ -195,7 +199,8 @@ int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void
  * The reference reads a model from a GGUF file in three steps: gguf::parse (crates/forgellm-frontend/src/gguf.rs:484-551),
  * load_config (crates/forgellm-cli/src/main.rs:700-830) and `forge export-weights` (main.rs:2585-2757, tensor names
  * mapped by weight_loader.rs:400-447), whose output file is the blob forge_hip_model_create takes.  These entry points are
- * those three steps.  Supported: architectures "llama" and "mistral" (without a sliding window shorter than max_seq);
+ * those three steps.  Supported: architectures "llama", "qwen2" (sets FORGE_HIP_FLAG_QKV_BIAS) and "mistral" (without a sliding
+ * window shorter than max_seq);
  * tensors of GGML type F32, F16, BF16, Q8_0, Q4_0 and -- turned into Q8_0 blocks when they are read, as the reference's loader
  * does (weight_loader.rs:219-229) -- Q4_1, Q4_K, Q5_K, Q6_K, Q8_K; projections mostly Q8_0 or mostly Q4_0 by the reference's
  * majority vote, which counts those other types as Q8_0 (a file whose projections are mostly Q4_K is refused: the reference

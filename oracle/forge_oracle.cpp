@@ -593,11 +593,12 @@ struct fo_config {
     float rms_eps, rope_theta;
     uint32_t wdtype;        // 8 = Q8_0, 2 = Q4_0 (GGML type ids)
     uint32_t lm_head_dtype; // same coding
-    uint32_t flags;
+    uint32_t flags;         // bit 1 (value 2): the blob carries QKV bias vectors (Qwen2, emit.rs:3906-3915)
 };
 
 struct fo_layer {
     const float* attn_norm; const uint8_t *q, *k, *v, *o; const float* ffn_norm; const uint8_t *gate, *up, *down;
+    const float *q_bias = nullptr, *k_bias = nullptr, *v_bias = nullptr;      // project.rs:286-292: after the v weights
 };
 
 struct fo_model {
@@ -616,7 +617,7 @@ static int64_t wsize(uint32_t dtype, int64_t n, int64_t k) { return n * ((k + QK
 uint64_t fo_weights_nbytes(const fo_config* c) {
     int64_t H = c->hidden, I = c->inter, QKS = (int64_t)c->heads * c->head_dim, KV = (int64_t)c->kv_heads * c->head_dim;
     int64_t per_layer = H * 4 + wsize(c->wdtype, QKS, H) + 2 * wsize(c->wdtype, KV, H) + wsize(c->wdtype, H, QKS) + H * 4 +
-                        2 * wsize(c->wdtype, I, H) + wsize(c->wdtype, H, I);
+                        2 * wsize(c->wdtype, I, H) + wsize(c->wdtype, H, I) + ((c->flags & 2u) ? (QKS + 2 * KV) * 4 : 0);
     return (uint64_t)((int64_t)c->vocab * H * 4 + c->layers * per_layer + H * 4 + wsize(c->lm_head_dtype, c->vocab, H));
 }
 
@@ -634,6 +635,11 @@ fo_model* fo_model_create(const fo_config* c, const uint8_t* blob, uint64_t nbyt
         L.q = p; p += wsize(c->wdtype, QKS, H);
         L.k = p; p += wsize(c->wdtype, KV, H);
         L.v = p; p += wsize(c->wdtype, KV, H);
+        if (c->flags & 2u) {
+            L.q_bias = (const float*)p; p += QKS * 4;
+            L.k_bias = (const float*)p; p += KV * 4;
+            L.v_bias = (const float*)p; p += KV * 4;
+        }
         L.o = p; p += wsize(c->wdtype, H, QKS);
         L.ffn_norm = (const float*)p; p += H * 4;
         L.gate = p; p += wsize(c->wdtype, I, H);
@@ -691,6 +697,11 @@ int fo_forward(fo_model* m, uint32_t token, float* logits) {
         matmul_vec(c.wdtype, m->variant, q.data(), normed.data(), L.q, H, QKS, 0);
         matmul_vec(c.wdtype, m->variant, k.data(), normed.data(), L.k, H, KV, 0);
         matmul_vec(c.wdtype, m->variant, v.data(), normed.data(), L.v, H, KV, 0);
+        if (L.q_bias) {                                       // emit.rs:4105-4120
+            for (int64_t i = 0; i < QKS; i++) q[i] += L.q_bias[i];
+            for (int64_t i = 0; i < KV; i++) k[i] += L.k_bias[i];
+            for (int64_t i = 0; i < KV; i++) v[i] += L.v_bias[i];
+        }
         rope(q.data(), pos, c.head_dim, c.heads, m->freqs.data());
         rope(k.data(), pos, c.head_dim, c.kv_heads, m->freqs.data());
         store_kv(m, l, pos, k.data(), v.data());
@@ -730,6 +741,11 @@ int fo_prefill_batched(fo_model* m, const uint32_t* tokens, int64_t n, float* lo
         matmul_mat(c.wdtype, m->variant, k.data(), n, normed.data(), L.k, H, KV);
         matmul_mat(c.wdtype, m->variant, v.data(), n, normed.data(), L.v, H, KV);
         for (int64_t r = 0; r < n; r++) {
+            if (L.q_bias) {                                   // emit.rs:5246-5260
+                for (int64_t i = 0; i < QKS; i++) q[r * QKS + i] += L.q_bias[i];
+                for (int64_t i = 0; i < KV; i++) k[r * KV + i] += L.k_bias[i];
+                for (int64_t i = 0; i < KV; i++) v[r * KV + i] += L.v_bias[i];
+            }
             rope(&q[r * QKS], base + r, c.head_dim, c.heads, m->freqs.data());
             rope(&k[r * KV], base + r, c.head_dim, c.kv_heads, m->freqs.data());
             store_kv(m, l, base + r, &k[r * KV], &v[r * KV]);

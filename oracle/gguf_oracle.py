@@ -122,7 +122,7 @@ def _get(g, key, types):
 
 def config(g, max_seq=0, flags=0) -> dict:
     arch = _get(g, "general.architecture", (8,)) or "unknown"
-    if arch not in ("llama", "mistral"):
+    if arch not in ("llama", "mistral", "qwen2"):
         raise GgufError(f"unsupported GGUF architecture: {arch}")
     p = arch + "."
     hidden = _get(g, p + "embedding_length", (4,)) or 0
@@ -186,7 +186,8 @@ def config(g, max_seq=0, flags=0) -> dict:
     f = np.float32
     return {"hidden": hidden, "inter": inter, "layers": layers, "heads": heads, "kv_heads": kv, "head_dim": hidden // heads,
             "vocab": vocab, "max_seq": seq, "rms_eps": float(f(1e-5) if eps is None else f(eps)),
-            "rope_theta": float(f(10000.0) if theta is None else f(theta)), "wdtype": wd, "lm_head_dtype": lm, "flags": flags}
+            "rope_theta": float(f(10000.0) if theta is None else f(theta)), "wdtype": wd, "lm_head_dtype": lm,
+            "flags": flags | (2 if arch == "qwen2" else 0)}                  # qkv_bias goes with the architecture, main.rs:770
 
 
 F = np.float32
@@ -309,7 +310,10 @@ def export_weights(oracle, g, data, cfg) -> np.ndarray:
     for l in range(cfg["layers"]):
         b = f"blk.{l}."
         parts += [f32(b + "attn_norm.weight", H), quant(b + "attn_q.weight", QKS * H, wd), quant(b + "attn_k.weight", KV * H, wd),
-                  quant(b + "attn_v.weight", KV * H, wd), quant(b + "attn_output.weight", H * QKS, wd), f32(b + "ffn_norm.weight", H),
+                  quant(b + "attn_v.weight", KV * H, wd)]
+        if cfg["flags"] & 2:
+            parts += [f32(b + "attn_q.bias", QKS), f32(b + "attn_k.bias", KV), f32(b + "attn_v.bias", KV)]
+        parts += [quant(b + "attn_output.weight", H * QKS, wd), f32(b + "ffn_norm.weight", H),
                   quant(b + "ffn_gate.weight", I * H, wd), quant(b + "ffn_up.weight", I * H, wd), quant(b + "ffn_down.weight", H * I, wd)]
     parts.append(f32("output_norm.weight", H))
     lm_name = "output.weight" if "output.weight" in by_name else "lm_head.weight" if "lm_head.weight" in by_name else "token_embd.weight"

@@ -173,9 +173,13 @@ def test_parse_errors(fh, gg, go):
 
 @pytest.mark.parametrize("wd", [Q8, Q4])
 @pytest.mark.parametrize("tied", [True, False])
-def test_synthetic_model_round_trip(fh, gg, go, oracle, wd, tied, tmp_path):
-    """blob -> GGUF file -> (library) config + blob: identical bytes, identical configuration; same through the oracle."""
+@pytest.mark.parametrize("bias", [False, True])
+def test_synthetic_model_round_trip(fh, gg, go, oracle, wd, tied, bias, tmp_path):
+    """blob -> GGUF file -> (library) config + blob: identical bytes, identical configuration; same through the oracle.
+    bias: a Qwen2-style model (architecture qwen2, bias vectors after the v weights)."""
     cfg = fh.synth.tiny(wd, max_seq=640)
+    if bias:
+        cfg["flags"] = fh.FLAG_QKV_BIAS
     blob = fh.synth.make_weights_blob(cfg, seed=11)
     path = str(tmp_path / "m.gguf")
     data = gg.model_to_gguf(cfg, blob, tied=tied, path=path, tokens=tied)
@@ -186,7 +190,7 @@ def test_synthetic_model_round_trip(fh, gg, go, oracle, wd, tied, tmp_path):
         assert np.float32(got["rms_eps"]) == np.float32(cfg["rms_eps"]) and np.float32(got["rope_theta"]) == np.float32(cfg["rope_theta"])
         out = f.export_weights(got)
         assert out.size == blob.size and np.array_equal(out, blob)
-        assert f.config(max_seq=128, flags=1)["max_seq"] == 128 and f.config(max_seq=128, flags=1)["flags"] == 1
+        assert f.config(max_seq=128, flags=1)["max_seq"] == 128 and f.config(max_seq=128, flags=1)["flags"] == 1 | cfg.get("flags", 0)
         f.close()
     o = go.parse(data)
     ocfg = go.config(o)
@@ -262,7 +266,11 @@ def test_config_defaults_and_refusals(fh, gg, go):
         with pytest.raises(go.GgufError):
             go.config(go.parse(data))
 
-    refused([("general.architecture", gg.STRING, "qwen2")] + base[1:], text="unsupported GGUF architecture: qwen2")
+    refused([("general.architecture", gg.STRING, "gemma")] + base[1:], text="unsupported GGUF architecture: gemma")
+    # qwen2: the QKV bias goes with the architecture (main.rs:770)
+    qmeta = [("general.architecture", gg.STRING, "qwen2")] + [(k.replace("llama.", "qwen2."), t, v) for k, t, v in base[1:]]
+    cq = gg.GgufFile(make(qmeta)).config()
+    assert cq["flags"] == fh.FLAG_QKV_BIAS and cq == go.config(go.parse(make(qmeta)))
     refused(base[1:], text="unsupported GGUF architecture: unknown")
     refused(base[:2], text="could not extract model config")
     # get_u32 takes a Uint32 value only (gguf.rs:306-308): the same key as u64 does not count
@@ -511,6 +519,15 @@ def test_model_from_gguf_equals_model_from_blob(fh, gg, torch_gpu, tmp_path):
             assert ta == tb
             tok = ta
         assert np.array_equal(a.read_kv(1, 0), b.read_kv(1, 0))
+        a.close(); b.close()
+        # a Qwen2-style file (QKV bias): same check
+        cfgb = dict(cfg, flags=fh.FLAG_QKV_BIAS)
+        blobb = fh.synth.make_weights_blob(cfgb, seed=16)
+        pathb = str(tmp_path / f"b{wd}.gguf")
+        gg.model_to_gguf(cfgb, blobb, tied=True, path=pathb)
+        a, b = fh.HipModel(cfgb, blobb), fh.HipModel.from_gguf(pathb)
+        assert b.config["flags"] == fh.FLAG_QKV_BIAS
+        assert np.array_equal(a.forward_prefill(prompt).view(np.uint32), b.forward_prefill(prompt).view(np.uint32))
         a.close(); b.close()
         # a smaller cache than the file's context length, and the exact mode
         c = fh.HipModel.from_gguf(path, max_seq=600, flags=fh.FLAG_EXACT)
