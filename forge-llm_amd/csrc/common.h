@@ -177,7 +177,7 @@ struct PdState;
 // Leaves *out null (returning OK) when the shape or device is not covered; `state` = {position, token, next token, abort flag}.
 int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layers, const QWeight& lm_head, const float* embed,
                   const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, uint32_t* counts,
-                  PdState** out);
+                  const float* qkv_bias, PdState** out);
 int32_t pd_set_repeat_penalty(PdState* st, float penalty);
 void pd_destroy(PdState* st);
 int32_t pd_enqueue(PdState* st, bool profile, uint32_t token, hipStream_t s);

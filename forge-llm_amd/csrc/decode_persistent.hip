@@ -113,6 +113,7 @@ struct PdArgs {
     uint32_t host_seq;
     uint32_t q4, lm_q4;                        // weight formats: projections, lm_head
     uint32_t* counts;                          // u32 [vocab]: times each token id has been fed (this step's token is added here)
+    const float* qkv_bias;                     // optional [layers][QKS + 2 KV]: added to q, k, v before the rotation (Qwen2)
     float penalty;                             // > 1: the argmax is taken over the penalised logits
     uint32_t use_hint;                         // pollers wait for one watched element before re-reading a whole buffer
     uint32_t off_act_s, off_misc, off_big;     // LDS byte offsets (activation codes sit at 0)
@@ -368,6 +369,7 @@ struct GemvJob {
     uint32_t res_tag;          // EPI_ADD: tag of the residual's current version (0: embedding row)
     uint16_t* kc;              // EPI_ROPE
     uint16_t* vc;
+    const float* bias;         // EPI_ROPE, optional: this layer's q | k | v bias (emit.rs:4105-4120)
 };
 
 struct WReg { int4 v[PD_D]; uint32_t s[PD_D]; };
@@ -847,6 +849,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
             float v = 0.f;
             if (mine) v = ORDERED ? ordered_sum(big + cx.tid * pstride, h.nblk, segment_row_is_dot1(row, g.seg, g.nseg, g.tail_mod)) : (big[cx.tid * 4] + big[cx.tid * 4 + 1]) + (big[cx.tid * 4 + 2] + big[cx.tid * 4 + 3]);
             if (job.epi == EPI_ROPE) {
+                if (PEN && job.bias && mine) v = v + job.bias[row];      // the kernel variant with the optional extras carries it
                 // rope (emit.rs:508-528): rows 2i, 2i+1 of a head sit in neighbouring lanes
                 const float other = __shfl_xor(v, 1, WAVE);
                 if (mine) {
@@ -994,6 +997,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         job.tag_out = is_lm ? 0 : base + (ph == 0 ? 1u : ph == 1 ? 4u : ph == 2 ? 5u : 6u);
         job.res_tag = ph == 1 ? x_in : base + 4;
         job.kc = a.layers[l].kc;
+        job.bias = (PEN && a.qkv_bias && ph == 0) ? a.qkv_bias + (size_t)l * (a.QKS + 2 * a.KV) : nullptr;
         job.vc = a.layers[l].vc;
         if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
         else pd_gemv_phase<false, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
@@ -1097,12 +1101,12 @@ const void* pd_kernel_ord(const PdState* st) {
     if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2, ORD, PEN>);
     return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 1, ORD, PEN>) : reinterpret_cast<const void*>(decode_step_kernel<HD, 0, ORD, PEN>);
 }
-// The repeat penalty is code of its own in the lm_head epilogue: the default kernel is built without it (the ordered
-// variants always carry it).
+// The repeat penalty (lm_head epilogue) and the QKV bias (qkv epilogue) are code of their own: the default kernel is
+// built without them (the ordered variants always carry them).
 template <int HD>
 const void* pd_kernel(const PdState* st) {
     if (st->ordered) return pd_kernel_ord<HD, true, true>(st);
-    return st->args.penalty > 1.0f ? pd_kernel_ord<HD, false, true>(st) : pd_kernel_ord<HD, false, false>(st);
+    return (st->args.penalty > 1.0f || st->args.qkv_bias) ? pd_kernel_ord<HD, false, true>(st) : pd_kernel_ord<HD, false, false>(st);
 }
 template <int HD>
 hipError_t launch_pd_hd(const PdState* st, hipStream_t s) {
@@ -1119,7 +1123,7 @@ void pd_destroy(PdState* st) { delete st; }
 // device is outside what the kernel covers; the caller then keeps the multi-kernel step.
 int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layers, const QWeight& lm_head, const float* embed,
                   const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, uint32_t* counts,
-                  PdState** out) {
+                  const float* qkv_bias, PdState** out) {
     *out = nullptr;
     if (c.flags & FORGE_HIP_FLAG_EXACT) return FORGE_HIP_OK;
     if (c.head_dim != 64 && c.head_dim != 128) return FORGE_HIP_OK;
@@ -1132,6 +1136,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
 
     std::unique_ptr<PdState> st(new PdState());
     PdArgs& a = st->args;
+    a.qkv_bias = qkv_bias;                 // selects the kernel variant: before the residency check below
     const uint32_t H = c.hidden, I = c.inter, hd = c.head_dim, QKS = c.heads * hd, KV = c.kv_heads * hd;
     const uint32_t kmax = std::max(std::max(H, I), QKS);
     const uint32_t gsize = c.heads / c.kv_heads;

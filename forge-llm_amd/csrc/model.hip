@@ -464,15 +464,15 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
         (rc = m->ptok.alloc((size_t)R * 4)))
         return rc;
     const char* penv = getenv("FORGE_HIP_PERSIST");
-    // a model with QKV bias decodes with the kernel sequence (the resident kernel has no bias in its qkv epilogue)
-    if (!(penv && penv[0] == '0') && !has_bias) {
+    if (!(penv && penv[0] == '0')) {
         std::vector<PdLayerIn> pl(cfg->layers);
         for (uint32_t l = 0; l < cfg->layers; l++) {
             Layer& L = m->layers[l];
             pl[l] = PdLayerIn{&L.qkv, &L.o, &L.gate_up, &L.down, L.attn_norm, L.ffn_norm, m->kc(l), m->vc(l)};
         }
         rc = pd_create(*cfg, pl, m->lm_head, m->embed.as<float>(), m->final_norm.as<float>(), m->cos_t.as<float>(),
-                       m->sin_t.as<float>(), m->logits.as<float>(), m->state.as<uint32_t>(), m->counts.as<uint32_t>(), &m->pd);
+                       m->sin_t.as<float>(), m->logits.as<float>(), m->state.as<uint32_t>(), m->counts.as<uint32_t>(),
+                       has_bias ? m->biases.as<float>() : nullptr, &m->pd);
         if (rc) return rc;
     }
     FH_HIP(hipDeviceSynchronize());

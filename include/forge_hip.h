@@ -43,7 +43,7 @@ extern "C" {
 #define FORGE_HIP_FLAG_EXACT 1u
 /* Bit for config.flags only.  QKV_BIAS: the q, k and v projections add a bias vector before RoPE (Qwen2,
  * emit.rs:3906-3915, 4105-4120) and the weights blob carries, per layer after the v weights, q_bias [heads*head_dim],
- * k_bias and v_bias [kv_heads*head_dim] as f32 (project.rs:286-292).  Such a model decodes with the kernel sequence. */
+ * k_bias and v_bias [kv_heads*head_dim] as f32 (project.rs:286-292). */
 #define FORGE_HIP_FLAG_QKV_BIAS 2u
 
 #define FORGE_HIP_Q4_0 2u /* GGML type ids, crates/forgellm-frontend/src/gguf.rs:207-258 */
