@@ -196,7 +196,7 @@ def main():
     ap.add_argument("--no-alt", action="store_true", help="skip the second model that measures the kernel-sequence decode step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (known HBM traffic, for scaling counter readings)")
-    ap.add_argument("--model", choices=("llama32_1b", "llama32_3b", "smollm2_135m"), default="llama32_1b",
+    ap.add_argument("--model", choices=("llama32_1b", "llama32_3b", "smollm2_135m", "llama31_8b", "qwen25_1p5b"), default="llama32_1b",
                     help="shape of the synthetic model (default: the one the headline metric is quoted on)")
     ap.add_argument("--format", choices=("q8_0", "q4_0"), default="q8_0", help="weight format (default: the headline's)")
     ap.add_argument("--ops-table", action="store_true",
@@ -216,7 +216,8 @@ def main():
     wd = fh.Q8_0 if args.format == "q8_0" else fh.Q4_0
     cfg = getattr(fh.synth, args.model)(wd, max_seq=4096)
     headline = args.model == "llama32_1b" and args.format == "q8_0"
-    model_name = {"llama32_1b": "Llama-3.2-1B", "llama32_3b": "Llama-3.2-3B", "smollm2_135m": "SmolLM2-135M"}[args.model]
+    model_name = {"llama32_1b": "Llama-3.2-1B", "llama32_3b": "Llama-3.2-3B", "smollm2_135m": "SmolLM2-135M", "llama31_8b": "Llama-3.1-8B",
+                  "qwen25_1p5b": "Qwen2.5-1.5B"}[args.model]
     t0 = time.perf_counter()
     blob = fh.synth.make_weights_blob(cfg, seed=args.seed, threads=16)
     t_gen = time.perf_counter() - t0

@@ -80,6 +80,18 @@ def llama32_3b(wdtype=8, max_seq=4096):
     return _cfg(3072, 8192, 28, 24, 8, 128, 128256, max_seq, 500000.0, wdtype)
 
 
+def llama31_8b(wdtype=8, max_seq=4096):
+    return _cfg(4096, 14336, 32, 32, 8, 128, 128256, max_seq, 500000.0, wdtype)
+
+
+def qwen25_1p5b(wdtype=8, max_seq=4096):
+    """Qwen2.5-1.5B shape: QKV bias, 12 heads over 2 KV heads, head_dim 128, vocabulary 151 936."""
+    c = _cfg(1536, 8960, 28, 12, 2, 128, 151936, max_seq, 1000000.0, wdtype)
+    c["flags"] = 2
+    c["rms_eps"] = 1e-6
+    return c
+
+
 def tiny(wdtype=8, max_seq=640, hidden=256, inter=512, layers=2, heads=4, kv_heads=2, head_dim=64, vocab=1000):
     return _cfg(hidden, inter, layers, heads, kv_heads, head_dim, vocab, max_seq, 10000.0, wdtype)
 
