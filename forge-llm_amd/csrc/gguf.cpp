@@ -239,7 +239,7 @@ int32_t locate(const forge_hip_gguf* g, const std::string& name, uint64_t numel,
         return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor " + name + " has " + std::to_string(t->numel()) + " elements, the configuration needs " +
                                                std::to_string(numel));
     const uint64_t start = g->tensor_data_offset + t->offset, size = t->data_size();
-    if (start > g->nbytes || size > g->nbytes - start)
+    if (t->offset > g->nbytes || start > g->nbytes || size > g->nbytes - start)
         return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor " + name + " extends past end of file");      // weight_loader.rs:172-177
     out->t = t;
     out->bytes = g->data + start;

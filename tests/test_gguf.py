@@ -328,6 +328,33 @@ def test_export_errors(fh, gg):
         gg.GgufFile("/nonexistent/dir/model.gguf")
 
 
+def test_damaged_files_are_refused_or_read_but_never_crash(fh, gg):
+    """Random byte damage to a small valid model file: parsing, configuration and export each either succeed or come
+    back with an error code (the process survives; nothing is read outside the buffer)."""
+    cfg = fh.synth.tiny(Q8, max_seq=640, hidden=64, inter=64, layers=1, heads=1, kv_heads=1, head_dim=64, vocab=64)
+    blob = fh.synth.make_weights_blob(cfg, seed=17)
+    good = bytearray(gg.model_to_gguf(cfg, blob, tied=False, tokens=True))
+    head = gg.GgufFile(bytes(good)).tensor_data_offset
+    rng = np.random.default_rng(5)
+    outcomes = {"ok": 0, "refused": 0}
+    for trial in range(600):
+        data = bytearray(good)
+        for _ in range(int(rng.integers(1, 4))):
+            pos = int(rng.integers(0, head))                  # damage the header, metadata and descriptors
+            data[pos] = int(rng.integers(0, 256))
+        if trial % 5 == 0:
+            data = data[:int(rng.integers(0, len(data)))]
+        try:
+            f = gg.GgufFile(bytes(data))
+            c = f.config()
+            if fh.hip_model.weights_nbytes(c) < (1 << 26):    # a damaged size field may ask for gigabytes: skip those
+                f.export_weights(c)
+            outcomes["ok"] += 1
+        except fh.ForgeHipError:
+            outcomes["refused"] += 1
+    assert outcomes["refused"] > 50 and outcomes["ok"] > 5, outcomes
+
+
 # ---------------- the other block formats the reference's loader reads ----------------
 def f16le(bits):
     return struct.pack("<H", bits)
