@@ -283,6 +283,11 @@ def test_config_defaults_and_refusals(fh, gg, go):
     ck = gg.GgufFile(make(base, kq)).config()
     assert (ck["wdtype"], ck["lm_head_dtype"]) == (Q8, Q8) and ck == go.config(go.parse(make(base, kq)))
     refused(base + [("llama.attention.sliding_window", gg.U32, 1024)], text="sliding-window")
+    # a window that covers the whole cache is the same attention up to rounding: accepted, but not in exact mode
+    wide = gg.GgufFile(make(base + [("llama.attention.sliding_window", gg.U32, 4096)]))
+    assert wide.config()["max_seq"] == 2048
+    with pytest.raises(fh.ForgeHipError, match="sliding window"):
+        wide.config(flags=fh.FLAG_EXACT)
     # the vote: 2 x Q4_0 against 1 x Q8_0
     vote = (("blk.0.attn_q.weight", [64, 64], gg.Q4_0, None), ("blk.0.attn_k.weight", [64, 64], gg.Q4_0, None),
             ("blk.0.ffn_up.weight", [64, 64], gg.Q8_0, None), ("blk.0.attn_norm.weight", [64], gg.F32, None),
