@@ -1214,6 +1214,8 @@ e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, hd == 64 ? pd_kernel<6
     a.taq2 = t; t += n_taq2;
     a.tpart = t;
     a.tag_base = 0;
+    // FORGE_HIP_PD_TAG_START: start the tag sequence elsewhere (a test starts it just below the point where it is rewound)
+    { const char* e = getenv("FORGE_HIP_PD_TAG_START"); if (e) a.tag_base = (uint32_t)strtoul(e, nullptr, 0); }
     a.spin_limit = 400000;
     a.q4 = st->q4; a.lm_q4 = st->lmq4;
     { const char* e = getenv("FORGE_HIP_PD_HINT"); a.use_hint = (e && e[0] == '0') ? 0 : 1; }

@@ -234,6 +234,23 @@ def test_persistent_decode_kernel_equals_kernel_sequence(fh, torch_gpu, monkeypa
     seq.close(); one.close()
 
 
+def test_persistent_decode_kernel_rewinds_its_tags(fh, torch_gpu, monkeypatch):
+    """The hand-over tags count up from launch to launch and are rewound (buffers cleared) before they could wrap:
+    started just below that point, the one-kernel model goes through the rewind within a few steps and keeps giving
+    the kernel sequence's bits."""
+    cfg = tiny_cfg(fh, Q8, 0)
+    blob = fh.synth.make_weights_blob(cfg, seed=43)
+    toks = fh.synth.uniform_ids(44, 16, cfg["vocab"])
+    monkeypatch.setenv("FORGE_HIP_PD_TAG_START", str(0xF0000000 - 30))      # 13 tags per launch for 2 layers
+    seq, one = persistent_pair(fh, cfg, blob, monkeypatch)
+    monkeypatch.delenv("FORGE_HIP_PD_TAG_START")
+    for t in toks:
+        same_bits(one.forward(int(t)), seq.forward(int(t)))
+    for which in (0, 1):
+        assert np.array_equal(one.read_kv(1, which), seq.read_kv(1, which))
+    seq.close(); one.close()
+
+
 @pytest.mark.parametrize("wd", [Q8, Q4])
 def test_persistent_decode_kernel_default_summation(fh, oracle, torch_gpu, monkeypatch, wd):
     """The default one-kernel step adds a row's block products as they come (per lane, then across the wave) instead of
