@@ -1217,6 +1217,9 @@ e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, hd == 64 ? pd_kernel<6
     // FORGE_HIP_PD_TAG_START: start the tag sequence elsewhere (a test starts it just below the point where it is rewound)
     { const char* e = getenv("FORGE_HIP_PD_TAG_START"); if (e) a.tag_base = (uint32_t)strtoul(e, nullptr, 0); }
     a.spin_limit = 400000;
+    // FORGE_HIP_PD_SPIN_LIMIT: how often a wait re-reads before the workgroup gives up (a test sets it to 1 to walk the
+    // give-up path: every wait in the kernel is bounded by it, so the kernel still ends normally)
+    { const char* e = getenv("FORGE_HIP_PD_SPIN_LIMIT"); if (e && atoi(e) > 0) a.spin_limit = (uint32_t)atoi(e); }
     a.q4 = st->q4; a.lm_q4 = st->lmq4;
     { const char* e = getenv("FORGE_HIP_PD_HINT"); a.use_hint = (e && e[0] == '0') ? 0 : 1; }
     a.token = 0; a.token_from_arg = 0; a.host_out = nullptr; a.host_seq = 0;

@@ -251,6 +251,28 @@ def test_persistent_decode_kernel_rewinds_its_tags(fh, torch_gpu, monkeypatch):
     seq.close(); one.close()
 
 
+def test_persistent_decode_kernel_gives_up_instead_of_hanging(fh, torch_gpu, monkeypatch):
+    """Every wait of the one-kernel step is bounded.  With the bound set to a single re-read the workgroups give up at
+    the first hand-over that is not there yet: the kernel ends, the call comes back with FORGE_HIP_ERR_HIP and a message,
+    and the device goes on working (a model created afterwards decodes as usual)."""
+    cfg = tiny_cfg(fh, Q8, 0)
+    blob = fh.synth.make_weights_blob(cfg, seed=45)
+    monkeypatch.setenv("FORGE_HIP_PERSIST", "1")
+    monkeypatch.setenv("FORGE_HIP_PD_SPIN_LIMIT", "1")
+    impatient = fh.HipModel(cfg, blob)
+    assert impatient.decode_launches == 1
+    with pytest.raises(fh.ForgeHipError) as e:
+        for t in range(8):                                   # the first steps may get through if every hand-over is on time
+            impatient.forward_greedy(t)
+    assert e.value.code == fh.ERR_HIP and "gave up waiting" in str(e.value)
+    impatient.close()
+    monkeypatch.delenv("FORGE_HIP_PD_SPIN_LIMIT")
+    seq, one = persistent_pair(fh, cfg, blob, monkeypatch)
+    for t in fh.synth.uniform_ids(46, 6, cfg["vocab"]):
+        same_bits(one.forward(int(t)), seq.forward(int(t)))
+    seq.close(); one.close()
+
+
 @pytest.mark.parametrize("wd", [Q8, Q4])
 def test_persistent_decode_kernel_default_summation(fh, oracle, torch_gpu, monkeypatch, wd):
     """The default one-kernel step adds a row's block products as they come (per lane, then across the wave) instead of
