@@ -33,7 +33,8 @@ EXPORTS = [
     "forge_hip_f32_to_f16", "forge_hip_quantize_f32", "forge_hip_expf_host", "forge_hip_dequant", "forge_hip_qweight_create",
     "forge_hip_qweight_destroy", "forge_hip_quantize_act", "forge_hip_gemv_q", "forge_hip_gemm_q",
     "forge_hip_block_isums", "forge_hip_rms_norm", "forge_hip_silu_mul", "forge_hip_rope_kv_store",
-    "forge_hip_attn_prefill_f16kv", "forge_hip_attn_decode_f16kv", "forge_hip_argmax",
+    "forge_hip_attn_prefill_f16kv", "forge_hip_attn_decode_f16kv",
+    "forge_hip_attn_prefill_sliding_f16kv", "forge_hip_attn_decode_sliding_f16kv", "forge_hip_argmax",
     "forge_hip_gguf_open", "forge_hip_gguf_parse", "forge_hip_gguf_close", "forge_hip_gguf_version", "forge_hip_gguf_alignment",
     "forge_hip_gguf_tensor_data_offset", "forge_hip_gguf_tensor_count", "forge_hip_gguf_metadata_count", "forge_hip_gguf_tensor",
     "forge_hip_gguf_find_tensor", "forge_hip_gguf_meta", "forge_hip_gguf_config", "forge_hip_gguf_export_weights",
@@ -54,6 +55,7 @@ class Config(C.Structure):
         ("kv_heads", C.c_uint32), ("head_dim", C.c_uint32), ("vocab", C.c_uint32), ("max_seq", C.c_uint32),
         ("rms_eps", C.c_float), ("rope_theta", C.c_float),
         ("wdtype", C.c_uint32), ("lm_head_dtype", C.c_uint32), ("flags", C.c_uint32),
+        ("sliding_window", C.c_uint32),
     ]
 
 
@@ -134,6 +136,10 @@ def lib():
     L.forge_hip_attn_prefill_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]
     L.forge_hip_attn_decode_f16kv.restype = i32
     L.forge_hip_attn_decode_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, vp]
+    L.forge_hip_attn_prefill_sliding_f16kv.restype = i32
+    L.forge_hip_attn_prefill_sliding_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]
+    L.forge_hip_attn_decode_sliding_f16kv.restype = i32
+    L.forge_hip_attn_decode_sliding_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, vp]
     L.forge_hip_argmax.restype = i32
     L.forge_hip_argmax.argtypes = [vp, u32, vp, vp]
     L.forge_hip_model_set_repeat_penalty.restype = i32

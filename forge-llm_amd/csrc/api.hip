@@ -245,7 +245,20 @@ int32_t forge_hip_attn_prefill_f16kv(const float* q_dev, const uint16_t* k_cache
                           nullptr, M, base_pos, nullptr, heads, kv_heads, head_dim, (hipStream_t)stream);
     else
         launch_attn_prefill(q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, M, base_pos,
-                            heads, kv_heads, head_dim, (hipStream_t)stream);
+                            heads, kv_heads, head_dim, 0u, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_attn_prefill_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
+                                             float* out_dev, uint32_t M, uint32_t base_pos, uint32_t window, uint32_t heads,
+                                             uint32_t kv_heads, uint32_t head_dim, void* stream) {
+    FH_CHECK(q_dev && k_cache_dev && v_cache_dev && out_dev, "attn_prefill_sliding: null pointer");
+    FH_CHECK(window >= 1, "attn_prefill_sliding: window must be at least 1");
+    int32_t rc = check_attn_shape("attn_prefill_sliding", heads, kv_heads, head_dim);
+    if (rc) return rc;
+    launch_attn_prefill(q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, M, base_pos, heads,
+                        kv_heads, head_dim, window, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }
@@ -265,8 +278,24 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
         rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
         if (rc) return rc;
         launch_attn_decode(q_dev, k_cache_dev, v_cache_dev, out_dev, nullptr, nullptr, seq_len, nullptr, heads, kv_heads,
-                           head_dim, g_attn.p, (hipStream_t)stream);
+                           head_dim, 0u, g_attn.p, (hipStream_t)stream);
     }
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_attn_decode_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
+                                            float* out_dev, uint32_t seq_len, uint32_t window, uint32_t heads,
+                                            uint32_t kv_heads, uint32_t head_dim, void* stream) {
+    FH_CHECK(q_dev && k_cache_dev && v_cache_dev && out_dev, "attn_decode_sliding: null pointer");
+    FH_CHECK(seq_len >= 1, "attn_decode_sliding: seq_len must be at least 1");
+    FH_CHECK(window >= 1, "attn_decode_sliding: window must be at least 1");
+    int32_t rc = check_attn_shape("attn_decode_sliding", heads, kv_heads, head_dim);
+    if (rc) return rc;
+    rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
+    if (rc) return rc;
+    launch_attn_decode(q_dev, k_cache_dev, v_cache_dev, out_dev, nullptr, nullptr, seq_len, nullptr, heads, kv_heads, head_dim,
+                       window, g_attn.p, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }

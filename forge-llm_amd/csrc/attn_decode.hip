@@ -39,7 +39,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const float* __r
                                                                 const uint16_t* __restrict__ vc,
                                                                 float* __restrict__ ws, uint32_t seq_len_arg,
                                                                 const uint32_t* __restrict__ pos_dev, uint32_t heads,
-                                                                uint32_t kv_heads, uint32_t gsize) {
+                                                                uint32_t kv_heads, uint32_t gsize, uint32_t window) {
     constexpr int LPK = HD <= 64 ? 8 : 16;   // lanes per key row
     constexpr int KPW = 64 / LPK;            // keys per wave load
     constexpr int REC = HD + 2;
@@ -56,9 +56,11 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const float* __r
     const float scale = 1.0f / sqrtf((float)HD);
     const uint32_t kv_stride = kv_heads * HD;
 
-    uint32_t chunk = (seq + nsplit - 1) / nsplit;
+    // attention_sliding (emit.rs:598-627): only the last `window` rows are keys (window 0: all of them)
+    const uint32_t start = (window != 0 && seq > window) ? seq - window : 0;
+    uint32_t chunk = (seq - start + nsplit - 1) / nsplit;
     chunk = (chunk + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
-    const uint32_t t0 = split * chunk;
+    const uint32_t t0 = min(seq, start + split * chunk);
     const uint32_t t1 = min(seq, t0 + chunk);
 
     float qf[GT][8];
@@ -188,30 +190,30 @@ bool attn_head_dim_supported(uint32_t hd) { return hd == 64 || hd == 96 || hd ==
 namespace {
 template <int HD, int GT>
 void launch_split(const float* q, const uint16_t* kc, const uint16_t* vc, float* ws, uint32_t seq,
-                  const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, hipStream_t s) {
+                  const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t window, hipStream_t s) {
     const uint32_t gsize = heads / kv_heads;
     dim3 grid(kv_heads * (gsize / GT), DECODE_SPLITS);
-    fh::launch(attn_decode_split_kernel<HD, GT>, grid, 256, 0, s, q, kc, vc, ws, seq, pos_dev, heads, kv_heads, gsize);
+    fh::launch(attn_decode_split_kernel<HD, GT>, grid, 256, 0, s, q, kc, vc, ws, seq, pos_dev, heads, kv_heads, gsize, window);
 }
 template <int HD>
 void launch_hd(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
-               uint32_t seq, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, float* ws, hipStream_t s) {
+               uint32_t seq, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t window, float* ws, hipStream_t s) {
     const uint32_t gsize = heads / kv_heads;
-    if (gsize % 4 == 0) launch_split<HD, 4>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
-    else if (gsize % 3 == 0) launch_split<HD, 3>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
-    else if (gsize % 2 == 0) launch_split<HD, 2>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
-    else launch_split<HD, 1>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, s);
+    if (gsize % 4 == 0) launch_split<HD, 4>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, s);
+    else if (gsize % 3 == 0) launch_split<HD, 3>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, s);
+    else if (gsize % 2 == 0) launch_split<HD, 2>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, s);
+    else launch_split<HD, 1>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, s);
     fh::launch(attn_decode_combine_kernel<HD>, heads, HD, 0, s, ws, DECODE_SPLITS, out, oq, osc);
 }
 }  // namespace
 
 void launch_attn_decode(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
                         uint32_t seq_len, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd,
-                        void* workspace, hipStream_t s) {
+                        uint32_t window, void* workspace, hipStream_t s) {
     float* ws = reinterpret_cast<float*>(workspace);
-    if (hd == 64) launch_hd<64>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, ws, s);
-    else if (hd == 96) launch_hd<96>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, ws, s);
-    else launch_hd<128>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, ws, s);
+    if (hd == 64) launch_hd<64>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, s);
+    else if (hd == 96) launch_hd<96>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, s);
+    else launch_hd<128>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, s);
 }
 
 }  // namespace fh

@@ -34,11 +34,13 @@ constexpr int AP_THREADS = 512;
 // QUANT: instead of f32 rows the kernel writes what the o projection's GEMM reads, the activation quantiser's int8
 // codes oq[M][heads*HD] and fp16 scales osc[M][heads*HD/32] of the same values (a 32-element block is one 32-wide
 // head_dim tile of one query: 16 values in this lane, 16 in lane ^ 32).
-template <int HD, bool QUANT>
+// WIN: sliding-window attention (attention_sliding_batch, emit.rs:907-1046): the query at position p sees the keys
+// [max(0, p - window + 1), p]; key tiles that lie before the window of the workgroup's first query are never loaded.
+template <int HD, bool QUANT, bool WIN>
 __global__ __launch_bounds__(AP_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
 void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
                          float* __restrict__ out, uint32_t q_stride, uint32_t out_stride, uint32_t M, uint32_t base_pos,
-                         uint32_t heads, uint32_t kv_heads, int8_t* __restrict__ oq, uint16_t* __restrict__ osc) {
+                         uint32_t heads, uint32_t kv_heads, int8_t* __restrict__ oq, uint16_t* __restrict__ osc, uint32_t window) {
     constexpr int KS = HD + 8;    // K tile row stride (halfs): 16-byte pad
     constexpr int VS = KT + 4;    // V^T tile row stride (halfs): 8-byte pad
     constexpr int KTOTAL = KT * HD / 8;          // 16-byte pieces of K per tile
@@ -97,6 +99,10 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
     const uint32_t wave_max_pos = base_pos + min(q0 + qg * QW + QW, M) - 1;   // may underflow if the group is empty
     const uint32_t wave_min_pos = base_pos + q0 + qg * QW;                    // position of the group's first query
     const bool wave_active = q0 + qg * QW < M;
+    // first key any query of the workgroup / of this wave's group may see
+    const uint32_t wg_lo = (WIN && base_pos + q0 + 1 > window) ? base_pos + q0 + 1 - window : 0;
+    const uint32_t wave_lo = (WIN && wave_min_pos + 1 > window) ? wave_min_pos + 1 - window : 0;
+    const uint32_t tile0 = wg_lo / KT;
 
     int4 kreg[KPIECES];
     uint2 va[VITEMS], vb[VITEMS];
@@ -138,14 +144,14 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
         }
     };
 
-    load_tile(0);
-    store_tile(0);
+    load_tile(tile0);
+    store_tile(tile0 & 1);
     __syncthreads();
-    for (uint32_t kt = 0; kt < ntiles; kt++) {
+    for (uint32_t kt = tile0; kt < ntiles; kt++) {
         const uint32_t buf = kt & 1;
         if (kt + 1 < ntiles) load_tile(kt + 1);          // in flight while this tile is computed
         const uint32_t k0 = kt * KT + kh * 32;            // this wave's 32 keys of the tile
-        if (wave_active && k0 <= wave_max_pos) {         // else they lie entirely in the group's future
+        if (wave_active && k0 <= wave_max_pos && k0 + 32 > wave_lo) {   // else they lie entirely in the group's future, or before every window
             const _Float16* Kb = Ks(buf);
             const _Float16* Vb = Vt(buf);
             // ---- S^T tile: sacc[r] = q . k for key k0 + 8(r/4) + 4 lh + r%4, query lq
@@ -158,7 +164,13 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], sacc, 0, 0, 0);
             }
             // ---- causal mask: only keys past the group's first query can be masked for some query
-            if (k0 + 31 > wave_min_pos) {
+            if (WIN) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const uint32_t t = k0 + 8 * (r >> 2) + 4 * lh + (r & 3);
+                    sacc[r] = (t <= qpos && t + window > qpos) ? sacc[r] : -INFINITY;
+                }
+            } else if (k0 + 31 > wave_min_pos) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const uint32_t t = k0 + 8 * (r >> 2) + 4 * lh + (r & 3);
@@ -225,8 +237,8 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
     if (kh == 1) return;
     {
         const float m1 = mg[0], l1 = mg[1];
-        const float m = fmaxf(m_run, m1);            // finite: key 0 is in the even wave's half and visible to every query
-        const float a0 = __builtin_amdgcn_exp2f(m_run - m), a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - m);
+        const float m = fmaxf(m_run, m1);            // finite: every query sees itself (without a window, key 0 in the even half too)
+        const float a0 = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - m), a1 = m1 == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m1 - m);
         l_run = l_run * a0 + l1 * a1;
 #pragma unroll
         for (int d = 0; d < ND; d++)
@@ -273,26 +285,41 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
     }
 }
 
+namespace {
+template <int HD, bool QUANT>
+void launch_win(dim3 grid, hipStream_t s, const float* q, const uint16_t* kc, const uint16_t* vc, float* out, uint32_t q_stride,
+                uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, int8_t* oq, uint16_t* osc,
+                uint32_t window) {
+    // a window that covers every key of the call is plain causal attention
+    if (window != 0 && window < base_pos + M)
+        fh::launch(attn_prefill_kernel<HD, QUANT, true>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window);
+    else
+        fh::launch(attn_prefill_kernel<HD, QUANT, false>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, 0u);
+}
+template <bool QUANT>
+void launch_hd(uint32_t hd, dim3 grid, hipStream_t s, const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
+               uint32_t q_stride, uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, int8_t* oq,
+               uint16_t* osc, uint32_t window) {
+    if (hd == 64) launch_win<64, QUANT>(grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window);
+    else if (hd == 96) launch_win<96, QUANT>(grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window);
+    else launch_win<128, QUANT>(grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window);
+}
+}  // namespace
+
 void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, float* out,
                          uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
-                         uint32_t hd, hipStream_t s) {
+                         uint32_t hd, uint32_t window, hipStream_t s) {
     if (M == 0) return;
     dim3 grid(((M + QB - 1) / QB) * heads);
-    int8_t* nq = nullptr;
-    uint16_t* ns = nullptr;
-    if (hd == 64) fh::launch(attn_prefill_kernel<64, false>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, nq, ns);
-    else if (hd == 96) fh::launch(attn_prefill_kernel<96, false>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, nq, ns);
-    else fh::launch(attn_prefill_kernel<128, false>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, nq, ns);
+    launch_hd<false>(hd, grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, nullptr, nullptr, window);
 }
 
 void launch_attn_prefill_quant(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, int8_t* oq, uint16_t* osc,
-                               uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s) {
+                               uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, uint32_t hd, uint32_t window,
+                               hipStream_t s) {
     if (M == 0) return;
     dim3 grid(((M + QB - 1) / QB) * heads);
-    float* no = nullptr;
-    if (hd == 64) fh::launch(attn_prefill_kernel<64, true>, grid, AP_THREADS, 0, s, q, kc, vc, no, q_stride, 0u, M, base_pos, heads, kv_heads, oq, osc);
-    else if (hd == 96) fh::launch(attn_prefill_kernel<96, true>, grid, AP_THREADS, 0, s, q, kc, vc, no, q_stride, 0u, M, base_pos, heads, kv_heads, oq, osc);
-    else fh::launch(attn_prefill_kernel<128, true>, grid, AP_THREADS, 0, s, q, kc, vc, no, q_stride, 0u, M, base_pos, heads, kv_heads, oq, osc);
+    launch_hd<true>(hd, grid, s, q, kc, vc, nullptr, q_stride, 0u, M, base_pos, heads, kv_heads, oq, osc, window);
 }
 
 }  // namespace fh

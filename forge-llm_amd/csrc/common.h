@@ -138,20 +138,23 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
 constexpr uint32_t DECODE_SPLITS = 32;
 size_t attn_decode_workspace_bytes(uint32_t heads, uint32_t hd);
 // seq_len = pos_dev ? *pos_dev + 1 : seq_len.  Writes f32 out if non-null and quantised (q, sc) if q non-null.
+// window != 0: only the last `window` rows are keys (attention_sliding, emit.rs:598-627).
 void launch_attn_decode(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
                         uint32_t seq_len, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd,
-                        void* workspace, hipStream_t s);
+                        uint32_t window, void* workspace, hipStream_t s);
 
 // attn_prefill.hip
 // q rows / out rows have strides q_stride / out_stride floats (q may live inside a fused qkv buffer).
+// window != 0: the query at position p sees keys [max(0, p - window + 1), p] (attention_sliding_batch, emit.rs:907-1046).
 void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, float* out,
                          uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
-                         uint32_t hd, hipStream_t s);
+                         uint32_t hd, uint32_t window, hipStream_t s);
 
 // The same attention, written as the activation quantiser's output of its rows: int8 codes oq[M][heads*hd] and fp16 scales
 // osc[M][heads*hd/32] (bit-identical to launch_attn_prefill followed by launch_quantize_act).
 void launch_attn_prefill_quant(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, int8_t* oq, uint16_t* osc,
-                               uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s);
+                               uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, uint32_t hd, uint32_t window,
+                               hipStream_t s);
 
 bool attn_head_dim_supported(uint32_t hd);
 

@@ -115,6 +115,7 @@ struct PdArgs {
     uint32_t* counts;                          // u32 [vocab]: times each token id has been fed (this step's token is added here)
     const float* qkv_bias;                     // optional [layers][QKS + 2 KV]: added to q, k, v before the rotation (Qwen2)
     float penalty;                             // > 1: the argmax is taken over the penalised logits
+    uint32_t window;                           // != 0: attention over the last `window` positions only (sliding window)
     uint32_t use_hint;                         // pollers wait for one watched element before re-reading a whole buffer
     uint32_t off_act_s, off_misc, off_big;     // LDS byte offsets (activation codes sit at 0)
     unsigned long long* stamps;                // optional: wall clock at the start of every phase (workgroup 0)
@@ -545,14 +546,16 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
     const bool dvalid = c * 8 < HD;
     const float scale = 1.0f / sqrtf((float)HD);
     const uint32_t kv_stride = a.KV;
-    uint32_t chunk = (seq + DECODE_SPLITS - 1) / DECODE_SPLITS;
+    // attention_sliding (emit.rs:598-627): only the last `window` rows are keys (window 0: all of them)
+    const uint32_t start = (a.window != 0 && seq > a.window) ? seq - a.window : 0;
+    uint32_t chunk = (seq - start + DECODE_SPLITS - 1) / DECODE_SPLITS;
     chunk = (chunk + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
 
     for (uint32_t item = cx.wg; item < n_items; item += cx.G) {
         const uint32_t bx = item % nbx, split = item / nbx;
         const uint32_t kvh = bx / gpk, sub = bx % gpk;
         const uint32_t h0 = kvh * gsize + sub * gt;
-        const uint32_t t0 = split * chunk;
+        const uint32_t t0 = min(seq, start + split * chunk);
         const uint32_t t1 = min(seq, t0 + chunk);
         const bool has_new = t0 <= pos && pos < t1;
         // The cached K/V rows do not depend on q: the first key blocks of this wave are requested before q is awaited (loads
@@ -1195,6 +1198,7 @@ e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, hd == 64 ? pd_kernel<6
     a.n_layers = (uint32_t)layers.size();
     a.H = H; a.I = I; a.QKS = QKS; a.KV = KV; a.heads = c.heads; a.kv_heads = c.kv_heads;
     a.eps = c.rms_eps;
+    a.window = c.sliding_window;
     a.embed = embed; a.final_norm = final_norm; a.cos_t = cos_t; a.sin_t = sin_t;
     a.logits = logits; a.state = state;
     a.counts = counts; a.penalty = 1.0f;

@@ -551,9 +551,8 @@ int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_
                                                        "; this library reads " + SUPPORTED_TYPES + " tensors");
     }
     const uint64_t seq = max_seq ? max_seq : ctx;
-    if (has_window && window < seq)
-        return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: sliding-window attention (window " + std::to_string(window) + ") is not supported for max_seq " +
-                                                   std::to_string(seq));
+    // Some(0) would make the reference attend to nothing (emit.rs:604-605)
+    if (has_window && window == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: a sliding window of 0 positions");
     // a model with a window runs `attention_sliding` in the reference (emit.rs:598-627, 4156-4170), a plain softmax over the
     // window: within the window it equals full attention up to rounding, but not bit for bit
     if (has_window && (flags & FORGE_HIP_FLAG_EXACT))
@@ -566,6 +565,7 @@ int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_
     c.rms_eps = eps; c.rope_theta = theta;
     c.wdtype = wdtype; c.lm_head_dtype = lm;
     c.flags = flags | (arch == "qwen2" ? FORGE_HIP_FLAG_QKV_BIAS : 0u);
+    c.sliding_window = has_window ? window : 0u;     // main.rs:764-767
     *out = c;
     return FORGE_HIP_OK;
 }

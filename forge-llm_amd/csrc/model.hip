@@ -165,6 +165,10 @@ int32_t validate(const forge_hip_config* c) {
     // The reference switches to its non-flash attention (a different summation order) when
     // max_seq_len <= 512 (emit.rs:126-128); the order-faithful kernels follow the flash variants only.
     FH_CHECK(!(c->flags & FORGE_HIP_FLAG_EXACT) || c->max_seq > 512, "FORGE_HIP_FLAG_EXACT needs max_seq > 512");
+    // a model with a window runs attention_sliding in the reference (emit.rs:598-627, 4156-4170): a plain softmax over the
+    // window, which the order-faithful kernels do not restate
+    FH_CHECK(!(c->flags & FORGE_HIP_FLAG_EXACT) || c->sliding_window == 0,
+             "FORGE_HIP_FLAG_EXACT is not available for a model with a sliding window");
     FH_CHECK(gemv_k_supported(c->hidden) && gemv_k_supported(c->inter) && gemv_k_supported(c->heads * c->head_dim),
              "hidden, inter and heads*head_dim must be at most 16384");
     return FORGE_HIP_OK;
@@ -184,7 +188,7 @@ void enqueue_decode_attention(forge_hip_model* m, uint32_t l, const float* q, ui
                               c.kv_heads, c.head_dim, s);
         else
             launch_attn_decode(q, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads, c.head_dim,
-                               m->attn_ws.p, s);
+                               c.sliding_window, m->attn_ws.p, s);
     }
     { StageMark t(m, ST_O); launch_gemv(m->layers[l].o, aq, asc, m->x.as<float>(), true, GemvOrder::MatmulVec, s); }
 }
@@ -256,9 +260,9 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
     } else if (m->prefill_fuse_quant) {
         // the attention kernel writes the o projection's quantised input itself
         StageMark t(m, ST_ATTN);
-        launch_attn_prefill_quant(qkv, QKV, m->kc(l), m->vc(l), aq, asc, M, base_pos, c.heads, c.kv_heads, c.head_dim, s);
+        launch_attn_prefill_quant(qkv, QKV, m->kc(l), m->vc(l), aq, asc, M, base_pos, c.heads, c.kv_heads, c.head_dim, c.sliding_window, s);
     } else {
-        { StageMark t(m, ST_ATTN); launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, s); }
+        { StageMark t(m, ST_ATTN); launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, c.sliding_window, s); }
         { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
     }
     { StageMark t(m, ST_O); launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s); }

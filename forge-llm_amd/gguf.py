@@ -114,7 +114,8 @@ def model_to_gguf(cfg: dict, blob: np.ndarray, tied: bool = True, arch: str = No
     tied=False stores the f32 table and `output.weight`.  tokens=True also writes a `tokenizer.ggml.tokens` array of
     `vocab` one-character strings, the key the vocabulary size is read from first."""
     if arch is None:
-        arch = "qwen2" if cfg.get("flags", 0) & 2 else "llama"       # the reference ties QKV bias to the architecture
+        # the reference ties QKV bias to the architecture; a window is Mistral's
+        arch = "qwen2" if cfg.get("flags", 0) & 2 else "mistral" if cfg.get("sliding_window", 0) else "llama"
     t = split_blob(cfg, blob)
     if tied:
         dims, gtype, data = t.pop("output.weight")
@@ -130,6 +131,8 @@ def model_to_gguf(cfg: dict, blob: np.ndarray, tied: bool = True, arch: str = No
         (f"{arch}.attention.layer_norm_rms_epsilon", FLOAT32, cfg["rms_eps"]),
         (f"{arch}.rope.freq_base", FLOAT32, cfg["rope_theta"]),
     ]
+    if cfg.get("sliding_window", 0):
+        meta.append((f"{arch}.attention.sliding_window", U32, cfg["sliding_window"]))
     if tokens:
         meta.append(("tokenizer.ggml.tokens", ARRAY, (STRING, [chr(33 + i % 90) for i in range(cfg["vocab"])])))
     else:

@@ -235,6 +235,35 @@ def attention_flash(q, k_cache, v_cache, seq_len, heads, kv_heads, head_dim, fla
     return out
 
 
+def attention_sliding_batch(q, k_cache, v_cache, base_pos, window, heads, kv_heads, head_dim):
+    """attention_sliding_batch over an fp16 cache: row r (position base_pos + r) sees the last `window` positions up to its own."""
+    from . import check, lib
+    torch = _torch()
+    q = _dev(q, torch.float32)
+    k_cache, v_cache = _dev(k_cache, torch.int16), _dev(v_cache, torch.int16)
+    M = q.shape[0]
+    if base_pos + M > k_cache.shape[0]:
+        raise ValueError("cache holds fewer than base_pos + M rows")
+    out = torch.empty_like(q)
+    check(lib().forge_hip_attn_prefill_sliding_f16kv(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), M, base_pos, window,
+                                                     heads, kv_heads, head_dim, _stream()))
+    return out
+
+
+def attention_sliding(q, k_cache, v_cache, seq_len, window, heads, kv_heads, head_dim):
+    """attention_sliding over an fp16 cache: one query f32 [heads*hd] against the last min(window, seq_len) of seq_len rows."""
+    from . import check, lib
+    torch = _torch()
+    q = _dev(q, torch.float32)
+    k_cache, v_cache = _dev(k_cache, torch.int16), _dev(v_cache, torch.int16)
+    if seq_len > k_cache.shape[0]:
+        raise ValueError("cache holds fewer than seq_len rows")
+    out = torch.empty_like(q)
+    check(lib().forge_hip_attn_decode_sliding_f16kv(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), seq_len, window, heads,
+                                                    kv_heads, head_dim, _stream()))
+    return out
+
+
 def argmax(x):
     from . import check, lib
     torch = _torch()

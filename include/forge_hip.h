@@ -57,6 +57,9 @@ typedef struct forge_hip_config {
     uint32_t wdtype;        /* projection weights: FORGE_HIP_Q8_0 or FORGE_HIP_Q4_0 */
     uint32_t lm_head_dtype; /* same coding */
     uint32_t flags;         /* FORGE_HIP_FLAG_EXACT, FORGE_HIP_FLAG_QKV_BIAS, both or neither */
+    uint32_t sliding_window; /* ModelConfig::sliding_window_size (ir.rs:512), 0 = None: a position attends to itself and the
+                              * sliding_window - 1 positions before it (attention_sliding, emit.rs:598-627; attention_sliding_batch,
+                              * emit.rs:907-1046; Mistral).  Not available together with FORGE_HIP_FLAG_EXACT. */
 } forge_hip_config;
 
 typedef struct forge_hip_model forge_hip_model;
@@ -192,6 +195,18 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
                                     float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
                                     uint32_t head_dim, uint32_t flags, void* stream);
 
+/* attention_sliding_batch (emit.rs:907-1046) over an fp16 cache: as forge_hip_attn_prefill_f16kv, but the query at
+ * position p = base_pos + row sees only the keys [max(0, p - window + 1), p]; window >= 1.  Fast arithmetic only. */
+int32_t forge_hip_attn_prefill_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
+                                             float* out_dev, uint32_t M, uint32_t base_pos, uint32_t window, uint32_t heads,
+                                             uint32_t kv_heads, uint32_t head_dim, void* stream);
+
+/* attention_sliding (emit.rs:598-627) over an fp16 cache: one query against the last min(window, seq_len) of seq_len
+ * cached rows; window >= 1.  Fast arithmetic only. */
+int32_t forge_hip_attn_decode_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
+                                            float* out_dev, uint32_t seq_len, uint32_t window, uint32_t heads,
+                                            uint32_t kv_heads, uint32_t head_dim, void* stream);
+
 /* argmax (project.rs:501-503): index of the LAST maximum of n floats -> *out_dev (uint32). */
 int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void* stream);
 
@@ -199,8 +214,8 @@ int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void
  * The reference reads a model from a GGUF file in three steps: gguf::parse (crates/forgellm-frontend/src/gguf.rs:484-551),
  * load_config (crates/forgellm-cli/src/main.rs:700-830) and `forge export-weights` (main.rs:2585-2757, tensor names
  * mapped by weight_loader.rs:400-447), whose output file is the blob forge_hip_model_create takes.  These entry points are
- * those three steps.  Supported: architectures "llama", "qwen2" (sets FORGE_HIP_FLAG_QKV_BIAS) and "mistral" (without a sliding
- * window shorter than max_seq);
+ * those three steps.  Supported: architectures "llama", "qwen2" (sets FORGE_HIP_FLAG_QKV_BIAS) and "mistral"
+ * (`<arch>.attention.sliding_window` becomes config.sliding_window, main.rs:764-767);
  * tensors of GGML type F32, F16, BF16, Q8_0, Q4_0 and -- turned into Q8_0 blocks when they are read, as the reference's loader
  * does (weight_loader.rs:219-229) -- Q4_1, Q4_K, Q5_K, Q6_K, Q8_K; projections mostly Q8_0 or mostly Q4_0 by the reference's
  * majority vote, which counts those other types as Q8_0 (a file whose projections are mostly Q4_K is refused: the reference

@@ -23,6 +23,9 @@
 //   f16<->f32, dequant, weight quantisers, kv quantiser, rms_norm, silu, softmax, rope,
 //   argmax, attention vs attention_flash vs attention_flash_batch: pinned by the
 //   reference's own unit-test vectors and closed forms (tests/test_oracle_*.py).
+//   attention_sliding / attention_sliding_batch: no reference test executes them; pinned by
+//   an fp64 softmax over the window written from the definition, by window >= seq being
+//   attention_std, and by batch == per-token.
 //   block isums: pinned by brute-force int64.  f32 combines / matmuls: pinned against an
 //   fp64 evaluation of the same quantised operands.
 //   forward / forward_prefill_batched for Q8_0/Q4_0: PARITY UNPINNED by any reference
@@ -571,6 +574,108 @@ void attention_flash_batch(float* out, const float* qb, const KVView& c, int64_t
     }
 }
 
+// emit.rs:598-627 — plain softmax over the last `window` cached rows.
+void attention_sliding(float* out, const float* q, const KVView& c, int64_t seq, int64_t window, int nh, int nkv, int hd) {
+    int64_t start = seq > window ? seq - window : 0;
+    int64_t wl = seq - start;
+    int gsize = nh / nkv;
+    float scale = 1.0f / sqrtf((float)hd);
+    int64_t stride = (int64_t)nkv * hd;
+    std::vector<float> scores((size_t)wl);
+    for (int h = 0; h < nh; h++) {
+        int kvh = h / gsize;
+        const float* qh = q + (int64_t)h * hd;
+        for (int64_t si = 0; si < wl; si++) {
+            int64_t t = start + si;
+            scores[si] = kdot(c, qh, t, t * stride + (int64_t)kvh * hd, hd) * scale;
+        }
+        softmax(scores.data(), wl);
+        for (int d = 0; d < hd; d++) {
+            float sum = 0.0f;
+            for (int64_t si = 0; si < wl; si++) {
+                int64_t t = start + si;
+                sum += scores[si] * vval(c, t, t * stride + (int64_t)kvh * hd + d);
+            }
+            out[(int64_t)h * hd + d] = sum;
+        }
+    }
+}
+
+// emit.rs:907-1046 — 16-query tiles, 64-key blocks from the block that holds the tile's first visible key; per query
+// the keys [max(0, q_pos - window + 1), q_pos] take part, the others carry weight 0.
+void attention_sliding_batch(float* out, const float* qb, const KVView& c, int64_t m, int64_t base_pos, int64_t window,
+                             int nh, int nkv, int hd) {
+    constexpr int Q_TILE = 16;
+    int gsize = nh / nkv;
+    float scale = 1.0f / sqrtf((float)hd);
+    int64_t stride = (int64_t)nkv * hd;
+    int64_t ostride = (int64_t)nh * hd;
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int h = 0; h < nh; h++) {
+        int kvh = h / gsize;
+        int64_t qo = (int64_t)h * hd;
+        std::vector<float> acc((size_t)Q_TILE * hd);
+        std::vector<float> scores((size_t)Q_TILE * FLASH_BLOCK);
+        for (int64_t qs = 0; qs < m;) {
+            int64_t ql = std::min<int64_t>(Q_TILE, m - qs);
+            int64_t first_pos = base_pos + qs, last_pos = base_pos + qs + ql - 1;
+            int64_t tile_min_k = first_pos > window - 1 ? first_pos - (window - 1) : 0;
+            float m_state[Q_TILE], l_state[Q_TILE];
+            for (int i = 0; i < Q_TILE; i++) { m_state[i] = -INFINITY; l_state[i] = 0.0f; }
+            std::fill(acc.begin(), acc.end(), 0.0f);
+            for (int64_t bs = tile_min_k / FLASH_BLOCK * FLASH_BLOCK; bs <= last_pos;) {
+                int64_t be = std::min<int64_t>(bs + FLASH_BLOCK, last_pos + 1);
+                int64_t bl = be - bs;
+                std::fill(scores.begin(), scores.end(), 0.0f);
+                for (int64_t bi = 0; bi < bl; bi++) {
+                    int64_t t = bs + bi;
+                    for (int64_t qi = 0; qi < ql; qi++) {
+                        const float* qrow = qb + (qs + qi) * ostride + qo;
+                        scores[qi * FLASH_BLOCK + bi] = kdot(c, qrow, t, t * stride + (int64_t)kvh * hd, hd) * scale;
+                    }
+                }
+                for (int64_t qi = 0; qi < ql; qi++) {
+                    int64_t q_pos = base_pos + qs + qi;
+                    int64_t win_start = q_pos > window - 1 ? q_pos - (window - 1) : 0;
+                    int64_t lo = std::max(win_start, bs) - bs;
+                    int64_t hi = q_pos + 1 > bs ? q_pos + 1 - bs : 0;
+                    if (hi > bl) hi = bl;
+                    float* sc = &scores[qi * FLASH_BLOCK];
+                    if (lo >= hi) { for (int64_t bi = 0; bi < bl; bi++) sc[bi] = 0.0f; continue; }
+                    float m_block = -INFINITY;
+                    for (int64_t bi = lo; bi < hi; bi++) if (sc[bi] > m_block) m_block = sc[bi];
+                    float m_prev = m_state[qi];
+                    float m_new = fmaxf(m_prev, m_block);
+                    m_state[qi] = m_new;
+                    float exp_scale = expf(m_prev - m_new);
+                    l_state[qi] *= exp_scale;
+                    for (int d = 0; d < hd; d++) acc[qi * hd + d] *= exp_scale;
+                    float l_block = 0.0f;
+                    for (int64_t bi = lo; bi < hi; bi++) { float e = expf(sc[bi] - m_new); sc[bi] = e; l_block += e; }
+                    for (int64_t bi = 0; bi < lo; bi++) sc[bi] = 0.0f;
+                    for (int64_t bi = hi; bi < bl; bi++) sc[bi] = 0.0f;
+                    l_state[qi] += l_block;
+                }
+                for (int64_t bi = 0; bi < bl; bi++) {
+                    int64_t t = bs + bi;
+                    int64_t vo = t * stride + (int64_t)kvh * hd;
+                    for (int d = 0; d < hd; d++) {
+                        float v = vval(c, t, vo + d);
+                        for (int64_t qi = 0; qi < ql; qi++) acc[qi * hd + d] += scores[qi * FLASH_BLOCK + bi] * v;
+                    }
+                }
+                bs = be;
+            }
+            for (int64_t qi = 0; qi < ql; qi++) {
+                float inv_l = l_state[qi] > 0.0f ? 1.0f / l_state[qi] : 0.0f;
+                float* p = out + (qs + qi) * ostride + qo;
+                for (int d = 0; d < hd; d++) p[d] = acc[qi * hd + d] * inv_l;
+            }
+            qs += ql;
+        }
+    }
+}
+
 // crates/forgellm-codegen-cpu/src/project.rs:501-503 — Iterator::max_by returns the LAST
 // maximal element.
 uint32_t argmax_last(const float* v, int64_t n) {
@@ -594,6 +699,7 @@ struct fo_config {
     uint32_t wdtype;        // 8 = Q8_0, 2 = Q4_0 (GGML type ids)
     uint32_t lm_head_dtype; // same coding
     uint32_t flags;         // bit 1 (value 2): the blob carries QKV bias vectors (Qwen2, emit.rs:3906-3915)
+    uint32_t sliding_window; // ModelConfig::sliding_window_size, 0 = None (emit.rs:97-99, 4156-4170, 5312-5340)
 };
 
 struct fo_layer {
@@ -706,7 +812,8 @@ int fo_forward(fo_model* m, uint32_t token, float* logits) {
         rope(k.data(), pos, c.head_dim, c.kv_heads, m->freqs.data());
         store_kv(m, l, pos, k.data(), v.data());
         KVView cv = kv_view(m, l);
-        if (flash) attention_flash(attn.data(), q.data(), cv, pos + 1, c.heads, c.kv_heads, c.head_dim);
+        if (c.sliding_window) attention_sliding(attn.data(), q.data(), cv, pos + 1, c.sliding_window, c.heads, c.kv_heads, c.head_dim);
+        else if (flash) attention_flash(attn.data(), q.data(), cv, pos + 1, c.heads, c.kv_heads, c.head_dim);
         else attention_std(attn.data(), q.data(), cv, pos + 1, c.heads, c.kv_heads, c.head_dim);
         matmul_vec(c.wdtype, m->variant, proj.data(), attn.data(), L.o, QKS, H, 0);
         for (int64_t i = 0; i < H; i++) hs[i] += proj[i];
@@ -751,7 +858,8 @@ int fo_prefill_batched(fo_model* m, const uint32_t* tokens, int64_t n, float* lo
             store_kv(m, l, base + r, &k[r * KV], &v[r * KV]);
         }
         KVView cv = kv_view(m, l);
-        if (flash) attention_flash_batch(attn.data(), q.data(), cv, n, base, c.heads, c.kv_heads, c.head_dim);
+        if (c.sliding_window) attention_sliding_batch(attn.data(), q.data(), cv, n, base, c.sliding_window, c.heads, c.kv_heads, c.head_dim);
+        else if (flash) attention_flash_batch(attn.data(), q.data(), cv, n, base, c.heads, c.kv_heads, c.head_dim);
         else for (int64_t r = 0; r < n; r++)
             attention_std(&attn[r * QKS], &q[r * QKS], cv, base + r + 1, c.heads, c.kv_heads, c.head_dim);
         matmul_mat(c.wdtype, m->variant, proj.data(), n, attn.data(), L.o, QKS, H);
@@ -828,16 +936,18 @@ void fo_expf_array(const float* x, int64_t n, float* out) { for (int64_t i = 0; 
 
 // Attention over an externally supplied cache.  kvmode 0: k,v are int8 with ks/vs scales;
 // kvmode 1: k,v are fp16 bit patterns.  kind 0 standard, 1 flash, 2 flash_batch (then q is
-// [m][nh*hd], out likewise, and the cache holds base_pos+m rows).
+// [m][nh*hd], out likewise, and the cache holds base_pos+m rows), 3 sliding, 4 sliding_batch (both with `window`).
 void fo_attention(int kind, int kvmode, float* out, const float* q, const void* k, const void* v, const float* ks,
-                  const float* vs, int64_t seq_or_m, int64_t base_pos, int nh, int nkv, int hd) {
+                  const float* vs, int64_t seq_or_m, int64_t base_pos, int nh, int nkv, int hd, int64_t window) {
     KVView c{};
     c.mode = kvmode;
     if (kvmode == 0) { c.k8 = (const int8_t*)k; c.v8 = (const int8_t*)v; c.ks = ks; c.vs = vs; }
     else { c.k16 = (const uint16_t*)k; c.v16 = (const uint16_t*)v; }
     if (kind == 0) attention_std(out, q, c, seq_or_m, nh, nkv, hd);
     else if (kind == 1) attention_flash(out, q, c, seq_or_m, nh, nkv, hd);
-    else attention_flash_batch(out, q, c, seq_or_m, base_pos, nh, nkv, hd);
+    else if (kind == 2) attention_flash_batch(out, q, c, seq_or_m, base_pos, nh, nkv, hd);
+    else if (kind == 3) attention_sliding(out, q, c, seq_or_m, window, nh, nkv, hd);
+    else attention_sliding_batch(out, q, c, seq_or_m, base_pos, window, nh, nkv, hd);
 }
 
 int fo_num_threads(void) {

@@ -181,13 +181,14 @@ def config(g, max_seq=0, flags=0) -> dict:
             raise GgufError("output.weight has an unsupported GGML type")
     seq = max_seq or ctx
     window = _get(g, p + "attention.sliding_window", (4,))
-    if window is not None and window < seq:
-        raise GgufError("sliding-window attention is not supported")
+    if window == 0:
+        raise GgufError("a sliding window of 0 positions")
     f = np.float32
     return {"hidden": hidden, "inter": inter, "layers": layers, "heads": heads, "kv_heads": kv, "head_dim": hidden // heads,
             "vocab": vocab, "max_seq": seq, "rms_eps": float(f(1e-5) if eps is None else f(eps)),
             "rope_theta": float(f(10000.0) if theta is None else f(theta)), "wdtype": wd, "lm_head_dtype": lm,
-            "flags": flags | (2 if arch == "qwen2" else 0)}                  # qkv_bias goes with the architecture, main.rs:770
+            "flags": flags | (2 if arch == "qwen2" else 0),
+            "sliding_window": window or 0}                  # qkv_bias goes with the architecture, main.rs:770
 
 
 F = np.float32

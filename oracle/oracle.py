@@ -26,6 +26,7 @@ class Config(C.Structure):
         ("kv_heads", C.c_uint32), ("head_dim", C.c_uint32), ("vocab", C.c_uint32), ("max_seq", C.c_uint32),
         ("rms_eps", C.c_float), ("rope_theta", C.c_float),
         ("wdtype", C.c_uint32), ("lm_head_dtype", C.c_uint32), ("flags", C.c_uint32),
+        ("sliding_window", C.c_uint32),
     ]
 
 
@@ -79,7 +80,7 @@ def lib():
     L.fo_expf_array.argtypes = [vp, i64, vp]
     L.fo_argmax.restype = C.c_uint32
     L.fo_argmax.argtypes = [vp, i64]
-    L.fo_attention.argtypes = [i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32]
+    L.fo_attention.argtypes = [i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64]
     L.fo_num_threads.restype = i32
     L.fo_set_num_threads.argtypes = [i32]
     _lib = L
@@ -226,9 +227,12 @@ def argmax(v):
     return int(lib().fo_argmax(_p(v), v.size))
 
 
-def attention(kind, q, k, v, seq_or_m, nh, nkv, hd, base_pos=0, ks=None, vs=None):
-    """kind: 'std' | 'flash' | 'flash_batch'.  k, v: int8 (with ks, vs) or uint16 fp16 bits."""
-    kinds = {"std": 0, "flash": 1, "flash_batch": 2}
+def attention(kind, q, k, v, seq_or_m, nh, nkv, hd, base_pos=0, ks=None, vs=None, window=0):
+    """kind: 'std' | 'flash' | 'flash_batch' | 'sliding' | 'sliding_batch' (the last two need `window` >= 1).
+    k, v: int8 (with ks, vs) or uint16 fp16 bits."""
+    kinds = {"std": 0, "flash": 1, "flash_batch": 2, "sliding": 3, "sliding_batch": 4}
+    if kinds[kind] >= 3 and window < 1:
+        raise ValueError("sliding attention needs a window of at least 1")
     q = _f32(q)
     if k.dtype == np.int8:
         kvmode, ks, vs = KV_INT8, _f32(ks), _f32(vs)
@@ -237,7 +241,7 @@ def attention(kind, q, k, v, seq_or_m, nh, nkv, hd, base_pos=0, ks=None, vs=None
         kvmode = KV_F16
     k, v = np.ascontiguousarray(k), np.ascontiguousarray(v)
     out = np.empty_like(q)
-    lib().fo_attention(kinds[kind], kvmode, _p(out), _p(q), _p(k), _p(v), _p(ks), _p(vs), seq_or_m, base_pos, nh, nkv, hd)
+    lib().fo_attention(kinds[kind], kvmode, _p(out), _p(q), _p(k), _p(v), _p(ks), _p(vs), seq_or_m, base_pos, nh, nkv, hd, window)
     return out
 
 

@@ -282,12 +282,16 @@ def test_config_defaults_and_refusals(fh, gg, go):
     kq = (("blk.0.attn_q.weight", [256, 64], gg.Q5_K, None), ("output.weight", [256, 64], gg.Q6_K, None))
     ck = gg.GgufFile(make(base, kq)).config()
     assert (ck["wdtype"], ck["lm_head_dtype"]) == (Q8, Q8) and ck == go.config(go.parse(make(base, kq)))
-    refused(base + [("llama.attention.sliding_window", gg.U32, 1024)], text="sliding-window")
-    # a window that covers the whole cache is the same attention up to rounding: accepted, but not in exact mode
-    wide = gg.GgufFile(make(base + [("llama.attention.sliding_window", gg.U32, 4096)]))
-    assert wide.config()["max_seq"] == 2048
-    with pytest.raises(fh.ForgeHipError, match="sliding window"):
-        wide.config(flags=fh.FLAG_EXACT)
+    # the window travels into the config (main.rs:764-767); exact mode has no sliding attention
+    for w in (1024, 4096):
+        blob_w = make(base + [("llama.attention.sliding_window", gg.U32, w)])
+        win = gg.GgufFile(blob_w)
+        cw = win.config()
+        assert cw["sliding_window"] == w and cw["max_seq"] == 2048 and cw == go.config(go.parse(blob_w))
+        with pytest.raises(fh.ForgeHipError, match="sliding window"):
+            win.config(flags=fh.FLAG_EXACT)
+    assert c["sliding_window"] == 0
+    refused(base + [("llama.attention.sliding_window", gg.U32, 0)], text="sliding window of 0")
     # the vote: 2 x Q4_0 against 1 x Q8_0
     vote = (("blk.0.attn_q.weight", [64, 64], gg.Q4_0, None), ("blk.0.attn_k.weight", [64, 64], gg.Q4_0, None),
             ("blk.0.ffn_up.weight", [64, 64], gg.Q8_0, None), ("blk.0.attn_norm.weight", [64], gg.F32, None),
@@ -541,7 +545,7 @@ def test_model_from_gguf_equals_model_from_blob(fh, gg, torch_gpu, tmp_path):
         path = str(tmp_path / f"m{wd}.gguf")
         gg.model_to_gguf(cfg, blob, tied=True, path=path)
         a, b = fh.HipModel(cfg, blob), fh.HipModel.from_gguf(path)
-        assert b.config == {**cfg, "rms_eps": b.config["rms_eps"], "rope_theta": b.config["rope_theta"]}
+        assert b.config == {"sliding_window": 0, **cfg, "rms_eps": b.config["rms_eps"], "rope_theta": b.config["rope_theta"]}
         prompt = fh.synth.uniform_ids(5, 40, cfg["vocab"])
         la, lb = a.forward_prefill(prompt), b.forward_prefill(prompt)
         assert np.array_equal(la.view(np.uint32), lb.view(np.uint32))

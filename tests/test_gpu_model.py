@@ -408,3 +408,81 @@ def test_qkv_bias_model_matches_oracle(fh, oracle, torch_gpu, wd, monkeypatch):
     gm = fh.HipModel(nobias_cfg, np.concatenate(keep))
     assert not np.array_equal(gm.forward_prefill(prompt), olog)
     gm.close(); om.close()
+
+
+@pytest.mark.parametrize("wd", [Q8, Q4])
+@pytest.mark.parametrize("window", [1, 24, 100])
+def test_sliding_window_model_matches_oracle(fh, oracle, torch_gpu, wd, window, monkeypatch):
+    """A Mistral-style model (sliding_window_size: attention_sliding in decode, attention_sliding_batch in prefill,
+    emit.rs:4156-4170 and 5312-5340): prompt and decode both run past the window; logits within tolerance of the CPU
+    oracle with identical greedy tokens on these seeds, resident kernel and kernel sequence alike; prefill in two chunks
+    (the second starts beyond the window) equals one; and the window matters."""
+    cfg = tiny_cfg(fh, wd, 0)
+    cfg["sliding_window"] = window
+    blob = fh.synth.make_weights_blob(cfg, seed=61 + window)
+    prompt = fh.synth.uniform_ids(62, 150, cfg["vocab"])
+    om = oracle.Model(cfg, blob, A, KV_F16)
+    olog = om.prefill_batched(prompt)
+    otoks, ologits = [], []
+    tok = oracle.argmax(olog)
+    for _ in range(12):
+        ol = om.forward(tok)
+        ologits.append(ol)
+        tok = oracle.argmax(ol)
+        otoks.append(tok)
+    om.close()
+    runs = {}
+    # resident kernel with the default summation, resident kernel summing in the reference's block order, kernel sequence
+    for name, persist, ordered in (("resident", "1", "0"), ("resident_ordered", "1", "1"), ("sequence", "0", "0")):
+        monkeypatch.setenv("FORGE_HIP_PERSIST", persist)
+        monkeypatch.setenv("FORGE_HIP_PD_ORDERED", ordered)
+        gm = fh.HipModel(cfg, blob)
+        assert (gm.decode_launches == 1) == (persist == "1")
+        glog = gm.forward_prefill(prompt)
+        assert np.allclose(glog, olog, rtol=2e-2, atol=2e-2)
+        tok = fh.ops.argmax_host(glog)
+        assert tok == oracle.argmax(olog)
+        toks, logs = [], []
+        for _ in range(12):
+            lg = gm.forward(tok)
+            logs.append(lg)
+            tok = fh.ops.argmax_host(lg)
+            toks.append(tok)
+        runs[name] = (toks, logs)
+        gm.reset()
+        gm.forward_prefill(prompt[:101])
+        two = gm.forward_prefill(prompt[101:])
+        assert np.allclose(two, glog, rtol=1e-3, atol=1e-3)
+        gm.close()
+    monkeypatch.delenv("FORGE_HIP_PERSIST")
+    monkeypatch.delenv("FORGE_HIP_PD_ORDERED")
+    assert runs["resident"][0] == runs["resident_ordered"][0] == runs["sequence"][0] == otoks
+    for a, b, c, o in zip(runs["resident"][1], runs["resident_ordered"][1], runs["sequence"][1], ologits):
+        assert np.array_equal(b.view(np.uint32), c.view(np.uint32))          # same keys, same order, same merges
+        assert np.allclose(a, o, rtol=2e-2, atol=2e-2) and np.allclose(c, o, rtol=2e-2, atol=2e-2)
+    gm = fh.HipModel(dict(cfg, sliding_window=0), blob)
+    assert not np.allclose(gm.forward_prefill(prompt), olog, rtol=2e-2, atol=2e-2)
+    gm.close()
+    with pytest.raises(fh.ForgeHipError, match="sliding window"):
+        fh.HipModel(dict(cfg, flags=EXACT), blob)
+
+
+def test_sliding_window_model_from_gguf(fh, oracle, torch_gpu, tmp_path):
+    """`mistral.attention.sliding_window` reaches the kernels: a model read from a GGUF file with the key decodes like the
+    model created from the blob with config.sliding_window."""
+    cfg = tiny_cfg(fh, Q8, 0)
+    cfg["sliding_window"] = 40
+    blob = fh.synth.make_weights_blob(cfg, seed=71)
+    path = tmp_path / "mistral.gguf"
+    fh.gguf.model_to_gguf(cfg, blob, path=str(path))
+    a = fh.HipModel.from_gguf(str(path))
+    b = fh.HipModel(cfg, blob)
+    prompt = fh.synth.uniform_ids(72, 90, cfg["vocab"])
+    la, lb = a.forward_prefill(prompt), b.forward_prefill(prompt)
+    assert np.array_equal(la.view(np.uint32), lb.view(np.uint32))
+    tok = fh.ops.argmax_host(la)
+    for _ in range(6):
+        ta, tb = a.forward_greedy(tok), b.forward_greedy(tok)
+        assert ta == tb
+        tok = ta
+    a.close(); b.close()

@@ -208,6 +208,67 @@ def test_attention_prefill_parity(fh, oracle, torch_gpu, heads, kv_heads, hd, M,
     close(fh.ops.attention_flash_batch(qd, kd, vd, base, heads, kv_heads, hd, 0).cpu().numpy(), want, rtol=2e-3, atol=2e-3)
 
 
+@pytest.mark.parametrize("heads,kv_heads,hd", [(32, 8, 64), (9, 3, 64), (6, 6, 96), (24, 8, 128)])
+@pytest.mark.parametrize("seq,window", [(1, 1), (5, 3), (70, 1), (70, 64), (70, 70), (70, 4096), (900, 17), (900, 256), (900, 899)])
+def test_attention_sliding_decode_parity(fh, oracle, torch_gpu, heads, kv_heads, hd, seq, window):
+    """attention_sliding (emit.rs:598-627): one query against the last `window` cached rows."""
+    torch = torch_gpu
+    k16, v16 = _kv_cache(fh, oracle, seq, kv_heads, hd, seed=seq + hd + window)
+    q = fh.synth.normal(9, heads * hd, 1.0)
+    want = oracle.attention("sliding", q, k16, v16, seq, heads, kv_heads, hd, window=window)
+    qd, kd, vd = torch.from_numpy(q).cuda(), _dev16(torch, k16), _dev16(torch, v16)
+    got = fh.ops.attention_sliding(qd, kd, vd, seq, window, heads, kv_heads, hd).cpu().numpy()
+    close(got, want)
+    if window >= seq:       # then it is the plain decode attention, bit for bit
+        same_bits(got, fh.ops.attention_flash(qd, kd, vd, seq, heads, kv_heads, hd, 0).cpu().numpy())
+    else:                   # rows before the window do not count: poison them
+        kd2, vd2 = kd.clone(), vd.clone()
+        kd2[:seq - window] = 0x7BFF          # fp16 65504
+        vd2[:seq - window] = 0x7BFF
+        same_bits(fh.ops.attention_sliding(qd, kd2, vd2, seq, window, heads, kv_heads, hd).cpu().numpy(), got)
+
+
+@pytest.mark.parametrize("heads,kv_heads,hd", [(8, 2, 64), (6, 6, 96), (6, 2, 128)])
+@pytest.mark.parametrize("M,base,window", [(1, 0, 1), (33, 0, 5), (200, 0, 1), (200, 0, 31), (200, 0, 64), (200, 0, 100), (131, 77, 33),
+                                           (131, 77, 128), (131, 77, 207), (131, 77, 208), (300, 500, 129), (64, 64, 1000)])
+def test_attention_sliding_prefill_parity(fh, oracle, torch_gpu, heads, kv_heads, hd, M, base, window):
+    """attention_sliding_batch (emit.rs:907-1046): row r sees the keys [max(0, base + r - window + 1), base + r]."""
+    torch = torch_gpu
+    seq = base + M
+    k16, v16 = _kv_cache(fh, oracle, seq, kv_heads, hd, seed=M + hd + base + window)
+    q = oracle.f16_to_f32(oracle.f32_to_f16(fh.synth.normal(10, M * heads * hd, 1.0))).reshape(M, heads * hd)
+    want = oracle.attention("sliding_batch", q, k16, v16, M, heads, kv_heads, hd, base_pos=base, window=window)
+    qd, kd, vd = torch.from_numpy(q).cuda(), _dev16(torch, k16), _dev16(torch, v16)
+    got = fh.ops.attention_sliding_batch(qd, kd, vd, base, window, heads, kv_heads, hd).cpu().numpy()
+    close(got, want)
+    if window >= seq:       # every key of the call is inside every window: the causal kernel, bit for bit
+        same_bits(got, fh.ops.attention_flash_batch(qd, kd, vd, base, heads, kv_heads, hd, 0).cpu().numpy())
+    else:                   # rows before the first query's window are never read, and no query may see a row before its own
+        first = max(0, base - window + 1)
+        kd2, vd2 = kd.clone(), vd.clone()
+        kd2[:first] = 0x7BFF
+        vd2[:first] = 0x7BFF
+        same_bits(fh.ops.attention_sliding_batch(qd, kd2, vd2, base, window, heads, kv_heads, hd).cpu().numpy(), got)
+        r = M - 1                                  # the last query: poison everything before ITS window
+        lo = max(0, base + r - window + 1)
+        kd3, vd3 = kd.clone(), vd.clone()
+        kd3[:lo] = 0x7BFF
+        vd3[:lo] = 0x7BFF
+        close(fh.ops.attention_sliding_batch(qd, kd3, vd3, base, window, heads, kv_heads, hd).cpu().numpy()[r], want[r])
+
+
+def test_attention_sliding_refusals(fh, torch_gpu):
+    torch = torch_gpu
+    q = torch.zeros((4, 256), device="cuda")
+    kc = torch.zeros((8, 64), dtype=torch.int16, device="cuda")
+    with pytest.raises(fh.ForgeHipError, match="window"):
+        fh.ops.attention_sliding_batch(q, kc, kc, 0, 0, 4, 1, 64)
+    with pytest.raises(fh.ForgeHipError, match="window"):
+        fh.ops.attention_sliding(q[0].contiguous(), kc, kc, 4, 0, 4, 1, 64)
+    with pytest.raises(fh.ForgeHipError, match="head_dim"):
+        fh.ops.attention_sliding(q[0].contiguous(), kc, kc, 4, 2, 4, 1, 48)
+
+
 def test_attention_reference_vectors_shape_scaled(fh, oracle, torch_gpu):
     """The reference's deterministic attention inputs (emit.rs:6687-6741), widened to head_dim 64."""
     torch = torch_gpu

@@ -235,6 +235,101 @@ def test_flash_batch_rows_equal_per_token_flash(oracle, kvmode):
         assert np.max(np.abs(one - batch[r])) < 2e-6
 
 
+# ---- sliding-window attention (emit.rs:598-627, 907-1046): no reference test executes these two, so they are pinned
+# by what the definition fixes: an fp64 softmax over the window, window >= seq == attention, batch == per token
+def _windowed_fp64(q, k, v, nh, nkv, hd, qpos, window):
+    q2 = np.atleast_2d(q).astype(np.float64)
+    out = np.zeros_like(q2)
+    g = nh // nkv
+    for r in range(q2.shape[0]):
+        lo, hi = max(0, qpos[r] - window + 1), qpos[r] + 1
+        for h in range(nh):
+            kh = k[lo:hi, (h // g) * hd:(h // g + 1) * hd]
+            vh = v[lo:hi, (h // g) * hd:(h // g + 1) * hd]
+            s = kh @ q2[r, h * hd:(h + 1) * hd] / np.sqrt(hd)
+            p = np.exp(s - s.max())
+            out[r, h * hd:(h + 1) * hd] = (p / p.sum()) @ vh
+    return out
+
+
+@pytest.mark.parametrize("seq", [5, 64, 70, 200])
+def test_sliding_with_a_wide_window_is_standard_attention(oracle, seq):
+    """`When seq_len <= window, behaves identically to attention` (emit.rs:597): same bits, on the reference's inputs."""
+    hd, nh, nkv = 8, 3, 1
+    q, k, v = _ref_attention_inputs(seq)
+    k16, v16 = oracle.f32_to_f16(k), oracle.f32_to_f16(v)
+    std = oracle.attention("std", q, k16, v16, seq, nh, nkv, hd)
+    for window in (seq, seq + 1, 4096):
+        assert np.array_equal(oracle.attention("sliding", q, k16, v16, seq, nh, nkv, hd, window=window).view(np.uint32), std.view(np.uint32))
+    # a shorter window is attention over the tail of the cache
+    w = max(1, seq // 3)
+    tail = oracle.attention("std", q, k16.reshape(seq, -1)[seq - w:], v16.reshape(seq, -1)[seq - w:], w, nh, nkv, hd)
+    assert np.array_equal(oracle.attention("sliding", q, k16, v16, seq, nh, nkv, hd, window=w).view(np.uint32), tail.view(np.uint32))
+
+
+@pytest.mark.parametrize("kvmode", ["int8", "f16"])
+@pytest.mark.parametrize("window", [1, 7, 64, 65, 100, 1000])
+def test_sliding_batch_against_fp64_and_per_token(oracle, kvmode, window):
+    rng = np.random.default_rng(80 + window)
+    hd, nh, nkv, base, m = 16, 4, 2, 37, 150         # crosses 64-key blocks and 16-row query tiles
+    seq = base + m
+    q = rng.standard_normal((m, nh * hd)).astype(np.float32)
+    kf32 = rng.standard_normal((seq, nkv * hd)).astype(np.float32)
+    vf32 = rng.standard_normal((seq, nkv * hd)).astype(np.float32)
+    if kvmode == "int8":
+        kq = np.empty((seq, nkv * hd), np.int8); vq = np.empty_like(kq)
+        ks = np.empty(seq, np.float32); vs = np.empty(seq, np.float32)
+        for t in range(seq):
+            kq[t], ks[t] = oracle.quantize_kv(kf32[t])
+            vq[t], vs[t] = oracle.quantize_kv(vf32[t])
+        kw = dict(ks=ks, vs=vs)
+        kc, vc = kq, vq
+        kd = kq.astype(np.float64) * ks[:, None].astype(np.float64)
+        vd = vq.astype(np.float64) * vs[:, None].astype(np.float64)
+    else:
+        kc, vc = oracle.f32_to_f16(kf32), oracle.f32_to_f16(vf32)
+        kw = {}
+        kd, vd = oracle.f16_to_f32(kc).astype(np.float64), oracle.f16_to_f32(vc).astype(np.float64)
+    qpos = [base + r for r in range(m)]
+    batch = oracle.attention("sliding_batch", q, kc, vc, m, nh, nkv, hd, base_pos=base, window=window, **kw)
+    want = _windowed_fp64(q, kd, vd, nh, nkv, hd, qpos, window)
+    assert np.max(np.abs(batch - want)) < 2e-5
+    # a key one step outside the window must not count: moving it far away changes nothing
+    if window < seq:
+        r = m - 1
+        kc2 = kc.copy()
+        kc2[qpos[r] - window] = kc[qpos[r]]          # the row just before the last query's window
+        again = oracle.attention("sliding_batch", q, kc2, vc, m, nh, nkv, hd, base_pos=base, window=window, **kw)
+        assert np.array_equal(again[r], batch[r])
+    for r in (0, 1, 15, 16, 27, 90, 149):
+        n = base + r + 1
+        one = oracle.attention("sliding", q[r], kc[:n], vc[:n], n, nh, nkv, hd, window=window, **{k_: v_[:n] for k_, v_ in kw.items()})
+        assert np.max(np.abs(one - batch[r])) < 2e-6
+        assert np.max(np.abs(one - want[r])) < 2e-5
+    if window >= seq:                                 # then it is the causal flash attention, block for block
+        flash = oracle.attention("flash_batch", q, kc, vc, m, nh, nkv, hd, base_pos=base, **kw)
+        assert np.array_equal(flash.view(np.uint32), batch.view(np.uint32))
+
+
+def test_sliding_model_prefill_batched_equals_token_loop(oracle, fh):
+    """A model with a window: token loop (attention_sliding) and batched prefill (attention_sliding_batch) agree, and the
+    window matters (the same weights without it give other logits once the prompt is longer than the window)."""
+    cfg = fh.synth.tiny(wdtype=Q8, max_seq=640, hidden=128, inter=256, layers=2, heads=4, kv_heads=2, head_dim=32, vocab=300)
+    cfg["sliding_window"] = 9
+    blob = fh.synth.make_weights_blob(cfg, seed=3)
+    toks = fh.synth.uniform_ids(5, 40, cfg["vocab"])
+    m1 = oracle.Model(cfg, blob, A, 1)
+    for t in toks:
+        last = m1.forward(int(t))
+    batched = oracle.Model(cfg, blob, A, 1).prefill_batched(toks)
+    assert np.max(np.abs(last - batched)) < 1e-4 * max(1.0, float(np.max(np.abs(last))))
+    full = oracle.Model(dict(cfg, sliding_window=0), blob, A, 1).prefill_batched(toks)
+    assert np.max(np.abs(full - batched)) > 1e-3
+    # a prompt that fits the window sees every key either way (the summation order differs: flash blocks against plain softmax)
+    short = oracle.Model(dict(cfg, sliding_window=0), blob, A, 1).prefill_batched(toks[:9])
+    assert np.max(np.abs(short - oracle.Model(cfg, blob, A, 1).prefill_batched(toks[:9]))) < 1e-4
+
+
 # ---- whole model: per-token forward loop == batched prefill (the reference's own consistency claim)
 @pytest.mark.parametrize("wd", [Q8, Q4])
 @pytest.mark.parametrize("variant,kv", [(A, 1), (A, 0), (B, 0)])
