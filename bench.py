@@ -182,6 +182,24 @@ def ops_table(fh, reps=10):
             us = timed(lambda: ops.attention_flash(q1, k, v, seq, heads, kvh, hd))
             rows.append({"op": "attention_decode", "heads": heads, "kv_heads": kvh, "head_dim": hd, "cache": seq,
                          "us_per_call": round(us, 2), "kv_bytes": 2 * seq * kvh * hd * 2})
+    # sliding-window attention: the Llama-3.2-1B head shape with a 1024-position window and the Mistral-7B head shape
+    # (32 / 8 heads of 128) with its 4096-position window
+    for heads, kvh, hd, seq, window in ((32, 8, 64, 3001, 1024), (32, 8, 128, 8192, 4096)):
+        q = torch.from_numpy(fh.synth.normal(15, seq * heads * hd, 1.0).reshape(seq, heads * hd)).cuda()
+        k = torch.from_numpy(fh.synth.normal(16, seq * kvh * hd, 1.0).reshape(seq, kvh * hd)).cuda().half().view(torch.int16)
+        v = torch.from_numpy(fh.synth.normal(17, seq * kvh * hd, 1.0).reshape(seq, kvh * hd)).cuda().half().view(torch.int16)
+        pairs = sum(min(p + 1, window) for p in range(seq))
+        for w, name in ((window, "attention_prefill_sliding"), (0, "attention_prefill")):
+            us = timed((lambda: ops.attention_sliding_batch(q, k, v, 0, window, heads, kvh, hd)) if w else
+                       (lambda: ops.attention_flash_batch(q, k, v, 0, heads, kvh, hd)))
+            rows.append({"op": name, "heads": heads, "kv_heads": kvh, "head_dim": hd, "seq": seq, "window": w,
+                         "us_per_call": round(us, 2), "flops": 4 * heads * hd * (pairs if w else seq * (seq + 1) // 2)})
+        q1 = q[seq - 1].contiguous()
+        for w, name in ((window, "attention_decode_sliding"), (0, "attention_decode")):
+            us = timed((lambda: ops.attention_sliding(q1, k, v, seq, window, heads, kvh, hd)) if w else
+                       (lambda: ops.attention_flash(q1, k, v, seq, heads, kvh, hd)))
+            rows.append({"op": name, "heads": heads, "kv_heads": kvh, "head_dim": hd, "cache": seq, "window": w,
+                         "us_per_call": round(us, 2), "kv_bytes": 2 * (min(seq, w) if w else seq) * kvh * hd * 2})
     print(json.dumps({"ops_table": rows, "reps": reps}))
 
 

@@ -164,13 +164,14 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], sacc, 0, 0, 0);
             }
             // ---- causal mask: only keys past the group's first query can be masked for some query
-            if (WIN) {
+            // with a window, also keys that the group's last query no longer sees
+            if (WIN && (k0 + 31 > wave_min_pos || k0 + window <= wave_max_pos)) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const uint32_t t = k0 + 8 * (r >> 2) + 4 * lh + (r & 3);
                     sacc[r] = (t <= qpos && t + window > qpos) ? sacc[r] : -INFINITY;
                 }
-            } else if (k0 + 31 > wave_min_pos) {
+            } else if (!WIN && k0 + 31 > wave_min_pos) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
                     const uint32_t t = k0 + 8 * (r >> 2) + 4 * lh + (r & 3);
