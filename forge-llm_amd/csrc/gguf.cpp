@@ -386,6 +386,25 @@ int32_t write_quantised(const forge_hip_gguf* g, const std::string& name, uint32
     return FORGE_HIP_OK;
 }
 
+// Elements [first, first + numel) of a tensor of `total` elements, in the blob's format: one part of a fused Phi-3 tensor
+// (split_weight_three / split_weight_two, weight_loader.rs:543-583, 641-700).  The reference splits what its loader made of the
+// whole tensor, so a tensor in another format is converted whole and then cut; parts start on 32-element block boundaries
+// because every row has a multiple of 32 elements.
+int32_t write_quantised_part(const forge_hip_gguf* g, const std::string& name, uint32_t wdtype, uint64_t total, uint64_t first,
+                             uint64_t numel, uint8_t* out) {
+    Source s;
+    int32_t rc = locate(g, name, total, &s);
+    if (rc) return rc;
+    if (first % 32 || numel % 32 || first + numel > total)
+        return fail(FORGE_HIP_ERR_INVALID, "gguf: fused tensor " + name + " cannot be split on block boundaries");
+    if (s.t->type == wdtype) { memcpy(out, s.bytes + qbytes(wdtype, first), qbytes(wdtype, numel)); return FORGE_HIP_OK; }
+    std::vector<float> v(total);
+    rc = to_f32(s, total, v.data());
+    if (rc) return rc;
+    fh::quantize_host(wdtype, v.data() + first, numel, out);
+    return FORGE_HIP_OK;
+}
+
 int32_t write_f32(const forge_hip_gguf* g, const std::string& name, uint64_t numel, uint8_t* out) {
     Source s;
     const int32_t rc = locate(g, name, numel, &s);
@@ -489,9 +508,9 @@ int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_
     const MetaValue* arch_v = g->find("general.architecture");
     const std::string arch = arch_v && arch_v->type == 8 ? arch_v->str : "unknown";
     // The kernels here cover the Llama layer, with the QKV bias of Qwen2 (main.rs:770: the bias goes with the
-    // architecture): no GeLU or embedding scale (gemma), no fused QKV (phi3).  Mistral is the Llama layer plus an optional
-    // sliding window.
-    if (arch != "llama" && arch != "mistral" && arch != "qwen2")
+    // architecture): no GeLU or embedding scale (gemma).  Mistral is the Llama layer plus an optional sliding window;
+    // Phi-3 is the Llama layer with fused tensors in the file, which export_weights splits (main.rs:759).
+    if (arch != "llama" && arch != "mistral" && arch != "qwen2" && arch != "phi3" && arch != "phi")
         return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: unsupported GGUF architecture: " + arch);
     const std::string p = arch + ".";
     uint32_t hidden = 0, layers = 0, heads = 0, kv_heads = 0, inter = 0;
@@ -587,9 +606,17 @@ int32_t forge_hip_gguf_export_weights(const forge_hip_gguf* g, const forge_hip_c
     FH_STEP(write_f32(g, "token_embd.weight", V * H, p), V * H * 4);
     for (uint32_t l = 0; l < c->layers; l++) {
         FH_STEP(write_f32(g, blk(l, "attn_norm.weight"), H, p), H * 4);
-        FH_STEP(write_quantised(g, blk(l, "attn_q.weight"), wt, QKS * H, p), qbytes(wt, QKS * H));
-        FH_STEP(write_quantised(g, blk(l, "attn_k.weight"), wt, KV * H, p), qbytes(wt, KV * H));
-        FH_STEP(write_quantised(g, blk(l, "attn_v.weight"), wt, KV * H, p), qbytes(wt, KV * H));
+        if (!g->tensor(blk(l, "attn_q.weight")) && g->tensor(blk(l, "attn_qkv.weight"))) {
+            // Phi-3: Q|K|V rows in one tensor (weight_loader.rs:425-427, 552-567)
+            const uint64_t all = (QKS + 2 * KV) * H;
+            FH_STEP(write_quantised_part(g, blk(l, "attn_qkv.weight"), wt, all, 0, QKS * H, p), qbytes(wt, QKS * H));
+            FH_STEP(write_quantised_part(g, blk(l, "attn_qkv.weight"), wt, all, QKS * H, KV * H, p), qbytes(wt, KV * H));
+            FH_STEP(write_quantised_part(g, blk(l, "attn_qkv.weight"), wt, all, (QKS + KV) * H, KV * H, p), qbytes(wt, KV * H));
+        } else {
+            FH_STEP(write_quantised(g, blk(l, "attn_q.weight"), wt, QKS * H, p), qbytes(wt, QKS * H));
+            FH_STEP(write_quantised(g, blk(l, "attn_k.weight"), wt, KV * H, p), qbytes(wt, KV * H));
+            FH_STEP(write_quantised(g, blk(l, "attn_v.weight"), wt, KV * H, p), qbytes(wt, KV * H));
+        }
         if (c->flags & FORGE_HIP_FLAG_QKV_BIAS) {             // main.rs:2737-2742
             FH_STEP(write_f32(g, blk(l, "attn_q.bias"), QKS, p), QKS * 4);
             FH_STEP(write_f32(g, blk(l, "attn_k.bias"), KV, p), KV * 4);
@@ -597,8 +624,15 @@ int32_t forge_hip_gguf_export_weights(const forge_hip_gguf* g, const forge_hip_c
         }
         FH_STEP(write_quantised(g, blk(l, "attn_output.weight"), wt, H * QKS, p), qbytes(wt, H * QKS));
         FH_STEP(write_f32(g, blk(l, "ffn_norm.weight"), H, p), H * 4);
-        FH_STEP(write_quantised(g, blk(l, "ffn_gate.weight"), wt, I * H, p), qbytes(wt, I * H));
-        FH_STEP(write_quantised(g, blk(l, "ffn_up.weight"), wt, I * H, p), qbytes(wt, I * H));
+        const TensorInfo* up = g->tensor(blk(l, "ffn_up.weight"));
+        if (!g->tensor(blk(l, "ffn_gate.weight")) && up && up->numel() == 2 * I * H) {
+            // Phi-3: gate|up rows in one tensor (weight_loader.rs:569-580)
+            FH_STEP(write_quantised_part(g, blk(l, "ffn_up.weight"), wt, 2 * I * H, 0, I * H, p), qbytes(wt, I * H));
+            FH_STEP(write_quantised_part(g, blk(l, "ffn_up.weight"), wt, 2 * I * H, I * H, I * H, p), qbytes(wt, I * H));
+        } else {
+            FH_STEP(write_quantised(g, blk(l, "ffn_gate.weight"), wt, I * H, p), qbytes(wt, I * H));
+            FH_STEP(write_quantised(g, blk(l, "ffn_up.weight"), wt, I * H, p), qbytes(wt, I * H));
+        }
         FH_STEP(write_quantised(g, blk(l, "ffn_down.weight"), wt, H * I, p), qbytes(wt, H * I));
     }
     FH_STEP(write_f32(g, "output_norm.weight", H, p), H * 4);

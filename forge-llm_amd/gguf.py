@@ -107,7 +107,8 @@ def split_blob(cfg: dict, blob: np.ndarray) -> dict:
     return out
 
 
-def model_to_gguf(cfg: dict, blob: np.ndarray, tied: bool = True, arch: str = None, path=None, tokens: bool = False) -> bytes:
+def model_to_gguf(cfg: dict, blob: np.ndarray, tied: bool = True, arch: str = None, path=None, tokens: bool = False,
+                  fused: bool = False) -> bytes:
     """A weights blob as a GGUF v3 file with the metadata keys load_config reads (main.rs:700-830).
     tied=True stores the embedding once, as the quantised `token_embd.weight` (what llama.cpp does for models with tied
     embeddings; the blob's f32 table must then be the dequantised lm_head, as `synth.make_weights_blob` makes it);
@@ -115,8 +116,23 @@ def model_to_gguf(cfg: dict, blob: np.ndarray, tied: bool = True, arch: str = No
     `vocab` one-character strings, the key the vocabulary size is read from first."""
     if arch is None:
         # the reference ties QKV bias to the architecture; a window is Mistral's
-        arch = "qwen2" if cfg.get("flags", 0) & 2 else "mistral" if cfg.get("sliding_window", 0) else "llama"
+        arch = "qwen2" if cfg.get("flags", 0) & 2 else "mistral" if cfg.get("sliding_window", 0) else "phi3" if fused else "llama"
     t = split_blob(cfg, blob)
+    if fused:
+        # the Phi-3 file layout (weight_loader.rs:425-427, 531-534): q|k|v rows in `attn_qkv.weight`, gate|up rows in `ffn_up.weight`
+        fused_t = {}
+        for name, (dims, gtype, data) in t.items():
+            if name.endswith("attn_q.weight"):
+                b = name[:-len("attn_q.weight")]
+                k, v = t[b + "attn_k.weight"], t[b + "attn_v.weight"]
+                fused_t[b + "attn_qkv.weight"] = ([dims[0], dims[1] + k[0][1] + v[0][1]], gtype, np.concatenate([data, k[2], v[2]]))
+            elif name.endswith("ffn_gate.weight"):
+                b = name[:-len("ffn_gate.weight")]
+                u = t[b + "ffn_up.weight"]
+                fused_t[b + "ffn_up.weight"] = ([dims[0], dims[1] + u[0][1]], gtype, np.concatenate([data, u[2]]))
+            elif not name.endswith(("attn_k.weight", "attn_v.weight", "ffn_up.weight")):
+                fused_t[name] = (dims, gtype, data)
+        t = fused_t
     if tied:
         dims, gtype, data = t.pop("output.weight")
         t["token_embd.weight"] = (dims, gtype, data)

@@ -214,8 +214,9 @@ int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void
  * The reference reads a model from a GGUF file in three steps: gguf::parse (crates/forgellm-frontend/src/gguf.rs:484-551),
  * load_config (crates/forgellm-cli/src/main.rs:700-830) and `forge export-weights` (main.rs:2585-2757, tensor names
  * mapped by weight_loader.rs:400-447), whose output file is the blob forge_hip_model_create takes.  These entry points are
- * those three steps.  Supported: architectures "llama", "qwen2" (sets FORGE_HIP_FLAG_QKV_BIAS) and "mistral"
- * (`<arch>.attention.sliding_window` becomes config.sliding_window, main.rs:764-767);
+ * those three steps.  Supported: architectures "llama", "qwen2" (sets FORGE_HIP_FLAG_QKV_BIAS) , "mistral"
+ * (`<arch>.attention.sliding_window` becomes config.sliding_window, main.rs:764-767) and "phi3" / "phi" (main.rs:759; the fused
+ * attn_qkv.weight and ffn_up.weight tensors are cut apart like split_fused_tensors, weight_loader.rs:543-583);
  * tensors of GGML type F32, F16, BF16, Q8_0, Q4_0 and -- turned into Q8_0 blocks when they are read, as the reference's loader
  * does (weight_loader.rs:219-229) -- Q4_1, Q4_K, Q5_K, Q6_K, Q8_K; projections mostly Q8_0 or mostly Q4_0 by the reference's
  * majority vote, which counts those other types as Q8_0 (a file whose projections are mostly Q4_K is refused: the reference

@@ -122,7 +122,7 @@ def _get(g, key, types):
 
 def config(g, max_seq=0, flags=0) -> dict:
     arch = _get(g, "general.architecture", (8,)) or "unknown"
-    if arch not in ("llama", "mistral", "qwen2"):
+    if arch not in ("llama", "mistral", "qwen2", "phi3", "phi"):
         raise GgufError(f"unsupported GGUF architecture: {arch}")
     p = arch + "."
     hidden = _get(g, p + "embedding_length", (4,)) or 0
@@ -304,18 +304,39 @@ def export_weights(oracle, g, data, cfg) -> np.ndarray:
             return np.frombuffer(data, np.uint8, data_size(t), g["tensor_data_offset"] + t["offset"])
         return oracle.quantize_weights(wd, _tensor_f32(oracle, g, data, t))
 
+    def quant_parts(name, sizes, wd):
+        """A fused Phi-3 tensor cut into parts (split_weight_three / split_weight_two, weight_loader.rs:543-583, 641-700):
+        the loader converts the whole tensor first, the split cuts the result at element counts."""
+        whole = np.ascontiguousarray(quant(name, sum(sizes), wd), np.uint8)
+        bb = 34 if wd == 8 else 18
+        out, at = [], 0
+        for n in sizes:
+            if n % 32:
+                raise GgufError(f"fused tensor {name} cannot be split on block boundaries")
+            out.append(whole[at // 32 * bb:(at + n) // 32 * bb])
+            at += n
+        return out
+
     H, I = cfg["hidden"], cfg["inter"]
     QKS, KV, V = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"], cfg["vocab"]
     wd = cfg["wdtype"]
     parts = [f32("token_embd.weight", V * H)]
     for l in range(cfg["layers"]):
         b = f"blk.{l}."
-        parts += [f32(b + "attn_norm.weight", H), quant(b + "attn_q.weight", QKS * H, wd), quant(b + "attn_k.weight", KV * H, wd),
-                  quant(b + "attn_v.weight", KV * H, wd)]
+        parts.append(f32(b + "attn_norm.weight", H))
+        if b + "attn_q.weight" not in by_name and b + "attn_qkv.weight" in by_name:
+            parts += quant_parts(b + "attn_qkv.weight", [QKS * H, KV * H, KV * H], wd)
+        else:
+            parts += [quant(b + "attn_q.weight", QKS * H, wd), quant(b + "attn_k.weight", KV * H, wd), quant(b + "attn_v.weight", KV * H, wd)]
         if cfg["flags"] & 2:
             parts += [f32(b + "attn_q.bias", QKS), f32(b + "attn_k.bias", KV), f32(b + "attn_v.bias", KV)]
-        parts += [quant(b + "attn_output.weight", H * QKS, wd), f32(b + "ffn_norm.weight", H),
-                  quant(b + "ffn_gate.weight", I * H, wd), quant(b + "ffn_up.weight", I * H, wd), quant(b + "ffn_down.weight", H * I, wd)]
+        parts += [quant(b + "attn_output.weight", H * QKS, wd), f32(b + "ffn_norm.weight", H)]
+        up = by_name.get(b + "ffn_up.weight")
+        if b + "ffn_gate.weight" not in by_name and up is not None and numel(up) == 2 * I * H:
+            parts += quant_parts(b + "ffn_up.weight", [I * H, I * H], wd)
+        else:
+            parts += [quant(b + "ffn_gate.weight", I * H, wd), quant(b + "ffn_up.weight", I * H, wd)]
+        parts.append(quant(b + "ffn_down.weight", H * I, wd))
     parts.append(f32("output_norm.weight", H))
     lm_name = "output.weight" if "output.weight" in by_name else "lm_head.weight" if "lm_head.weight" in by_name else "token_embd.weight"
     parts.append(quant(lm_name, V * H, cfg["lm_head_dtype"]))

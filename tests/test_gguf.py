@@ -198,6 +198,73 @@ def test_synthetic_model_round_trip(fh, gg, go, oracle, wd, tied, bias, tmp_path
     assert np.array_equal(go.export_weights(oracle, o, data, ocfg), blob)
 
 
+@pytest.mark.parametrize("wd", [Q8, Q4])
+def test_phi3_fused_tensors_are_split(fh, gg, go, oracle, wd):
+    """A Phi-3 file keeps Q|K|V rows in `attn_qkv.weight` and gate|up rows in `ffn_up.weight`; the reference's loader cuts them
+    apart (split_fused_tensors, weight_loader.rs:543-583) before export-weights writes q, k, v, gate, up one by one.
+    blob -> fused GGUF -> blob: identical bytes; library == oracle; the fused tensors vote like any projection."""
+    cfg = fh.synth.tiny(wd, max_seq=640, heads=4, kv_heads=2, head_dim=96, hidden=384)     # Phi-3's head_dim, GQA so that q != k rows
+    blob = fh.synth.make_weights_blob(cfg, seed=21)
+    data = gg.model_to_gguf(cfg, blob, tied=False, fused=True)
+    f = gg.GgufFile(data)
+    names = {t["name"] for t in f.tensors}
+    assert "blk.0.attn_qkv.weight" in names and "blk.0.attn_q.weight" not in names and "blk.0.ffn_gate.weight" not in names
+    got = f.config()
+    assert got["wdtype"] == wd and got["head_dim"] == 96 and got["flags"] == 0
+    assert np.array_equal(f.export_weights(got), blob)
+    o = go.parse(data)
+    assert go.config(o) == got
+    assert np.array_equal(go.export_weights(oracle, o, data, got), blob)
+    f.close()
+    # "phi" is the same architecture to the reference (main.rs:759)
+    data_phi = gg.model_to_gguf(cfg, blob, tied=False, fused=True, arch="phi")
+    assert np.array_equal(gg.GgufFile(data_phi).export_weights(got), blob)
+
+
+def test_phi3_fused_tensors_in_other_formats(fh, gg, go, oracle):
+    """Fused tensors that are not in the blob's format are converted whole and then cut, as the reference's loader does:
+    an F16 `attn_qkv`, a Q6_K `ffn_up` (read as Q8_0) in a Q8_0 model; library == oracle, and each part equals what the same
+    rows give as a tensor of their own."""
+    cfg = fh.synth.tiny(Q8, max_seq=640, hidden=256, inter=512, heads=4, kv_heads=2, head_dim=64)
+    blob = fh.synth.make_weights_blob(cfg, seed=22)
+    t = gg.split_blob(cfg, blob)
+    H, I, QKS, KV = cfg["hidden"], cfg["inter"], 256, 128
+    qkv = np.concatenate([oracle.dequant(Q8, t[f"blk.0.attn_{n}.weight"][2], H * r) for n, r in (("q", QKS), ("k", KV), ("v", KV))])
+    for n in ("q", "k", "v"):
+        del t[f"blk.0.attn_{n}.weight"]
+    t["blk.0.attn_qkv.weight"] = ([H, QKS + 2 * KV], gg.F16, oracle.f32_to_f16(qkv).astype("<u2").view(np.uint8))
+    rng = np.random.default_rng(5)
+    q6 = rng.integers(0, 256, 2 * I * H // 256 * 210, dtype=np.uint8)
+    q6.reshape(-1, 210)[:, 208:] = np.frombuffer(np.float16(rng.uniform(0.001, 0.01, 2 * I * H // 256)).tobytes(), np.uint8).reshape(-1, 2)
+    del t["blk.0.ffn_gate.weight"]
+    t["blk.0.ffn_up.weight"] = ([H, 2 * I], gg.Q6_K, q6)
+    meta = [("general.architecture", gg.STRING, "phi3"), ("phi3.embedding_length", gg.U32, H), ("phi3.block_count", gg.U32, cfg["layers"]),
+            ("phi3.attention.head_count", gg.U32, cfg["heads"]), ("phi3.attention.head_count_kv", gg.U32, cfg["kv_heads"]),
+            ("phi3.feed_forward_length", gg.U32, I), ("phi3.vocab_size", gg.U32, cfg["vocab"]), ("phi3.context_length", gg.U32, 640)]
+    data = gg.write_gguf(meta, [(n, d, g, b) for n, (d, g, b) in t.items()])
+    f = gg.GgufFile(data)
+    got = f.config()
+    o = go.parse(data)
+    assert go.config(o) == got and got["wdtype"] == Q8
+    out = f.export_weights(got)
+    assert np.array_equal(out, go.export_weights(oracle, o, data, got))
+    parts = gg.split_blob(got, out)
+    # each part is what its own rows give when they are quantised as a tensor of their own
+    qkv16 = oracle.f16_to_f32(oracle.f32_to_f16(qkv))
+    for n, r, at in (("q", QKS, 0), ("k", KV, QKS), ("v", KV, QKS + KV)):
+        assert np.array_equal(parts[f"blk.0.attn_{n}.weight"][2], oracle.quantize_weights(Q8, qkv16[at * H:(at + r) * H]))
+    whole = oracle.quantize_weights(Q8, gg.dequant_ggml(gg.Q6_K, q6, 2 * I * H))
+    assert np.array_equal(parts["blk.0.ffn_gate.weight"][2], whole[:I * H // 32 * 34])
+    assert np.array_equal(parts["blk.0.ffn_up.weight"][2], whole[I * H // 32 * 34:])
+    # a fused tensor of the wrong size is refused like any other
+    t["blk.0.attn_qkv.weight"] = ([H, QKS + KV], gg.F16, oracle.f32_to_f16(qkv[:(QKS + KV) * H]).astype("<u2").view(np.uint8))
+    bad = gg.write_gguf(meta, [(n, d, g, b) for n, (d, g, b) in t.items()])
+    with pytest.raises(fh.ForgeHipError, match="elements"):
+        gg.GgufFile(bad).export_weights(got)
+    with pytest.raises(go.GgufError):
+        go.export_weights(oracle, go.parse(bad), bad, got)
+
+
 def test_tensors_in_other_formats_are_converted_like_the_oracle_does(fh, gg, go, oracle):
     """A Q8_0 model whose norms are F16, one projection F32, one BF16, one Q4_0, with an F16 embedding and a Q4_0 output
     matrix: the exporter dequantises / requantises with the reference's routines; library == oracle, byte for byte."""
@@ -570,3 +637,27 @@ def test_model_from_gguf_equals_model_from_blob(fh, gg, torch_gpu, tmp_path):
         assert c.config["max_seq"] == 600 and c.config["flags"] == fh.FLAG_EXACT
         c.forward_prefill(prompt)
         c.close()
+
+
+@pytest.mark.gpu
+def test_phi3_model_from_fused_gguf(fh, gg, oracle, torch_gpu, tmp_path):
+    """A Phi-3-style file (fused tensors, head_dim 96, no GQA) read by forge_hip_model_create_from_gguf: same logits and greedy
+    tokens as the model built from the blob, and the exact mode agrees with the CPU oracle bit for bit."""
+    cfg = fh.synth.tiny(Q8, max_seq=640, hidden=384, inter=768, heads=4, kv_heads=4, head_dim=96)
+    blob = fh.synth.make_weights_blob(cfg, seed=23)
+    path = str(tmp_path / "phi3.gguf")
+    gg.model_to_gguf(cfg, blob, tied=True, fused=True, path=path)
+    a, b = fh.HipModel(cfg, blob), fh.HipModel.from_gguf(path)
+    prompt = fh.synth.uniform_ids(6, 50, cfg["vocab"])
+    la, lb = a.forward_prefill(prompt), b.forward_prefill(prompt)
+    assert np.array_equal(la.view(np.uint32), lb.view(np.uint32))
+    tok = fh.ops.argmax_host(la)
+    for _ in range(6):
+        ta, tb = a.forward_greedy(tok), b.forward_greedy(tok)
+        assert ta == tb
+        tok = ta
+    a.close(); b.close()
+    e = fh.HipModel.from_gguf(path, flags=fh.FLAG_EXACT)
+    om = oracle.Model(dict(cfg, flags=fh.FLAG_EXACT), blob, 0, 1)
+    assert np.array_equal(e.forward_prefill(prompt).view(np.uint32), om.prefill_batched(prompt).view(np.uint32))
+    e.close(); om.close()
