@@ -59,7 +59,9 @@ def prefill_flops(cfg, m):
     H, I = cfg["hidden"], cfg["inter"]
     QKS, KV = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"]
     gemm = 2 * m * cfg["layers"] * (H * QKS + 2 * H * KV + QKS * H + 2 * H * I + I * H)
-    attn = cfg["layers"] * 4 * cfg["head_dim"] * cfg["heads"] * m * (m + 1) // 2
+    w = cfg.get("sliding_window", 0)
+    pairs = m * (m + 1) // 2 if not w or w >= m else w * (w + 1) // 2 + (m - w) * w      # sum over positions of min(p + 1, w)
+    attn = cfg["layers"] * 4 * cfg["head_dim"] * cfg["heads"] * pairs
     return gemm, attn
 
 
@@ -97,7 +99,8 @@ def decode_profile(fh, model, cfg, tok, context, prof_steps=8):
     stage_us = {s: round(v * 1e3, 1) for s, v in stage_ms.items() if v > 0}
     if model.decode_launches == 1:
         # one resident kernel per token: its phases are the stages, timed by the kernel's own clock stamps
-        kv_bytes = cfg["layers"] * 2 * context * cfg["kv_heads"] * cfg["head_dim"] * 2
+        rows = min(context, cfg.get("sliding_window", 0) or context)          # a sliding window bounds the rows a step reads
+        kv_bytes = cfg["layers"] * 2 * rows * cfg["kv_heads"] * cfg["head_dim"] * 2
         total = gemv_bytes_total + kv_bytes
         kernel_ms = sum(stage_ms.values())
         achieved = total / (kernel_ms * 1e-3) / 1e9
@@ -204,6 +207,7 @@ def ops_table(fh, reps=10):
 
 
 def main():
+    global PROMPT_TOKENS
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
@@ -214,9 +218,11 @@ def main():
     ap.add_argument("--no-alt", action="store_true", help="skip the second model that measures the kernel-sequence decode step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (known HBM traffic, for scaling counter readings)")
-    ap.add_argument("--model", choices=("llama32_1b", "llama32_3b", "smollm2_135m", "llama31_8b", "qwen25_1p5b"), default="llama32_1b",
+    ap.add_argument("--model", choices=("llama32_1b", "llama32_3b", "smollm2_135m", "llama31_8b", "qwen25_1p5b", "mistral_7b"), default="llama32_1b",
                     help="shape of the synthetic model (default: the one the headline metric is quoted on)")
     ap.add_argument("--format", choices=("q8_0", "q4_0"), default="q8_0", help="weight format (default: the headline's)")
+    ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
+                    help="length of the prompt (default: the 2502 tokens the metric is quoted on); the cache is sized to fit")
     ap.add_argument("--ops-table", action="store_true",
                     help="instead of the model benchmark, run the isolated kernels at the benchmark configurations' sizes")
     args = ap.parse_args()
@@ -232,10 +238,11 @@ def main():
         ops_table(fh)
         return
     wd = fh.Q8_0 if args.format == "q8_0" else fh.Q4_0
-    cfg = getattr(fh.synth, args.model)(wd, max_seq=4096)
-    headline = args.model == "llama32_1b" and args.format == "q8_0"
+    PROMPT_TOKENS = args.prompt_tokens
+    cfg = getattr(fh.synth, args.model)(wd, max_seq=max(4096, (PROMPT_TOKENS + 2 * (args.warmup + args.steps) + 16 + 1023) // 1024 * 1024))
+    headline = args.model == "llama32_1b" and args.format == "q8_0" and PROMPT_TOKENS == 2502
     model_name = {"llama32_1b": "Llama-3.2-1B", "llama32_3b": "Llama-3.2-3B", "smollm2_135m": "SmolLM2-135M", "llama31_8b": "Llama-3.1-8B",
-                  "qwen25_1p5b": "Qwen2.5-1.5B"}[args.model]
+                  "qwen25_1p5b": "Qwen2.5-1.5B", "mistral_7b": "Mistral-7B (sliding window 4096)"}[args.model]
     t0 = time.perf_counter()
     blob = fh.synth.make_weights_blob(cfg, seed=args.seed, threads=16)
     t_gen = time.perf_counter() - t0

@@ -84,6 +84,13 @@ def llama31_8b(wdtype=8, max_seq=4096):
     return _cfg(4096, 14336, 32, 32, 8, 128, 128256, max_seq, 500000.0, wdtype)
 
 
+def mistral_7b(wdtype=8, max_seq=8192):
+    """Mistral-7B-v0.1 shape: the Llama layer with a sliding window of 4096 positions, vocabulary 32 000."""
+    c = _cfg(4096, 14336, 32, 32, 8, 128, 32000, max_seq, 10000.0, wdtype)
+    c["sliding_window"] = 4096
+    return c
+
+
 def qwen25_1p5b(wdtype=8, max_seq=4096):
     """Qwen2.5-1.5B shape: QKV bias, 12 heads over 2 KV heads, head_dim 128, vocabulary 151 936."""
     c = _cfg(1536, 8960, 28, 12, 2, 128, 151936, max_seq, 1000000.0, wdtype)
