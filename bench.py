@@ -218,7 +218,7 @@ def main():
     ap.add_argument("--no-alt", action="store_true", help="skip the second model that measures the kernel-sequence decode step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (known HBM traffic, for scaling counter readings)")
-    ap.add_argument("--model", choices=("llama32_1b", "llama32_3b", "smollm2_135m", "llama31_8b", "qwen25_1p5b", "mistral_7b"), default="llama32_1b",
+    ap.add_argument("--model", choices=("llama32_1b", "llama32_3b", "smollm2_135m", "llama31_8b", "qwen25_1p5b", "mistral_7b", "phi3_mini"), default="llama32_1b",
                     help="shape of the synthetic model (default: the one the headline metric is quoted on)")
     ap.add_argument("--format", choices=("q8_0", "q4_0"), default="q8_0", help="weight format (default: the headline's)")
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
@@ -242,7 +242,7 @@ def main():
     cfg = getattr(fh.synth, args.model)(wd, max_seq=max(4096, (PROMPT_TOKENS + 2 * (args.warmup + args.steps) + 16 + 1023) // 1024 * 1024))
     headline = args.model == "llama32_1b" and args.format == "q8_0" and PROMPT_TOKENS == 2502
     model_name = {"llama32_1b": "Llama-3.2-1B", "llama32_3b": "Llama-3.2-3B", "smollm2_135m": "SmolLM2-135M", "llama31_8b": "Llama-3.1-8B",
-                  "qwen25_1p5b": "Qwen2.5-1.5B", "mistral_7b": "Mistral-7B (sliding window 4096)"}[args.model]
+                  "qwen25_1p5b": "Qwen2.5-1.5B", "mistral_7b": "Mistral-7B (sliding window 4096)", "phi3_mini": "Phi-3-mini"}[args.model]
     t0 = time.perf_counter()
     blob = fh.synth.make_weights_blob(cfg, seed=args.seed, threads=16)
     t_gen = time.perf_counter() - t0

@@ -536,10 +536,16 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
     constexpr int KPW = 64 / LPK;
     constexpr int REC = HD + 2;
     const uint32_t wave = cx.wave & 3u, lane = cx.lane;
-    float* sh = big;                                                  // [4 waves][4][REC]
+    const uint32_t gt = a.gt, gsize = a.heads / a.kv_heads, gpk = gsize / gt;
+    // With one query head per item only four of the eight waves have keys to walk: the other four then take an item of
+    // their own at the same time (own LDS area, own 256 threads; the barriers are shared).
+    const bool dual = gt == 1;
+    const uint32_t grp = dual ? cx.wave >> 2 : 0u;
+    const uint32_t ltid = dual ? (cx.tid & 255u) : cx.tid, lthreads = dual ? 256u : (uint32_t)PD_THREADS;
+    constexpr int AREA = 16 * REC + 6 * HD;
+    float* sh = big + grp * AREA;                                     // [4 waves][4][REC]
     float* q_lds = sh + 16 * REC;                                     // [gt][HD]
     uint32_t* kvn = reinterpret_cast<uint32_t*>(q_lds + 4 * HD);      // [2][HD] fp16 bits of this position's K and V
-    const uint32_t gt = a.gt, gsize = a.heads / a.kv_heads, gpk = gsize / gt;
     const uint32_t nbx = a.kv_heads * gpk, n_items = nbx * DECODE_SPLITS;
     const uint32_t seq = pos + 1;
     const uint32_t c = lane % LPK, slot = lane / LPK;
@@ -551,11 +557,17 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
     uint32_t chunk = (seq - start + DECODE_SPLITS - 1) / DECODE_SPLITS;
     chunk = (chunk + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
 
-    for (uint32_t item = cx.wg; item < n_items; item += cx.G) {
+    // every workgroup walks the same number of rounds (the barriers inside are workgroup-wide); a wave group whose item
+    // number is past the end only takes part in the barriers
+    const uint32_t per_round = dual ? 2 * cx.G : cx.G;
+    const uint32_t rounds = (n_items + per_round - 1) / per_round;
+    for (uint32_t it = 0; it < rounds; it++) {
+        const uint32_t item = cx.wg + (dual ? 2 * it + grp : it) * cx.G;
+        const bool on = item < n_items;
         const uint32_t bx = item % nbx, split = item / nbx;
         const uint32_t kvh = bx / gpk, sub = bx % gpk;
         const uint32_t h0 = kvh * gsize + sub * gt;
-        const uint32_t t0 = min(seq, start + split * chunk);
+        const uint32_t t0 = on ? min(seq, start + split * chunk) : seq;      // no item: an empty key range
         const uint32_t t1 = min(seq, t0 + chunk);
         const bool has_new = t0 <= pos && pos < t1;
         // The cached K/V rows do not depend on q: the first key blocks of this wave are requested before q is awaited (loads
@@ -575,7 +587,7 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
             }
         }
         // q is awaited even when the split is empty: the wait orders this item's records after the previous layer's readers
-        for (uint32_t e = cx.tid; e < gt * HD || (has_new && e < 2 * HD); e += PD_THREADS) {
+        for (uint32_t e = ltid; on && (e < gt * HD || (has_new && e < 2 * HD)); e += lthreads) {
             const bool need_q = e < gt * HD, need_kv = has_new && e < 2 * HD;
             const uint64_t* pq = a.tq + (size_t)h0 * HD + e;
             const uint64_t* pkv = a.tkv + (e < HD ? kvh * HD + e : a.KV + kvh * HD + (e - HD));
@@ -599,7 +611,7 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
             }
         }
 
-        for (uint32_t g = cx.wave >> 2; g < gt; g += PD_WAVES / 4) {
+        for (uint32_t g = dual ? 0u : cx.wave >> 2; g < gt; g += PD_WAVES / 4) {
             float qf[8], acc[8], m = -INFINITY, l = 0.f;
 #pragma unroll
             for (int i = 0; i < 8; i++) { acc[i] = 0.f; qf[i] = dvalid ? q_lds[g * HD + c * 8 + i] : 0.f; }
@@ -671,7 +683,7 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
         }
         __syncthreads();
         // merge the four key waves: one thread per output element
-        for (uint32_t e = cx.tid; e < gt * HD; e += PD_THREADS) {
+        for (uint32_t e = ltid; on && e < gt * HD; e += lthreads) {
             const uint32_t gg = e / HD, d = e % HD;
             float mm = sh[gg * REC + HD], ll = sh[gg * REC + HD + 1], av = sh[gg * REC + d];
             for (int w = 1; w < 4; w++) {
@@ -1118,6 +1130,10 @@ hipError_t launch_pd_hd(const PdState* st, hipStream_t s) {
     return hipLaunchCooperativeKernel(pd_kernel<HD>(st), dim3(st->grid), dim3(PD_THREADS), kargs, st->lds, s);
 }
 
+const void* pd_kernel_for(const PdState* st) {
+    return st->hd == 64 ? pd_kernel<64>(st) : st->hd == 96 ? pd_kernel<96>(st) : pd_kernel<128>(st);
+}
+
 }  // namespace
 
 void pd_destroy(PdState* st) { delete st; }
@@ -1129,7 +1145,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
                   const float* qkv_bias, PdState** out) {
     *out = nullptr;
     if (c.flags & FORGE_HIP_FLAG_EXACT) return FORGE_HIP_OK;
-    if (c.head_dim != 64 && c.head_dim != 128) return FORGE_HIP_OK;
+    if (c.head_dim != 64 && c.head_dim != 96 && c.head_dim != 128) return FORGE_HIP_OK;
     int dev = 0, coop = 0, cus = 0, khz = 0;
     FH_HIP(hipGetDevice(&dev));
     FH_HIP(hipDeviceGetAttribute(&coop, hipDeviceAttributeCooperativeLaunch, dev));
@@ -1158,7 +1174,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     a.off_big = a.off_misc + PD_MISC_BYTES;
     if (a.off_big + 4096 > PD_LDS_BYTES) return FORGE_HIP_OK;
     const uint32_t big = PD_LDS_BYTES - 64 - a.off_big;
-    const uint32_t attn_bytes = (16 * (hd + 2) + 6 * hd) * 4;
+    const uint32_t attn_bytes = (a.gt == 1 ? 2 : 1) * (16 * (hd + 2) + 6 * hd) * 4;      // two items at a time when a group has one head
     if ((H + 32) * 4 > big || attn_bytes > big || DECODE_SPLITS * (hd + 2) * 4 > big) return FORGE_HIP_OK;
     st->lds = a.off_big + big;
 
@@ -1191,7 +1207,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     {
         int per_cu = 0;
         hipError_t e = hipErrorInvalidValue;
-e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, hd == 64 ? pd_kernel<64>(st.get()) : pd_kernel<128>(st.get()), PD_THREADS, st->lds);
+        e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, pd_kernel_for(st.get()), PD_THREADS, st->lds);
         if (e != hipSuccess || per_cu < 1) { (void)hipGetLastError(); return FORGE_HIP_OK; }
     }
 
@@ -1259,7 +1275,7 @@ int32_t pd_set_repeat_penalty(PdState* st, float penalty) {
     const float old = st->args.penalty;
     st->args.penalty = penalty;
     int per_cu = 0;
-    const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, st->hd == 64 ? pd_kernel<64>(st) : pd_kernel<128>(st), PD_THREADS, st->lds);
+    const hipError_t e = hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, pd_kernel_for(st), PD_THREADS, st->lds);
     if (e != hipSuccess || per_cu < 1) {
         (void)hipGetLastError();
         st->args.penalty = old;
@@ -1286,7 +1302,7 @@ int32_t pd_enqueue(PdState* st, bool profile, uint32_t token, hipStream_t s) {
     }
     unsigned long long* keep = a.stamps;
     if (!profile) a.stamps = nullptr;
-    const hipError_t e = st->hd == 64 ? launch_pd_hd<64>(st, s) : launch_pd_hd<128>(st, s);
+    const hipError_t e = st->hd == 64 ? launch_pd_hd<64>(st, s) : st->hd == 96 ? launch_pd_hd<96>(st, s) : launch_pd_hd<128>(st, s);
     a.stamps = keep;
     if (e != hipSuccess) return fail(FORGE_HIP_ERR_HIP, std::string("persistent decode launch: ") + hipGetErrorString(e));
     a.tag_base += st->tags_per_launch;

@@ -84,6 +84,11 @@ def llama31_8b(wdtype=8, max_seq=4096):
     return _cfg(4096, 14336, 32, 32, 8, 128, 128256, max_seq, 500000.0, wdtype)
 
 
+def phi3_mini(wdtype=8, max_seq=4096):
+    """Phi-3-mini-4k shape: 32 heads of 96 with a KV head each, vocabulary 32 064."""
+    return _cfg(3072, 8192, 32, 32, 32, 96, 32064, max_seq, 10000.0, wdtype)
+
+
 def mistral_7b(wdtype=8, max_seq=8192):
     """Mistral-7B-v0.1 shape: the Llama layer with a sliding window of 4096 positions, vocabulary 32 000."""
     c = _cfg(4096, 14336, 32, 32, 8, 128, 32000, max_seq, 10000.0, wdtype)

@@ -296,12 +296,25 @@ def test_persistent_decode_kernel_default_summation(fh, oracle, torch_gpu, monke
     seq.close(); one.close()
 
 
-@pytest.mark.parametrize("shape", ["smollm2_135m", "llama_1b_2layers", "llama_3b_2layers"])
+@pytest.mark.parametrize("shape", ["smollm2_135m", "llama_1b_2layers", "llama_3b_2layers", "phi3_mini_2layers", "hd96_gqa", "mha_12_heads"])
 def test_persistent_decode_kernel_real_shapes(fh, torch_gpu, monkeypatch, shape):
     """Same check on the shapes that matter: SmolLM2-135M (hidden 576, 9 heads over 3 KV heads: partial weight
-    units, three heads per group), the Llama-3.2-1B layer shape at a context that spans every split, and the
-    Llama-3.2-3B layer shape (hidden 3072: three weight units per row, head_dim 128, three heads per group)."""
-    if shape == "smollm2_135m":
+    units, three heads per group), the Llama-3.2-1B layer shape at a context that spans every split, the
+    Llama-3.2-3B layer shape (hidden 3072: three weight units per row, head_dim 128, three heads per group), the
+    Phi-3-mini layer shape (head_dim 96: 12 of a key row's 16 lanes carry data; 32 heads with a KV head each) and a small
+    head_dim 96 model with two heads per KV head.  With a KV head per query head the attention phase gives each half of a
+    workgroup's waves an item of its own: Phi-3-mini has 1024 items (two full rounds), 12 heads of 64 have 384 (in the only
+    round the second halves of workgroups 128-255 have none)."""
+    if shape == "mha_12_heads":
+        cfg = fh.synth.tiny(Q8, max_seq=1024, hidden=768, inter=1024, layers=2, heads=12, kv_heads=12, head_dim=64, vocab=2000)
+        n_prompt = 500
+    elif shape == "phi3_mini_2layers":
+        cfg = fh.synth.tiny(Q8, max_seq=1024, hidden=3072, inter=8192, layers=2, heads=32, kv_heads=32, head_dim=96, vocab=32064)
+        n_prompt = 700
+    elif shape == "hd96_gqa":
+        cfg = fh.synth.tiny(Q4, max_seq=1024, hidden=384, inter=768, layers=3, heads=4, kv_heads=2, head_dim=96, vocab=1000)
+        n_prompt = 333
+    elif shape == "smollm2_135m":
         cfg = fh.synth.smollm2_135m(Q8, max_seq=1024)
         n_prompt = 300
     elif shape == "llama_3b_2layers":
