@@ -177,3 +177,56 @@ int main(void) {
     env = dict(os.environ, LD_LIBRARY_PATH=libdir + ":/opt/rocm/lib:" + os.environ.get("LD_LIBRARY_PATH", ""))
     r = subprocess.run([str(exe)], capture_output=True, text=True, env=env, timeout=120)
     assert r.returncode == 0 and r.stdout.strip() == "ok", (r.returncode, r.stdout, r.stderr)
+
+
+def _c_declarations(header_text):
+    """{name: [parameter declarations]} of every function the header declares."""
+    import re
+    text = re.sub(r"/\*.*?\*/", " ", header_text, flags=re.S)
+    text = re.sub(r"^\s*#.*$", " ", text, flags=re.M)
+    out = {}
+    for m in re.finditer(r"\b(forge_hip_\w+)\s*\(([^;{}]*?)\)\s*;", text, flags=re.S):
+        params = m.group(2).strip()
+        out[m.group(1)] = [] if params in ("", "void") else [p.strip() for p in params.split(",")]
+    return out, text
+
+
+def test_rust_binding_matches_the_header():
+    """The crate text that the reference's maintainers would add (forgellm-codegen-hip) cannot be compiled here, so its
+    `extern "C"` block and its `#[repr(C)]` config are held to include/forge_hip.h: every function it names is declared
+    there with the same number of parameters, in the same order by name, pointer for pointer; the struct has the header's
+    fields in the header's order; placeholders and braces are balanced."""
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    rust = open(os.path.join(root, "forge-llm_amd", "bindings", "forgellm-codegen-hip", "src", "lib.rs")).read()
+    decls, ctext = _c_declarations(open(os.path.join(root, "include", "forge_hip.h")).read())
+    block = re.search(r'extern "C" \{(.*?)\n\}', rust, flags=re.S).group(1)
+    fns = re.findall(r"fn (forge_hip_\w+)\((.*?)\)(?: -> ([\w\s\*]+))?;", block)
+    assert len(fns) >= 14
+    ctype = {"u32": "uint32_t", "u64": "uint64_t", "i32": "int32_t", "i64": "int64_t", "f32": "float", "u8": "uint8_t", "c_char": "char",
+             "ForgeHipConfig": "forge_hip_config", "ForgeHipModel": "forge_hip_model"}
+    for name, params, _ret in fns:
+        assert name in decls, name
+        rparams = [p.strip() for p in params.split(",")] if params.strip() else []
+        assert len(rparams) == len(decls[name]), (name, rparams, decls[name])
+        for rp, cp in zip(rparams, decls[name]):
+            rname, rtype = [x.strip() for x in rp.split(":")]
+            assert re.search(r"\b" + re.escape(rname) + r"$", cp), (name, rp, cp)          # same parameter name
+            assert rtype.count("*") == cp.count("*"), (name, rp, cp)                         # same level of indirection
+            assert ("*const" in rtype) == ("const" in cp) or "*" not in rtype, (name, rp, cp)
+            base = rtype.replace("*const", "").replace("*mut", "").strip()
+            assert ctype[base] in cp, (name, rp, cp)
+    # the struct: same fields, same order, same types
+    cstruct = re.search(r"typedef struct forge_hip_config \{(.*?)\} forge_hip_config;", ctext, flags=re.S).group(1)
+    cfields = []
+    for ty, names in re.findall(r"(uint32_t|float)\s+([^;]+);", cstruct):
+        cfields += [(n.strip(), ty) for n in names.split(",")]
+    rstruct = re.search(r"pub struct ForgeHipConfig \{(.*?)\}", rust, flags=re.S).group(1)
+    rfields = [(n, ctype[t]) for n, t in re.findall(r"pub (\w+): (\w+),", rstruct)]
+    assert rfields == cfields
+    # every template placeholder is replaced by a .replace() of the generator
+    for ph in set(re.findall(r"@[A-Z_]+@", rust)):
+        assert f'.replace("{ph}"' in rust, ph
+    for text in re.findall(r'r#"(.*?)"#', rust, flags=re.S) + [re.sub(r'r#".*?"#', '""', rust, flags=re.S)]:
+        code = re.sub(r'"(?:[^"\\\n]|\\.)*"', '""', text)           # string literals may hold a lone bracket
+        assert code.count("{") == code.count("}") and code.count("(") == code.count(")"), text[:60]
