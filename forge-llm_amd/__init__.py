@@ -137,9 +137,9 @@ def lib():
     L.forge_hip_attn_decode_f16kv.restype = i32
     L.forge_hip_attn_decode_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, vp]
     L.forge_hip_attn_prefill_sliding_f16kv.restype = i32
-    L.forge_hip_attn_prefill_sliding_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]
+    L.forge_hip_attn_prefill_sliding_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, vp]
     L.forge_hip_attn_decode_sliding_f16kv.restype = i32
-    L.forge_hip_attn_decode_sliding_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, vp]
+    L.forge_hip_attn_decode_sliding_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]
     L.forge_hip_argmax.restype = i32
     L.forge_hip_argmax.argtypes = [vp, u32, vp, vp]
     L.forge_hip_model_set_repeat_penalty.restype = i32

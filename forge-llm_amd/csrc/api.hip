@@ -5,6 +5,8 @@
 
 #include <vector>
 
+#include <algorithm>
+
 #include "common.h"
 #include "expf_ref.h"
 
@@ -242,7 +244,7 @@ int32_t forge_hip_attn_prefill_f16kv(const float* q_dev, const uint16_t* k_cache
     if (rc) return rc;
     if (flags & FORGE_HIP_FLAG_EXACT)
         launch_attn_exact(true, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr,
-                          nullptr, M, base_pos, nullptr, heads, kv_heads, head_dim, (hipStream_t)stream);
+                          nullptr, M, base_pos, nullptr, heads, kv_heads, head_dim, 0u, 0u, (hipStream_t)stream);
     else
         launch_attn_prefill(q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, M, base_pos,
                             heads, kv_heads, head_dim, 0u, (hipStream_t)stream);
@@ -252,13 +254,18 @@ int32_t forge_hip_attn_prefill_f16kv(const float* q_dev, const uint16_t* k_cache
 
 int32_t forge_hip_attn_prefill_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                              float* out_dev, uint32_t M, uint32_t base_pos, uint32_t window, uint32_t heads,
-                                             uint32_t kv_heads, uint32_t head_dim, void* stream) {
+                                             uint32_t kv_heads, uint32_t head_dim, uint32_t flags, void* stream) {
     FH_CHECK(q_dev && k_cache_dev && v_cache_dev && out_dev, "attn_prefill_sliding: null pointer");
     FH_CHECK(window >= 1, "attn_prefill_sliding: window must be at least 1");
+    FH_CHECK((flags & ~FORGE_HIP_FLAG_EXACT) == 0, "attn_prefill_sliding: unknown flag bits");
     int32_t rc = check_attn_shape("attn_prefill_sliding", heads, kv_heads, head_dim);
     if (rc) return rc;
-    launch_attn_prefill(q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, M, base_pos, heads,
-                        kv_heads, head_dim, window, (hipStream_t)stream);
+    if (flags & FORGE_HIP_FLAG_EXACT)
+        launch_attn_exact(true, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr, nullptr, M,
+                          base_pos, nullptr, heads, kv_heads, head_dim, window, base_pos + M, (hipStream_t)stream);
+    else
+        launch_attn_prefill(q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, M, base_pos, heads,
+                            kv_heads, head_dim, window, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }
@@ -273,7 +280,7 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
     if (rc) return rc;
     if (flags & FORGE_HIP_FLAG_EXACT) {
         launch_attn_exact(false, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr,
-                          nullptr, 1, seq_len - 1, nullptr, heads, kv_heads, head_dim, (hipStream_t)stream);
+                          nullptr, 1, seq_len - 1, nullptr, heads, kv_heads, head_dim, 0u, 0u, (hipStream_t)stream);
     } else {
         rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
         if (rc) return rc;
@@ -286,16 +293,23 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
 
 int32_t forge_hip_attn_decode_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                             float* out_dev, uint32_t seq_len, uint32_t window, uint32_t heads,
-                                            uint32_t kv_heads, uint32_t head_dim, void* stream) {
+                                            uint32_t kv_heads, uint32_t head_dim, uint32_t flags, void* stream) {
     FH_CHECK(q_dev && k_cache_dev && v_cache_dev && out_dev, "attn_decode_sliding: null pointer");
     FH_CHECK(seq_len >= 1, "attn_decode_sliding: seq_len must be at least 1");
     FH_CHECK(window >= 1, "attn_decode_sliding: window must be at least 1");
+    FH_CHECK((flags & ~FORGE_HIP_FLAG_EXACT) == 0, "attn_decode_sliding: unknown flag bits");
     int32_t rc = check_attn_shape("attn_decode_sliding", heads, kv_heads, head_dim);
     if (rc) return rc;
-    rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
-    if (rc) return rc;
-    launch_attn_decode(q_dev, k_cache_dev, v_cache_dev, out_dev, nullptr, nullptr, seq_len, nullptr, heads, kv_heads, head_dim,
-                       window, g_attn.p, (hipStream_t)stream);
+    if (flags & FORGE_HIP_FLAG_EXACT) {
+        FH_CHECK(std::min(window, seq_len) <= attn_exact_max_window(), "attn_decode_sliding: the exact kernel keeps at most 12288 scores");
+        launch_attn_exact(false, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr, nullptr, 1,
+                          seq_len - 1, nullptr, heads, kv_heads, head_dim, window, seq_len, (hipStream_t)stream);
+    } else {
+        rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
+        if (rc) return rc;
+        launch_attn_decode(q_dev, k_cache_dev, v_cache_dev, out_dev, nullptr, nullptr, seq_len, nullptr, heads, kv_heads, head_dim,
+                           window, g_attn.p, (hipStream_t)stream);
+    }
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }

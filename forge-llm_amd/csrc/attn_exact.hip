@@ -10,6 +10,8 @@
 // It is a VALU kernel: one workgroup per (query row, head), keys across lanes for the
 // scores, head dims across lanes for P.V.  The MFMA / split-sequence kernels are the fast
 // path and agree with it to the float tolerance.
+#include <algorithm>
+
 #include "common.h"
 #include "device_utils.h"
 #include "expf_ref.h"
@@ -22,7 +24,7 @@ template <int HD, bool BATCH>
 __global__ void attn_exact_kernel(const float* __restrict__ q, uint32_t q_stride, const uint16_t* __restrict__ kc,
                                   const uint16_t* __restrict__ vc, float* __restrict__ out, uint32_t out_stride,
                                   int8_t* __restrict__ oq, uint16_t* __restrict__ osc, uint32_t base_pos,
-                                  const uint32_t* __restrict__ pos_dev, uint32_t heads, uint32_t kv_heads) {
+                                  const uint32_t* __restrict__ pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t window) {
     __shared__ float qs[HD];
     __shared__ float e[XB];
     __shared__ float red[2];
@@ -38,11 +40,17 @@ __global__ void attn_exact_kernel(const float* __restrict__ q, uint32_t q_stride
     __syncthreads();
 
     float m_i = -INFINITY, l_i = 0.f, acc = 0.f;   // acc: head dim `tid`
-    for (uint32_t bs = 0; bs < seq; bs += XB) {
+    // attention_sliding_batch (emit.rs:907-1046, BATCH only): the same 64-key blocks, aligned at multiples of 64; blocks
+    // that end before the query's window leave its state untouched, so the walk starts at the block that holds the
+    // window's first key, and in that block the keys before it take no part (maximum, sums) or carry weight 0 (P.V:
+    // adding 0 * v changes nothing).
+    const uint32_t win_start = (window != 0 && seq > window) ? seq - window : 0;
+    for (uint32_t bs = win_start / XB * XB; bs < seq; bs += XB) {
         const uint32_t bl = min((uint32_t)XB, seq - bs);
+        const uint32_t lo = win_start > bs ? win_start - bs : 0;
         // ---- scores: thread bi owns key bs+bi; sum += q[i]*k[i] in order, then * scale
         float s = -INFINITY;
-        if (tid < bl) {
+        if (tid >= lo && tid < bl) {
             const uint16_t* krow = kc + (size_t)(bs + tid) * kv_stride + kvh * HD;
             float sum = 0.f;
 #pragma unroll
@@ -69,20 +77,20 @@ __global__ void attn_exact_kernel(const float* __restrict__ q, uint32_t q_stride
         const float exp_scale = expf_ref<true>(m_prev - m_i);
         l_i = l_i * exp_scale;
         acc = acc * exp_scale;
-        if (tid < bl) e[tid] = expf_ref<true>(s - m_i);
+        if (tid >= lo && tid < bl) e[tid] = expf_ref<true>(s - m_i);
         __syncthreads();
         // ---- l_block: sequential over the block (every thread redundantly: same bits)
         float l_block = 0.f;
-        for (uint32_t bi = 0; bi < bl; bi++) l_block = l_block + e[bi];
+        for (uint32_t bi = lo; bi < bl; bi++) l_block = l_block + e[bi];
         l_i = l_i + l_block;
         // ---- P.V for head dim tid
         if (tid < HD) {
             const uint16_t* vcol = vc + (size_t)bs * kv_stride + kvh * HD + tid;
             if (BATCH) {
-                for (uint32_t bi = 0; bi < bl; bi++) acc = acc + e[bi] * f16_bits_to_f32(vcol[(size_t)bi * kv_stride]);
+                for (uint32_t bi = lo; bi < bl; bi++) acc = acc + e[bi] * f16_bits_to_f32(vcol[(size_t)bi * kv_stride]);
             } else {
                 float sum = 0.f;
-                for (uint32_t bi = 0; bi < bl; bi++) sum = sum + e[bi] * f16_bits_to_f32(vcol[(size_t)bi * kv_stride]);
+                for (uint32_t bi = lo; bi < bl; bi++) sum = sum + e[bi] * f16_bits_to_f32(vcol[(size_t)bi * kv_stride]);
                 acc = acc + sum;
             }
         }
@@ -106,14 +114,97 @@ __global__ void attn_exact_kernel(const float* __restrict__ q, uint32_t q_stride
     }
 }
 
+// attention_sliding (emit.rs:598-627), the decode attention of a model with a window: no blocks, a plain softmax over the
+// last min(window, seq) rows — scores, their maximum, exp and a sequential sum, a multiplication by the reciprocal, then
+// for every head dim a sequential sum of weight * v.  The scores live in dynamic LDS (wl floats).
+template <int HD>
+__global__ void attn_exact_sliding_kernel(const float* __restrict__ q, uint32_t q_stride, const uint16_t* __restrict__ kc,
+                                          const uint16_t* __restrict__ vc, float* __restrict__ out, uint32_t out_stride,
+                                          int8_t* __restrict__ oq, uint16_t* __restrict__ osc, uint32_t base_pos,
+                                          const uint32_t* __restrict__ pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t window) {
+    extern __shared__ float sc[];          // [wl] scores, then weights
+    __shared__ float qs[HD];
+    __shared__ float red[4];
+    const uint32_t tid = threadIdx.x, nt = blockDim.x;
+    const uint32_t h = blockIdx.x, r = blockIdx.y;
+    const uint32_t kvh = h / (heads / kv_heads);
+    const uint32_t seq = (pos_dev ? *pos_dev : base_pos) + r + 1;
+    const uint32_t start = seq > window ? seq - window : 0, wl = seq - start;
+    const uint32_t kv_stride = kv_heads * HD;
+    const float scale = 1.0f / sqrtf((float)HD);
+    if (tid < HD) qs[tid] = q[(size_t)r * q_stride + h * HD + tid];
+    __syncthreads();
+    float mx = -INFINITY;
+    for (uint32_t si = tid; si < wl; si += nt) {
+        const uint16_t* krow = kc + (size_t)(start + si) * kv_stride + kvh * HD;
+        float sum = 0.f;
+#pragma unroll
+        for (int c = 0; c < HD / 8; c++) {
+            const uint4 w = *reinterpret_cast<const uint4*>(krow + c * 8);
+            const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                sum = sum + qs[c * 8 + 2 * j] * f16_bits_to_f32((uint16_t)(ww[j] & 0xFFFFu));
+                sum = sum + qs[c * 8 + 2 * j + 1] * f16_bits_to_f32((uint16_t)(ww[j] >> 16));
+            }
+        }
+        const float s = sum * scale;
+        sc[si] = s;
+        mx = fmaxf(mx, s);
+    }
+    mx = wave_max(mx);                      // the maximum does not depend on the order
+    if ((tid & 63u) == 0) red[tid >> 6] = mx;
+    __syncthreads();
+    mx = red[0];
+    for (uint32_t w = 1; w < nt / 64; w++) mx = fmaxf(mx, red[w]);
+    for (uint32_t si = tid; si < wl; si += nt) sc[si] = expf_ref<true>(sc[si] - mx);
+    __syncthreads();
+    float sum = 0.f;                        // sequential, by every thread: same bits
+    for (uint32_t si = 0; si < wl; si++) sum = sum + sc[si];
+    const float inv = sum > 0.0f ? 1.0f / sum : 0.0f;
+    __syncthreads();
+    for (uint32_t si = tid; si < wl; si += nt) sc[si] = sc[si] * inv;
+    __syncthreads();
+    float o = 0.f;
+    if (tid < HD) {
+        const uint16_t* vcol = vc + (size_t)start * kv_stride + kvh * HD + tid;
+        for (uint32_t si = 0; si < wl; si++) o = o + sc[si] * f16_bits_to_f32(vcol[(size_t)si * kv_stride]);
+        if (out) out[(size_t)r * out_stride + h * HD + tid] = o;
+    }
+    if (oq) {
+        float amax = tid < HD ? fabsf(o) : 0.f;
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+        float qinv;
+        const float qsc = act_scale(amax, qinv);
+        if (tid < HD) {
+            const size_t idx = (size_t)r * heads * HD + h * HD + tid;
+            oq[idx] = (int8_t)quant_code(o * qinv);
+            if ((tid & 31) == 0) osc[idx / 32] = f32_to_f16_bits(qsc);
+        }
+    }
+}
+
+// Longest window (rows whose scores one workgroup keeps in LDS) the order-faithful decode attention takes.
+uint32_t attn_exact_max_window() { return 12288; }
+
 void launch_attn_exact(bool batch_order, const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc,
                        float* out, uint32_t out_stride, int8_t* oq, uint16_t* osc, uint32_t M, uint32_t base_pos,
-                       const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s) {
+                       const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, uint32_t window, uint32_t max_rows,
+                       hipStream_t s) {
     if (M == 0) return;
     dim3 grid(heads, M);
     const uint32_t threads = hd <= 64 ? 64 : 128;
+    if (window != 0 && !batch_order) {
+        // max_rows: the most rows the cache can hold (the position may be known to the device only)
+        const size_t lds = (size_t)std::min(window, max_rows) * sizeof(float);
+        if (hd == 64) fh::launch(attn_exact_sliding_kernel<64>, grid, 128, lds, s, q, q_stride, kc, vc, out, out_stride, oq, osc, base_pos, pos_dev, heads, kv_heads, window);
+        else if (hd == 96) fh::launch(attn_exact_sliding_kernel<96>, grid, 128, lds, s, q, q_stride, kc, vc, out, out_stride, oq, osc, base_pos, pos_dev, heads, kv_heads, window);
+        else fh::launch(attn_exact_sliding_kernel<128>, grid, 128, lds, s, q, q_stride, kc, vc, out, out_stride, oq, osc, base_pos, pos_dev, heads, kv_heads, window);
+        return;
+    }
 #define FH_AX(HD_, B_) \
-    fh::launch(attn_exact_kernel<HD_, B_>, grid, threads, 0, s, q, q_stride, kc, vc, out, out_stride, oq, osc, base_pos, pos_dev, heads, kv_heads)
+    fh::launch(attn_exact_kernel<HD_, B_>, grid, threads, 0, s, q, q_stride, kc, vc, out, out_stride, oq, osc, base_pos, pos_dev, heads, kv_heads, window)
     if (hd == 64) { if (batch_order) FH_AX(64, true); else FH_AX(64, false); }
     else if (hd == 96) { if (batch_order) FH_AX(96, true); else FH_AX(96, false); }
     else { if (batch_order) FH_AX(128, true); else FH_AX(128, false); }

@@ -160,10 +160,14 @@ bool attn_head_dim_supported(uint32_t hd);
 
 // attn_exact.hip — order-faithful attention (one workgroup per row and head).  batch_order selects
 // attention_flash_batch's accumulation order, otherwise attention_flash's.  Row r sits at position
-// (pos_dev ? *pos_dev : base_pos) + r and sees keys [0, that position].
+// (pos_dev ? *pos_dev : base_pos) + r and sees keys [0, that position].  window != 0: attention_sliding_batch's order
+// (batch_order) or attention_sliding's plain softmax over the last `window` rows, whose scores take min(window, max_rows)
+// floats of LDS (max_rows = the rows the cache can hold; window <= attn_exact_max_window() or max_rows <= it).
 void launch_attn_exact(bool batch_order, const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc,
                        float* out, uint32_t out_stride, int8_t* oq, uint16_t* osc, uint32_t M, uint32_t base_pos,
-                       const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s);
+                       const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, uint32_t window, uint32_t max_rows,
+                       hipStream_t s);
+uint32_t attn_exact_max_window();
 
 // decode_persistent.hip — the whole decode step as one resident kernel (fast mode only)
 struct PdLayerIn {

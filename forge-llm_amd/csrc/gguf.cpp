@@ -572,10 +572,6 @@ int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_
     const uint64_t seq = max_seq ? max_seq : ctx;
     // Some(0) would make the reference attend to nothing (emit.rs:604-605)
     if (has_window && window == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: a sliding window of 0 positions");
-    // a model with a window runs `attention_sliding` in the reference (emit.rs:598-627, 4156-4170), a plain softmax over the
-    // window: within the window it equals full attention up to rounding, but not bit for bit
-    if (has_window && (flags & FORGE_HIP_FLAG_EXACT))
-        return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: FORGE_HIP_FLAG_EXACT is not available for a model with a sliding window");
     FH_CHECK(vocab <= 0xFFFFFFFFull && seq <= 0xFFFFFFFFull, "gguf: vocabulary or context length out of range");
     forge_hip_config c{};
     c.hidden = hidden; c.inter = inter; c.layers = layers; c.heads = heads; c.kv_heads = kv_heads;

@@ -165,10 +165,10 @@ int32_t validate(const forge_hip_config* c) {
     // The reference switches to its non-flash attention (a different summation order) when
     // max_seq_len <= 512 (emit.rs:126-128); the order-faithful kernels follow the flash variants only.
     FH_CHECK(!(c->flags & FORGE_HIP_FLAG_EXACT) || c->max_seq > 512, "FORGE_HIP_FLAG_EXACT needs max_seq > 512");
-    // a model with a window runs attention_sliding in the reference (emit.rs:598-627, 4156-4170): a plain softmax over the
-    // window, which the order-faithful kernels do not restate
-    FH_CHECK(!(c->flags & FORGE_HIP_FLAG_EXACT) || c->sliding_window == 0,
-             "FORGE_HIP_FLAG_EXACT is not available for a model with a sliding window");
+    // a model with a window runs attention_sliding in the reference (emit.rs:598-627, 4156-4170), whose order-faithful
+    // restatement keeps one row of scores in LDS
+    FH_CHECK(!(c->flags & FORGE_HIP_FLAG_EXACT) || c->sliding_window == 0 || std::min(c->sliding_window, c->max_seq) <= attn_exact_max_window(),
+             "FORGE_HIP_FLAG_EXACT with a sliding window needs min(sliding_window, max_seq) <= 12288");
     FH_CHECK(gemv_k_supported(c->hidden) && gemv_k_supported(c->inter) && gemv_k_supported(c->heads * c->head_dim),
              "hidden, inter and heads*head_dim must be at most 16384");
     return FORGE_HIP_OK;
@@ -185,7 +185,7 @@ void enqueue_decode_attention(forge_hip_model* m, uint32_t l, const float* q, ui
         StageMark t(m, ST_ATTN);
         if (exact)
             launch_attn_exact(false, q, q_stride, m->kc(l), m->vc(l), nullptr, m->QKS, aq, asc, 1, 0, m->d_pos(), c.heads,
-                              c.kv_heads, c.head_dim, s);
+                              c.kv_heads, c.head_dim, c.sliding_window, c.max_seq, s);
         else
             launch_attn_decode(q, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads, c.head_dim,
                                c.sliding_window, m->attn_ws.p, s);
@@ -255,7 +255,7 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
                              c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s);
     }
     if (exact) {
-        { StageMark t(m, ST_ATTN); launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, s); }
+        { StageMark t(m, ST_ATTN); launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, c.sliding_window, c.max_seq, s); }
         { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
     } else if (m->prefill_fuse_quant) {
         // the attention kernel writes the o projection's quantised input itself

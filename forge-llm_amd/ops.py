@@ -235,7 +235,7 @@ def attention_flash(q, k_cache, v_cache, seq_len, heads, kv_heads, head_dim, fla
     return out
 
 
-def attention_sliding_batch(q, k_cache, v_cache, base_pos, window, heads, kv_heads, head_dim):
+def attention_sliding_batch(q, k_cache, v_cache, base_pos, window, heads, kv_heads, head_dim, flags=0):
     """attention_sliding_batch over an fp16 cache: row r (position base_pos + r) sees the last `window` positions up to its own."""
     from . import check, lib
     torch = _torch()
@@ -246,11 +246,11 @@ def attention_sliding_batch(q, k_cache, v_cache, base_pos, window, heads, kv_hea
         raise ValueError("cache holds fewer than base_pos + M rows")
     out = torch.empty_like(q)
     check(lib().forge_hip_attn_prefill_sliding_f16kv(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), M, base_pos, window,
-                                                     heads, kv_heads, head_dim, _stream()))
+                                                     heads, kv_heads, head_dim, flags, _stream()))
     return out
 
 
-def attention_sliding(q, k_cache, v_cache, seq_len, window, heads, kv_heads, head_dim):
+def attention_sliding(q, k_cache, v_cache, seq_len, window, heads, kv_heads, head_dim, flags=0):
     """attention_sliding over an fp16 cache: one query f32 [heads*hd] against the last min(window, seq_len) of seq_len rows."""
     from . import check, lib
     torch = _torch()
@@ -260,7 +260,7 @@ def attention_sliding(q, k_cache, v_cache, seq_len, window, heads, kv_heads, hea
         raise ValueError("cache holds fewer than seq_len rows")
     out = torch.empty_like(q)
     check(lib().forge_hip_attn_decode_sliding_f16kv(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), seq_len, window, heads,
-                                                    kv_heads, head_dim, _stream()))
+                                                    kv_heads, head_dim, flags, _stream()))
     return out
 
 

@@ -59,7 +59,7 @@ typedef struct forge_hip_config {
     uint32_t flags;         /* FORGE_HIP_FLAG_EXACT, FORGE_HIP_FLAG_QKV_BIAS, both or neither */
     uint32_t sliding_window; /* ModelConfig::sliding_window_size (ir.rs:512), 0 = None: a position attends to itself and the
                               * sliding_window - 1 positions before it (attention_sliding, emit.rs:598-627; attention_sliding_batch,
-                              * emit.rs:907-1046; Mistral).  Not available together with FORGE_HIP_FLAG_EXACT. */
+                              * emit.rs:907-1046; Mistral).  With FORGE_HIP_FLAG_EXACT min(sliding_window, max_seq) must be <= 12288. */
 } forge_hip_config;
 
 typedef struct forge_hip_model forge_hip_model;
@@ -196,16 +196,16 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
                                     uint32_t head_dim, uint32_t flags, void* stream);
 
 /* attention_sliding_batch (emit.rs:907-1046) over an fp16 cache: as forge_hip_attn_prefill_f16kv, but the query at
- * position p = base_pos + row sees only the keys [max(0, p - window + 1), p]; window >= 1.  Fast arithmetic only. */
+ * position p = base_pos + row sees only the keys [max(0, p - window + 1), p]; window >= 1. */
 int32_t forge_hip_attn_prefill_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                              float* out_dev, uint32_t M, uint32_t base_pos, uint32_t window, uint32_t heads,
-                                             uint32_t kv_heads, uint32_t head_dim, void* stream);
+                                             uint32_t kv_heads, uint32_t head_dim, uint32_t flags, void* stream);
 
 /* attention_sliding (emit.rs:598-627) over an fp16 cache: one query against the last min(window, seq_len) of seq_len
- * cached rows; window >= 1.  Fast arithmetic only. */
+ * cached rows; window >= 1.  With FORGE_HIP_FLAG_EXACT at most 12288 rows (their scores stay in LDS). */
 int32_t forge_hip_attn_decode_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                             float* out_dev, uint32_t seq_len, uint32_t window, uint32_t heads,
-                                            uint32_t kv_heads, uint32_t head_dim, void* stream);
+                                            uint32_t kv_heads, uint32_t head_dim, uint32_t flags, void* stream);
 
 /* argmax (project.rs:501-503): index of the LAST maximum of n floats -> *out_dev (uint32). */
 int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void* stream);

@@ -349,14 +349,13 @@ def test_config_defaults_and_refusals(fh, gg, go):
     kq = (("blk.0.attn_q.weight", [256, 64], gg.Q5_K, None), ("output.weight", [256, 64], gg.Q6_K, None))
     ck = gg.GgufFile(make(base, kq)).config()
     assert (ck["wdtype"], ck["lm_head_dtype"]) == (Q8, Q8) and ck == go.config(go.parse(make(base, kq)))
-    # the window travels into the config (main.rs:764-767); exact mode has no sliding attention
+    # the window travels into the config (main.rs:764-767)
     for w in (1024, 4096):
         blob_w = make(base + [("llama.attention.sliding_window", gg.U32, w)])
         win = gg.GgufFile(blob_w)
         cw = win.config()
         assert cw["sliding_window"] == w and cw["max_seq"] == 2048 and cw == go.config(go.parse(blob_w))
-        with pytest.raises(fh.ForgeHipError, match="sliding window"):
-            win.config(flags=fh.FLAG_EXACT)
+        assert win.config(flags=fh.FLAG_EXACT)["flags"] == fh.FLAG_EXACT
     assert c["sliding_window"] == 0
     refused(base + [("llama.attention.sliding_window", gg.U32, 0)], text="sliding window of 0")
     # the vote: 2 x Q4_0 against 1 x Q8_0

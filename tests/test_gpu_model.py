@@ -429,7 +429,7 @@ def test_sliding_window_model_matches_oracle(fh, oracle, torch_gpu, wd, window, 
     """A Mistral-style model (sliding_window_size: attention_sliding in decode, attention_sliding_batch in prefill,
     emit.rs:4156-4170 and 5312-5340): prompt and decode both run past the window; logits within tolerance of the CPU
     oracle with identical greedy tokens on these seeds, resident kernel and kernel sequence alike; prefill in two chunks
-    (the second starts beyond the window) equals one; and the window matters."""
+    (the second starts beyond the window) equals one; the window matters; and the exact mode gives the oracle's bits."""
     cfg = tiny_cfg(fh, wd, 0)
     cfg["sliding_window"] = window
     blob = fh.synth.make_weights_blob(cfg, seed=61 + window)
@@ -476,8 +476,20 @@ def test_sliding_window_model_matches_oracle(fh, oracle, torch_gpu, wd, window, 
     gm = fh.HipModel(dict(cfg, sliding_window=0), blob)
     assert not np.allclose(gm.forward_prefill(prompt), olog, rtol=2e-2, atol=2e-2)
     gm.close()
-    with pytest.raises(fh.ForgeHipError, match="sliding window"):
-        fh.HipModel(dict(cfg, flags=EXACT), blob)
+    # exact mode: attention_sliding_batch and attention_sliding in the reference's order of operations, bit for bit
+    for fuse in ("1", "0"):
+        monkeypatch.setenv("FORGE_HIP_FUSE", fuse)
+        gm = fh.HipModel(dict(cfg, flags=EXACT), blob)
+        assert np.array_equal(gm.forward_prefill(prompt).view(np.uint32), olog.view(np.uint32))
+        tok = oracle.argmax(olog)
+        for i in range(12):
+            gl = gm.forward(tok)
+            assert np.array_equal(gl.view(np.uint32), ologits[i].view(np.uint32)), (fuse, i)
+            tok = oracle.argmax(gl)
+        gm.close()
+    monkeypatch.delenv("FORGE_HIP_FUSE")
+    with pytest.raises(fh.ForgeHipError, match="12288"):
+        fh.HipModel(dict(cfg, flags=EXACT, sliding_window=20000, max_seq=16384), blob)
 
 
 def test_sliding_window_model_from_gguf(fh, oracle, torch_gpu, tmp_path):

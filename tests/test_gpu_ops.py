@@ -219,6 +219,7 @@ def test_attention_sliding_decode_parity(fh, oracle, torch_gpu, heads, kv_heads,
     qd, kd, vd = torch.from_numpy(q).cuda(), _dev16(torch, k16), _dev16(torch, v16)
     got = fh.ops.attention_sliding(qd, kd, vd, seq, window, heads, kv_heads, hd).cpu().numpy()
     close(got, want)
+    same_bits(fh.ops.attention_sliding(qd, kd, vd, seq, window, heads, kv_heads, hd, EXACT).cpu().numpy(), want)
     if window >= seq:       # then it is the plain decode attention, bit for bit
         same_bits(got, fh.ops.attention_flash(qd, kd, vd, seq, heads, kv_heads, hd, 0).cpu().numpy())
     else:                   # rows before the window do not count: poison them
@@ -241,6 +242,7 @@ def test_attention_sliding_prefill_parity(fh, oracle, torch_gpu, heads, kv_heads
     qd, kd, vd = torch.from_numpy(q).cuda(), _dev16(torch, k16), _dev16(torch, v16)
     got = fh.ops.attention_sliding_batch(qd, kd, vd, base, window, heads, kv_heads, hd).cpu().numpy()
     close(got, want)
+    same_bits(fh.ops.attention_sliding_batch(qd, kd, vd, base, window, heads, kv_heads, hd, EXACT).cpu().numpy(), want)
     if window >= seq:       # every key of the call is inside every window: the causal kernel, bit for bit
         same_bits(got, fh.ops.attention_flash_batch(qd, kd, vd, base, heads, kv_heads, hd, 0).cpu().numpy())
     else:                   # rows before the first query's window are never read, and no query may see a row before its own
