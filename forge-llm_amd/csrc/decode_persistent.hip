@@ -611,11 +611,23 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
             }
         }
 
-        for (uint32_t g = dual ? 0u : cx.wave >> 2; g < gt; g += PD_WAVES / 4) {
-            float qf[8], acc[8], m = -INFINITY, l = 0.f;
+        // A wave carries the heads gA and gA + 2 of the group (those that exist) through ONE walk over its keys: each K/V
+        // block is fetched once and used for both, every head's own sequence of operations is what a walk of its own gives.
+        {
+            const uint32_t gA = dual ? 0u : cx.wave >> 2;
+            constexpr int NH = PD_WAVES / 4 == 2 ? 2 : 1;
+            static_assert(PD_WAVES == 8, "two head slots per wave cover groups of up to four heads");
+            bool has[NH];
+            float qf[NH][8], acc[NH][8], m[NH], l[NH];
 #pragma unroll
-            for (int i = 0; i < 8; i++) { acc[i] = 0.f; qf[i] = dvalid ? q_lds[g * HD + c * 8 + i] : 0.f; }
-            for (uint32_t tb0 = tbw; tb0 < t1; tb0 += UNR * 4 * KPW) {
+            for (int hh = 0; hh < NH; hh++) {
+                const uint32_t g = gA + 2 * hh;
+                has[hh] = g < gt;
+                m[hh] = -INFINITY; l[hh] = 0.f;
+#pragma unroll
+                for (int i = 0; i < 8; i++) { acc[hh][i] = 0.f; qf[hh][i] = (dvalid && has[hh]) ? q_lds[g * HD + c * 8 + i] : 0.f; }
+            }
+            for (uint32_t tb0 = tbw; tb0 < t1 && has[0]; tb0 += UNR * 4 * KPW) {
                 Half8 kr[UNR], vr[UNR];
 #pragma unroll
                 for (int u = 0; u < UNR; u++) {
@@ -647,38 +659,46 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
                         float kf[8], vf[8];
                         unpack8(kr[u], kf);
                         unpack8(vr[u], vf);
-                        float d = 0.f;
 #pragma unroll
-                        for (int i = 0; i < 8; i++) d = fmaf(qf[i], kf[i], d);
+                        for (int hh = 0; hh < NH; hh++) {
+                            if (!has[hh]) continue;
+                            float d = 0.f;
 #pragma unroll
-                        for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, WAVE);
-                        if (valid) {
-                            const float sc = d * scale;
-                            const float mn = fmaxf(m, sc);
-                            const float alpha = __expf(m - mn);   // m = -inf on the first key: exp(-inf) = 0
-                            const float p = __expf(sc - mn);
-                            l = fmaf(l, alpha, p);
+                            for (int i = 0; i < 8; i++) d = fmaf(qf[hh][i], kf[i], d);
 #pragma unroll
-                            for (int i = 0; i < 8; i++) acc[i] = fmaf(acc[i], alpha, p * vf[i]);
-                            m = mn;
+                            for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, WAVE);
+                            if (valid) {
+                                const float sc = d * scale;
+                                const float mn = fmaxf(m[hh], sc);
+                                const float alpha = __expf(m[hh] - mn);   // m = -inf on the first key: exp(-inf) = 0
+                                const float p = __expf(sc - mn);
+                                l[hh] = fmaf(l[hh], alpha, p);
+#pragma unroll
+                                for (int i = 0; i < 8; i++) acc[hh][i] = fmaf(acc[hh][i], alpha, p * vf[i]);
+                                m[hh] = mn;
+                            }
                         }
                     }
                 }
             }
-            // merge the key slots of the wave
 #pragma unroll
-            for (int o = LPK; o < 64; o <<= 1) {
-                float m2 = __shfl_xor(m, o, WAVE), l2 = __shfl_xor(l, o, WAVE);
-                float a2[8];
+            for (int hh = 0; hh < NH; hh++) {
+                if (!has[hh]) continue;
+                // merge the key slots of the wave
 #pragma unroll
-                for (int i = 0; i < 8; i++) a2[i] = __shfl_xor(acc[i], o, WAVE);
-                merge_state<8>(m, l, acc, m2, l2, a2);
-            }
-            if (slot == 0 && dvalid) {
-                float* rec = sh + (wave * 4 + g) * REC;
+                for (int o = LPK; o < 64; o <<= 1) {
+                    float m2 = __shfl_xor(m[hh], o, WAVE), l2 = __shfl_xor(l[hh], o, WAVE);
+                    float a2[8];
 #pragma unroll
-                for (int i = 0; i < 8; i++) rec[c * 8 + i] = acc[i];
-                if (c == 0) { rec[HD] = m; rec[HD + 1] = l; }
+                    for (int i = 0; i < 8; i++) a2[i] = __shfl_xor(acc[hh][i], o, WAVE);
+                    merge_state<8>(m[hh], l[hh], acc[hh], m2, l2, a2);
+                }
+                if (slot == 0 && dvalid) {
+                    float* rec = sh + (wave * 4 + gA + 2 * hh) * REC;
+#pragma unroll
+                    for (int i = 0; i < 8; i++) rec[c * 8 + i] = acc[hh][i];
+                    if (c == 0) { rec[HD] = m[hh]; rec[HD + 1] = l[hh]; }
+                }
             }
         }
         __syncthreads();
