@@ -97,7 +97,8 @@ def decode_profile(fh, model, cfg, tok, context, prof_steps=8):
     gemv_bytes_total = sum(gbytes.values())
     per_stage = {s: {"GB/s": round(gbytes[s] / (stage_ms[s] * 1e-3) / 1e9, 1), "us_per_token": round(stage_ms[s] * 1e3, 1)} for s in gbytes}
     stage_us = {s: round(v * 1e3, 1) for s, v in stage_ms.items() if v > 0}
-    if model.decode_launches == 1:
+    n_launch = model.decode_launches
+    if n_launch <= (cfg["layers"] + 33) // 34:
         # one resident kernel per token: its phases are the stages, timed by the kernel's own clock stamps
         rows = min(context, cfg.get("sliding_window", 0) or context)          # a sliding window bounds the rows a step reads
         kv_bytes = cfg["layers"] * 2 * rows * cfg["kv_heads"] * cfg["head_dim"] * 2
@@ -106,8 +107,8 @@ def decode_profile(fh, model, cfg, tok, context, prof_steps=8):
         achieved = total / (kernel_ms * 1e-3) / 1e9
         roof = {"kernel": "decode_step_kernel (the whole decode step: every quantised GEMV, decode attention, norms, argmax)",
                 "bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-                "traffic": STEP_KERNEL_HBM_BYTES_PER_LAUNCH, "bytes_per_launch": total, "us_per_launch": kernel_ms * 1e3,
-                "launches_per_step": 1, "weights_and_vectors_bytes": gemv_bytes_total, "kv_cache_bytes": kv_bytes,
+                "traffic": STEP_KERNEL_HBM_BYTES_PER_LAUNCH, "bytes_per_launch": total / n_launch, "us_per_launch": kernel_ms * 1e3 / n_launch,
+                "launches_per_step": n_launch, "weights_and_vectors_bytes": gemv_bytes_total, "kv_cache_bytes": kv_bytes,
                 "per_phase": per_stage}
     else:
         gemv_ms = sum(stage_ms[s] for s in gbytes)
@@ -218,7 +219,7 @@ def main():
     ap.add_argument("--no-alt", action="store_true", help="skip the second model that measures the kernel-sequence decode step")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (known HBM traffic, for scaling counter readings)")
-    ap.add_argument("--model", choices=("llama32_1b", "llama32_3b", "smollm2_135m", "llama31_8b", "qwen25_1p5b", "mistral_7b", "phi3_mini"), default="llama32_1b",
+    ap.add_argument("--model", choices=("llama32_1b", "llama32_3b", "smollm2_135m", "llama31_8b", "qwen25_1p5b", "mistral_7b", "phi3_mini", "qwen25_14b"), default="llama32_1b",
                     help="shape of the synthetic model (default: the one the headline metric is quoted on)")
     ap.add_argument("--format", choices=("q8_0", "q4_0"), default="q8_0", help="weight format (default: the headline's)")
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
@@ -242,7 +243,7 @@ def main():
     cfg = getattr(fh.synth, args.model)(wd, max_seq=max(4096, (PROMPT_TOKENS + 2 * (args.warmup + args.steps) + 16 + 1023) // 1024 * 1024))
     headline = args.model == "llama32_1b" and args.format == "q8_0" and PROMPT_TOKENS == 2502
     model_name = {"llama32_1b": "Llama-3.2-1B", "llama32_3b": "Llama-3.2-3B", "smollm2_135m": "SmolLM2-135M", "llama31_8b": "Llama-3.1-8B",
-                  "qwen25_1p5b": "Qwen2.5-1.5B", "mistral_7b": "Mistral-7B (sliding window 4096)", "phi3_mini": "Phi-3-mini"}[args.model]
+                  "qwen25_1p5b": "Qwen2.5-1.5B", "mistral_7b": "Mistral-7B (sliding window 4096)", "phi3_mini": "Phi-3-mini", "qwen25_14b": "Qwen2.5-14B"}[args.model]
     t0 = time.perf_counter()
     blob = fh.synth.make_weights_blob(cfg, seed=args.seed, threads=16)
     t_gen = time.perf_counter() - t0
@@ -296,7 +297,9 @@ def main():
     model.reset()
     tok2 = fh.ops.argmax_host(model.forward_prefill(prompt[:32]))
     t_decode_short, _ = timed_decode(model, tok2, 4, args.steps)
-    path = "one resident kernel per token" if model.decode_launches == 1 else f"{model.decode_launches} kernels per token (graph replay)"
+    path = ("one resident kernel per token" if model.decode_launches == 1 else
+            f"{model.decode_launches} launches of the resident kernel per token (34 layers each)"
+            if model.decode_launches <= (cfg["layers"] + 33) // 34 else f"{model.decode_launches} kernels per token (graph replay)")
 
     # ---- the reference's default loop: greedy with repeat penalty 1.1 over every token fed (project.rs:607-611, 742-744)
     model.reset()

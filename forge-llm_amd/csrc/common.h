@@ -182,6 +182,7 @@ struct PdLayerIn {
 };
 struct PdState;
 // Leaves *out null (returning OK) when the shape or device is not covered; `state` = {position, token, next token, abort flag}.
+uint32_t pd_launches_per_step(const PdState* st);
 int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layers, const QWeight& lm_head, const float* embed,
                   const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, uint32_t* counts,
                   const float* qkv_bias, PdState** out);

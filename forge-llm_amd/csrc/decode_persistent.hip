@@ -86,12 +86,17 @@ struct PdLayer {
     uint16_t* kc;
     uint16_t* vc;
 };
-constexpr uint32_t PD_MAX_LAYERS = 34;       // the descriptors travel as kernel arguments (4 KB in all)
+constexpr uint32_t PD_MAX_LAYERS = 34;       // per launch: the descriptors travel as kernel arguments (4 KB in all)
+constexpr uint32_t PD_MAX_SEGMENTS = 8;
 enum { PD_QKV = 0, PD_O = 1, PD_GU = 2, PD_DOWN = 3, PD_LM = 4 };
 
 struct PdArgs {
     PdGemv shape[5];           // qkv, o, gate_up, down (addresses per layer, below) and lm_head (addresses here)
-    uint32_t n_layers, H, I, QKS, KV, heads, kv_heads, gt;
+    uint32_t n_layers, H, I, QKS, KV, heads, kv_heads, gt;   // n_layers: the layers of THIS launch, layers[0 .. n_layers)
+    // A model of more layers than the descriptor array holds runs its step as several launches in a row: layers
+    // [layer0, layer0 + n_layers) of total_layers; the first launch starts from the embedding row, the last one ends with
+    // the lm_head and the argmax.  Tags and exchange buffers carry over from launch to launch unchanged.
+    uint32_t layer0, total_layers, seg_last;
     float eps;
     const float* embed;
     const float* final_norm;
@@ -988,23 +993,25 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
 
     // steps 4 l + {0: qkv, 1: attention then o, 2: gate/up, 3: down}; step 4 L: lm_head.  Phase instance k of this
     // launch carries tag tag_base + k: per layer 1 qkv, 2 attention split, 3 attention merge, 4 o, 5 gate/up, 6 down.
+    const uint32_t n_steps = 4 * L + (a.seg_last ? 1u : 0u);
 #pragma nounroll
-    for (uint32_t step = 0; step <= 4 * L; step++) {
+    for (uint32_t step = 0; step < n_steps; step++) {
         const bool is_lm = step == 4 * L;
-        const uint32_t l = is_lm ? L - 1 : step >> 2, ph = is_lm ? 4u : (step & 3u);
-        const uint32_t base = a.tag_base + 6 * l;
-        const uint32_t x_in = l ? base : 0;                  // tag of x entering layer l (0: still the embedding row)
+        const uint32_t l = is_lm ? L - 1 : step >> 2, ph = is_lm ? 4u : (step & 3u);     // l: index into a.layers
+        const uint32_t lg = a.layer0 + l;                     // the layer's number in the model
+        const uint32_t base = a.tag_base + 6 * lg;
+        const uint32_t x_in = lg ? base : 0;                 // tag of x entering the layer (0: still the embedding row)
         if (ph == 1) {
-            if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * l + 1] = wall_clock64();
+            if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * lg + 1] = wall_clock64();
             pd_attn_split<HD>(a, a.layers[l].kc, a.layers[l].vc, pos, base + 1, base + 2, big, cx);
             if (sh_abort) return;
-            if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * l + 2] = wall_clock64();
+            if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * lg + 2] = wall_clock64();
             pd_attn_combine<HD>(a, base + 2, base + 3, misc, big, cx);
             if (sh_abort) return;
         }
         if (a.stamps && cx.wg == 0 && cx.tid == 0) {
             static const int slot[5] = {0, 3, 4, 5, 6};
-            a.stamps[6 * l + slot[ph]] = wall_clock64();
+            a.stamps[6 * lg + slot[ph]] = wall_clock64();
         }
         GemvJob job;
         job.which = ph;
@@ -1017,7 +1024,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
             const bool n_lm = ns == 4 * L;
             const uint32_t nl = n_lm ? L - 1 : ns >> 2, nph = n_lm ? 4u : (ns & 3u);
             // the O projection follows attention, which needs every wave at once: its (few) weights are loaded when it starts
-            next.valid = ns <= 4 * L && nph != 1;
+            next.valid = ns < n_steps && nph != 1;
             next.which = nph;
             next.qs = n_lm ? a.shape[PD_LM].qs : a.layers[next.valid ? nl : 0].qs[nph & 3u];
             next.ws = n_lm ? a.shape[PD_LM].ws : a.layers[next.valid ? nl : 0].ws[nph & 3u];
@@ -1032,7 +1039,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         job.tag_out = is_lm ? 0 : base + (ph == 0 ? 1u : ph == 1 ? 4u : ph == 2 ? 5u : 6u);
         job.res_tag = ph == 1 ? x_in : base + 4;
         job.kc = a.layers[l].kc;
-        job.bias = (PEN && a.qkv_bias && ph == 0) ? a.qkv_bias + (size_t)l * (a.QKS + 2 * a.KV) : nullptr;
+        job.bias = (PEN && a.qkv_bias && ph == 0) ? a.qkv_bias + (size_t)lg * (a.QKS + 2 * a.KV) : nullptr;
         job.vc = a.layers[l].vc;
         if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
         else pd_gemv_phase<false, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
@@ -1040,14 +1047,15 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         if (sh_abort) return;
     }
 
+    if (!a.seg_last) return;          // the next launch goes on from the exchange buffers
     // ---------------- argmax (and the position / token advance) ----------------
-    const uint32_t th = a.tag_base + 6 * L + 1;
+    const uint32_t th = a.tag_base + 6 * a.total_layers + 1;
     best = arg_wg(best, misc, cx);
     if (cx.tid == 0) {
         stc64(a.tpart + 2 * cx.wg, th, __float_as_uint(best.v));
         stc64(a.tpart + 2 * cx.wg + 1, th, best.i);
     }
-    if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * L + 1] = wall_clock64();
+    if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * a.total_layers + 1] = wall_clock64();
     if (cx.wg == 0) {
         ArgPair p{-INFINITY, 0};
         for (uint32_t w = cx.tid; w < cx.G; w += PD_THREADS) {
@@ -1062,7 +1070,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
             a.state[1] = p.i;
             a.state[0] = pos + 1;
             if (!PEN) a.counts[token] += 1;          // nobody read the counters in this launch
-            if (a.stamps) a.stamps[6 * L + 2] = wall_clock64();
+            if (a.stamps) a.stamps[6 * a.total_layers + 2] = wall_clock64();
             // the host may be spinning on this word instead of waiting for the stream
             if (a.host_out)
                 __hip_atomic_store(a.host_out, ((unsigned long long)a.host_seq << 32) | p.i, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -1090,6 +1098,7 @@ struct PdState {
     size_t tagged_bytes = 0;
     void* tagged_base = nullptr;
     std::vector<unsigned long long> stamps_host;
+    std::vector<PdLayer> all_layers;           // every layer's descriptors; a launch takes a slice of at most PD_MAX_LAYERS
     int wall_khz = 0;
     unsigned long long* host_out = nullptr;    // pinned, mapped into the device's address space
     unsigned long long* host_out_dev = nullptr;
@@ -1158,6 +1167,9 @@ const void* pd_kernel_for(const PdState* st) {
 
 void pd_destroy(PdState* st) { delete st; }
 
+// Kernel launches of one decode step: 1, or one per slice of PD_MAX_LAYERS layers for a deeper model.
+uint32_t pd_launches_per_step(const PdState* st) { return (st->args.total_layers + PD_MAX_LAYERS - 1) / PD_MAX_LAYERS; }
+
 // Plans the persistent decode step for a model.  Leaves *out null (and returns OK) when the shape or the
 // device is outside what the kernel covers; the caller then keeps the multi-kernel step.
 int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layers, const QWeight& lm_head, const float* embed,
@@ -1198,7 +1210,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     if ((H + 32) * 4 > big || attn_bytes > big || DECODE_SPLITS * (hd + 2) * 4 > big) return FORGE_HIP_OK;
     st->lds = a.off_big + big;
 
-    if (layers.empty() || layers.size() > PD_MAX_LAYERS) return FORGE_HIP_OK;
+    if (layers.empty() || layers.size() > PD_MAX_LAYERS * PD_MAX_SEGMENTS) return FORGE_HIP_OK;
     {
         const PdLayerIn& in = layers[0];
         const uint32_t wt = c.wdtype;
@@ -1214,7 +1226,8 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     }
     for (size_t l = 0; l < layers.size(); l++) {
         const PdLayerIn& in = layers[l];
-        PdLayer& L = a.layers[l];
+        st->all_layers.emplace_back();
+        PdLayer& L = st->all_layers.back();
         const QWeight* w[4] = {in.qkv, in.o, in.gate_up, in.down};
         for (int k = 0; k < 4; k++) { L.qs[k] = w[k]->qs; L.ws[k] = w[k]->scales; }
         L.attn_norm = in.attn_norm; L.ffn_norm = in.ffn_norm; L.kc = in.kc; L.vc = in.vc;
@@ -1231,7 +1244,11 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
         if (e != hipSuccess || per_cu < 1) { (void)hipGetLastError(); return FORGE_HIP_OK; }
     }
 
-    a.n_layers = (uint32_t)layers.size();
+    a.total_layers = (uint32_t)layers.size();
+    a.layer0 = 0;
+    a.n_layers = std::min<uint32_t>(a.total_layers, PD_MAX_LAYERS);
+    a.seg_last = a.n_layers == a.total_layers;
+    for (uint32_t l = 0; l < a.n_layers; l++) a.layers[l] = st->all_layers[l];
     a.H = H; a.I = I; a.QKS = QKS; a.KV = KV; a.heads = c.heads; a.kv_heads = c.kv_heads;
     a.eps = c.rms_eps;
     a.window = c.sliding_window;
@@ -1283,8 +1300,8 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
             (void)hipGetLastError();
         }
     }
-    st->tags_per_launch = 6 * a.n_layers + 1;
-    st->n_stamps = 6 * a.n_layers + 3;
+    st->tags_per_launch = 6 * a.total_layers + 1;
+    st->n_stamps = 6 * a.total_layers + 3;
     a.stamps = nullptr;
     *out = st.release();
     return FORGE_HIP_OK;
@@ -1322,7 +1339,16 @@ int32_t pd_enqueue(PdState* st, bool profile, uint32_t token, hipStream_t s) {
     }
     unsigned long long* keep = a.stamps;
     if (!profile) a.stamps = nullptr;
-    const hipError_t e = st->hd == 64 ? launch_pd_hd<64>(st, s) : st->hd == 96 ? launch_pd_hd<96>(st, s) : launch_pd_hd<128>(st, s);
+    hipError_t e = hipSuccess;
+    for (uint32_t l0 = 0; l0 < a.total_layers && e == hipSuccess; l0 += PD_MAX_LAYERS) {
+        if (a.total_layers > PD_MAX_LAYERS) {       // one launch per slice of layers (the arguments are copied at launch)
+            a.layer0 = l0;
+            a.n_layers = std::min<uint32_t>(PD_MAX_LAYERS, a.total_layers - l0);
+            a.seg_last = l0 + a.n_layers == a.total_layers;
+            for (uint32_t l = 0; l < a.n_layers; l++) a.layers[l] = st->all_layers[l0 + l];
+        }
+        e = st->hd == 64 ? launch_pd_hd<64>(st, s) : st->hd == 96 ? launch_pd_hd<96>(st, s) : launch_pd_hd<128>(st, s);
+    }
     a.stamps = keep;
     if (e != hipSuccess) return fail(FORGE_HIP_ERR_HIP, std::string("persistent decode launch: ") + hipGetErrorString(e));
     a.tag_base += st->tags_per_launch;

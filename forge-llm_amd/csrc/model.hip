@@ -593,7 +593,7 @@ int32_t forge_hip_prefill_profile(forge_hip_model* m, const uint32_t* tokens, ui
 
 int32_t forge_hip_model_decode_launches(const forge_hip_model* m) {
     if (!m) return -1;
-    if (m->pd) return 1;
+    if (m->pd) return (int32_t)pd_launches_per_step(m->pd);
     const bool exact = (m->cfg.flags & FORGE_HIP_FLAG_EXACT) != 0;
     const int attn = exact ? 1 : 2;
     const int layer = (m->fuse_norm ? 1 : 3) + attn + 1 + (m->fuse_silu ? 1 : 3) + 1;

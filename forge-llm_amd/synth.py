@@ -89,6 +89,15 @@ def phi3_mini(wdtype=8, max_seq=4096):
     return _cfg(3072, 8192, 32, 32, 32, 96, 32064, max_seq, 10000.0, wdtype)
 
 
+def qwen25_14b(wdtype=8, max_seq=4096):
+    """Qwen2.5-14B shape: 48 layers (more than one launch of the resident decode kernel carries), QKV bias, 40 heads over
+    8 KV heads, head_dim 128, vocabulary 152 064."""
+    c = _cfg(5120, 13824, 48, 40, 8, 128, 152064, max_seq, 1000000.0, wdtype)
+    c["flags"] = 2
+    c["rms_eps"] = 1e-6
+    return c
+
+
 def mistral_7b(wdtype=8, max_seq=8192):
     """Mistral-7B-v0.1 shape: the Llama layer with a sliding window of 4096 positions, vocabulary 32 000."""
     c = _cfg(4096, 14336, 32, 32, 8, 128, 32000, max_seq, 10000.0, wdtype)

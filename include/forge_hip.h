@@ -115,7 +115,7 @@ int32_t forge_hip_prefill_profile(forge_hip_model* m, const uint32_t* tokens_hos
                                   uint32_t* stage_launches_host);
 
 /* Kernel launches one decode step costs on this model: 1 when the whole step runs as one resident kernel
- * (fast mode, covered shapes), otherwise the length of the kernel sequence.  The Metal backend's counterpart
+ * (fast mode, covered shapes; one launch per 34 layers for a deeper model), otherwise the length of the kernel sequence.  The Metal backend's counterpart
  * is the fixed encoder sequence of MetalModel::forward (metal:5070-5300). */
 int32_t forge_hip_model_decode_launches(const forge_hip_model* m);
 

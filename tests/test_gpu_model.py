@@ -234,6 +234,39 @@ def test_persistent_decode_kernel_equals_kernel_sequence(fh, torch_gpu, monkeypa
     seq.close(); one.close()
 
 
+@pytest.mark.parametrize("layers", [35, 70])
+def test_persistent_decode_kernel_deep_models(fh, torch_gpu, monkeypatch, layers):
+    """A model of more than 34 layers runs its step as one launch per slice of 34 layers (the layer descriptors of a launch
+    travel as kernel arguments); tags and exchange buffers carry over between the launches, so the bits are those of the
+    kernel sequence: logits from an empty cache and after a prefill, greedy tokens, the last layer's cache."""
+    cfg = fh.synth.tiny(Q8, max_seq=640, hidden=128, inter=256, layers=layers, heads=2, kv_heads=1, head_dim=64, vocab=500)
+    blob = fh.synth.make_weights_blob(cfg, seed=91)
+    toks = fh.synth.uniform_ids(92, 60, cfg["vocab"])
+    monkeypatch.setenv("FORGE_HIP_PERSIST", "0")
+    seq = fh.HipModel(cfg, blob)
+    monkeypatch.setenv("FORGE_HIP_PERSIST", "1")
+    monkeypatch.setenv("FORGE_HIP_PD_ORDERED", "1")
+    one = fh.HipModel(cfg, blob)
+    assert one.decode_launches == (layers + 33) // 34 and seq.decode_launches > layers
+    for t in toks[:6]:
+        same_bits(one.forward(int(t)), seq.forward(int(t)))
+    seq.reset(); one.reset()
+    same_bits(one.forward_prefill(toks[:40]), seq.forward_prefill(toks[:40]))
+    a = b = int(toks[40])
+    for _ in range(10):
+        a, b = one.forward_greedy(a), seq.forward_greedy(b)
+        assert a == b
+    same_bits(one.forward(7), seq.forward(7))
+    assert np.array_equal(one.read_kv(layers - 1, 0), seq.read_kv(layers - 1, 0))
+    prof = one.forward_profile(a)
+    assert prof["qkv_matmul"][1] == layers and prof["lm_head_matmul"][0] > 0
+    one.set_repeat_penalty(1.1); seq.set_repeat_penalty(1.1)          # the variant with the optional extras, same slices
+    for _ in range(4):
+        a, b = one.forward_greedy(a), seq.forward_greedy(b)
+        assert a == b
+    seq.close(); one.close()
+
+
 def test_persistent_decode_kernel_rewinds_its_tags(fh, torch_gpu, monkeypatch):
     """The hand-over tags count up from launch to launch and are rewound (buffers cleared) before they could wrap:
     started just below that point, the one-kernel model goes through the rewind within a few steps and keeps giving
