@@ -298,10 +298,16 @@ inline bool row_is_dot1(int64_t row, int64_t n, int64_t chunk, int tail_mod) {
     return i >= len - (len % tail_mod);
 }
 
+// The switch to 256-row chunks compares N * ceil(K/32) * 34 with one megabyte for Q8_0 (emit.rs:1971) and, with the
+// same 34-byte figure, for Q4_0 (emit.rs:2837); the lm_head loops are always chunked (emit.rs:4304, 5452).
+inline bool matmul_vec_is_chunked(int64_t k, int64_t n, int lm_head_mode) {
+    return lm_head_mode != 0 || n * ((k + QK - 1) / QK * Q8_BYTES) >= 1000000;
+}
+
 void matmul_vec(int wdtype, int variant, float* out, const float* in, const uint8_t* w,
                 int64_t k, int64_t n, int lm_head_mode /*0 vec,1 forward lm,2 prefill lm*/) {
     int64_t row_bytes = (k + QK - 1) / QK * wbytes(wdtype);
-    bool par = lm_head_mode != 0 || n * ((k + QK - 1) / QK * wbytes(wdtype)) >= 1000000;
+    bool par = matmul_vec_is_chunked(k, n, lm_head_mode);
     int64_t chunk = par ? 256 : 0;
     int tail_mod = lm_head_mode == 2 ? 8 : 4;
     if (variant == 0) {
@@ -931,6 +937,16 @@ void fo_rope_table(int64_t n_pos, int head_dim, float theta, float* cos_out, flo
 }
 float fo_quantize_kv(const float* v, int64_t n, int8_t* out) { return quantize_kv(v, n, out); }
 uint32_t fo_argmax(const float* v, int64_t n) { return argmax_last(v, n); }
+// Which output rows add their block products in the 4-accumulator (dot1) order: out[r] = 1 for those rows.
+// mode: 0 matmul_vec, 1 lm_head of forward, 2 lm_head of forward_prefill_batched, 3 matmul_mat.  wdtype does not enter
+// the rule (both formats compare 34-byte blocks with the threshold); it is an argument so that callers state the format.
+void fo_row_order(int wdtype, int64_t k, int64_t n, int mode, uint8_t* out) {
+    (void)wdtype;
+    for (int64_t r = 0; r < n; r++) {
+        if (mode == 3) out[r] = row_is_dot1(r, n, 0, 4);
+        else out[r] = row_is_dot1(r, n, matmul_vec_is_chunked(k, n, mode) ? 256 : 0, mode == 2 ? 8 : 4);
+    }
+}
 // The C library's expf (what Rust's f32::exp calls on Linux), element-wise.
 void fo_expf_array(const float* x, int64_t n, float* out) { for (int64_t i = 0; i < n; i++) out[i] = expf(x[i]); }
 

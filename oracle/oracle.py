@@ -81,6 +81,7 @@ def lib():
     L.fo_argmax.restype = C.c_uint32
     L.fo_argmax.argtypes = [vp, i64]
     L.fo_attention.argtypes = [i32, i32, vp, vp, vp, vp, vp, vp, i64, i64, i32, i32, i32, i64]
+    L.fo_row_order.argtypes = [i32, i64, i64, i32, vp]
     L.fo_num_threads.restype = i32
     L.fo_set_num_threads.argtypes = [i32]
     _lib = L
@@ -225,6 +226,13 @@ def expf(x):
 def argmax(v):
     v = _f32(v)
     return int(lib().fo_argmax(_p(v), v.size))
+
+
+def row_order(wdtype, k, n, mode):
+    """Output rows of a variant-A matmul that take the 4-accumulator order; mode: 'vec' | 'lm_forward' | 'lm_prefill' | 'mat'."""
+    out = np.empty(n, np.uint8)
+    lib().fo_row_order(wdtype, k, n, {"vec": 0, "lm_forward": 1, "lm_prefill": 2, "mat": 3}[mode], _p(out))
+    return [int(i) for i in np.flatnonzero(out)]
 
 
 def attention(kind, q, k, v, seq_or_m, nh, nkv, hd, base_pos=0, ks=None, vs=None, window=0):
