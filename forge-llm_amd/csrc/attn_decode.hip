@@ -5,6 +5,8 @@
 // lanes of a wave cover 64/LPK keys per load and every key slot keeps its own online-softmax
 // state, so the loop needs no cross-slot traffic; slots, waves and splits are merged at
 // the end with the usual (max, sum, acc) rescaling.
+#include <mutex>
+
 #include "common.h"
 #include "device_utils.h"
 
@@ -217,3 +219,56 @@ void launch_attn_decode(const float* q, const uint16_t* kc, const uint16_t* vc, 
 }
 
 }  // namespace fh
+
+// ---- decode attention for callers that cannot allocate ----------------------------------------------------------
+// The split records of the two kernels above normally live in a lazily grown allocation of the op-level API.  Code
+// under HIP graph capture, tight serving loops and harnesses that forbid allocation get the same kernels over a
+// fixed array in the library's own device image instead.  Each GPU holds its own copy of the array (until the
+// process ends) at its own address, which the host learns once per device with hipGetSymbolAddress: the array's
+// name in host code is only a handle for that query, never a device address.
+namespace {
+constexpr uint32_t NOALLOC_MAX_HEADS = 128, NOALLOC_MAX_HEAD_DIM = 128;
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)NOALLOC_MAX_HEADS * fh::DECODE_SPLITS * (NOALLOC_MAX_HEAD_DIM + 2) * sizeof(float);
+constexpr int NOALLOC_MAX_DEVICES = 64;
+
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[NOALLOC_MAX_DEVICES] = {};
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int32_t scratch_on_current_device(void** out) {
+    int dev = -1;
+    FH_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= NOALLOC_MAX_DEVICES) return fh::fail(FORGE_HIP_ERR_INVALID, "attn_decode_noalloc: device index out of range");
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        FH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fh::fail(FORGE_HIP_ERR_HIP, "attn_decode_noalloc: hipGetSymbolAddress returned a null address");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return FORGE_HIP_OK;
+}
+}  // namespace
+
+extern "C" int32_t forge_hip_attn_decode_f16kv_noalloc(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
+                                                       float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
+                                                       uint32_t head_dim, void* stream) {
+    FH_CHECK(q_dev && k_cache_dev && v_cache_dev && out_dev, "attn_decode_noalloc: null pointer");
+    FH_CHECK(seq_len >= 1, "attn_decode_noalloc: seq_len must be at least 1");
+    FH_CHECK(fh::attn_head_dim_supported(head_dim), "attn_decode_noalloc: head_dim must be 64, 96 or 128");
+    FH_CHECK(kv_heads != 0 && heads != 0 && heads % kv_heads == 0, "attn_decode_noalloc: heads must be a positive multiple of kv_heads");
+    FH_CHECK(heads <= NOALLOC_MAX_HEADS && fh::attn_decode_workspace_bytes(heads, head_dim) <= NOALLOC_SCRATCH_BYTES,
+             "attn_decode_noalloc: more than 128 query heads do not fit the fixed scratch array");
+    void* ws = nullptr;
+    int32_t rc = scratch_on_current_device(&ws);
+    if (rc) return rc;
+    // every (head, split) record is written by the split kernel before the merge kernel reads it, empty splits
+    // included, so nothing of the previous call's contents has to be cleared
+    fh::launch_attn_decode(q_dev, k_cache_dev, v_cache_dev, out_dev, nullptr, nullptr, seq_len, nullptr, heads, kv_heads, head_dim, 0u,
+                           ws, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}

@@ -235,6 +235,21 @@ def attention_flash(q, k_cache, v_cache, seq_len, heads, kv_heads, head_dim, fla
     return out
 
 
+def attention_flash_noalloc(q, k_cache, v_cache, seq_len, heads, kv_heads, head_dim, out):
+    """attention_flash (fast mode) through the entry point that allocates nothing: the caller brings `out` (f32 [heads*hd],
+    on the device) as well as the inputs, all already of the right type and contiguous."""
+    from . import check, lib
+    torch = _torch()
+    for t, dt in ((q, torch.float32), (out, torch.float32), (k_cache, torch.int16), (v_cache, torch.int16)):
+        if not (t.is_cuda and t.dtype == dt and t.is_contiguous()):
+            raise ValueError("attention_flash_noalloc takes contiguous device tensors (q, out f32; caches int16 bit patterns)")
+    if seq_len > k_cache.shape[0] or out.numel() != q.numel():
+        raise ValueError("cache holds fewer than seq_len rows, or out has another size than q")
+    check(lib().forge_hip_attn_decode_f16kv_noalloc(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), seq_len, heads, kv_heads,
+                                                    head_dim, _stream()))
+    return out
+
+
 def attention_sliding_batch(q, k_cache, v_cache, base_pos, window, heads, kv_heads, head_dim, flags=0):
     """attention_sliding_batch over an fp16 cache: row r (position base_pos + r) sees the last `window` positions up to its own."""
     from . import check, lib

@@ -195,6 +195,16 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
                                     float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
                                     uint32_t head_dim, uint32_t flags, void* stream);
 
+/* forge_hip_attn_decode_f16kv without FORGE_HIP_FLAG_EXACT for callers that cannot allocate: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same kernels, same
+ * results bit for bit; the split records (heads * 32 * (head_dim + 2) floats) go to a fixed 2 129 920-byte array in the
+ * library's device image (one copy per GPU, held until the process ends) instead of the op-level API's lazily grown
+ * allocation, and the call makes no hipMalloc / hipFree.  heads <= 128, else FORGE_HIP_ERR_INVALID.  Every call on a GPU
+ * uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not. */
+int32_t forge_hip_attn_decode_f16kv_noalloc(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
+                                            float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
+                                            uint32_t head_dim, void* stream);
+
 /* attention_sliding_batch (emit.rs:907-1046) over an fp16 cache: as forge_hip_attn_prefill_f16kv, but the query at
  * position p = base_pos + row sees only the keys [max(0, p - window + 1), p]; window >= 1. */
 int32_t forge_hip_attn_prefill_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
