@@ -7,6 +7,10 @@ problem and compares the parts the oracle can do in seconds, using what the oper
     up to its position: sampled rows are checked against the oracle run on exactly those rows;
   * the same rows computed alone on the GPU must equal the rows of the full launch bit for bit
     (tiling, batching and chunking may not change a result)."""
+import hashlib
+import json
+import os
+
 import numpy as np
 import pytest
 
@@ -160,3 +164,80 @@ def test_llama_3b_shape_two_layers_identical_tokens(fh, oracle, torch_gpu):
     for which in (0, 1):
         same_bits(oracle.f16_to_f32(gm.read_kv(1, which)), om.read_kv(1, which))
     gm.close(); om.close()
+
+
+# ---------------- Llama-3.2-3B shape at full size: 28 layers, 2500-token prompt, 128 greedy tokens ----------------
+_FIXTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "config5_llama32_3b_q8.json")
+_full_3b = {}
+
+
+def full_3b(fh):
+    """The model and prompt of tests/golden/config5_llama32_3b_q8.json, regenerated from its seeds (once per session)."""
+    if not _full_3b:
+        with open(_FIXTURE) as f:
+            fx = json.load(f)
+        cfg = fh.synth.llama32_3b(Q8, max_seq=4096)
+        assert {k: cfg[k] for k in cfg} == {k: fx["config"][k] for k in cfg}
+        blob = fh.synth.make_weights_blob(cfg, seed=fx["weight_seed"], threads=16)
+        prompt = fh.synth.uniform_ids(fx["prompt_seed"], fx["prompt_tokens"], cfg["vocab"])
+        assert [int(t) for t in prompt[:8]] == fx["prompt_head"]
+        _full_3b.update(fx=fx, cfg=cfg, blob=blob, prompt=prompt)
+    return _full_3b["fx"], _full_3b["cfg"], _full_3b["blob"], _full_3b["prompt"]
+
+
+def _sha(a):
+    return hashlib.sha256(np.ascontiguousarray(a, np.float32).tobytes()).hexdigest()
+
+
+@pytest.mark.timeout(900)
+def test_llama_3b_full_size_exact_mode_holds_the_oracle_fixture(fh, torch_gpu):
+    """The whole workload -- 28 layers, batched prefill of 2500 tokens, 128 greedy tokens -- in exact mode against what the
+    CPU oracle produced for it (a quarter of an hour on 8 cores, run once by tests/golden/make_config5_fixture.py): identical
+    token ids, and the prefill logits and the logits behind the last token identical in every bit (SHA-256 of the f32 words)."""
+    fx, cfg, blob, prompt = full_3b(fh)
+    gm = fh.HipModel(dict(cfg, flags=EXACT), blob)
+    logits = gm.forward_prefill(prompt)
+    assert [int(i) for i in np.argsort(logits)[-5:][::-1]] == fx["prefill_top5"]
+    assert _sha(logits) == fx["prefill_logits_sha256"]
+    tokens = [fh.ops.argmax_host(logits)]
+    for _ in range(len(fx["tokens"]) - 1):
+        logits = gm.forward(tokens[-1])
+        tokens.append(fh.ops.argmax_host(logits))
+    first_bad = next((i for i, (a, b) in enumerate(zip(tokens, fx["tokens"])) if a != b), None)
+    assert first_bad is None, f"token {first_bad} differs: {tokens[first_bad]} against the oracle's {fx['tokens'][first_bad]}"
+    assert _sha(logits) == fx["last_logits_sha256"]
+    gm.close()
+
+
+@pytest.mark.timeout(900)
+def test_llama_3b_full_size_resident_kernel_equals_kernel_sequence(fh, torch_gpu, monkeypatch):
+    """Fast mode at full depth and context: after the same 2500-token prefill, 128 greedy steps of the one-kernel decode step
+    (summing in the reference order) and of the kernel sequence give the same tokens, the same logits and the same cache,
+    bit for bit; and the default summation of the one-kernel step stays within the fast mode's bound of the sequence over a
+    single step from identical state."""
+    fx, cfg, blob, prompt = full_3b(fh)
+    monkeypatch.setenv("FORGE_HIP_PERSIST", "0")
+    seq = fh.HipModel(cfg, blob)
+    monkeypatch.setenv("FORGE_HIP_PERSIST", "1")
+    monkeypatch.setenv("FORGE_HIP_PD_ORDERED", "1")
+    one = fh.HipModel(cfg, blob)
+    monkeypatch.setenv("FORGE_HIP_PD_ORDERED", "0")
+    fast = fh.HipModel(cfg, blob)
+    assert one.decode_launches == 1 and fast.decode_launches == 1 and seq.decode_launches > 1
+    la = seq.forward_prefill(prompt)
+    same_bits(one.forward_prefill(prompt), la)
+    fast.forward_prefill_batch(prompt)
+    a = b = fh.ops.argmax_host(la)
+    lf, ls = fast.forward(a), seq.forward(a)                                   # one step, identical state
+    assert np.max(np.abs(lf - ls)) < 5e-2 * max(1.0, float(np.std(ls))) and np.corrcoef(lf, ls)[0, 1] > 0.999
+    same_bits(one.forward(a), ls)
+    a = b = fh.ops.argmax_host(ls)
+    for step in range(126):
+        a2, b2 = one.forward_greedy(a), seq.forward_greedy(b)
+        assert a2 == b2, f"step {step}: {a2} against {b2}"
+        a, b = a2, b2
+    same_bits(one.forward(a), seq.forward(b))
+    for layer in (0, 13, 27):
+        assert np.array_equal(one.read_kv(layer, 0), seq.read_kv(layer, 0))
+        assert np.array_equal(one.read_kv(layer, 1), seq.read_kv(layer, 1))
+    seq.close(); one.close(); fast.close()
