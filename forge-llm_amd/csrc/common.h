@@ -187,6 +187,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
                   const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, uint32_t* counts,
                   const float* qkv_bias, PdState** out);
 int32_t pd_set_repeat_penalty(PdState* st, float penalty);
+void pd_set_poll_limit(PdState* st, uint32_t n);
 void pd_destroy(PdState* st);
 int32_t pd_enqueue(PdState* st, bool profile, uint32_t token, hipStream_t s);
 // Spins on the host word the kernel writes last; false = not available, wait for the stream instead.

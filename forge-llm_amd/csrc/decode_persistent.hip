@@ -114,6 +114,7 @@ struct PdArgs {
     uint32_t* state;   // [0] position  [1] token  [2] next token  [3] abort flag
     uint32_t tag_base, spin_limit;
     uint32_t token, token_from_arg;            // the step's input token when the host passes it with the launch
+    uint32_t step_seq;                         // number of this step (never 0): left in state[4] by whoever counts the step's token
     unsigned long long* host_out;              // host-mapped {next token, launch number}: written last, or null
     uint32_t host_seq;
     uint32_t q4, lm_q4;                        // weight formats: projections, lm_head
@@ -943,7 +944,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
                     if (PEN) {
                         const bool fed = row == cx.token;
                         const uint32_t c = a.counts[row] + (fed ? 1u : 0u);
-                        if (fed) a.counts[row] = c;
+                        if (fed) { a.counts[row] = c; a.state[4] = a.step_seq; }      // so that a step that gives up later can be undone
                         if (a.penalty > 1.0f) v = repeat_penalised(v, c, a.penalty);
                     }
                     best = arg_better(best, ArgPair{v, row});
@@ -1307,6 +1308,9 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     return FORGE_HIP_OK;
 }
 
+// Polls before a workgroup gives up (0: the default).  A test knob: 1 makes every wait fail that is not satisfied at once.
+void pd_set_poll_limit(PdState* st, uint32_t n) { st->args.spin_limit = n ? n : 400000u; }
+
 // A penalty > 1 selects the kernel variant that carries the penalty code: check that it, too, fits one workgroup per CU.
 int32_t pd_set_repeat_penalty(PdState* st, float penalty) {
     const float old = st->args.penalty;
@@ -1327,6 +1331,7 @@ int32_t pd_enqueue(PdState* st, bool profile, uint32_t token, hipStream_t s) {
     PdArgs& a = st->args;
     a.token = token;
     a.token_from_arg = 1;
+    a.step_seq = a.step_seq + 1 ? a.step_seq + 1 : 1;
     a.host_out = st->host_out_dev;
     if (a.host_out) a.host_seq = ++st->seq;
     if (a.tag_base > 0xF0000000u) {      // tags are about to wrap: start again from zeroed buffers
@@ -1375,6 +1380,22 @@ bool pd_wait_token(PdState* st, uint32_t* next) {
 int32_t pd_after_sync(PdState* st, uint32_t abort_flag, hipStream_t s) {
     if (!abort_flag) return FORGE_HIP_OK;
     PdArgs& a = st->args;
+    // The step did not happen: the position was not advanced (the kernel does that last), the cache row of this position
+    // will be written again; what may have happened is the count of the step's token (the kernel variant with the repeat
+    // penalty counts it in its lm_head phase).  It says so in state[4]: take the count back.
+    {
+        uint32_t seq = 0;
+        FH_HIP(hipMemcpyAsync(&seq, a.state + 4, 4, hipMemcpyDeviceToHost, s));
+        FH_HIP(hipStreamSynchronize(s));
+        if (seq == a.step_seq && a.counts) {
+            uint32_t c = 0;
+            FH_HIP(hipMemcpyAsync(&c, a.counts + a.token, 4, hipMemcpyDeviceToHost, s));
+            FH_HIP(hipStreamSynchronize(s));
+            if (c) c -= 1;
+            FH_HIP(hipMemcpyAsync(a.counts + a.token, &c, 4, hipMemcpyHostToDevice, s));
+            FH_HIP(hipStreamSynchronize(s));
+        }
+    }
     FH_HIP(hipMemsetAsync(st->tagged_base, 0, st->tagged_bytes, s));
     FH_HIP(hipMemsetAsync(a.state + 3, 0, 4, s));
     FH_HIP(hipStreamSynchronize(s));

@@ -334,6 +334,8 @@ int32_t finish_decode_step(forge_hip_model* m) {
     return FORGE_HIP_OK;
 }
 
+// Enqueues a decode step.  The position is counted as advanced here; a step that turns out not to have happened (the
+// resident kernel gave up) is taken back by step_failed().
 int32_t forward_common(forge_hip_model* m, uint32_t token) {
     FH_CHECK(m, "model is null");
     if (m->pos >= (int64_t)m->cfg.max_seq) return fail(FORGE_HIP_ERR_POSITION, "KV cache is full (pos == max_seq)");
@@ -342,6 +344,14 @@ int32_t forward_common(forge_hip_model* m, uint32_t token) {
     if (rc) return rc;
     m->pos += 1;
     return FORGE_HIP_OK;
+}
+
+// finish_decode_step() with the host's view put back in line with the device's when the step failed: the device position
+// was not advanced, so neither is the host's, and the same token can be fed again.
+int32_t finish_or_undo(forge_hip_model* m) {
+    const int32_t rc = finish_decode_step(m);
+    if (rc && m->pos > 0) m->pos -= 1;
+    return rc;
 }
 
 }  // namespace
@@ -495,7 +505,7 @@ int32_t forge_hip_forward(forge_hip_model* m, uint32_t token, float* logits_host
     int32_t rc = forward_common(m, token);
     if (rc) return rc;
     FH_HIP(hipMemcpyAsync(logits_host, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, m->stream));
-    return finish_decode_step(m);
+    return finish_or_undo(m);
 }
 
 int32_t forge_hip_forward_greedy(forge_hip_model* m, uint32_t token, uint32_t* next_token_host) {
@@ -504,7 +514,7 @@ int32_t forge_hip_forward_greedy(forge_hip_model* m, uint32_t token, uint32_t* n
     if (rc) return rc;
     // the resident kernel hands the token over through host memory as soon as it is final
     if (m->pd && pd_wait_token(m->pd, next_token_host)) return FORGE_HIP_OK;
-    rc = finish_decode_step(m);
+    rc = finish_or_undo(m);
     if (rc) return rc;
     *next_token_host = m->h_stage[4];
     return FORGE_HIP_OK;
@@ -623,6 +633,13 @@ int32_t forge_hip_model_set_repeat_penalty(forge_hip_model* m, float penalty) {
     m->repeat_penalty = penalty;
     // the captured kernel sequence carries the old value in its launch arguments: capture again at the next step
     if (m->decode_graph) { (void)hipGraphExecDestroy(m->decode_graph); m->decode_graph = nullptr; }
+    return FORGE_HIP_OK;
+}
+
+int32_t forge_hip_model_set_poll_limit(forge_hip_model* m, uint32_t polls) {
+    FH_CHECK(m, "set_poll_limit: model is null");
+    FH_HIP(hipStreamSynchronize(m->stream));
+    if (m->pd) pd_set_poll_limit(m->pd, polls);
     return FORGE_HIP_OK;
 }
 

@@ -122,6 +122,11 @@ class HipModel:
             out.append(nxt)
         return out
 
+    def set_poll_limit(self, polls: int) -> None:
+        """Polls a workgroup of the resident decode kernel spends on one hand-over before the step gives up (0: default).
+        A step that gives up raises ForgeHipError(ERR_HIP) and leaves position, token counts and context as they were."""
+        self._check(self._lib.forge_hip_model_set_poll_limit(self._h, int(polls)))
+
     def set_repeat_penalty(self, penalty: float) -> None:
         """With a penalty > 1, forward_greedy takes the argmax of the logits after apply_repeat_penalty over every token
         fed since the last reset (project.rs:505-513, 742-744), on the device."""

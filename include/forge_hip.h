@@ -123,6 +123,13 @@ int32_t forge_hip_model_decode_launches(const forge_hip_model* m);
 int32_t forge_hip_reset(forge_hip_model* m);
 /* Current position (KVCache.len, emit.rs:3960). */
 int64_t forge_hip_model_pos(const forge_hip_model* m);
+/* How often a workgroup of the resident decode kernel polls for another workgroup's data before the step gives up
+ * (0: the default, 400000 polls, far beyond any wait of a healthy step).  A step that gives up returns
+ * FORGE_HIP_ERR_HIP from forge_hip_forward / forge_hip_forward_greedy and has not happened: the position, the token
+ * counts of the repeat penalty and the context in the cache are what they were before the call, and the same token can
+ * be fed again.  No counterpart in the reference (its CPU loop has nothing to wait for); a no-op for a model that runs
+ * the kernel sequence. */
+int32_t forge_hip_model_set_poll_limit(forge_hip_model* m, uint32_t polls);
 /* Debug/parity: copy layer `layer`'s cached K (which=0) or V (which=1) rows [0,pos) to host as
  * fp16 bit patterns, row-major [pos][kv_heads*head_dim]. */
 int32_t forge_hip_model_read_kv(forge_hip_model* m, uint32_t layer, uint32_t which, uint16_t* out_host);

@@ -284,25 +284,52 @@ def test_persistent_decode_kernel_rewinds_its_tags(fh, torch_gpu, monkeypatch):
     seq.close(); one.close()
 
 
-def test_persistent_decode_kernel_gives_up_instead_of_hanging(fh, torch_gpu, monkeypatch):
+@pytest.mark.parametrize("penalty", [1.0, 1.1])
+def test_persistent_decode_kernel_gives_up_instead_of_hanging(fh, torch_gpu, monkeypatch, penalty):
     """Every wait of the one-kernel step is bounded.  With the bound set to a single re-read the workgroups give up at
     the first hand-over that is not there yet: the kernel ends, the call comes back with FORGE_HIP_ERR_HIP and a message,
-    and the device goes on working (a model created afterwards decodes as usual)."""
+    and the step has not happened: the position is the one before the call, and with the bound lifted the SAME model
+    takes the same token again and goes on bit-identical to the kernel sequence -- logits, greedy tokens (with the
+    repeat penalty too, whose count of the failed step's token must not stay) and the cache."""
     cfg = tiny_cfg(fh, Q8, 0)
     blob = fh.synth.make_weights_blob(cfg, seed=45)
-    monkeypatch.setenv("FORGE_HIP_PERSIST", "1")
-    monkeypatch.setenv("FORGE_HIP_PD_SPIN_LIMIT", "1")
-    impatient = fh.HipModel(cfg, blob)
-    assert impatient.decode_launches == 1
-    with pytest.raises(fh.ForgeHipError) as e:
-        for t in range(8):                                   # the first steps may get through if every hand-over is on time
-            impatient.forward_greedy(t)
-    assert e.value.code == fh.ERR_HIP and "gave up waiting" in str(e.value)
-    impatient.close()
-    monkeypatch.delenv("FORGE_HIP_PD_SPIN_LIMIT")
+    toks = [int(t) for t in fh.synth.uniform_ids(46, 14, cfg["vocab"])]
+    toks[5] = toks[2]                                        # a repeated id, so the count of toks[2] matters below
     seq, one = persistent_pair(fh, cfg, blob, monkeypatch)
-    for t in fh.synth.uniform_ids(46, 6, cfg["vocab"]):
-        same_bits(one.forward(int(t)), seq.forward(int(t)))
+    seq.set_repeat_penalty(penalty); one.set_repeat_penalty(penalty)
+    for t in toks[:2]:
+        assert one.forward_greedy(t) == seq.forward_greedy(t)
+    one.set_poll_limit(1)
+    failures = 0
+    for attempt in range(8):                                 # a step may get through if every hand-over is on time
+        before = one.pos
+        try:
+            one.forward_greedy(toks[2])
+        except fh.ForgeHipError as e:
+            assert e.code == fh.ERR_HIP and "gave up waiting" in str(e)
+            assert one.pos == before
+            failures += 1
+            if failures == 3:
+                break
+        else:                                                # it got through: keep the other model in step
+            assert one.pos == before + 1
+            seq.forward_greedy(toks[2])
+    assert failures, "no step gave up with a poll limit of 1"
+    one.set_poll_limit(0)
+    fed = one.pos - 2                                        # times toks[2] went through after all
+    if fed == 0:
+        assert one.forward_greedy(toks[2]) == seq.forward_greedy(toks[2])
+    assert one.pos == seq.pos
+    for t in toks[3:10]:
+        assert one.forward_greedy(t) == seq.forward_greedy(t)
+    for t in toks[10:]:
+        same_bits(one.forward(t), seq.forward(t))
+    for which in (0, 1):
+        assert np.array_equal(one.read_kv(1, which), seq.read_kv(1, which))
+    # a batched prefill after the failures starts from the host's position: it must be the device's too
+    more = fh.synth.uniform_ids(47, 40, cfg["vocab"])
+    same_bits(one.forward_prefill(more), seq.forward_prefill(more))
+    assert one.forward_greedy(3) == seq.forward_greedy(3)
     seq.close(); one.close()
 
 
