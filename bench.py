@@ -13,9 +13,14 @@ With FORGE_HIP_PERSIST=0 the step is a sequence of kernels and the figure is tha
 launches, each timed by a pair of HIP events attached to its dispatch.  The line also carries the other
 path's figures under "kernel_sequence_path".  `peak` = 8 TB/s (MI355X HBM3E).
 
+exact_mode: the same workload on a model created with FORGE_HIP_FLAG_EXACT (bit-identical to the reference's
+generated kernels): its prefill and decode throughput, and the fast mode's distance from it (first greedy token
+that differs, largest logit difference before that).
+
 cpu_baseline: the CPU restatement of the reference's generated kernels (oracle/), in the arithmetic
-the reference runs on an x86 host (f32 activations x dequantised weights, int8 KV), per-token decode,
-timed on this host's cores on a bounded sample.
+the reference runs on an x86 host (f32 activations x dequantised weights, int8 KV) and beside it in the
+aarch64 arithmetic (int8 activation blocks): batched prefill and per-token decode, timed on this host's cores
+on a bounded sample.
 """
 import argparse
 import json
@@ -31,6 +36,7 @@ HBM_PEAK_GBS = 8000.0
 MFMA_I8_PEAK_TOPS = 5000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 PROMPT_TOKENS = 2502
+DIVERGENCE_STEPS = 128         # greedy steps over which the fast mode's tokens are compared with the exact mode's
 # HBM bytes per GEMV launch of this workload, averaged over the 65 GEMV launches of one decode step: FETCH_SIZE and
 # WRITE_SIZE counters of two profiler runs of this script, each scaled by what the same counter reads for the 1 GiB
 # copy of --calibrate-copy (FETCH_SIZE x2.000, WRITE_SIZE x1.000).  Summary: profiles/gemv_hbm_traffic_pmc.md.
@@ -65,24 +71,38 @@ def prefill_flops(cfg, m):
     return gemm, attn
 
 
-def cpu_baseline(fh, cfg, blob, prompt, budget_s=20.0):
+def cpu_baseline(fh, cfg, blob, prompt, budget_s=24.0):
+    """The CPU restatement of the reference's generated kernels, timed on this host's cores on a bounded sample of the same
+    workload: a batched prefill of the first CTX prompt tokens (forward_prefill_batched), then greedy decode tokens at that
+    context (forward).  `value` is the decode rate in the arithmetic an x86 build of the reference runs (variant B: f32
+    activations x dequantised weights, int8 KV); the aarch64 arithmetic (variant A: int8 activation blocks, the one the
+    GPU's exact mode reproduces bit for bit) is timed beside it on the same sample."""
     from oracle import oracle
-    om = oracle.Model(cfg, blob, oracle.VARIANT_B, oracle.KV_INT8)
     threads = oracle.num_threads()
-    ctx = 8
-    for t in prompt[:ctx]:
-        logits = om.forward(int(t))          # per-token path fills a short cache
-    tok = oracle.argmax(logits)
-    t0 = time.perf_counter()
-    n = 0
-    while n < 32 and (time.perf_counter() - t0 < budget_s or n < 2):
-        tok = oracle.argmax(om.forward(tok))
-        n += 1
-    dt = time.perf_counter() - t0
-    om.close()
-    return {"value": n / dt, "unit": "tok/s", "cores": threads, "kind": "port",
-            "sample": f"{n} greedy decode tokens after an {ctx}-token prompt, same model and weights; f32 x dequantised-weight "
-                      f"arithmetic of the reference's x86 build, int8 KV, OpenMP over rows with {threads} threads"}
+    ctx, n_decode = 64, 16
+    rows = {}
+    for name, variant, kv, share in (("B", oracle.VARIANT_B, oracle.KV_INT8, 0.7), ("A", oracle.VARIANT_A, oracle.KV_F16, 0.3)):
+        om = oracle.Model(cfg, blob, variant, kv)
+        t0 = time.perf_counter()
+        tok = oracle.argmax(om.prefill_batched(prompt[:ctx]))
+        t_prefill = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        n = 0
+        while n < n_decode and (time.perf_counter() - t0 < budget_s * share / 2 or n < 2):
+            tok = oracle.argmax(om.forward(tok))
+            n += 1
+        t_decode = time.perf_counter() - t0
+        om.close()
+        rows[name] = {"decode_tok_per_s": n / t_decode, "decode_tokens": n, "prefill_tok_per_s": ctx / t_prefill,
+                      "prefill_tokens": ctx}
+    return {"value": rows["B"]["decode_tok_per_s"], "unit": "tok/s", "cores": threads, "kind": "port",
+            "decode_context": ctx, "prefill_tok_per_s": rows["B"]["prefill_tok_per_s"],
+            "variant_a": {"decode_tok_per_s": rows["A"]["decode_tok_per_s"], "prefill_tok_per_s": rows["A"]["prefill_tok_per_s"],
+                          "arithmetic": "int8 activation blocks x int8 weight blocks (the reference's aarch64 kernels), fp16 KV"},
+            "sample": f"same model and weights: forward_prefill_batched over the first {ctx} prompt tokens, then "
+                      f"{rows['B']['decode_tokens']} greedy decode tokens at context {ctx}..{ctx + n_decode} (the GPU figures are at "
+                      f"context {len(prompt)}; the CPU's attention share at that context would lower its rate further); f32 x "
+                      f"dequantised-weight arithmetic of the reference's x86 build, int8 KV, OpenMP over rows with {threads} threads"}
 
 
 def decode_profile(fh, model, cfg, tok, context, prof_steps=8):
@@ -132,6 +152,54 @@ def timed_decode(model, tok, warmup, steps):
         tok = model.forward_greedy(tok)
     torch.cuda.synchronize()
     return time.perf_counter() - t0, tok
+
+
+def greedy_with_logits(fh, model, prompt, n):
+    """Prefill, then n greedy picks, every step through `forward` so the logits come back: tokens [n] and logits
+    [n][vocab] (logits[i] are the ones whose argmax is tokens[i])."""
+    import numpy as np
+    model.reset()
+    logits = [model.forward_prefill(prompt)]
+    toks = [fh.ops.argmax_host(logits[0])]
+    for _ in range(n - 1):
+        logits.append(model.forward(toks[-1]))
+        toks.append(fh.ops.argmax_host(logits[-1]))
+    return toks, np.stack(logits)
+
+
+def exact_mode_figures(fh, cfg, blob, prompt, warmup, steps, fast_tokens, fast_logits):
+    """The same workload with FORGE_HIP_FLAG_EXACT (the arithmetic that reproduces the reference's generated kernels bit
+    for bit: ordered block sums, the reference's softmax and exponential): prefill and decode throughput, and how far the
+    fast mode measured above is from it -- the first greedy token at which the two differ over `len(fast_tokens)` steps,
+    the largest logit difference while both still had the same context, and the margin between the two largest exact
+    logits at the step where they part (how close that choice was)."""
+    import numpy as np
+    import torch
+    m = fh.HipModel(dict(cfg, flags=cfg.get("flags", 0) | fh.FLAG_EXACT), blob)
+    m.forward_prefill_batch(prompt)
+    m.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    logits = m.forward_prefill(prompt)
+    torch.cuda.synchronize()
+    t_prefill = time.perf_counter() - t0
+    t_decode, _ = timed_decode(m, fh.ops.argmax_host(logits), warmup, steps)
+    launches = m.decode_launches
+    toks, lg = greedy_with_logits(fh, m, prompt, len(fast_tokens))
+    m.close()
+    same = [a == b for a, b in zip(toks, fast_tokens)]
+    first = same.index(False) if False in same else None
+    shared = len(toks) if first is None else first + 1            # logits[i] come from identical contexts for i <= first
+    delta = np.abs(lg[:shared].astype(np.float64) - fast_logits[:shared]).max(axis=1)
+    out = {"decode_tok_per_s": steps / t_decode, "ms_per_step": t_decode / steps * 1e3, "prefill_tok_per_s": len(prompt) / t_prefill,
+           "prefill_ms": t_prefill * 1e3, "decode_path": f"{launches} kernels per token (graph replay), order-faithful kernels",
+           "fast_vs_exact": {"greedy_steps_compared": len(toks), "first_divergent_token": first,
+                             "max_logit_delta": float(delta.max()), "prefill_logit_delta": float(delta[0]),
+                             "logit_absmax": float(np.abs(lg[:shared]).max())}}
+    if first is not None:
+        top2 = np.partition(lg[first], -2)[-2:]
+        out["fast_vs_exact"]["exact_top2_margin_at_divergence"] = float(top2[1] - top2[0])
+    return out
 
 
 def ops_table(fh, reps=10):
@@ -217,6 +285,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-gguf", action="store_true", help="create the model from the weights blob instead of from a GGUF file")
     ap.add_argument("--no-alt", action="store_true", help="skip the second model that measures the kernel-sequence decode step")
+    ap.add_argument("--no-exact", action="store_true",
+                    help="skip the third model that measures the exact mode and the fast mode's distance from it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (known HBM traffic, for scaling counter readings)")
     ap.add_argument("--model", choices=("llama32_1b", "llama32_3b", "smollm2_135m", "llama31_8b", "qwen25_1p5b", "mistral_7b", "phi3_mini", "qwen25_14b"), default="llama32_1b",
@@ -240,7 +310,7 @@ def main():
         return
     wd = fh.Q8_0 if args.format == "q8_0" else fh.Q4_0
     PROMPT_TOKENS = args.prompt_tokens
-    cfg = getattr(fh.synth, args.model)(wd, max_seq=max(4096, (PROMPT_TOKENS + 2 * (args.warmup + args.steps) + 16 + 1023) // 1024 * 1024))
+    cfg = getattr(fh.synth, args.model)(wd, max_seq=max(4096, (PROMPT_TOKENS + max(2 * (args.warmup + args.steps), DIVERGENCE_STEPS) + 16 + 1023) // 1024 * 1024))
     headline = args.model == "llama32_1b" and args.format == "q8_0" and PROMPT_TOKENS == 2502
     model_name = {"llama32_1b": "Llama-3.2-1B", "llama32_3b": "Llama-3.2-3B", "smollm2_135m": "SmolLM2-135M", "llama31_8b": "Llama-3.1-8B",
                   "qwen25_1p5b": "Qwen2.5-1.5B", "mistral_7b": "Mistral-7B (sliding window 4096)", "phi3_mini": "Phi-3-mini", "qwen25_14b": "Qwen2.5-14B"}[args.model]
@@ -301,6 +371,9 @@ def main():
             f"{model.decode_launches} launches of the resident kernel per token (34 layers each)"
             if model.decode_launches <= (cfg["layers"] + 33) // 34 else f"{model.decode_launches} kernels per token (graph replay)")
 
+    # ---- the fast mode's greedy tokens and logits over DIVERGENCE_STEPS steps, for the comparison with the exact mode
+    fast_tokens, fast_logits = (None, None) if args.no_exact else greedy_with_logits(fh, model, prompt, DIVERGENCE_STEPS)
+
     # ---- the reference's default loop: greedy with repeat penalty 1.1 over every token fed (project.rs:607-611, 742-744)
     model.reset()
     model.set_repeat_penalty(1.1)
@@ -324,6 +397,7 @@ def main():
             m2.close()
         finally:
             os.environ["FORGE_HIP_PERSIST"] = "1"
+    exact = None if args.no_exact else exact_mode_figures(fh, cfg, blob, prompt, args.warmup, args.steps, fast_tokens, fast_logits)
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)     # 1 GiB
         dst = torch.empty_like(src)
@@ -354,6 +428,7 @@ def main():
         "decode_tok_per_s_short_context": args.steps / t_decode_short,
         "decode_tok_per_s_repeat_penalty_1.1": args.steps / t_decode_pen,
         "decode_weight_stream_GBps_end_to_end": fh.synth.decode_weight_bytes(cfg) * args.steps / t_decode / 1e9,
+        "exact_mode": exact,
         "roofline": roofline,
         "prefill_rooflines": {
             "gemm": {"bound": "mfma", "achieved": gemm_flops / (gemm_ms * 1e-3) / 1e12, "peak": MFMA_I8_PEAK_TOPS,

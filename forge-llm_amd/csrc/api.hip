@@ -160,7 +160,7 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
 int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, uint32_t M, int32_t* out_dev,
                               uint32_t path, void* stream) {
     FH_CHECK(w && x_dev && out_dev, "block_isums: null pointer");
-    FH_CHECK(path <= 1, "block_isums: path must be 0 (GEMV kernel) or 1 (MFMA GEMM kernel)");
+    FH_CHECK(path <= 2, "block_isums: path must be 0 (GEMV kernel), 1 (MFMA GEMM kernel, exact mode) or 2 (MFMA GEMM kernel, fast mode)");
     if (M == 0) return FORGE_HIP_OK;
     int8_t* q; uint16_t* sc;
     int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream);
@@ -176,7 +176,7 @@ int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, ui
         Scratch& sink = g_attn;
         rc = sink.reserve((size_t)M * w->w.N * sizeof(float));
         if (rc) return rc;
-        launch_gemm(w->w, q, sc, M, reinterpret_cast<float*>(sink.p), w->w.N, false, true, out_dev, (hipStream_t)stream);
+        launch_gemm(w->w, q, sc, M, reinterpret_cast<float*>(sink.p), w->w.N, false, path == 1, out_dev, (hipStream_t)stream);
     }
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;

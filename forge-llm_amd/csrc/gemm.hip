@@ -77,7 +77,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                    const uint16_t* __restrict__ asc, float* __restrict__ y, int32_t* __restrict__ isums, uint32_t M,
                    uint32_t N, uint32_t K, uint32_t ldy, int accumulate) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    constexpr bool MAGIC = !EXACT && !DUMP;
+    constexpr bool MAGIC = !EXACT;               // DUMP && !EXACT: the fast arithmetic, with its block sums written out too
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // uniform: the compiler keeps it scalar
@@ -286,8 +286,15 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                     const uint32_t mb = m0 + wm * WM + tm * 32 + 4 * lhalf;
                     const uint32_t base = (n < N && b < nblk) ? ((mb * N + n) * nblk + b) * 4 : OOB;
 #pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        __builtin_amdgcn_raw_buffer_store_b32((uint32_t)isum[r], rdump, base + (8 * (r >> 2) + (r & 3)) * N * nblk * 4, 0, 0);
+                    for (int r = 0; r < 16; r++) {
+                        int32_t v = isum[r];
+                        if (MAGIC) {                 // what the biased accumulator holds, turned back into the block sum
+                            v -= (int32_t)MAGIC_BITS;
+                            if (kb & 1) v = -v;      // odd blocks ran on negated activation codes
+                            if (Q4) v >>= 4;         // nibble codes were fed as 16 (c - 8)
+                        }
+                        __builtin_amdgcn_raw_buffer_store_b32((uint32_t)v, rdump, base + (8 * (r >> 2) + (r & 3)) * N * nblk * 4, 0, 0);
+                    }
                 }
                 isum = isum_n;
                 S = S_n;
@@ -402,11 +409,13 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
             const uint64_t tiles64 = (uint64_t)((nc + BN - 1) / BN) * ((mc + 63) / 64);
             const bool small_tiles = tiles64 <= (uint64_t)cus && mc > 64;
             if (q4) {
-                if (isums) FH_GEMM_LAUNCH(true, true, true);
+                if (isums && exact) FH_GEMM_LAUNCH(true, true, true);
+                else if (isums) FH_GEMM_LAUNCH(true, true, false);
                 else if (exact) FH_GEMM_LAUNCH(true, false, true);
                 else FH_GEMM_LAUNCH(true, false, false);
             } else {
-                if (isums) FH_GEMM_LAUNCH(false, true, true);
+                if (isums && exact) FH_GEMM_LAUNCH(false, true, true);
+                else if (isums) FH_GEMM_LAUNCH(false, true, false);
                 else if (exact) FH_GEMM_LAUNCH(false, false, true);
                 else FH_GEMM_LAUNCH(false, false, false);
             }

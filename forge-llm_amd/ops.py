@@ -163,7 +163,7 @@ def matmul_mat_q(w: QWeight, x, flags=0):
 
 
 def block_isums(w: QWeight, x, path):
-    """int32 block sums [M][N][K/32]; path 0 = GEMV kernel, 1 = MFMA GEMM kernel."""
+    """int32 block sums [M][N][K/32]; path 0 = GEMV kernel, 1 = MFMA GEMM kernel (exact mode), 2 = the same in fast mode."""
     from . import check, lib
     torch = _torch()
     x = _dev(x, torch.float32)

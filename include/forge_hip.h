@@ -171,7 +171,9 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
 
 /* The int32 block sums the two calls above combine: out_dev int32 [M][N][K/32]
  * (dot_q8_0_q8_0 / dot_q4_0_q8_0 `vaddvq_s32(acc)`, emit.rs:1543-1553, 2522-2552).
- * path 0 = the GEMV kernel's dot, path 1 = the MFMA GEMM kernel's tiles. */
+ * path 0 = the GEMV kernel's dot, path 1 = the MFMA GEMM kernel's tiles in exact mode, path 2 = the same kernel in the
+ * fast mode (which accumulates the sums on top of a floating-point bias, negates odd blocks and feeds 4-bit codes times
+ * 16: the sums written out are recovered from those accumulators, so they show what the fast arithmetic really summed). */
 int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, uint32_t M, int32_t* out_dev,
                               uint32_t path, void* stream);
 

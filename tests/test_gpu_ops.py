@@ -55,7 +55,7 @@ def test_quantize_act_bit_exact(fh, oracle, torch_gpu, M, K):
 
 @pytest.mark.parametrize("wd", [Q8, Q4])
 @pytest.mark.parametrize("N,K", [(8, 32), (13, 576), (260, 2048), (64, 8192), (70, 3072)])
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 def test_block_isums_bit_exact(fh, oracle, torch_gpu, wd, N, K, path):
     torch = torch_gpu
     M = 1 if path == 0 else 37
@@ -68,7 +68,7 @@ def test_block_isums_bit_exact(fh, oracle, torch_gpu, wd, N, K, path):
         assert np.array_equal(got[r], want), f"row {r}"
 
 
-@pytest.mark.parametrize("path", [0, 1])
+@pytest.mark.parametrize("path", [0, 1, 2])
 def test_block_isums_extreme_codes(fh, oracle, torch_gpu, path):
     """All +-127 activations against all +-127 weights: |isum| = 516128, the int32 extreme of a block."""
     torch = torch_gpu
