@@ -244,7 +244,7 @@ int32_t forge_hip_attn_prefill_f16kv(const float* q_dev, const uint16_t* k_cache
     if (rc) return rc;
     if (flags & FORGE_HIP_FLAG_EXACT)
         launch_attn_exact(true, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr,
-                          nullptr, M, base_pos, nullptr, heads, kv_heads, head_dim, 0u, 0u, (hipStream_t)stream);
+                          nullptr, M, base_pos, nullptr, heads, kv_heads, head_dim, 0u, 0u, nullptr, (hipStream_t)stream);
     else
         launch_attn_prefill(q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, M, base_pos,
                             heads, kv_heads, head_dim, 0u, (hipStream_t)stream);
@@ -262,7 +262,7 @@ int32_t forge_hip_attn_prefill_sliding_f16kv(const float* q_dev, const uint16_t*
     if (rc) return rc;
     if (flags & FORGE_HIP_FLAG_EXACT)
         launch_attn_exact(true, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr, nullptr, M,
-                          base_pos, nullptr, heads, kv_heads, head_dim, window, base_pos + M, (hipStream_t)stream);
+                          base_pos, nullptr, heads, kv_heads, head_dim, window, base_pos + M, nullptr, (hipStream_t)stream);
     else
         launch_attn_prefill(q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, M, base_pos, heads,
                             kv_heads, head_dim, window, (hipStream_t)stream);
@@ -279,8 +279,15 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
     int32_t rc = check_attn_shape("attn_decode", heads, kv_heads, head_dim);
     if (rc) return rc;
     if (flags & FORGE_HIP_FLAG_EXACT) {
+        // spread over (key block, head) workgroups when the cache is short enough for that kernel's tables
+        const size_t xb = attn_exact_decode_workspace_bytes(heads, head_dim, seq_len);
+        if (xb) {
+            rc = g_attn.reserve(xb);
+            if (rc) return rc;
+        }
         launch_attn_exact(false, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr,
-                          nullptr, 1, seq_len - 1, nullptr, heads, kv_heads, head_dim, 0u, 0u, (hipStream_t)stream);
+                          nullptr, 1, seq_len - 1, nullptr, heads, kv_heads, head_dim, 0u, seq_len, xb ? g_attn.p : nullptr,
+                          (hipStream_t)stream);
     } else {
         rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
         if (rc) return rc;
@@ -303,7 +310,7 @@ int32_t forge_hip_attn_decode_sliding_f16kv(const float* q_dev, const uint16_t* 
     if (flags & FORGE_HIP_FLAG_EXACT) {
         FH_CHECK(std::min(window, seq_len) <= attn_exact_max_window(), "attn_decode_sliding: the exact kernel keeps at most 12288 scores");
         launch_attn_exact(false, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr, nullptr, 1,
-                          seq_len - 1, nullptr, heads, kv_heads, head_dim, window, seq_len, (hipStream_t)stream);
+                          seq_len - 1, nullptr, heads, kv_heads, head_dim, window, seq_len, nullptr, (hipStream_t)stream);
     } else {
         rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
         if (rc) return rc;

@@ -185,14 +185,173 @@ __global__ void attn_exact_sliding_kernel(const float* __restrict__ q, uint32_t 
     }
 }
 
+// ---- attention_flash for ONE query row (the decode step), spread over the chip.
+// The reference's loop over 64-key blocks looks serial, but only a thin thread of it is: per block it needs the running
+// maximum (a prefix maximum of the block maxima: order-free), then exp(s - m_i) per key, the block's sequential sums
+// l_block and sum[d] -- all of which depend on nothing but this block's scores and m_i -- and only then the recurrence
+//     l_i = l_i * exp_scale + l_block,   acc[d] = acc[d] * exp_scale + sum[d]        (two roundings each, in that order)
+// that ties the blocks together.  So: (1) one workgroup per (block, head) computes the block's scores and maximum;
+// (2) one workgroup per (block, head) computes m_i, the weights, l_block and sum[d], every sequential sum in the
+// reference's order; (3) one workgroup per head runs the recurrence over the blocks' records.  Every f32 operation has
+// the operands and the order it has in the one-workgroup kernel above, so the bits are the same; the work of steps 1
+// and 2 (all the memory traffic and all but a few operations per block) runs on as many workgroups as there are blocks.
+// Workspace per head: scores [rows_cap], then per block: maximum, m_i, l_block, sum[HD]  (nb_cap = rows_cap / 64 blocks).
+constexpr uint32_t XD_MAX_BLOCKS = 4096;     // blocks whose exp_scale the last step keeps in LDS: caches up to 262144 rows
+
+__host__ __device__ inline size_t xd_head_floats(uint32_t nb_cap, uint32_t hd) { return (size_t)nb_cap * (XB + 3 + hd); }
+
+struct XdWs {
+    float *scores, *bmax, *mi, *lblk, *sums;
+};
+__device__ __forceinline__ XdWs xd_ws(float* ws, uint32_t h, uint32_t nb_cap, uint32_t hd) {
+    float* p = ws + (size_t)h * xd_head_floats(nb_cap, hd);
+    return XdWs{p, p + (size_t)nb_cap * XB, p + (size_t)nb_cap * (XB + 1), p + (size_t)nb_cap * (XB + 2), p + (size_t)nb_cap * (XB + 3)};
+}
+
+template <int HD>
+__global__ __launch_bounds__(64) void attn_exact_decode_scores_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc,
+                                                                     float* __restrict__ ws, uint32_t base_pos,
+                                                                     const uint32_t* __restrict__ pos_dev, uint32_t heads,
+                                                                     uint32_t kv_heads, uint32_t nb_cap) {
+    __shared__ float qs[HD];
+    const uint32_t tid = threadIdx.x, b = blockIdx.x, h = blockIdx.y;
+    const uint32_t seq = (pos_dev ? *pos_dev : base_pos) + 1, bs = b * XB;
+    if (bs >= seq) return;
+    const uint32_t kvh = h / (heads / kv_heads), kv_stride = kv_heads * HD, bl = min((uint32_t)XB, seq - bs);
+    const float scale = 1.0f / sqrtf((float)HD);
+    for (uint32_t i = tid; i < HD; i += 64) qs[i] = q[h * HD + i];
+    __syncthreads();
+    float sc = -INFINITY;
+    if (tid < bl) {
+        const uint16_t* krow = kc + (size_t)(bs + tid) * kv_stride + kvh * HD;
+        float sum = 0.f;
+#pragma unroll
+        for (int c = 0; c < HD / 8; c++) {
+            const uint4 w = *reinterpret_cast<const uint4*>(krow + c * 8);
+            const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                sum = sum + qs[c * 8 + 2 * j] * f16_bits_to_f32((uint16_t)(ww[j] & 0xFFFFu));
+                sum = sum + qs[c * 8 + 2 * j + 1] * f16_bits_to_f32((uint16_t)(ww[j] >> 16));
+            }
+        }
+        sc = sum * scale;
+    }
+    const XdWs w = xd_ws(ws, h, nb_cap, HD);
+    if (tid < bl) w.scores[bs + tid] = sc;
+    const float mb = wave_max(sc);
+    if (tid == 0) w.bmax[b] = mb;
+}
+
+template <int HD>
+__global__ __launch_bounds__(HD <= 64 ? 64 : 128) void attn_exact_decode_block_kernel(const uint16_t* __restrict__ vc, float* __restrict__ ws,
+                                                                                    uint32_t base_pos, const uint32_t* __restrict__ pos_dev,
+                                                                                    uint32_t heads, uint32_t kv_heads, uint32_t nb_cap) {
+    __shared__ float e[XB];
+    __shared__ float red[1];
+    const uint32_t tid = threadIdx.x, b = blockIdx.x, h = blockIdx.y;
+    const uint32_t seq = (pos_dev ? *pos_dev : base_pos) + 1, bs = b * XB;
+    if (bs >= seq) return;
+    const uint32_t kvh = h / (heads / kv_heads), kv_stride = kv_heads * HD, bl = min((uint32_t)XB, seq - bs);
+    const XdWs w = xd_ws(ws, h, nb_cap, HD);
+    if (tid < 64) {
+        // m_i after this block: the largest block maximum so far (`if m_block > m_i { m_i = m_block }` from -inf on)
+        float m = -INFINITY;
+        for (uint32_t i = tid; i <= b; i += 64) m = fmaxf(m, w.bmax[i]);
+        m = wave_max(m);
+        if (tid == 0) { red[0] = m; w.mi[b] = m; }
+        if (tid < bl) e[tid] = expf_ref<true>(w.scores[bs + tid] - m);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        float l_block = 0.f;
+        for (uint32_t bi = 0; bi < bl; bi++) l_block = l_block + e[bi];
+        w.lblk[b] = l_block;
+    }
+    if (tid < HD) {
+        const uint16_t* vcol = vc + (size_t)bs * kv_stride + kvh * HD + tid;
+        float sum = 0.f;
+        if (bl == XB) {
+#pragma unroll 16
+            for (uint32_t bi = 0; bi < XB; bi++) sum = sum + e[bi] * f16_bits_to_f32(vcol[(size_t)bi * kv_stride]);
+        } else {
+            for (uint32_t bi = 0; bi < bl; bi++) sum = sum + e[bi] * f16_bits_to_f32(vcol[(size_t)bi * kv_stride]);
+        }
+        w.sums[(size_t)b * HD + tid] = sum;
+    }
+}
+
+template <int HD>
+__global__ __launch_bounds__(HD <= 64 ? 64 : 128) void attn_exact_decode_chain_kernel(float* __restrict__ ws, float* __restrict__ out,
+                                                                                    int8_t* __restrict__ oq, uint16_t* __restrict__ osc,
+                                                                                    uint32_t base_pos, const uint32_t* __restrict__ pos_dev,
+                                                                                    uint32_t heads, uint32_t nb_cap) {
+    __shared__ float es[XD_MAX_BLOCKS];
+    const uint32_t tid = threadIdx.x, nt = blockDim.x, h = blockIdx.x;
+    const uint32_t seq = (pos_dev ? *pos_dev : base_pos) + 1, nb = (seq + XB - 1) / XB;
+    const XdWs w = xd_ws(ws, h, nb_cap, HD);
+    // exp_scale of every block: exp(m_prev - m_i), m_prev = -inf before the first block
+    for (uint32_t i = tid; i < nb; i += nt) es[i] = expf_ref<true>((i ? w.mi[i - 1] : -INFINITY) - w.mi[i]);
+    __syncthreads();
+    float l_i = 0.f, acc = 0.f;
+    const uint32_t d = tid < HD ? tid : 0;
+#pragma unroll 4
+    for (uint32_t i = 0; i < nb; i++) {
+        const float exp_scale = es[i];
+        l_i = l_i * exp_scale;
+        acc = acc * exp_scale;
+        l_i = l_i + w.lblk[i];
+        acc = acc + w.sums[(size_t)i * HD + d];
+    }
+    const float inv_l = 1.0f / l_i;
+    const float o = acc * inv_l;
+    if (tid < HD && out) out[h * HD + tid] = o;
+    if (oq) {
+        float amax = tid < HD ? fabsf(o) : 0.f;
+#pragma unroll
+        for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+        float inv;
+        const float sc = act_scale(amax, inv);
+        if (tid < HD) {
+            const size_t idx = (size_t)h * HD + tid;
+            oq[idx] = (int8_t)quant_code(o * inv);
+            if ((tid & 31) == 0) osc[idx / 32] = f32_to_f16_bits(sc);
+        }
+    }
+}
+
+// Workspace of the spread-out decode attention for a cache of up to max_rows rows; 0 if it does not apply (then the
+// one-workgroup kernel runs).
+size_t attn_exact_decode_workspace_bytes(uint32_t heads, uint32_t hd, uint32_t max_rows) {
+    const uint32_t nb_cap = (max_rows + XB - 1) / XB;
+    if (max_rows == 0 || nb_cap > XD_MAX_BLOCKS) return 0;
+    return (size_t)heads * xd_head_floats(nb_cap, hd) * sizeof(float);
+}
+
 // Longest window (rows whose scores one workgroup keeps in LDS) the order-faithful decode attention takes.
 uint32_t attn_exact_max_window() { return 12288; }
 
 void launch_attn_exact(bool batch_order, const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc,
                        float* out, uint32_t out_stride, int8_t* oq, uint16_t* osc, uint32_t M, uint32_t base_pos,
                        const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, uint32_t window, uint32_t max_rows,
-                       hipStream_t s) {
+                       void* ws, hipStream_t s) {
     if (M == 0) return;
+    if (ws && !batch_order && window == 0 && M == 1 && attn_exact_decode_workspace_bytes(heads, hd, max_rows) != 0) {
+        const uint32_t nb_cap = (max_rows + XB - 1) / XB;
+        // blocks past the position (known to the device only when pos_dev is set) return at once
+        const uint32_t nb = pos_dev ? nb_cap : (base_pos + XB) / XB;
+        float* w = static_cast<float*>(ws);
+        dim3 g2(nb, heads);
+#define FH_XD(HD_)                                                                                                              \
+    do {                                                                                                                        \
+        fh::launch(attn_exact_decode_scores_kernel<HD_>, g2, 64, 0, s, q, kc, w, base_pos, pos_dev, heads, kv_heads, nb_cap);   \
+        fh::launch(attn_exact_decode_block_kernel<HD_>, g2, HD_ <= 64 ? 64 : 128, 0, s, vc, w, base_pos, pos_dev, heads, kv_heads, nb_cap); \
+        fh::launch(attn_exact_decode_chain_kernel<HD_>, dim3(heads), HD_ <= 64 ? 64 : 128, 0, s, w, out, oq, osc, base_pos, pos_dev, heads, nb_cap); \
+    } while (0)
+        if (hd == 64) FH_XD(64); else if (hd == 96) FH_XD(96); else FH_XD(128);
+#undef FH_XD
+        return;
+    }
     dim3 grid(heads, M);
     const uint32_t threads = hd <= 64 ? 64 : 128;
     if (window != 0 && !batch_order) {

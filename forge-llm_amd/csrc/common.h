@@ -166,7 +166,10 @@ bool attn_head_dim_supported(uint32_t hd);
 void launch_attn_exact(bool batch_order, const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc,
                        float* out, uint32_t out_stride, int8_t* oq, uint16_t* osc, uint32_t M, uint32_t base_pos,
                        const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, uint32_t window, uint32_t max_rows,
-                       hipStream_t s);
+                       void* ws, hipStream_t s);
+// One decode row without a window runs spread over (key block, head) workgroups when `ws` holds
+// attn_exact_decode_workspace_bytes(heads, hd, max_rows) bytes (0: caches that long keep the one-workgroup kernel): same bits.
+size_t attn_exact_decode_workspace_bytes(uint32_t heads, uint32_t hd, uint32_t max_rows);
 uint32_t attn_exact_max_window();
 
 // decode_persistent.hip — the whole decode step as one resident kernel (fast mode only)

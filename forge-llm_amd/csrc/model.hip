@@ -185,7 +185,7 @@ void enqueue_decode_attention(forge_hip_model* m, uint32_t l, const float* q, ui
         StageMark t(m, ST_ATTN);
         if (exact)
             launch_attn_exact(false, q, q_stride, m->kc(l), m->vc(l), nullptr, m->QKS, aq, asc, 1, 0, m->d_pos(), c.heads,
-                              c.kv_heads, c.head_dim, c.sliding_window, c.max_seq, s);
+                              c.kv_heads, c.head_dim, c.sliding_window, c.max_seq, m->attn_ws.p, s);
         else
             launch_attn_decode(q, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads, c.head_dim,
                                c.sliding_window, m->attn_ws.p, s);
@@ -255,7 +255,7 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
                              c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s);
     }
     if (exact) {
-        { StageMark t(m, ST_ATTN); launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, c.sliding_window, c.max_seq, s); }
+        { StageMark t(m, ST_ATTN); launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, c.sliding_window, c.max_seq, nullptr, s); }
         { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
     } else if (m->prefill_fuse_quant) {
         // the attention kernel writes the o projection's quantised input itself
@@ -466,7 +466,7 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
     // ---- scratch ----
     if ((rc = m->x.alloc(H * 4)) || (rc = m->qkv.alloc(m->QKV * 4)) || (rc = m->gu.alloc(2 * (size_t)I * 4)) ||
         (rc = m->logits.alloc((size_t)cfg->vocab * 4)) || (rc = m->aq.alloc(m->KMAX)) ||
-        (rc = m->asc.alloc(m->KMAX / 32 * 2)) || (rc = m->attn_ws.alloc(attn_decode_workspace_bytes(cfg->heads, cfg->head_dim))) ||
+        (rc = m->asc.alloc(m->KMAX / 32 * 2)) || (rc = m->attn_ws.alloc(std::max(attn_decode_workspace_bytes(cfg->heads, cfg->head_dim), (cfg->flags & FORGE_HIP_FLAG_EXACT) ? attn_exact_decode_workspace_bytes(cfg->heads, cfg->head_dim, cfg->max_seq) : (size_t)0))) ||
         (rc = m->state.alloc(64)) || (rc = m->argmax_ws.alloc(ARGMAX_BLOCKS * 8)) || (rc = m->counts.alloc((size_t)cfg->vocab * 4)))
         return rc;
     FH_HIP(hipMemset(m->state.p, 0, 64));
