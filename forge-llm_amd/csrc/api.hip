@@ -58,14 +58,14 @@ inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 bool valid_wdtype(uint32_t t) { return t == FORGE_HIP_Q8_0 || t == FORGE_HIP_Q4_0; }
 
 // Quantise x[M][K] into the shared scratch; returns pointers.
-int32_t quantise_into_scratch(const float* x, uint32_t M, uint32_t K, int8_t** q, uint16_t** sc, hipStream_t s) {
+int32_t quantise_into_scratch(const float* x, uint32_t M, uint32_t K, int8_t** q, uint16_t** sc, hipStream_t s, bool neg_odd = false) {
     const size_t qbytes = align256((size_t)M * K);
     const size_t sbytes = (size_t)M * (K / 32) * 2;
     int32_t rc = g_act.reserve(qbytes + sbytes);
     if (rc) return rc;
     *q = reinterpret_cast<int8_t*>(g_act.p);
     *sc = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(g_act.p) + qbytes);
-    launch_quantize_act(x, M, K, *q, *sc, s);
+    launch_quantize_act(x, M, K, *q, *sc, s, neg_odd);
     return FORGE_HIP_OK;
 }
 
@@ -150,9 +150,10 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
     FH_CHECK((flags & ~FORGE_HIP_FLAG_EXACT) == 0, "gemm_q: unknown flag bits");
     if (M == 0) return FORGE_HIP_OK;
     int8_t* q; uint16_t* sc;
-    int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream);
+    const bool exact = (flags & FORGE_HIP_FLAG_EXACT) != 0;
+    int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream, !exact);   // the fast kernel takes odd blocks negated
     if (rc) return rc;
-    launch_gemm(w->w, q, sc, M, y_dev, w->w.N, false, (flags & FORGE_HIP_FLAG_EXACT) != 0, nullptr, (hipStream_t)stream);
+    launch_gemm(w->w, q, sc, M, y_dev, w->w.N, false, exact, nullptr, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }
@@ -163,7 +164,7 @@ int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, ui
     FH_CHECK(path <= 2, "block_isums: path must be 0 (GEMV kernel), 1 (MFMA GEMM kernel, exact mode) or 2 (MFMA GEMM kernel, fast mode)");
     if (M == 0) return FORGE_HIP_OK;
     int8_t* q; uint16_t* sc;
-    int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream);
+    int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream, path == 2);
     if (rc) return rc;
     const size_t nblk = w->w.K / 32;
     if (path == 0) {

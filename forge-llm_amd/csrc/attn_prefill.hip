@@ -260,6 +260,8 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
             amax = fmaxf(amax, __shfl_xor(amax, 32, WAVE));
             float inv;
             const float sc = act_scale(amax, inv);
+            // QUANT has no f32 output, so out_stride carries a flag instead: store the odd blocks of a row negated
+            if (out_stride != 0 && ((head * (HD / 32) + d) & 1u) != 0) inv = -inv;
             if (qrow < M) {
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
@@ -317,10 +319,10 @@ void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, 
 
 void launch_attn_prefill_quant(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, int8_t* oq, uint16_t* osc,
                                uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, uint32_t hd, uint32_t window,
-                               hipStream_t s) {
+                               hipStream_t s, bool neg_odd) {
     if (M == 0) return;
     dim3 grid(((M + QB - 1) / QB) * heads);
-    launch_hd<true>(hd, grid, s, q, kc, vc, nullptr, q_stride, 0u, M, base_pos, heads, kv_heads, oq, osc, window);
+    launch_hd<true>(hd, grid, s, q, kc, vc, nullptr, q_stride, neg_odd ? 1u : 0u, M, base_pos, heads, kv_heads, oq, osc, window);
 }
 
 }  // namespace fh

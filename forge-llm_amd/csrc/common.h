@@ -87,14 +87,15 @@ void qweight_free(QWeight* w);
 // All are asynchronous on `s` and validate nothing: callers check shapes first.
 
 // elementwise.hip
-void launch_quantize_act(const float* x, uint32_t M, uint32_t K, int8_t* q, uint16_t* sc, hipStream_t s);
+// neg_odd (here and below): the codes of a row's odd blocks are stored negated, as the fast prefill GEMM takes them.
+void launch_quantize_act(const float* x, uint32_t M, uint32_t K, int8_t* q, uint16_t* sc, hipStream_t s, bool neg_odd = false);
 // rms_norm of M rows; writes f32 `normed` if non-null and the quantised row (q, sc) if q non-null.
 void launch_rmsnorm(const float* x, const float* w, float eps, uint32_t M, uint32_t H, float* normed, int8_t* q,
-                    uint16_t* sc, hipStream_t s);
+                    uint16_t* sc, hipStream_t s, bool neg_odd = false);
 // out = silu(gate)*up over M rows where gate = gu[r][0..I), up = gu[r][I..2I) when fused, else two
 // pointers; writes f32 out if non-null and quantised (q, sc) if q non-null.
 void launch_silu_mul(const float* gate, const float* up, uint32_t M, uint32_t I, uint32_t row_stride, float* out,
-                     int8_t* q, uint16_t* sc, hipStream_t s);
+                     int8_t* q, uint16_t* sc, hipStream_t s, bool neg_odd = false);
 // Interleaved-pair RoPE on q,k and fp16 cache write of k,v.  Position of row r is
 // (pos_dev ? *pos_dev : base_pos) + r.  q/k/v rows have strides q_stride/kv_stride floats.
 void launch_rope_kv_store(float* q, float* k, const float* v, uint32_t q_stride, uint32_t kv_stride, uint16_t* kc,
@@ -130,7 +131,8 @@ void launch_gemv_norm_silu_quant(const QWeight& wgu, const float* x, const float
                                  uint16_t* osc, hipStream_t s);
 
 // gemm.hip — y[m][n] (=|+=) ...; aq int8 [M][K], as fp16 [M][K/32].  isums (optional) int32 [M][N][K/32].
-// exact: unfused multiply/add per block (bit-identical to the CPU path); otherwise one FMA per block.
+// exact: unfused multiply/add per block (bit-identical to the CPU path); otherwise one FMA per block, and then the
+// activation codes of every row's odd blocks must come negated (the neg_odd flag of the quantising launchers).
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
                  bool accumulate, bool exact, int32_t* isums, hipStream_t s);
 
@@ -154,7 +156,7 @@ void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, 
 // osc[M][heads*hd/32] (bit-identical to launch_attn_prefill followed by launch_quantize_act).
 void launch_attn_prefill_quant(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, int8_t* oq, uint16_t* osc,
                                uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, uint32_t hd, uint32_t window,
-                               hipStream_t s);
+                               hipStream_t s, bool neg_odd = false);
 
 bool attn_head_dim_supported(uint32_t hd);
 

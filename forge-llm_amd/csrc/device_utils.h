@@ -57,7 +57,9 @@ __device__ __forceinline__ float wave_max(float v) {
 
 // Quantise 4 consecutive floats held by each of 8 consecutive lanes (one 32-element block).
 // Returns the packed 4 int8 codes; lane%8==0 also gets the fp16 scale bits via `scale_bits`.
-__device__ __forceinline__ uint32_t quantize_block_part(float4 v, uint16_t& scale_bits) {
+// `negate`: store -code instead of code (the scale stays positive): the fast prefill GEMM wants the odd blocks of a row
+// that way (gemm.hip).
+__device__ __forceinline__ uint32_t quantize_block_part(float4 v, uint16_t& scale_bits, bool negate = false) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = fmaxf(amax, __shfl_xor(amax, 1, WAVE));
     amax = fmaxf(amax, __shfl_xor(amax, 2, WAVE));
@@ -65,6 +67,7 @@ __device__ __forceinline__ uint32_t quantize_block_part(float4 v, uint16_t& scal
     float inv;
     float s = act_scale(amax, inv);
     scale_bits = f32_to_f16_bits(s);
+    if (negate) inv = -inv;          // rounding and clamping are symmetric: round(-x) = -round(x)
     uint32_t q0 = (uint32_t)quant_code(v.x * inv) & 0xFFu;
     uint32_t q1 = (uint32_t)quant_code(v.y * inv) & 0xFFu;
     uint32_t q2 = (uint32_t)quant_code(v.z * inv) & 0xFFu;

@@ -10,23 +10,25 @@ namespace fh {
 
 // ---- quantize_to_q8_0_blocks_into (emit.rs:1410-1440), planes instead of 34-byte blocks ----
 __global__ __launch_bounds__(256) void quantize_act_kernel(const float* __restrict__ x, uint64_t n4,
-                                                           uint32_t* __restrict__ q, uint16_t* __restrict__ sc) {
+                                                           uint32_t* __restrict__ q, uint16_t* __restrict__ sc,
+                                                           uint32_t neg_odd_blocks_per_row) {
     uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
     if (i < n4) v = reinterpret_cast<const float4*>(x)[i];
     uint16_t sb;
-    uint32_t packed = quantize_block_part(v, sb);
+    const bool neg = neg_odd_blocks_per_row != 0 && (((i >> 3) % neg_odd_blocks_per_row) & 1) != 0;
+    uint32_t packed = quantize_block_part(v, sb, neg);
     if (i < n4) {
         q[i] = packed;
         if ((i & 7) == 0) sc[i >> 3] = sb;
     }
 }
 
-void launch_quantize_act(const float* x, uint32_t M, uint32_t K, int8_t* q, uint16_t* sc, hipStream_t s) {
+void launch_quantize_act(const float* x, uint32_t M, uint32_t K, int8_t* q, uint16_t* sc, hipStream_t s, bool neg_odd) {
     uint64_t n4 = (uint64_t)M * K / 4;
     if (n4 == 0) return;
     uint32_t grid = (uint32_t)((n4 + 255) / 256);
-    fh::launch(quantize_act_kernel, grid, 256, 0, s, x, n4, reinterpret_cast<uint32_t*>(q), sc);
+    fh::launch(quantize_act_kernel, grid, 256, 0, s, x, n4, reinterpret_cast<uint32_t*>(q), sc, neg_odd ? K / 32 : 0u);
 }
 
 // ---- rms_norm (emit.rs:327-334) + optional block quantisation -------------------------------
@@ -36,7 +38,7 @@ void launch_quantize_act(const float* x, uint32_t M, uint32_t K, int8_t* q, uint
 // then the H mod 16 tail added in order.  inv = 1/sqrt(ss/n + eps), out = (x*inv)*w.
 __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w,
                                                       float eps, uint32_t H, float* __restrict__ normed,
-                                                      uint32_t* __restrict__ q, uint16_t* __restrict__ sc) {
+                                                      uint32_t* __restrict__ q, uint16_t* __restrict__ sc, uint32_t neg_odd) {
     extern __shared__ float xs[];          // the row, then 16 partial sums, then the result
     const uint32_t row = blockIdx.x, tid = threadIdx.x;
     const float4* xr = reinterpret_cast<const float4*>(x + (size_t)row * H);
@@ -80,7 +82,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
         }
         if (q) {
             uint16_t sb;
-            uint32_t packed = quantize_block_part(o, sb);
+            uint32_t packed = quantize_block_part(o, sb, neg_odd != 0 && ((i >> 3) & 1) != 0);
             if (i < n4) {
                 q[(size_t)row * n4 + i] = packed;
                 if ((i & 7) == 0) sc[(size_t)row * (H / 32) + (i >> 3)] = sb;
@@ -90,18 +92,19 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
 }
 
 void launch_rmsnorm(const float* x, const float* w, float eps, uint32_t M, uint32_t H, float* normed, int8_t* q,
-                    uint16_t* sc, hipStream_t s) {
+                    uint16_t* sc, hipStream_t s, bool neg_odd) {
     if (M == 0) return;
-    fh::launch(rmsnorm_kernel, M, 256, (H + 32) * sizeof(float), s, x, w, eps, H, normed, reinterpret_cast<uint32_t*>(q), sc);
+    fh::launch(rmsnorm_kernel, M, 256, (H + 32) * sizeof(float), s, x, w, eps, H, normed, reinterpret_cast<uint32_t*>(q), sc, neg_odd ? 1u : 0u);
 }
 
 // ---- silu_mul (emit.rs:380-386) + optional block quantisation --------------------------------
 __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__ gate, const float* __restrict__ up,
                                                        uint32_t I4, uint32_t row_stride, uint64_t total4,
                                                        float* __restrict__ out, uint32_t* __restrict__ q,
-                                                       uint16_t* __restrict__ sc) {
+                                                       uint16_t* __restrict__ sc, uint32_t neg_odd) {
     uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+    const bool neg = neg_odd != 0 && (((i % I4) >> 3) & 1) != 0;
     if (i < total4) {
         uint64_t r = i / I4, c = i % I4;
         float4 g = reinterpret_cast<const float4*>(gate + r * row_stride)[c];
@@ -115,7 +118,7 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
     }
     if (q) {
         uint16_t sb;
-        uint32_t packed = quantize_block_part(o, sb);
+        uint32_t packed = quantize_block_part(o, sb, neg);
         if (i < total4) {
             q[i] = packed;
             if ((i & 7) == 0) sc[i >> 3] = sb;
@@ -124,11 +127,11 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
 }
 
 void launch_silu_mul(const float* gate, const float* up, uint32_t M, uint32_t I, uint32_t row_stride, float* out,
-                     int8_t* q, uint16_t* sc, hipStream_t s) {
+                     int8_t* q, uint16_t* sc, hipStream_t s, bool neg_odd) {
     uint64_t total4 = (uint64_t)M * I / 4;
     if (total4 == 0) return;
     uint32_t grid = (uint32_t)((total4 + 255) / 256);
-    fh::launch(silu_mul_kernel, grid, 256, 0, s, gate, up, I / 4, row_stride, total4, out, reinterpret_cast<uint32_t*>(q), sc);
+    fh::launch(silu_mul_kernel, grid, 256, 0, s, gate, up, I / 4, row_stride, total4, out, reinterpret_cast<uint32_t*>(q), sc, neg_odd ? 1u : 0u);
 }
 
 // ---- rope (emit.rs:508-528) + fp16 KV write ------------------------------------------------------

@@ -13,8 +13,9 @@
 // 64 cycles of MFMA), so the fast mode halves it by never converting: the integer MFMA starts from
 // C = 0x4B400000 in every element, which makes its int32 result, read as f32, the number 12582912 + isum
 // exactly (|isum| <= 516128 < 2^22), and one FMA per element adds S * (12582912 + isum).  To keep the
-// accumulators near their true size the bias alternates in sign: in odd blocks the activation codes are
-// negated before the MFMA and the weight scale carries a minus sign, which adds S * (isum - 12582912).  What
+// accumulators near their true size the bias alternates in sign: in odd blocks the activation codes come
+// negated (the quantising kernels store them so for this kernel: no work here) and the weight scale carries a
+// minus sign, which adds S * (isum - 12582912).  What
 // is left of the bias after 8 blocks, 12582912 * sum_b (+-)S_b, is itself a product of the scales: one more
 // f16 MFMA (k = the 8 blocks) gives it, and one FMA per element takes it out.  Block sums stay exact; the
 // f32 accumulation carries a rounding error of about 2e-5 of the typical output (measured; 1e-7 in the
@@ -57,12 +58,6 @@ constexpr uint32_t OOB = 0x80000000u;         // an offset no descriptor here co
 
 #define FH_LDS3(p) ((__attribute__((address_space(3))) void*)(p))
 
-// -x for each of four int8 codes (none is -128).
-__device__ __forceinline__ uint32_t neg4(uint32_t x) {
-    const uint32_t y = ~x;
-    return ((y & 0x7F7F7F7Fu) + 0x01010101u) ^ (y & 0x80808080u);
-}
-
 // (c - 8) for each of four nibble codes c held in the low nibbles of the four bytes.
 __device__ __forceinline__ uint32_t nib_minus8(uint32_t x) {
     return ((x | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
@@ -88,11 +83,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     const uint32_t lrow = lane & 31, lhalf = lane >> 5;
     const uint32_t wrow = Q4 ? K / 2 : K;   // bytes of one weight row
 
-    const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc((void*)aq, 0, M * K, RSRC_FLAGS);
-    const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void*)wq, 0, N * wrow, RSRC_FLAGS);
-    const __amdgpu_buffer_rsrc_t ras = __builtin_amdgcn_make_buffer_rsrc((void*)asc, 0, M * nblk * 2, RSRC_FLAGS);
     const __amdgpu_buffer_rsrc_t rdump = __builtin_amdgcn_make_buffer_rsrc((void*)isums, 0, DUMP ? M * N * nblk * 4 : 0, RSRC_FLAGS);
-    const __amdgpu_buffer_rsrc_t rws = __builtin_amdgcn_make_buffer_rsrc((void*)wsc, 0, N * nblk * 2, RSRC_FLAGS);
 
     // ---- loader mapping: load i of wave w fills LDS rows (4i + w) * 8 .. + 8 of a tile, lane -> (row, position)
     const uint32_t ld_row = wave * 8 + (lane >> 3);                        // + 32 i
@@ -110,24 +101,37 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     v4i rb[2];
     uint32_t rs[KB];
 
+    // The K position of a stage moves the descriptors (scalar work: base + k0, records - k0), not the lanes' offsets: the
+    // range check still sees the whole offset (a scalar offset operand would be left out of it), and the per-lane
+    // offsets stay the same from stage to stage.
     auto issue_stage = [&](uint32_t k0, uint32_t buf) {
+        const uint32_t kq = Q4 ? k0 / 2 : k0, ks = (k0 / 32) * 2;
+        // 0 records: every access is out of range.  (readfirstlane: the value is uniform, and a descriptor word in a
+        // vector register would cost a loop over its values around every load.)
+        auto left = [](uint32_t total, uint32_t skip) {
+            return (uint32_t)__builtin_amdgcn_readfirstlane((int)(total > skip ? total - skip : 0u));
+        };
+        const __amdgpu_buffer_rsrc_t ra_k = __builtin_amdgcn_make_buffer_rsrc((void*)(aq + k0), 0, left(M * K, k0), RSRC_FLAGS);
+        const __amdgpu_buffer_rsrc_t rw_k = __builtin_amdgcn_make_buffer_rsrc((void*)(wq + kq), 0, left(N * wrow, kq), RSRC_FLAGS);
+        const __amdgpu_buffer_rsrc_t ras_k = __builtin_amdgcn_make_buffer_rsrc((void*)((const uint8_t*)asc + ks), 0, left(M * nblk * 2, ks), RSRC_FLAGS);
+        const __amdgpu_buffer_rsrc_t rws_k = __builtin_amdgcn_make_buffer_rsrc((void*)((const uint8_t*)wsc + ks), 0, left(N * nblk * 2, ks), RSRC_FLAGS);
 #pragma unroll
         for (int i = 0; i < 2 * TM; i++)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, FH_LDS3(lds + LDS_A + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
-                                                     a_voff + i * 32 * K + k0, 0, 0, 0);
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra_k, FH_LDS3(lds + LDS_A + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
+                                                     a_voff + i * 32 * K, 0, 0, 0);
         if (Q4) {
 #pragma unroll
-            for (int i = 0; i < 2; i++) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rw, q4_voff + i * 64 * nblk * 16 + (k0 / 32) * 16, 0, 0);
+            for (int i = 0; i < 2; i++) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rw_k, q4_voff + i * 64 * nblk * 16, 0, 0);
         } else {
 #pragma unroll
             for (int i = 0; i < 4; i++)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, FH_LDS3(lds + LDS_B + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
-                                                         w_voff + i * 32 * K + k0, 0, 0, 0);
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rw_k, FH_LDS3(lds + LDS_B + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
+                                                         w_voff + i * 32 * K, 0, 0, 0);
         }
 #pragma unroll
         for (int b = 0; b < KB; b++) {
-            const uint32_t v = sc_is_a ? __builtin_amdgcn_raw_buffer_load_b16(ras, sc_voff + b * 2 + (k0 / 32) * 2, 0, 0)
-                                       : __builtin_amdgcn_raw_buffer_load_b16(rws, sc_voff + b * 2 + (k0 / 32) * 2, 0, 0);
+            const uint32_t v = sc_is_a ? __builtin_amdgcn_raw_buffer_load_b16(ras_k, sc_voff + b * 2, 0, 0)
+                                       : __builtin_amdgcn_raw_buffer_load_b16(rws_k, sc_voff + b * 2, 0, 0);
             rs[b] = v;              // looked at only when the stage is committed: nothing at the start of a stage waits for it
         }
     };
@@ -207,10 +211,6 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         for (int t = 0; t < TM; t++) {
             f.af[t] = *reinterpret_cast<const v4i*>(A + ((fa_off ^ (kb * 32)) + t * 32 * BK));
             f.sa[t] = *reinterpret_cast<const uint16_t*>(lds + sa_off + slot * s_slot_stride + t * s_t_stride + kb * 2);
-            if (MAGIC && (kb & 1)) {
-                f.af[t].x = (int)neg4((uint32_t)f.af[t].x); f.af[t].y = (int)neg4((uint32_t)f.af[t].y);
-                f.af[t].z = (int)neg4((uint32_t)f.af[t].z); f.af[t].w = (int)neg4((uint32_t)f.af[t].w);
-            }
         }
     };
     auto scale_operand = [](uint32_t bits) {

@@ -246,8 +246,8 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
     float* attn = m->pattn.as<float>();
     int8_t* aq = m->paq.as<int8_t>();
     uint16_t* asc = m->pasc.as<uint16_t>();
-    const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
-    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
+    const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;      // the fast GEMM takes the odd blocks of its activations negated
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s, !exact); }
     { StageMark t(m, ST_QKV); launch_gemm(L.qkv, aq, asc, M, qkv, QKV, false, exact, nullptr, s); }
     {
         StageMark t(m, ST_ROPE);
@@ -260,15 +260,15 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
     } else if (m->prefill_fuse_quant) {
         // the attention kernel writes the o projection's quantised input itself
         StageMark t(m, ST_ATTN);
-        launch_attn_prefill_quant(qkv, QKV, m->kc(l), m->vc(l), aq, asc, M, base_pos, c.heads, c.kv_heads, c.head_dim, c.sliding_window, s);
+        launch_attn_prefill_quant(qkv, QKV, m->kc(l), m->vc(l), aq, asc, M, base_pos, c.heads, c.kv_heads, c.head_dim, c.sliding_window, s, true);
     } else {
         { StageMark t(m, ST_ATTN); launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, c.sliding_window, s); }
-        { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
+        { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s, true); }
     }
     { StageMark t(m, ST_O); launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s); }
-    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s, !exact); }
     { StageMark t(m, ST_GATE_UP); launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s); }
-    { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s); }
+    { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s, !exact); }
     { StageMark t(m, ST_DOWN); launch_gemm(L.down, aq, asc, M, x, H, true, exact, nullptr, s); }
 }
 
