@@ -326,18 +326,72 @@ pub fn sample(logits: &mut [f32], temperature: f32, top_k: usize, top_p: f32, rn
 "#;
 
 const MAIN_RS: &str = r#"//! @MODEL_NAME@ on AMD MI355X through libforge_hip.  Generated by forgellm-codegen-hip.
+//!
+//! Same command line as the binaries of the other ForgeLLM backends (flags, defaults, what goes to stdout and what to
+//! stderr); the first argument may also be a GGUF file.
 mod model;
 
 use std::io::Write;
+use std::time::Instant;
 
 use model::{apply_repeat_penalty, sample, HipModel};
 
-fn parse_f32_arg(args: &[String], flag: &str, default: f32) -> f32 {
-    args.windows(2).find(|w| w[0] == flag).and_then(|w| w[1].parse::<f32>().ok()).unwrap_or(default)
+/// Everything the command line can say.  Defaults are those of the CPU backend's binary.
+struct Options {
+    weights: String,
+    tokenizer: String,
+    prompt: String,
+    temperature: f32,
+    top_k: usize,
+    top_p: f32,
+    max_tokens: usize,
+    repeat_penalty: f32,
+    seed: u64,
+    quiet: bool,
 }
 
-fn parse_usize_arg(args: &[String], flag: &str, default: usize) -> usize {
-    args.windows(2).find(|w| w[0] == flag).and_then(|w| w[1].parse::<usize>().ok()).unwrap_or(default)
+const USAGE_FLAGS: &str = "[prompt] [--temp T] [--top-k K] [--top-p P] [--max-tokens N] [--repeat-penalty R] [--seed S] [--quiet]";
+
+impl Options {
+    /// One pass over the arguments after the two paths: `--flag value` pairs fill their field (a value that does not parse
+    /// leaves the default), `--quiet` / `-q` is a switch, any other dash argument is skipped, the rest is the prompt.
+    fn from_args(args: &[String]) -> Options {
+        let mut o = Options {
+            weights: args[1].clone(),
+            tokenizer: args[2].clone(),
+            prompt: String::new(),
+            temperature: 0.0,
+            top_k: 0,
+            top_p: 0.9,
+            max_tokens: 128,
+            repeat_penalty: 1.1,
+            seed: 0xdeadbeef12345678,
+            quiet: false,
+        };
+        let mut words: Vec<&str> = Vec::new();
+        let mut rest = args[3..].iter();
+        while let Some(arg) = rest.next() {
+            match arg.as_str() {
+                "--quiet" | "-q" => o.quiet = true,
+                "--temp" => set(&mut o.temperature, rest.next()),
+                "--top-k" => set(&mut o.top_k, rest.next()),
+                "--top-p" => set(&mut o.top_p, rest.next()),
+                "--max-tokens" => set(&mut o.max_tokens, rest.next()),
+                "--repeat-penalty" => set(&mut o.repeat_penalty, rest.next()),
+                "--seed" => set(&mut o.seed, rest.next()),
+                other if other.starts_with('-') => {}
+                word => words.push(word),
+            }
+        }
+        o.prompt = if words.is_empty() { "Hello".to_string() } else { words.join(" ") };
+        o
+    }
+}
+
+fn set<T: std::str::FromStr>(field: &mut T, value: Option<&String>) {
+    if let Some(v) = value.and_then(|v| v.parse::<T>().ok()) {
+        *field = v;
+    }
 }
 
 fn main() {
@@ -347,101 +401,73 @@ fn main() {
         return;
     }
     if args.len() < 3 {
-        eprintln!("Usage: {} <weights.bin | model.gguf> <tokenizer.json> [prompt] [--temp T] [--top-k K] [--top-p P] [--max-tokens N] [--repeat-penalty R] [--seed S] [--quiet]", args[0]);
+        eprintln!("Usage: {} <weights.bin | model.gguf> <tokenizer.json> {}", args[0], USAGE_FLAGS);
         eprintln!("AOT-compiled @ARCH@ | @LAYERS@ layers | hidden=@HIDDEN@ | HIP (gfx950)");
         std::process::exit(1);
     }
-    let weights_path = &args[1];
-    let tokenizer_path = &args[2];
-    let temperature = parse_f32_arg(&args, "--temp", 0.0);
-    let top_k = parse_usize_arg(&args, "--top-k", 0);
-    let top_p = parse_f32_arg(&args, "--top-p", 0.9);
-    let max_tokens = parse_usize_arg(&args, "--max-tokens", 128);
-    let repeat_penalty = parse_f32_arg(&args, "--repeat-penalty", 1.1);
-    let seed = args.windows(2).find(|w| w[0] == "--seed").and_then(|w| w[1].parse::<u64>().ok()).unwrap_or(0xdeadbeef12345678);
-    let quiet = args.iter().any(|a| a == "--quiet" || a == "-q");
-    let prompt = {
-        let value_flags = ["--temp", "--top-k", "--top-p", "--max-tokens", "--repeat-penalty", "--seed"];
-        let mut parts: Vec<String> = Vec::new();
-        let mut i = 3;
-        while i < args.len() {
-            let a = &args[i];
-            if value_flags.contains(&a.as_str()) {
-                i += 2;
-                continue;
-            }
-            if a.starts_with('-') {
-                i += 1;
-                continue;
-            }
-            parts.push(a.clone());
-            i += 1;
-        }
-        parts.join(" ")
-    };
-    let prompt = if prompt.is_empty() { "Hello".to_string() } else { prompt };
-
+    let opt = Options::from_args(&args);
     if model::device_count() < 1 {
         eprintln!("no AMD GPU visible to HIP");
         std::process::exit(1);
     }
-    let tokenizer = tokenizers::Tokenizer::from_file(tokenizer_path).expect("failed to load tokenizer");
-    let mut m = if weights_path.ends_with(".gguf") {
-        HipModel::from_gguf(weights_path)
+    let tokenizer = tokenizers::Tokenizer::from_file(&opt.tokenizer).expect("failed to load tokenizer");
+    let mut gpu = if opt.weights.ends_with(".gguf") {
+        HipModel::from_gguf(&opt.weights)
     } else {
-        let bytes = std::fs::read(weights_path).expect("failed to read weights");
-        HipModel::new(&bytes)
+        HipModel::new(&std::fs::read(&opt.weights).expect("failed to read weights"))
     };
 
-    let enc = tokenizer.encode(prompt.as_str(), false).expect("encode failed");
-    let prompt_tokens: Vec<u32> = enc.get_ids().to_vec();
-    eprintln!("Prompt: {} tokens | temp={} top_k={} max_tokens={}", prompt_tokens.len(), temperature, top_k, max_tokens);
+    let prompt_ids: Vec<u32> = tokenizer.encode(opt.prompt.as_str(), false).expect("encode failed").get_ids().to_vec();
+    eprintln!("Prompt: {} tokens | temp={} top_k={} max_tokens={}", prompt_ids.len(), opt.temperature, opt.top_k, opt.max_tokens);
 
-    let t0 = std::time::Instant::now();
-    let mut rng_state: u64 = seed;
-    let mut logits = m.forward_prefill(&prompt_tokens);
-    let mut next = sample(&mut logits, temperature, top_k, top_p, &mut rng_state);
-    eprintln!("Prefill: {:.1} tok/s", prompt_tokens.len() as f64 / t0.elapsed().as_secs_f64());
+    // prompt in one batched pass; the first token is sampled from its logits without a penalty
+    let mut rng = opt.seed;
+    let started = Instant::now();
+    let mut first_logits = gpu.forward_prefill(&prompt_ids);
+    let first = sample(&mut first_logits, opt.temperature, opt.top_k, opt.top_p, &mut rng);
+    eprintln!("Prefill: {:.1} tok/s", prompt_ids.len() as f64 / started.elapsed().as_secs_f64());
 
-    if !quiet {
-        print!("{}", prompt);
+    if !opt.quiet {
+        print!("{}", opt.prompt);
     }
-    let t1 = std::time::Instant::now();
-    let eos_tokens: Vec<u32> = ["</s>", "<|endoftext|>", "<|im_end|>", "<|eot_id|>"]
-        .iter()
-        .filter_map(|t| tokenizer.token_to_id(t))
-        .collect();
-    // Greedy decoding keeps the whole loop on the GPU: the library counts every token it is fed and takes the argmax over the
-    // penalised logits itself, so 4 bytes per token come back.  With a temperature the logits come back and are sampled here.
-    let greedy = temperature <= 0.0;
-    if greedy {
-        m.set_repeat_penalty(repeat_penalty);
-    }
-    let mut recent_tokens: Vec<u32> = prompt_tokens.clone();
-    let mut gen_count = 0usize;
-    for _ in 0..max_tokens {
-        if eos_tokens.contains(&next) {
-            break;
-        }
-        if !quiet {
-            let text = tokenizer.decode(&[next], true).unwrap_or_default();
-            print!("{}", text);
-            std::io::stdout().flush().ok();
-        }
-        recent_tokens.push(next);
-        if greedy {
-            next = m.forward_greedy(next);
-        } else {
-            let mut l = m.forward(next);
-            apply_repeat_penalty(&mut l, &recent_tokens, repeat_penalty);
-            next = sample(&mut l, temperature, top_k, top_p, &mut rng_state);
-        }
-        gen_count += 1;
-    }
-    if !quiet {
+    let started = Instant::now();
+    let produced = generate(&mut gpu, &tokenizer, &opt, prompt_ids, first, &mut rng);
+    if !opt.quiet {
         println!();
     }
-    eprintln!("Generate: {} tokens in {:.2}s ({:.1} tok/s)", gen_count, t1.elapsed().as_secs_f64(), gen_count as f64 / t1.elapsed().as_secs_f64());
+    let secs = started.elapsed().as_secs_f64();
+    eprintln!("Generate: {} tokens in {:.2}s ({:.1} tok/s)", produced, secs, produced as f64 / secs);
+}
+
+/// Feeds `token`, then whatever is chosen next, until an end-of-sequence id or `max_tokens`; returns how many were fed.
+/// With temperature <= 0 the choice stays on the GPU: the library counts every token it has been fed (the prompt's too) and
+/// takes the argmax of the penalised logits itself, so 4 bytes per token come back.  Otherwise the logits come back and the
+/// penalty over all tokens so far and the sampler run here.
+fn generate(gpu: &mut HipModel, tokenizer: &tokenizers::Tokenizer, opt: &Options, prompt_ids: Vec<u32>, first: u32, rng: &mut u64) -> usize {
+    let stop: Vec<u32> = ["</s>", "<|endoftext|>", "<|im_end|>", "<|eot_id|>"].iter().filter_map(|t| tokenizer.token_to_id(t)).collect();
+    let on_gpu = opt.temperature <= 0.0;
+    if on_gpu {
+        gpu.set_repeat_penalty(opt.repeat_penalty);
+    }
+    let mut seen = prompt_ids;
+    let mut token = first;
+    let mut fed = 0usize;
+    while fed < opt.max_tokens && !stop.contains(&token) {
+        if !opt.quiet {
+            print!("{}", tokenizer.decode(&[token], true).unwrap_or_default());
+            std::io::stdout().flush().ok();
+        }
+        seen.push(token);
+        token = if on_gpu {
+            gpu.forward_greedy(token)
+        } else {
+            let mut logits = gpu.forward(token);
+            apply_repeat_penalty(&mut logits, &seen, opt.repeat_penalty);
+            sample(&mut logits, opt.temperature, opt.top_k, opt.top_p, rng)
+        };
+        fed += 1;
+    }
+    fed
 }
 "#;
 

@@ -136,6 +136,10 @@ void launch_gemv_norm_silu_quant(const QWeight& wgu, const float* x, const float
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
                  bool accumulate, bool exact, int32_t* isums, hipStream_t s);
 
+// model.hip — the part of forge_hip_model_create's checks that sizes depend on (formats, dimensions the kernels cover);
+// sets the error message.
+int32_t validate_config_shape(const forge_hip_config* c);
+
 // attn_decode.hip
 constexpr uint32_t DECODE_SPLITS = 32;
 size_t attn_decode_workspace_bytes(uint32_t heads, uint32_t hd);

@@ -18,6 +18,7 @@
 #include <map>
 #include <memory>
 #include <new>
+#include <stdexcept>
 
 #include "common.h"
 
@@ -48,6 +49,9 @@ struct MetaValue {
     uint32_t elem_type = 0;      // type 9
     uint64_t count = 0;          // type 9: number of elements (elements themselves are skipped, only counted)
 };
+
+// No tensor of a real file comes near this; below it, element counts times bytes per block cannot wrap 64 bits.
+constexpr uint64_t MAX_TENSOR_ELEMENTS = 1ull << 48;
 
 struct TensorInfo {
     std::string name;
@@ -207,6 +211,14 @@ int32_t parse_into(forge_hip_gguf* g) {
         if (r.ok && t.n_dims > 4)
             return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor dimension count " + std::to_string(t.n_dims) + " exceeds maximum (4)");
         for (uint32_t d = 0; d < t.n_dims; d++) t.dims[d] = r.get<uint64_t>();
+        {
+            // the sizes below are products of these: refuse what no file can hold before anything multiplies them
+            uint64_t n = 1;
+            bool over = false;
+            for (uint32_t d = 0; d < t.n_dims; d++) over = over || __builtin_mul_overflow(n, t.dims[d], &n);
+            if (r.ok && (over || n > MAX_TENSOR_ELEMENTS))
+                return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor " + t.name + " has more than 2^48 elements");
+        }
         t.type = r.get<uint32_t>();
         t.offset = r.get<uint64_t>();
         if (!r.ok) return fail(FORGE_HIP_ERR_INVALID, "gguf: file ends inside the tensor descriptors");
@@ -414,44 +426,60 @@ int32_t write_f32(const forge_hip_gguf* g, const std::string& name, uint64_t num
 
 }  // namespace
 
+// An allocation that fails (a vector sized from a damaged or hostile file) must not leave through the C boundary.
+template <typename F>
+int32_t no_throw(const char* name, F&& body) {
+    try {
+        return body();
+    } catch (const std::bad_alloc&) {
+        return fh::fail(FORGE_HIP_ERR_INVALID, std::string(name) + ": out of host memory");
+    } catch (const std::length_error&) {
+        return fh::fail(FORGE_HIP_ERR_INVALID, std::string(name) + ": a size in the file is too large");
+    }
+}
+
 extern "C" {
 
 int32_t forge_hip_gguf_parse(const uint8_t* data_host, uint64_t nbytes, forge_hip_gguf** out) {
-    FH_CHECK(out, "gguf_parse: null out");
-    *out = nullptr;
-    FH_CHECK(data_host || nbytes == 0, "gguf_parse: null data");
-    std::unique_ptr<forge_hip_gguf> g(new forge_hip_gguf());
-    g->data = data_host;
-    g->nbytes = nbytes;
-    const int32_t rc = parse_into(g.get());
-    if (rc) return rc;
-    *out = g.release();
-    return FORGE_HIP_OK;
+    return no_throw("gguf_parse", [&]() -> int32_t {
+        FH_CHECK(out, "gguf_parse: null out");
+        *out = nullptr;
+        FH_CHECK(data_host || nbytes == 0, "gguf_parse: null data");
+        std::unique_ptr<forge_hip_gguf> g(new forge_hip_gguf());
+        g->data = data_host;
+        g->nbytes = nbytes;
+        const int32_t rc = parse_into(g.get());
+        if (rc) return rc;
+        *out = g.release();
+        return FORGE_HIP_OK;
+    });
 }
 
 int32_t forge_hip_gguf_open(const char* path, forge_hip_gguf** out) {
-    FH_CHECK(out, "gguf_open: null out");
-    *out = nullptr;
-    FH_CHECK(path, "gguf_open: null path");
-    const int fd = open(path, O_RDONLY);
-    if (fd < 0) return fh::fail(FORGE_HIP_ERR_INVALID, std::string("gguf_open: cannot open ") + path + ": " + strerror(errno));
-    struct stat st;
-    if (fstat(fd, &st) != 0 || st.st_size <= 0) {
+    return no_throw("gguf_open", [&]() -> int32_t {
+        FH_CHECK(out, "gguf_open: null out");
+        *out = nullptr;
+        FH_CHECK(path, "gguf_open: null path");
+        const int fd = open(path, O_RDONLY);
+        if (fd < 0) return fh::fail(FORGE_HIP_ERR_INVALID, std::string("gguf_open: cannot open ") + path + ": " + strerror(errno));
+        struct stat st;
+        if (fstat(fd, &st) != 0 || st.st_size <= 0) {
+            close(fd);
+            return fh::fail(FORGE_HIP_ERR_INVALID, std::string("gguf_open: cannot read ") + path);
+        }
+        void* map = mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
         close(fd);
-        return fh::fail(FORGE_HIP_ERR_INVALID, std::string("gguf_open: cannot read ") + path);
-    }
-    void* map = mmap(nullptr, (size_t)st.st_size, PROT_READ, MAP_PRIVATE, fd, 0);
-    close(fd);
-    if (map == MAP_FAILED) return fh::fail(FORGE_HIP_ERR_INVALID, std::string("gguf_open: cannot map ") + path + ": " + strerror(errno));
-    std::unique_ptr<forge_hip_gguf> g(new forge_hip_gguf());
-    g->map = map;
-    g->map_len = (uint64_t)st.st_size;
-    g->data = reinterpret_cast<const uint8_t*>(map);
-    g->nbytes = g->map_len;
-    const int32_t rc = parse_into(g.get());
-    if (rc) return rc;
-    *out = g.release();
-    return FORGE_HIP_OK;
+        if (map == MAP_FAILED) return fh::fail(FORGE_HIP_ERR_INVALID, std::string("gguf_open: cannot map ") + path + ": " + strerror(errno));
+        std::unique_ptr<forge_hip_gguf> g(new forge_hip_gguf());
+        g->map = map;
+        g->map_len = (uint64_t)st.st_size;
+        g->data = reinterpret_cast<const uint8_t*>(map);
+        g->nbytes = g->map_len;
+        const int32_t rc = parse_into(g.get());
+        if (rc) return rc;
+        *out = g.release();
+        return FORGE_HIP_OK;
+    });
 }
 
 void forge_hip_gguf_close(forge_hip_gguf* g) { delete g; }
@@ -497,165 +525,182 @@ int32_t forge_hip_gguf_meta(const forge_hip_gguf* g, const char* key, uint32_t* 
 }
 
 int32_t forge_hip_dequant_ggml(uint32_t ggml_type, const uint8_t* data_host, uint64_t n, float* out_host) {
-    FH_CHECK(data_host && out_host, "dequant_ggml: null pointer");
-    if (!dequant_ggml(ggml_type, data_host, n, out_host))
-        return fh::fail(FORGE_HIP_ERR_INVALID, "dequant_ggml: GGML type " + std::to_string(ggml_type) + " is not one of " + SUPPORTED_TYPES);
-    return FORGE_HIP_OK;
+    return no_throw("dequant_ggml", [&]() -> int32_t {
+        FH_CHECK(data_host && out_host, "dequant_ggml: null pointer");
+        if (!dequant_ggml(ggml_type, data_host, n, out_host))
+            return fh::fail(FORGE_HIP_ERR_INVALID, "dequant_ggml: GGML type " + std::to_string(ggml_type) + " is not one of " + SUPPORTED_TYPES);
+        return FORGE_HIP_OK;
+    });
 }
 
 int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_t flags, forge_hip_config* out) {
-    FH_CHECK(g && out, "gguf_config: null argument");
-    const MetaValue* arch_v = g->find("general.architecture");
-    const std::string arch = arch_v && arch_v->type == 8 ? arch_v->str : "unknown";
-    // The kernels here cover the Llama layer, with the QKV bias of Qwen2 (main.rs:770: the bias goes with the
-    // architecture): no GeLU or embedding scale (gemma).  Mistral is the Llama layer plus an optional sliding window;
-    // Phi-3 is the Llama layer with fused tensors in the file, which export_weights splits (main.rs:759).
-    if (arch != "llama" && arch != "mistral" && arch != "qwen2" && arch != "phi3" && arch != "phi")
-        return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: unsupported GGUF architecture: " + arch);
-    const std::string p = arch + ".";
-    uint32_t hidden = 0, layers = 0, heads = 0, kv_heads = 0, inter = 0;
-    g->get_u32(p + "embedding_length", &hidden);
-    g->get_u32(p + "block_count", &layers);
-    g->get_u32(p + "attention.head_count", &heads);
-    if (!g->get_u32(p + "attention.head_count_kv", &kv_heads)) kv_heads = heads;
-    if (hidden == 0 || layers == 0 || heads == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: could not extract model config from GGUF metadata");
-    if (!g->get_u32(p + "feed_forward_length", &inter)) inter = hidden * 4;
-    uint64_t vocab = 32000, ctx = 2048;
-    const MetaValue* tokens = g->find("tokenizer.ggml.tokens");
-    if (tokens && tokens->type == 9) vocab = tokens->count;
-    else g->get_u64(p + "vocab_size", &vocab);
-    g->get_u64(p + "context_length", &ctx);
-    float eps = 1e-5f, theta = 10000.0f;
-    g->get_f32(p + "attention.layer_norm_rms_epsilon", &eps);
-    g->get_f32(p + "rope.freq_base", &theta);
-    uint32_t window = 0;
-    const bool has_window = g->get_u32(p + "attention.sliding_window", &window);
-
-    // majority vote over the projection tensors (main.rs:479-555)
-    uint64_t q8 = 0, q4 = 0, q4k = 0, f16 = 0, f32 = 0;
-    for (const auto& t : g->tensors) {
-        const std::string& n = t.name;
-        const bool proj = n.find(".weight") != std::string::npos && n.find("token_embd") == std::string::npos &&
-                          n.find("output.weight") == std::string::npos && n.find("_norm") == std::string::npos;
-        if (!proj) continue;
-        switch (t.type) {
-            case T_Q8_0: q8++; break;
-            case T_Q4_0: q4++; break;
-            case 12: q4k++; break;
-            case T_F16: case T_BF16: f16++; break;
-            case T_F32: f32++; break;
-            case 3: case 20: case 23: case 6: case 7: case 9: case 10: case 11: case 13: case 14: case 15: case 16: case 17: case 22:
-            case 18: case 21: case 19: case 29: q8++; break;
-            default: break;
+    return no_throw("gguf_config", [&]() -> int32_t {
+        FH_CHECK(g && out, "gguf_config: null argument");
+        const MetaValue* arch_v = g->find("general.architecture");
+        const std::string arch = arch_v && arch_v->type == 8 ? arch_v->str : "unknown";
+        // The kernels here cover the Llama layer, with the QKV bias of Qwen2 (main.rs:770: the bias goes with the
+        // architecture): no GeLU or embedding scale (gemma).  Mistral is the Llama layer plus an optional sliding window;
+        // Phi-3 is the Llama layer with fused tensors in the file, which export_weights splits (main.rs:759).
+        if (arch != "llama" && arch != "mistral" && arch != "qwen2" && arch != "phi3" && arch != "phi")
+            return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: unsupported GGUF architecture: " + arch);
+        const std::string p = arch + ".";
+        uint32_t hidden = 0, layers = 0, heads = 0, kv_heads = 0, inter = 0;
+        g->get_u32(p + "embedding_length", &hidden);
+        g->get_u32(p + "block_count", &layers);
+        g->get_u32(p + "attention.head_count", &heads);
+        if (!g->get_u32(p + "attention.head_count_kv", &kv_heads)) kv_heads = heads;
+        if (hidden == 0 || layers == 0 || heads == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: could not extract model config from GGUF metadata");
+    if (!g->get_u32(p + "feed_forward_length", &inter)) {
+            FH_CHECK(hidden <= 0x3FFFFFFFu, "gguf: embedding_length out of range");
+            inter = hidden * 4;
         }
-    }
-    const uint64_t total = q8 + q4 + q4k + f16 + f32;
-    uint32_t wdtype = 0;
-    if (total && q4k <= total / 2) {
-        if (q8 > total / 2) wdtype = FORGE_HIP_Q8_0;
-        else if (q4 > total / 2) wdtype = FORGE_HIP_Q4_0;
-    }
-    if (!wdtype) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: the projection weights are neither mostly Q8_0 nor mostly Q4_0");
-    // lm_head: the type of output.weight after loading (main.rs:567-581, gguf.rs:168-205); without that tensor the
-    // embedding table serves, converted to the projections' format
-    uint32_t lm = wdtype;
-    const TensorInfo* ot = g->tensor("output.weight");
-    if (!ot) ot = g->tensor("lm_head.weight");
-    if (ot) {
-        if (ot->type == T_Q4_0) lm = FORGE_HIP_Q4_0;
-        else if (ot->type == T_Q8_0) lm = FORGE_HIP_Q8_0;
-        else if (ot->type == T_F32 || ot->type == T_F16 || ot->type == T_BF16) lm = wdtype;   // dense: quantised like the projections
-        else if (requantised_on_load(ot->type)) lm = FORGE_HIP_Q8_0;                          // GGMLType::to_dtype, gguf.rs:168-205
-        else return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: output.weight has GGML type " + std::to_string(ot->type) +
-                                                       "; this library reads " + SUPPORTED_TYPES + " tensors");
-    }
-    const uint64_t seq = max_seq ? max_seq : ctx;
-    // Some(0) would make the reference attend to nothing (emit.rs:604-605)
-    if (has_window && window == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: a sliding window of 0 positions");
-    FH_CHECK(vocab <= 0xFFFFFFFFull && seq <= 0xFFFFFFFFull, "gguf: vocabulary or context length out of range");
-    forge_hip_config c{};
-    c.hidden = hidden; c.inter = inter; c.layers = layers; c.heads = heads; c.kv_heads = kv_heads;
-    c.head_dim = hidden / heads;                     // main.rs:731
-    c.vocab = (uint32_t)vocab; c.max_seq = (uint32_t)seq;
-    c.rms_eps = eps; c.rope_theta = theta;
-    c.wdtype = wdtype; c.lm_head_dtype = lm;
-    c.flags = flags | (arch == "qwen2" ? FORGE_HIP_FLAG_QKV_BIAS : 0u);
-    c.sliding_window = has_window ? window : 0u;     // main.rs:764-767
-    *out = c;
-    return FORGE_HIP_OK;
+        uint64_t vocab = 32000, ctx = 2048;
+        const MetaValue* tokens = g->find("tokenizer.ggml.tokens");
+        if (tokens && tokens->type == 9) vocab = tokens->count;
+        else g->get_u64(p + "vocab_size", &vocab);
+        g->get_u64(p + "context_length", &ctx);
+        float eps = 1e-5f, theta = 10000.0f;
+        g->get_f32(p + "attention.layer_norm_rms_epsilon", &eps);
+        g->get_f32(p + "rope.freq_base", &theta);
+        uint32_t window = 0;
+        const bool has_window = g->get_u32(p + "attention.sliding_window", &window);
+
+        // majority vote over the projection tensors (main.rs:479-555)
+        uint64_t q8 = 0, q4 = 0, q4k = 0, f16 = 0, f32 = 0;
+        for (const auto& t : g->tensors) {
+            const std::string& n = t.name;
+            const bool proj = n.find(".weight") != std::string::npos && n.find("token_embd") == std::string::npos &&
+                              n.find("output.weight") == std::string::npos && n.find("_norm") == std::string::npos;
+            if (!proj) continue;
+            switch (t.type) {
+                case T_Q8_0: q8++; break;
+                case T_Q4_0: q4++; break;
+                case 12: q4k++; break;
+                case T_F16: case T_BF16: f16++; break;
+                case T_F32: f32++; break;
+                case 3: case 20: case 23: case 6: case 7: case 9: case 10: case 11: case 13: case 14: case 15: case 16: case 17: case 22:
+                case 18: case 21: case 19: case 29: q8++; break;
+                default: break;
+            }
+        }
+        const uint64_t total = q8 + q4 + q4k + f16 + f32;
+        uint32_t wdtype = 0;
+        if (total && q4k <= total / 2) {
+            if (q8 > total / 2) wdtype = FORGE_HIP_Q8_0;
+            else if (q4 > total / 2) wdtype = FORGE_HIP_Q4_0;
+        }
+        if (!wdtype) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: the projection weights are neither mostly Q8_0 nor mostly Q4_0");
+        // lm_head: the type of output.weight after loading (main.rs:567-581, gguf.rs:168-205); without that tensor the
+        // embedding table serves, converted to the projections' format
+        uint32_t lm = wdtype;
+        const TensorInfo* ot = g->tensor("output.weight");
+        if (!ot) ot = g->tensor("lm_head.weight");
+        if (ot) {
+            if (ot->type == T_Q4_0) lm = FORGE_HIP_Q4_0;
+            else if (ot->type == T_Q8_0) lm = FORGE_HIP_Q8_0;
+            else if (ot->type == T_F32 || ot->type == T_F16 || ot->type == T_BF16) lm = wdtype;   // dense: quantised like the projections
+            else if (requantised_on_load(ot->type)) lm = FORGE_HIP_Q8_0;                          // GGMLType::to_dtype, gguf.rs:168-205
+            else return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: output.weight has GGML type " + std::to_string(ot->type) +
+                                                           "; this library reads " + SUPPORTED_TYPES + " tensors");
+        }
+        const uint64_t seq = max_seq ? max_seq : ctx;
+        // Some(0) would make the reference attend to nothing (emit.rs:604-605)
+        if (has_window && window == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: a sliding window of 0 positions");
+        FH_CHECK(vocab <= 0xFFFFFFFFull && seq <= 0xFFFFFFFFull, "gguf: vocabulary or context length out of range");
+        forge_hip_config c{};
+        c.hidden = hidden; c.inter = inter; c.layers = layers; c.heads = heads; c.kv_heads = kv_heads;
+        c.head_dim = hidden / heads;                     // main.rs:731
+        c.vocab = (uint32_t)vocab; c.max_seq = (uint32_t)seq;
+        c.rms_eps = eps; c.rope_theta = theta;
+        c.wdtype = wdtype; c.lm_head_dtype = lm;
+        c.flags = flags | (arch == "qwen2" ? FORGE_HIP_FLAG_QKV_BIAS : 0u);
+        c.sliding_window = has_window ? window : 0u;     // main.rs:764-767
+        // what the kernels cannot run is refused here, before any size is computed from these numbers
+        const int32_t vrc = fh::validate_config_shape(&c);
+        if (vrc) return vrc;
+        *out = c;
+        return FORGE_HIP_OK;
+    });
 }
 
 int32_t forge_hip_gguf_export_weights(const forge_hip_gguf* g, const forge_hip_config* c, uint8_t* out_host, uint64_t nbytes) {
-    FH_CHECK(g && c && out_host, "gguf_export_weights: null argument");
-    FH_CHECK(c->wdtype == FORGE_HIP_Q8_0 || c->wdtype == FORGE_HIP_Q4_0, "gguf_export_weights: wdtype must be Q8_0 or Q4_0");
-    FH_CHECK(c->lm_head_dtype == FORGE_HIP_Q8_0 || c->lm_head_dtype == FORGE_HIP_Q4_0, "gguf_export_weights: lm_head_dtype must be Q8_0 or Q4_0");
-    FH_CHECK(c->hidden % 32 == 0 && c->inter % 32 == 0 && (c->heads * c->head_dim) % 32 == 0, "gguf_export_weights: row lengths must be multiples of 32");
-    const uint64_t need = forge_hip_weights_nbytes(c);
-    if (nbytes != need)
-        return fh::fail(FORGE_HIP_ERR_BLOB_SIZE, "gguf_export_weights: buffer is " + std::to_string(nbytes) + " bytes, config needs " + std::to_string(need));
-    const uint64_t H = c->hidden, I = c->inter, QKS = (uint64_t)c->heads * c->head_dim, KV = (uint64_t)c->kv_heads * c->head_dim, V = c->vocab;
-    const uint32_t wt = c->wdtype;
-    uint8_t* p = out_host;
-    int32_t rc;
-#define FH_STEP(call, bytes) do { rc = (call); if (rc) return rc; p += (bytes); } while (0)
-    // the embedding table is always f32 in the blob (main.rs:2690-2722)
-    FH_STEP(write_f32(g, "token_embd.weight", V * H, p), V * H * 4);
-    for (uint32_t l = 0; l < c->layers; l++) {
-        FH_STEP(write_f32(g, blk(l, "attn_norm.weight"), H, p), H * 4);
-        if (!g->tensor(blk(l, "attn_q.weight")) && g->tensor(blk(l, "attn_qkv.weight"))) {
-            // Phi-3: Q|K|V rows in one tensor (weight_loader.rs:425-427, 552-567)
-            const uint64_t all = (QKS + 2 * KV) * H;
-            FH_STEP(write_quantised_part(g, blk(l, "attn_qkv.weight"), wt, all, 0, QKS * H, p), qbytes(wt, QKS * H));
-            FH_STEP(write_quantised_part(g, blk(l, "attn_qkv.weight"), wt, all, QKS * H, KV * H, p), qbytes(wt, KV * H));
-            FH_STEP(write_quantised_part(g, blk(l, "attn_qkv.weight"), wt, all, (QKS + KV) * H, KV * H, p), qbytes(wt, KV * H));
-        } else {
-            FH_STEP(write_quantised(g, blk(l, "attn_q.weight"), wt, QKS * H, p), qbytes(wt, QKS * H));
-            FH_STEP(write_quantised(g, blk(l, "attn_k.weight"), wt, KV * H, p), qbytes(wt, KV * H));
-            FH_STEP(write_quantised(g, blk(l, "attn_v.weight"), wt, KV * H, p), qbytes(wt, KV * H));
+    return no_throw("gguf_export_weights", [&]() -> int32_t {
+        FH_CHECK(g && c && out_host, "gguf_export_weights: null argument");
+        FH_CHECK(c->wdtype == FORGE_HIP_Q8_0 || c->wdtype == FORGE_HIP_Q4_0, "gguf_export_weights: wdtype must be Q8_0 or Q4_0");
+        FH_CHECK(c->lm_head_dtype == FORGE_HIP_Q8_0 || c->lm_head_dtype == FORGE_HIP_Q4_0, "gguf_export_weights: lm_head_dtype must be Q8_0 or Q4_0");
+        FH_CHECK(c->hidden % 32 == 0 && c->inter % 32 == 0 && (c->heads * c->head_dim) % 32 == 0, "gguf_export_weights: row lengths must be multiples of 32");
+        const int32_t vrc = fh::validate_config_shape(c);
+        if (vrc) return vrc;
+        const uint64_t need = forge_hip_weights_nbytes(c);
+        if (need == 0 || nbytes != need)
+            return fh::fail(FORGE_HIP_ERR_BLOB_SIZE, "gguf_export_weights: buffer is " + std::to_string(nbytes) + " bytes, config needs " + std::to_string(need));
+        const uint64_t H = c->hidden, I = c->inter, QKS = (uint64_t)c->heads * c->head_dim, KV = (uint64_t)c->kv_heads * c->head_dim, V = c->vocab;
+        const uint32_t wt = c->wdtype;
+        uint8_t* p = out_host;
+        int32_t rc;
+    #define FH_STEP(call, bytes) do { rc = (call); if (rc) return rc; p += (bytes); } while (0)
+        // the embedding table is always f32 in the blob (main.rs:2690-2722)
+        FH_STEP(write_f32(g, "token_embd.weight", V * H, p), V * H * 4);
+        for (uint32_t l = 0; l < c->layers; l++) {
+            FH_STEP(write_f32(g, blk(l, "attn_norm.weight"), H, p), H * 4);
+            if (!g->tensor(blk(l, "attn_q.weight")) && g->tensor(blk(l, "attn_qkv.weight"))) {
+                // Phi-3: Q|K|V rows in one tensor (weight_loader.rs:425-427, 552-567)
+                const uint64_t all = (QKS + 2 * KV) * H;
+                FH_STEP(write_quantised_part(g, blk(l, "attn_qkv.weight"), wt, all, 0, QKS * H, p), qbytes(wt, QKS * H));
+                FH_STEP(write_quantised_part(g, blk(l, "attn_qkv.weight"), wt, all, QKS * H, KV * H, p), qbytes(wt, KV * H));
+                FH_STEP(write_quantised_part(g, blk(l, "attn_qkv.weight"), wt, all, (QKS + KV) * H, KV * H, p), qbytes(wt, KV * H));
+            } else {
+                FH_STEP(write_quantised(g, blk(l, "attn_q.weight"), wt, QKS * H, p), qbytes(wt, QKS * H));
+                FH_STEP(write_quantised(g, blk(l, "attn_k.weight"), wt, KV * H, p), qbytes(wt, KV * H));
+                FH_STEP(write_quantised(g, blk(l, "attn_v.weight"), wt, KV * H, p), qbytes(wt, KV * H));
+            }
+            if (c->flags & FORGE_HIP_FLAG_QKV_BIAS) {             // main.rs:2737-2742
+                FH_STEP(write_f32(g, blk(l, "attn_q.bias"), QKS, p), QKS * 4);
+                FH_STEP(write_f32(g, blk(l, "attn_k.bias"), KV, p), KV * 4);
+                FH_STEP(write_f32(g, blk(l, "attn_v.bias"), KV, p), KV * 4);
+            }
+            FH_STEP(write_quantised(g, blk(l, "attn_output.weight"), wt, H * QKS, p), qbytes(wt, H * QKS));
+            FH_STEP(write_f32(g, blk(l, "ffn_norm.weight"), H, p), H * 4);
+            const TensorInfo* up = g->tensor(blk(l, "ffn_up.weight"));
+            if (!g->tensor(blk(l, "ffn_gate.weight")) && up && up->numel() == 2 * I * H) {
+                // Phi-3: gate|up rows in one tensor (weight_loader.rs:569-580)
+                FH_STEP(write_quantised_part(g, blk(l, "ffn_up.weight"), wt, 2 * I * H, 0, I * H, p), qbytes(wt, I * H));
+                FH_STEP(write_quantised_part(g, blk(l, "ffn_up.weight"), wt, 2 * I * H, I * H, I * H, p), qbytes(wt, I * H));
+            } else {
+                FH_STEP(write_quantised(g, blk(l, "ffn_gate.weight"), wt, I * H, p), qbytes(wt, I * H));
+                FH_STEP(write_quantised(g, blk(l, "ffn_up.weight"), wt, I * H, p), qbytes(wt, I * H));
+            }
+            FH_STEP(write_quantised(g, blk(l, "ffn_down.weight"), wt, H * I, p), qbytes(wt, H * I));
         }
-        if (c->flags & FORGE_HIP_FLAG_QKV_BIAS) {             // main.rs:2737-2742
-            FH_STEP(write_f32(g, blk(l, "attn_q.bias"), QKS, p), QKS * 4);
-            FH_STEP(write_f32(g, blk(l, "attn_k.bias"), KV, p), KV * 4);
-            FH_STEP(write_f32(g, blk(l, "attn_v.bias"), KV, p), KV * 4);
-        }
-        FH_STEP(write_quantised(g, blk(l, "attn_output.weight"), wt, H * QKS, p), qbytes(wt, H * QKS));
-        FH_STEP(write_f32(g, blk(l, "ffn_norm.weight"), H, p), H * 4);
-        const TensorInfo* up = g->tensor(blk(l, "ffn_up.weight"));
-        if (!g->tensor(blk(l, "ffn_gate.weight")) && up && up->numel() == 2 * I * H) {
-            // Phi-3: gate|up rows in one tensor (weight_loader.rs:569-580)
-            FH_STEP(write_quantised_part(g, blk(l, "ffn_up.weight"), wt, 2 * I * H, 0, I * H, p), qbytes(wt, I * H));
-            FH_STEP(write_quantised_part(g, blk(l, "ffn_up.weight"), wt, 2 * I * H, I * H, I * H, p), qbytes(wt, I * H));
-        } else {
-            FH_STEP(write_quantised(g, blk(l, "ffn_gate.weight"), wt, I * H, p), qbytes(wt, I * H));
-            FH_STEP(write_quantised(g, blk(l, "ffn_up.weight"), wt, I * H, p), qbytes(wt, I * H));
-        }
-        FH_STEP(write_quantised(g, blk(l, "ffn_down.weight"), wt, H * I, p), qbytes(wt, H * I));
-    }
-    FH_STEP(write_f32(g, "output_norm.weight", H, p), H * 4);
-    // lm_head: output.weight, or the embedding table of a model with tied weights (main.rs:2632-2676)
-    const char* lm_name = g->tensor("output.weight") ? "output.weight" : g->tensor("lm_head.weight") ? "lm_head.weight" : "token_embd.weight";
-    FH_STEP(write_quantised(g, lm_name, c->lm_head_dtype, V * H, p), qbytes(c->lm_head_dtype, V * H));
-#undef FH_STEP
-    if ((uint64_t)(p - out_host) != need) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf_export_weights: internal size mismatch");
-    return FORGE_HIP_OK;
+        FH_STEP(write_f32(g, "output_norm.weight", H, p), H * 4);
+        // lm_head: output.weight, or the embedding table of a model with tied weights (main.rs:2632-2676)
+        const char* lm_name = g->tensor("output.weight") ? "output.weight" : g->tensor("lm_head.weight") ? "lm_head.weight" : "token_embd.weight";
+        FH_STEP(write_quantised(g, lm_name, c->lm_head_dtype, V * H, p), qbytes(c->lm_head_dtype, V * H));
+    #undef FH_STEP
+        if ((uint64_t)(p - out_host) != need) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf_export_weights: internal size mismatch");
+        return FORGE_HIP_OK;
+    });
 }
 
 int32_t forge_hip_model_create_from_gguf(const char* path, uint32_t max_seq, uint32_t flags, forge_hip_model** out) {
-    FH_CHECK(out, "model_create_from_gguf: null out");
-    *out = nullptr;
-    forge_hip_gguf* g = nullptr;
-    int32_t rc = forge_hip_gguf_open(path, &g);
-    if (rc) return rc;
-    std::unique_ptr<forge_hip_gguf> hold(g);
-    forge_hip_config c;
-    rc = forge_hip_gguf_config(g, max_seq, flags, &c);
-    if (rc) return rc;
-    const uint64_t n = forge_hip_weights_nbytes(&c);
-    std::unique_ptr<uint8_t[]> blob(new (std::nothrow) uint8_t[n]);
-    if (!blob) return fh::fail(FORGE_HIP_ERR_INVALID, "model_create_from_gguf: out of host memory for " + std::to_string(n) + " bytes");
-    rc = forge_hip_gguf_export_weights(g, &c, blob.get(), n);
-    if (rc) return rc;
-    return forge_hip_model_create(&c, blob.get(), n, out);
+    return no_throw("model_create_from_gguf", [&]() -> int32_t {
+        FH_CHECK(out, "model_create_from_gguf: null out");
+        *out = nullptr;
+        forge_hip_gguf* g = nullptr;
+        int32_t rc = forge_hip_gguf_open(path, &g);
+        if (rc) return rc;
+        std::unique_ptr<forge_hip_gguf> hold(g);
+        forge_hip_config c;
+        rc = forge_hip_gguf_config(g, max_seq, flags, &c);
+        if (rc) return rc;
+        const uint64_t n = forge_hip_weights_nbytes(&c);
+        if (n == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "model_create_from_gguf: the configuration's weight size does not fit 64 bits");
+        std::unique_ptr<uint8_t[]> blob(new (std::nothrow) uint8_t[n]);
+        if (!blob) return fh::fail(FORGE_HIP_ERR_INVALID, "model_create_from_gguf: out of host memory for " + std::to_string(n) + " bytes");
+        rc = forge_hip_gguf_export_weights(g, &c, blob.get(), n);
+        if (rc) return rc;
+        return forge_hip_model_create(&c, blob.get(), n, out);
+    });
 }
 
 }  // extern "C"

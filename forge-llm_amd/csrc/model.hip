@@ -152,7 +152,8 @@ int32_t collect_profile(forge_hip_model* m, float* stage_ms, uint32_t* stage_lau
 
 size_t wsize(uint32_t dtype, uint64_t n, uint64_t k) { return (size_t)(n * (k / 32) * (dtype == FORGE_HIP_Q8_0 ? 34 : 18)); }
 
-int32_t validate(const forge_hip_config* c) {
+// The numbers sizes are computed from: formats, dimensions the kernels cover.
+int32_t validate_shape(const forge_hip_config* c) {
     FH_CHECK(c, "config is null");
     FH_CHECK(c->wdtype == FORGE_HIP_Q8_0 || c->wdtype == FORGE_HIP_Q4_0, "wdtype must be Q8_0 (8) or Q4_0 (2)");
     FH_CHECK(c->lm_head_dtype == FORGE_HIP_Q8_0 || c->lm_head_dtype == FORGE_HIP_Q4_0, "lm_head_dtype must be Q8_0 (8) or Q4_0 (2)");
@@ -161,6 +162,14 @@ int32_t validate(const forge_hip_config* c) {
     FH_CHECK(c->layers >= 1 && c->vocab >= 1 && c->max_seq >= 1, "layers, vocab and max_seq must be positive");
     FH_CHECK(c->heads >= 1 && c->kv_heads >= 1 && c->heads % c->kv_heads == 0, "heads must be a positive multiple of kv_heads");
     FH_CHECK(attn_head_dim_supported(c->head_dim), "head_dim must be 64, 96 or 128");
+    FH_CHECK(c->heads <= 16384 / 64 && gemv_k_supported(c->hidden) && gemv_k_supported(c->inter) && gemv_k_supported(c->heads * c->head_dim),
+             "hidden, inter and heads*head_dim must be at most 16384");
+    return FORGE_HIP_OK;
+}
+
+int32_t validate_cfg(const forge_hip_config* c) {
+    const int32_t rc = validate_shape(c);
+    if (rc) return rc;
     FH_CHECK((c->flags & ~(FORGE_HIP_FLAG_EXACT | FORGE_HIP_FLAG_QKV_BIAS)) == 0, "unknown bits in flags");
     // The reference switches to its non-flash attention (a different summation order) when
     // max_seq_len <= 512 (emit.rs:126-128); the order-faithful kernels follow the flash variants only.
@@ -169,8 +178,6 @@ int32_t validate(const forge_hip_config* c) {
     // restatement keeps one row of scores in LDS
     FH_CHECK(!(c->flags & FORGE_HIP_FLAG_EXACT) || c->sliding_window == 0 || std::min(c->sliding_window, c->max_seq) <= attn_exact_max_window(),
              "FORGE_HIP_FLAG_EXACT with a sliding window needs min(sliding_window, max_seq) <= 12288");
-    FH_CHECK(gemv_k_supported(c->hidden) && gemv_k_supported(c->inter) && gemv_k_supported(c->heads * c->head_dim),
-             "hidden, inter and heads*head_dim must be at most 16384");
     return FORGE_HIP_OK;
 }
 
@@ -356,21 +363,32 @@ int32_t finish_or_undo(forge_hip_model* m) {
 
 }  // namespace
 
+namespace fh {
+int32_t validate_config_shape(const forge_hip_config* c) { return validate_shape(c); }
+}  // namespace fh
+
 extern "C" {
 
 uint64_t forge_hip_weights_nbytes(const forge_hip_config* c) {
     if (!c) return 0;
-    const uint64_t H = c->hidden, I = c->inter, QKS = (uint64_t)c->heads * c->head_dim, KV = (uint64_t)c->kv_heads * c->head_dim;
-    const uint64_t per_layer = H * 4 + wsize(c->wdtype, QKS, H) + 2 * wsize(c->wdtype, KV, H) + wsize(c->wdtype, H, QKS) +
-                               H * 4 + 2 * wsize(c->wdtype, I, H) + wsize(c->wdtype, H, I) +
-                               ((c->flags & FORGE_HIP_FLAG_QKV_BIAS) ? (QKS + 2 * KV) * 4 : 0);
-    return (uint64_t)c->vocab * H * 4 + c->layers * per_layer + H * 4 + wsize(c->lm_head_dtype, c->vocab, H);
+    // every field is a caller's (or a file's) 32-bit number: the sum is formed with checked arithmetic and is 0 when
+    // it does not fit 64 bits -- no blob has that length, so forge_hip_model_create refuses such a configuration
+    bool over = false;
+    auto mul = [&](uint64_t a, uint64_t b) { uint64_t r = 0; over = over || __builtin_mul_overflow(a, b, &r); return r; };
+    auto add = [&](uint64_t a, uint64_t b) { uint64_t r = 0; over = over || __builtin_add_overflow(a, b, &r); return r; };
+    auto w = [&](uint32_t t, uint64_t n, uint64_t k) { return mul(mul(n, k / 32), t == FORGE_HIP_Q8_0 ? 34 : 18); };
+    const uint64_t H = c->hidden, I = c->inter, QKS = mul(c->heads, c->head_dim), KV = mul(c->kv_heads, c->head_dim);
+    uint64_t per_layer = add(mul(H, 8), add(add(w(c->wdtype, QKS, H), mul(2, w(c->wdtype, KV, H))), w(c->wdtype, H, QKS)));
+    per_layer = add(per_layer, add(mul(2, w(c->wdtype, I, H)), w(c->wdtype, H, I)));
+    if (c->flags & FORGE_HIP_FLAG_QKV_BIAS) per_layer = add(per_layer, mul(add(QKS, mul(2, KV)), 4));
+    const uint64_t total = add(add(mul(mul(c->vocab, H), 4), mul(c->layers, per_layer)), add(mul(H, 4), w(c->lm_head_dtype, c->vocab, H)));
+    return over ? 0 : total;
 }
 
 int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob, uint64_t nbytes, forge_hip_model** out) {
     FH_CHECK(out, "model_create: null out");
     *out = nullptr;
-    int32_t rc = validate(cfg);
+    int32_t rc = validate_cfg(cfg);
     if (rc) return rc;
     FH_CHECK(blob, "model_create: null weights");
     if (nbytes != forge_hip_weights_nbytes(cfg))

@@ -431,6 +431,58 @@ def test_damaged_files_are_refused_or_read_but_never_crash(fh, gg):
 
 
 # ---------------- the other block formats the reference's loader reads ----------------
+def test_hostile_sizes_are_refused_before_anything_is_computed_from_them(fh, gg, tmp_path):
+    """Numbers a file controls (tensor dimensions, embedding length, vocabulary, layer count) are checked before any size
+    is derived from them: products that wrap 64 bits, dimensions no kernel covers, a blob size beyond 64 bits, an
+    allocation that cannot be had.  Every case comes back as an error code."""
+    base = [("general.architecture", gg.STRING, "llama"), ("llama.embedding_length", gg.U32, 64), ("llama.block_count", gg.U32, 1),
+            ("llama.attention.head_count", gg.U32, 1)]
+    q = ("blk.0.attn_q.weight", [64, 64], gg.Q8_0, None)
+    # tensor dimensions: a product that wraps to 0, one that wraps to a small number, one that is merely absurd
+    for dims in ([1 << 32, 1 << 32], [(1 << 63) + 1, 2, 1, 1], [1 << 40, 1 << 20], [1 << 49]):
+        assert "more than 2^48 elements" in err(fh, gg.write_gguf(base, [q, ("blk.0.attn_k.weight", dims, gg.F16, None)]))
+    gg.GgufFile(gg.write_gguf(base, [q, ("blk.0.attn_k.weight", [1 << 24, 1 << 24], gg.F16, None)]))      # 2^48 itself parses
+
+    def config_error(meta):
+        with pytest.raises(fh.ForgeHipError) as e:
+            gg.GgufFile(gg.write_gguf(meta, [q])).config()
+        assert e.value.code == fh.ERR_INVALID
+        return str(e.value)
+
+    def with_(key, vtype, value):
+        return [(k, t, value if k == key else v) for k, t, v in base] if any(k == key for k, _, _ in base) else base + [(key, vtype, value)]
+
+    assert "embedding_length out of range" in config_error(with_("llama.embedding_length", gg.U32, 0xFFFFFFE0))   # 4 * hidden would wrap
+    assert "hidden must be" in config_error(with_("llama.embedding_length", gg.U32, 1 << 20))
+    assert "hidden must be" in config_error(with_("llama.embedding_length", gg.U32, 1 << 20) + [("llama.feed_forward_length", gg.U32, 64)])
+    assert "head_dim must be" in config_error(with_("llama.attention.head_count", gg.U32, 0xFFFFFFFF))
+    assert "inter must be" in config_error(with_("llama.feed_forward_length", gg.U32, 0xFFFFFFFF))
+    assert "at most 16384" in config_error(with_("llama.feed_forward_length", gg.U32, 0xFFFFFFE0))
+    assert "out of range" in config_error(with_("llama.vocab_size", gg.U64, 1 << 40))
+    assert "out of range" in config_error(with_("llama.context_length", gg.U64, 1 << 33))
+    # numbers that pass (a 32-bit vocabulary and layer count on a small hidden size): the sizes are real, just unobtainable
+    big = gg.GgufFile(gg.write_gguf(base + [("llama.vocab_size", gg.U64, 0xFFFFFFFF)], [q]))
+    c = big.config()
+    assert c["vocab"] == 0xFFFFFFFF
+    n = fh.hip_model.weights_nbytes(c)
+    assert n > (1 << 40)
+    from ctypes import byref, c_void_p
+    small = np.empty(16, np.uint8)
+    assert fh.lib().forge_hip_gguf_export_weights(big._h, byref(fh.Config(**c)), small.ctypes.data_as(c_void_p), 16) == fh.ERR_BLOB_SIZE
+    path = str(tmp_path / "big.gguf")
+    gg.write_gguf(base + [("llama.vocab_size", gg.U64, 0xFFFFFFFF)], [q], path=path)
+    h = c_void_p()
+    rc = fh.lib().forge_hip_model_create_from_gguf(path.encode(), 0, 0, byref(h))
+    assert rc == fh.ERR_INVALID and not h.value               # no terabyte to be had, or no such tensors: an error either way
+    # a configuration whose blob size does not fit 64 bits has size 0, and no model is made from it
+    wild = dict(c, hidden=16352, inter=0xFFFFFFE0, layers=0xFFFFFFFF, vocab=0xFFFFFFFF, heads=128, kv_heads=128, head_dim=128)
+    assert fh.hip_model.weights_nbytes(wild) == 0
+    with pytest.raises(fh.ForgeHipError):
+        fh.HipModel(wild, np.zeros(16, np.uint8))
+    with pytest.raises(fh.ForgeHipError):
+        big.export_weights(wild)
+
+
 def f16le(bits):
     return struct.pack("<H", bits)
 
