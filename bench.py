@@ -232,6 +232,10 @@ def ops_table(fh, reps=10):
             us = timed(lambda: ops.matmul_vec_q(w, x))
             rows.append({"op": "gemv", "fmt": name, "K": K, "N": N, "us_per_call": round(us, 2),
                          "weight_bytes": N * (K // 32) * bpb})
+            if (K, N) == (2048, 8192):      # the reference's x86 arithmetic (f32 activations, sequential row sums) on the same matrix
+                us = timed(lambda: ops.matmul_vec_q_portable(w, x))
+                rows.append({"op": "gemv_portable_dot", "fmt": name, "K": K, "N": N, "us_per_call": round(us, 2),
+                             "weight_bytes": N * (K // 32) * bpb})
             if N <= 8192:
                 for M in (352, 902, 1603, 2502):
                     xm = torch.from_numpy(fh.synth.normal(8, M * K, 1.0).reshape(M, K)).cuda()

@@ -158,6 +158,13 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
     return FORGE_HIP_OK;
 }
 
+int32_t forge_hip_gemv_q_f32act(const forge_hip_qweight* w, const float* x_dev, float* y_dev, void* stream) {
+    FH_CHECK(w && x_dev && y_dev, "gemv_q_f32act: null pointer");
+    launch_gemv_f32(w->w, x_dev, y_dev, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
 int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, uint32_t M, int32_t* out_dev,
                               uint32_t path, void* stream) {
     FH_CHECK(w && x_dev && out_dev, "block_isums: null pointer");

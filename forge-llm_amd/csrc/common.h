@@ -130,6 +130,10 @@ void launch_gemv_norm_rope_kv(const QWeight& wqkv, const float* x, const float* 
 void launch_gemv_norm_silu_quant(const QWeight& wgu, const float* x, const float* norm_w, float eps, int8_t* oq,
                                  uint16_t* osc, hipStream_t s);
 
+// gemv_f32.hip — the reference's portable row dot (f32 activations x weights dequantised on the fly, one sequential sum
+// per row): y[n] = sum_k x[k] * (f32(q[n][k]) * w_s[n][k/32]).
+void launch_gemv_f32(const QWeight& w, const float* x, float* y, hipStream_t s);
+
 // gemm.hip — y[m][n] (=|+=) ...; aq int8 [M][K], as fp16 [M][K/32].  isums (optional) int32 [M][N][K/32].
 // exact: unfused multiply/add per block (bit-identical to the CPU path); otherwise one FMA per block, and then the
 // activation codes of every row's odd blocks must come negated (the neg_odd flag of the quantising launchers).

@@ -140,6 +140,19 @@ def matmul_vec_q(w: QWeight, x):
     return y
 
 
+def matmul_vec_q_portable(w: QWeight, x):
+    """The same matmul through the reference's portable row dot (the x86 arithmetic: f32 activations, weights dequantised
+    on the fly, one sequential sum per row; emit.rs:1359-1377, 2337-2359)."""
+    from . import check, lib
+    torch = _torch()
+    x = _dev(x, torch.float32)
+    if x.numel() != w.K:
+        raise ValueError("input length must equal K")
+    y = torch.empty(w.N, dtype=torch.float32, device=x.device)
+    check(lib().forge_hip_gemv_q_f32act(w._h, _ptr(x), _ptr(y), _stream()))
+    return y
+
+
 def expf_host(x) -> np.ndarray:
     """exp as the GPU kernels evaluate it (host twin; bit-identical to the C library's expf)."""
     from . import check, lib

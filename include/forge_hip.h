@@ -164,6 +164,12 @@ int32_t forge_hip_quantize_act(const float* x_dev, uint32_t M, uint32_t K, int8_
  * x_dev f32 [K], y_dev f32 [N]. */
 int32_t forge_hip_gemv_q(const forge_hip_qweight* w, const float* x_dev, float* y_dev, void* stream);
 
+/* The same matmul in the arithmetic the reference runs on hosts other than aarch64: its portable dot_q8_0 / dot_q4_0
+ * (emit.rs:1359-1377, 2337-2359) called once per row by matmul_vec (emit.rs:2046-2092) -- f32 activations against
+ * weights dequantised on the fly, y[n] = sum_k x[k] * (f32(q) * scale) added element by element in order (Q4_0: low
+ * nibble j, then high nibble j + 16, per byte).  Bit-identical to that code; no activation quantiser is involved. */
+int32_t forge_hip_gemv_q_f32act(const forge_hip_qweight* w, const float* x_dev, float* y_dev, void* stream);
+
 /* matmul_mat_q8_0_KxN / matmul_mat_q4_0_KxN (emit.rs:2108-2302, 3667-3817):
  * y[M][N] = x[M][K] W^T, row-major. */
 int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, uint32_t flags,

@@ -101,6 +101,30 @@ def test_matmul_vec_bit_exact(fh, oracle, torch_gpu, wd, K, N):
 
 
 @pytest.mark.parametrize("wd", [Q8, Q4])
+@pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 512), (8192, 2048), (576, 1536), (3072, 1029), (32, 5), (96, 7), (160, 64),
+                                 (2048, 1283)])
+def test_matmul_vec_portable_dot_bit_exact(fh, oracle, torch_gpu, wd, K, N):
+    """The reference's x86 arithmetic (variant B: f32 activations against weights dequantised on the fly, one sequential
+    sum per row, emit.rs:1359-1377 / 2337-2359): identical bits, row counts that are not multiples of 64, K that is not a
+    multiple of the kernel's 128-element tile, and activations with large and tiny blocks side by side."""
+    torch = torch_gpu
+    wraw = make_weight(fh, wd, N, K, seed=7 * N + K)
+    x = fh.synth.normal(17 + K, K, 1.0)
+    x[:32] *= 1e4
+    if K >= 64:
+        x[32:64] *= 1e-6
+    w = fh.ops.QWeight(wd, wraw, K, N)
+    y = fh.ops.matmul_vec_q_portable(w, torch.from_numpy(x).cuda()).cpu().numpy()
+    want = oracle.matmul_vec(wd, 1, x, wraw, K, N)
+    same_bits(y, want)
+    # and it is a different arithmetic from the int8 block-dot path: close, not equal
+    ya = fh.ops.matmul_vec_q(w, torch.from_numpy(x).cuda()).cpu().numpy()
+    assert np.abs(ya - want).max() <= 2e-2 * max(1.0, float(np.abs(want).max()))
+    if K >= 2048:
+        assert not np.array_equal(ya, want)
+
+
+@pytest.mark.parametrize("wd", [Q8, Q4])
 @pytest.mark.parametrize("M,K,N", [(1, 2048, 512), (37, 576, 960), (352, 2048, 2048), (130, 8192, 320), (129, 3072, 256)])
 def test_matmul_mat_parity(fh, oracle, torch_gpu, wd, M, K, N):
     torch = torch_gpu
