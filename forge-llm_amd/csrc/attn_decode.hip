@@ -2,25 +2,18 @@
 // sequence so that one query fills the GPU ("flash decoding"): grid = (kv head groups,
 // DECODE_SPLITS).  HBM-bound: each K/V row is read once per group of query heads that share
 // it.  A key row of head_dim fp16 values is spread over LPK lanes (16 bytes each); the
-// lanes of a wave cover 64/LPK keys per load and every key slot keeps its own online-softmax
-// state, so the loop needs no cross-slot traffic; slots, waves and splits are merged at
-// the end with the usual (max, sum, acc) rescaling.
+// lanes of a wave cover 64/LPK keys per load, a wave keeps four such loads of K and of V in flight
+// (and the next four requested before it computes), and every key slot keeps its own online-softmax
+// state, advanced two keys at a time (one new maximum and one rescale per pair), so the loop
+// needs no cross-slot traffic; slots, waves and splits are merged at the end with the usual
+// (max, sum, acc) rescaling.
 #include <mutex>
 
+#include "attn_decode_math.h"
 #include "common.h"
 #include "device_utils.h"
 
 namespace fh {
-
-struct __attribute__((aligned(16))) Half8 { uint32_t w[4]; };
-
-__device__ __forceinline__ void unpack8(const Half8& h, float* f) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        f[2 * i] = f16_bits_to_f32((uint16_t)(h.w[i] & 0xFFFFu));
-        f[2 * i + 1] = f16_bits_to_f32((uint16_t)(h.w[i] >> 16));
-    }
-}
 
 // merge (m2,l2,a2) into (m,l,a)
 template <int NV>
@@ -79,35 +72,43 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const float* __r
         for (int i = 0; i < 8; i++) acc[g][i] = 0.f;
     }
 
-    for (uint32_t tb = t0 + wave * KPW; tb < t1; tb += 4 * KPW) {
-        const uint32_t t = tb + slot;
-        const bool valid = t < t1;
-        Half8 kr = {{0, 0, 0, 0}}, vr = {{0, 0, 0, 0}};
-        if (valid && dvalid) {
-            const size_t off = (size_t)t * kv_stride + kvh * HD + c * 8;
-            kr = *reinterpret_cast<const Half8*>(kc + off);
-            vr = *reinterpret_cast<const Half8*>(vc + off);
-        }
-        float kf[8], vf[8];
-        unpack8(kr, kf);
-        unpack8(vr, vf);
+    // A wave takes UNR key blocks (UNR * KPW keys) per step, all their K and V loads in flight together and the next step's
+    // issued before this step's arithmetic; every key slot advances its online softmax by UNR keys at once.
+    constexpr int UNR = 4;
+    const uint32_t tbw = t0 + wave * KPW, tstep = UNR * 4 * KPW;
+    auto load_step = [&](uint32_t tb0, Half8 (&kr)[UNR], Half8 (&vr)[UNR]) {
 #pragma unroll
-        for (int g = 0; g < GT; g++) {
-            float d = 0.f;
-#pragma unroll
-            for (int i = 0; i < 8; i++) d = fmaf(qf[g][i], kf[i], d);
-#pragma unroll
-            for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, WAVE);
-            if (valid) {
-                const float s = d * scale;
-                const float mn = fmaxf(m[g], s);
-                const float alpha = __expf(m[g] - mn);   // m = -inf on the first key: exp(-inf) = 0
-                const float p = __expf(s - mn);
-                l[g] = fmaf(l[g], alpha, p);
-#pragma unroll
-                for (int i = 0; i < 8; i++) acc[g][i] = fmaf(acc[g][i], alpha, p * vf[i]);
-                m[g] = mn;
+        for (int u = 0; u < UNR; u++) {
+            const uint32_t t = tb0 + u * 4 * KPW + slot;
+            kr[u] = Half8{{0, 0, 0, 0}};
+            vr[u] = Half8{{0, 0, 0, 0}};
+            if (t < t1 && dvalid) {
+                const size_t off = (size_t)t * kv_stride + kvh * HD + c * 8;
+                kr[u] = *reinterpret_cast<const Half8*>(kc + off);
+                vr[u] = *reinterpret_cast<const Half8*>(vc + off);
             }
+        }
+    };
+    Half8 kr[UNR], vr[UNR], kn[UNR], vn[UNR];
+    if (tbw < t1) load_step(tbw, kr, vr);
+    for (uint32_t tb0 = tbw; tb0 < t1; tb0 += tstep) {
+        const bool more = tb0 + tstep < t1;
+        if (more) load_step(tb0 + tstep, kn, vn);
+#pragma unroll
+        for (int u0 = 0; u0 < UNR; u0 += 2)
+#pragma unroll
+            for (int g = 0; g < GT; g++) {
+                float sc[2];
+#pragma unroll
+                for (int u = 0; u < 2; u++) {
+                    const float d = key_dot<LPK>(qf[g], kr[u0 + u]);
+                    sc[u] = tb0 + (u0 + u) * 4 * KPW + slot < t1 ? d * scale : -INFINITY;
+                }
+                softmax_block_update<2>(m[g], l[g], acc[g], sc, vr + u0);
+            }
+        if (more) {
+#pragma unroll
+            for (int u = 0; u < UNR; u++) { kr[u] = kn[u]; vr[u] = vn[u]; }
         }
     }
 

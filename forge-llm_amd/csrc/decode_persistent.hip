@@ -45,6 +45,7 @@
 
 #include <chrono>
 
+#include "attn_decode_math.h"
 #include "common.h"
 #include "device_utils.h"
 #include "expf_ref.h"
@@ -509,16 +510,6 @@ __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& 
 }
 
 // ---- attention ------------------------------------------------------------------------------------------
-struct __attribute__((aligned(16))) Half8 { uint32_t w[4]; };
-
-__device__ __forceinline__ void unpack8(const Half8& h, float* f) {
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        f[2 * i] = f16_bits_to_f32((uint16_t)(h.w[i] & 0xFFFFu));
-        f[2 * i + 1] = f16_bits_to_f32((uint16_t)(h.w[i] >> 16));
-    }
-}
-
 template <int NV>
 __device__ __forceinline__ void merge_state(float& m, float& l, float* a, float m2, float l2, const float* a2) {
     const float mn = fmaxf(m, m2);
@@ -657,35 +648,20 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
                         vr[u] = Half8{{0, 0, 0, 0}};
                     }
                 }
+                // every key slot advances two keys at a time (attn_decode_math.h: the kernel pair's arithmetic)
 #pragma unroll
-                for (int u = 0; u < UNR; u++) {
-                    const uint32_t tb = tb0 + u * 4 * KPW;
-                    if (tb < t1) {
-                        const bool valid = tb + slot < t1;
-                        float kf[8], vf[8];
-                        unpack8(kr[u], kf);
-                        unpack8(vr[u], vf);
+                for (int u0 = 0; u0 < UNR; u0 += 2)
 #pragma unroll
-                        for (int hh = 0; hh < NH; hh++) {
-                            if (!has[hh]) continue;
-                            float d = 0.f;
+                    for (int hh = 0; hh < NH; hh++) {
+                        if (!has[hh]) continue;
+                        float sc[2];
 #pragma unroll
-                            for (int i = 0; i < 8; i++) d = fmaf(qf[hh][i], kf[i], d);
-#pragma unroll
-                            for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, WAVE);
-                            if (valid) {
-                                const float sc = d * scale;
-                                const float mn = fmaxf(m[hh], sc);
-                                const float alpha = __expf(m[hh] - mn);   // m = -inf on the first key: exp(-inf) = 0
-                                const float p = __expf(sc - mn);
-                                l[hh] = fmaf(l[hh], alpha, p);
-#pragma unroll
-                                for (int i = 0; i < 8; i++) acc[hh][i] = fmaf(acc[hh][i], alpha, p * vf[i]);
-                                m[hh] = mn;
-                            }
+                        for (int u = 0; u < 2; u++) {
+                            const float d = key_dot<LPK>(qf[hh], kr[u0 + u]);
+                            sc[u] = tb0 + (u0 + u) * 4 * KPW + slot < t1 ? d * scale : -INFINITY;
                         }
+                        softmax_block_update<2>(m[hh], l[hh], acc[hh], sc, vr + u0);
                     }
-                }
             }
 #pragma unroll
             for (int hh = 0; hh < NH; hh++) {
