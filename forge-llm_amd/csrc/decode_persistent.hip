@@ -583,6 +583,11 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
                 vr0[u] = ldg(reinterpret_cast<const Half8*>(vc + off));
             }
         }
+        // The phase before this one is a GEMV whose rows the poller waves may still be summing out of the LDS area that q,
+        // this position's K/V row and the wave records are about to be written to: in a GEMV phase only the pollers write
+        // LDS inputs, here every wave does, and a streamer wave gets here as soon as it has issued its loads.  (The loads
+        // above touch no LDS: they stay in front of the barrier.)
+        if (it == 0) __syncthreads();
         // q is awaited even when the split is empty: the wait orders this item's records after the previous layer's readers
         for (uint32_t e = ltid; on && (e < gt * HD || (has_new && e < 2 * HD)); e += lthreads) {
             const bool need_q = e < gt * HD, need_kv = has_new && e < 2 * HD;

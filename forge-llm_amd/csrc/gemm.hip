@@ -213,9 +213,12 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
             f.sa[t] = *reinterpret_cast<const uint16_t*>(lds + sa_off + slot * s_slot_stride + t * s_t_stride + kb * 2);
         }
     };
+    // operand of the rank-1 product: the scale in k = 0, zeros in the other slots (the K = 8 form of the MFMA: two registers
+    // per operand, one of them the zero, where the K = 16 form needs three zero registers beside every scale)
+    typedef _Float16 v4s __attribute__((ext_vector_type(4)));
     auto scale_operand = [](uint32_t bits) {
         const _Float16 z = (_Float16)0.0f;
-        return (v8h){__builtin_bit_cast(_Float16, (uint16_t)bits), z, z, z, z, z, z, z};
+        return (v4s){__builtin_bit_cast(_Float16, (uint16_t)bits), z, z, z};
     };
 
     const v16i zero_i = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
@@ -243,7 +246,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         Frag fr[2];
         read_frag(fr[0], buf, slot, 0);
         v16i isum = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[0].af[0], fr[0].bf[0], c_in, 0, 0, 0);
-        v16f S = __builtin_amdgcn_mfma_f32_32x32x16_f16(scale_operand(fr[0].sa[0]), scale_operand(fr[0].sb[0]), zero_f, 0, 0, 0);
+        v16f S = __builtin_amdgcn_mfma_f32_32x32x8f16(scale_operand(fr[0].sa[0]), scale_operand(fr[0].sb[0]), zero_f, 0, 0, 0);
 #pragma unroll
         for (int kb = 0; kb < KB; kb++) {
             Frag& f = fr[kb & 1];
@@ -263,6 +266,9 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                 v16i isum_n = zero_i;
                 v16f S_n = zero_f;
                 if (has_next) isum_n = __builtin_amdgcn_mfma_i32_32x32x32_i8(fn.af[tm2], fn.bf[tn2], c_in, 0, 0, 0);
+                // pin each MFMA where it is written: left alone, the scheduler sinks it below the FMAs of its region, right in
+                // front of its own first reader, and pays the matrix pipe's latency in wait states every tile
+                __builtin_amdgcn_sched_barrier(0);
                 const v16f biased = __builtin_bit_cast(v16f, isum);   // fast mode: 12582912 +- isum, exactly
                 auto combine = [&](int r) {
                     if (MAGIC) {
@@ -277,7 +283,8 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                 for (int r = 0; r < 8; r++) combine(r);
                 __builtin_amdgcn_sched_barrier(0);
                 if (has_next)
-                    S_n = __builtin_amdgcn_mfma_f32_32x32x16_f16(scale_operand(fn.sa[tm2]), scale_operand(fn.sb[tn2]), zero_f, 0, 0, 0);
+                    S_n = __builtin_amdgcn_mfma_f32_32x32x8f16(scale_operand(fn.sa[tm2]), scale_operand(fn.sb[tn2]), zero_f, 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int r = 8; r < 16; r++) combine(r);
                 if (DUMP) {
