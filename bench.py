@@ -243,6 +243,18 @@ def ops_table(fh, reps=10):
                     rows.append({"op": "gemm", "fmt": name, "M": M, "K": K, "N": N, "us_per_call": round(us, 2),
                                  "int8_ops": 2 * M * K * N})
             w.close()
+    # K-quant GEMVs (matmul_vec_q4_k / matmul_vec_q6_k): random super-blocks with sane fp16 scales
+    rng = np.random.default_rng(5)
+    for ty, name, sbb in ((fh.Q4_K, "Q4_K", 144), (fh.Q6_K, "Q6_K", 210)):
+        for K, N in ((2048, 8192), (8192, 2048), (2048, 128256)):
+            raw = rng.integers(0, 256, (N * K // 256, sbb), dtype=np.uint8)
+            for off in ((0, 2) if ty == fh.Q4_K else (208,)):
+                raw[:, off:off + 2] = rng.normal(0, 0.05, raw.shape[0]).astype(np.float16).view(np.uint8).reshape(-1, 2)
+            w = ops.QWeight(ty, raw.reshape(-1), K, N)
+            x = torch.from_numpy(fh.synth.normal(7, K, 1.0)).cuda()
+            us = timed(lambda: ops.matmul_vec_q(w, x))
+            rows.append({"op": "gemv", "fmt": name, "K": K, "N": N, "us_per_call": round(us, 2), "weight_bytes": N * (K // 256) * sbb})
+            w.close()
     for heads, kvh, hd in ((32, 8, 64), (32, 32, 96)):
         for seq in (801, 1501, 3001):
             q = torch.from_numpy(fh.synth.normal(9, seq * heads * hd, 1.0).reshape(seq, heads * hd)).cuda()

@@ -15,6 +15,7 @@ LIB_PATH = os.path.join(_HERE, "libforge_hip.so")
 
 Q4_0 = 2
 Q8_0 = 8
+Q4_K, Q6_K = 12, 14   # op level only: ops.QWeight + ops.matmul_vec_q
 FLAG_EXACT = 1   # config.flags / op flags: order-faithful f32 arithmetic (bit-identical to the CPU path)
 FLAG_QKV_BIAS = 2   # config.flags: q, k, v projections add a bias vector before RoPE (Qwen2); the blob carries the vectors
 

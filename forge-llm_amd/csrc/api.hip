@@ -16,8 +16,9 @@ int32_t qweight_upload(uint32_t wdtype, const uint8_t* raw_host, uint32_t K, uin
     QWeight w;
     w.wdtype = wdtype; w.K = K; w.N = N; w.owns = true;
     std::vector<uint8_t> qs(w.qs_bytes());
-    std::vector<uint16_t> sc((size_t)N * (K / 32));
-    repack_host(wdtype, raw_host, K, N, qs.data(), sc.data());
+    std::vector<uint16_t> sc((w.scales_bytes() + 1) / 2);
+    if (w.kquant()) repack_kquant_host(wdtype, raw_host, K, N, qs.data(), reinterpret_cast<uint8_t*>(sc.data()));
+    else repack_host(wdtype, raw_host, K, N, qs.data(), sc.data());
     FH_HIP(hipMalloc((void**)&w.qs, std::max<size_t>(qs.size(), 16)));
     hipError_t e = hipMalloc((void**)&w.scales, std::max<size_t>(w.scales_bytes(), 16));
     if (e != hipSuccess) { (void)hipFree(w.qs); return fail(FORGE_HIP_ERR_HIP, "hipMalloc(scales) failed"); }
@@ -107,9 +108,11 @@ int32_t forge_hip_qweight_create(uint32_t wdtype, const uint8_t* raw_host, uint3
                                  forge_hip_qweight** out) {
     FH_CHECK(out, "qweight_create: null out");
     *out = nullptr;
-    FH_CHECK(valid_wdtype(wdtype), "qweight_create: wdtype must be Q8_0 (8) or Q4_0 (2)");
+    const bool kq = wdtype == FORGE_HIP_Q4_K || wdtype == FORGE_HIP_Q6_K;
+    FH_CHECK(valid_wdtype(wdtype) || kq, "qweight_create: wdtype must be Q8_0 (8), Q4_0 (2), Q4_K (12) or Q6_K (14)");
     FH_CHECK(raw_host, "qweight_create: null weights");
     FH_CHECK(K >= 32 && K % 32 == 0 && N >= 1, "qweight_create: K must be a positive multiple of 32 and N >= 1");
+    FH_CHECK(!kq || kquant_k_supported(K), "qweight_create: a K-quant matrix needs K to be a multiple of 256, at most 16384");
     if (forge_hip_device_count() < 1) return fail(FORGE_HIP_ERR_NO_DEVICE, "no HIP device");
     forge_hip_qweight* h = new forge_hip_qweight();
     int32_t rc = qweight_upload(wdtype, raw_host, K, N, &h->w);
@@ -139,7 +142,8 @@ int32_t forge_hip_gemv_q(const forge_hip_qweight* w, const float* x_dev, float* 
     int8_t* q; uint16_t* sc;
     int32_t rc = quantise_into_scratch(x_dev, 1, w->w.K, &q, &sc, (hipStream_t)stream);
     if (rc) return rc;
-    launch_gemv(w->w, q, sc, y_dev, false, GemvOrder::MatmulVec, (hipStream_t)stream);
+    if (w->w.kquant()) launch_gemv_kquant(w->w, q, sc, y_dev, false, (hipStream_t)stream);
+    else launch_gemv(w->w, q, sc, y_dev, false, GemvOrder::MatmulVec, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }
@@ -147,6 +151,7 @@ int32_t forge_hip_gemv_q(const forge_hip_qweight* w, const float* x_dev, float* 
 int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, uint32_t flags,
                          void* stream) {
     FH_CHECK(w && x_dev && y_dev, "gemm_q: null pointer");
+    FH_CHECK(!w->w.kquant(), "gemm_q: K-quant matrices have no batched matmul (the reference runs them through matmul_vec)");
     FH_CHECK((flags & ~FORGE_HIP_FLAG_EXACT) == 0, "gemm_q: unknown flag bits");
     if (M == 0) return FORGE_HIP_OK;
     int8_t* q; uint16_t* sc;
@@ -160,6 +165,7 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
 
 int32_t forge_hip_gemv_q_f32act(const forge_hip_qweight* w, const float* x_dev, float* y_dev, void* stream) {
     FH_CHECK(w && x_dev && y_dev, "gemv_q_f32act: null pointer");
+    FH_CHECK(!w->w.kquant(), "gemv_q_f32act: Q8_0 and Q4_0 matrices only");
     launch_gemv_f32(w->w, x_dev, y_dev, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
@@ -168,6 +174,7 @@ int32_t forge_hip_gemv_q_f32act(const forge_hip_qweight* w, const float* x_dev, 
 int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, uint32_t M, int32_t* out_dev,
                               uint32_t path, void* stream) {
     FH_CHECK(w && x_dev && out_dev, "block_isums: null pointer");
+    FH_CHECK(!w->w.kquant(), "block_isums: Q8_0 and Q4_0 matrices only");
     FH_CHECK(path <= 2, "block_isums: path must be 0 (GEMV kernel), 1 (MFMA GEMM kernel, exact mode) or 2 (MFMA GEMM kernel, fast mode)");
     if (M == 0) return FORGE_HIP_OK;
     int8_t* q; uint16_t* sc;

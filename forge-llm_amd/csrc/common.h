@@ -65,9 +65,12 @@ struct QWeight {
     uint8_t* qs = nullptr;
     uint16_t* scales = nullptr;
     bool owns = false;
-    size_t qs_row_bytes() const { return wdtype == FORGE_HIP_Q8_0 ? K : K / 2; }
+    bool kquant() const { return wdtype == FORGE_HIP_Q4_K || wdtype == FORGE_HIP_Q6_K; }
+    // K-quants (gemv_kquant.hip): qs = nibble bytes (Q4_K, K/2 per row) or low nibbles + high bit pairs (Q6_K, 192 per
+    // super-block); `scales` then points at the second plane (16 / 32 bytes per super-block)
+    size_t qs_row_bytes() const { return wdtype == FORGE_HIP_Q6_K ? (size_t)K / 256 * 192 : wdtype == FORGE_HIP_Q8_0 ? K : K / 2; }
     size_t qs_bytes() const { return (size_t)N * qs_row_bytes(); }
-    size_t scales_bytes() const { return (size_t)N * (K / 32) * 2; }
+    size_t scales_bytes() const { return kquant() ? (size_t)N * (K / 256) * (wdtype == FORGE_HIP_Q4_K ? 16 : 32) : (size_t)N * (K / 32) * 2; }
 };
 
 // Split raw GGUF rows into the two planes (host side).
@@ -133,6 +136,11 @@ void launch_gemv_norm_silu_quant(const QWeight& wgu, const float* x, const float
 // gemv_f32.hip — the reference's portable row dot (f32 activations x weights dequantised on the fly, one sequential sum
 // per row): y[n] = sum_k x[k] * (f32(q[n][k]) * w_s[n][k/32]).
 void launch_gemv_f32(const QWeight& w, const float* x, float* y, hipStream_t s);
+
+// gemv_kquant.hip — matmul_vec_q4_k / matmul_vec_q6_k: Q8_0-quantised activations against 256-element super-blocks.
+void repack_kquant_host(uint32_t wdtype, const uint8_t* raw, uint32_t K, uint64_t N, uint8_t* qs, uint8_t* meta);
+bool kquant_k_supported(uint32_t K);
+void launch_gemv_kquant(const QWeight& w, const int8_t* aq, const uint16_t* as, float* y, bool accumulate, hipStream_t s);
 
 // gemm.hip — y[m][n] (=|+=) ...; aq int8 [M][K], as fp16 [M][K/32].  isums (optional) int32 [M][N][K/32].
 // exact: unfused multiply/add per block (bit-identical to the CPU path); otherwise one FMA per block, and then the

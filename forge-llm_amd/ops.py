@@ -96,7 +96,9 @@ class QWeight:
         from . import check, lib, require_gpu
         require_gpu()
         raw = np.ascontiguousarray(raw, dtype=np.uint8)
-        if raw.size != N * (K // 32) * block_bytes(wdtype):
+        # Q8_0 / Q4_0: 34- / 18-byte blocks of 32; Q4_K (12) / Q6_K (14): 144- / 210-byte super-blocks of 256
+        expect = N * (K // 256) * {12: 144, 14: 210}[wdtype] if wdtype in (12, 14) else N * (K // 32) * block_bytes(wdtype)
+        if raw.size != expect:
             raise ValueError("raw weight bytes do not match N x K")
         self.wdtype, self.K, self.N = wdtype, K, N
         self._lib = lib()

@@ -48,6 +48,8 @@ extern "C" {
 
 #define FORGE_HIP_Q4_0 2u /* GGML type ids, crates/forgellm-frontend/src/gguf.rs:207-258 */
 #define FORGE_HIP_Q8_0 8u
+#define FORGE_HIP_Q4_K 12u /* op level only: forge_hip_qweight_create + forge_hip_gemv_q */
+#define FORGE_HIP_Q6_K 14u
 
 /* Mirrors the fields of ModelConfig (crates/forgellm-frontend/src/ir.rs:484-519) that the
  * code generators read. */
@@ -150,7 +152,10 @@ int32_t forge_hip_dequant(uint32_t wdtype, const uint8_t* data_host, uint64_t n,
 /* ---------------- op-level API ---------------- */
 
 /* Upload one weight matrix given as raw GGUF blocks, row-major [N][K/32] (the `weight: &[u8]`
- * argument of matmul_vec_q8_0_KxN, emit.rs:1958).  K must be a multiple of 32. */
+ * argument of matmul_vec_q8_0_KxN, emit.rs:1958).  K must be a multiple of 32.
+ * wdtype FORGE_HIP_Q4_K / FORGE_HIP_Q6_K: raw 144- / 210-byte super-blocks, row-major [N][K/256] (the `weight` argument of
+ * matmul_vec_q4_k_KxN / matmul_vec_q6_k_KxN, emit.rs:3411, 3636); K a multiple of 256, at most 16384.  Such a handle is
+ * taken by forge_hip_gemv_q only: the reference has no batched matmul for these formats. */
 int32_t forge_hip_qweight_create(uint32_t wdtype, const uint8_t* raw_host, uint32_t K, uint32_t N,
                                  forge_hip_qweight** out);
 void forge_hip_qweight_destroy(forge_hip_qweight* w);
@@ -161,7 +166,8 @@ int32_t forge_hip_quantize_act(const float* x_dev, uint32_t M, uint32_t K, int8_
                                void* stream);
 
 /* matmul_vec_q8_0_KxN / matmul_vec_q4_0_KxN (emit.rs:1926-2092, 2797-2958): y[N] = W x.
- * x_dev f32 [K], y_dev f32 [N]. */
+ * x_dev f32 [K], y_dev f32 [N].  For a Q4_K / Q6_K handle: matmul_vec_q4_k_KxN / matmul_vec_q6_k_KxN (emit.rs:3388-3490,
+ * 3622-3655; dots emit.rs:3035-3306, 3553-3612), bit-identical f32. */
 int32_t forge_hip_gemv_q(const forge_hip_qweight* w, const float* x_dev, float* y_dev, void* stream);
 
 /* The same matmul in the arithmetic the reference runs on hosts other than aarch64: its portable dot_q8_0 / dot_q4_0

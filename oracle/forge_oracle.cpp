@@ -697,7 +697,103 @@ uint32_t argmax_last(const float* v, int64_t n) {
 // Model (emit.rs:3875-4019 Weights/LayerWeights/KVCache; blob layout project.rs:342-407,
 // writer order crates/forgellm-cli/src/main.rs:2714-2757).
 // ---------------------------------------------------------------------------------------
+// ---- K-quant row dots (emit.rs:2978-3310 Q4_K, emit.rs:3508-3615 Q6_K) ---------------------------------------------------
+// Both take the SAME Q8_0-quantised activation blocks as the Q8_0/Q4_0 dots (one 32-element block per 32 weights) and
+// are one arithmetic on every host: the aarch64 forms (sdot, one row or four rows at a time, emit.rs:3035-3243) compute
+// the same integers and combine them with the same f32 operations in the same order as the scalar forms restated here.
+
+// get_scale_min_k4, emit.rs:3013-3021.
+static inline void scale_min_k4(int j, const uint8_t* sc, int* scale, int* mn) {
+    if (j < 4) { *scale = sc[j] & 63; *mn = sc[j + 4] & 63; }
+    else { *scale = (sc[j + 4] & 0x0F) | ((sc[j - 4] >> 6) << 4); *mn = (sc[j + 4] >> 4) | ((sc[j] >> 6) << 4); }
+}
+
+// dot_q4_k_q8_0, emit.rs:3246-3306: per 256-element super-block (144 bytes: d, dmin, 12 bytes of 6-bit scales and
+// minima, 128 bytes of nibbles), four chunks of 32 bytes; a chunk's low nibbles are sub-block 2c, its high nibbles
+// sub-block 2c+1;  acc += x_scale * (d*sc * dot - dmin*m * sum)  for the one, then for the other.
+float dot_q4_k(const uint8_t* a_q8, const uint8_t* w, int64_t k) {
+    const int64_t num_sb = k / 256;
+    float acc = 0.0f;
+    for (int64_t sb = 0; sb < num_sb; sb++) {
+        const uint8_t* blk = w + sb * 144;
+        const float d = f16_to_f32(rd16(blk)), dmin = f16_to_f32(rd16(blk + 2));
+        const uint8_t* scales = blk + 4;
+        const uint8_t* qs = blk + 16;
+        for (int chunk = 0; chunk < 4; chunk++) {
+            const int is = chunk * 2;
+            int sc1, m1, sc2, m2;
+            scale_min_k4(is, scales, &sc1, &m1);
+            scale_min_k4(is + 1, scales, &sc2, &m2);
+            const float d1_w = d * (float)sc1, m1_w = dmin * (float)m1, d2_w = d * (float)sc2, m2_w = dmin * (float)m2;
+            const uint8_t* qc = qs + chunk * 32;
+            const uint8_t* x1 = a_q8 + (sb * 8 + is) * Q8_BYTES;
+            const uint8_t* x2 = a_q8 + (sb * 8 + is + 1) * Q8_BYTES;
+            const float x1_scale = f16_to_f32(rd16(x1)), x2_scale = f16_to_f32(rd16(x2));
+            int32_t dot1 = 0, sum1 = 0, dot2 = 0, sum2 = 0;
+            for (int i = 0; i < 32; i++) {
+                const int xi = (int8_t)x1[2 + i];
+                dot1 += xi * (qc[i] & 0x0F);
+                sum1 += xi;
+            }
+            acc += x1_scale * (d1_w * (float)dot1 - m1_w * (float)sum1);
+            for (int i = 0; i < 32; i++) {
+                const int xi = (int8_t)x2[2 + i];
+                dot2 += xi * (qc[i] >> 4);
+                sum2 += xi;
+            }
+            acc += x2_scale * (d2_w * (float)dot2 - m2_w * (float)sum2);
+        }
+    }
+    return acc;
+}
+
+// dot_q6_k_q8_0, emit.rs:3553-3612: per super-block (210 bytes: 128 of low nibbles, 64 of high bit pairs, 16 int8 scales,
+// d) eight activation blocks; block b takes its 32 six-bit values (minus 32) from the table's nibble and bit-pair fields,
+// 16 under scale 2b and 16 under scale 2b+1;  acc += d * x_scale * (sc_lo * dot_lo + sc_hi * dot_hi).
+float dot_q6_k(const uint8_t* a_q8, const uint8_t* w, int64_t k) {
+    static const int T[8][5] = {{0, 0, 0, 0, 0}, {32, 0, 0, 2, 2}, {0, 0, 4, 4, 4}, {32, 0, 4, 6, 6},
+                                {64, 32, 0, 0, 8}, {96, 32, 0, 2, 10}, {64, 32, 4, 4, 12}, {96, 32, 4, 6, 14}};
+    const int64_t num_sb = k / 256;
+    float acc = 0.0f;
+    for (int64_t sb = 0; sb < num_sb; sb++) {
+        const uint8_t* blk = w + sb * 210;
+        const uint8_t* ql = blk;
+        const uint8_t* qh = blk + 128;
+        const int8_t* scales = reinterpret_cast<const int8_t*>(blk + 192);
+        const float d = f16_to_f32(rd16(blk + 208));
+        for (int b = 0; b < 8; b++) {
+            const uint8_t* x = a_q8 + (sb * 8 + b) * Q8_BYTES;
+            const float x_scale = f16_to_f32(rd16(x));
+            const int sc_lo = scales[T[b][4]], sc_hi = scales[T[b][4] + 1];
+            int32_t dot_lo = 0, dot_hi = 0;
+            for (int l = 0; l < 32; l++) {
+                const int q6 = (((ql[T[b][0] + l] >> T[b][2]) & 0x0F) | (((qh[T[b][1] + l] >> T[b][3]) & 0x03) << 4)) - 32;
+                const int xi = (int8_t)x[2 + l];
+                if (l < 16) dot_lo += q6 * xi; else dot_hi += q6 * xi;
+            }
+            acc += d * x_scale * ((float)sc_lo * (float)dot_lo + (float)sc_hi * (float)dot_hi);
+        }
+    }
+    return acc;
+}
+
+// matmul_vec_q4_k_KxN / matmul_vec_q6_k_KxN (emit.rs:3388-3490, 3622-3655): quantise the input once, one dot per row.
+void matmul_vec_kquant(int ggml_type, float* out, const float* in, const uint8_t* w, int64_t k, int64_t n) {
+    std::vector<uint8_t> a_q8((size_t)(k / QK * Q8_BYTES));
+    quantize_act_q8_0(in, k, a_q8.data());
+    const int64_t row_bytes = k / 256 * (ggml_type == 12 ? 144 : 210);
+#pragma omp parallel for schedule(static)
+    for (int64_t r = 0; r < n; r++)
+        out[r] = ggml_type == 12 ? dot_q4_k(a_q8.data(), w + r * row_bytes, k) : dot_q6_k(a_q8.data(), w + r * row_bytes, k);
+}
+
 extern "C" {
+float fo_dot_kquant(int ggml_type, const uint8_t* a_q8, const uint8_t* w, int64_t k) {
+    return ggml_type == 12 ? dot_q4_k(a_q8, w, k) : dot_q6_k(a_q8, w, k);
+}
+void fo_matmul_vec_kquant(int ggml_type, float* out, const float* in, const uint8_t* w, int64_t k, int64_t n) {
+    matmul_vec_kquant(ggml_type, out, in, w, k, n);
+}
 
 struct fo_config {
     uint32_t hidden, inter, layers, heads, kv_heads, head_dim, vocab, max_seq;

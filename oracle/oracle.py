@@ -168,6 +168,24 @@ def matmul_vec(wdtype, variant, x, w, k, n):
     return out
 
 
+def dot_kquant(ggml_type, a_q8, w, k):
+    """dot_q4_k_q8_0 (ggml_type 12) / dot_q6_k_q8_0 (14) of a weight row with Q8_0-quantised activation blocks."""
+    L = lib()
+    L.fo_dot_kquant.restype = C.c_float
+    L.fo_dot_kquant.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64]
+    return float(L.fo_dot_kquant(ggml_type, _p(_u8(a_q8)), _p(_u8(w)), k))
+
+
+def matmul_vec_kquant(ggml_type, x, w, k, n):
+    """matmul_vec_q4_k_KxN / matmul_vec_q6_k_KxN: quantise x to Q8_0 blocks, one dot per row."""
+    L = lib()
+    L.fo_matmul_vec_kquant.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64]
+    x, w = _f32(x), _u8(w)
+    out = np.empty(n, np.float32)
+    L.fo_matmul_vec_kquant(ggml_type, _p(out), _p(x), _p(w), k, n)
+    return out
+
+
 def matmul_mat(wdtype, variant, x, w, m, k, n):
     x, w = _f32(x), _u8(w)
     out = np.empty((m, n), np.float32)

@@ -124,6 +124,35 @@ def test_matmul_vec_portable_dot_bit_exact(fh, oracle, torch_gpu, wd, K, N):
         assert not np.array_equal(ya, want)
 
 
+def random_superblocks(ty, n, seed):
+    """Random K-quant super-blocks with sane fp16 scale fields (every other bit pattern is a valid block)."""
+    rng = np.random.default_rng(seed)
+    b = rng.integers(0, 256, (n, {12: 144, 14: 210}[ty]), dtype=np.uint8)
+    for off in {12: (0, 2), 14: (208,)}[ty]:
+        b[:, off:off + 2] = rng.normal(0, 0.05, n).astype(np.float16).view(np.uint8).reshape(n, 2)
+    return b.reshape(-1)
+
+
+@pytest.mark.parametrize("ty", [12, 14])
+@pytest.mark.parametrize("K,N", [(256, 3), (2048, 512), (2048, 2048), (8192, 300), (3072, 1029), (4096, 64)])
+def test_matmul_vec_kquant_bit_exact(fh, oracle, torch_gpu, ty, K, N):
+    """matmul_vec_q4_k / matmul_vec_q6_k (emit.rs:3388-3490, 3622-3655): exact sub-block integers and the reference's one
+    f32 order per row, so the bits are the oracle's (whose dots are held to a float64 evaluation of the dequantised
+    operands in tests/test_oracle_math.py)."""
+    torch = torch_gpu
+    wraw = random_superblocks(ty, N * K // 256, seed=ty * 1000 + K + N)
+    x = fh.synth.normal(23 + K, K, 1.0)
+    x[:32] = 0.0                                             # an all-zero activation block
+    w = fh.ops.QWeight(ty, wraw, K, N)
+    y = fh.ops.matmul_vec_q(w, torch.from_numpy(x).cuda()).cpu().numpy()
+    same_bits(y, oracle.matmul_vec_kquant(ty, x, wraw, K, N))
+    with pytest.raises(fh.ForgeHipError):
+        fh.ops.matmul_mat_q(w, torch.from_numpy(np.stack([x, x])).cuda())       # no batched matmul for these formats
+    w.close()
+    with pytest.raises(fh.ForgeHipError):
+        fh.ops.QWeight(ty, random_superblocks(ty, 1, 1), 288, 1)                # K must be a multiple of 256
+
+
 @pytest.mark.parametrize("wd", [Q8, Q4])
 @pytest.mark.parametrize("M,K,N", [(1, 2048, 512), (37, 576, 960), (352, 2048, 2048), (130, 8192, 320), (129, 3072, 256)])
 def test_matmul_mat_parity(fh, oracle, torch_gpu, wd, M, K, N):

@@ -355,3 +355,72 @@ def test_model_prefill_batched_equals_token_loop(oracle, fh, wd, variant, kv):
     assert not np.allclose(other, batched)
     with pytest.raises(ValueError):
         oracle.Model(cfg, blob[:-1], variant, kv)
+
+
+# ---------------- K-quant row dots (emit.rs:3035-3306 Q4_K, 3553-3612 Q6_K) ----------------
+def _superblocks(ty, n, seed):
+    rng = np.random.default_rng(seed)
+    b = rng.integers(0, 256, (n, {12: 144, 14: 210}[ty]), dtype=np.uint8)
+    for off in {12: (0, 2), 14: (208,)}[ty]:
+        b[:, off:off + 2] = rng.normal(0, 0.05, n).astype(np.float16).view(np.uint8).reshape(n, 2)
+    return b.reshape(-1)
+
+
+@pytest.mark.parametrize("ty", [12, 14])
+@pytest.mark.parametrize("K", [256, 1024, 4096])
+def test_kquant_dots_against_fp64_of_the_dequantised_operands(oracle, ty, K):
+    """The reference has no test that runs dot_q4_k_q8_0 / dot_q6_k_q8_0.  What pins the restatement: the dot of a
+    K-quant row with Q8_0 activation blocks is, up to f32 rounding, the float64 dot of the two DEQUANTISED vectors, and
+    both dequantisers are held to the reference's own block fixtures (tests/test_gguf.py).  A wrong nibble or bit-pair
+    field, scale index, minimum term or block order moves the result by its own magnitude."""
+    from oracle import gguf_oracle as go
+    w = _superblocks(ty, K // 256, seed=ty + K)
+    x = np.random.default_rng(K).normal(0, 1, K).astype(np.float32)
+    aq = oracle.quantize_act(x)
+    got = oracle.dot_kquant(ty, aq, w, K)
+    wd = go.dequant_ggml(oracle, ty, w, K).astype(np.float64)
+    xd = oracle.dequant(Q8, aq, K).astype(np.float64)
+    assert abs(got - float(np.dot(wd, xd))) <= 2e-6 * float(np.sum(np.abs(wd * xd)))
+
+
+@pytest.mark.parametrize("ty", [12, 14])
+def test_kquant_dot_special_cases(oracle, ty):
+    """One super-block by hand.  Q4_K with every nibble c, sub-block scales sc and minima m:  x_s * (d sc c - dmin m) * sum(xq)
+    per sub-block; Q6_K with every 6-bit value v and scales s:  d x_s s (v - 32) * sum(xq) per block.  Zero activations
+    give exactly 0 whatever the weights."""
+    K = 256
+    x = np.tile(np.arange(1, 33, dtype=np.float32), 8)                 # every block the same codes, scale 32/127
+    aq = oracle.quantize_act(x)
+    codes = oracle.dequant(Q8, aq, K) / np.float32(oracle.f16_to_f32(np.frombuffer(aq[:2].tobytes(), np.uint16))[0])
+    sumq = float(np.round(codes[:32]).sum())
+    xs = float(oracle.f16_to_f32(np.frombuffer(aq[:2].tobytes(), np.uint16))[0])
+    if ty == 12:
+        blk = np.zeros(144, np.uint8)
+        blk[0:2] = np.frombuffer(np.float16(0.5).tobytes(), np.uint8)   # d
+        blk[2:4] = np.frombuffer(np.float16(0.25).tobytes(), np.uint8)  # dmin
+        blk[4:8] = 3                                                    # scales of sub-blocks 0..3 (j < 4: low 6 bits)
+        blk[8:12] = 2                                                   # minima of sub-blocks 0..3
+        blk[12:16] = 3 | (2 << 4)                                       # sub-blocks 4..7: scale low nibble, minimum high nibble
+        blk[16:144] = 0x55                                              # every nibble 5
+        want = 8 * xs * (0.5 * 3 * 5 * sumq - 0.25 * 2 * sumq)
+    else:
+        blk = np.zeros(210, np.uint8)
+        blk[0:128] = 0x99                                               # low nibbles 9
+        blk[128:192] = 0xAA                                             # bit pairs 2: v = 9 | 2 << 4 = 41
+        blk[192:208] = np.array([7], np.int8).view(np.uint8)[0]         # scales
+        blk[208:210] = np.frombuffer(np.float16(0.125).tobytes(), np.uint8)
+        want = 8 * 0.125 * xs * 7 * (41 - 32) * sumq
+    got = oracle.dot_kquant(ty, aq, blk, K)
+    assert abs(got - want) <= 1e-5 * abs(want)
+    assert oracle.dot_kquant(ty, oracle.quantize_act(np.zeros(K, np.float32)), _superblocks(ty, 1, 3), K) == 0.0
+
+
+@pytest.mark.parametrize("ty", [12, 14])
+def test_matmul_vec_kquant_is_one_dot_per_row(oracle, ty):
+    K, N = 512, 5
+    w = _superblocks(ty, N * K // 256, seed=9)
+    x = np.random.default_rng(4).normal(0, 1, K).astype(np.float32)
+    rb = K // 256 * {12: 144, 14: 210}[ty]
+    aq = oracle.quantize_act(x)
+    want = np.array([oracle.dot_kquant(ty, aq, w[r * rb:(r + 1) * rb], K) for r in range(N)], np.float32)
+    assert np.array_equal(oracle.matmul_vec_kquant(ty, x, w, K, N).view(np.uint32), want.view(np.uint32))
