@@ -17,6 +17,36 @@
  *  - Arithmetic: activations are quantised per 32-element block to int8 exactly as
  *    emit.rs:1410-1440, block dot products are exact int32 (emit.rs:1543-1553,
  *    2522-2552), the per-block combine and everything else is f32.  KV cache is fp16.
+ *
+ * Supported envelope (anything outside it is refused with FORGE_HIP_ERR_INVALID and a message, never
+ * computed wrongly):
+ *  - model API: projection and lm_head weights Q8_0 or Q4_0; hidden a multiple of 32 in [32, 16352];
+ *    inter and heads*head_dim multiples of 32, at most 16384; head_dim 64, 96 or 128; heads a multiple
+ *    of kv_heads, at most 256; FORGE_HIP_FLAG_EXACT needs max_seq > 512 (below that the reference runs
+ *    its non-flash attention, which has no order-faithful kernel here) and, with a sliding window,
+ *    min(sliding_window, max_seq) <= 12288.  forge_hip_prefill_batch takes any n up to the free cache;
+ *    it works through the prompt in chunks of at most 4096 rows, so its scratch does not grow with n.
+ *  - op-level API: K a multiple of 32, at most 16384 (K-quants: a multiple of 256); M and S bounded
+ *    only by memory; head_dim as above.
+ *
+ * Device memory and threads
+ *  - A model allocates all its device buffers in forge_hip_model_create (weights, KV cache for max_seq,
+ *    activations for one prefill chunk); later calls allocate no device memory (the kernel-sequence
+ *    decode path instantiates its HIP graph at the first decode step).
+ *  - The op-level calls keep three process-wide scratch areas (quantised activations, attention / argmax
+ *    partial results, RoPE tables) that GROW ON DEMAND: a call that needs more than any earlier call
+ *    did frees the old area, which waits for the device, and allocates a larger one (hipFree +
+ *    hipMalloc on the call path).  They are shared by all streams and not locked: use the
+ *    op-level API from one thread and one stream at a time, and call the largest shape once at start-up
+ *    if the allocation must not happen later.  forge_hip_attn_decode_f16kv_noalloc is the one op-level
+ *    call that never allocates.
+ *  - The one-kernel decode step (forge_hip_model_decode_launches() == 1) runs one workgroup per compute
+ *    unit and its workgroups wait on each other's results, so all of them must be resident at once:
+ *    the library assumes that the process has the GPU to itself.  If another process or another
+ *    stream of this process holds compute units for long enough, the kernel's bounded wait expires,
+ *    the call returns FORGE_HIP_ERR_HIP with the model's position and repeat counts unchanged, and the
+ *    caller may repeat it or set FORGE_HIP_PERSIST=0 before model_create to use the kernel sequence,
+ *    which has no such requirement.
  */
 #ifndef FORGE_HIP_H
 #define FORGE_HIP_H
