@@ -53,6 +53,7 @@ struct Scratch {
 Scratch g_act;    // quantised activations: codes then scales
 Scratch g_attn;   // decode-attention partials / argmax partials
 Scratch g_rope;   // cos | sin tables
+Scratch g_gemm;   // partial tiles and counters of the GEMM's K-range variant
 
 inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
@@ -158,7 +159,15 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
     const bool exact = (flags & FORGE_HIP_FLAG_EXACT) != 0;
     int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream, !exact);   // the fast kernel takes odd blocks negated
     if (rc) return rc;
-    launch_gemm(w->w, q, sc, M, y_dev, w->w.N, false, exact, nullptr, (hipStream_t)stream);
+    // large fast-mode problems may cut left-over tiles along K: that kernel parks partial tiles in a workspace
+    void* split_ws = nullptr;
+    if (!exact && (uint64_t)((M + 127) / 128) * ((w->w.N + 127) / 128) > 256) {
+        const bool fresh = g_gemm.cap < gemm_split_workspace_bytes();
+        if ((rc = g_gemm.reserve(gemm_split_workspace_bytes()))) return rc;
+        if (fresh) FH_HIP(hipMemset(g_gemm.p, 0, gemm_split_workspace_bytes()));   // its counters start at zero and are left at zero
+        split_ws = g_gemm.p;
+    }
+    launch_gemm(w->w, q, sc, M, y_dev, w->w.N, false, exact, nullptr, (hipStream_t)stream, split_ws);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }

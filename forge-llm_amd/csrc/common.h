@@ -145,8 +145,12 @@ void launch_gemv_kquant(const QWeight& w, const int8_t* aq, const uint16_t* as, 
 // gemm.hip — y[m][n] (=|+=) ...; aq int8 [M][K], as fp16 [M][K/32].  isums (optional) int32 [M][N][K/32].
 // exact: unfused multiply/add per block (bit-identical to the CPU path); otherwise one FMA per block, and then the
 // activation codes of every row's odd blocks must come negated (the neg_odd flag of the quantising launchers).
+// split_ws (optional, gemm_split_workspace_bytes() bytes, its last KB zero before the first use and left zero by every
+// launch): lets the fast mode cut the tiles that do not fill a whole round of CUs along K; launches that share a
+// workspace must be ordered (one stream).  With it a row's low bits may depend on where in the batch the row sits.
+size_t gemm_split_workspace_bytes();
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
-                 bool accumulate, bool exact, int32_t* isums, hipStream_t s);
+                 bool accumulate, bool exact, int32_t* isums, hipStream_t s, void* split_ws = nullptr);
 
 // model.hip — the part of forge_hip_model_create's checks that sizes depend on (formats, dimensions the kernels cover);
 // sets the error message.

@@ -55,6 +55,7 @@ constexpr int LDS_A = 0, LDS_B = 2 * TILE_BYTES, LDS_ASC = 4 * TILE_BYTES, LDS_B
 constexpr uint32_t MAGIC_BITS = 0x4B400000u;  // 12582912.0f = 1.5 * 2^23: ulp 1, room for +-2^22
 constexpr uint32_t RSRC_FLAGS = 0x00020000;   // raw buffer, 32-bit data format
 constexpr uint32_t OOB = 0x80000000u;         // an offset no descriptor here covers
+constexpr uint32_t GEMM_SPLIT_MAX_ITEMS = 256; // K ranges one launch may park in the split workspace (64 KB each)
 
 #define FH_LDS3(p) ((__attribute__((address_space(3))) void*)(p))
 
@@ -66,19 +67,49 @@ __device__ __forceinline__ uint32_t nib_minus8(uint32_t x) {
 // EXACT: multiply then add per block (bit-identical to the CPU path); otherwise one FMA per block.
 // TM: 32-row tiles per wave along m.  2 = the 128-row workgroup tile; 1 = a 64-row tile for problems so small that even
 // twice the workgroups leave CUs idle (a workgroup's time per K stage halves with its tile).
-template <bool Q4, bool DUMP, bool EXACT, int TM>
+// SPLIT (fast mode only): a one-dimensional grid of work items.  The first `full_tiles` output tiles (row-major over the
+// tile grid) are worked over the whole of K by one workgroup each, as in the other variants; each of the remaining tiles
+// is cut into `split` ranges of `stages_per_part` K stages, one workgroup per range, whose partial tiles go to
+// `partials`; the workgroup that finishes a tile's last range adds the ranges in range order (so the result does not
+// depend on who came last) and stores the tile.  The launch code uses it when the tiles fill the CUs once and a fraction:
+// the fraction is what gets cut, so that every CU ends up with the same amount of work.
+struct GemmSplit {
+    uint32_t full_tiles, split, stages_per_part;
+    float* partials;        // [tiles - full_tiles][split][tile elements]
+    uint32_t* counters;     // [tiles - full_tiles], zero between launches
+};
+
+template <bool Q4, bool DUMP, bool EXACT, int TM, bool SPLIT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ wsc, const int8_t* __restrict__ aq,
                    const uint16_t* __restrict__ asc, float* __restrict__ y, int32_t* __restrict__ isums, uint32_t M,
-                   uint32_t N, uint32_t K, uint32_t ldy, int accumulate) {
+                   uint32_t N, uint32_t K, uint32_t ldy, int accumulate, GemmSplit sp) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr bool MAGIC = !EXACT;               // DUMP && !EXACT: the fast arithmetic, with its block sums written out too
+    static_assert(!SPLIT || (MAGIC && !DUMP), "K ranges change the order of the block sum: fast mode only");
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // uniform: the compiler keeps it scalar
     const uint32_t wm = wave >> 1, wn = wave & 1;
     constexpr int WM = 32 * TM;                  // rows of a wave's tile
-    const uint32_t m0 = blockIdx.y * (2 * WM), n0 = blockIdx.x * BN;
+    const uint32_t stages = (K + BK - 1) / BK;
+    uint32_t tile_x = blockIdx.x, tile_y = blockIdx.y, s_begin = 0, s_end = stages;
+    bool ranged = false;                         // this workgroup holds one K range of its tile
+    uint32_t range_tile = 0;                     // index of the tile among the cut ones
+    if (SPLIT) {
+        const uint32_t gx = (N + BN - 1) / BN;
+        uint32_t tile = blockIdx.x;
+        if (tile >= sp.full_tiles) {
+            const uint32_t r = tile - sp.full_tiles;
+            range_tile = r / sp.split;
+            tile = sp.full_tiles + range_tile;
+            s_begin = (r % sp.split) * sp.stages_per_part;       // even: the bias is taken out per pair of stages
+            s_end = s_begin + sp.stages_per_part < stages ? s_begin + sp.stages_per_part : stages;
+            ranged = true;
+        }
+        tile_x = tile % gx; tile_y = tile / gx;
+    }
+    const uint32_t m0 = tile_y * (2 * WM), n0 = tile_x * BN;
     const uint32_t nblk = K / 32;
     const uint32_t lrow = lane & 31, lhalf = lane >> 5;
     const uint32_t wrow = Q4 ? K / 2 : K;   // bytes of one weight row
@@ -230,9 +261,8 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         for (int r = 0; r < 16; r++) c_in[r] = (int)MAGIC_BITS;
     }
 
-    const uint32_t stages = (K + BK - 1) / BK;
-    issue_stage(0, 0);
-    commit_stage(0, 0, 0);
+    issue_stage(s_begin * BK, 0);
+    commit_stage(0, s_begin & 3, s_begin * KB);
     __builtin_amdgcn_s_waitcnt(0);      // vmcnt(0): the tiles of stage 0 are in LDS
     __syncthreads();
 
@@ -317,7 +347,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     // the 8 blocks left of the bias: 12582912 * sum_b a_s[m][b] * (+-w_s[n][b]), the sum being one f16 MFMA.
     const uint32_t ta_off = lhalf ? (uint32_t)LDS_ZERO : LDS_ASC + (wm * WM + lrow) * SC_ROW;
     const uint32_t tb_off = lhalf ? (uint32_t)LDS_ZERO : LDS_BSC + (wn * 64 + lrow) * SC_ROW;
-    for (uint32_t s = 0; s < stages; s += 2) {
+    for (uint32_t s = s_begin; s < s_end; s += 2) {
         run_stage(s, 0);
         run_stage(s + 1, 1);
         if (MAGIC) {
@@ -347,6 +377,40 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         }
     }
 
+    if (SPLIT && ranged) {
+        // Park this range's tile (thread-major: element e of thread t at [e][t], the same mapping in every workgroup).
+        // Partial tiles cross between CUs whose L2 caches do not see each other's lines, so they travel as device-scope
+        // (write-through / cache-bypassing) stores and loads rather than behind device-scope fences, which would write
+        // back and invalidate a whole L2 per workgroup: the stores are waited for, then counted, and the workgroup that
+        // counts last reads them all.
+        constexpr uint32_t TILE_ELEMS = TM * 2 * 16 * 256;
+        float* mine = sp.partials + ((size_t)range_tile * sp.split + s_begin / sp.stages_per_part) * TILE_ELEMS;
+#pragma unroll
+        for (int e = 0; e < TM * 2 * 16; e++)
+            __hip_atomic_store(mine + e * 256 + tid, acc[e / 32][(e / 16) & 1][e & 15], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");   // for the compiler: the stores stay above this line
+        __builtin_amdgcn_s_waitcnt(0);                           // vmcnt(0): they have been acknowledged
+        __syncthreads();
+        __shared__ uint32_t arrived;
+        if (tid == 0) arrived = __hip_atomic_fetch_add(sp.counters + range_tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();
+        if (arrived != sp.split - 1) return;      // whole workgroup: not the last range of this tile
+        const float* all = sp.partials + (size_t)range_tile * sp.split * TILE_ELEMS;
+        // ranges in K order, whoever arrived last; a whole range's loads in flight at a time
+        for (uint32_t p = 0; p < sp.split; p++) {
+            float part[TM * 2 * 16];
+#pragma unroll
+            for (int e = 0; e < TM * 2 * 16; e++)
+                part[e] = __hip_atomic_load(all + (size_t)p * TILE_ELEMS + e * 256 + tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+#pragma unroll
+            for (int e = 0; e < TM * 2 * 16; e++) {
+                float& dst = acc[e / 32][(e / 16) & 1][e & 15];
+                dst = p == 0 ? part[e] : dst + part[e];
+            }
+        }
+        if (tid == 0) __hip_atomic_store(sp.counters + range_tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch (stream order)
+    }
+
     // epilogue: lane holds column n = lrow, rows 8g + 4*lhalf + (r&3); the descriptor drops rows >= M
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc((void*)y, 0, M * ldy * 4, RSRC_FLAGS);
 #pragma unroll
@@ -369,8 +433,10 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
 
 // The kernel addresses each matrix with 32-bit byte offsets below 2^31: larger problems are cut into
 // row ranges of the activations and of the weights, one launch each.
+size_t gemm_split_workspace_bytes() { return (size_t)GEMM_SPLIT_MAX_ITEMS * BM * BN * sizeof(float) + GEMM_SPLIT_MAX_ITEMS * sizeof(uint32_t); }
+
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
-                 bool accumulate, bool exact, int32_t* isums, hipStream_t s) {
+                 bool accumulate, bool exact, int32_t* isums, hipStream_t s, void* split_ws) {
     if (M == 0 || w.N == 0) return;
     const int accf = accumulate ? 1 : 0;
     const bool q4 = w.wdtype == FORGE_HIP_Q4_0;
@@ -394,7 +460,7 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
         (void)lds_ok;                                                                                                   \
         dim3 grid((nc + BN - 1) / BN, (mc + 64 * TM_ - 1) / (64 * TM_));                                                \
         fh::launch(gemm_q_kernel<Q4_, DUMP_, EXACT_, TM_>, grid, 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c, y_c, is_c, \
-                   mc, nc, w.K, ldy, accf);                                                                             \
+                   mc, nc, w.K, ldy, accf, GemmSplit{});                                                                \
     } while (0)
 #define FH_GEMM_LAUNCH(Q4_, DUMP_, EXACT_)                         \
     do {                                                           \
@@ -415,6 +481,36 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
             // halves with its tile, and a larger tile would only leave more CUs idle
             const uint64_t tiles64 = (uint64_t)((nc + BN - 1) / BN) * ((mc + 63) / 64);
             const bool small_tiles = tiles64 <= (uint64_t)cus && mc > 64;
+            // 128-row tiles that fill the CUs a few times and a fraction (fast mode, caller gave a workspace): the
+            // tiles of the fraction are cut along K so that they spread over all CUs
+            if (split_ws && !exact && !isums && !small_tiles && mc == M && nc == w.N) {
+                const uint32_t tiles = ((nc + BN - 1) / BN) * ((mc + BM - 1) / BM), stages = (w.K + BK - 1) / BK;
+                const uint32_t rem = tiles % (uint32_t)cus;
+                uint32_t split = rem ? std::min<uint32_t>({(uint32_t)cus / rem, 8u, stages / 2, GEMM_SPLIT_MAX_ITEMS / rem}) : 0;
+                if (tiles > (uint32_t)cus && tiles / (uint32_t)cus < 4 && split >= 2) {
+                    GemmSplit sp{};
+                    sp.stages_per_part = ((stages + split - 1) / split + 1) & ~1u;
+                    sp.split = (stages + sp.stages_per_part - 1) / sp.stages_per_part;
+                    sp.full_tiles = tiles - rem;
+                    sp.partials = reinterpret_cast<float*>(split_ws);
+                    sp.counters = reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(split_ws) + (size_t)GEMM_SPLIT_MAX_ITEMS * BM * BN * sizeof(float));
+                    if (sp.split >= 2) {
+                        const uint32_t items = sp.full_tiles + rem * sp.split;
+#define FH_GEMM_LAUNCH_SPLIT(Q4_)                                                                                            \
+    do {                                                                                                                    \
+        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, false, false, 2, true>,       \
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES);   \
+        (void)lds_ok;                                                                                                       \
+        fh::launch(gemm_q_kernel<Q4_, false, false, 2, true>, dim3(items), 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c, y_c, \
+                   is_c, mc, nc, w.K, ldy, accf, sp);                                                                       \
+    } while (0)
+                        if (q4) FH_GEMM_LAUNCH_SPLIT(true);
+                        else FH_GEMM_LAUNCH_SPLIT(false);
+#undef FH_GEMM_LAUNCH_SPLIT
+                        continue;
+                    }
+                }
+            }
             if (q4) {
                 if (isums && exact) FH_GEMM_LAUNCH(true, true, true);
                 else if (isums) FH_GEMM_LAUNCH(true, true, false);

@@ -59,7 +59,7 @@ struct forge_hip_model {
     DevBuf kcache, vcache;               // fp16 [layers][max_seq][KV]
     DevBuf cos_t, sin_t;
     // decode scratch
-    DevBuf x, qkv, gu, logits, aq, asc, attn_ws, state, argmax_ws;
+    DevBuf x, qkv, gu, logits, aq, asc, attn_ws, gemm_ws, state, argmax_ws;
     DevBuf counts;                       // u32 [vocab]: how often each token id has been fed since the last reset
     float repeat_penalty = 1.0f;         // > 1: forward_greedy picks the maximum of the penalised logits
     // prefill scratch (chunk_rows rows)
@@ -255,7 +255,7 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
     uint16_t* asc = m->pasc.as<uint16_t>();
     const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;      // the fast GEMM takes the odd blocks of its activations negated
     { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s, !exact); }
-    { StageMark t(m, ST_QKV); launch_gemm(L.qkv, aq, asc, M, qkv, QKV, false, exact, nullptr, s); }
+    { StageMark t(m, ST_QKV); launch_gemm(L.qkv, aq, asc, M, qkv, QKV, false, exact, nullptr, s, m->gemm_ws.p); }
     {
         StageMark t(m, ST_ROPE);
         launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos, nullptr, c.heads,
@@ -272,11 +272,11 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
         { StageMark t(m, ST_ATTN); launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, c.sliding_window, s); }
         { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s, true); }
     }
-    { StageMark t(m, ST_O); launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s); }
+    { StageMark t(m, ST_O); launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s, m->gemm_ws.p); }
     { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s, !exact); }
-    { StageMark t(m, ST_GATE_UP); launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s); }
+    { StageMark t(m, ST_GATE_UP); launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s, m->gemm_ws.p); }
     { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s, !exact); }
-    { StageMark t(m, ST_DOWN); launch_gemm(L.down, aq, asc, M, x, H, true, exact, nullptr, s); }
+    { StageMark t(m, ST_DOWN); launch_gemm(L.down, aq, asc, M, x, H, true, exact, nullptr, s, m->gemm_ws.p); }
 }
 
 // Final norm of one row + lm_head GEMV + argmax (+ pos/token advance when `advance`).
@@ -495,6 +495,12 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
         (rc = m->paq.alloc((size_t)R * m->KMAX)) || (rc = m->pasc.alloc((size_t)R * (m->KMAX / 32) * 2)) ||
         (rc = m->ptok.alloc((size_t)R * 4)))
         return rc;
+    // fast mode: the prefill GEMMs may cut left-over tiles along K (FORGE_HIP_GEMM_SPLIT=0: never)
+    const char* senv = getenv("FORGE_HIP_GEMM_SPLIT");
+    if (!(cfg->flags & FORGE_HIP_FLAG_EXACT) && !(senv && senv[0] == '0')) {
+        if ((rc = m->gemm_ws.alloc(gemm_split_workspace_bytes()))) return rc;
+        FH_HIP(hipMemset(m->gemm_ws.p, 0, gemm_split_workspace_bytes()));
+    }
     const char* penv = getenv("FORGE_HIP_PERSIST");
     if (!(penv && penv[0] == '0')) {
         std::vector<PdLayerIn> pl(cfg->layers);

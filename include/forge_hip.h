@@ -33,8 +33,8 @@
  *  - A model allocates all its device buffers in forge_hip_model_create (weights, KV cache for max_seq,
  *    activations for one prefill chunk); later calls allocate no device memory (the kernel-sequence
  *    decode path instantiates its HIP graph at the first decode step).
- *  - The op-level calls keep three process-wide scratch areas (quantised activations, attention / argmax
- *    partial results, RoPE tables) that GROW ON DEMAND: a call that needs more than any earlier call
+ *  - The op-level calls keep four process-wide scratch areas (quantised activations, attention / argmax
+ *    partial results, RoPE tables, 16 MB of partial GEMM tiles) that GROW ON DEMAND: a call that needs more than any earlier call
  *    did frees the old area, which waits for the device, and allocates a larger one (hipFree +
  *    hipMalloc on the call path).  They are shared by all streams and not locked: use the
  *    op-level API from one thread and one stream at a time, and call the largest shape once at start-up

@@ -6,7 +6,8 @@ problem and compares the parts the oracle can do in seconds, using what the oper
   * a GEMM row depends only on its own activation row, an attention row only on its own query and the keys
     up to its position: sampled rows are checked against the oracle run on exactly those rows;
   * the same rows computed alone on the GPU must equal the rows of the full launch bit for bit
-    (tiling, batching and chunking may not change a result)."""
+    (tiling, batching and chunking may not change a result) -- in EXACT mode and for attention; the fast GEMM
+    promises it within its tolerance only."""
 import hashlib
 import json
 import os
@@ -90,7 +91,10 @@ def test_gemm_llama_1b_shapes(fh, oracle, torch_gpu, wd, K, N, M):
     # the sampled rows as a batch of their own: same bits as inside the full batch
     xs = torch.from_numpy(np.ascontiguousarray(x[rows])).cuda()
     same_bits(fh.ops.matmul_mat_q(w, xs, EXACT).cpu().numpy(), exact[rows])
-    same_bits(fh.ops.matmul_mat_q(w, xs, 0).cpu().numpy(), fast[rows])
+    # fast mode: a large batch may have its left-over tiles cut along K (another f32 order for the rows in them), so
+    # only the tolerance holds between batches; within one batch size the result is reproducible
+    close(fh.ops.matmul_mat_q(w, xs, 0).cpu().numpy(), fast[rows], rtol=1e-4, atol=1e-4)
+    same_bits(fh.ops.matmul_mat_q(w, xd, 0).cpu().numpy(), fast)
 
 
 # ---------------- attention over an fp16 cache ----------------

@@ -166,6 +166,26 @@ def test_matmul_mat_parity(fh, oracle, torch_gpu, wd, M, K, N):
     close(fh.ops.matmul_mat_q(w, xd, 0).cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("wd", [Q8, Q4])
+@pytest.mark.parametrize("M,K,N", [(2502, 2048, 2048), (2502, 8192, 2048), (2100, 1152, 3072), (2502, 576, 2176)])
+def test_matmul_mat_k_ranges_of_leftover_tiles(fh, torch_gpu, wd, M, K, N):
+    """Fast mode, more 128 x 128 tiles than CUs but not a whole number of rounds: the left-over tiles are cut into K ranges
+    that meet in a workspace.  Held to the fast mode's tolerance against EXACT mode (which is bit-identical to the CPU path,
+    see the parity test above and never cuts K), twice in a row (the second call finds the counters the first one left),
+    and the result must not depend on the run (ranges are added in K order, whoever finishes last)."""
+    torch = torch_gpu
+    wraw = make_weight(fh, wd, N, K, seed=3 * N + K + M)
+    x = fh.synth.normal(17 + K, M * K, 1.0).reshape(M, K)
+    w = fh.ops.QWeight(wd, wraw, K, N)
+    xd = torch.from_numpy(x).cuda()
+    want = fh.ops.matmul_mat_q(w, xd, EXACT).cpu().numpy()
+    first = fh.ops.matmul_mat_q(w, xd, 0).cpu().numpy()
+    close(first, want)
+    for _ in range(3):
+        same_bits(fh.ops.matmul_mat_q(w, xd, 0).cpu().numpy(), first)
+    w.close()
+
+
 def test_matmul_mat_ragged_n_within_tolerance(fh, oracle, torch_gpu):
     """N % 4 != 0: the reference's last rows use the 4-accumulator order; the GEMM kernel keeps one
     order for all rows, so those rows agree to tolerance only."""
