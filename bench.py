@@ -446,6 +446,7 @@ def main():
         "decode_weight_stream_GBps_end_to_end": fh.synth.decode_weight_bytes(cfg) * args.steps / t_decode / 1e9,
         "exact_mode": exact,
         "roofline": roofline,
+        "prefill_stage_ms": {k: round(v[0], 3) for k, v in pp.items() if v[1]},
         "prefill_rooflines": {
             "gemm": {"bound": "mfma", "achieved": gemm_flops / (gemm_ms * 1e-3) / 1e12, "peak": MFMA_I8_PEAK_TOPS,
                      "unit": "TOP/s (int8)", "frac": gemm_flops / (gemm_ms * 1e-3) / 1e12 / MFMA_I8_PEAK_TOPS, "ms": gemm_ms},
