@@ -159,9 +159,9 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
     const bool exact = (flags & FORGE_HIP_FLAG_EXACT) != 0;
     int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream, !exact);   // the fast kernel takes odd blocks negated
     if (rc) return rc;
-    // large fast-mode problems may cut left-over tiles along K: that kernel parks partial tiles in a workspace
+    // fast mode may cut tiles along K to fill the CUs: that kernel parks partial tiles in a workspace
     void* split_ws = nullptr;
-    if (!exact && (uint64_t)((M + 127) / 128) * ((w->w.N + 127) / 128) > 256) {
+    if (!exact && M > 64) {
         const bool fresh = g_gemm.cap < gemm_split_workspace_bytes();
         if ((rc = g_gemm.reserve(gemm_split_workspace_bytes()))) return rc;
         if (fresh) FH_HIP(hipMemset(g_gemm.p, 0, gemm_split_workspace_bytes()));   // its counters start at zero and are left at zero

@@ -464,7 +464,7 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
     } while (0)
 #define FH_GEMM_LAUNCH(Q4_, DUMP_, EXACT_)                         \
     do {                                                           \
-        if (small_tiles) FH_GEMM_LAUNCH_TM(Q4_, DUMP_, EXACT_, 1); \
+        if (tm == 1) FH_GEMM_LAUNCH_TM(Q4_, DUMP_, EXACT_, 1);     \
         else FH_GEMM_LAUNCH_TM(Q4_, DUMP_, EXACT_, 2);             \
     } while (0)
     for (uint32_t mlo = 0; mlo < M; mlo += m_step)
@@ -481,34 +481,55 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
             // halves with its tile, and a larger tile would only leave more CUs idle
             const uint64_t tiles64 = (uint64_t)((nc + BN - 1) / BN) * ((mc + 63) / 64);
             const bool small_tiles = tiles64 <= (uint64_t)cus && mc > 64;
-            // 128-row tiles that fill the CUs a few times and a fraction (fast mode, caller gave a workspace): the
-            // tiles of the fraction are cut along K so that they spread over all CUs
-            if (split_ws && !exact && !isums && !small_tiles && mc == M && nc == w.N) {
-                const uint32_t tiles = ((nc + BN - 1) / BN) * ((mc + BM - 1) / BM), stages = (w.K + BK - 1) / BK;
-                const uint32_t rem = tiles % (uint32_t)cus;
-                uint32_t split = rem ? std::min<uint32_t>({(uint32_t)cus / rem, 8u, stages / 2, GEMM_SPLIT_MAX_ITEMS / rem}) : 0;
-                if (tiles > (uint32_t)cus && tiles / (uint32_t)cus < 4 && split >= 2) {
-                    GemmSplit sp{};
-                    sp.stages_per_part = ((stages + split - 1) / split + 1) & ~1u;
-                    sp.split = (stages + sp.stages_per_part - 1) / sp.stages_per_part;
-                    sp.full_tiles = tiles - rem;
-                    sp.partials = reinterpret_cast<float*>(split_ws);
-                    sp.counters = reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(split_ws) + (size_t)GEMM_SPLIT_MAX_ITEMS * BM * BN * sizeof(float));
-                    if (sp.split >= 2) {
-                        const uint32_t items = sp.full_tiles + rem * sp.split;
-#define FH_GEMM_LAUNCH_SPLIT(Q4_)                                                                                            \
+            int tm = small_tiles ? 1 : 2;
+            // Fast mode with a workspace from the caller: tiles that fill the CUs a few times and a fraction have the tiles of
+            // the fraction cut along K, so that they spread over all CUs; a problem with fewer tiles than half the CUs is
+            // all fraction.  Which tile height then fills the CUs best is decided by a small cost model (microseconds per K
+            // stage of a workgroup that has a CU to itself, measured: 1.3 for a 128-row tile, 1.1 for a 64-row one).
+            if (split_ws && !exact && !isums && mc == M && nc == w.N) {
+                struct Plan { int tm; GemmSplit sp; uint32_t items; double cost; };
+                const uint32_t stages = (w.K + BK - 1) / BK;
+                auto plan = [&](int tm_) {
+                    const uint32_t tile_rows = 64 * tm_, tiles = ((nc + BN - 1) / BN) * ((mc + tile_rows - 1) / tile_rows);
+                    const double t_stage = tm_ == 1 ? 1.1 : 1.3;
+                    Plan p{tm_, GemmSplit{}, 0, (double)((tiles + cus - 1) / cus) * stages * t_stage};   // items 0: not cut
+                    const uint32_t rem = tiles % (uint32_t)cus;
+                    const uint32_t split = rem ? std::min<uint32_t>({(uint32_t)cus / rem, 8u, stages / 2, GEMM_SPLIT_MAX_ITEMS / rem}) : 0;
+                    if (tiles / (uint32_t)cus < 4 && split >= 2) {
+                        GemmSplit sp{};
+                        sp.stages_per_part = ((stages + split - 1) / split + 1) & ~1u;
+                        sp.split = (stages + sp.stages_per_part - 1) / sp.stages_per_part;
+                        sp.full_tiles = tiles - rem;
+                        sp.partials = reinterpret_cast<float*>(split_ws);
+                        sp.counters = reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(split_ws) + (size_t)GEMM_SPLIT_MAX_ITEMS * BM * BN * sizeof(float));
+                        // parking, counting and adding partial tiles: 12 us (64-row tiles) to 18 us (128-row tiles) end to end
+                        // when every workgroup does it at the same moment, 5 when whole tiles are still being worked beside it
+                        const double cost = ((double)(sp.full_tiles / cus) * stages + sp.stages_per_part) * t_stage +
+                                            (sp.full_tiles ? 5.0 : tm_ == 1 ? 12.0 : 18.0);
+                        if (sp.split >= 2 && cost < p.cost) { p.sp = sp; p.items = sp.full_tiles + rem * sp.split; p.cost = cost; }
+                    }
+                    return p;
+                };
+                Plan best = plan(tm);
+                if (tm == 1) { const Plan other = plan(2); if (other.cost < best.cost) best = other; }
+                tm = best.tm;
+                if (best.items) {
+                    const GemmSplit sp = best.sp;
+                    const uint32_t items = best.items;
+#define FH_GEMM_LAUNCH_SPLIT(Q4_, TM_)                                                                                       \
     do {                                                                                                                    \
-        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, false, false, 2, true>,       \
+        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, false, false, TM_, true>,     \
                                                              hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES);   \
         (void)lds_ok;                                                                                                       \
-        fh::launch(gemm_q_kernel<Q4_, false, false, 2, true>, dim3(items), 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c, y_c, \
-                   is_c, mc, nc, w.K, ldy, accf, sp);                                                                       \
+        fh::launch(gemm_q_kernel<Q4_, false, false, TM_, true>, dim3(items), 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c,   \
+                   y_c, is_c, mc, nc, w.K, ldy, accf, sp);                                                                  \
     } while (0)
-                        if (q4) FH_GEMM_LAUNCH_SPLIT(true);
-                        else FH_GEMM_LAUNCH_SPLIT(false);
+                    if (q4 && tm == 1) FH_GEMM_LAUNCH_SPLIT(true, 1);
+                    else if (q4) FH_GEMM_LAUNCH_SPLIT(true, 2);
+                    else if (tm == 1) FH_GEMM_LAUNCH_SPLIT(false, 1);
+                    else FH_GEMM_LAUNCH_SPLIT(false, 2);
 #undef FH_GEMM_LAUNCH_SPLIT
-                        continue;
-                    }
+                    continue;
                 }
             }
             if (q4) {
