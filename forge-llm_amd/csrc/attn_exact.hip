@@ -114,6 +114,174 @@ __global__ void attn_exact_kernel(const float* __restrict__ q, uint32_t q_stride
     }
 }
 
+// attention_flash_batch for many rows (batched prefill without a window), the same arithmetic as attn_exact_kernel<HD, true>
+// value for value, arranged so that a key block is fetched once for 16 queries instead of once per query: a workgroup is
+// ONE wave that carries up to 16 queries of one KV head (rows_per_wg consecutive rows x the heads that share the KV head)
+// through the key blocks.  Per block: lane = key for the scores (the key's row in registers, the queries broadcast from
+// LDS, 64-step sequential sums, four queries interleaved so that their chains overlap); lane = query for the running
+// maximum, the rescale factor and the sequential block sum; lane = key again for the exponentials; lane = head dim for
+// P.V (the block's V column in registers, the weights broadcast from LDS, added in key order straight into the
+// accumulator).  Every query keeps the reference's own per-row block structure: blocks start at multiples of 64, a block
+// past a row's last key leaves that row untouched, a row's last block is walked for its own number of keys only.
+template <int HD>
+__global__ __launch_bounds__(64) void attn_exact_batch_group_kernel(const float* __restrict__ q, uint32_t q_stride,
+                                                                    const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+                                                                    float* __restrict__ out, uint32_t out_stride, uint32_t base_pos,
+                                                                    uint32_t M, uint32_t heads, uint32_t kv_heads, uint32_t rows_per_wg) {
+    constexpr int NQ = 16;                 // queries a wave carries
+    constexpr int DPL = (HD + 63) / 64;    // head dims per lane in P.V: lane, lane + 64
+    __shared__ __attribute__((aligned(16))) float qs[NQ][HD];
+    __shared__ __attribute__((aligned(16))) float se[NQ][XB + 4];   // scores, then weights (rows 16-byte aligned)
+    __shared__ float mi[NQ], es[NQ];
+    const uint32_t lane = threadIdx.x;
+    const uint32_t kvh = blockIdx.x, r0 = blockIdx.y * rows_per_wg;
+    const uint32_t G = heads / kv_heads;
+    const uint32_t rows = min(rows_per_wg, M - r0), nq = rows * G;
+    const uint32_t kv_stride = kv_heads * HD;
+    const float scale = 1.0f / sqrtf((float)HD);
+
+    for (uint32_t i = lane; i < NQ * HD; i += 64) {
+        const uint32_t qi = i / HD, d = i % HD;
+        qs[qi][d] = qi < nq ? q[(size_t)(r0 + qi / G) * q_stride + (kvh * G + qi % G) * HD + d] : 0.f;
+    }
+    // lane j < nq keeps the softmax state of query j
+    const uint32_t my_seq = lane < nq ? base_pos + r0 + lane / G + 1 : 0;
+    float m_i = -INFINITY, l_i = 0.f;
+    float acc[NQ][DPL];
+#pragma unroll
+    for (int qi = 0; qi < NQ; qi++)
+#pragma unroll
+        for (int t = 0; t < DPL; t++) acc[qi][t] = 0.f;
+    const uint32_t seq_max = base_pos + r0 + rows;      // keys the last row sees
+    __syncthreads();
+
+    for (uint32_t bs = 0; bs < seq_max; bs += XB) {
+        // ---- scores: lane = key bs + lane
+        const uint32_t key = bs + lane;
+        float sreg[NQ];
+        {
+            float kf[HD];
+            if (key < seq_max) {
+                const uint16_t* krow = kc + (size_t)key * kv_stride + kvh * HD;
+#pragma unroll
+                for (int c = 0; c < HD / 8; c++) {
+                    const uint4 w = *reinterpret_cast<const uint4*>(krow + c * 8);
+                    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+#pragma unroll
+                    for (int j = 0; j < 4; j++) {
+                        kf[c * 8 + 2 * j] = f16_bits_to_f32((uint16_t)(ww[j] & 0xFFFFu));
+                        kf[c * 8 + 2 * j + 1] = f16_bits_to_f32((uint16_t)(ww[j] >> 16));
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int d = 0; d < HD; d++) kf[d] = 0.f;
+            }
+#pragma unroll
+            for (int q0 = 0; q0 < NQ; q0 += 4) {
+                float sum[4] = {0.f, 0.f, 0.f, 0.f};
+                if ((uint32_t)q0 < nq) {
+#pragma unroll
+                for (int d = 0; d < HD; d++)
+#pragma unroll
+                    for (int u = 0; u < 4; u++) sum[u] = sum[u] + qs[q0 + u][d] * kf[d];
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++) {
+                    const uint32_t seq_q = base_pos + r0 + (q0 + u) / G + 1;     // uniform
+                    sreg[q0 + u] = ((uint32_t)(q0 + u) < nq && key < seq_q) ? sum[u] * scale : -INFINITY;
+                    se[q0 + u][lane] = sreg[q0 + u];
+                }
+            }
+        }
+        __syncthreads();
+        // ---- lane = query: block maximum, running maximum, rescale factor
+        const uint32_t my_bl = my_seq > bs ? min((uint32_t)XB, my_seq - bs) : 0;
+        if (lane < nq) {
+            float exp_scale = 1.0f;                 // a block past this row's keys: x * 1.0f is x
+            if (my_bl) {
+                float m_block = -INFINITY;
+#pragma unroll 16
+                for (int bi = 0; bi < XB; bi++) m_block = fmaxf(m_block, se[lane][bi]);   // keys past the row read -inf
+                const float m_prev = m_i;
+                if (m_block > m_i) m_i = m_block;
+                exp_scale = expf_ref<true>(m_prev - m_i);
+                l_i = l_i * exp_scale;
+            }
+            es[lane] = exp_scale;
+            mi[lane] = m_i;
+        }
+        __syncthreads();
+        // ---- lane = key: weights
+#pragma unroll
+        for (int qi = 0; qi < NQ; qi++) {
+            if ((uint32_t)qi < nq) se[qi][lane] = sreg[qi] == -INFINITY ? 0.f : expf_ref<true>(sreg[qi] - mi[qi]);
+        }
+        __syncthreads();
+        // ---- lane = query: sequential block sum over the row's own keys of the block
+        if (lane < nq && my_bl) {
+            float l_block = 0.f;
+            if (my_bl == XB) {
+#pragma unroll
+                for (int bi = 0; bi < XB; bi++) l_block = l_block + se[lane][bi];
+            } else {
+#pragma unroll
+                for (int bi = 0; bi < XB; bi++) l_block = (uint32_t)bi < my_bl ? l_block + se[lane][bi] : l_block;
+            }
+            l_i = l_i + l_block;
+        }
+        // ---- P.V: lane = head dim (and lane + 64)
+        {
+            float vf[XB][DPL];
+#pragma unroll
+            for (int bi = 0; bi < XB; bi++)
+#pragma unroll
+                for (int t = 0; t < DPL; t++) {
+                    const uint32_t d = lane + 64 * t;
+                    vf[bi][t] = (bs + bi < seq_max && d < HD) ? f16_bits_to_f32(vc[(size_t)(bs + bi) * kv_stride + kvh * HD + d]) : 0.f;
+                }
+#pragma unroll
+            for (int qi = 0; qi < NQ; qi++) {
+                const uint32_t seq_q = base_pos + r0 + qi / G + 1;               // uniform
+                // (a guard, not a break or continue: the loop must unroll completely, acc[] lives in registers)
+                if ((uint32_t)qi < nq && seq_q > bs) {                           // else the block lies past this row's keys
+                const uint32_t bl = min((uint32_t)XB, seq_q - bs);
+                const float exp_scale = es[qi];
+#pragma unroll
+                for (int t = 0; t < DPL; t++) acc[qi][t] = acc[qi][t] * exp_scale;
+                if (bl == XB) {
+#pragma unroll
+                    for (int bi = 0; bi < XB; bi++) {
+                        const float e = se[qi][bi];
+#pragma unroll
+                        for (int t = 0; t < DPL; t++) acc[qi][t] = acc[qi][t] + e * vf[bi][t];
+                    }
+                } else {
+#pragma unroll
+                    for (int bi = 0; bi < XB; bi++) {
+                        const float e = se[qi][bi];
+#pragma unroll
+                        for (int t = 0; t < DPL; t++) acc[qi][t] = (uint32_t)bi < bl ? acc[qi][t] + e * vf[bi][t] : acc[qi][t];
+                    }
+                }
+                }
+            }
+        }
+        __syncthreads();   // se, es and mi are rewritten by the next block
+    }
+    if (lane < nq) es[lane] = 1.0f / l_i;
+    __syncthreads();
+#pragma unroll
+    for (int qi = 0; qi < NQ; qi++) {
+        const float inv_l = es[qi];
+#pragma unroll
+        for (int t = 0; t < DPL; t++) {
+            const uint32_t d = lane + 64 * t;
+            if ((uint32_t)qi < nq && d < HD) out[(size_t)(r0 + qi / G) * out_stride + (kvh * G + qi % G) * HD + d] = acc[qi][t] * inv_l;
+        }
+    }
+}
+
 // attention_sliding (emit.rs:598-627), the decode attention of a model with a window: no blocks, a plain softmax over the
 // last min(window, seq) rows — scores, their maximum, exp and a sequential sum, a multiplication by the reciprocal, then
 // for every head dim a sequential sum of weight * v.  The scores live in dynamic LDS (wl floats).
@@ -350,6 +518,17 @@ void launch_attn_exact(bool batch_order, const float* q, uint32_t q_stride, cons
     } while (0)
         if (hd == 64) FH_XD(64); else if (hd == 96) FH_XD(96); else FH_XD(128);
 #undef FH_XD
+        return;
+    }
+    // batched prefill without a window: a wave per 16 queries of one KV head (needs the f32 output form and at most 16
+    // heads per KV head; FORGE_HIP_EXACT_GROUP=0: the one-query kernel)
+    static const bool group_ok = [] { const char* e = getenv("FORGE_HIP_EXACT_GROUP"); return !(e && e[0] == '0'); }();
+    if (group_ok && batch_order && window == 0 && M > 1 && out && !oq && !pos_dev && heads / kv_heads <= 16) {
+        const uint32_t rows_per_wg = 16 / (heads / kv_heads);
+        dim3 gg(kv_heads, (M + rows_per_wg - 1) / rows_per_wg);
+        if (hd == 64) fh::launch(attn_exact_batch_group_kernel<64>, gg, 64, 0, s, q, q_stride, kc, vc, out, out_stride, base_pos, M, heads, kv_heads, rows_per_wg);
+        else if (hd == 96) fh::launch(attn_exact_batch_group_kernel<96>, gg, 64, 0, s, q, q_stride, kc, vc, out, out_stride, base_pos, M, heads, kv_heads, rows_per_wg);
+        else fh::launch(attn_exact_batch_group_kernel<128>, gg, 64, 0, s, q, q_stride, kc, vc, out, out_stride, base_pos, M, heads, kv_heads, rows_per_wg);
         return;
     }
     dim3 grid(heads, M);
