@@ -134,7 +134,8 @@ __global__ __launch_bounds__(64) void attn_exact_batch_group_kernel(const float*
     __shared__ __attribute__((aligned(16))) float se[NQ][XB + 4];   // scores, then weights (rows 16-byte aligned)
     __shared__ float mi[NQ], es[NQ];
     const uint32_t lane = threadIdx.x;
-    const uint32_t kvh = blockIdx.x, r0 = blockIdx.y * rows_per_wg;
+    // the last rows walk the most key blocks: they are handed out first, the short ones fill the end
+    const uint32_t kvh = blockIdx.x, r0 = (gridDim.y - 1 - blockIdx.y) * rows_per_wg;
     const uint32_t G = heads / kv_heads;
     const uint32_t rows = min(rows_per_wg, M - r0), nq = rows * G;
     const uint32_t kv_stride = kv_heads * HD;
@@ -153,29 +154,32 @@ __global__ __launch_bounds__(64) void attn_exact_batch_group_kernel(const float*
 #pragma unroll
         for (int t = 0; t < DPL; t++) acc[qi][t] = 0.f;
     const uint32_t seq_max = base_pos + r0 + rows;      // keys the last row sees
+    // the key row of the NEXT block travels while this block is worked (zeros past the last key)
+    uint4 kraw[HD / 8];
+    auto fetch_k = [&](uint32_t bs) {
+        const uint32_t key = bs + lane;
+#pragma unroll
+        for (int c = 0; c < HD / 8; c++)
+            kraw[c] = key < seq_max ? *reinterpret_cast<const uint4*>(kc + (size_t)key * kv_stride + kvh * HD + c * 8) : make_uint4(0, 0, 0, 0);
+    };
+    fetch_k(0);
     __syncthreads();
 
     for (uint32_t bs = 0; bs < seq_max; bs += XB) {
         // ---- scores: lane = key bs + lane
         const uint32_t key = bs + lane;
         float sreg[NQ];
+        float vf[XB][DPL];
         {
             float kf[HD];
-            if (key < seq_max) {
-                const uint16_t* krow = kc + (size_t)key * kv_stride + kvh * HD;
 #pragma unroll
-                for (int c = 0; c < HD / 8; c++) {
-                    const uint4 w = *reinterpret_cast<const uint4*>(krow + c * 8);
-                    const uint32_t ww[4] = {w.x, w.y, w.z, w.w};
+            for (int c = 0; c < HD / 8; c++) {
+                const uint32_t ww[4] = {kraw[c].x, kraw[c].y, kraw[c].z, kraw[c].w};
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
-                        kf[c * 8 + 2 * j] = f16_bits_to_f32((uint16_t)(ww[j] & 0xFFFFu));
-                        kf[c * 8 + 2 * j + 1] = f16_bits_to_f32((uint16_t)(ww[j] >> 16));
-                    }
+                for (int j = 0; j < 4; j++) {
+                    kf[c * 8 + 2 * j] = f16_bits_to_f32((uint16_t)(ww[j] & 0xFFFFu));
+                    kf[c * 8 + 2 * j + 1] = f16_bits_to_f32((uint16_t)(ww[j] >> 16));
                 }
-            } else {
-#pragma unroll
-                for (int d = 0; d < HD; d++) kf[d] = 0.f;
             }
 #pragma unroll
             for (int q0 = 0; q0 < NQ; q0 += 4) {
@@ -194,6 +198,14 @@ __global__ __launch_bounds__(64) void attn_exact_batch_group_kernel(const float*
                 }
             }
         }
+        // the block's V column (lane = head dim) is requested now and used after the softmax phases
+#pragma unroll
+        for (int bi = 0; bi < XB; bi++)
+#pragma unroll
+            for (int t = 0; t < DPL; t++) {
+                const uint32_t d = lane + 64 * t;
+                vf[bi][t] = (bs + bi < seq_max && d < HD) ? f16_bits_to_f32(vc[(size_t)(bs + bi) * kv_stride + kvh * HD + d]) : 0.f;
+            }
         __syncthreads();
         // ---- lane = query: block maximum, running maximum, rescale factor
         const uint32_t my_bl = my_seq > bs ? min((uint32_t)XB, my_seq - bs) : 0;
@@ -232,14 +244,7 @@ __global__ __launch_bounds__(64) void attn_exact_batch_group_kernel(const float*
         }
         // ---- P.V: lane = head dim (and lane + 64)
         {
-            float vf[XB][DPL];
-#pragma unroll
-            for (int bi = 0; bi < XB; bi++)
-#pragma unroll
-                for (int t = 0; t < DPL; t++) {
-                    const uint32_t d = lane + 64 * t;
-                    vf[bi][t] = (bs + bi < seq_max && d < HD) ? f16_bits_to_f32(vc[(size_t)(bs + bi) * kv_stride + kvh * HD + d]) : 0.f;
-                }
+            fetch_k(bs + XB);
 #pragma unroll
             for (int qi = 0; qi < NQ; qi++) {
                 const uint32_t seq_q = base_pos + r0 + qi / G + 1;               // uniform
