@@ -29,15 +29,19 @@ typedef float v16f __attribute__((ext_vector_type(16)));
 constexpr int QW = 32;        // queries per wave pair
 constexpr int QB = 128;       // queries per workgroup
 constexpr int KT = 64;        // keys per tile
-constexpr int AP_THREADS = 512;
+constexpr int AP_THREADS = 512;   // the 8-wave form; the 4-wave form runs 256
 
 // QUANT: instead of f32 rows the kernel writes what the o projection's GEMM reads, the activation quantiser's int8
 // codes oq[M][heads*HD] and fp16 scales osc[M][heads*HD/32] of the same values (a 32-element block is one 32-wide
 // head_dim tile of one query: 16 values in this lane, 16 in lane ^ 32).
 // WIN: sliding-window attention (attention_sliding_batch, emit.rs:907-1046): the query at position p sees the keys
 // [max(0, p - window + 1), p]; key tiles that lie before the window of the workgroup's first query are never loaded.
-template <int HD, bool QUANT, bool WIN>
-__global__ __launch_bounds__(AP_THREADS) __attribute__((amdgpu_waves_per_eu(2)))
+// KH: 32-key halves of a tile that one wave works.  1 = the 8-wave form described above (two waves share a query group and
+// merge at the end: twice the waves on the longest chain, for short sequences); 2 = 4 waves, each takes its 32 queries
+// through all 64 keys of a tile: two independent score tiles per step to overlap, one maximum / rescale / lane exchange
+// per 64 keys, no merge.
+template <int HD, bool QUANT, bool WIN, int KH>
+__global__ __launch_bounds__(AP_THREADS / KH) __attribute__((amdgpu_waves_per_eu(2)))
 void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
                          float* __restrict__ out, uint32_t q_stride, uint32_t out_stride, uint32_t M, uint32_t base_pos,
                          uint32_t heads, uint32_t kv_heads, int8_t* __restrict__ oq, uint16_t* __restrict__ osc, uint32_t window) {
@@ -45,20 +49,21 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
     constexpr int VS = KT + 4;    // V^T tile row stride (halfs): 8-byte pad
     constexpr int KTOTAL = KT * HD / 8;          // 16-byte pieces of K per tile
     constexpr int VTOTAL = KT * HD / 8;          // (key pair, 4 dims) items of V per tile
-    constexpr int KPIECES = (KTOTAL + AP_THREADS - 1) / AP_THREADS, VITEMS = (VTOTAL + AP_THREADS - 1) / AP_THREADS;
+    constexpr int NT = AP_THREADS / KH;           // threads of the workgroup
+    constexpr int KPIECES = (KTOTAL + NT - 1) / NT, VITEMS = (VTOTAL + NT - 1) / NT;
     constexpr int DG = HD / 4;    // groups of 4 head dims
     constexpr int NS = HD / 16;   // MFMA k-steps over head_dim
     constexpr int ND = HD / 32;   // 32-wide head_dim tiles of the output
     constexpr int KBYTES = KT * KS * 2, VBYTES = HD * VS * 2;
     constexpr int MERGE_FLOATS = 2 + ND * 16;    // per lane: m, l and the output accumulators
-    static_assert(2 * (KBYTES + VBYTES) >= 4 * 64 * MERGE_FLOATS * 4, "the merge reuses the tile buffers");
+    static_assert(KH == 2 || 2 * (KBYTES + VBYTES) >= 4 * 64 * MERGE_FLOATS * 4, "the merge reuses the tile buffers");
     // two tiles each: the loads of tile t+1 are written while tile t is read, one barrier per tile
     __shared__ __attribute__((aligned(16))) uint8_t smem[2 * (KBYTES + VBYTES)];
     auto Ks = [&](uint32_t buf) { return reinterpret_cast<_Float16*>(smem + buf * KBYTES); };
     auto Vt = [&](uint32_t buf) { return reinterpret_cast<_Float16*>(smem + 2 * KBYTES + buf * VBYTES); };
 
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t qg = wave >> 1, kh = wave & 1;      // query group of 32, half of every key tile
+    const uint32_t qg = KH == 1 ? wave >> 1 : wave, kh = KH == 1 ? (wave & 1) : 0;   // query group of 32, (first) half of every key tile
     const uint32_t lq = lane & 31, lh = lane >> 5;
     // tile-major order, heaviest (latest) query tiles first: they stream the most keys, and whatever does not fit the
     // machine at once is the light end, handed out as the first workgroups finish
@@ -109,7 +114,7 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
     auto load_tile = [&](uint32_t kt) {
 #pragma unroll
         for (int i = 0; i < KPIECES; i++) {
-            const uint32_t idx = tid + AP_THREADS * i, key = idx / (HD / 8), dc = idx % (HD / 8);
+            const uint32_t idx = tid + NT * i, key = idx / (HD / 8), dc = idx % (HD / 8);
             const uint32_t t = kt * KT + key;
             kreg[i] = (idx < KTOTAL && t < seq_total) ? *reinterpret_cast<const int4*>(kc + (size_t)t * kv_stride + kvh * HD + dc * 8)
                                                      : make_int4(0, 0, 0, 0);
@@ -117,7 +122,7 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
         // V: an item is 4 head dims of two consecutive keys (seq rows t, t+1)
 #pragma unroll
         for (int i = 0; i < VITEMS; i++) {
-            const uint32_t idx = tid + AP_THREADS * i, kp = idx / DG, dg = idx % DG;
+            const uint32_t idx = tid + NT * i, kp = idx / DG, dg = idx % DG;
             const uint32_t t = kt * KT + 2 * kp;
             const uint16_t* src = vc + (size_t)t * kv_stride + kvh * HD + dg * 4;
             va[i] = (idx < VTOTAL && t < seq_total) ? *reinterpret_cast<const uint2*>(src) : make_uint2(0, 0);
@@ -127,13 +132,13 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
     auto store_tile = [&](uint32_t buf) {
 #pragma unroll
         for (int i = 0; i < KPIECES; i++) {
-            const uint32_t idx = tid + AP_THREADS * i, key = idx / (HD / 8), dc = idx % (HD / 8);
+            const uint32_t idx = tid + NT * i, key = idx / (HD / 8), dc = idx % (HD / 8);
             if (idx < KTOTAL) *reinterpret_cast<int4*>(Ks(buf) + key * KS + dc * 8) = kreg[i];
         }
         // V^T[d][key]: the two keys' values of one head dim side by side in a dword
 #pragma unroll
         for (int i = 0; i < VITEMS; i++) {
-            const uint32_t idx = tid + AP_THREADS * i, kp = idx / DG, dg = idx % DG;
+            const uint32_t idx = tid + NT * i, kp = idx / DG, dg = idx % DG;
             if (idx < VTOTAL) {
                 uint32_t* vt = reinterpret_cast<uint32_t*>(Vt(buf) + (dg * 4) * VS + 2 * kp);
                 vt[0 * (VS / 2)] = __builtin_amdgcn_perm(vb[i].x, va[i].x, 0x05040100u);
@@ -150,53 +155,66 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
     for (uint32_t kt = tile0; kt < ntiles; kt++) {
         const uint32_t buf = kt & 1;
         if (kt + 1 < ntiles) load_tile(kt + 1);          // in flight while this tile is computed
-        const uint32_t k0 = kt * KT + kh * 32;            // this wave's 32 keys of the tile
-        if (wave_active && k0 <= wave_max_pos && k0 + 32 > wave_lo) {   // else they lie entirely in the group's future, or before every window
+        const uint32_t k0 = kt * KT + kh * 32;            // this wave's first 32 keys of the tile
+        constexpr uint32_t KW = 32 * KH;                  // keys of the tile this wave works
+        if (wave_active && k0 <= wave_max_pos && k0 + KW > wave_lo) {   // else they lie entirely in the group's future, or before every window
             const _Float16* Kb = Ks(buf);
             const _Float16* Vb = Vt(buf);
-            // ---- S^T tile: sacc[r] = q . k for key k0 + 8(r/4) + 4 lh + r%4, query lq
-            v16f sacc;
+            // ---- S^T tiles: sacc[h][r] = q . k for key k0 + 32 h + 8(r/4) + 4 lh + r%4, query lq
+            v16f sacc[KH];
 #pragma unroll
-            for (int r = 0; r < 16; r++) sacc[r] = 0.f;
+            for (int h = 0; h < KH; h++)
 #pragma unroll
-            for (int s = 0; s < NS; s++) {
-                v8h kf = *reinterpret_cast<const v8h*>(Kb + (kh * 32 + lq) * KS + 16 * s + 8 * lh);
-                sacc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], sacc, 0, 0, 0);
-            }
+                for (int r = 0; r < 16; r++) sacc[h][r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < NS; s++)
+#pragma unroll
+                for (int h = 0; h < KH; h++) {
+                    v8h kf = *reinterpret_cast<const v8h*>(Kb + ((kh + h) * 32 + lq) * KS + 16 * s + 8 * lh);
+                    sacc[h] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf, qf[s], sacc[h], 0, 0, 0);
+                }
             // ---- causal mask: only keys past the group's first query can be masked for some query
             // with a window, also keys that the group's last query no longer sees
-            if (WIN && (k0 + 31 > wave_min_pos || k0 + window <= wave_max_pos)) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const uint32_t t = k0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                    sacc[r] = (t <= qpos && t + window > qpos) ? sacc[r] : -INFINITY;
-                }
-            } else if (!WIN && k0 + 31 > wave_min_pos) {
+            for (int h = 0; h < KH; h++) {
+                const uint32_t kb = k0 + 32 * h;
+                if (WIN && (kb + 31 > wave_min_pos || kb + window <= wave_max_pos)) {
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const uint32_t t = k0 + 8 * (r >> 2) + 4 * lh + (r & 3);
-                    sacc[r] = (t <= qpos) ? sacc[r] : -INFINITY;
+                    for (int r = 0; r < 16; r++) {
+                        const uint32_t t = kb + 8 * (r >> 2) + 4 * lh + (r & 3);
+                        sacc[h][r] = (t <= qpos && t + window > qpos) ? sacc[h][r] : -INFINITY;
+                    }
+                } else if (!WIN && kb + 31 > wave_min_pos) {
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const uint32_t t = kb + 8 * (r >> 2) + 4 * lh + (r & 3);
+                        sacc[h][r] = (t <= qpos) ? sacc[h][r] : -INFINITY;
+                    }
                 }
             }
             // ---- online softmax in base 2 (per-lane scalars: a lane owns one query)
             float m_tile = -INFINITY;
 #pragma unroll
-            for (int r = 0; r < 16; r++) m_tile = fmaxf(m_tile, sacc[r]);
+            for (int h = 0; h < KH; h++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) m_tile = fmaxf(m_tile, sacc[h][r]);
             m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, WAVE)) * c2;      // c2 > 0: max commutes with the scaling
             const float m_new = fmaxf(m_run, m_tile);
-            // a query that has seen no key yet (all of this half tile masked for it) keeps m = -inf: exponentiate
+            // a query that has seen no key yet (all of these keys masked for it) keeps m = -inf: exponentiate
             // against 0 instead, every p is then 2^-inf = 0
             const float m_exp = m_new == -INFINITY ? 0.f : m_new;
             float l_tile = 0.f;
-            v8h pb[2];
+            v8h pb[KH][2];
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int h = 0; h < KH; h++)
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const float p = __builtin_amdgcn_exp2f(fmaf(sacc[8 * j + e], c2, -m_exp));   // 2^-inf = 0 for masked keys
-                    l_tile += p;
-                    pb[j][e] = (_Float16)p;
-                }
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        const float p = __builtin_amdgcn_exp2f(fmaf(sacc[h][8 * j + e], c2, -m_exp));   // 2^-inf = 0 for masked keys
+                        l_tile += p;
+                        pb[h][j][e] = (_Float16)p;
+                    }
             // rescale what has been accumulated, unless no query of the wave saw a new maximum
             if (__builtin_amdgcn_ballot_w64(m_new > m_run) != 0) {
                 const float alpha = m_run == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_run - m_new);
@@ -208,17 +226,19 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
             }
             l_run += l_tile;
             m_run = m_new;
-            // ---- O^T += V^T P^T over this wave's 32 keys
+            // ---- O^T += V^T P^T over this wave's keys
 #pragma unroll
-            for (int d = 0; d < ND; d++)
+            for (int h = 0; h < KH; h++)
 #pragma unroll
-                for (int j = 0; j < 2; j++) {
-                    const _Float16* vrow = Vb + (d * 32 + lq) * VS + kh * 32 + 16 * j + 4 * lh;
-                    v4h v0 = *reinterpret_cast<const v4h*>(vrow);
-                    v4h v1 = *reinterpret_cast<const v4h*>(vrow + 8);
-                    v8h vf = (v8h){v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
-                    oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pb[j], oacc[d], 0, 0, 0);
-                }
+                for (int j = 0; j < 2; j++)
+#pragma unroll
+                    for (int d = 0; d < ND; d++) {
+                        const _Float16* vrow = Vb + (d * 32 + lq) * VS + (kh + h) * 32 + 16 * j + 4 * lh;
+                        v4h v0 = *reinterpret_cast<const v4h*>(vrow);
+                        v4h v1 = *reinterpret_cast<const v4h*>(vrow + 8);
+                        v8h vf = (v8h){v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+                        oacc[d] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pb[h][j], oacc[d], 0, 0, 0);
+                    }
         }
         if (kt + 1 < ntiles) store_tile(buf ^ 1);   // nobody reads that buffer: its tile was finished before the last barrier
         __syncthreads();
@@ -226,6 +246,7 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
 
     // ---- the two waves of a query group merge their halves: the odd one hands (m, l, O) over through LDS
     float* mg = reinterpret_cast<float*>(smem) + (qg * 64 + lane) * MERGE_FLOATS;
+    if (KH == 1) {
     if (kh == 1) {
         mg[0] = m_run;
         mg[1] = l_run;
@@ -245,6 +266,7 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
         for (int d = 0; d < ND; d++)
 #pragma unroll
             for (int r = 0; r < 16; r++) oacc[d][r] = oacc[d][r] * a0 + mg[2 + d * 16 + r] * a1;
+    }
     }
 
     // ---- normalise and store: lane (lq, lh) holds out[qrow][32 d + 8 g + 4 lh + 0..3]
@@ -293,11 +315,26 @@ template <int HD, bool QUANT>
 void launch_win(dim3 grid, hipStream_t s, const float* q, const uint16_t* kc, const uint16_t* vc, float* out, uint32_t q_stride,
                 uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, int8_t* oq, uint16_t* osc,
                 uint32_t window) {
+    // The 4-wave form when there are clearly more workgroups than the machine holds at once (three per CU at head_dim 64,
+    // two above: then throughput decides, and a wave with two score tiles per step does 15-30 % more of it); the 8-wave form
+    // when they all fit (then the longest workgroup's chain of tile steps decides, and twice the waves halve its steps).
+    // Measured, 32 heads: 3001 tokens of head_dim 96 143 -> 108 us, 8192 tokens of head_dim 128 978 -> 842 us; 2502 tokens of
+    // head_dim 64 59 -> 67 us, which is why the count decides.  FORGE_HIP_ATTN_WAVES=8 / 4 forces one.
+    static const int forced = [] { const char* e = getenv("FORGE_HIP_ATTN_WAVES"); return e ? atoi(e) : 0; }();
+    static const int cus = [] {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) n = 256;
+        return n > 0 ? n : 256;
+    }();
+    const uint32_t slots = (uint32_t)cus * (HD == 64 ? 3 : 2);
+    const bool four = forced == 4 || (forced != 8 && grid.x * 4 >= slots * 5);
     // a window that covers every key of the call is plain causal attention
-    if (window != 0 && window < base_pos + M)
-        fh::launch(attn_prefill_kernel<HD, QUANT, true>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window);
-    else
-        fh::launch(attn_prefill_kernel<HD, QUANT, false>, grid, AP_THREADS, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, 0u);
+    const bool win = window != 0 && window < base_pos + M;
+#define FH_AP(WIN_, KH_) \
+    fh::launch(attn_prefill_kernel<HD, QUANT, WIN_, KH_>, grid, AP_THREADS / KH_, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, WIN_ ? window : 0u)
+    if (win) { if (four) FH_AP(true, 2); else FH_AP(true, 1); }
+    else { if (four) FH_AP(false, 2); else FH_AP(false, 1); }
+#undef FH_AP
 }
 template <bool QUANT>
 void launch_hd(uint32_t hd, dim3 grid, hipStream_t s, const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
