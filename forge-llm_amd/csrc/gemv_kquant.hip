@@ -37,18 +37,20 @@ __device__ __forceinline__ int sub32x4(uint32_t x) { return (int)(((x | 0x808080
 
 constexpr int KQ_WAVES = 4;
 
-// LDS: the activation codes [K], their scales as f32 [K/32], (Q4_K) their sums as f32 [K/32], then per wave the products [K/32]
-template <bool Q6>
+// LDS: the activation codes [K], their scales as f32 [K/32], (Q4_K) their sums as f32 [K/32], then per wave the products
+// [RW][K/32 + 1].  A wave works RW rows at a time: all their loads are issued before the first is used (one row of
+// K = 2048 is a single kilobyte, far too little in flight for HBM), and lane r adds row r's products in block order.
+template <bool Q6, int RW>
 __global__ __launch_bounds__(KQ_WAVES * 64) void gemv_kquant_kernel(const uint8_t* __restrict__ qs, const uint8_t* __restrict__ meta,
                                                                   const int8_t* __restrict__ aq, const uint16_t* __restrict__ as,
                                                                   float* __restrict__ y, uint32_t K, uint32_t N, int accumulate) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t nblk = K / 32, nsb = K / 256;
+    const uint32_t nblk = K / 32, nsb = K / 256, pstride = nblk + 1;
     int8_t* xa = reinterpret_cast<int8_t*>(lds);
     float* xs = reinterpret_cast<float*>(lds + K);
     float* xsum = xs + nblk;
-    float* prod = xsum + nblk + (size_t)wave * (nblk + 1);
+    float* prod = xsum + nblk + (size_t)wave * RW * pstride;
     for (uint32_t i = tid; i < K / 16; i += KQ_WAVES * 64) reinterpret_cast<int4*>(xa)[i] = reinterpret_cast<const int4*>(aq)[i];
     for (uint32_t b = tid; b < nblk; b += KQ_WAVES * 64) {
         xs[b] = f16_bits_to_f32(as[b]);
@@ -62,7 +64,7 @@ __global__ __launch_bounds__(KQ_WAVES * 64) void gemv_kquant_kernel(const uint8_
 
     // a row is nsb * 8 pieces of 16 bytes of the first plane; piece p = 8 sb + t belongs to lane p % 64 of pass p / 64
     const uint32_t pieces = nsb * 8;
-    for (uint32_t row = blockIdx.x * KQ_WAVES + wave; row < N; row += gridDim.x * KQ_WAVES) {
+    for (uint32_t row0 = (blockIdx.x * KQ_WAVES + wave) * RW; row0 < N; row0 += gridDim.x * KQ_WAVES * RW) {
         for (uint32_t p0 = 0; p0 < pieces; p0 += 64) {
             const uint32_t p = p0 + lane;
             if (p < pieces) {
@@ -71,70 +73,93 @@ __global__ __launch_bounds__(KQ_WAVES * 64) void gemv_kquant_kernel(const uint8_
                     // piece t: bytes [16 t, +16) of the super-block's nibbles = elements [16 e, +16) of sub-blocks 2c (low
                     // nibbles) and 2c + 1 (high nibbles), c = t / 2
                     const uint32_t c = t >> 1;
-                    const int4 w = *reinterpret_cast<const int4*>(qs + ((size_t)row * nsb + sb) * 128 + t * 16);
-                    const uint4 mt = *reinterpret_cast<const uint4*>(meta + ((size_t)row * nsb + sb) * 16);
-                    const int m = 0x0F0F0F0F;
-                    const int4 lo = make_int4(w.x & m, w.y & m, w.z & m, w.w & m);
-                    const int4 hi = make_int4((w.x >> 4) & m, (w.y >> 4) & m, (w.z >> 4) & m, (w.w >> 4) & m);
+                    int4 wv[RW];
+                    uint4 mv[RW];
+#pragma unroll
+                    for (int r = 0; r < RW; r++) {
+                        const size_t row = min(row0 + r, N - 1);          // past the end: the last row again, never stored
+                        wv[r] = *reinterpret_cast<const int4*>(qs + (row * nsb + sb) * 128 + t * 16);
+                        mv[r] = *reinterpret_cast<const uint4*>(meta + (row * nsb + sb) * 16);
+                    }
                     const uint32_t b_lo = sb * 8 + 2 * c;
                     const int4 a_lo = *reinterpret_cast<const int4*>(xa + b_lo * 32 + e * 16);
                     const int4 a_hi = *reinterpret_cast<const int4*>(xa + (b_lo + 1) * 32 + e * 16);
-                    int d_lo = kq_dot16(lo, a_lo, 0), d_hi = kq_dot16(hi, a_hi, 0);
-                    d_lo += pair_swap(d_lo);                     // the other 16 elements sit in the neighbouring lane
-                    d_hi += pair_swap(d_hi);
                     // the even lane of the pair finishes sub-block 2c, the odd lane 2c + 1
-                    const uint32_t j = 2 * c + e;
-                    const int dot = e ? d_hi : d_lo;
-                    const uint32_t sc12[3] = {mt.y, mt.z, mt.w};
-                    uint32_t sc, mn;                             // get_scale_min_k4, emit.rs:3013-3021
-                    if (j < 4) { sc = byte_of(sc12, j) & 63u; mn = byte_of(sc12, j + 4) & 63u; }
-                    else {
-                        sc = (byte_of(sc12, j + 4) & 0x0Fu) | ((byte_of(sc12, j - 4) >> 6) << 4);
-                        mn = (byte_of(sc12, j + 4) >> 4) | ((byte_of(sc12, j) >> 6) << 4);
+                    const uint32_t j = 2 * c + e, b = sb * 8 + j;
+                    const float x_s = xs[b], x_sum = xsum[b];
+#pragma unroll
+                    for (int r = 0; r < RW; r++) {
+                        const int4 w = wv[r];
+                        const uint4 mt = mv[r];
+                        const int m = 0x0F0F0F0F;
+                        const int4 lo = make_int4(w.x & m, w.y & m, w.z & m, w.w & m);
+                        const int4 hi = make_int4((w.x >> 4) & m, (w.y >> 4) & m, (w.z >> 4) & m, (w.w >> 4) & m);
+                        int d_lo = kq_dot16(lo, a_lo, 0), d_hi = kq_dot16(hi, a_hi, 0);
+                        d_lo += pair_swap(d_lo);                     // the other 16 elements sit in the neighbouring lane
+                        d_hi += pair_swap(d_hi);
+                        const int dot = e ? d_hi : d_lo;
+                        const uint32_t sc12[3] = {mt.y, mt.z, mt.w};
+                        uint32_t sc, mn;                             // get_scale_min_k4, emit.rs:3013-3021
+                        if (j < 4) { sc = byte_of(sc12, j) & 63u; mn = byte_of(sc12, j + 4) & 63u; }
+                        else {
+                            sc = (byte_of(sc12, j + 4) & 0x0Fu) | ((byte_of(sc12, j - 4) >> 6) << 4);
+                            mn = (byte_of(sc12, j + 4) >> 4) | ((byte_of(sc12, j) >> 6) << 4);
+                        }
+                        const float d = f16_bits_to_f32((uint16_t)(mt.x & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(mt.x >> 16));
+                        const float d_w = d * (float)sc, m_w = dmin * (float)mn;
+                        prod[r * pstride + b] = x_s * (d_w * (float)dot - m_w * x_sum);
                     }
-                    const float d = f16_bits_to_f32((uint16_t)(mt.x & 0xFFFFu)), dmin = f16_bits_to_f32((uint16_t)(mt.x >> 16));
-                    const float d_w = d * (float)sc, m_w = dmin * (float)mn;
-                    const uint32_t b = sb * 8 + j;
-                    prod[b] = xs[b] * (d_w * (float)dot - m_w * xsum[b]);
                 } else {
                     // piece t = 4 h + 2 p + e: elements [16 e, +16) of blocks 4h + p (low nibbles of ql[64h + 32p ..], bit pair
                     // 2p of qh[32h ..]) and 4h + 2 + p (high nibbles, bit pair 2 + p)
                     const uint32_t h = t >> 2, pp = (t >> 1) & 1;
-                    const uint8_t* sbp = qs + ((size_t)row * nsb + sb) * 192;
-                    const uint4 ql = *reinterpret_cast<const uint4*>(sbp + 64 * h + 32 * pp + 16 * e);
-                    const uint4 qh = *reinterpret_cast<const uint4*>(sbp + 128 + 32 * h + 16 * e);
-                    const uint8_t* mp = meta + ((size_t)row * nsb + sb) * 32;
-                    const uint32_t qlw[4] = {ql.x, ql.y, ql.z, ql.w}, qhw[4] = {qh.x, qh.y, qh.z, qh.w};
-                    const uint32_t bA = sb * 8 + 4 * h + pp, bB = bA + 2;
-                    int4 qa, qb;
-                    int* qav = reinterpret_cast<int*>(&qa);
-                    int* qbv = reinterpret_cast<int*>(&qb);
+                    uint4 qlv[RW], qhv[RW], scv[RW];
+                    uint32_t dv[RW];
 #pragma unroll
-                    for (int i = 0; i < 4; i++) {
-                        qav[i] = sub32x4((qlw[i] & 0x0F0F0F0Fu) | (((qhw[i] >> (2 * pp)) & 0x03030303u) << 4));
-                        qbv[i] = sub32x4(((qlw[i] >> 4) & 0x0F0F0F0Fu) | (((qhw[i] >> (4 + 2 * pp)) & 0x03030303u) << 4));
+                    for (int r = 0; r < RW; r++) {
+                        const size_t row = min(row0 + r, N - 1);
+                        const uint8_t* sbp = qs + (row * nsb + sb) * 192;
+                        qlv[r] = *reinterpret_cast<const uint4*>(sbp + 64 * h + 32 * pp + 16 * e);
+                        qhv[r] = *reinterpret_cast<const uint4*>(sbp + 128 + 32 * h + 16 * e);
+                        const uint8_t* mp = meta + (row * nsb + sb) * 32;
+                        scv[r] = *reinterpret_cast<const uint4*>(mp);                 // the 16 int8 sub-block scales
+                        dv[r] = *reinterpret_cast<const uint32_t*>(mp + 16);          // d (fp16) in the low half
                     }
+                    const uint32_t bA = sb * 8 + 4 * h + pp, bB = bA + 2;
                     const int4 xA = *reinterpret_cast<const int4*>(xa + bA * 32 + e * 16);
                     const int4 xB = *reinterpret_cast<const int4*>(xa + bB * 32 + e * 16);
-                    const int dA = kq_dot16(qa, xA, 0), dB = kq_dot16(qb, xB, 0);
-                    // this lane's 16 elements go under scale 2b + e; the even lane adds the pair: sc_lo*dot_lo + sc_hi*dot_hi
-                    const float sA = (float)(int)(int8_t)mp[2 * (4 * h + pp) + e], sB = (float)(int)(int8_t)mp[2 * (4 * h + 2 + pp) + e];
-                    const float tA = sA * (float)dA, tB = sB * (float)dB;
-                    const float uA = tA + pair_swap(tA), uB = tB + pair_swap(tB);      // even lane: lo + hi
-                    if (!e) {
-                        const float d = f16_bits_to_f32((uint16_t)(mp[16] | (mp[17] << 8)));
-                        prod[bA] = (d * xs[bA]) * uA;
-                        prod[bB] = (d * xs[bB]) * uB;
+                    const float xsA = xs[bA], xsB = xs[bB];
+#pragma unroll
+                    for (int r = 0; r < RW; r++) {
+                        const uint32_t qlw[4] = {qlv[r].x, qlv[r].y, qlv[r].z, qlv[r].w}, qhw[4] = {qhv[r].x, qhv[r].y, qhv[r].z, qhv[r].w};
+                        const uint32_t scw[4] = {scv[r].x, scv[r].y, scv[r].z, scv[r].w};
+                        int4 qa, qb;
+                        int* qav = reinterpret_cast<int*>(&qa);
+                        int* qbv = reinterpret_cast<int*>(&qb);
+#pragma unroll
+                        for (int i = 0; i < 4; i++) {
+                            qav[i] = sub32x4((qlw[i] & 0x0F0F0F0Fu) | (((qhw[i] >> (2 * pp)) & 0x03030303u) << 4));
+                            qbv[i] = sub32x4(((qlw[i] >> 4) & 0x0F0F0F0Fu) | (((qhw[i] >> (4 + 2 * pp)) & 0x03030303u) << 4));
+                        }
+                        const int dA = kq_dot16(qa, xA, 0), dB = kq_dot16(qb, xB, 0);
+                        // this lane's 16 elements go under scale 2b + e; the even lane adds the pair: sc_lo*dot_lo + sc_hi*dot_hi
+                        const float sA = (float)(int)(int8_t)byte_of(scw, 2 * (4 * h + pp) + e), sB = (float)(int)(int8_t)byte_of(scw, 2 * (4 * h + 2 + pp) + e);
+                        const float tA = sA * (float)dA, tB = sB * (float)dB;
+                        const float uA = tA + pair_swap(tA), uB = tB + pair_swap(tB);      // even lane: lo + hi
+                        if (!e) {
+                            const float d = f16_bits_to_f32((uint16_t)(dv[r] & 0xFFFFu));
+                            prod[r * pstride + bA] = (d * xsA) * uA;
+                            prod[r * pstride + bB] = (d * xsB) * uB;
+                        }
                     }
                 }
             }
         }
-        // LDS operations of one wave execute in order: the products are there
-        float r = 0.f;
-        if (lane == 0) {
-            r = ordered_sum(prod, nblk, false);
-            if (accumulate) r = y[row] + r;
-            y[row] = r;
+        // LDS operations of one wave execute in order: the products are there.  Lane r adds row r's.
+        if (lane < RW && row0 + lane < N) {
+            float r = ordered_sum(prod + lane * pstride, nblk, false);
+            if (accumulate) r = y[row0 + lane] + r;
+            y[row0 + lane] = r;
         }
     }
 }
@@ -168,12 +193,17 @@ bool kquant_k_supported(uint32_t K) { return K >= 256 && K % 256 == 0 && K <= 16
 void launch_gemv_kquant(const QWeight& w, const int8_t* aq, const uint16_t* as, float* y, bool accumulate, hipStream_t s) {
     if (w.N == 0) return;
     const uint32_t nblk = w.K / 32;
-    const size_t lds = (size_t)w.K + (size_t)nblk * 8 + (size_t)KQ_WAVES * (nblk + 1) * 4;
-    uint32_t grid = (w.N + KQ_WAVES - 1) / KQ_WAVES;
+    // rows a wave keeps in flight: four when that still leaves every CU several workgroups
+    const int rw = w.N >= 16384 ? 4 : w.N >= 4096 ? 2 : 1;
+    const size_t lds = (size_t)w.K + (size_t)nblk * 8 + (size_t)KQ_WAVES * rw * (nblk + 1) * 4;
+    uint32_t grid = (w.N + KQ_WAVES * rw - 1) / (KQ_WAVES * rw);
     if (grid > 256 * 8) grid = 256 * 8;
     const uint8_t* meta = reinterpret_cast<const uint8_t*>(w.scales);
-    if (w.wdtype == FORGE_HIP_Q6_K) fh::launch(gemv_kquant_kernel<true>, grid, KQ_WAVES * 64, lds, s, w.qs, meta, aq, as, y, w.K, w.N, accumulate ? 1 : 0);
-    else fh::launch(gemv_kquant_kernel<false>, grid, KQ_WAVES * 64, lds, s, w.qs, meta, aq, as, y, w.K, w.N, accumulate ? 1 : 0);
+    const int acc = accumulate ? 1 : 0;
+#define FH_KQ(Q6_, RW_) fh::launch(gemv_kquant_kernel<Q6_, RW_>, grid, KQ_WAVES * 64, lds, s, w.qs, meta, aq, as, y, w.K, w.N, acc)
+    if (w.wdtype == FORGE_HIP_Q6_K) { if (rw == 4) FH_KQ(true, 4); else if (rw == 2) FH_KQ(true, 2); else FH_KQ(true, 1); }
+    else { if (rw == 4) FH_KQ(false, 4); else if (rw == 2) FH_KQ(false, 2); else FH_KQ(false, 1); }
+#undef FH_KQ
 }
 
 }  // namespace fh
