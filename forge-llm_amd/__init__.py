@@ -34,7 +34,7 @@ EXPORTS = [
     "forge_hip_f32_to_f16", "forge_hip_quantize_f32", "forge_hip_expf_host", "forge_hip_dequant", "forge_hip_qweight_create",
     "forge_hip_qweight_destroy", "forge_hip_quantize_act", "forge_hip_gemv_q", "forge_hip_gemm_q",
     "forge_hip_block_isums", "forge_hip_gemv_q_f32act", "forge_hip_rms_norm", "forge_hip_silu_mul", "forge_hip_rope_kv_store",
-    "forge_hip_attn_prefill_f16kv", "forge_hip_attn_decode_f16kv", "forge_hip_attn_decode_f16kv_noalloc",
+    "forge_hip_attn_prefill_f16kv", "forge_hip_attn_decode_f16kv", "forge_hip_attn_decode_f16kv_noalloc", "forge_hip_attn_decode_f16kv_paged",
     "forge_hip_attn_prefill_sliding_f16kv", "forge_hip_attn_decode_sliding_f16kv", "forge_hip_argmax",
     "forge_hip_gguf_open", "forge_hip_gguf_parse", "forge_hip_gguf_close", "forge_hip_gguf_version", "forge_hip_gguf_alignment",
     "forge_hip_gguf_tensor_data_offset", "forge_hip_gguf_tensor_count", "forge_hip_gguf_metadata_count", "forge_hip_gguf_tensor",
@@ -141,6 +141,8 @@ def lib():
     L.forge_hip_attn_prefill_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp]
     L.forge_hip_attn_decode_f16kv.restype = i32
     L.forge_hip_attn_decode_f16kv.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, u32, vp]
+    L.forge_hip_attn_decode_f16kv_paged.restype = i32
+    L.forge_hip_attn_decode_f16kv_paged.argtypes = [vp, vp, vp, vp, u32, vp, u32, u32, u32, u32, vp]
     L.forge_hip_attn_decode_f16kv_noalloc.restype = i32
     L.forge_hip_attn_decode_f16kv_noalloc.argtypes = [vp, vp, vp, vp, u32, u32, u32, u32, vp]
     L.forge_hip_attn_prefill_sliding_f16kv.restype = i32

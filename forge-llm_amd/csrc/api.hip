@@ -322,6 +322,23 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
     return FORGE_HIP_OK;
 }
 
+int32_t forge_hip_attn_decode_f16kv_paged(const float* q_dev, const uint16_t* k_pool_dev, const uint16_t* v_pool_dev,
+                                          const uint32_t* page_table_dev, uint32_t page_rows, float* out_dev, uint32_t seq_len,
+                                          uint32_t heads, uint32_t kv_heads, uint32_t head_dim, void* stream) {
+    FH_CHECK(q_dev && k_pool_dev && v_pool_dev && page_table_dev && out_dev, "attn_decode_paged: null pointer");
+    FH_CHECK(seq_len >= 1, "attn_decode_paged: seq_len must be at least 1");
+    int32_t rc = check_attn_shape("attn_decode_paged", heads, kv_heads, head_dim);
+    if (rc) return rc;
+    FH_CHECK(page_rows >= 1 && (page_rows & (page_rows - 1)) == 0, "attn_decode_paged: page_rows must be a power of two");
+    FH_CHECK(attn_decode_paged_supported(seq_len, page_rows), "attn_decode_paged: pages too small for a sequence this long (more than 2048 table entries per split)");
+    rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
+    if (rc) return rc;
+    launch_attn_decode_paged(q_dev, k_pool_dev, v_pool_dev, page_table_dev, page_rows, out_dev, seq_len, heads, kv_heads, head_dim,
+                             g_attn.p, (hipStream_t)stream);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
 int32_t forge_hip_attn_decode_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                             float* out_dev, uint32_t seq_len, uint32_t window, uint32_t heads,
                                             uint32_t kv_heads, uint32_t head_dim, uint32_t flags, void* stream) {

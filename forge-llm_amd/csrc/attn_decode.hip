@@ -27,14 +27,23 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float* a, float 
     m = mn;
 }
 
+// A paged cache (PAGED): kc / vc are pools of pages of 2^page_shift rows, and row t of the sequence is row t % page of
+// pool page page_table[t / page].  A split's table entries are copied into LDS first (they are few), so the address of
+// a key costs one LDS read more than in the flat cache; nothing else changes, the bits included.
+constexpr uint32_t PAGE_ENTRIES_MAX = 2048;   // table entries one split may span (else: contiguous-only)
+struct PageTable {
+    const uint32_t* table;   // nullptr unless PAGED
+    uint32_t shift;          // log2(rows per page)
+};
+
 // workspace record per (kv group, split, head-in-group): [HD acc][m][l]
-template <int HD, int GT>
+template <int HD, int GT, bool PAGED = false>
 __global__ __launch_bounds__(256) void attn_decode_split_kernel(const float* __restrict__ q,
                                                                 const uint16_t* __restrict__ kc,
                                                                 const uint16_t* __restrict__ vc,
                                                                 float* __restrict__ ws, uint32_t seq_len_arg,
                                                                 const uint32_t* __restrict__ pos_dev, uint32_t heads,
-                                                                uint32_t kv_heads, uint32_t gsize, uint32_t window) {
+                                                                uint32_t kv_heads, uint32_t gsize, uint32_t window, PageTable pt) {
     constexpr int LPK = HD <= 64 ? 8 : 16;   // lanes per key row
     constexpr int KPW = 64 / LPK;            // keys per wave load
     constexpr int REC = HD + 2;
@@ -57,6 +66,19 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const float* __r
     chunk = (chunk + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
     const uint32_t t0 = min(seq, start + split * chunk);
     const uint32_t t1 = min(seq, t0 + chunk);
+
+    __shared__ uint32_t pt_s[PAGED ? PAGE_ENTRIES_MAX : 1];
+    const uint32_t pt_first = PAGED ? t0 >> pt.shift : 0;
+    if (PAGED) {
+        const uint32_t n_entries = t1 > t0 ? ((t1 - 1) >> pt.shift) - pt_first + 1 : 0;
+        for (uint32_t i = threadIdx.x; i < n_entries; i += 256) pt_s[i] = pt.table[pt_first + i];
+        __syncthreads();
+    }
+    // row of the cache (pool) that holds position t
+    auto row_of = [&](uint32_t t) -> size_t {
+        if (!PAGED) return t;
+        return ((size_t)pt_s[(t >> pt.shift) - pt_first] << pt.shift) + (t & ((1u << pt.shift) - 1));
+    };
 
     float qf[GT][8];
 #pragma unroll
@@ -83,7 +105,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const float* __r
             kr[u] = Half8{{0, 0, 0, 0}};
             vr[u] = Half8{{0, 0, 0, 0}};
             if (t < t1 && dvalid) {
-                const size_t off = (size_t)t * kv_stride + kvh * HD + c * 8;
+                const size_t off = row_of(t) * kv_stride + kvh * HD + c * 8;
                 kr[u] = *reinterpret_cast<const Half8*>(kc + off);
                 vr[u] = *reinterpret_cast<const Half8*>(vc + off);
             }
@@ -193,30 +215,51 @@ bool attn_head_dim_supported(uint32_t hd) { return hd == 64 || hd == 96 || hd ==
 namespace {
 template <int HD, int GT>
 void launch_split(const float* q, const uint16_t* kc, const uint16_t* vc, float* ws, uint32_t seq,
-                  const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t window, hipStream_t s) {
+                  const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t window, PageTable pt, hipStream_t s) {
     const uint32_t gsize = heads / kv_heads;
     dim3 grid(kv_heads * (gsize / GT), DECODE_SPLITS);
-    fh::launch(attn_decode_split_kernel<HD, GT>, grid, 256, 0, s, q, kc, vc, ws, seq, pos_dev, heads, kv_heads, gsize, window);
+    if (pt.table) fh::launch(attn_decode_split_kernel<HD, GT, true>, grid, 256, 0, s, q, kc, vc, ws, seq, pos_dev, heads, kv_heads, gsize, window, pt);
+    else fh::launch(attn_decode_split_kernel<HD, GT, false>, grid, 256, 0, s, q, kc, vc, ws, seq, pos_dev, heads, kv_heads, gsize, window, pt);
 }
 template <int HD>
 void launch_hd(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
-               uint32_t seq, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t window, float* ws, hipStream_t s) {
+               uint32_t seq, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t window, float* ws, PageTable pt,
+               hipStream_t s) {
     const uint32_t gsize = heads / kv_heads;
-    if (gsize % 4 == 0) launch_split<HD, 4>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, s);
-    else if (gsize % 3 == 0) launch_split<HD, 3>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, s);
-    else if (gsize % 2 == 0) launch_split<HD, 2>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, s);
-    else launch_split<HD, 1>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, s);
+    if (gsize % 4 == 0) launch_split<HD, 4>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, pt, s);
+    else if (gsize % 3 == 0) launch_split<HD, 3>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, pt, s);
+    else if (gsize % 2 == 0) launch_split<HD, 2>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, pt, s);
+    else launch_split<HD, 1>(q, kc, vc, ws, seq, pos_dev, heads, kv_heads, window, pt, s);
     fh::launch(attn_decode_combine_kernel<HD>, heads, HD, 0, s, ws, DECODE_SPLITS, out, oq, osc);
 }
 }  // namespace
+
+// Whether a paged call with these sizes is covered: pages of a power of two of rows, and no split spanning more table
+// entries than the kernel keeps in LDS.
+bool attn_decode_paged_supported(uint32_t seq_len, uint32_t page_rows) {
+    if (page_rows == 0 || (page_rows & (page_rows - 1)) != 0) return false;
+    const uint32_t per_split = (seq_len + DECODE_SPLITS - 1) / DECODE_SPLITS + 64;
+    return per_split / page_rows + 2 <= PAGE_ENTRIES_MAX;
+}
+
+void launch_attn_decode_paged(const float* q, const uint16_t* k_pool, const uint16_t* v_pool, const uint32_t* page_table,
+                              uint32_t page_rows, float* out, uint32_t seq_len, uint32_t heads, uint32_t kv_heads, uint32_t hd,
+                              void* workspace, hipStream_t s) {
+    float* ws = reinterpret_cast<float*>(workspace);
+    PageTable pt{page_table, (uint32_t)__builtin_ctz(page_rows)};
+    if (hd == 64) launch_hd<64>(q, k_pool, v_pool, out, nullptr, nullptr, seq_len, nullptr, heads, kv_heads, 0u, ws, pt, s);
+    else if (hd == 96) launch_hd<96>(q, k_pool, v_pool, out, nullptr, nullptr, seq_len, nullptr, heads, kv_heads, 0u, ws, pt, s);
+    else launch_hd<128>(q, k_pool, v_pool, out, nullptr, nullptr, seq_len, nullptr, heads, kv_heads, 0u, ws, pt, s);
+}
 
 void launch_attn_decode(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
                         uint32_t seq_len, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd,
                         uint32_t window, void* workspace, hipStream_t s) {
     float* ws = reinterpret_cast<float*>(workspace);
-    if (hd == 64) launch_hd<64>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, s);
-    else if (hd == 96) launch_hd<96>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, s);
-    else launch_hd<128>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, s);
+    const PageTable pt{nullptr, 0};
+    if (hd == 64) launch_hd<64>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, pt, s);
+    else if (hd == 96) launch_hd<96>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, pt, s);
+    else launch_hd<128>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, pt, s);
 }
 
 }  // namespace fh

@@ -164,6 +164,12 @@ size_t attn_decode_workspace_bytes(uint32_t heads, uint32_t hd);
 void launch_attn_decode(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
                         uint32_t seq_len, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd,
                         uint32_t window, void* workspace, hipStream_t s);
+// The same over a paged cache: k_pool / v_pool fp16 [pages][page_rows][kv_heads*hd], row t of the sequence is row
+// t % page_rows of pool page page_table[t / page_rows].  f32 output, no window.
+bool attn_decode_paged_supported(uint32_t seq_len, uint32_t page_rows);
+void launch_attn_decode_paged(const float* q, const uint16_t* k_pool, const uint16_t* v_pool, const uint32_t* page_table,
+                              uint32_t page_rows, float* out, uint32_t seq_len, uint32_t heads, uint32_t kv_heads, uint32_t hd,
+                              void* workspace, hipStream_t s);
 
 // attn_prefill.hip
 // q rows / out rows have strides q_stride / out_stride floats (q may live inside a fused qkv buffer).

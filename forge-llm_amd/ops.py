@@ -250,6 +250,19 @@ def attention_flash(q, k_cache, v_cache, seq_len, heads, kv_heads, head_dim, fla
     return out
 
 
+def attention_flash_paged(q, k_pool, v_pool, page_table, page_rows, seq_len, heads, kv_heads, head_dim):
+    """attention_flash over a paged fp16 cache: pools [pages][page_rows][kv_heads*head_dim] (int16 bit patterns),
+    page_table int32/uint32 [ceil(seq_len / page_rows)] of pool page indices."""
+    from . import check, lib
+    torch = _torch()
+    q = _dev(q, torch.float32)
+    pt = page_table.to(torch.int32).contiguous()
+    out = torch.empty(heads * head_dim, dtype=torch.float32, device=q.device)
+    check(lib().forge_hip_attn_decode_f16kv_paged(_ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(pt), page_rows, _ptr(out), seq_len,
+                                                  heads, kv_heads, head_dim, _stream()))
+    return out
+
+
 def attention_flash_noalloc(q, k_cache, v_cache, seq_len, heads, kv_heads, head_dim, out):
     """attention_flash (fast mode) through the entry point that allocates nothing: the caller brings `out` (f32 [heads*hd],
     on the device) as well as the inputs, all already of the right type and contiguous."""

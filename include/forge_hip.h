@@ -256,6 +256,16 @@ int32_t forge_hip_attn_decode_f16kv_noalloc(const float* q_dev, const uint16_t* 
                                             float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
                                             uint32_t head_dim, void* stream);
 
+/* forge_hip_attn_decode_f16kv (fast arithmetic) over a PAGED fp16 cache, for hosts whose KV memory is a pool of pages
+ * shared by several sequences.  The reference's own cache is one flat array per model (emit.rs:532-545, metal:3525-3553), so
+ * this has no reference call to replace; its result is, bit for bit, that of forge_hip_attn_decode_f16kv on the same rows
+ * laid out flat.  k_pool_dev / v_pool_dev: fp16 [pages][page_rows][kv_heads*head_dim]; row t of the sequence is row
+ * t % page_rows of pool page page_table_dev[t / page_rows] (uint32 indices, ceil(seq_len / page_rows) entries);
+ * page_rows a power of two (a 262 144-row sequence needs pages of at least 8 rows). */
+int32_t forge_hip_attn_decode_f16kv_paged(const float* q_dev, const uint16_t* k_pool_dev, const uint16_t* v_pool_dev,
+                                          const uint32_t* page_table_dev, uint32_t page_rows, float* out_dev, uint32_t seq_len,
+                                          uint32_t heads, uint32_t kv_heads, uint32_t head_dim, void* stream);
+
 /* attention_sliding_batch (emit.rs:907-1046) over an fp16 cache: as forge_hip_attn_prefill_f16kv, but the query at
  * position p = base_pos + row sees only the keys [max(0, p - window + 1), p]; window >= 1. */
 int32_t forge_hip_attn_prefill_sliding_f16kv(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,

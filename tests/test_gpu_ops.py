@@ -263,6 +263,46 @@ def test_attention_decode_parity(fh, oracle, torch_gpu, heads, kv_heads, hd, seq
     close(fh.ops.attention_flash(qd, kd, vd, seq, heads, kv_heads, hd, 0).cpu().numpy(), want)
 
 
+@pytest.mark.parametrize("heads,kv_heads,hd", [(32, 8, 64), (9, 3, 64), (32, 32, 96), (24, 8, 128)])
+@pytest.mark.parametrize("seq,page_rows", [(1, 16), (70, 16), (900, 64), (2250, 16), (2250, 256), (8192, 128), (777, 1)])
+def test_attention_decode_paged_cache(fh, oracle, torch_gpu, heads, kv_heads, hd, seq, page_rows):
+    """The sequence's rows scattered over a pool of pages in a random order (with pages of other sequences, poisoned, in
+    between): the paged call must give the flat call's bits, and stays within the tolerance of the oracle."""
+    torch = torch_gpu
+    k16, v16 = _kv_cache(fh, oracle, seq, kv_heads, hd, seed=seq + hd + page_rows)
+    q = fh.synth.normal(19, heads * hd, 1.0)
+    n_pages = (seq + page_rows - 1) // page_rows
+    rng = np.random.default_rng(seq * 31 + page_rows)
+    pool_pages = 2 * n_pages + 3
+    table = rng.permutation(pool_pages)[:n_pages].astype(np.int32)
+    kvw = kv_heads * hd
+    k_pool = np.full((pool_pages, page_rows, kvw), 0x7E00, np.uint16)       # NaN bit patterns wherever the sequence is not
+    v_pool = np.full((pool_pages, page_rows, kvw), 0x7E00, np.uint16)
+    for i, pg in enumerate(table):
+        rows = slice(i * page_rows, min(seq, (i + 1) * page_rows))
+        n = rows.stop - rows.start
+        k_pool[pg, :n] = k16[rows]
+        v_pool[pg, :n] = v16[rows]
+    qd = torch.from_numpy(q).cuda()
+    flat = fh.ops.attention_flash(qd, _dev16(torch, k16), _dev16(torch, v16), seq, heads, kv_heads, hd, 0).cpu().numpy()
+    paged = fh.ops.attention_flash_paged(qd, _dev16(torch, k_pool), _dev16(torch, v_pool), torch.from_numpy(table).cuda(), page_rows,
+                                         seq, heads, kv_heads, hd).cpu().numpy()
+    same_bits(paged, flat)
+    if seq <= 900:
+        close(paged, oracle.attention("flash", q, k16, v16, seq, heads, kv_heads, hd))
+
+
+def test_attention_decode_paged_cache_refusals(fh, torch_gpu):
+    torch = torch_gpu
+    q = torch.zeros(8 * 64, device="cuda")
+    pool = torch.zeros((4, 24, 2 * 64), dtype=torch.int16, device="cuda")
+    table = torch.zeros(4, dtype=torch.int32, device="cuda")
+    with pytest.raises(fh.ForgeHipError):
+        fh.ops.attention_flash_paged(q, pool, pool, table, 24, 50, 8, 2, 64)          # pages of 24 rows: not a power of two
+    with pytest.raises(fh.ForgeHipError):
+        fh.ops.attention_flash_paged(q, pool, pool, table, 16, 50, 8, 2, 80)          # head_dim
+
+
 @pytest.mark.parametrize("heads,kv_heads,hd", [(8, 2, 64), (6, 6, 96), (6, 2, 128)])
 @pytest.mark.parametrize("M,base", [(1, 0), (33, 0), (200, 0), (131, 77), (64, 64)])
 def test_attention_prefill_parity(fh, oracle, torch_gpu, heads, kv_heads, hd, M, base):
