@@ -402,12 +402,13 @@ def test_persistent_decode_kernel_real_shapes(fh, torch_gpu, monkeypatch, shape)
     seq.close(); one.close()
 
 
-def test_prefill_gemm_k_ranges_at_model_level(fh, torch_gpu, monkeypatch):
+@pytest.mark.parametrize("wd", [Q8, Q4])
+def test_prefill_gemm_k_ranges_at_model_level(fh, torch_gpu, monkeypatch, wd):
     """Two Llama-3.2-1B-shaped layers over a 2502-token prompt (fast mode): the o and down projections have 320 tiles for 256
     CUs, so their left-over tiles are cut along K.  With the cut switched off the logits agree as closely as fast mode
     agrees with itself under any other change of f32 summation order, and a second pass over the same
     prompt reproduces the first bit for bit (ranges are added in K order, whichever workgroup finishes last)."""
-    cfg = fh.synth.llama32_1b(Q8, max_seq=2560)
+    cfg = fh.synth.llama32_1b(wd, max_seq=2560)
     cfg["layers"], cfg["vocab"] = 2, 8000
     blob = fh.synth.make_weights_blob(cfg, seed=91, threads=16)
     toks = fh.synth.uniform_ids(92, 2502, cfg["vocab"])
