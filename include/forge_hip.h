@@ -69,7 +69,10 @@ extern "C" {
  * fused multiply-add, 64-key attention blocks with sequential sums, the C library's expf), so
  * results are bit-identical to the CPU path and greedy tokens are identical.  Without it the
  * prefill GEMM fuses its per-block multiply-add and attention runs on the MFMA / split-sequence
- * kernels: same integer block sums, f32 results within rel 1e-3 / abs 1e-3, much faster. */
+ * kernels: same integer block sums, f32 results within rel 1e-3 / abs 1e-3, much faster.  Only EXACT
+ * results are independent of how rows are batched: without the flag the GEMM may add a row's blocks in
+ * K ranges chosen from the batch size, so the same row can differ in its last bits between two batch
+ * sizes (a repeated call with the same sizes reproduces its bits). */
 #define FORGE_HIP_FLAG_EXACT 1u
 /* Bit for config.flags only.  QKV_BIAS: the q, k and v projections add a bias vector before RoPE (Qwen2,
  * emit.rs:3906-3915, 4105-4120) and the weights blob carries, per layer after the v weights, q_bias [heads*head_dim],
