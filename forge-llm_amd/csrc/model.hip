@@ -68,6 +68,7 @@ struct forge_hip_model {
     uint32_t chunk_rows = 0;
     // pinned host staging: [0] token, [1] next token, [2] position
     uint32_t* h_stage = nullptr;
+    float* h_logits = nullptr;          // pinned: logits come home at PCIe speed and are copied to the caller's (pageable) buffer from here
     int64_t pos = 0;
     bool use_graph = true;
     bool fuse_norm = false, fuse_silu = false;   // fused GEMV prologue/epilogue variants fit LDS for this model
@@ -93,6 +94,7 @@ struct forge_hip_model {
         for (auto& L : layers) { qweight_free(&L.qkv); qweight_free(&L.o); qweight_free(&L.gate_up); qweight_free(&L.down); }
         qweight_free(&lm_head);
         if (h_stage) (void)hipHostFree(h_stage);
+        if (h_logits) (void)hipHostFree(h_logits);
         if (stream) (void)hipStreamDestroy(stream);
     }
 };
@@ -411,6 +413,7 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
     m->prefill_fuse_quant = fuse_ok;
     FH_HIP(hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking));
     FH_HIP(hipHostMalloc((void**)&m->h_stage, 64, hipHostMallocDefault));
+    FH_HIP(hipHostMalloc((void**)&m->h_logits, (size_t)cfg->vocab * 4, hipHostMallocDefault));
 
     // ---- weights (blob order: project.rs:342-407) ----
     const uint8_t* p = blob;
@@ -528,8 +531,11 @@ int32_t forge_hip_forward(forge_hip_model* m, uint32_t token, float* logits_host
     FH_CHECK(logits_host, "forward: null logits");
     int32_t rc = forward_common(m, token);
     if (rc) return rc;
-    FH_HIP(hipMemcpyAsync(logits_host, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, m->stream));
-    return finish_or_undo(m);
+    FH_HIP(hipMemcpyAsync(m->h_logits, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, m->stream));
+    rc = finish_or_undo(m);
+    if (rc) return rc;
+    memcpy(logits_host, m->h_logits, (size_t)m->cfg.vocab * 4);
+    return FORGE_HIP_OK;
 }
 
 int32_t forge_hip_forward_greedy(forge_hip_model* m, uint32_t token, uint32_t* next_token_host) {
@@ -570,9 +576,10 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint
     if (logits_host) {
         enqueue_head(m, m->px.as<float>() + (size_t)(last_rows - 1) * m->H, true, false);
         FH_HIP(hipGetLastError());
-        FH_HIP(hipMemcpyAsync(logits_host, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, s));
+        FH_HIP(hipMemcpyAsync(m->h_logits, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, s));
     }
     FH_HIP(hipStreamSynchronize(s));
+    if (logits_host) memcpy(logits_host, m->h_logits, (size_t)m->cfg.vocab * 4);
     return FORGE_HIP_OK;
 }
 
