@@ -411,24 +411,49 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         if (tid == 0) __hip_atomic_store(sp.counters + range_tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch (stream order)
     }
 
-    // epilogue: lane holds column n = lrow, rows 8g + 4*lhalf + (r&3); the descriptor drops rows >= M
+    // epilogue: lane holds column n = lrow, rows 8g + 4*lhalf + (r&3); the descriptor drops rows >= M.
+    // y += ...: all of a lane's old values are requested before the first is used (a load, its wait, the add and the
+    // store per element would be 64 memory round trips one after the other: every wait also waits for the store before it)
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc((void*)y, 0, M * ldy * 4, RSRC_FLAGS);
+    auto offset_of = [&](int tm, int tn, int r) {
+        const uint32_t n = n0 + wn * 64 + tn * 32 + lrow;
+        const uint32_t mb = m0 + wm * WM + tm * 32 + 4 * lhalf;
+        const uint32_t base = n < N ? (mb * ldy + n) * 4 : OOB;
+        return base + (8 * (r >> 2) + (r & 3)) * ldy * 4;
+    };
+    if (accumulate) {
+        float old[TM][2][16];
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) old[tm][tn][r] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ry, offset_of(tm, tn, r), 0, 0));
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float v = acc[tm][tn][r];
+                    if (MAGIC && Q4) v *= 0.0625f;
+                    acc[tm][tn][r] = old[tm][tn][r] + v;
+                }
+    } else if (MAGIC && Q4) {
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[tm][tn][r] *= 0.0625f;
+    }
 #pragma unroll
     for (int tm = 0; tm < TM; tm++)
 #pragma unroll
-        for (int tn = 0; tn < 2; tn++) {
-            const uint32_t n = n0 + wn * 64 + tn * 32 + lrow;
-            const uint32_t mb = m0 + wm * WM + tm * 32 + 4 * lhalf;
-            const uint32_t base = n < N ? (mb * ldy + n) * 4 : OOB;
+        for (int tn = 0; tn < 2; tn++)
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                const uint32_t off = base + (8 * (r >> 2) + (r & 3)) * ldy * 4;
-                float v = acc[tm][tn][r];
-                if (MAGIC && Q4) v *= 0.0625f;
-                if (accumulate) v = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(ry, off, 0, 0)) + v;
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), ry, off, 0, 0);
-            }
-        }
+            for (int r = 0; r < 16; r++)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, acc[tm][tn][r]), ry, offset_of(tm, tn, r), 0, 0);
 }
 
 // The kernel addresses each matrix with 32-bit byte offsets below 2^31: larger problems are cut into
