@@ -869,7 +869,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
         }
         if (cx.tid < ((t.rows + 63u) & ~63u)) {
             float v = 0.f;
-            if (mine) v = ORDERED ? ordered_sum(big + cx.tid * pstride, h.nblk, segment_row_is_dot1(row, g.seg, g.nseg, g.tail_mod)) : (big[cx.tid * 4] + big[cx.tid * 4 + 1]) + (big[cx.tid * 4 + 2] + big[cx.tid * 4 + 3]);
+            if (mine) v = ORDERED ? ordered_sum_words(big + cx.tid * pstride, h.nblk, segment_row_is_dot1(row, g.seg, g.nseg, g.tail_mod)) : (big[cx.tid * 4] + big[cx.tid * 4 + 1]) + (big[cx.tid * 4 + 2] + big[cx.tid * 4 + 3]);
             if (job.epi == EPI_ROPE) {
                 if (PEN && job.bias && mine) v = v + job.bias[row];      // the kernel variant with the optional extras carries it
                 // rope (emit.rs:508-528): rows 2i, 2i+1 of a head sit in neighbouring lanes

@@ -80,29 +80,39 @@ __device__ __forceinline__ bool row_is_dot1(uint32_t row, const GemvArgs& a) {
     return segment_row_is_dot1(row, a.seg, a.nseg, a.tail_mod);
 }
 
-template <bool Q4, int NCH, int RW, int WAVES, Pro PRO, Epi EPI>
+// KS > 1: a group's rows are worked by KS waves, each taking every KS-th chunk of K (its share of the activation
+// fragment, of the loads to issue and of the products) — a wave that is alone on its SIMD issues an instruction only
+// every few nanoseconds, so on the small matrices, where there is one workgroup per CU, what a wave has to issue is
+// what the kernel takes.  The products meet in LDS as before and the first of the KS waves adds them in order.
+template <bool Q4, int NCH, int RW, int WAVES, int KS, Pro PRO, Epi EPI>
 __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
-    extern __shared__ float lds[];
+    static_assert(NCH % KS == 0 && WAVES % KS == 0, "K split must divide the chunks and the waves");
+    static_assert(KS == 1 || (EPI != Epi::SiluQuant && EPI != Epi::Isums), "no K split in these variants");
+    extern __shared__ __align__(16) float lds[];
     constexpr uint32_t THREADS = WAVES * 64;
+    constexpr int NL = NCH / KS;                             // chunks per wave
+    constexpr uint32_t RWAVES = WAVES / KS;                  // row groups per workgroup
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t kpart = KS == 1 ? 0u : wave % KS, rwave = KS == 1 ? wave : wave / KS;
     const uint32_t K = a.K, N = a.N, nblk = K / 32;
-    const uint32_t pstride = nblk + 1;                       // +1: conflict-free column reads
-    float* prod = lds + (size_t)wave * a.rc * pstride;
-    float* shared_tail = lds + (size_t)WAVES * a.rc * pstride;   // prologue / epilogue scratch
+    const uint32_t pstride = prod_stride(nblk);
+    float* prod = lds + (size_t)rwave * a.rc * pstride;
+    float* shared_tail = lds + (size_t)RWAVES * a.rc * pstride;   // prologue / epilogue scratch
+    auto chunk = [&](int j) -> uint32_t { return (uint32_t)j * KS + kpart; };   // this wave's j-th chunk of K
 
-    uint32_t blk[NCH];
-    bool own[NCH];                                           // this lane reports block blk[j]
+    uint32_t blk[NL];
+    bool own[NL];                                            // this lane reports block blk[j]
 #pragma unroll
-    for (int j = 0; j < NCH; j++) {
-        if (Q4) { blk[j] = j * 64 + lane; own[j] = blk[j] < nblk; }
-        else { const uint32_t off = j * 1024 + lane * 16; blk[j] = off / 32; own[j] = off < K && !(lane & 1); }
+    for (int j = 0; j < NL; j++) {
+        if (Q4) { blk[j] = chunk(j) * 64 + lane; own[j] = blk[j] < nblk; }
+        else { const uint32_t off = chunk(j) * 1024 + lane * 16; blk[j] = off / 32; own[j] = off < K && !(lane & 1); }
     }
 
     // ---- row groups.  Standard: wave w of workgroup-group g0 owns rows [(g0+w) rc, +rc).
     //      SiluQuant (WAVES = 16, rc = 4): workgroup G owns inter indices [32 G, +32): waves 0..7 take the
     //      gate rows, waves 8..15 the up rows, four rows each.
     const uint32_t ngroups = EPI == Epi::SiluQuant ? (a.inter + 31) / 32 : (N + a.rc - 1) / a.rc;
-    const uint32_t gstep = EPI == Epi::SiluQuant ? 1 : WAVES;
+    const uint32_t gstep = EPI == Epi::SiluQuant ? 1 : RWAVES;
     auto rows_of = [&](uint32_t g0, uint32_t& row_base, uint32_t& row_end) -> bool {
         if (EPI == Epi::SiluQuant) {
             const uint32_t i0 = g0 * 32 + (wave & 7) * 4;
@@ -110,27 +120,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
             row_end = (wave >> 3) * a.inter + min(a.inter, i0 + 4);
             return i0 < a.inter;
         }
-        const uint32_t g = g0 + wave;                        // may be >= ngroups: idle but keeps the barriers uniform
+        const uint32_t g = g0 + rwave;                       // may be >= ngroups: idle but keeps the barriers uniform
         row_base = g * a.rc;
         row_end = min(N, row_base + a.rc);
         return g < ngroups;
     };
 
-    int4 wv[RW][NCH];
-    uint16_t wsb[RW][NCH];
+    int4 wv[RW][NL];
+    uint16_t wsb[RW][NL];
     auto load_rows = [&](uint32_t row0, uint32_t row_end) {
 #pragma unroll
         for (int r = 0; r < RW; r++) {
             const uint32_t row = min(row0 + r, row_end - 1);
 #pragma unroll
-            for (int j = 0; j < NCH; j++) {
+            for (int j = 0; j < NL; j++) {
                 if (Q4) {
                     if (blk[j] < nblk) {
                         wv[r][j] = *reinterpret_cast<const int4*>(a.qs + ((size_t)row * nblk + blk[j]) * 16);
                         wsb[r][j] = a.ws[(size_t)row * nblk + blk[j]];
                     } else { wv[r][j] = make_int4(0, 0, 0, 0); wsb[r][j] = 0; }
                 } else {
-                    const uint32_t off = j * 1024 + lane * 16;
+                    const uint32_t off = chunk(j) * 1024 + lane * 16;
                     if (off < K) {
                         wv[r][j] = *reinterpret_cast<const int4*>(a.qs + (size_t)row * K + off);
                         wsb[r][j] = a.ws[(size_t)row * nblk + blk[j]];
@@ -141,17 +151,27 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
     };
 
     // Weights do not depend on the activations: start streaming the first rows before the prologue.
+    // The order in which this lane will add its row's products (lane i of a wave adds row i of the wave's group) is
+    // worked out here as well, for the first group: a lone wave on a SIMD issues an instruction every few nanoseconds,
+    // and these hundred-odd cost nothing while the loads are in flight.  Pinned, or the compiler moves them down in
+    // front of their use behind the products barrier.
     bool prefetched = false;
+    uint32_t d1_first = 0;
     {
         uint32_t rb, re;
         const uint32_t g0 = blockIdx.x * gstep;
-        if (g0 < ngroups && rows_of(g0, rb, re) && rb < re) { load_rows(rb, re); prefetched = true; }
+        if (g0 < ngroups && rows_of(g0, rb, re) && rb < re) {
+            load_rows(rb, re); prefetched = true;
+            if (EPI != Epi::Isums && kpart == 0 && lane < a.rc && rb + lane < re) d1_first = row_is_dot1(rb + lane, a);
+        }
+        asm volatile("" : "+v"(d1_first));
     }
+    bool first_group = true;
 
     // ---- activation fragment, resident for the whole kernel
-    int4 av[NCH], av2[Q4 ? NCH : 1];
-    int asum8[Q4 ? NCH : 1];
-    float asf[NCH];
+    int4 av[NL], av2[Q4 ? NL : 1];
+    int asum8[Q4 ? NL : 1];
+    float asf[NL];
     if (PRO == Pro::RmsNorm) {
         // rms_norm of x[K] in the reference's summation order, then block quantisation, all in-kernel
         float* xs = shared_tail;                              // K floats + 17
@@ -183,9 +203,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
         __syncthreads();
         const float inv_rms = 1.0f / sqrtf(part[16] / (float)K + a.eps);
 #pragma unroll
-        for (int j = 0; j < NCH; j++) {
-            // the 16 (Q8 layout) or 32 (Q4 layout) consecutive elements this lane holds of chunk j
-            const uint32_t e0 = Q4 ? (j * 64 + lane) * 32 : j * 1024 + lane * 16;
+        for (int j = 0; j < NL; j++) {
+            // the 16 (Q8 layout) or 32 (Q4 layout) consecutive elements this lane holds of its j-th chunk
+            const uint32_t e0 = Q4 ? (chunk(j) * 64 + lane) * 32 : chunk(j) * 1024 + lane * 16;
             constexpr int CNT = Q4 ? 32 : 16;
             float v[CNT];
             float amax = 0.f;
@@ -215,14 +235,14 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
         __syncthreads();   // xs is free again (SiluQuant reuses the tail)
     } else {
 #pragma unroll
-        for (int j = 0; j < NCH; j++) {
+        for (int j = 0; j < NL; j++) {
             if (Q4) {
                 if (own[j]) {
                     av[j] = *reinterpret_cast<const int4*>(a.aq + (size_t)blk[j] * 32);
                     av2[j] = *reinterpret_cast<const int4*>(a.aq + (size_t)blk[j] * 32 + 16);
                 } else { av[j] = av2[j] = make_int4(0, 0, 0, 0); }
             } else {
-                const uint32_t off = j * 1024 + lane * 16;
+                const uint32_t off = chunk(j) * 1024 + lane * 16;
                 av[j] = off < K ? *reinterpret_cast<const int4*>(a.aq + off) : make_int4(0, 0, 0, 0);
             }
             asf[j] = (EPI != Epi::Isums && blk[j] < nblk) ? f16_bits_to_f32(a.as[blk[j]]) : 0.f;
@@ -231,12 +251,18 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
     if (Q4) {
         const int4 ones = make_int4(0x01010101, 0x01010101, 0x01010101, 0x01010101);
 #pragma unroll
-        for (int j = 0; j < NCH; j++) asum8[j] = 8 * dot16(ones, av2[j], dot16(ones, av[j], 0));
+        for (int j = 0; j < NL; j++) asum8[j] = 8 * dot16(ones, av2[j], dot16(ones, av[j], 0));
     }
 
     for (uint32_t g0 = blockIdx.x * gstep; g0 < ngroups; g0 += gridDim.x * gstep) {
         uint32_t row_base, row_end;   // this wave's rows [row_base, row_end)
         const bool wave_on = rows_of(g0, row_base, row_end);
+        uint32_t d1 = d1_first;
+        if (!first_group) {
+            d1 = (EPI != Epi::Isums && wave_on && kpart == 0 && lane < a.rc && row_base + lane < row_end) ? row_is_dot1(row_base + lane, a) : 0u;
+            asm volatile("" : "+v"(d1));
+        }
+        first_group = false;
         if (wave_on) {
             for (uint32_t sub = 0; sub < a.rc; sub += RW) {
                 if (row_base + sub >= row_end) break;
@@ -246,7 +272,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
                 for (int r = 0; r < RW; r++) {
                     const uint32_t row = row_base + sub + r;
 #pragma unroll
-                    for (int j = 0; j < NCH; j++) {
+                    for (int j = 0; j < NL; j++) {
                         int isum;
                         if (Q4) {
                             const int4 w = wv[r][j];
@@ -269,11 +295,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
         prefetched = false;
         if (EPI == Epi::Isums) continue;
         __syncthreads();
-        // ---- ordered sums: lane i of the wave owns row row_base + i
+        // ---- ordered sums: lane i of the group's (first) wave owns row row_base + i
         const uint32_t row = row_base + lane;
-        const bool active = wave_on && lane < a.rc && row < row_end;
+        const bool active = wave_on && kpart == 0 && lane < a.rc && row < row_end;
         float r = 0.f;
-        if (active) r = ordered_sum(prod + lane * pstride, nblk, row_is_dot1(row, a));
+        if (active) r = ordered_sum(prod + lane * pstride, nblk, d1 != 0);
         if (EPI == Epi::Store) {
             if (active) a.y[row] = r;
         } else if (EPI == Epi::Add) {
@@ -315,8 +341,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
             }
             // the next iteration's first barrier orders these reads before res[] is rewritten
         }
-        // the product area is private to the wave and LDS operations of one wave execute in order,
-        // so no barrier is needed before the next group overwrites it
+        // KS = 1: the product area is private to the wave and LDS operations of one wave execute in order, so no
+        // barrier is needed before the next group overwrites it; shared between waves it is
+        if (KS > 1) __syncthreads();
     }
 }
 
@@ -341,45 +368,63 @@ size_t lds_tail_bytes(bool norm, bool silu, uint32_t K) {
     return tail;
 }
 
-template <bool Q4, int NCH, int RW, Pro PRO, Epi EPI>
+template <bool Q4, int NCH, int RW, Pro PRO, Epi EPI, int KS = 1>
 void launch_one(GemvArgs a, hipStream_t s) {
-    constexpr int WAVES = EPI == Epi::SiluQuant ? 16 : 4;
+    constexpr int WAVES = EPI == Epi::SiluQuant ? 16 : 4;      // waves that own row groups; the kernel runs WAVES * KS
     const uint32_t nblk = a.K / 32;
     const size_t tail = lds_tail_bytes(PRO == Pro::RmsNorm, EPI == Epi::SiluQuant, a.K);
     a.rc = EPI == Epi::SiluQuant ? 4 : rows_per_group(nblk, a.N, RW);
     // shrink the group if the products and the prologue's copy of x do not fit LDS together
     constexpr uint32_t step = RW < 2 ? 2 : RW;
-    while (EPI != Epi::SiluQuant && a.rc > step && (size_t)WAVES * a.rc * (nblk + 1) * sizeof(float) + tail > LDS_LIMIT) a.rc -= step;
+    while (EPI != Epi::SiluQuant && a.rc > step && (size_t)WAVES * a.rc * prod_stride(nblk) * sizeof(float) + tail > LDS_LIMIT) a.rc -= step;
     const uint32_t ngroups = EPI == Epi::SiluQuant ? (a.inter + 31) / 32 : ((a.N + a.rc - 1) / a.rc + WAVES - 1) / WAVES;
     uint32_t grid = ngroups;
     if (grid > 256 * 8) grid = 256 * 8;
-    const size_t lds = EPI == Epi::Isums ? 0 : (size_t)WAVES * a.rc * (nblk + 1) * sizeof(float);
-    fh::launch(gemv_kernel<Q4, NCH, (EPI == Epi::SiluQuant ? (RW > 4 ? 4 : RW) : RW), WAVES, PRO, EPI>, grid, WAVES * 64, lds + tail, s, a);
+    const size_t lds = EPI == Epi::Isums ? 0 : (size_t)WAVES * a.rc * prod_stride(nblk) * sizeof(float);
+    fh::launch(gemv_kernel<Q4, NCH, (EPI == Epi::SiluQuant ? (RW > 4 ? 4 : RW) : RW), WAVES * KS, KS, PRO, EPI>, grid, WAVES * KS * 64, lds + tail, s, a);
 }
 
 template <Pro PRO, Epi EPI>
 void dispatch(uint32_t wdtype, const GemvArgs& a, hipStream_t s) {
-    // SiluQuant walks 16 rows per wave; RW must divide 16 (it always does)
+    // SiluQuant walks 16 rows per wave; RW must divide 16 (it always does).
+    // Matrices of few rows (everything but an lm_head) leave a CU with a handful of waves: there K is dealt to KS waves
+    // per row group, the largest KS on offer that keeps the launch within 16 waves per CU.
+    constexpr bool CAN_SPLIT = EPI != Epi::SiluQuant && EPI != Epi::Isums;
+    auto fits = [&](int rw, int ks) {
+        const uint32_t rc = rows_per_group(a.K / 32, a.N, rw);
+        return (uint64_t)((a.N + rc - 1) / rc) * ks <= 256u * 16u;
+    };
+#define FH_GEMV_ONE(Q4_, NCH_, RW_, KSA_, KSB_)                                                   \
+    do {                                                                                          \
+        if constexpr (CAN_SPLIT && KSA_ > 1) {                                                    \
+            if (fits(RW_, KSA_)) { launch_one<Q4_, NCH_, RW_, PRO, EPI, KSA_>(a, s); break; }     \
+        }                                                                                         \
+        if constexpr (CAN_SPLIT && KSB_ > 1) {                                                    \
+            if (fits(RW_, KSB_)) { launch_one<Q4_, NCH_, RW_, PRO, EPI, KSB_>(a, s); break; }     \
+        }                                                                                         \
+        launch_one<Q4_, NCH_, RW_, PRO, EPI>(a, s);                                               \
+    } while (0)
     if (wdtype == FORGE_HIP_Q8_0) {
         const uint32_t nch = (a.K + 1023) / 1024;
         switch (nch) {
-            case 1: launch_one<false, 1, 4, PRO, EPI>(a, s); break;
-            case 2: launch_one<false, 2, 4, PRO, EPI>(a, s); break;
-            case 3: launch_one<false, 3, 2, PRO, EPI>(a, s); break;
-            case 4: launch_one<false, 4, 2, PRO, EPI>(a, s); break;
-            case 5: case 6: launch_one<false, 6, 2, PRO, EPI>(a, s); break;
-            case 7: case 8: launch_one<false, 8, 2, PRO, EPI>(a, s); break;
-            default: launch_one<false, 16, 1, PRO, EPI>(a, s); break;
+            case 1: FH_GEMV_ONE(false, 1, 4, 1, 1); break;
+            case 2: FH_GEMV_ONE(false, 2, 4, 2, 1); break;
+            case 3: FH_GEMV_ONE(false, 3, 2, 1, 1); break;
+            case 4: FH_GEMV_ONE(false, 4, 2, 4, 2); break;
+            case 5: case 6: FH_GEMV_ONE(false, 6, 2, 2, 1); break;
+            case 7: case 8: FH_GEMV_ONE(false, 8, 2, 4, 2); break;
+            default: FH_GEMV_ONE(false, 16, 1, 4, 2); break;
         }
     } else {
         const uint32_t nch = (a.K + 2047) / 2048;
         switch (nch) {
-            case 1: launch_one<true, 1, 4, PRO, EPI>(a, s); break;
-            case 2: launch_one<true, 2, 4, PRO, EPI>(a, s); break;
-            case 3: case 4: launch_one<true, 4, 2, PRO, EPI>(a, s); break;
-            default: launch_one<true, 8, 1, PRO, EPI>(a, s); break;
+            case 1: FH_GEMV_ONE(true, 1, 4, 1, 1); break;
+            case 2: FH_GEMV_ONE(true, 2, 4, 2, 1); break;
+            case 3: case 4: FH_GEMV_ONE(true, 4, 2, 4, 2); break;
+            default: FH_GEMV_ONE(true, 8, 1, 4, 2); break;
         }
     }
+#undef FH_GEMV_ONE
 }
 
 GemvArgs base_args(const QWeight& w, GemvOrder order) {
@@ -398,10 +443,10 @@ bool gemv_k_supported(uint32_t K) { return K % 32 == 0 && K >= 32 && K <= 16384;
 // Whether the fused prologue / epilogue variants fit LDS for this K (else the caller launches the
 // separate kernels).
 bool gemv_norm_fusable(uint32_t K) {
-    return gemv_k_supported(K) && (size_t)4 * 4 * (K / 32 + 1) * sizeof(float) + lds_tail_bytes(true, false, K) <= LDS_LIMIT;
+    return gemv_k_supported(K) && (size_t)4 * 4 * prod_stride(K / 32) * sizeof(float) + lds_tail_bytes(true, false, K) <= LDS_LIMIT;
 }
 bool gemv_silu_fusable(uint32_t K) {
-    return gemv_k_supported(K) && (size_t)16 * 4 * (K / 32 + 1) * sizeof(float) + lds_tail_bytes(true, true, K) <= LDS_LIMIT;
+    return gemv_k_supported(K) && (size_t)16 * 4 * prod_stride(K / 32) * sizeof(float) + lds_tail_bytes(true, true, K) <= LDS_LIMIT;
 }
 
 void launch_gemv(const QWeight& w, const int8_t* aq, const uint16_t* as, float* y, bool accumulate, GemvOrder order,

@@ -38,7 +38,7 @@ __device__ __forceinline__ int sub32x4(uint32_t x) { return (int)(((x | 0x808080
 constexpr int KQ_WAVES = 4;
 
 // LDS: the activation codes [K], their scales as f32 [K/32], (Q4_K) their sums as f32 [K/32], then per wave the products
-// [RW][K/32 + 1].  A wave works RW rows at a time: all their loads are issued before the first is used (one row of
+// [RW][prod_stride(K/32)].  A wave works RW rows at a time: all their loads are issued before the first is used (one row of
 // K = 2048 is a single kilobyte, far too little in flight for HBM), and lane r adds row r's products in block order.
 template <bool Q6, int RW>
 __global__ __launch_bounds__(KQ_WAVES * 64) void gemv_kquant_kernel(const uint8_t* __restrict__ qs, const uint8_t* __restrict__ meta,
@@ -46,7 +46,7 @@ __global__ __launch_bounds__(KQ_WAVES * 64) void gemv_kquant_kernel(const uint8_
                                                                   float* __restrict__ y, uint32_t K, uint32_t N, int accumulate) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t nblk = K / 32, nsb = K / 256, pstride = nblk + 1;
+    const uint32_t nblk = K / 32, nsb = K / 256, pstride = prod_stride(nblk);
     int8_t* xa = reinterpret_cast<int8_t*>(lds);
     float* xs = reinterpret_cast<float*>(lds + K);
     float* xsum = xs + nblk;
@@ -195,7 +195,7 @@ void launch_gemv_kquant(const QWeight& w, const int8_t* aq, const uint16_t* as, 
     const uint32_t nblk = w.K / 32;
     // rows a wave keeps in flight: four when that still leaves every CU several workgroups
     const int rw = w.N >= 16384 ? 4 : w.N >= 4096 ? 2 : 1;
-    const size_t lds = (size_t)w.K + (size_t)nblk * 8 + (size_t)KQ_WAVES * rw * (nblk + 1) * 4;
+    const size_t lds = (size_t)w.K + (size_t)nblk * 8 + (size_t)KQ_WAVES * rw * prod_stride(nblk) * 4;
     uint32_t grid = (w.N + KQ_WAVES * rw - 1) / (KQ_WAVES * rw);
     if (grid > 256 * 8) grid = 256 * 8;
     const uint8_t* meta = reinterpret_cast<const uint8_t*>(w.scales);
