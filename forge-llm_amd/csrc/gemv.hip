@@ -150,6 +150,20 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
         }
     };
 
+    // Pro::RmsNorm: x and the norm weights are requested first (the first XE float4 per thread; what lies beyond is
+    // fetched later, behind the weights): loads return in issue order, so behind the weights they would arrive only after them, and the
+    // norm would wait for the weights instead of running while they travel.
+    constexpr int XE = THREADS >= 1024 ? 1 : THREADS >= 512 ? 2 : 4;   // 4096 elements, at 16 waves within their 128 registers
+    float4 xe[PRO == Pro::RmsNorm ? XE : 1], we[PRO == Pro::RmsNorm ? XE : 1];
+    if (PRO == Pro::RmsNorm) {
+#pragma unroll
+        for (int i = 0; i < XE; i++) {
+            const uint32_t e4 = i * THREADS + tid;
+            xe[i] = we[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (e4 < K / 4) { xe[i] = reinterpret_cast<const float4*>(a.x)[e4]; we[i] = reinterpret_cast<const float4*>(a.norm_w)[e4]; }
+        }
+    }
+
     // Weights do not depend on the activations: start streaming the first rows before the prologue.
     // The order in which this lane will add its row's products (lane i of a wave adds row i of the wave's group) is
     // worked out here as well, for the first group: a lone wave on a SIMD issues an instruction every few nanoseconds,
@@ -173,10 +187,15 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
     int asum8[Q4 ? NL : 1];
     float asf[NL];
     if (PRO == Pro::RmsNorm) {
-        // rms_norm of x[K] in the reference's summation order, then block quantisation, all in-kernel
-        float* xs = shared_tail;                              // K floats + 17
-        float* part = xs + K;
-        for (uint32_t i = tid; i < K / 4; i += THREADS) reinterpret_cast<float4*>(xs)[i] = reinterpret_cast<const float4*>(a.x)[i];
+        // rms_norm of x[K] in the reference's summation order, then block quantisation, once per workgroup: 8 lanes
+        // share a block of 32, codes and scales go to LDS and every wave picks its fragment up from there
+        float* xs = shared_tail;                              // K floats
+        float* part = xs + K;                                 // 17 (32 reserved)
+        float* qsc = part + 32;                               // K/32 scales, as the f32 value of their fp16 rounding
+        uint32_t* qcd = reinterpret_cast<uint32_t*>(qsc + ((nblk + 3u) & ~3u));   // K codes, 16-byte aligned
+#pragma unroll
+        for (int i = 0; i < XE; i++) { const uint32_t e4 = i * THREADS + tid; if (e4 < K / 4) reinterpret_cast<float4*>(xs)[e4] = xe[i]; }
+        for (uint32_t e4 = XE * THREADS + tid; e4 < K / 4; e4 += THREADS) reinterpret_cast<float4*>(xs)[e4] = reinterpret_cast<const float4*>(a.x)[e4];
         __syncthreads();
         if (tid < 16) {
             float s = 0.f;
@@ -202,37 +221,30 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
         }
         __syncthreads();
         const float inv_rms = 1.0f / sqrtf(part[16] / (float)K + a.eps);
+        auto quantise4 = [&](uint32_t e4, float4 xv, float4 w4) {
+            const float4 v = make_float4(xv.x * inv_rms * w4.x, xv.y * inv_rms * w4.y, xv.z * inv_rms * w4.z, xv.w * inv_rms * w4.w);
+            uint16_t sb;
+            qcd[e4] = quantize_block_part(v, sb);
+            if ((e4 & 7u) == 0) qsc[e4 >> 3] = f16_bits_to_f32(sb);
+        };
+        // (K / 4 is a multiple of 8 and so is THREADS: the 8 lanes of a block are in or out together)
+#pragma unroll
+        for (int i = 0; i < XE; i++) { const uint32_t e4 = i * THREADS + tid; if (e4 < K / 4) quantise4(e4, reinterpret_cast<const float4*>(xs)[e4], we[i]); }
+        for (uint32_t e4 = XE * THREADS + tid; e4 < K / 4; e4 += THREADS) quantise4(e4, reinterpret_cast<const float4*>(xs)[e4], reinterpret_cast<const float4*>(a.norm_w)[e4]);
+        __syncthreads();
 #pragma unroll
         for (int j = 0; j < NL; j++) {
-            // the 16 (Q8 layout) or 32 (Q4 layout) consecutive elements this lane holds of its j-th chunk
-            const uint32_t e0 = Q4 ? (chunk(j) * 64 + lane) * 32 : chunk(j) * 1024 + lane * 16;
-            constexpr int CNT = Q4 ? 32 : 16;
-            float v[CNT];
-            float amax = 0.f;
-            const bool in = e0 < K;
-#pragma unroll
-            for (int i = 0; i < CNT / 4; i++) {
-                float4 xv = make_float4(0.f, 0.f, 0.f, 0.f), wv4 = xv;
-                if (in) { xv = reinterpret_cast<const float4*>(xs + e0)[i]; wv4 = reinterpret_cast<const float4*>(a.norm_w + e0)[i]; }
-                v[4 * i] = xv.x * inv_rms * wv4.x; v[4 * i + 1] = xv.y * inv_rms * wv4.y;
-                v[4 * i + 2] = xv.z * inv_rms * wv4.z; v[4 * i + 3] = xv.w * inv_rms * wv4.w;
+            const uint8_t* codes = reinterpret_cast<const uint8_t*>(qcd);
+            if (Q4) {
+                av[j] = av2[j] = make_int4(0, 0, 0, 0);
+                if (own[j]) { av[j] = *reinterpret_cast<const int4*>(codes + (size_t)blk[j] * 32); av2[j] = *reinterpret_cast<const int4*>(codes + (size_t)blk[j] * 32 + 16); }
+            } else {
+                const uint32_t off = chunk(j) * 1024 + lane * 16;
+                av[j] = off < K ? *reinterpret_cast<const int4*>(codes + off) : make_int4(0, 0, 0, 0);
             }
-#pragma unroll
-            for (int i = 0; i < CNT; i++) amax = fmaxf(amax, fabsf(v[i]));
-            if (!Q4) amax = fmaxf(amax, __shfl_xor(amax, 1, WAVE));   // the other half of the block
-            float inv;
-            const float sc = act_scale(amax, inv);
-            asf[j] = in ? f16_bits_to_f32(f32_to_f16_bits(sc)) : 0.f;
-            uint32_t pk[CNT / 4];
-#pragma unroll
-            for (int i = 0; i < CNT / 4; i++) {
-                pk[i] = ((uint32_t)quant_code(v[4 * i] * inv) & 0xFFu) | (((uint32_t)quant_code(v[4 * i + 1] * inv) & 0xFFu) << 8) |
-                        (((uint32_t)quant_code(v[4 * i + 2] * inv) & 0xFFu) << 16) | (((uint32_t)quant_code(v[4 * i + 3] * inv) & 0xFFu) << 24);
-            }
-            av[j] = make_int4((int)pk[0], (int)pk[1], (int)pk[2], (int)pk[3]);
-            if (Q4) av2[j] = make_int4((int)pk[CNT / 4 - 4], (int)pk[CNT / 4 - 3], (int)pk[CNT / 4 - 2], (int)pk[CNT / 4 - 1]);
+            asf[j] = blk[j] < nblk ? qsc[blk[j]] : 0.f;
         }
-        __syncthreads();   // xs is free again (SiluQuant reuses the tail)
+        // (the SiluQuant epilogue reuses the first words of the tail: x, which nobody reads after the barrier above)
     } else {
 #pragma unroll
         for (int j = 0; j < NL; j++) {
@@ -256,6 +268,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
 
     for (uint32_t g0 = blockIdx.x * gstep; g0 < ngroups; g0 += gridDim.x * gstep) {
         uint32_t row_base, row_end;   // this wave's rows [row_base, row_end)
+        // the row distance is read afresh in every pass: otherwise the LDS address of every (row, chunk) product is
+        // worked out ahead of the loop and kept, which at 16 waves per workgroup (128 registers) ends in spills that
+        // are reloaded, one memory round trip each, between the products
+        uint32_t ps = pstride;
+        asm volatile("" : "+s"(ps));
         const bool wave_on = rows_of(g0, row_base, row_end);
         uint32_t d1 = d1_first;
         if (!first_group) {
@@ -286,7 +303,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
                         }
                         if (own[j] && row < row_end) {
                             if (EPI == Epi::Isums) a.isums[(size_t)row * nblk + blk[j]] = isum;
-                            else prod[(sub + r) * pstride + blk[j]] = (asf[j] * f16_bits_to_f32(wsb[r][j])) * (float)isum;
+                            else prod[(sub + r) * ps + blk[j]] = (asf[j] * f16_bits_to_f32(wsb[r][j])) * (float)isum;
                         }
                     }
                 }
@@ -299,7 +316,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
         const uint32_t row = row_base + lane;
         const bool active = wave_on && kpart == 0 && lane < a.rc && row < row_end;
         float r = 0.f;
-        if (active) r = ordered_sum(prod + lane * pstride, nblk, d1 != 0);
+        if (active) r = ordered_sum(prod + lane * ps, nblk, d1 != 0);
         if (EPI == Epi::Store) {
             if (active) a.y[row] = r;
         } else if (EPI == Epi::Add) {
@@ -363,7 +380,8 @@ uint32_t rows_per_group(uint32_t nblk, uint32_t N, uint32_t rw) {
 
 constexpr size_t LDS_LIMIT = 64 * 1024;
 size_t lds_tail_bytes(bool norm, bool silu, uint32_t K) {
-    size_t tail = norm ? (size_t)(K + 32) * sizeof(float) : 0;
+    // the norm prologue: x [K] f32, 32 words of partial sums, the scales [K/32] f32 (padded to 16 bytes), the codes [K]
+    size_t tail = norm ? (size_t)(K + 32 + ((K / 32 + 3) & ~3u)) * sizeof(float) + K : 0;
     if (silu && tail < 64 * sizeof(float)) tail = 64 * sizeof(float);
     return tail;
 }
