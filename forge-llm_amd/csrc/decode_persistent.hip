@@ -978,6 +978,10 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     const uint32_t n_steps = 4 * L + (a.seg_last ? 1u : 0u);
 #pragma nounroll
     for (uint32_t step = 0; step < n_steps; step++) {
+        // The thread's number is read afresh in every step: otherwise LDS addresses derived from it are worked out
+        // ahead of the loop, where they do not all fit the 256 registers, and the ones that were parked in scratch
+        // memory came back through a load and a wait for every outstanding load in front of the norm's LDS writes.
+        asm volatile("" : "+v"(cx.tid), "+v"(cx.lane));
         const bool is_lm = step == 4 * L;
         const uint32_t l = is_lm ? L - 1 : step >> 2, ph = is_lm ? 4u : (step & 3u);     // l: index into a.layers
         const uint32_t lg = a.layer0 + l;                     // the layer's number in the model
