@@ -176,6 +176,6 @@ def require_gpu():
 
 
 from .hip_model import HipModel  # noqa: E402
-from . import gguf, ops, synth  # noqa: E402
+from . import gguf, ops, serve, synth  # noqa: E402
 
-__all__ = ["HipModel", "ops", "synth", "Config", "ForgeHipError", "lib", "check", "device_count", "Q4_0", "Q8_0", "FLAG_EXACT"]
+__all__ = ["HipModel", "ops", "serve", "synth", "Config", "ForgeHipError", "lib", "check", "device_count", "Q4_0", "Q8_0", "FLAG_EXACT"]
