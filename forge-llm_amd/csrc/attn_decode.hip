@@ -137,14 +137,16 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(const float* __r
     // merge the key slots of the wave
 #pragma unroll
     for (int g = 0; g < GT; g++) {
-#pragma unroll
-        for (int o = LPK; o < 64; o <<= 1) {
-            float m2 = __shfl_xor(m[g], o, WAVE), l2 = __shfl_xor(l[g], o, WAVE);
+        auto merge_with = [&](auto O) {
+            const float m2 = lane_xor<O.value>(m[g]), l2 = lane_xor<O.value>(l[g]);
             float a2[8];
 #pragma unroll
-            for (int i = 0; i < 8; i++) a2[i] = __shfl_xor(acc[g][i], o, WAVE);
+            for (int i = 0; i < 8; i++) a2[i] = lane_xor<O.value>(acc[g][i]);
             merge_state<8>(m[g], l[g], acc[g], m2, l2, a2);
-        }
+        };
+        if (LPK == 8) merge_with(std::integral_constant<int, 8>{});
+        merge_with(std::integral_constant<int, 16>{});
+        merge_with(std::integral_constant<int, 32>{});
         if (slot == 0 && dvalid) {
 #pragma unroll
             for (int i = 0; i < 8; i++) sh[wave][g][c * 8 + i] = acc[g][i];
@@ -196,9 +198,7 @@ __global__ void attn_decode_combine_kernel(const float* __restrict__ ws, uint32_
     const float o = num * (1.0f / den_s);
     if (out) out[(size_t)h * HD + d] = o;
     if (oq) {
-        float amax = fabsf(o);
-#pragma unroll
-        for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+        const float amax = half_wave_max(fabsf(o));
         float inv;
         const float sc = act_scale(amax, inv);
         oq[(size_t)h * HD + d] = (int8_t)quant_code(o * inv);

@@ -24,8 +24,9 @@ __device__ __forceinline__ float key_dot(const float (&qf)[8], const Half8& kr) 
     float d = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; i++) d = fmaf(qf[i], kf[i], d);
-#pragma unroll
-    for (int o = 1; o < LPK; o <<= 1) d += __shfl_xor(d, o, WAVE);
+    static_assert(LPK == 8 || LPK == 16, "a key row over 8 or 16 lanes");
+    d = lane_xor_add<1>(d); d = lane_xor_add<2>(d); d = lane_xor_add<4>(d);
+    if (LPK == 16) d = lane_xor_add<8>(d);
     return d;
 }
 

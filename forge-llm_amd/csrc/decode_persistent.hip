@@ -672,14 +672,16 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
             for (int hh = 0; hh < NH; hh++) {
                 if (!has[hh]) continue;
                 // merge the key slots of the wave
-#pragma unroll
-                for (int o = LPK; o < 64; o <<= 1) {
-                    float m2 = __shfl_xor(m[hh], o, WAVE), l2 = __shfl_xor(l[hh], o, WAVE);
+                auto merge_with = [&](auto O) {
+                    const float m2 = lane_xor<O.value>(m[hh]), l2 = lane_xor<O.value>(l[hh]);
                     float a2[8];
 #pragma unroll
-                    for (int i = 0; i < 8; i++) a2[i] = __shfl_xor(acc[hh][i], o, WAVE);
+                    for (int i = 0; i < 8; i++) a2[i] = lane_xor<O.value>(acc[hh][i]);
                     merge_state<8>(m[hh], l[hh], acc[hh], m2, l2, a2);
-                }
+                };
+                if (LPK == 8) merge_with(std::integral_constant<int, 8>{});
+                merge_with(std::integral_constant<int, 16>{});
+                merge_with(std::integral_constant<int, 32>{});
                 if (slot == 0 && dvalid) {
                     float* rec = sh + (wave * 4 + gA + 2 * hh) * REC;
 #pragma unroll
@@ -735,15 +737,12 @@ __device__ __forceinline__ void pd_attn_combine(const PdArgs& a, uint32_t tag_in
 #pragma unroll
             for (uint32_t s = 0; s < DECODE_SPLITS; s++) num = fmaf(wgt_s[s], recs[s * REC + d], num);
             const float o = num * (1.0f / wgt_s[DECODE_SPLITS]);
-            float amax = fabsf(o);
-#pragma unroll
-            for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+            const float amax = half_wave_max(fabsf(o));
             float inv;
             const float sc = act_scale(amax, inv);
             const uint32_t code = (uint32_t)quant_code(o * inv) & 0xFFu;
-            const uint32_t base_lane = cx.lane & ~3u;
-            const uint32_t pk = __shfl(code, base_lane, WAVE) | (__shfl(code, base_lane + 1, WAVE) << 8) |
-                                (__shfl(code, base_lane + 2, WAVE) << 16) | (__shfl(code, base_lane + 3, WAVE) << 24);
+            const uint32_t pk = quad_broadcast<0>(code) | (quad_broadcast<1>(code) << 8) | (quad_broadcast<2>(code) << 16) |
+                                (quad_broadcast<3>(code) << 24);
             const uint32_t e = h * HD + d;
             if ((d & 3u) == 0) stc64(a.taq + e / 4, tag_out, pk);
             if ((d & 31u) == 0) stc64(a.taq + a.QKS / 4 + e / 32, tag_out, f32_to_f16_bits(sc));
@@ -873,7 +872,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
             if (job.epi == EPI_ROPE) {
                 if (PEN && job.bias && mine) v = v + job.bias[row];      // the kernel variant with the optional extras carries it
                 // rope (emit.rs:508-528): rows 2i, 2i+1 of a head sit in neighbouring lanes
-                const float other = __shfl_xor(v, 1, WAVE);
+                const float other = lane_xor<1>(v);
                 if (mine) {
                     if (row < a.QKS + a.KV) {
                         const float o = (row & 1u) ? other * rs + v * rc : v * rc - other * rs;
@@ -900,19 +899,16 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
             } else if (job.epi == EPI_SILU) {
                 // lanes 0..31 hold the gate rows of inter indices [32 tile, +32), lanes 32..63 the up rows
                 const uint32_t lr = cx.tid;
-                const float ux = __shfl(v, (cx.lane & 31u) + 32, WAVE);
+                const float ux = lane_xor<32>(v);         // lanes 0..31: the up row of the same inter index
                 if (lr < 32) {
                     // silu_mul, emit.rs:380-386; the C library's expf bit for bit where the reference order is asked for
                     const float o = (v / (1.0f + (ORDERED ? expf_ref<true>(-v) : __expf(-v)))) * ux;
-                    float amax = fabsf(o);
-#pragma unroll
-                    for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+                    const float amax = half_wave_max(fabsf(o));
                     float inv;
                     const float sc = act_scale(amax, inv);
                     const uint32_t code = (uint32_t)quant_code(o * inv) & 0xFFu;
-                    const uint32_t bl = lr & ~3u;
-                    const uint32_t pk = __shfl(code, bl, WAVE) | (__shfl(code, bl + 1, WAVE) << 8) | (__shfl(code, bl + 2, WAVE) << 16) |
-                                        (__shfl(code, bl + 3, WAVE) << 24);
+                    const uint32_t pk = quad_broadcast<0>(code) | (quad_broadcast<1>(code) << 8) | (quad_broadcast<2>(code) << 16) |
+                                        (quad_broadcast<3>(code) << 24);
                     if ((lr & 3u) == 0) stc64(a.taq2 + tile * 8 + lr / 4, job.tag_out, pk);
                     if (lr == 0) stc64(a.taq2 + a.I / 4 + tile, job.tag_out, f32_to_f16_bits(sc));
                 }

@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace fh {
 
 constexpr int WAVE = 64;
@@ -44,14 +46,64 @@ __device__ __forceinline__ float repeat_penalised(float v, uint32_t count, float
     return v;
 }
 
+// Lane exchange lane <-> lane ^ O without the LDS crossbar (`__shfl_xor` compiles to ds_bpermute_b32: an LDS
+// instruction and its latency per step, which is what the short dependent chains of the decode kernels are made of).
+// Inside a row of 16 lanes: DPP moves; across rows: the lane-swap instructions of gfx950.  Every lane of the pairs
+// involved must be active.
+template <int CTRL, typename T>
+__device__ __forceinline__ T dpp_move(T v) { return __builtin_amdgcn_update_dpp((T)0, v, CTRL, 0xF, 0xF, false); }
+template <int O>
+__device__ __forceinline__ uint32_t lane_xor_bits(uint32_t v) {
+    static_assert(O == 1 || O == 2 || O == 4 || O == 8 || O == 16 || O == 32, "one bit of the lane number");
+    if constexpr (O == 1) return dpp_move<0xB1>(v);                      // quad_perm [1,0,3,2]
+    else if constexpr (O == 2) return dpp_move<0x4E>(v);                 // quad_perm [2,3,0,1]
+    else if constexpr (O == 4) {
+        uint32_t r = __builtin_amdgcn_update_dpp(v, v, 0x104, 0xF, 0x5, false);      // row_shl:4 into lanes 0-3, 8-11
+        return __builtin_amdgcn_update_dpp(r, v, 0x114, 0xF, 0xA, false);            // row_shr:4 into lanes 4-7, 12-15
+    } else if constexpr (O == 8) return dpp_move<0x128>(v);              // row_ror:8
+    else if constexpr (O == 16) {
+        // rows 1 and 3 of the first operand change places with rows 0 and 2 of the second
+        const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+        return (__lane_id() & 16u) ? r[0] : r[1];
+    } else {
+        const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+        return (__lane_id() & 32u) ? r[0] : r[1];
+    }
+}
+template <int O> __device__ __forceinline__ float lane_xor(float v) { return __uint_as_float(lane_xor_bits<O>(__float_as_uint(v))); }
+template <int O> __device__ __forceinline__ uint32_t lane_xor(uint32_t v) { return lane_xor_bits<O>(v); }
+template <int O> __device__ __forceinline__ int lane_xor(int v) { return (int)lane_xor_bits<O>((uint32_t)v); }
+
+// v + (lane ^ O's v) and the maximum likewise: across rows both halves of a swap are used as they come (the sum of a
+// pair is the same number whichever of the two lanes computes it).
+template <int O> __device__ __forceinline__ float lane_xor_add(float v) {
+    if constexpr (O == 16) { const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false); return __uint_as_float(r[0]) + __uint_as_float(r[1]); }
+    else if constexpr (O == 32) { const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false); return __uint_as_float(r[0]) + __uint_as_float(r[1]); }
+    else return v + lane_xor<O>(v);
+}
+template <int O> __device__ __forceinline__ float lane_xor_max(float v) {
+    if constexpr (O == 16) { const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false); return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1])); }
+    else if constexpr (O == 32) { const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false); return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1])); }
+    else return fmaxf(v, lane_xor<O>(v));
+}
+// The value of lane (lane & ~3) + I, for the four lanes of a quad.
+template <int I> __device__ __forceinline__ uint32_t quad_broadcast(uint32_t v) { return dpp_move<I * 0x55>(v); }
+
+// Sum over the wave in the pairing order 32, 16, ..., 1 (every lane ends with the same bits).
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
+    v = lane_xor_add<32>(v); v = lane_xor_add<16>(v); v = lane_xor_add<8>(v);
+    v = lane_xor_add<4>(v); v = lane_xor_add<2>(v); v = lane_xor_add<1>(v);
     return v;
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, WAVE));
+    v = lane_xor_max<1>(v); v = lane_xor_max<2>(v); v = lane_xor_max<4>(v);
+    v = lane_xor_max<8>(v); v = lane_xor_max<16>(v); v = lane_xor_max<32>(v);
+    return v;
+}
+// Maximum over the aligned group of 32 lanes.
+__device__ __forceinline__ float half_wave_max(float v) {
+    v = lane_xor_max<1>(v); v = lane_xor_max<2>(v); v = lane_xor_max<4>(v);
+    v = lane_xor_max<8>(v); v = lane_xor_max<16>(v);
     return v;
 }
 
@@ -61,9 +113,9 @@ __device__ __forceinline__ float wave_max(float v) {
 // that way (gemm.hip).
 __device__ __forceinline__ uint32_t quantize_block_part(float4 v, uint16_t& scale_bits, bool negate = false) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-    amax = fmaxf(amax, __shfl_xor(amax, 1, WAVE));
-    amax = fmaxf(amax, __shfl_xor(amax, 2, WAVE));
-    amax = fmaxf(amax, __shfl_xor(amax, 4, WAVE));
+    amax = lane_xor_max<1>(amax);
+    amax = lane_xor_max<2>(amax);
+    amax = lane_xor_max<4>(amax);
     float inv;
     float s = act_scale(amax, inv);
     scale_bits = f32_to_f16_bits(s);

@@ -299,7 +299,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
                             isum = dot16(hi, av2[j], dot16(lo, av[j], 0)) - asum8[j];
                         } else {
                             const int half = dot16(wv[r][j], av[j], 0);
-                            isum = half + __shfl_xor(half, 1, WAVE);
+                            isum = half + lane_xor<1>(half);
                         }
                         if (own[j] && row < row_end) {
                             if (EPI == Epi::Isums) a.isums[(size_t)row * nblk + blk[j]] = isum;
@@ -324,7 +324,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
         } else if (EPI == Epi::RopeKv) {
             // rows 2i, 2i+1 of a head sit in lanes 2i, 2i+1 (row_base and rc are even)
             if (a.bias && active) r = r + a.bias[row];
-            const float other = __shfl_xor(r, 1, WAVE);
+            const float other = lane_xor<1>(r);
             if (active) {
                 const uint32_t pos = *a.pos_dev;
                 if (row < a.qks + a.kv) {
@@ -346,9 +346,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
                 const bool in = i < a.inter;
                 const float gx = in ? res[tid] : 0.f, ux = in ? res[32 + tid] : 0.f;
                 const float o = in ? (gx / (1.0f + expf_ref<true>(-gx))) * ux : 0.f;
-                float amax = fabsf(o);
-#pragma unroll
-                for (int off = 1; off < 32; off <<= 1) amax = fmaxf(amax, __shfl_xor(amax, off, WAVE));
+                const float amax = half_wave_max(fabsf(o));
                 float inv;
                 const float sc = act_scale(amax, inv);
                 if (in) {
