@@ -198,7 +198,7 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
             for (int h = 0; h < KH; h++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) m_tile = fmaxf(m_tile, sacc[h][r]);
-            m_tile = fmaxf(m_tile, __shfl_xor(m_tile, 32, WAVE)) * c2;      // c2 > 0: max commutes with the scaling
+            m_tile = lane_xor_max<32>(m_tile) * c2;      // c2 > 0: max commutes with the scaling
             const float m_new = fmaxf(m_run, m_tile);
             // a query that has seen no key yet (all of these keys masked for it) keeps m = -inf: exponentiate
             // against 0 instead, every p is then 2^-inf = 0
@@ -270,7 +270,7 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
     }
 
     // ---- normalise and store: lane (lq, lh) holds out[qrow][32 d + 8 g + 4 lh + 0..3]
-    const float l_tot = l_run + __shfl_xor(l_run, 32, WAVE);
+    const float l_tot = lane_xor_add<32>(l_run);
     if (QUANT) {
         const float inv_l = 1.0f / l_tot;
         const uint32_t width = heads * HD;
@@ -279,7 +279,7 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
             float o[16], amax = 0.f;
 #pragma unroll
             for (int r = 0; r < 16; r++) { o[r] = oacc[d][r] * inv_l; amax = fmaxf(amax, fabsf(o[r])); }
-            amax = fmaxf(amax, __shfl_xor(amax, 32, WAVE));
+            amax = lane_xor_max<32>(amax);
             float inv;
             const float sc = act_scale(amax, inv);
             // QUANT has no f32 output, so out_stride carries a flag instead: store the odd blocks of a row negated

@@ -758,13 +758,9 @@ __device__ __forceinline__ ArgPair arg_better(ArgPair a, ArgPair b) {
     return take_b ? b : a;
 }
 __device__ __forceinline__ ArgPair arg_wg(ArgPair a, float* misc, const PdCtx& cx) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        ArgPair b;
-        b.v = __shfl_xor(a.v, o, WAVE);
-        b.i = __shfl_xor(a.i, o, WAVE);
-        a = arg_better(a, b);
-    }
+    auto fold = [&](auto O) { a = arg_better(a, ArgPair{lane_xor<O.value>(a.v), lane_xor<O.value>(a.i)}); };
+    fold(std::integral_constant<int, 32>{}); fold(std::integral_constant<int, 16>{}); fold(std::integral_constant<int, 8>{});
+    fold(std::integral_constant<int, 4>{}); fold(std::integral_constant<int, 2>{}); fold(std::integral_constant<int, 1>{});
     ArgPair* sh = reinterpret_cast<ArgPair*>(misc + PD_MISC_SCRATCH);
     __syncthreads();
     if (cx.lane == 0) sh[cx.wave] = a;

@@ -222,13 +222,9 @@ __device__ __forceinline__ ArgPair arg_better(ArgPair a, ArgPair b) {
     return take_b ? b : a;
 }
 __device__ __forceinline__ ArgPair arg_wave(ArgPair a) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        ArgPair b;
-        b.v = __shfl_xor(a.v, o, WAVE);
-        b.i = __shfl_xor(a.i, o, WAVE);
-        a = arg_better(a, b);
-    }
+    auto fold = [&](auto O) { a = arg_better(a, ArgPair{lane_xor<O.value>(a.v), lane_xor<O.value>(a.i)}); };
+    fold(std::integral_constant<int, 32>{}); fold(std::integral_constant<int, 16>{}); fold(std::integral_constant<int, 8>{});
+    fold(std::integral_constant<int, 4>{}); fold(std::integral_constant<int, 2>{}); fold(std::integral_constant<int, 1>{});
     return a;
 }
 __device__ __forceinline__ ArgPair arg_block(ArgPair a, ArgPair* sh) {
