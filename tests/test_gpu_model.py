@@ -159,12 +159,22 @@ def test_graph_replay_matches_eager(fh, torch_gpu, monkeypatch):
 
 
 @pytest.mark.parametrize("wd", [Q8, Q4])
-def test_fused_decode_kernels_equal_separate_kernels(fh, torch_gpu, monkeypatch, wd):
+@pytest.mark.parametrize("shape", ["tiny", "hidden_1536", "hidden_5120"])
+def test_fused_decode_kernels_equal_separate_kernels(fh, torch_gpu, monkeypatch, wd, shape):
     """The decode step with rms_norm / rope / silu fused into the GEMV launches gives the same bits as the
-    step made of separate kernels (same f32 operation order in both)."""
-    cfg = tiny_cfg(fh, wd, EXACT)
+    step made of separate kernels (same f32 operation order in both).  The wider shapes reach what the tiny one does
+    not: a last 1024-element chunk of K that is half empty and K dealt to several waves per row group (1536), a vector
+    longer than what the norm prologue's threads request ahead of the weights (5120)."""
+    if shape == "tiny":
+        cfg = tiny_cfg(fh, wd, EXACT)
+    elif shape == "hidden_1536":
+        cfg = fh.synth.tiny(wdtype=wd, max_seq=640, hidden=1536, inter=2560, layers=2, heads=6, kv_heads=2, head_dim=64, vocab=600)
+        cfg["flags"] = EXACT
+    else:
+        cfg = fh.synth.tiny(wdtype=wd, max_seq=640, hidden=5120, inter=1024, layers=2, heads=8, kv_heads=2, head_dim=128, vocab=600)
+        cfg["flags"] = EXACT
     blob = fh.synth.make_weights_blob(cfg, seed=31)
-    toks = fh.synth.uniform_ids(32, 70, cfg["vocab"])
+    toks = fh.synth.uniform_ids(32, 70 if shape == "tiny" else 24, cfg["vocab"])
     monkeypatch.setenv("FORGE_HIP_FUSE", "0")
     plain = fh.HipModel(cfg, blob)
     monkeypatch.setenv("FORGE_HIP_FUSE", "1")

@@ -88,10 +88,14 @@ def test_block_isums_extreme_codes(fh, oracle, torch_gpu, path):
 
 @pytest.mark.parametrize("wd", [Q8, Q4])
 @pytest.mark.parametrize("K,N", [(2048, 2048), (2048, 512), (8192, 2048), (576, 1536), (3072, 1029), (32, 5),
-                                 (2048, 1283), (96, 7)])
+                                 (2048, 1283), (96, 7), (1536, 301), (5120, 98), (4096, 130), (16384, 42), (8192, 4099),
+                                 (2048, 18001)])
 def test_matmul_vec_bit_exact(fh, oracle, torch_gpu, wd, K, N):
     """Sequential per-block combine, unfused, tail rows in the 4-accumulator order: identical bits.
-    (2048, 1283) is over 1 MB, so the reference chunks rows by 256 and the tail rule applies per chunk."""
+    (2048, 1283) is over 1 MB, so the reference chunks rows by 256 and the tail rule applies per chunk.  The shapes from
+    (1536, 301) on walk the ways K is dealt to the waves of a row group: a half-empty last chunk, six chunks over two
+    waves, four and sixteen over four, a row count at which the split is narrowed to keep the launch within the CUs, and
+    one (18001 rows) at which it is off and a workgroup walks several row groups."""
     torch = torch_gpu
     wraw = make_weight(fh, wd, N, K, seed=3 * N + K)
     x = fh.synth.normal(11 + K, K, 1.0)
