@@ -76,6 +76,7 @@ struct PdGemv {
     uint32_t inter;               // != 0: fused [gate;up] matrix, rows [0,inter) gate, [inter, 2 inter) up
     uint32_t nseg, tail_mod;
     Segment seg[3];
+    uint32_t umagic;              // floor(2^32 / U) + 1: p / U = mulhi(p, umagic) for the few hundred positions of a tile (U >= 2)
 };
 
 // What differs from layer to layer: addresses only.  The shapes of the four matrices are shared.
@@ -385,11 +386,11 @@ struct WReg { int4 v[PD_D]; uint32_t s[PD_D]; };
 __device__ __forceinline__ uint32_t sgpr(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
 
 // The scalar fields of a shape, read once per phase into scalar registers.
-struct Shape { uint32_t K, N, nblk, U, T, ntiles, inter; };
+struct Shape { uint32_t K, N, nblk, U, T, ntiles, inter, umagic; };
 __device__ __forceinline__ Shape pd_shape(const PdGemv& g) {
     Shape h;
     h.K = sgpr(g.K); h.N = sgpr(g.N); h.nblk = sgpr(g.nblk); h.U = sgpr(g.U); h.T = sgpr(g.T); h.ntiles = sgpr(g.ntiles);
-    h.inter = sgpr(g.inter);
+    h.inter = sgpr(g.inter); h.umagic = sgpr(g.umagic);
     return h;
 }
 
@@ -405,7 +406,8 @@ __device__ __forceinline__ TilePos pd_tile(const Shape& g, uint32_t tile) {
     return t;
 }
 __device__ __forceinline__ uint32_t pd_row(const TilePos& t, uint32_t lr) { return t.row0 + lr + (lr >= t.split ? t.jump : 0u); }
-__device__ __forceinline__ uint32_t sdiv(uint32_t a, uint32_t b) { return sgpr(a / b); }
+// position / U without a division: a scalar multiply (host: umagic = floor(2^32 / U) + 1, exact while position * U < 2^32)
+__device__ __forceinline__ uint32_t pos_div_u(uint32_t p, const Shape& h) { return h.U == 1 ? p : sgpr(__umulhi(p, h.umagic)); }
 
 // The weight streamers of a workgroup (waves PD_POLL_WAVES .. PD_WAVES-1, numbered sw = 0 .. PD_STREAM_WAVES-1) split a
 // tile by rows: streamer sw takes tile rows sw, sw + PD_STREAM_WAVES, ... and walks each row's U weight units (1 KB:
@@ -420,7 +422,7 @@ __device__ __forceinline__ void pd_load_round(const GemvJob& job, const Shape& h
     constexpr uint32_t BPU = Q4 ? 64 : 32, BPB = Q4 ? 16 : 32;
     const uint32_t U = h.U, nblk = h.nblk;
     const uint32_t lb = Q4 ? lane : lane >> 1;
-    const uint32_t q = sdiv(round * PD_D, U);
+    const uint32_t q = pos_div_u(round * PD_D, h);
     uint32_t j = round * PD_D - q * U, lr = sw + q * PD_STREAM_WAVES;
 #pragma unroll
     for (int d = 0; d < PD_D; d++) {
@@ -463,7 +465,7 @@ __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& 
     constexpr uint32_t BPU = Q4 ? 64 : 32;
     const uint32_t U = h.U, nblk = h.nblk;
     const uint32_t lb = Q4 ? lane : lane >> 1;
-    const uint32_t q = sdiv(round * PD_D, U);
+    const uint32_t q = pos_div_u(round * PD_D, h);
     uint32_t j = round * PD_D - q * U, lr = sw + q * PD_STREAM_WAVES;
 #pragma unroll
     for (int d = 0; d < PD_D; d++) {
@@ -1096,6 +1098,7 @@ bool plan_gemv(const QWeight& w, uint32_t inter, uint32_t nseg, const Segment* s
     g->qs = w.qs; g->ws = w.scales; g->K = w.K; g->N = w.N; g->nblk = w.K / 32;
     const uint32_t epu = w.wdtype == FORGE_HIP_Q8_0 ? 1024 : 2048;
     g->U = (w.K + epu - 1) / epu;
+    g->umagic = g->U >= 2 ? (uint32_t)(0x100000000ull / g->U) + 1u : 0u;
     g->inter = inter;
     g->nseg = nseg; g->tail_mod = tail_mod;
     for (uint32_t i = 0; i < nseg; i++) g->seg[i] = seg[i];
