@@ -4,7 +4,8 @@
 //
 // HBM-bound: every weight byte is read once, with 16-byte loads that are contiguous
 // across the wave; the int8 products run on v_dot4, no MFMA.  A wave owns RW consecutive
-// rows at a time and keeps the quantised activation vector in registers for all of them.
+// rows at a time and keeps the quantised activation vector in registers for all of them
+// (on matrices of few rows: its share of the vector, K being dealt to KS waves per row group).
 //
 // Q8_0: lane l of chunk j holds bytes [1024 j + 16 l, +16) of the row = half of block
 //       32 j + l/2; the two halves are added as integers across the lane pair.
@@ -21,7 +22,8 @@
 // A kernel boundary costs several microseconds on this GPU, more than streaming a small
 // matrix, so the decode step's neighbours are fused in:
 //   prologue  RmsNorm: rms_norm (emit.rs:327-334, the 16-lane FMA order of emit.rs:272-295) and the
-//             activation quantiser (emit.rs:1410-1440), recomputed by every workgroup from x
+//             activation quantiser (emit.rs:1410-1440), recomputed by every workgroup from x, once per
+//             workgroup: codes and scales go to LDS, every wave reads its fragment from there
 //   epilogue  Add: residual_add (emit.rs:455-459);  RopeKv: rope (emit.rs:508-528) on the q and k
 //             rows and the fp16 KV-cache write;  SiluQuant: silu_mul (emit.rs:380-386) of the gate
 //             and up rows of a fused [gate;up] matrix and the quantisation of the result.
