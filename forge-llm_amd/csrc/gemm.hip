@@ -135,7 +135,8 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     // The K position of a stage moves the descriptors (scalar work: base + k0, records - k0), not the lanes' offsets: the
     // range check still sees the whole offset (a scalar offset operand would be left out of it), and the per-lane
     // offsets stay the same from stage to stage.
-    auto issue_stage = [&](uint32_t k0, uint32_t buf) {
+    // part: which of the stage's loads to issue (1: activation tile, 2: weight tile, 4: scales; 7: all)
+    auto issue_stage = [&](uint32_t k0, uint32_t buf, int part = 7) {
         const uint32_t kq = Q4 ? k0 / 2 : k0, ks = (k0 / 32) * 2;
         // 0 records: every access is out of range.  (readfirstlane: the value is uniform, and a descriptor word in a
         // vector register would cost a loop over its values around every load.)
@@ -146,24 +147,28 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         const __amdgpu_buffer_rsrc_t rw_k = __builtin_amdgcn_make_buffer_rsrc((void*)(wq + kq), 0, left(N * wrow, kq), RSRC_FLAGS);
         const __amdgpu_buffer_rsrc_t ras_k = __builtin_amdgcn_make_buffer_rsrc((void*)((const uint8_t*)asc + ks), 0, left(M * nblk * 2, ks), RSRC_FLAGS);
         const __amdgpu_buffer_rsrc_t rws_k = __builtin_amdgcn_make_buffer_rsrc((void*)((const uint8_t*)wsc + ks), 0, left(N * nblk * 2, ks), RSRC_FLAGS);
+        if (part & 1) {
 #pragma unroll
-        for (int i = 0; i < 2 * TM; i++)
-            __builtin_amdgcn_raw_ptr_buffer_load_lds(ra_k, FH_LDS3(lds + LDS_A + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
-                                                     a_voff + i * 32 * K, 0, 0, 0);
-        if (Q4) {
+            for (int i = 0; i < 2 * TM; i++)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ra_k, FH_LDS3(lds + LDS_A + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
+                                                         a_voff + i * 32 * K, 0, 0, 0);
+        }
+        if ((part & 2) && Q4) {
 #pragma unroll
             for (int i = 0; i < 2; i++) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rw_k, q4_voff + i * 64 * nblk * 16, 0, 0);
-        } else {
+        } else if (part & 2) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rw_k, FH_LDS3(lds + LDS_B + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
                                                          w_voff + i * 32 * K, 0, 0, 0);
         }
+        if (part & 4) {
 #pragma unroll
-        for (int b = 0; b < KB; b++) {
-            const uint32_t v = sc_is_a ? __builtin_amdgcn_raw_buffer_load_b16(ras_k, sc_voff + b * 2, 0, 0)
-                                       : __builtin_amdgcn_raw_buffer_load_b16(rws_k, sc_voff + b * 2, 0, 0);
-            rs[b] = v;              // looked at only when the stage is committed: nothing at the start of a stage waits for it
+            for (int b = 0; b < KB; b++) {
+                const uint32_t v = sc_is_a ? __builtin_amdgcn_raw_buffer_load_b16(ras_k, sc_voff + b * 2, 0, 0)
+                                           : __builtin_amdgcn_raw_buffer_load_b16(rws_k, sc_voff + b * 2, 0, 0);
+                rs[b] = v;          // looked at only when the stage is committed: nothing at the start of a stage waits for it
+            }
         }
     };
 
@@ -270,8 +275,11 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     auto run_stage = [&](uint32_t s, uint32_t buf) {
         const uint32_t slot = s & 3;
         // unconditionally: past the last stage this fetches blocks that do not exist (zeros or the next row's
-        // bytes, with scale 0), which keeps the loop body one straight block of code
-        issue_stage((s + 1) * BK, buf ^ 1);
+        // bytes, with scale 0), which keeps the loop body one straight block of code.  The next stage's loads go out in
+        // three portions, the activation tile here, the weight tile and the scales behind the first and the second block:
+        // a wave that issues all twelve at once sits in their issue for a fifth to a third of the stage (time stamps),
+        // longer the fuller the memory pipeline is
+        issue_stage((s + 1) * BK, buf ^ 1, 1);
 
         Frag fr[2];
         read_frag(fr[0], buf, slot, 0);
@@ -337,6 +345,8 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                 S = S_n;
                 __builtin_amdgcn_sched_barrier(0);   // keep the tiles in this order: one tile of temporaries ahead, no more
             }
+            if (kb == 0) { issue_stage((s + 1) * BK, buf ^ 1, 2); __builtin_amdgcn_sched_barrier(0); }
+            if (kb == 1) { issue_stage((s + 1) * BK, buf ^ 1, 4); __builtin_amdgcn_sched_barrier(0); }
         }
         commit_stage(buf ^ 1, (s + 1) & 3, (s + 1) * KB);
         __builtin_amdgcn_s_waitcnt(0);   // this wave's share of stage s+1 has landed
