@@ -1259,7 +1259,11 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     // give-up path: every wait in the kernel is bounded by it, so the kernel still ends normally)
     { const char* e = getenv("FORGE_HIP_PD_SPIN_LIMIT"); if (e && atoi(e) > 0) a.spin_limit = (uint32_t)atoi(e); }
     a.q4 = st->q4; a.lm_q4 = st->lmq4;
-    { const char* e = getenv("FORGE_HIP_PD_HINT"); a.use_hint = (e && e[0] == '0') ? 0 : 1; }
+    // The watcher (one thread polls one element of a buffer, the other pollers wait for its word in LDS before they re-read
+    // what they missed) pays on narrow models, where a phase is nothing but its hand-over (hidden 576: +2 %); from a hidden
+    // size of 1024 up the pollers re-read on their own (1B +1.0 %, 3B +1.7 %, 8B +0.9 % over the watcher).
+    // FORGE_HIP_PD_HINT=0 / 1 forces either.
+    { const char* e = getenv("FORGE_HIP_PD_HINT"); a.use_hint = e ? (e[0] == '0' ? 0 : 1) : (a.H < 1024 ? 1 : 0); }
     a.token = 0; a.token_from_arg = 0; a.host_out = nullptr; a.host_seq = 0;
     // All workgroups are co-resident by construction (one per CU, checked above), and every wait in the kernel is
     // bounded, so an ordinary launch is enough; it costs ~7 us less per step than a cooperative one.
