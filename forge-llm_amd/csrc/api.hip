@@ -115,6 +115,7 @@ int32_t forge_hip_qweight_create(uint32_t wdtype, const uint8_t* raw_host, uint3
     FH_CHECK(K >= 32 && K % 32 == 0 && N >= 1, "qweight_create: K must be a positive multiple of 32 and N >= 1");
     FH_CHECK(!kq || kquant_k_supported(K), "qweight_create: a K-quant matrix needs K to be a multiple of 256, at most 16384");
     if (forge_hip_device_count() < 1) return fail(FORGE_HIP_ERR_NO_DEVICE, "no HIP device");
+    attn_decode_noalloc_prepare();
     forge_hip_qweight* h = new forge_hip_qweight();
     int32_t rc = qweight_upload(wdtype, raw_host, K, N, &h->w);
     if (rc) { delete h; return rc; }
@@ -164,7 +165,10 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
     if (!exact && M > 64) {
         const bool fresh = g_gemm.cap < gemm_split_workspace_bytes();
         if ((rc = g_gemm.reserve(gemm_split_workspace_bytes()))) return rc;
-        if (fresh) FH_HIP(hipMemset(g_gemm.p, 0, gemm_split_workspace_bytes()));   // its counters start at zero and are left at zero
+        // its counters start at zero and are left at zero; cleared on the caller's stream, so that the clear is ordered
+        // before the kernel whatever kind of stream that is (a null-stream memset does not wait for, and is not waited
+        // for by, a non-blocking stream)
+        if (fresh) FH_HIP(hipMemsetAsync(g_gemm.p, 0, gemm_split_workspace_bytes(), (hipStream_t)stream));
         split_ws = g_gemm.p;
     }
     launch_gemm(w->w, q, sc, M, y_dev, w->w.N, false, exact, nullptr, (hipStream_t)stream, split_ws);

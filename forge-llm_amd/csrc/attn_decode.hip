@@ -297,6 +297,14 @@ int32_t scratch_on_current_device(void** out) {
 }
 }  // namespace
 
+// Set-up calls (forge_hip_model_create, forge_hip_qweight_create) look the address up for their device, so that a caller
+// who has made one of them never pays the lookup (which may load the code object) inside forge_hip_attn_decode_f16kv_noalloc,
+// for instance under a stream capture.  A failure is left for the entry point itself to report.
+void fh::attn_decode_noalloc_prepare() {
+    void* p = nullptr;
+    if (scratch_on_current_device(&p) != FORGE_HIP_OK) (void)hipGetLastError();
+}
+
 extern "C" int32_t forge_hip_attn_decode_f16kv_noalloc(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                                        float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
                                                        uint32_t head_dim, void* stream) {

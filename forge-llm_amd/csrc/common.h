@@ -171,6 +171,10 @@ void launch_attn_decode_paged(const float* q, const uint16_t* k_pool, const uint
                               uint32_t page_rows, float* out, uint32_t seq_len, uint32_t heads, uint32_t kv_heads, uint32_t hd,
                               void* workspace, hipStream_t s);
 
+// Looks up, once per device, the address of the fixed scratch array of forge_hip_attn_decode_f16kv_noalloc on the current
+// device; called from the library's set-up entry points.
+void attn_decode_noalloc_prepare();
+
 // attn_prefill.hip
 // q rows / out rows have strides q_stride / out_stride floats (q may live inside a fused qkv buffer).
 // window != 0: the query at position p sees keys [max(0, p - window + 1), p] (attention_sliding_batch, emit.rs:907-1046).

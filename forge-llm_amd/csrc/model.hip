@@ -397,6 +397,7 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
         return fail(FORGE_HIP_ERR_BLOB_SIZE, "weights blob is " + std::to_string(nbytes) + " bytes, config needs " +
                                                  std::to_string(forge_hip_weights_nbytes(cfg)));
     if (forge_hip_device_count() < 1) return fail(FORGE_HIP_ERR_NO_DEVICE, "no HIP device");
+    attn_decode_noalloc_prepare();
 
     std::unique_ptr<forge_hip_model> m(new forge_hip_model());
     m->cfg = *cfg;

@@ -271,8 +271,10 @@ def attention_flash_noalloc(q, k_cache, v_cache, seq_len, heads, kv_heads, head_
     for t, dt in ((q, torch.float32), (out, torch.float32), (k_cache, torch.int16), (v_cache, torch.int16)):
         if not (t.is_cuda and t.dtype == dt and t.is_contiguous()):
             raise ValueError("attention_flash_noalloc takes contiguous device tensors (q, out f32; caches int16 bit patterns)")
-    if seq_len > k_cache.shape[0] or out.numel() != q.numel():
-        raise ValueError("cache holds fewer than seq_len rows, or out has another size than q")
+    if seq_len > k_cache.shape[0] or out.numel() != q.numel() or q.numel() != heads * head_dim:
+        raise ValueError("cache holds fewer than seq_len rows, or q / out do not hold heads * head_dim values")
+    if k_cache.numel() < seq_len * kv_heads * head_dim or v_cache.numel() < seq_len * kv_heads * head_dim:
+        raise ValueError("a cache holds fewer than seq_len rows of kv_heads * head_dim values")
     check(lib().forge_hip_attn_decode_f16kv_noalloc(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), seq_len, heads, kv_heads,
                                                     head_dim, _stream()))
     return out

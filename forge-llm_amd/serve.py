@@ -22,6 +22,7 @@ from http.server import BaseHTTPRequestHandler, HTTPServer
 
 EOS_TOKEN = 2            # lib.rs:8757
 DEFAULT_MAX_TOKENS = 256  # lib.rs:8729
+MAX_BODY_BYTES = 16 << 20  # a larger request body is refused with 413 before it is read (the reference reads any length)
 MODEL_ID = "forgellm-hip"
 
 
@@ -112,23 +113,38 @@ class ChatServer:
         except Exception as e:
             return 500, {}, json.dumps({"error": "Tokenization failed: %s" % e}).encode()
         model = self.model
-        model.reset()
-        if hasattr(model, "set_repeat_penalty"):
-            model.set_repeat_penalty(1.0)                # the serve loop is a plain argmax
-        t0 = time.perf_counter()
-        next_token = self._prefill(tokens)
-        prefill_s = time.perf_counter() - t0
-        t0 = time.perf_counter()
-        pieces, generated = [], 0
-        for _ in range(req["max_tokens"]):
-            if next_token == EOS_TOKEN:
-                break
-            text = self._decode_one(next_token)
-            if text is not None:
-                pieces.append(text)
-            generated += 1
-            next_token = model.forward_greedy(next_token)
-        gen_s = time.perf_counter() - t0
+        # The cache holds max_seq positions and every token fed takes one: a prompt that fills it is refused up front, and
+        # the decode loop stops at the last free position with finish_reason "length".  (The reference has neither check:
+        # its generated binary panics on the slice index; here the model call would raise in the middle of the request.)
+        max_seq = int(getattr(model, "config", {}).get("max_seq", 0) or 0)
+        if max_seq and len(tokens) >= max_seq:
+            return 400, {}, json.dumps({"error": "Prompt too long: %d tokens, the model's context holds %d"
+                                                 % (len(tokens), max_seq)}).encode()
+        room = max_seq - len(tokens) if max_seq else req["max_tokens"]      # decode steps the cache still has rows for
+        finish = "stop"
+        try:
+            model.reset()
+            if hasattr(model, "set_repeat_penalty"):
+                model.set_repeat_penalty(1.0)                # the serve loop is a plain argmax
+            t0 = time.perf_counter()
+            next_token = self._prefill(tokens)
+            prefill_s = time.perf_counter() - t0
+            t0 = time.perf_counter()
+            pieces, generated = [], 0
+            for _ in range(req["max_tokens"]):
+                if next_token == EOS_TOKEN:
+                    break
+                text = self._decode_one(next_token)
+                if text is not None:
+                    pieces.append(text)
+                generated += 1
+                if generated > room:                         # feeding this token would need a row past the cache's end
+                    finish = "length"
+                    break
+                next_token = model.forward_greedy(next_token)
+            gen_s = time.perf_counter() - t0
+        except Exception as e:                               # a failed model call is an answer, not a dropped connection
+            return 500, {}, json.dumps({"error": "Generation failed: %s" % e}).encode()
         tok_s = generated / gen_s if gen_s > 0.0 else 0.0
         if req["stream"]:
             out = []
@@ -139,10 +155,10 @@ class ChatServer:
             usage = ('{"prefill_tokens":%d,"prefill_time_ms":%.1f,"generation_tokens":%d,"generation_time_ms":%.1f,'
                      '"tokens_per_sec":%.1f}' % (len(tokens), prefill_s * 1e3, generated, gen_s * 1e3, tok_s))
             out.append('data: {"id":"chatcmpl-1","object":"chat.completion.chunk","choices":[{"index":0,"delta":{},'
-                       '"finish_reason":"stop"}],"usage":%s}\n\ndata: [DONE]\n\n' % usage)
+                       '"finish_reason":"%s"}],"usage":%s}\n\ndata: [DONE]\n\n' % (finish, usage))
             return 200, {"Content-Type": "text/event-stream", "Cache-Control": "no-cache"}, "".join(out).encode("utf-8")
         resp = {"id": "chatcmpl-1", "object": "chat.completion",
-                "choices": [{"index": 0, "message": {"role": "assistant", "content": "".join(pieces)}, "finish_reason": "stop"}],
+                "choices": [{"index": 0, "message": {"role": "assistant", "content": "".join(pieces)}, "finish_reason": finish}],
                 "usage": {"prefill_tokens": len(tokens), "prefill_time_ms": int(prefill_s * 1e3),
                           "generation_tokens": generated, "generation_time_ms": int(gen_s * 1e3), "tokens_per_sec": tok_s}}
         return 200, {"Content-Type": "application/json"}, json.dumps(resp, ensure_ascii=False).encode("utf-8")
@@ -166,9 +182,16 @@ def make_http_server(model, tokenizer, port: int, host: str = "0.0.0.0") -> HTTP
         protocol_version = "HTTP/1.1"
 
         def _respond(self, method):
-            n = int(self.headers.get("Content-Length") or 0)
-            body = self.rfile.read(n) if n > 0 else b""
-            status, headers, payload = chat.handle(method, self.path, body)
+            try:
+                n = int(self.headers.get("Content-Length") or 0)
+            except ValueError:
+                n = -1
+            if n < 0 or n > MAX_BODY_BYTES:
+                status, headers, payload = 413, {}, json.dumps({"error": "Request body too large"}).encode()
+                self.close_connection = True                 # the unread body must not be taken for the next request
+            else:
+                body = self.rfile.read(n) if n > 0 else b""
+                status, headers, payload = chat.handle(method, self.path, body)
             self.send_response(status)
             for k, v in headers.items():
                 self.send_header(k, v)

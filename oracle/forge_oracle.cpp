@@ -993,6 +993,17 @@ void fo_model_read_kv(fo_model* m, int layer, int which, float* out) {
         }
 }
 
+// The inverse of fo_model_read_kv: rows [0, n) of one layer's K and V cache are stored from f32 rows through the model's own
+// cache write (int8 + per-token scale, or fp16), and the cache length is set to n.  Lets a model take over the context
+// another one has computed (a timing aid: a decode step at a long context without this model's own prefill of it).
+int fo_model_write_kv(fo_model* m, int layer, int64_t n, const float* k, const float* v) {
+    int64_t KV = (int64_t)m->cfg.kv_heads * m->cfg.head_dim;
+    if (layer < 0 || layer >= (int)m->cfg.layers || n < 0 || n > (int64_t)m->cfg.max_seq) return -3;
+    for (int64_t t = 0; t < n; t++) store_kv(m, layer, t, k + t * KV, v + t * KV);
+    m->len = n;
+    return 0;
+}
+
 // ---- op-level entry points ----
 float fo_f16_to_f32(uint16_t b) { return f16_to_f32(b); }
 uint16_t fo_f32_to_f16(float x) { return f32_to_f16(x); }

@@ -54,6 +54,8 @@ def lib():
     L.fo_prefill_batched.restype = i32
     L.fo_prefill_batched.argtypes = [vp, vp, i64, vp]
     L.fo_model_read_kv.argtypes = [vp, i32, i32, vp]
+    L.fo_model_write_kv.restype = i32
+    L.fo_model_write_kv.argtypes = [vp, i32, i64, vp, vp]
     L.fo_f16_to_f32.restype = f32
     L.fo_f16_to_f32.argtypes = [C.c_uint16]
     L.fo_f32_to_f16.restype = C.c_uint16
@@ -311,6 +313,15 @@ class Model:
         out = np.empty((n, kv), np.float32)
         lib().fo_model_read_kv(self._h, layer, which, _p(out))
         return out
+
+    def adopt_context(self, other):
+        """Take over the cached context of another oracle model of the same shape (its K/V rows pass through this
+        model's own cache write); the position becomes the other model's."""
+        for l in range(self.cfg.layers):
+            k, v = other.read_kv(l, 0), other.read_kv(l, 1)
+            rc = lib().fo_model_write_kv(self._h, l, k.shape[0], _p(k), _p(v))
+            if rc != 0:
+                raise RuntimeError(f"oracle write_kv failed: {rc}")
 
     @property
     def pos(self):

@@ -53,6 +53,23 @@ def test_quantize_act_bit_exact(fh, oracle, torch_gpu, M, K):
     assert np.array_equal(sc.cpu().numpy().view(np.uint16), bits)
 
 
+def test_quantize_act_rounding_ties(fh, torch_gpu):
+    """Elements exactly half way between two codes go AWAY from zero (f32::round, emit.rs:1433).  Block 0 has its largest
+    magnitude at 127 (scale and reciprocal exactly 1), block 1 at 254 (scale 2, reciprocal 0.5); expected codes by hand."""
+    torch = torch_gpu
+    ties = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 126.5, -126.5, 127.0, 0.25, -0.75, 3.0]
+    want = [1, -1, 2, -2, 3, -3, 127, -127, 127, 0, -1, 3]
+    x = np.zeros((2, 64), np.float32)
+    x[0, :12] = ties
+    x[0, 32:44] = [2.0 * t for t in ties]
+    x[1, 32:44] = ties                                      # and in another row, second block
+    q, sc = fh.ops.quantize_act(torch.from_numpy(x).cuda())
+    q, sc = q.cpu().numpy(), sc.cpu().numpy().view(np.uint16)
+    assert q[0, :12].tolist() == want and q[0, 32:44].tolist() == want and q[1, 32:44].tolist() == want
+    assert sc[0].tolist() == [0x3C00, 0x4000] and sc[1].tolist() == [0x3C00, 0x3C00]    # row 1, block 0: all zero -> scale 1.0
+    assert not q[0, 12:32].any() and not q[1, :32].any()
+
+
 @pytest.mark.parametrize("wd", [Q8, Q4])
 @pytest.mark.parametrize("N,K", [(8, 32), (13, 576), (260, 2048), (64, 8192), (70, 3072)])
 @pytest.mark.parametrize("path", [0, 1, 2])

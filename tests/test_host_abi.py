@@ -48,6 +48,21 @@ def test_host_quantisers_bit_identical_to_oracle(fh, oracle, wd):
     assert fh.ops.quantize_weights(wd, np.zeros(0, np.float32)).size == 0
 
 
+def test_host_quantisers_rounding_ties(fh):
+    """Elements exactly half way between two codes (scale 1.0 exactly: largest magnitude 127 resp. 8) go AWAY from zero,
+    as f32::round does (weight_loader.rs:1482, 1534-1535); expected codes written by hand."""
+    v = np.zeros(32, np.float32)
+    v[:12] = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 126.5, -126.5, 127.0, 0.25, -0.75, 3.0]
+    raw = fh.ops.quantize_weights(Q8, v)
+    assert (int(raw[0]) | (int(raw[1]) << 8)) == 0x3C00
+    assert raw[2:14].view(np.int8).tolist() == [1, -1, 2, -2, 3, -3, 127, -127, 127, 0, -1, 3]
+    v[:12] = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 6.5, -7.5, 8.0, -8.0, 7.5, 0.25]
+    raw = fh.ops.quantize_weights(Q4, v)
+    assert (int(raw[0]) | (int(raw[1]) << 8)) == 0x3C00
+    codes = np.concatenate([raw[2:] & 0x0F, raw[2:] >> 4])
+    assert codes[:12].tolist() == [9, 7, 10, 6, 11, 5, 15, 0, 15, 0, 15, 8]
+
+
 def test_expf_twin_matches_c_library(fh, oracle):
     """The kernels' exp (host twin) against the C library's expf, which the CPU path calls: dense
     sweep of the softmax/silu range plus the overflow/underflow edges.  (Over all 2.2e9 finite inputs

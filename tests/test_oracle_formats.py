@@ -169,6 +169,47 @@ def test_activation_quantiser_invariants(oracle):
         assert np.array_equal(codes[b].astype(np.float64), want)
 
 
+# ---- rounding ties: f32::round is half AWAY from zero (weight_loader.rs:1482, 1534-1535; emit.rs:1433)
+# A block whose largest magnitude is 127.0 (Q8_0, activations) or 8.0 (Q4_0) has scale 1.0 and reciprocal 1.0 exactly, so
+# x * inv is x itself and the elements below sit exactly half way between two codes.  The expected codes are written out
+# by hand; round-half-to-even (rintf, numpy.round) would give 0, 0, 2, 2, 2, 2, 126, -126 for the first eight.
+TIE_INPUT = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 126.5, -126.5, 127.0, 0.25, -0.75, 3.0]
+TIE_Q8_CODES = [1, -1, 2, -2, 3, -3, 127, -127, 127, 0, -1, 3]
+TIE4_INPUT = [0.5, -0.5, 1.5, -1.5, 2.5, -2.5, 6.5, -7.5, 8.0, -8.0, 7.5, 0.25]
+TIE4_CODES = [9, 7, 10, 6, 11, 5, 15, 0, 15, 0, 15, 8]          # round(x) + 8, clamped to [0, 15]
+
+
+def tie_block(values):
+    v = np.zeros(32, np.float32)
+    v[:len(values)] = values
+    return v
+
+
+def test_weight_quantiser_q8_0_rounding_ties(oracle):
+    raw = oracle.quantize_weights(Q8, tie_block(TIE_INPUT))
+    assert (int(raw[0]) | (int(raw[1]) << 8)) == 0x3C00                      # scale 127 / 127 = 1.0
+    assert raw[2:2 + len(TIE_Q8_CODES)].view(np.int8).tolist() == TIE_Q8_CODES
+    assert np.all(raw[2 + len(TIE_Q8_CODES):] == 0)
+
+
+def test_weight_quantiser_q4_0_rounding_ties(oracle):
+    raw = oracle.quantize_weights(Q4, tie_block(TIE4_INPUT))
+    assert (int(raw[0]) | (int(raw[1]) << 8)) == 0x3C00                      # scale 8 / 8 = 1.0
+    codes = np.concatenate([raw[2:] & 0x0F, raw[2:] >> 4])                   # elements 0..15, then 16..31
+    assert codes[:len(TIE4_CODES)].tolist() == TIE4_CODES
+    assert np.all(codes[len(TIE4_CODES):] == 8)                              # zeros sit at the offset
+
+
+def test_activation_quantiser_rounding_ties(oracle):
+    raw = oracle.quantize_act(tie_block(TIE_INPUT))
+    assert (int(raw[0]) | (int(raw[1]) << 8)) == 0x3C00
+    assert raw[2:2 + len(TIE_Q8_CODES)].view(np.int8).tolist() == TIE_Q8_CODES
+    # the same ties at another power-of-two scale: absmax 254 -> s = 2, inv = 0.5, x * inv = 0.5 (k + 0.5)
+    raw = oracle.quantize_act(tie_block([2.0 * t for t in TIE_INPUT]))
+    assert (int(raw[0]) | (int(raw[1]) << 8)) == 0x4000
+    assert raw[2:2 + len(TIE_Q8_CODES)].view(np.int8).tolist() == TIE_Q8_CODES
+
+
 # ---- KV int8 quantiser: the reference's fixture (emit.rs:6813-6852)
 def test_kv_quantiser_reference_fixture(oracle):
     v = (((np.arange(64) * 7 + 3).astype(np.float32) * np.float32(0.1) - np.float32(3.0)) * np.float32(0.5)).astype(np.float32)

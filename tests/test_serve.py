@@ -155,6 +155,59 @@ def test_tokenizer_failure_is_500(fh):
     assert status == 500 and json.loads(body)["error"] == "Tokenization failed: no vocabulary"
 
 
+class LimitedModel(ScriptedModel):
+    """A scripted model with a cache of `max_seq` rows that raises, like HipModel, when a token is fed past its end."""
+
+    def __init__(self, script, max_seq):
+        super().__init__(script)
+        self.config = {"max_seq": max_seq}
+        self.pos = 0
+
+    def reset(self):
+        super().reset()
+        self.pos = 0
+
+    def forward_prefill_batch(self, tokens):
+        if self.pos + len(tokens) > self.config["max_seq"]:
+            raise RuntimeError("prompt does not fit the KV cache")
+        super().forward_prefill_batch(tokens)
+        self.pos += len(tokens)
+
+    def forward_greedy(self, token):
+        if self.pos >= self.config["max_seq"]:
+            raise RuntimeError("KV cache is full (pos == max_seq)")
+        self.pos += 1
+        return super().forward_greedy(token)
+
+
+def test_context_limit_is_an_answer_not_an_exception(fh):
+    """The cache's end: a prompt that fills it is a 400, a generation that reaches it ends with finish_reason "length"
+    after exactly the tokens that fit, and a model call that fails all the same comes back as a 500 body."""
+    n = len(PROMPT)
+    s = fh.serve.ChatServer(LimitedModel([tok("a")] * 64, n), CharTokenizer())
+    status, _, body = post(s, {"messages": MSGS})
+    assert status == 400 and "Prompt too long" in json.loads(body)["error"]
+    # room for 3 more rows: the prompt's n tokens, then the tokens "a", "a", "a" can still be fed; the 4th pick is the last
+    m = LimitedModel([tok("a")] * 64, n + 3)
+    s = fh.serve.ChatServer(m, CharTokenizer())
+    status, _, body = post(s, {"messages": MSGS, "max_tokens": 50})
+    resp = json.loads(body)
+    assert status == 200 and resp["choices"][0]["finish_reason"] == "length"
+    assert resp["choices"][0]["message"]["content"] == "aaaa" and resp["usage"]["generation_tokens"] == 4
+    assert m.pos == n + 3
+    status, _, body = post(s, {"messages": MSGS, "max_tokens": 50, "stream": True})
+    assert status == 200 and b'"finish_reason":"length"' in body
+    # max_tokens below the room: an ordinary stop
+    status, _, body = post(s, {"messages": MSGS, "max_tokens": 2})
+    assert json.loads(body)["choices"][0]["finish_reason"] == "stop"
+
+    class Broken(ScriptedModel):
+        def forward_greedy(self, token):
+            raise RuntimeError("device lost")
+    status, _, body = post(fh.serve.ChatServer(Broken([]), CharTokenizer()), {"messages": MSGS})
+    assert status == 500 and "device lost" in json.loads(body)["error"]
+
+
 def test_other_routes(fh):
     s = fh.serve.ChatServer(ScriptedModel([2]), CharTokenizer())
     status, headers, body = s.handle("GET", "/v1/models")
