@@ -53,6 +53,12 @@ constexpr int SC_ROW = KB * 2, SC_SLOT = BM * SC_ROW;
 constexpr int LDS_A = 0, LDS_B = 2 * TILE_BYTES, LDS_ASC = 4 * TILE_BYTES, LDS_BSC = LDS_ASC + 4 * SC_SLOT,
               LDS_ZERO = LDS_BSC + 4 * SC_SLOT, GEMM_LDS_BYTES = LDS_ZERO + 512;
 constexpr uint32_t MAGIC_BITS = 0x4B400000u;  // 12582912.0f = 1.5 * 2^23: ulp 1, room for +-2^22
+// The fast mode's bias removal multiplies the activation scales by 2^SCALE_A_LOG2 and the weight scales by
+// 2^(23 - SCALE_A_LOG2) (and half of that) on their way into an f16 MFMA.  The factors themselves (256, 32768) and the
+// products are exact fp16 numbers while a_s < 2^(16 - SCALE_A_LOG2) = 256 (a block's largest activation below 32 512) and
+// w_s < 2 (Q8_0 weights below 254, Q4_0 weights below 16 in magnitude).
+constexpr int SCALE_A_LOG2 = 8;
+static_assert(23 - SCALE_A_LOG2 <= 15, "2^16 is not an fp16 number");
 constexpr uint32_t RSRC_FLAGS = 0x00020000;   // raw buffer, 32-bit data format
 constexpr uint32_t OOB = 0x80000000u;         // an offset no descriptor here covers
 constexpr uint32_t GEMM_SPLIT_MAX_ITEMS = 256; // K ranges one launch may park in the split workspace (64 KB each)
@@ -353,36 +359,45 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         __syncthreads();
     };
 
-    // Stages go in pairs (an odd count runs one stage of zero scales).  After a pair the fast mode removes what
-    // the 8 blocks left of the bias: 12582912 * sum_b a_s[m][b] * (+-w_s[n][b]), the sum being one f16 MFMA.
-    const uint32_t ta_off = lhalf ? (uint32_t)LDS_ZERO : LDS_ASC + (wm * WM + lrow) * SC_ROW;
-    const uint32_t tb_off = lhalf ? (uint32_t)LDS_ZERO : LDS_BSC + (wn * 64 + lrow) * SC_ROW;
+    // Stages go in pairs (an odd count runs one stage of zero scales).  After a pair the fast mode removes what the 8
+    // blocks left of the bias, 1.5 * 2^23 * sum_b a_s[m][b] * (+-w_s[n][b]).  That is sum_b (2^8 a_s[b]) * (2^15 w[b] +
+    // 2^14 w[b]), sixteen products of fp16 numbers, so one f16 MFMA subtracts it from the accumulators directly: the
+    // activation side holds 2^8 a_s[b] in both halves of the wave, the weight side -2^15 w[b] in the lanes of the lower
+    // half (k = 0..7) and -2^14 w[b] in the upper half (k = 8..15).  (Before: the sum from the MFMA and one FMA per
+    // element to apply it, 64 VALU instructions per wave and stage pair instead of 16 packed multiplies.)
+    const uint32_t ta_off = LDS_ASC + (wm * WM + lrow) * SC_ROW;
+    const uint32_t tb_off = LDS_BSC + (wn * 64 + lrow) * SC_ROW;
     for (uint32_t s = s_begin; s < s_end; s += 2) {
         run_stage(s, 0);
         run_stage(s + 1, 1);
         if (MAGIC) {
-            const uint32_t pair = lhalf ? 0u : (s & 2u) * (uint32_t)SC_SLOT;      // slots {0,1} or {2,3}
+            const uint32_t pair = (s & 2u) * (uint32_t)SC_SLOT;      // slots {0,1} or {2,3}
             typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+            const _Float16 bf = lhalf ? (_Float16)(-(float)(1 << (22 - SCALE_A_LOG2))) : (_Float16)(-(float)(1 << (23 - SCALE_A_LOG2)));
+            const _Float16 af = (_Float16)(float)(1 << SCALE_A_LOG2);
+            const v8h bfv = (v8h){bf, bf, bf, bf, bf, bf, bf, bf}, afv = (v8h){af, af, af, af, af, af, af, af};
             v8h ta[TM], tb[2];
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-                const v4h b0 = *reinterpret_cast<const v4h*>(lds + tb_off + pair + t * s_t_stride);
-                const v4h b1 = *reinterpret_cast<const v4h*>(lds + tb_off + pair + s_slot_stride + t * s_t_stride);
-                tb[t] = (v8h){b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]};
+                const v4h b0 = *reinterpret_cast<const v4h*>(lds + tb_off + pair + t * (32 * SC_ROW));
+                const v4h b1 = *reinterpret_cast<const v4h*>(lds + tb_off + pair + SC_SLOT + t * (32 * SC_ROW));
+                tb[t] = (v8h){b0[0], b0[1], b0[2], b0[3], b1[0], b1[1], b1[2], b1[3]} * bfv;
             }
 #pragma unroll
             for (int t = 0; t < TM; t++) {
-                const v4h a0 = *reinterpret_cast<const v4h*>(lds + ta_off + pair + t * s_t_stride);
-                const v4h a1 = *reinterpret_cast<const v4h*>(lds + ta_off + pair + s_slot_stride + t * s_t_stride);
-                ta[t] = (v8h){a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                const v4h a0 = *reinterpret_cast<const v4h*>(lds + ta_off + pair + t * (32 * SC_ROW));
+                const v4h a1 = *reinterpret_cast<const v4h*>(lds + ta_off + pair + SC_SLOT + t * (32 * SC_ROW));
+                ta[t] = (v8h){a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]} * afv;
             }
 #pragma unroll
             for (int t = 0; t < 2 * TM; t++) {
                 const int tm = t >> 1, tn = t & 1;
-                const v16f T = __builtin_amdgcn_mfma_f32_32x32x16_f16(ta[tm], tb[tn], zero_f, 0, 0, 0);
+                v16f c;
 #pragma unroll
-                for (int r = 0; r < 16; r++)
-                    acc[tm][tn][r] = fmaf(-__builtin_bit_cast(float, MAGIC_BITS), T[r], acc[tm][tn][r]);
+                for (int r = 0; r < 16; r++) c[r] = acc[tm][tn][r];
+                c = __builtin_amdgcn_mfma_f32_32x32x16_f16(ta[tm], tb[tn], c, 0, 0, 0);
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[tm][tn][r] = c[r];
             }
         }
     }
