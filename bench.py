@@ -401,6 +401,21 @@ def main():
     model.set_repeat_penalty(1.1)
     tok3 = fh.ops.argmax_host(model.forward_prefill(prompt))
     t_decode_pen, _ = timed_decode(model, tok3, args.warmup, args.steps)
+
+    # ---- the same prompt and decode steps over a PAGED cache: pages of 64 rows in a shuffled order
+    model.reset()
+    model.set_repeat_penalty(1.0)
+    n_pages = cfg["max_seq"] // 64
+    model.set_kv_pages(64, np.random.default_rng(args.seed).permutation(n_pages).astype(np.uint32))
+    model.forward_prefill_batch(prompt)
+    model.reset()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    logits_paged = model.forward_prefill(prompt)
+    torch.cuda.synchronize()
+    t_prefill_paged = time.perf_counter() - t0
+    paged_same = bool(np.array_equal(logits_paged.view(np.uint32), logits.view(np.uint32)))
+    t_decode_paged, _ = timed_decode(model, fh.ops.argmax_host(logits_paged), args.warmup, args.steps)
     model.close()
 
     # ---- the other decode path, for comparison: the step as a sequence of kernels
@@ -449,6 +464,8 @@ def main():
         "prefill_ms": t_prefill * 1e3,
         "decode_tok_per_s_short_context": args.steps / t_decode_short,
         "decode_tok_per_s_repeat_penalty_1.1": args.steps / t_decode_pen,
+        "paged_kv_cache": {"page_rows": 64, "page_order": "shuffled", "decode_tok_per_s": args.steps / t_decode_paged,
+                           "prefill_tok_per_s": PROMPT_TOKENS / t_prefill_paged, "prefill_logits_bit_identical_to_flat_cache": paged_same},
         "decode_weight_stream_GBps_end_to_end": fh.synth.decode_weight_bytes(cfg) * args.steps / t_decode / 1e9,
         "exact_mode": exact,
         "roofline": roofline,

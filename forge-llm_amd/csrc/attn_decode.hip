@@ -31,10 +31,6 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float* a, float 
 // pool page page_table[t / page].  A split's table entries are copied into LDS first (they are few), so the address of
 // a key costs one LDS read more than in the flat cache; nothing else changes, the bits included.
 constexpr uint32_t PAGE_ENTRIES_MAX = 2048;   // table entries one split may span (else: contiguous-only)
-struct PageTable {
-    const uint32_t* table;   // nullptr unless PAGED
-    uint32_t shift;          // log2(rows per page)
-};
 
 // workspace record per (kv group, split, head-in-group): [HD acc][m][l]
 template <int HD, int GT, bool PAGED = false>
@@ -254,9 +250,8 @@ void launch_attn_decode_paged(const float* q, const uint16_t* k_pool, const uint
 
 void launch_attn_decode(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
                         uint32_t seq_len, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd,
-                        uint32_t window, void* workspace, hipStream_t s) {
+                        uint32_t window, void* workspace, hipStream_t s, PageTable pt) {
     float* ws = reinterpret_cast<float*>(workspace);
-    const PageTable pt{nullptr, 0};
     if (hd == 64) launch_hd<64>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, pt, s);
     else if (hd == 96) launch_hd<96>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, pt, s);
     else launch_hd<128>(q, kc, vc, out, oq, osc, seq_len, pos_dev, heads, kv_heads, window, ws, pt, s);

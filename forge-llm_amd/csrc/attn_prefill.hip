@@ -42,9 +42,10 @@ constexpr int AP_THREADS = 512;   // the 8-wave form; the 4-wave form runs 256
 // per 64 keys, no merge.
 template <int HD, bool QUANT, bool WIN, int KH>
 __global__ __launch_bounds__(AP_THREADS / KH) __attribute__((amdgpu_waves_per_eu(2)))
-void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
+void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict__ kc_flat, const uint16_t* __restrict__ vc_flat,
                          float* __restrict__ out, uint32_t q_stride, uint32_t out_stride, uint32_t M, uint32_t base_pos,
-                         uint32_t heads, uint32_t kv_heads, int8_t* __restrict__ oq, uint16_t* __restrict__ osc, uint32_t window) {
+                         uint32_t heads, uint32_t kv_heads, int8_t* __restrict__ oq, uint16_t* __restrict__ osc, uint32_t window,
+                         PageTable pt) {
     constexpr int KS = HD + 8;    // K tile row stride (halfs): 16-byte pad
     constexpr int VS = KT + 4;    // V^T tile row stride (halfs): 8-byte pad
     constexpr int KTOTAL = KT * HD / 8;          // 16-byte pieces of K per tile
@@ -112,6 +113,10 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
     int4 kreg[KPIECES];
     uint2 va[VITEMS], vb[VITEMS];
     auto load_tile = [&](uint32_t kt) {
+        // a paged cache: a tile of 64 keys lies within one page (pages are multiples of 64 rows), `shift` rows further on
+        const ptrdiff_t shift = pt.table ? (ptrdiff_t)paged_row(pt, kt * KT) - (ptrdiff_t)(kt * KT) : 0;
+        const uint16_t* kc = kc_flat + shift * (ptrdiff_t)kv_stride;
+        const uint16_t* vc = vc_flat + shift * (ptrdiff_t)kv_stride;
 #pragma unroll
         for (int i = 0; i < KPIECES; i++) {
             const uint32_t idx = tid + NT * i, key = idx / (HD / 8), dc = idx % (HD / 8);
@@ -314,7 +319,7 @@ namespace {
 template <int HD, bool QUANT>
 void launch_win(dim3 grid, hipStream_t s, const float* q, const uint16_t* kc, const uint16_t* vc, float* out, uint32_t q_stride,
                 uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, int8_t* oq, uint16_t* osc,
-                uint32_t window) {
+                uint32_t window, PageTable pt) {
     // The 4-wave form when there are clearly more workgroups than the machine holds at once (three per CU at head_dim 64,
     // two above: then throughput decides, and a wave with two score tiles per step does 15-30 % more of it); the 8-wave form
     // when they all fit (then the longest workgroup's chain of tile steps decides, and twice the waves halve its steps).
@@ -331,7 +336,7 @@ void launch_win(dim3 grid, hipStream_t s, const float* q, const uint16_t* kc, co
     // a window that covers every key of the call is plain causal attention
     const bool win = window != 0 && window < base_pos + M;
 #define FH_AP(WIN_, KH_) \
-    fh::launch(attn_prefill_kernel<HD, QUANT, WIN_, KH_>, grid, AP_THREADS / KH_, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, WIN_ ? window : 0u)
+    fh::launch(attn_prefill_kernel<HD, QUANT, WIN_, KH_>, grid, AP_THREADS / KH_, 0, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, WIN_ ? window : 0u, pt)
     if (win) { if (four) FH_AP(true, 2); else FH_AP(true, 1); }
     else { if (four) FH_AP(false, 2); else FH_AP(false, 1); }
 #undef FH_AP
@@ -339,27 +344,27 @@ void launch_win(dim3 grid, hipStream_t s, const float* q, const uint16_t* kc, co
 template <bool QUANT>
 void launch_hd(uint32_t hd, dim3 grid, hipStream_t s, const float* q, const uint16_t* kc, const uint16_t* vc, float* out,
                uint32_t q_stride, uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, int8_t* oq,
-               uint16_t* osc, uint32_t window) {
-    if (hd == 64) launch_win<64, QUANT>(grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window);
-    else if (hd == 96) launch_win<96, QUANT>(grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window);
-    else launch_win<128, QUANT>(grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window);
+               uint16_t* osc, uint32_t window, PageTable pt) {
+    if (hd == 64) launch_win<64, QUANT>(grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window, pt);
+    else if (hd == 96) launch_win<96, QUANT>(grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window, pt);
+    else launch_win<128, QUANT>(grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, oq, osc, window, pt);
 }
 }  // namespace
 
 void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, float* out,
                          uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
-                         uint32_t hd, uint32_t window, hipStream_t s) {
+                         uint32_t hd, uint32_t window, hipStream_t s, PageTable pt) {
     if (M == 0) return;
     dim3 grid(((M + QB - 1) / QB) * heads);
-    launch_hd<false>(hd, grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, nullptr, nullptr, window);
+    launch_hd<false>(hd, grid, s, q, kc, vc, out, q_stride, out_stride, M, base_pos, heads, kv_heads, nullptr, nullptr, window, pt);
 }
 
 void launch_attn_prefill_quant(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, int8_t* oq, uint16_t* osc,
                                uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, uint32_t hd, uint32_t window,
-                               hipStream_t s, bool neg_odd) {
+                               hipStream_t s, bool neg_odd, PageTable pt) {
     if (M == 0) return;
     dim3 grid(((M + QB - 1) / QB) * heads);
-    launch_hd<true>(hd, grid, s, q, kc, vc, nullptr, q_stride, neg_odd ? 1u : 0u, M, base_pos, heads, kv_heads, oq, osc, window);
+    launch_hd<true>(hd, grid, s, q, kc, vc, nullptr, q_stride, neg_odd ? 1u : 0u, M, base_pos, heads, kv_heads, oq, osc, window, pt);
 }
 
 }  // namespace fh

@@ -86,6 +86,18 @@ const char* last_error_cstr();
 int32_t qweight_upload(uint32_t wdtype, const uint8_t* raw_host, uint32_t K, uint32_t N, QWeight* out);
 void qweight_free(QWeight* w);
 
+// ---- paged KV cache --------------------------------------------------------------------------
+// A cache may be a pool of pages of 2^shift rows: row t of the sequence is then row t % page of pool page
+// table[t / page] (table: uint32 in device memory).  table == nullptr: the flat cache, row t is row t.
+struct PageTable {
+    const uint32_t* table = nullptr;
+    uint32_t shift = 0;          // log2(rows per page)
+};
+__device__ __forceinline__ size_t paged_row(const PageTable& pt, uint32_t t) {
+    if (!pt.table) return t;
+    return ((size_t)pt.table[t >> pt.shift] << pt.shift) + (t & ((1u << pt.shift) - 1u));
+}
+
 // ---- kernel launchers ------------------------------------------------------------------------
 // All are asynchronous on `s` and validate nothing: callers check shapes first.
 
@@ -103,7 +115,8 @@ void launch_silu_mul(const float* gate, const float* up, uint32_t M, uint32_t I,
 // (pos_dev ? *pos_dev : base_pos) + r.  q/k/v rows have strides q_stride/kv_stride floats.
 void launch_rope_kv_store(float* q, float* k, const float* v, uint32_t q_stride, uint32_t kv_stride, uint16_t* kc,
                           uint16_t* vc, uint32_t M, uint32_t base_pos, const uint32_t* pos_dev, uint32_t heads,
-                          uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, const float* bias, hipStream_t s);
+                          uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, const float* bias, hipStream_t s,
+                          PageTable pt = PageTable{});
 void launch_embedding(const float* table, const uint32_t* tokens_dev, uint32_t M, uint32_t H, float* out, uint32_t* counts,
                       hipStream_t s);
 // Index of the LAST maximum.  `scratch` needs 2*ARGMAX_BLOCKS uint32/float pairs.
@@ -128,7 +141,8 @@ void launch_gemv_norm(const QWeight& w, const float* x, const float* norm_w, flo
 // fused [q;k;v] matrix: q rows -> q_out (rotated), k rows -> K cache (rotated, fp16), v rows -> V cache, at *pos_dev
 void launch_gemv_norm_rope_kv(const QWeight& wqkv, const float* x, const float* norm_w, float eps, const float* bias, float* q_out,
                               uint16_t* kc, uint16_t* vc, const float* cos_t, const float* sin_t,
-                              const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s);
+                              const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s,
+                              PageTable pt = PageTable{});
 // fused [gate;up] matrix: quant(silu(gate)*up) -> (oq, osc)
 void launch_gemv_norm_silu_quant(const QWeight& wgu, const float* x, const float* norm_w, float eps, int8_t* oq,
                                  uint16_t* osc, hipStream_t s);
@@ -163,7 +177,7 @@ size_t attn_decode_workspace_bytes(uint32_t heads, uint32_t hd);
 // window != 0: only the last `window` rows are keys (attention_sliding, emit.rs:598-627).
 void launch_attn_decode(const float* q, const uint16_t* kc, const uint16_t* vc, float* out, int8_t* oq, uint16_t* osc,
                         uint32_t seq_len, const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd,
-                        uint32_t window, void* workspace, hipStream_t s);
+                        uint32_t window, void* workspace, hipStream_t s, PageTable pt = PageTable{});
 // The same over a paged cache: k_pool / v_pool fp16 [pages][page_rows][kv_heads*hd], row t of the sequence is row
 // t % page_rows of pool page page_table[t / page_rows].  f32 output, no window.
 bool attn_decode_paged_supported(uint32_t seq_len, uint32_t page_rows);
@@ -178,15 +192,16 @@ void attn_decode_noalloc_prepare();
 // attn_prefill.hip
 // q rows / out rows have strides q_stride / out_stride floats (q may live inside a fused qkv buffer).
 // window != 0: the query at position p sees keys [max(0, p - window + 1), p] (attention_sliding_batch, emit.rs:907-1046).
+// pt: a paged cache needs pages of a multiple of 64 rows (a key tile then lies within one page).
 void launch_attn_prefill(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, float* out,
                          uint32_t out_stride, uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads,
-                         uint32_t hd, uint32_t window, hipStream_t s);
+                         uint32_t hd, uint32_t window, hipStream_t s, PageTable pt = PageTable{});
 
 // The same attention, written as the activation quantiser's output of its rows: int8 codes oq[M][heads*hd] and fp16 scales
 // osc[M][heads*hd/32] (bit-identical to launch_attn_prefill followed by launch_quantize_act).
 void launch_attn_prefill_quant(const float* q, uint32_t q_stride, const uint16_t* kc, const uint16_t* vc, int8_t* oq, uint16_t* osc,
                                uint32_t M, uint32_t base_pos, uint32_t heads, uint32_t kv_heads, uint32_t hd, uint32_t window,
-                               hipStream_t s, bool neg_odd = false);
+                               hipStream_t s, bool neg_odd = false, PageTable pt = PageTable{});
 
 bool attn_head_dim_supported(uint32_t hd);
 
@@ -223,6 +238,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
                   const float* qkv_bias, PdState** out);
 int32_t pd_set_repeat_penalty(PdState* st, float penalty);
 void pd_set_poll_limit(PdState* st, uint32_t n);
+int32_t pd_set_kv_pages(PdState* st, PageTable pt, uint32_t max_seq);
 void pd_destroy(PdState* st);
 int32_t pd_enqueue(PdState* st, bool profile, uint32_t token, hipStream_t s);
 // Spins on the host word the kernel writes last; false = not available, wait for the stream instead.

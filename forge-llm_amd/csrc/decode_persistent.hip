@@ -67,6 +67,9 @@ constexpr int PD_STREAM_WAVES = PD_WAVES - PD_POLL_WAVES;
 constexpr int PD_POLL_N = 20;                 // tagged elements a poller thread takes per round trip
 // misc LDS (floats): [0,33) norm partial sums, [40] hint flag, [64,128) phase scratch
 constexpr int PD_MISC_HINT = 40, PD_MISC_SCRATCH = 64;
+// misc LDS words [PD_MISC_PT, 512): page-table entries of this workgroup's attention items, staged once per step (an item's
+// key range is the same in every layer); slot (round, wave group) holds pt_cap entries
+constexpr int PD_MISC_PT = 128, PD_MISC_PT_WORDS = 512 - PD_MISC_PT;
 
 struct PdGemv {
     const uint8_t* qs;
@@ -124,6 +127,8 @@ struct PdArgs {
     const float* qkv_bias;                     // optional [layers][QKS + 2 KV]: added to q, k, v before the rotation (Qwen2)
     float penalty;                             // > 1: the argmax is taken over the penalised logits
     uint32_t window;                           // != 0: attention over the last `window` positions only (sliding window)
+    PageTable pt;                              // paged KV cache (table == nullptr: flat); pt_cap: table entries an attention item may span
+    uint32_t pt_cap;
     uint32_t use_hint;                         // pollers wait for one watched element before re-reading a whole buffer
     uint32_t off_act_s, off_misc, off_big;     // LDS byte offsets (activation codes sit at 0)
     unsigned long long* stamps;                // optional: wall clock at the start of every phase (workgroup 0)
@@ -523,6 +528,45 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float* a, float 
     m = mn;
 }
 
+// Key range [t0, t1) of attention work item number `round` of wave group `grp` of this workgroup (the items of
+// attn_decode_split_kernel: kv head group x split), and which item it is.  The same in every layer of a step.
+struct PdItem { uint32_t item, n_items, nbx, t0, t1, seq, start, chunk; bool on; };
+template <int HD>
+__device__ __forceinline__ PdItem pd_attn_item(const PdArgs& a, uint32_t pos, uint32_t round, uint32_t grp, const PdCtx& cx) {
+    constexpr int LPK = HD <= 64 ? 8 : 16;
+    constexpr int KPW = 64 / LPK;
+    const bool dual = a.gt == 1;
+    const uint32_t gsize = a.heads / a.kv_heads, gpk = gsize / a.gt;
+    PdItem r;
+    r.nbx = a.kv_heads * gpk; r.n_items = r.nbx * DECODE_SPLITS;
+    r.seq = pos + 1;
+    // attention_sliding (emit.rs:598-627): only the last `window` rows are keys (window 0: all of them)
+    r.start = (a.window != 0 && r.seq > a.window) ? r.seq - a.window : 0;
+    r.chunk = (r.seq - r.start + DECODE_SPLITS - 1) / DECODE_SPLITS;
+    r.chunk = (r.chunk + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
+    r.item = cx.wg + (dual ? 2 * round + grp : round) * cx.G;
+    r.on = r.item < r.n_items;
+    const uint32_t split = r.item / r.nbx;
+    r.t0 = r.on ? min(r.seq, r.start + split * r.chunk) : r.seq;      // no item: an empty key range
+    r.t1 = min(r.seq, r.t0 + r.chunk);
+    return r;
+}
+
+// Paged cache: the table entries of every item of this workgroup, into LDS, once per step.
+template <int HD>
+__device__ __forceinline__ void pd_stage_pages(const PdArgs& a, uint32_t pos, uint32_t* pts, const PdCtx& cx) {
+    if (!a.pt.table) return;
+    const bool dual = a.gt == 1;
+    const PdItem any = pd_attn_item<HD>(a, pos, 0, 0, cx);
+    const uint32_t per_round = dual ? 2 * cx.G : cx.G, rounds = (any.n_items + per_round - 1) / per_round;
+    for (uint32_t s = 0; s < rounds * (dual ? 2u : 1u); s++) {
+        const PdItem it = pd_attn_item<HD>(a, pos, dual ? s >> 1 : s, dual ? s & 1u : 0u, cx);
+        if (it.t1 <= it.t0) continue;
+        const uint32_t first = it.t0 >> a.pt.shift, n = ((it.t1 - 1) >> a.pt.shift) - first + 1;
+        for (uint32_t i = cx.tid; i < n && i < a.pt_cap; i += PD_THREADS) pts[s * a.pt_cap + i] = a.pt.table[first + i];
+    }
+}
+
 // P2: the work items of attn_decode_split_kernel (kv head group x split), one per workgroup at a time.  The
 // separate kernel gives an item four waves that each carry all `gt` query heads of the group; here wave
 // 4 g + w carries head g over the keys wave w would take (same keys, same order, same merges), which
@@ -530,7 +574,7 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float* a, float 
 // row and q from the tagged buffers P1 filled.
 template <int HD>
 __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* kc, const uint16_t* vc, uint32_t pos, uint32_t tag_in,
-                                              uint32_t tag_out, float* big, const PdCtx& cx) {
+                                              uint32_t tag_out, float* big, const uint32_t* pts, const PdCtx& cx) {
     constexpr int LPK = HD <= 64 ? 8 : 16;
     constexpr int KPW = 64 / LPK;
     constexpr int REC = HD + 2;
@@ -546,29 +590,32 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
     float* q_lds = sh + 16 * REC;                                     // [gt][HD]
     uint32_t* kvn = reinterpret_cast<uint32_t*>(q_lds + 4 * HD);      // [2][HD] fp16 bits of this position's K and V
     const uint32_t nbx = a.kv_heads * gpk, n_items = nbx * DECODE_SPLITS;
-    const uint32_t seq = pos + 1;
     const uint32_t c = lane % LPK, slot = lane / LPK;
     const bool dvalid = c * 8 < HD;
     const float scale = 1.0f / sqrtf((float)HD);
     const uint32_t kv_stride = a.KV;
-    // attention_sliding (emit.rs:598-627): only the last `window` rows are keys (window 0: all of them)
-    const uint32_t start = (a.window != 0 && seq > a.window) ? seq - a.window : 0;
-    uint32_t chunk = (seq - start + DECODE_SPLITS - 1) / DECODE_SPLITS;
-    chunk = (chunk + 4 * KPW - 1) / (4 * KPW) * (4 * KPW);
+    const bool paged = a.pt.table != nullptr;
 
     // every workgroup walks the same number of rounds (the barriers inside are workgroup-wide); a wave group whose item
     // number is past the end only takes part in the barriers
     const uint32_t per_round = dual ? 2 * cx.G : cx.G;
     const uint32_t rounds = (n_items + per_round - 1) / per_round;
     for (uint32_t it = 0; it < rounds; it++) {
-        const uint32_t item = cx.wg + (dual ? 2 * it + grp : it) * cx.G;
-        const bool on = item < n_items;
+        const PdItem itm = pd_attn_item<HD>(a, pos, it, grp, cx);
+        const uint32_t item = itm.item;
+        const bool on = itm.on;
         const uint32_t bx = item % nbx, split = item / nbx;
         const uint32_t kvh = bx / gpk, sub = bx % gpk;
         const uint32_t h0 = kvh * gsize + sub * gt;
-        const uint32_t t0 = on ? min(seq, start + split * chunk) : seq;      // no item: an empty key range
-        const uint32_t t1 = min(seq, t0 + chunk);
+        const uint32_t t0 = itm.t0, t1 = itm.t1;
         const bool has_new = t0 <= pos && pos < t1;
+        // row of the cache (pool) that holds position t of this item's range: the item's table entries sit in LDS
+        const uint32_t* my_pts = pts + (dual ? 2 * it + grp : it) * a.pt_cap;
+        const uint32_t pt_first = t0 >> a.pt.shift, pt_mask = (1u << a.pt.shift) - 1u;
+        auto row_of = [&](uint32_t t) -> size_t {
+            if (!paged) return t;
+            return ((size_t)my_pts[(t >> a.pt.shift) - pt_first] << a.pt.shift) + (t & pt_mask);
+        };
         // The cached K/V rows do not depend on q: the first key blocks of this wave are requested before q is awaited (loads
         // return in order, so the wait for q then costs the longer of the two latencies, not their sum).
         constexpr int UNR = 4;        // key blocks whose K/V loads are issued together
@@ -580,7 +627,7 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
             kr0[u] = Half8{{0, 0, 0, 0}};
             vr0[u] = Half8{{0, 0, 0, 0}};
             if (t < t1 && dvalid && t != pos) {
-                const size_t off = (size_t)t * kv_stride + kvh * HD + c * 8;
+                const size_t off = row_of(t) * kv_stride + kvh * HD + c * 8;
                 kr0[u] = ldg(reinterpret_cast<const Half8*>(kc + off));
                 vr0[u] = ldg(reinterpret_cast<const Half8*>(vc + off));
             }
@@ -646,7 +693,7 @@ __device__ __forceinline__ void pd_attn_split(const PdArgs& a, const uint16_t* k
                                 vr[u].w[i] = (kvn[HD + c * 8 + 2 * i] & 0xFFFFu) | (kvn[HD + c * 8 + 2 * i + 1] << 16);
                             }
                         } else {
-                            const size_t off = (size_t)t * kv_stride + kvh * HD + c * 8;
+                            const size_t off = row_of(t) * kv_stride + kvh * HD + c * 8;
                             kr[u] = ldg(reinterpret_cast<const Half8*>(kc + off));
                             vr[u] = ldg(reinterpret_cast<const Half8*>(vc + off));
                         }
@@ -779,7 +826,7 @@ __device__ __forceinline__ ArgPair arg_wg(ArgPair a, float* misc, const PdCtx& c
 //   tiles     compute a round from registers, issue the next round (or the next tile's first), sum, finish the rows
 template <bool Q4, int HD, int FMT, bool ORDERED, bool PEN>
 __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& job, const Mat& next, bool early, WReg& W, WReg& W1, const float* emb,
-                                              uint32_t pos, uint32_t* aq_lds, float* as_lds, float* misc, float* big, ArgPair& best,
+                                              uint32_t pos, size_t crow, uint32_t* aq_lds, float* as_lds, float* misc, float* big, ArgPair& best,
                                               const PdCtx& cx) {
     const PdGemv& g = a.shape[job.which];
     const Shape h = pd_shape(g);
@@ -878,12 +925,12 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
                             stc64(a.tq + row, job.tag_out, __float_as_uint(o));
                         } else {
                             const uint16_t hb = f32_to_f16_bits(o);
-                            stg(job.kc + (size_t)pos * a.KV + (row - a.QKS), hb);
+                            stg(job.kc + crow * a.KV + (row - a.QKS), hb);
                             stc64(a.tkv + (row - a.QKS), job.tag_out, hb);
                         }
                     } else {
                         const uint16_t hb = f32_to_f16_bits(v);
-                        stg(job.vc + (size_t)pos * a.KV + (row - a.QKS - a.KV), hb);
+                        stg(job.vc + crow * a.KV + (row - a.QKS - a.KV), hb);
                         stc64(a.tkv + a.KV + (row - a.QKS - a.KV), job.tag_out, hb);
                     }
                 }
@@ -960,6 +1007,9 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     __syncthreads();
 
     const uint32_t pos = a.state[0], token = a.token_from_arg ? a.token : a.state[1];
+    const size_t crow = paged_row(a.pt, pos);        // row of the cache (pool) that this position's K and V go to
+    uint32_t* pts = reinterpret_cast<uint32_t*>(misc) + PD_MISC_PT;
+    pd_stage_pages<HD>(a, pos, pts, cx);             // published by the first barrier of the first phase
     const float* emb = a.embed + (size_t)token * a.H;
     cx.token = token;
     const uint32_t L = a.n_layers;
@@ -983,7 +1033,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         const uint32_t x_in = lg ? base : 0;                 // tag of x entering the layer (0: still the embedding row)
         if (ph == 1) {
             if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * lg + 1] = wall_clock64();
-            pd_attn_split<HD>(a, a.layers[l].kc, a.layers[l].vc, pos, base + 1, base + 2, big, cx);
+            pd_attn_split<HD>(a, a.layers[l].kc, a.layers[l].vc, pos, base + 1, base + 2, big, pts, cx);
             if (sh_abort) return;
             if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * lg + 2] = wall_clock64();
             pd_attn_combine<HD>(a, base + 2, base + 3, misc, big, cx);
@@ -1021,8 +1071,8 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         job.kc = a.layers[l].kc;
         job.bias = (PEN && a.qkv_bias && ph == 0) ? a.qkv_bias + (size_t)lg * (a.QKS + 2 * a.KV) : nullptr;
         job.vc = a.layers[l].vc;
-        if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
-        else pd_gemv_phase<false, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, aq_lds, as_lds, misc, big, best, cx);
+        if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
+        else pd_gemv_phase<false, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
         early = next.valid;
         if (sh_abort) return;
     }
@@ -1233,6 +1283,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     a.H = H; a.I = I; a.QKS = QKS; a.KV = KV; a.heads = c.heads; a.kv_heads = c.kv_heads;
     a.eps = c.rms_eps;
     a.window = c.sliding_window;
+    a.pt = PageTable{}; a.pt_cap = 0;
     a.embed = embed; a.final_norm = final_norm; a.cos_t = cos_t; a.sin_t = sin_t;
     a.logits = logits; a.state = state;
     a.counts = counts; a.penalty = 1.0f;
@@ -1289,6 +1340,23 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     st->n_stamps = 6 * a.total_layers + 3;
     a.stamps = nullptr;
     *out = st.release();
+    return FORGE_HIP_OK;
+}
+
+// Paged KV cache (pt.table == nullptr: back to the flat cache).  The kernel keeps the table entries of a workgroup's
+// attention items in a fixed LDS area: fails if `max_seq` rows in pages this small would need more.
+int32_t pd_set_kv_pages(PdState* st, PageTable pt, uint32_t max_seq) {
+    PdArgs& a = st->args;
+    if (!pt.table) { a.pt = PageTable{}; a.pt_cap = 0; return FORGE_HIP_OK; }
+    const bool dual = a.gt == 1;
+    const uint32_t n_items = a.kv_heads * ((a.heads / a.kv_heads) / a.gt) * DECODE_SPLITS;
+    const uint32_t per_round = (dual ? 2u : 1u) * st->grid, slots = (n_items + per_round - 1) / per_round * (dual ? 2u : 1u);
+    const uint32_t max_chunk = round_up((max_seq + DECODE_SPLITS - 1) / DECODE_SPLITS, 32);       // 4 KPW <= 32 keys
+    const uint32_t cap = (max_chunk >> pt.shift) + 2;
+    if (slots * cap > (uint32_t)PD_MISC_PT_WORDS)
+        return fail(FORGE_HIP_ERR_INVALID, "kv pages: pages this small need more page-table entries per attention item than the decode kernel keeps (" +
+                                               std::to_string(slots * cap) + " > " + std::to_string(PD_MISC_PT_WORDS) + "): use larger pages");
+    a.pt = pt; a.pt_cap = cap;
     return FORGE_HIP_OK;
 }
 

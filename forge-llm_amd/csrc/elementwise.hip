@@ -146,10 +146,11 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(float* __restrict__ 
                                                             uint32_t kv_heads, uint32_t hd,
                                                             const float* __restrict__ cos_t,
                                                             const float* __restrict__ sin_t,
-                                                            const float* __restrict__ bias) {
+                                                            const float* __restrict__ bias, PageTable pt) {
     // bias (optional): q | k | v bias vectors, added before the rotation (Qwen2, emit.rs:4105-4120)
     const uint32_t r = blockIdx.y;
     const uint32_t pos = (pos_dev ? *pos_dev : base_pos) + r;
+    const size_t crow = paged_row(pt, pos);          // row of the cache (pool) that holds this position
     const uint32_t half = hd / 2;
     const uint32_t qp = heads * half, kp = kv_heads * half;
     const uint32_t p = blockIdx.x * 256 + threadIdx.x;
@@ -174,24 +175,25 @@ __global__ __launch_bounds__(256) void rope_kv_store_kernel(float* __restrict__ 
         o.y = __fadd_rn(__fmul_rn(x.x, s), __fmul_rn(x.y, c));
         *ptr = o;
         uint32_t packed = (uint32_t)f32_to_f16_bits(o.x) | ((uint32_t)f32_to_f16_bits(o.y) << 16);
-        reinterpret_cast<uint32_t*>(kc + (size_t)pos * kv_heads * hd)[pk] = packed;
+        reinterpret_cast<uint32_t*>(kc + crow * kv_heads * hd)[pk] = packed;
     } else if (p < qp + 2 * kp) {
         const uint32_t pv = p - qp - kp;
         float2 x = reinterpret_cast<const float2*>(v + (size_t)r * kv_stride)[pv];
         if (bias) { x.x = x.x + bias[2 * (qp + kp) + 2 * pv]; x.y = x.y + bias[2 * (qp + kp) + 2 * pv + 1]; }
         uint32_t packed = (uint32_t)f32_to_f16_bits(x.x) | ((uint32_t)f32_to_f16_bits(x.y) << 16);
-        reinterpret_cast<uint32_t*>(vc + (size_t)pos * kv_heads * hd)[pv] = packed;
+        reinterpret_cast<uint32_t*>(vc + crow * kv_heads * hd)[pv] = packed;
     }
 }
 
 void launch_rope_kv_store(float* q, float* k, const float* v, uint32_t q_stride, uint32_t kv_stride, uint16_t* kc,
                           uint16_t* vc, uint32_t M, uint32_t base_pos, const uint32_t* pos_dev, uint32_t heads,
-                          uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, const float* bias, hipStream_t s) {
+                          uint32_t kv_heads, uint32_t hd, const float* cos_t, const float* sin_t, const float* bias, hipStream_t s,
+                          PageTable pt) {
     if (M == 0) return;
     uint32_t per_row = (heads + 2 * kv_heads) * hd / 2;
     dim3 grid((per_row + 255) / 256, M);
     fh::launch(rope_kv_store_kernel, grid, 256, 0, s, q, k, v, q_stride, kv_stride, kc, vc, base_pos, pos_dev, heads, kv_heads,
-                                              hd, cos_t, sin_t, bias);
+                                              hd, cos_t, sin_t, bias, pt);
 }
 
 // ---- embedding (emit.rs:585-589) -----------------------------------------------------------------

@@ -70,6 +70,7 @@ struct GemvArgs {
     const float* cos_t;
     const float* sin_t;
     const uint32_t* pos_dev;
+    PageTable pt;            // where position *pos_dev lives in a paged cache
     const float* bias;       // optional: q | k | v bias, added before the rotation (Qwen2, emit.rs:4105-4120)
     uint32_t qks, kv, hd;
     // Epi::SiluQuant: rows [0,I) gate, [I,2I) up -> oq int8 [I], osc fp16 [I/32]
@@ -334,9 +335,9 @@ __global__ __launch_bounds__(WAVES * 64) void gemv_kernel(GemvArgs a) {
                     const float c = a.cos_t[(size_t)pos * (a.hd / 2) + d / 2], s = a.sin_t[(size_t)pos * (a.hd / 2) + d / 2];
                     const float o = (row & 1) ? other * s + r * c : r * c - other * s;
                     if (row < a.qks) a.q_out[row] = o;
-                    else a.kc[(size_t)pos * a.kv + (row - a.qks)] = f32_to_f16_bits(o);
+                    else a.kc[paged_row(a.pt, pos) * a.kv + (row - a.qks)] = f32_to_f16_bits(o);
                 } else {
-                    a.vc[(size_t)pos * a.kv + (row - a.qks - a.kv)] = f32_to_f16_bits(r);
+                    a.vc[paged_row(a.pt, pos) * a.kv + (row - a.qks - a.kv)] = f32_to_f16_bits(r);
                 }
             }
         } else if (EPI == Epi::SiluQuant) {
@@ -490,10 +491,12 @@ void launch_gemv_norm(const QWeight& w, const float* x, const float* norm_w, flo
 
 void launch_gemv_norm_rope_kv(const QWeight& wqkv, const float* x, const float* norm_w, float eps, const float* bias, float* q_out,
                               uint16_t* kc, uint16_t* vc, const float* cos_t, const float* sin_t,
-                              const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s) {
+                              const uint32_t* pos_dev, uint32_t heads, uint32_t kv_heads, uint32_t hd, hipStream_t s,
+                              PageTable pt) {
     GemvArgs a = base_args(wqkv, GemvOrder::MatmulVec);
     a.x = x; a.norm_w = norm_w; a.eps = eps;
     a.q_out = q_out; a.kc = kc; a.vc = vc; a.cos_t = cos_t; a.sin_t = sin_t; a.pos_dev = pos_dev;
+    a.pt = pt;
     a.bias = bias;
     a.qks = heads * hd; a.kv = kv_heads * hd; a.hd = hd;
     a.nseg = 3;

@@ -61,6 +61,9 @@ struct forge_hip_model {
     // decode scratch
     DevBuf x, qkv, gu, logits, aq, asc, attn_ws, gemm_ws, state, argmax_ws;
     DevBuf counts;                       // u32 [vocab]: how often each token id has been fed since the last reset
+    DevBuf page_table;                   // u32 [max_seq / page_rows]: pool page of each page of the sequence (paged KV cache)
+    PageTable pt;                        // table == nullptr: the flat cache
+    std::vector<uint32_t> page_table_host;
     float repeat_penalty = 1.0f;         // > 1: forward_greedy picks the maximum of the penalised logits
     // prefill scratch (chunk_rows rows)
     DevBuf px, pqkv, pattn, pgu, paq, pasc, ptok;
@@ -197,7 +200,7 @@ void enqueue_decode_attention(forge_hip_model* m, uint32_t l, const float* q, ui
                               c.kv_heads, c.head_dim, c.sliding_window, c.max_seq, m->attn_ws.p, s);
         else
             launch_attn_decode(q, m->kc(l), m->vc(l), nullptr, aq, asc, 0, m->d_pos(), c.heads, c.kv_heads, c.head_dim,
-                               c.sliding_window, m->attn_ws.p, s);
+                               c.sliding_window, m->attn_ws.p, s, m->pt);
     }
     { StageMark t(m, ST_O); launch_gemv(m->layers[l].o, aq, asc, m->x.as<float>(), true, GemvOrder::MatmulVec, s); }
 }
@@ -220,7 +223,7 @@ void enqueue_decode_layer(forge_hip_model* m, uint32_t l) {
     if (m->fuse_norm) {
         StageMark t(m, ST_QKV);
         launch_gemv_norm_rope_kv(L.qkv, x, L.attn_norm, c.rms_eps, L.qkv_bias, qkv, m->kc(l), m->vc(l), m->cos_t.as<float>(),
-                                 m->sin_t.as<float>(), m->d_pos(), c.heads, c.kv_heads, c.head_dim, s);
+                                 m->sin_t.as<float>(), m->d_pos(), c.heads, c.kv_heads, c.head_dim, s, m->pt);
         // q now sits compact in qkv[0, QKS)
     } else {
         { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, 1, H, nullptr, aq, asc, s); }
@@ -228,7 +231,7 @@ void enqueue_decode_layer(forge_hip_model* m, uint32_t l) {
         {
             StageMark t(m, ST_ROPE);
             launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), 1, 0, m->d_pos(), c.heads,
-                                 c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s);
+                                 c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s, m->pt);
         }
     }
     enqueue_decode_attention(m, l, qkv, QKS);
@@ -261,7 +264,7 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
     {
         StageMark t(m, ST_ROPE);
         launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos, nullptr, c.heads,
-                             c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s);
+                             c.kv_heads, c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s, m->pt);
     }
     if (exact) {
         { StageMark t(m, ST_ATTN); launch_attn_exact(true, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, c.sliding_window, c.max_seq, nullptr, s); }
@@ -269,9 +272,9 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
     } else if (m->prefill_fuse_quant) {
         // the attention kernel writes the o projection's quantised input itself
         StageMark t(m, ST_ATTN);
-        launch_attn_prefill_quant(qkv, QKV, m->kc(l), m->vc(l), aq, asc, M, base_pos, c.heads, c.kv_heads, c.head_dim, c.sliding_window, s, true);
+        launch_attn_prefill_quant(qkv, QKV, m->kc(l), m->vc(l), aq, asc, M, base_pos, c.heads, c.kv_heads, c.head_dim, c.sliding_window, s, true, m->pt);
     } else {
-        { StageMark t(m, ST_ATTN); launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, c.sliding_window, s); }
+        { StageMark t(m, ST_ATTN); launch_attn_prefill(qkv, QKV, m->kc(l), m->vc(l), attn, QKS, M, base_pos, c.heads, c.kv_heads, c.head_dim, c.sliding_window, s, m->pt); }
         { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s, true); }
     }
     { StageMark t(m, ST_O); launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s, m->gemm_ws.p); }
@@ -677,12 +680,59 @@ int32_t forge_hip_model_set_poll_limit(forge_hip_model* m, uint32_t polls) {
 
 int64_t forge_hip_model_pos(const forge_hip_model* m) { return m ? m->pos : -1; }
 
+int32_t forge_hip_model_set_kv_pages(forge_hip_model* m, uint32_t page_rows, const uint32_t* page_table_host, uint32_t n_pages) {
+    FH_CHECK(m, "set_kv_pages: model is null");
+    FH_CHECK(m->pos == 0, "set_kv_pages: the cache layout can only change while the cache is empty (after create or reset)");
+    FH_HIP(hipStreamSynchronize(m->stream));
+    PageTable pt{};
+    std::vector<uint32_t> table;
+    if (page_rows != 0) {
+        FH_CHECK(!(m->cfg.flags & FORGE_HIP_FLAG_EXACT), "set_kv_pages: the order-faithful kernels (FORGE_HIP_FLAG_EXACT) read a flat cache only");
+        FH_CHECK((page_rows & (page_rows - 1)) == 0 && page_rows >= 64, "set_kv_pages: page_rows must be a power of two, at least 64");
+        FH_CHECK(m->cfg.max_seq % page_rows == 0 && n_pages == m->cfg.max_seq / page_rows,
+                 "set_kv_pages: n_pages must be max_seq / page_rows (max_seq a multiple of page_rows)");
+        FH_CHECK(page_table_host, "set_kv_pages: null page table");
+        // every pool page at most once: two pages of the sequence must not share memory
+        std::vector<uint8_t> seen(n_pages, 0);
+        for (uint32_t i = 0; i < n_pages; i++) {
+            FH_CHECK(page_table_host[i] < n_pages && !seen[page_table_host[i]], "set_kv_pages: the table must name every pool page below n_pages at most once");
+            seen[page_table_host[i]] = 1;
+        }
+        table.assign(page_table_host, page_table_host + n_pages);
+        if (!m->page_table.p) {
+            const int32_t rc = m->page_table.alloc((size_t)m->cfg.max_seq / 64 * 4);      // room for the smallest page size
+            if (rc) return rc;
+        }
+        FH_HIP(hipMemcpy(m->page_table.p, table.data(), (size_t)n_pages * 4, hipMemcpyHostToDevice));
+        pt.table = m->page_table.as<uint32_t>();
+        pt.shift = (uint32_t)__builtin_ctz(page_rows);
+    }
+    if (m->pd) {
+        const int32_t rc = pd_set_kv_pages(m->pd, pt, m->cfg.max_seq);
+        if (rc) return rc;
+    }
+    m->pt = pt;
+    m->page_table_host.swap(table);
+    // the captured kernel sequence carries the old layout in its launch arguments: capture again at the next step
+    if (m->decode_graph) { (void)hipGraphExecDestroy(m->decode_graph); m->decode_graph = nullptr; }
+    return FORGE_HIP_OK;
+}
+
 int32_t forge_hip_model_read_kv(forge_hip_model* m, uint32_t layer, uint32_t which, uint16_t* out_host) {
     FH_CHECK(m && out_host, "read_kv: null pointer");
     FH_CHECK(layer < m->cfg.layers && which <= 1, "read_kv: layer or selector out of range");
     FH_HIP(hipStreamSynchronize(m->stream));
     const uint16_t* src = which == 0 ? m->kc(layer) : m->vc(layer);
-    if (m->pos > 0) FH_HIP(hipMemcpy(out_host, src, (size_t)m->pos * m->KV * 2, hipMemcpyDeviceToHost));
+    if (m->pos > 0 && !m->pt.table) FH_HIP(hipMemcpy(out_host, src, (size_t)m->pos * m->KV * 2, hipMemcpyDeviceToHost));
+    if (m->pos > 0 && m->pt.table) {
+        // paged cache: the sequence's rows page by page, in sequence order
+        const uint64_t page_rows = 1ull << m->pt.shift;
+        for (uint64_t t0 = 0; t0 < (uint64_t)m->pos; t0 += page_rows) {
+            const uint64_t rows = std::min<uint64_t>(page_rows, (uint64_t)m->pos - t0);
+            const uint64_t pool_row = (uint64_t)m->page_table_host[t0 >> m->pt.shift] << m->pt.shift;
+            FH_HIP(hipMemcpy(out_host + t0 * m->KV, src + pool_row * m->KV, rows * m->KV * 2, hipMemcpyDeviceToHost));
+        }
+    }
     return FORGE_HIP_OK;
 }
 

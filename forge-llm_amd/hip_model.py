@@ -110,6 +110,16 @@ class HipModel:
         self._check(self._lib.forge_hip_model_read_kv(self._h, layer, which, out.ctypes.data_as(C.c_void_p)))
         return out
 
+    def set_kv_pages(self, page_rows: int, page_table=None) -> None:
+        """Paged KV cache: position t lives in row t % page_rows of pool page page_table[t // page_rows] (a permutation of
+        range(max_seq // page_rows); page_rows a power of two >= 64).  page_rows = 0: the flat cache.  Only while the cache
+        is empty; same results bit for bit under either layout."""
+        if not page_rows:
+            self._check(self._lib.forge_hip_model_set_kv_pages(self._h, 0, None, 0))
+            return
+        t = np.ascontiguousarray(page_table, dtype=np.uint32)
+        self._check(self._lib.forge_hip_model_set_kv_pages(self._h, int(page_rows), t.ctypes.data_as(C.c_void_p), t.size))
+
     def generate_greedy(self, prompt, n_tokens: int):
         """The reference's greedy loop (crates/forgellm-codegen-cpu/src/project.rs:714-751 with
         temperature 0 and repeat penalty 1.0): prefill, argmax, then feed tokens back."""

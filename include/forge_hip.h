@@ -165,6 +165,17 @@ int64_t forge_hip_model_pos(const forge_hip_model* m);
  * be fed again.  No counterpart in the reference (its CPU loop has nothing to wait for); a no-op for a model that runs
  * the kernel sequence. */
 int32_t forge_hip_model_set_poll_limit(forge_hip_model* m, uint32_t polls);
+/* A PAGED KV cache for the model: the cache memory of every layer is taken as a pool of n_pages = max_seq / page_rows pages
+ * of page_rows rows, and position t of the sequence lives in row t % page_rows of pool page page_table[t / page_rows].  For
+ * hosts that hand a sequence its cache pages from a shared allocator; it has no counterpart in the reference, whose
+ * model object owns one flat array per layer (emit.rs:3954-4019, metal:3525-3553).  Every kernel of the fast mode follows
+ * the table (prefill: RoPE + cache write, MFMA attention; decode: the resident kernel and the kernel sequence), and the
+ * results are, bit for bit, those of the flat cache.  page_rows: a power of two, at least 64 (a 64-key attention tile
+ * then lies within one page), dividing max_seq; page_table_host: n_pages pool page numbers, each below n_pages, none
+ * twice.  page_rows = 0 switches back to the flat cache.  Only while the cache is empty (after create or reset); not with
+ * FORGE_HIP_FLAG_EXACT (the order-faithful kernels read a flat cache).  forge_hip_model_read_kv returns rows in sequence
+ * order under either layout. */
+int32_t forge_hip_model_set_kv_pages(forge_hip_model* m, uint32_t page_rows, const uint32_t* page_table_host, uint32_t n_pages);
 /* Debug/parity: copy layer `layer`'s cached K (which=0) or V (which=1) rows [0,pos) to host as
  * fp16 bit patterns, row-major [pos][kv_heads*head_dim]. */
 int32_t forge_hip_model_read_kv(forge_hip_model* m, uint32_t layer, uint32_t which, uint16_t* out_host);

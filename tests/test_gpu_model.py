@@ -412,6 +412,89 @@ def test_persistent_decode_kernel_real_shapes(fh, torch_gpu, monkeypatch, shape)
     seq.close(); one.close()
 
 
+@pytest.mark.parametrize("persist", ["1", "0"])
+@pytest.mark.parametrize("shape", ["llama_1b_2layers", "llama_3b_2layers", "phi3_mini_2layers", "window_hd64"])
+def test_paged_kv_cache_equals_flat_cache(fh, torch_gpu, monkeypatch, shape, persist):
+    """The model over a PAGED cache (forge_hip_model_set_kv_pages: pages in a shuffled order, so that consecutive positions
+    sit far apart in the pool) against the same model over the flat cache: prefill in two calls (the second starts inside
+    a page and reads keys of pages the first one wrote), decode steps through the resident kernel and through the kernel
+    sequence, greedy tokens, logits and the cache rows in sequence order -- all bit for bit.  Pages of 64 and of 256 rows;
+    a model with a sliding window; a second sequence after reset with another table."""
+    if shape == "phi3_mini_2layers":
+        cfg = fh.synth.tiny(Q8, max_seq=1024, hidden=3072, inter=8192, layers=2, heads=32, kv_heads=32, head_dim=96, vocab=32064)
+        n_prompt, page_rows = 700, 64
+    elif shape == "llama_3b_2layers":
+        cfg = fh.synth.llama32_3b(Q8, max_seq=1024)
+        cfg["layers"], cfg["vocab"] = 2, 32000
+        n_prompt, page_rows = 700, 256
+    elif shape == "window_hd64":
+        cfg = fh.synth.tiny(Q4, max_seq=1024, hidden=512, inter=1024, layers=2, heads=8, kv_heads=2, head_dim=64, vocab=3000)
+        cfg["sliding_window"] = 200
+        n_prompt, page_rows = 600, 64
+    else:
+        cfg = fh.synth.llama32_1b(Q8, max_seq=2048)
+        cfg["layers"], cfg["vocab"] = 2, 32000
+        n_prompt, page_rows = 1500, 64
+    monkeypatch.setenv("FORGE_HIP_PERSIST", persist)
+    blob = fh.synth.make_weights_blob(cfg, seed=131, threads=16)
+    toks = fh.synth.uniform_ids(132, n_prompt + 12, cfg["vocab"])
+    flat, paged = fh.HipModel(cfg, blob), fh.HipModel(cfg, blob)
+    assert (flat.decode_launches == 1) == (persist == "1")
+    n_pages = cfg["max_seq"] // page_rows
+    table = np.random.default_rng(7).permutation(n_pages).astype(np.uint32)
+    paged.set_kv_pages(page_rows, table)
+    first = n_prompt // 2 + 13                                   # not a multiple of the page size
+    for m in (flat, paged):
+        m.forward_prefill_batch(toks[:first])
+    same_bits(paged.forward_prefill(toks[first:n_prompt]), flat.forward_prefill(toks[first:n_prompt]))
+    for t in toks[n_prompt:n_prompt + 6]:
+        same_bits(paged.forward(int(t)), flat.forward(int(t)))
+    a = b = int(toks[n_prompt + 6])
+    for _ in range(6):
+        a, b = paged.forward_greedy(a), flat.forward_greedy(b)
+        assert a == b
+    for layer in range(cfg["layers"]):
+        for which in (0, 1):
+            assert np.array_equal(paged.read_kv(layer, which), flat.read_kv(layer, which))
+    # the layout can change only while the cache is empty; a new sequence may use another table
+    with pytest.raises(fh.ForgeHipError):
+        paged.set_kv_pages(page_rows, table)
+    paged.reset(); flat.reset()
+    paged.set_kv_pages(page_rows, table[::-1].copy())
+    same_bits(paged.forward_prefill(toks[:90]), flat.forward_prefill(toks[:90]))
+    assert paged.forward_greedy(5) == flat.forward_greedy(5)
+    paged.reset(); flat.reset()
+    paged.set_kv_pages(0)                                        # back to the flat cache
+    same_bits(paged.forward_prefill(toks[:70]), flat.forward_prefill(toks[:70]))
+    flat.close(); paged.close()
+
+
+def test_paged_kv_cache_refusals(fh, torch_gpu):
+    cfg = tiny_cfg(fh, Q8, 0)                                    # max_seq 640
+    blob = fh.synth.make_weights_blob(cfg, seed=11)
+    m = fh.HipModel(cfg, blob)
+    ok = np.arange(10, dtype=np.uint32)
+    for rows, table in ((32, np.arange(20, dtype=np.uint32)),    # pages below 64 rows
+                        (96, np.arange(6, dtype=np.uint32)),     # not a power of two
+                        (128, np.arange(5, dtype=np.uint32)),    # 640 / 128 = 5 pages, fine in number, but checked below
+                        (64, np.arange(9, dtype=np.uint32)),     # wrong number of pages
+                        (64, np.array([0, 1, 2, 3, 4, 5, 6, 7, 8, 8], np.uint32)),   # a pool page twice
+                        (64, np.array([0, 1, 2, 3, 4, 5, 6, 7, 8, 10], np.uint32))): # a page beyond the pool
+        if rows == 128:
+            m.set_kv_pages(rows, table)                          # this one is valid
+            m.set_kv_pages(0)
+            continue
+        with pytest.raises(fh.ForgeHipError) as e:
+            m.set_kv_pages(rows, table)
+        assert e.value.code == fh.ERR_INVALID
+    m.set_kv_pages(64, ok)
+    m.close()
+    x = fh.HipModel(dict(tiny_cfg(fh, Q8, EXACT)), blob)
+    with pytest.raises(fh.ForgeHipError):
+        x.set_kv_pages(64, ok)                                   # the order-faithful kernels read a flat cache
+    x.close()
+
+
 @pytest.mark.parametrize("wd", [Q8, Q4])
 def test_prefill_gemm_k_ranges_at_model_level(fh, torch_gpu, monkeypatch, wd):
     """Two Llama-3.2-1B-shaped layers over a 2502-token prompt (fast mode): the o and down projections have 320 tiles for 256
