@@ -29,6 +29,7 @@ ERR_HIP = -5
 # every symbol include/forge_hip.h declares
 EXPORTS = [
     "forge_hip_last_error", "forge_hip_device_count", "forge_hip_weights_nbytes", "forge_hip_model_create",
+    "forge_hip_weights_nbytes_mixed", "forge_hip_model_create_mixed",
     "forge_hip_model_destroy", "forge_hip_forward", "forge_hip_forward_greedy", "forge_hip_prefill_batch",
     "forge_hip_forward_profile", "forge_hip_prefill_profile", "forge_hip_model_decode_launches", "forge_hip_reset", "forge_hip_model_pos", "forge_hip_model_set_poll_limit", "forge_hip_model_set_kv_pages", "forge_hip_model_read_kv", "forge_hip_f16_to_f32",
     "forge_hip_f32_to_f16", "forge_hip_quantize_f32", "forge_hip_expf_host", "forge_hip_dequant", "forge_hip_qweight_create",
@@ -107,6 +108,10 @@ def lib():
     L.forge_hip_model_set_poll_limit.argtypes = [vp, C.c_uint32]
     L.forge_hip_model_read_kv.restype = i32
     L.forge_hip_model_read_kv.argtypes = [vp, u32, u32, vp]
+    L.forge_hip_weights_nbytes_mixed.restype = u64
+    L.forge_hip_weights_nbytes_mixed.argtypes = [C.POINTER(Config), vp]
+    L.forge_hip_model_create_mixed.restype = i32
+    L.forge_hip_model_create_mixed.argtypes = [C.POINTER(Config), vp, vp, u64, C.POINTER(vp)]
     L.forge_hip_model_set_kv_pages.restype = i32
     L.forge_hip_model_set_kv_pages.argtypes = [vp, u32, vp, u32]
     L.forge_hip_f16_to_f32.restype = C.c_float

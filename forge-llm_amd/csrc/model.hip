@@ -28,6 +28,7 @@ struct Layer {
     float* attn_norm = nullptr;
     float* ffn_norm = nullptr;
     QWeight qkv, o, gate_up, down;
+    QWeight q, k, v, gate, up;           // a model with a storage format per projection keeps these five apart (qkv, gate_up unused)
     float* qkv_bias = nullptr;           // [QKS + 2 KV]: q | k | v bias, in the row order of the fused qkv matrix (FLAG_QKV_BIAS)
 };
 
@@ -77,6 +78,11 @@ struct forge_hip_model {
     bool fuse_norm = false, fuse_silu = false;   // fused GEMV prologue/epilogue variants fit LDS for this model
     hipGraphExec_t decode_graph = nullptr;
     PdState* pd = nullptr;               // the decode step as one resident kernel, when the shape is covered
+    // ProjectionDTypes (ir.rs:410-421): q, k, v, o, gate, up, down each in its own storage format (GGML ids 8, 2, 12, 14).
+    // `mixed`: they are not all cfg.wdtype, or the lm_head is a K-quant: every projection is then a GEMV launch of its own
+    // and a prompt is walked token by token, as the reference does for such models (emit.rs:4530-4534, 4621-5040).
+    bool mixed = false;
+    uint32_t pd_types[7] = {0, 0, 0, 0, 0, 0, 0};
     // forward_profile / prefill_profile: one event pair per kernel launch, tagged with the stage of the
     // enclosing StageMark (ST_COUNT = outside any stage, not measured)
     int prof_cur = 0;
@@ -94,7 +100,10 @@ struct forge_hip_model {
         if (decode_graph) (void)hipGraphExecDestroy(decode_graph);
         pd_destroy(pd);
         for (hipEvent_t e : prof_ev) (void)hipEventDestroy(e);
-        for (auto& L : layers) { qweight_free(&L.qkv); qweight_free(&L.o); qweight_free(&L.gate_up); qweight_free(&L.down); }
+        for (auto& L : layers) {
+            qweight_free(&L.qkv); qweight_free(&L.o); qweight_free(&L.gate_up); qweight_free(&L.down);
+            qweight_free(&L.q); qweight_free(&L.k); qweight_free(&L.v); qweight_free(&L.gate); qweight_free(&L.up);
+        }
         qweight_free(&lm_head);
         if (h_stage) (void)hipHostFree(h_stage);
         if (h_logits) (void)hipHostFree(h_logits);
@@ -155,13 +164,19 @@ int32_t collect_profile(forge_hip_model* m, float* stage_ms, uint32_t* stage_lau
     return FORGE_HIP_OK;
 }
 
-size_t wsize(uint32_t dtype, uint64_t n, uint64_t k) { return (size_t)(n * (k / 32) * (dtype == FORGE_HIP_Q8_0 ? 34 : 18)); }
+bool is_kquant(uint32_t d) { return d == FORGE_HIP_Q4_K || d == FORGE_HIP_Q6_K; }
+// bytes of an [n][k] matrix in a storage format (project.rs:195-213)
+size_t wsize(uint32_t dtype, uint64_t n, uint64_t k) {
+    if (is_kquant(dtype)) return (size_t)(n * (k / 256) * (dtype == FORGE_HIP_Q4_K ? 144 : 210));
+    return (size_t)(n * (k / 32) * (dtype == FORGE_HIP_Q8_0 ? 34 : 18));
+}
 
 // The numbers sizes are computed from: formats, dimensions the kernels cover.
-int32_t validate_shape(const forge_hip_config* c) {
+int32_t validate_shape(const forge_hip_config* c, bool lm_head_kquant_ok = false) {
     FH_CHECK(c, "config is null");
     FH_CHECK(c->wdtype == FORGE_HIP_Q8_0 || c->wdtype == FORGE_HIP_Q4_0, "wdtype must be Q8_0 (8) or Q4_0 (2)");
-    FH_CHECK(c->lm_head_dtype == FORGE_HIP_Q8_0 || c->lm_head_dtype == FORGE_HIP_Q4_0, "lm_head_dtype must be Q8_0 (8) or Q4_0 (2)");
+    FH_CHECK(c->lm_head_dtype == FORGE_HIP_Q8_0 || c->lm_head_dtype == FORGE_HIP_Q4_0 || (lm_head_kquant_ok && is_kquant(c->lm_head_dtype)),
+             "lm_head_dtype must be Q8_0 (8) or Q4_0 (2) (Q4_K (12) / Q6_K (14): forge_hip_model_create_mixed)");
     FH_CHECK(c->hidden >= 32 && c->hidden % 32 == 0 && c->hidden <= 16352, "hidden must be a multiple of 32 in [32, 16352]");
     FH_CHECK(c->inter >= 32 && c->inter % 32 == 0, "inter must be a positive multiple of 32");
     FH_CHECK(c->layers >= 1 && c->vocab >= 1 && c->max_seq >= 1, "layers, vocab and max_seq must be positive");
@@ -172,8 +187,8 @@ int32_t validate_shape(const forge_hip_config* c) {
     return FORGE_HIP_OK;
 }
 
-int32_t validate_cfg(const forge_hip_config* c) {
-    const int32_t rc = validate_shape(c);
+int32_t validate_cfg(const forge_hip_config* c, bool lm_head_kquant_ok = false) {
+    const int32_t rc = validate_shape(c, lm_head_kquant_ok);
     if (rc) return rc;
     FH_CHECK((c->flags & ~(FORGE_HIP_FLAG_EXACT | FORGE_HIP_FLAG_QKV_BIAS)) == 0, "unknown bits in flags");
     // The reference switches to its non-flash attention (a different summation order) when
@@ -205,11 +220,65 @@ void enqueue_decode_attention(forge_hip_model* m, uint32_t l, const float* q, ui
     { StageMark t(m, ST_O); launch_gemv(m->layers[l].o, aq, asc, m->x.as<float>(), true, GemvOrder::MatmulVec, s); }
 }
 
+// One projection in its own storage format (matmul_call, emit.rs:3316-3334): y (=|+=) W * the quantised vector.
+void gemv_any(const QWeight& w, const int8_t* aq, const uint16_t* asc, float* y, bool accumulate, GemvOrder order, hipStream_t s) {
+    if (w.kquant()) launch_gemv_kquant(w, aq, asc, y, accumulate, s);
+    else launch_gemv(w, aq, asc, y, accumulate, order, s);
+}
+
+// One decoder layer for ONE row of a model with a storage format per projection (model::forward, emit.rs:4029-4500, with
+// the projection calls of emit.rs:4085-4100, 4200-4260): every projection a launch of its own kernel family.  The row sits
+// at `pos` (pos_dev == nullptr: a token of a prompt) or at *pos_dev (a decode step).
+void enqueue_mixed_layer(forge_hip_model* m, uint32_t l, uint32_t pos, const uint32_t* pos_dev) {
+    const forge_hip_config& c = m->cfg;
+    Layer& L = m->layers[l];
+    hipStream_t s = m->stream;
+    const uint32_t H = m->H, I = m->I, QKS = m->QKS, KV = m->KV, QKV = m->QKV;
+    float* x = m->x.as<float>();
+    float* qkv = m->qkv.as<float>();
+    float* gu = m->gu.as<float>();
+    int8_t* aq = m->aq.as<int8_t>();
+    uint16_t* asc = m->asc.as<uint16_t>();
+    const GemvOrder mv = GemvOrder::MatmulVec;
+    const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, 1, H, nullptr, aq, asc, s); }
+    {
+        StageMark t(m, ST_QKV);
+        gemv_any(L.q, aq, asc, qkv, false, mv, s);
+        gemv_any(L.k, aq, asc, qkv + QKS, false, mv, s);
+        gemv_any(L.v, aq, asc, qkv + QKS + KV, false, mv, s);
+    }
+    {
+        StageMark t(m, ST_ROPE);
+        launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), 1, pos, pos_dev, c.heads, c.kv_heads,
+                             c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), nullptr, s, m->pt);
+    }
+    {
+        StageMark t(m, ST_ATTN);
+        if (exact)
+            launch_attn_exact(false, qkv, QKS, m->kc(l), m->vc(l), nullptr, QKS, aq, asc, 1, pos, pos_dev, c.heads, c.kv_heads,
+                              c.head_dim, 0u, c.max_seq, m->attn_ws.p, s);
+        else
+            launch_attn_decode(qkv, m->kc(l), m->vc(l), nullptr, aq, asc, pos + 1, pos_dev, c.heads, c.kv_heads, c.head_dim, 0u,
+                               m->attn_ws.p, s, m->pt);
+    }
+    { StageMark t(m, ST_O); gemv_any(L.o, aq, asc, x, true, mv, s); }
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, 1, H, nullptr, aq, asc, s); }
+    {
+        StageMark t(m, ST_GATE_UP);
+        gemv_any(L.gate, aq, asc, gu, false, mv, s);
+        gemv_any(L.up, aq, asc, gu + I, false, mv, s);
+    }
+    { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, 1, I, 2 * I, nullptr, aq, asc, s); }
+    { StageMark t(m, ST_DOWN); gemv_any(L.down, aq, asc, x, true, mv, s); }
+}
+
 // One decoder layer of the decode step (one row, position read from device memory).  Six launches
 // when the fused GEMV variants fit LDS: [norm+quant | qkv GEMV | rope + KV write], attention split,
 // attention merge + quant, [o GEMV | residual], [norm+quant | gate/up GEMV | silu*up + quant],
 // [down GEMV | residual].
 void enqueue_decode_layer(forge_hip_model* m, uint32_t l) {
+    if (m->mixed) { enqueue_mixed_layer(m, l, 0, m->d_pos()); return; }
     const forge_hip_config& c = m->cfg;
     Layer& L = m->layers[l];
     hipStream_t s = m->stream;
@@ -290,7 +359,17 @@ void enqueue_head(forge_hip_model* m, const float* xrow, bool after_prefill, boo
     const GemvOrder order = after_prefill ? GemvOrder::LmHeadAfterPrefill : GemvOrder::LmHead;
     // The lm_head runs thousands of workgroups; repeating the norm prologue in each costs more than the
     // one extra launch, so the fused form is used only for small vocabularies.
-    if (m->fuse_norm && m->cfg.vocab <= 16384) {
+    if (m->mixed) {
+        // the per-token forward_prefill ends with the lm_head loop of forward (emit.rs:4880-5040), not with the batched one's
+        {
+            StageMark t(m, ST_RMSNORM);
+            launch_rmsnorm(xrow, m->final_norm.as<float>(), m->cfg.rms_eps, 1, m->H, nullptr, m->aq.as<int8_t>(), m->asc.as<uint16_t>(), s);
+        }
+        {
+            StageMark t(m, ST_LM_HEAD);
+            gemv_any(m->lm_head, m->aq.as<int8_t>(), m->asc.as<uint16_t>(), m->logits.as<float>(), false, GemvOrder::LmHead, s);
+        }
+    } else if (m->fuse_norm && m->cfg.vocab <= 16384) {
         StageMark t(m, ST_LM_HEAD);
         launch_gemv_norm(m->lm_head, xrow, m->final_norm.as<float>(), m->cfg.rms_eps, m->logits.as<float>(), order, s);
     } else {
@@ -390,20 +469,68 @@ uint64_t forge_hip_weights_nbytes(const forge_hip_config* c) {
     return over ? 0 : total;
 }
 
+uint64_t forge_hip_weights_nbytes_mixed(const forge_hip_config* c, const uint32_t* pd) {
+    if (!c || !pd) return 0;
+    bool over = false;
+    auto mul = [&](uint64_t a, uint64_t b) { uint64_t r = 0; over = over || __builtin_mul_overflow(a, b, &r); return r; };
+    auto add = [&](uint64_t a, uint64_t b) { uint64_t r = 0; over = over || __builtin_add_overflow(a, b, &r); return r; };
+    auto w = [&](uint32_t t, uint64_t n, uint64_t k) {
+        if (is_kquant(t)) return mul(mul(n, k / 256), t == FORGE_HIP_Q4_K ? 144 : 210);
+        return mul(mul(n, k / 32), t == FORGE_HIP_Q8_0 ? 34 : 18);
+    };
+    const uint64_t H = c->hidden, I = c->inter, QKS = mul(c->heads, c->head_dim), KV = mul(c->kv_heads, c->head_dim);
+    uint64_t per_layer = add(mul(H, 8), add(add(w(pd[0], QKS, H), add(w(pd[1], KV, H), w(pd[2], KV, H))), w(pd[3], H, QKS)));
+    per_layer = add(per_layer, add(add(w(pd[4], I, H), w(pd[5], I, H)), w(pd[6], H, I)));
+    const uint64_t total = add(add(mul(mul(c->vocab, H), 4), mul(c->layers, per_layer)), add(mul(H, 4), w(c->lm_head_dtype, c->vocab, H)));
+    return over ? 0 : total;
+}
+
+static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd, const uint8_t* blob, uint64_t nbytes, forge_hip_model** out);
+
 int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob, uint64_t nbytes, forge_hip_model** out) {
+    return model_create_impl(cfg, nullptr, blob, nbytes, out);
+}
+
+int32_t forge_hip_model_create_mixed(const forge_hip_config* cfg, const uint32_t* proj_dtypes, const uint8_t* blob, uint64_t nbytes,
+                                     forge_hip_model** out) {
+    FH_CHECK(out, "model_create_mixed: null out");
+    *out = nullptr;
+    FH_CHECK(cfg && proj_dtypes, "model_create_mixed: null pointer");
+    bool mixed = is_kquant(cfg->lm_head_dtype);
+    for (int i = 0; i < 7; i++) {
+        const uint32_t d = proj_dtypes[i];
+        FH_CHECK(d == FORGE_HIP_Q8_0 || d == FORGE_HIP_Q4_0 || is_kquant(d), "model_create_mixed: a projection's format must be Q8_0 (8), Q4_0 (2), Q4_K (12) or Q6_K (14)");
+        mixed = mixed || d != cfg->wdtype;
+    }
+    return model_create_impl(cfg, mixed ? proj_dtypes : nullptr, blob, nbytes, out);
+}
+
+static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd, const uint8_t* blob, uint64_t nbytes, forge_hip_model** out) {
     FH_CHECK(out, "model_create: null out");
     *out = nullptr;
-    int32_t rc = validate_cfg(cfg);
+    int32_t rc = validate_cfg(cfg, pd != nullptr);
     if (rc) return rc;
     FH_CHECK(blob, "model_create: null weights");
-    if (nbytes != forge_hip_weights_nbytes(cfg))
-        return fail(FORGE_HIP_ERR_BLOB_SIZE, "weights blob is " + std::to_string(nbytes) + " bytes, config needs " +
-                                                 std::to_string(forge_hip_weights_nbytes(cfg)));
+    if (pd) {
+        // what the per-projection path covers: no QKV bias, no sliding window (the reference's per-token prefill runs full
+        // attention even for a model with a window, emit.rs:4717-4720: not restated), K-quant matrices over K % 256 == 0
+        FH_CHECK((cfg->flags & FORGE_HIP_FLAG_QKV_BIAS) == 0 && cfg->sliding_window == 0,
+                 "model_create_mixed: QKV bias and sliding windows are covered for uniformly Q8_0 / Q4_0 models only");
+        const uint32_t kin[7] = {cfg->hidden, cfg->hidden, cfg->hidden, cfg->heads * cfg->head_dim, cfg->hidden, cfg->hidden, cfg->inter};
+        for (int i = 0; i < 7; i++)
+            FH_CHECK(!is_kquant(pd[i]) || kquant_k_supported(kin[i]), "model_create_mixed: a K-quant projection needs an input width that is a multiple of 256, at most 16384");
+        FH_CHECK(!is_kquant(cfg->lm_head_dtype) || kquant_k_supported(cfg->hidden), "model_create_mixed: a K-quant lm_head needs hidden to be a multiple of 256");
+    }
+    const uint64_t want = pd ? forge_hip_weights_nbytes_mixed(cfg, pd) : forge_hip_weights_nbytes(cfg);
+    if (nbytes != want)
+        return fail(FORGE_HIP_ERR_BLOB_SIZE, "weights blob is " + std::to_string(nbytes) + " bytes, config needs " + std::to_string(want));
     if (forge_hip_device_count() < 1) return fail(FORGE_HIP_ERR_NO_DEVICE, "no HIP device");
     attn_decode_noalloc_prepare();
 
     std::unique_ptr<forge_hip_model> m(new forge_hip_model());
     m->cfg = *cfg;
+    m->mixed = pd != nullptr;
+    if (pd) memcpy(m->pd_types, pd, sizeof(m->pd_types));
     const uint32_t H = m->H = cfg->hidden, I = m->I = cfg->inter;
     const uint32_t QKS = m->QKS = cfg->heads * cfg->head_dim, KV = m->KV = cfg->kv_heads * cfg->head_dim;
     m->QKV = QKS + 2 * KV;
@@ -412,8 +539,8 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
     m->use_graph = !(genv && genv[0] == '0');
     const char* fenv = getenv("FORGE_HIP_FUSE");
     const bool fuse_ok = !(fenv && fenv[0] == '0');
-    m->fuse_norm = fuse_ok && gemv_norm_fusable(H);
-    m->fuse_silu = fuse_ok && gemv_silu_fusable(H);
+    m->fuse_norm = fuse_ok && !pd && gemv_norm_fusable(H);
+    m->fuse_silu = fuse_ok && !pd && gemv_silu_fusable(H);
     m->prefill_fuse_quant = fuse_ok;
     FH_HIP(hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking));
     FH_HIP(hipHostMalloc((void**)&m->h_stage, 64, hipHostMallocDefault));
@@ -440,6 +567,25 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
         L.ffn_norm = L.attn_norm + H;
         FH_HIP(hipMemcpy(L.attn_norm, p, H * 4, hipMemcpyHostToDevice));
         p += H * 4;
+        if (pd) {
+            if ((rc = qweight_upload(pd[0], p, H, QKS, &L.q))) return rc;
+            p += wsize(pd[0], QKS, H);
+            if ((rc = qweight_upload(pd[1], p, H, KV, &L.k))) return rc;
+            p += wsize(pd[1], KV, H);
+            if ((rc = qweight_upload(pd[2], p, H, KV, &L.v))) return rc;
+            p += wsize(pd[2], KV, H);
+            if ((rc = qweight_upload(pd[3], p, QKS, H, &L.o))) return rc;
+            p += wsize(pd[3], H, QKS);
+            FH_HIP(hipMemcpy(L.ffn_norm, p, H * 4, hipMemcpyHostToDevice));
+            p += H * 4;
+            if ((rc = qweight_upload(pd[4], p, H, I, &L.gate))) return rc;
+            p += wsize(pd[4], I, H);
+            if ((rc = qweight_upload(pd[5], p, H, I, &L.up))) return rc;
+            p += wsize(pd[5], I, H);
+            if ((rc = qweight_upload(pd[6], p, I, H, &L.down))) return rc;
+            p += wsize(pd[6], H, I);
+            continue;
+        }
         // q, k, v are adjacent in the blob and all have K = hidden: upload as one matrix.
         rc = qweight_upload(wt, p, H, m->QKV, &L.qkv);
         if (rc) return rc;
@@ -509,7 +655,7 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* blob,
         FH_HIP(hipMemset(m->gemm_ws.p, 0, gemm_split_workspace_bytes()));
     }
     const char* penv = getenv("FORGE_HIP_PERSIST");
-    if (!(penv && penv[0] == '0')) {
+    if (!pd && !(penv && penv[0] == '0')) {       // the resident kernel carries Q8_0 / Q4_0 weight units only
         std::vector<PdLayerIn> pl(cfg->layers);
         for (uint32_t l = 0; l < cfg->layers; l++) {
             Layer& L = m->layers[l];
@@ -562,6 +708,33 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint
     for (uint64_t i = 0; i < n; i++)
         if (tokens[i] >= m->cfg.vocab) return fail(FORGE_HIP_ERR_POSITION, "token id out of range");
     hipStream_t s = m->stream;
+    if (m->mixed) {
+        // forward_prefill of a model that is not uniformly Q8_0 or Q4_0 (emit.rs:4530-4534, 4621-5040): one token at a time
+        // through forward's own operations, the lm_head once after the last token
+        uint64_t fed = 0;
+        while (fed < n) {
+            const uint32_t rows = (uint32_t)std::min<uint64_t>(m->chunk_rows, n - fed);
+            FH_HIP(hipMemcpyAsync(m->ptok.p, tokens + fed, (size_t)rows * 4, hipMemcpyHostToDevice, s));
+            for (uint32_t r = 0; r < rows; r++) {
+                launch_embedding(m->embed.as<float>(), m->ptok.as<uint32_t>() + r, 1, m->H, m->x.as<float>(), m->counts.as<uint32_t>(), s);
+                for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_mixed_layer(m, l, (uint32_t)(m->pos + fed + r), nullptr);
+            }
+            FH_HIP(hipGetLastError());
+            FH_HIP(hipStreamSynchronize(s));          // the token staging area is reused by the next chunk
+            fed += rows;
+        }
+        m->pos += (int64_t)n;
+        m->h_stage[2] = (uint32_t)m->pos;
+        FH_HIP(hipMemcpyAsync(m->d_pos(), &m->h_stage[2], 4, hipMemcpyHostToDevice, s));
+        if (logits_host) {
+            enqueue_head(m, m->x.as<float>(), true, false);
+            FH_HIP(hipGetLastError());
+            FH_HIP(hipMemcpyAsync(m->h_logits, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, s));
+        }
+        FH_HIP(hipStreamSynchronize(s));
+        if (logits_host) memcpy(logits_host, m->h_logits, (size_t)m->cfg.vocab * 4);
+        return FORGE_HIP_OK;
+    }
     uint64_t done = 0;
     uint32_t last_rows = 0;
     while (done < n) {
@@ -641,6 +814,7 @@ int32_t forge_hip_model_decode_launches(const forge_hip_model* m) {
     if (m->pd) return (int32_t)pd_launches_per_step(m->pd);
     const bool exact = (m->cfg.flags & FORGE_HIP_FLAG_EXACT) != 0;
     const int attn = exact ? 1 : 2;
+    if (m->mixed) return 1 + (int)m->cfg.layers * (1 + 3 + 1 + attn + 1 + 1 + 2 + 1 + 1) + 4;
     const int layer = (m->fuse_norm ? 1 : 3) + attn + 1 + (m->fuse_silu ? 1 : 3) + 1;
     const int head = ((m->fuse_norm && m->cfg.vocab <= 16384) ? 1 : 2) + 2;
     return 1 + (int)m->cfg.layers * layer + head;

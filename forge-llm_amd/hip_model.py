@@ -13,9 +13,11 @@ import numpy as np
 
 
 class HipModel:
-    def __init__(self, config: dict, weights):
+    def __init__(self, config: dict, weights, proj_dtypes=None):
         """config: dict with the forge_hip_config fields; weights: the weights.bin bytes
-        (numpy uint8 array, bytes or memoryview).  The blob is copied to the GPU."""
+        (numpy uint8 array, bytes or memoryview).  The blob is copied to the GPU.
+        proj_dtypes: the GGML type ids of (q, k, v, o, gate, up, down) for a model with a storage format per
+        projection (ProjectionDTypes, crates/forgellm-frontend/src/ir.rs:410-421); None: all in config["wdtype"]."""
         from . import Config, check, lib
         self._lib = lib()
         self._check = check
@@ -24,7 +26,14 @@ class HipModel:
         w = np.frombuffer(weights, dtype=np.uint8) if not isinstance(weights, np.ndarray) else weights
         w = np.ascontiguousarray(w, dtype=np.uint8)
         h = C.c_void_p()
-        check(self._lib.forge_hip_model_create(C.byref(self._cfg), w.ctypes.data_as(C.c_void_p), w.size, C.byref(h)))
+        if proj_dtypes is None:
+            check(self._lib.forge_hip_model_create(C.byref(self._cfg), w.ctypes.data_as(C.c_void_p), w.size, C.byref(h)))
+        else:
+            pd = np.ascontiguousarray(proj_dtypes, dtype=np.uint32)
+            if pd.size != 7:
+                raise ValueError("proj_dtypes: seven GGML type ids (q, k, v, o, gate, up, down)")
+            check(self._lib.forge_hip_model_create_mixed(C.byref(self._cfg), pd.ctypes.data_as(C.c_void_p),
+                                                         w.ctypes.data_as(C.c_void_p), w.size, C.byref(h)))
         self._h = h
         self.vocab = int(config["vocab"])
 
@@ -184,3 +193,13 @@ def weights_nbytes(config: dict) -> int:
     from . import Config, lib
     c = Config(**config)
     return int(lib().forge_hip_weights_nbytes(C.byref(c)))
+
+
+def weights_nbytes_mixed(config: dict, proj_dtypes) -> int:
+    """Byte length of a weights.bin whose projections (q, k, v, o, gate, up, down) are stored in proj_dtypes."""
+    from . import Config, lib
+    c = Config(**config)
+    pd = np.ascontiguousarray(proj_dtypes, dtype=np.uint32)
+    if pd.size != 7:
+        raise ValueError("proj_dtypes: seven GGML type ids (q, k, v, o, gate, up, down)")
+    return int(lib().forge_hip_weights_nbytes_mixed(C.byref(c), pd.ctypes.data_as(C.c_void_p)))

@@ -163,6 +163,66 @@ def make_weights_blob(cfg: dict, seed: int, std: float = 0.02, norm_jitter: floa
     return blob
 
 
+def kquant_blocks(rng, ggml_type: int, n_blocks: int, std: float = 0.02) -> np.ndarray:
+    """n_blocks random Q4_K (144-byte) or Q6_K (210-byte) super-blocks whose 256 weights each have zero mean and a standard
+    deviation near `std`: every payload byte uniform, the fp16 super-block scales chosen for that spread.  (Not a
+    quantisation of anything: the tests need valid blocks of sane magnitude, not a particular matrix.)"""
+    if ggml_type == 12:
+        raw = rng.integers(0, 256, (n_blocks, 144), dtype=np.uint8)
+        # w = d * sc * q - dmin * m with sc, m uniform in 0..63 and q in 0..15: zero mean for dmin = 7.5 d, spread 258 d
+        d = (std / 258.0) * rng.uniform(0.7, 1.3, n_blocks)
+        raw[:, 0:2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+        raw[:, 2:4] = (7.5 * d).astype(np.float16).view(np.uint8).reshape(-1, 2)
+    elif ggml_type == 14:
+        raw = rng.integers(0, 256, (n_blocks, 210), dtype=np.uint8)
+        # w = d * scale * (q - 32), scale an int8 kept within +-15 here, q in 0..63: spread about 165 d
+        raw[:, 192:208] = rng.integers(-15, 16, (n_blocks, 16)).astype(np.int8).view(np.uint8)
+        d = (std / 165.0) * rng.uniform(0.7, 1.3, n_blocks)
+        raw[:, 208:210] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+    else:
+        raise ValueError("kquant_blocks: Q4_K (12) or Q6_K (14)")
+    return raw.reshape(-1)
+
+
+def matrix_bytes(n: int, k: int, dtype: int) -> int:
+    """Bytes of an [n][k] matrix in a storage format (GGML type id 8, 2, 12 or 14)."""
+    if dtype in (12, 14):
+        return n * (k // 256) * (144 if dtype == 12 else 210)
+    return n * (k // 32) * (34 if dtype == 8 else 18)
+
+
+def make_weights_blob_mixed(cfg: dict, proj_dtypes, seed: int, std: float = 0.02, norm_jitter: float = 0.1, threads: int = 8) -> np.ndarray:
+    """Random-init model as weights.bin bytes with a storage format per projection: proj_dtypes = (q, k, v, o, gate, up,
+    down) as GGML type ids, the lm_head in cfg["lm_head_dtype"]; Q8_0 / Q4_0 matrices are quantised normal weights, Q4_K /
+    Q6_K matrices random super-blocks (kquant_blocks).  The f32 embedding table is drawn on its own (untied)."""
+    from .ops import quantize_weights
+    H, I = cfg["hidden"], cfg["inter"]
+    QKS, KV = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"]
+    rng = np.random.default_rng(seed)
+    counter = [0]
+
+    def sub_seed():
+        counter[0] += 1
+        return (seed * 1000003 + counter[0] * 7919) & 0xFFFFFFFFFFFFFFFF
+
+    def mat(n, k, dtype):
+        if dtype in (12, 14):
+            assert k % 256 == 0, "a K-quant matrix needs K to be a multiple of 256"
+            return kquant_blocks(rng, dtype, n * (k // 256), std)
+        return quantize_weights(dtype, normal(sub_seed(), n * k, std, threads))
+
+    def norm_vec():
+        return (1.0 + norm_jitter * normal(sub_seed(), H, 1.0, 1)).astype(np.float32)
+
+    pq, pk, pv, po, pg, pu, pdn = [int(x) for x in proj_dtypes]
+    parts = [normal(sub_seed(), cfg["vocab"] * H, std, threads).view(np.uint8)]
+    for _ in range(cfg["layers"]):
+        parts += [norm_vec().view(np.uint8), mat(QKS, H, pq), mat(KV, H, pk), mat(KV, H, pv), mat(H, QKS, po),
+                  norm_vec().view(np.uint8), mat(I, H, pg), mat(I, H, pu), mat(H, I, pdn)]
+    parts += [norm_vec().view(np.uint8), mat(cfg["vocab"], H, cfg["lm_head_dtype"])]
+    return np.concatenate(parts)
+
+
 def gemv_bytes(n: int, k: int, wdtype: int) -> int:
     """Algorithmic bytes of one quantised GEMV: the GGUF blocks of the matrix (34 or 18 bytes
     per 32 weights) plus the f32 input and output vectors."""

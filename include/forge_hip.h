@@ -20,7 +20,8 @@
  *
  * Supported envelope (anything outside it is refused with FORGE_HIP_ERR_INVALID and a message, never
  * computed wrongly):
- *  - model API: projection and lm_head weights Q8_0 or Q4_0; hidden a multiple of 32 in [32, 16352];
+ *  - model API: projection and lm_head weights Q8_0 or Q4_0 (forge_hip_model_create_mixed: also Q4_K and Q6_K, a
+ *    format per projection); hidden a multiple of 32 in [32, 16352];
  *    inter and heads*head_dim multiples of 32, at most 16384; head_dim 64, 96 or 128; heads a multiple
  *    of kv_heads, at most 256; FORGE_HIP_FLAG_EXACT needs max_seq > 512 (below that the reference runs
  *    its non-flash attention, which has no order-faithful kernel here) and, with a sliding window,
@@ -115,6 +116,22 @@ uint64_t forge_hip_weights_nbytes(const forge_hip_config* cfg);
  * keeps ownership of `weights_bin` and may free it on return. */
 int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* weights_bin_host, uint64_t nbytes,
                                forge_hip_model** out);
+
+/* A model whose projections do not share one storage format (ProjectionDTypes, crates/forgellm-frontend/src/ir.rs:410-421;
+ * chosen per GGUF tensor category by detect_gguf_proj_dtypes, crates/forgellm-cli/src/main.rs:608-680; each projection then
+ * calls the kernel of its own format, matmul_call, emit.rs:3316-3334).  proj_dtypes = the GGML type ids of
+ * {q, k, v, o, gate, up, down}, each Q8_0 (8), Q4_0 (2), Q4_K (12) or Q6_K (14); the lm_head's format is
+ * cfg->lm_head_dtype and may be a K-quant too; cfg->wdtype is not read unless all seven agree with it.  The blob has
+ * forge_hip_model_create's layout with every matrix in its own format, K-quant matrices as the GGUF file's own
+ * super-blocks (144 bytes per 256 weights for Q4_K, 210 for Q6_K).  As in the reference, such a model has no batched
+ * prefill (model_is_q8/q4 gate, emit.rs:4530-4534): forge_hip_prefill_batch walks the prompt one token at a time through
+ * the decode operations (forward_prefill, emit.rs:4621-5040) and runs the lm_head once, in forward's order.  Decode runs
+ * the kernel sequence (one GEMV launch per projection), captured in a graph; the resident decode kernel carries Q8_0 and
+ * Q4_0 weights only.  K-quant matrices need an input width that is a multiple of 256; QKV bias and sliding windows are
+ * refused.  When all seven formats equal cfg->wdtype and the lm_head is Q8_0 or Q4_0 this is forge_hip_model_create. */
+uint64_t forge_hip_weights_nbytes_mixed(const forge_hip_config* cfg, const uint32_t* proj_dtypes);
+int32_t forge_hip_model_create_mixed(const forge_hip_config* cfg, const uint32_t* proj_dtypes, const uint8_t* weights_bin_host,
+                                     uint64_t nbytes, forge_hip_model** out);
 void forge_hip_model_destroy(forge_hip_model* m);
 
 /* MetalModel::forward(token_id) -> Vec<f32> (metal:5070) / model::forward (emit.rs:4029):

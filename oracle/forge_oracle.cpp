@@ -812,6 +812,10 @@ struct fo_layer {
 struct fo_model {
     fo_config cfg;
     int variant, kvmode;
+    // storage format of q, k, v, o, gate, up, down (ProjectionDTypes, ir.rs:410-421): 8 = Q8_0, 2 = Q4_0, 12 = Q4_K, 14 = Q6_K
+    // (GGML ids); `mixed`: not all equal to cfg.wdtype, or the lm_head a K-quant
+    uint32_t pd[7];
+    bool mixed = false;
     std::vector<uint8_t> blob;
     const float* embed; std::vector<fo_layer> layers; const float* final_norm; const uint8_t* lm_head;
     std::vector<std::vector<int8_t>> k8, v8; std::vector<std::vector<float>> ks, vs;
@@ -820,7 +824,18 @@ struct fo_model {
     int64_t len;
 };
 
-static int64_t wsize(uint32_t dtype, int64_t n, int64_t k) { return n * ((k + QK - 1) / QK) * (dtype == 8 ? Q8_BYTES : Q4_BYTES); }
+// bytes of an [n][k] matrix in a storage format (project.rs:195-213: 34 / 18 bytes per 32, 144 / 210 bytes per 256 elements)
+static int64_t wsize(uint32_t dtype, int64_t n, int64_t k) {
+    if (dtype == 12 || dtype == 14) return n * ((k + 255) / 256) * (dtype == 12 ? 144 : 210);
+    return n * ((k + QK - 1) / QK) * (dtype == 8 ? Q8_BYTES : Q4_BYTES);
+}
+static bool is_kquant(uint32_t d) { return d == 12 || d == 14; }
+// One projection in its own storage format (matmul_call, emit.rs:3316-3334).  The K-quant kernels quantise their input to
+// Q8_0 blocks on every target architecture (emit.rs:3388-3490, 3622-3655), so `variant` does not reach them.
+static void matmul_vec_any(uint32_t dtype, int variant, float* out, const float* in, const uint8_t* w, int64_t k, int64_t n, int lm_mode) {
+    if (is_kquant(dtype)) matmul_vec_kquant((int)dtype, out, in, w, k, n);
+    else matmul_vec((int)dtype, variant, out, in, w, k, n, lm_mode);
+}
 
 uint64_t fo_weights_nbytes(const fo_config* c) {
     int64_t H = c->hidden, I = c->inter, QKS = (int64_t)c->heads * c->head_dim, KV = (int64_t)c->kv_heads * c->head_dim;
@@ -829,10 +844,26 @@ uint64_t fo_weights_nbytes(const fo_config* c) {
     return (uint64_t)((int64_t)c->vocab * H * 4 + c->layers * per_layer + H * 4 + wsize(c->lm_head_dtype, c->vocab, H));
 }
 
+// The same with a storage format per projection: pd = {q, k, v, o, gate, up, down}; the lm_head's is c->lm_head_dtype.
+uint64_t fo_weights_nbytes_mixed(const fo_config* c, const uint32_t* pd) {
+    int64_t H = c->hidden, I = c->inter, QKS = (int64_t)c->heads * c->head_dim, KV = (int64_t)c->kv_heads * c->head_dim;
+    int64_t per_layer = H * 4 + wsize(pd[0], QKS, H) + wsize(pd[1], KV, H) + wsize(pd[2], KV, H) + wsize(pd[3], H, QKS) + H * 4 +
+                        wsize(pd[4], I, H) + wsize(pd[5], I, H) + wsize(pd[6], H, I) + ((c->flags & 2u) ? (QKS + 2 * KV) * 4 : 0);
+    return (uint64_t)((int64_t)c->vocab * H * 4 + c->layers * per_layer + H * 4 + wsize(c->lm_head_dtype, c->vocab, H));
+}
+
+fo_model* fo_model_create_mixed(const fo_config* c, const uint32_t* pd, const uint8_t* blob, uint64_t nbytes, int variant, int kvmode);
 fo_model* fo_model_create(const fo_config* c, const uint8_t* blob, uint64_t nbytes, int variant, int kvmode) {
-    if (nbytes != fo_weights_nbytes(c)) return nullptr;
+    const uint32_t pd[7] = {c->wdtype, c->wdtype, c->wdtype, c->wdtype, c->wdtype, c->wdtype, c->wdtype};
+    return fo_model_create_mixed(c, pd, blob, nbytes, variant, kvmode);
+}
+
+fo_model* fo_model_create_mixed(const fo_config* c, const uint32_t* pd, const uint8_t* blob, uint64_t nbytes, int variant, int kvmode) {
+    if (nbytes != fo_weights_nbytes_mixed(c, pd)) return nullptr;
     fo_model* m = new fo_model();
     m->cfg = *c; m->variant = variant; m->kvmode = kvmode; m->len = 0;
+    for (int i = 0; i < 7; i++) { m->pd[i] = pd[i]; m->mixed = m->mixed || pd[i] != c->wdtype; }
+    m->mixed = m->mixed || is_kquant(c->lm_head_dtype);
     m->blob.assign(blob, blob + nbytes);
     const uint8_t* p = m->blob.data();
     int64_t H = c->hidden, I = c->inter, QKS = (int64_t)c->heads * c->head_dim, KV = (int64_t)c->kv_heads * c->head_dim;
@@ -840,19 +871,19 @@ fo_model* fo_model_create(const fo_config* c, const uint8_t* blob, uint64_t nbyt
     for (uint32_t l = 0; l < c->layers; l++) {
         fo_layer L;
         L.attn_norm = (const float*)p; p += H * 4;
-        L.q = p; p += wsize(c->wdtype, QKS, H);
-        L.k = p; p += wsize(c->wdtype, KV, H);
-        L.v = p; p += wsize(c->wdtype, KV, H);
+        L.q = p; p += wsize(pd[0], QKS, H);
+        L.k = p; p += wsize(pd[1], KV, H);
+        L.v = p; p += wsize(pd[2], KV, H);
         if (c->flags & 2u) {
             L.q_bias = (const float*)p; p += QKS * 4;
             L.k_bias = (const float*)p; p += KV * 4;
             L.v_bias = (const float*)p; p += KV * 4;
         }
-        L.o = p; p += wsize(c->wdtype, H, QKS);
+        L.o = p; p += wsize(pd[3], H, QKS);
         L.ffn_norm = (const float*)p; p += H * 4;
-        L.gate = p; p += wsize(c->wdtype, I, H);
-        L.up = p; p += wsize(c->wdtype, I, H);
-        L.down = p; p += wsize(c->wdtype, H, I);
+        L.gate = p; p += wsize(pd[4], I, H);
+        L.up = p; p += wsize(pd[5], I, H);
+        L.down = p; p += wsize(pd[6], H, I);
         m->layers.push_back(L);
     }
     m->final_norm = (const float*)p; p += H * 4;
@@ -891,6 +922,7 @@ static void store_kv(fo_model* m, int l, int64_t pos, const float* k, const floa
 }
 
 // emit.rs:4029-4500.  Returns 0, or -3 when the cache is full.
+// logits == NULL: the lm_head is skipped (a token of the per-token forward_prefill that is not the last one, emit.rs:4553-5048).
 int fo_forward(fo_model* m, uint32_t token, float* logits) {
     const fo_config& c = m->cfg;
     int64_t H = c.hidden, I = c.inter, QKS = (int64_t)c.heads * c.head_dim, KV = (int64_t)c.kv_heads * c.head_dim;
@@ -902,9 +934,9 @@ int fo_forward(fo_model* m, uint32_t token, float* logits) {
     for (uint32_t l = 0; l < c.layers; l++) {
         const fo_layer& L = m->layers[l];
         rms_norm(normed.data(), hs.data(), L.attn_norm, H, c.rms_eps, m->variant);
-        matmul_vec(c.wdtype, m->variant, q.data(), normed.data(), L.q, H, QKS, 0);
-        matmul_vec(c.wdtype, m->variant, k.data(), normed.data(), L.k, H, KV, 0);
-        matmul_vec(c.wdtype, m->variant, v.data(), normed.data(), L.v, H, KV, 0);
+        matmul_vec_any(m->pd[0], m->variant, q.data(), normed.data(), L.q, H, QKS, 0);
+        matmul_vec_any(m->pd[1], m->variant, k.data(), normed.data(), L.k, H, KV, 0);
+        matmul_vec_any(m->pd[2], m->variant, v.data(), normed.data(), L.v, H, KV, 0);
         if (L.q_bias) {                                       // emit.rs:4105-4120
             for (int64_t i = 0; i < QKS; i++) q[i] += L.q_bias[i];
             for (int64_t i = 0; i < KV; i++) k[i] += L.k_bias[i];
@@ -917,17 +949,19 @@ int fo_forward(fo_model* m, uint32_t token, float* logits) {
         if (c.sliding_window) attention_sliding(attn.data(), q.data(), cv, pos + 1, c.sliding_window, c.heads, c.kv_heads, c.head_dim);
         else if (flash) attention_flash(attn.data(), q.data(), cv, pos + 1, c.heads, c.kv_heads, c.head_dim);
         else attention_std(attn.data(), q.data(), cv, pos + 1, c.heads, c.kv_heads, c.head_dim);
-        matmul_vec(c.wdtype, m->variant, proj.data(), attn.data(), L.o, QKS, H, 0);
+        matmul_vec_any(m->pd[3], m->variant, proj.data(), attn.data(), L.o, QKS, H, 0);
         for (int64_t i = 0; i < H; i++) hs[i] += proj[i];
         rms_norm(normed.data(), hs.data(), L.ffn_norm, H, c.rms_eps, m->variant);
-        matmul_vec(c.wdtype, m->variant, gate.data(), normed.data(), L.gate, H, I, 0);
-        matmul_vec(c.wdtype, m->variant, up.data(), normed.data(), L.up, H, I, 0);
+        matmul_vec_any(m->pd[4], m->variant, gate.data(), normed.data(), L.gate, H, I, 0);
+        matmul_vec_any(m->pd[5], m->variant, up.data(), normed.data(), L.up, H, I, 0);
         silu_mul(ffn.data(), gate.data(), up.data(), I);
-        matmul_vec(c.wdtype, m->variant, ffo.data(), ffn.data(), L.down, I, H, 0);
+        matmul_vec_any(m->pd[6], m->variant, ffo.data(), ffn.data(), L.down, I, H, 0);
         for (int64_t i = 0; i < H; i++) hs[i] += ffo[i];
     }
-    rms_norm(normed.data(), hs.data(), m->final_norm, H, c.rms_eps, m->variant);
-    matmul_vec(c.lm_head_dtype, m->variant, logits, normed.data(), m->lm_head, H, c.vocab, 1);
+    if (logits) {
+        rms_norm(normed.data(), hs.data(), m->final_norm, H, c.rms_eps, m->variant);
+        matmul_vec_any(c.lm_head_dtype, m->variant, logits, normed.data(), m->lm_head, H, c.vocab, 1);
+    }
     m->len += 1;
     return 0;
 }
@@ -939,6 +973,17 @@ int fo_prefill_batched(fo_model* m, const uint32_t* tokens, int64_t n, float* lo
     int64_t base = m->len;
     if (n <= 0 || base + n > c.max_seq) return -3;
     for (int64_t r = 0; r < n; r++) if (tokens[r] >= c.vocab) return -3;
+    if (m->mixed) {
+        // forward_prefill hands the prompt to the batched function only when every projection is Q8_0 or every one Q4_0
+        // (emit.rs:4530-4534); otherwise it walks the tokens one at a time with forward's own operations and runs the
+        // lm_head once, after the last (emit.rs:4621-5040: chunks of 256 rows, dot8 / dot4 groups and a dot1 tail like
+        // forward's)
+        for (int64_t r = 0; r < n; r++) {
+            const int rc = fo_forward(m, tokens[r], r == n - 1 ? logits : nullptr);
+            if (rc) return rc;
+        }
+        return 0;
+    }
     std::vector<float> hs((size_t)n * H), normed((size_t)n * H), q((size_t)n * QKS), k((size_t)n * KV), v((size_t)n * KV),
         attn((size_t)n * QKS), proj((size_t)n * H), gate((size_t)n * I), up((size_t)n * I), ffn((size_t)n * I), ffo((size_t)n * H);
     for (int64_t r = 0; r < n; r++) std::memcpy(&hs[r * H], m->embed + (int64_t)tokens[r] * H, H * 4);

@@ -45,6 +45,10 @@ def lib():
     L.fo_weights_nbytes.argtypes = [C.POINTER(Config)]
     L.fo_model_create.restype = vp
     L.fo_model_create.argtypes = [C.POINTER(Config), vp, C.c_uint64, i32, i32]
+    L.fo_model_create_mixed.restype = vp
+    L.fo_model_create_mixed.argtypes = [C.POINTER(Config), vp, vp, C.c_uint64, i32, i32]
+    L.fo_weights_nbytes_mixed.restype = C.c_uint64
+    L.fo_weights_nbytes_mixed.argtypes = [C.POINTER(Config), vp]
     L.fo_model_destroy.argtypes = [vp]
     L.fo_model_reset.argtypes = [vp]
     L.fo_model_pos.restype = i64
@@ -284,11 +288,18 @@ def set_num_threads(n):
 class Model:
     """Oracle model: forward / forward_prefill_batched over a weights.bin blob."""
 
-    def __init__(self, cfg: dict, blob, variant=VARIANT_A, kvmode=KV_F16):
+    def __init__(self, cfg: dict, blob, variant=VARIANT_A, kvmode=KV_F16, proj_dtypes=None):
+        """proj_dtypes (optional): storage format of q, k, v, o, gate, up, down as GGML type ids (8, 2, 12, 14); the
+        lm_head's is cfg["lm_head_dtype"].  Default: cfg["wdtype"] for all seven."""
         self.cfg = Config(**cfg)
         blob = _u8(blob)
         self.vocab = cfg["vocab"]
-        self._h = lib().fo_model_create(C.byref(self.cfg), _p(blob), blob.size, variant, kvmode)
+        if proj_dtypes is None:
+            self._h = lib().fo_model_create(C.byref(self.cfg), _p(blob), blob.size, variant, kvmode)
+        else:
+            pd = np.ascontiguousarray(proj_dtypes, dtype=np.uint32)
+            assert pd.size == 7
+            self._h = lib().fo_model_create_mixed(C.byref(self.cfg), _p(pd), _p(blob), blob.size, variant, kvmode)
         if not self._h:
             raise ValueError("oracle: weights blob size does not match the config")
 
@@ -340,6 +351,11 @@ class Model:
             self.close()
         except Exception:
             pass
+
+
+def weights_nbytes_mixed(cfg: dict, proj_dtypes):
+    pd = np.ascontiguousarray(proj_dtypes, dtype=np.uint32)
+    return int(lib().fo_weights_nbytes_mixed(C.byref(Config(**cfg)), _p(pd)))
 
 
 def weights_nbytes(cfg: dict):

@@ -1,0 +1,150 @@
+"""GPU parity of models that keep a storage format per projection (ProjectionDTypes,
+crates/forgellm-frontend/src/ir.rs:410-421): Q8_0, Q4_0, Q4_K and Q6_K matrices side by side, as the reference builds
+them from GGUF files whose tensor categories differ (detect_gguf_proj_dtypes, crates/forgellm-cli/src/main.rs:608-680).
+
+The oracle is the CPU restatement of model::forward with matmul_call's per-projection dispatch (emit.rs:3316-3334) and of
+forward_prefill's per-token walk (emit.rs:4621-5040); tests/test_oracle_model_pin.py holds it to a float64 model.  With
+FLAG_EXACT every operation on the GPU is in the CPU path's order: logits, cache rows and greedy tokens are compared bit
+for bit.  Without it the decode attention is the split-sequence kernel (within 1e-3 per call), held to the loose
+end-to-end bound of the uniform models."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+Q8, Q4, Q4K, Q6K = 8, 2, 12, 14
+A, KV_F16 = 0, 1
+EXACT, QKV_BIAS = 1, 2
+
+MIXES = {
+    "q4_k_m": ((Q4K, Q4K, Q6K, Q4K, Q4K, Q4K, Q6K), Q6K),        # llama.cpp's Q4_K_M recipe
+    "all_four": ((Q8, Q4, Q4K, Q8, Q6K, Q4, Q4K), Q8),
+    "kquant_lm_head_only": ((Q4, Q4, Q4, Q4, Q4, Q4, Q4), Q6K),
+    "q6_k": ((Q6K,) * 7, Q6K),
+}
+
+
+def same_bits(got, want):
+    got, want = np.ascontiguousarray(got, np.float32), np.ascontiguousarray(want, np.float32)
+    diff = got.view(np.uint32) != want.view(np.uint32)
+    assert not diff.any(), f"{diff.sum()} of {diff.size} differ in bits; max abs err {np.max(np.abs(got - want)):.3e}"
+
+
+def tiny(fh, lm, flags, **kw):
+    shape = dict(hidden=256, inter=512, layers=2, heads=4, kv_heads=2, head_dim=64, vocab=1000)
+    shape.update(kw)
+    cfg = fh.synth.tiny(wdtype=Q8, max_seq=640, **shape)
+    cfg["lm_head_dtype"] = lm
+    cfg["flags"] = flags
+    return cfg
+
+
+@pytest.mark.parametrize("mix", list(MIXES))
+def test_mixed_model_exact_mode_is_bit_identical(fh, oracle, torch_gpu, mix):
+    pd, lm = MIXES[mix]
+    cfg = tiny(fh, lm, EXACT)
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=21, std=0.05)
+    toks = fh.synth.uniform_ids(12, 40, cfg["vocab"])
+    gm = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    om = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
+    gl, ol = gm.forward_prefill(toks), om.prefill_batched(toks)
+    assert gm.pos == om.pos == 40
+    same_bits(gl, ol)
+    for layer in range(cfg["layers"]):
+        for which in (0, 1):
+            same_bits(oracle.f16_to_f32(gm.read_kv(layer, which)), om.read_kv(layer, which))
+    tok = oracle.argmax(ol)
+    for _ in range(16):                                     # greedy decode, logits compared at every step
+        g, o = gm.forward(tok), om.forward(tok)
+        same_bits(g, o)
+        tok = oracle.argmax(o)
+    # a second prompt chunk continues the cache (a chat turn)
+    more = fh.synth.uniform_ids(13, 9, cfg["vocab"])
+    same_bits(gm.forward_prefill(more), om.prefill_batched(more))
+    gm.reset()
+    same_bits(gm.forward_prefill(toks), gl)
+    gm.close()
+
+
+def test_mixed_model_greedy_tokens_at_a_real_width(fh, oracle, torch_gpu):
+    """Llama-3.2-1B's widths (hidden 2048 = 8 super-blocks per row, inter 8192, 32:8 heads of 64) in the Q4_K_M recipe:
+    prompt + 24 greedy tokens, ids identical to the oracle's."""
+    pd, lm = MIXES["q4_k_m"]
+    cfg = tiny(fh, lm, EXACT, hidden=2048, inter=8192, heads=32, kv_heads=8, vocab=4096)
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=3, std=0.02)
+    prompt = fh.synth.uniform_ids(5, 24, cfg["vocab"])
+    gm = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    om = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
+    want = [oracle.argmax(om.prefill_batched(prompt))]
+    for _ in range(23):
+        want.append(oracle.argmax(om.forward(want[-1])))
+    assert gm.generate_greedy(prompt, 24) == want
+    gm.close()
+
+
+@pytest.mark.parametrize("mix", ["q4_k_m", "all_four"])
+def test_mixed_model_fast_mode(fh, oracle, torch_gpu, mix, monkeypatch):
+    pd, lm = MIXES[mix]
+    cfg = tiny(fh, lm, 0)
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=21, std=0.05)
+    toks = fh.synth.uniform_ids(12, 40, cfg["vocab"])
+    gm = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    assert gm.decode_launches > 1                           # the kernel sequence: one launch per projection
+    om = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
+    gl, ol = gm.forward_prefill(toks), om.prefill_batched(toks)
+    # layer 0's K/V rows depend on embedding -> rms_norm -> GEMV -> rope only, all order-faithful: same bits
+    for which in (0, 1):
+        same_bits(oracle.f16_to_f32(gm.read_kv(0, which)), om.read_kv(0, which))
+    assert np.max(np.abs(gl - ol)) < 0.1 * max(1.0, float(np.std(ol)) * 4)
+    assert np.corrcoef(gl, ol)[0, 1] > 0.995
+    # the captured graph replays what the eager launches compute
+    steps = [int(t) for t in fh.synth.uniform_ids(14, 6, cfg["vocab"])]
+    graph = [gm.forward(t) for t in steps]
+    gm.close()
+    monkeypatch.setenv("FORGE_HIP_GRAPH", "0")
+    ge = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    assert np.array_equal(ge.forward_prefill(toks), gl)
+    for t, want in zip(steps, graph):
+        assert np.array_equal(ge.forward(t), want)
+    ge.close()
+
+
+def test_uniform_formats_through_the_mixed_entry_point_are_the_plain_model(fh, torch_gpu):
+    cfg = tiny(fh, Q8, 0)
+    cfg["wdtype"] = Q4
+    blob = fh.synth.make_weights_blob(cfg, seed=4)
+    toks = fh.synth.uniform_ids(2, 33, cfg["vocab"])
+    a = fh.HipModel(cfg, blob)
+    b = fh.HipModel(cfg, blob, proj_dtypes=[Q4] * 7)
+    assert b.decode_launches == a.decode_launches == 1      # the resident kernel, as for forge_hip_model_create
+    assert np.array_equal(a.forward_prefill(toks), b.forward_prefill(toks))
+    assert a.generate_greedy([1, 2, 3], 8) == b.generate_greedy([1, 2, 3], 8)
+    a.close()
+    b.close()
+
+
+def test_mixed_model_refusals(fh, torch_gpu):
+    pd, lm = MIXES["q4_k_m"]
+    cfg = tiny(fh, lm, 0)
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=1)
+    with pytest.raises(fh.ForgeHipError) as e:                 # a format the kernels do not carry
+        fh.HipModel(cfg, blob, proj_dtypes=[13] + list(pd[1:]))
+    assert e.value.code == fh.ERR_INVALID
+    with pytest.raises(fh.ForgeHipError) as e:                 # blob of another mix
+        fh.HipModel(cfg, blob, proj_dtypes=MIXES["all_four"][0])
+    assert e.value.code == fh.ERR_BLOB_SIZE
+    for bad in (dict(flags=QKV_BIAS), dict(sliding_window=64)):
+        c = dict(cfg)
+        c.update(bad)
+        with pytest.raises(fh.ForgeHipError) as e:
+            fh.HipModel(c, blob, proj_dtypes=pd)
+        assert e.value.code == fh.ERR_INVALID
+    # SmolLM2's hidden 576 is no multiple of a 256-weight super-block
+    c = tiny(fh, Q8, 0, hidden=576, inter=1536, heads=9, kv_heads=3)
+    with pytest.raises(fh.ForgeHipError) as e:
+        fh.HipModel(c, np.zeros(16, np.uint8), proj_dtypes=pd)
+    assert e.value.code == fh.ERR_INVALID
+    # a K-quant lm_head needs the per-projection entry point
+    with pytest.raises(fh.ForgeHipError) as e:
+        fh.HipModel(cfg, blob)
+    assert e.value.code == fh.ERR_INVALID

@@ -120,6 +120,22 @@ def test_blob_size_contract(fh, oracle):
     assert np.array_equal(table, oracle.dequant(Q8, lm_raw, V * H))
 
 
+def test_blob_size_contract_with_a_format_per_projection(fh, oracle):
+    """project.rs:195-213 sizes every projection by its own format: 34 / 18 bytes per 32 weights, 144 / 210 per 256."""
+    from forge_llm_amd.hip_model import weights_nbytes, weights_nbytes_mixed
+    cfg = fh.synth.tiny(wdtype=Q8, max_seq=640, hidden=256, inter=512, layers=2, heads=4, kv_heads=2, head_dim=64, vocab=301)
+    for pd, lm in (((12, 12, 14, 12, 12, 12, 14), 14), ((8, 2, 12, 8, 14, 2, 12), 8), ((2,) * 7, 2)):
+        c = dict(cfg, lm_head_dtype=lm)
+        n = weights_nbytes_mixed(c, pd)
+        assert n == oracle.weights_nbytes_mixed(c, pd)
+        assert fh.synth.make_weights_blob_mixed(c, pd, seed=1).size == n
+    assert weights_nbytes_mixed(dict(cfg, wdtype=Q4, lm_head_dtype=Q4), (2,) * 7) == weights_nbytes(dict(cfg, wdtype=Q4, lm_head_dtype=Q4))
+    # by hand for one matrix mix: H = 256, I = 512, QKS = 256, KV = 128, 2 layers, vocab 301
+    c = dict(cfg, lm_head_dtype=14)
+    per_layer = 2 * 256 * 4 + 256 * 144 + 128 * 144 + 128 * 210 + 256 * 144 + 2 * 512 * 144 + 256 * 2 * 210
+    assert weights_nbytes_mixed(c, (12, 12, 14, 12, 12, 12, 14)) == 301 * 256 * 4 + 2 * per_layer + 256 * 4 + 301 * 210
+
+
 def test_errors_are_codes_not_crashes(fh):
     L = fh.lib()
     cfg = fh.synth.tiny(Q8)

@@ -34,11 +34,26 @@ def _dequant(raw, wd, n, k):
     return (codes * scale[:, None]).reshape(n, k)
 
 
-def _cut(cfg, blob):
-    """Named tensors of a weights.bin, by the running byte offset of project.rs:342-407."""
+def _dequant_any(oracle, raw, dt, n, k):
+    """Q8_0 / Q4_0 by the routine above; Q4_K (12) and Q6_K (14) super-blocks by the numpy restatement of
+    weight_loader.rs:997-1201, which its own tests pin against the reference's fixtures."""
+    if dt in (Q8, Q4):
+        return _dequant(raw, dt, n, k)
+    from oracle import gguf_oracle
+    return gguf_oracle.dequant_ggml(oracle, dt, np.ascontiguousarray(raw), n * k).astype(np.float64).reshape(n, k)
+
+
+def _nbytes(dt, n, k):
+    return n * (k // 256) * (144 if dt == 12 else 210) if dt in (12, 14) else n * (k // 32) * (34 if dt == Q8 else 18)
+
+
+def _cut(cfg, blob, pd=None, oracle=None):
+    """Named tensors of a weights.bin, by the running byte offset of project.rs:342-407.  pd: the storage formats of
+    (q, k, v, o, gate, up, down) when they differ (ProjectionDTypes, ir.rs:410-421)."""
     H, I, V = cfg["hidden"], cfg["inter"], cfg["vocab"]
     QK, KV = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"]
     wd, lm = cfg["wdtype"], cfg["lm_head_dtype"]
+    pq, pk, pv, po, pg, pu, pdn = pd if pd is not None else [wd] * 7
     boff = [0]
 
     def f32(n):
@@ -47,19 +62,19 @@ def _cut(cfg, blob):
         return v
 
     def mat(n, k, dt):
-        nb = n * (k // 32) * (34 if dt == Q8 else 18)
-        w = _dequant(blob[boff[0]:boff[0] + nb], dt, n, k)
+        nb = _nbytes(dt, n, k)
+        w = _dequant_any(oracle, blob[boff[0]:boff[0] + nb], dt, n, k)
         boff[0] += nb
         return w
 
     t = {"embed": f32(V * H).reshape(V, H), "layers": []}
     for _ in range(cfg["layers"]):
-        L = {"attn_norm": f32(H), "q": mat(QK, H, wd), "k": mat(KV, H, wd), "v": mat(KV, H, wd)}
+        L = {"attn_norm": f32(H), "q": mat(QK, H, pq), "k": mat(KV, H, pk), "v": mat(KV, H, pv)}
         if cfg.get("flags", 0) & FLAG_QKV_BIAS:
             L["qb"], L["kb"], L["vb"] = f32(QK), f32(KV), f32(KV)
-        L["o"] = mat(H, QK, wd)
+        L["o"] = mat(H, QK, po)
         L["ffn_norm"] = f32(H)
-        L["gate"], L["up"], L["down"] = mat(I, H, wd), mat(I, H, wd), mat(H, I, wd)
+        L["gate"], L["up"], L["down"] = mat(I, H, pg), mat(I, H, pu), mat(H, I, pdn)
         t["layers"].append(L)
     t["final_norm"] = f32(H)
     t["lm_head"] = mat(V, H, lm)
@@ -109,19 +124,23 @@ def _kv_round(x, mode):
     return np.clip(np.sign(y) * np.floor(np.abs(y) + 0.5), -127, 127) * np.where(amax > 0, scale, 0.0)
 
 
-def _forward64(cfg, blob, tokens, variant, kvmode):
+def _forward64(cfg, blob, tokens, variant, kvmode, pd=None, oracle=None):
     """Logits of every prompt position [m][vocab] and the cached K/V per layer, all float64."""
-    t = _cut(cfg, blob)
+    t = _cut(cfg, blob, pd, oracle)
     H, hd, nh, nkv = cfg["hidden"], cfg["head_dim"], cfg["heads"], cfg["kv_heads"]
     eps, theta, win = cfg["rms_eps"], cfg["rope_theta"], cfg.get("sliding_window", 0)
     m = len(tokens)
     pos = np.arange(m)
     act = _quant_act if variant == A else (lambda v: v)
+    # a K-quant projection quantises its input on every target (emit.rs:3388-3490), a Q8_0 / Q4_0 one under variant A only
+    kq = (lambda dt: dt in (12, 14))
+    pdl = list(pd) if pd is not None else [cfg["wdtype"]] * 7
+    acts = [(_quant_act if kq(dt) else act) for dt in pdl] + [_quant_act if kq(cfg["lm_head_dtype"]) else act]
     x = t["embed"][np.asarray(tokens, np.int64)].copy()
     caches = []
     for L in t["layers"]:
-        n = act(_rms(x, L["attn_norm"], eps))
-        q, k, v = n @ L["q"].T, n @ L["k"].T, n @ L["v"].T
+        n = _rms(x, L["attn_norm"], eps)
+        q, k, v = acts[0](n) @ L["q"].T, acts[1](n) @ L["k"].T, acts[2](n) @ L["v"].T
         if "qb" in L:
             q, k, v = q + L["qb"], k + L["kb"], v + L["vb"]
         q, k = _rope(q, pos, nh, hd, theta), _rope(k, pos, nkv, hd, theta)
@@ -137,11 +156,11 @@ def _forward64(cfg, blob, tokens, variant, kvmode):
             s = np.where(keep, s, -np.inf)
             p = np.exp(s - s.max(axis=1, keepdims=True))
             out[:, h * hd:(h + 1) * hd] = (p / p.sum(axis=1, keepdims=True)) @ v[:, g * hd:(g + 1) * hd]
-        x = x + act(out) @ L["o"].T
-        n = act(_rms(x, L["ffn_norm"], eps))
-        gate, up = n @ L["gate"].T, n @ L["up"].T
-        x = x + act(gate / (1.0 + np.exp(-gate)) * up) @ L["down"].T
-    return act(_rms(x, t["final_norm"], eps)) @ t["lm_head"].T, caches
+        x = x + acts[3](out) @ L["o"].T
+        n = _rms(x, L["ffn_norm"], eps)
+        gate, up = acts[4](n) @ L["gate"].T, acts[5](n) @ L["up"].T
+        x = x + acts[6](gate / (1.0 + np.exp(-gate)) * up) @ L["down"].T
+    return acts[7](_rms(x, t["final_norm"], eps)) @ t["lm_head"].T, caches
 
 
 def _cfg(fh, wd, heads, kv_heads, hd, max_seq=640, layers=2, bias=False, window=0, vocab=301):
@@ -334,3 +353,42 @@ def test_tail_rows_really_use_the_other_order(oracle, wd):
         assert y[r] == np.float32(four if r in scalar_rows else seq)
         differs += seq != four
     assert differs > 0
+
+
+
+# ---------------------------------------------------------------- a storage format per projection
+Q4K, Q6K = 12, 14
+MIXES = [  # (q, k, v, o, gate, up, down), lm_head
+    ((Q4K, Q4K, Q6K, Q4K, Q4K, Q4K, Q6K), Q6K),     # what llama.cpp's Q4_K_M files hold
+    ((Q8, Q4, Q4K, Q8, Q6K, Q4, Q4K), Q8),          # every format next to every other
+    ((Q4, Q4, Q4, Q4, Q4, Q4, Q4), Q6K),            # uniform projections under a K-quant lm_head
+]
+
+
+@pytest.mark.parametrize("variant", [A, B])
+@pytest.mark.parametrize("pd,lm", MIXES)
+def test_model_with_a_format_per_projection_matches_float64_model(oracle, fh, pd, lm, variant):
+    """Each projection must reach the kernel of ITS format with ITS slice of the blob (matmul_call, emit.rs:3316-3334;
+    reader offsets project.rs:342-407 with per-projection byte counts :195-213): a projection read with another's format
+    or byte count turns the logits into noise.  The prompt goes through forward_prefill's per-token walk (emit.rs:4621-5040),
+    which has to give forward's own numbers bit for bit."""
+    cfg = fh.synth.tiny(wdtype=Q8, max_seq=640, hidden=256, inter=512, layers=2, heads=4, kv_heads=2, head_dim=64, vocab=301)
+    cfg["rope_theta"] = 10000.0
+    cfg["lm_head_dtype"] = lm
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=11 + variant, std=0.05)
+    assert blob.size == oracle.weights_nbytes_mixed(cfg, pd)
+    toks = np.random.default_rng(5).integers(0, cfg["vocab"], 19).astype(np.uint32)
+    want, _ = _forward64(cfg, blob, toks, variant, KV_F16, pd, oracle)
+    m = oracle.Model(cfg, blob, variant, KV_F16, proj_dtypes=pd)
+    rows = np.stack([m.forward(int(t)) for t in toks])
+    scale = np.abs(want).max()
+    assert scale > 0.05
+    # an activation code a hair from a rounding tie may fall the other way in f32 than in f64: from that position on the
+    # difference is one quantisation step; before it (and for most rows) the two agree to f32 rounding
+    per_row = np.abs(rows - want).max(axis=1)
+    assert per_row[0] < 1e-5 * scale and (per_row < 1e-4 * scale).sum() >= 3
+    assert per_row.max() < 3e-2 * scale          # a wiring mistake moves the logits by their own magnitude
+    m2 = oracle.Model(cfg, blob, variant, KV_F16, proj_dtypes=pd)
+    last = m2.prefill_batched(toks)
+    assert np.array_equal(last, rows[-1])
+    assert np.array_equal(m2.forward(7), m.forward(7))
