@@ -40,6 +40,7 @@ EXPORTS = [
     "forge_hip_gguf_open", "forge_hip_gguf_parse", "forge_hip_gguf_close", "forge_hip_gguf_version", "forge_hip_gguf_alignment",
     "forge_hip_gguf_tensor_data_offset", "forge_hip_gguf_tensor_count", "forge_hip_gguf_metadata_count", "forge_hip_gguf_tensor",
     "forge_hip_gguf_find_tensor", "forge_hip_gguf_meta", "forge_hip_gguf_config", "forge_hip_gguf_export_weights",
+    "forge_hip_gguf_config_mixed", "forge_hip_gguf_export_weights_mixed", "forge_hip_quantize_kquant",
     "forge_hip_model_create_from_gguf", "forge_hip_dequant_ggml", "forge_hip_model_set_repeat_penalty", "forge_hip_apply_repeat_penalty", "forge_hip_sample",
 ]
 

@@ -365,6 +365,169 @@ bool dequant_ggml(uint32_t type, const uint8_t* d, uint64_t n, float* out) {
     }
 }
 
+// ---- the K-quant weight quantisers (weight_loader.rs:1646-2140): used when a tensor's format differs from the format its
+// projection category is stored in (load_from_file_mixed_per_tensor, weight_loader.rs:193-218) -----------------------------
+
+inline float round_away(float v) { return roundf(v); }          // f32::round: halves away from zero
+inline float clampf(float v, float lo, float hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// make_qkx2_quants (weight_loader.rs:1666-1768) for one sub-block of 32: returns scale and the_min (>= 0) with
+// dequant(L) = scale * L - the_min, L in [0, nmax]; a search over nstep + 1 slightly shifted inverse scales, each refitted by
+// two-parameter least squares, keeping the candidate with the least squared error.
+void make_qkx2_quants(const float* x, float nmax, float rmin, float rdelta, int nstep, float* scale_out, float* min_out, uint8_t* L) {
+    const int n = 32;
+    float mn = x[0], mx = x[0];
+    for (int i = 1; i < n; i++) { if (x[i] < mn) mn = x[i]; if (x[i] > mx) mx = x[i]; }
+    if (mx == mn) { *scale_out = 0.0f; *min_out = -mn; memset(L, 0, n); return; }
+    if (mn > 0.0f) mn = 0.0f;
+    const float iscale = nmax / (mx - mn);
+    const float scale = 1.0f / iscale;
+    float best_mad = 0.0f;
+    for (int i = 0; i < n; i++) {
+        const float li = clampf(round_away((x[i] - mn) * iscale), 0.0f, nmax);
+        L[i] = (uint8_t)li;
+        const float diff = scale * (float)L[i] + mn - x[i];
+        best_mad += diff * diff;
+    }
+    float best_min = mn, best_scale = scale;
+    uint8_t laux[32];
+    for (int is = 0; is <= nstep && nstep > 0; is++) {
+        const float iscale_try = (rmin + rdelta * (float)is + nmax) / (mx - mn);
+        float sum_l = 0.0f, sum_l2 = 0.0f, sum_x = 0.0f, sum_xl = 0.0f;
+        for (int i = 0; i < n; i++) {
+            laux[i] = (uint8_t)clampf(round_away((x[i] - mn) * iscale_try), 0.0f, nmax);
+            const float lif = (float)laux[i];
+            sum_l += lif;
+            sum_l2 += lif * lif;
+            sum_x += x[i];
+            sum_xl += lif * x[i];
+        }
+        const float nf = (float)n;
+        const float det = nf * sum_l2 - sum_l * sum_l;
+        if (!(det > 0.0f)) continue;
+        float this_scale = (nf * sum_xl - sum_x * sum_l) / det;
+        float this_min = (sum_l2 * sum_x - sum_l * sum_xl) / det;
+        if (this_min > 0.0f) {
+            this_min = 0.0f;
+            if (sum_l2 > 0.0f) this_scale = sum_xl / sum_l2;
+        }
+        if (!(this_scale > 0.0f)) continue;
+        float mad = 0.0f;
+        for (int i = 0; i < n; i++) {
+            const float diff = this_scale * (float)laux[i] + this_min - x[i];
+            mad += diff * diff;
+        }
+        if (mad < best_mad) { memcpy(L, laux, n); best_mad = mad; best_scale = this_scale; best_min = this_min; }
+    }
+    *scale_out = best_scale;
+    *min_out = -best_min;
+}
+
+// quantize_f32_to_q4_k, weight_loader.rs:1773-1882: n floats -> ceil(n / 256) super-blocks of 144 bytes (a tail is padded with zeros).
+void quantize_q4_k(const float* data, uint64_t n, uint8_t* out) {
+    const uint64_t nsb = (n + 255) / 256;
+    for (uint64_t sb = 0; sb < nsb; sb++) {
+        float padded[256] = {0};
+        const uint64_t have = std::min<uint64_t>(256, n - sb * 256);
+        memcpy(padded, data + sb * 256, have * 4);
+        float sub_scale[8], sub_min[8];
+        uint8_t q[8][32];
+        for (int j = 0; j < 8; j++) make_qkx2_quants(padded + j * 32, 15.0f, -1.0f, 0.1f, 20, &sub_scale[j], &sub_min[j], q[j]);
+        float max_scale = 0.0f, max_min = 0.0f;
+        for (int j = 0; j < 8; j++) { if (sub_scale[j] > max_scale) max_scale = sub_scale[j]; if (sub_min[j] > max_min) max_min = sub_min[j]; }
+        const float inv_scale = max_scale > 0.0f ? 63.0f / max_scale : 0.0f;
+        const float inv_min = max_min > 0.0f ? 63.0f / max_min : 0.0f;
+        const float d = max_scale > 0.0f ? max_scale / 63.0f : 0.0f;
+        const float dmin = max_min > 0.0f ? max_min / 63.0f : 0.0f;
+        uint8_t sq[8], mq[8];
+        for (int j = 0; j < 8; j++) {
+            sq[j] = (uint8_t)clampf(round_away(sub_scale[j] * inv_scale), 0.0f, 63.0f);
+            mq[j] = (uint8_t)clampf(round_away(sub_min[j] * inv_min), 0.0f, 63.0f);
+        }
+        // the codes are fitted again to the scales as stored (6 bits under an fp16 super-block scale), :1826-1850
+        const uint16_t d_bits = fh::f32_to_f16_host(d), dmin_bits = fh::f32_to_f16_host(dmin);
+        const float d_stored = fh::f16_to_f32_host(d_bits), dmin_stored = fh::f16_to_f32_host(dmin_bits);
+        for (int j = 0; j < 8; j++) {
+            const float s_eff = d_stored * (float)sq[j];
+            if (s_eff == 0.0f) { memset(q[j], 0, 32); continue; }
+            const float inv_s_eff = 1.0f / s_eff;
+            const float dm_eff = dmin_stored * (float)mq[j];
+            for (int i = 0; i < 32; i++) q[j][i] = (uint8_t)clampf(round_away((padded[j * 32 + i] + dm_eff) * inv_s_eff), 0.0f, 15.0f);
+        }
+        uint8_t* o = out + sb * 144;
+        o[0] = (uint8_t)d_bits; o[1] = (uint8_t)(d_bits >> 8); o[2] = (uint8_t)dmin_bits; o[3] = (uint8_t)(dmin_bits >> 8);
+        for (int i = 0; i < 4; i++) {                 // inverse of get_scale_min_k4
+            o[4 + i] = (uint8_t)((sq[i] & 63) | (((sq[i + 4] >> 4) & 3) << 6));
+            o[8 + i] = (uint8_t)((mq[i] & 63) | (((mq[i + 4] >> 4) & 3) << 6));
+            o[12 + i] = (uint8_t)((sq[i + 4] & 0x0F) | ((mq[i + 4] & 0x0F) << 4));
+        }
+        for (int c = 0; c < 4; c++)
+            for (int i = 0; i < 32; i++) o[16 + c * 32 + i] = (uint8_t)((q[2 * c][i] & 0x0F) | (q[2 * c + 1][i] << 4));
+    }
+}
+
+// make_q6k_quants' scale (weight_loader.rs:1987-2010): -max/32 for the signed value of largest magnitude (the FIRST of equals), 0 for a
+// sub-block of zeros.  The codes it also fits are not used by the caller.
+float q6k_sub_scale(const float* x) {
+    float mx = 0.0f, amax = 0.0f;
+    for (int i = 0; i < 16; i++) { const float av = fabsf(x[i]); if (av > amax) { amax = av; mx = x[i]; } }
+    if (amax < 1e-30f) return 0.0f;
+    const float iscale = -32.0f / mx;
+    return 1.0f / iscale;
+}
+
+// quantize_f32_to_q6_k, weight_loader.rs:2025-2140: n floats -> ceil(n / 256) super-blocks of 210 bytes.
+void quantize_q6_k(const float* data, uint64_t n, uint8_t* out) {
+    const uint64_t nsb = (n + 255) / 256;
+    for (uint64_t sb = 0; sb < nsb; sb++) {
+        float padded[256] = {0};
+        const uint64_t have = std::min<uint64_t>(256, n - sb * 256);
+        memcpy(padded, data + sb * 256, have * 4);
+        float sub[16];
+        float max_scale = 0.0f, max_abs = 0.0f;
+        for (int j = 0; j < 16; j++) {
+            sub[j] = q6k_sub_scale(padded + j * 16);
+            if (fabsf(sub[j]) > max_abs) { max_abs = fabsf(sub[j]); max_scale = sub[j]; }
+        }
+        uint8_t* o = out + sb * 210;
+        memset(o, 0, 210);
+        if (max_abs < 1e-30f) continue;
+        const float super_iscale = -128.0f / max_scale;
+        const float super_d = 1.0f / super_iscale;
+        const uint16_t d_bits = fh::f32_to_f16_host(super_d);
+        o[208] = (uint8_t)d_bits; o[209] = (uint8_t)(d_bits >> 8);
+        int8_t sq[16];
+        for (int j = 0; j < 16; j++) {
+            int v = (int)round_away(super_iscale * sub[j]);
+            v = v < -128 ? -128 : (v > 127 ? 127 : v);
+            sq[j] = (int8_t)v;
+            o[192 + j] = (uint8_t)sq[j];
+        }
+        const float d_stored = fh::f16_to_f32_host(d_bits);
+        int8_t L[256] = {0};
+        for (int j = 0; j < 16; j++) {
+            const float s_eff = d_stored * (float)sq[j];
+            if (s_eff == 0.0f) continue;
+            const float inv = 1.0f / s_eff;
+            for (int i = 0; i < 16; i++) {
+                int v = (int)round_away(inv * padded[j * 16 + i]);
+                L[j * 16 + i] = (int8_t)(v < -32 ? -32 : (v > 31 ? 31 : v));
+            }
+        }
+        for (int half = 0; half < 2; half++) {
+            uint8_t* ql = o + half * 64;
+            uint8_t* qh = o + 128 + half * 32;
+            const int8_t* l = L + half * 128;
+            for (int i = 0; i < 32; i++) {
+                const uint8_t q1 = (uint8_t)(l[i] + 32), q2 = (uint8_t)(l[i + 32] + 32), q3 = (uint8_t)(l[i + 64] + 32), q4 = (uint8_t)(l[i + 96] + 32);
+                ql[i] = (uint8_t)((q1 & 0x0F) | ((q3 & 0x0F) << 4));
+                ql[i + 32] = (uint8_t)((q2 & 0x0F) | ((q4 & 0x0F) << 4));
+                qh[i] = (uint8_t)((q1 >> 4) | ((q2 >> 4) << 2) | ((q3 >> 4) << 4) | ((q4 >> 4) << 6));
+            }
+        }
+    }
+}
+
 const char* const SUPPORTED_TYPES = "F32, F16, BF16, Q8_0, Q4_0, Q4_1, Q4_K, Q5_K, Q6_K and Q8_K";
 
 // f32 values of a tensor as the reference holds it after loading: dense types and Q8_0 / Q4_0 decode directly
@@ -533,9 +696,14 @@ int32_t forge_hip_dequant_ggml(uint32_t ggml_type, const uint8_t* data_host, uin
     });
 }
 
-int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_t flags, forge_hip_config* out) {
-    return no_throw("gguf_config", [&]() -> int32_t {
-        FH_CHECK(g && out, "gguf_config: null argument");
+}  // extern "C"
+
+namespace {
+
+// Everything of load_config (main.rs:700-830) but the weight formats: shape, context, RoPE, window, bias flag; `majority` =
+// detect_gguf_dtype's vote over the projection tensors (main.rs:479-555): Q8_0 (8), Q4_0 (2), Q4_K (12), or 0 for a dense majority.
+int32_t config_base(const forge_hip_gguf* g, uint32_t max_seq, uint32_t flags, forge_hip_config* out, uint32_t* majority) {
+    {
         const MetaValue* arch_v = g->find("general.architecture");
         const std::string arch = arch_v && arch_v->type == 8 ? arch_v->str : "unknown";
         // The kernels here cover the Llama layer, with the QKV bias of Qwen2 (main.rs:770: the bias goes with the
@@ -584,12 +752,139 @@ int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_
             }
         }
         const uint64_t total = q8 + q4 + q4k + f16 + f32;
-        uint32_t wdtype = 0;
-        if (total && q4k <= total / 2) {
-            if (q8 > total / 2) wdtype = FORGE_HIP_Q8_0;
-            else if (q4 > total / 2) wdtype = FORGE_HIP_Q4_0;
+        *majority = 0;
+        if (total) {
+            if (q4k > total / 2) *majority = FORGE_HIP_Q4_K;
+            else if (q8 > total / 2) *majority = FORGE_HIP_Q8_0;
+            else if (q4 > total / 2) *majority = FORGE_HIP_Q4_0;
         }
-        if (!wdtype) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: the projection weights are neither mostly Q8_0 nor mostly Q4_0");
+        const uint64_t seq = max_seq ? max_seq : ctx;
+        // Some(0) would make the reference attend to nothing (emit.rs:604-605)
+        if (has_window && window == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: a sliding window of 0 positions");
+        FH_CHECK(vocab <= 0xFFFFFFFFull && seq <= 0xFFFFFFFFull, "gguf: vocabulary or context length out of range");
+        forge_hip_config c{};
+        c.hidden = hidden; c.inter = inter; c.layers = layers; c.heads = heads; c.kv_heads = kv_heads;
+        c.head_dim = hidden / heads;                     // main.rs:731
+        c.vocab = (uint32_t)vocab; c.max_seq = (uint32_t)seq;
+        c.rms_eps = eps; c.rope_theta = theta;
+        c.flags = flags | (arch == "qwen2" ? FORGE_HIP_FLAG_QKV_BIAS : 0u);
+        c.sliding_window = has_window ? window : 0u;     // main.rs:764-767
+        *out = c;
+        return FORGE_HIP_OK;
+    }
+}
+
+// ---- a storage format per projection category (detect_gguf_proj_dtypes, main.rs:608-680) ------------------------------------
+
+enum Cat { C_EMBED, C_Q, C_K, C_V, C_O, C_GATE, C_UP, C_DOWN, C_LM, C_COUNT, C_NONE };
+constexpr uint32_t DENSE = 1;      // the reference's DType::F16, which stands for every dense tensor type here
+
+// ProjCategory::from_gguf_name, ir.rs:382-401
+Cat category_of(const std::string& name) {
+    if (name == "token_embd.weight") return C_EMBED;
+    if (name == "output.weight" || name == "lm_head.weight") return C_LM;
+    if (name.compare(0, 4, "blk.") != 0) return C_NONE;
+    const size_t dot = name.find('.', 4);
+    if (dot == std::string::npos) return C_NONE;
+    const std::string suffix = name.substr(dot + 1);
+    if (suffix == "attn_q.weight") return C_Q;
+    if (suffix == "attn_k.weight") return C_K;
+    if (suffix == "attn_v.weight") return C_V;
+    if (suffix == "attn_output.weight") return C_O;
+    if (suffix == "ffn_gate.weight") return C_GATE;
+    if (suffix == "ffn_up.weight") return C_UP;
+    if (suffix == "ffn_down.weight") return C_DOWN;
+    return C_NONE;
+}
+
+// ggml_type_storage_dtype, main.rs:586-599: the format a tensor of this type can be kept in; 0 = none (the tensor does not vote)
+uint32_t storage_dtype(uint32_t type) {
+    switch (type) {
+        case T_Q8_0: return FORGE_HIP_Q8_0;
+        case T_Q4_0: return FORGE_HIP_Q4_0;
+        case 12: return FORGE_HIP_Q4_K;
+        case 14: return FORGE_HIP_Q6_K;
+        case T_F32: case T_F16: case T_BF16: return DENSE;
+        default: return 0;
+    }
+}
+
+// precision_rank, main.rs:630-640: decides a tie of counts in favour of the more precise format
+int precision_rank(uint32_t d) {
+    switch (d) {
+        case DENSE: return 5;
+        case FORGE_HIP_Q8_0: return 4;
+        case FORGE_HIP_Q6_K: return 3;
+        case FORGE_HIP_Q4_K: return 2;
+        case FORGE_HIP_Q4_0: return 1;
+        default: return 0;
+    }
+}
+
+// The nine category formats: the majority among the category's tensors, `fallback` for a category without a tensor that votes;
+// a file without an output tensor takes the embedding's format for the lm_head (main.rs:668-678).
+void detect_categories(const forge_hip_gguf* g, uint32_t fallback, uint32_t out[C_COUNT]) {
+    static const uint32_t kinds[5] = {FORGE_HIP_Q8_0, FORGE_HIP_Q4_0, FORGE_HIP_Q4_K, FORGE_HIP_Q6_K, DENSE};
+    uint64_t counts[C_COUNT][5] = {};
+    bool has_lm = false;
+    for (const auto& t : g->tensors) {
+        const Cat c = category_of(t.name);
+        if (c == C_NONE) continue;
+        if (c == C_LM) has_lm = true;
+        const uint32_t d = storage_dtype(t.type);
+        for (int k = 0; k < 5; k++) if (kinds[k] == d) counts[c][k]++;
+    }
+    for (int c = 0; c < C_COUNT; c++) {
+        uint32_t best = fallback;
+        uint64_t best_n = 0;
+        for (int k = 0; k < 5; k++)
+            if (counts[c][k] > best_n || (counts[c][k] == best_n && best_n > 0 && precision_rank(kinds[k]) > precision_rank(best))) {
+                best = kinds[k];
+                best_n = counts[c][k];
+            }
+        out[c] = best;
+    }
+    if (!has_lm) out[C_LM] = out[C_EMBED];
+}
+
+uint64_t qbytes_any(uint32_t dtype, uint64_t numel) {
+    if (dtype == FORGE_HIP_Q4_K) return numel / 256 * 144;
+    if (dtype == FORGE_HIP_Q6_K) return numel / 256 * 210;
+    return qbytes(dtype, numel);
+}
+
+// One tensor in the format of its category (load_from_file_mixed_per_tensor, weight_loader.rs:190-230): the file's bytes when the
+// tensor already has that format; for a K-quant target its values (dequantised directly) quantised with that format's
+// quantiser; for a Q8_0 / Q4_0 target the conversion of the uniform export.
+int32_t write_in_format(const forge_hip_gguf* g, const std::string& name, uint32_t dtype, uint64_t numel, uint8_t* out) {
+    if (dtype == FORGE_HIP_Q8_0 || dtype == FORGE_HIP_Q4_0) return write_quantised(g, name, dtype, numel, out);
+    Source s;
+    int32_t rc = locate(g, name, numel, &s);
+    if (rc) return rc;
+    if (numel % 256) return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor " + name + " is no whole number of 256-weight super-blocks");
+    if (s.t->type == dtype) { memcpy(out, s.bytes, qbytes_any(dtype, numel)); return FORGE_HIP_OK; }
+    std::vector<float> v(numel);
+    if (!dequant_ggml(s.t->type, s.bytes, numel, v.data()))
+        return fail(FORGE_HIP_ERR_INVALID, "gguf: tensor " + name + " has GGML type " + std::to_string(s.t->type) + "; this library reads " +
+                                               SUPPORTED_TYPES + " tensors");
+    if (dtype == FORGE_HIP_Q4_K) quantize_q4_k(v.data(), numel, out);
+    else quantize_q6_k(v.data(), numel, out);
+    return FORGE_HIP_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_t flags, forge_hip_config* out) {
+    return no_throw("gguf_config", [&]() -> int32_t {
+        FH_CHECK(g && out, "gguf_config: null argument");
+        forge_hip_config c{};
+        uint32_t wdtype = 0;
+        const int32_t brc = config_base(g, max_seq, flags, &c, &wdtype);
+        if (brc) return brc;
+        if (wdtype != FORGE_HIP_Q8_0 && wdtype != FORGE_HIP_Q4_0)
+            return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: the projection weights are neither mostly Q8_0 nor mostly Q4_0");
         // lm_head: the type of output.weight after loading (main.rs:567-581, gguf.rs:168-205); without that tensor the
         // embedding table serves, converted to the projections' format
         uint32_t lm = wdtype;
@@ -603,18 +898,7 @@ int32_t forge_hip_gguf_config(const forge_hip_gguf* g, uint32_t max_seq, uint32_
             else return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: output.weight has GGML type " + std::to_string(ot->type) +
                                                            "; this library reads " + SUPPORTED_TYPES + " tensors");
         }
-        const uint64_t seq = max_seq ? max_seq : ctx;
-        // Some(0) would make the reference attend to nothing (emit.rs:604-605)
-        if (has_window && window == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: a sliding window of 0 positions");
-        FH_CHECK(vocab <= 0xFFFFFFFFull && seq <= 0xFFFFFFFFull, "gguf: vocabulary or context length out of range");
-        forge_hip_config c{};
-        c.hidden = hidden; c.inter = inter; c.layers = layers; c.heads = heads; c.kv_heads = kv_heads;
-        c.head_dim = hidden / heads;                     // main.rs:731
-        c.vocab = (uint32_t)vocab; c.max_seq = (uint32_t)seq;
-        c.rms_eps = eps; c.rope_theta = theta;
         c.wdtype = wdtype; c.lm_head_dtype = lm;
-        c.flags = flags | (arch == "qwen2" ? FORGE_HIP_FLAG_QKV_BIAS : 0u);
-        c.sliding_window = has_window ? window : 0u;     // main.rs:764-767
         // what the kernels cannot run is refused here, before any size is computed from these numbers
         const int32_t vrc = fh::validate_config_shape(&c);
         if (vrc) return vrc;
@@ -682,6 +966,89 @@ int32_t forge_hip_gguf_export_weights(const forge_hip_gguf* g, const forge_hip_c
     });
 }
 
+int32_t forge_hip_quantize_kquant(uint32_t ggml_type, const float* data_host, uint64_t n, uint8_t* out_host) {
+    return no_throw("quantize_kquant", [&]() -> int32_t {
+        FH_CHECK(ggml_type == FORGE_HIP_Q4_K || ggml_type == FORGE_HIP_Q6_K, "quantize_kquant: the type must be Q4_K (12) or Q6_K (14)");
+        FH_CHECK(out_host && (data_host || n == 0), "quantize_kquant: null pointer");
+        if (ggml_type == FORGE_HIP_Q4_K) quantize_q4_k(data_host, n, out_host);
+        else quantize_q6_k(data_host, n, out_host);
+        return FORGE_HIP_OK;
+    });
+}
+
+int32_t forge_hip_gguf_config_mixed(const forge_hip_gguf* g, uint32_t max_seq, uint32_t flags, forge_hip_config* out, uint32_t* proj_dtypes,
+                                    uint32_t* embed_dtype) {
+    return no_throw("gguf_config_mixed", [&]() -> int32_t {
+        FH_CHECK(g && out && proj_dtypes, "gguf_config_mixed: null argument");
+        forge_hip_config c{};
+        uint32_t majority = 0;
+        const int32_t brc = config_base(g, max_seq, flags, &c, &majority);
+        if (brc) return brc;
+        if (!majority) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: the projection weights are neither mostly Q8_0, Q4_0 nor Q4_K");
+        uint32_t cat[C_COUNT];
+        detect_categories(g, majority, cat);
+        if (embed_dtype) *embed_dtype = cat[C_EMBED];
+        // The blob keeps the embedding table as f32 whatever the file holds (main.rs:2690-2722).  A dense projection category or a
+        // dense lm_head is stored in the majority format here, as the uniform export does (the reference would keep f32 weights
+        // and run its f32 dot product, which this library does not carry).
+        const uint32_t dense_as = majority == FORGE_HIP_Q4_K ? (uint32_t)FORGE_HIP_Q8_0 : majority;
+        for (int i = C_Q; i <= C_LM; i++) if (cat[i] == DENSE) cat[i] = dense_as;
+        for (int i = 0; i < 7; i++) proj_dtypes[i] = cat[C_Q + i];
+        c.wdtype = (majority == FORGE_HIP_Q8_0 || majority == FORGE_HIP_Q4_0) ? majority : (uint32_t)FORGE_HIP_Q8_0;
+        c.lm_head_dtype = cat[C_LM];
+        *out = c;
+        return FORGE_HIP_OK;
+    });
+}
+
+int32_t forge_hip_gguf_export_weights_mixed(const forge_hip_gguf* g, const forge_hip_config* c, const uint32_t* pd, uint8_t* out_host,
+                                            uint64_t nbytes) {
+    return no_throw("gguf_export_weights_mixed", [&]() -> int32_t {
+        FH_CHECK(g && c && pd && out_host, "gguf_export_weights_mixed: null argument");
+        const uint64_t need = forge_hip_weights_nbytes_mixed(c, pd);
+        if (need == 0 || nbytes != need)
+            return fh::fail(FORGE_HIP_ERR_BLOB_SIZE, "gguf_export_weights_mixed: buffer is " + std::to_string(nbytes) + " bytes, config needs " + std::to_string(need));
+        FH_CHECK(!(c->flags & FORGE_HIP_FLAG_QKV_BIAS), "gguf_export_weights_mixed: QKV bias goes with uniformly Q8_0 / Q4_0 models only");
+        const uint64_t H = c->hidden, I = c->inter, QKS = (uint64_t)c->heads * c->head_dim, KV = (uint64_t)c->kv_heads * c->head_dim, V = c->vocab;
+        auto known = [](uint32_t d) { return d == FORGE_HIP_Q8_0 || d == FORGE_HIP_Q4_0 || d == FORGE_HIP_Q4_K || d == FORGE_HIP_Q6_K; };
+        for (int i = 0; i < 7; i++) FH_CHECK(known(pd[i]), "gguf_export_weights_mixed: a projection's format must be Q8_0, Q4_0, Q4_K or Q6_K");
+        FH_CHECK(known(c->lm_head_dtype), "gguf_export_weights_mixed: lm_head_dtype must be Q8_0, Q4_0, Q4_K or Q6_K");
+        FH_CHECK(H % 32 == 0 && I % 32 == 0 && QKS % 32 == 0, "gguf_export_weights_mixed: row lengths must be multiples of 32");
+        uint8_t* p = out_host;
+        int32_t rc;
+    #define FH_STEP(call, bytes) do { rc = (call); if (rc) return rc; p += (bytes); } while (0)
+        {
+            // the per-tensor loader keeps a Q4_K / Q6_K embedding table in its own format, and the exporter dequantises that
+            // directly (main.rs:2697-2712); every other type goes the way of the uniform export
+            Source e;
+            rc = locate(g, "token_embd.weight", V * H, &e);
+            if (rc) return rc;
+            if (e.t->type == 12 || e.t->type == 14) dequant_ggml(e.t->type, e.bytes, V * H, reinterpret_cast<float*>(p));
+            else if ((rc = write_f32(g, "token_embd.weight", V * H, p))) return rc;
+            p += V * H * 4;
+        }
+        for (uint32_t l = 0; l < c->layers; l++) {
+            if (!g->tensor(blk(l, "attn_q.weight")) || !g->tensor(blk(l, "ffn_gate.weight")))
+                return fh::fail(FORGE_HIP_ERR_INVALID, "gguf: fused attn_qkv / gate-up tensors are split for uniformly Q8_0 / Q4_0 files only");
+            FH_STEP(write_f32(g, blk(l, "attn_norm.weight"), H, p), H * 4);
+            FH_STEP(write_in_format(g, blk(l, "attn_q.weight"), pd[0], QKS * H, p), qbytes_any(pd[0], QKS * H));
+            FH_STEP(write_in_format(g, blk(l, "attn_k.weight"), pd[1], KV * H, p), qbytes_any(pd[1], KV * H));
+            FH_STEP(write_in_format(g, blk(l, "attn_v.weight"), pd[2], KV * H, p), qbytes_any(pd[2], KV * H));
+            FH_STEP(write_in_format(g, blk(l, "attn_output.weight"), pd[3], H * QKS, p), qbytes_any(pd[3], H * QKS));
+            FH_STEP(write_f32(g, blk(l, "ffn_norm.weight"), H, p), H * 4);
+            FH_STEP(write_in_format(g, blk(l, "ffn_gate.weight"), pd[4], I * H, p), qbytes_any(pd[4], I * H));
+            FH_STEP(write_in_format(g, blk(l, "ffn_up.weight"), pd[5], I * H, p), qbytes_any(pd[5], I * H));
+            FH_STEP(write_in_format(g, blk(l, "ffn_down.weight"), pd[6], H * I, p), qbytes_any(pd[6], H * I));
+        }
+        FH_STEP(write_f32(g, "output_norm.weight", H, p), H * 4);
+        const char* lm_name = g->tensor("output.weight") ? "output.weight" : g->tensor("lm_head.weight") ? "lm_head.weight" : "token_embd.weight";
+        FH_STEP(write_in_format(g, lm_name, c->lm_head_dtype, V * H, p), qbytes_any(c->lm_head_dtype, V * H));
+    #undef FH_STEP
+        if ((uint64_t)(p - out_host) != need) return fh::fail(FORGE_HIP_ERR_INVALID, "gguf_export_weights_mixed: internal size mismatch");
+        return FORGE_HIP_OK;
+    });
+}
+
 int32_t forge_hip_model_create_from_gguf(const char* path, uint32_t max_seq, uint32_t flags, forge_hip_model** out) {
     return no_throw("model_create_from_gguf", [&]() -> int32_t {
         FH_CHECK(out, "model_create_from_gguf: null out");
@@ -691,15 +1058,23 @@ int32_t forge_hip_model_create_from_gguf(const char* path, uint32_t max_seq, uin
         if (rc) return rc;
         std::unique_ptr<forge_hip_gguf> hold(g);
         forge_hip_config c;
-        rc = forge_hip_gguf_config(g, max_seq, flags, &c);
+        uint32_t pd[7];
+        rc = forge_hip_gguf_config_mixed(g, max_seq, flags, &c, pd, nullptr);
         if (rc) return rc;
-        const uint64_t n = forge_hip_weights_nbytes(&c);
+        bool uniform = c.lm_head_dtype == FORGE_HIP_Q8_0 || c.lm_head_dtype == FORGE_HIP_Q4_0;
+        for (int i = 0; i < 7; i++) uniform = uniform && pd[i] == c.wdtype;
+        if (uniform) {
+            // every projection in the majority format, Q8_0 or Q4_0: the export and the model of the uniform case
+            rc = forge_hip_gguf_config(g, max_seq, flags, &c);
+            if (rc) return rc;
+        }
+        const uint64_t n = uniform ? forge_hip_weights_nbytes(&c) : forge_hip_weights_nbytes_mixed(&c, pd);
         if (n == 0) return fh::fail(FORGE_HIP_ERR_INVALID, "model_create_from_gguf: the configuration's weight size does not fit 64 bits");
         std::unique_ptr<uint8_t[]> blob(new (std::nothrow) uint8_t[n]);
         if (!blob) return fh::fail(FORGE_HIP_ERR_INVALID, "model_create_from_gguf: out of host memory for " + std::to_string(n) + " bytes");
-        rc = forge_hip_gguf_export_weights(g, &c, blob.get(), n);
+        rc = uniform ? forge_hip_gguf_export_weights(g, &c, blob.get(), n) : forge_hip_gguf_export_weights_mixed(g, &c, pd, blob.get(), n);
         if (rc) return rc;
-        return forge_hip_model_create(&c, blob.get(), n, out);
+        return uniform ? forge_hip_model_create(&c, blob.get(), n, out) : forge_hip_model_create_mixed(&c, pd, blob.get(), n, out);
     });
 }
 

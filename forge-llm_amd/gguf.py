@@ -222,6 +222,29 @@ class GgufFile:
         self._check(self._lib.forge_hip_gguf_config(self._h, max_seq, flags, C.byref(c)))
         return {k: getattr(c, k) for k, _ in Config._fields_}
 
+    def config_mixed(self, max_seq: int = 0, flags: int = 0):
+        """detect_gguf_proj_dtypes on top of load_config (crates/forgellm-cli/src/main.rs:608-680, 782-793): the
+        configuration, the storage formats of (q, k, v, o, gate, up, down) as GGML type ids, and the embedding table's
+        (1 = dense).  config["lm_head_dtype"] is the lm_head category's format."""
+        from . import Config
+        c = Config()
+        pd = np.zeros(7, np.uint32)
+        embed = C.c_uint32()
+        self._check(self._lib.forge_hip_gguf_config_mixed(self._h, max_seq, flags, C.byref(c), pd.ctypes.data_as(C.c_void_p), C.byref(embed)))
+        return {name: getattr(c, name) for name, _ in Config._fields_}, [int(x) for x in pd], int(embed.value)
+
+    def export_weights_mixed(self, cfg: dict, proj_dtypes) -> np.ndarray:
+        """The weights.bin bytes with every projection in the format of its category (load_from_file_mixed_per_tensor,
+        crates/forgellm-frontend/src/weight_loader.rs:152-238; blob order main.rs:2714-2757)."""
+        from . import Config
+        from .hip_model import weights_nbytes_mixed
+        c = Config(**cfg)
+        pd = np.ascontiguousarray(proj_dtypes, dtype=np.uint32)
+        out = np.empty(weights_nbytes_mixed(cfg, pd), np.uint8)
+        self._check(self._lib.forge_hip_gguf_export_weights_mixed(self._h, C.byref(c), pd.ctypes.data_as(C.c_void_p),
+                                                            out.ctypes.data_as(C.c_void_p), out.size))
+        return out
+
     def export_weights(self, cfg: dict) -> np.ndarray:
         from . import Config
         c = Config(**cfg)
@@ -275,3 +298,15 @@ def _declare(L):
     L.forge_hip_model_create_from_gguf.restype = i32
     L.forge_hip_model_create_from_gguf.argtypes = [C.c_char_p, u32, u32, C.POINTER(vp)]
     L._gguf_declared = True
+
+
+def quantize_kquant(ggml_type: int, x) -> np.ndarray:
+    """quantize_f32_to_q4_k / quantize_f32_to_q6_k (crates/forgellm-frontend/src/weight_loader.rs:1773-1882, 2025-2140):
+    f32 array -> ceil(n / 256) super-blocks of 144 (Q4_K, type 12) or 210 (Q6_K, type 14) bytes."""
+    from . import check, lib
+    L = lib()
+    _declare(L)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    out = np.empty((x.size + 255) // 256 * (144 if ggml_type == 12 else 210), np.uint8)
+    check(L.forge_hip_quantize_kquant(ggml_type, x.ctypes.data_as(C.c_void_p), x.size, out.ctypes.data_as(C.c_void_p)))
+    return out

@@ -46,11 +46,14 @@ class HipModel:
         L = lib()
         _declare(L)
         g = GgufFile(path)
-        cfg = g.config(max_seq, flags)
+        cfg, pd, _ = g.config_mixed(max_seq, flags)
+        if all(d == cfg["wdtype"] for d in pd) and cfg["lm_head_dtype"] in (8, 2):
+            cfg, pd = g.config(max_seq, flags), None       # every projection in one format: the uniform rules
         g.close()
         self = cls.__new__(cls)
         self._lib, self._check = L, check
         self.config = cfg
+        self.proj_dtypes = pd
         h = C.c_void_p()
         check(L.forge_hip_model_create_from_gguf(path.encode(), max_seq, flags, C.byref(h)))
         self._h = h

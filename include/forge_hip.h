@@ -365,7 +365,31 @@ int32_t forge_hip_gguf_export_weights(const forge_hip_gguf* g, const forge_hip_c
 /* `dequantize` (weight_loader.rs:809-825) for one tensor's bytes: GGML types F32 (0), F16 (1), BF16 (30), Q8_0 (8), Q4_0 (2),
  * Q4_1 (3), Q4_K (12), Q5_K (13), Q6_K (14), Q8_K (15); n = number of elements. */
 int32_t forge_hip_dequant_ggml(uint32_t ggml_type, const uint8_t* data_host, uint64_t n, float* out_host);
-/* open + config + export_weights + forge_hip_model_create. */
+/* A GGUF file whose tensor categories are not all stored alike (llama.cpp's Q4_K_M: Q4_K for most projections, Q6_K for
+ * half of attn_v / ffn_down and for the output matrix).  detect_gguf_proj_dtypes (main.rs:608-680): per category (q, k, v, o,
+ * gate, up, down, the embedding table, the output matrix) the format most of its tensors have among Q8_0, Q4_0, Q4_K, Q6_K
+ * and "dense" (F32 / F16 / BF16), equal counts going to the more precise one; a category none of whose tensors votes takes
+ * the file's majority format (forge_hip_gguf_config's vote, which here may also come out as Q4_K); without an output tensor
+ * the lm_head takes the embedding's format.  proj_dtypes receives the seven projection formats, *embed_dtype (may be NULL)
+ * the embedding's (1 = dense), out->lm_head_dtype the lm_head's; out->wdtype is the majority format when that is Q8_0 or
+ * Q4_0, else Q8_0 (forge_hip_model_create_mixed does not read it).  A dense projection or lm_head category is reported as
+ * the majority format (Q8_0 under a Q4_K majority): the reference would keep such weights as f32, which this library does
+ * not carry. */
+int32_t forge_hip_gguf_config_mixed(const forge_hip_gguf* g, uint32_t max_seq, uint32_t flags, forge_hip_config* out,
+                                    uint32_t* proj_dtypes, uint32_t* embed_dtype);
+/* The blob of forge_hip_model_create_mixed (exactly forge_hip_weights_nbytes_mixed(cfg, proj_dtypes) bytes) from the file's
+ * tensors, as load_from_file_mixed_per_tensor + export-weights produce it (weight_loader.rs:152-238, main.rs:2556-2757): a
+ * tensor that already has its category's format is copied; for a Q4_K / Q6_K category any other tensor is dequantised and
+ * quantised again with quantize_f32_to_q4_k / _q6_k; for a Q8_0 / Q4_0 category the conversion is that of
+ * forge_hip_gguf_export_weights; a Q4_K / Q6_K embedding table is dequantised directly into the f32 table.  Fused Phi-3
+ * tensors and QKV bias are refused here. */
+int32_t forge_hip_gguf_export_weights_mixed(const forge_hip_gguf* g, const forge_hip_config* cfg, const uint32_t* proj_dtypes,
+                                            uint8_t* out_host, uint64_t nbytes);
+/* quantize_f32_to_q4_k (weight_loader.rs:1773-1882, sub-block fit make_qkx2_quants :1666-1768) and quantize_f32_to_q6_k
+ * (:2025-2140): n floats -> ceil(n / 256) super-blocks of 144 (ggml_type 12) or 210 (14) bytes; a tail is padded with zeros. */
+int32_t forge_hip_quantize_kquant(uint32_t ggml_type, const float* data_host, uint64_t n, uint8_t* out_host);
+/* open + config + export_weights + forge_hip_model_create; a file that forge_hip_gguf_config_mixed finds to hold several
+ * formats (or a K-quant lm_head) goes through the _mixed functions and forge_hip_model_create_mixed instead. */
 int32_t forge_hip_model_create_from_gguf(const char* path, uint32_t max_seq, uint32_t flags, forge_hip_model** out);
 
 /* ---------------- sampling (the loop of the generated main.rs, project.rs:714-751) ----------------

@@ -341,3 +341,262 @@ def export_weights(oracle, g, data, cfg) -> np.ndarray:
     lm_name = "output.weight" if "output.weight" in by_name else "lm_head.weight" if "lm_head.weight" in by_name else "token_embd.weight"
     parts.append(quant(lm_name, V * H, cfg["lm_head_dtype"]))
     return np.concatenate([np.ascontiguousarray(p, np.uint8) for p in parts])
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# A storage format per projection category: detect_gguf_proj_dtypes (main.rs:608-680), load_from_file_mixed_per_tensor
+# (weight_loader.rs:152-238), and the K-quant weight quantisers that loader calls (weight_loader.rs:1666-1882, 1987-2140).
+# The quantisers are written here in array form (all sub-blocks at once, f32 sums kept sequential), from the reference's text;
+# the reference holds no input/output vectors for them, only quality bounds (weight_loader.rs:2735-2990), which
+# tests/test_gguf.py applies to the reference tests' own inputs: beyond those bounds their parity is unpinned.
+
+DENSE = 1
+_CATS = ("embed", "q", "k", "v", "o", "gate", "up", "down", "lm_head")
+_SUFFIX = {"attn_q.weight": "q", "attn_k.weight": "k", "attn_v.weight": "v", "attn_output.weight": "o", "ffn_gate.weight": "gate",
+           "ffn_up.weight": "up", "ffn_down.weight": "down"}
+_RANK = {DENSE: 5, 8: 4, 14: 3, 12: 2, 2: 1}
+
+
+def _category(name):
+    """ProjCategory::from_gguf_name, ir.rs:382-401."""
+    if name == "token_embd.weight":
+        return "embed"
+    if name in ("output.weight", "lm_head.weight"):
+        return "lm_head"
+    if not name.startswith("blk."):
+        return None
+    rest = name[4:]
+    if "." not in rest:
+        return None
+    return _SUFFIX.get(rest[rest.index(".") + 1:])
+
+
+def _storage(ty):
+    """ggml_type_storage_dtype, main.rs:586-599."""
+    return ty if ty in (8, 2, 12, 14) else DENSE if ty in (0, 1, 30) else None
+
+
+def _majority(g):
+    """detect_gguf_dtype, main.rs:479-555: 8, 2, 12, or None for a dense majority."""
+    q8 = q4 = q4k = f16 = f32 = 0
+    as_q8 = {3, 20, 23, 6, 7, 9, 10, 11, 13, 14, 15, 16, 17, 22, 18, 21, 19, 29}
+    for t in g["tensors"]:
+        n = t["name"]
+        if not (".weight" in n and "token_embd" not in n and "output.weight" not in n and "_norm" not in n):
+            continue
+        ty = t["ggml_type"]
+        q8 += ty == 8 or ty in as_q8
+        q4 += ty == 2
+        q4k += ty == 12
+        f16 += ty in (1, 30)
+        f32 += ty == 0
+    total = q8 + q4 + q4k + f16 + f32
+    if total == 0:
+        return None
+    return 12 if q4k > total // 2 else 8 if q8 > total // 2 else 2 if q4 > total // 2 else None
+
+
+def proj_dtypes(g, fallback):
+    """The nine category formats {category: type id} (DENSE = 1 for F32 / F16 / BF16)."""
+    out = {}
+    for cat in _CATS:
+        counts = {}
+        for t in g["tensors"]:
+            if _category(t["name"]) == cat and _storage(t["ggml_type"]) is not None:
+                d = _storage(t["ggml_type"])
+                counts[d] = counts.get(d, 0) + 1
+        out[cat] = max(counts.items(), key=lambda kv: (kv[1], _RANK[kv[0]]))[0] if counts else fallback
+    if not any(_category(t["name"]) == "lm_head" for t in g["tensors"]):
+        out["lm_head"] = out["embed"]
+    return out
+
+
+def config_mixed(g, max_seq=0, flags=0):
+    """(config, [q, k, v, o, gate, up, down], embed) as forge_hip_gguf_config_mixed reports them."""
+    maj = _majority(g)
+    if maj is None:
+        raise GgufError("projection weights are neither mostly Q8_0, Q4_0 nor Q4_K")
+    # the shape part of load_config does not depend on the formats: take it from config() of a file voted Q8_0
+    shape_only = dict(g, tensors=[dict(t, ggml_type=8) for t in g["tensors"]])
+    cfg = config(shape_only, max_seq, flags)
+    cats = proj_dtypes(g, maj)
+    dense_as = 8 if maj == 12 else maj
+    fixed = {c: (dense_as if d == DENSE and c != "embed" else d) for c, d in cats.items()}
+    cfg["wdtype"] = maj if maj in (8, 2) else 8
+    cfg["lm_head_dtype"] = fixed["lm_head"]
+    return cfg, [fixed[c] for c in _CATS[1:8]], cats["embed"]
+
+
+def _round_away(x):
+    """f32::round: halves away from zero (exact: the fraction of an f32 is itself an f32)."""
+    a = np.abs(x)
+    fl = np.floor(a)
+    return np.copysign(fl + ((a - fl) >= F(0.5)), x).astype(F)
+
+
+def _seq_sum(v):
+    acc = np.zeros(v.shape[0], F)
+    for i in range(v.shape[1]):
+        acc = (acc + v[:, i]).astype(F)
+    return acc
+
+
+def _make_qkx2(x, nmax=15.0, rmin=-1.0, rdelta=0.1, nstep=20):
+    """make_qkx2_quants (weight_loader.rs:1666-1768) for S sub-blocks at once: x [S][32] -> scale [S], the_min [S], L [S][32]."""
+    x = np.ascontiguousarray(x, F)
+    nmax, rmin, rdelta = F(nmax), F(rmin), F(rdelta)
+    mn0, mx = x.min(axis=1), x.max(axis=1)
+    flat = mx == mn0
+    mn = np.minimum(mn0, F(0.0)).astype(F)
+    span = np.where(flat, F(1.0), mx - mn).astype(F)
+    iscale = (nmax / span).astype(F)
+    scale = (F(1.0) / iscale).astype(F)
+    L = np.clip(_round_away(((x - mn[:, None]) * iscale[:, None]).astype(F)), 0, nmax).astype(F)
+    diff = ((scale[:, None] * L).astype(F) + mn[:, None]).astype(F) - x
+    best_mad = _seq_sum((diff * diff).astype(F))
+    best_scale, best_min, best_L = scale.copy(), mn.copy(), L.copy()
+    nf = F(32.0)
+    with np.errstate(all="ignore"):
+        for step in range(nstep + 1):
+            num = F(F(rmin + F(rdelta * F(step))) + nmax)
+            itry = (num / span).astype(F)
+            la = np.clip(_round_away(((x - mn[:, None]) * itry[:, None]).astype(F)), 0, nmax).astype(F)
+            sum_l, sum_l2 = _seq_sum(la), _seq_sum((la * la).astype(F))
+            sum_x, sum_xl = _seq_sum(x), _seq_sum((la * x).astype(F))
+            det = ((nf * sum_l2).astype(F) - (sum_l * sum_l).astype(F)).astype(F)
+            ok = det > 0
+            sdet = np.where(ok, det, F(1.0))
+            ts = ((((nf * sum_xl).astype(F) - (sum_x * sum_l).astype(F)).astype(F)) / sdet).astype(F)
+            tm = ((((sum_l2 * sum_x).astype(F) - (sum_l * sum_xl).astype(F)).astype(F)) / sdet).astype(F)
+            pos = tm > 0
+            alt = (sum_xl / np.where(sum_l2 > 0, sum_l2, F(1.0))).astype(F)
+            ts = np.where(pos & (sum_l2 > 0), alt, ts).astype(F)
+            tm = np.where(pos, F(0.0), tm).astype(F)
+            ok &= ts > 0
+            d = ((ts[:, None] * la).astype(F) + tm[:, None]).astype(F) - x
+            mad = _seq_sum((d * d).astype(F))
+            better = ok & (mad < best_mad) & ~flat
+            best_L[better], best_mad[better], best_scale[better], best_min[better] = la[better], mad[better], ts[better], tm[better]
+    best_scale[flat], best_min[flat], best_L[flat] = 0.0, mn0[flat], 0.0
+    return best_scale, (-best_min).astype(F), best_L.astype(np.uint8)
+
+
+def quantize_q4_k(oracle, data):
+    """quantize_f32_to_q4_k, weight_loader.rs:1773-1882."""
+    data = np.ascontiguousarray(data, F).reshape(-1)
+    nsb = (data.size + 255) // 256
+    x = np.zeros(nsb * 256, F)
+    x[:data.size] = data
+    sc, mn, q = _make_qkx2(x.reshape(nsb * 8, 32))
+    sc, mn, q = sc.reshape(nsb, 8), mn.reshape(nsb, 8), q.reshape(nsb, 8, 32)
+    max_scale, max_min = np.maximum(sc.max(axis=1), F(0.0)), np.maximum(mn.max(axis=1), F(0.0))
+    with np.errstate(all="ignore"):
+        inv_scale = np.where(max_scale > 0, F(63.0) / max_scale, F(0.0)).astype(F)
+        inv_min = np.where(max_min > 0, F(63.0) / max_min, F(0.0)).astype(F)
+    d = np.where(max_scale > 0, max_scale / F(63.0), F(0.0)).astype(F)
+    dmin = np.where(max_min > 0, max_min / F(63.0), F(0.0)).astype(F)
+    sq = np.clip(_round_away((sc * inv_scale[:, None]).astype(F)), 0, 63).astype(np.uint8)
+    mq = np.clip(_round_away((mn * inv_min[:, None]).astype(F)), 0, 63).astype(np.uint8)
+    d_bits, dmin_bits = oracle.f32_to_f16(d), oracle.f32_to_f16(dmin)
+    d_st, dmin_st = oracle.f16_to_f32(d_bits).astype(F), oracle.f16_to_f32(dmin_bits).astype(F)
+    s_eff = (d_st[:, None] * sq.astype(F)).astype(F)
+    dm_eff = (dmin_st[:, None] * mq.astype(F)).astype(F)
+    with np.errstate(all="ignore"):
+        inv = (F(1.0) / np.where(s_eff == 0, F(1.0), s_eff)).astype(F)
+    xs = x.reshape(nsb, 8, 32)
+    codes = np.clip(_round_away(((xs + dm_eff[:, :, None]).astype(F) * inv[:, :, None]).astype(F)), 0, 15).astype(np.uint8)
+    codes[s_eff == 0] = 0
+    out = np.zeros((nsb, 144), np.uint8)
+    out[:, 0:2] = np.ascontiguousarray(d_bits, "<u2").view(np.uint8).reshape(nsb, 2)
+    out[:, 2:4] = np.ascontiguousarray(dmin_bits, "<u2").view(np.uint8).reshape(nsb, 2)
+    out[:, 4:8] = (sq[:, :4] & 63) | (((sq[:, 4:] >> 4) & 3) << 6)
+    out[:, 8:12] = (mq[:, :4] & 63) | (((mq[:, 4:] >> 4) & 3) << 6)
+    out[:, 12:16] = (sq[:, 4:] & 0x0F) | ((mq[:, 4:] & 0x0F) << 4)
+    out[:, 16:] = ((codes[:, 0::2] & 0x0F) | (codes[:, 1::2] << 4)).reshape(nsb, 128)
+    return out.reshape(-1)
+
+
+def quantize_q6_k(oracle, data):
+    """quantize_f32_to_q6_k, weight_loader.rs:2025-2140 (sub-block scale: make_q6k_quants :1987-2010)."""
+    data = np.ascontiguousarray(data, F).reshape(-1)
+    nsb = (data.size + 255) // 256
+    x = np.zeros(nsb * 256, F)
+    x[:data.size] = data
+    xs = x.reshape(nsb, 16, 16)
+    first = np.abs(xs).argmax(axis=2)                                  # the first element of largest magnitude
+    mx = np.take_along_axis(xs, first[:, :, None], axis=2)[:, :, 0]
+    zero = np.abs(mx) < F(1e-30)
+    with np.errstate(all="ignore"):
+        isc = (F(-32.0) / np.where(zero, F(1.0), mx)).astype(F)
+        sub = np.where(zero, F(0.0), (F(1.0) / isc).astype(F)).astype(F)
+    top = np.abs(sub).argmax(axis=1)
+    max_scale = sub[np.arange(nsb), top]
+    dead = np.abs(max_scale) < F(1e-30)
+    with np.errstate(all="ignore"):
+        sup_i = (F(-128.0) / np.where(dead, F(1.0), max_scale)).astype(F)
+        sup_d = (F(1.0) / sup_i).astype(F)
+    d_bits = oracle.f32_to_f16(sup_d)
+    sq = np.clip(_round_away((sup_i[:, None] * sub).astype(F)), -128, 127).astype(np.int8)
+    d_st = oracle.f16_to_f32(d_bits).astype(F)
+    s_eff = (d_st[:, None] * sq.astype(F)).astype(F)
+    with np.errstate(all="ignore"):
+        inv = (F(1.0) / np.where(s_eff == 0, F(1.0), s_eff)).astype(F)
+    L = np.clip(_round_away((inv[:, :, None] * xs).astype(F)), -32, 31).astype(np.int32)
+    L[s_eff == 0] = 0
+    q = (L.reshape(nsb, 2, 4, 32) + 32).astype(np.uint8)               # [block][half][quarter of 32][l]
+    out = np.zeros((nsb, 210), np.uint8)
+    ql = out[:, :128].reshape(nsb, 2, 64)
+    qh = out[:, 128:192].reshape(nsb, 2, 32)
+    ql[:, :, :32] = (q[:, :, 0] & 0x0F) | ((q[:, :, 2] & 0x0F) << 4)
+    ql[:, :, 32:] = (q[:, :, 1] & 0x0F) | ((q[:, :, 3] & 0x0F) << 4)
+    qh[:] = (q[:, :, 0] >> 4) | ((q[:, :, 1] >> 4) << 2) | ((q[:, :, 2] >> 4) << 4) | ((q[:, :, 3] >> 4) << 6)
+    out[:, 192:208] = sq.view(np.uint8)
+    out[:, 208:210] = np.ascontiguousarray(d_bits, "<u2").view(np.uint8).reshape(nsb, 2)
+    out[dead] = 0
+    return out.reshape(-1)
+
+
+def export_weights_mixed(oracle, g, data, cfg, pd) -> np.ndarray:
+    """The weights.bin bytes with each projection in its category's format."""
+    data = bytes(data)
+    by_name = {t["name"]: t for t in g["tensors"]}
+
+    def find(name, n):
+        t = by_name.get(name)
+        if t is None:
+            raise GgufError(f"weight not found: {name}")
+        if numel(t) != n:
+            raise GgufError(f"tensor {name} has the wrong number of elements")
+        return t
+
+    def raw(t):
+        return np.frombuffer(data, np.uint8, data_size(t), g["tensor_data_offset"] + t["offset"])
+
+    def f32(name, n):
+        return _tensor_f32(oracle, g, data, find(name, n)).astype("<f4").view(np.uint8)
+
+    def put(name, n, dt):
+        t = find(name, n)
+        if t["ggml_type"] == dt:
+            return raw(t)
+        if dt in (8, 2):
+            return oracle.quantize_weights(dt, _tensor_f32(oracle, g, data, t))
+        v = dequant_ggml(oracle, t["ggml_type"], raw(t), n)                  # directly: no Q8_0 stage for a K-quant target
+        return quantize_q4_k(oracle, v) if dt == 12 else quantize_q6_k(oracle, v)
+
+    H, I = cfg["hidden"], cfg["inter"]
+    QKS, KV, V = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"], cfg["vocab"]
+    emb = find("token_embd.weight", V * H)
+    if emb["ggml_type"] in (12, 14):
+        parts = [dequant_ggml(oracle, emb["ggml_type"], raw(emb), V * H).astype("<f4").view(np.uint8)]
+    else:
+        parts = [f32("token_embd.weight", V * H)]
+    for l in range(cfg["layers"]):
+        b = f"blk.{l}."
+        parts += [f32(b + "attn_norm.weight", H), put(b + "attn_q.weight", QKS * H, pd[0]), put(b + "attn_k.weight", KV * H, pd[1]),
+                  put(b + "attn_v.weight", KV * H, pd[2]), put(b + "attn_output.weight", H * QKS, pd[3]), f32(b + "ffn_norm.weight", H),
+                  put(b + "ffn_gate.weight", I * H, pd[4]), put(b + "ffn_up.weight", I * H, pd[5]), put(b + "ffn_down.weight", H * I, pd[6])]
+    parts.append(f32("output_norm.weight", H))
+    lm_name = "output.weight" if "output.weight" in by_name else "lm_head.weight" if "lm_head.weight" in by_name else "token_embd.weight"
+    parts.append(put(lm_name, V * H, cfg["lm_head_dtype"]))
+    return np.concatenate([np.ascontiguousarray(p, np.uint8) for p in parts])

@@ -712,3 +712,235 @@ def test_phi3_model_from_fused_gguf(fh, gg, oracle, torch_gpu, tmp_path):
     om = oracle.Model(dict(cfg, flags=fh.FLAG_EXACT), blob, 0, 1)
     assert np.array_equal(e.forward_prefill(prompt).view(np.uint32), om.prefill_batched(prompt).view(np.uint32))
     e.close(); om.close()
+
+
+# ---------------------------------------------------------------- a storage format per projection category
+def _xorshift(state):
+    def nxt():
+        s = nxt.s
+        s ^= (s << 13) & 0xFFFFFFFF
+        s ^= s >> 17
+        s ^= (s << 5) & 0xFFFFFFFF
+        nxt.s = s
+        return s
+    nxt.s = state
+    return nxt
+
+
+def _gauss_like_the_reference_tests(seed, n):
+    """Box-Muller over a 32-bit xorshift, sigma 0.05 (the inputs of weight_loader.rs:2783-2840, 2924-2966; numpy's cos / ln need
+    not round like Rust's: the bounds below hold for the distribution, not for particular bits)."""
+    nxt = _xorshift(seed)
+    out = []
+    while len(out) < n:
+        u1 = max(nxt() / 0xFFFFFFFF, 1e-7)
+        u2 = nxt() / 0xFFFFFFFF
+        r = np.sqrt(-2.0 * np.log(u1))
+        out += [0.05 * r * np.cos(2 * np.pi * u2), 0.05 * r * np.sin(2 * np.pi * u2)]
+    return np.asarray(out[:n], np.float32)
+
+
+KQ_INPUTS = {
+    "gauss": lambda: np.random.default_rng(1).normal(0, 0.05, 256 * 24).astype(np.float32),
+    "heavy_tail": lambda: (np.random.default_rng(2).standard_t(3, 256 * 16) * 0.02).astype(np.float32),
+    "ramp": lambda: ((np.arange(512) - 256.0) * 0.005).astype(np.float32),
+    "zeros": lambda: np.zeros(512, np.float32),
+    "flat_and_positive": lambda: np.concatenate([np.full(256, 0.25, np.float32), np.abs(np.random.default_rng(3).normal(0, 1, 256)).astype(np.float32),
+                                                 np.full(128, -1.5, np.float32), np.zeros(128, np.float32)]),
+    "ragged_tail": lambda: np.random.default_rng(4).normal(0, 1, 300).astype(np.float32),
+    "one_outlier": lambda: np.concatenate([np.random.default_rng(5).normal(0, 0.01, 255).astype(np.float32), np.float32([3.0])]),
+    "ties": lambda: np.tile(np.float32([-32, -31.5, -0.5, 0.5, 1.5, 2.5, 30.5, 31, 0, 0, 0, 0, 0, 0, 0, 0]), 16),
+}
+
+
+@pytest.mark.parametrize("ty", [12, 14])
+@pytest.mark.parametrize("name", list(KQ_INPUTS))
+def test_kquant_quantisers_library_equals_restatement(fh, gg, go, oracle, ty, name):
+    """The library's quantize_f32_to_q4_k / _q6_k (C++ loops) against the array-form restatement, byte for byte, and what the
+    format itself fixes: every code is the NEAREST one under the scales as stored (the refit step, weight_loader.rs:1826-1850,
+    2085-2100), checked through the fixture-pinned dequantisers."""
+    x = KQ_INPUTS[name]()
+    got = gg.quantize_kquant(ty, x)
+    want = (go.quantize_q4_k if ty == 12 else go.quantize_q6_k)(oracle, x)
+    assert got.size == (x.size + 255) // 256 * (144 if ty == 12 else 210)
+    assert np.array_equal(got, want)
+    n = (x.size + 255) // 256 * 256
+    xp = np.zeros(n, np.float32)
+    xp[:x.size] = x
+    back = gg.dequant_ggml(ty, got, n).astype(np.float64)
+    if ty == 14:
+        b = got.reshape(-1, 210)
+        d = oracle.f16_to_f32(b[:, 208:210].copy().view("<u2")[:, 0]).astype(np.float64)
+        step = np.abs(d[:, None] * b[:, 192:208].view(np.int8).astype(np.float64))           # [block][16 sub-blocks]
+        step = np.repeat(step, 16, axis=1).reshape(-1)
+        inside = (np.abs(xp) <= 31 * step)                       # codes -32 .. 31: beyond 31 steps a positive value is clamped
+        assert np.all(np.abs(back - xp)[inside] <= 0.5 * step[inside] * (1 + 1e-5) + 1e-12)
+    else:
+        b = got.reshape(-1, 144)
+        d = oracle.f16_to_f32(b[:, 0:2].copy().view("<u2")[:, 0]).astype(np.float64)
+        dmin = oracle.f16_to_f32(b[:, 2:4].copy().view("<u2")[:, 0]).astype(np.float64)
+        sc, mn = go._scale_min_k4(b[:, 4:16])                                                  # [block][8 sub-blocks]
+        step = np.repeat(d[:, None] * sc, 32, axis=1).reshape(-1)
+        low = -np.repeat(dmin[:, None] * mn, 32, axis=1).reshape(-1)                           # the value of code 0
+        inside = (xp >= low) & (xp <= low + 15 * step)
+        assert np.all(np.abs(back - xp)[inside] <= 0.5 * step[inside] * (1 + 1e-5) + 1e-12)
+        assert inside.mean() > 0.9 or name not in ("gauss", "heavy_tail", "ramp")      # the check must bite where it can
+
+
+def test_kquant_quantisers_meet_the_reference_tests_bounds(fh, gg, oracle):
+    """The reference's own unit tests for the two quantisers (weight_loader.rs:2735-2990), on their inputs."""
+    ramp = ((np.arange(512) - 256.0) * 0.005).astype(np.float32)
+    q = gg.quantize_kquant(12, ramp)
+    assert q.size == 2 * 144 and np.abs(gg.dequant_ggml(12, q, 512) - ramp).max() < 0.05                     # :2735-2755
+    q = gg.quantize_kquant(14, ramp)
+    assert q.size == 2 * 210 and np.abs(gg.dequant_ggml(14, q, 512) - ramp).max() < 0.02                     # :2906-2921
+    state, vals = 0xDEADBEEF, []
+    for _ in range(512):                                                                                      # :2758-2780
+        state = (state * 1664525 + 1013904223) & 0xFFFFFFFF
+        vals.append((np.float32(state >> 16) / np.float32(65535) - np.float32(0.5)) * np.float32(0.2))
+    v = np.asarray(vals, np.float32)
+    e = gg.dequant_ggml(12, gg.quantize_kquant(12, v), 512).astype(np.float64) - v
+    assert np.sqrt(np.mean(e * e)) < 0.005
+    for ty, seed in ((12, 0x13579BDF), (14, 0xFEEDBABE)):                                                     # :2783-2840, :2924-2966
+        v = _gauss_like_the_reference_tests(seed, 4096)
+        e = gg.dequant_ggml(ty, gg.quantize_kquant(ty, v), 4096).astype(np.float64) - v
+        assert abs(e.mean()) < 5 * np.sqrt(np.mean(e * e)) / np.sqrt(4096)
+    nxt = _xorshift(0xACEDF00D)                                                                               # :2844-2892
+    vals = []
+    for i in range(8192):
+        u1 = max(nxt() / 0xFFFFFFFF * 0.99, 1e-6)
+        u2 = max(nxt() / 0xFFFFFFFF, 1e-6)
+        z = np.sqrt(-2 * np.log(u1)) * np.cos(2 * np.pi * u2)
+        vals.append(0.3 * np.sign(z) if i % 200 == 0 else 0.05 * z)
+    v = np.asarray(vals, np.float32)
+    e = gg.dequant_ggml(12, gg.quantize_kquant(12, v), 8192).astype(np.float64) - v
+    assert abs(e.mean()) < 5 * np.sqrt(np.mean(e * e)) / np.sqrt(8192)
+    for ty in (12, 14):                                                                                       # :2895-2903, :2969-2976
+        assert np.abs(gg.dequant_ggml(ty, gg.quantize_kquant(ty, np.zeros(256, np.float32)), 256)).max() < 1e-3
+    with pytest.raises(fh.ForgeHipError):
+        gg.quantize_kquant(13, np.zeros(256, np.float32))
+
+
+def _kquant_file(fh, gg, recipe, seed=31, layers=4, tied=False, embed_ty=12, lm_ty=14, extra=None):
+    """A llama-architecture GGUF file of a small random model whose tensors are stored by `recipe(layer, suffix) -> type id`
+    (12 = Q4_K, 14 = Q6_K, 8, 2); returns (bytes, {name: (type, raw bytes)}, shape dict)."""
+    shape = dict(hidden=256, inter=512, layers=layers, heads=4, kv_heads=2, head_dim=64, vocab=512)
+    H, I, V = shape["hidden"], shape["inter"], shape["vocab"]
+    QKS, KV = 256, 128
+    rng = np.random.default_rng(seed)
+
+    def store(ty, n_rows, k):
+        w = rng.normal(0, 0.05, n_rows * k).astype(np.float32)
+        if ty in (12, 14):
+            return gg.quantize_kquant(ty, w)
+        if ty == 13:
+            return random_blocks(13, n_rows * k // 256, int(rng.integers(1 << 30)))
+        return fh.ops.quantize_weights(ty, w)
+
+    t = {"token_embd.weight": ([H, V], embed_ty, store(embed_ty, V, H))}
+    for l in range(layers):
+        t[f"blk.{l}.attn_norm.weight"] = ([H], gg.F32, (1 + 0.1 * rng.normal(0, 1, H)).astype(np.float32).view(np.uint8))
+        t[f"blk.{l}.ffn_norm.weight"] = ([H], gg.F32, (1 + 0.1 * rng.normal(0, 1, H)).astype(np.float32).view(np.uint8))
+        for suffix, n_rows, k in (("attn_q", QKS, H), ("attn_k", KV, H), ("attn_v", KV, H), ("attn_output", H, QKS), ("ffn_gate", I, H),
+                                  ("ffn_up", I, H), ("ffn_down", H, I)):
+            ty = recipe(l, suffix)
+            t[f"blk.{l}.{suffix}.weight"] = ([k, n_rows], ty, store(ty, n_rows, k))
+    t["output_norm.weight"] = ([H], gg.F32, (1 + 0.1 * rng.normal(0, 1, H)).astype(np.float32).view(np.uint8))
+    if not tied:
+        t["output.weight"] = ([H, V], lm_ty, store(lm_ty, V, H))
+    meta = [("general.architecture", gg.STRING, "llama"), ("llama.embedding_length", gg.U32, H), ("llama.block_count", gg.U32, layers),
+            ("llama.attention.head_count", gg.U32, 4), ("llama.attention.head_count_kv", gg.U32, 2), ("llama.feed_forward_length", gg.U32, I),
+            ("llama.vocab_size", gg.U32, V), ("llama.context_length", gg.U32, 640), ("llama.attention.layer_norm_rms_epsilon", gg.FLOAT32, 1e-5),
+            ("llama.rope.freq_base", gg.FLOAT32, 10000.0)] + list(extra or [])
+    data = gg.write_gguf(meta, [(n, d, g, b) for n, (d, g, b) in t.items()])
+    return data, {n: (g, np.ascontiguousarray(b, np.uint8).reshape(-1)) for n, (d, g, b) in t.items()}, shape
+
+
+def _q4_k_m(l, suffix):
+    """llama.cpp's Q4_K_M over four layers: attn_v and ffn_down are Q6_K in half of the layers, everything else Q4_K."""
+    return 14 if suffix in ("attn_v", "ffn_down") and l in (0, 3) else 12
+
+
+def test_q4_k_m_file_keeps_a_format_per_category(fh, gg, go, oracle):
+    data, raw, shape = _kquant_file(fh, gg, _q4_k_m)
+    f, o = gg.GgufFile(data), go.parse(data)
+    with pytest.raises(fh.ForgeHipError):
+        f.config()                                                     # no Q8_0 / Q4_0 majority: the uniform rules do not apply
+    cfg, pd, embed = f.config_mixed()
+    # v and down: two Q4_K against two Q6_K tensors, the tie goes to the more precise format (main.rs:626-640)
+    assert pd == [12, 12, 14, 12, 12, 12, 14] and cfg["lm_head_dtype"] == 14 and embed == 12
+    assert (cfg, pd, embed) == go.config_mixed(o)
+    assert {k: cfg[k] for k in shape} == shape
+    blob = f.export_weights_mixed(cfg, pd)
+    assert np.array_equal(blob, go.export_weights_mixed(oracle, o, data, cfg, pd))
+    H, V = 256, 512
+    # the f32 table is the Q4_K table dequantised directly; tensors already in their category's format are the file's bytes
+    assert np.array_equal(blob[:V * H * 4].view(np.float32), gg.dequant_ggml(12, raw["token_embd.weight"][1], V * H))
+    at = V * H * 4 + H * 4
+    assert np.array_equal(blob[at:at + raw["blk.0.attn_q.weight"][1].size], raw["blk.0.attn_q.weight"][1])
+    assert np.array_equal(blob[-raw["output.weight"][1].size:], raw["output.weight"][1])
+    # layer 1's attn_v is Q4_K in a Q6_K category: dequantised and quantised again (weight_loader.rs:208-218)
+    per_layer = (blob.size - V * H * 4 - H * 4 - raw["output.weight"][1].size) // 4
+    v_at = V * H * 4 + per_layer + H * 4 + 256 * 144 + 128 * 144
+    want = gg.quantize_kquant(14, gg.dequant_ggml(12, raw["blk.1.attn_v.weight"][1], 128 * 256))
+    assert np.array_equal(blob[v_at:v_at + want.size], want)
+
+
+def test_category_rules_on_other_files(fh, gg, go, oracle):
+    # a Q4_0 file whose output matrix is Q6_K (llama.cpp's default): Q4_0 projections under a Q6_K lm_head
+    data, raw, _ = _kquant_file(fh, gg, lambda l, s: 2, embed_ty=2, lm_ty=14, layers=2)
+    f, o = gg.GgufFile(data), go.parse(data)
+    cfg, pd, embed = f.config_mixed()
+    assert pd == [2] * 7 and (cfg["wdtype"], cfg["lm_head_dtype"], embed) == (2, 14, 2) and (cfg, pd, embed) == go.config_mixed(o)
+    assert np.array_equal(f.export_weights_mixed(cfg, pd), go.export_weights_mixed(oracle, o, data, cfg, pd))
+    # tied embeddings stored as Q6_K: the lm_head takes the embedding's format and bytes (main.rs:668-678, 2632-2676)
+    data, raw, _ = _kquant_file(fh, gg, lambda l, s: 12, embed_ty=14, tied=True, layers=2)
+    f, o = gg.GgufFile(data), go.parse(data)
+    cfg, pd, embed = f.config_mixed()
+    assert pd == [12] * 7 and (cfg["lm_head_dtype"], embed) == (14, 14) and (cfg, pd, embed) == go.config_mixed(o)
+    blob = f.export_weights_mixed(cfg, pd)
+    assert np.array_equal(blob, go.export_weights_mixed(oracle, o, data, cfg, pd))
+    assert np.array_equal(blob[-raw["token_embd.weight"][1].size:], raw["token_embd.weight"][1])
+    # a category whose tensors are all Q5_K has no vote and takes the file's majority format; its tensors are converted
+    data, raw, _ = _kquant_file(fh, gg, lambda l, s: 13 if s == "ffn_up" else 12, layers=2)
+    f, o = gg.GgufFile(data), go.parse(data)
+    cfg, pd, embed = f.config_mixed()
+    assert pd == [12] * 7 and (cfg, pd, embed) == go.config_mixed(o)
+    blob = f.export_weights_mixed(cfg, pd)
+    assert np.array_equal(blob, go.export_weights_mixed(oracle, o, data, cfg, pd))
+    # a uniform Q8_0 file reports seven times Q8_0: forge_hip_model_create_from_gguf then takes the uniform rules
+    cfg8 = fh.synth.tiny(Q8, max_seq=640)
+    data = gg.model_to_gguf(cfg8, fh.synth.make_weights_blob(cfg8, seed=2), tied=True)
+    cfg, pd, embed = gg.GgufFile(data).config_mixed()
+    assert pd == [8] * 7 and cfg["lm_head_dtype"] == 8 and embed == 8
+    # refusals: wrong buffer size, an unknown format
+    f = gg.GgufFile(_kquant_file(fh, gg, _q4_k_m)[0])
+    cfg, pd, _ = f.config_mixed()
+    with pytest.raises(fh.ForgeHipError):
+        f.export_weights_mixed(cfg, [13] + pd[1:])
+
+
+@pytest.mark.gpu
+def test_q4_k_m_model_from_gguf_matches_the_oracle(fh, gg, go, oracle, torch_gpu, tmp_path):
+    """forge_hip_model_create_from_gguf on a Q4_K_M-style file, order-faithful mode: prompt logits, cache rows and 12 greedy
+    steps bit for bit those of the CPU oracle run on the oracle's own export of the same file."""
+    data, _, _ = _kquant_file(fh, gg, _q4_k_m)
+    path = str(tmp_path / "q4km.gguf")
+    with open(path, "wb") as fp:
+        fp.write(data)
+    o = go.parse(data)
+    cfg, pd, _ = go.config_mixed(o, flags=fh.FLAG_EXACT)
+    blob = go.export_weights_mixed(oracle, o, data, cfg, pd)
+    gm = fh.HipModel.from_gguf(path, flags=fh.FLAG_EXACT)
+    assert gm.proj_dtypes == pd and gm.config["lm_head_dtype"] == 14 and gm.decode_launches > 1
+    om = oracle.Model(cfg, blob, 0, 1, proj_dtypes=pd)
+    prompt = fh.synth.uniform_ids(8, 24, cfg["vocab"])
+    gl, ol = gm.forward_prefill(prompt), om.prefill_batched(prompt)
+    assert np.array_equal(gl.view(np.uint32), ol.view(np.uint32))
+    tok = oracle.argmax(ol)
+    for _ in range(12):
+        g, w = gm.forward(tok), om.forward(tok)
+        assert np.array_equal(g.view(np.uint32), w.view(np.uint32))
+        tok = oracle.argmax(w)
+    assert np.array_equal(oracle.f16_to_f32(gm.read_kv(3, 1)), om.read_kv(3, 1))
+    gm.close()
