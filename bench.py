@@ -205,6 +205,22 @@ def exact_mode_figures(fh, cfg, blob, prompt, warmup, steps, fast_tokens, fast_l
     if first is not None:
         top2 = np.partition(lg[first], -2)[-2:]
         out["fast_vs_exact"]["exact_top2_margin_at_divergence"] = float(top2[1] - top2[0])
+    # the same mode with the whole step as one resident kernel (ordered row sums, attention walked in the reference's
+    # 64-key blocks): bit-identical to the kernel sequence, measured beside it; the library's default is the sequence
+    if cfg.get("sliding_window", 0) == 0:
+        import os
+        os.environ["FORGE_HIP_PD_EXACT"] = "1"
+        try:
+            m = fh.HipModel(dict(cfg, flags=cfg.get("flags", 0) | fh.FLAG_EXACT), blob)
+            if m.decode_launches < launches:
+                m.forward_prefill_batch(prompt)
+                t1, _ = timed_decode(m, fh.ops.argmax_host(logits), warmup, steps)
+                one_toks, _ = greedy_with_logits(fh, m, prompt, min(16, len(toks)))
+                out["one_resident_kernel"] = {"decode_tok_per_s": steps / t1, "ms_per_step": t1 / steps * 1e3, "launches_per_token": m.decode_launches,
+                                              "tokens_identical_to_kernel_sequence": one_toks == toks[:len(one_toks)], "selected_by": "FORGE_HIP_PD_EXACT=1"}
+            m.close()
+        finally:
+            del os.environ["FORGE_HIP_PD_EXACT"]
     return out
 
 

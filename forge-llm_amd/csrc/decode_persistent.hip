@@ -115,6 +115,9 @@ struct PdArgs {
     uint64_t* taq;     // [QKS/4 + QKS/32]  attention output, int8 codes (4 per element) then fp16 scales
     uint64_t* taq2;    // [I/4 + I/32]      silu(gate)*up, same format
     uint64_t* tpart;   // [2 G]          per-workgroup argmax candidates
+    uint64_t* tbm;     // [heads][nb_cap]          order-faithful attention: block maxima
+    uint64_t* trec;    // [heads][nb_cap][hd + 2]  order-faithful attention: per block sum[d], then m_i, l_block
+    uint32_t exact_attn, nb_cap;               // exact_attn: attention in the reference's own order (ordered kernel variants only)
     float* logits;
     uint32_t* state;   // [0] position  [1] token  [2] next token  [3] abort flag
     uint32_t tag_base, spin_limit;
@@ -389,6 +392,14 @@ struct GemvJob {
 struct WReg { int4 v[PD_D]; uint32_t s[PD_D]; };
 
 __device__ __forceinline__ uint32_t sgpr(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+
+// Tells the register allocator that a weight register set holds nothing from here on (no instruction is emitted): whether a
+// phase finds its first round already loaded is a run-time flag, so without this the set stays reserved through code that
+// runs only when it is empty (the attention phases).
+__device__ __forceinline__ void pd_forget(WReg& W) {
+#pragma unroll
+    for (int d = 0; d < PD_D; d++) asm volatile("" : "=v"(W.v[d].x), "=v"(W.v[d].y), "=v"(W.v[d].z), "=v"(W.v[d].w), "=v"(W.s[d]));
+}
 
 // The scalar fields of a shape, read once per phase into scalar registers.
 struct Shape { uint32_t K, N, nblk, U, T, ntiles, inter, umagic; };
@@ -800,6 +811,216 @@ __device__ __forceinline__ void pd_attn_combine(const PdArgs& a, uint32_t tag_in
     }
 }
 
+// ---- attention in the reference's order (attention_flash, emit.rs:656-715) ---------------------------------
+// The reference walks the keys in blocks of 64; per block: scores (sequential q.k sums), the block maximum, the running
+// maximum m_i, exp(s - m_i), the sequential sums l_block and sum[d], and the recurrence
+//     l_i = l_i * exp_scale + l_block,   acc[d] = acc[d] * exp_scale + sum[d],   exp_scale = exp(m_prev - m_i)
+// which is the only part that ties the blocks together; m_i is a prefix maximum of the block maxima (order-free).  So a
+// (block, head) pair is a work item of ONE WAVE here: lane = key for the scores, lane = head dim for sum[d], the weights
+// and q broadcast from registers (v_readlane), no LDS.  A wave first computes the scores of all its items and publishes
+// their maxima, then, per item, reads the maxima of the blocks before it, forms the weights and publishes the block's
+// record; one workgroup per head then runs the recurrence over the records and quantises the row for the O projection.
+// Every f32 operation has the operands and the order it has in attn_exact.hip's kernels (and in the reference).
+constexpr uint32_t PX_B = 64;        // FLASH_ATTN_BLOCK_SIZE, emit.rs:201
+constexpr uint32_t PX_CHUNK = 64;    // block records the recurrence takes into LDS at a time
+constexpr uint32_t PX_MAX_BLOCKS = 4096;
+
+// What the two stages need of the kernel arguments.
+struct PxArgs {
+    const uint64_t* tq;
+    const uint64_t* tkv;
+    uint64_t* tbm;
+    uint64_t* trec;
+    uint64_t* taq;
+    uint32_t nb_cap, heads, kv_heads, KV, QKS;
+};
+__device__ __forceinline__ PxArgs px_args(const PdArgs& a) {
+    return PxArgs{a.tq, a.tkv, a.tbm, a.trec, a.taq, a.nb_cap, a.heads, a.kv_heads, a.KV, a.QKS};
+}
+
+template <int HD>
+__device__ __forceinline__ void pd_attn_exact_blocks(const PxArgs& a, const uint16_t* kc, const uint16_t* vc, uint32_t pos, uint32_t tag_in,
+                                                     uint32_t tag_out, const PdCtx& cx) {
+    constexpr int REC = HD + 2;
+    constexpr int NQ = (HD + 63) / 64;            // registers per lane of a head-sized vector spread over the wave
+    constexpr int VB = 64 / NQ;                   // keys whose V elements a lane requests together (64 registers)
+    const uint32_t lane = cx.lane;
+    const uint32_t seq = pos + 1, nb = (seq + PX_B - 1) / PX_B, n_items = nb * a.heads;
+    const uint32_t gsize = a.heads / a.kv_heads, kv_stride = a.KV;
+    const float scale = 1.0f / sqrtf((float)HD);
+    const uint32_t slots = cx.G * PD_WAVES;
+    // Items in block-major order, item = block * heads + head, one per wave and pass.  What an item waits for (the maxima
+    // of the earlier blocks of its head) belongs to items of a lower number, which their waves reach in the same or an
+    // earlier pass; the score stage of a pass waits for nothing but q, so every pass completes.
+#pragma nounroll
+    for (uint32_t item = sgpr(cx.wg + cx.G * cx.wave); item < n_items; item += slots) {
+        const uint32_t b = item / a.heads, h = item - b * a.heads, kvh = h / gsize;
+        const uint32_t bs = b * PX_B, bl = min(PX_B, seq - bs), t = bs + lane;
+        const bool has_new = b == nb - 1;                    // the block that holds this position
+        // the key's row and the first V elements do not depend on q: requested first (loads return in order)
+        uint4 kr[HD / 8];
+#pragma unroll
+        for (int c = 0; c < HD / 8; c++) kr[c] = make_uint4(0, 0, 0, 0);
+        if (lane < bl && t != pos) {
+            const uint16_t* krow = kc + (size_t)t * kv_stride + kvh * HD;
+#pragma unroll
+            for (int c = 0; c < HD / 8; c++) kr[c] = ldg(reinterpret_cast<const uint4*>(krow + c * 8));
+        }
+        const uint16_t* vcol = vc + (size_t)bs * kv_stride + kvh * HD + lane;
+        uint16_t vv[VB][NQ];
+        auto load_v = [&](uint32_t k0) {
+#pragma unroll
+            for (int u = 0; u < VB; u++)
+#pragma unroll
+                for (int j = 0; j < NQ; j++) {
+                    const uint32_t bi = k0 + (uint32_t)u;
+                    vv[u][j] = 0;
+                    if (bi < bl && bs + bi != pos && lane + 64u * (uint32_t)j < (uint32_t)HD) vv[u][j] = ldg(vcol + (size_t)bi * kv_stride + 64 * j);
+                }
+        };
+        // (heads of more than 64 dims: the key row alone takes 48-64 registers, the V elements are requested after the scores)
+        if (NQ == 1) load_v(0);
+        // q of this head, and with the last block this position's K and V rows: one round trip; a lane without an
+        // element of its own re-reads its first one
+        uint32_t got[3 * NQ];
+        {
+            const uint64_t* pq = a.tq + (size_t)h * HD;
+            const uint64_t* pk = a.tkv + kvh * HD;
+            const uint64_t* pv = a.tkv + a.KV + kvh * HD;
+            auto addr = [&](int i) -> const uint64_t* {
+                const int j = i % NQ;
+                const uint32_t e = lane + 64u * (uint32_t)j < (uint32_t)HD ? lane + 64u * (uint32_t)j : lane % 32u;
+                return (i < NQ || !has_new) ? pq + e : (i < 2 * NQ ? pk + e : pv + e);
+            };
+            poll_many<3 * NQ>(addr, 3 * NQ, tag_in, got, cx, Hint{nullptr, nullptr});
+        }
+        // ---- scores (sequential q.k sums, lane = key) and the block maximum
+        float sum = 0.f;
+        const bool mine_new = has_new && t == pos;
+#pragma unroll
+        for (int i = 0; i < HD; i++) {
+            const float qi = __int_as_float(__builtin_amdgcn_readlane((int)got[i / 64], i % 64));
+            const uint4 w4 = kr[i / 8];
+            const uint32_t w = (i % 8) / 2 == 0 ? w4.x : (i % 8) / 2 == 1 ? w4.y : (i % 8) / 2 == 2 ? w4.z : w4.w;
+            uint32_t kb = (i & 1) ? w >> 16 : w & 0xFFFFu;
+            if (has_new) {
+                const uint32_t kn = (uint32_t)__builtin_amdgcn_readlane((int)got[NQ + i / 64], i % 64);
+                kb = mine_new ? kn & 0xFFFFu : kb;
+            }
+            sum = sum + qi * f16_bits_to_f32((uint16_t)kb);
+        }
+        if (NQ != 1) load_v(0);
+        const float sc = lane < bl ? sum * scale : -INFINITY;
+        const float mb = wave_max(sc);
+        if (lane == 0) stc64(a.tbm + (size_t)h * a.nb_cap + b, tag_out, __float_as_uint(mb));
+        // ---- m_i after this block: the largest block maximum so far (`if m_block > m_i { m_i = m_block }` from -inf on)
+        float m = mb;
+        for (uint32_t j0 = 0; j0 < b; j0 += 128) {
+            uint32_t v[2];
+            poll_many<2>([&](int i) { return a.tbm + (size_t)h * a.nb_cap + min(j0 + lane + 64u * (uint32_t)i, b - 1); }, 2, tag_out, v, cx,
+                         Hint{nullptr, nullptr});
+            m = fmaxf(m, fmaxf(__uint_as_float(v[0]), __uint_as_float(v[1])));
+        }
+        m = wave_max(m);
+        // ---- weights, l_block and sum[d] (sequential over the block's keys; lane = head dim)
+        const float e = lane < bl ? expf_ref<true>(sc - m) : 0.f;
+        float l_block = 0.f, acc[NQ];
+#pragma unroll
+        for (int j = 0; j < NQ; j++) acc[j] = 0.f;
+#pragma nounroll
+        for (uint32_t k0 = 0; k0 < bl; k0 += VB) {
+            if (k0) load_v(k0);
+#pragma unroll
+            for (int u = 0; u < VB; u++) {
+                const uint32_t bi = k0 + (uint32_t)u;
+                if (bi < bl) {                                  // wave-uniform
+                    const float eb = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(e), (int)bi));
+                    l_block = l_block + eb;
+#pragma unroll
+                    for (int j = 0; j < NQ; j++) {
+                        const uint16_t hb = bs + bi == pos ? (uint16_t)got[2 * NQ + j] : vv[u][j];
+                        acc[j] = acc[j] + eb * f16_bits_to_f32(hb);
+                    }
+                }
+            }
+        }
+        uint64_t* rec = a.trec + ((size_t)h * a.nb_cap + b) * REC;
+#pragma unroll
+        for (int j = 0; j < NQ; j++)
+            if (lane + 64u * (uint32_t)j < (uint32_t)HD) stc64(rec + lane + 64 * j, tag_out, __float_as_uint(acc[j]));
+        if (lane == 0) { stc64(rec + HD, tag_out, __float_as_uint(m)); stc64(rec + HD + 1, tag_out, __float_as_uint(l_block)); }
+    }
+}
+
+// The recurrence over a head's block records (one head per workgroup at a time), the division by l_i and the quantised row
+// for the O projection (attn_exact_decode_chain_kernel's arithmetic).
+template <int HD>
+__device__ __forceinline__ void pd_attn_exact_chain(const PxArgs& a, uint32_t pos, uint32_t tag_in, uint32_t tag_out, float* misc, float* big,
+                                                    const PdCtx& cx) {
+    constexpr int REC = HD + 2;
+    const uint32_t tid = cx.tid;
+    const uint32_t nb = (pos + PX_B) / PX_B;
+    float* es = misc + PD_MISC_SCRATCH;          // [PX_CHUNK] exp_scale of the chunk's blocks
+    float* recs = big;                           // [PX_CHUNK][REC]
+    __syncthreads();                             // the GEMV phase before may still be summing rows out of `big`
+    for (uint32_t h = cx.wg; h < a.heads; h += cx.G) {
+        float l_i = 0.f, acc = 0.f, m_prev = -INFINITY;
+        for (uint32_t c0 = 0; c0 < nb; c0 += PX_CHUNK) {
+            const uint32_t n = min(PX_CHUNK, nb - c0);
+            const uint64_t* base = a.trec + ((size_t)h * a.nb_cap + c0) * REC;
+            poll_vec<(PX_CHUNK * REC + PD_THREADS - 1) / PD_THREADS>(base, n * REC, tag_in, PD_THREADS, cx, Hint{nullptr, nullptr},
+                        [&](uint32_t i, uint32_t p) { recs[i] = __uint_as_float(p); });
+            __syncthreads();
+            if (*cx.sh_abort) return;
+            // exp_scale = exp(m_prev - m_i), m_prev = -inf before the first block
+            if (tid < n) es[tid] = expf_ref<true>((tid ? recs[(tid - 1) * REC + HD] : m_prev) - recs[tid * REC + HD]);
+            m_prev = recs[(n - 1) * REC + HD];
+            __syncthreads();
+            if (tid < HD) {
+                // the four operations of a block form two dependent chains; the operands of the next eight blocks are read
+                // from LDS while the current eight are worked through
+                auto step = [&](float exp_scale, float lb, float sd) {
+                    l_i = l_i * exp_scale;
+                    acc = acc * exp_scale;
+                    l_i = l_i + lb;
+                    acc = acc + sd;
+                };
+                uint32_t i = 0;
+                if (n >= 8) {
+                    float e0[8], b0[8], s0[8], e1[8], b1[8], s1[8];
+#pragma unroll
+                    for (int k = 0; k < 8; k++) { e0[k] = es[k]; b0[k] = recs[k * REC + HD + 1]; s0[k] = recs[k * REC + tid]; }
+                    for (i = 8; i + 8 <= n; i += 8) {
+#pragma unroll
+                        for (int k = 0; k < 8; k++) { e1[k] = es[i + k]; b1[k] = recs[(i + k) * REC + HD + 1]; s1[k] = recs[(i + k) * REC + tid]; }
+#pragma unroll
+                        for (int k = 0; k < 8; k++) step(e0[k], b0[k], s0[k]);
+#pragma unroll
+                        for (int k = 0; k < 8; k++) { e0[k] = e1[k]; b0[k] = b1[k]; s0[k] = s1[k]; }
+                    }
+#pragma unroll
+                    for (int k = 0; k < 8; k++) step(e0[k], b0[k], s0[k]);
+                }
+                for (; i < n; i++) step(es[i], recs[i * REC + HD + 1], recs[i * REC + tid]);
+            }
+            __syncthreads();
+        }
+        if (tid < HD) {
+            const float inv_l = 1.0f / l_i;
+            const float o = acc * inv_l;
+            const float amax = half_wave_max(fabsf(o));
+            float inv;
+            const float scq = act_scale(amax, inv);
+            const uint32_t code = (uint32_t)quant_code(o * inv) & 0xFFu;
+            const uint32_t pk = quad_broadcast<0>(code) | (quad_broadcast<1>(code) << 8) | (quad_broadcast<2>(code) << 16) |
+                                (quad_broadcast<3>(code) << 24);
+            const uint32_t e = h * HD + tid;
+            if ((tid & 3u) == 0) stc64(a.taq + e / 4, tag_out, pk);
+            if ((tid & 31u) == 0) stc64(a.taq + a.QKS / 4 + e / 32, tag_out, f32_to_f16_bits(scq));
+        }
+    }
+}
+
 // ---- argmax (project.rs:501-503): the LAST index among equal maxima --------------------------------------
 struct ArgPair { float v; uint32_t i; };
 __device__ __forceinline__ ArgPair arg_better(ArgPair a, ArgPair b) {
@@ -1033,11 +1254,21 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         const uint32_t x_in = lg ? base : 0;                 // tag of x entering the layer (0: still the embedding row)
         if (ph == 1) {
             if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * lg + 1] = wall_clock64();
-            pd_attn_split<HD>(a, a.layers[l].kc, a.layers[l].vc, pos, base + 1, base + 2, big, pts, cx);
-            if (sh_abort) return;
-            if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * lg + 2] = wall_clock64();
-            pd_attn_combine<HD>(a, base + 2, base + 3, misc, big, cx);
-            if (sh_abort) return;
+            if (ORD && a.exact_attn) {
+                pd_attn_exact_blocks<HD>(px_args(a), a.layers[l].kc, a.layers[l].vc, pos, base + 1, base + 2, cx);
+                if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * lg + 2] = wall_clock64();
+                pd_attn_exact_chain<HD>(px_args(a), pos, base + 2, base + 3, misc, big, cx);
+                __syncthreads();
+                if (sh_abort) return;
+            } else {
+                pd_attn_split<HD>(a, a.layers[l].kc, a.layers[l].vc, pos, base + 1, base + 2, big, pts, cx);
+                if (sh_abort) return;
+                if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * lg + 2] = wall_clock64();
+                pd_attn_combine<HD>(a, base + 2, base + 3, misc, big, cx);
+                if (sh_abort) return;
+            }
+            pd_forget(W);          // the O projection loads its first round itself (`early` is false here)
+            pd_forget(W1);
         }
         if (a.stamps && cx.wg == 0 && cx.tid == 0) {
             static const int slot[5] = {0, 3, 4, 5, 6};
@@ -1207,7 +1438,16 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
                   const float* final_norm, const float* cos_t, const float* sin_t, float* logits, uint32_t* state, uint32_t* counts,
                   const float* qkv_bias, PdState** out) {
     *out = nullptr;
-    if (c.flags & FORGE_HIP_FLAG_EXACT) return FORGE_HIP_OK;
+    // The order-faithful mode can run as this kernel too: the ordered variant with the attention phases in the reference's
+    // order.  It is bit-identical to the kernel sequence but not faster (Llama-3.2-1B shape at 2.5k context: 954 against
+    // 940 us per token; 3B: 2199 against 2115; SmolLM2-135M: 1215 against 996 -- the ordered row sums cost every GEMV
+    // phase 2-4 us that the separate kernels hide behind their launches), so the sequence stays the default and
+    // FORGE_HIP_PD_EXACT=1 asks for the kernel.  A window (attention_sliding: another algorithm) and caches of more than
+    // 4096 blocks always keep the sequence.
+    const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
+    const uint32_t nb_cap = (c.max_seq + PX_B - 1) / PX_B;
+    if (exact && (c.sliding_window != 0 || nb_cap > PX_MAX_BLOCKS)) return FORGE_HIP_OK;
+    { const char* e = getenv("FORGE_HIP_PD_EXACT"); if (exact && !(e && e[0] == '1')) return FORGE_HIP_OK; }
     if (c.head_dim != 64 && c.head_dim != 96 && c.head_dim != 128) return FORGE_HIP_OK;
     int dev = 0, coop = 0, cus = 0, khz = 0;
     FH_HIP(hipGetDevice(&dev));
@@ -1229,7 +1469,9 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     st->lmq4 = c.lm_head_dtype == FORGE_HIP_Q4_0;
     st->wall_khz = khz;
     // FORGE_HIP_PD_ORDERED=1: GEMV rows summed in the reference's block order, bit-identical to the kernel sequence
-    { const char* e = getenv("FORGE_HIP_PD_ORDERED"); st->ordered = e && e[0] == '1'; }
+    { const char* e = getenv("FORGE_HIP_PD_ORDERED"); st->ordered = exact || (e && e[0] == '1'); }
+    a.exact_attn = exact ? 1u : 0u;
+    a.nb_cap = nb_cap;
 
     // LDS: activation codes | activation scales | misc | big
     a.off_act_s = round_up(kmax, 16);
@@ -1239,6 +1481,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     const uint32_t big = PD_LDS_BYTES - 64 - a.off_big;
     const uint32_t attn_bytes = (a.gt == 1 ? 2 : 1) * (16 * (hd + 2) + 6 * hd) * 4;      // two items at a time when a group has one head
     if ((H + 32) * 4 > big || attn_bytes > big || DECODE_SPLITS * (hd + 2) * 4 > big) return FORGE_HIP_OK;
+    if (exact && (PX_CHUNK * (hd + 2) * 4 > big || c.heads > st->grid * PD_WAVES)) return FORGE_HIP_OK;
     st->lds = a.off_big + big;
 
     if (layers.empty() || layers.size() > PD_MAX_LAYERS * PD_MAX_SEGMENTS) return FORGE_HIP_OK;
@@ -1290,7 +1533,8 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     // one allocation for all tagged buffers (zeroed: tag 0 is never expected)
     const size_t n_tx = H, n_tq = QKS, n_tkv = 2 * (size_t)KV, n_tws = (size_t)c.heads * DECODE_SPLITS * (hd + 2),
                  n_taq = QKS / 4 + QKS / 32, n_taq2 = I / 4 + I / 32, n_tpart = 2 * (size_t)st->grid;
-    const size_t total = n_tx + n_tq + n_tkv + n_tws + n_taq + n_taq2 + n_tpart;
+    const size_t n_tbm = exact ? (size_t)c.heads * nb_cap : 0, n_trec = n_tbm * (hd + 2);
+    const size_t total = n_tx + n_tq + n_tkv + n_tws + n_taq + n_taq2 + n_tpart + n_tbm + n_trec;
     uint64_t* t = dev_alloc<uint64_t>(total * 8, st->owned);
     if (!t) return fail(FORGE_HIP_ERR_HIP, "persistent decode: out of device memory");
     FH_HIP(hipMemset(t, 0, total * 8));
@@ -1301,7 +1545,9 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     a.tws = t; t += n_tws;
     a.taq = t; t += n_taq;
     a.taq2 = t; t += n_taq2;
-    a.tpart = t;
+    a.tpart = t; t += n_tpart;
+    a.tbm = t; t += n_tbm;
+    a.trec = t;
     a.tag_base = 0;
     // FORGE_HIP_PD_TAG_START: start the tag sequence elsewhere (a test starts it just below the point where it is rewound)
     { const char* e = getenv("FORGE_HIP_PD_TAG_START"); if (e) a.tag_base = (uint32_t)strtoul(e, nullptr, 0); }

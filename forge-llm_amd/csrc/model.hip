@@ -775,7 +775,9 @@ int32_t forge_hip_forward_profile(forge_hip_model* m, uint32_t token, float* sta
         rc = pd_phase_ms(m->pd, &ph, m->stream);
         if (rc) return rc;
         for (int i = 0; i < ST_COUNT; i++) { stage_ms[i] = 0.f; if (stage_launches) stage_launches[i] = 0; }
-        static const int phase_stage[6] = {ST_QKV, ST_ATTN, ST_ATTN, ST_O, ST_GATE_UP, ST_DOWN};
+        // the second attention phase (merge of the splits, or the recurrence over the blocks, and the quantised row for the O
+        // projection) is reported as the quantise stage
+        static const int phase_stage[6] = {ST_QKV, ST_ATTN, ST_QUANT, ST_O, ST_GATE_UP, ST_DOWN};
         for (size_t i = 0; i < ph.size(); i++) {
             const size_t nl = 6 * (size_t)m->cfg.layers;
             const int st = i < nl ? phase_stage[i % 6] : (i == nl ? ST_LM_HEAD : ST_ARGMAX);
