@@ -33,7 +33,7 @@ EXPORTS = [
     "forge_hip_model_destroy", "forge_hip_forward", "forge_hip_forward_greedy", "forge_hip_prefill_batch",
     "forge_hip_forward_profile", "forge_hip_prefill_profile", "forge_hip_model_decode_launches", "forge_hip_reset", "forge_hip_model_pos", "forge_hip_model_set_poll_limit", "forge_hip_model_set_kv_pages", "forge_hip_model_read_kv", "forge_hip_f16_to_f32",
     "forge_hip_f32_to_f16", "forge_hip_quantize_f32", "forge_hip_expf_host", "forge_hip_dequant", "forge_hip_qweight_create",
-    "forge_hip_qweight_destroy", "forge_hip_quantize_act", "forge_hip_gemv_q", "forge_hip_gemm_q",
+    "forge_hip_qweight_destroy", "forge_hip_quantize_act", "forge_hip_gemv_q", "forge_hip_gemm_q", "forge_hip_gemm_silu_q",
     "forge_hip_block_isums", "forge_hip_gemv_q_f32act", "forge_hip_rms_norm", "forge_hip_silu_mul", "forge_hip_rope_kv_store",
     "forge_hip_attn_prefill_f16kv", "forge_hip_attn_decode_f16kv", "forge_hip_attn_decode_f16kv_noalloc", "forge_hip_attn_decode_f16kv_paged",
     "forge_hip_attn_prefill_sliding_f16kv", "forge_hip_attn_decode_sliding_f16kv", "forge_hip_argmax",
@@ -133,6 +133,8 @@ def lib():
     L.forge_hip_gemv_q.argtypes = [vp, vp, vp, vp]
     L.forge_hip_gemm_q.restype = i32
     L.forge_hip_gemm_q.argtypes = [vp, vp, u32, vp, u32, vp]
+    L.forge_hip_gemm_silu_q.restype = i32
+    L.forge_hip_gemm_silu_q.argtypes = [vp, vp, u32, vp, vp, vp]
     L.forge_hip_expf_host.restype = i32
     L.forge_hip_expf_host.argtypes = [vp, u64, vp]
     L.forge_hip_gemv_q_f32act.restype = i32

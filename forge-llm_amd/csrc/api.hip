@@ -176,6 +176,28 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
     return FORGE_HIP_OK;
 }
 
+int32_t forge_hip_gemm_silu_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, int8_t* out_q_dev, uint16_t* out_scales_dev,
+                              void* stream) {
+    FH_CHECK(w && x_dev && out_q_dev && out_scales_dev, "gemm_silu_q: null pointer");
+    FH_CHECK(!w->w.kquant(), "gemm_silu_q: Q8_0 and Q4_0 matrices only");
+    if (M == 0) return FORGE_HIP_OK;
+    FH_CHECK(w->w.N % 128 == 0 && gemm_silu_supported(w->w, w->w.N / 2, M),
+             "gemm_silu_q: the matrix must hold gate rows then up rows, a multiple of 64 each, and M * max(K, N / 2) must stay below 2^31");
+    int8_t* q; uint16_t* sc;
+    int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream, true);
+    if (rc) return rc;
+    void* split_ws = nullptr;
+    if (M > 64) {
+        const bool fresh = g_gemm.cap < gemm_split_workspace_bytes();
+        if ((rc = g_gemm.reserve(gemm_split_workspace_bytes()))) return rc;
+        if (fresh) FH_HIP(hipMemsetAsync(g_gemm.p, 0, gemm_split_workspace_bytes(), (hipStream_t)stream));
+        split_ws = g_gemm.p;
+    }
+    launch_gemm(w->w, q, sc, M, nullptr, w->w.N, false, false, nullptr, (hipStream_t)stream, split_ws, out_q_dev, out_scales_dev);
+    FH_HIP(hipGetLastError());
+    return FORGE_HIP_OK;
+}
+
 int32_t forge_hip_gemv_q_f32act(const forge_hip_qweight* w, const float* x_dev, float* y_dev, void* stream) {
     FH_CHECK(w && x_dev && y_dev, "gemv_q_f32act: null pointer");
     FH_CHECK(!w->w.kquant(), "gemv_q_f32act: Q8_0 and Q4_0 matrices only");

@@ -163,8 +163,13 @@ void launch_gemv_kquant(const QWeight& w, const int8_t* aq, const uint16_t* as, 
 // launch): lets the fast mode cut the tiles that do not fill a whole round of CUs along K; launches that share a
 // workspace must be ordered (one stream).  With it a row's low bits may depend on where in the batch the row sits.
 size_t gemm_split_workspace_bytes();
+// silu_q / silu_sc (fast mode, no isums, gemm_silu_supported(w, w.N / 2, M)): w is a fused [gate; up] matrix; instead of y
+// the launch writes quantize(silu(gate) * up) for the down projection: codes [M][N / 2] with odd blocks negated and fp16
+// scales [M][N / 64] (silu_mul emit.rs:380-386 with the hardware exponential, quantiser emit.rs:1410-1440).
+bool gemm_silu_supported(const QWeight& w, uint32_t inter, uint32_t M);
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
-                 bool accumulate, bool exact, int32_t* isums, hipStream_t s, void* split_ws = nullptr);
+                 bool accumulate, bool exact, int32_t* isums, hipStream_t s, void* split_ws = nullptr, int8_t* silu_q = nullptr,
+                 uint16_t* silu_sc = nullptr);
 
 // model.hip — the part of forge_hip_model_create's checks that sizes depend on (formats, dimensions the kernels cover);
 // sets the error message.

@@ -79,13 +79,22 @@ __device__ __forceinline__ uint32_t nib_minus8(uint32_t x) {
 // `partials`; the workgroup that finishes a tile's last range adds the ranges in range order (so the result does not
 // depend on who came last) and stores the tile.  The launch code uses it when the tiles fill the CUs once and a fraction:
 // the fraction is what gets cut, so that every CU ends up with the same amount of work.
+// SILU (fast mode only): the matrix is a fused [gate; up] pair of `inter` rows each (emit.rs:5390-5420 computes both from
+// the same normalised row).  A workgroup's 128 columns are then 64 consecutive inter indices: each wave's first 32-column
+// tile holds gate rows i0 .. i0 + 32, its second the up rows of the same indices, so a lane ends up with gate and up of
+// one (row, index) pair and the epilogue is silu(gate) * up (emit.rs:380-386, hardware exp) and the activation quantiser
+// (emit.rs:1410-1440: the 32 indices of a tile are exactly one block, spread over 32 lanes) -- the down projection's
+// input, codes and scales, instead of 2 * inter floats per row written and read back.
 struct GemmSplit {
     uint32_t full_tiles, split, stages_per_part;
     float* partials;        // [tiles - full_tiles][split][tile elements]
     uint32_t* counters;     // [tiles - full_tiles], zero between launches
+    int8_t* silu_q;         // SILU: [M][inter] codes (odd blocks negated, as the fast GEMM takes its activations)
+    uint16_t* silu_sc;      // SILU: [M][inter / 32] fp16 scales
+    uint32_t inter;
 };
 
-template <bool Q4, bool DUMP, bool EXACT, int TM, bool SPLIT = false>
+template <bool Q4, bool DUMP, bool EXACT, int TM, bool SPLIT = false, bool SILU = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ wsc, const int8_t* __restrict__ aq,
                    const uint16_t* __restrict__ asc, float* __restrict__ y, int32_t* __restrict__ isums, uint32_t M,
@@ -93,6 +102,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr bool MAGIC = !EXACT;               // DUMP && !EXACT: the fast arithmetic, with its block sums written out too
     static_assert(!SPLIT || (MAGIC && !DUMP), "K ranges change the order of the block sum: fast mode only");
+    static_assert(!SILU || (MAGIC && !DUMP), "the fused SiLU epilogue belongs to the fast mode");
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // uniform: the compiler keeps it scalar
@@ -126,14 +136,21 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     const uint32_t ld_row = wave * 8 + (lane >> 3);                        // + 32 i
     const uint32_t ld_chunk = (lane & 7) ^ ((ld_row >> 1) & 7);            // global chunk for LDS position lane & 7
     const uint32_t a_voff = (m0 + ld_row) * K + ld_chunk * 16;             // + 32 i K + k0
-    const uint32_t w_voff = (n0 + ld_row) * K + ld_chunk * 16;             // Q8_0 only
+    // SILU: tile row j is weight row i0 + (j / 64) * 32 + j % 32 (+ inter for the up half, (j / 32) odd), i0 = 64 tile_x
+    const uint32_t s_inter = SILU ? sp.inter : 0u, si0 = tile_x * 64;
+    const uint32_t w_voff = (SILU ? si0 + ld_row : n0 + ld_row) * K + ld_chunk * 16;     // Q8_0 only; load i: + w_step[i]
     // Q4_0: piece idx = tid + 256 i: row = idx / 4, block = idx % 4 (16 packed bytes -> 32 codes)
     const uint32_t q4_row = tid >> 2, q4_blk = tid & 3;                    // + 64 i
-    const uint32_t q4_voff = ((n0 + q4_row) * nblk + q4_blk) * 16;         // + 64 i nblk 16 + (k0/32) 16
+    const uint32_t q4_wrow = SILU ? si0 + (q4_row & 31) + (q4_row >> 5) * s_inter : n0 + q4_row;
+    const uint32_t q4_voff = (q4_wrow * nblk + q4_blk) * 16;               // + q4_step i + (k0/32) 16
     // scales: threads 0..127 take activation row tid, threads 128..255 weight row tid - 128
     const bool sc_is_a = wave < 2;
     const uint32_t sc_row = tid & 127;
-    const uint32_t sc_voff = ((sc_is_a ? m0 : n0) + sc_row) * nblk * 2;
+    const uint32_t sc_wrow = SILU ? si0 + (sc_row >> 6) * 32 + (sc_row & 31) + ((sc_row >> 5) & 1) * s_inter : n0 + sc_row;
+    const uint32_t sc_voff = (sc_is_a ? m0 + sc_row : sc_wrow) * nblk * 2;
+    // uniform steps from load to load (rows 32 i further on; SILU: 32 (i / 2) further on, odd loads in the up half)
+    const uint32_t w_step[4] = {0u, SILU ? s_inter * K : 32 * K, SILU ? 32 * K : 64 * K, SILU ? 32 * K + s_inter * K : 96 * K};
+    const uint32_t q4_step = (SILU ? 32u : 64u) * nblk * 16;
 
     v4i rb[2];
     uint32_t rs[KB];
@@ -161,12 +178,12 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         }
         if ((part & 2) && Q4) {
 #pragma unroll
-            for (int i = 0; i < 2; i++) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rw_k, q4_voff + i * 64 * nblk * 16, 0, 0);
+            for (int i = 0; i < 2; i++) rb[i] = __builtin_amdgcn_raw_buffer_load_b128(rw_k, q4_voff + i * q4_step, 0, 0);
         } else if (part & 2) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(rw_k, FH_LDS3(lds + LDS_B + buf * TILE_BYTES + (i * 4 + wave) * 1024), 16,
-                                                         w_voff + i * 32 * K, 0, 0, 0);
+                                                         w_voff + w_step[i], 0, 0, 0);
         }
         if (part & 4) {
 #pragma unroll
@@ -436,6 +453,35 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         if (tid == 0) __hip_atomic_store(sp.counters + range_tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch (stream order)
     }
 
+    if (SILU) {
+        // lane: inter index i0 + 32 wn + lrow, gate in the first column tile, up in the second; rows as below
+        const uint32_t inter = sp.inter, blk = tile_x * 2 + wn;           // the quant block this wave's 32 indices are
+        const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc((void*)sp.silu_q, 0, M * inter, RSRC_FLAGS);
+        const __amdgpu_buffer_rsrc_t rsc = __builtin_amdgcn_make_buffer_rsrc((void*)sp.silu_sc, 0, M * (inter / 32) * 2, RSRC_FLAGS);
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float g = acc[tm][0][r], u = acc[tm][1][r];
+                if (Q4) { g *= 0.0625f; u *= 0.0625f; }
+                // fast mode: reciprocals instead of divisions (1 ulp), round-to-nearest-even instead of half-away (they part
+                // on exact ties only); |o * inv| <= 127 up to rounding, so the conversion needs no clamp
+                const float o = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
+                const float amax = half_wave_max(fabsf(o));               // the 32 lanes that share lhalf: one block of one row
+                const float scl = amax > 0.f ? amax * (1.0f / 127.0f) : 1.0f;
+                float inv = amax > 0.f ? 127.0f * __builtin_amdgcn_rcpf(amax) : 0.f;
+                if (blk & 1u) inv = -inv;                                 // odd blocks negated for the GEMM that reads them
+                const uint32_t code = (uint32_t)(int)__builtin_rintf(o * inv) & 0xFFu;
+                const uint32_t pk = quad_broadcast<0>(code) | (quad_broadcast<1>(code) << 8) | (quad_broadcast<2>(code) << 16) |
+                                    (quad_broadcast<3>(code) << 24);
+                const uint32_t m = m0 + wm * WM + tm * 32 + 4 * lhalf + 8 * (r >> 2) + (r & 3);
+                // rows >= M lie past the end of the descriptors and are dropped
+                if ((lrow & 3u) == 0) __builtin_amdgcn_raw_buffer_store_b32(pk, rq, m * inter + blk * 32 + lrow, 0, 0);
+                if (lrow == 0) __builtin_amdgcn_raw_buffer_store_b16((uint16_t)f32_to_f16_bits(scl), rsc, (m * (inter / 32) + blk) * 2, 0, 0);
+            }
+        return;
+    }
+
     // epilogue: lane holds column n = lrow, rows 8g + 4*lhalf + (r&3); the descriptor drops rows >= M.
     // y += ...: all of a lane's old values are requested before the first is used (a load, its wait, the add and the
     // store per element would be 64 memory round trips one after the other: every wait also waits for the store before it)
@@ -485,9 +531,17 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
 // row ranges of the activations and of the weights, one launch each.
 size_t gemm_split_workspace_bytes() { return (size_t)GEMM_SPLIT_MAX_ITEMS * BM * BN * sizeof(float) + GEMM_SPLIT_MAX_ITEMS * sizeof(uint32_t); }
 
+// Whether launch_gemm's fused SiLU epilogue covers a fused [gate; up] matrix of 2 * inter rows for M activation rows.
+bool gemm_silu_supported(const QWeight& w, uint32_t inter, uint32_t M) {
+    const uint64_t LIMIT = 0x7FFFFFFFull - 2 * BK;
+    return w.N == 2 * (uint64_t)inter && inter % 64 == 0 && (uint64_t)M * std::max<uint64_t>(w.K, inter) <= LIMIT &&
+           (uint64_t)w.N * std::max<uint64_t>(w.qs_row_bytes(), (uint64_t)(w.K / 32) * 2) <= LIMIT;
+}
+
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
-                 bool accumulate, bool exact, int32_t* isums, hipStream_t s, void* split_ws) {
+                 bool accumulate, bool exact, int32_t* isums, hipStream_t s, void* split_ws, int8_t* silu_q, uint16_t* silu_sc) {
     if (M == 0 || w.N == 0) return;
+    const bool silu = silu_q != nullptr;      // caller: gemm_silu_supported, fast mode, no block-sum dump
     const int accf = accumulate ? 1 : 0;
     const bool q4 = w.wdtype == FORGE_HIP_Q4_0;
     const uint64_t LIMIT = 0x7FFFFFFFull - 2 * BK;
@@ -563,6 +617,25 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
                 Plan best = plan(tm);
                 if (tm == 1) { const Plan other = plan(2); if (other.cost < best.cost) best = other; }
                 tm = best.tm;
+                if (best.items && silu) {
+                    GemmSplit sp = best.sp;
+                    sp.silu_q = silu_q; sp.silu_sc = silu_sc; sp.inter = w.N / 2;
+                    const uint32_t items = best.items;
+#define FH_GEMM_LAUNCH_SPLIT_SILU(Q4_, TM_)                                                                                  \
+    do {                                                                                                                    \
+        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, false, false, TM_, true, true>, \
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES);   \
+        (void)lds_ok;                                                                                                       \
+        fh::launch(gemm_q_kernel<Q4_, false, false, TM_, true, true>, dim3(items), 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c,   \
+                   as_c, y_c, is_c, mc, nc, w.K, ldy, accf, sp);                                                            \
+    } while (0)
+                    if (q4 && tm == 1) FH_GEMM_LAUNCH_SPLIT_SILU(true, 1);
+                    else if (q4) FH_GEMM_LAUNCH_SPLIT_SILU(true, 2);
+                    else if (tm == 1) FH_GEMM_LAUNCH_SPLIT_SILU(false, 1);
+                    else FH_GEMM_LAUNCH_SPLIT_SILU(false, 2);
+#undef FH_GEMM_LAUNCH_SPLIT_SILU
+                    continue;
+                }
                 if (best.items) {
                     const GemmSplit sp = best.sp;
                     const uint32_t items = best.items;
@@ -581,6 +654,25 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
 #undef FH_GEMM_LAUNCH_SPLIT
                     continue;
                 }
+            }
+            if (silu) {
+                GemmSplit sp{};
+                sp.silu_q = silu_q; sp.silu_sc = silu_sc; sp.inter = w.N / 2;
+#define FH_GEMM_LAUNCH_SILU(Q4_, TM_)                                                                                         \
+    do {                                                                                                                    \
+        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, false, false, TM_, false, true>, \
+                                                             hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES);   \
+        (void)lds_ok;                                                                                                       \
+        dim3 grid((nc + BN - 1) / BN, (mc + 64 * TM_ - 1) / (64 * TM_));                                                    \
+        fh::launch(gemm_q_kernel<Q4_, false, false, TM_, false, true>, grid, 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c,   \
+                   y_c, is_c, mc, nc, w.K, ldy, accf, sp);                                                                  \
+    } while (0)
+                if (q4 && tm == 1) FH_GEMM_LAUNCH_SILU(true, 1);
+                else if (q4) FH_GEMM_LAUNCH_SILU(true, 2);
+                else if (tm == 1) FH_GEMM_LAUNCH_SILU(false, 1);
+                else FH_GEMM_LAUNCH_SILU(false, 2);
+#undef FH_GEMM_LAUNCH_SILU
+                continue;
             }
             if (q4) {
                 if (isums && exact) FH_GEMM_LAUNCH(true, true, true);

@@ -67,8 +67,9 @@ struct forge_hip_model {
     std::vector<uint32_t> page_table_host;
     float repeat_penalty = 1.0f;         // > 1: forward_greedy picks the maximum of the penalised logits
     // prefill scratch (chunk_rows rows)
-    DevBuf px, pqkv, pattn, pgu, paq, pasc, ptok;
+    DevBuf px, pqkv, pattn, pgu, paq, pasc, paq2, pasc2, ptok;
     bool prefill_fuse_quant = true;              // fast mode: attention writes int8 codes + scales (FORGE_HIP_FUSE=0: separate quantiser)
+    bool prefill_fuse_silu = false;              // fast mode: the gate/up GEMM writes silu(gate) * up quantised (FORGE_HIP_FUSE=0: separate kernel)
     uint32_t chunk_rows = 0;
     // pinned host staging: [0] token, [1] next token, [2] position
     uint32_t* h_stage = nullptr;
@@ -348,8 +349,17 @@ void enqueue_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t 
     }
     { StageMark t(m, ST_O); launch_gemm(L.o, aq, asc, M, x, H, true, exact, nullptr, s, m->gemm_ws.p); }
     { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s, !exact); }
-    { StageMark t(m, ST_GATE_UP); launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s, m->gemm_ws.p); }
-    { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s, !exact); }
+    if (m->prefill_fuse_silu && gemm_silu_supported(L.gate_up, I, M)) {
+        // the GEMM's epilogue writes silu(gate) * up quantised: the [M][2 I] floats never exist.  The kernel reads `aq` while
+        // it runs, so its output goes to the second code buffer and the down projection reads that.
+        StageMark t(m, ST_GATE_UP);
+        launch_gemm(L.gate_up, aq, asc, M, nullptr, 2 * I, false, false, nullptr, s, m->gemm_ws.p, m->paq2.as<int8_t>(), m->pasc2.as<uint16_t>());
+        aq = m->paq2.as<int8_t>();
+        asc = m->pasc2.as<uint16_t>();
+    } else {
+        { StageMark t(m, ST_GATE_UP); launch_gemm(L.gate_up, aq, asc, M, gu, 2 * I, false, exact, nullptr, s, m->gemm_ws.p); }
+        { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s, !exact); }
+    }
     { StageMark t(m, ST_DOWN); launch_gemm(L.down, aq, asc, M, x, H, true, exact, nullptr, s, m->gemm_ws.p); }
 }
 
@@ -542,6 +552,10 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
     m->fuse_norm = fuse_ok && !pd && gemv_norm_fusable(H);
     m->fuse_silu = fuse_ok && !pd && gemv_silu_fusable(H);
     m->prefill_fuse_quant = fuse_ok;
+    // FORGE_HIP_FUSE_SILU_GEMM=0: the gate/up GEMM writes floats and silu_mul + the quantiser run as a kernel of their own
+    // (the fused epilogue uses the hardware exponential and reciprocals: same values to the fast mode's tolerance, not the same bits)
+    const char* senv2 = getenv("FORGE_HIP_FUSE_SILU_GEMM");
+    m->prefill_fuse_silu = fuse_ok && !(senv2 && senv2[0] == '0') && !(cfg->flags & FORGE_HIP_FLAG_EXACT) && !pd && I % 64 == 0;
     FH_HIP(hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking));
     FH_HIP(hipHostMalloc((void**)&m->h_stage, 64, hipHostMallocDefault));
     FH_HIP(hipHostMalloc((void**)&m->h_logits, (size_t)cfg->vocab * 4, hipHostMallocDefault));
@@ -648,6 +662,7 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
         (rc = m->paq.alloc((size_t)R * m->KMAX)) || (rc = m->pasc.alloc((size_t)R * (m->KMAX / 32) * 2)) ||
         (rc = m->ptok.alloc((size_t)R * 4)))
         return rc;
+    if (m->prefill_fuse_silu && ((rc = m->paq2.alloc((size_t)R * I)) || (rc = m->pasc2.alloc((size_t)R * (I / 32) * 2)))) return rc;
     // fast mode: the prefill GEMMs may cut left-over tiles along K (FORGE_HIP_GEMM_SPLIT=0: never)
     const char* senv = getenv("FORGE_HIP_GEMM_SPLIT");
     if (!(cfg->flags & FORGE_HIP_FLAG_EXACT) && !(senv && senv[0] == '0')) {

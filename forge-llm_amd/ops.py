@@ -164,6 +164,22 @@ def expf_host(x) -> np.ndarray:
     return out
 
 
+def gate_up_silu_q(w: QWeight, x):
+    """The gate / up matmuls, silu_mul and the activation quantiser of the batched feed-forward block in one launch
+    (crates/forgellm-codegen-cpu/src/emit.rs:5390-5420): w holds the gate rows then the up rows; x: f32 [M][K] on the GPU.
+    Returns (codes int8 [M][N/2] with odd blocks negated, scales as fp16 bit patterns int16 [M][N/64])."""
+    from . import check, lib
+    torch = _torch()
+    x = _dev(x, torch.float32)
+    if x.dim() != 2 or x.shape[1] != w.K:
+        raise ValueError("input must be [M][K]")
+    M = x.shape[0]
+    q = torch.empty((M, w.N // 2), dtype=torch.int8, device=x.device)
+    sc = torch.empty((M, w.N // 64), dtype=torch.int16, device=x.device)
+    check(lib().forge_hip_gemm_silu_q(w._h, _ptr(x), M, _ptr(q), _ptr(sc), _stream()))
+    return q, sc
+
+
 def matmul_mat_q(w: QWeight, x, flags=0):
     """matmul_mat_q8_0_KxN / matmul_mat_q4_0_KxN: x f32 [M][K] -> f32 [M][N]."""
     from . import check, lib

@@ -242,6 +242,16 @@ int32_t forge_hip_gemv_q_f32act(const forge_hip_qweight* w, const float* x_dev, 
 int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, uint32_t flags,
                          void* stream);
 
+/* The gate / up half of the batched feed-forward block in one launch (fast mode): for a handle whose N rows are the gate
+ * projection's rows followed by the up projection's (N / 2 each, a multiple of 64), gate = x Wg^T and up = x Wu^T as
+ * forge_hip_gemm_q computes them, then silu_mul (emit.rs:380-386, hardware exponential) and the activation quantiser
+ * (quantize_to_q8_0_blocks_into, emit.rs:1410-1440) in the kernel's epilogue: out_q_dev int8 [M][N / 2] with the codes of
+ * every row's odd blocks negated (the form forge_hip_gemm_q's fast kernel takes its activations in), out_scales_dev
+ * fp16 bits [M][N / 64].  What forward_prefill_batched does between the gate / up matmuls and the down matmul
+ * (emit.rs:5390-5420) without the [M][N] floats in memory. */
+int32_t forge_hip_gemm_silu_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, int8_t* out_q_dev, uint16_t* out_scales_dev,
+                              void* stream);
+
 /* The int32 block sums the two calls above combine: out_dev int32 [M][N][K/32]
  * (dot_q8_0_q8_0 / dot_q4_0_q8_0 `vaddvq_s32(acc)`, emit.rs:1543-1553, 2522-2552).
  * path 0 = the GEMV kernel's dot, path 1 = the MFMA GEMM kernel's tiles in exact mode, path 2 = the same kernel in the

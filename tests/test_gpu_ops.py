@@ -207,6 +207,38 @@ def test_matmul_mat_k_ranges_of_leftover_tiles(fh, torch_gpu, wd, M, K, N):
     w.close()
 
 
+@pytest.mark.parametrize("wd", [Q8, Q4])
+@pytest.mark.parametrize("M,K,I", [(2502, 2048, 8192), (37, 576, 1536), (300, 256, 64), (700, 3072, 1024), (65, 8192, 128)])
+def test_gate_up_matmul_with_silu_and_quantiser_in_the_epilogue(fh, oracle, torch_gpu, wd, M, K, I):
+    """forge_hip_gemm_silu_q: gate / up matmuls (fast arithmetic), silu(gate) * up and the activation quantiser in one kernel.
+    Checked against the order-faithful matmul (bit-identical to the CPU path, see above) followed by silu_mul and the
+    quantiser's definition in float64: every scale is absmax / 127 of its block to the fast mode's tolerance, every code is
+    the nearest one (half a step, plus the tolerance on the value that was rounded), odd blocks come negated; rows past M
+    stay untouched; the result does not depend on the run."""
+    torch = torch_gpu
+    wraw = make_weight(fh, wd, 2 * I, K, seed=7 * I + K + M)
+    x = fh.synth.normal(19 + K, M * K, 1.0).reshape(M, K)
+    w = fh.ops.QWeight(wd, wraw, K, 2 * I)
+    xd = torch.from_numpy(x).cuda()
+    y = fh.ops.matmul_mat_q(w, xd, EXACT).cpu().numpy().astype(np.float64)
+    gate, up = y[:, :I], y[:, I:]
+    o = gate / (1.0 + np.exp(-gate)) * up
+    q, sc = fh.ops.gate_up_silu_q(w, xd)
+    q2, sc2 = fh.ops.gate_up_silu_q(w, xd)
+    assert torch.equal(q, q2) and torch.equal(sc, sc2)
+    codes = q.cpu().numpy().astype(np.float64).reshape(M, I // 32, 32)
+    scales = oracle.f16_to_f32(sc.cpu().numpy().view(np.uint16)).astype(np.float64).reshape(M, I // 32)
+    ob = o.reshape(M, I // 32, 32)
+    amax = np.abs(ob).max(axis=2)
+    tol = 2e-3 * amax + 1e-6
+    assert np.all(np.abs(scales - amax / 127.0) <= tol / 127.0 + amax / 127.0 * 2.0 ** -10)      # fp16 rounding of the scale
+    sign = np.where(np.arange(I // 32) % 2 == 1, -1.0, 1.0)[None, :, None]
+    recon = codes * sign * scales[:, :, None]
+    assert np.all(np.abs(recon - ob) <= 0.5 * scales[:, :, None] * (1 + 2.0 ** -9) + tol[:, :, None])
+    assert np.abs(codes).max() == 127                          # every block reaches its own maximum
+    w.close()
+
+
 def test_matmul_mat_ragged_n_within_tolerance(fh, oracle, torch_gpu):
     """N % 4 != 0: the reference's last rows use the 4-accumulator order; the GEMM kernel keeps one
     order for all rows, so those rows agree to tolerance only."""
