@@ -70,6 +70,15 @@ constexpr int PD_MISC_HINT = 40, PD_MISC_SCRATCH = 64;
 // misc LDS words [PD_MISC_PT, 512): page-table entries of this workgroup's attention items, staged once per step (an item's
 // key range is the same in every layer); slot (round, wave group) holds pt_cap entries
 constexpr int PD_MISC_PT = 128, PD_MISC_PT_WORDS = 512 - PD_MISC_PT;
+// `big` area: a GEMV phase's row sums sit at its start -- [rows][4] partial sums by default, [rows][nblk + 1] block products
+// in the ordered variants -- and the residual row that a norm phase fetches (H floats) starts PD_X_WORDS further on.  The
+// two poller waves leave a GEMV phase one after the other (the one without rows does not wait for the one that still adds
+// its rows up) and the first thing a norm phase does is write that row: with the default sums (at most PD_MAX_TILE_ROWS
+// rows of 4 words) the two ranges are disjoint by this offset; the ordered variants' products can reach anywhere, so they
+// put a barrier in front of a norm phase's input instead.
+constexpr uint32_t PD_X_WORDS = 512;
+static_assert(PD_MAX_TILE_ROWS * 4 <= PD_X_WORDS, "default row sums must end before the residual row begins");
+static_assert(PD_MISC_SCRATCH + 64 <= PD_MISC_PT, "phase scratch (64 floats: merge weights, argmax pairs, exp_scale chunk) ends before the page table words");
 
 struct PdGemv {
     const uint8_t* qs;
@@ -824,6 +833,7 @@ __device__ __forceinline__ void pd_attn_combine(const PdArgs& a, uint32_t tag_in
 constexpr uint32_t PX_B = 64;        // FLASH_ATTN_BLOCK_SIZE, emit.rs:201
 constexpr uint32_t PX_CHUNK = 64;    // block records the recurrence takes into LDS at a time
 constexpr uint32_t PX_MAX_BLOCKS = 4096;
+static_assert(PX_CHUNK <= 64 && DECODE_SPLITS + 1 <= 64 && PD_WAVES * 2 <= 64, "users of the 64 floats of phase scratch in the misc area");
 
 // What the two stages need of the kernel arguments.
 struct PxArgs {
@@ -1062,6 +1072,10 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     const uint32_t K = job.in_len, U = h.U;
     TilePos t = pd_tile(h, cx.wg);
 
+    float* xs = big + PD_X_WORDS;                           // the residual row of a norm phase
+    // ordered variants: the other poller wave may still be adding up the previous phase's block products, which can lie
+    // where this phase's input is about to be written (see PD_X_WORDS)
+    if (ORDERED && job.pro == PRO_NORM) __syncthreads();
     // ---- inputs (norm weights are requested before this wave's weights: loads return in order)
     float4 nw = make_float4(0.f, 0.f, 0.f, 0.f);
     if (job.pro == PRO_NORM && cx.tid * 4 < K) nw = ldg(reinterpret_cast<const float4*>(job.norm_w + cx.tid * 4));
@@ -1070,8 +1084,8 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     } else {
         float ssq = 0.f;
         if (job.pro == PRO_AQ) pd_load_aq(job.tin, job.tin_tag, K, aq_lds, as_lds, misc, a.use_hint != 0, cx);
-        else if (job.tin_tag) pd_load_x(job.tin, job.tin_tag, K, big, misc, a.use_hint != 0, cx, ssq);
-        else for (uint32_t i = cx.tid; i < K; i += PD_POLL_THREADS) { const float v = emb[i]; big[i] = v; ssq += v * v; }
+        else if (job.tin_tag) pd_load_x(job.tin, job.tin_tag, K, xs, misc, a.use_hint != 0, cx, ssq);
+        else for (uint32_t i = cx.tid; i < K; i += PD_POLL_THREADS) { const float v = emb[i]; xs[i] = v; ssq += v * v; }
         if (!ORDERED && job.pro == PRO_NORM) {
             // the pollers square what they fetched: the sum of squares needs no pass (and no barrier) of its own
             ssq += __builtin_amdgcn_update_dpp(0.f, ssq, 0xB1, 0xF, 0xF, false);      // quad_perm [1,0,3,2]
@@ -1083,8 +1097,8 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     }
     __syncthreads();
     if (*cx.sh_abort) return;
-    // the norm reads big[0..K); the products reuse the area afterwards
-    if (job.pro == PRO_NORM) pd_norm_quant<ORDERED>(big, job.norm_w, nw, a.eps, K, aq_lds, as_lds, misc, cx);
+    // the norm reads the row; the products use the area from its start afterwards
+    if (job.pro == PRO_NORM) pd_norm_quant<ORDERED>(xs, job.norm_w, nw, a.eps, K, aq_lds, as_lds, misc, cx);
 
     // ---- tiles
     float acc = 0.f;
@@ -1480,7 +1494,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     if (a.off_big + 4096 > PD_LDS_BYTES) return FORGE_HIP_OK;
     const uint32_t big = PD_LDS_BYTES - 64 - a.off_big;
     const uint32_t attn_bytes = (a.gt == 1 ? 2 : 1) * (16 * (hd + 2) + 6 * hd) * 4;      // two items at a time when a group has one head
-    if ((H + 32) * 4 > big || attn_bytes > big || DECODE_SPLITS * (hd + 2) * 4 > big) return FORGE_HIP_OK;
+    if ((H + 32 + PD_X_WORDS) * 4 > big || attn_bytes > big || DECODE_SPLITS * (hd + 2) * 4 > big) return FORGE_HIP_OK;
     if (exact && (PX_CHUNK * (hd + 2) * 4 > big || c.heads > st->grid * PD_WAVES)) return FORGE_HIP_OK;
     st->lds = a.off_big + big;
 
