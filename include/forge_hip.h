@@ -238,7 +238,10 @@ int32_t forge_hip_gemv_q(const forge_hip_qweight* w, const float* x_dev, float* 
 int32_t forge_hip_gemv_q_f32act(const forge_hip_qweight* w, const float* x_dev, float* y_dev, void* stream);
 
 /* matmul_mat_q8_0_KxN / matmul_mat_q4_0_KxN (emit.rs:2108-2302, 3667-3817):
- * y[M][N] = x[M][K] W^T, row-major. */
+ * y[M][N] = x[M][K] W^T, row-major.  With FORGE_HIP_FLAG_EXACT every row has the CPU path's bits.  Without it the block sums
+ * are still exact and the f32 combine is within 1e-3, for data whose per-block activation scale is below 256 (largest
+ * activation of a block below 32 512) and whose weight scales are below 2: the kernel removes a bias from its block sums with
+ * an fp16 matrix instruction on scales multiplied by powers of two, which is exact inside that range only. */
 int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, uint32_t flags,
                          void* stream);
 
@@ -292,7 +295,10 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
  * results bit for bit; the split records (heads * 32 * (head_dim + 2) floats) go to a fixed 2 129 920-byte array in the
  * library's device image (one copy per GPU, held until the process ends) instead of the op-level API's lazily grown
  * allocation, and the call makes no hipMalloc / hipFree.  heads <= 128, else FORGE_HIP_ERR_INVALID.  Every call on a GPU
- * uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not. */
+ * uses that GPU's one array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not.
+ * The array's device address is looked up once per device when a model or a weight handle is created there
+ * (forge_hip_model_create*, forge_hip_qweight_create), else at the first call on the device: a caller that holds neither
+ * makes one call outside a graph capture first. */
 int32_t forge_hip_attn_decode_f16kv_noalloc(const float* q_dev, const uint16_t* k_cache_dev, const uint16_t* v_cache_dev,
                                             float* out_dev, uint32_t seq_len, uint32_t heads, uint32_t kv_heads,
                                             uint32_t head_dim, void* stream);
