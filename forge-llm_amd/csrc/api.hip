@@ -153,10 +153,18 @@ int32_t forge_hip_gemv_q(const forge_hip_qweight* w, const float* x_dev, float* 
 int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, uint32_t flags,
                          void* stream) {
     FH_CHECK(w && x_dev && y_dev, "gemm_q: null pointer");
-    FH_CHECK(!w->w.kquant(), "gemm_q: K-quant matrices have no batched matmul (the reference runs them through matmul_vec)");
     FH_CHECK((flags & ~FORGE_HIP_FLAG_EXACT) == 0, "gemm_q: unknown flag bits");
     if (M == 0) return FORGE_HIP_OK;
     int8_t* q; uint16_t* sc;
+    if (w->w.kquant()) {
+        // the reference has no batched matmul for these formats: M rows of matmul_vec, the matrix read once per 8 rows
+        FH_CHECK(kquant_k_supported(w->w.K), "gemm_q: K must be a multiple of 256, at most 16384");
+        int32_t rck = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream, false);
+        if (rck) return rck;
+        launch_gemv_kquant_rows(w->w, q, sc, M, y_dev, w->w.N, false, (hipStream_t)stream);
+        FH_HIP(hipGetLastError());
+        return FORGE_HIP_OK;
+    }
     const bool exact = (flags & FORGE_HIP_FLAG_EXACT) != 0;
     int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream, !exact);   // the fast kernel takes odd blocks negated
     if (rc) return rc;

@@ -155,6 +155,16 @@ void launch_gemv_f32(const QWeight& w, const float* x, float* y, hipStream_t s);
 void repack_kquant_host(uint32_t wdtype, const uint8_t* raw, uint32_t K, uint64_t N, uint8_t* qs, uint8_t* meta);
 bool kquant_k_supported(uint32_t K);
 void launch_gemv_kquant(const QWeight& w, const int8_t* aq, const uint16_t* as, float* y, bool accumulate, hipStream_t s);
+// Up to three Q4_K / Q6_K matrices of the same K over one quantised vector in a single launch (q, k, v; gate, up).
+void launch_gemv_kquant_multi(const QWeight* const* w, float* const* y, uint32_t n, const int8_t* aq, const uint16_t* as, bool accumulate,
+                              hipStream_t s);
+// ... over quantise(rms_norm(x) * norm_w), normed and quantised inside the kernel (the norm kernel's bits).
+void launch_gemv_kquant_multi_norm(const QWeight* const* w, float* const* y, uint32_t n, const float* x, const float* norm_w, float eps,
+                                   hipStream_t s);
+// The same for M rows of quantised activations (codes [M][K], scales [M][K/32]); rows of y are ldy floats apart.  Every row has the
+// bits launch_gemv_kquant gives it alone.
+void launch_gemv_kquant_rows(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy, bool accumulate,
+                             hipStream_t s);
 
 // gemm.hip — y[m][n] (=|+=) ...; aq int8 [M][K], as fp16 [M][K/32].  isums (optional) int32 [M][N][K/32].
 // exact: unfused multiply/add per block (bit-identical to the CPU path); otherwise one FMA per block, and then the

@@ -69,6 +69,8 @@ struct forge_hip_model {
     // prefill scratch (chunk_rows rows)
     DevBuf px, pqkv, pattn, pgu, paq, pasc, paq2, pasc2, ptok;
     bool prefill_fuse_quant = true;              // fast mode: attention writes int8 codes + scales (FORGE_HIP_FUSE=0: separate quantiser)
+    bool mixed_fuse = true;          // K-quant projections over a normed row norm and quantise it themselves: a launch less, the same bits
+    bool mixed_batched = false;                  // per-projection formats: the prompt runs in batches of rows (see enqueue_mixed_prefill_layer)
     bool prefill_fuse_silu = false;              // fast mode: the gate/up GEMM writes silu(gate) * up quantised (FORGE_HIP_FUSE=0: separate kernel)
     uint32_t chunk_rows = 0;
     // pinned host staging: [0] token, [1] next token, [2] position
@@ -227,6 +229,30 @@ void gemv_any(const QWeight& w, const int8_t* aq, const uint16_t* asc, float* y,
     else launch_gemv(w, aq, asc, y, accumulate, order, s);
 }
 
+// Projections that multiply quantise(rms_norm(x) * norm_w).  All K-quant: one launch that norms, quantises and multiplies.
+// Otherwise the norm kernel first, then the K-quant ones among them in one launch and the others one each.
+static void norm_gemv_group(forge_hip_model* m, const float* norm_w, const QWeight* const* w, float* const* y, uint32_t n, int stage) {
+    hipStream_t s = m->stream;
+    int8_t* aq = m->aq.as<int8_t>();
+    uint16_t* asc = m->asc.as<uint16_t>();
+    const QWeight* kw[3];
+    float* ky[3];
+    uint32_t nk = 0;
+    for (uint32_t i = 0; i < n; i++)
+        if (w[i]->kquant()) { kw[nk] = w[i]; ky[nk++] = y[i]; }
+    if (nk == n && m->mixed_fuse) {
+        StageMark t(m, stage);
+        launch_gemv_kquant_multi_norm(kw, ky, nk, m->x.as<float>(), norm_w, m->cfg.rms_eps, s);
+        return;
+    }
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(m->x.as<float>(), norm_w, m->cfg.rms_eps, 1, m->H, nullptr, aq, asc, s); }
+    StageMark t(m, stage);
+    for (uint32_t i = 0; i < n; i++)
+        if (!w[i]->kquant()) launch_gemv(*w[i], aq, asc, y[i], false, GemvOrder::MatmulVec, s);
+    if (nk == 1) launch_gemv_kquant(*kw[0], aq, asc, ky[0], false, s);
+    else if (nk > 1) launch_gemv_kquant_multi(kw, ky, nk, aq, asc, false, s);
+}
+
 // One decoder layer for ONE row of a model with a storage format per projection (model::forward, emit.rs:4029-4500, with
 // the projection calls of emit.rs:4085-4100, 4200-4260): every projection a launch of its own kernel family.  The row sits
 // at `pos` (pos_dev == nullptr: a token of a prompt) or at *pos_dev (a decode step).
@@ -234,7 +260,7 @@ void enqueue_mixed_layer(forge_hip_model* m, uint32_t l, uint32_t pos, const uin
     const forge_hip_config& c = m->cfg;
     Layer& L = m->layers[l];
     hipStream_t s = m->stream;
-    const uint32_t H = m->H, I = m->I, QKS = m->QKS, KV = m->KV, QKV = m->QKV;
+    const uint32_t I = m->I, QKS = m->QKS, KV = m->KV, QKV = m->QKV;
     float* x = m->x.as<float>();
     float* qkv = m->qkv.as<float>();
     float* gu = m->gu.as<float>();
@@ -242,12 +268,10 @@ void enqueue_mixed_layer(forge_hip_model* m, uint32_t l, uint32_t pos, const uin
     uint16_t* asc = m->asc.as<uint16_t>();
     const GemvOrder mv = GemvOrder::MatmulVec;
     const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
-    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, 1, H, nullptr, aq, asc, s); }
     {
-        StageMark t(m, ST_QKV);
-        gemv_any(L.q, aq, asc, qkv, false, mv, s);
-        gemv_any(L.k, aq, asc, qkv + QKS, false, mv, s);
-        gemv_any(L.v, aq, asc, qkv + QKS + KV, false, mv, s);
+        const QWeight* w[3] = {&L.q, &L.k, &L.v};
+        float* y[3] = {qkv, qkv + QKS, qkv + QKS + KV};
+        norm_gemv_group(m, L.attn_norm, w, y, 3, ST_QKV);
     }
     {
         StageMark t(m, ST_ROPE);
@@ -264,11 +288,10 @@ void enqueue_mixed_layer(forge_hip_model* m, uint32_t l, uint32_t pos, const uin
                                m->attn_ws.p, s, m->pt);
     }
     { StageMark t(m, ST_O); gemv_any(L.o, aq, asc, x, true, mv, s); }
-    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, 1, H, nullptr, aq, asc, s); }
     {
-        StageMark t(m, ST_GATE_UP);
-        gemv_any(L.gate, aq, asc, gu, false, mv, s);
-        gemv_any(L.up, aq, asc, gu + I, false, mv, s);
+        const QWeight* w[2] = {&L.gate, &L.up};
+        float* y[2] = {gu, gu + I};
+        norm_gemv_group(m, L.ffn_norm, w, y, 2, ST_GATE_UP);
     }
     { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, 1, I, 2 * I, nullptr, aq, asc, s); }
     { StageMark t(m, ST_DOWN); gemv_any(L.down, aq, asc, x, true, mv, s); }
@@ -314,6 +337,62 @@ void enqueue_decode_layer(forge_hip_model* m, uint32_t l) {
         { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, 1, I, 2 * I, nullptr, aq, asc, s); }
     }
     { StageMark t(m, ST_DOWN); launch_gemv(L.down, aq, asc, x, true, mv, s); }
+}
+
+// M rows through one projection of a model with a format per projection: K-quant matrices with the multi-row GEMV (each row
+// has the one-row kernel's bits), Q8_0 / Q4_0 matrices with the order-faithful GEMM (plain activation codes, as the K-quant
+// kernel takes them).
+void matmul_rows_any(forge_hip_model* m, const QWeight& w, const int8_t* aq, const uint16_t* asc, uint32_t M, float* y, uint32_t ldy,
+                     bool accumulate) {
+    if (w.kquant()) launch_gemv_kquant_rows(w, aq, asc, M, y, ldy, accumulate, m->stream);
+    else launch_gemm(w, aq, asc, M, y, ldy, accumulate, true, nullptr, m->stream, nullptr);
+}
+
+// One decoder layer for M rows of a model with a format per projection.  The reference walks such a prompt token by token
+// (emit.rs:4530-4534, 4621-5040); the operations of a token depend on earlier tokens only through the K/V cache, so a layer can
+// take all rows of a chunk at once: every projection row is the row the one-token kernel computes (K-quant matrices: bit for
+// bit), the cache rows of the chunk are written before attention reads them.  Fast mode: MFMA attention.  Order-faithful mode
+// (only when all seven projections are K-quants, so that no row's bits depend on the batch): attention_flash's own order per row.
+void enqueue_mixed_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t base_pos) {
+    const forge_hip_config& c = m->cfg;
+    Layer& L = m->layers[l];
+    hipStream_t s = m->stream;
+    const uint32_t H = m->H, I = m->I, QKS = m->QKS, KV = m->KV, QKV = m->QKV;
+    float* x = m->px.as<float>();
+    float* qkv = m->pqkv.as<float>();
+    float* gu = m->pgu.as<float>();
+    float* attn = m->pattn.as<float>();
+    int8_t* aq = m->paq.as<int8_t>();
+    uint16_t* asc = m->pasc.as<uint16_t>();
+    const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
+    {
+        StageMark t(m, ST_QKV);
+        matmul_rows_any(m, L.q, aq, asc, M, qkv, QKV, false);
+        matmul_rows_any(m, L.k, aq, asc, M, qkv + QKS, QKV, false);
+        matmul_rows_any(m, L.v, aq, asc, M, qkv + QKS + KV, QKV, false);
+    }
+    {
+        StageMark t(m, ST_ROPE);
+        launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos, nullptr, c.heads, c.kv_heads,
+                             c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), nullptr, s, m->pt);
+    }
+    if (exact) {
+        { StageMark t(m, ST_ATTN); launch_attn_exact(false, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, 0u, c.max_seq, nullptr, s); }
+        { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
+    } else {
+        StageMark t(m, ST_ATTN);
+        launch_attn_prefill_quant(qkv, QKV, m->kc(l), m->vc(l), aq, asc, M, base_pos, c.heads, c.kv_heads, c.head_dim, 0u, s, false, m->pt);
+    }
+    { StageMark t(m, ST_O); matmul_rows_any(m, L.o, aq, asc, M, x, H, true); }
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s); }
+    {
+        StageMark t(m, ST_GATE_UP);
+        matmul_rows_any(m, L.gate, aq, asc, M, gu, 2 * I, false);
+        matmul_rows_any(m, L.up, aq, asc, M, gu + I, 2 * I, false);
+    }
+    { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s); }
+    { StageMark t(m, ST_DOWN); matmul_rows_any(m, L.down, aq, asc, M, x, H, true); }
 }
 
 // One decoder layer of a batched prefill: M rows at positions base_pos.. .
@@ -540,7 +619,18 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
     std::unique_ptr<forge_hip_model> m(new forge_hip_model());
     m->cfg = *cfg;
     m->mixed = pd != nullptr;
-    if (pd) memcpy(m->pd_types, pd, sizeof(m->pd_types));
+    if (pd) {
+        memcpy(m->pd_types, pd, sizeof(m->pd_types));
+        // The prompt runs in batches of rows when no row's bits can depend on the batch in the mode asked for: always in the fast
+        // mode; in the order-faithful mode when all seven projections are K-quants (their multi-row kernel gives every row the
+        // one-row kernel's bits).  FORGE_HIP_MIXED_BATCH=0: token by token, as the reference walks such a prompt.
+        bool all_k = true;
+        for (int i = 0; i < 7; i++) all_k = all_k && is_kquant(pd[i]);
+        const char* benv = getenv("FORGE_HIP_MIXED_BATCH");
+        const char* fenv = getenv("FORGE_HIP_MIXED_FUSE");
+        m->mixed_fuse = !(fenv && fenv[0] == '0');
+        m->mixed_batched = !(benv && benv[0] == '0') && (all_k || !(cfg->flags & FORGE_HIP_FLAG_EXACT));
+    }
     const uint32_t H = m->H = cfg->hidden, I = m->I = cfg->inter;
     const uint32_t QKS = m->QKS = cfg->heads * cfg->head_dim, KV = m->KV = cfg->kv_heads * cfg->head_dim;
     m->QKV = QKS + 2 * KV;
@@ -723,6 +813,30 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint
     for (uint64_t i = 0; i < n; i++)
         if (tokens[i] >= m->cfg.vocab) return fail(FORGE_HIP_ERR_POSITION, "token id out of range");
     hipStream_t s = m->stream;
+    if (m->mixed && m->mixed_batched) {
+        uint64_t fed = 0;
+        uint32_t last_rows = 0;
+        while (fed < n) {
+            const uint32_t rows = (uint32_t)std::min<uint64_t>(m->chunk_rows, n - fed);
+            FH_HIP(hipMemcpyAsync(m->ptok.p, tokens + fed, (size_t)rows * 4, hipMemcpyHostToDevice, s));
+            launch_embedding(m->embed.as<float>(), m->ptok.as<uint32_t>(), rows, m->H, m->px.as<float>(), m->counts.as<uint32_t>(), s);
+            for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_mixed_prefill_layer(m, l, rows, (uint32_t)(m->pos + fed));
+            FH_HIP(hipGetLastError());
+            fed += rows;
+            last_rows = rows;
+        }
+        m->pos += (int64_t)n;
+        m->h_stage[2] = (uint32_t)m->pos;
+        FH_HIP(hipMemcpyAsync(m->d_pos(), &m->h_stage[2], 4, hipMemcpyHostToDevice, s));
+        if (logits_host) {
+            enqueue_head(m, m->px.as<float>() + (size_t)(last_rows - 1) * m->H, true, false);
+            FH_HIP(hipGetLastError());
+            FH_HIP(hipMemcpyAsync(m->h_logits, m->logits.p, (size_t)m->cfg.vocab * 4, hipMemcpyDeviceToHost, s));
+        }
+        FH_HIP(hipStreamSynchronize(s));
+        if (logits_host) memcpy(logits_host, m->h_logits, (size_t)m->cfg.vocab * 4);
+        return FORGE_HIP_OK;
+    }
     if (m->mixed) {
         // forward_prefill of a model that is not uniformly Q8_0 or Q4_0 (emit.rs:4530-4534, 4621-5040): one token at a time
         // through forward's own operations, the lm_head once after the last token
@@ -831,7 +945,17 @@ int32_t forge_hip_model_decode_launches(const forge_hip_model* m) {
     if (m->pd) return (int32_t)pd_launches_per_step(m->pd);
     const bool exact = (m->cfg.flags & FORGE_HIP_FLAG_EXACT) != 0;
     const int attn = exact ? 1 : 2;
-    if (m->mixed) return 1 + (int)m->cfg.layers * (1 + 3 + 1 + attn + 1 + 1 + 2 + 1 + 1) + 4;
+    if (m->mixed) {
+        // a group of projections over the same normed vector: all K-quant -> one launch that norms as well; else the norm, one
+        // launch for the K-quant ones and one for each of the others
+        auto kq = [&](int cat) { return m->pd_types[cat] == FORGE_HIP_Q4_K || m->pd_types[cat] == FORGE_HIP_Q6_K; };
+        auto group = [&](std::initializer_list<int> cats) {
+            int plain = 0, k = 0;
+            for (int cat : cats) (kq(cat) ? k : plain)++;
+            return (plain == 0 && m->mixed_fuse) ? 1 : 1 + plain + (k ? 1 : 0);
+        };
+        return 1 + (int)m->cfg.layers * (group({0, 1, 2}) + 1 + attn + 1 + group({4, 5}) + 2) + 4;
+    }
     const int layer = (m->fuse_norm ? 1 : 3) + attn + 1 + (m->fuse_silu ? 1 : 3) + 1;
     const int head = ((m->fuse_norm && m->cfg.vocab <= 16384) ? 1 : 2) + 2;
     return 1 + (int)m->cfg.layers * layer + head;

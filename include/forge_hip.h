@@ -241,7 +241,9 @@ int32_t forge_hip_gemv_q_f32act(const forge_hip_qweight* w, const float* x_dev, 
  * y[M][N] = x[M][K] W^T, row-major.  With FORGE_HIP_FLAG_EXACT every row has the CPU path's bits.  Without it the block sums
  * are still exact and the f32 combine is within 1e-3, for data whose per-block activation scale is below 256 (largest
  * activation of a block below 32 512) and whose weight scales are below 2: the kernel removes a bias from its block sums with
- * an fp16 matrix instruction on scales multiplied by powers of two, which is exact inside that range only. */
+ * an fp16 matrix instruction on scales multiplied by powers of two, which is exact inside that range only.
+ * A Q4_K / Q6_K handle: the reference has no batched matmul for these formats; the call computes M rows of
+ * matmul_vec_q4_k / _q6_k (each row with forge_hip_gemv_q's bits, whatever `flags` says), reading the matrix once per 8 rows. */
 int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, uint32_t flags,
                          void* stream);
 

@@ -66,6 +66,36 @@ def test_mixed_model_exact_mode_is_bit_identical(fh, oracle, torch_gpu, mix):
     gm.close()
 
 
+@pytest.mark.parametrize("flags", [EXACT, 0])
+def test_mixed_model_prompt_in_batches_equals_token_by_token(fh, torch_gpu, monkeypatch, flags):
+    """A prompt through a K-quant model in batches of rows (every matrix read once per 8 rows) against the reference's
+    token-by-token walk (FORGE_HIP_MIXED_BATCH=0).  Order-faithful mode: logits, cache rows and the tokens that follow, bit
+    for bit (prompt lengths that end inside a batch of 8, at its end, and longer than one chunk would be).  Fast mode: the
+    projections are still the one-row kernel's rows, attention is the MFMA kernel: the first layer's cache rows bit for bit,
+    the logits to the fast mode's bound."""
+    pd, lm = MIXES["q4_k_m"]
+    cfg = tiny(fh, lm, flags)
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=33, std=0.05)
+    monkeypatch.setenv("FORGE_HIP_MIXED_BATCH", "0")
+    walk = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    monkeypatch.delenv("FORGE_HIP_MIXED_BATCH")
+    batch = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    for n in (1, 7, 8, 77):
+        toks = fh.synth.uniform_ids(40 + n, n + 5, cfg["vocab"])
+        walk.reset(); batch.reset()
+        a, b = walk.forward_prefill(toks[:n]), batch.forward_prefill(toks[:n])
+        for which in (0, 1):
+            assert np.array_equal(batch.read_kv(0, which), walk.read_kv(0, which))
+        if flags & EXACT:
+            same_bits(b, a)
+            more_a, more_b = walk.forward_prefill(toks[n:]), batch.forward_prefill(toks[n:])      # a second chunk continues the cache
+            same_bits(more_b, more_a)
+            assert np.array_equal(batch.read_kv(1, 1), walk.read_kv(1, 1))
+        else:
+            assert np.max(np.abs(a - b)) < 0.1 * max(1.0, float(np.std(a)) * 4) and (n < 8 or np.corrcoef(a, b)[0, 1] > 0.99)
+    walk.close(); batch.close()
+
+
 def test_mixed_model_greedy_tokens_at_a_real_width(fh, oracle, torch_gpu):
     """Llama-3.2-1B's widths (hidden 2048 = 8 super-blocks per row, inter 8192, 32:8 heads of 64) in the Q4_K_M recipe:
     prompt + 24 greedy tokens, ids identical to the oracle's."""
@@ -107,6 +137,28 @@ def test_mixed_model_fast_mode(fh, oracle, torch_gpu, mix, monkeypatch):
     for t, want in zip(steps, graph):
         assert np.array_equal(ge.forward(t), want)
     ge.close()
+
+
+def test_mixed_model_grouped_launches_keep_the_bits(fh, torch_gpu, monkeypatch):
+    """K-quant projections that read the same normed row (q, k, v; gate, up) go out as ONE launch that norms and quantises
+    the row itself; FORGE_HIP_MIXED_FUSE=0 keeps the norm kernel in front.  Same logits and cache rows bit for bit, fewer
+    launches per step.  A mix with a Q8_0 matrix in the group keeps the norm kernel for it."""
+    for mix, fewer in (("q4_k_m", True), ("all_four", False)):
+        pd, lm = MIXES[mix]
+        cfg = tiny(fh, lm, EXACT)
+        blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=5, std=0.05)
+        toks = fh.synth.uniform_ids(9, 19, cfg["vocab"])
+        monkeypatch.setenv("FORGE_HIP_MIXED_FUSE", "0")
+        plain = fh.HipModel(cfg, blob, proj_dtypes=pd)
+        monkeypatch.delenv("FORGE_HIP_MIXED_FUSE")
+        fused = fh.HipModel(cfg, blob, proj_dtypes=pd)
+        assert (fused.decode_launches < plain.decode_launches) == fewer
+        same_bits(fused.forward_prefill(toks), plain.forward_prefill(toks))
+        for t in (3, 77, 500):
+            same_bits(fused.forward(t), plain.forward(t))
+        for layer in range(cfg["layers"]):
+            assert np.array_equal(fused.read_kv(layer, 0), plain.read_kv(layer, 0))
+        plain.close(); fused.close()
 
 
 def test_uniform_formats_through_the_mixed_entry_point_are_the_plain_model(fh, torch_gpu):

@@ -167,8 +167,12 @@ def test_matmul_vec_kquant_bit_exact(fh, oracle, torch_gpu, ty, K, N):
     w = fh.ops.QWeight(ty, wraw, K, N)
     y = fh.ops.matmul_vec_q(w, torch.from_numpy(x).cuda()).cpu().numpy()
     same_bits(y, oracle.matmul_vec_kquant(ty, x, wraw, K, N))
-    with pytest.raises(fh.ForgeHipError):
-        fh.ops.matmul_mat_q(w, torch.from_numpy(np.stack([x, x])).cuda())       # no batched matmul for these formats
+    # M rows at once: the reference has no batched matmul for these formats, so every row is matmul_vec's, bit for bit,
+    # whatever its place in the batch (1 row, a ragged 11, more than one workgroup's 8)
+    rows = np.stack([x, -x, 0.5 * x] + [fh.synth.normal(31 + i, K, 1.0) for i in range(8)])
+    want = np.stack([oracle.matmul_vec_kquant(ty, r, wraw, K, N) for r in rows])
+    for M in (1, 11):
+        same_bits(fh.ops.matmul_mat_q(w, torch.from_numpy(rows[:M]).cuda()).cpu().numpy(), want[:M])
     w.close()
     with pytest.raises(fh.ForgeHipError):
         fh.ops.QWeight(ty, random_superblocks(ty, 1, 1), 288, 1)                # K must be a multiple of 256
