@@ -10,7 +10,7 @@ INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 BUILD = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libforge_hip.so")
 
-SOURCES = ["format.hip", "elementwise.hip", "gemv.hip", "gemv_f32.hip", "gemv_kquant.hip", "gemm.hip", "attn_decode.hip", "attn_prefill.hip",
+SOURCES = ["format.hip", "elementwise.hip", "gemv.hip", "gemv_f32.hip", "gemv_kquant.hip", "kquant_prefill.hip", "gemm.hip", "attn_decode.hip", "attn_prefill.hip",
            "attn_exact.hip", "decode_persistent.hip", "api.hip", "model.hip", "gguf.cpp", "sampling.cpp"]
 
 # -packed-fp32-ops off: keep hipcc from forming packed FP32 instructions.

@@ -54,6 +54,7 @@ Scratch g_act;    // quantised activations: codes then scales
 Scratch g_attn;   // decode-attention partials / argmax partials
 Scratch g_rope;   // cos | sin tables
 Scratch g_gemm;   // partial tiles and counters of the GEMM's K-range variant
+Scratch g_twin;   // K-quant twins: block sums of the activations, or the activations with every block twice
 
 inline size_t align256(size_t n) { return (n + 255) & ~(size_t)255; }
 
@@ -76,7 +77,12 @@ int32_t quantise_into_scratch(const float* x, uint32_t M, uint32_t K, int8_t** q
 
 using namespace fh;
 
-struct forge_hip_qweight { QWeight w; };
+struct forge_hip_qweight {
+    QWeight w;
+    // K-quant matrices: the matrix as the int8 MFMA GEMM takes it, built by the first forge_hip_gemm_q without FLAG_EXACT
+    KqTwin twin;
+    bool twin_tried = false, twin_covered = false;
+};
 
 extern "C" {
 
@@ -126,6 +132,7 @@ int32_t forge_hip_qweight_create(uint32_t wdtype, const uint8_t* raw_host, uint3
 void forge_hip_qweight_destroy(forge_hip_qweight* w) {
     if (!w) return;
     qweight_free(&w->w);
+    kquant_twin_free(&w->twin);
     delete w;
 }
 
@@ -156,16 +163,51 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
     FH_CHECK((flags & ~FORGE_HIP_FLAG_EXACT) == 0, "gemm_q: unknown flag bits");
     if (M == 0) return FORGE_HIP_OK;
     int8_t* q; uint16_t* sc;
+    const bool exact = (flags & FORGE_HIP_FLAG_EXACT) != 0;
     if (w->w.kquant()) {
-        // the reference has no batched matmul for these formats: M rows of matmul_vec, the matrix read once per 8 rows
         FH_CHECK(kquant_k_supported(w->w.K), "gemm_q: K must be a multiple of 256, at most 16384");
-        int32_t rck = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream, false);
+        hipStream_t s = (hipStream_t)stream;
+        forge_hip_qweight* h = const_cast<forge_hip_qweight*>(w);
+        if (!exact && !h->twin_tried) {
+            int32_t rct = kquant_twin_create(h->w, &h->twin, &h->twin_covered, s);
+            if (rct) return rct;
+            h->twin_tried = true;
+        }
+        if (exact || !h->twin_covered) {
+            // the reference has no batched matmul for these formats: M rows of matmul_vec, the matrix read once per 8 rows
+            int32_t rck = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, s, false);
+            if (rck) return rck;
+            launch_gemv_kquant_rows(w->w, q, sc, M, y_dev, w->w.N, false, s);
+            FH_HIP(hipGetLastError());
+            return FORGE_HIP_OK;
+        }
+        // fast mode: the matrix's twin on the int8 MFMA GEMM (kquant_prefill.hip)
+        const uint32_t K = w->w.K;
+        int32_t rck = quantise_into_scratch(x_dev, M, K, &q, &sc, s, true);
         if (rck) return rck;
-        launch_gemv_kquant_rows(w->w, q, sc, M, y_dev, w->w.N, false, (hipStream_t)stream);
+        void* split_ws = nullptr;
+        if (M > 64) {
+            const bool fresh = g_gemm.cap < gemm_split_workspace_bytes();
+            if ((rck = g_gemm.reserve(gemm_split_workspace_bytes()))) return rck;
+            if (fresh) FH_HIP(hipMemsetAsync(g_gemm.p, 0, gemm_split_workspace_bytes(), s));
+            split_ws = g_gemm.p;
+        }
+        if (h->twin.coef) {
+            if ((rck = g_twin.reserve((size_t)M * (K / 32) * 4))) return rck;
+            launch_act_block_sums(q, sc, M, K, true, reinterpret_cast<float*>(g_twin.p), s);
+            launch_gemm(h->twin.w, q, sc, M, y_dev, w->w.N, false, false, nullptr, s, split_ws);
+            launch_kq_min_term(reinterpret_cast<const float*>(g_twin.p), h->twin.coef, M, w->w.N, K, y_dev, w->w.N, s);
+        } else {
+            const size_t qbytes = align256((size_t)M * K * 2);
+            if ((rck = g_twin.reserve(qbytes + (size_t)M * (K / 32) * 4))) return rck;
+            int8_t* q2 = reinterpret_cast<int8_t*>(g_twin.p);
+            uint16_t* sc2 = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(g_twin.p) + qbytes);
+            launch_act_twice(q, sc, M, K, q2, sc2, s);
+            launch_gemm(h->twin.w, q2, sc2, M, y_dev, w->w.N, false, false, nullptr, s, split_ws);
+        }
         FH_HIP(hipGetLastError());
         return FORGE_HIP_OK;
     }
-    const bool exact = (flags & FORGE_HIP_FLAG_EXACT) != 0;
     int32_t rc = quantise_into_scratch(x_dev, M, w->w.K, &q, &sc, (hipStream_t)stream, !exact);   // the fast kernel takes odd blocks negated
     if (rc) return rc;
     // fast mode may cut tiles along K to fill the CUs: that kernel parks partial tiles in a workspace

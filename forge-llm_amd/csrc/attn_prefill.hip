@@ -296,7 +296,8 @@ void attn_prefill_kernel(const float* __restrict__ q, const uint16_t* __restrict
                                         (((uint32_t)quant_code(o[4 * g + 2] * inv) & 0xFFu) << 16) | (((uint32_t)quant_code(o[4 * g + 3] * inv) & 0xFFu) << 24);
                     *reinterpret_cast<uint32_t*>(oq + (size_t)qrow * width + head * HD + 32 * d + 8 * g + 4 * lh) = pk;
                 }
-                if (lh == 0) osc[(size_t)qrow * (width / 32) + head * (HD / 32) + d] = f32_to_f16_bits(sc);
+                // (for the fast GEMM an all-zero block carries the scale 0, see quantize_block_part)
+                if (lh == 0) osc[(size_t)qrow * (width / 32) + head * (HD / 32) + d] = (out_stride != 0 && amax == 0.f) ? (uint16_t)0 : f32_to_f16_bits(sc);
             }
         }
         return;

@@ -102,7 +102,8 @@ __device__ __forceinline__ size_t paged_row(const PageTable& pt, uint32_t t) {
 // All are asynchronous on `s` and validate nothing: callers check shapes first.
 
 // elementwise.hip
-// neg_odd (here and below): the codes of a row's odd blocks are stored negated, as the fast prefill GEMM takes them.
+// neg_odd (here and below): the codes of a row's odd blocks are stored negated and an all-zero block gets the scale 0
+// (the reference's quantiser gives it 1.0), as the fast prefill GEMM takes them.
 void launch_quantize_act(const float* x, uint32_t M, uint32_t K, int8_t* q, uint16_t* sc, hipStream_t s, bool neg_odd = false);
 // rms_norm of M rows; writes f32 `normed` if non-null and the quantised row (q, sc) if q non-null.
 void launch_rmsnorm(const float* x, const float* w, float eps, uint32_t M, uint32_t H, float* normed, int8_t* q,
@@ -161,6 +162,22 @@ void launch_gemv_kquant_multi(const QWeight* const* w, float* const* y, uint32_t
 // ... over quantise(rms_norm(x) * norm_w), normed and quantised inside the kernel (the norm kernel's bits).
 void launch_gemv_kquant_multi_norm(const QWeight* const* w, float* const* y, uint32_t n, const float* x, const float* norm_w, float eps,
                                    hipStream_t s);
+// kquant_prefill.hip -- K-quant matrices on the int8 MFMA GEMM (fast mode).  The twin of a matrix is the same weights in
+// the Q8_0 layout: Q4_K as codes (q - 8) * g of depth K plus one f32 coefficient per (row, block) for the minimum term,
+// Q6_K as the hi and lo parts of sc * q, two blocks per block (depth 2K), under the exact scales 64 d and d.
+struct KqTwin {
+    QWeight w;                 // Q8_0 layout, [N][K] (Q4_K) or [N][2K] (Q6_K)
+    float* coef = nullptr;     // Q4_K: [N][K/32], 8 * d * sc - dmin * min
+    bool present() const { return w.qs != nullptr; }
+};
+int32_t kquant_twin_create(const QWeight& w, KqTwin* out, bool* covered, hipStream_t s);
+void kquant_twin_free(KqTwin* t);
+// out[m][b] = a_s[m][b] * (sum of block b's codes), f32 [M][K/32]
+void launch_act_block_sums(const int8_t* aq, const uint16_t* as, uint32_t M, uint32_t K, bool neg_odd, float* out, hipStream_t s);
+// every pair of blocks twice: codes [M][2K], scales [M][2K/32]; blocks 2p, 2p + 1 -> 2p, 2p + 1, 2p, 2p + 1
+void launch_act_twice(const int8_t* aq, const uint16_t* as, uint32_t M, uint32_t K, int8_t* oq, uint16_t* os, hipStream_t s);
+// y[m][n] += sum_b block_sums[m][b] * coef[n][b]
+void launch_kq_min_term(const float* block_sums, const float* coef, uint32_t M, uint32_t N, uint32_t K, float* y, uint32_t ldy, hipStream_t s);
 // The same for M rows of quantised activations (codes [M][K], scales [M][K/32]); rows of y are ldy floats apart.  Every row has the
 // bits launch_gemv_kquant gives it alone.
 void launch_gemv_kquant_rows(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy, bool accumulate,

@@ -111,14 +111,17 @@ __device__ __forceinline__ float half_wave_max(float v) {
 // Returns the packed 4 int8 codes; lane%8==0 also gets the fp16 scale bits via `scale_bits`.
 // `negate`: store -code instead of code (the scale stays positive): the fast prefill GEMM wants the odd blocks of a row
 // that way (gemm.hip).
-__device__ __forceinline__ uint32_t quantize_block_part(float4 v, uint16_t& scale_bits, bool negate = false) {
+// `empty_zero`: an all-zero block gets the scale 0 instead of the reference's 1.0.  Its codes are zero either way; the fast
+// prefill GEMM adds scale * (bias +- block sum) per block, and a scale of 1.0 next to neighbours of 0.01 would push the
+// running sums to a magnitude where their low bits are lost.
+__device__ __forceinline__ uint32_t quantize_block_part(float4 v, uint16_t& scale_bits, bool negate = false, bool empty_zero = false) {
     float amax = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
     amax = lane_xor_max<1>(amax);
     amax = lane_xor_max<2>(amax);
     amax = lane_xor_max<4>(amax);
     float inv;
     float s = act_scale(amax, inv);
-    scale_bits = f32_to_f16_bits(s);
+    scale_bits = (empty_zero && amax == 0.0f) ? (uint16_t)0 : f32_to_f16_bits(s);
     if (negate) inv = -inv;          // rounding and clamping are symmetric: round(-x) = -round(x)
     uint32_t q0 = (uint32_t)quant_code(v.x * inv) & 0xFFu;
     uint32_t q1 = (uint32_t)quant_code(v.y * inv) & 0xFFu;

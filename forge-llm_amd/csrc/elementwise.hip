@@ -17,7 +17,7 @@ __global__ __launch_bounds__(256) void quantize_act_kernel(const float* __restri
     if (i < n4) v = reinterpret_cast<const float4*>(x)[i];
     uint16_t sb;
     const bool neg = neg_odd_blocks_per_row != 0 && (((i >> 3) % neg_odd_blocks_per_row) & 1) != 0;
-    uint32_t packed = quantize_block_part(v, sb, neg);
+    uint32_t packed = quantize_block_part(v, sb, neg, neg_odd_blocks_per_row != 0);
     if (i < n4) {
         q[i] = packed;
         if ((i & 7) == 0) sc[i >> 3] = sb;
@@ -82,7 +82,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
         }
         if (q) {
             uint16_t sb;
-            uint32_t packed = quantize_block_part(o, sb, neg_odd != 0 && ((i >> 3) & 1) != 0);
+            uint32_t packed = quantize_block_part(o, sb, neg_odd != 0 && ((i >> 3) & 1) != 0, neg_odd != 0);
             if (i < n4) {
                 q[(size_t)row * n4 + i] = packed;
                 if ((i & 7) == 0) sc[(size_t)row * (H / 32) + (i >> 3)] = sb;
@@ -118,7 +118,7 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const float* __restrict__
     }
     if (q) {
         uint16_t sb;
-        uint32_t packed = quantize_block_part(o, sb, neg);
+        uint32_t packed = quantize_block_part(o, sb, neg, neg_odd != 0);
         if (i < total4) {
             q[i] = packed;
             if ((i & 7) == 0) sc[i >> 3] = sb;

@@ -468,7 +468,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
                 // on exact ties only); |o * inv| <= 127 up to rounding, so the conversion needs no clamp
                 const float o = g * __builtin_amdgcn_rcpf(1.0f + __expf(-g)) * u;
                 const float amax = half_wave_max(fabsf(o));               // the 32 lanes that share lhalf: one block of one row
-                const float scl = amax > 0.f ? amax * (1.0f / 127.0f) : 1.0f;
+                const float scl = amax * (1.0f / 127.0f);                 // an all-zero block: scale 0 (see quantize_block_part)
                 float inv = amax > 0.f ? 127.0f * __builtin_amdgcn_rcpf(amax) : 0.f;
                 if (blk & 1u) inv = -inv;                                 // odd blocks negated for the GEMM that reads them
                 const uint32_t code = (uint32_t)(int)__builtin_rintf(o * inv) & 0xFFu;

@@ -1,0 +1,249 @@
+// Prompt matmuls for K-quant weights on the matrix unit (fast mode).
+//
+// The reference multiplies a Q4_K / Q6_K matrix one vector at a time (matmul_vec_q4_k_KxN, emit.rs:3388-3490; matmul_vec_q6_k_KxN,
+// emit.rs:3622-3655) and walks a prompt through such a model token by token (emit.rs:4530-4534).  The order-faithful mode
+// keeps that arithmetic (gemv_kquant.hip).  The fast mode re-expresses each matrix, once, as a matrix the int8 MFMA GEMM
+// (gemm.hip) already multiplies -- int8 codes under one fp16 scale per block of 32, the Q8_0 layout -- its "twin":
+//
+//   Q4_K  w = d*sc_j * q - dmin*m_j, q = 0..15, per 32-element sub-block j, i.e.
+//             sum_k x_k w_k  =  d*sc_j * sum x_k (q_k - 8)  +  (8 d*sc_j - dmin*m_j) * sum x_k
+//         First term: codes (q - 8) * g under the scale fp16(d*sc_j / g), with the integer g = 9..15 that brings g * fp16(d*sc_j / g)
+//         closest to d*sc_j (d*sc_j has up to 17 significant bits, fp16 has 11: among seven distinct roundings the best is
+//         typically within 4e-5 of it, relative; that residue times the block's centred dot product is all that is dropped).
+//         Second term: the block sums of the activations times an f32 coefficient per (row, block), a small f32 matmul of
+//         depth K/32 (kq_min_term_kernel).
+//   Q6_K  w = d * sc_h * q, q = -32..31, sc_h an int8 per 16-element half.  sc_h * q = 64 hi + lo with lo in [-32, 31] and hi
+//         in [-63, 64]: a block becomes two blocks of a matrix of depth 2K, the hi codes under the scale 64 d and the lo codes
+//         under d.  Both scales are exact fp16 numbers (d is one), so nothing is dropped at all; the activations go in twice
+//         (act_twice_kernel).  Blocks 2p, 2p + 1 of a row become hi(2p), hi(2p + 1), lo(2p), lo(2p + 1): neighbours of equal
+//         scale, which is what the GEMM's alternating bias wants.
+//
+// Integer block sums stay exact; against the order-faithful result the difference is the order of the f32 additions and, for
+// Q4_K, the residue above.
+#include "common.h"
+#include "device_utils.h"
+
+namespace fh {
+
+namespace {
+
+// One thread per (row, 32-element block).  Planes of the source as gemv_kquant.hip lays them out.
+__global__ __launch_bounds__(256) void twin_q4k_kernel(const uint8_t* __restrict__ qs, const uint8_t* __restrict__ meta, uint32_t K, uint64_t total,
+                                                     int8_t* __restrict__ tq, uint16_t* __restrict__ ts, float* __restrict__ coef,
+                                                     uint32_t* __restrict__ bad) {
+    const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;       // n * nblk + b
+    if (id >= total) return;
+    const uint32_t nblk = K / 32;
+    const uint64_t n = id / nblk;
+    const uint32_t b = (uint32_t)(id % nblk), sb = b >> 3, j = b & 7, c = j >> 1;
+    const uint8_t* mp = meta + (n * (K / 256) + sb) * 16;
+    const float d = f16_bits_to_f32((uint16_t)(mp[0] | (mp[1] << 8))), dmin = f16_bits_to_f32((uint16_t)(mp[2] | (mp[3] << 8)));
+    const uint8_t* s12 = mp + 4;
+    uint32_t sc, mn;                                                       // get_scale_min_k4, emit.rs:3013-3021
+    if (j < 4) { sc = s12[j] & 63u; mn = s12[j + 4] & 63u; }
+    else {
+        sc = (s12[j + 4] & 0x0Fu) | ((s12[j - 4] >> 6) << 4);
+        mn = (s12[j + 4] >> 4) | ((s12[j] >> 6) << 4);
+    }
+    const float s = d * (float)sc;                                         // exact: 11 x 6 bits
+    if (!(s >= 0.f) || !(s < 2.0f)) *bad = 1u;                             // outside what the GEMM's scale arithmetic covers
+    // multipliers 9..15: seven different roundings (their odd parts differ), and codes that use the int8 range, which keeps
+    // the GEMM's accumulation error small against the block sums
+    int g = 15;
+    uint16_t s16 = f32_to_f16_bits(s / 15.0f);
+    float err = fabsf(f16_bits_to_f32(s16) * 15.0f - s);
+    for (int cand = 14; cand >= 9; cand--) {
+        const uint16_t h = f32_to_f16_bits(s / (float)cand);
+        const float e = fabsf(f16_bits_to_f32(h) * (float)cand - s);
+        if (e < err) { err = e; g = cand; s16 = h; }
+    }
+    ts[id] = s16;
+    coef[id] = 8.0f * s - dmin * (float)mn;
+    // sub-block j = 2c + hi: element i is the low (hi = 0) or high nibble of byte 32 c + i
+    const uint8_t* src = qs + (n * (K / 256) + sb) * 128 + 32 * c;
+    const uint32_t sh = (j & 1) * 4;
+    int8_t* dst = tq + id * 32;
+    for (uint32_t i = 0; i < 32; i++) dst[i] = (int8_t)(((int)((src[i] >> sh) & 15u) - 8) * g);
+}
+
+__global__ __launch_bounds__(256) void twin_q6k_kernel(const uint8_t* __restrict__ qs, const uint8_t* __restrict__ meta, uint32_t K, uint64_t total,
+                                                     int8_t* __restrict__ tq, uint16_t* __restrict__ ts, uint32_t* __restrict__ bad) {
+    const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;       // n * nblk + b
+    if (id >= total) return;
+    const uint32_t nblk = K / 32;
+    const uint64_t n = id / nblk;
+    const uint32_t b = (uint32_t)(id % nblk), sb = b >> 3, jb = b & 7, h = jb >> 2, r = jb & 3;
+    const uint8_t* sp = qs + (n * (K / 256) + sb) * 192;
+    const uint8_t* mp = meta + (n * (K / 256) + sb) * 32;
+    const float d = f16_bits_to_f32((uint16_t)(mp[16] | (mp[17] << 8)));
+    const float mag = fabsf(d);
+    if (!(mag * 64.0f < 2.0f)) *bad = 1u;
+    const int sign = d < 0.f ? -1 : 1;
+    // block 4h + r of the super-block: r = 0, 1 the low nibbles of ql[64h + 32r ..], r = 2, 3 the high nibbles of
+    // ql[64h + 32(r - 2) ..]; bit pair r of qh[32h ..]
+    const uint8_t* ql = sp + 64 * h + 32 * (r & 1);
+    const uint8_t* qh = sp + 128 + 32 * h;
+    const uint32_t nib_shift = (r >> 1) * 4, pair_shift = 2 * r;
+    // blocks 2p + e of the row -> twin blocks 4p + e (hi) and 4p + 2 + e (lo)
+    const uint64_t tb = n * 2 * nblk + 4 * (uint64_t)(b >> 1) + (b & 1);
+    ts[tb] = f32_to_f16_bits(mag * 64.0f);                                 // exact: a power of two times an fp16 number
+    ts[tb + 2] = f32_to_f16_bits(mag);
+    int8_t* dst = tq + tb * 32;
+    for (uint32_t i = 0; i < 32; i++) {
+        const int q = (int)(((ql[i] >> nib_shift) & 15u) | (((qh[i] >> pair_shift) & 3u) << 4)) - 32;
+        const int p = sign * (int)(int8_t)mp[2 * jb + (i >> 4)] * q;       // |p| <= 4096
+        const int hi = (p + 32) >> 6;                                      // floor((p + 32) / 64): arithmetic shift
+        dst[i] = (int8_t)hi;
+        dst[64 + i] = (int8_t)(p - 64 * hi);
+    }
+}
+
+// a_s[m][b] * sum of block b's codes, f32 [M][K/32].  `neg_odd`: the codes of odd blocks arrive negated.
+__global__ __launch_bounds__(256) void act_block_sums_kernel(const int8_t* __restrict__ aq, const uint16_t* __restrict__ as, uint64_t total,
+                                                           uint32_t nblk, uint32_t neg_odd, float* __restrict__ out) {
+    const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;       // m * nblk + b
+    if (id >= total) return;
+    const int4* p = reinterpret_cast<const int4*>(aq + id * 32);
+    const int4 a0 = p[0], a1 = p[1];
+    const int ones = 0x01010101;
+    int sum = 0;
+    sum = __builtin_amdgcn_sdot4(a0.x, ones, sum, false); sum = __builtin_amdgcn_sdot4(a0.y, ones, sum, false);
+    sum = __builtin_amdgcn_sdot4(a0.z, ones, sum, false); sum = __builtin_amdgcn_sdot4(a0.w, ones, sum, false);
+    sum = __builtin_amdgcn_sdot4(a1.x, ones, sum, false); sum = __builtin_amdgcn_sdot4(a1.y, ones, sum, false);
+    sum = __builtin_amdgcn_sdot4(a1.z, ones, sum, false); sum = __builtin_amdgcn_sdot4(a1.w, ones, sum, false);
+    if (neg_odd && ((id % nblk) & 1u)) sum = -sum;
+    out[id] = f16_bits_to_f32(as[id]) * (float)sum;
+}
+
+// Every pair of activation blocks twice, [M][2 K/32] blocks: blocks 2p, 2p + 1 of a row become 2p, 2p + 1, 2p, 2p + 1 (the hi
+// and the lo blocks of a Q6_K twin meet the same activations).  Odd blocks stay odd, so codes that arrive with their odd
+// blocks negated leave that way.
+__global__ __launch_bounds__(256) void act_twice_kernel(const int8_t* __restrict__ aq, const uint16_t* __restrict__ as, uint64_t pairs,
+                                                      int8_t* __restrict__ oq, uint16_t* __restrict__ os) {
+    const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;       // pair * 4 + sixteen-byte quarter of the pair
+    if (id >= pairs * 4) return;
+    const uint64_t pair = id >> 2;
+    const uint32_t part = (uint32_t)(id & 3);
+    const int4 v = reinterpret_cast<const int4*>(aq)[id];
+    int4* o = reinterpret_cast<int4*>(oq);
+    o[pair * 8 + part] = v;
+    o[pair * 8 + 4 + part] = v;
+    if (part == 0) {
+        const uint32_t s2 = reinterpret_cast<const uint32_t*>(as)[pair];
+        reinterpret_cast<uint32_t*>(os)[pair * 2] = s2;
+        reinterpret_cast<uint32_t*>(os)[pair * 2 + 1] = s2;
+    }
+}
+
+// y[m][n] += sum_b bs[m][b] * coef[n][b]: the minimum term of a Q4_K matrix for M rows.  One wave per 32 x 32 tile of y,
+// v_mfma_f32_32x32x2_f32; a lane fetches four consecutive b of its row per operand (the order of k inside the sum is free), so
+// eight b go through four MFMAs.  Both operands are small and re-read from L2.
+__global__ __launch_bounds__(256) void kq_min_term_kernel(const float* __restrict__ bs, const float* __restrict__ coef, uint32_t M, uint32_t N,
+                                                        uint32_t nblk, float* __restrict__ y, uint32_t ldy) {
+    typedef float v16f __attribute__((ext_vector_type(16)));
+    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t m0 = blockIdx.y * 64 + (wave >> 1) * 32, n0 = blockIdx.x * 64 + (wave & 1) * 32;
+    if (m0 >= M || n0 >= N) return;
+    const uint32_t lrow = lane & 31, lhalf = lane >> 5;
+    const float* ap = bs + (size_t)min(m0 + lrow, M - 1) * nblk + 4 * lhalf;
+    const float* bp = coef + (size_t)min(n0 + lrow, N - 1) * nblk + 4 * lhalf;
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    for (uint32_t g = 0; g < nblk; g += 8) {
+        const float4 a = *reinterpret_cast<const float4*>(ap + g), b = *reinterpret_cast<const float4*>(bp + g);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc, 0, 0, 0);
+    }
+    // lane holds column n0 + lrow, rows m0 + 8 (r / 4) + 4 lhalf + r % 4
+    const uint32_t n = n0 + lrow;
+    if (n >= N) return;
+    float old[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const uint32_t m = m0 + 8 * (r >> 2) + 4 * lhalf + (r & 3);
+        old[r] = m < M ? y[(size_t)m * ldy + n] : 0.f;
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const uint32_t m = m0 + 8 * (r >> 2) + 4 * lhalf + (r & 3);
+        if (m < M) y[(size_t)m * ldy + n] = old[r] + acc[r];
+    }
+}
+
+}  // namespace
+
+// `*covered` = false (and no twin) when a block scale lies outside what the fast GEMM's scale arithmetic covers (a negative
+// Q4_K scale, d * sc or 64 |d| not below 2): the caller keeps the multi-row GEMV for that matrix.
+int32_t kquant_twin_create(const QWeight& w, KqTwin* out, bool* covered, hipStream_t s) {
+    *covered = false;
+    if (!w.kquant() || w.K % 256 != 0) { set_error("kquant twin: not a K-quant matrix"); return FORGE_HIP_ERR_INVALID; }
+    const uint32_t nblk = w.K / 32;
+    const uint64_t total = (uint64_t)w.N * nblk;
+    const bool q6 = w.wdtype == FORGE_HIP_Q6_K;
+    QWeight t;
+    t.wdtype = FORGE_HIP_Q8_0;
+    t.K = q6 ? 2 * w.K : w.K;
+    t.N = w.N;
+    t.owns = true;
+    uint32_t* bad = nullptr;
+    float* coef = nullptr;
+    auto fail = [&](int32_t rc) {
+        if (t.qs) (void)hipFree(t.qs);
+        if (t.scales) (void)hipFree(t.scales);
+        if (coef) (void)hipFree(coef);
+        if (bad) (void)hipFree(bad);
+        return rc;
+    };
+    if (hipMalloc(&t.qs, t.qs_bytes()) != hipSuccess || hipMalloc(&t.scales, t.scales_bytes()) != hipSuccess ||
+        hipMalloc(&bad, 4) != hipSuccess || (!q6 && hipMalloc(&coef, total * 4) != hipSuccess)) {
+        (void)hipGetLastError();
+        set_error("kquant twin: out of device memory");
+        return fail(FORGE_HIP_ERR_HIP);
+    }
+    if (hipMemsetAsync(bad, 0, 4, s) != hipSuccess) return fail(FORGE_HIP_ERR_HIP);
+    const uint32_t grid = (uint32_t)((total + 255) / 256);
+    const uint8_t* meta = reinterpret_cast<const uint8_t*>(w.scales);
+    if (q6) fh::launch(twin_q6k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, reinterpret_cast<int8_t*>(t.qs), t.scales, bad);
+    else fh::launch(twin_q4k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, reinterpret_cast<int8_t*>(t.qs), t.scales, coef, bad);
+    uint32_t flag = 0;
+    if (hipMemcpyAsync(&flag, bad, 4, hipMemcpyDeviceToHost, s) != hipSuccess || hipStreamSynchronize(s) != hipSuccess) {
+        set_error("kquant twin: conversion kernel failed");
+        return fail(FORGE_HIP_ERR_HIP);
+    }
+    (void)hipFree(bad);
+    bad = nullptr;
+    if (flag) return fail(FORGE_HIP_OK);
+    *covered = true;
+    out->w = t;
+    out->coef = coef;
+    return FORGE_HIP_OK;
+}
+
+void kquant_twin_free(KqTwin* t) {
+    if (!t) return;
+    qweight_free(&t->w);
+    if (t->coef) (void)hipFree(t->coef);
+    t->coef = nullptr;
+}
+
+void launch_act_block_sums(const int8_t* aq, const uint16_t* as, uint32_t M, uint32_t K, bool neg_odd, float* out, hipStream_t s) {
+    const uint64_t total = (uint64_t)M * (K / 32);
+    if (total == 0) return;
+    fh::launch(act_block_sums_kernel, (uint32_t)((total + 255) / 256), 256, 0, s, aq, as, total, K / 32, neg_odd ? 1u : 0u, out);
+}
+
+void launch_act_twice(const int8_t* aq, const uint16_t* as, uint32_t M, uint32_t K, int8_t* oq, uint16_t* os, hipStream_t s) {
+    const uint64_t pairs = (uint64_t)M * (K / 64);
+    if (pairs == 0) return;
+    fh::launch(act_twice_kernel, (uint32_t)((pairs * 4 + 255) / 256), 256, 0, s, aq, as, pairs, oq, os);
+}
+
+void launch_kq_min_term(const float* block_sums, const float* coef, uint32_t M, uint32_t N, uint32_t K, float* y, uint32_t ldy, hipStream_t s) {
+    if (M == 0 || N == 0) return;
+    fh::launch(kq_min_term_kernel, dim3((N + 63) / 64, (M + 63) / 64), 256, 0, s, block_sums, coef, M, N, K / 32, y, ldy);
+}
+
+}  // namespace fh

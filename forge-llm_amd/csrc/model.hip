@@ -29,6 +29,7 @@ struct Layer {
     float* ffn_norm = nullptr;
     QWeight qkv, o, gate_up, down;
     QWeight q, k, v, gate, up;           // a model with a storage format per projection keeps these five apart (qkv, gate_up unused)
+    KqTwin twin[7];                      // fast mode: the K-quant ones among q, k, v, o, gate, up, down as matrices of the int8 MFMA GEMM
     float* qkv_bias = nullptr;           // [QKS + 2 KV]: q | k | v bias, in the row order of the fused qkv matrix (FLAG_QKV_BIAS)
 };
 
@@ -68,6 +69,8 @@ struct forge_hip_model {
     float repeat_penalty = 1.0f;         // > 1: forward_greedy picks the maximum of the penalised logits
     // prefill scratch (chunk_rows rows)
     DevBuf px, pqkv, pattn, pgu, paq, pasc, paq2, pasc2, ptok;
+    DevBuf pbsum, paq3, pasc3;           // K-quant twins: block sums of the activations (f32), the activations with every block twice
+    bool mixed_twins = false;            // fast mode: K-quant projections of a prompt run on the MFMA GEMM (kquant_prefill.hip)
     bool prefill_fuse_quant = true;              // fast mode: attention writes int8 codes + scales (FORGE_HIP_FUSE=0: separate quantiser)
     bool mixed_fuse = true;          // K-quant projections over a normed row norm and quantise it themselves: a launch less, the same bits
     bool mixed_batched = false;                  // per-projection formats: the prompt runs in batches of rows (see enqueue_mixed_prefill_layer)
@@ -106,6 +109,7 @@ struct forge_hip_model {
         for (auto& L : layers) {
             qweight_free(&L.qkv); qweight_free(&L.o); qweight_free(&L.gate_up); qweight_free(&L.down);
             qweight_free(&L.q); qweight_free(&L.k); qweight_free(&L.v); qweight_free(&L.gate); qweight_free(&L.up);
+            for (KqTwin& t : L.twin) kquant_twin_free(&t);
         }
         qweight_free(&lm_head);
         if (h_stage) (void)hipHostFree(h_stage);
@@ -393,6 +397,88 @@ void enqueue_mixed_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uin
     }
     { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s); }
     { StageMark t(m, ST_DOWN); matmul_rows_any(m, L.down, aq, asc, M, x, H, true); }
+}
+
+// What the twins among `tw` need of the quantised rows in (paq, pasc) (odd blocks negated): Q4_K twins the scaled block sums,
+// Q6_K twins every block twice.
+static void twin_inputs(forge_hip_model* m, const QWeight* const* w, const KqTwin* const* tw, int n, uint32_t M, uint32_t K) {
+    bool sums = false, twice = false;
+    for (int i = 0; i < n; i++) {
+        if (!w[i]->kquant()) continue;
+        (tw[i]->coef ? sums : twice) = true;
+    }
+    if (sums) launch_act_block_sums(m->paq.as<int8_t>(), m->pasc.as<uint16_t>(), M, K, true, m->pbsum.as<float>(), m->stream);
+    if (twice) launch_act_twice(m->paq.as<int8_t>(), m->pasc.as<uint16_t>(), M, K, m->paq3.as<int8_t>(), m->pasc3.as<uint16_t>(), m->stream);
+}
+
+// y (=|+=) rows * W^T on the MFMA GEMM, whatever W's format (fast mode).
+static void matmul_rows_mfma(forge_hip_model* m, const QWeight& w, const KqTwin& tw, uint32_t M, float* y, uint32_t ldy, bool accumulate) {
+    hipStream_t s = m->stream;
+    const int8_t* aq = m->paq.as<int8_t>();
+    const uint16_t* asc = m->pasc.as<uint16_t>();
+    if (!w.kquant()) launch_gemm(w, aq, asc, M, y, ldy, accumulate, false, nullptr, s, m->gemm_ws.p);
+    else if (tw.coef) {
+        launch_gemm(tw.w, aq, asc, M, y, ldy, accumulate, false, nullptr, s, m->gemm_ws.p);
+        launch_kq_min_term(m->pbsum.as<float>(), tw.coef, M, w.N, w.K, y, ldy, s);
+    } else launch_gemm(tw.w, m->paq3.as<int8_t>(), m->pasc3.as<uint16_t>(), M, y, ldy, accumulate, false, nullptr, s, m->gemm_ws.p);
+}
+
+// The same layer in fast mode with every projection on the int8 MFMA GEMM: Q8_0 / Q4_0 matrices as they are, K-quant
+// matrices through their twins.  Block sums are exact integers as in the one-row kernels; scales of K-quant blocks are rounded
+// to fp16 and the f32 accumulation order is the GEMM's.
+void enqueue_mixed_prefill_layer_mfma(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t base_pos) {
+    const forge_hip_config& c = m->cfg;
+    Layer& L = m->layers[l];
+    hipStream_t s = m->stream;
+    const uint32_t H = m->H, I = m->I, QKS = m->QKS, KV = m->KV, QKV = m->QKV;
+    float* x = m->px.as<float>();
+    float* qkv = m->pqkv.as<float>();
+    float* gu = m->pgu.as<float>();
+    int8_t* aq = m->paq.as<int8_t>();
+    uint16_t* asc = m->pasc.as<uint16_t>();
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s, true); }
+    {
+        StageMark t(m, ST_QKV);
+        const QWeight* w[3] = {&L.q, &L.k, &L.v};
+        const KqTwin* tw[3] = {&L.twin[0], &L.twin[1], &L.twin[2]};
+        twin_inputs(m, w, tw, 3, M, H);
+        matmul_rows_mfma(m, L.q, L.twin[0], M, qkv, QKV, false);
+        matmul_rows_mfma(m, L.k, L.twin[1], M, qkv + QKS, QKV, false);
+        matmul_rows_mfma(m, L.v, L.twin[2], M, qkv + QKS + KV, QKV, false);
+    }
+    {
+        StageMark t(m, ST_ROPE);
+        launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos, nullptr, c.heads, c.kv_heads,
+                             c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), nullptr, s, m->pt);
+    }
+    {
+        StageMark t(m, ST_ATTN);
+        launch_attn_prefill_quant(qkv, QKV, m->kc(l), m->vc(l), aq, asc, M, base_pos, c.heads, c.kv_heads, c.head_dim, 0u, s, true, m->pt);
+    }
+    {
+        StageMark t(m, ST_O);
+        const QWeight* w[1] = {&L.o};
+        const KqTwin* tw[1] = {&L.twin[3]};
+        twin_inputs(m, w, tw, 1, M, QKS);
+        matmul_rows_mfma(m, L.o, L.twin[3], M, x, H, true);
+    }
+    { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s, true); }
+    {
+        StageMark t(m, ST_GATE_UP);
+        const QWeight* w[2] = {&L.gate, &L.up};
+        const KqTwin* tw[2] = {&L.twin[4], &L.twin[5]};
+        twin_inputs(m, w, tw, 2, M, H);
+        matmul_rows_mfma(m, L.gate, L.twin[4], M, gu, 2 * I, false);
+        matmul_rows_mfma(m, L.up, L.twin[5], M, gu + I, 2 * I, false);
+    }
+    { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s, true); }
+    {
+        StageMark t(m, ST_DOWN);
+        const QWeight* w[1] = {&L.down};
+        const KqTwin* tw[1] = {&L.twin[6]};
+        twin_inputs(m, w, tw, 1, M, I);
+        matmul_rows_mfma(m, L.down, L.twin[6], M, x, H, true);
+    }
 }
 
 // One decoder layer of a batched prefill: M rows at positions base_pos.. .
@@ -759,6 +845,32 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
         if ((rc = m->gemm_ws.alloc(gemm_split_workspace_bytes()))) return rc;
         FH_HIP(hipMemset(m->gemm_ws.p, 0, gemm_split_workspace_bytes()));
     }
+    // fast mode, prompt in batches: the K-quant projections get twins for the MFMA GEMM (FORGE_HIP_KQ_MFMA=0: the multi-row
+    // GEMV, whose rows are the one-row kernel's bit for bit).  A matrix with a block scale outside the GEMM's scale
+    // arithmetic keeps the whole model on the GEMV.
+    const char* tenv = getenv("FORGE_HIP_KQ_MFMA");
+    if (pd && m->mixed_batched && !(cfg->flags & FORGE_HIP_FLAG_EXACT) && !(tenv && tenv[0] == '0')) {
+        bool all = true, any_k = false;
+        for (uint32_t l = 0; l < cfg->layers && all; l++) {
+            Layer& L = m->layers[l];
+            const QWeight* w[7] = {&L.q, &L.k, &L.v, &L.o, &L.gate, &L.up, &L.down};
+            for (int i = 0; i < 7 && all; i++) {
+                if (!w[i]->kquant()) continue;
+                any_k = true;
+                bool covered = false;
+                if ((rc = kquant_twin_create(*w[i], &L.twin[i], &covered, m->stream))) return rc;
+                all = covered;
+            }
+        }
+        if (!all)
+            for (auto& L : m->layers)
+                for (KqTwin& t : L.twin) kquant_twin_free(&t);
+        m->mixed_twins = all;
+        if (all && any_k &&
+            ((rc = m->pbsum.alloc((size_t)R * (m->KMAX / 32) * 4)) || (rc = m->paq3.alloc((size_t)R * m->KMAX * 2)) ||
+             (rc = m->pasc3.alloc((size_t)R * (m->KMAX / 32) * 2 * 2))))
+            return rc;
+    }
     const char* penv = getenv("FORGE_HIP_PERSIST");
     if (!pd && !(penv && penv[0] == '0')) {       // the resident kernel carries Q8_0 / Q4_0 weight units only
         std::vector<PdLayerIn> pl(cfg->layers);
@@ -820,7 +932,10 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint
             const uint32_t rows = (uint32_t)std::min<uint64_t>(m->chunk_rows, n - fed);
             FH_HIP(hipMemcpyAsync(m->ptok.p, tokens + fed, (size_t)rows * 4, hipMemcpyHostToDevice, s));
             launch_embedding(m->embed.as<float>(), m->ptok.as<uint32_t>(), rows, m->H, m->px.as<float>(), m->counts.as<uint32_t>(), s);
-            for (uint32_t l = 0; l < m->cfg.layers; l++) enqueue_mixed_prefill_layer(m, l, rows, (uint32_t)(m->pos + fed));
+            for (uint32_t l = 0; l < m->cfg.layers; l++) {
+                if (m->mixed_twins) enqueue_mixed_prefill_layer_mfma(m, l, rows, (uint32_t)(m->pos + fed));
+                else enqueue_mixed_prefill_layer(m, l, rows, (uint32_t)(m->pos + fed));
+            }
             FH_HIP(hipGetLastError());
             fed += rows;
             last_rows = rows;

@@ -145,12 +145,15 @@ def test_matmul_vec_portable_dot_bit_exact(fh, oracle, torch_gpu, wd, K, N):
         assert not np.array_equal(ya, want)
 
 
-def random_superblocks(ty, n, seed):
-    """Random K-quant super-blocks with sane fp16 scale fields (every other bit pattern is a valid block)."""
+def random_superblocks(ty, n, seed, positive=False):
+    """Random K-quant super-blocks with sane fp16 scale fields (every other bit pattern is a valid block).  `positive`:
+    d and dmin >= 0, as every quantiser writes them."""
     rng = np.random.default_rng(seed)
     b = rng.integers(0, 256, (n, {12: 144, 14: 210}[ty]), dtype=np.uint8)
     for off in {12: (0, 2), 14: (208,)}[ty]:
-        b[:, off:off + 2] = rng.normal(0, 0.05, n).astype(np.float16).view(np.uint8).reshape(n, 2)
+        # (positive: small enough that d times a 6-bit / int8 sub-block scale stays below 2, the fast matmul's envelope)
+        d = np.abs(rng.normal(0, 0.003, n)) if positive else rng.normal(0, 0.05, n)
+        b[:, off:off + 2] = d.astype(np.float16).view(np.uint8).reshape(n, 2)
     return b.reshape(-1)
 
 
@@ -172,10 +175,53 @@ def test_matmul_vec_kquant_bit_exact(fh, oracle, torch_gpu, ty, K, N):
     rows = np.stack([x, -x, 0.5 * x] + [fh.synth.normal(31 + i, K, 1.0) for i in range(8)])
     want = np.stack([oracle.matmul_vec_kquant(ty, r, wraw, K, N) for r in rows])
     for M in (1, 11):
-        same_bits(fh.ops.matmul_mat_q(w, torch.from_numpy(rows[:M]).cuda()).cpu().numpy(), want[:M])
+        same_bits(fh.ops.matmul_mat_q(w, torch.from_numpy(rows[:M]).cuda(), EXACT).cpu().numpy(), want[:M])
     w.close()
     with pytest.raises(fh.ForgeHipError):
         fh.ops.QWeight(ty, random_superblocks(ty, 1, 1), 288, 1)                # K must be a multiple of 256
+
+
+@pytest.mark.parametrize("ty", [12, 14])
+@pytest.mark.parametrize("M,K,N", [(1, 256, 32), (11, 2048, 512), (352, 2048, 2048), (130, 8192, 320), (700, 3072, 1029), (2502, 2048, 1024)])
+def test_matmul_mat_kquant_on_the_matrix_unit(fh, oracle, torch_gpu, ty, M, K, N):
+    """Fast mode for K-quant matrices: the matrix re-expressed once for the int8 MFMA GEMM (Q4_K: the nibbles as a Q4_0
+    matrix under fp16(d * sc) plus the minimum term as a matmul over the activations' block sums; Q6_K: every 16-element half
+    a block of a Q8_0 matrix of depth 2K under fp16(|d * sc|)).  Block sums stay exact; what differs from matmul_vec is the
+    fp16 rounding of the block scales (2^-11 relative at most) and the order of the f32 additions.  Tolerance: 1e-3 of
+    |value| + the row's root mean square (a sum of K signed products has no smaller natural unit).  With the order-faithful
+    flag the same call gives matmul_vec's bits."""
+    torch = torch_gpu
+    wraw = random_superblocks(ty, N * K // 256, seed=ty * 77 + K + N + M, positive=True)
+    x = fh.synth.normal(5 + K + M, M * K, 1.0).reshape(M, K)
+    x[0, :32] = 0.0
+    w = fh.ops.QWeight(ty, wraw, K, N)
+    xd = torch.from_numpy(x).cuda()
+    exact = fh.ops.matmul_mat_q(w, xd, EXACT).cpu().numpy()
+    for m in {0, M // 2, M - 1}:
+        same_bits(exact[m], oracle.matmul_vec_kquant(ty, x[m], wraw, K, N))
+    fast = fh.ops.matmul_mat_q(w, xd, 0).cpu().numpy()
+    again = fh.ops.matmul_mat_q(w, xd, 0).cpu().numpy()
+    assert np.array_equal(fast, again)
+    rms = np.sqrt(np.mean(exact.astype(np.float64) ** 2, axis=1, keepdims=True))
+    err = np.abs(fast.astype(np.float64) - exact)
+    assert np.all(err <= 1e-3 * (np.abs(exact) + rms)), f"max err / (|v| + rms) = {np.max(err / (np.abs(exact) + rms)):.3e}"
+    assert np.sqrt(np.mean(err ** 2)) < 2e-4 * float(np.mean(rms))
+    if M * N * K >= 2048 * 2048:
+        assert not np.array_equal(fast, exact)                 # it IS the other arithmetic
+    w.close()
+
+
+def test_matmul_mat_kquant_scales_outside_the_fast_arithmetic_keep_the_exact_rows(fh, oracle, torch_gpu):
+    """A Q4_K matrix with a negative d (no quantiser writes one, the format allows it) has no twin: the fast call then
+    runs the order-faithful rows."""
+    torch = torch_gpu
+    K, N, M = 512, 64, 9
+    wraw = random_superblocks(12, N * K // 256, seed=3)          # d of either sign
+    x = fh.synth.normal(8, M * K, 1.0).reshape(M, K)
+    w = fh.ops.QWeight(12, wraw, K, N)
+    xd = torch.from_numpy(x).cuda()
+    same_bits(fh.ops.matmul_mat_q(w, xd, 0).cpu().numpy(), fh.ops.matmul_mat_q(w, xd, EXACT).cpu().numpy())
+    w.close()
 
 
 @pytest.mark.parametrize("wd", [Q8, Q4])
@@ -184,6 +230,7 @@ def test_matmul_mat_parity(fh, oracle, torch_gpu, wd, M, K, N):
     torch = torch_gpu
     wraw = make_weight(fh, wd, N, K, seed=5 * N + K + M)
     x = fh.synth.normal(13 + K, M * K, 1.0).reshape(M, K)
+    x[M // 2, 32:64] = 0.0            # an all-zero activation block (reference scale 1.0: the fast kernel must not let it swamp its sums)
     w = fh.ops.QWeight(wd, wraw, K, N)
     want = oracle.matmul_mat(wd, 0, x, wraw, M, K, N)
     xd = torch.from_numpy(x).cuda()
