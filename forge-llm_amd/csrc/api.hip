@@ -169,7 +169,8 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
         hipStream_t s = (hipStream_t)stream;
         forge_hip_qweight* h = const_cast<forge_hip_qweight*>(w);
         if (!exact && !h->twin_tried) {
-            int32_t rct = kquant_twin_create(h->w, &h->twin, &h->twin_covered, s);
+            const QWeight* one[1] = {&h->w};
+            int32_t rct = kquant_twin_create(one, 1, &h->twin, &h->twin_covered, s);
             if (rct) return rct;
             h->twin_tried = true;
         }
@@ -195,8 +196,8 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
         if (h->twin.coef) {
             if ((rck = g_twin.reserve((size_t)M * (K / 32) * 4))) return rck;
             launch_act_block_sums(q, sc, M, K, true, reinterpret_cast<float*>(g_twin.p), s);
-            launch_gemm(h->twin.w, q, sc, M, y_dev, w->w.N, false, false, nullptr, s, split_ws);
-            launch_kq_min_term(reinterpret_cast<const float*>(g_twin.p), h->twin.coef, M, w->w.N, K, y_dev, w->w.N, s);
+            launch_gemm(h->twin.w, q, sc, M, y_dev, w->w.N, false, false, nullptr, s, split_ws, nullptr, nullptr,
+                        reinterpret_cast<const float*>(g_twin.p), h->twin.coef);
         } else {
             const size_t qbytes = align256((size_t)M * K * 2);
             if ((rck = g_twin.reserve(qbytes + (size_t)M * (K / 32) * 4))) return rck;

@@ -170,14 +170,12 @@ struct KqTwin {
     float* coef = nullptr;     // Q4_K: [N][K/32], 8 * d * sc - dmin * min
     bool present() const { return w.qs != nullptr; }
 };
-int32_t kquant_twin_create(const QWeight& w, KqTwin* out, bool* covered, hipStream_t s);
+int32_t kquant_twin_create(const QWeight* const* ws, uint32_t n, KqTwin* out, bool* covered, hipStream_t s);
 void kquant_twin_free(KqTwin* t);
 // out[m][b] = a_s[m][b] * (sum of block b's codes), f32 [M][K/32]
 void launch_act_block_sums(const int8_t* aq, const uint16_t* as, uint32_t M, uint32_t K, bool neg_odd, float* out, hipStream_t s);
 // every pair of blocks twice: codes [M][2K], scales [M][2K/32]; blocks 2p, 2p + 1 -> 2p, 2p + 1, 2p, 2p + 1
 void launch_act_twice(const int8_t* aq, const uint16_t* as, uint32_t M, uint32_t K, int8_t* oq, uint16_t* os, hipStream_t s);
-// y[m][n] += sum_b block_sums[m][b] * coef[n][b]
-void launch_kq_min_term(const float* block_sums, const float* coef, uint32_t M, uint32_t N, uint32_t K, float* y, uint32_t ldy, hipStream_t s);
 // The same for M rows of quantised activations (codes [M][K], scales [M][K/32]); rows of y are ldy floats apart.  Every row has the
 // bits launch_gemv_kquant gives it alone.
 void launch_gemv_kquant_rows(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy, bool accumulate,
@@ -194,9 +192,11 @@ size_t gemm_split_workspace_bytes();
 // the launch writes quantize(silu(gate) * up) for the down projection: codes [M][N / 2] with odd blocks negated and fp16
 // scales [M][N / 64] (silu_mul emit.rs:380-386 with the hardware exponential, quantiser emit.rs:1410-1440).
 bool gemm_silu_supported(const QWeight& w, uint32_t inter, uint32_t M);
+// mt_a / mt_w (fast mode, Q8_0-layout matrices, no isums): f32 [M][K/32] and [N][K/32]; every element of the result
+// additionally receives sum_b mt_a[m][b] * mt_w[n][b] (before the SiLU epilogue, if any).
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
                  bool accumulate, bool exact, int32_t* isums, hipStream_t s, void* split_ws = nullptr, int8_t* silu_q = nullptr,
-                 uint16_t* silu_sc = nullptr);
+                 uint16_t* silu_sc = nullptr, const float* mt_a = nullptr, const float* mt_w = nullptr);
 
 // model.hip — the part of forge_hip_model_create's checks that sizes depend on (formats, dimensions the kernels cover);
 // sets the error message.

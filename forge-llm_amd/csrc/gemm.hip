@@ -34,6 +34,8 @@
 // All global accesses go through buffer descriptors: rows past the end of a matrix read as zero and
 // stores past the end are dropped by the hardware's range check, so the loops carry no predication.
 // A K tail (K % 128) reads whatever follows in the row-major matrix; those blocks get scale 0.
+#include <type_traits>
+
 #include "common.h"
 #include "device_utils.h"
 
@@ -92,9 +94,14 @@ struct GemmSplit {
     int8_t* silu_q;         // SILU: [M][inter] codes (odd blocks negated, as the fast GEMM takes its activations)
     uint16_t* silu_sc;      // SILU: [M][inter / 32] fp16 scales
     uint32_t inter;
+    const float* mt_a;      // MINT: [M][K / 32] f32, one value per activation block
+    const float* mt_w;      // MINT: [N][K / 32] f32, one value per weight block
 };
 
-template <bool Q4, bool DUMP, bool EXACT, int TM, bool SPLIT = false, bool SILU = false>
+// MINT: the tile additionally receives sum_b mt_a[m][b] * mt_w[n][b], an f32 matmul of depth K / 32 on the matrix unit in
+// front of the epilogue (the minimum term of a Q4_K matrix: activation block sums times a coefficient per weight block,
+// kquant_prefill.hip) -- so that it costs no pass over the result and may precede the SiLU epilogue.
+template <bool Q4, bool DUMP, bool EXACT, int TM, bool SPLIT = false, bool SILU = false, bool MINT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
 void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ wsc, const int8_t* __restrict__ aq,
                    const uint16_t* __restrict__ asc, float* __restrict__ y, int32_t* __restrict__ isums, uint32_t M,
@@ -103,6 +110,7 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     constexpr bool MAGIC = !EXACT;               // DUMP && !EXACT: the fast arithmetic, with its block sums written out too
     static_assert(!SPLIT || (MAGIC && !DUMP), "K ranges change the order of the block sum: fast mode only");
     static_assert(!SILU || (MAGIC && !DUMP), "the fused SiLU epilogue belongs to the fast mode");
+    static_assert(!MINT || (MAGIC && !DUMP && !Q4), "the extra f32 term belongs to the fast mode on Q8_0-layout matrices (no 1/16 pending)");
 
     const uint32_t tid = threadIdx.x, lane = tid & 63;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));   // uniform: the compiler keeps it scalar
@@ -453,6 +461,34 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
         if (tid == 0) __hip_atomic_store(sp.counters + range_tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next launch (stream order)
     }
 
+    if (MINT) {
+        // A: lane = (row lrow of the tile, k = lhalf), B: lane = (column lrow, k = lhalf), v_mfma_f32_32x32x2_f32; a lane fetches
+        // four consecutive b per operand (the order of k inside a sum is free), so eight b pass through four MFMAs.  The
+        // result tile has the accumulators' layout.
+        typedef float v16f32 __attribute__((ext_vector_type(16)));
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+            for (int tn = 0; tn < 2; tn++) {
+                const uint32_t mrow = min(m0 + wm * WM + tm * 32 + lrow, M - 1);
+                const uint32_t nrow = SILU ? si0 + 32 * wn + lrow + tn * s_inter : min(n0 + wn * 64 + tn * 32 + lrow, N - 1);
+                const float* ap = sp.mt_a + (size_t)mrow * nblk + 4 * lhalf;
+                const float* bp = sp.mt_w + (size_t)nrow * nblk + 4 * lhalf;
+                v16f32 c;
+#pragma unroll
+                for (int r = 0; r < 16; r++) c[r] = acc[tm][tn][r];
+                for (uint32_t g = 0; g < nblk; g += 8) {
+                    const float4 a = *reinterpret_cast<const float4*>(ap + g), b = *reinterpret_cast<const float4*>(bp + g);
+                    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, c, 0, 0, 0);
+                    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, c, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[tm][tn][r] = c[r];
+            }
+    }
+
     if (SILU) {
         // lane: inter index i0 + 32 wn + lrow, gate in the first column tile, up in the second; rows as below
         const uint32_t inter = sp.inter, blk = tile_x * 2 + wn;           // the quant block this wave's 32 indices are
@@ -539,7 +575,8 @@ bool gemm_silu_supported(const QWeight& w, uint32_t inter, uint32_t M) {
 }
 
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
-                 bool accumulate, bool exact, int32_t* isums, hipStream_t s, void* split_ws, int8_t* silu_q, uint16_t* silu_sc) {
+                 bool accumulate, bool exact, int32_t* isums, hipStream_t s, void* split_ws, int8_t* silu_q, uint16_t* silu_sc,
+                 const float* mt_a, const float* mt_w) {
     if (M == 0 || w.N == 0) return;
     const bool silu = silu_q != nullptr;      // caller: gemm_silu_supported, fast mode, no block-sum dump
     const int accf = accumulate ? 1 : 0;
@@ -590,6 +627,8 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
             // the fraction cut along K, so that they spread over all CUs; a problem with fewer tiles than half the CUs is
             // all fraction.  Which tile height then fills the CUs best is decided by a small cost model (microseconds per K
             // stage of a workgroup that has a CU to itself, measured: 1.3 for a 128-row tile, 1.1 for a 64-row one).
+            GemmSplit fsp{};
+            uint32_t items = 0;
             if (split_ws && !exact && !isums && mc == M && nc == w.N) {
                 struct Plan { int tm; GemmSplit sp; uint32_t items; double cost; };
                 const uint32_t stages = (w.K + BK - 1) / BK;
@@ -617,61 +656,40 @@ void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_
                 Plan best = plan(tm);
                 if (tm == 1) { const Plan other = plan(2); if (other.cost < best.cost) best = other; }
                 tm = best.tm;
-                if (best.items && silu) {
-                    GemmSplit sp = best.sp;
-                    sp.silu_q = silu_q; sp.silu_sc = silu_sc; sp.inter = w.N / 2;
-                    const uint32_t items = best.items;
-#define FH_GEMM_LAUNCH_SPLIT_SILU(Q4_, TM_)                                                                                  \
-    do {                                                                                                                    \
-        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, false, false, TM_, true, true>, \
-                                                             hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES);   \
-        (void)lds_ok;                                                                                                       \
-        fh::launch(gemm_q_kernel<Q4_, false, false, TM_, true, true>, dim3(items), 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c,   \
-                   as_c, y_c, is_c, mc, nc, w.K, ldy, accf, sp);                                                            \
-    } while (0)
-                    if (q4 && tm == 1) FH_GEMM_LAUNCH_SPLIT_SILU(true, 1);
-                    else if (q4) FH_GEMM_LAUNCH_SPLIT_SILU(true, 2);
-                    else if (tm == 1) FH_GEMM_LAUNCH_SPLIT_SILU(false, 1);
-                    else FH_GEMM_LAUNCH_SPLIT_SILU(false, 2);
-#undef FH_GEMM_LAUNCH_SPLIT_SILU
-                    continue;
-                }
-                if (best.items) {
-                    const GemmSplit sp = best.sp;
-                    const uint32_t items = best.items;
-#define FH_GEMM_LAUNCH_SPLIT(Q4_, TM_)                                                                                       \
-    do {                                                                                                                    \
-        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, false, false, TM_, true>,     \
-                                                             hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES);   \
-        (void)lds_ok;                                                                                                       \
-        fh::launch(gemm_q_kernel<Q4_, false, false, TM_, true>, dim3(items), 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c,   \
-                   y_c, is_c, mc, nc, w.K, ldy, accf, sp);                                                                  \
-    } while (0)
-                    if (q4 && tm == 1) FH_GEMM_LAUNCH_SPLIT(true, 1);
-                    else if (q4) FH_GEMM_LAUNCH_SPLIT(true, 2);
-                    else if (tm == 1) FH_GEMM_LAUNCH_SPLIT(false, 1);
-                    else FH_GEMM_LAUNCH_SPLIT(false, 2);
-#undef FH_GEMM_LAUNCH_SPLIT
-                    continue;
-                }
+                if (best.items) { fsp = best.sp; items = best.items; }
             }
-            if (silu) {
-                GemmSplit sp{};
-                sp.silu_q = silu_q; sp.silu_sc = silu_sc; sp.inter = w.N / 2;
-#define FH_GEMM_LAUNCH_SILU(Q4_, TM_)                                                                                         \
-    do {                                                                                                                    \
-        static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, false, false, TM_, false, true>, \
-                                                             hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES);   \
-        (void)lds_ok;                                                                                                       \
-        dim3 grid((nc + BN - 1) / BN, (mc + 64 * TM_ - 1) / (64 * TM_));                                                    \
-        fh::launch(gemm_q_kernel<Q4_, false, false, TM_, false, true>, grid, 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c,   \
-                   y_c, is_c, mc, nc, w.K, ldy, accf, sp);                                                                  \
-    } while (0)
-                if (q4 && tm == 1) FH_GEMM_LAUNCH_SILU(true, 1);
-                else if (q4) FH_GEMM_LAUNCH_SILU(true, 2);
-                else if (tm == 1) FH_GEMM_LAUNCH_SILU(false, 1);
-                else FH_GEMM_LAUNCH_SILU(false, 2);
-#undef FH_GEMM_LAUNCH_SILU
+            if (items || silu || mt_a) {
+                // the fast kernel's variants: tiles cut along K, the SiLU epilogue, the extra f32 term
+                if (silu) { fsp.silu_q = silu_q; fsp.silu_sc = silu_sc; fsp.inter = w.N / 2; }
+                if (mt_a) { fsp.mt_a = mt_a + (size_t)mlo * nblk; fsp.mt_w = mt_w + (size_t)nlo * nblk; }
+                const dim3 grid = items ? dim3(items) : dim3((nc + BN - 1) / BN, (mc + 64 * tm - 1) / (64 * tm));
+                auto go = [&](auto q4_, auto tm_, auto split_, auto silu_, auto mint_) {
+                    constexpr bool Q4_ = decltype(q4_)::value, SPLIT_ = decltype(split_)::value, SILU_ = decltype(silu_)::value,
+                                   MINT_ = decltype(mint_)::value;
+                    constexpr int TM_ = decltype(tm_)::value;
+                    static const hipError_t lds_ok = hipFuncSetAttribute((const void*)gemm_q_kernel<Q4_, false, false, TM_, SPLIT_, SILU_, MINT_>,
+                                                                         hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS_BYTES);
+                    (void)lds_ok;
+                    fh::launch(gemm_q_kernel<Q4_, false, false, TM_, SPLIT_, SILU_, MINT_>, grid, 256, GEMM_LDS_BYTES, s, wq, wsc, aq_c, as_c,
+                               y_c, is_c, mc, nc, w.K, ldy, accf, fsp);
+                };
+                using T = std::true_type;
+                using F = std::false_type;
+                using One = std::integral_constant<int, 1>;
+                using Two = std::integral_constant<int, 2>;
+                auto by_tm = [&](auto q4_, auto split_, auto silu_, auto mint_) {
+                    if (tm == 1) go(q4_, One{}, split_, silu_, mint_);
+                    else go(q4_, Two{}, split_, silu_, mint_);
+                };
+                auto by_shape = [&](auto q4_, auto mint_) {
+                    if (items && silu) by_tm(q4_, T{}, T{}, mint_);
+                    else if (items) by_tm(q4_, T{}, F{}, mint_);
+                    else if (silu) by_tm(q4_, F{}, T{}, mint_);
+                    else by_tm(q4_, F{}, F{}, mint_);
+                };
+                if (mt_a) by_shape(F{}, T{});          // caller: a Q8_0-layout matrix
+                else if (q4) by_shape(T{}, F{});
+                else by_shape(F{}, F{});
                 continue;
             }
             if (q4) {

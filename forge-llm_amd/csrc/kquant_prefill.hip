@@ -11,7 +11,7 @@
 //         closest to d*sc_j (d*sc_j has up to 17 significant bits, fp16 has 11: among seven distinct roundings the best is
 //         typically within 4e-5 of it, relative; that residue times the block's centred dot product is all that is dropped).
 //         Second term: the block sums of the activations times an f32 coefficient per (row, block), a small f32 matmul of
-//         depth K/32 (kq_min_term_kernel).
+//         depth K/32 that the GEMM kernel runs on the matrix unit in front of its epilogue (its mt_a / mt_w operands).
 //   Q6_K  w = d * sc_h * q, q = -32..31, sc_h an int8 per 16-element half.  sc_h * q = 64 hi + lo with lo in [-32, 31] and hi
 //         in [-63, 64]: a block becomes two blocks of a matrix of depth 2K, the hi codes under the scale 64 d and the lo codes
 //         under d.  Both scales are exact fp16 numbers (d is one), so nothing is dropped at all; the activations go in twice
@@ -135,58 +135,28 @@ __global__ __launch_bounds__(256) void act_twice_kernel(const int8_t* __restrict
     }
 }
 
-// y[m][n] += sum_b bs[m][b] * coef[n][b]: the minimum term of a Q4_K matrix for M rows.  One wave per 32 x 32 tile of y,
-// v_mfma_f32_32x32x2_f32; a lane fetches four consecutive b of its row per operand (the order of k inside the sum is free), so
-// eight b go through four MFMAs.  Both operands are small and re-read from L2.
-__global__ __launch_bounds__(256) void kq_min_term_kernel(const float* __restrict__ bs, const float* __restrict__ coef, uint32_t M, uint32_t N,
-                                                        uint32_t nblk, float* __restrict__ y, uint32_t ldy) {
-    typedef float v16f __attribute__((ext_vector_type(16)));
-    const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t m0 = blockIdx.y * 64 + (wave >> 1) * 32, n0 = blockIdx.x * 64 + (wave & 1) * 32;
-    if (m0 >= M || n0 >= N) return;
-    const uint32_t lrow = lane & 31, lhalf = lane >> 5;
-    const float* ap = bs + (size_t)min(m0 + lrow, M - 1) * nblk + 4 * lhalf;
-    const float* bp = coef + (size_t)min(n0 + lrow, N - 1) * nblk + 4 * lhalf;
-    v16f acc;
-#pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] = 0.f;
-    for (uint32_t g = 0; g < nblk; g += 8) {
-        const float4 a = *reinterpret_cast<const float4*>(ap + g), b = *reinterpret_cast<const float4*>(bp + g);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, acc, 0, 0, 0);
-    }
-    // lane holds column n0 + lrow, rows m0 + 8 (r / 4) + 4 lhalf + r % 4
-    const uint32_t n = n0 + lrow;
-    if (n >= N) return;
-    float old[16];
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const uint32_t m = m0 + 8 * (r >> 2) + 4 * lhalf + (r & 3);
-        old[r] = m < M ? y[(size_t)m * ldy + n] : 0.f;
-    }
-#pragma unroll
-    for (int r = 0; r < 16; r++) {
-        const uint32_t m = m0 + 8 * (r >> 2) + 4 * lhalf + (r & 3);
-        if (m < M) y[(size_t)m * ldy + n] = old[r] + acc[r];
-    }
-}
-
 }  // namespace
 
-// `*covered` = false (and no twin) when a block scale lies outside what the fast GEMM's scale arithmetic covers (a negative
-// Q4_K scale, d * sc or 64 |d| not below 2): the caller keeps the multi-row GEMV for that matrix.
-int32_t kquant_twin_create(const QWeight& w, KqTwin* out, bool* covered, hipStream_t s) {
+// One twin for `n` matrices of the same format and depth, their rows one after the other (q then k; gate then up): one GEMM
+// launch for the group.  `*covered` = false (and no twin) when a block scale lies outside what the fast GEMM's scale
+// arithmetic covers (a negative Q4_K scale, d * sc or 64 |d| not below 2): the caller keeps the multi-row GEMV.
+int32_t kquant_twin_create(const QWeight* const* ws, uint32_t n, KqTwin* out, bool* covered, hipStream_t s) {
     *covered = false;
-    if (!w.kquant() || w.K % 256 != 0) { set_error("kquant twin: not a K-quant matrix"); return FORGE_HIP_ERR_INVALID; }
-    const uint32_t nblk = w.K / 32;
-    const uint64_t total = (uint64_t)w.N * nblk;
-    const bool q6 = w.wdtype == FORGE_HIP_Q6_K;
+    const QWeight& w0 = *ws[0];
+    uint64_t rows = 0;
+    for (uint32_t i = 0; i < n; i++) {
+        if (!ws[i]->kquant() || ws[i]->K % 256 != 0 || ws[i]->wdtype != w0.wdtype || ws[i]->K != w0.K) {
+            set_error("kquant twin: K-quant matrices of one format and depth only");
+            return FORGE_HIP_ERR_INVALID;
+        }
+        rows += ws[i]->N;
+    }
+    const uint32_t nblk = w0.K / 32;
+    const bool q6 = w0.wdtype == FORGE_HIP_Q6_K;
     QWeight t;
     t.wdtype = FORGE_HIP_Q8_0;
-    t.K = q6 ? 2 * w.K : w.K;
-    t.N = w.N;
+    t.K = q6 ? 2 * w0.K : w0.K;
+    t.N = (uint32_t)rows;
     t.owns = true;
     uint32_t* bad = nullptr;
     float* coef = nullptr;
@@ -198,16 +168,24 @@ int32_t kquant_twin_create(const QWeight& w, KqTwin* out, bool* covered, hipStre
         return rc;
     };
     if (hipMalloc(&t.qs, t.qs_bytes()) != hipSuccess || hipMalloc(&t.scales, t.scales_bytes()) != hipSuccess ||
-        hipMalloc(&bad, 4) != hipSuccess || (!q6 && hipMalloc(&coef, total * 4) != hipSuccess)) {
+        hipMalloc(&bad, 4) != hipSuccess || (!q6 && hipMalloc(&coef, rows * nblk * 4) != hipSuccess)) {
         (void)hipGetLastError();
         set_error("kquant twin: out of device memory");
         return fail(FORGE_HIP_ERR_HIP);
     }
     if (hipMemsetAsync(bad, 0, 4, s) != hipSuccess) return fail(FORGE_HIP_ERR_HIP);
-    const uint32_t grid = (uint32_t)((total + 255) / 256);
-    const uint8_t* meta = reinterpret_cast<const uint8_t*>(w.scales);
-    if (q6) fh::launch(twin_q6k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, reinterpret_cast<int8_t*>(t.qs), t.scales, bad);
-    else fh::launch(twin_q4k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, reinterpret_cast<int8_t*>(t.qs), t.scales, coef, bad);
+    uint64_t row0 = 0;
+    for (uint32_t i = 0; i < n; i++) {
+        const QWeight& w = *ws[i];
+        const uint64_t total = (uint64_t)w.N * nblk;
+        const uint32_t grid = (uint32_t)((total + 255) / 256);
+        const uint8_t* meta = reinterpret_cast<const uint8_t*>(w.scales);
+        int8_t* tq = reinterpret_cast<int8_t*>(t.qs) + row0 * t.K;
+        uint16_t* ts = t.scales + row0 * (t.K / 32);
+        if (q6) fh::launch(twin_q6k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, tq, ts, bad);
+        else fh::launch(twin_q4k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, tq, ts, coef + row0 * nblk, bad);
+        row0 += w.N;
+    }
     uint32_t flag = 0;
     if (hipMemcpyAsync(&flag, bad, 4, hipMemcpyDeviceToHost, s) != hipSuccess || hipStreamSynchronize(s) != hipSuccess) {
         set_error("kquant twin: conversion kernel failed");
@@ -239,11 +217,6 @@ void launch_act_twice(const int8_t* aq, const uint16_t* as, uint32_t M, uint32_t
     const uint64_t pairs = (uint64_t)M * (K / 64);
     if (pairs == 0) return;
     fh::launch(act_twice_kernel, (uint32_t)((pairs * 4 + 255) / 256), 256, 0, s, aq, as, pairs, oq, os);
-}
-
-void launch_kq_min_term(const float* block_sums, const float* coef, uint32_t M, uint32_t N, uint32_t K, float* y, uint32_t ldy, hipStream_t s) {
-    if (M == 0 || N == 0) return;
-    fh::launch(kq_min_term_kernel, dim3((N + 63) / 64, (M + 63) / 64), 256, 0, s, block_sums, coef, M, N, K / 32, y, ldy);
 }
 
 }  // namespace fh

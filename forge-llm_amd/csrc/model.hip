@@ -29,7 +29,10 @@ struct Layer {
     float* ffn_norm = nullptr;
     QWeight qkv, o, gate_up, down;
     QWeight q, k, v, gate, up;           // a model with a storage format per projection keeps these five apart (qkv, gate_up unused)
-    KqTwin twin[7];                      // fast mode: the K-quant ones among q, k, v, o, gate, up, down as matrices of the int8 MFMA GEMM
+    // fast mode: the K-quant ones among q, k, v, o, gate, up, down as matrices of the int8 MFMA GEMM.  Neighbours of one format
+    // that read the same rows (q, k, v; gate, up) share a twin: twin[i] then covers twin_span[i] projections from i on
+    KqTwin twin[7];
+    uint8_t twin_span[7] = {0, 0, 0, 0, 0, 0, 0};
     float* qkv_bias = nullptr;           // [QKS + 2 KV]: q | k | v bias, in the row order of the fused qkv matrix (FLAG_QKV_BIAS)
 };
 
@@ -399,33 +402,38 @@ void enqueue_mixed_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uin
     { StageMark t(m, ST_DOWN); matmul_rows_any(m, L.down, aq, asc, M, x, H, true); }
 }
 
-// What the twins among `tw` need of the quantised rows in (paq, pasc) (odd blocks negated): Q4_K twins the scaled block sums,
-// Q6_K twins every block twice.
-static void twin_inputs(forge_hip_model* m, const QWeight* const* w, const KqTwin* const* tw, int n, uint32_t M, uint32_t K) {
-    bool sums = false, twice = false;
-    for (int i = 0; i < n; i++) {
-        if (!w[i]->kquant()) continue;
-        (tw[i]->coef ? sums : twice) = true;
-    }
-    if (sums) launch_act_block_sums(m->paq.as<int8_t>(), m->pasc.as<uint16_t>(), M, K, true, m->pbsum.as<float>(), m->stream);
-    if (twice) launch_act_twice(m->paq.as<int8_t>(), m->pasc.as<uint16_t>(), M, K, m->paq3.as<int8_t>(), m->pasc3.as<uint16_t>(), m->stream);
-}
-
-// y (=|+=) rows * W^T on the MFMA GEMM, whatever W's format (fast mode).
-static void matmul_rows_mfma(forge_hip_model* m, const QWeight& w, const KqTwin& tw, uint32_t M, float* y, uint32_t ldy, bool accumulate) {
+// The projections ids[0..n) of a layer multiply the same quantised rows (aq, asc: depth K, odd blocks negated) and write
+// neighbouring columns of y, all on the int8 MFMA GEMM (fast mode): Q8_0 / Q4_0 matrices as they are, K-quant matrices
+// through their twins, which first get what they need of the rows (Q4_K: the scaled block sums; Q6_K: every block twice).
+// silu_q: the group is gate, up under ONE twin and the launch writes quantize(silu(gate) * up) instead of y.
+static void matmul_group_mfma(forge_hip_model* m, Layer& L, const int* ids, int n, const int8_t* aq, const uint16_t* asc, uint32_t M,
+                              uint32_t K, float* y, uint32_t ldy, bool accumulate, int8_t* silu_q = nullptr, uint16_t* silu_sc = nullptr) {
     hipStream_t s = m->stream;
-    const int8_t* aq = m->paq.as<int8_t>();
-    const uint16_t* asc = m->pasc.as<uint16_t>();
-    if (!w.kquant()) launch_gemm(w, aq, asc, M, y, ldy, accumulate, false, nullptr, s, m->gemm_ws.p);
-    else if (tw.coef) {
-        launch_gemm(tw.w, aq, asc, M, y, ldy, accumulate, false, nullptr, s, m->gemm_ws.p);
-        launch_kq_min_term(m->pbsum.as<float>(), tw.coef, M, w.N, w.K, y, ldy, s);
-    } else launch_gemm(tw.w, m->paq3.as<int8_t>(), m->pasc3.as<uint16_t>(), M, y, ldy, accumulate, false, nullptr, s, m->gemm_ws.p);
+    const QWeight* w[7] = {&L.q, &L.k, &L.v, &L.o, &L.gate, &L.up, &L.down};
+    bool sums = false, twice = false;
+    for (int j = 0; j < n; j++)
+        if (L.twin_span[ids[j]]) (L.twin[ids[j]].coef ? sums : twice) = true;
+    if (sums) launch_act_block_sums(aq, asc, M, K, true, m->pbsum.as<float>(), s);
+    if (twice) launch_act_twice(aq, asc, M, K, m->paq3.as<int8_t>(), m->pasc3.as<uint16_t>(), s);
+    float* col = y;
+    for (int j = 0; j < n;) {
+        const int id = ids[j];
+        if (!w[id]->kquant()) {
+            launch_gemm(*w[id], aq, asc, M, col, ldy, accumulate, false, nullptr, s, m->gemm_ws.p);
+            col += w[id]->N;
+            j++;
+            continue;
+        }
+        const KqTwin& t = L.twin[id];
+        if (t.coef) launch_gemm(t.w, aq, asc, M, col, ldy, accumulate, false, nullptr, s, m->gemm_ws.p, silu_q, silu_sc, m->pbsum.as<float>(), t.coef);
+        else launch_gemm(t.w, m->paq3.as<int8_t>(), m->pasc3.as<uint16_t>(), M, col, ldy, accumulate, false, nullptr, s, m->gemm_ws.p, silu_q, silu_sc);
+        col += t.w.N;
+        j += L.twin_span[id];
+    }
 }
 
-// The same layer in fast mode with every projection on the int8 MFMA GEMM: Q8_0 / Q4_0 matrices as they are, K-quant
-// matrices through their twins.  Block sums are exact integers as in the one-row kernels; scales of K-quant blocks are rounded
-// to fp16 and the f32 accumulation order is the GEMM's.
+// The same layer in fast mode with every projection on the int8 MFMA GEMM.  Block sums are exact integers as in the one-row
+// kernels; the f32 accumulation order is the GEMM's, and the scale of a Q4_K block is rounded as kquant_prefill.hip says.
 void enqueue_mixed_prefill_layer_mfma(forge_hip_model* m, uint32_t l, uint32_t M, uint32_t base_pos) {
     const forge_hip_config& c = m->cfg;
     Layer& L = m->layers[l];
@@ -436,16 +444,9 @@ void enqueue_mixed_prefill_layer_mfma(forge_hip_model* m, uint32_t l, uint32_t M
     float* gu = m->pgu.as<float>();
     int8_t* aq = m->paq.as<int8_t>();
     uint16_t* asc = m->pasc.as<uint16_t>();
+    static const int qkv_ids[3] = {0, 1, 2}, o_ids[1] = {3}, gu_ids[2] = {4, 5}, down_ids[1] = {6};
     { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.attn_norm, c.rms_eps, M, H, nullptr, aq, asc, s, true); }
-    {
-        StageMark t(m, ST_QKV);
-        const QWeight* w[3] = {&L.q, &L.k, &L.v};
-        const KqTwin* tw[3] = {&L.twin[0], &L.twin[1], &L.twin[2]};
-        twin_inputs(m, w, tw, 3, M, H);
-        matmul_rows_mfma(m, L.q, L.twin[0], M, qkv, QKV, false);
-        matmul_rows_mfma(m, L.k, L.twin[1], M, qkv + QKS, QKV, false);
-        matmul_rows_mfma(m, L.v, L.twin[2], M, qkv + QKS + KV, QKV, false);
-    }
+    { StageMark t(m, ST_QKV); matmul_group_mfma(m, L, qkv_ids, 3, aq, asc, M, H, qkv, QKV, false); }
     {
         StageMark t(m, ST_ROPE);
         launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos, nullptr, c.heads, c.kv_heads,
@@ -455,30 +456,18 @@ void enqueue_mixed_prefill_layer_mfma(forge_hip_model* m, uint32_t l, uint32_t M
         StageMark t(m, ST_ATTN);
         launch_attn_prefill_quant(qkv, QKV, m->kc(l), m->vc(l), aq, asc, M, base_pos, c.heads, c.kv_heads, c.head_dim, 0u, s, true, m->pt);
     }
-    {
-        StageMark t(m, ST_O);
-        const QWeight* w[1] = {&L.o};
-        const KqTwin* tw[1] = {&L.twin[3]};
-        twin_inputs(m, w, tw, 1, M, QKS);
-        matmul_rows_mfma(m, L.o, L.twin[3], M, x, H, true);
-    }
+    { StageMark t(m, ST_O); matmul_group_mfma(m, L, o_ids, 1, aq, asc, M, QKS, x, H, true); }
     { StageMark t(m, ST_RMSNORM); launch_rmsnorm(x, L.ffn_norm, c.rms_eps, M, H, nullptr, aq, asc, s, true); }
-    {
-        StageMark t(m, ST_GATE_UP);
-        const QWeight* w[2] = {&L.gate, &L.up};
-        const KqTwin* tw[2] = {&L.twin[4], &L.twin[5]};
-        twin_inputs(m, w, tw, 2, M, H);
-        matmul_rows_mfma(m, L.gate, L.twin[4], M, gu, 2 * I, false);
-        matmul_rows_mfma(m, L.up, L.twin[5], M, gu + I, 2 * I, false);
+    if (m->prefill_fuse_silu && L.twin_span[4] == 2 && gemm_silu_supported(L.twin[4].w, I, M)) {
+        // gate and up under one twin: the GEMM's epilogue writes silu(gate) * up quantised, the [M][2 inter] floats never exist
+        { StageMark t(m, ST_GATE_UP); matmul_group_mfma(m, L, gu_ids, 2, aq, asc, M, H, nullptr, 2 * I, false, m->paq2.as<int8_t>(), m->pasc2.as<uint16_t>()); }
+        aq = m->paq2.as<int8_t>();
+        asc = m->pasc2.as<uint16_t>();
+    } else {
+        { StageMark t(m, ST_GATE_UP); matmul_group_mfma(m, L, gu_ids, 2, aq, asc, M, H, gu, 2 * I, false); }
+        { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s, true); }
     }
-    { StageMark t(m, ST_SILU); launch_silu_mul(gu, gu + I, M, I, 2 * I, nullptr, aq, asc, s, true); }
-    {
-        StageMark t(m, ST_DOWN);
-        const QWeight* w[1] = {&L.down};
-        const KqTwin* tw[1] = {&L.twin[6]};
-        twin_inputs(m, w, tw, 1, M, I);
-        matmul_rows_mfma(m, L.down, L.twin[6], M, x, H, true);
-    }
+    { StageMark t(m, ST_DOWN); matmul_group_mfma(m, L, down_ids, 1, aq, asc, M, I, x, H, true); }
 }
 
 // One decoder layer of a batched prefill: M rows at positions base_pos.. .
@@ -839,6 +828,7 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
         (rc = m->ptok.alloc((size_t)R * 4)))
         return rc;
     if (m->prefill_fuse_silu && ((rc = m->paq2.alloc((size_t)R * I)) || (rc = m->pasc2.alloc((size_t)R * (I / 32) * 2)))) return rc;
+    const bool fuse_silu_twins = fuse_ok && !(senv2 && senv2[0] == '0') && I % 64 == 0;
     // fast mode: the prefill GEMMs may cut left-over tiles along K (FORGE_HIP_GEMM_SPLIT=0: never)
     const char* senv = getenv("FORGE_HIP_GEMM_SPLIT");
     if (!(cfg->flags & FORGE_HIP_FLAG_EXACT) && !(senv && senv[0] == '0')) {
@@ -851,25 +841,37 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
     const char* tenv = getenv("FORGE_HIP_KQ_MFMA");
     if (pd && m->mixed_batched && !(cfg->flags & FORGE_HIP_FLAG_EXACT) && !(tenv && tenv[0] == '0')) {
         bool all = true, any_k = false;
+        static const int groups[4][4] = {{0, 1, 2, -1}, {3, -1, -1, -1}, {4, 5, -1, -1}, {6, -1, -1, -1}};
         for (uint32_t l = 0; l < cfg->layers && all; l++) {
             Layer& L = m->layers[l];
             const QWeight* w[7] = {&L.q, &L.k, &L.v, &L.o, &L.gate, &L.up, &L.down};
-            for (int i = 0; i < 7 && all; i++) {
-                if (!w[i]->kquant()) continue;
-                any_k = true;
-                bool covered = false;
-                if ((rc = kquant_twin_create(*w[i], &L.twin[i], &covered, m->stream))) return rc;
-                all = covered;
-            }
+            for (int g = 0; g < 4 && all; g++)
+                for (int j = 0; groups[g][j] >= 0 && all;) {
+                    const int id = groups[g][j];
+                    if (!w[id]->kquant()) { j++; continue; }
+                    // this projection and the neighbours of its format that follow it in the group
+                    const QWeight* part[3];
+                    uint32_t span = 0;
+                    while (groups[g][j] >= 0 && w[groups[g][j]]->wdtype == w[id]->wdtype) part[span++] = w[groups[g][j++]];
+                    any_k = true;
+                    bool covered = false;
+                    if ((rc = kquant_twin_create(part, span, &L.twin[id], &covered, m->stream))) return rc;
+                    L.twin_span[id] = (uint8_t)span;
+                    all = covered;
+                }
         }
         if (!all)
             for (auto& L : m->layers)
-                for (KqTwin& t : L.twin) kquant_twin_free(&t);
+                for (int i = 0; i < 7; i++) { kquant_twin_free(&L.twin[i]); L.twin_span[i] = 0; }
         m->mixed_twins = all;
         if (all && any_k &&
             ((rc = m->pbsum.alloc((size_t)R * (m->KMAX / 32) * 4)) || (rc = m->paq3.alloc((size_t)R * m->KMAX * 2)) ||
              (rc = m->pasc3.alloc((size_t)R * (m->KMAX / 32) * 2 * 2))))
             return rc;
+        if (all && fuse_silu_twins) {
+            m->prefill_fuse_silu = true;
+            if ((rc = m->paq2.alloc((size_t)R * I)) || (rc = m->pasc2.alloc((size_t)R * (I / 32) * 2))) return rc;
+        }
     }
     const char* penv = getenv("FORGE_HIP_PERSIST");
     if (!pd && !(penv && penv[0] == '0')) {       // the resident kernel carries Q8_0 / Q4_0 weight units only
