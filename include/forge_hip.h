@@ -123,11 +123,15 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* weigh
  * {q, k, v, o, gate, up, down}, each Q8_0 (8), Q4_0 (2), Q4_K (12) or Q6_K (14); the lm_head's format is
  * cfg->lm_head_dtype and may be a K-quant too; cfg->wdtype is not read unless all seven agree with it.  The blob has
  * forge_hip_model_create's layout with every matrix in its own format, K-quant matrices as the GGUF file's own
- * super-blocks (144 bytes per 256 weights for Q4_K, 210 for Q6_K).  As in the reference, such a model has no batched
- * prefill (model_is_q8/q4 gate, emit.rs:4530-4534): forge_hip_prefill_batch walks the prompt one token at a time through
- * the decode operations (forward_prefill, emit.rs:4621-5040) and runs the lm_head once, in forward's order.  Decode runs
- * the kernel sequence (one GEMV launch per projection), captured in a graph; the resident decode kernel carries Q8_0 and
- * Q4_0 weights only.  K-quant matrices need an input width that is a multiple of 256; QKV bias and sliding windows are
+ * super-blocks (144 bytes per 256 weights for Q4_K, 210 for Q6_K).  In the reference such a model has no batched
+ * prefill (model_is_q8/q4 gate, emit.rs:4530-4534): the prompt goes one token at a time through the decode operations
+ * (forward_prefill, emit.rs:4621-5040) and the lm_head runs once, in forward's order.  forge_hip_prefill_batch takes the
+ * prompt in batches of rows where that changes no bit the mode promises: with FORGE_HIP_FLAG_EXACT when all seven
+ * projections are K-quants (multi-row K-quant GEMV: every row has the one-row kernel's bits, so logits, cache and tokens are
+ * the token-by-token walk's), otherwise token by token; without the flag always, on the int8 MFMA GEMM (K-quant matrices
+ * through re-expressions built at create time, see forge_hip_gemm_q: the device then holds both forms of those matrices).
+ * Decode runs the kernel sequence (K-quant projections over the same normed row share a launch), captured in a graph; the
+ * resident decode kernel carries Q8_0 and Q4_0 weights only.  K-quant matrices need an input width that is a multiple of 256; QKV bias and sliding windows are
  * refused.  When all seven formats equal cfg->wdtype and the lm_head is Q8_0 or Q4_0 this is forge_hip_model_create. */
 uint64_t forge_hip_weights_nbytes_mixed(const forge_hip_config* cfg, const uint32_t* proj_dtypes);
 int32_t forge_hip_model_create_mixed(const forge_hip_config* cfg, const uint32_t* proj_dtypes, const uint8_t* weights_bin_host,
@@ -242,8 +246,16 @@ int32_t forge_hip_gemv_q_f32act(const forge_hip_qweight* w, const float* x_dev, 
  * are still exact and the f32 combine is within 1e-3, for data whose per-block activation scale is below 256 (largest
  * activation of a block below 32 512) and whose weight scales are below 2: the kernel removes a bias from its block sums with
  * an fp16 matrix instruction on scales multiplied by powers of two, which is exact inside that range only.
- * A Q4_K / Q6_K handle: the reference has no batched matmul for these formats; the call computes M rows of
- * matmul_vec_q4_k / _q6_k (each row with forge_hip_gemv_q's bits, whatever `flags` says), reading the matrix once per 8 rows. */
+ * A Q4_K / Q6_K handle: the reference has no batched matmul for these formats.  With FORGE_HIP_FLAG_EXACT the call computes M
+ * rows of matmul_vec_q4_k / _q6_k, each row with forge_hip_gemv_q's bits, reading the matrix once per 8 rows.  Without the
+ * flag it runs the int8 MFMA kernel on a re-expression of the matrix in int8 codes and fp16 block scales (Q4_K: codes
+ * (q - 8) * g with the multiplier g that makes fp16(d * sc / g) * g closest to d * sc, the minimum term as an f32 product over
+ * the activations' block sums; Q6_K: sc * q split into hi and lo codes under the exact scales 64 d and d): block sums stay
+ * exact, results lie within 1e-3 of |value| + the row's root mean square.  The first such call builds the re-expression in
+ * device memory (Q4_K: 9.5 bits per weight, Q6_K: 17) and the handle keeps it, so the handle must not be used from two
+ * threads at once; a matrix with a negative Q4_K d or a block scale of 2 or more falls back to the order-faithful rows.
+ * An all-zero block of activations goes into the fast kernel with the scale 0 (the reference's quantiser says 1.0; the codes
+ * are zero either way). */
 int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_t M, float* y_dev, uint32_t flags,
                          void* stream);
 
