@@ -17,6 +17,10 @@ exact_mode: the same workload on a model created with FORGE_HIP_FLAG_EXACT (bit-
 generated kernels): its prefill and decode throughput, and the fast mode's distance from it (first greedy token
 that differs, largest logit difference before that).
 
+kquant_model: the same shape with a storage format per projection (llama.cpp's Q4_K_M recipe, random super-blocks):
+prompt and decode throughput in fast mode (prompt on the MFMA GEMM through re-expressed matrices, decode as a kernel
+sequence) and in the order-faithful mode (prompt through the multi-row K-quant GEMV).
+
 cpu_baseline: the CPU restatement of the reference's generated kernels (oracle/) on this host's cores, on the same
 model and prompt: in the aarch64 arithmetic (int8 activation blocks) the whole prompt as a batched prefill and
 decode steps at that context; in the arithmetic the reference runs on an x86 host (f32 activations x dequantised
@@ -224,6 +228,40 @@ def exact_mode_figures(fh, cfg, blob, prompt, warmup, steps, fast_tokens, fast_l
     return out
 
 
+def kquant_model_figures(fh, cfg, prompt, warmup, steps, seed):
+    """The same shape with llama.cpp's Q4_K_M recipe (Q4_K q/k/o/gate/up, Q6_K v/down/lm_head; random super-blocks): the model
+    with a storage format per projection.  Fast mode: prompt on the int8 MFMA GEMM through the matrices' twins, decode as a
+    kernel sequence; order-faithful mode: prompt through the multi-row K-quant GEMV (bit for bit the reference's
+    token-by-token walk)."""
+    kcfg = dict(cfg)
+    kcfg["lm_head_dtype"] = 14
+    pd = (12, 12, 14, 12, 12, 12, 14)
+    blob = fh.synth.make_weights_blob_mixed(kcfg, pd, seed=seed)
+    t0 = time.perf_counter()
+    m = fh.HipModel(kcfg, blob, proj_dtypes=pd)
+    t_create = time.perf_counter() - t0
+    m.forward_prefill(prompt)                                # first pass: kernels loaded, workspaces touched
+    m.reset()
+    t0 = time.perf_counter()
+    tok = fh.ops.argmax_host(m.forward_prefill(prompt))
+    t_prefill = time.perf_counter() - t0
+    t_decode, tok = timed_decode(m, tok, warmup, steps)
+    out = {"formats": "Q4_K q/k/o/gate/up, Q6_K v/down/lm_head", "weights_bytes": int(blob.size),
+           "prefill_tok_per_s": len(prompt) / t_prefill, "prefill_ms": t_prefill * 1e3,
+           "decode_tok_per_s": steps / t_decode, "decode_launches_per_token": m.decode_launches,
+           "create_s_incl_twins": round(t_create, 2)}
+    m.close()
+    ecfg = dict(kcfg, flags=fh.FLAG_EXACT)
+    e = fh.HipModel(ecfg, blob, proj_dtypes=pd)
+    t0 = time.perf_counter()
+    tok = fh.ops.argmax_host(e.forward_prefill(prompt))
+    t_eprefill = time.perf_counter() - t0
+    t_edecode, tok = timed_decode(e, tok, warmup, steps)
+    out["order_faithful"] = {"prefill_tok_per_s": len(prompt) / t_eprefill, "decode_tok_per_s": steps / t_edecode}
+    e.close()
+    return out
+
+
 def ops_table(fh, reps=10):
     """The isolated kernels at the sizes of the benchmark configurations (GEMV and GEMM at Llama-3.2-1B projection
     shapes, prefill attention at 801/1501/3001 tokens, decode attention over 900/2250/8192-token caches), `reps` calls
@@ -325,6 +363,7 @@ def main():
     ap.add_argument("--no-alt", action="store_true", help="skip the second model that measures the kernel-sequence decode step")
     ap.add_argument("--no-exact", action="store_true",
                     help="skip the third model that measures the exact mode and the fast mode's distance from it")
+    ap.add_argument("--no-kquant", action="store_true", help="skip the Q4_K_M-recipe model of the same shape")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one 1 GiB device-to-device copy kernel (known HBM traffic, for scaling counter readings)")
     ap.add_argument("--model", choices=("llama32_1b", "llama32_3b", "smollm2_135m", "llama31_8b", "qwen25_1p5b", "mistral_7b", "phi3_mini", "qwen25_14b"), default="llama32_1b",
@@ -451,6 +490,9 @@ def main():
         finally:
             os.environ["FORGE_HIP_PERSIST"] = "1"
     exact = None if args.no_exact else exact_mode_figures(fh, cfg, blob, prompt, args.warmup, args.steps, fast_tokens, fast_logits)
+    kquant = None
+    if not args.no_kquant and cfg["hidden"] % 256 == 0 and cfg["inter"] % 256 == 0 and not cfg.get("sliding_window") and not (cfg.get("flags", 0) & 2):
+        kquant = kquant_model_figures(fh, cfg, prompt, args.warmup, args.steps, args.seed)
     if args.calibrate_copy:
         src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").fill_(1.0)     # 1 GiB
         dst = torch.empty_like(src)
@@ -495,6 +537,7 @@ def main():
         },
         "decode_stage_us": stage_us,
         "kernel_sequence_path": alt,
+        "kquant_model": kquant,
         "setup_s": {"generate_weights": round(t_gen, 1), "upload_and_repack": round(t_load, 1)},
         "gguf_load": gguf_info,
     }
