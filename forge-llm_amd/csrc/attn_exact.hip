@@ -123,7 +123,10 @@ __global__ void attn_exact_kernel(const float* __restrict__ q, uint32_t q_stride
 // P.V (the block's V column in registers, the weights broadcast from LDS, added in key order straight into the
 // accumulator).  Every query keeps the reference's own per-row block structure: blocks start at multiples of 64, a block
 // past a row's last key leaves that row untouched, a row's last block is walked for its own number of keys only.
-template <int HD>
+// BATCH = false: the rows in attention_flash's own order (emit.rs:656-715: a block's weighted values are summed first and the
+// sum is added to the accumulator), for the rows of a prompt that the reference walks token by token through the decode
+// attention (models with a format per projection).
+template <int HD, bool BATCH = true>
 __global__ __launch_bounds__(64) void attn_exact_batch_group_kernel(const float* __restrict__ q, uint32_t q_stride,
                                                                     const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
                                                                     float* __restrict__ out, uint32_t out_stride, uint32_t base_pos,
@@ -254,21 +257,26 @@ __global__ __launch_bounds__(64) void attn_exact_batch_group_kernel(const float*
                 const float exp_scale = es[qi];
 #pragma unroll
                 for (int t = 0; t < DPL; t++) acc[qi][t] = acc[qi][t] * exp_scale;
+                float part[DPL];                 // BATCH: the accumulator itself; else the block's own sum
+#pragma unroll
+                for (int t = 0; t < DPL; t++) part[t] = BATCH ? acc[qi][t] : 0.f;
                 if (bl == XB) {
 #pragma unroll
                     for (int bi = 0; bi < XB; bi++) {
                         const float e = se[qi][bi];
 #pragma unroll
-                        for (int t = 0; t < DPL; t++) acc[qi][t] = acc[qi][t] + e * vf[bi][t];
+                        for (int t = 0; t < DPL; t++) part[t] = part[t] + e * vf[bi][t];
                     }
                 } else {
 #pragma unroll
                     for (int bi = 0; bi < XB; bi++) {
                         const float e = se[qi][bi];
 #pragma unroll
-                        for (int t = 0; t < DPL; t++) acc[qi][t] = (uint32_t)bi < bl ? acc[qi][t] + e * vf[bi][t] : acc[qi][t];
+                        for (int t = 0; t < DPL; t++) part[t] = (uint32_t)bi < bl ? part[t] + e * vf[bi][t] : part[t];
                     }
                 }
+#pragma unroll
+                for (int t = 0; t < DPL; t++) acc[qi][t] = BATCH ? part[t] : acc[qi][t] + part[t];
                 }
             }
         }
@@ -525,15 +533,18 @@ void launch_attn_exact(bool batch_order, const float* q, uint32_t q_stride, cons
 #undef FH_XD
         return;
     }
-    // batched prefill without a window: a wave per 16 queries of one KV head (needs the f32 output form and at most 16
-    // heads per KV head; FORGE_HIP_EXACT_GROUP=0: the one-query kernel)
+    // many rows without a window, in either order: a wave per 16 queries of one KV head (needs the f32 output form and at most
+    // 16 heads per KV head; FORGE_HIP_EXACT_GROUP=0: the one-query kernel)
     static const bool group_ok = [] { const char* e = getenv("FORGE_HIP_EXACT_GROUP"); return !(e && e[0] == '0'); }();
-    if (group_ok && batch_order && window == 0 && M > 1 && out && !oq && !pos_dev && heads / kv_heads <= 16) {
+    if (group_ok && window == 0 && M > 1 && out && !oq && !pos_dev && heads / kv_heads <= 16) {
         const uint32_t rows_per_wg = 16 / (heads / kv_heads);
         dim3 gg(kv_heads, (M + rows_per_wg - 1) / rows_per_wg);
-        if (hd == 64) fh::launch(attn_exact_batch_group_kernel<64>, gg, 64, 0, s, q, q_stride, kc, vc, out, out_stride, base_pos, M, heads, kv_heads, rows_per_wg);
-        else if (hd == 96) fh::launch(attn_exact_batch_group_kernel<96>, gg, 64, 0, s, q, q_stride, kc, vc, out, out_stride, base_pos, M, heads, kv_heads, rows_per_wg);
-        else fh::launch(attn_exact_batch_group_kernel<128>, gg, 64, 0, s, q, q_stride, kc, vc, out, out_stride, base_pos, M, heads, kv_heads, rows_per_wg);
+#define FH_AXG(HD_, B_) \
+    fh::launch(attn_exact_batch_group_kernel<HD_, B_>, gg, 64, 0, s, q, q_stride, kc, vc, out, out_stride, base_pos, M, heads, kv_heads, rows_per_wg)
+        if (hd == 64) { if (batch_order) FH_AXG(64, true); else FH_AXG(64, false); }
+        else if (hd == 96) { if (batch_order) FH_AXG(96, true); else FH_AXG(96, false); }
+        else { if (batch_order) FH_AXG(128, true); else FH_AXG(128, false); }
+#undef FH_AXG
         return;
     }
     dim3 grid(heads, M);
