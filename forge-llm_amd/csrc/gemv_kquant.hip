@@ -525,9 +525,10 @@ template <KqPro PRO>
 void launch_kq_multi(const QWeight* const* w, float* const* y, uint32_t n, const KqIn& in, bool accumulate, hipStream_t s) {
     if (n == 0) return;
     const uint32_t K = w[0]->K, nblk = K / 32;
-    uint32_t nmax = 0;
-    for (uint32_t i = 0; i < n; i++) nmax = std::max(nmax, w[i]->N);
-    const int rw = nmax >= 16384 ? 4 : nmax >= 4096 ? 2 : 1;
+    uint32_t ntot = 0;
+    for (uint32_t i = 0; i < n; i++) ntot += w[i]->N;
+    // rows a wave keeps in flight, by the rows of the whole launch
+    const int rw = ntot >= 16384 ? 4 : ntot >= 4096 ? 2 : 1;
     KqMulti a{};
     a.n = n;
     uint32_t total = 0;
