@@ -1008,7 +1008,6 @@ int32_t forge_hip_gguf_export_weights_mixed(const forge_hip_gguf* g, const forge
         const uint64_t need = forge_hip_weights_nbytes_mixed(c, pd);
         if (need == 0 || nbytes != need)
             return fh::fail(FORGE_HIP_ERR_BLOB_SIZE, "gguf_export_weights_mixed: buffer is " + std::to_string(nbytes) + " bytes, config needs " + std::to_string(need));
-        FH_CHECK(!(c->flags & FORGE_HIP_FLAG_QKV_BIAS), "gguf_export_weights_mixed: QKV bias goes with uniformly Q8_0 / Q4_0 models only");
         const uint64_t H = c->hidden, I = c->inter, QKS = (uint64_t)c->heads * c->head_dim, KV = (uint64_t)c->kv_heads * c->head_dim, V = c->vocab;
         auto known = [](uint32_t d) { return d == FORGE_HIP_Q8_0 || d == FORGE_HIP_Q4_0 || d == FORGE_HIP_Q4_K || d == FORGE_HIP_Q6_K; };
         for (int i = 0; i < 7; i++) FH_CHECK(known(pd[i]), "gguf_export_weights_mixed: a projection's format must be Q8_0, Q4_0, Q4_K or Q6_K");
@@ -1034,6 +1033,11 @@ int32_t forge_hip_gguf_export_weights_mixed(const forge_hip_gguf* g, const forge
             FH_STEP(write_in_format(g, blk(l, "attn_q.weight"), pd[0], QKS * H, p), qbytes_any(pd[0], QKS * H));
             FH_STEP(write_in_format(g, blk(l, "attn_k.weight"), pd[1], KV * H, p), qbytes_any(pd[1], KV * H));
             FH_STEP(write_in_format(g, blk(l, "attn_v.weight"), pd[2], KV * H, p), qbytes_any(pd[2], KV * H));
+            if (c->flags & FORGE_HIP_FLAG_QKV_BIAS) {      // main.rs:2737-2742
+                FH_STEP(write_f32(g, blk(l, "attn_q.bias"), QKS, p), QKS * 4);
+                FH_STEP(write_f32(g, blk(l, "attn_k.bias"), KV, p), KV * 4);
+                FH_STEP(write_f32(g, blk(l, "attn_v.bias"), KV, p), KV * 4);
+            }
             FH_STEP(write_in_format(g, blk(l, "attn_output.weight"), pd[3], H * QKS, p), qbytes_any(pd[3], H * QKS));
             FH_STEP(write_f32(g, blk(l, "ffn_norm.weight"), H, p), H * 4);
             FH_STEP(write_in_format(g, blk(l, "ffn_gate.weight"), pd[4], I * H, p), qbytes_any(pd[4], I * H));

@@ -283,7 +283,7 @@ void enqueue_mixed_layer(forge_hip_model* m, uint32_t l, uint32_t pos, const uin
     {
         StageMark t(m, ST_ROPE);
         launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), 1, pos, pos_dev, c.heads, c.kv_heads,
-                             c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), nullptr, s, m->pt);
+                             c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s, m->pt);
     }
     {
         StageMark t(m, ST_ATTN);
@@ -382,7 +382,7 @@ void enqueue_mixed_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uin
     {
         StageMark t(m, ST_ROPE);
         launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos, nullptr, c.heads, c.kv_heads,
-                             c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), nullptr, s, m->pt);
+                             c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s, m->pt);
     }
     if (exact) {
         { StageMark t(m, ST_ATTN); launch_attn_exact(false, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, 0u, c.max_seq, nullptr, s); }
@@ -450,7 +450,7 @@ void enqueue_mixed_prefill_layer_mfma(forge_hip_model* m, uint32_t l, uint32_t M
     {
         StageMark t(m, ST_ROPE);
         launch_rope_kv_store(qkv, qkv + QKS, qkv + QKS + KV, QKV, QKV, m->kc(l), m->vc(l), M, base_pos, nullptr, c.heads, c.kv_heads,
-                             c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), nullptr, s, m->pt);
+                             c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s, m->pt);
     }
     {
         StageMark t(m, ST_ATTN);
@@ -645,6 +645,7 @@ uint64_t forge_hip_weights_nbytes_mixed(const forge_hip_config* c, const uint32_
     const uint64_t H = c->hidden, I = c->inter, QKS = mul(c->heads, c->head_dim), KV = mul(c->kv_heads, c->head_dim);
     uint64_t per_layer = add(mul(H, 8), add(add(w(pd[0], QKS, H), add(w(pd[1], KV, H), w(pd[2], KV, H))), w(pd[3], H, QKS)));
     per_layer = add(per_layer, add(add(w(pd[4], I, H), w(pd[5], I, H)), w(pd[6], H, I)));
+    if (c->flags & FORGE_HIP_FLAG_QKV_BIAS) per_layer = add(per_layer, mul(add(QKS, mul(KV, 2)), 4));       // q | k | v bias, project.rs:286-292
     const uint64_t total = add(add(mul(mul(c->vocab, H), 4), mul(c->layers, per_layer)), add(mul(H, 4), w(c->lm_head_dtype, c->vocab, H)));
     return over ? 0 : total;
 }
@@ -676,10 +677,9 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
     if (rc) return rc;
     FH_CHECK(blob, "model_create: null weights");
     if (pd) {
-        // what the per-projection path covers: no QKV bias, no sliding window (the reference's per-token prefill runs full
-        // attention even for a model with a window, emit.rs:4717-4720: not restated), K-quant matrices over K % 256 == 0
-        FH_CHECK((cfg->flags & FORGE_HIP_FLAG_QKV_BIAS) == 0 && cfg->sliding_window == 0,
-                 "model_create_mixed: QKV bias and sliding windows are covered for uniformly Q8_0 / Q4_0 models only");
+        // what the per-projection path covers: no sliding window (the reference's per-token prefill runs full attention even
+        // for a model with a window, emit.rs:4717-4720: not restated), K-quant matrices over K % 256 == 0
+        FH_CHECK(cfg->sliding_window == 0, "model_create_mixed: sliding windows are covered for uniformly Q8_0 / Q4_0 models only");
         const uint32_t kin[7] = {cfg->hidden, cfg->hidden, cfg->hidden, cfg->heads * cfg->head_dim, cfg->hidden, cfg->hidden, cfg->inter};
         for (int i = 0; i < 7; i++)
             FH_CHECK(!is_kquant(pd[i]) || kquant_k_supported(kin[i]), "model_create_mixed: a K-quant projection needs an input width that is a multiple of 256, at most 16384");
@@ -753,6 +753,11 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
             p += wsize(pd[1], KV, H);
             if ((rc = qweight_upload(pd[2], p, H, KV, &L.v))) return rc;
             p += wsize(pd[2], KV, H);
+            if (has_bias) {                                   // q_bias | k_bias | v_bias, project.rs:286-292
+                L.qkv_bias = m->biases.as<float>() + (size_t)l * m->QKV;
+                FH_HIP(hipMemcpy(L.qkv_bias, p, (size_t)m->QKV * 4, hipMemcpyHostToDevice));
+                p += (size_t)m->QKV * 4;
+            }
             if ((rc = qweight_upload(pd[3], p, QKS, H, &L.o))) return rc;
             p += wsize(pd[3], H, QKS);
             FH_HIP(hipMemcpy(L.ffn_norm, p, H * 4, hipMemcpyHostToDevice));

@@ -216,9 +216,12 @@ def make_weights_blob_mixed(cfg: dict, proj_dtypes, seed: int, std: float = 0.02
 
     pq, pk, pv, po, pg, pu, pdn = [int(x) for x in proj_dtypes]
     parts = [normal(sub_seed(), cfg["vocab"] * H, std, threads).view(np.uint8)]
+    has_bias = bool(cfg.get("flags", 0) & 2)
     for _ in range(cfg["layers"]):
-        parts += [norm_vec().view(np.uint8), mat(QKS, H, pq), mat(KV, H, pk), mat(KV, H, pv), mat(H, QKS, po),
-                  norm_vec().view(np.uint8), mat(I, H, pg), mat(I, H, pu), mat(H, I, pdn)]
+        parts += [norm_vec().view(np.uint8), mat(QKS, H, pq), mat(KV, H, pk), mat(KV, H, pv)]
+        if has_bias:                                        # q_bias | k_bias | v_bias, f32 (project.rs:286-292)
+            parts.append(normal(sub_seed(), QKS + 2 * KV, 0.5, 1).astype(np.float32).view(np.uint8))
+        parts += [mat(H, QKS, po), norm_vec().view(np.uint8), mat(I, H, pg), mat(I, H, pu), mat(H, I, pdn)]
     parts += [norm_vec().view(np.uint8), mat(cfg["vocab"], H, cfg["lm_head_dtype"])]
     return np.concatenate(parts)
 

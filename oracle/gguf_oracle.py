@@ -594,7 +594,10 @@ def export_weights_mixed(oracle, g, data, cfg, pd) -> np.ndarray:
     for l in range(cfg["layers"]):
         b = f"blk.{l}."
         parts += [f32(b + "attn_norm.weight", H), put(b + "attn_q.weight", QKS * H, pd[0]), put(b + "attn_k.weight", KV * H, pd[1]),
-                  put(b + "attn_v.weight", KV * H, pd[2]), put(b + "attn_output.weight", H * QKS, pd[3]), f32(b + "ffn_norm.weight", H),
+                  put(b + "attn_v.weight", KV * H, pd[2])]
+        if cfg.get("flags", 0) & 2:                                          # main.rs:2737-2742
+            parts += [f32(b + "attn_q.bias", QKS), f32(b + "attn_k.bias", KV), f32(b + "attn_v.bias", KV)]
+        parts += [put(b + "attn_output.weight", H * QKS, pd[3]), f32(b + "ffn_norm.weight", H),
                   put(b + "ffn_gate.weight", I * H, pd[4]), put(b + "ffn_up.weight", I * H, pd[5]), put(b + "ffn_down.weight", H * I, pd[6])]
     parts.append(f32("output_norm.weight", H))
     lm_name = "output.weight" if "output.weight" in by_name else "lm_head.weight" if "lm_head.weight" in by_name else "token_embd.weight"

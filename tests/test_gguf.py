@@ -821,7 +821,7 @@ def test_kquant_quantisers_meet_the_reference_tests_bounds(fh, gg, oracle):
         gg.quantize_kquant(13, np.zeros(256, np.float32))
 
 
-def _kquant_file(fh, gg, recipe, seed=31, layers=4, tied=False, embed_ty=12, lm_ty=14, extra=None):
+def _kquant_file(fh, gg, recipe, seed=31, layers=4, tied=False, embed_ty=12, lm_ty=14, extra=None, arch="llama"):
     """A llama-architecture GGUF file of a small random model whose tensors are stored by `recipe(layer, suffix) -> type id`
     (12 = Q4_K, 14 = Q6_K, 8, 2); returns (bytes, {name: (type, raw bytes)}, shape dict)."""
     shape = dict(hidden=256, inter=512, layers=layers, heads=4, kv_heads=2, head_dim=64, vocab=512)
@@ -845,13 +845,16 @@ def _kquant_file(fh, gg, recipe, seed=31, layers=4, tied=False, embed_ty=12, lm_
                                   ("ffn_up", I, H), ("ffn_down", H, I)):
             ty = recipe(l, suffix)
             t[f"blk.{l}.{suffix}.weight"] = ([k, n_rows], ty, store(ty, n_rows, k))
+        if arch == "qwen2":                                   # the bias vectors go with the architecture (main.rs:770)
+            for suffix, n in (("attn_q", QKS), ("attn_k", KV), ("attn_v", KV)):
+                t[f"blk.{l}.{suffix}.bias"] = ([n], gg.F32, rng.normal(0, 0.5, n).astype(np.float32).view(np.uint8))
     t["output_norm.weight"] = ([H], gg.F32, (1 + 0.1 * rng.normal(0, 1, H)).astype(np.float32).view(np.uint8))
     if not tied:
         t["output.weight"] = ([H, V], lm_ty, store(lm_ty, V, H))
-    meta = [("general.architecture", gg.STRING, "llama"), ("llama.embedding_length", gg.U32, H), ("llama.block_count", gg.U32, layers),
-            ("llama.attention.head_count", gg.U32, 4), ("llama.attention.head_count_kv", gg.U32, 2), ("llama.feed_forward_length", gg.U32, I),
-            ("llama.vocab_size", gg.U32, V), ("llama.context_length", gg.U32, 640), ("llama.attention.layer_norm_rms_epsilon", gg.FLOAT32, 1e-5),
-            ("llama.rope.freq_base", gg.FLOAT32, 10000.0)] + list(extra or [])
+    meta = [("general.architecture", gg.STRING, arch), (arch + ".embedding_length", gg.U32, H), (arch + ".block_count", gg.U32, layers),
+            (arch + ".attention.head_count", gg.U32, 4), (arch + ".attention.head_count_kv", gg.U32, 2), (arch + ".feed_forward_length", gg.U32, I),
+            (arch + ".vocab_size", gg.U32, V), (arch + ".context_length", gg.U32, 640), (arch + ".attention.layer_norm_rms_epsilon", gg.FLOAT32, 1e-5),
+            (arch + ".rope.freq_base", gg.FLOAT32, 10000.0)] + list(extra or [])
     data = gg.write_gguf(meta, [(n, d, g, b) for n, (d, g, b) in t.items()])
     return data, {n: (g, np.ascontiguousarray(b, np.uint8).reshape(-1)) for n, (d, g, b) in t.items()}, shape
 
@@ -918,6 +921,44 @@ def test_category_rules_on_other_files(fh, gg, go, oracle):
     cfg, pd, _ = f.config_mixed()
     with pytest.raises(fh.ForgeHipError):
         f.export_weights_mixed(cfg, [13] + pd[1:])
+
+
+def test_qwen2_q4_k_m_file_carries_its_bias_vectors(fh, gg, go, oracle):
+    """A Qwen2 file in the Q4_K_M recipe: the bias flag comes with the architecture (main.rs:770) and the export writes
+    q | k | v bias after the v weights of every layer (main.rs:2737-2742), whatever the weight formats."""
+    data, raw, shape = _kquant_file(fh, gg, _q4_k_m, arch="qwen2", layers=2)
+    f, o = gg.GgufFile(data), go.parse(data)
+    cfg, pd, embed = f.config_mixed()
+    assert cfg["flags"] & 2 and pd == [12, 12, 14, 12, 12, 12, 14] and (cfg, pd, embed) == go.config_mixed(o)
+    blob = f.export_weights_mixed(cfg, pd)
+    assert np.array_equal(blob, go.export_weights_mixed(oracle, o, data, cfg, pd))
+    H, V = 256, 512
+    at = V * H * 4 + H * 4 + 256 * 144 + 128 * 144 + 128 * 210          # embedding, layer 0: norm, q, k (Q4_K), v (Q6_K)
+    want = np.concatenate([raw[f"blk.0.attn_{n}.bias"][1] for n in ("q", "k", "v")])
+    assert np.array_equal(blob[at:at + want.size], want)
+
+
+@pytest.mark.gpu
+def test_qwen2_q4_k_m_model_from_gguf_matches_the_oracle(fh, gg, go, oracle, torch_gpu, tmp_path):
+    data, _, _ = _kquant_file(fh, gg, _q4_k_m, arch="qwen2", layers=2)
+    path = str(tmp_path / "qwen2_q4km.gguf")
+    with open(path, "wb") as fp:
+        fp.write(data)
+    o = go.parse(data)
+    cfg, pd, _ = go.config_mixed(o, flags=fh.FLAG_EXACT)
+    blob = go.export_weights_mixed(oracle, o, data, cfg, pd)
+    gm = fh.HipModel.from_gguf(path, flags=fh.FLAG_EXACT)
+    assert gm.proj_dtypes == pd and gm.config["flags"] & 2
+    om = oracle.Model(cfg, blob, 0, 1, proj_dtypes=pd)
+    prompt = fh.synth.uniform_ids(9, 21, cfg["vocab"])
+    gl, ol = gm.forward_prefill(prompt), om.prefill_batched(prompt)
+    assert np.array_equal(gl.view(np.uint32), ol.view(np.uint32))
+    tok = oracle.argmax(ol)
+    for _ in range(8):
+        g, w = gm.forward(tok), om.forward(tok)
+        assert np.array_equal(g.view(np.uint32), w.view(np.uint32))
+        tok = oracle.argmax(w)
+    gm.close()
 
 
 @pytest.mark.gpu

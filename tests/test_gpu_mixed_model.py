@@ -107,6 +107,42 @@ def test_mixed_model_prompt_in_batches_equals_token_by_token(fh, oracle, torch_g
     walk.close(); batch.close()
 
 
+@pytest.mark.parametrize("mix", ["q4_k_m", "all_four"])
+def test_mixed_model_with_qkv_bias(fh, oracle, torch_gpu, monkeypatch, mix):
+    """Qwen2's q / k / v bias (emit.rs:4105-4120 in forward, :4663-4675 in the token-by-token prompt; blob project.rs:286-292)
+    in a model with a format per projection.  Order-faithful mode: prompt (in batches for the all-K-quant mix, token by
+    token for the other), cache rows and 12 greedy steps bit for bit the oracle's; the batched prompt equals the walk.  Fast
+    mode (prompt on the MFMA GEMM): first-layer cache rows and logits to the fast mode's bounds."""
+    pd, lm = MIXES[mix]
+    cfg = tiny(fh, lm, EXACT | QKV_BIAS)
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=61, std=0.05)
+    toks = fh.synth.uniform_ids(19, 45, cfg["vocab"])
+    gm = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    om = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
+    gl, ol = gm.forward_prefill(toks), om.prefill_batched(toks)
+    same_bits(gl, ol)
+    for layer in range(cfg["layers"]):
+        for which in (0, 1):
+            same_bits(oracle.f16_to_f32(gm.read_kv(layer, which)), om.read_kv(layer, which))
+    first_layer = [om.read_kv(0, which).copy() for which in (0, 1)]
+    tok = oracle.argmax(ol)
+    for _ in range(12):
+        g, o = gm.forward(tok), om.forward(tok)
+        same_bits(g, o)
+        tok = oracle.argmax(o)
+    monkeypatch.setenv("FORGE_HIP_MIXED_BATCH", "0")
+    walk = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    monkeypatch.delenv("FORGE_HIP_MIXED_BATCH")
+    same_bits(walk.forward_prefill(toks), gl)
+    walk.close(); gm.close()
+    fast = fh.HipModel(dict(cfg, flags=QKV_BIAS), blob, proj_dtypes=pd)
+    fl = fast.forward_prefill(toks)
+    for which in (0, 1):
+        rows_close(oracle.f16_to_f32(fast.read_kv(0, which)), first_layer[which])
+    assert np.max(np.abs(fl - ol)) < 0.1 * max(1.0, float(np.std(ol)) * 4) and np.corrcoef(fl, ol)[0, 1] > 0.995
+    fast.close()
+
+
 def test_mixed_model_greedy_tokens_at_a_real_width(fh, oracle, torch_gpu):
     """Llama-3.2-1B's widths (hidden 2048 = 8 super-blocks per row, inter 8192, 32:8 heads of 64) in the Q4_K_M recipe:
     prompt + 24 greedy tokens, ids identical to the oracle's."""
@@ -229,12 +265,12 @@ def test_mixed_model_refusals(fh, torch_gpu):
     with pytest.raises(fh.ForgeHipError) as e:                 # blob of another mix
         fh.HipModel(cfg, blob, proj_dtypes=MIXES["all_four"][0])
     assert e.value.code == fh.ERR_BLOB_SIZE
-    for bad in (dict(flags=QKV_BIAS), dict(sliding_window=64)):
-        c = dict(cfg)
-        c.update(bad)
-        with pytest.raises(fh.ForgeHipError) as e:
-            fh.HipModel(c, blob, proj_dtypes=pd)
-        assert e.value.code == fh.ERR_INVALID
+    with pytest.raises(fh.ForgeHipError) as e:                 # a window: the reference's token-by-token prompt ignores it, not restated
+        fh.HipModel(dict(cfg, sliding_window=64), blob, proj_dtypes=pd)
+    assert e.value.code == fh.ERR_INVALID
+    with pytest.raises(fh.ForgeHipError) as e:                 # the bias flag without bias vectors in the blob
+        fh.HipModel(dict(cfg, flags=QKV_BIAS), blob, proj_dtypes=pd)
+    assert e.value.code == fh.ERR_BLOB_SIZE
     # SmolLM2's hidden 576 is no multiple of a 256-weight super-block
     c = tiny(fh, Q8, 0, hidden=576, inter=1536, heads=9, kv_heads=3)
     with pytest.raises(fh.ForgeHipError) as e:

@@ -130,6 +130,11 @@ def test_blob_size_contract_with_a_format_per_projection(fh, oracle):
         assert n == oracle.weights_nbytes_mixed(c, pd)
         assert fh.synth.make_weights_blob_mixed(c, pd, seed=1).size == n
     assert weights_nbytes_mixed(dict(cfg, wdtype=Q4, lm_head_dtype=Q4), (2,) * 7) == weights_nbytes(dict(cfg, wdtype=Q4, lm_head_dtype=Q4))
+    # Qwen2's bias vectors (project.rs:286-292) add (QKS + 2 KV) floats per layer whatever the formats
+    cb = dict(cfg, lm_head_dtype=14, flags=2)
+    pdm = (12, 12, 14, 12, 12, 12, 14)
+    assert weights_nbytes_mixed(cb, pdm) == weights_nbytes_mixed(dict(cb, flags=0), pdm) + 2 * (256 + 2 * 128) * 4 == oracle.weights_nbytes_mixed(cb, pdm)
+    assert fh.synth.make_weights_blob_mixed(cb, pdm, seed=1).size == weights_nbytes_mixed(cb, pdm)
     # by hand for one matrix mix: H = 256, I = 512, QKS = 256, KV = 128, 2 layers, vocab 301
     c = dict(cfg, lm_head_dtype=14)
     per_layer = 2 * 256 * 4 + 256 * 144 + 128 * 144 + 128 * 210 + 256 * 144 + 2 * 512 * 144 + 256 * 2 * 210

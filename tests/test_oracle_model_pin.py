@@ -365,6 +365,45 @@ MIXES = [  # (q, k, v, o, gate, up, down), lm_head
 ]
 
 
+def test_model_with_a_format_per_projection_and_qkv_bias_matches_float64_model(oracle, fh):
+    """Qwen2's bias vectors (project.rs:286-292: after the v weights, whatever the formats) in a model with a format per
+    projection: a bias read from the wrong offset, or left out, moves every logit."""
+    pd, lm = MIXES[0]
+    cfg = fh.synth.tiny(wdtype=Q8, max_seq=640, hidden=256, inter=512, layers=2, heads=4, kv_heads=2, head_dim=64, vocab=301)
+    cfg["rope_theta"] = 10000.0
+    cfg["lm_head_dtype"] = lm
+    cfg["flags"] = FLAG_QKV_BIAS
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=17, std=0.05)
+    assert blob.size == oracle.weights_nbytes_mixed(cfg, pd)
+    toks = np.random.default_rng(6).integers(0, cfg["vocab"], 17).astype(np.uint32)
+    want, _ = _forward64(cfg, blob, toks, A, KV_F16, pd, oracle)
+    without, _ = _forward64(dict(cfg, flags=0), np.concatenate([blob[:0], _strip_bias(cfg, blob, pd)]), toks, A, KV_F16, pd, oracle)
+    m = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
+    rows = np.stack([m.forward(int(t)) for t in toks])
+    scale = np.abs(want).max()
+    per_row = np.abs(rows - want).max(axis=1)
+    assert per_row[0] < 1e-5 * scale and (per_row < 1e-4 * scale).sum() >= 3 and per_row.max() < 3e-2 * scale
+    assert np.abs(without - want).max() > 0.2 * scale          # the bias matters at this size: leaving it out is not within the bound
+    m2 = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
+    assert np.array_equal(m2.prefill_batched(toks), rows[-1])
+
+
+def _strip_bias(cfg, blob, pd):
+    """The same blob without its bias vectors."""
+    H, I, V = cfg["hidden"], cfg["inter"], cfg["vocab"]
+    QK, KV = cfg["heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"]
+    parts, at = [blob[:V * H * 4]], V * H * 4
+    for _ in range(cfg["layers"]):
+        n = H * 4 + _nbytes(pd[0], QK, H) + 2 * _nbytes(pd[1], KV, H) if pd[1] == pd[2] else H * 4 + _nbytes(pd[0], QK, H) + _nbytes(pd[1], KV, H) + _nbytes(pd[2], KV, H)
+        parts.append(blob[at:at + n])
+        at += n + (QK + 2 * KV) * 4
+        n = _nbytes(pd[3], H, QK) + H * 4 + _nbytes(pd[4], I, H) + _nbytes(pd[5], I, H) + _nbytes(pd[6], H, I)
+        parts.append(blob[at:at + n])
+        at += n
+    parts.append(blob[at:])
+    return np.concatenate(parts)
+
+
 @pytest.mark.parametrize("variant", [A, B])
 @pytest.mark.parametrize("pd,lm", MIXES)
 def test_model_with_a_format_per_projection_matches_float64_model(oracle, fh, pd, lm, variant):
