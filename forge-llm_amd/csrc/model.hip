@@ -287,12 +287,16 @@ void enqueue_mixed_layer(forge_hip_model* m, uint32_t l, uint32_t pos, const uin
     }
     {
         StageMark t(m, ST_ATTN);
+        // a model with a window: decode steps attend to the last `sliding_window` rows (attention_sliding, emit.rs:4156-4170); a
+        // token of a prompt to every row so far through `attention` (emit.rs:4717-4720), which is attention_sliding's
+        // arithmetic with a window that covers everything
+        const uint32_t win = c.sliding_window == 0 ? 0u : pos_dev ? c.sliding_window : c.max_seq;
         if (exact)
             launch_attn_exact(false, qkv, QKS, m->kc(l), m->vc(l), nullptr, QKS, aq, asc, 1, pos, pos_dev, c.heads, c.kv_heads,
-                              c.head_dim, 0u, c.max_seq, m->attn_ws.p, s);
+                              c.head_dim, win, c.max_seq, m->attn_ws.p, s);
         else
-            launch_attn_decode(qkv, m->kc(l), m->vc(l), nullptr, aq, asc, pos + 1, pos_dev, c.heads, c.kv_heads, c.head_dim, 0u,
-                               m->attn_ws.p, s, m->pt);
+            launch_attn_decode(qkv, m->kc(l), m->vc(l), nullptr, aq, asc, pos + 1, pos_dev, c.heads, c.kv_heads, c.head_dim,
+                               pos_dev ? c.sliding_window : 0u, m->attn_ws.p, s, m->pt);
     }
     { StageMark t(m, ST_O); gemv_any(L.o, aq, asc, x, true, mv, s); }
     {
@@ -385,7 +389,8 @@ void enqueue_mixed_prefill_layer(forge_hip_model* m, uint32_t l, uint32_t M, uin
                              c.head_dim, m->cos_t.as<float>(), m->sin_t.as<float>(), L.qkv_bias, s, m->pt);
     }
     if (exact) {
-        { StageMark t(m, ST_ATTN); launch_attn_exact(false, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, 0u, c.max_seq, nullptr, s); }
+        // (a model with a window: `attention` over all rows so far, see enqueue_mixed_layer)
+        { StageMark t(m, ST_ATTN); launch_attn_exact(false, qkv, QKV, m->kc(l), m->vc(l), attn, QKS, nullptr, nullptr, M, base_pos, nullptr, c.heads, c.kv_heads, c.head_dim, c.sliding_window ? c.max_seq : 0u, c.max_seq, nullptr, s); }
         { StageMark t(m, ST_QUANT); launch_quantize_act(attn, M, QKS, aq, asc, s); }
     } else {
         StageMark t(m, ST_ATTN);
@@ -677,9 +682,11 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
     if (rc) return rc;
     FH_CHECK(blob, "model_create: null weights");
     if (pd) {
-        // what the per-projection path covers: no sliding window (the reference's per-token prefill runs full attention even
-        // for a model with a window, emit.rs:4717-4720: not restated), K-quant matrices over K % 256 == 0
-        FH_CHECK(cfg->sliding_window == 0, "model_create_mixed: sliding windows are covered for uniformly Q8_0 / Q4_0 models only");
+        // what the per-projection path covers: K-quant matrices over K % 256 == 0.  (A model with a sliding window: its prompt
+        // rows see ALL earlier positions -- the reference's token-by-token prompt calls `attention`, not `attention_sliding`,
+        // emit.rs:4717-4720 with use_flash_attention false for such a model, emit.rs:126-128 -- and only decode steps the window.)
+        FH_CHECK(!(cfg->flags & FORGE_HIP_FLAG_EXACT) || cfg->sliding_window == 0 || cfg->max_seq <= attn_exact_max_window(),
+                 "model_create_mixed: FORGE_HIP_FLAG_EXACT with a sliding window needs max_seq <= 12288 (a prompt row's scores sit in LDS)");
         const uint32_t kin[7] = {cfg->hidden, cfg->hidden, cfg->hidden, cfg->heads * cfg->head_dim, cfg->hidden, cfg->hidden, cfg->inter};
         for (int i = 0; i < 7; i++)
             FH_CHECK(!is_kquant(pd[i]) || kquant_k_supported(kin[i]), "model_create_mixed: a K-quant projection needs an input width that is a multiple of 256, at most 16384");

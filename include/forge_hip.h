@@ -133,8 +133,10 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* weigh
  * Decode runs the kernel sequence (K-quant projections over the same normed row share a launch), captured in a graph; the
  * resident decode kernel carries Q8_0 and Q4_0 weights only.  K-quant matrices need an input width that is a multiple of 256.
  * FORGE_HIP_FLAG_QKV_BIAS works as in forge_hip_model_create (the bias vectors follow the v weights of every layer,
- * project.rs:286-292); a sliding window is refused (the reference's token-by-token prompt runs full attention for such a
- * model, emit.rs:4717-4720: not restated).  When all seven formats equal cfg->wdtype and the lm_head is Q8_0 or Q4_0 this is forge_hip_model_create. */
+ * project.rs:286-292).  A sliding window follows the reference's rule for such models: the rows of a prompt see ALL earlier
+ * positions (its token-by-token prompt calls `attention`, never attention_sliding, emit.rs:4717-4720 with
+ * use_flash_attention false, emit.rs:126-128) and only decode steps apply the window (emit.rs:4156-4170); with
+ * FORGE_HIP_FLAG_EXACT such a model needs max_seq <= 12288.  When all seven formats equal cfg->wdtype and the lm_head is Q8_0 or Q4_0 this is forge_hip_model_create. */
 uint64_t forge_hip_weights_nbytes_mixed(const forge_hip_config* cfg, const uint32_t* proj_dtypes);
 int32_t forge_hip_model_create_mixed(const forge_hip_config* cfg, const uint32_t* proj_dtypes, const uint8_t* weights_bin_host,
                                      uint64_t nbytes, forge_hip_model** out);

@@ -921,9 +921,13 @@ static void store_kv(fo_model* m, int l, int64_t pos, const float* k, const floa
     }
 }
 
-// emit.rs:4029-4500.  Returns 0, or -3 when the cache is full.
-// logits == NULL: the lm_head is skipped (a token of the per-token forward_prefill that is not the last one, emit.rs:4553-5048).
-int fo_forward(fo_model* m, uint32_t token, float* logits) {
+// model::forward (emit.rs:4029-4500) and one token of the per-token forward_prefill (emit.rs:4553-5048; logits == NULL: not
+// the prompt's last token, the lm_head is skipped).
+// prompt_walk: the token belongs to a prompt that forward_prefill walks one token at a time (models with a format per
+// projection).  The walk's attention is `attention_flash` when use_flash_attention(config) and plain `attention` otherwise
+// (emit.rs:4717-4720) -- it never calls attention_sliding, so a model with a window (for which use_flash_attention is false,
+// emit.rs:126-128) lets every prompt row see ALL earlier positions; only decode steps apply the window (emit.rs:4156-4170).
+static int forward_impl(fo_model* m, uint32_t token, float* logits, bool prompt_walk) {
     const fo_config& c = m->cfg;
     int64_t H = c.hidden, I = c.inter, QKS = (int64_t)c.heads * c.head_dim, KV = (int64_t)c.kv_heads * c.head_dim;
     int64_t pos = m->len;
@@ -946,8 +950,8 @@ int fo_forward(fo_model* m, uint32_t token, float* logits) {
         rope(k.data(), pos, c.head_dim, c.kv_heads, m->freqs.data());
         store_kv(m, l, pos, k.data(), v.data());
         KVView cv = kv_view(m, l);
-        if (c.sliding_window) attention_sliding(attn.data(), q.data(), cv, pos + 1, c.sliding_window, c.heads, c.kv_heads, c.head_dim);
-        else if (flash) attention_flash(attn.data(), q.data(), cv, pos + 1, c.heads, c.kv_heads, c.head_dim);
+        if (c.sliding_window && !prompt_walk) attention_sliding(attn.data(), q.data(), cv, pos + 1, c.sliding_window, c.heads, c.kv_heads, c.head_dim);
+        else if (flash && !c.sliding_window) attention_flash(attn.data(), q.data(), cv, pos + 1, c.heads, c.kv_heads, c.head_dim);
         else attention_std(attn.data(), q.data(), cv, pos + 1, c.heads, c.kv_heads, c.head_dim);
         matmul_vec_any(m->pd[3], m->variant, proj.data(), attn.data(), L.o, QKS, H, 0);
         for (int64_t i = 0; i < H; i++) hs[i] += proj[i];
@@ -966,6 +970,10 @@ int fo_forward(fo_model* m, uint32_t token, float* logits) {
     return 0;
 }
 
+// emit.rs:4029-4500.  Returns 0, or -3 when the cache is full.
+// logits == NULL: the lm_head is skipped.
+int fo_forward(fo_model* m, uint32_t token, float* logits) { return forward_impl(m, token, logits, false); }
+
 // emit.rs:5118-5486.  logits may be NULL (then the lm_head is skipped).
 int fo_prefill_batched(fo_model* m, const uint32_t* tokens, int64_t n, float* logits) {
     const fo_config& c = m->cfg;
@@ -979,7 +987,7 @@ int fo_prefill_batched(fo_model* m, const uint32_t* tokens, int64_t n, float* lo
         // lm_head once, after the last (emit.rs:4621-5040: chunks of 256 rows, dot8 / dot4 groups and a dot1 tail like
         // forward's)
         for (int64_t r = 0; r < n; r++) {
-            const int rc = fo_forward(m, tokens[r], r == n - 1 ? logits : nullptr);
+            const int rc = forward_impl(m, tokens[r], r == n - 1 ? logits : nullptr, true);
             if (rc) return rc;
         }
         return 0;

@@ -938,6 +938,37 @@ def test_qwen2_q4_k_m_file_carries_its_bias_vectors(fh, gg, go, oracle):
     assert np.array_equal(blob[at:at + want.size], want)
 
 
+def test_mistral_q4_k_m_file_keeps_its_window(fh, gg, go, oracle):
+    data, _, _ = _kquant_file(fh, gg, _q4_k_m, arch="mistral", layers=2, extra=[("mistral.attention.sliding_window", gg.U32, 32)])
+    f, o = gg.GgufFile(data), go.parse(data)
+    cfg, pd, embed = f.config_mixed()
+    assert cfg["sliding_window"] == 32 and not cfg["flags"] & 2 and (cfg, pd, embed) == go.config_mixed(o)
+    assert np.array_equal(f.export_weights_mixed(cfg, pd), go.export_weights_mixed(oracle, o, data, cfg, pd))
+
+
+@pytest.mark.gpu
+def test_mistral_q4_k_m_model_from_gguf_matches_the_oracle(fh, gg, go, oracle, torch_gpu, tmp_path):
+    data, _, _ = _kquant_file(fh, gg, _q4_k_m, arch="mistral", layers=2, extra=[("mistral.attention.sliding_window", gg.U32, 16)])
+    path = str(tmp_path / "mistral_q4km.gguf")
+    with open(path, "wb") as fp:
+        fp.write(data)
+    o = go.parse(data)
+    cfg, pd, _ = go.config_mixed(o, flags=fh.FLAG_EXACT)
+    blob = go.export_weights_mixed(oracle, o, data, cfg, pd)
+    gm = fh.HipModel.from_gguf(path, flags=fh.FLAG_EXACT)
+    assert gm.config["sliding_window"] == 16
+    om = oracle.Model(cfg, blob, 0, 1, proj_dtypes=pd)
+    prompt = fh.synth.uniform_ids(10, 40, cfg["vocab"])
+    gl, ol = gm.forward_prefill(prompt), om.prefill_batched(prompt)
+    assert np.array_equal(gl.view(np.uint32), ol.view(np.uint32))
+    tok = oracle.argmax(ol)
+    for _ in range(8):
+        g, w = gm.forward(tok), om.forward(tok)
+        assert np.array_equal(g.view(np.uint32), w.view(np.uint32))
+        tok = oracle.argmax(w)
+    gm.close()
+
+
 @pytest.mark.gpu
 def test_qwen2_q4_k_m_model_from_gguf_matches_the_oracle(fh, gg, go, oracle, torch_gpu, tmp_path):
     data, _, _ = _kquant_file(fh, gg, _q4_k_m, arch="qwen2", layers=2)

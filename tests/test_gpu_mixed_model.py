@@ -143,6 +143,45 @@ def test_mixed_model_with_qkv_bias(fh, oracle, torch_gpu, monkeypatch, mix):
     fast.close()
 
 
+@pytest.mark.parametrize("mix", ["q4_k_m", "all_four"])
+def test_mixed_model_with_a_sliding_window(fh, oracle, torch_gpu, monkeypatch, mix):
+    """A model with a window and a format per projection (Mistral files in K-quant recipes).  The reference walks its prompt
+    token by token through `attention` over ALL earlier rows (emit.rs:4717-4720; never attention_sliding) and applies the
+    window in decode steps only (emit.rs:4156-4170).  Order-faithful mode: prompt longer than the window (in batches for the
+    all-K-quant mix), a second chunk, cache rows and 14 greedy steps bit for bit the oracle's; fast mode to its bounds."""
+    pd, lm = MIXES[mix]
+    cfg = tiny(fh, lm, EXACT)
+    cfg["sliding_window"] = 24
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=71, std=0.05)
+    toks = fh.synth.uniform_ids(23, 70, cfg["vocab"])
+    gm = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    om = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
+    gl, ol = gm.forward_prefill(toks[:50]), om.prefill_batched(toks[:50])
+    same_bits(gl, ol)
+    first_layer = [om.read_kv(0, which).copy() for which in (0, 1)]
+    same_bits(gm.forward_prefill(toks[50:]), om.prefill_batched(toks[50:]))
+    for which in (0, 1):
+        same_bits(oracle.f16_to_f32(gm.read_kv(1, which)), om.read_kv(1, which))
+    tok = 7
+    for _ in range(14):
+        g, o = gm.forward(tok), om.forward(tok)
+        same_bits(g, o)
+        tok = oracle.argmax(o)
+    gm.close()
+    fast = fh.HipModel(dict(cfg, flags=0), blob, proj_dtypes=pd)
+    fl = fast.forward_prefill(toks[:50])
+    for which in (0, 1):
+        rows_close(oracle.f16_to_f32(fast.read_kv(0, which)), first_layer[which])
+    assert np.max(np.abs(fl - ol)) < 0.1 * max(1.0, float(np.std(ol)) * 4) and np.corrcoef(fl, ol)[0, 1] > 0.995
+    # decode steps with the window: against the oracle fed the same tokens (teacher forcing keeps the contexts equal)
+    om2 = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
+    om2.prefill_batched(toks[:50])
+    for t in (3, 99, 500, 41):
+        a, b = fast.forward(t), om2.forward(t)
+        assert np.max(np.abs(a - b)) < 0.1 * max(1.0, float(np.std(b)) * 4) and np.corrcoef(a, b)[0, 1] > 0.99
+    fast.close()
+
+
 def test_mixed_model_greedy_tokens_at_a_real_width(fh, oracle, torch_gpu):
     """Llama-3.2-1B's widths (hidden 2048 = 8 super-blocks per row, inter 8192, 32:8 heads of 64) in the Q4_K_M recipe:
     prompt + 24 greedy tokens, ids identical to the oracle's."""
@@ -265,8 +304,8 @@ def test_mixed_model_refusals(fh, torch_gpu):
     with pytest.raises(fh.ForgeHipError) as e:                 # blob of another mix
         fh.HipModel(cfg, blob, proj_dtypes=MIXES["all_four"][0])
     assert e.value.code == fh.ERR_BLOB_SIZE
-    with pytest.raises(fh.ForgeHipError) as e:                 # a window: the reference's token-by-token prompt ignores it, not restated
-        fh.HipModel(dict(cfg, sliding_window=64), blob, proj_dtypes=pd)
+    with pytest.raises(fh.ForgeHipError) as e:                 # order-faithful mode keeps a prompt row's scores in LDS: max_seq <= 12288
+        fh.HipModel(dict(cfg, sliding_window=64, max_seq=16384, flags=EXACT), blob, proj_dtypes=pd)
     assert e.value.code == fh.ERR_INVALID
     with pytest.raises(fh.ForgeHipError) as e:                 # the bias flag without bias vectors in the blob
         fh.HipModel(dict(cfg, flags=QKV_BIAS), blob, proj_dtypes=pd)

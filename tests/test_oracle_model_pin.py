@@ -124,8 +124,9 @@ def _kv_round(x, mode):
     return np.clip(np.sign(y) * np.floor(np.abs(y) + 0.5), -127, 127) * np.where(amax > 0, scale, 0.0)
 
 
-def _forward64(cfg, blob, tokens, variant, kvmode, pd=None, oracle=None):
-    """Logits of every prompt position [m][vocab] and the cached K/V per layer, all float64."""
+def _forward64(cfg, blob, tokens, variant, kvmode, pd=None, oracle=None, win_from=0):
+    """Logits of every prompt position [m][vocab] and the cached K/V per layer, all float64.  win_from: the first row the
+    sliding window applies to (rows before it see every earlier position)."""
     t = _cut(cfg, blob, pd, oracle)
     H, hd, nh, nkv = cfg["hidden"], cfg["head_dim"], cfg["heads"], cfg["kv_heads"]
     eps, theta, win = cfg["rms_eps"], cfg["rope_theta"], cfg.get("sliding_window", 0)
@@ -152,7 +153,7 @@ def _forward64(cfg, blob, tokens, variant, kvmode, pd=None, oracle=None):
             s = q[:, h * hd:(h + 1) * hd] @ k[:, g * hd:(g + 1) * hd].T / np.sqrt(hd)
             keep = pos[None, :] <= pos[:, None]
             if win:
-                keep &= pos[None, :] > pos[:, None] - win
+                keep &= (pos[None, :] > pos[:, None] - win) | (pos[:, None] < win_from)
             s = np.where(keep, s, -np.inf)
             p = np.exp(s - s.max(axis=1, keepdims=True))
             out[:, h * hd:(h + 1) * hd] = (p / p.sum(axis=1, keepdims=True)) @ v[:, g * hd:(g + 1) * hd]
@@ -386,6 +387,32 @@ def test_model_with_a_format_per_projection_and_qkv_bias_matches_float64_model(o
     assert np.abs(without - want).max() > 0.2 * scale          # the bias matters at this size: leaving it out is not within the bound
     m2 = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
     assert np.array_equal(m2.prefill_batched(toks), rows[-1])
+
+
+def test_model_with_a_format_per_projection_and_a_window_walks_its_prompt_with_full_attention(oracle, fh):
+    """forward_prefill's token-by-token walk calls `attention` (or attention_flash), never attention_sliding (emit.rs:4717-4720;
+    use_flash_attention is false for a model with a window, emit.rs:126-128): the rows of a prompt see every earlier
+    position, decode steps only the window (emit.rs:4156-4170).  The float64 model with exactly that mask rule; the rule
+    that every row is windowed, and the rule that none is, both miss by far more than the bound."""
+    pd, lm = MIXES[0]
+    cfg = fh.synth.tiny(wdtype=Q8, max_seq=640, hidden=256, inter=512, layers=2, heads=4, kv_heads=2, head_dim=64, vocab=301)
+    cfg["rope_theta"] = 10000.0
+    cfg["lm_head_dtype"] = lm
+    cfg["sliding_window"] = 6
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=23, std=0.05)
+    toks = np.random.default_rng(8).integers(0, cfg["vocab"], 26).astype(np.uint32)
+    n_prompt = 17
+    want, _ = _forward64(cfg, blob, toks, A, KV_F16, pd, oracle, win_from=n_prompt)
+    all_windowed, _ = _forward64(cfg, blob, toks, A, KV_F16, pd, oracle)
+    none_windowed, _ = _forward64(dict(cfg, sliding_window=0), blob, toks, A, KV_F16, pd, oracle)
+    m = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
+    rows = [m.prefill_batched(toks[:n_prompt])] + [m.forward(int(t)) for t in toks[n_prompt:]]
+    got = np.stack(rows)
+    ref = want[n_prompt - 1:]
+    scale = np.abs(want).max()
+    assert np.abs(got - ref).max() < 3e-2 * scale and np.abs(got[0] - ref[0]).max() < 2e-3 * scale
+    assert np.abs(all_windowed[n_prompt - 1] - ref[0]).max() > 0.1 * scale       # the prompt's last row does see more than 6 positions
+    assert np.abs(none_windowed[-1] - ref[-1]).max() > 0.1 * scale               # and the decode rows do not
 
 
 def _strip_bias(cfg, blob, pd):
