@@ -253,14 +253,18 @@ uint32_t attn_exact_max_window();
 
 // decode_persistent.hip — the whole decode step as one resident kernel (fast mode only)
 struct PdLayerIn {
-    const QWeight* qkv;
+    const QWeight* qkv;        // uniform models: the fused matrices
     const QWeight* o;
     const QWeight* gate_up;
     const QWeight* down;
+
     const float* attn_norm;
     const float* ffn_norm;
     uint16_t* kc;
     uint16_t* vc;
+    // K-quant models (every matrix Q4_K or Q6_K; qkv and gate_up are then null): the projections one by one, re-laid out for
+    // the kernel by pd_create.  q and k must share a format, gate and up too; v may have its own.
+    const QWeight *q = nullptr, *k = nullptr, *v = nullptr, *gate = nullptr, *up = nullptr;
 };
 struct PdState;
 // Leaves *out null (returning OK) when the shape or device is not covered; `state` = {position, token, next token, abort flag}.

@@ -95,17 +95,25 @@ struct PdGemv {
 struct PdLayer {
     const uint8_t* qs[4];      // qkv, o, gate_up, down
     const uint16_t* ws[4];
-    const float* attn_norm;
-    const float* ffn_norm;
+    const float* attn_norm;    // [2][H]: the layer's attention norm weights, then its feed-forward norm weights
     uint16_t* kc;
     uint16_t* vc;
 };
 constexpr uint32_t PD_MAX_LAYERS = 34;       // per launch: the descriptors travel as kernel arguments (4 KB in all)
 constexpr uint32_t PD_MAX_SEGMENTS = 8;
-enum { PD_QKV = 0, PD_O = 1, PD_GU = 2, PD_DOWN = 3, PD_LM = 4 };
+enum { PD_QKV = 0, PD_O = 1, PD_GU = 2, PD_DOWN = 3, PD_LM = 4, PD_V = 5 };
+// Weight formats of a phase's matrix.  Q8_0 and Q6_K units hold 32 blocks (two lanes per block), Q4_0 and Q4_K units 64 (a lane per
+// block).  The K-quant matrices are re-laid out for this kernel when the model is created (pd_create_kquant):
+//   Q4_K  codes: 16 bytes per 32-weight sub-block in Q4_0's byte order (byte i = weight i | weight i + 16 << 4), values 0..15;
+//         one word per sub-block b: fp16 bits of d (b even) or dmin (b odd) | 6-bit scale << 16 | 6-bit minimum << 24 -- the two
+//         sub-blocks of a pair belong to one super-block, so a lane gets the other half from its neighbour
+//   Q6_K  16 bytes per 16-weight half block: byte i of the first eight = code i % 4 + 8 (i / 4)'s low nibble | code + 4's << 4,
+//         bytes 8..11 the 2-bit high parts (byte i: codes i, i + 4, i + 8, i + 12), byte 12 the int8 scale, bytes 14..15 d (fp16)
+enum { WF_Q8 = 0, WF_Q4 = 1, WF_Q4K = 2, WF_Q6K = 3 };
+__host__ __device__ constexpr bool wf_lane_per_block(int wf) { return wf == WF_Q4 || wf == WF_Q4K; }
 
 struct PdArgs {
-    PdGemv shape[5];           // qkv, o, gate_up, down (addresses per layer, below) and lm_head (addresses here)
+    PdGemv shape[6];           // qkv, o, gate_up, down (addresses per layer, below), lm_head (addresses here) and, with split_v, v
     uint32_t n_layers, H, I, QKS, KV, heads, kv_heads, gt;   // n_layers: the layers of THIS launch, layers[0 .. n_layers)
     // A model of more layers than the descriptor array holds runs its step as several launches in a row: layers
     // [layer0, layer0 + n_layers) of total_layers; the first launch starts from the embedding row, the last one ends with
@@ -134,7 +142,11 @@ struct PdArgs {
     uint32_t step_seq;                         // number of this step (never 0): left in state[4] by whoever counts the step's token
     unsigned long long* host_out;              // host-mapped {next token, launch number}: written last, or null
     uint32_t host_seq;
-    uint32_t q4, lm_q4;                        // weight formats: projections, lm_head
+    // weight format of each matrix (WF_*): [PD_QKV .. PD_LM] and [PD_V].  split_v: the v rows are a matrix of their own
+    // (shape[PD_V], another format than q and k: llama.cpp's K-quant recipes), its planes `v_qs_off` / `v_ws_off` bytes
+    // behind the layer's q;k planes; shape[PD_QKV] then holds the q and k rows only.
+    uint32_t wf[6];
+    uint32_t split_v, v_qs_off, v_ws_off;
     uint32_t* counts;                          // u32 [vocab]: times each token id has been fed (this step's token is added here)
     const float* qkv_bias;                     // optional [layers][QKS + 2 KV]: added to q, k, v before the rotation (Qwen2)
     float penalty;                             // > 1: the argmax is taken over the penalised logits
@@ -385,7 +397,8 @@ struct GemvJob {
     uint32_t which;            // index of the shape in the kernel arguments (PD_QKV .. PD_LM)
     const uint8_t* qs;
     const uint16_t* ws;
-    bool q4;
+    uint32_t wf;               // WF_*
+    uint32_t row_off;          // EPI_ROPE: the matrix's first row is row `row_off` of q | k | v (the v matrix of a split phase)
     int pro, epi;
     const float* norm_w;       // PRO_NORM
     const uint64_t* tin;       // tagged input: residual stream (PRO_NORM) or quantised vector (PRO_AQ)
@@ -441,9 +454,10 @@ __device__ __forceinline__ uint32_t pos_div_u(uint32_t p, const Shape& h) { retu
 // Every slot issues its two loads whatever the shape (slots past the wave's rows and lanes past a row's end re-read a
 // valid address and their data is ignored): the number of loads in flight is then known at compile time and a round can
 // be consumed while the next one is still arriving.
-template <bool Q4>
+template <int WF>
 __device__ __forceinline__ void pd_load_round(const GemvJob& job, const Shape& h, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane,
                                               WReg& W) {
+    constexpr bool Q4 = wf_lane_per_block(WF);
     constexpr uint32_t BPU = Q4 ? 64 : 32, BPB = Q4 ? 16 : 32;
     const uint32_t U = h.U, nblk = h.nblk;
     const uint32_t lb = Q4 ? lane : lane >> 1;
@@ -456,7 +470,9 @@ __device__ __forceinline__ void pd_load_round(const GemvJob& job, const Shape& h
         const uint32_t bc = b < nblk ? b : nblk - 1;
         const uint32_t bi = pd_row(t, lrc) * nblk + bc;             // block index in the matrix (fits 32 bits: N K / 32)
         W.v[d] = ldg(reinterpret_cast<const int4*>(job.qs + (size_t)bi * BPB + (Q4 ? 0u : (lane & 1u) * 16u)));
-        W.s[d] = ldg(job.ws + bi);
+        if (WF == WF_Q4K) W.s[d] = ldg(reinterpret_cast<const uint32_t*>(job.ws) + bi);
+        else if (WF == WF_Q6K) W.s[d] = 0u;                       // scale and d travel inside the 16 bytes
+        else W.s[d] = ldg(job.ws + bi);
         j += 1;
         if (j == U) { j = 0; lr += PD_STREAM_WAVES; }
     }
@@ -467,7 +483,8 @@ struct Mat {
     uint32_t which;            // shape index; valid == false: nothing follows
     const uint8_t* qs;
     const uint16_t* ws;
-    bool q4, valid;
+    uint32_t wf;
+    bool valid;
 };
 template <int FMT>
 __device__ __forceinline__ void pd_load_first(const PdArgs& a, const Mat& m, uint32_t wg, uint32_t sw, uint32_t lane, WReg& W) {
@@ -476,17 +493,21 @@ __device__ __forceinline__ void pd_load_first(const PdArgs& a, const Mat& m, uin
     const TilePos t = pd_tile(h, wg);
     GemvJob j{};
     j.qs = m.qs; j.ws = m.ws;
-    if (FMT == 1 || (FMT == 2 && m.q4)) pd_load_round<true>(j, h, t, 0, sw, lane, W);
-    else pd_load_round<false>(j, h, t, 0, sw, lane, W);
+    if (FMT == 3) {
+        if (m.wf == WF_Q4K) pd_load_round<WF_Q4K>(j, h, t, 0, sw, lane, W);
+        else pd_load_round<WF_Q6K>(j, h, t, 0, sw, lane, W);
+    } else if (FMT == 1 || (FMT == 2 && m.wf == WF_Q4)) pd_load_round<WF_Q4>(j, h, t, 0, sw, lane, W);
+    else pd_load_round<WF_Q8>(j, h, t, 0, sw, lane, W);
 }
 
 // Exact int32 block dots on v_dot4 and one f32 product (a_s*w_s)*f32(isum) per block.
 //   ORDERED   the products are parked in LDS (prod[row][block]) and summed later in the reference's order
 //   otherwise each lane adds its products of a row as they come (`acc`, carried across rounds) and the wave folds
 //             them when the row's last unit is done: rowsum[row].  Same terms, another order of addition.
-template <bool Q4, bool ORDERED>
+template <int WF, bool ORDERED>
 __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane, const WReg& W,
                                                  const uint32_t* aq_lds, const float* as_lds, float* prod, uint32_t pstride, float& acc) {
+    constexpr bool Q4 = wf_lane_per_block(WF);
     constexpr uint32_t BPU = Q4 ? 64 : 32;
     const uint32_t U = h.U, nblk = h.nblk;
     const uint32_t lb = Q4 ? lane : lane >> 1;
@@ -498,6 +519,63 @@ __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& 
             const uint32_t b = j * BPU + lb;
             const bool in = b < nblk;
             const uint32_t bs = in ? b : 0;
+            if (WF == WF_Q4K || WF == WF_Q6K) {
+                // K-quants: the block's term of dot_q4_k_q8_0 / dot_q6_k_q8_0 (emit.rs:3035-3306, 3553-3612) as gemv_kquant.hip forms it
+                float term;
+                bool mine;                                            // this lane reports the block
+                if (WF == WF_Q4K) {
+                    const int4 a0 = *reinterpret_cast<const int4*>(aq_lds + bs * 8);
+                    const int4 a1 = *reinterpret_cast<const int4*>(aq_lds + bs * 8 + 4);
+                    const int4 w = W.v[d];
+                    const int m = 0x0F0F0F0F;
+                    const int4 lo = make_int4(w.x & m, w.y & m, w.z & m, w.w & m);
+                    const int4 hi = make_int4((w.x >> 4) & m, (w.y >> 4) & m, (w.z >> 4) & m, (w.w >> 4) & m);
+                    const int4 ones = make_int4(0x01010101, 0x01010101, 0x01010101, 0x01010101);
+                    const int asum = dot16(ones, a1, dot16(ones, a0, 0));
+                    const int dot = dot16(hi, a1, dot16(lo, a0, 0));
+                    const uint32_t sw_ = W.s[d];
+                    const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)sw_, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
+                    const bool even = !(lane & 1u);
+                    const float dd = f16_bits_to_f32((uint16_t)((even ? sw_ : other) & 0xFFFFu));
+                    const float dmin = f16_bits_to_f32((uint16_t)((even ? other : sw_) & 0xFFFFu));
+                    const float d_w = dd * (float)((sw_ >> 16) & 0xFFu), m_w = dmin * (float)(sw_ >> 24);
+                    term = as_lds[bs] * (d_w * (float)dot - m_w * (float)asum);
+                    mine = in;
+                } else {
+                    const int4 a = *reinterpret_cast<const int4*>(aq_lds + bs * 8 + (lane & 1u) * 4);
+                    const int4 w = W.v[d];
+                    const uint32_t m4 = 0x0F0F0F0Fu, m2 = 0x03030303u;
+                    const uint32_t wx = (uint32_t)w.x, wy = (uint32_t)w.y, wz = (uint32_t)w.z, ww = (uint32_t)w.w;
+                    auto minus32 = [](uint32_t x) { return (int)(((x | 0x80808080u) - 0x20202020u) ^ 0x80808080u); };   // bytes 0..63 -> -32..31
+                    int4 q;
+                    q.x = minus32((wx & m4) | ((wz & m2) << 4));
+                    q.y = minus32(((wx >> 4) & m4) | (((wz >> 2) & m2) << 4));
+                    q.z = minus32((wy & m4) | (((wz >> 4) & m2) << 4));
+                    q.w = minus32(((wy >> 4) & m4) | (((wz >> 6) & m2) << 4));
+                    const int dh = in ? dot16(q, a, 0) : 0;
+                    const float th = (float)(int)(int8_t)(ww & 0xFFu) * (float)dh;
+                    const float u = th + __builtin_amdgcn_update_dpp(0.f, th, 0xB1, 0xF, 0xF, false);       // lo + hi (even lane)
+                    term = (f16_bits_to_f32((uint16_t)(ww >> 16)) * as_lds[bs]) * u;
+                    mine = in && !(lane & 1u);
+                }
+                if (ORDERED) {
+                    if (mine) prod[lr * pstride + b] = term;
+                } else {
+                    if (mine) acc += term;
+                    if (j == U - 1) {
+                        float r = acc;
+                        r += __builtin_amdgcn_update_dpp(0.f, r, 0xB1, 0xF, 0xF, false);     // quad_perm [1,0,3,2]
+                        r += __builtin_amdgcn_update_dpp(0.f, r, 0x4E, 0xF, 0xF, false);     // quad_perm [2,3,0,1]
+                        r += __builtin_amdgcn_update_dpp(0.f, r, 0x141, 0xF, 0xF, false);    // row_half_mirror
+                        r += __builtin_amdgcn_update_dpp(0.f, r, 0x140, 0xF, 0xF, false);    // row_mirror
+                        if ((lane & 15u) == 0) prod[lr * 4 + (lane >> 4)] = r;
+                        acc = 0.f;
+                    }
+                }
+                j += 1;
+                if (j == U) { j = 0; lr += PD_STREAM_WAVES; }
+                continue;
+            }
             int isum;
             if (Q4) {
                 const int4 a0 = *reinterpret_cast<const int4*>(aq_lds + bs * 8);
@@ -1055,7 +1133,7 @@ __device__ __forceinline__ ArgPair arg_wg(ArgPair a, float* misc, const PdCtx& c
 //   inputs    the streamers issue the first weight loads of their rows at once; the poller wave fetches the activation
 //             vector (it never has weights in flight, so nothing delays what it polls)
 //   tiles     compute a round from registers, issue the next round (or the next tile's first), sum, finish the rows
-template <bool Q4, int HD, int FMT, bool ORDERED, bool PEN>
+template <int WF, int HD, int FMT, bool ORDERED, bool PEN>
 __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& job, const Mat& next, bool early, WReg& W, WReg& W1, const float* emb,
                                               uint32_t pos, size_t crow, uint32_t* aq_lds, float* as_lds, float* misc, float* big, ArgPair& best,
                                               const PdCtx& cx) {
@@ -1080,7 +1158,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     float4 nw = make_float4(0.f, 0.f, 0.f, 0.f);
     if (job.pro == PRO_NORM && cx.tid * 4 < K) nw = ldg(reinterpret_cast<const float4*>(job.norm_w + cx.tid * 4));
     if (streamer) {
-        if (!early) pd_load_round<Q4>(job, h, t, 0, sw, cx.lane, W);      // otherwise the previous phase's tail issued them
+        if (!early) pd_load_round<WF>(job, h, t, 0, sw, cx.lane, W);      // otherwise the previous phase's tail issued them
     } else {
         float ssq = 0.f;
         if (job.pro == PRO_AQ) pd_load_aq(job.tin, job.tin_tag, K, aq_lds, as_lds, misc, a.use_hint != 0, cx);
@@ -1111,12 +1189,13 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
         // up to 64 rows)
         const bool mine = cx.tid < t.rows;
         const uint32_t row = pd_row(t, mine ? cx.tid : 0);
+        const uint32_t erow = row + (job.epi == EPI_ROPE ? job.row_off : 0u);      // row of q | k | v
         float rc = 0.f, rs = 0.f;
         uint64_t res_w = 0;
         float res_e = 0.f;
         if (mine) {
-            if (job.epi == EPI_ROPE && row < a.QKS + a.KV) {
-                const uint32_t d = row < a.QKS ? row % HD : (row - a.QKS) % HD;
+            if (job.epi == EPI_ROPE && erow < a.QKS + a.KV) {
+                const uint32_t d = erow < a.QKS ? erow % HD : (erow - a.QKS) % HD;
                 rc = a.cos_t[(size_t)pos * (HD / 2) + d / 2];
                 rs = a.sin_t[(size_t)pos * (HD / 2) + d / 2];
             } else if (job.epi == EPI_ADD) {
@@ -1129,11 +1208,11 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
             // always in W
 #pragma nounroll
             for (uint32_t r = 0; r < rounds; r += 2) {
-                if (r + 1 < rounds) pd_load_round<Q4>(job, h, t, r + 1, sw, cx.lane, W1);
-                pd_compute_round<Q4, ORDERED>(h, t, r, sw, cx.lane, W, aq_lds, as_lds, big, pstride, acc);
+                if (r + 1 < rounds) pd_load_round<WF>(job, h, t, r + 1, sw, cx.lane, W1);
+                pd_compute_round<WF, ORDERED>(h, t, r, sw, cx.lane, W, aq_lds, as_lds, big, pstride, acc);
                 if (r + 1 < rounds) {
-                    if (r + 2 < rounds) pd_load_round<Q4>(job, h, t, r + 2, sw, cx.lane, W);
-                    pd_compute_round<Q4, ORDERED>(h, t, r + 1, sw, cx.lane, W1, aq_lds, as_lds, big, pstride, acc);
+                    if (r + 2 < rounds) pd_load_round<WF>(job, h, t, r + 2, sw, cx.lane, W);
+                    pd_compute_round<WF, ORDERED>(h, t, r + 1, sw, cx.lane, W1, aq_lds, as_lds, big, pstride, acc);
                 }
             }
         }
@@ -1143,30 +1222,30 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
         // long as the data takes to arrive (the memory pipeline holds only so many misses), so it must not sit between
         // the products and the sums.
         if (streamer) {
-            if (more) pd_load_round<Q4>(job, h, tn, 0, sw, cx.lane, W);
+            if (more) pd_load_round<WF>(job, h, tn, 0, sw, cx.lane, W);
             else if (next.valid) pd_load_first<FMT>(a, next, cx.wg, sw, cx.lane, W);
         }
         if (cx.tid < ((t.rows + 63u) & ~63u)) {
             float v = 0.f;
             if (mine) v = ORDERED ? ordered_sum_words(big + cx.tid * pstride, h.nblk, segment_row_is_dot1(row, g.seg, g.nseg, g.tail_mod)) : (big[cx.tid * 4] + big[cx.tid * 4 + 1]) + (big[cx.tid * 4 + 2] + big[cx.tid * 4 + 3]);
             if (job.epi == EPI_ROPE) {
-                if (PEN && job.bias && mine) v = v + job.bias[row];      // the kernel variant with the optional extras carries it
+                if (PEN && job.bias && mine) v = v + job.bias[erow];     // the kernel variant with the optional extras carries it
                 // rope (emit.rs:508-528): rows 2i, 2i+1 of a head sit in neighbouring lanes
                 const float other = lane_xor<1>(v);
                 if (mine) {
-                    if (row < a.QKS + a.KV) {
-                        const float o = (row & 1u) ? other * rs + v * rc : v * rc - other * rs;
-                        if (row < a.QKS) {
-                            stc64(a.tq + row, job.tag_out, __float_as_uint(o));
+                    if (erow < a.QKS + a.KV) {
+                        const float o = (erow & 1u) ? other * rs + v * rc : v * rc - other * rs;
+                        if (erow < a.QKS) {
+                            stc64(a.tq + erow, job.tag_out, __float_as_uint(o));
                         } else {
                             const uint16_t hb = f32_to_f16_bits(o);
-                            stg(job.kc + crow * a.KV + (row - a.QKS), hb);
-                            stc64(a.tkv + (row - a.QKS), job.tag_out, hb);
+                            stg(job.kc + crow * a.KV + (erow - a.QKS), hb);
+                            stc64(a.tkv + (erow - a.QKS), job.tag_out, hb);
                         }
                     } else {
                         const uint16_t hb = f32_to_f16_bits(v);
-                        stg(job.vc + crow * a.KV + (row - a.QKS - a.KV), hb);
-                        stc64(a.tkv + a.KV + (row - a.QKS - a.KV), job.tag_out, hb);
+                        stg(job.vc + crow * a.KV + (erow - a.QKS - a.KV), hb);
+                        stc64(a.tkv + a.KV + (erow - a.QKS - a.KV), job.tag_out, hb);
                     }
                 }
             } else if (job.epi == EPI_ADD) {
@@ -1292,7 +1371,8 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         job.which = ph;
         job.qs = is_lm ? a.shape[PD_LM].qs : a.layers[l].qs[ph];
         job.ws = is_lm ? a.shape[PD_LM].ws : a.layers[l].ws[ph];
-        job.q4 = is_lm ? a.lm_q4 != 0 : a.q4 != 0;
+        job.wf = a.wf[is_lm ? (uint32_t)PD_LM : ph];
+        job.row_off = 0;
         Mat next;
         {
             const uint32_t ns = step + 1;
@@ -1303,11 +1383,11 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
             next.which = nph;
             next.qs = n_lm ? a.shape[PD_LM].qs : a.layers[next.valid ? nl : 0].qs[nph & 3u];
             next.ws = n_lm ? a.shape[PD_LM].ws : a.layers[next.valid ? nl : 0].ws[nph & 3u];
-            next.q4 = n_lm ? a.lm_q4 != 0 : a.q4 != 0;
+            next.wf = a.wf[n_lm ? (uint32_t)PD_LM : nph];
         }
         job.pro = (ph == 1 || ph == 3) ? PRO_AQ : PRO_NORM;
         job.epi = ph == 0 ? EPI_ROPE : ph == 2 ? EPI_SILU : ph == 4 ? EPI_LOGITS : EPI_ADD;
-        job.norm_w = ph == 0 ? a.layers[l].attn_norm : ph == 2 ? a.layers[l].ffn_norm : a.final_norm;
+        job.norm_w = ph == 0 ? a.layers[l].attn_norm : ph == 2 ? a.layers[l].attn_norm + a.H : a.final_norm;
         job.tin = ph == 1 ? a.taq : ph == 3 ? a.taq2 : a.tx;
         job.tin_tag = ph == 0 ? x_in : ph == 1 ? base + 3 : ph == 2 ? base + 4 : ph == 3 ? base + 5 : base + 6;
         job.in_len = ph == 1 ? a.QKS : ph == 3 ? a.I : a.H;
@@ -1316,8 +1396,39 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         job.kc = a.layers[l].kc;
         job.bias = (PEN && a.qkv_bias && ph == 0) ? a.qkv_bias + (size_t)lg * (a.QKS + 2 * a.KV) : nullptr;
         job.vc = a.layers[l].vc;
-        if (FMT == 1 || (FMT == 2 && job.q4)) pd_gemv_phase<true, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
-        else pd_gemv_phase<false, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
+        if (FMT == 3) {
+            // K-quant models: a phase's matrix is Q4_K or Q6_K.  When v has another format than q and k (split_v) the q;k;v phase
+            // is two matrices one after the other: both read the same normed row and write q | k | v rows under the same tag, so
+            // nothing changes for the phases around them; the second one fetches and norms the row again (it is there already).
+            auto run = [&](const GemvJob& jb, const Mat& nx, bool ea) {
+                if (jb.wf == WF_Q4K) pd_gemv_phase<WF_Q4K, HD, FMT, ORD, PEN>(a, jb, nx, ea, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
+                else pd_gemv_phase<WF_Q6K, HD, FMT, ORD, PEN>(a, jb, nx, ea, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
+            };
+            if (ph == 0 && a.split_v) {
+                Mat vmat;
+                vmat.valid = true;
+                vmat.which = PD_V;
+                vmat.qs = job.qs + a.v_qs_off;
+                vmat.ws = reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(job.ws) + a.v_ws_off);
+                vmat.wf = a.wf[PD_V];
+                run(job, vmat, early);
+                if (sh_abort) return;
+                __syncthreads();          // the q;k rows are summed and stored before the second matrix's input and sums use the same LDS
+                GemvJob jv = job;
+                jv.which = PD_V;
+                jv.qs = vmat.qs;
+                jv.ws = vmat.ws;
+                jv.wf = vmat.wf;
+                jv.row_off = a.QKS + a.KV;
+                run(jv, next, true);
+            } else {
+                run(job, next, early);
+            }
+        } else if (FMT == 1 || (FMT == 2 && job.wf == WF_Q4)) {
+            pd_gemv_phase<WF_Q4, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
+        } else {
+            pd_gemv_phase<WF_Q8, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
+        }
         early = next.valid;
         if (sh_abort) return;
     }
@@ -1369,7 +1480,7 @@ struct PdState {
     PdArgs args{};
     std::vector<void*> owned;
     uint32_t grid = 0, lds = 0, hd = 0, tags_per_launch = 0, n_stamps = 0;
-    bool q4 = false, lmq4 = false, ordered = false, cooperative = true;
+    bool q4 = false, lmq4 = false, kquant = false, ordered = false, cooperative = true;
     size_t tagged_bytes = 0;
     void* tagged_base = nullptr;
     std::vector<unsigned long long> stamps_host;
@@ -1386,12 +1497,87 @@ struct PdState {
 
 namespace {
 
+// K-quant matrices as this kernel's weight units (layouts at WF_*), from the planes gemv_kquant.hip keeps.  One thread per
+// (row, 32-weight block).
+__global__ __launch_bounds__(256) void pd_repack_q4k_kernel(const uint8_t* __restrict__ qs, const uint8_t* __restrict__ meta, uint32_t K, uint64_t total,
+                                                          uint8_t* __restrict__ codes, uint32_t* __restrict__ words) {
+    const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;       // n * nblk + b
+    if (id >= total) return;
+    const uint32_t nblk = K / 32;
+    const uint64_t n = id / nblk;
+    const uint32_t b = (uint32_t)(id % nblk), sb = b >> 3, j = b & 7, c = j >> 1;
+    const uint8_t* mp = meta + (n * (K / 256) + sb) * 16;
+    const uint8_t* s12 = mp + 4;
+    uint32_t sc, mn;                                                       // get_scale_min_k4, emit.rs:3013-3021
+    if (j < 4) { sc = s12[j] & 63u; mn = s12[j + 4] & 63u; }
+    else {
+        sc = (s12[j + 4] & 0x0Fu) | ((s12[j - 4] >> 6) << 4);
+        mn = (s12[j + 4] >> 4) | ((s12[j] >> 6) << 4);
+    }
+    const uint32_t h16 = (b & 1u) ? (uint32_t)(mp[2] | (mp[3] << 8)) : (uint32_t)(mp[0] | (mp[1] << 8));     // odd: dmin, even: d
+    words[id] = h16 | (sc << 16) | (mn << 24);
+    // sub-block j = 2c + hi: weight i is the low (hi = 0) or high nibble of byte 32 c + i of the super-block
+    const uint8_t* src = qs + (n * (K / 256) + sb) * 128 + 32 * c;
+    const uint32_t sh = (j & 1) * 4;
+    uint8_t* dst = codes + id * 16;
+    for (uint32_t i = 0; i < 16; i++) dst[i] = (uint8_t)(((src[i] >> sh) & 15u) | (((src[i + 16] >> sh) & 15u) << 4));
+}
+
+__global__ __launch_bounds__(256) void pd_repack_q6k_kernel(const uint8_t* __restrict__ qs, const uint8_t* __restrict__ meta, uint32_t K, uint64_t total,
+                                                          uint8_t* __restrict__ codes) {
+    const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;       // n * nblk + b
+    if (id >= total) return;
+    const uint32_t nblk = K / 32;
+    const uint64_t n = id / nblk;
+    const uint32_t b = (uint32_t)(id % nblk), sb = b >> 3, jb = b & 7, h = jb >> 2, r = jb & 3;
+    const uint8_t* sp = qs + (n * (K / 256) + sb) * 192;
+    const uint8_t* mp = meta + (n * (K / 256) + sb) * 32;
+    // block 4h + r of the super-block: r = 0, 1 the low nibbles of ql[64h + 32r ..], r = 2, 3 the high nibbles of
+    // ql[64h + 32(r - 2) ..]; bit pair r of qh[32h ..]
+    const uint8_t* ql = sp + 64 * h + 32 * (r & 1);
+    const uint8_t* qh = sp + 128 + 32 * h;
+    const uint32_t nib_shift = (r >> 1) * 4, pair_shift = 2 * r;
+    for (uint32_t half = 0; half < 2; half++) {
+        uint32_t c[16];
+        for (uint32_t i = 0; i < 16; i++) {
+            const uint32_t e = 16 * half + i;
+            c[i] = ((ql[e] >> nib_shift) & 15u) | (((qh[e] >> pair_shift) & 3u) << 4);        // 0..63, the weight is this minus 32
+        }
+        uint8_t* dst = codes + (id * 2 + half) * 16;
+        for (uint32_t k = 0; k < 4; k++) {
+            dst[k] = (uint8_t)((c[k] & 15u) | ((c[4 + k] & 15u) << 4));
+            dst[4 + k] = (uint8_t)((c[8 + k] & 15u) | ((c[12 + k] & 15u) << 4));
+            dst[8 + k] = (uint8_t)((c[k] >> 4) | ((c[4 + k] >> 4) << 2) | ((c[8 + k] >> 4) << 4) | ((c[12 + k] >> 4) << 6));
+        }
+        dst[12] = mp[2 * jb + half];          // the int8 scale of this half
+        dst[13] = 0;
+        dst[14] = mp[16];                     // d (fp16)
+        dst[15] = mp[17];
+    }
+}
+
+// Bytes of the two planes of an [N][K] K-quant matrix in the kernel's layout.
+size_t pd_kq_code_bytes(uint32_t wdtype, uint64_t N, uint32_t K) { return wdtype == FORGE_HIP_Q4_K ? N * (K / 32) * 16 : N * (K / 32) * 32; }
+size_t pd_kq_word_bytes(uint32_t wdtype, uint64_t N, uint32_t K) { return wdtype == FORGE_HIP_Q4_K ? N * (K / 32) * 4 : 0; }
+
+void pd_repack_kquant(const QWeight& w, uint8_t* codes, uint8_t* words, hipStream_t s) {
+    const uint64_t total = (uint64_t)w.N * (w.K / 32);
+    const uint32_t grid = (uint32_t)((total + 255) / 256);
+    const uint8_t* meta = reinterpret_cast<const uint8_t*>(w.scales);
+    if (w.wdtype == FORGE_HIP_Q4_K) fh::launch(pd_repack_q4k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, codes, reinterpret_cast<uint32_t*>(words));
+    else fh::launch(pd_repack_q6k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, codes);
+}
+
+uint32_t wf_of(uint32_t wdtype) {
+    return wdtype == FORGE_HIP_Q8_0 ? WF_Q8 : wdtype == FORGE_HIP_Q4_0 ? WF_Q4 : wdtype == FORGE_HIP_Q4_K ? WF_Q4K : WF_Q6K;
+}
+
 // Tile plan of one matrix: rows per tile so that the tiles spread evenly over the grid and a tile's block
 // products fit `big_bytes` of LDS.  Returns false if they cannot.
 bool plan_gemv(const QWeight& w, uint32_t inter, uint32_t nseg, const Segment* seg, uint32_t tail_mod, uint32_t grid,
                uint32_t big_bytes, PdGemv* g) {
     g->qs = w.qs; g->ws = w.scales; g->K = w.K; g->N = w.N; g->nblk = w.K / 32;
-    const uint32_t epu = w.wdtype == FORGE_HIP_Q8_0 ? 1024 : 2048;
+    const uint32_t epu = (w.wdtype == FORGE_HIP_Q8_0 || w.wdtype == FORGE_HIP_Q6_K) ? 1024 : 2048;
     g->U = (w.K + epu - 1) / epu;
     g->umagic = g->U >= 2 ? (uint32_t)(0x100000000ull / g->U) + 1u : 0u;
     g->inter = inter;
@@ -1418,6 +1604,8 @@ bool plan_gemv(const QWeight& w, uint32_t inter, uint32_t nseg, const Segment* s
 
 template <int HD, bool ORD, bool PEN>
 const void* pd_kernel_ord(const PdState* st) {
+    // (K-quant models always run the variant with the optional extras: half as many kernels to build for a path that is opt-in)
+    if (st->kquant) return reinterpret_cast<const void*>(decode_step_kernel<HD, 3, ORD, true>);
     if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2, ORD, PEN>);
     return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 1, ORD, PEN>) : reinterpret_cast<const void*>(decode_step_kernel<HD, 0, ORD, PEN>);
 }
@@ -1481,6 +1669,16 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     st->hd = hd;
     st->q4 = c.wdtype == FORGE_HIP_Q4_0;
     st->lmq4 = c.lm_head_dtype == FORGE_HIP_Q4_0;
+    // a model of K-quant matrices: every projection and the lm_head Q4_K or Q6_K, q and k of one format, gate and up too
+    if (layers.empty()) return FORGE_HIP_OK;
+    st->kquant = layers[0].q != nullptr;
+    if (st->kquant) {
+        const PdLayerIn& in = layers[0];
+        const QWeight* all[7] = {in.q, in.k, in.v, in.o, in.gate, in.up, in.down};
+        for (const QWeight* w : all)
+            if (!w || !w->kquant()) return FORGE_HIP_OK;
+        if (!lm_head.kquant() || in.q->wdtype != in.k->wdtype || in.gate->wdtype != in.up->wdtype) return FORGE_HIP_OK;
+    }
     st->wall_khz = khz;
     // FORGE_HIP_PD_ORDERED=1: GEMV rows summed in the reference's block order, bit-identical to the kernel sequence
     { const char* e = getenv("FORGE_HIP_PD_ORDERED"); st->ordered = exact || (e && e[0] == '1'); }
@@ -1499,7 +1697,74 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     st->lds = a.off_big + big;
 
     if (layers.empty() || layers.size() > PD_MAX_LAYERS * PD_MAX_SEGMENTS) return FORGE_HIP_OK;
-    {
+    QWeight lm_res = lm_head;                     // K-quant models: the lm_head in the kernel's layout
+    if (st->kquant) {
+        const PdLayerIn& in0 = layers[0];
+        // descriptors of the matrices as the kernel sees them: q;k (with v behind it when v shares their format), o, gate;up, down
+        const bool split_v = in0.v->wdtype != in0.q->wdtype;
+        auto desc = [](uint32_t wdtype, uint32_t K, uint32_t N) { QWeight d; d.wdtype = wdtype; d.K = K; d.N = N; return d; };
+        const QWeight dqk = desc(in0.q->wdtype, H, split_v ? QKS + KV : QKS + 2 * KV), dv = desc(in0.v->wdtype, H, KV),
+                      dgu = desc(in0.gate->wdtype, H, 2 * I);
+        if (!plan_gemv(dqk, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_QKV]) || !plan_gemv(*in0.o, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_O]) ||
+            !plan_gemv(dgu, I, 0, nullptr, 4, st->grid, big, &a.shape[PD_GU]) || !plan_gemv(*in0.down, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_DOWN]) ||
+            (split_v && !plan_gemv(dv, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_V])) ||
+            !plan_gemv(lm_head, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_LM]))
+            return FORGE_HIP_OK;
+        for (int k = 0; k < 6; k++) { a.shape[k].qs = nullptr; a.shape[k].ws = nullptr; }
+        a.wf[PD_QKV] = wf_of(dqk.wdtype); a.wf[PD_O] = wf_of(in0.o->wdtype); a.wf[PD_GU] = wf_of(dgu.wdtype);
+        a.wf[PD_DOWN] = wf_of(in0.down->wdtype); a.wf[PD_LM] = wf_of(lm_head.wdtype); a.wf[PD_V] = wf_of(dv.wdtype);
+        a.split_v = split_v ? 1u : 0u;
+        // the layout per layer: codes [q | k | v], words [q | k | v] (a Q6_K matrix has no words), then o, gate;up, down each
+        const size_t cq = pd_kq_code_bytes(in0.q->wdtype, QKS, H), ck = pd_kq_code_bytes(in0.k->wdtype, KV, H), cv = pd_kq_code_bytes(in0.v->wdtype, KV, H);
+        const size_t wq = pd_kq_word_bytes(in0.q->wdtype, QKS, H), wk = pd_kq_word_bytes(in0.k->wdtype, KV, H), wv = pd_kq_word_bytes(in0.v->wdtype, KV, H);
+        a.v_qs_off = (uint32_t)(cq + ck);
+        a.v_ws_off = (uint32_t)(wq + wk);
+        if (cq + ck + cv > 0xFFFFFFFFull) return FORGE_HIP_OK;
+        for (size_t l = 0; l < layers.size(); l++) {
+            const PdLayerIn& in = layers[l];
+            const QWeight* all[7] = {in.q, in.k, in.v, in.o, in.gate, in.up, in.down};
+            for (int i = 0; i < 7; i++)
+                if (!all[i] || all[i]->wdtype != (i == 0 || i == 1 ? in0.q->wdtype : i == 2 ? in0.v->wdtype : i == 3 ? in0.o->wdtype : i < 6 ? in0.gate->wdtype : in0.down->wdtype))
+                    return FORGE_HIP_OK;
+            st->all_layers.emplace_back();
+            PdLayer& L = st->all_layers.back();
+            auto plane = [&](size_t n) -> uint8_t* { return n ? dev_alloc<uint8_t>(n, st->owned) : nullptr; };
+            uint8_t* c_qkv = plane(cq + ck + cv);
+            uint8_t* w_qkv = plane(wq + wk + wv);
+            const size_t co = pd_kq_code_bytes(in.o->wdtype, H, QKS), wo = pd_kq_word_bytes(in.o->wdtype, H, QKS);
+            const size_t cg = pd_kq_code_bytes(in.gate->wdtype, I, H), wg = pd_kq_word_bytes(in.gate->wdtype, I, H);
+            const size_t cd = pd_kq_code_bytes(in.down->wdtype, H, I), wd = pd_kq_word_bytes(in.down->wdtype, H, I);
+            uint8_t *c_o = plane(co), *w_o = plane(wo), *c_gu = plane(2 * cg), *w_gu = plane(2 * wg), *c_d = plane(cd), *w_d = plane(wd);
+            if (!c_qkv || !c_o || !c_gu || !c_d || (wq + wk + wv && !w_qkv) || (wo && !w_o) || (wg && !w_gu) || (wd && !w_d))
+                return fail(FORGE_HIP_ERR_HIP, "persistent decode: out of device memory for the K-quant weight units");
+            pd_repack_kquant(*in.q, c_qkv, w_qkv, nullptr);
+            pd_repack_kquant(*in.k, c_qkv + cq, w_qkv ? w_qkv + wq : nullptr, nullptr);
+            pd_repack_kquant(*in.v, c_qkv + cq + ck, w_qkv ? w_qkv + wq + wk : nullptr, nullptr);
+            pd_repack_kquant(*in.o, c_o, w_o, nullptr);
+            pd_repack_kquant(*in.gate, c_gu, w_gu, nullptr);
+            pd_repack_kquant(*in.up, c_gu + cg, w_gu ? w_gu + wg : nullptr, nullptr);
+            pd_repack_kquant(*in.down, c_d, w_d, nullptr);
+            L.qs[0] = c_qkv; L.ws[0] = reinterpret_cast<const uint16_t*>(w_qkv);
+            L.qs[1] = c_o; L.ws[1] = reinterpret_cast<const uint16_t*>(w_o);
+            L.qs[2] = c_gu; L.ws[2] = reinterpret_cast<const uint16_t*>(w_gu);
+            L.qs[3] = c_d; L.ws[3] = reinterpret_cast<const uint16_t*>(w_d);
+            if (in.ffn_norm != in.attn_norm + H) return FORGE_HIP_OK;          // the kernel finds the second norm H floats behind the first
+            L.attn_norm = in.attn_norm; L.kc = in.kc; L.vc = in.vc;
+        }
+        {
+            const size_t cl = pd_kq_code_bytes(lm_head.wdtype, c.vocab, H), wl = pd_kq_word_bytes(lm_head.wdtype, c.vocab, H);
+            uint8_t* c_l = dev_alloc<uint8_t>(cl, st->owned);
+            uint8_t* w_l = wl ? dev_alloc<uint8_t>(wl, st->owned) : nullptr;
+            if (!c_l || (wl && !w_l)) return fail(FORGE_HIP_ERR_HIP, "persistent decode: out of device memory for the K-quant weight units");
+            pd_repack_kquant(lm_head, c_l, w_l, nullptr);
+            lm_res.qs = c_l;
+            lm_res.scales = reinterpret_cast<uint16_t*>(w_l);
+            a.shape[PD_LM].qs = c_l;
+            a.shape[PD_LM].ws = reinterpret_cast<const uint16_t*>(w_l);
+        }
+        FH_HIP(hipDeviceSynchronize());
+        FH_HIP(hipGetLastError());
+    } else {
         const PdLayerIn& in = layers[0];
         const uint32_t wt = c.wdtype;
         Segment sq[3] = {make_segment(wt, H, 0, QKS, false), make_segment(wt, H, QKS, KV, false), make_segment(wt, H, QKS + KV, KV, false)};
@@ -1512,18 +1777,23 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
             return FORGE_HIP_OK;
         for (int k = 0; k < 4; k++) { a.shape[k].qs = nullptr; a.shape[k].ws = nullptr; }
     }
-    for (size_t l = 0; l < layers.size(); l++) {
+    for (size_t l = 0; l < layers.size() && !st->kquant; l++) {
         const PdLayerIn& in = layers[l];
         st->all_layers.emplace_back();
         PdLayer& L = st->all_layers.back();
         const QWeight* w[4] = {in.qkv, in.o, in.gate_up, in.down};
         for (int k = 0; k < 4; k++) { L.qs[k] = w[k]->qs; L.ws[k] = w[k]->scales; }
-        L.attn_norm = in.attn_norm; L.ffn_norm = in.ffn_norm; L.kc = in.kc; L.vc = in.vc;
+        if (in.ffn_norm != in.attn_norm + H) return FORGE_HIP_OK;          // the kernel finds the second norm H floats behind the first
+            L.attn_norm = in.attn_norm; L.kc = in.kc; L.vc = in.vc;
     }
-    {
+    if (!st->kquant) {
         Segment sl[1] = {make_segment(c.lm_head_dtype, H, 0, c.vocab, true)};
         if (!plan_gemv(lm_head, 0, 1, sl, 4, st->grid, big, &a.shape[PD_LM])) return FORGE_HIP_OK;
+        a.wf[PD_QKV] = a.wf[PD_O] = a.wf[PD_GU] = a.wf[PD_DOWN] = a.wf[PD_V] = st->q4 ? WF_Q4 : WF_Q8;
+        a.wf[PD_LM] = st->lmq4 ? WF_Q4 : WF_Q8;
+        a.split_v = 0; a.v_qs_off = 0; a.v_ws_off = 0;
     }
+    (void)lm_res;
     // cooperative residency: one workgroup per CU must fit
     {
         int per_cu = 0;
@@ -1569,7 +1839,6 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     // FORGE_HIP_PD_SPIN_LIMIT: how often a wait re-reads before the workgroup gives up (a test sets it to 1 to walk the
     // give-up path: every wait in the kernel is bounded by it, so the kernel still ends normally)
     { const char* e = getenv("FORGE_HIP_PD_SPIN_LIMIT"); if (e && atoi(e) > 0) a.spin_limit = (uint32_t)atoi(e); }
-    a.q4 = st->q4; a.lm_q4 = st->lmq4;
     // The watcher (one thread polls one element of a buffer, the other pollers wait for its word in LDS before they re-read
     // what they missed) pays on narrow models, where a phase is nothing but its hand-over (hidden 576: +2 %); from a hidden
     // size of 1024 up the pollers re-read on their own (1B +1.0 %, 3B +1.7 %, 8B +0.9 % over the watcher).

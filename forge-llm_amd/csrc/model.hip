@@ -886,7 +886,29 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
         }
     }
     const char* penv = getenv("FORGE_HIP_PERSIST");
-    if (!pd && !(penv && penv[0] == '0')) {       // the resident kernel carries Q8_0 / Q4_0 weight units only
+    const char* kenv = getenv("FORGE_HIP_PD_KQUANT");
+    if (pd && !(penv && penv[0] == '0') && kenv && kenv[0] == '1') {
+        // a model whose matrices are all Q4_K / Q6_K (q and k of one format, gate and up too) can run its decode step as the
+        // resident kernel with K-quant weight units: bit-identical to the kernel sequence in the ordered variant, but not
+        // faster (Q4_K_M-recipe 1B shape: 920 against 868 us per token: the K-quant block decoders are instruction-bound on
+        // the kernel's six streaming waves, and a v matrix of another format than q and k costs a phase of its own), so the
+        // sequence stays the default and FORGE_HIP_PD_KQUANT=1 asks for the kernel.  pd_create leaves m->pd null for any
+        // other mix.
+        bool all_k = is_kquant(cfg->lm_head_dtype);
+        for (int i = 0; i < 7; i++) all_k = all_k && is_kquant(pd[i]);
+        if (all_k && pd[0] == pd[1] && pd[4] == pd[5]) {
+            std::vector<PdLayerIn> pl(cfg->layers);
+            for (uint32_t l = 0; l < cfg->layers; l++) {
+                Layer& L = m->layers[l];
+                pl[l] = PdLayerIn{nullptr, &L.o, nullptr, &L.down, L.attn_norm, L.ffn_norm, m->kc(l), m->vc(l), &L.q, &L.k, &L.v, &L.gate, &L.up};
+            }
+            rc = pd_create(*cfg, pl, m->lm_head, m->embed.as<float>(), m->final_norm.as<float>(), m->cos_t.as<float>(),
+                           m->sin_t.as<float>(), m->logits.as<float>(), m->state.as<uint32_t>(), m->counts.as<uint32_t>(),
+                           has_bias ? m->biases.as<float>() : nullptr, &m->pd);
+            if (rc) return rc;
+        }
+    }
+    if (!pd && !(penv && penv[0] == '0')) {       // uniform Q8_0 / Q4_0 models
         std::vector<PdLayerIn> pl(cfg->layers);
         for (uint32_t l = 0; l < cfg->layers; l++) {
             Layer& L = m->layers[l];

@@ -280,6 +280,48 @@ def test_mixed_model_grouped_launches_keep_the_bits(fh, torch_gpu, monkeypatch):
         plain.close(); fused.close()
 
 
+@pytest.mark.parametrize("mix,extra", [("q4_k_m", {}), ("q6_k", {}), ("q4_k_m", dict(flags=QKV_BIAS)), ("q4_k_m", dict(sliding_window=24)),
+                                       ("q4_k_m", dict(hidden=512, inter=1024, heads=4, kv_heads=4, head_dim=128))])
+def test_kquant_weight_units_in_the_resident_kernel(fh, torch_gpu, monkeypatch, mix, extra):
+    """FORGE_HIP_PD_KQUANT=1: the decode step of a model whose matrices are all Q4_K / Q6_K as ONE resident kernel, the matrices
+    re-laid out as its weight units (Q4_K: Q4_0-ordered nibbles + a word of d | dmin, scale and minimum per sub-block; Q6_K:
+    16 bytes per 16 weights with scale and d inside); a v matrix of another format than q and k is a phase of its own.  With
+    the ordered row sums (FORGE_HIP_PD_ORDERED=1) every logit equals the kernel sequence's bit for bit, step after step, and
+    the cache rows too; the default sums differ by the order of additions (and by the int8 activation codes that this moves)."""
+    pd, lm = MIXES[mix]
+    flags = extra.get("flags", 0)
+    shape = {k: v for k, v in extra.items() if k not in ("flags", "sliding_window")}
+    cfg = tiny(fh, lm, flags, **shape)
+    cfg["sliding_window"] = extra.get("sliding_window", 0)
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=29, std=0.05)
+    toks = fh.synth.uniform_ids(31, 45, cfg["vocab"])
+    seq = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    assert seq.decode_launches > 1
+    monkeypatch.setenv("FORGE_HIP_PD_KQUANT", "1")
+    fast = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    monkeypatch.setenv("FORGE_HIP_PD_ORDERED", "1")
+    ordered = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    monkeypatch.delenv("FORGE_HIP_PD_ORDERED")
+    monkeypatch.delenv("FORGE_HIP_PD_KQUANT")
+    assert fast.decode_launches == ordered.decode_launches == 1
+    a = seq.forward_prefill(toks)
+    assert np.array_equal(a, ordered.forward_prefill(toks)) and np.array_equal(a, fast.forward_prefill(toks))
+    tok = int(np.argmax(a))
+    for _ in range(30):                                     # past the window where there is one
+        x, y, z = seq.forward(tok), ordered.forward(tok), fast.forward(tok)
+        same_bits(y, x)
+        # a last-bit difference in a norm can move an int8 activation code by one: quantisation noise, not rounding noise
+        assert np.corrcoef(z, x)[0, 1] > 0.999 and np.max(np.abs(z - x)) < 0.05 * max(1.0, float(np.std(x)))
+        tok = int(np.argmax(x))
+    for layer in range(cfg["layers"]):
+        for which in (0, 1):
+            assert np.array_equal(ordered.read_kv(layer, which), seq.read_kv(layer, which))
+    # greedy decoding on the device, and a reset
+    seq.reset(); ordered.reset()
+    assert ordered.generate_greedy(toks[:9], 12) == seq.generate_greedy(toks[:9], 12)
+    seq.close(); ordered.close(); fast.close()
+
+
 def test_uniform_formats_through_the_mixed_entry_point_are_the_plain_model(fh, torch_gpu):
     cfg = tiny(fh, Q8, 0)
     cfg["wdtype"] = Q4
