@@ -18,8 +18,9 @@ generated kernels): its prefill and decode throughput, and the fast mode's dista
 that differs, largest logit difference before that).
 
 kquant_model: the same shape with a storage format per projection (llama.cpp's Q4_K_M recipe, random super-blocks):
-prompt and decode throughput in fast mode (prompt on the MFMA GEMM through re-expressed matrices, decode as a kernel
-sequence) and in the order-faithful mode (prompt through the multi-row K-quant GEMV).
+prompt and decode throughput in fast mode (prompt on the MFMA GEMM through re-expressed matrices, decode as one resident
+kernel with K-quant weight units, the kernel sequence beside it) and in the order-faithful mode (prompt through the
+multi-row K-quant GEMV).
 
 cpu_baseline: the CPU restatement of the reference's generated kernels (oracle/) on this host's cores, on the same
 model and prompt: in the aarch64 arithmetic (int8 activation blocks) the whole prompt as a batched prefill and
@@ -230,8 +231,8 @@ def exact_mode_figures(fh, cfg, blob, prompt, warmup, steps, fast_tokens, fast_l
 
 def kquant_model_figures(fh, cfg, prompt, warmup, steps, seed):
     """The same shape with llama.cpp's Q4_K_M recipe (Q4_K q/k/o/gate/up, Q6_K v/down/lm_head; random super-blocks): the model
-    with a storage format per projection.  Fast mode: prompt on the int8 MFMA GEMM through the matrices' twins, decode as a
-    kernel sequence; order-faithful mode: prompt through the multi-row K-quant GEMV (bit for bit the reference's
+    with a storage format per projection.  Fast mode: prompt on the int8 MFMA GEMM through the matrices' twins, decode as one
+    resident kernel (the kernel sequence timed beside it); order-faithful mode: prompt through the multi-row K-quant GEMV (bit for bit the reference's
     token-by-token walk)."""
     kcfg = dict(cfg)
     kcfg["lm_head_dtype"] = 14
@@ -251,6 +252,16 @@ def kquant_model_figures(fh, cfg, prompt, warmup, steps, seed):
            "decode_tok_per_s": steps / t_decode, "decode_launches_per_token": m.decode_launches,
            "create_s_incl_twins": round(t_create, 2)}
     m.close()
+    import os
+    os.environ["FORGE_HIP_PD_KQUANT"] = "0"                  # the same step as a sequence of kernels (grouped K-quant GEMVs)
+    try:
+        m = fh.HipModel(kcfg, blob, proj_dtypes=pd)
+        tok = fh.ops.argmax_host(m.forward_prefill(prompt))
+        t_seq, tok = timed_decode(m, tok, warmup, steps)
+        out["kernel_sequence"] = {"decode_tok_per_s": steps / t_seq, "decode_launches_per_token": m.decode_launches}
+        m.close()
+    finally:
+        del os.environ["FORGE_HIP_PD_KQUANT"]
     ecfg = dict(kcfg, flags=fh.FLAG_EXACT)
     e = fh.HipModel(ecfg, blob, proj_dtypes=pd)
     t0 = time.perf_counter()

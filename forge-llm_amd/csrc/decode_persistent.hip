@@ -107,8 +107,8 @@ enum { PD_QKV = 0, PD_O = 1, PD_GU = 2, PD_DOWN = 3, PD_LM = 4, PD_V = 5 };
 //   Q4_K  codes: 16 bytes per 32-weight sub-block in Q4_0's byte order (byte i = weight i | weight i + 16 << 4), values 0..15;
 //         one word per sub-block b: fp16 bits of d (b even) or dmin (b odd) | 6-bit scale << 16 | 6-bit minimum << 24 -- the two
 //         sub-blocks of a pair belong to one super-block, so a lane gets the other half from its neighbour
-//   Q6_K  16 bytes per 16-weight half block: byte i of the first eight = code i % 4 + 8 (i / 4)'s low nibble | code + 4's << 4,
-//         bytes 8..11 the 2-bit high parts (byte i: codes i, i + 4, i + 8, i + 12), byte 12 the int8 scale, bytes 14..15 d (fp16)
+//   Q6_K  codes: the 32 weights of a block as int8 (-32..31) in order (8 bits for 6: the streaming waves are bound by the
+//         instructions per weight, not by the bytes); one word per block: the int8 scales of its two halves | fp16 bits of d << 16
 enum { WF_Q8 = 0, WF_Q4 = 1, WF_Q4K = 2, WF_Q6K = 3 };
 __host__ __device__ constexpr bool wf_lane_per_block(int wf) { return wf == WF_Q4 || wf == WF_Q4K; }
 
@@ -146,7 +146,7 @@ struct PdArgs {
     // (shape[PD_V], another format than q and k: llama.cpp's K-quant recipes), its planes `v_qs_off` / `v_ws_off` bytes
     // behind the layer's q;k planes; shape[PD_QKV] then holds the q and k rows only.
     uint32_t wf[6];
-    uint32_t split_v, v_qs_off, v_ws_off;
+    uint32_t split_v, v_qs_off, v_ws_off, v_wg0;
     uint32_t* counts;                          // u32 [vocab]: times each token id has been fed (this step's token is added here)
     const float* qkv_bias;                     // optional [layers][QKS + 2 KV]: added to q, k, v before the rotation (Qwen2)
     float penalty;                             // > 1: the argmax is taken over the penalised logits
@@ -470,8 +470,7 @@ __device__ __forceinline__ void pd_load_round(const GemvJob& job, const Shape& h
         const uint32_t bc = b < nblk ? b : nblk - 1;
         const uint32_t bi = pd_row(t, lrc) * nblk + bc;             // block index in the matrix (fits 32 bits: N K / 32)
         W.v[d] = ldg(reinterpret_cast<const int4*>(job.qs + (size_t)bi * BPB + (Q4 ? 0u : (lane & 1u) * 16u)));
-        if (WF == WF_Q4K) W.s[d] = ldg(reinterpret_cast<const uint32_t*>(job.ws) + bi);
-        else if (WF == WF_Q6K) W.s[d] = 0u;                       // scale and d travel inside the 16 bytes
+        if (WF == WF_Q4K || WF == WF_Q6K) W.s[d] = ldg(reinterpret_cast<const uint32_t*>(job.ws) + bi);
         else W.s[d] = ldg(job.ws + bi);
         j += 1;
         if (j == U) { j = 0; lr += PD_STREAM_WAVES; }
@@ -484,6 +483,7 @@ struct Mat {
     const uint8_t* qs;
     const uint16_t* ws;
     uint32_t wf;
+    uint32_t wg_off;           // the matrix's tiles are spread over workgroups wg_off .. (a phase of two matrices side by side)
     bool valid;
 };
 template <int FMT>
@@ -506,7 +506,8 @@ __device__ __forceinline__ void pd_load_first(const PdArgs& a, const Mat& m, uin
 //             them when the row's last unit is done: rowsum[row].  Same terms, another order of addition.
 template <int WF, bool ORDERED>
 __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& t, uint32_t round, uint32_t sw, uint32_t lane, const WReg& W,
-                                                 const uint32_t* aq_lds, const float* as_lds, float* prod, uint32_t pstride, float& acc) {
+                                                 const uint32_t* aq_lds, const float* as_lds, const float* asum_w, float* prod, uint32_t pstride,
+                                                 float& acc) {
     constexpr bool Q4 = wf_lane_per_block(WF);
     constexpr uint32_t BPU = Q4 ? 64 : 32;
     const uint32_t U = h.U, nblk = h.nblk;
@@ -530,8 +531,6 @@ __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& 
                     const int m = 0x0F0F0F0F;
                     const int4 lo = make_int4(w.x & m, w.y & m, w.z & m, w.w & m);
                     const int4 hi = make_int4((w.x >> 4) & m, (w.y >> 4) & m, (w.z >> 4) & m, (w.w >> 4) & m);
-                    const int4 ones = make_int4(0x01010101, 0x01010101, 0x01010101, 0x01010101);
-                    const int asum = dot16(ones, a1, dot16(ones, a0, 0));
                     const int dot = dot16(hi, a1, dot16(lo, a0, 0));
                     const uint32_t sw_ = W.s[d];
                     const uint32_t other = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)sw_, 0xB1, 0xF, 0xF, false);   // quad_perm [1,0,3,2]
@@ -539,21 +538,13 @@ __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& 
                     const float dd = f16_bits_to_f32((uint16_t)((even ? sw_ : other) & 0xFFFFu));
                     const float dmin = f16_bits_to_f32((uint16_t)((even ? other : sw_) & 0xFFFFu));
                     const float d_w = dd * (float)((sw_ >> 16) & 0xFFu), m_w = dmin * (float)(sw_ >> 24);
-                    term = as_lds[bs] * (d_w * (float)dot - m_w * (float)asum);
+                    term = as_lds[bs] * (d_w * (float)dot - m_w * asum_w[bs]);      // the block's sum of codes: left there by this lane
                     mine = in;
                 } else {
                     const int4 a = *reinterpret_cast<const int4*>(aq_lds + bs * 8 + (lane & 1u) * 4);
-                    const int4 w = W.v[d];
-                    const uint32_t m4 = 0x0F0F0F0Fu, m2 = 0x03030303u;
-                    const uint32_t wx = (uint32_t)w.x, wy = (uint32_t)w.y, wz = (uint32_t)w.z, ww = (uint32_t)w.w;
-                    auto minus32 = [](uint32_t x) { return (int)(((x | 0x80808080u) - 0x20202020u) ^ 0x80808080u); };   // bytes 0..63 -> -32..31
-                    int4 q;
-                    q.x = minus32((wx & m4) | ((wz & m2) << 4));
-                    q.y = minus32(((wx >> 4) & m4) | (((wz >> 2) & m2) << 4));
-                    q.z = minus32((wy & m4) | (((wz >> 4) & m2) << 4));
-                    q.w = minus32(((wy >> 4) & m4) | (((wz >> 6) & m2) << 4));
-                    const int dh = in ? dot16(q, a, 0) : 0;
-                    const float th = (float)(int)(int8_t)(ww & 0xFFu) * (float)dh;
+                    const int dh = in ? dot16(W.v[d], a, 0) : 0;      // this lane's 16 weights are one scale's
+                    const uint32_t ww = W.s[d];
+                    const float th = (float)((int)(ww << (24u - (lane & 1u) * 8u)) >> 24) * (float)dh;      // the int8 scale of this lane's half
                     const float u = th + __builtin_amdgcn_update_dpp(0.f, th, 0xB1, 0xF, 0xF, false);       // lo + hi (even lane)
                     term = (f16_bits_to_f32((uint16_t)(ww >> 16)) * as_lds[bs]) * u;
                     mine = in && !(lane & 1u);
@@ -1133,7 +1124,11 @@ __device__ __forceinline__ ArgPair arg_wg(ArgPair a, float* misc, const PdCtx& c
 //   inputs    the streamers issue the first weight loads of their rows at once; the poller wave fetches the activation
 //             vector (it never has weights in flight, so nothing delays what it polls)
 //   tiles     compute a round from registers, issue the next round (or the next tile's first), sum, finish the rows
-template <int WF, int HD, int FMT, bool ORDERED, bool PEN>
+// One instance per kernel: the prologues and epilogues are most of the code and do not depend on the weight format, so a
+// kernel that carries two formats chooses between them (a scalar branch on job.wf) only where the streamers load and
+// multiply.  The step runs every phase's code once per layer: what does not fit the instruction cache is fetched again
+// each time.
+template <int HD, int FMT, bool ORDERED, bool PEN>
 __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& job, const Mat& next, bool early, WReg& W, WReg& W1, const float* emb,
                                               uint32_t pos, size_t crow, uint32_t* aq_lds, float* as_lds, float* misc, float* big, ArgPair& best,
                                               const PdCtx& cx) {
@@ -1141,9 +1136,16 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     const Shape h = pd_shape(g);
     const bool streamer = cx.wave >= (uint32_t)PD_POLL_WAVES;
     const uint32_t sw = cx.wave - PD_POLL_WAVES;
+    constexpr int WFA = FMT == 0 ? WF_Q8 : FMT == 1 ? WF_Q4 : FMT == 2 ? WF_Q8 : WF_Q4K;      // the format(s) this kernel carries
+    constexpr int WFB = FMT == 2 ? WF_Q4 : FMT == 3 ? WF_Q6K : WFA;
+    const bool second = WFB != WFA && job.wf == (uint32_t)WFB;
+    auto load_round = [&](const TilePos& tt, uint32_t r, WReg& w) {
+        if (second) pd_load_round<WFB>(job, h, tt, r, sw, cx.lane, w);
+        else pd_load_round<WFA>(job, h, tt, r, sw, cx.lane, w);
+    };
     if (cx.wg >= h.ntiles) {
         // nothing to do here; the streamers still start on the matrix that follows
-        if (streamer && next.valid) pd_load_first<FMT>(a, next, cx.wg, sw, cx.lane, W);
+        if (streamer && next.valid) pd_load_first<FMT>(a, next, cx.wg - next.wg_off, sw, cx.lane, W);
         return;
     }
     const uint32_t pstride = h.nblk + 1;                    // +1: conflict-free column reads
@@ -1158,7 +1160,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     float4 nw = make_float4(0.f, 0.f, 0.f, 0.f);
     if (job.pro == PRO_NORM && cx.tid * 4 < K) nw = ldg(reinterpret_cast<const float4*>(job.norm_w + cx.tid * 4));
     if (streamer) {
-        if (!early) pd_load_round<WF>(job, h, t, 0, sw, cx.lane, W);      // otherwise the previous phase's tail issued them
+        if (!early) load_round(t, 0, W);                                  // otherwise the previous phase's tail issued them
     } else {
         float ssq = 0.f;
         if (job.pro == PRO_AQ) pd_load_aq(job.tin, job.tin_tag, K, aq_lds, as_lds, misc, a.use_hint != 0, cx);
@@ -1177,6 +1179,23 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     if (*cx.sh_abort) return;
     // the norm reads the row; the products use the area from its start afterwards
     if (job.pro == PRO_NORM) pd_norm_quant<ORDERED>(xs, job.norm_w, nw, a.eps, K, aq_lds, as_lds, misc, cx);
+    // Q4_K: the sum of a block's activation codes (the minimum's factor) is the same for every row; a lane only ever multiplies
+    // blocks lane, lane + 64, ..., so it leaves their sums in its wave's own strip of LDS once per phase (no barrier: lanes read
+    // what they wrote themselves)
+    const float* asum_w = nullptr;
+    if (FMT == 3) {
+        const uint32_t strip = (a.off_misc - a.off_act_s) / (4u * (PD_STREAM_WAVES + 1));     // floats per strip; strip 0 holds the scales
+        float* mine_w = as_lds + ((streamer ? sw : 0u) + 1) * strip;
+        asum_w = mine_w;
+        if (streamer && !second) {
+            const int4 ones = make_int4(0x01010101, 0x01010101, 0x01010101, 0x01010101);
+            for (uint32_t b = cx.lane; b < h.nblk; b += 64) {
+                const int4 a0 = *reinterpret_cast<const int4*>(aq_lds + b * 8);
+                const int4 a1 = *reinterpret_cast<const int4*>(aq_lds + b * 8 + 4);
+                mine_w[b] = (float)dot16(ones, a1, dot16(ones, a0, 0));
+            }
+        }
+    }
 
     // ---- tiles
     float acc = 0.f;
@@ -1208,11 +1227,13 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
             // always in W
 #pragma nounroll
             for (uint32_t r = 0; r < rounds; r += 2) {
-                if (r + 1 < rounds) pd_load_round<WF>(job, h, t, r + 1, sw, cx.lane, W1);
-                pd_compute_round<WF, ORDERED>(h, t, r, sw, cx.lane, W, aq_lds, as_lds, big, pstride, acc);
+                if (r + 1 < rounds) load_round(t, r + 1, W1);
+                if (second) pd_compute_round<WFB, ORDERED>(h, t, r, sw, cx.lane, W, aq_lds, as_lds, asum_w, big, pstride, acc);
+                else pd_compute_round<WFA, ORDERED>(h, t, r, sw, cx.lane, W, aq_lds, as_lds, asum_w, big, pstride, acc);
                 if (r + 1 < rounds) {
-                    if (r + 2 < rounds) pd_load_round<WF>(job, h, t, r + 2, sw, cx.lane, W);
-                    pd_compute_round<WF, ORDERED>(h, t, r + 1, sw, cx.lane, W1, aq_lds, as_lds, big, pstride, acc);
+                    if (r + 2 < rounds) load_round(t, r + 2, W);
+                    if (second) pd_compute_round<WFB, ORDERED>(h, t, r + 1, sw, cx.lane, W1, aq_lds, as_lds, asum_w, big, pstride, acc);
+                    else pd_compute_round<WFA, ORDERED>(h, t, r + 1, sw, cx.lane, W1, aq_lds, as_lds, asum_w, big, pstride, acc);
                 }
             }
         }
@@ -1222,8 +1243,8 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
         // long as the data takes to arrive (the memory pipeline holds only so many misses), so it must not sit between
         // the products and the sums.
         if (streamer) {
-            if (more) pd_load_round<WF>(job, h, tn, 0, sw, cx.lane, W);
-            else if (next.valid) pd_load_first<FMT>(a, next, cx.wg, sw, cx.lane, W);
+            if (more) load_round(tn, 0, W);
+            else if (next.valid) pd_load_first<FMT>(a, next, cx.wg - next.wg_off, sw, cx.lane, W);
         }
         if (cx.tid < ((t.rows + 63u) & ~63u)) {
             float v = 0.f;
@@ -1367,6 +1388,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
             static const int slot[5] = {0, 3, 4, 5, 6};
             a.stamps[6 * lg + slot[ph]] = wall_clock64();
         }
+        const bool vside = FMT == 3 && a.split_v && cx.wg >= a.v_wg0;
         GemvJob job;
         job.which = ph;
         job.qs = is_lm ? a.shape[PD_LM].qs : a.layers[l].qs[ph];
@@ -1384,6 +1406,14 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
             next.qs = n_lm ? a.shape[PD_LM].qs : a.layers[next.valid ? nl : 0].qs[nph & 3u];
             next.ws = n_lm ? a.shape[PD_LM].ws : a.layers[next.valid ? nl : 0].ws[nph & 3u];
             next.wf = a.wf[n_lm ? (uint32_t)PD_LM : nph];
+            next.wg_off = 0;
+            if (FMT == 3 && a.split_v && nph == 0 && !n_lm && vside) {      // this workgroup's share of the q;k;v phase is the v matrix
+                next.which = PD_V;
+                next.qs += a.v_qs_off;
+                next.ws = reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(next.ws) + a.v_ws_off);
+                next.wf = a.wf[PD_V];
+                next.wg_off = a.v_wg0;
+            }
         }
         job.pro = (ph == 1 || ph == 3) ? PRO_AQ : PRO_NORM;
         job.epi = ph == 0 ? EPI_ROPE : ph == 2 ? EPI_SILU : ph == 4 ? EPI_LOGITS : EPI_ADD;
@@ -1396,39 +1426,24 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         job.kc = a.layers[l].kc;
         job.bias = (PEN && a.qkv_bias && ph == 0) ? a.qkv_bias + (size_t)lg * (a.QKS + 2 * a.KV) : nullptr;
         job.vc = a.layers[l].vc;
-        if (FMT == 3) {
-            // K-quant models: a phase's matrix is Q4_K or Q6_K.  When v has another format than q and k (split_v) the q;k;v phase
-            // is two matrices one after the other: both read the same normed row and write q | k | v rows under the same tag, so
-            // nothing changes for the phases around them; the second one fetches and norms the row again (it is there already).
-            auto run = [&](const GemvJob& jb, const Mat& nx, bool ea) {
-                if (jb.wf == WF_Q4K) pd_gemv_phase<WF_Q4K, HD, FMT, ORD, PEN>(a, jb, nx, ea, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
-                else pd_gemv_phase<WF_Q6K, HD, FMT, ORD, PEN>(a, jb, nx, ea, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
-            };
-            if (ph == 0 && a.split_v) {
-                Mat vmat;
-                vmat.valid = true;
-                vmat.which = PD_V;
-                vmat.qs = job.qs + a.v_qs_off;
-                vmat.ws = reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(job.ws) + a.v_ws_off);
-                vmat.wf = a.wf[PD_V];
-                run(job, vmat, early);
-                if (sh_abort) return;
-                __syncthreads();          // the q;k rows are summed and stored before the second matrix's input and sums use the same LDS
-                GemvJob jv = job;
-                jv.which = PD_V;
-                jv.qs = vmat.qs;
-                jv.ws = vmat.ws;
-                jv.wf = vmat.wf;
-                jv.row_off = a.QKS + a.KV;
-                run(jv, next, true);
+        // v in another format than q and k (K-quant recipes): two matrices side by side in the q;k;v phase.  The first v_wg0
+        // workgroups take the q;k rows, the others the v rows, each side tiling its matrix over its own share of the grid;
+        // both read the same normed row and write q | k | v rows under the same tag, so nothing changes for the phases
+        // around them.  (One call for every case: the phase's code is in the kernel once.)
+        PdCtx side = cx;
+        if (FMT == 3 && a.split_v && ph == 0) {
+            if (vside) {
+                side.wg = cx.wg - a.v_wg0; side.G = cx.G - a.v_wg0;
+                job.which = PD_V;
+                job.qs += a.v_qs_off;
+                job.ws = reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(job.ws) + a.v_ws_off);
+                job.wf = a.wf[PD_V];
+                job.row_off = a.QKS + a.KV;
             } else {
-                run(job, next, early);
+                side.G = a.v_wg0;
             }
-        } else if (FMT == 1 || (FMT == 2 && job.wf == WF_Q4)) {
-            pd_gemv_phase<WF_Q4, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
-        } else {
-            pd_gemv_phase<WF_Q8, HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, cx);
         }
+        pd_gemv_phase<HD, FMT, ORD, PEN>(a, job, next, early, W, W1, emb, pos, crow, aq_lds, as_lds, misc, big, best, side);
         early = next.valid;
         if (sh_abort) return;
     }
@@ -1524,7 +1539,7 @@ __global__ __launch_bounds__(256) void pd_repack_q4k_kernel(const uint8_t* __res
 }
 
 __global__ __launch_bounds__(256) void pd_repack_q6k_kernel(const uint8_t* __restrict__ qs, const uint8_t* __restrict__ meta, uint32_t K, uint64_t total,
-                                                          uint8_t* __restrict__ codes) {
+                                                          uint8_t* __restrict__ codes, uint32_t* __restrict__ words) {
     const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;       // n * nblk + b
     if (id >= total) return;
     const uint32_t nblk = K / 32;
@@ -1537,35 +1552,25 @@ __global__ __launch_bounds__(256) void pd_repack_q6k_kernel(const uint8_t* __res
     const uint8_t* ql = sp + 64 * h + 32 * (r & 1);
     const uint8_t* qh = sp + 128 + 32 * h;
     const uint32_t nib_shift = (r >> 1) * 4, pair_shift = 2 * r;
-    for (uint32_t half = 0; half < 2; half++) {
-        uint32_t c[16];
-        for (uint32_t i = 0; i < 16; i++) {
-            const uint32_t e = 16 * half + i;
-            c[i] = ((ql[e] >> nib_shift) & 15u) | (((qh[e] >> pair_shift) & 3u) << 4);        // 0..63, the weight is this minus 32
-        }
-        uint8_t* dst = codes + (id * 2 + half) * 16;
-        for (uint32_t k = 0; k < 4; k++) {
-            dst[k] = (uint8_t)((c[k] & 15u) | ((c[4 + k] & 15u) << 4));
-            dst[4 + k] = (uint8_t)((c[8 + k] & 15u) | ((c[12 + k] & 15u) << 4));
-            dst[8 + k] = (uint8_t)((c[k] >> 4) | ((c[4 + k] >> 4) << 2) | ((c[8 + k] >> 4) << 4) | ((c[12 + k] >> 4) << 6));
-        }
-        dst[12] = mp[2 * jb + half];          // the int8 scale of this half
-        dst[13] = 0;
-        dst[14] = mp[16];                     // d (fp16)
-        dst[15] = mp[17];
+    uint8_t* dst = codes + id * 32;
+    for (uint32_t e = 0; e < 32; e++) {
+        const int c = (int)(((ql[e] >> nib_shift) & 15u) | (((qh[e] >> pair_shift) & 3u) << 4)) - 32;       // the weight: -32..31
+        dst[e] = (uint8_t)(int8_t)c;
     }
+    // the int8 scales of the block's two halves, then d (fp16)
+    words[id] = (uint32_t)mp[2 * jb] | ((uint32_t)mp[2 * jb + 1] << 8) | ((uint32_t)mp[16] << 16) | ((uint32_t)mp[17] << 24);
 }
 
 // Bytes of the two planes of an [N][K] K-quant matrix in the kernel's layout.
 size_t pd_kq_code_bytes(uint32_t wdtype, uint64_t N, uint32_t K) { return wdtype == FORGE_HIP_Q4_K ? N * (K / 32) * 16 : N * (K / 32) * 32; }
-size_t pd_kq_word_bytes(uint32_t wdtype, uint64_t N, uint32_t K) { return wdtype == FORGE_HIP_Q4_K ? N * (K / 32) * 4 : 0; }
+size_t pd_kq_word_bytes(uint32_t, uint64_t N, uint32_t K) { return N * (K / 32) * 4; }
 
 void pd_repack_kquant(const QWeight& w, uint8_t* codes, uint8_t* words, hipStream_t s) {
     const uint64_t total = (uint64_t)w.N * (w.K / 32);
     const uint32_t grid = (uint32_t)((total + 255) / 256);
     const uint8_t* meta = reinterpret_cast<const uint8_t*>(w.scales);
     if (w.wdtype == FORGE_HIP_Q4_K) fh::launch(pd_repack_q4k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, codes, reinterpret_cast<uint32_t*>(words));
-    else fh::launch(pd_repack_q6k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, codes);
+    else fh::launch(pd_repack_q6k_kernel, grid, 256, 0, s, w.qs, meta, w.K, total, codes, reinterpret_cast<uint32_t*>(words));
 }
 
 uint32_t wf_of(uint32_t wdtype) {
@@ -1687,7 +1692,8 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
 
     // LDS: activation codes | activation scales | misc | big
     a.off_act_s = round_up(kmax, 16);
-    a.off_misc = a.off_act_s + round_up(kmax / 32 * 4, 16);
+    // K-quant models: one more strip of kmax / 32 floats per streaming wave behind the scales (each wave's sums of activation codes)
+    a.off_misc = a.off_act_s + round_up(kmax / 32 * 4, 16) * (st->kquant ? PD_STREAM_WAVES + 1 : 1);
     a.off_big = a.off_misc + PD_MISC_BYTES;
     if (a.off_big + 4096 > PD_LDS_BYTES) return FORGE_HIP_OK;
     const uint32_t big = PD_LDS_BYTES - 64 - a.off_big;
@@ -1699,15 +1705,26 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     if (layers.empty() || layers.size() > PD_MAX_LAYERS * PD_MAX_SEGMENTS) return FORGE_HIP_OK;
     QWeight lm_res = lm_head;                     // K-quant models: the lm_head in the kernel's layout
     if (st->kquant) {
+        if (exact) return FORGE_HIP_OK;           // order-faithful K-quant models keep the kernel sequence
         const PdLayerIn& in0 = layers[0];
         // descriptors of the matrices as the kernel sees them: q;k (with v behind it when v shares their format), o, gate;up, down
         const bool split_v = in0.v->wdtype != in0.q->wdtype;
         auto desc = [](uint32_t wdtype, uint32_t K, uint32_t N) { QWeight d; d.wdtype = wdtype; d.K = K; d.N = N; return d; };
         const QWeight dqk = desc(in0.q->wdtype, H, split_v ? QKS + KV : QKS + 2 * KV), dv = desc(in0.v->wdtype, H, KV),
                       dgu = desc(in0.gate->wdtype, H, 2 * I);
-        if (!plan_gemv(dqk, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_QKV]) || !plan_gemv(*in0.o, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_O]) ||
+        // a v matrix of its own shares the grid with q;k in proportion to the bytes each side streams
+        uint32_t g_qk = st->grid;
+        if (split_v) {
+            if (st->grid < 2) return FORGE_HIP_OK;
+            const double bq = (double)(pd_kq_code_bytes(dqk.wdtype, dqk.N, H) + pd_kq_word_bytes(dqk.wdtype, dqk.N, H)),
+                         bv = (double)(pd_kq_code_bytes(dv.wdtype, dv.N, H) + pd_kq_word_bytes(dv.wdtype, dv.N, H));
+            g_qk = (uint32_t)((double)st->grid * bq / (bq + bv) + 0.5);
+            g_qk = std::min(std::max(g_qk, 1u), st->grid - 1);
+        }
+        a.v_wg0 = g_qk;
+        if (!plan_gemv(dqk, 0, 0, nullptr, 4, g_qk, big, &a.shape[PD_QKV]) || !plan_gemv(*in0.o, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_O]) ||
             !plan_gemv(dgu, I, 0, nullptr, 4, st->grid, big, &a.shape[PD_GU]) || !plan_gemv(*in0.down, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_DOWN]) ||
-            (split_v && !plan_gemv(dv, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_V])) ||
+            (split_v && !plan_gemv(dv, 0, 0, nullptr, 4, st->grid - g_qk, big, &a.shape[PD_V])) ||
             !plan_gemv(lm_head, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_LM]))
             return FORGE_HIP_OK;
         for (int k = 0; k < 6; k++) { a.shape[k].qs = nullptr; a.shape[k].ws = nullptr; }
@@ -1791,7 +1808,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
         if (!plan_gemv(lm_head, 0, 1, sl, 4, st->grid, big, &a.shape[PD_LM])) return FORGE_HIP_OK;
         a.wf[PD_QKV] = a.wf[PD_O] = a.wf[PD_GU] = a.wf[PD_DOWN] = a.wf[PD_V] = st->q4 ? WF_Q4 : WF_Q8;
         a.wf[PD_LM] = st->lmq4 ? WF_Q4 : WF_Q8;
-        a.split_v = 0; a.v_qs_off = 0; a.v_ws_off = 0;
+        a.split_v = 0; a.v_qs_off = 0; a.v_ws_off = 0; a.v_wg0 = 0;
     }
     (void)lm_res;
     // cooperative residency: one workgroup per CU must fit

@@ -887,13 +887,11 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
     }
     const char* penv = getenv("FORGE_HIP_PERSIST");
     const char* kenv = getenv("FORGE_HIP_PD_KQUANT");
-    if (pd && !(penv && penv[0] == '0') && kenv && kenv[0] == '1') {
-        // a model whose matrices are all Q4_K / Q6_K (q and k of one format, gate and up too) can run its decode step as the
-        // resident kernel with K-quant weight units: bit-identical to the kernel sequence in the ordered variant, but not
-        // faster (Q4_K_M-recipe 1B shape: 920 against 868 us per token: the K-quant block decoders are instruction-bound on
-        // the kernel's six streaming waves, and a v matrix of another format than q and k costs a phase of its own), so the
-        // sequence stays the default and FORGE_HIP_PD_KQUANT=1 asks for the kernel.  pd_create leaves m->pd null for any
-        // other mix.
+    if (pd && !(penv && penv[0] == '0') && !(kenv && kenv[0] == '0')) {
+        // a model whose matrices are all Q4_K / Q6_K (q and k of one format, gate and up too) runs its decode step as the
+        // resident kernel with K-quant weight units (a second copy of the matrices in the kernel's layout): bit-identical to
+        // the kernel sequence in the ordered variant.  FORGE_HIP_PD_KQUANT=0 keeps the kernel sequence for such models;
+        // pd_create leaves m->pd null for any other mix.
         bool all_k = is_kquant(cfg->lm_head_dtype);
         for (int i = 0; i < 7; i++) all_k = all_k && is_kquant(pd[i]);
         if (all_k && pd[0] == pd[1] && pd[4] == pd[5]) {

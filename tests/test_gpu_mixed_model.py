@@ -205,7 +205,8 @@ def test_mixed_model_fast_mode(fh, oracle, torch_gpu, mix, monkeypatch):
     blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=21, std=0.05)
     toks = fh.synth.uniform_ids(12, 40, cfg["vocab"])
     gm = fh.HipModel(cfg, blob, proj_dtypes=pd)
-    assert gm.decode_launches > 1                           # the kernel sequence: one launch per projection
+    # all matrices Q4_K / Q6_K: one resident kernel per step; a mix with Q8_0 / Q4_0 matrices: the kernel sequence
+    assert (gm.decode_launches == 1) == (mix == "q4_k_m")
     om = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
     gl, ol = gm.forward_prefill(toks), om.prefill_batched(toks)
     # layer 0's K/V rows depend on embedding -> rms_norm -> matmul -> rope only: the fast matmul's bound
@@ -283,9 +284,10 @@ def test_mixed_model_grouped_launches_keep_the_bits(fh, torch_gpu, monkeypatch):
 @pytest.mark.parametrize("mix,extra", [("q4_k_m", {}), ("q6_k", {}), ("q4_k_m", dict(flags=QKV_BIAS)), ("q4_k_m", dict(sliding_window=24)),
                                        ("q4_k_m", dict(hidden=512, inter=1024, heads=4, kv_heads=4, head_dim=128))])
 def test_kquant_weight_units_in_the_resident_kernel(fh, torch_gpu, monkeypatch, mix, extra):
-    """FORGE_HIP_PD_KQUANT=1: the decode step of a model whose matrices are all Q4_K / Q6_K as ONE resident kernel, the matrices
-    re-laid out as its weight units (Q4_K: Q4_0-ordered nibbles + a word of d | dmin, scale and minimum per sub-block; Q6_K:
-    16 bytes per 16 weights with scale and d inside); a v matrix of another format than q and k is a phase of its own.  With
+    """The decode step of a model whose matrices are all Q4_K / Q6_K is ONE resident kernel (FORGE_HIP_PD_KQUANT=0: the kernel
+    sequence), the matrices re-laid out as its weight units (Q4_K: Q4_0-ordered nibbles + a word of d | dmin, scale and minimum
+    per sub-block; Q6_K: 16 bytes per 16 weights with scale and d inside); a v matrix of another format than q and k shares
+    the q;k;v phase with them, each side on its own share of the workgroups.  With
     the ordered row sums (FORGE_HIP_PD_ORDERED=1) every logit equals the kernel sequence's bit for bit, step after step, and
     the cache rows too; the default sums differ by the order of additions (and by the int8 activation codes that this moves)."""
     pd, lm = MIXES[mix]
@@ -295,14 +297,14 @@ def test_kquant_weight_units_in_the_resident_kernel(fh, torch_gpu, monkeypatch, 
     cfg["sliding_window"] = extra.get("sliding_window", 0)
     blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=29, std=0.05)
     toks = fh.synth.uniform_ids(31, 45, cfg["vocab"])
+    monkeypatch.setenv("FORGE_HIP_PD_KQUANT", "0")
     seq = fh.HipModel(cfg, blob, proj_dtypes=pd)
     assert seq.decode_launches > 1
-    monkeypatch.setenv("FORGE_HIP_PD_KQUANT", "1")
+    monkeypatch.delenv("FORGE_HIP_PD_KQUANT")
     fast = fh.HipModel(cfg, blob, proj_dtypes=pd)
     monkeypatch.setenv("FORGE_HIP_PD_ORDERED", "1")
     ordered = fh.HipModel(cfg, blob, proj_dtypes=pd)
     monkeypatch.delenv("FORGE_HIP_PD_ORDERED")
-    monkeypatch.delenv("FORGE_HIP_PD_KQUANT")
     assert fast.decode_launches == ordered.decode_launches == 1
     a = seq.forward_prefill(toks)
     assert np.array_equal(a, ordered.forward_prefill(toks)) and np.array_equal(a, fast.forward_prefill(toks))
