@@ -1320,7 +1320,9 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
 // fits the instruction cache matters more than one binary for all models.
 // ORD: the GEMV rows are summed in the reference's block order (bit-identical to the kernel sequence) instead of as the
 // products come.
-template <int HD, int FMT, bool ORD, bool PEN>
+// XA (ordered variants only): the attention walks the keys in the reference's own order instead of in splits; each kernel
+// carries one of the two.
+template <int HD, int FMT, bool ORD, bool PEN, bool XA>
 __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     extern __shared__ __align__(16) uint8_t smem[];
     __shared__ uint32_t sh_abort;
@@ -1368,7 +1370,7 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
         const uint32_t x_in = lg ? base : 0;                 // tag of x entering the layer (0: still the embedding row)
         if (ph == 1) {
             if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * lg + 1] = wall_clock64();
-            if (ORD && a.exact_attn) {
+            if (XA) {
                 pd_attn_exact_blocks<HD>(px_args(a), a.layers[l].kc, a.layers[l].vc, pos, base + 1, base + 2, cx);
                 if (a.stamps && cx.wg == 0 && cx.tid == 0) a.stamps[6 * lg + 2] = wall_clock64();
                 pd_attn_exact_chain<HD>(px_args(a), pos, base + 2, base + 3, misc, big, cx);
@@ -1607,19 +1609,20 @@ bool plan_gemv(const QWeight& w, uint32_t inter, uint32_t nseg, const Segment* s
     return true;
 }
 
-template <int HD, bool ORD, bool PEN>
+template <int HD, bool ORD, bool PEN, bool XA>
 const void* pd_kernel_ord(const PdState* st) {
-    // (K-quant models always run the variant with the optional extras: half as many kernels to build for a path that is opt-in)
-    if (st->kquant) return reinterpret_cast<const void*>(decode_step_kernel<HD, 3, ORD, true>);
-    if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2, ORD, PEN>);
-    return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 1, ORD, PEN>) : reinterpret_cast<const void*>(decode_step_kernel<HD, 0, ORD, PEN>);
+    // (K-quant models always run the variant with the optional extras, and never the reference-order attention)
+    if (st->kquant) return reinterpret_cast<const void*>(decode_step_kernel<HD, 3, ORD, true, false>);
+    if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2, ORD, PEN, XA>);
+    return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 1, ORD, PEN, XA>)
+                  : reinterpret_cast<const void*>(decode_step_kernel<HD, 0, ORD, PEN, XA>);
 }
 // The repeat penalty (lm_head epilogue) and the QKV bias (qkv epilogue) are code of their own: the default kernel is
 // built without them (the ordered variants always carry them).
 template <int HD>
 const void* pd_kernel(const PdState* st) {
-    if (st->ordered) return pd_kernel_ord<HD, true, true>(st);
-    return (st->args.penalty > 1.0f || st->args.qkv_bias) ? pd_kernel_ord<HD, false, true>(st) : pd_kernel_ord<HD, false, false>(st);
+    if (st->ordered) return st->args.exact_attn ? pd_kernel_ord<HD, true, true, true>(st) : pd_kernel_ord<HD, true, true, false>(st);
+    return (st->args.penalty > 1.0f || st->args.qkv_bias) ? pd_kernel_ord<HD, false, true, false>(st) : pd_kernel_ord<HD, false, false, false>(st);
 }
 template <int HD>
 hipError_t launch_pd_hd(const PdState* st, hipStream_t s) {
