@@ -60,7 +60,7 @@ constexpr int PD_WAVES = PD_THREADS / 64;
 constexpr int PD_D = 8;                       // weight units (1 KB) a wave holds in registers per round
 constexpr uint32_t PD_MAX_TILE_ROWS = 128;      // = 64 PD_POLL_WAVES: the pollers own a tile's rows
 constexpr uint32_t PD_LDS_BYTES = 64 * 1024;
-constexpr uint32_t PD_MISC_BYTES = 2048;
+constexpr uint32_t PD_MISC_BYTES = 2048 + 256;
 constexpr int PD_POLL_WAVES = 2;              // waves that fetch a phase's input; the others stream weights
 constexpr int PD_POLL_THREADS = PD_POLL_WAVES * 64;
 constexpr int PD_STREAM_WAVES = PD_WAVES - PD_POLL_WAVES;
@@ -70,6 +70,8 @@ constexpr int PD_MISC_HINT = 40, PD_MISC_SCRATCH = 64;
 // misc LDS words [PD_MISC_PT, 512): page-table entries of this workgroup's attention items, staged once per step (an item's
 // key range is the same in every layer); slot (round, wave group) holds pt_cap entries
 constexpr int PD_MISC_PT = 128, PD_MISC_PT_WORDS = 512 - PD_MISC_PT;
+// misc LDS words [512, 576): the 32 table entries of expf_ref (ordered variants), so that an exp costs an LDS read, not a trip to memory
+constexpr int PD_MISC_EXP = 512;
 // `big` area: a GEMV phase's row sums sit at its start -- [rows][4] partial sums by default, [rows][nblk + 1] block products
 // in the ordered variants -- and the residual row that a norm phase fetches (H floats) starts PD_X_WORDS further on.  The
 // two poller waves leave a GEMV phase one after the other (the one without rows does not wait for the one that still adds
@@ -206,7 +208,14 @@ struct PdCtx {
     uint32_t spin_limit;
     uint32_t* sh_abort;      // LDS
     uint32_t* abort_flag;    // global
+    const uint64_t* exp_tab; // LDS: expf_ref's table (ordered variants)
 };
+struct LdsExpTab {
+    const uint64_t* p;
+    __device__ __forceinline__ uint64_t operator()(int i) const { return p[i]; }
+};
+template <bool kFma>
+__device__ __forceinline__ float pd_expf(float x, const PdCtx& cx) { return expf_ref_with<kFma>(x, LdsExpTab{cx.exp_tab}); }
 
 // Re-read one element until it carries `tag`; bounded.
 __device__ __forceinline__ uint32_t poll(const uint64_t* p, uint32_t tag, const PdCtx& cx) {
@@ -1002,7 +1011,7 @@ __device__ __forceinline__ void pd_attn_exact_blocks(const PxArgs& a, const uint
         }
         m = wave_max(m);
         // ---- weights, l_block and sum[d] (sequential over the block's keys; lane = head dim)
-        const float e = lane < bl ? expf_ref<true>(sc - m) : 0.f;
+        const float e = lane < bl ? pd_expf<true>(sc - m, cx) : 0.f;
         float l_block = 0.f, acc[NQ];
 #pragma unroll
         for (int j = 0; j < NQ; j++) acc[j] = 0.f;
@@ -1052,7 +1061,7 @@ __device__ __forceinline__ void pd_attn_exact_chain(const PxArgs& a, uint32_t po
             __syncthreads();
             if (*cx.sh_abort) return;
             // exp_scale = exp(m_prev - m_i), m_prev = -inf before the first block
-            if (tid < n) es[tid] = expf_ref<true>((tid ? recs[(tid - 1) * REC + HD] : m_prev) - recs[tid * REC + HD]);
+            if (tid < n) es[tid] = pd_expf<true>((tid ? recs[(tid - 1) * REC + HD] : m_prev) - recs[tid * REC + HD], cx);
             m_prev = recs[(n - 1) * REC + HD];
             __syncthreads();
             if (tid < HD) {
@@ -1282,7 +1291,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
                 const float ux = lane_xor<32>(v);         // lanes 0..31: the up row of the same inter index
                 if (lr < 32) {
                     // silu_mul, emit.rs:380-386; the C library's expf bit for bit where the reference order is asked for
-                    const float o = (v / (1.0f + (ORDERED ? expf_ref<true>(-v) : __expf(-v)))) * ux;
+                    const float o = (v / (1.0f + (ORDERED ? pd_expf<true>(-v, cx) : __expf(-v)))) * ux;
                     const float amax = half_wave_max(fabsf(o));
                     float inv;
                     const float sc = act_scale(amax, inv);
@@ -1341,6 +1350,8 @@ __global__ __launch_bounds__(PD_THREADS) void decode_step_kernel(PdArgs a) {
     cx.sh_abort = &sh_abort;
     cx.abort_flag = a.state + 3;
     if (cx.tid == 0) { sh_abort = 0; reinterpret_cast<uint32_t*>(misc)[PD_MISC_HINT] = 0; }
+    cx.exp_tab = reinterpret_cast<const uint64_t*>(misc + PD_MISC_EXP);
+    if (ORD && cx.tid < 32) reinterpret_cast<uint64_t*>(misc + PD_MISC_EXP)[cx.tid] = expf_detail::tab((int)cx.tid);
     __syncthreads();
 
     const uint32_t pos = a.state[0], token = a.token_from_arg ? a.token : a.state[1];
@@ -1590,6 +1601,15 @@ bool plan_gemv(const QWeight& w, uint32_t inter, uint32_t nseg, const Segment* s
     g->inter = inter;
     g->nseg = nseg; g->tail_mod = tail_mod;
     for (uint32_t i = 0; i < nseg; i++) g->seg[i] = seg[i];
+    // rows in the four-accumulator order are the last len % tail_mod of each chunk: a matrix without any (the usual case:
+    // every chunk a multiple of tail_mod rows) tells the kernel so by carrying no segments, and no row asks
+    bool any_dot1 = false;
+    for (uint32_t i = 0; i < nseg && tail_mod; i++) {
+        const Segment& sg = seg[i];
+        if (!sg.chunk) any_dot1 = any_dot1 || sg.len % tail_mod != 0;
+        else any_dot1 = any_dot1 || sg.chunk % tail_mod != 0 || (sg.len % sg.chunk) % tail_mod != 0;
+    }
+    if (!any_dot1) g->nseg = 0;
     const uint32_t row_bytes = (g->nblk + 1) * 4;
     uint32_t cap = big_bytes / row_bytes;
     if (cap > PD_MAX_TILE_ROWS) cap = PD_MAX_TILE_ROWS;
@@ -1649,9 +1669,9 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
                   const float* qkv_bias, PdState** out) {
     *out = nullptr;
     // The order-faithful mode can run as this kernel too: the ordered variant with the attention phases in the reference's
-    // order.  It is bit-identical to the kernel sequence but not faster (Llama-3.2-1B shape at 2.5k context: 954 against
-    // 940 us per token; 3B: 2199 against 2115; SmolLM2-135M: 1215 against 996 -- the ordered row sums cost every GEMV
-    // phase 2-4 us that the separate kernels hide behind their launches), so the sequence stays the default and
+    // order.  It is bit-identical to the kernel sequence but not faster across shapes (Llama-3.2-1B shape at 2.5k context:
+    // 925 against 935 us per token; 3B: 2125 against 2118; SmolLM2-135M: 1204 against 1041 -- the ordered norm and row sums
+    // cost every GEMV phase 1-2 us that the separate kernels hide behind their launches), so the sequence stays the default and
     // FORGE_HIP_PD_EXACT=1 asks for the kernel.  A window (attention_sliding: another algorithm) and caches of more than
     // 4096 blocks always keep the sequence.
     const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;

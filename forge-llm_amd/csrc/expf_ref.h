@@ -53,8 +53,9 @@ FH_HD inline uint64_t double_as_u64(double d) {
 }
 }  // namespace expf_detail
 
-template <bool kFma>
-FH_HD inline float expf_ref(float x) {
+// `lookup(i)` returns tab(i): a kernel that keeps a copy of the table close by (LDS) passes its own.
+template <bool kFma, typename Lookup>
+FH_HD inline float expf_ref_with(float x, Lookup lookup) {
     using namespace expf_detail;
     constexpr double N = 32.0;
     constexpr double InvLn2N = 0x1.71547652b82fep+0 * N;
@@ -71,7 +72,7 @@ FH_HD inline float expf_ref(float x) {
     const uint64_t ki = double_as_u64(kd);
     kd -= Shift;
     const double r = z - kd;
-    uint64_t t = tab((int)(ki & 31));
+    uint64_t t = lookup((int)(ki & 31));
     t += ki << 47;
     const double s = u64_as_double(t);
     double y;
@@ -89,5 +90,12 @@ FH_HD inline float expf_ref(float x) {
     y = y * s;
     return (float)y;
 }
+
+namespace expf_detail {
+struct TabLookup { FH_HD uint64_t operator()(int i) const { return tab(i); } };
+}  // namespace expf_detail
+
+template <bool kFma>
+FH_HD inline float expf_ref(float x) { return expf_ref_with<kFma>(x, expf_detail::TabLookup{}); }
 
 }  // namespace fh
