@@ -553,7 +553,7 @@ __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& 
                     const int4 a = *reinterpret_cast<const int4*>(aq_lds + bs * 8 + (lane & 1u) * 4);
                     const int dh = in ? dot16(W.v[d], a, 0) : 0;      // this lane's 16 weights are one scale's
                     const uint32_t ww = W.s[d];
-                    const float th = (float)((int)(ww << (24u - (lane & 1u) * 8u)) >> 24) * (float)dh;      // the int8 scale of this lane's half
+                    const float th = (float)((int)(ww << (24u - (lane & 1u) * 8u)) >> 24) * (float)dh;      // the int8 scale of this lane's half (two shifts: the signed bit-field builtin gave wrong values with a lane-dependent offset)
                     const float u = th + __builtin_amdgcn_update_dpp(0.f, th, 0xB1, 0xF, 0xF, false);       // lo + hi (even lane)
                     term = (f16_bits_to_f32((uint16_t)(ww >> 16)) * as_lds[bs]) * u;
                     mine = in && !(lane & 1u);
