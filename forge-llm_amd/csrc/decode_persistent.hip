@@ -113,6 +113,10 @@ enum { PD_QKV = 0, PD_O = 1, PD_GU = 2, PD_DOWN = 3, PD_LM = 4, PD_V = 5 };
 //         instructions per weight, not by the bytes); one word per block: the int8 scales of its two halves | fp16 bits of d << 16
 enum { WF_Q8 = 0, WF_Q4 = 1, WF_Q4K = 2, WF_Q6K = 3 };
 __host__ __device__ constexpr bool wf_lane_per_block(int wf) { return wf == WF_Q4 || wf == WF_Q4K; }
+// The (at most two) weight formats a kernel variant FMT carries code for: 0 Q8_0, 1 Q4_0, 2 both, 3 Q4_K + Q6_K,
+// 4 Q4_0 + Q6_K, 5 Q8_0 + Q6_K (the last two: uniform projections under a Q6_K lm_head).
+__host__ __device__ constexpr int fmt_first(int fmt) { return fmt == 0 || fmt == 2 || fmt == 5 ? WF_Q8 : fmt == 3 ? WF_Q4K : WF_Q4; }
+__host__ __device__ constexpr int fmt_second(int fmt) { return fmt == 2 ? WF_Q4 : fmt >= 3 ? WF_Q6K : fmt_first(fmt); }
 
 struct PdArgs {
     PdGemv shape[6];           // qkv, o, gate_up, down (addresses per layer, below), lm_head (addresses here) and, with split_v, v
@@ -502,11 +506,9 @@ __device__ __forceinline__ void pd_load_first(const PdArgs& a, const Mat& m, uin
     const TilePos t = pd_tile(h, wg);
     GemvJob j{};
     j.qs = m.qs; j.ws = m.ws;
-    if (FMT == 3) {
-        if (m.wf == WF_Q4K) pd_load_round<WF_Q4K>(j, h, t, 0, sw, lane, W);
-        else pd_load_round<WF_Q6K>(j, h, t, 0, sw, lane, W);
-    } else if (FMT == 1 || (FMT == 2 && m.wf == WF_Q4)) pd_load_round<WF_Q4>(j, h, t, 0, sw, lane, W);
-    else pd_load_round<WF_Q8>(j, h, t, 0, sw, lane, W);
+    constexpr int WFA = fmt_first(FMT), WFB = fmt_second(FMT);
+    if (WFB != WFA && m.wf == (uint32_t)WFB) pd_load_round<WFB>(j, h, t, 0, sw, lane, W);
+    else pd_load_round<WFA>(j, h, t, 0, sw, lane, W);
 }
 
 // Exact int32 block dots on v_dot4 and one f32 product (a_s*w_s)*f32(isum) per block.
@@ -1145,8 +1147,7 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     const Shape h = pd_shape(g);
     const bool streamer = cx.wave >= (uint32_t)PD_POLL_WAVES;
     const uint32_t sw = cx.wave - PD_POLL_WAVES;
-    constexpr int WFA = FMT == 0 ? WF_Q8 : FMT == 1 ? WF_Q4 : FMT == 2 ? WF_Q8 : WF_Q4K;      // the format(s) this kernel carries
-    constexpr int WFB = FMT == 2 ? WF_Q4 : FMT == 3 ? WF_Q6K : WFA;
+    constexpr int WFA = fmt_first(FMT), WFB = fmt_second(FMT);      // the format(s) this kernel carries
     const bool second = WFB != WFA && job.wf == (uint32_t)WFB;
     auto load_round = [&](const TilePos& tt, uint32_t r, WReg& w) {
         if (second) pd_load_round<WFB>(job, h, tt, r, sw, cx.lane, w);
@@ -1325,8 +1326,8 @@ __device__ __forceinline__ void pd_gemv_phase(const PdArgs& a, const GemvJob& jo
     }
 }
 
-// FMT: which weight formats the kernel carries code for (0: Q8_0 only, 1: Q4_0 only, 2: both) -- a kernel that
-// fits the instruction cache matters more than one binary for all models.
+// FMT: which weight formats the kernel carries code for (fmt_first / fmt_second) -- a kernel that fits the instruction
+// cache matters more than one binary for all models.
 // ORD: the GEMV rows are summed in the reference's block order (bit-identical to the kernel sequence) instead of as the
 // products come.
 // XA (ordered variants only): the attention walks the keys in the reference's own order instead of in splits; each kernel
@@ -1509,6 +1510,7 @@ struct PdState {
     std::vector<void*> owned;
     uint32_t grid = 0, lds = 0, hd = 0, tags_per_launch = 0, n_stamps = 0;
     bool q4 = false, lmq4 = false, kquant = false, ordered = false, cooperative = true;
+    bool lmk = false;              // a K-quant (Q6_K) lm_head over Q8_0 / Q4_0 projections
     size_t tagged_bytes = 0;
     void* tagged_base = nullptr;
     std::vector<unsigned long long> stamps_host;
@@ -1633,6 +1635,8 @@ template <int HD, bool ORD, bool PEN, bool XA>
 const void* pd_kernel_ord(const PdState* st) {
     // (K-quant models always run the variant with the optional extras, and never the reference-order attention)
     if (st->kquant) return reinterpret_cast<const void*>(decode_step_kernel<HD, 3, ORD, true, false>);
+    if (st->lmk) return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 4, ORD, true, false>)
+                               : reinterpret_cast<const void*>(decode_step_kernel<HD, 5, ORD, true, false>);
     if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2, ORD, PEN, XA>);
     return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 1, ORD, PEN, XA>)
                   : reinterpret_cast<const void*>(decode_step_kernel<HD, 0, ORD, PEN, XA>);
@@ -1700,6 +1704,9 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     // a model of K-quant matrices: every projection and the lm_head Q4_K or Q6_K, q and k of one format, gate and up too
     if (layers.empty()) return FORGE_HIP_OK;
     st->kquant = layers[0].q != nullptr;
+    // Q8_0 / Q4_0 projections under a Q6_K lm_head (fast mode only, like the all-K-quant models)
+    st->lmk = !st->kquant && lm_head.kquant();
+    if (st->lmk && (lm_head.wdtype != FORGE_HIP_Q6_K || exact)) return FORGE_HIP_OK;
     if (st->kquant) {
         const PdLayerIn& in = layers[0];
         const QWeight* all[7] = {in.q, in.k, in.v, in.o, in.gate, in.up, in.down};
@@ -1827,11 +1834,26 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
             L.attn_norm = in.attn_norm; L.kc = in.kc; L.vc = in.vc;
     }
     if (!st->kquant) {
-        Segment sl[1] = {make_segment(c.lm_head_dtype, H, 0, c.vocab, true)};
-        if (!plan_gemv(lm_head, 0, 1, sl, 4, st->grid, big, &a.shape[PD_LM])) return FORGE_HIP_OK;
         a.wf[PD_QKV] = a.wf[PD_O] = a.wf[PD_GU] = a.wf[PD_DOWN] = a.wf[PD_V] = st->q4 ? WF_Q4 : WF_Q8;
-        a.wf[PD_LM] = st->lmq4 ? WF_Q4 : WF_Q8;
         a.split_v = 0; a.v_qs_off = 0; a.v_ws_off = 0; a.v_wg0 = 0;
+        if (st->lmk) {
+            // a Q6_K lm_head over Q8_0 / Q4_0 projections: the matrix in the kernel's layout, its rows summed in block order
+            if (!plan_gemv(lm_head, 0, 0, nullptr, 4, st->grid, big, &a.shape[PD_LM])) return FORGE_HIP_OK;
+            const size_t cl = pd_kq_code_bytes(lm_head.wdtype, c.vocab, H), wl = pd_kq_word_bytes(lm_head.wdtype, c.vocab, H);
+            uint8_t* c_l = dev_alloc<uint8_t>(cl, st->owned);
+            uint8_t* w_l = dev_alloc<uint8_t>(wl, st->owned);
+            if (!c_l || !w_l) return fail(FORGE_HIP_ERR_HIP, "persistent decode: out of device memory for the K-quant weight units");
+            pd_repack_kquant(lm_head, c_l, w_l, nullptr);
+            FH_HIP(hipDeviceSynchronize());
+            FH_HIP(hipGetLastError());
+            a.shape[PD_LM].qs = c_l;
+            a.shape[PD_LM].ws = reinterpret_cast<const uint16_t*>(w_l);
+            a.wf[PD_LM] = WF_Q6K;
+        } else {
+            Segment sl[1] = {make_segment(c.lm_head_dtype, H, 0, c.vocab, true)};
+            if (!plan_gemv(lm_head, 0, 1, sl, 4, st->grid, big, &a.shape[PD_LM])) return FORGE_HIP_OK;
+            a.wf[PD_LM] = st->lmq4 ? WF_Q4 : WF_Q8;
+        }
     }
     (void)lm_res;
     // cooperative residency: one workgroup per CU must fit

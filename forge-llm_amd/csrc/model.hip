@@ -754,12 +754,27 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
         FH_HIP(hipMemcpy(L.attn_norm, p, H * 4, hipMemcpyHostToDevice));
         p += H * 4;
         if (pd) {
-            if ((rc = qweight_upload(pd[0], p, H, QKS, &L.q))) return rc;
-            p += wsize(pd[0], QKS, H);
-            if ((rc = qweight_upload(pd[1], p, H, KV, &L.k))) return rc;
-            p += wsize(pd[1], KV, H);
-            if ((rc = qweight_upload(pd[2], p, H, KV, &L.v))) return rc;
-            p += wsize(pd[2], KV, H);
+            // Q8_0 / Q4_0 neighbours of one format (q, k, v; gate, up) go up as one matrix, as in the uniform model (the
+            // resident decode kernel multiplies them in one phase); the per-projection launches see its row ranges
+            auto rows_of = [](const QWeight& whole, uint32_t row0, uint32_t rows) {
+                QWeight v;
+                v.wdtype = whole.wdtype; v.K = whole.K; v.N = rows;
+                v.qs = whole.qs + (size_t)row0 * whole.qs_row_bytes();
+                v.scales = whole.scales + (size_t)row0 * (whole.K / 32);
+                return v;                                     // owns stays false
+            };
+            if (!is_kquant(pd[0]) && pd[0] == pd[1] && pd[1] == pd[2]) {
+                if ((rc = qweight_upload(pd[0], p, H, m->QKV, &L.qkv))) return rc;
+                p += wsize(pd[0], m->QKV, H);
+                L.q = rows_of(L.qkv, 0, QKS); L.k = rows_of(L.qkv, QKS, KV); L.v = rows_of(L.qkv, QKS + KV, KV);
+            } else {
+                if ((rc = qweight_upload(pd[0], p, H, QKS, &L.q))) return rc;
+                p += wsize(pd[0], QKS, H);
+                if ((rc = qweight_upload(pd[1], p, H, KV, &L.k))) return rc;
+                p += wsize(pd[1], KV, H);
+                if ((rc = qweight_upload(pd[2], p, H, KV, &L.v))) return rc;
+                p += wsize(pd[2], KV, H);
+            }
             if (has_bias) {                                   // q_bias | k_bias | v_bias, project.rs:286-292
                 L.qkv_bias = m->biases.as<float>() + (size_t)l * m->QKV;
                 FH_HIP(hipMemcpy(L.qkv_bias, p, (size_t)m->QKV * 4, hipMemcpyHostToDevice));
@@ -769,10 +784,16 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
             p += wsize(pd[3], H, QKS);
             FH_HIP(hipMemcpy(L.ffn_norm, p, H * 4, hipMemcpyHostToDevice));
             p += H * 4;
-            if ((rc = qweight_upload(pd[4], p, H, I, &L.gate))) return rc;
-            p += wsize(pd[4], I, H);
-            if ((rc = qweight_upload(pd[5], p, H, I, &L.up))) return rc;
-            p += wsize(pd[5], I, H);
+            if (!is_kquant(pd[4]) && pd[4] == pd[5]) {
+                if ((rc = qweight_upload(pd[4], p, H, 2 * I, &L.gate_up))) return rc;
+                p += wsize(pd[4], 2 * (uint64_t)I, H);
+                L.gate = rows_of(L.gate_up, 0, I); L.up = rows_of(L.gate_up, I, I);
+            } else {
+                if ((rc = qweight_upload(pd[4], p, H, I, &L.gate))) return rc;
+                p += wsize(pd[4], I, H);
+                if ((rc = qweight_upload(pd[5], p, H, I, &L.up))) return rc;
+                p += wsize(pd[5], I, H);
+            }
             if ((rc = qweight_upload(pd[6], p, I, H, &L.down))) return rc;
             p += wsize(pd[6], H, I);
             continue;
@@ -901,6 +922,25 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
                 pl[l] = PdLayerIn{nullptr, &L.o, nullptr, &L.down, L.attn_norm, L.ffn_norm, m->kc(l), m->vc(l), &L.q, &L.k, &L.v, &L.gate, &L.up};
             }
             rc = pd_create(*cfg, pl, m->lm_head, m->embed.as<float>(), m->final_norm.as<float>(), m->cos_t.as<float>(),
+                           m->sin_t.as<float>(), m->logits.as<float>(), m->state.as<uint32_t>(), m->counts.as<uint32_t>(),
+                           has_bias ? m->biases.as<float>() : nullptr, &m->pd);
+            if (rc) return rc;
+        }
+    }
+    if (pd && !m->pd && !(penv && penv[0] == '0') && !(kenv && kenv[0] == '0') && cfg->lm_head_dtype == FORGE_HIP_Q6_K && !is_kquant(pd[0])) {
+        // seven Q8_0 or seven Q4_0 projections under a Q6_K lm_head (what llama.cpp writes for its Q4_0 / Q8_0 recipes with
+        // a K-quant output matrix): the uniform model's resident kernel with the lm_head as K-quant weight units
+        bool same = true;
+        for (int i = 1; i < 7; i++) same = same && pd[i] == pd[0];
+        if (same) {
+            forge_hip_config c2 = *cfg;
+            c2.wdtype = pd[0];
+            std::vector<PdLayerIn> pl(cfg->layers);
+            for (uint32_t l = 0; l < cfg->layers; l++) {
+                Layer& L = m->layers[l];
+                pl[l] = PdLayerIn{&L.qkv, &L.o, &L.gate_up, &L.down, L.attn_norm, L.ffn_norm, m->kc(l), m->vc(l)};
+            }
+            rc = pd_create(c2, pl, m->lm_head, m->embed.as<float>(), m->final_norm.as<float>(), m->cos_t.as<float>(),
                            m->sin_t.as<float>(), m->logits.as<float>(), m->state.as<uint32_t>(), m->counts.as<uint32_t>(),
                            has_bias ? m->biases.as<float>() : nullptr, &m->pd);
             if (rc) return rc;

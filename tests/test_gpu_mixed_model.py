@@ -21,6 +21,7 @@ MIXES = {
     "all_four": ((Q8, Q4, Q4K, Q8, Q6K, Q4, Q4K), Q8),
     "kquant_lm_head_only": ((Q4, Q4, Q4, Q4, Q4, Q4, Q4), Q6K),
     "q6_k": ((Q6K,) * 7, Q6K),
+    "q8_0_under_q6_k": ((Q8,) * 7, Q6K),
 }
 
 
@@ -282,12 +283,16 @@ def test_mixed_model_grouped_launches_keep_the_bits(fh, torch_gpu, monkeypatch):
 
 
 @pytest.mark.parametrize("mix,extra", [("q4_k_m", {}), ("q6_k", {}), ("q4_k_m", dict(flags=QKV_BIAS)), ("q4_k_m", dict(sliding_window=24)),
-                                       ("q4_k_m", dict(hidden=512, inter=1024, heads=4, kv_heads=4, head_dim=128))])
+                                       ("q4_k_m", dict(hidden=512, inter=1024, heads=4, kv_heads=4, head_dim=128)),
+                                       ("kquant_lm_head_only", {}), ("q8_0_under_q6_k", dict(flags=QKV_BIAS)),
+                                       ("kquant_lm_head_only", dict(sliding_window=24, hidden=512, inter=1024, heads=4, kv_heads=4, head_dim=96))])
 def test_kquant_weight_units_in_the_resident_kernel(fh, torch_gpu, monkeypatch, mix, extra):
     """The decode step of a model whose matrices are all Q4_K / Q6_K is ONE resident kernel (FORGE_HIP_PD_KQUANT=0: the kernel
     sequence), the matrices re-laid out as its weight units (Q4_K: Q4_0-ordered nibbles + a word of d | dmin, scale and minimum
     per sub-block; Q6_K: 16 bytes per 16 weights with scale and d inside); a v matrix of another format than q and k shares
-    the q;k;v phase with them, each side on its own share of the workgroups.  With
+    the q;k;v phase with them, each side on its own share of the workgroups.  Seven Q4_0 or seven Q8_0 projections under a
+    Q6_K lm_head (llama.cpp's Q4_0 / Q8_0 files with a K-quant output matrix) run the uniform model's kernel with the lm_head as
+    K-quant weight units.  With
     the ordered row sums (FORGE_HIP_PD_ORDERED=1) every logit equals the kernel sequence's bit for bit, step after step, and
     the cache rows too; the default sums differ by the order of additions (and by the int8 activation codes that this moves)."""
     pd, lm = MIXES[mix]
