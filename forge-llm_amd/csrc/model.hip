@@ -76,6 +76,7 @@ struct forge_hip_model {
     bool mixed_twins = false;            // fast mode: K-quant projections of a prompt run on the MFMA GEMM (kquant_prefill.hip)
     bool prefill_fuse_quant = true;              // fast mode: attention writes int8 codes + scales (FORGE_HIP_FUSE=0: separate quantiser)
     bool mixed_fuse = true;          // K-quant projections over a normed row norm and quantise it themselves: a launch less, the same bits
+    bool mixed_plain_layers = false;     // per-projection formats, but all seven are one of Q8_0 / Q4_0 (only the lm_head differs): decode layers run the uniform model's launches
     bool mixed_batched = false;                  // per-projection formats: the prompt runs in batches of rows (see enqueue_mixed_prefill_layer)
     bool prefill_fuse_silu = false;              // fast mode: the gate/up GEMM writes silu(gate) * up quantised (FORGE_HIP_FUSE=0: separate kernel)
     uint32_t chunk_rows = 0;
@@ -313,7 +314,7 @@ void enqueue_mixed_layer(forge_hip_model* m, uint32_t l, uint32_t pos, const uin
 // attention merge + quant, [o GEMV | residual], [norm+quant | gate/up GEMV | silu*up + quant],
 // [down GEMV | residual].
 void enqueue_decode_layer(forge_hip_model* m, uint32_t l) {
-    if (m->mixed) { enqueue_mixed_layer(m, l, 0, m->d_pos()); return; }
+    if (m->mixed && !m->mixed_plain_layers) { enqueue_mixed_layer(m, l, 0, m->d_pos()); return; }
     const forge_hip_config& c = m->cfg;
     Layer& L = m->layers[l];
     hipStream_t s = m->stream;
@@ -721,8 +722,12 @@ static int32_t model_create_impl(const forge_hip_config* cfg, const uint32_t* pd
     m->use_graph = !(genv && genv[0] == '0');
     const char* fenv = getenv("FORGE_HIP_FUSE");
     const bool fuse_ok = !(fenv && fenv[0] == '0');
-    m->fuse_norm = fuse_ok && !pd && gemv_norm_fusable(H);
-    m->fuse_silu = fuse_ok && !pd && gemv_silu_fusable(H);
+    // seven projections of one plain format (the lm_head is what differs): the layers of a decode step are the uniform model's
+    bool plain_layers = pd != nullptr && !is_kquant(pd[0]);
+    for (int i = 1; i < 7 && plain_layers; i++) plain_layers = pd[i] == pd[0];
+    m->mixed_plain_layers = plain_layers;
+    m->fuse_norm = fuse_ok && (!pd || plain_layers) && gemv_norm_fusable(H);
+    m->fuse_silu = fuse_ok && (!pd || plain_layers) && gemv_silu_fusable(H);
     m->prefill_fuse_quant = fuse_ok;
     // FORGE_HIP_FUSE_SILU_GEMM=0: the gate/up GEMM writes floats and silu_mul + the quantiser run as a kernel of their own
     // (the fused epilogue uses the hardware exponential and reciprocals: same values to the fast mode's tolerance, not the same bits)
@@ -1134,6 +1139,8 @@ int32_t forge_hip_model_decode_launches(const forge_hip_model* m) {
     if (m->pd) return (int32_t)pd_launches_per_step(m->pd);
     const bool exact = (m->cfg.flags & FORGE_HIP_FLAG_EXACT) != 0;
     const int attn = exact ? 1 : 2;
+    if (m->mixed && m->mixed_plain_layers)
+        return 1 + (int)m->cfg.layers * ((m->fuse_norm ? 1 : 3) + attn + 1 + (m->fuse_silu ? 1 : 3) + 1) + 4;
     if (m->mixed) {
         // a group of projections over the same normed vector: all K-quant -> one launch that norms as well; else the norm, one
         // launch for the K-quant ones and one for each of the others
