@@ -1011,8 +1011,12 @@ int32_t forge_hip_prefill_batch(forge_hip_model* m, const uint32_t* tokens, uint
             const uint32_t rows = (uint32_t)std::min<uint64_t>(m->chunk_rows, n - fed);
             FH_HIP(hipMemcpyAsync(m->ptok.p, tokens + fed, (size_t)rows * 4, hipMemcpyHostToDevice, s));
             launch_embedding(m->embed.as<float>(), m->ptok.as<uint32_t>(), rows, m->H, m->px.as<float>(), m->counts.as<uint32_t>(), s);
+            // seven projections of one plain format, fast mode, no window (whose rule differs for these models): the uniform
+            // model's layer, with q;k;v and gate;up as one GEMM each and the fused epilogues
+            const bool uniform_rows = m->mixed_plain_layers && m->mixed_twins && m->cfg.sliding_window == 0;
             for (uint32_t l = 0; l < m->cfg.layers; l++) {
-                if (m->mixed_twins) enqueue_mixed_prefill_layer_mfma(m, l, rows, (uint32_t)(m->pos + fed));
+                if (uniform_rows) enqueue_prefill_layer(m, l, rows, (uint32_t)(m->pos + fed));
+                else if (m->mixed_twins) enqueue_mixed_prefill_layer_mfma(m, l, rows, (uint32_t)(m->pos + fed));
                 else enqueue_mixed_prefill_layer(m, l, rows, (uint32_t)(m->pos + fed));
             }
             FH_HIP(hipGetLastError());
