@@ -109,8 +109,8 @@ enum { PD_QKV = 0, PD_O = 1, PD_GU = 2, PD_DOWN = 3, PD_LM = 4, PD_V = 5 };
 //   Q4_K  codes: 16 bytes per 32-weight sub-block in Q4_0's byte order (byte i = weight i | weight i + 16 << 4), values 0..15;
 //         one word per sub-block b: fp16 bits of d (b even) or dmin (b odd) | 6-bit scale << 16 | 6-bit minimum << 24 -- the two
 //         sub-blocks of a pair belong to one super-block, so a lane gets the other half from its neighbour
-//   Q6_K  codes: the 32 weights of a block as int8 (-32..31) in order (8 bits for 6: the streaming waves are bound by the
-//         instructions per weight, not by the bytes); one word per block: the int8 scales of its two halves | fp16 bits of d << 16
+//   Q6_K  codes: the 32 weights of a block as int8 (-32..31) in order (8 bits for 6: unpacking 6-bit codes cost a phase more
+//         time than the bytes saved); one word per block: the int8 scales of its two halves | fp16 bits of d << 16
 enum { WF_Q8 = 0, WF_Q4 = 1, WF_Q4K = 2, WF_Q6K = 3 };
 __host__ __device__ constexpr bool wf_lane_per_block(int wf) { return wf == WF_Q4 || wf == WF_Q4K; }
 // The (at most two) weight formats a kernel variant FMT carries code for: 0 Q8_0, 1 Q4_0, 2 both, 3 Q4_K + Q6_K,
