@@ -199,15 +199,16 @@ def test_mixed_model_greedy_tokens_at_a_real_width(fh, oracle, torch_gpu):
     gm.close()
 
 
-@pytest.mark.parametrize("mix", ["q4_k_m", "all_four"])
+@pytest.mark.parametrize("mix", ["q4_k_m", "all_four", "kquant_lm_head_only"])
 def test_mixed_model_fast_mode(fh, oracle, torch_gpu, mix, monkeypatch):
     pd, lm = MIXES[mix]
     cfg = tiny(fh, lm, 0)
     blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=21, std=0.05)
     toks = fh.synth.uniform_ids(12, 40, cfg["vocab"])
     gm = fh.HipModel(cfg, blob, proj_dtypes=pd)
-    # all matrices Q4_K / Q6_K: one resident kernel per step; a mix with Q8_0 / Q4_0 matrices: the kernel sequence
-    assert (gm.decode_launches == 1) == (mix == "q4_k_m")
+    # all matrices Q4_K / Q6_K, or seven plain projections of one format under a Q6_K lm_head: one resident kernel per step;
+    # any other mix: the kernel sequence
+    assert (gm.decode_launches == 1) == (mix != "all_four")
     om = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
     gl, ol = gm.forward_prefill(toks), om.prefill_batched(toks)
     # layer 0's K/V rows depend on embedding -> rms_norm -> matmul -> rope only: the fast matmul's bound
