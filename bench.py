@@ -20,7 +20,8 @@ that differs, largest logit difference before that).
 kquant_model: the same shape with a storage format per projection (llama.cpp's Q4_K_M recipe, random super-blocks):
 prompt and decode throughput in fast mode (prompt on the MFMA GEMM through re-expressed matrices, decode as one resident
 kernel with K-quant weight units, the kernel sequence beside it) and in the order-faithful mode (prompt through the
-multi-row K-quant GEMV).
+multi-row K-quant GEMV); and llama.cpp's Q4_0 recipe with a K-quant output matrix (seven Q4_0 projections under a Q6_K
+lm_head) in fast mode.
 
 cpu_baseline: the CPU restatement of the reference's generated kernels (oracle/) on this host's cores, on the same
 model and prompt: in the aarch64 arithmetic (int8 activation blocks) the whole prompt as a batched prefill and
@@ -270,6 +271,20 @@ def kquant_model_figures(fh, cfg, prompt, warmup, steps, seed):
     t_edecode, tok = timed_decode(e, tok, warmup, steps)
     out["order_faithful"] = {"prefill_tok_per_s": len(prompt) / t_eprefill, "decode_tok_per_s": steps / t_edecode}
     e.close()
+    # llama.cpp's Q4_0 recipe with a K-quant output matrix: seven Q4_0 projections under a Q6_K lm_head (fast mode)
+    qcfg = dict(cfg, wdtype=2, lm_head_dtype=14)
+    qpd = (2,) * 7
+    qblob = fh.synth.make_weights_blob_mixed(qcfg, qpd, seed=seed)
+    q = fh.HipModel(qcfg, qblob, proj_dtypes=qpd)
+    q.forward_prefill(prompt)
+    q.reset()
+    t0 = time.perf_counter()
+    tok = fh.ops.argmax_host(q.forward_prefill(prompt))
+    t_qprefill = time.perf_counter() - t0
+    t_qdecode, tok = timed_decode(q, tok, warmup, steps)
+    out["q4_0_under_q6_k_lm_head"] = {"prefill_tok_per_s": len(prompt) / t_qprefill, "decode_tok_per_s": steps / t_qdecode,
+                                      "decode_launches_per_token": q.decode_launches, "weights_bytes": int(qblob.size)}
+    q.close()
     return out
 
 
