@@ -105,7 +105,7 @@ constexpr uint32_t PD_MAX_LAYERS = 34;       // per launch: the descriptors trav
 constexpr uint32_t PD_MAX_SEGMENTS = 8;
 enum { PD_QKV = 0, PD_O = 1, PD_GU = 2, PD_DOWN = 3, PD_LM = 4, PD_V = 5 };
 // Weight formats of a phase's matrix.  Q8_0 and Q6_K units hold 32 blocks (two lanes per block), Q4_0 and Q4_K units 64 (a lane per
-// block).  The K-quant matrices are re-laid out for this kernel when the model is created (pd_create_kquant):
+// block).  The K-quant matrices are re-laid out for this kernel when the model is created (pd_create):
 //   Q4_K  codes: 16 bytes per 32-weight sub-block in Q4_0's byte order (byte i = weight i | weight i + 16 << 4), values 0..15;
 //         one word per sub-block b: fp16 bits of d (b even) or dmin (b odd) | 6-bit scale << 16 | 6-bit minimum << 24 -- the two
 //         sub-blocks of a pair belong to one super-block, so a lane gets the other half from its neighbour
@@ -1761,7 +1761,7 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
         a.wf[PD_QKV] = wf_of(dqk.wdtype); a.wf[PD_O] = wf_of(in0.o->wdtype); a.wf[PD_GU] = wf_of(dgu.wdtype);
         a.wf[PD_DOWN] = wf_of(in0.down->wdtype); a.wf[PD_LM] = wf_of(lm_head.wdtype); a.wf[PD_V] = wf_of(dv.wdtype);
         a.split_v = split_v ? 1u : 0u;
-        // the layout per layer: codes [q | k | v], words [q | k | v] (a Q6_K matrix has no words), then o, gate;up, down each
+        // the layout per layer: codes [q | k | v], words [q | k | v], then o, gate;up, down each
         const size_t cq = pd_kq_code_bytes(in0.q->wdtype, QKS, H), ck = pd_kq_code_bytes(in0.k->wdtype, KV, H), cv = pd_kq_code_bytes(in0.v->wdtype, KV, H);
         const size_t wq = pd_kq_word_bytes(in0.q->wdtype, QKS, H), wk = pd_kq_word_bytes(in0.k->wdtype, KV, H), wv = pd_kq_word_bytes(in0.v->wdtype, KV, H);
         a.v_qs_off = (uint32_t)(cq + ck);
