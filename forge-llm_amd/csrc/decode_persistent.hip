@@ -556,9 +556,15 @@ __device__ __forceinline__ void pd_compute_round(const Shape& h, const TilePos& 
                     const int dh = in ? dot16(W.v[d], a, 0) : 0;      // this lane's 16 weights are one scale's
                     const uint32_t ww = W.s[d];
                     const float th = (float)((int)(ww << (24u - (lane & 1u) * 8u)) >> 24) * (float)dh;      // the int8 scale of this lane's half (two shifts: the signed bit-field builtin gave wrong values with a lane-dependent offset)
-                    const float u = th + __builtin_amdgcn_update_dpp(0.f, th, 0xB1, 0xF, 0xF, false);       // lo + hi (even lane)
-                    term = (f16_bits_to_f32((uint16_t)(ww >> 16)) * as_lds[bs]) * u;
-                    mine = in && !(lane & 1u);
+                    if (ORDERED) {
+                        const float u = th + __builtin_amdgcn_update_dpp(0.f, th, 0xB1, 0xF, 0xF, false);       // lo + hi (even lane)
+                        term = (f16_bits_to_f32((uint16_t)(ww >> 16)) * as_lds[bs]) * u;
+                        mine = in && !(lane & 1u);
+                    } else {
+                        // each lane adds its own half (the sum of the two halves is formed with the row's other terms)
+                        term = (f16_bits_to_f32((uint16_t)(ww >> 16)) * as_lds[bs]) * th;
+                        mine = in;
+                    }
                 }
                 if (ORDERED) {
                     if (mine) prod[lr * pstride + b] = term;

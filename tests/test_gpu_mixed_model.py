@@ -315,11 +315,12 @@ def test_kquant_weight_units_in_the_resident_kernel(fh, torch_gpu, monkeypatch, 
     a = seq.forward_prefill(toks)
     assert np.array_equal(a, ordered.forward_prefill(toks)) and np.array_equal(a, fast.forward_prefill(toks))
     tok = int(np.argmax(a))
-    for _ in range(30):                                     # past the window where there is one
+    for step in range(30):                                  # past the window where there is one
         x, y, z = seq.forward(tok), ordered.forward(tok), fast.forward(tok)
         same_bits(y, x)
-        # a last-bit difference in a norm can move an int8 activation code by one: quantisation noise, not rounding noise
-        assert np.corrcoef(z, x)[0, 1] > 0.999 and np.max(np.abs(z - x)) < 0.05 * max(1.0, float(np.std(x)))
+        # a last-bit difference in a norm can move an int8 activation code by one: quantisation noise, not rounding noise, and
+        # the caches of the two models drift apart by it from step to step
+        assert np.corrcoef(z, x)[0, 1] > 0.999 and np.max(np.abs(z - x)) < (0.03 if step == 0 else 0.15) * max(1.0, float(np.std(x)))
         tok = int(np.argmax(x))
     for layer in range(cfg["layers"]):
         for which in (0, 1):
