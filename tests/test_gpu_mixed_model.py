@@ -285,6 +285,7 @@ def test_mixed_model_grouped_launches_keep_the_bits(fh, torch_gpu, monkeypatch):
 
 @pytest.mark.parametrize("mix,extra", [("q4_k_m", {}), ("q6_k", {}), ("q4_k_m", dict(flags=QKV_BIAS)), ("q4_k_m", dict(sliding_window=24)),
                                        ("q4_k_m", dict(hidden=512, inter=1024, heads=4, kv_heads=4, head_dim=128)),
+                                       ("q4_k_m", dict(layers=36)), ("kquant_lm_head_only", dict(layers=35)),      # two launches per step
                                        ("kquant_lm_head_only", {}), ("q8_0_under_q6_k", dict(flags=QKV_BIAS)),
                                        ("kquant_lm_head_only", dict(sliding_window=24, hidden=512, inter=1024, heads=4, kv_heads=4, head_dim=96))])
 def test_kquant_weight_units_in_the_resident_kernel(fh, torch_gpu, monkeypatch, mix, extra):
@@ -311,7 +312,7 @@ def test_kquant_weight_units_in_the_resident_kernel(fh, torch_gpu, monkeypatch, 
     monkeypatch.setenv("FORGE_HIP_PD_ORDERED", "1")
     ordered = fh.HipModel(cfg, blob, proj_dtypes=pd)
     monkeypatch.delenv("FORGE_HIP_PD_ORDERED")
-    assert fast.decode_launches == ordered.decode_launches == 1
+    assert fast.decode_launches == ordered.decode_launches == (cfg["layers"] + 33) // 34
     a = seq.forward_prefill(toks)
     assert np.array_equal(a, ordered.forward_prefill(toks)) and np.array_equal(a, fast.forward_prefill(toks))
     tok = int(np.argmax(a))
