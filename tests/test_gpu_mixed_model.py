@@ -371,3 +371,31 @@ def test_mixed_model_refusals(fh, torch_gpu):
     with pytest.raises(fh.ForgeHipError) as e:
         fh.HipModel(cfg, blob)
     assert e.value.code == fh.ERR_INVALID
+
+
+@pytest.mark.parametrize("mix", ["q4_k_m", "kquant_lm_head_only", "all_four"])
+def test_mixed_model_on_a_paged_cache(fh, torch_gpu, mix):
+    """A model with a format per projection over a PAGED cache (pages in a shuffled order): prompt in two chunks, logits of
+    decode steps, greedy tokens and the cache rows equal the flat cache's bit for bit -- with the resident kernel (K-quant
+    weight units; plain projections under a Q6_K lm_head) and with the kernel sequence (the mix of all four formats)."""
+    pd, lm = MIXES[mix]
+    cfg = tiny(fh, lm, 0)
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=61, std=0.05)
+    toks = fh.synth.uniform_ids(62, 300, cfg["vocab"])
+    flat, paged = fh.HipModel(cfg, blob, proj_dtypes=pd), fh.HipModel(cfg, blob, proj_dtypes=pd)
+    page_rows = 64
+    table = np.random.default_rng(9).permutation(cfg["max_seq"] // page_rows).astype(np.uint32)
+    paged.set_kv_pages(page_rows, table)
+    for m in (flat, paged):
+        m.forward_prefill_batch(toks[:150])
+    same_bits(paged.forward_prefill(toks[150:280]), flat.forward_prefill(toks[150:280]))
+    for t in toks[280:290]:
+        same_bits(paged.forward(int(t)), flat.forward(int(t)))
+    a = b = int(toks[290])
+    for _ in range(8):
+        a, b = paged.forward_greedy(a), flat.forward_greedy(b)
+        assert a == b
+    for layer in range(cfg["layers"]):
+        for which in (0, 1):
+            assert np.array_equal(paged.read_kv(layer, which), flat.read_kv(layer, which))
+    flat.close(); paged.close()
