@@ -329,6 +329,11 @@ def test_kquant_weight_units_in_the_resident_kernel(fh, torch_gpu, monkeypatch, 
     # greedy decoding on the device, and a reset
     seq.reset(); ordered.reset()
     assert ordered.generate_greedy(toks[:9], 12) == seq.generate_greedy(toks[:9], 12)
+    # the repeat penalty on the device (the lm_head phase's epilogue; the sequence's argmax kernel)
+    seq.reset(); ordered.reset()
+    seq.set_repeat_penalty(1.3); ordered.set_repeat_penalty(1.3)
+    pa, pb = seq.generate_greedy(toks[:9], 16), ordered.generate_greedy(toks[:9], 16)
+    assert pa == pb
     seq.close(); ordered.close(); fast.close()
 
 
