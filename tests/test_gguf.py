@@ -1016,3 +1016,18 @@ def test_q4_k_m_model_from_gguf_matches_the_oracle(fh, gg, go, oracle, torch_gpu
         tok = oracle.argmax(w)
     assert np.array_equal(oracle.f16_to_f32(gm.read_kv(3, 1)), om.read_kv(3, 1))
     gm.close()
+    # the same file in fast mode: one resident kernel per decode step, the model built from the oracle's export of the file
+    # gives the same bits (same kernels on the same planes), and the logits stay near the order-faithful ones
+    fm = fh.HipModel.from_gguf(path)
+    assert fm.decode_launches == 1
+    fcfg = dict(cfg, flags=0)
+    bm = fh.HipModel(fcfg, blob, proj_dtypes=pd)
+    fl = fm.forward_prefill(prompt)
+    assert np.array_equal(fl, bm.forward_prefill(prompt))
+    assert np.corrcoef(fl, ol)[0, 1] > 0.995
+    t = int(np.argmax(fl))
+    for _ in range(6):
+        a, b = fm.forward(t), bm.forward(t)
+        assert np.array_equal(a, b)
+        t = int(np.argmax(a))
+    fm.close(); bm.close()
