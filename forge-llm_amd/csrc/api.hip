@@ -39,14 +39,26 @@ void qweight_free(QWeight* w) {
 
 namespace {
 
+// One area per device (the process may drive several): it grows when a call needs more than any earlier call on that device,
+// in steps of at least half its size again, so that a run of growing shapes re-allocates a few times and not at every call.
 struct Scratch {
-    void* p = nullptr;
-    size_t cap = 0;
+    static constexpr int MAX_DEVICES = 16;
+    void* area[MAX_DEVICES] = {};
+    size_t cap[MAX_DEVICES] = {};
+    static int device() {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) dev = 0;
+        return dev;
+    }
+    void* ptr() const { return area[device()]; }
+    size_t capacity() const { return cap[device()]; }
     int32_t reserve(size_t n) {
-        if (n <= cap) return FORGE_HIP_OK;
-        if (p) { FH_HIP(hipFree(p)); p = nullptr; cap = 0; }
-        FH_HIP(hipMalloc(&p, n));
-        cap = n;
+        const int d = device();
+        if (n <= cap[d]) return FORGE_HIP_OK;
+        const size_t want = std::max(n, cap[d] + cap[d] / 2);
+        if (area[d]) { FH_HIP(hipFree(area[d])); area[d] = nullptr; cap[d] = 0; }      // waits for the device
+        FH_HIP(hipMalloc(&area[d], want));
+        cap[d] = want;
         return FORGE_HIP_OK;
     }
 };
@@ -66,8 +78,8 @@ int32_t quantise_into_scratch(const float* x, uint32_t M, uint32_t K, int8_t** q
     const size_t sbytes = (size_t)M * (K / 32) * 2;
     int32_t rc = g_act.reserve(qbytes + sbytes);
     if (rc) return rc;
-    *q = reinterpret_cast<int8_t*>(g_act.p);
-    *sc = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(g_act.p) + qbytes);
+    *q = reinterpret_cast<int8_t*>(g_act.ptr());
+    *sc = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(g_act.ptr()) + qbytes);
     launch_quantize_act(x, M, K, *q, *sc, s, neg_odd);
     return FORGE_HIP_OK;
 }
@@ -188,21 +200,21 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
         if (rck) return rck;
         void* split_ws = nullptr;
         if (M > 64) {
-            const bool fresh = g_gemm.cap < gemm_split_workspace_bytes();
+            const bool fresh = g_gemm.capacity() < gemm_split_workspace_bytes();
             if ((rck = g_gemm.reserve(gemm_split_workspace_bytes()))) return rck;
-            if (fresh) FH_HIP(hipMemsetAsync(g_gemm.p, 0, gemm_split_workspace_bytes(), s));
-            split_ws = g_gemm.p;
+            if (fresh) FH_HIP(hipMemsetAsync(g_gemm.ptr(), 0, gemm_split_workspace_bytes(), s));
+            split_ws = g_gemm.ptr();
         }
         if (h->twin.coef) {
             if ((rck = g_twin.reserve((size_t)M * (K / 32) * 4))) return rck;
-            launch_act_block_sums(q, sc, M, K, true, reinterpret_cast<float*>(g_twin.p), s);
+            launch_act_block_sums(q, sc, M, K, true, reinterpret_cast<float*>(g_twin.ptr()), s);
             launch_gemm(h->twin.w, q, sc, M, y_dev, w->w.N, false, false, nullptr, s, split_ws, nullptr, nullptr,
-                        reinterpret_cast<const float*>(g_twin.p), h->twin.coef);
+                        reinterpret_cast<const float*>(g_twin.ptr()), h->twin.coef);
         } else {
             const size_t qbytes = align256((size_t)M * K * 2);
             if ((rck = g_twin.reserve(qbytes + (size_t)M * (K / 32) * 4))) return rck;
-            int8_t* q2 = reinterpret_cast<int8_t*>(g_twin.p);
-            uint16_t* sc2 = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(g_twin.p) + qbytes);
+            int8_t* q2 = reinterpret_cast<int8_t*>(g_twin.ptr());
+            uint16_t* sc2 = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(g_twin.ptr()) + qbytes);
             launch_act_twice(q, sc, M, K, q2, sc2, s);
             launch_gemm(h->twin.w, q2, sc2, M, y_dev, w->w.N, false, false, nullptr, s, split_ws);
         }
@@ -214,13 +226,13 @@ int32_t forge_hip_gemm_q(const forge_hip_qweight* w, const float* x_dev, uint32_
     // fast mode may cut tiles along K to fill the CUs: that kernel parks partial tiles in a workspace
     void* split_ws = nullptr;
     if (!exact && M > 64) {
-        const bool fresh = g_gemm.cap < gemm_split_workspace_bytes();
+        const bool fresh = g_gemm.capacity() < gemm_split_workspace_bytes();
         if ((rc = g_gemm.reserve(gemm_split_workspace_bytes()))) return rc;
         // its counters start at zero and are left at zero; cleared on the caller's stream, so that the clear is ordered
         // before the kernel whatever kind of stream that is (a null-stream memset does not wait for, and is not waited
         // for by, a non-blocking stream)
-        if (fresh) FH_HIP(hipMemsetAsync(g_gemm.p, 0, gemm_split_workspace_bytes(), (hipStream_t)stream));
-        split_ws = g_gemm.p;
+        if (fresh) FH_HIP(hipMemsetAsync(g_gemm.ptr(), 0, gemm_split_workspace_bytes(), (hipStream_t)stream));
+        split_ws = g_gemm.ptr();
     }
     launch_gemm(w->w, q, sc, M, y_dev, w->w.N, false, exact, nullptr, (hipStream_t)stream, split_ws);
     FH_HIP(hipGetLastError());
@@ -239,10 +251,10 @@ int32_t forge_hip_gemm_silu_q(const forge_hip_qweight* w, const float* x_dev, ui
     if (rc) return rc;
     void* split_ws = nullptr;
     if (M > 64) {
-        const bool fresh = g_gemm.cap < gemm_split_workspace_bytes();
+        const bool fresh = g_gemm.capacity() < gemm_split_workspace_bytes();
         if ((rc = g_gemm.reserve(gemm_split_workspace_bytes()))) return rc;
-        if (fresh) FH_HIP(hipMemsetAsync(g_gemm.p, 0, gemm_split_workspace_bytes(), (hipStream_t)stream));
-        split_ws = g_gemm.p;
+        if (fresh) FH_HIP(hipMemsetAsync(g_gemm.ptr(), 0, gemm_split_workspace_bytes(), (hipStream_t)stream));
+        split_ws = g_gemm.ptr();
     }
     launch_gemm(w->w, q, sc, M, nullptr, w->w.N, false, false, nullptr, (hipStream_t)stream, split_ws, out_q_dev, out_scales_dev);
     FH_HIP(hipGetLastError());
@@ -277,7 +289,7 @@ int32_t forge_hip_block_isums(const forge_hip_qweight* w, const float* x_dev, ui
         Scratch& sink = g_attn;
         rc = sink.reserve((size_t)M * w->w.N * sizeof(float));
         if (rc) return rc;
-        launch_gemm(w->w, q, sc, M, reinterpret_cast<float*>(sink.p), w->w.N, false, path == 1, out_dev, (hipStream_t)stream);
+        launch_gemm(w->w, q, sc, M, reinterpret_cast<float*>(sink.ptr()), w->w.N, false, path == 1, out_dev, (hipStream_t)stream);
     }
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
@@ -319,9 +331,9 @@ int32_t forge_hip_rope_kv_store(float* q_dev, float* k_dev, const float* v_dev, 
     }
     int32_t rc = g_rope.reserve(tab.size() * sizeof(float));
     if (rc) return rc;
-    FH_HIP(hipMemcpyAsync(g_rope.p, tab.data(), tab.size() * sizeof(float), hipMemcpyHostToDevice, (hipStream_t)stream));
+    FH_HIP(hipMemcpyAsync(g_rope.ptr(), tab.data(), tab.size() * sizeof(float), hipMemcpyHostToDevice, (hipStream_t)stream));
     FH_HIP(hipStreamSynchronize((hipStream_t)stream));   // `tab` is pageable and about to go out of scope
-    const float* cos_t = reinterpret_cast<const float*>(g_rope.p);
+    const float* cos_t = reinterpret_cast<const float*>(g_rope.ptr());
     const float* sin_t = cos_t + (size_t)n_pos * half;
     launch_rope_kv_store(q_dev, k_dev, v_dev, heads * head_dim, kv_heads * head_dim, k_cache_dev, v_cache_dev, M,
                          base_pos, nullptr, heads, kv_heads, head_dim, cos_t, sin_t, nullptr, (hipStream_t)stream);
@@ -387,13 +399,13 @@ int32_t forge_hip_attn_decode_f16kv(const float* q_dev, const uint16_t* k_cache_
             if (rc) return rc;
         }
         launch_attn_exact(false, q_dev, heads * head_dim, k_cache_dev, v_cache_dev, out_dev, heads * head_dim, nullptr,
-                          nullptr, 1, seq_len - 1, nullptr, heads, kv_heads, head_dim, 0u, seq_len, xb ? g_attn.p : nullptr,
+                          nullptr, 1, seq_len - 1, nullptr, heads, kv_heads, head_dim, 0u, seq_len, xb ? g_attn.ptr() : nullptr,
                           (hipStream_t)stream);
     } else {
         rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
         if (rc) return rc;
         launch_attn_decode(q_dev, k_cache_dev, v_cache_dev, out_dev, nullptr, nullptr, seq_len, nullptr, heads, kv_heads,
-                           head_dim, 0u, g_attn.p, (hipStream_t)stream);
+                           head_dim, 0u, g_attn.ptr(), (hipStream_t)stream);
     }
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
@@ -411,7 +423,7 @@ int32_t forge_hip_attn_decode_f16kv_paged(const float* q_dev, const uint16_t* k_
     rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
     if (rc) return rc;
     launch_attn_decode_paged(q_dev, k_pool_dev, v_pool_dev, page_table_dev, page_rows, out_dev, seq_len, heads, kv_heads, head_dim,
-                             g_attn.p, (hipStream_t)stream);
+                             g_attn.ptr(), (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }
@@ -433,7 +445,7 @@ int32_t forge_hip_attn_decode_sliding_f16kv(const float* q_dev, const uint16_t* 
         rc = g_attn.reserve(attn_decode_workspace_bytes(heads, head_dim));
         if (rc) return rc;
         launch_attn_decode(q_dev, k_cache_dev, v_cache_dev, out_dev, nullptr, nullptr, seq_len, nullptr, heads, kv_heads, head_dim,
-                           window, g_attn.p, (hipStream_t)stream);
+                           window, g_attn.ptr(), (hipStream_t)stream);
     }
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
@@ -449,7 +461,7 @@ int32_t forge_hip_argmax(const float* x_dev, uint32_t n, uint32_t* out_dev, void
     FH_CHECK(x_dev && out_dev && n >= 1, "argmax: null pointer or empty input");
     int32_t rc = g_attn.reserve(ARGMAX_BLOCKS * 8);
     if (rc) return rc;
-    launch_argmax(x_dev, n, out_dev, g_attn.p, nullptr, nullptr, nullptr, 1.0f, (hipStream_t)stream);
+    launch_argmax(x_dev, n, out_dev, g_attn.ptr(), nullptr, nullptr, nullptr, 1.0f, (hipStream_t)stream);
     FH_HIP(hipGetLastError());
     return FORGE_HIP_OK;
 }

@@ -34,12 +34,12 @@
  *  - A model allocates all its device buffers in forge_hip_model_create (weights, KV cache for max_seq,
  *    activations for one prefill chunk); later calls allocate no device memory (the kernel-sequence
  *    decode path instantiates its HIP graph at the first decode step).
- *  - The op-level calls keep four process-wide scratch areas (quantised activations, attention / argmax
- *    partial results, RoPE tables, 16 MB of partial GEMM tiles) that GROW ON DEMAND: a call that needs more than any earlier call
- *    did frees the old area, which waits for the device, and allocates a larger one (hipFree +
- *    hipMalloc on the call path).  They are shared by all streams and not locked: use the
- *    op-level API from one thread and one stream at a time, and call the largest shape once at start-up
- *    if the allocation must not happen later.  forge_hip_attn_decode_f16kv_noalloc is the one op-level
+ *  - The op-level calls keep a few scratch areas per device (quantised activations, attention / argmax
+ *    partial results, RoPE tables, 16 MB of partial GEMM tiles, K-quant operands) that GROW ON DEMAND: a call that needs more
+ *    than any earlier call on that device did frees the old area, which waits for the device, and allocates one at least half
+ *    as large again (hipFree + hipMalloc on the call path, a few times over a run of growing shapes).  They are shared by
+ *    all streams of a device and not locked: use the op-level API from one thread and one stream per device at a time, and call
+ *    the largest shape once at start-up if the allocation must not happen later.  forge_hip_attn_decode_f16kv_noalloc is the one op-level
  *    call that never allocates.
  *  - The one-kernel decode step (forge_hip_model_decode_launches() == 1) runs one workgroup per compute
  *    unit and its workgroups wait on each other's results, so all of them must be resident at once:
