@@ -1639,8 +1639,8 @@ bool plan_gemv(const QWeight& w, uint32_t inter, uint32_t nseg, const Segment* s
 
 template <int HD, bool ORD, bool PEN, bool XA>
 const void* pd_kernel_ord(const PdState* st) {
-    // (K-quant models always run the variant with the optional extras, and never the reference-order attention)
-    if (st->kquant) return reinterpret_cast<const void*>(decode_step_kernel<HD, 3, ORD, true, false>);
+    // (K-quant models always run the variant with the optional extras)
+    if (st->kquant) return reinterpret_cast<const void*>(decode_step_kernel<HD, 3, ORD, true, XA>);
     if (st->lmk) return st->q4 ? reinterpret_cast<const void*>(decode_step_kernel<HD, 4, ORD, true, false>)
                                : reinterpret_cast<const void*>(decode_step_kernel<HD, 5, ORD, true, false>);
     if (st->q4 != st->lmq4) return reinterpret_cast<const void*>(decode_step_kernel<HD, 2, ORD, PEN, XA>);
@@ -1681,13 +1681,19 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     // The order-faithful mode can run as this kernel too: the ordered variant with the attention phases in the reference's
     // order.  It is bit-identical to the kernel sequence but not faster across shapes (Llama-3.2-1B shape at 2.5k context:
     // 925 against 935 us per token; 3B: 2125 against 2118; SmolLM2-135M: 1204 against 1041 -- the ordered norm and row sums
-    // cost every GEMV phase 1-2 us that the separate kernels hide behind their launches), so the sequence stays the default and
-    // FORGE_HIP_PD_EXACT=1 asks for the kernel.  A window (attention_sliding: another algorithm) and caches of more than
-    // 4096 blocks always keep the sequence.
+    // cost every GEMV phase 1-2 us that the separate kernels hide behind their launches), so for Q8_0 / Q4_0 models the sequence
+    // stays the default and FORGE_HIP_PD_EXACT=1 asks for the kernel.  Models of K-quant matrices, whose sequence has a launch
+    // per projection group (117 per token at 16 layers), take the kernel by default (Q4_K_M recipe, 1B shape: 928 against 989
+    // us per token); FORGE_HIP_PD_EXACT=0 keeps their sequence.  A window (attention_sliding: another algorithm) and caches of
+    // more than 4096 blocks always keep the sequence.
     const bool exact = (c.flags & FORGE_HIP_FLAG_EXACT) != 0;
     const uint32_t nb_cap = (c.max_seq + PX_B - 1) / PX_B;
     if (exact && (c.sliding_window != 0 || nb_cap > PX_MAX_BLOCKS)) return FORGE_HIP_OK;
-    { const char* e = getenv("FORGE_HIP_PD_EXACT"); if (exact && !(e && e[0] == '1')) return FORGE_HIP_OK; }
+    if (exact) {
+        const char* e = getenv("FORGE_HIP_PD_EXACT");
+        const bool kquant_model = !layers.empty() && layers[0].q != nullptr;
+        if (!(e ? e[0] == '1' : kquant_model)) return FORGE_HIP_OK;
+    }
     if (c.head_dim != 64 && c.head_dim != 96 && c.head_dim != 128) return FORGE_HIP_OK;
     int dev = 0, coop = 0, cus = 0, khz = 0;
     FH_HIP(hipGetDevice(&dev));
@@ -1741,7 +1747,6 @@ int32_t pd_create(const forge_hip_config& c, const std::vector<PdLayerIn>& layer
     if (layers.empty() || layers.size() > PD_MAX_LAYERS * PD_MAX_SEGMENTS) return FORGE_HIP_OK;
     QWeight lm_res = lm_head;                     // K-quant models: the lm_head in the kernel's layout
     if (st->kquant) {
-        if (exact) return FORGE_HIP_OK;           // order-faithful K-quant models keep the kernel sequence
         const PdLayerIn& in0 = layers[0];
         // descriptors of the matrices as the kernel sees them: q;k (with v behind it when v shares their format), o, gate;up, down
         const bool split_v = in0.v->wdtype != in0.q->wdtype;

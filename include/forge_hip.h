@@ -130,11 +130,12 @@ int32_t forge_hip_model_create(const forge_hip_config* cfg, const uint8_t* weigh
  * projections are K-quants (multi-row K-quant GEMV: every row has the one-row kernel's bits, so logits, cache and tokens are
  * the token-by-token walk's), otherwise token by token; without the flag always, on the int8 MFMA GEMM (K-quant matrices
  * through re-expressions built at create time, see forge_hip_gemm_q: the device then holds both forms of those matrices).
- * Decode: a model whose seven projections and lm_head are all Q4_K / Q6_K (q and k of one format, gate and up too), without
- * FORGE_HIP_FLAG_EXACT, runs the step as one resident kernel over a third form of the matrices built at create time (K-quant
- * weight units: 5 bits per weight for Q4_K, 9 for Q6_K; FORGE_HIP_PD_KQUANT=0 in the environment keeps the kernel
- * sequence), and so does a model of seven Q8_0 or seven Q4_0 projections under a Q6_K lm_head (the uniform model's kernel with
- * the lm_head as weight units); any other mix runs the kernel sequence (K-quant projections over the same normed row share a launch), captured
+ * Decode: a model whose seven projections and lm_head are all Q4_K / Q6_K (q and k of one format, gate and up too) runs the
+ * step as one resident kernel over a third form of the matrices built at create time (K-quant weight units: 5 bits per weight
+ * for Q4_K, 9 for Q6_K; FORGE_HIP_PD_KQUANT=0 in the environment keeps the kernel sequence) -- with FORGE_HIP_FLAG_EXACT in the
+ * kernel's order-faithful variant, bit for bit the sequence (FORGE_HIP_PD_EXACT=0 keeps the sequence; a sliding window always
+ * does) -- and so does, without the flag, a model of seven Q8_0 or seven Q4_0 projections under a Q6_K lm_head (the uniform
+ * model's kernel with the lm_head as weight units); any other mix runs the kernel sequence (K-quant projections over the same normed row share a launch), captured
  * in a graph.  K-quant matrices need an input width that is a multiple of 256.
  * FORGE_HIP_FLAG_QKV_BIAS works as in forge_hip_model_create (the bias vectors follow the v weights of every layer,
  * project.rs:286-292).  A sliding window follows the reference's rule for such models: the rows of a prompt see ALL earlier

@@ -265,6 +265,7 @@ def test_mixed_model_grouped_launches_keep_the_bits(fh, torch_gpu, monkeypatch):
     """K-quant projections that read the same normed row (q, k, v; gate, up) go out as ONE launch that norms and quantises
     the row itself; FORGE_HIP_MIXED_FUSE=0 keeps the norm kernel in front.  Same logits and cache rows bit for bit, fewer
     launches per step.  A mix with a Q8_0 matrix in the group keeps the norm kernel for it."""
+    monkeypatch.setenv("FORGE_HIP_PD_EXACT", "0")            # the kernel sequence (all-K-quant models default to the resident kernel)
     for mix, fewer in (("q4_k_m", True), ("all_four", False)):
         pd, lm = MIXES[mix]
         cfg = tiny(fh, lm, EXACT)
@@ -404,3 +405,34 @@ def test_mixed_model_on_a_paged_cache(fh, torch_gpu, mix):
         for which in (0, 1):
             assert np.array_equal(paged.read_kv(layer, which), flat.read_kv(layer, which))
     flat.close(); paged.close()
+
+
+@pytest.mark.parametrize("mix", ["q4_k_m", "q6_k"])
+def test_order_faithful_kquant_model_on_the_resident_kernel(fh, oracle, torch_gpu, monkeypatch, mix):
+    """The order-faithful decode step of an all-K-quant model is ONE resident kernel (ordered row sums, the attention walked in
+    the reference's 64-key blocks; FORGE_HIP_PD_EXACT=0: the kernel sequence): prompt, 16 greedy steps and the cache rows of
+    both bit for bit the CPU oracle's."""
+    pd, lm = MIXES[mix]
+    cfg = tiny(fh, lm, EXACT)
+    blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=77, std=0.05)
+    toks = fh.synth.uniform_ids(78, 70, cfg["vocab"])
+    monkeypatch.setenv("FORGE_HIP_PD_EXACT", "0")
+    seq = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    assert seq.decode_launches > 1
+    monkeypatch.delenv("FORGE_HIP_PD_EXACT")
+    one = fh.HipModel(cfg, blob, proj_dtypes=pd)
+    assert one.decode_launches == 1
+    om = oracle.Model(cfg, blob, A, KV_F16, proj_dtypes=pd)
+    ol = om.prefill_batched(toks)
+    same_bits(one.forward_prefill(toks), ol)
+    same_bits(seq.forward_prefill(toks), ol)
+    tok = oracle.argmax(ol)
+    for _ in range(16):
+        w = om.forward(tok)
+        same_bits(one.forward(tok), w)
+        same_bits(seq.forward(tok), w)
+        tok = oracle.argmax(w)
+    for layer in range(cfg["layers"]):
+        for which in (0, 1):
+            assert np.array_equal(one.read_kv(layer, which), seq.read_kv(layer, which))
+    seq.close(); one.close()
