@@ -249,18 +249,23 @@ def test_llama_3b_full_size_resident_kernel_equals_kernel_sequence(fh, torch_gpu
 
 
 @pytest.mark.timeout(600)
-@pytest.mark.parametrize("name,pd,lm", [("q4_k_m", (12, 12, 14, 12, 12, 12, 14), 14), ("q4_0_under_q6_k", (2,) * 7, 14)])
+@pytest.mark.parametrize("name,pd,lm", [("q4_k_m", (12, 12, 14, 12, 12, 12, 14), 14), ("q4_0_under_q6_k", (2,) * 7, 14),
+                                        ("q4_k_m_order_faithful", (12, 12, 14, 12, 12, 12, 14), 14)])
 def test_llama_1b_shape_kquant_resident_kernel_equals_kernel_sequence(fh, torch_gpu, monkeypatch, name, pd, lm):
     """The Llama-3.2-1B shape with llama.cpp's Q4_K_M recipe (Q4_K q/k/o/gate/up, Q6_K v/down/lm_head: the v matrix shares the
     q;k;v phase on its own share of the 256 workgroups) and with seven Q4_0 projections under a Q6_K lm_head: after the same
     700-token prompt, 300 greedy steps of the one-kernel decode step (summing in the reference order) and of the kernel
-    sequence give the same tokens, the same logits and the same cache, bit for bit."""
+    sequence give the same tokens, the same logits and the same cache, bit for bit.  Third case: the order-faithful mode of the
+    Q4_K_M recipe, whose default is the kernel with the reference-order attention."""
     cfg = fh.synth.llama32_1b(Q4 if pd[0] == Q4 else Q8, max_seq=2048)
     cfg["lm_head_dtype"] = lm
+    exact = name.endswith("order_faithful")
+    if exact:
+        cfg["flags"] = EXACT
     blob = fh.synth.make_weights_blob_mixed(cfg, pd, seed=5)
-    monkeypatch.setenv("FORGE_HIP_PD_KQUANT", "0")
+    monkeypatch.setenv("FORGE_HIP_PD_EXACT" if exact else "FORGE_HIP_PD_KQUANT", "0")
     seq = fh.HipModel(cfg, blob, proj_dtypes=pd)
-    monkeypatch.delenv("FORGE_HIP_PD_KQUANT")
+    monkeypatch.delenv("FORGE_HIP_PD_EXACT" if exact else "FORGE_HIP_PD_KQUANT")
     monkeypatch.setenv("FORGE_HIP_PD_ORDERED", "1")
     one = fh.HipModel(cfg, blob, proj_dtypes=pd)
     monkeypatch.delenv("FORGE_HIP_PD_ORDERED")
