@@ -20,7 +20,7 @@ that differs, largest logit difference before that).
 kquant_model: the same shape with a storage format per projection (llama.cpp's Q4_K_M recipe, random super-blocks):
 prompt and decode throughput in fast mode (prompt on the MFMA GEMM through re-expressed matrices, decode as one resident
 kernel with K-quant weight units, the kernel sequence beside it) and in the order-faithful mode (prompt through the
-multi-row K-quant GEMV); and llama.cpp's Q4_0 recipe with a K-quant output matrix (seven Q4_0 projections under a Q6_K
+multi-row K-quant GEMV, decode as the resident kernel's ordered variant); and llama.cpp's Q4_0 recipe with a K-quant output matrix (seven Q4_0 projections under a Q6_K
 lm_head) in fast mode.
 
 cpu_baseline: the CPU restatement of the reference's generated kernels (oracle/) on this host's cores, on the same
