@@ -167,7 +167,7 @@ void launch_gemv_kquant_multi_norm(const QWeight* const* w, float* const* y, uin
 // Q6_K as the hi and lo parts of sc * q, two blocks per block (depth 2K), under the exact scales 64 d and d.
 struct KqTwin {
     QWeight w;                 // Q8_0 layout, [N][K] (Q4_K) or [N][2K] (Q6_K)
-    float* coef = nullptr;     // Q4_K: [N][K/32], 8 * d * sc - dmin * min
+    float* coef = nullptr;     // Q4_K: [N][K/32] slots, (8 * d * sc - dmin * min) * 2^8 as a hi | lo pair of fp16 numbers
     bool present() const { return w.qs != nullptr; }
 };
 int32_t kquant_twin_create(const QWeight* const* ws, uint32_t n, KqTwin* out, bool* covered, hipStream_t s);
@@ -192,8 +192,9 @@ size_t gemm_split_workspace_bytes();
 // the launch writes quantize(silu(gate) * up) for the down projection: codes [M][N / 2] with odd blocks negated and fp16
 // scales [M][N / 64] (silu_mul emit.rs:380-386 with the hardware exponential, quantiser emit.rs:1410-1440).
 bool gemm_silu_supported(const QWeight& w, uint32_t inter, uint32_t M);
-// mt_a / mt_w (fast mode, Q8_0-layout matrices, no isums): f32 [M][K/32] and [N][K/32]; every element of the result
-// additionally receives sum_b mt_a[m][b] * mt_w[n][b] (before the SiLU epilogue, if any).
+// mt_a / mt_w (fast mode, Q8_0-layout matrices, no isums): [M][K/32] and [N][K/32] slots of 4 bytes, each a hi | lo pair of
+// fp16 numbers (launch_act_block_sums, kquant_twin_create write them); every element of the result additionally receives
+// sum_b mt_a[m][b] * mt_w[n][b] (before the SiLU epilogue, if any).
 void launch_gemm(const QWeight& w, const int8_t* aq, const uint16_t* as, uint32_t M, float* y, uint32_t ldy,
                  bool accumulate, bool exact, int32_t* isums, hipStream_t s, void* split_ws = nullptr, int8_t* silu_q = nullptr,
                  uint16_t* silu_sc = nullptr, const float* mt_a = nullptr, const float* mt_w = nullptr);

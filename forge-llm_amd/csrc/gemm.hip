@@ -94,12 +94,12 @@ struct GemmSplit {
     int8_t* silu_q;         // SILU: [M][inter] codes (odd blocks negated, as the fast GEMM takes its activations)
     uint16_t* silu_sc;      // SILU: [M][inter / 32] fp16 scales
     uint32_t inter;
-    const float* mt_a;      // MINT: [M][K / 32] f32, one value per activation block
-    const float* mt_w;      // MINT: [N][K / 32] f32, one value per weight block
+    const float* mt_a;      // MINT: [M][K / 32] slots of 4 bytes (a hi | lo pair of fp16 numbers), one per activation block
+    const float* mt_w;      // MINT: [N][K / 32] slots likewise, one per weight block
 };
 
-// MINT: the tile additionally receives sum_b mt_a[m][b] * mt_w[n][b], an f32 matmul of depth K / 32 on the matrix unit in
-// front of the epilogue (the minimum term of a Q4_K matrix: activation block sums times a coefficient per weight block,
+// MINT: the tile additionally receives sum_b mt_a[m][b] * mt_w[n][b], a matmul of depth K / 32 on the f16 matrix unit (operands
+// as hi | lo pairs of fp16 numbers) in front of the epilogue (the minimum term of a Q4_K matrix: activation block sums times a coefficient per weight block,
 // kquant_prefill.hip) -- so that it costs no pass over the result and may precede the SiLU epilogue.
 template <bool Q4, bool DUMP, bool EXACT, int TM, bool SPLIT = false, bool SILU = false, bool MINT = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2)))
@@ -462,31 +462,74 @@ void gemm_q_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
     }
 
     if (MINT) {
-        // A: lane = (row lrow of the tile, k = lhalf), B: lane = (column lrow, k = lhalf), v_mfma_f32_32x32x2_f32; a lane fetches
-        // four consecutive b per operand (the order of k inside a sum is free), so eight b pass through four MFMAs.  The
-        // result tile has the accumulators' layout.
-        typedef float v16f32 __attribute__((ext_vector_type(16)));
+        // On the f16 matrix unit, sixteen b per step: every operand arrives as a hi | lo pair of fp16 numbers in a 4-byte slot
+        // (kquant_prefill.hip: hi = fp16(x), lo = fp16(x - hi), x scaled by a power of two that cancels between the sides) and the
+        // three products hi*hi + hi*lo + lo*hi carry it to 2^-22 relative -- a sixteenth of the f32 MFMA's time, which for
+        // K = 2048 was as long as the tile's whole int8 loop.
+        // A: lane = (row lrow of the tile, b = 8 lhalf .. + 8 of each group of sixteen), B: lane = (column lrow, the same b).
+        auto split = [](const float4& x0, const float4& x1, v8h& hi, v8h& lo) {
+            const uint32_t p[8] = {__float_as_uint(x0.x), __float_as_uint(x0.y), __float_as_uint(x0.z), __float_as_uint(x0.w),
+                                   __float_as_uint(x1.x), __float_as_uint(x1.y), __float_as_uint(x1.z), __float_as_uint(x1.w)};
+            uint32_t h[4], l[4];
 #pragma unroll
-        for (int tm = 0; tm < TM; tm++)
+            for (int i = 0; i < 4; i++) {
+                h[i] = __builtin_amdgcn_perm(p[2 * i + 1], p[2 * i], 0x05040100u);      // the two low halves
+                l[i] = __builtin_amdgcn_perm(p[2 * i + 1], p[2 * i], 0x07060302u);      // the two high halves
+            }
+            hi = __builtin_bit_cast(v8h, make_uint4(h[0], h[1], h[2], h[3]));
+            lo = __builtin_bit_cast(v8h, make_uint4(l[0], l[1], l[2], l[3]));
+        };
+        // The operand rows (256 bytes per 64 blocks) come through LDS, which the main loop no longer needs: a lane that fetched its
+        // own row from memory touched one cache line per lane and load, and the term cost as much as a third of the tile.
+        // Chunks of 64 blocks; rows 272 bytes apart (a row's 32-byte fragments of neighbouring rows on different banks).
+        constexpr uint32_t MT_ROW = 272, MT_B = 128 * MT_ROW;          // the B rows start behind 128 A rows
+        static_assert(2 * 128 * 272 <= GEMM_LDS_BYTES, "the minimum term's operand rows fit the kernel's LDS");
+        for (uint32_t b0 = 0; b0 < nblk; b0 += 64) {
+            const uint32_t nb = min(64u, nblk - b0);                   // a multiple of 8
+            __syncthreads();                                           // the previous chunk (or the main loop) is done with LDS
+            // thread: 16-byte piece (tid % 16) of rows tid / 16, + 16, ...
+            const uint32_t piece = tid & 15, r0 = tid >> 4;
+            if (piece * 4 < nb) {
 #pragma unroll
-            for (int tn = 0; tn < 2; tn++) {
-                const uint32_t mrow = min(m0 + wm * WM + tm * 32 + lrow, M - 1);
-                const uint32_t nrow = SILU ? si0 + 32 * wn + lrow + tn * s_inter : min(n0 + wn * 64 + tn * 32 + lrow, N - 1);
-                const float* ap = sp.mt_a + (size_t)mrow * nblk + 4 * lhalf;
-                const float* bp = sp.mt_w + (size_t)nrow * nblk + 4 * lhalf;
-                v16f32 c;
-#pragma unroll
-                for (int r = 0; r < 16; r++) c[r] = acc[tm][tn][r];
-                for (uint32_t g = 0; g < nblk; g += 8) {
-                    const float4 a = *reinterpret_cast<const float4*>(ap + g), b = *reinterpret_cast<const float4*>(bp + g);
-                    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, b.x, c, 0, 0, 0);
-                    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, b.y, c, 0, 0, 0);
-                    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, b.z, c, 0, 0, 0);
-                    c = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, b.w, c, 0, 0, 0);
+                for (uint32_t r = r0; r < 2 * WM; r += 16) {
+                    const uint32_t mrow = min(m0 + r, M - 1);
+                    *reinterpret_cast<float4*>(lds + r * MT_ROW + piece * 16) = *reinterpret_cast<const float4*>(sp.mt_a + (size_t)mrow * nblk + b0 + piece * 4);
                 }
 #pragma unroll
-                for (int r = 0; r < 16; r++) acc[tm][tn][r] = c[r];
+                for (uint32_t c = r0; c < 128; c += 16) {
+                    const uint32_t cwn = c >> 6, ctn = (c >> 5) & 1, clr = c & 31;
+                    const uint32_t nrow = SILU ? si0 + 32 * cwn + clr + ctn * s_inter : min(n0 + c, N - 1);
+                    *reinterpret_cast<float4*>(lds + MT_B + c * MT_ROW + piece * 16) = *reinterpret_cast<const float4*>(sp.mt_w + (size_t)nrow * nblk + b0 + piece * 4);
+                }
             }
+            __syncthreads();
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int tn = 0; tn < 2; tn++) {
+                    const uint8_t* ap = lds + (wm * WM + tm * 32 + lrow) * MT_ROW + lhalf * 32;
+                    const uint8_t* bp = lds + MT_B + (wn * 64 + tn * 32 + lrow) * MT_ROW + lhalf * 32;
+                    v16f c;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) c[r] = acc[tm][tn][r];
+                    for (uint32_t g = 0; g < nb; g += 16) {
+                        // the upper half-wave of a last, half group reads the group's first half again and multiplies it by zeros
+                        const bool in = g + 8 * lhalf < nb;
+                        const uint32_t go = (in ? g : g - 8 * lhalf) * 4;
+                        const float4 a0 = *reinterpret_cast<const float4*>(ap + go), a1 = *reinterpret_cast<const float4*>(ap + go + 16);
+                        float4 b0v = *reinterpret_cast<const float4*>(bp + go), b1v = *reinterpret_cast<const float4*>(bp + go + 16);
+                        if (!in) { b0v = make_float4(0.f, 0.f, 0.f, 0.f); b1v = b0v; }
+                        v8h ah, al, bh, bl;
+                        split(a0, a1, ah, al);
+                        split(b0v, b1v, bh, bl);
+                        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bh, c, 0, 0, 0);
+                        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bl, c, 0, 0, 0);
+                        c = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bh, c, 0, 0, 0);
+                    }
+#pragma unroll
+                    for (int r = 0; r < 16; r++) acc[tm][tn][r] = c[r];
+                }
+        }
     }
 
     if (SILU) {

@@ -10,8 +10,8 @@
 //         First term: codes (q - 8) * g under the scale fp16(d*sc_j / g), with the integer g = 9..15 that brings g * fp16(d*sc_j / g)
 //         closest to d*sc_j (d*sc_j has up to 17 significant bits, fp16 has 11: among seven distinct roundings the best is
 //         typically within 4e-5 of it, relative; that residue times the block's centred dot product is all that is dropped).
-//         Second term: the block sums of the activations times an f32 coefficient per (row, block), a small f32 matmul of
-//         depth K/32 that the GEMM kernel runs on the matrix unit in front of its epilogue (its mt_a / mt_w operands).
+//         Second term: the block sums of the activations times a coefficient per (row, block), a small matmul of depth K/32
+//         that the GEMM kernel runs on the f16 matrix unit in front of its epilogue (its mt_a / mt_w operands: hi | lo pairs).
 //   Q6_K  w = d * sc_h * q, q = -32..31, sc_h an int8 per 16-element half.  sc_h * q = 64 hi + lo with lo in [-32, 31] and hi
 //         in [-63, 64]: a block becomes two blocks of a matrix of depth 2K, the hi codes under the scale 64 d and the lo codes
 //         under d.  Both scales are exact fp16 numbers (d is one), so nothing is dropped at all; the activations go in twice
@@ -26,6 +26,15 @@
 namespace fh {
 
 namespace {
+
+// The operands of the minimum term travel as two fp16 numbers in the 4 bytes of an f32 slot: hi = fp16(x), lo = fp16(x - hi)
+// (x to 2^-22 relative).  The GEMM multiplies them on the f16 matrix unit as hi*hi + hi*lo + lo*hi.  Powers of two keep both
+// sides in fp16's range: activation block sums (up to 32 times the largest activation) arrive times 2^-8, coefficients times 2^8.
+__device__ __forceinline__ float hi_lo_f16(float x) {
+    const uint16_t h = f32_to_f16_bits(x);
+    const uint16_t l = f32_to_f16_bits(x - f16_bits_to_f32(h));
+    return __uint_as_float((uint32_t)h | ((uint32_t)l << 16));
+}
 
 // One thread per (row, 32-element block).  Planes of the source as gemv_kquant.hip lays them out.
 __global__ __launch_bounds__(256) void twin_q4k_kernel(const uint8_t* __restrict__ qs, const uint8_t* __restrict__ meta, uint32_t K, uint64_t total,
@@ -58,7 +67,7 @@ __global__ __launch_bounds__(256) void twin_q4k_kernel(const uint8_t* __restrict
         if (e < err) { err = e; g = cand; s16 = h; }
     }
     ts[id] = s16;
-    coef[id] = 8.0f * s - dmin * (float)mn;
+    coef[id] = hi_lo_f16((8.0f * s - dmin * (float)mn) * 256.0f);
     // sub-block j = 2c + hi: element i is the low (hi = 0) or high nibble of byte 32 c + i
     const uint8_t* src = qs + (n * (K / 256) + sb) * 128 + 32 * c;
     const uint32_t sh = (j & 1) * 4;
@@ -98,7 +107,7 @@ __global__ __launch_bounds__(256) void twin_q6k_kernel(const uint8_t* __restrict
     }
 }
 
-// a_s[m][b] * sum of block b's codes, f32 [M][K/32].  `neg_odd`: the codes of odd blocks arrive negated.
+// a_s[m][b] * sum of block b's codes * 2^-8 as a hi | lo pair of fp16 numbers, [M][K/32] slots of 4 bytes.  `neg_odd`: the codes of odd blocks arrive negated.
 __global__ __launch_bounds__(256) void act_block_sums_kernel(const int8_t* __restrict__ aq, const uint16_t* __restrict__ as, uint64_t total,
                                                            uint32_t nblk, uint32_t neg_odd, float* __restrict__ out) {
     const uint64_t id = (uint64_t)blockIdx.x * 256 + threadIdx.x;       // m * nblk + b
@@ -112,7 +121,7 @@ __global__ __launch_bounds__(256) void act_block_sums_kernel(const int8_t* __res
     sum = __builtin_amdgcn_sdot4(a1.x, ones, sum, false); sum = __builtin_amdgcn_sdot4(a1.y, ones, sum, false);
     sum = __builtin_amdgcn_sdot4(a1.z, ones, sum, false); sum = __builtin_amdgcn_sdot4(a1.w, ones, sum, false);
     if (neg_odd && ((id % nblk) & 1u)) sum = -sum;
-    out[id] = f16_bits_to_f32(as[id]) * (float)sum;
+    out[id] = hi_lo_f16(f16_bits_to_f32(as[id]) * (float)sum * 0.00390625f);
 }
 
 // Every pair of activation blocks twice, [M][2 K/32] blocks: blocks 2p, 2p + 1 of a row become 2p, 2p + 1, 2p, 2p + 1 (the hi
